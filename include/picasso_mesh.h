@@ -1,0 +1,168 @@
+/*
+ * picasso_mesh.h -- C ABI of libpicasso_mesh.so (MI355X / gfx950).
+ *
+ * Replaces, for the mesh-convolution and mesh (un)pooling path, the three pybind11
+ * torch extensions of EnyaHermite/PicassoPlus:
+ *     mesh_conv3d   (picasso/mesh/pi_modules/source/mesh_conv3d.cpp:272-279)
+ *     mesh_pool3d   (picasso/mesh/pi_modules/source/mesh_pool3d.cpp:151-157)
+ *     mesh_unpool3d (picasso/mesh/pi_modules/source/mesh_unpool3d.cpp:81-85)
+ *
+ * Conventions
+ *   - Every pointer is a DEVICE pointer owned by the caller (PyTorch's allocator in the
+ *     Python binding).  Features are float32, indices int32, all arrays row-major and
+ *     densely packed, exactly what the reference's CHECK_INPUT macros enforce
+ *     (mesh_conv3d.cpp:24-30).
+ *   - Outputs and workspaces are allocated by the caller; the library never allocates
+ *     device memory.  Outputs need no pre-clearing: every element is written.
+ *   - `stream` is a hipStream_t passed as void*; work is enqueued there and the call
+ *     returns without synchronising.
+ *   - Return value 0 = success.  Non-zero = failure; pmesh_last_error() then returns a
+ *     thread-local message.  Argument errors are detected before anything is launched.
+ *   - Reductions run over sorted adjacency (CSR) in a fixed order: results are
+ *     bit-reproducible from run to run, unlike the reference's float atomics.
+ *   - Entry points are re-entrant; they keep no global mutable state.
+ *
+ * Symbols: cout = c*r + m is the depth-multiplied output channel of the V2F / F2V
+ * convolutions, (C, r) = filter.shape[1:].
+ */
+#ifndef PICASSO_MESH_H
+#define PICASSO_MESH_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void *pmesh_stream_t;
+
+/* ABI revision of this header; bumped on any signature change. */
+int pmesh_abi_version(void);
+/* Message of the last failing call on the calling thread ("" if none). */
+const char *pmesh_last_error(void);
+
+/* ------------------------------------------------------------------ adjacency (CSR)
+ * The reference scatters with float atomics and therefore needs no adjacency.  Here the
+ * scatter ops are segmented reductions over these arrays, built once per index tensor
+ * and reused by every conv of a mesh level (forward and backward).
+ */
+
+/* Vertex -> incident (facet, corner) list.
+ *   key(e) = vt_map ? vt_map[face[e]] : face[e]   for e = 3*f + corner, e in [0, 3*Nf)
+ *   rowptr[v] .. rowptr[v+1]: slots of row v, v in [0, n_rows); colidx holds e, ascending
+ *   within a row; entries with key < 0 are dropped (rowptr[n_rows] = number kept).
+ *   rowptr: n_rows+1 ints, colidx: 3*Nf ints.
+ * Serves facet2vertex forward (rows = output vertices, mesh_conv3d_gpu.cu:318-326) and
+ * vertex2facet input-backward (rows = input vertices, vt_map = NULL, :213-216). */
+size_t pmesh_vertex_csr_workspace_bytes(int64_t n_facets, int64_t n_rows);
+int pmesh_build_vertex_csr(const int32_t *face, const int32_t *vt_map, int64_t n_facets,
+                           int64_t n_vt_map, int64_t n_rows, int32_t *rowptr, int32_t *colidx,
+                           void *workspace, size_t workspace_bytes, pmesh_stream_t stream);
+
+/* Coarse vertex -> member list of a decimation cluster map.
+ *   rep(v) = vt_replace[v] < 0 ? -vt_replace[v] : v ;  key(v) = vt_map[rep(v)]
+ *   rowptr: n_coarse+1 ints; members: n_fine ints, ascending within a row.
+ * Serves max/avg pool forward and unpool backward (mesh_pool3d_gpu.cu:39-58,109-129,
+ * mesh_unpool3d_gpu.cu:27-46). */
+size_t pmesh_cluster_csr_workspace_bytes(int64_t n_fine, int64_t n_coarse);
+int pmesh_build_cluster_csr(const int32_t *vt_replace, const int32_t *vt_map, int64_t n_fine,
+                            int64_t n_coarse, int32_t *rowptr, int32_t *members,
+                            void *workspace, size_t workspace_bytes, pmesh_stream_t stream);
+
+/* ------------------------------------------------------------------ vertex2facet
+ * replaces vertex2facet_forward / vertex2facet_backward (mesh_conv3d.cpp:123-188)
+ *   input (Nv,C)  filter (3,C,r)  face (Nf,3)  ->  output (Nf,C*r)
+ */
+int pmesh_v2f_fwd(const float *input, const float *filter, const int32_t *face, float *output,
+                  int64_t Nv, int64_t Nf, int C, int r, pmesh_stream_t stream);
+
+/* grad_input (Nv,C), grad_filter (3,C,r).  rowptr/colidx: vertex CSR with vt_map = NULL,
+ * n_rows = Nv.  workspace: pmesh_v2f_bwd_workspace_bytes(C, r) bytes. */
+size_t pmesh_v2f_bwd_workspace_bytes(int C, int r);
+int pmesh_v2f_bwd(const float *grad_output, const float *input, const float *filter,
+                  const int32_t *face, const int32_t *rowptr, const int32_t *colidx,
+                  float *grad_input, float *grad_filter, void *workspace, size_t workspace_bytes,
+                  int64_t Nv, int64_t Nf, int C, int r, pmesh_stream_t stream);
+
+/* ------------------------------------------------------------------ facet2vertex
+ * replaces facet2vertex_forward / facet2vertex_backward (mesh_conv3d.cpp:33-122)
+ *   input (Nf,C)  filter (K,C,r)  coeff (Nf,K)  face (Nf,3)  nf_count (NvOut)  vt_map (NvIn)
+ *   -> output (NvOut, C*r).  rowptr/colidx: vertex CSR with this vt_map, n_rows = NvOut.
+ */
+int pmesh_f2v_fwd(const float *input, const float *filter, const float *coeff,
+                  const int32_t *nf_count, const int32_t *rowptr, const int32_t *colidx,
+                  float *output, int64_t Nf, int64_t NvOut, int C, int r, int K,
+                  pmesh_stream_t stream);
+
+/* grad_input (Nf,C), grad_filter (K,C,r).  workspace: pmesh_f2v_bwd_workspace_bytes(C,r,K). */
+size_t pmesh_f2v_bwd_workspace_bytes(int C, int r, int K);
+int pmesh_f2v_bwd(const float *grad_output, const float *input, const float *filter,
+                  const float *coeff, const int32_t *face, const int32_t *nf_count,
+                  const int32_t *vt_map, float *grad_input, float *grad_filter, void *workspace,
+                  size_t workspace_bytes, int64_t Nf, int64_t NvIn, int64_t NvOut, int C, int r,
+                  int K, pmesh_stream_t stream);
+
+/* ------------------------------------------------------------------ facet2facet
+ * replaces facet2facet_forward / facet2facet_backward (mesh_conv3d.cpp:192-269)
+ *   texture (T,Cin)  filter (Cout,Cin,F)  bary_coeff (T,F)  cum_texture (Nf, inclusive
+ *   running total of texture points per facet, as layers.py:57 prepares it)
+ *   -> output (Nf,Cout).   F <= 50 as in mesh_conv3d.cpp:211.
+ */
+int pmesh_f2f_fwd(const float *texture, const float *filter, const float *bary_coeff,
+                  const int32_t *cum_texture, float *output, int64_t T, int64_t Nf, int Cin,
+                  int Cout, int F, pmesh_stream_t stream);
+
+/* grad_texture (T,Cin), grad_filter (Cout,Cin,F).
+ * workspace: pmesh_f2f_bwd_workspace_bytes(Cin,Cout,F). */
+size_t pmesh_f2f_bwd_workspace_bytes(int Cin, int Cout, int F);
+int pmesh_f2f_bwd(const float *grad_output, const float *texture, const float *filter,
+                  const float *bary_coeff, const int32_t *cum_texture, float *grad_texture,
+                  float *grad_filter, void *workspace, size_t workspace_bytes, int64_t T,
+                  int64_t Nf, int Cin, int Cout, int F, pmesh_stream_t stream);
+
+/* ------------------------------------------------------------------ mesh pooling
+ * replaces max_forward / max_backward / avg_forward / avg_backward
+ * (mesh_pool3d.cpp:29-148).  rowptr/members: cluster CSR of (vt_replace, vt_map).
+ *   input (NvIn,C) -> output (NvOut,C) [, max_index (NvOut,C) int32]
+ * Ties in the arg-max resolve to the smallest vertex index; rows without members get
+ * value 0 and index 0, as the reference's zero-filled outputs do (mesh_pool3d.cpp:53-54).
+ */
+int pmesh_pool_max_fwd(const float *input, const int32_t *rowptr, const int32_t *members,
+                       float *output, int32_t *max_index, int64_t NvIn, int64_t NvOut, int C,
+                       pmesh_stream_t stream);
+/* grad_input (NvIn,C).  With vt_replace/vt_map given, grad_input is produced by a gather
+ * (row v takes grad_output where max_index names v) -- valid when max_index came from
+ * pmesh_pool_max_fwd on the same maps.  With both NULL it is the reference's zero-fill
+ * plus scatter by max_index (mesh_pool3d_gpu.cu:90-102). */
+int pmesh_pool_max_bwd(const float *grad_output, const int32_t *max_index,
+                       const int32_t *vt_replace, const int32_t *vt_map, float *grad_input,
+                       int64_t NvIn, int64_t NvOut, int C, pmesh_stream_t stream);
+int pmesh_pool_avg_fwd(const float *input, const int32_t *vt_replace, const int32_t *rowptr,
+                       const int32_t *members, float *output, int64_t NvIn, int64_t NvOut, int C,
+                       pmesh_stream_t stream);
+int pmesh_pool_avg_bwd(const float *grad_output, const int32_t *vt_replace,
+                       const int32_t *vt_map, float *grad_input, int64_t NvIn, int64_t NvOut,
+                       int C, pmesh_stream_t stream);
+
+/* ------------------------------------------------------------------ mesh unpooling
+ * replaces forward / backward of mesh_unpool3d (mesh_unpool3d.cpp:20-78)
+ *   input (NvCoarse,C) -> output (NvFine,C): every fine vertex copies its cluster's row.
+ */
+int pmesh_unpool_fwd(const float *input, const int32_t *vt_replace, const int32_t *vt_map,
+                     float *output, int64_t NvCoarse, int64_t NvFine, int C,
+                     pmesh_stream_t stream);
+int pmesh_unpool_bwd(const float *grad_output, const int32_t *rowptr, const int32_t *members,
+                     float *grad_input, int64_t NvCoarse, int64_t NvFine, int C,
+                     pmesh_stream_t stream);
+
+/* ------------------------------------------------------------------ spherical harmonics
+ * replaces SphHarmCoeff.__call__ + torch_sph_harm_reorder (picasso/mesh/layers.py:348-356,
+ * picasso/math_utils.py:10-62): real SH basis of degree <= L (L <= 5) at the directions
+ * xyz (N,3) -> out (N,(L+1)^2); a zero vector evaluates at direction (1,0,0). */
+int pmesh_sph_harm(const float *xyz, float *out, int64_t N, int L, pmesh_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* PICASSO_MESH_H */

@@ -1,0 +1,84 @@
+"""ctypes binding of libpicasso_mesh.so (declared in include/picasso_mesh.h).
+
+The library is the only compute path of this package: when it is missing the ops raise,
+they never fall back to another implementation.
+"""
+import ctypes
+import os
+
+from ctypes import c_char_p, c_int, c_int64, c_size_t, c_void_p
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "csrc", "libpicasso_mesh.so")
+ABI_VERSION = 1
+
+P, I, L, Z = c_void_p, c_int, c_int64, c_size_t
+
+# name -> (restype, argtypes); mirrors include/picasso_mesh.h one to one
+SIGNATURES = {
+    "pmesh_abi_version": (I, []),
+    "pmesh_last_error": (c_char_p, []),
+    "pmesh_vertex_csr_workspace_bytes": (Z, [L, L]),
+    "pmesh_build_vertex_csr": (I, [P, P, L, L, L, P, P, P, Z, P]),
+    "pmesh_cluster_csr_workspace_bytes": (Z, [L, L]),
+    "pmesh_build_cluster_csr": (I, [P, P, L, L, P, P, P, Z, P]),
+    "pmesh_v2f_fwd": (I, [P, P, P, P, L, L, I, I, P]),
+    "pmesh_v2f_bwd_workspace_bytes": (Z, [I, I]),
+    "pmesh_v2f_bwd": (I, [P, P, P, P, P, P, P, P, P, Z, L, L, I, I, P]),
+    "pmesh_f2v_fwd": (I, [P, P, P, P, P, P, P, L, L, I, I, I, P]),
+    "pmesh_f2v_bwd_workspace_bytes": (Z, [I, I, I]),
+    "pmesh_f2v_bwd": (I, [P, P, P, P, P, P, P, P, P, P, Z, L, L, L, I, I, I, P]),
+    "pmesh_f2f_fwd": (I, [P, P, P, P, P, L, L, I, I, I, P]),
+    "pmesh_f2f_bwd_workspace_bytes": (Z, [I, I, I]),
+    "pmesh_f2f_bwd": (I, [P, P, P, P, P, P, P, P, Z, L, L, I, I, I, P]),
+    "pmesh_pool_max_fwd": (I, [P, P, P, P, P, L, L, I, P]),
+    "pmesh_pool_max_bwd": (I, [P, P, P, P, P, L, L, I, P]),
+    "pmesh_pool_avg_fwd": (I, [P, P, P, P, P, L, L, I, P]),
+    "pmesh_pool_avg_bwd": (I, [P, P, P, P, L, L, I, P]),
+    "pmesh_unpool_fwd": (I, [P, P, P, P, L, L, I, P]),
+    "pmesh_unpool_bwd": (I, [P, P, P, P, L, L, I, P]),
+    "pmesh_sph_harm": (I, [P, P, L, I, P]),
+}
+
+_lib = None
+
+
+class NativeLibraryError(RuntimeError):
+    pass
+
+
+def load():
+    """Load the shared library once; raise loudly when it is absent or stale."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise NativeLibraryError(
+            "libpicasso_mesh.so is not built (%s). Build it with `python -m picassoplus_amd.build`; "
+            "this package has no other compute path." % LIB_PATH)
+    lib = ctypes.CDLL(LIB_PATH)
+    for name, (res, args) in SIGNATURES.items():
+        try:
+            fn = getattr(lib, name)
+        except AttributeError as exc:
+            raise NativeLibraryError("libpicasso_mesh.so lacks symbol %s; rebuild it" % name) from exc
+        fn.restype, fn.argtypes = res, args
+    if lib.pmesh_abi_version() != ABI_VERSION:
+        raise NativeLibraryError("libpicasso_mesh.so has ABI %d, binding expects %d; rebuild it"
+                                 % (lib.pmesh_abi_version(), ABI_VERSION))
+    _lib = lib
+    return lib
+
+
+def call(name, *args):
+    """Invoke an int-returning entry point; non-zero becomes RuntimeError(last error)."""
+    lib = load()
+    rc = getattr(lib, name)(*args)
+    if rc != 0:
+        msg = lib.pmesh_last_error()
+        raise RuntimeError("%s failed: %s" % (name, msg.decode() if msg else "unknown error"))
+
+
+def query(name, *args):
+    """Invoke a size query (host only)."""
+    return int(getattr(load(), name)(*args))

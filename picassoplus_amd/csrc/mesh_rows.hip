@@ -1,0 +1,809 @@
+// HBM-bound row kernels of the mesh-conv path: vertex2facet, facet2vertex, mesh pooling and
+// unpooling, spherical-harmonic basis.  gfx950, wave64.
+//
+// Common shape: one feature row (C floats) is owned by a power-of-two group of lanes, each
+// lane moving V consecutive channels per access (V = 4 -> 16-byte accesses, used whenever the
+// depth multiplier r is 1 and C is a multiple of 4; V = 1 covers every other shape).
+// Scatter-type ops of the reference (float atomicAdd / CAS atomicMax) are run here as
+// gathers over sorted CSR adjacency, so every sum has a fixed order and no atomics exist.
+// Filter gradients are reduced in two stages: per-workgroup partial sums written to a
+// workspace, then a fixed-order reduction over workgroups.
+#include "common.h"
+#include "../../include/picasso_mesh.h"
+
+namespace pmesh {
+
+// ----------------------------------------------------------------------------------------
+// small device helpers
+// ----------------------------------------------------------------------------------------
+__device__ __forceinline__ void load_coeff16(const float *p, int kc, bool vec_ok, float (&cf)[16])
+{
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+        if (vec_ok && 4 * g + 4 <= kc) {
+            const float4 t = *reinterpret_cast<const float4 *>(p + 4 * g);
+            cf[4 * g] = t.x; cf[4 * g + 1] = t.y; cf[4 * g + 2] = t.z; cf[4 * g + 3] = t.w;
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) cf[4 * g + i] = (4 * g + i < kc) ? p[4 * g + i] : 0.f;
+        }
+    }
+}
+
+// Sum `acc` over the row slots of a workgroup in slot order and let slot 0 store the result.
+template <int V>
+__device__ __forceinline__ void block_reduce_store(const Pack<V> &acc, float *red, float *dst,
+                                                   bool active, int lane, int slot, int lpr, int rpb)
+{
+#pragma unroll
+    for (int i = 0; i < V; ++i) red[threadIdx.x * V + i] = acc.v[i];
+    __syncthreads();
+    if (slot == 0 && active) {
+        Pack<V> s = zero_pack<V>();
+        for (int t = 0; t < rpb; ++t)
+#pragma unroll
+            for (int i = 0; i < V; ++i) s.v[i] += red[(t * lpr + lane) * V + i];
+        stp<V>(dst, s);
+    }
+    __syncthreads();
+}
+
+// out[o] = sum_g partial[g*n + o], g ascending within four interleaved slices, slices added
+// in order.  One workgroup covers 64 outputs.
+__global__ __launch_bounds__(kBlock) void reduce_partials_k(const float *__restrict__ partial,
+                                                            float *__restrict__ out, int G, int n)
+{
+    __shared__ float red[4][64];
+    const int j = threadIdx.x & 63, s = threadIdx.x >> 6;
+    const int o = blockIdx.x * 64 + j;
+    float sum = 0.f;
+    if (o < n)
+        for (int g = s; g < G; g += 4) sum += partial[(size_t)g * n + o];
+    red[s][j] = sum;
+    __syncthreads();
+    if (s == 0 && o < n) out[o] = ((red[0][j] + red[1][j]) + red[2][j]) + red[3][j];
+}
+
+__global__ __launch_bounds__(kBlock) void fill_zero_k(float *__restrict__ p, int64_t n)
+{
+    const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i < n) p[i] = 0.f;
+}
+
+// ----------------------------------------------------------------------------------------
+// vertex2facet forward:  out[f, c*r+m] = sum_k filt[k,c,m] * in[face[f,k], c]
+// ----------------------------------------------------------------------------------------
+template <int V>
+__global__ __launch_bounds__(kBlock) void v2f_fwd_k(const float *__restrict__ in,
+                                                    const float *__restrict__ filt,
+                                                    const int *__restrict__ face,
+                                                    float *__restrict__ out, int64_t Nf, int C, int r,
+                                                    int Q, int lpr_log2)
+{
+    const int lpr = 1 << lpr_log2;
+    const int lane = threadIdx.x & (lpr - 1), slot = threadIdx.x >> lpr_log2;
+    const int64_t f = (int64_t)blockIdx.x * (kBlock >> lpr_log2) + slot;
+    if (f >= Nf) return;
+    const int Co = C * r;
+    const int64_t v0 = face[3 * f], v1 = face[3 * f + 1], v2 = face[3 * f + 2];
+    for (int q = lane; q < Q; q += lpr) {
+        const int co = q * V;
+        const int c = (V == 4) ? co : co / r;
+        const Pack<V> a0 = ldp<V>(in + v0 * C + c), a1 = ldp<V>(in + v1 * C + c), a2 = ldp<V>(in + v2 * C + c);
+        const Pack<V> f0 = ldp<V>(filt + co), f1 = ldp<V>(filt + Co + co), f2 = ldp<V>(filt + 2 * Co + co);
+        Pack<V> o;
+#pragma unroll
+        for (int i = 0; i < V; ++i) o.v[i] = fmaf(f2.v[i], a2.v[i], fmaf(f1.v[i], a1.v[i], f0.v[i] * a0.v[i]));
+        stp<V>(out + f * Co + co, o);
+    }
+}
+
+// ----------------------------------------------------------------------------------------
+// vertex2facet backward, one pass over the vertex -> (facet, corner) adjacency:
+//   gin[v,c]     = sum_{(f,k) at v} sum_m gout[f,c*r+m] * filt[k,c,m]
+//   gfilt[k,c,m] = sum_v in[v,c] * sum_{(f,k) at v} gout[f,c*r+m]        (per-workgroup partials)
+// Lanes own input channels; the depth multiplier is an outer loop (V = 4 implies r = 1).
+// ----------------------------------------------------------------------------------------
+template <int V>
+__global__ __launch_bounds__(kBlock) void v2f_bwd_k(const float *__restrict__ gout,
+                                                    const float *__restrict__ in,
+                                                    const float *__restrict__ filt,
+                                                    const int *__restrict__ rowptr,
+                                                    const int *__restrict__ colidx,
+                                                    float *__restrict__ gin, float *__restrict__ partial,
+                                                    int64_t Nv, int C, int r, int Q, int lpr_log2,
+                                                    int64_t rows_per_block)
+{
+    __shared__ float red[kBlock * V];
+    const int lpr = 1 << lpr_log2, rpb = kBlock >> lpr_log2;
+    const int lane = threadIdx.x & (lpr - 1), slot = threadIdx.x >> lpr_log2;
+    const int Co = C * r;
+    const int64_t rbeg = (int64_t)blockIdx.x * rows_per_block;
+    const int64_t rend = (rbeg + rows_per_block < Nv) ? rbeg + rows_per_block : Nv;
+    for (int m = 0; m < r; ++m)
+        for (int q0 = 0; q0 < Q; q0 += lpr) {
+            const int q = q0 + lane;
+            const bool active = q < Q;
+            const int c = q * V;
+            const int co = (V == 4) ? c : c * r + m;
+            Pack<V> fk[3], acc[3];
+#pragma unroll
+            for (int k = 0; k < 3; ++k) {
+                fk[k] = active ? ldp<V>(filt + k * Co + co) : zero_pack<V>();
+                acc[k] = zero_pack<V>();
+            }
+            if (active)
+                for (int64_t row = rbeg + slot; row < rend; row += rpb) {
+                    const int e0 = rowptr[row], e1 = rowptr[row + 1];
+                    const Pack<V> x = ldp<V>(in + row * C + c);
+                    Pack<V> g = zero_pack<V>(), s[3];
+#pragma unroll
+                    for (int k = 0; k < 3; ++k) s[k] = zero_pack<V>();
+                    for (int e = e0; e < e1; ++e) {
+                        const int ent = colidx[e];
+                        const int f = ent / 3, k = ent - 3 * f;
+                        const Pack<V> go = ldp<V>(gout + (int64_t)f * Co + co);
+#pragma unroll
+                        for (int i = 0; i < V; ++i) {
+                            const float w = (k == 0) ? fk[0].v[i] : (k == 1) ? fk[1].v[i] : fk[2].v[i];
+                            g.v[i] = fmaf(go.v[i], w, g.v[i]);
+                            s[0].v[i] += (k == 0) ? go.v[i] : 0.f;
+                            s[1].v[i] += (k == 1) ? go.v[i] : 0.f;
+                            s[2].v[i] += (k == 2) ? go.v[i] : 0.f;
+                        }
+                    }
+#pragma unroll
+                    for (int k = 0; k < 3; ++k)
+#pragma unroll
+                        for (int i = 0; i < V; ++i) acc[k].v[i] = fmaf(s[k].v[i], x.v[i], acc[k].v[i]);
+                    float *gp = gin + row * C + c;
+                    if (m == 0) {
+                        stp<V>(gp, g);
+                    } else {
+#pragma unroll
+                        for (int i = 0; i < V; ++i) gp[i] += g.v[i];
+                    }
+                }
+#pragma unroll
+            for (int k = 0; k < 3; ++k)
+                block_reduce_store<V>(acc[k], red, partial + ((size_t)blockIdx.x * 3 + k) * Co + co, active,
+                                      lane, slot, lpr, rpb);
+        }
+}
+
+// ----------------------------------------------------------------------------------------
+// facet2vertex forward over the output-vertex -> facet adjacency:
+//   out[vo,co] = (1/nf[vo]) * sum_{f at vo} in[f,c] * sum_k coeff[f,k] * filt[k,co]
+// ----------------------------------------------------------------------------------------
+template <int V>
+__global__ __launch_bounds__(kBlock) void f2v_fwd_k(const float *__restrict__ in,
+                                                    const float *__restrict__ filt,
+                                                    const float *__restrict__ coeff,
+                                                    const int *__restrict__ nfcount,
+                                                    const int *__restrict__ rowptr,
+                                                    const int *__restrict__ colidx,
+                                                    float *__restrict__ out, int64_t NvOut, int C, int r,
+                                                    int K, int Q, int lpr_log2, int coeff_vec)
+{
+    const int lpr = 1 << lpr_log2;
+    const int lane = threadIdx.x & (lpr - 1), slot = threadIdx.x >> lpr_log2;
+    const int64_t row = (int64_t)blockIdx.x * (kBlock >> lpr_log2) + slot;
+    if (row >= NvOut) return;
+    const int Co = C * r;
+    const int e0 = rowptr[row], e1 = rowptr[row + 1];
+    const float inv = (e1 > e0) ? 1.0f / (float)nfcount[row] : 0.f;
+    for (int q = lane; q < Q; q += lpr) {
+        const int co = q * V;
+        const int c = (V == 4) ? co : co / r;
+        Pack<V> acc = zero_pack<V>();
+        for (int k0 = 0; k0 < K; k0 += 16) {
+            const int kc = (K - k0 < 16) ? K - k0 : 16;
+            Pack<V> fl[16];
+#pragma unroll
+            for (int k = 0; k < 16; ++k) fl[k] = (k < kc) ? ldp<V>(filt + (size_t)(k0 + k) * Co + co) : zero_pack<V>();
+            for (int e = e0; e < e1; ++e) {
+                const int64_t f = colidx[e] / 3;
+                const Pack<V> x = ldp<V>(in + f * C + c);
+                float cf[16];
+                load_coeff16(coeff + f * K + k0, kc, coeff_vec != 0, cf);
+                Pack<V> w = zero_pack<V>();
+#pragma unroll
+                for (int k = 0; k < 16; ++k)
+#pragma unroll
+                    for (int i = 0; i < V; ++i) w.v[i] = fmaf(cf[k], fl[k].v[i], w.v[i]);
+#pragma unroll
+                for (int i = 0; i < V; ++i) acc.v[i] = fmaf(w.v[i], x.v[i], acc.v[i]);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < V; ++i) acc.v[i] *= inv;
+        stp<V>(out + row * Co + co, acc);
+    }
+}
+
+// ----------------------------------------------------------------------------------------
+// facet2vertex backward, one pass over the facets:
+//   s[f,co]      = sum_{corner j, vo_j >= 0} gout[vo_j,co] / nf[vo_j]
+//   gin[f,c]     = sum_m s[f,co] * w[f,co],   w = sum_k coeff[f,k] * filt[k,co]
+//   gfilt[k,co]  = sum_f coeff[f,k] * in[f,c] * s[f,co]                (per-workgroup partials)
+// ----------------------------------------------------------------------------------------
+template <int V>
+__global__ __launch_bounds__(kBlock) void f2v_bwd_k(const float *__restrict__ gout,
+                                                    const float *__restrict__ in,
+                                                    const float *__restrict__ filt,
+                                                    const float *__restrict__ coeff,
+                                                    const int *__restrict__ face,
+                                                    const int *__restrict__ nfcount,
+                                                    const int *__restrict__ vtmap,
+                                                    float *__restrict__ gin, float *__restrict__ partial,
+                                                    int64_t Nf, int64_t NvOut, int C, int r, int K, int Q,
+                                                    int lpr_log2, int coeff_vec, int64_t rows_per_block)
+{
+    __shared__ float red[kBlock * V];
+    const int lpr = 1 << lpr_log2, rpb = kBlock >> lpr_log2;
+    const int lane = threadIdx.x & (lpr - 1), slot = threadIdx.x >> lpr_log2;
+    const int Co = C * r;
+    const int64_t fbeg = (int64_t)blockIdx.x * rows_per_block;
+    const int64_t fend = (fbeg + rows_per_block < Nf) ? fbeg + rows_per_block : Nf;
+    for (int m = 0; m < r; ++m)
+        for (int q0 = 0; q0 < Q; q0 += lpr) {
+            const int q = q0 + lane;
+            const bool active = q < Q;
+            const int c = q * V;
+            const int co = (V == 4) ? c : c * r + m;
+            for (int k0 = 0; k0 < K; k0 += 16) {
+                const int kc = (K - k0 < 16) ? K - k0 : 16;
+                const bool first = (m == 0 && k0 == 0);
+                Pack<V> fl[16], acc[16];
+#pragma unroll
+                for (int k = 0; k < 16; ++k) {
+                    fl[k] = (active && k < kc) ? ldp<V>(filt + (size_t)(k0 + k) * Co + co) : zero_pack<V>();
+                    acc[k] = zero_pack<V>();
+                }
+                if (active)
+                    for (int64_t f = fbeg + slot; f < fend; f += rpb) {
+                        Pack<V> s = zero_pack<V>();
+#pragma unroll
+                        for (int j = 0; j < 3; ++j) {
+                            const int vo = vtmap[face[3 * f + j]];
+                            if (vo >= 0 && vo < NvOut) {
+                                const float inv = 1.0f / (float)nfcount[vo];
+                                const Pack<V> g = ldp<V>(gout + (int64_t)vo * Co + co);
+#pragma unroll
+                                for (int i = 0; i < V; ++i) s.v[i] = fmaf(g.v[i], inv, s.v[i]);
+                            }
+                        }
+                        const Pack<V> x = ldp<V>(in + f * C + c);
+                        float cf[16];
+                        load_coeff16(coeff + f * K + k0, kc, coeff_vec != 0, cf);
+                        Pack<V> w = zero_pack<V>(), t;
+#pragma unroll
+                        for (int k = 0; k < 16; ++k)
+#pragma unroll
+                            for (int i = 0; i < V; ++i) w.v[i] = fmaf(cf[k], fl[k].v[i], w.v[i]);
+#pragma unroll
+                        for (int i = 0; i < V; ++i) t.v[i] = x.v[i] * s.v[i];
+#pragma unroll
+                        for (int k = 0; k < 16; ++k)
+#pragma unroll
+                            for (int i = 0; i < V; ++i) acc[k].v[i] = fmaf(cf[k], t.v[i], acc[k].v[i]);
+                        float *gp = gin + f * C + c;
+                        if (first) {
+                            Pack<V> gi;
+#pragma unroll
+                            for (int i = 0; i < V; ++i) gi.v[i] = s.v[i] * w.v[i];
+                            stp<V>(gp, gi);
+                        } else {
+#pragma unroll
+                            for (int i = 0; i < V; ++i) gp[i] = fmaf(s.v[i], w.v[i], gp[i]);
+                        }
+                    }
+#pragma unroll
+                for (int k = 0; k < 16; ++k)
+                    if (k < kc)
+                        block_reduce_store<V>(acc[k], red,
+                                              partial + ((size_t)blockIdx.x * K + k0 + k) * Co + co, active,
+                                              lane, slot, lpr, rpb);
+            }
+        }
+}
+
+// ----------------------------------------------------------------------------------------
+// pooling / unpooling over decimation clusters
+//   rep(v) = vt_replace[v] < 0 ? -vt_replace[v] : v ;  vo(v) = vt_map[rep(v)] ;
+//   cnt(v) = vt_replace[rep(v)] + 1
+// ----------------------------------------------------------------------------------------
+__device__ __forceinline__ int cluster_of(const int *__restrict__ vtrep, const int *__restrict__ vtmap,
+                                          int64_t v, int64_t n_fine, int64_t n_coarse, int *cnt)
+{
+    const int rp = vtrep[v];
+    const int64_t rep = rp < 0 ? -(int64_t)rp : v;
+    if (rep >= n_fine) return -1;
+    const int vo = vtmap[rep];
+    if (vo < 0 || vo >= n_coarse) return -1;
+    if (cnt) *cnt = vtrep[rep] + 1;
+    return vo;
+}
+
+// max pooling forward over the coarse-vertex -> members adjacency (members ascending):
+// running maximum that ignores NaN, first (smallest) member attaining it is the arg-max.
+template <int V>
+__global__ __launch_bounds__(kBlock) void pool_max_fwd_k(const float *__restrict__ in,
+                                                         const int *__restrict__ rowptr,
+                                                         const int *__restrict__ members,
+                                                         float *__restrict__ out, int *__restrict__ maxidx,
+                                                         int64_t NvOut, int C, int Q, int lpr_log2)
+{
+    const int lpr = 1 << lpr_log2;
+    const int lane = threadIdx.x & (lpr - 1), slot = threadIdx.x >> lpr_log2;
+    const int64_t row = (int64_t)blockIdx.x * (kBlock >> lpr_log2) + slot;
+    if (row >= NvOut) return;
+    const int e0 = rowptr[row], e1 = rowptr[row + 1];
+    for (int q = lane; q < Q; q += lpr) {
+        const int c = q * V;
+        Pack<V> best = zero_pack<V>();
+        int idx[V];
+#pragma unroll
+        for (int i = 0; i < V; ++i) idx[i] = 0;
+        for (int e = e0; e < e1; ++e) {
+            const int v = members[e];
+            const Pack<V> x = ldp<V>(in + (int64_t)v * C + c);
+#pragma unroll
+            for (int i = 0; i < V; ++i) {
+                const float b = best.v[i], y = x.v[i];
+                const bool take = (e == e0) || (y > b) || (b != b && y == y);
+                best.v[i] = take ? y : b;
+                idx[i] = take ? ((y == y) ? v : 0) : idx[i];
+            }
+        }
+        stp<V>(out + row * C + c, best);
+        if constexpr (V == 4) {
+            *reinterpret_cast<int4 *>(maxidx + row * C + c) = make_int4(idx[0], idx[1], idx[2], idx[3]);
+        } else {
+#pragma unroll
+            for (int i = 0; i < V; ++i) maxidx[row * C + c + i] = idx[i];
+        }
+    }
+}
+
+// segmented sum over cluster members: AVG weights each member by 1/cnt(member) (avg pool
+// forward), otherwise plain sum (unpool backward).
+template <int V, bool AVG>
+__global__ __launch_bounds__(kBlock) void cluster_sum_k(const float *__restrict__ in,
+                                                        const int *__restrict__ vtrep,
+                                                        const int *__restrict__ rowptr,
+                                                        const int *__restrict__ members,
+                                                        float *__restrict__ out, int64_t NvFine,
+                                                        int64_t NvOut, int C, int Q, int lpr_log2)
+{
+    const int lpr = 1 << lpr_log2;
+    const int lane = threadIdx.x & (lpr - 1), slot = threadIdx.x >> lpr_log2;
+    const int64_t row = (int64_t)blockIdx.x * (kBlock >> lpr_log2) + slot;
+    if (row >= NvOut) return;
+    const int e0 = rowptr[row], e1 = rowptr[row + 1];
+    for (int q = lane; q < Q; q += lpr) {
+        const int c = q * V;
+        Pack<V> acc = zero_pack<V>();
+        for (int e = e0; e < e1; ++e) {
+            const int64_t v = members[e];
+            float wgt = 1.f;
+            if constexpr (AVG) {
+                const int rp = vtrep[v];
+                const int64_t rep = rp < 0 ? -(int64_t)rp : v;
+                wgt = 1.0f / (float)(vtrep[rep < NvFine ? rep : v] + 1);
+            }
+            const Pack<V> x = ldp<V>(in + v * C + c);
+#pragma unroll
+            for (int i = 0; i < V; ++i) acc.v[i] = AVG ? fmaf(x.v[i], wgt, acc.v[i]) : acc.v[i] + x.v[i];
+        }
+        stp<V>(out + row * C + c, acc);
+    }
+}
+
+// per-fine-vertex gathers from the cluster's coarse row.
+enum FineMode { kUnpoolFwd = 0, kAvgBwd = 1, kMaxBwdGather = 2 };
+
+template <int V, int MODE>
+__global__ __launch_bounds__(kBlock) void fine_gather_k(const float *__restrict__ coarse,
+                                                        const int *__restrict__ maxidx,
+                                                        const int *__restrict__ vtrep,
+                                                        const int *__restrict__ vtmap,
+                                                        float *__restrict__ fine, int64_t NvFine,
+                                                        int64_t NvCoarse, int C, int Q, int lpr_log2)
+{
+    const int lpr = 1 << lpr_log2;
+    const int lane = threadIdx.x & (lpr - 1), slot = threadIdx.x >> lpr_log2;
+    const int64_t v = (int64_t)blockIdx.x * (kBlock >> lpr_log2) + slot;
+    if (v >= NvFine) return;
+    int cnt = 1;
+    const int vo = cluster_of(vtrep, vtmap, v, NvFine, NvCoarse, &cnt);
+    for (int q = lane; q < Q; q += lpr) {
+        const int c = q * V;
+        Pack<V> o = zero_pack<V>();
+        if (vo >= 0) {
+            const Pack<V> g = ldp<V>(coarse + (int64_t)vo * C + c);
+            if constexpr (MODE == kUnpoolFwd) {
+                o = g;
+            } else if constexpr (MODE == kAvgBwd) {
+                const float d = (float)cnt;
+#pragma unroll
+                for (int i = 0; i < V; ++i) o.v[i] = g.v[i] / d;
+            } else {
+#pragma unroll
+                for (int i = 0; i < V; ++i) o.v[i] = (maxidx[(int64_t)vo * C + c + i] == (int)v) ? g.v[i] : 0.f;
+            }
+        }
+        stp<V>(fine + v * C + c, o);
+    }
+}
+
+// reference form of max-pool backward: scatter by max_index into a cleared gradient.
+__global__ __launch_bounds__(kBlock) void pool_max_bwd_scatter_k(const float *__restrict__ gout,
+                                                                 const int *__restrict__ maxidx,
+                                                                 float *__restrict__ gin, int64_t n,
+                                                                 int C, int64_t NvIn)
+{
+    const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= n) return;
+    const int ch = (int)(i % C);
+    const int64_t v = maxidx[i];
+    if (v >= 0 && v < NvIn) gin[v * C + ch] = gout[i];
+}
+
+// ----------------------------------------------------------------------------------------
+// real spherical-harmonic basis, degree <= 5, cartesian closed forms on the unit direction
+// ----------------------------------------------------------------------------------------
+__global__ __launch_bounds__(kBlock) void sph_harm_k(const float *__restrict__ xyz, float *__restrict__ out,
+                                                     int64_t N, int L)
+{
+    const int64_t n = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (n >= N) return;
+    float x = xyz[3 * n], y = xyz[3 * n + 1], z = xyz[3 * n + 2];
+    // scale-free normalisation; the zero vector evaluates at (1,0,0) like atan2(0,0) = 0 does
+    const float mx = fmaxf(fabsf(x), fmaxf(fabsf(y), fabsf(z)));
+    if (mx > 0.f && mx < INFINITY) {
+        x /= mx; y /= mx; z /= mx;
+        const float inv = 1.0f / sqrtf(x * x + y * y + z * z);
+        x *= inv; y *= inv; z *= inv;
+    } else {
+        x = 1.f; y = 0.f; z = 0.f;
+    }
+    const float PI = 3.14159265358979323846f;
+    const int B = (L + 1) * (L + 1);
+    float v[36];
+    const float x2 = x * x, y2 = y * y, z2 = z * z, xy = x * y;
+    const float c2 = x2 - y2, s2 = 2.f * xy;                      // sin^2(th) cos/sin(2 phi)
+    const float c3 = x * (x2 - 3.f * y2), s3 = y * (3.f * x2 - y2);  // sin^3(th) cos/sin(3 phi)
+    v[0] = 0.5f * sqrtf(1.f / PI);
+    if (L >= 1) {
+        const float a = 0.5f * sqrtf(1.5f / PI);
+        v[1] = a * x; v[2] = 0.5f * sqrtf(3.f / PI) * z; v[3] = a * y;
+    }
+    if (L >= 2) {
+        const float a = 0.25f * sqrtf(7.5f / PI), b = 0.5f * sqrtf(7.5f / PI);
+        v[4] = a * c2; v[5] = b * x * z; v[6] = 0.25f * sqrtf(5.f / PI) * (3.f * z2 - 1.f);
+        v[7] = a * s2; v[8] = b * y * z;
+    }
+    if (L >= 3) {
+        const float a = 0.125f * sqrtf(35.f / PI), b = 0.25f * sqrtf(52.5f / PI), d = 0.125f * sqrtf(21.f / PI);
+        const float t = 5.f * z2 - 1.f;
+        v[9] = a * c3; v[10] = b * z * c2; v[11] = d * x * t;
+        v[12] = 0.25f * sqrtf(7.f / PI) * z * (5.f * z2 - 3.f);
+        v[13] = a * s3; v[14] = b * z * s2; v[15] = d * y * t;
+    }
+    if (L >= 4) {
+        const float c4 = x2 * x2 - 6.f * x2 * y2 + y2 * y2, s4 = 4.f * xy * c2;
+        const float a = 0.1875f * sqrtf(17.5f / PI), b = 0.375f * sqrtf(35.f / PI);
+        const float d = 0.375f * sqrtf(2.5f / PI), e = 0.375f * sqrtf(5.f / PI);
+        const float t2 = 7.f * z2 - 1.f, t1 = z * (7.f * z2 - 3.f);
+        v[16] = a * c4; v[17] = b * z * c3; v[18] = d * c2 * t2; v[19] = e * x * t1;
+        v[20] = 0.1875f * sqrtf(1.f / PI) * (35.f * z2 * z2 - 30.f * z2 + 3.f);
+        v[21] = a * s4; v[22] = b * z * s3; v[23] = d * s2 * t2; v[24] = e * y * t1;
+    }
+    if (L >= 5) {
+        const float c4 = x2 * x2 - 6.f * x2 * y2 + y2 * y2, s4 = 4.f * xy * c2;
+        const float c5 = x * (x2 * x2 - 10.f * x2 * y2 + 5.f * y2 * y2);
+        const float s5 = y * (5.f * x2 * x2 - 10.f * x2 * y2 + y2 * y2);
+        const float a = 0.09375f * sqrtf(77.f / PI), b = 0.1875f * sqrtf(192.5f / PI);
+        const float d = 0.03125f * sqrtf(385.f / PI), e = 0.125f * sqrtf(577.5f / PI);
+        const float g = 0.0625f * sqrtf(82.5f / PI);
+        const float t3 = 9.f * z2 - 1.f, t2 = z * (3.f * z2 - 1.f), t1 = 21.f * z2 * z2 - 14.f * z2 + 1.f;
+        v[25] = a * c5; v[26] = b * z * c4; v[27] = d * c3 * t3; v[28] = e * c2 * t2; v[29] = g * x * t1;
+        v[30] = 0.0625f * sqrtf(11.f / PI) * z * (63.f * z2 * z2 - 70.f * z2 + 15.f);
+        v[31] = a * s5; v[32] = b * z * s4; v[33] = d * s3 * t3; v[34] = e * s2 * t2; v[35] = g * y * t1;
+    }
+    float *o = out + n * B;
+    for (int i = 0; i < B; ++i) o[i] = v[i];
+}
+
+// ----------------------------------------------------------------------------------------
+// host side
+// ----------------------------------------------------------------------------------------
+static inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// V = 4 needs r == 1, C % 4 == 0 and 16-byte aligned feature arrays.
+static inline int pick_v(int C, int r, std::initializer_list<const void *> ptrs)
+{
+    if (r != 1 || (C & 3)) return 1;
+    for (const void *p : ptrs)
+        if (!aligned16(p)) return 1;
+    return 4;
+}
+
+static int reduce_partials(const float *partial, float *out, int G, int n, hipStream_t st)
+{
+    reduce_partials_k<<<dim3((unsigned)ceil_div(n, 64)), dim3(kBlock), 0, st>>>(partial, out, G, n);
+    PM_LAUNCHED("reduce_partials");
+    return 0;
+}
+
+}  // namespace pmesh
+
+using namespace pmesh;
+
+#define PM_DIMS(name)                                                                     \
+    PM_REQUIRE(C > 0 && r > 0 && (int64_t)C * r <= (1 << 20), name ": bad channel counts C=%d r=%d", C, r)
+
+extern "C" int pmesh_v2f_fwd(const float *input, const float *filter, const int32_t *face, float *output,
+                             int64_t Nv, int64_t Nf, int C, int r, pmesh_stream_t stream)
+{
+    clear_error();
+    PM_DIMS("v2f_fwd");
+    PM_REQUIRE(Nv >= 0 && Nf >= 0, "v2f_fwd: negative size");
+    if (Nf == 0) return 0;
+    PM_REQUIRE(input && filter && face && output, "v2f_fwd: null pointer");
+    PM_REQUIRE(Nv <= INT32_MAX && Nf <= INT32_MAX / 3, "v2f_fwd: sizes exceed int32 indexing");
+    hipStream_t st = (hipStream_t)stream;
+    const int V = pick_v(C, r, {input, filter, output});
+    const RowShape rs = row_shape(C * r / V);
+    const int64_t blocks = ceil_div(Nf, rs.rpb);
+    PM_REQUIRE(grid_ok(blocks), "v2f_fwd: grid too large");
+    if (V == 4)
+        v2f_fwd_k<4><<<dim3((unsigned)blocks), dim3(kBlock), 0, st>>>(input, filter, face, output, Nf, C, r, rs.items, rs.lpr_log2);
+    else
+        v2f_fwd_k<1><<<dim3((unsigned)blocks), dim3(kBlock), 0, st>>>(input, filter, face, output, Nf, C, r, rs.items, rs.lpr_log2);
+    PM_LAUNCHED("v2f_fwd");
+    return 0;
+}
+
+// workspace = per-workgroup partial filter gradients, worst case 1024 workgroups
+extern "C" size_t pmesh_v2f_bwd_workspace_bytes(int C, int r) { return (size_t)1024 * 3 * C * r * sizeof(float); }
+
+extern "C" int pmesh_v2f_bwd(const float *grad_output, const float *input, const float *filter,
+                             const int32_t *face, const int32_t *rowptr, const int32_t *colidx,
+                             float *grad_input, float *grad_filter, void *workspace, size_t workspace_bytes,
+                             int64_t Nv, int64_t Nf, int C, int r, pmesh_stream_t stream)
+{
+    clear_error();
+    (void)face;
+    PM_DIMS("v2f_bwd");
+    PM_REQUIRE(Nv >= 0 && Nf >= 0, "v2f_bwd: negative size");
+    PM_REQUIRE(grad_filter, "v2f_bwd: null grad_filter");
+    PM_REQUIRE(Nv <= INT32_MAX && Nf <= INT32_MAX / 3, "v2f_bwd: sizes exceed int32 indexing");
+    hipStream_t st = (hipStream_t)stream;
+    const int Co = C * r;
+    if (Nv == 0) {
+        fill_zero_k<<<dim3((unsigned)ceil_div(3 * Co, kBlock)), dim3(kBlock), 0, st>>>(grad_filter, 3 * Co);
+        PM_LAUNCHED("v2f_bwd(fill)");
+        return 0;
+    }
+    PM_REQUIRE(grad_output && input && filter && rowptr && colidx && grad_input && workspace, "v2f_bwd: null pointer");
+    const int V = pick_v(C, r, {grad_output, input, filter, grad_input, workspace});
+    const RowShape rs = row_shape(C / V);
+    const int G = persistent_blocks(Nv, rs.rpb);
+    const int64_t rows_per_block = ceil_div(ceil_div(Nv, G), rs.rpb) * rs.rpb;
+    PM_REQUIRE(workspace_bytes >= (size_t)G * 3 * Co * sizeof(float), "v2f_bwd: workspace too small (%zu bytes)", workspace_bytes);
+    float *partial = (float *)workspace;
+    if (V == 4)
+        v2f_bwd_k<4><<<dim3(G), dim3(kBlock), 0, st>>>(grad_output, input, filter, rowptr, colidx, grad_input, partial, Nv, C, r, rs.items, rs.lpr_log2, rows_per_block);
+    else
+        v2f_bwd_k<1><<<dim3(G), dim3(kBlock), 0, st>>>(grad_output, input, filter, rowptr, colidx, grad_input, partial, Nv, C, r, rs.items, rs.lpr_log2, rows_per_block);
+    PM_LAUNCHED("v2f_bwd");
+    return reduce_partials(partial, grad_filter, G, 3 * Co, st);
+}
+
+extern "C" int pmesh_f2v_fwd(const float *input, const float *filter, const float *coeff,
+                             const int32_t *nf_count, const int32_t *rowptr, const int32_t *colidx,
+                             float *output, int64_t Nf, int64_t NvOut, int C, int r, int K,
+                             pmesh_stream_t stream)
+{
+    clear_error();
+    PM_DIMS("f2v_fwd");
+    PM_REQUIRE(K > 0 && K <= 4096, "f2v_fwd: bad filter size K=%d", K);
+    PM_REQUIRE(Nf >= 0 && NvOut >= 0, "f2v_fwd: negative size");
+    if (NvOut == 0) return 0;
+    PM_REQUIRE(input && filter && coeff && nf_count && rowptr && colidx && output, "f2v_fwd: null pointer");
+    PM_REQUIRE(NvOut <= INT32_MAX && Nf <= INT32_MAX / 3, "f2v_fwd: sizes exceed int32 indexing");
+    hipStream_t st = (hipStream_t)stream;
+    const int V = pick_v(C, r, {input, filter, output});
+    const RowShape rs = row_shape(C * r / V);
+    const int64_t blocks = ceil_div(NvOut, rs.rpb);
+    PM_REQUIRE(grid_ok(blocks), "f2v_fwd: grid too large");
+    const int cvec = ((K & 3) == 0 && aligned16(coeff)) ? 1 : 0;
+    if (V == 4)
+        f2v_fwd_k<4><<<dim3((unsigned)blocks), dim3(kBlock), 0, st>>>(input, filter, coeff, nf_count, rowptr, colidx, output, NvOut, C, r, K, rs.items, rs.lpr_log2, cvec);
+    else
+        f2v_fwd_k<1><<<dim3((unsigned)blocks), dim3(kBlock), 0, st>>>(input, filter, coeff, nf_count, rowptr, colidx, output, NvOut, C, r, K, rs.items, rs.lpr_log2, cvec);
+    PM_LAUNCHED("f2v_fwd");
+    return 0;
+}
+
+extern "C" size_t pmesh_f2v_bwd_workspace_bytes(int C, int r, int K) { return (size_t)1024 * K * C * r * sizeof(float); }
+
+extern "C" int pmesh_f2v_bwd(const float *grad_output, const float *input, const float *filter,
+                             const float *coeff, const int32_t *face, const int32_t *nf_count,
+                             const int32_t *vt_map, float *grad_input, float *grad_filter, void *workspace,
+                             size_t workspace_bytes, int64_t Nf, int64_t NvIn, int64_t NvOut, int C, int r,
+                             int K, pmesh_stream_t stream)
+{
+    clear_error();
+    (void)NvIn;
+    PM_DIMS("f2v_bwd");
+    PM_REQUIRE(K > 0 && K <= 4096, "f2v_bwd: bad filter size K=%d", K);
+    PM_REQUIRE(Nf >= 0 && NvOut >= 0, "f2v_bwd: negative size");
+    PM_REQUIRE(grad_filter, "f2v_bwd: null grad_filter");
+    PM_REQUIRE(NvOut <= INT32_MAX && Nf <= INT32_MAX / 3, "f2v_bwd: sizes exceed int32 indexing");
+    hipStream_t st = (hipStream_t)stream;
+    const int Co = C * r;
+    if (Nf == 0) {
+        fill_zero_k<<<dim3((unsigned)ceil_div((int64_t)K * Co, kBlock)), dim3(kBlock), 0, st>>>(grad_filter, (int64_t)K * Co);
+        PM_LAUNCHED("f2v_bwd(fill)");
+        return 0;
+    }
+    PM_REQUIRE(grad_output && input && filter && coeff && face && nf_count && vt_map && grad_input && workspace, "f2v_bwd: null pointer");
+    const int V = pick_v(C, r, {grad_output, input, filter, grad_input, workspace});
+    const RowShape rs = row_shape(C / V);
+    const int G = persistent_blocks(Nf, rs.rpb);
+    const int64_t rows_per_block = ceil_div(ceil_div(Nf, G), rs.rpb) * rs.rpb;
+    PM_REQUIRE(workspace_bytes >= (size_t)G * K * Co * sizeof(float), "f2v_bwd: workspace too small (%zu bytes)", workspace_bytes);
+    const int cvec = ((K & 3) == 0 && aligned16(coeff)) ? 1 : 0;
+    float *partial = (float *)workspace;
+    if (V == 4)
+        f2v_bwd_k<4><<<dim3(G), dim3(kBlock), 0, st>>>(grad_output, input, filter, coeff, face, nf_count, vt_map, grad_input, partial, Nf, NvOut, C, r, K, rs.items, rs.lpr_log2, cvec, rows_per_block);
+    else
+        f2v_bwd_k<1><<<dim3(G), dim3(kBlock), 0, st>>>(grad_output, input, filter, coeff, face, nf_count, vt_map, grad_input, partial, Nf, NvOut, C, r, K, rs.items, rs.lpr_log2, cvec, rows_per_block);
+    PM_LAUNCHED("f2v_bwd");
+    return reduce_partials(partial, grad_filter, G, K * Co, st);
+}
+
+// ---- pooling ---------------------------------------------------------------------------
+#define PM_POOL_DIMS(name)                                                                      \
+    PM_REQUIRE(C > 0 && C <= (1 << 20), name ": bad channel count C=%d", C);                   \
+    PM_REQUIRE(NvIn >= 0 && NvOut >= 0 && NvIn <= INT32_MAX && NvOut <= INT32_MAX, name ": bad vertex counts")
+
+extern "C" int pmesh_pool_max_fwd(const float *input, const int32_t *rowptr, const int32_t *members,
+                                  float *output, int32_t *max_index, int64_t NvIn, int64_t NvOut, int C,
+                                  pmesh_stream_t stream)
+{
+    clear_error();
+    PM_POOL_DIMS("pool_max_fwd");
+    if (NvOut == 0) return 0;
+    PM_REQUIRE(input && rowptr && members && output && max_index, "pool_max_fwd: null pointer");
+    hipStream_t st = (hipStream_t)stream;
+    const int V = (pick_v(C, 1, {input, output, max_index}));
+    const RowShape rs = row_shape(C / V);
+    const int64_t blocks = ceil_div(NvOut, rs.rpb);
+    PM_REQUIRE(grid_ok(blocks), "pool_max_fwd: grid too large");
+    if (V == 4)
+        pool_max_fwd_k<4><<<dim3((unsigned)blocks), dim3(kBlock), 0, st>>>(input, rowptr, members, output, max_index, NvOut, C, rs.items, rs.lpr_log2);
+    else
+        pool_max_fwd_k<1><<<dim3((unsigned)blocks), dim3(kBlock), 0, st>>>(input, rowptr, members, output, max_index, NvOut, C, rs.items, rs.lpr_log2);
+    PM_LAUNCHED("pool_max_fwd");
+    return 0;
+}
+
+template <int MODE>
+static int launch_fine_gather(const char *name, const float *coarse, const int32_t *maxidx,
+                              const int32_t *vtrep, const int32_t *vtmap, float *fine, int64_t NvFine,
+                              int64_t NvCoarse, int C, hipStream_t st)
+{
+    const int V = pick_v(C, 1, {coarse, fine, maxidx ? (const void *)maxidx : (const void *)coarse});
+    const RowShape rs = row_shape(C / V);
+    const int64_t blocks = ceil_div(NvFine, rs.rpb);
+    PM_REQUIRE(grid_ok(blocks), "%s: grid too large", name);
+    if (V == 4)
+        fine_gather_k<4, MODE><<<dim3((unsigned)blocks), dim3(kBlock), 0, st>>>(coarse, maxidx, vtrep, vtmap, fine, NvFine, NvCoarse, C, rs.items, rs.lpr_log2);
+    else
+        fine_gather_k<1, MODE><<<dim3((unsigned)blocks), dim3(kBlock), 0, st>>>(coarse, maxidx, vtrep, vtmap, fine, NvFine, NvCoarse, C, rs.items, rs.lpr_log2);
+    PM_LAUNCHED(name);
+    return 0;
+}
+
+extern "C" int pmesh_pool_max_bwd(const float *grad_output, const int32_t *max_index,
+                                  const int32_t *vt_replace, const int32_t *vt_map, float *grad_input,
+                                  int64_t NvIn, int64_t NvOut, int C, pmesh_stream_t stream)
+{
+    clear_error();
+    PM_POOL_DIMS("pool_max_bwd");
+    if (NvIn == 0) return 0;
+    PM_REQUIRE(grad_input, "pool_max_bwd: null pointer");
+    PM_REQUIRE((vt_replace == nullptr) == (vt_map == nullptr), "pool_max_bwd: pass both cluster maps or neither");
+    hipStream_t st = (hipStream_t)stream;
+    if (vt_replace) {
+        PM_REQUIRE(NvOut == 0 || (grad_output && max_index), "pool_max_bwd: null pointer");
+        return launch_fine_gather<kMaxBwdGather>("pool_max_bwd", grad_output, max_index, vt_replace, vt_map,
+                                                 grad_input, NvIn, NvOut, C, st);
+    }
+    const int64_t n_in = NvIn * C, n_out = NvOut * C;
+    PM_REQUIRE(grid_ok(ceil_div(n_in, kBlock)), "pool_max_bwd: grid too large");
+    fill_zero_k<<<dim3((unsigned)ceil_div(n_in, kBlock)), dim3(kBlock), 0, st>>>(grad_input, n_in);
+    PM_LAUNCHED("pool_max_bwd(fill)");
+    if (n_out == 0) return 0;
+    PM_REQUIRE(grad_output && max_index, "pool_max_bwd: null pointer");
+    pool_max_bwd_scatter_k<<<dim3((unsigned)ceil_div(n_out, kBlock)), dim3(kBlock), 0, st>>>(grad_output, max_index, grad_input, n_out, C, NvIn);
+    PM_LAUNCHED("pool_max_bwd(scatter)");
+    return 0;
+}
+
+template <bool AVG>
+static int launch_cluster_sum(const char *name, const float *in, const int32_t *vtrep, const int32_t *rowptr,
+                              const int32_t *members, float *out, int64_t NvFine, int64_t NvOut, int C,
+                              hipStream_t st)
+{
+    const int V = pick_v(C, 1, {in, out});
+    const RowShape rs = row_shape(C / V);
+    const int64_t blocks = ceil_div(NvOut, rs.rpb);
+    PM_REQUIRE(grid_ok(blocks), "%s: grid too large", name);
+    if (V == 4)
+        cluster_sum_k<4, AVG><<<dim3((unsigned)blocks), dim3(kBlock), 0, st>>>(in, vtrep, rowptr, members, out, NvFine, NvOut, C, rs.items, rs.lpr_log2);
+    else
+        cluster_sum_k<1, AVG><<<dim3((unsigned)blocks), dim3(kBlock), 0, st>>>(in, vtrep, rowptr, members, out, NvFine, NvOut, C, rs.items, rs.lpr_log2);
+    PM_LAUNCHED(name);
+    return 0;
+}
+
+extern "C" int pmesh_pool_avg_fwd(const float *input, const int32_t *vt_replace, const int32_t *rowptr,
+                                  const int32_t *members, float *output, int64_t NvIn, int64_t NvOut, int C,
+                                  pmesh_stream_t stream)
+{
+    clear_error();
+    PM_POOL_DIMS("pool_avg_fwd");
+    if (NvOut == 0) return 0;
+    PM_REQUIRE(input && vt_replace && rowptr && members && output, "pool_avg_fwd: null pointer");
+    return launch_cluster_sum<true>("pool_avg_fwd", input, vt_replace, rowptr, members, output, NvIn, NvOut, C, (hipStream_t)stream);
+}
+
+extern "C" int pmesh_pool_avg_bwd(const float *grad_output, const int32_t *vt_replace, const int32_t *vt_map,
+                                  float *grad_input, int64_t NvIn, int64_t NvOut, int C, pmesh_stream_t stream)
+{
+    clear_error();
+    PM_POOL_DIMS("pool_avg_bwd");
+    if (NvIn == 0) return 0;
+    PM_REQUIRE(vt_replace && vt_map && grad_input && (NvOut == 0 || grad_output), "pool_avg_bwd: null pointer");
+    return launch_fine_gather<kAvgBwd>("pool_avg_bwd", grad_output, nullptr, vt_replace, vt_map, grad_input, NvIn, NvOut, C, (hipStream_t)stream);
+}
+
+extern "C" int pmesh_unpool_fwd(const float *input, const int32_t *vt_replace, const int32_t *vt_map,
+                                float *output, int64_t NvCoarse, int64_t NvFine, int C, pmesh_stream_t stream)
+{
+    clear_error();
+    const int64_t NvIn = NvFine, NvOut = NvCoarse;
+    PM_POOL_DIMS("unpool_fwd");
+    if (NvFine == 0) return 0;
+    PM_REQUIRE(vt_replace && vt_map && output && (NvCoarse == 0 || input), "unpool_fwd: null pointer");
+    return launch_fine_gather<kUnpoolFwd>("unpool_fwd", input, nullptr, vt_replace, vt_map, output, NvFine, NvCoarse, C, (hipStream_t)stream);
+}
+
+extern "C" int pmesh_unpool_bwd(const float *grad_output, const int32_t *rowptr, const int32_t *members,
+                                float *grad_input, int64_t NvCoarse, int64_t NvFine, int C, pmesh_stream_t stream)
+{
+    clear_error();
+    const int64_t NvIn = NvFine, NvOut = NvCoarse;
+    PM_POOL_DIMS("unpool_bwd");
+    if (NvCoarse == 0) return 0;
+    PM_REQUIRE(rowptr && members && grad_input && (NvFine == 0 || grad_output), "unpool_bwd: null pointer");
+    return launch_cluster_sum<false>("unpool_bwd", grad_output, nullptr, rowptr, members, grad_input, NvFine, NvCoarse, C, (hipStream_t)stream);
+}
+
+extern "C" int pmesh_sph_harm(const float *xyz, float *out, int64_t N, int L, pmesh_stream_t stream)
+{
+    clear_error();
+    PM_REQUIRE(L >= 0 && L <= 5, "sph_harm: degree %d not supported (0..5)", L);
+    PM_REQUIRE(N >= 0, "sph_harm: negative size");
+    if (N == 0) return 0;
+    PM_REQUIRE(xyz && out, "sph_harm: null pointer");
+    PM_REQUIRE(grid_ok(ceil_div(N, kBlock)), "sph_harm: grid too large");
+    sph_harm_k<<<dim3((unsigned)ceil_div(N, kBlock)), dim3(kBlock), 0, (hipStream_t)stream>>>(xyz, out, N, L);
+    PM_LAUNCHED("sph_harm");
+    return 0;
+}

@@ -1,0 +1,156 @@
+"""Native mesh convolution ops: counterpart of the reference's ``mesh_conv3d`` extension.
+
+Same six functions, argument order and result shapes as the pybind module defined in
+picasso/mesh/pi_modules/source/mesh_conv3d.cpp:272-279; the arithmetic runs in
+libpicasso_mesh.so (HIP, gfx950) through the C ABI of include/picasso_mesh.h.
+"""
+import torch
+
+from ... import _lib
+from .. import topology
+from ._check import F32, I32, check_input, same_device, stream_of, workspace
+
+
+# ---------------------------------------------------------------- vertex2facet
+def _v2f_dims(input, filter, face):
+    check_input(input, "input", 2, F32)
+    check_input(filter, "filter", 3, F32)
+    check_input(face, "face", 2, I32)
+    C, r = input.shape[1], filter.shape[2]
+    if filter.shape[0] != 3 or filter.shape[1] != C:
+        raise RuntimeError("3 filters required, or input Channel size error of the filter")
+    if face.shape[1] != 3:
+        raise RuntimeError("face must have shape (NfIn, 3)")
+    return input.shape[0], face.shape[0], C, r
+
+
+def vertex2facet_forward(input, filter, face):
+    """mesh_conv3d.cpp:123-152: (NvIn,C),(3,C,r),(NfIn,3) -> (NfIn,C*r)."""
+    Nv, Nf, C, r = _v2f_dims(input, filter, face)
+    dev = same_device(input, filter, face)
+    if Nf and Nv:
+        topology._check_range_cached(face, Nv)
+    with torch.cuda.device(dev):
+        out = torch.empty((Nf, C * r), dtype=F32, device=dev)
+        _lib.call("pmesh_v2f_fwd", input.data_ptr(), filter.data_ptr(), face.data_ptr(), out.data_ptr(),
+                  Nv, Nf, C, r, stream_of(input))
+    return out
+
+
+def vertex2facet_backward(grad_output, input, filter, face):
+    """mesh_conv3d.cpp:153-188 -> [grad_input (NvIn,C), grad_filter (3,C,r)]."""
+    Nv, Nf, C, r = _v2f_dims(input, filter, face)
+    check_input(grad_output, "grad_output", 2, F32)
+    if tuple(grad_output.shape) != (Nf, C * r):
+        raise RuntimeError("grad_output must have shape (NfIn, C*r)")
+    dev = same_device(grad_output, input, filter, face)
+    rowptr, colidx = topology.vertex_csr(face, None, Nv)
+    with torch.cuda.device(dev):
+        gin = torch.empty((Nv, C), dtype=F32, device=dev)
+        gfilt = torch.empty((3, C, r), dtype=F32, device=dev)
+        nbytes = _lib.query("pmesh_v2f_bwd_workspace_bytes", C, r)
+        ws = workspace(nbytes, dev)
+        _lib.call("pmesh_v2f_bwd", grad_output.data_ptr(), input.data_ptr(), filter.data_ptr(), face.data_ptr(),
+                  rowptr.data_ptr(), colidx.data_ptr(), gin.data_ptr(), gfilt.data_ptr(), ws.data_ptr(), nbytes,
+                  Nv, Nf, C, r, stream_of(input))
+    return [gin, gfilt]
+
+
+# ---------------------------------------------------------------- facet2vertex
+def _f2v_dims(input, filter, coeff, face, nf_count, vt_map):
+    check_input(input, "input", 2, F32)
+    check_input(filter, "filter", 3, F32)
+    check_input(coeff, "coeff", 2, F32)
+    check_input(face, "face", 2, I32)
+    check_input(nf_count, "nf_count", 1, I32)
+    check_input(vt_map, "vt_map", 1, I32)
+    Nf, C = input.shape
+    K, r = filter.shape[0], filter.shape[2]
+    if filter.shape[1] != C:
+        raise RuntimeError("Input Channel size error of the filter")
+    if tuple(coeff.shape) != (Nf, K):
+        raise RuntimeError("coeff must have shape (NfIn, filter_size)")
+    if tuple(face.shape) != (Nf, 3):
+        raise RuntimeError("face must have shape (NfIn, 3)")
+    return Nf, C, K, r, nf_count.shape[0], vt_map.shape[0]
+
+
+def facet2vertex_forward(input, filter, coeff, face, nf_count, vt_map):
+    """mesh_conv3d.cpp:33-74 -> (NvOut, C*r)."""
+    Nf, C, K, r, NvOut, NvIn = _f2v_dims(input, filter, coeff, face, nf_count, vt_map)
+    dev = same_device(input, filter, coeff, face, nf_count, vt_map)
+    rowptr, colidx = topology.vertex_csr(face, vt_map, NvOut)
+    with torch.cuda.device(dev):
+        out = torch.empty((NvOut, C * r), dtype=F32, device=dev)
+        _lib.call("pmesh_f2v_fwd", input.data_ptr(), filter.data_ptr(), coeff.data_ptr(), nf_count.data_ptr(),
+                  rowptr.data_ptr(), colidx.data_ptr(), out.data_ptr(), Nf, NvOut, C, r, K, stream_of(input))
+    return out
+
+
+def facet2vertex_backward(grad_output, input, filter, coeff, face, nf_count, vt_map):
+    """mesh_conv3d.cpp:75-122 -> [grad_input (NfIn,C), grad_filter (K,C,r)]."""
+    Nf, C, K, r, NvOut, NvIn = _f2v_dims(input, filter, coeff, face, nf_count, vt_map)
+    check_input(grad_output, "grad_output", 2, F32)
+    if tuple(grad_output.shape) != (NvOut, C * r):
+        raise RuntimeError("grad_output must have shape (NvOut, C*r)")
+    dev = same_device(grad_output, input, filter, coeff, face, nf_count, vt_map)
+    if Nf:
+        topology._check_range_cached(face, NvIn)
+    with torch.cuda.device(dev):
+        gin = torch.empty((Nf, C), dtype=F32, device=dev)
+        gfilt = torch.empty((K, C, r), dtype=F32, device=dev)
+        nbytes = _lib.query("pmesh_f2v_bwd_workspace_bytes", C, r, K)
+        ws = workspace(nbytes, dev)
+        _lib.call("pmesh_f2v_bwd", grad_output.data_ptr(), input.data_ptr(), filter.data_ptr(), coeff.data_ptr(),
+                  face.data_ptr(), nf_count.data_ptr(), vt_map.data_ptr(), gin.data_ptr(), gfilt.data_ptr(),
+                  ws.data_ptr(), nbytes, Nf, NvIn, NvOut, C, r, K, stream_of(input))
+    return [gin, gfilt]
+
+
+# ---------------------------------------------------------------- facet2facet
+def _f2f_dims(input, filter, bary_coeff, num_texture, forward):
+    check_input(input, "input", 2, F32)
+    check_input(filter, "filter", 3, F32)
+    check_input(bary_coeff, "bary_coeff", 2, F32)
+    check_input(num_texture, "num_texture", 1, I32)
+    T, Cin = input.shape
+    Cout, _, F = filter.shape
+    if filter.shape[1] != Cin:
+        raise RuntimeError("input Channel size error of the filter.")
+    if F > 50:
+        raise RuntimeError("A maximum of 50 filters are supported in face2face convolution.")
+    if bary_coeff.shape[1] != F:
+        raise RuntimeError("Dimension of bary_coeff mismatches number of filters.")
+    if bary_coeff.shape[0] != T:
+        raise RuntimeError("The shape of bary_coeff should be (NiK, Dim)).")
+    return T, Cin, Cout, F, num_texture.shape[0]
+
+
+def facet2facet_forward(input, filter, bary_coeff, num_texture):
+    """mesh_conv3d.cpp:192-228; ``num_texture`` is the inclusive running total per facet."""
+    T, Cin, Cout, F, Nf = _f2f_dims(input, filter, bary_coeff, num_texture, True)
+    dev = same_device(input, filter, bary_coeff, num_texture)
+    with torch.cuda.device(dev):
+        out = torch.empty((Nf, Cout), dtype=F32, device=dev)
+        _lib.call("pmesh_f2f_fwd", input.data_ptr(), filter.data_ptr(), bary_coeff.data_ptr(),
+                  num_texture.data_ptr(), out.data_ptr(), T, Nf, Cin, Cout, F, stream_of(input))
+    return out
+
+
+def facet2facet_backward(grad_output, input, filter, bary_coeff, num_texture):
+    """mesh_conv3d.cpp:229-269 -> [grad_input (NiK,Cin), grad_filter (Cout,Cin,F)]."""
+    T, Cin, Cout, F, Nf = _f2f_dims(input, filter, bary_coeff, num_texture, False)
+    check_input(grad_output, "grad_output", 2, F32)
+    if tuple(grad_output.shape) != (Nf, Cout):
+        raise RuntimeError("grad_output must have shape (NfIn, Cout)")
+    dev = same_device(grad_output, input, filter, bary_coeff, num_texture)
+    with torch.cuda.device(dev):
+        # rows past the last facet's segment receive no gradient
+        gin = torch.zeros((T, Cin), dtype=F32, device=dev)
+        gfilt = torch.empty((Cout, Cin, F), dtype=F32, device=dev)
+        nbytes = _lib.query("pmesh_f2f_bwd_workspace_bytes", Cin, Cout, F)
+        ws = workspace(nbytes, dev)
+        _lib.call("pmesh_f2f_bwd", grad_output.data_ptr(), input.data_ptr(), filter.data_ptr(),
+                  bary_coeff.data_ptr(), num_texture.data_ptr(), gin.data_ptr(), gfilt.data_ptr(),
+                  ws.data_ptr(), nbytes, T, Nf, Cin, Cout, F, stream_of(input))
+    return [gin, gfilt]

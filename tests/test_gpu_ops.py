@@ -1,0 +1,265 @@
+"""Parity of the HIP kernels with the CPU oracle, called through the reference-shaped API.
+
+Reference arithmetic: brute-force loops (oracle/mesh_loops.inc) in float64 for small cases,
+the vectorised float64 restatement (oracle/torch_ref.py) for medium ones.  Bar: index arrays
+and arg-max indices bit-exact, float32 features and gradients within 1e-5 of max |reference|.
+"""
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import loops, torch_ref
+from picassoplus_amd import synthetic as S
+from picassoplus_amd.mesh import topology
+from picassoplus_amd.mesh.layers import sph_harm_values
+from picassoplus_amd.mesh.pi_modules import (conv3d, mesh_conv3d, mesh_pool3d, mesh_unpool3d, pool3d,
+                                             unpool3d)
+from util import assert_close, dev, mesh_case, rel_err, strided_vt_map, texture_case
+
+pytestmark = pytest.mark.gpu
+
+
+def say(*a):
+    print(*a, flush=True)
+    sys.stdout.flush()
+
+
+# ------------------------------------------------------------------ adjacency
+@pytest.mark.parametrize("mesh", ["tetra", "octa", "sphere2", "room_small"])
+@pytest.mark.parametrize("strided", [False, True])
+def test_vertex_csr_exact(cuda, mesh, strided):
+    say("case vertex_csr", mesh, strided)
+    v, f = mesh_case(mesh)
+    rng = np.random.default_rng(1)
+    nv = v.shape[0]
+    if strided:
+        vt_map, n_rows = strided_vt_map(rng, nv)
+        keys = vt_map[f.reshape(-1).astype(np.int64)]
+    else:
+        vt_map, n_rows = None, nv
+        keys = f.reshape(-1).astype(np.int64)
+    e = np.arange(keys.shape[0])
+    ok = keys >= 0
+    order = np.argsort(keys[ok], kind="stable")
+    col_ref = e[ok][order].astype(np.int32)
+    rowptr_ref = np.concatenate([[0], np.cumsum(np.bincount(keys[ok], minlength=n_rows))]).astype(np.int32)
+    rowptr, colidx = topology.vertex_csr(dev(f, cuda), dev(vt_map, cuda) if strided else None, n_rows)
+    torch.cuda.synchronize()
+    assert np.array_equal(rowptr.cpu().numpy(), rowptr_ref)
+    assert np.array_equal(colidx.cpu().numpy()[:col_ref.shape[0]], col_ref)
+
+
+@pytest.mark.parametrize("spatial", [True, False])
+def test_cluster_csr_exact(cuda, spatial):
+    say("case cluster_csr", spatial)
+    rng = np.random.default_rng(2)
+    vt_replace, vt_map, nvo = S.cluster_maps(rng, 5000, spatial=spatial, orphan_frac=0.05)
+    vo, _ = torch_ref.cluster_maps(torch.from_numpy(vt_replace), torch.from_numpy(vt_map))
+    vo = vo.numpy().astype(np.int64)
+    ok = vo >= 0
+    ids = np.arange(vo.shape[0])
+    order = np.argsort(vo[ok], kind="stable")
+    mem_ref = ids[ok][order].astype(np.int32)
+    rowptr_ref = np.concatenate([[0], np.cumsum(np.bincount(vo[ok], minlength=nvo))]).astype(np.int32)
+    rowptr, members = topology.cluster_csr(dev(vt_replace, cuda), dev(vt_map, cuda), nvo)
+    torch.cuda.synchronize()
+    assert np.array_equal(rowptr.cpu().numpy(), rowptr_ref)
+    assert np.array_equal(members.cpu().numpy()[:mem_ref.shape[0]], mem_ref)
+
+
+# ------------------------------------------------------------------ vertex2facet
+@pytest.mark.parametrize("mesh,C,r", [("tetra", 4, 1), ("octa", 5, 2), ("sphere2", 32, 1), ("sphere3", 64, 1),
+                                      ("room_small", 64, 1), ("sphere2", 7, 3), ("torus", 130, 1),
+                                      ("octa", 2048, 1), ("sphere2", 96, 1)])
+def test_v2f_parity(cuda, mesh, C, r):
+    say("case v2f", mesh, C, r)
+    v, f = mesh_case(mesh)
+    rng = np.random.default_rng(10)
+    nv, nf = v.shape[0], f.shape[0]
+    x = rng.uniform(-1, 1, (nv, C))
+    filt = rng.normal(0, 0.5, (3, C, r))
+    gout = rng.normal(0, 1, (nf, C * r))
+    out_ref = loops.v2f_fwd(x, filt, f)
+    gin_ref, gfilt_ref = loops.v2f_bwd(gout, x, filt, f)
+    xt = dev(x, cuda, torch.float32).requires_grad_(True)
+    ft = dev(filt, cuda, torch.float32).requires_grad_(True)
+    out = conv3d.vertex2facet(xt, ft, dev(f, cuda))
+    out.backward(dev(gout, cuda, torch.float32))
+    torch.cuda.synchronize()
+    assert_close(out, out_ref, "v2f out")
+    assert_close(xt.grad, gin_ref, "v2f grad_input")
+    assert_close(ft.grad, gfilt_ref, "v2f grad_filter")
+
+
+# ------------------------------------------------------------------ facet2vertex
+@pytest.mark.parametrize("mesh,C,r,K,strided", [("tetra", 4, 1, 16, False), ("octa", 6, 2, 9, True),
+                                                ("sphere2", 32, 1, 16, False), ("sphere3", 64, 1, 16, True),
+                                                ("room_small", 64, 1, 16, False), ("torus", 20, 1, 36, False),
+                                                ("sphere2", 5, 3, 4, True), ("sphere2", 128, 1, 16, False)])
+def test_f2v_parity(cuda, mesh, C, r, K, strided):
+    say("case f2v", mesh, C, r, K, strided)
+    v, f = mesh_case(mesh)
+    rng = np.random.default_rng(11)
+    nv, nf = v.shape[0], f.shape[0]
+    if strided:
+        vt_map, nvo = strided_vt_map(rng, nv)
+    else:
+        vt_map, nvo = np.arange(nv, dtype=np.int32), nv
+    nfc = S.vertex_facet_count(f, vt_map, nvo)
+    x = rng.uniform(-1, 1, (nf, C))
+    filt = rng.normal(0, 0.5, (K, C, r))
+    coeff = rng.normal(0, 0.5, (nf, K))
+    gout = rng.normal(0, 1, (nvo, C * r))
+    out_ref = loops.f2v_fwd(x, filt, coeff, f, np.maximum(nfc, 1), vt_map)
+    gin_ref, gfilt_ref = loops.f2v_bwd(gout, x, filt, coeff, f, np.maximum(nfc, 1), vt_map)
+    xt = dev(x, cuda, torch.float32).requires_grad_(True)
+    ft = dev(filt, cuda, torch.float32).requires_grad_(True)
+    out = conv3d.facet2vertex(xt, ft, dev(coeff, cuda, torch.float32), dev(f, cuda),
+                              dev(np.maximum(nfc, 1), cuda), dev(vt_map, cuda))
+    out.backward(dev(gout, cuda, torch.float32))
+    torch.cuda.synchronize()
+    assert_close(out, out_ref, "f2v out")
+    assert_close(xt.grad, gin_ref, "f2v grad_input")
+    assert_close(ft.grad, gfilt_ref, "f2v grad_filter")
+
+
+def test_f2v_unit_count_is_plain_scatter(cuda):
+    """nf_count = 1 and a one-hot coeff reduce facet2vertex to a scatter-add of filt[k0]*x."""
+    say("case f2v one-hot")
+    v, f = mesh_case("sphere2")
+    rng = np.random.default_rng(12)
+    nv, nf, C, K = v.shape[0], f.shape[0], 8, 16
+    x = rng.uniform(-1, 1, (nf, C)).astype(np.float32)
+    filt = rng.normal(0, 1, (K, C, 1)).astype(np.float32)
+    coeff = np.zeros((nf, K), np.float32)
+    coeff[:, 3] = 1
+    ref = np.zeros((nv, C))
+    np.add.at(ref, f.reshape(-1), np.repeat(x.astype(np.float64) * filt[3, :, 0], 3, axis=0))
+    out = mesh_conv3d.facet2vertex_forward(dev(x, cuda), dev(filt, cuda), dev(coeff, cuda), dev(f, cuda),
+                                           dev(np.ones(nv, np.int32), cuda), dev(np.arange(nv, dtype=np.int32), cuda))
+    torch.cuda.synchronize()
+    assert_close(out, ref, "f2v scatter form")
+
+
+# ------------------------------------------------------------------ facet2facet
+@pytest.mark.parametrize("nf,Cin,Cout,F,kmax", [(10, 3, 8, 16, 3), (100, 3, 32, 16, 5), (200, 64, 64, 16, 9),
+                                                (333, 16, 96, 16, 4), (70, 5, 7, 9, 3), (65, 4, 6, 36, 2),
+                                                (64, 3, 5, 50, 2), (129, 130, 64, 4, 3), (50, 8, 8, 1, 2)])
+def test_f2f_parity(cuda, nf, Cin, Cout, F, kmax):
+    say("case f2f", nf, Cin, Cout, F, kmax)
+    rng = np.random.default_rng(13)
+    counts, bary, owner = texture_case(rng, nf, kmax)
+    T = int(counts.sum())
+    cum = np.cumsum(counts).astype(np.int32)
+    tex = rng.uniform(-1, 1, (T, Cin))
+    sh = rng.normal(0, 0.5, (T, F))
+    filt = rng.normal(0, 0.3, (Cout, Cin, F))
+    gout = rng.normal(0, 1, (nf, Cout))
+    out_ref = loops.f2f_fwd(tex, filt, sh, cum)
+    gin_ref, gfilt_ref = loops.f2f_bwd(gout, tex, filt, sh, cum)
+    tt = dev(tex, cuda, torch.float32).requires_grad_(True)
+    ft = dev(filt, cuda, torch.float32).requires_grad_(True)
+    out = conv3d.facet2facet(tt, ft, dev(sh, cuda, torch.float32), dev(cum, cuda))
+    out.backward(dev(gout, cuda, torch.float32))
+    torch.cuda.synchronize()
+    assert_close(out, out_ref, "f2f out")
+    assert_close(tt.grad, gin_ref, "f2f grad_texture")
+    assert_close(ft.grad, gfilt_ref, "f2f grad_filter")
+
+
+# ------------------------------------------------------------------ pooling
+@pytest.mark.parametrize("nv,C,spatial,orphans", [(50, 4, True, 0.0), (3000, 128, True, 0.05), (3000, 5, False, 0.1),
+                                                  (777, 64, False, 0.0), (100, 1100, True, 0.0)])
+def test_pool_unpool_parity(cuda, nv, C, spatial, orphans):
+    say("case pool", nv, C, spatial, orphans)
+    rng = np.random.default_rng(14)
+    vt_replace, vt_map, nvo = S.cluster_maps(rng, nv, spatial=spatial, orphan_frac=orphans)
+    x = rng.normal(0, 1, (nv, C)).astype(np.float32)
+    gout = rng.normal(0, 1, (nvo, C)).astype(np.float32)
+    gfine = rng.normal(0, 1, (nv, C)).astype(np.float32)
+    vr, vm = dev(vt_replace, cuda), dev(vt_map, cuda)
+    vt_out = torch.zeros(nvo, 3, device=cuda)
+
+    # max pool: value and arg-max bit-exact (inputs are float32 on both sides)
+    out_ref, idx_ref = loops.maxpool_fwd(x, vt_replace, vt_map, nvo, dtype=np.float32)
+    xt = dev(x, cuda).requires_grad_(True)
+    out, idx = mesh_pool3d.max_forward(xt.detach(), vr, vm, vt_out)
+    torch.cuda.synchronize()
+    assert np.array_equal(out.cpu().numpy(), out_ref)
+    assert np.array_equal(idx.cpu().numpy(), idx_ref)
+    y = pool3d.maxPool(xt, vr, vm, vt_out)
+    y.backward(dev(gout, cuda))
+    gin_ref = loops.maxpool_bwd(gout, nv, idx_ref, dtype=np.float32)
+    torch.cuda.synchronize()
+    assert np.array_equal(xt.grad.cpu().numpy(), gin_ref)
+    gin_scatter = mesh_pool3d.max_backward(dev(gout, cuda), xt.detach(), idx)
+    torch.cuda.synchronize()
+    assert np.array_equal(gin_scatter.cpu().numpy(), gin_ref)
+
+    # avg pool
+    xt = dev(x, cuda).requires_grad_(True)
+    y = pool3d.avgPool(xt, vr, vm, vt_out)
+    y.backward(dev(gout, cuda))
+    torch.cuda.synchronize()
+    assert_close(y, loops.avgpool_fwd(x, vt_replace, vt_map, nvo), "avg out")
+    assert_close(xt.grad, loops.avgpool_bwd(gout, vt_replace, vt_map), "avg grad")
+
+    # unpool (copy: exact) and its backward
+    ct = dev(gout, cuda).requires_grad_(True)
+    up = unpool3d.interpolate(ct, vr, vm)
+    up.backward(dev(gfine, cuda))
+    torch.cuda.synchronize()
+    assert np.array_equal(up.detach().cpu().numpy(), loops.unpool_fwd(gout, vt_replace, vt_map, dtype=np.float32))
+    assert_close(ct.grad, loops.unpool_bwd(gfine, nvo, vt_replace, vt_map), "unpool grad")
+
+
+def test_max_pool_tie_rule_and_empty_rows(cuda):
+    """Equal values: the smallest vertex id wins.  Output rows past the last cluster stay 0 / index 0."""
+    say("case pool ties")
+    vt_replace = np.array([0, 2, -1, -1, 0, -6, 1], np.int32)   # clusters {0}, {1,2,3}, {4}, {6,5}
+    vt_map = np.array([0, 1, -1, -1, 2, -1, 3], np.int32)
+    x = np.array([[1, 5], [7, 2], [7, 9], [3, 9], [-4, -4], [0.5, 6], [0.5, -1]], np.float32)
+    out, idx = mesh_pool3d.max_forward(dev(x, cuda), dev(vt_replace, cuda), dev(vt_map, cuda),
+                                       torch.zeros(6, 3, device=cuda))
+    torch.cuda.synchronize()
+    assert out.cpu().tolist() == [[1, 5], [7, 9], [-4, -4], [0.5, 6], [0, 0], [0, 0]]
+    assert idx.cpu().tolist() == [[0, 0], [1, 2], [4, 4], [5, 5], [0, 0], [0, 0]]
+
+
+# ------------------------------------------------------------------ spherical harmonics
+@pytest.mark.parametrize("L", [0, 1, 2, 3, 4, 5])
+def test_sph_harm_parity(cuda, L):
+    say("case sph_harm", L)
+    rng = np.random.default_rng(15)
+    xyz = rng.normal(0, 1, (2000, 3)) * rng.uniform(1e-3, 1e3, (2000, 1))
+    xyz[:7] = [[0, 0, 0], [1, 0, 0], [0, 1, 0], [0, 0, 1], [-1, 0, 0], [0, -1, 0], [0, 0, -1]]
+    xyz32 = xyz.astype(np.float32)
+    ref = loops.sph_harm(xyz32.astype(np.float64), L)
+    out = sph_harm_values(dev(xyz32, cuda), L)
+    torch.cuda.synchronize()
+    assert_close(out, ref, "sph_harm L=%d" % L)
+
+
+# ------------------------------------------------------------------ determinism
+def test_bitwise_reproducible(cuda):
+    say("case determinism")
+    v, f = mesh_case("sphere3")
+    rng = np.random.default_rng(16)
+    nv, nf, C, K = v.shape[0], f.shape[0], 64, 16
+    x = dev(rng.uniform(-1, 1, (nf, C)), cuda, torch.float32)
+    filt = dev(rng.normal(0, 0.5, (K, C, 1)), cuda, torch.float32)
+    coeff = dev(rng.normal(0, 0.5, (nf, K)), cuda, torch.float32)
+    gout = dev(rng.normal(0, 1, (nv, C)), cuda, torch.float32)
+    ft, nfc, vm = dev(f, cuda), dev(S.vertex_facet_count(f, np.arange(nv), nv), cuda), dev(np.arange(nv, dtype=np.int32), cuda)
+    runs = []
+    for _ in range(3):
+        o = mesh_conv3d.facet2vertex_forward(x, filt, coeff, ft, nfc, vm)
+        gi, gf = mesh_conv3d.facet2vertex_backward(gout, x, filt, coeff, ft, nfc, vm)
+        runs.append((o.clone(), gi.clone(), gf.clone()))
+    torch.cuda.synchronize()
+    for a, b in zip(runs[0], runs[1]):
+        assert torch.equal(a, b)
+    for a, b in zip(runs[0], runs[2]):
+        assert torch.equal(a, b)

@@ -1,0 +1,74 @@
+"""Helpers shared by the tests: seeded cases and the parity metric."""
+import numpy as np
+import torch
+
+from picassoplus_amd import synthetic as S
+
+TOL_F32 = 1e-5   # max |y - y*| / max |y*| against the float64 oracle
+
+
+def rel_err(y, ref):
+    y = np.asarray(y, dtype=np.float64)
+    ref = np.asarray(ref, dtype=np.float64)
+    assert y.shape == ref.shape, (y.shape, ref.shape)
+    if ref.size == 0:
+        return 0.0
+    den = np.abs(ref).max()
+    num = np.abs(y - ref).max()
+    return float(num / den) if den > 0 else float(num)
+
+
+def assert_close(y, ref, what, tol=TOL_F32):
+    e = rel_err(y.detach().cpu().numpy() if isinstance(y, torch.Tensor) else y, ref)
+    assert e <= tol, "%s: max rel err %.3e > %.1e" % (what, e, tol)
+    return e
+
+
+def dev(a, device, dtype=None):
+    t = torch.from_numpy(np.ascontiguousarray(a))
+    if dtype is not None:
+        t = t.to(dtype)
+    return t.to(device)
+
+
+def tiny_meshes():
+    """Tetrahedron, octahedron and a 2x2 planar grid: (vertex, face) pairs."""
+    tet_v = np.array([[1, 1, 1], [1, -1, -1], [-1, 1, -1], [-1, -1, 1]], np.float64)
+    tet_f = np.array([[0, 1, 2], [0, 3, 1], [0, 2, 3], [1, 3, 2]], np.int32)
+    oct_v = np.array([[1, 0, 0], [-1, 0, 0], [0, 1, 0], [0, -1, 0], [0, 0, 1], [0, 0, -1]], np.float64)
+    oct_f = np.array([[0, 2, 4], [2, 1, 4], [1, 3, 4], [3, 0, 4], [2, 0, 5], [1, 2, 5], [3, 1, 5], [0, 3, 5]], np.int32)
+    grid_v, grid_f = S.grid_patch(np.random.default_rng(0), 2, 2, (0, 0, 0), (1, 0, 0), (0, 1, 0))
+    return {"tetra": (tet_v, tet_f), "octa": (oct_v, oct_f), "grid2": (grid_v, grid_f)}
+
+
+def mesh_case(name, seed=0):
+    """(vertex, face) for a named mesh."""
+    tm = tiny_meshes()
+    if name in tm:
+        return tm[name]
+    rng = np.random.default_rng(seed)
+    if name.startswith("sphere"):
+        return S.icosphere(int(name[6:]))
+    if name == "torus":
+        return S.torus(24, 16)
+    if name == "room_small":
+        return S.room(rng, scale=0.01)
+    if name == "shapes_small":
+        w = S.shapes_workload(seed=seed, n_meshes=2)
+        return w["vertex"], w["face"]
+    raise KeyError(name)
+
+
+def strided_vt_map(rng, nv, keep=0.6):
+    """Input->output vertex map with dropped vertices (-1), ascending on the kept ones."""
+    kept = rng.random(nv) < keep
+    kept[0] = True
+    vt_map = np.where(kept, np.cumsum(kept) - 1, -1).astype(np.int32)
+    return vt_map, int(kept.sum())
+
+
+def texture_case(rng, nf, kmax=5, empty_frac=0.1):
+    counts = rng.integers(1, kmax + 1, nf).astype(np.int32)
+    counts[rng.random(nf) < empty_frac] = 0
+    counts, bary, owner = S.texture_points(rng, nf, counts)
+    return counts, bary, owner

@@ -1,0 +1,285 @@
+#!/usr/bin/env python3
+"""Benchmark of the mesh-conv hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload scene|shapes|pool] [--scale S]
+
+A step is one forward+backward pass of the layer over one batch of seeded synthetic meshes
+already resident in HBM.  Default workload ``scene``: 8 room-like meshes of about 300 k
+facets each, texture points per facet 1..9 by area, F2F (64 -> 64, SH degree 3) followed by
+F2V (64 -> 64) in float32, gradient dL/dy ~ N(0,1) -- the native ops only; the pointwise
+matmul / bias / ReLU / batch-norm tail of the modules is ordinary PyTorch and not timed.
+
+Prints ONE JSON line with the whole-job throughput in Mfacets/s, the roofline figure of the
+dominant kernel (HIP events on the launch stream, inside the timed region) and the CPU
+baseline (the vectorised oracle in float32 on the host cores, on a bounded sample).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+MFMA_F32_PEAK_TFLOPS = 157.3
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="scene", choices=["scene", "shapes", "pool"])
+    ap.add_argument("--scale", type=float, default=1.0, help="facet-count scale of the scene workload")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    return ap.parse_args()
+
+
+# ---------------------------------------------------------------------------- inputs
+def build_conv_inputs(mesh, C, L, seed, tex_counts="area"):
+    from picassoplus_amd import synthetic as S
+    rng = np.random.default_rng(seed)
+    v, f = mesh["vertex"], mesh["face"]
+    nv, nf = v.shape[0], f.shape[0]
+    normal, area = S.triangle_normals_areas(v, f)
+    counts = S.area_scaled_texture_counts(area) if tex_counts == "area" else np.full(nf, int(tex_counts), np.int32)
+    counts, bary, owner = S.texture_points(rng, nf, counts)
+    B = (L + 1) ** 2
+    return dict(
+        nv=nv, nf=nf, T=int(counts.sum()), C=C, B=B, L=L, face=f, normal=normal.astype(np.float32),
+        counts=counts, bary=bary.astype(np.float32), owner=owner,
+        vt_map=np.arange(nv, dtype=np.int32), nf_count=np.maximum(S.vertex_facet_count(f, np.arange(nv), nv), 1),
+        x=rng.uniform(-1, 1, (nv, C)).astype(np.float32),
+        w_f2f=S.xavier_uniform(rng, (C, C, B), C * B, C * B).astype(np.float32),
+        w_f2v=S.xavier_uniform(rng, (B, C, 1), C, B * C).astype(np.float32),
+        w_v2f=S.xavier_uniform(rng, (3, C, 1), C, 3 * C).astype(np.float32),
+        mf_in=mesh["mf_in"], nv_in=mesh["nv_in"])
+
+
+def conv_bytes_flops(d, ops):
+    """Algorithmic HBM bytes / flops per op: every input read once, every output written once."""
+    Nf, Nv, T, C, B = d["nf"], d["nv"], d["T"], d["C"], d["B"]
+    tab = {
+        "v2f_fwd": (4 * Nv * C + 12 * Nf + 4 * Nf * C, 6 * Nf * C),
+        "v2f_bwd": (4 * Nf * C + 12 * Nf + 8 * Nv * C, 12 * Nf * C),
+        "f2v_fwd": (4 * Nf * C + 4 * Nf * B + 12 * Nf + 8 * Nv + 4 * Nv * C, Nf * C * (2 * B + 7)),
+        "f2v_bwd": (4 * Nv * C + 8 * Nf * C + 4 * Nf * B + 12 * Nf + 8 * Nv, Nf * C * (4 * B + 12)),
+        "f2f_fwd": (4 * T * C + 4 * T * B + 4 * Nf + 4 * C * C * B + 4 * Nf * C, 2 * T * C * B + 2 * Nf * C * B * C),
+        "f2f_bwd_texture": (4 * Nf * C + 4 * T * B + 4 * Nf + 4 * C * C * B + 4 * T * C, 2 * Nf * C * B * C + 2 * T * C * B),
+        "f2f_bwd_filter": (4 * Nf * C + 4 * T * C + 4 * T * B + 4 * Nf + 4 * C * C * B, 2 * Nf * C * B * C + 2 * T * C * B),
+    }
+    return {k: tab[k] for k in ops}
+
+
+class EventTimer:
+    """Brackets every native call with HIP events on the launch stream."""
+
+    def __init__(self, torch):
+        self.torch, self.open, self.pairs, self.on = torch, {}, [], False
+
+    def __call__(self, name, phase):
+        if not self.on:
+            return
+        ev = self.torch.cuda.Event(enable_timing=True)
+        ev.record()
+        if phase == "begin":
+            self.open[name] = ev
+        else:
+            self.pairs.append((name, self.open.pop(name), ev))
+
+    def summary(self):
+        tot, cnt = {}, {}
+        for name, a, b in self.pairs:
+            key = name.replace("pmesh_", "")
+            tot[key] = tot.get(key, 0.0) + a.elapsed_time(b)
+            cnt[key] = cnt.get(key, 0) + 1
+        return {k: tot[k] / cnt[k] for k in tot}
+
+
+# ---------------------------------------------------------------------------- workloads
+def run_conv_layer(args, torch, kind):
+    from picassoplus_amd import _lib, synthetic as S
+    from picassoplus_amd.mesh.layers import sph_harm_values
+    from picassoplus_amd.mesh.pi_modules import conv3d
+    dev = torch.device("cuda:0")
+    C, L = 64, 3
+    if kind == "scene":
+        mesh = S.scene_workload(seed=3000, n_rooms=8, scale=args.scale)
+        d = build_conv_inputs(mesh, C, L, seed=3000)
+        ops = ["f2f_fwd", "f2v_fwd", "f2v_bwd", "f2f_bwd_texture", "f2f_bwd_filter"]
+        name = "scene8x300k_F2F+F2V_C64_L3_fp32_fwd+bwd"
+    else:
+        mesh = S.shapes_workload(seed=2000, n_meshes=16)
+        d = build_conv_inputs(mesh, C, L, seed=2000, tex_counts=3)
+        ops = ["v2f_fwd", "f2f_fwd", "f2v_fwd", "f2v_bwd", "f2f_bwd_texture", "f2f_bwd_filter", "v2f_bwd"]
+        name = "shapes16_V2F+F2F+F2V_C64_L3_fp32_fwd+bwd"
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+    face, vt_map, nfc = t(d["face"]), t(d["vt_map"]), t(d["nf_count"].astype(np.int32))
+    cum = torch.cumsum(t(d["counts"]), 0, dtype=torch.int32)
+    bary = t(d["bary"])
+    owner = t(d["owner"])
+    x = t(d["x"])
+    # texture-point features: barycentric interpolation of the vertex features (set-up, untimed)
+    corner = face.long()[owner]
+    tex = (x[corner[:, 0]] * bary[:, 0:1] + x[corner[:, 1]] * bary[:, 1:2] + x[corner[:, 2]] * bary[:, 2:3]).contiguous()
+    del corner, owner
+    sh = sph_harm_values(bary, L)
+    coeff = sph_harm_values(t(d["normal"]), L)
+    w_f2f, w_f2v, w_v2f = t(d["w_f2f"]), t(d["w_f2v"]), t(d["w_v2f"])
+    gy = torch.randn(d["nv"], C, device=dev, generator=torch.Generator(device=dev).manual_seed(1))
+    tex.requires_grad_(True); w_f2f.requires_grad_(True); w_f2v.requires_grad_(True)
+    if kind == "shapes":
+        x.requires_grad_(True); w_v2f.requires_grad_(True)
+
+    def step():
+        if kind == "scene":
+            y1 = conv3d.facet2facet(tex, w_f2f, sh, cum)
+            y = conv3d.facet2vertex(y1, w_f2v, coeff, face, nfc, vt_map)
+            return torch.autograd.grad(y, [tex, w_f2f, w_f2v], gy)
+        y0 = conv3d.vertex2facet(x, w_v2f, face)
+        y1 = conv3d.facet2facet(tex, w_f2f, sh, cum)
+        y = conv3d.facet2vertex(y0 + y1, w_f2v, coeff, face, nfc, vt_map)
+        return torch.autograd.grad(y, [x, tex, w_v2f, w_f2f, w_f2v], gy)
+
+    timer = EventTimer(torch)
+    _lib.set_call_hook(timer)
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    timer.on = True
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    timer.on = False
+    _lib.set_call_hook(None)
+    ms = (t1 - t0) * 1e3 / args.steps
+    per_op = timer.summary()
+    bf = conv_bytes_flops(d, ops)
+    total_bytes = sum(b for b, _ in bf.values())
+    dom = max(ops, key=lambda k: per_op.get(k, 0.0))
+    dom_ms = per_op[dom]
+    if dom.startswith("f2f"):
+        roof = dict(bound="mfma", achieved=bf[dom][1] / (dom_ms * 1e-3) / 1e12, peak=MFMA_F32_PEAK_TFLOPS, unit="TFLOP/s")
+    else:
+        roof = dict(bound="hbm", achieved=bf[dom][0] / (dom_ms * 1e-3) / 1e9, peak=HBM_PEAK_GBS, unit="GB/s")
+    roof.update(frac=roof["achieved"] / roof["peak"], traffic=None, kernel=dom, kernel_ms=dom_ms)
+    ops_report = {k: dict(ms=per_op.get(k), gbps=bf[k][0] / (per_op[k] * 1e-3) / 1e9,
+                          tflops=bf[k][1] / (per_op[k] * 1e-3) / 1e12) for k in ops if k in per_op}
+    res = dict(value=d["nf"] / (ms * 1e-3) / 1e6, ms_per_step=ms, roofline=roof, ops=ops_report,
+               hbm_gbps=total_bytes / (ms * 1e-3) / 1e9, hbm_frac=total_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+               config=dict(workload=name, facets=d["nf"], vertices=d["nv"], texture_points=d["T"], channels=C,
+                           sh_degree=L, meshes=int(len(d["mf_in"])), algorithmic_bytes=total_bytes))
+    if not args.no_cpu_baseline:
+        res["cpu_baseline"] = cpu_baseline_conv(d, kind, torch)
+    return res
+
+
+def cpu_baseline_conv(d, kind, torch):
+    """Vectorised oracle (float32) on the host cores over the first mesh of the batch only."""
+    from oracle import torch_ref as R
+    torch.set_num_threads(os.cpu_count() or 1)
+    nf, nv = int(d["mf_in"][0]), int(d["nv_in"][0])
+    T = int(d["counts"][:nf].sum())
+    f = torch.from_numpy(d["face"][:nf])
+    cum = torch.cumsum(torch.from_numpy(d["counts"][:nf]), 0, dtype=torch.int32)
+    bary = torch.from_numpy(d["bary"][:T])
+    x = torch.from_numpy(d["x"][:nv])
+    own = torch.from_numpy(d["owner"][:T])
+    corner = f.long()[own]
+    tex = x[corner[:, 0]] * bary[:, 0:1] + x[corner[:, 1]] * bary[:, 1:2] + x[corner[:, 2]] * bary[:, 2:3]
+    sh, coeff = R.sph_harm(bary, d["L"]), R.sph_harm(torch.from_numpy(d["normal"][:nf]), d["L"])
+    w_f2f, w_f2v, w_v2f = (torch.from_numpy(d[k]) for k in ("w_f2f", "w_f2v", "w_v2f"))
+    vt_map, nfc = torch.from_numpy(d["vt_map"][:nv]), torch.from_numpy(d["nf_count"][:nv].astype(np.int32))
+    gy = torch.randn(nv, d["C"])
+    t0 = time.perf_counter()
+    y1 = R.f2f_fwd(tex, w_f2f, sh, cum)
+    if kind == "shapes":
+        y1 = y1 + R.v2f_fwd(x, w_v2f, f)
+    R.f2v_fwd(y1, w_f2v, coeff, f, nfc, vt_map)
+    g1, _ = R.f2v_bwd(gy, y1, w_f2v, coeff, f, nfc, vt_map)
+    R.f2f_bwd(g1, tex, w_f2f, sh, cum)
+    if kind == "shapes":
+        R.v2f_bwd(g1, x, w_v2f, f)
+    dt = time.perf_counter() - t0
+    return dict(value=nf / dt / 1e6, unit="Mfacets/s", cores=torch.get_num_threads(), kind="port",
+                sample="first mesh of the batch (%d facets, %d texture points), one pass, %.1f s" % (nf, T, dt))
+
+
+def run_pool(args, torch):
+    from picassoplus_amd import _lib, synthetic as S
+    from picassoplus_amd.mesh.pi_modules import pool3d, unpool3d
+    dev = torch.device("cuda:0")
+    C, n = 128, 1024
+    rng = np.random.default_rng(4000)
+    nv = n * n
+    vt_replace, vt_map, nvo = S.cluster_maps(rng, nv, mean=4.0, lo=1, hi=12, spatial=True)
+    vr, vm = torch.from_numpy(vt_replace).to(dev), torch.from_numpy(vt_map).to(dev)
+    x = torch.randn(nv, C, device=dev, requires_grad=True)
+    vt_out = torch.zeros(nvo, 3, device=dev)
+    g_c, g_f = torch.randn(nvo, C, device=dev), torch.randn(nv, C, device=dev)
+
+    def step():
+        y = pool3d.maxPool(x, vr, vm, vt_out)
+        torch.autograd.grad(y, x, g_c)
+        y = pool3d.avgPool(x, vr, vm, vt_out)
+        torch.autograd.grad(y, x, g_c)
+        c = y.detach().requires_grad_(True)
+        u = unpool3d.interpolate(c, vr, vm)
+        torch.autograd.grad(u, c, g_f)
+
+    timer = EventTimer(torch)
+    _lib.set_call_hook(timer)
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    timer.on = True
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    _lib.set_call_hook(None)
+    per_op = timer.summary()
+    nb = {"pool_max_fwd": 4 * nv * C + 8 * nv + 8 * nvo * C, "pool_max_bwd": 8 * nvo * C + 4 * nv * C,
+          "pool_avg_fwd": 4 * nv * C + 8 * nv + 4 * nvo * C, "pool_avg_bwd": 4 * nv * C + 8 * nv + 4 * nvo * C,
+          "unpool_fwd": 4 * nvo * C + 8 * nv + 4 * nv * C, "unpool_bwd": 4 * nvo * C + 8 * nv + 4 * nv * C}
+    dom = max(nb, key=lambda k: per_op[k])
+    ach = nb[dom] / (per_op[dom] * 1e-3) / 1e9
+    total = sum(nb.values())
+    return dict(value=nv / (ms * 1e-3) / 1e6, unit="Mvertices/s", ms_per_step=ms,
+                roofline=dict(bound="hbm", achieved=ach, peak=HBM_PEAK_GBS, unit="GB/s", frac=ach / HBM_PEAK_GBS,
+                              traffic=None, kernel=dom, kernel_ms=per_op[dom]),
+                ops={k: dict(ms=per_op[k], gbps=nb[k] / (per_op[k] * 1e-3) / 1e9) for k in nb},
+                hbm_gbps=total / (ms * 1e-3) / 1e9, hbm_frac=total / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                config=dict(workload="plane1024_pool_max+avg+unpool_C128_fp32_fwd+bwd", vertices=nv, coarse=nvo, channels=C))
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this path keeps whole meshes on one device and nothing here "
+              "uses a second one; run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    from picassoplus_amd import _lib
+    _lib.load()
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU (torch.cuda.is_available() is False)", file=sys.stderr)
+        sys.exit(2)
+    torch.cuda.set_device(0)
+    res = run_pool(args, torch) if args.workload == "pool" else run_conv_layer(args, torch, args.workload)
+    line = dict(metric="mesh-conv layer fwd+bwd throughput", value=res.pop("value"), unit=res.pop("unit", "Mfacets/s"),
+                n_gpus=1, steps=args.steps, warmup=args.warmup, ms_per_step=res.pop("ms_per_step"),
+                higher_is_better=True, scaling="weak", vs_baseline=None, dtype="f32", data="synthetic")
+    line.update(res)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -114,12 +114,23 @@ int pmesh_f2f_fwd(const float *texture, const float *filter, const float *bary_c
                   int Cout, int F, pmesh_stream_t stream);
 
 /* grad_texture (T,Cin), grad_filter (Cout,Cin,F).
- * workspace: pmesh_f2f_bwd_workspace_bytes(Cin,Cout,F). */
+ * workspace: pmesh_f2f_bwd_workspace_bytes(Cin,Cout,F).  Only rows of grad_texture that belong
+ * to a facet are written; the caller clears it when texture rows may lie outside every facet.
+ * pmesh_f2f_bwd is the texture half followed by the filter half; each half can be called
+ * alone when only one gradient is wanted (the reference always computes both,
+ * mesh_conv3d_gpu.cu:144-168). */
 size_t pmesh_f2f_bwd_workspace_bytes(int Cin, int Cout, int F);
 int pmesh_f2f_bwd(const float *grad_output, const float *texture, const float *filter,
                   const float *bary_coeff, const int32_t *cum_texture, float *grad_texture,
                   float *grad_filter, void *workspace, size_t workspace_bytes, int64_t T,
                   int64_t Nf, int Cin, int Cout, int F, pmesh_stream_t stream);
+int pmesh_f2f_bwd_texture(const float *grad_output, const float *filter, const float *bary_coeff,
+                          const int32_t *cum_texture, float *grad_texture, int64_t T, int64_t Nf,
+                          int Cin, int Cout, int F, pmesh_stream_t stream);
+int pmesh_f2f_bwd_filter(const float *grad_output, const float *texture, const float *bary_coeff,
+                         const int32_t *cum_texture, float *grad_filter, void *workspace,
+                         size_t workspace_bytes, int64_t T, int64_t Nf, int Cin, int Cout, int F,
+                         pmesh_stream_t stream);
 
 /* ------------------------------------------------------------------ mesh pooling
  * replaces max_forward / max_backward / avg_forward / avg_backward

@@ -31,6 +31,8 @@ SIGNATURES = {
     "pmesh_f2f_fwd": (I, [P, P, P, P, P, L, L, I, I, I, P]),
     "pmesh_f2f_bwd_workspace_bytes": (Z, [I, I, I]),
     "pmesh_f2f_bwd": (I, [P, P, P, P, P, P, P, P, Z, L, L, I, I, I, P]),
+    "pmesh_f2f_bwd_texture": (I, [P, P, P, P, P, L, L, I, I, I, P]),
+    "pmesh_f2f_bwd_filter": (I, [P, P, P, P, P, P, Z, L, L, I, I, I, P]),
     "pmesh_pool_max_fwd": (I, [P, P, P, P, P, L, L, I, P]),
     "pmesh_pool_max_bwd": (I, [P, P, P, P, P, L, L, I, P]),
     "pmesh_pool_avg_fwd": (I, [P, P, P, P, P, L, L, I, P]),
@@ -70,10 +72,25 @@ def load():
     return lib
 
 
+_call_hook = None
+
+
+def set_call_hook(hook):
+    """Install ``hook(name, phase)`` (phase "begin"/"end") around every native call, or None.
+    The benchmark uses it to bracket calls with HIP events on the launch stream."""
+    global _call_hook
+    _call_hook = hook
+
+
 def call(name, *args):
     """Invoke an int-returning entry point; non-zero becomes RuntimeError(last error)."""
     lib = load()
+    hook = _call_hook
+    if hook is not None:
+        hook(name, "begin")
     rc = getattr(lib, name)(*args)
+    if hook is not None:
+        hook(name, "end")
     if rc != 0:
         msg = lib.pmesh_last_error()
         raise RuntimeError("%s failed: %s" % (name, msg.decode() if msg else "unknown error"))

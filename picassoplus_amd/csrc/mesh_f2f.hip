@@ -345,41 +345,64 @@ extern "C" size_t pmesh_f2f_bwd_workspace_bytes(int Cin, int Cout, int F)
     return (size_t)kFiltMaxSplits * Cout * Cin * F * sizeof(float);
 }
 
+extern "C" int pmesh_f2f_bwd_texture(const float *grad_output, const float *filter, const float *bary_coeff,
+                                     const int32_t *cum_texture, float *grad_texture, int64_t T, int64_t Nf,
+                                     int Cin, int Cout, int F, pmesh_stream_t stream)
+{
+    clear_error();
+    PM_F2F_DIMS("f2f_bwd_texture");
+    if (Nf == 0 || T == 0) return 0;
+    PM_REQUIRE(grad_output && filter && bary_coeff && cum_texture && grad_texture, "f2f_bwd_texture: null pointer");
+    const ChunkGeom cg = chunk_geom(Cin, F);
+    const int64_t gx = ceil_div(Nf, 64);
+    PM_REQUIRE(grid_ok(gx), "f2f_bwd_texture: grid too large");
+    const int sh_vec = ((F & 3) == 0 && (reinterpret_cast<uintptr_t>(bary_coeff) & 15u) == 0) ? 1 : 0;
+    f2f_bwd_tex_k<<<dim3((unsigned)gx), dim3(256), 0, (hipStream_t)stream>>>(
+        grad_output, filter, bary_coeff, cum_texture, grad_texture, Nf, (int)T, Cin, Cout, cg, sh_vec);
+    PM_LAUNCHED("f2f_bwd_texture");
+    return 0;
+}
+
+extern "C" int pmesh_f2f_bwd_filter(const float *grad_output, const float *texture, const float *bary_coeff,
+                                    const int32_t *cum_texture, float *grad_filter, void *workspace,
+                                    size_t workspace_bytes, int64_t T, int64_t Nf, int Cin, int Cout, int F,
+                                    pmesh_stream_t stream)
+{
+    clear_error();
+    PM_F2F_DIMS("f2f_bwd_filter");
+    PM_REQUIRE(grad_filter, "f2f_bwd_filter: null grad_filter");
+    hipStream_t st = (hipStream_t)stream;
+    const int64_t nW = (int64_t)Cout * Cin * F;
+    if (Nf == 0 || T == 0) {
+        f2f_fill_zero_k<<<dim3((unsigned)ceil_div(nW, kBlock)), dim3(kBlock), 0, st>>>(grad_filter, nW);
+        PM_LAUNCHED("f2f_bwd_filter(fill)");
+        return 0;
+    }
+    PM_REQUIRE(grad_output && texture && bary_coeff && cum_texture && workspace, "f2f_bwd_filter: null pointer");
+    const ChunkGeom cg = chunk_geom(Cin, F);
+    const int S = filt_splits(Nf);
+    PM_REQUIRE(workspace_bytes >= (size_t)S * nW * sizeof(float), "f2f_bwd_filter: workspace too small (%zu bytes)",
+               workspace_bytes);
+    const int waves = cg.n_chunks < kFiltMaxWaves ? cg.n_chunks : kFiltMaxWaves;
+    const int64_t gy = ceil_div(cg.n_chunks, waves), gz = ceil_div(Cout, 64);
+    PM_REQUIRE(gy <= 65535 && gz <= 65535, "f2f_bwd_filter: grid too large");
+    const int64_t fps = ceil_div(ceil_div(Nf, S), kFiltFB) * kFiltFB;
+    f2f_bwd_filt_k<<<dim3((unsigned)S, (unsigned)gy, (unsigned)gz), dim3(64 * waves), 0, st>>>(
+        grad_output, texture, bary_coeff, cum_texture, (float *)workspace, Nf, (int)T, Cin, Cout, cg, fps, waves);
+    PM_LAUNCHED("f2f_bwd_filter");
+    f2f_reduce_k<<<dim3((unsigned)ceil_div(nW, 64)), dim3(kBlock), 0, st>>>((const float *)workspace, grad_filter, S, nW);
+    PM_LAUNCHED("f2f_bwd_filter(reduce)");
+    return 0;
+}
+
 extern "C" int pmesh_f2f_bwd(const float *grad_output, const float *texture, const float *filter,
                              const float *bary_coeff, const int32_t *cum_texture, float *grad_texture,
                              float *grad_filter, void *workspace, size_t workspace_bytes, int64_t T,
                              int64_t Nf, int Cin, int Cout, int F, pmesh_stream_t stream)
 {
-    clear_error();
-    PM_F2F_DIMS("f2f_bwd");
-    PM_REQUIRE(grad_filter, "f2f_bwd: null grad_filter");
-    hipStream_t st = (hipStream_t)stream;
-    const int64_t nW = (int64_t)Cout * Cin * F;
-    if (Nf == 0 || T == 0) {
-        f2f_fill_zero_k<<<dim3((unsigned)ceil_div(nW, kBlock)), dim3(kBlock), 0, st>>>(grad_filter, nW);
-        PM_LAUNCHED("f2f_bwd(fill)");
-        return 0;
-    }
-    PM_REQUIRE(grad_output && texture && filter && bary_coeff && cum_texture && grad_texture && workspace,
-               "f2f_bwd: null pointer");
-    const ChunkGeom cg = chunk_geom(Cin, F);
-    const int64_t gx = ceil_div(Nf, 64);
-    PM_REQUIRE(grid_ok(gx), "f2f_bwd: grid too large");
-    const int sh_vec = ((F & 3) == 0 && (reinterpret_cast<uintptr_t>(bary_coeff) & 15u) == 0) ? 1 : 0;
-    f2f_bwd_tex_k<<<dim3((unsigned)gx), dim3(256), 0, st>>>(grad_output, filter, bary_coeff, cum_texture,
-                                                            grad_texture, Nf, (int)T, Cin, Cout, cg, sh_vec);
-    PM_LAUNCHED("f2f_bwd(texture)");
-
-    const int S = filt_splits(Nf);
-    PM_REQUIRE(workspace_bytes >= (size_t)S * nW * sizeof(float), "f2f_bwd: workspace too small (%zu bytes)", workspace_bytes);
-    const int waves = cg.n_chunks < kFiltMaxWaves ? cg.n_chunks : kFiltMaxWaves;
-    const int64_t gy = ceil_div(cg.n_chunks, waves), gz = ceil_div(Cout, 64);
-    PM_REQUIRE(gy <= 65535 && gz <= 65535, "f2f_bwd: grid too large");
-    const int64_t fps = ceil_div(ceil_div(Nf, S), kFiltFB) * kFiltFB;
-    f2f_bwd_filt_k<<<dim3((unsigned)S, (unsigned)gy, (unsigned)gz), dim3(64 * waves), 0, st>>>(
-        grad_output, texture, bary_coeff, cum_texture, (float *)workspace, Nf, (int)T, Cin, Cout, cg, fps, waves);
-    PM_LAUNCHED("f2f_bwd(filter)");
-    f2f_reduce_k<<<dim3((unsigned)ceil_div(nW, 64)), dim3(kBlock), 0, st>>>((const float *)workspace, grad_filter, S, nW);
-    PM_LAUNCHED("f2f_bwd(reduce)");
-    return 0;
+    int rc = pmesh_f2f_bwd_texture(grad_output, filter, bary_coeff, cum_texture, grad_texture, T, Nf, Cin, Cout, F,
+                                   stream);
+    if (rc) return rc;
+    return pmesh_f2f_bwd_filter(grad_output, texture, bary_coeff, cum_texture, grad_filter, workspace,
+                                workspace_bytes, T, Nf, Cin, Cout, F, stream);
 }

@@ -150,7 +150,9 @@ def facet2facet_backward(grad_output, input, filter, bary_coeff, num_texture):
         gfilt = torch.empty((Cout, Cin, F), dtype=F32, device=dev)
         nbytes = _lib.query("pmesh_f2f_bwd_workspace_bytes", Cin, Cout, F)
         ws = workspace(nbytes, dev)
-        _lib.call("pmesh_f2f_bwd", grad_output.data_ptr(), input.data_ptr(), filter.data_ptr(),
-                  bary_coeff.data_ptr(), num_texture.data_ptr(), gin.data_ptr(), gfilt.data_ptr(),
-                  ws.data_ptr(), nbytes, T, Nf, Cin, Cout, F, stream_of(input))
+        st = stream_of(input)
+        _lib.call("pmesh_f2f_bwd_texture", grad_output.data_ptr(), filter.data_ptr(), bary_coeff.data_ptr(),
+                  num_texture.data_ptr(), gin.data_ptr(), T, Nf, Cin, Cout, F, st)
+        _lib.call("pmesh_f2f_bwd_filter", grad_output.data_ptr(), input.data_ptr(), bary_coeff.data_ptr(),
+                  num_texture.data_ptr(), gfilt.data_ptr(), ws.data_ptr(), nbytes, T, Nf, Cin, Cout, F, st)
     return [gin, gfilt]

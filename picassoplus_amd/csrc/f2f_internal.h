@@ -1,0 +1,20 @@
+// Internal launchers of the F = 16 (spherical-harmonic degree 3) fast path of facet2facet.
+#pragma once
+#include "common.h"
+
+namespace pmesh {
+
+// The fast path needs F == 16, Cin % 4 == 0 and 16-byte aligned texture / SH / filter arrays.
+bool f2f16_usable(const void *tex, const void *W, const void *sh, int Cin, int F);
+
+int f2f16_fwd(const float *tex, const float *W, const float *sh, const int *cum, float *out, int64_t T,
+              int64_t Nf, int Cin, int Cout, hipStream_t st);
+
+int f2f16_bwd_texture(const float *gout, const float *W, const float *sh, const int *cum, float *gtex, int64_t T,
+                      int64_t Nf, int Cin, int Cout, hipStream_t st);
+
+// writes `splits` partial (Cout x Cin*16) blocks; the caller reduces them in split order
+int f2f16_bwd_filter_partials(const float *gout, const float *tex, const float *sh, const int *cum, float *partial,
+                              int splits, int64_t T, int64_t Nf, int Cin, int Cout, hipStream_t st);
+
+}  // namespace pmesh

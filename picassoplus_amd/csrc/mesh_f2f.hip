@@ -16,7 +16,9 @@
 // CB = max(1, 64 / F) channels = QC = CB*F <= 64 columns (zero padded to 64), so that a chunk
 // of H holds every d of its channels.
 #include "common.h"
+#include "f2f_internal.h"
 #include "../../include/picasso_mesh.h"
+#include <cstdlib>
 
 namespace pmesh {
 
@@ -313,6 +315,14 @@ static inline int filt_splits(int64_t Nf)
     return (int)s;
 }
 
+// PMESH_F2F_GENERIC=1 routes every shape through the shape-generic kernels of this file
+// (read on every call so that tests can flip it).
+static inline bool force_generic()
+{
+    const char *e = getenv("PMESH_F2F_GENERIC");
+    return e && e[0] == '1';
+}
+
 }  // namespace pmesh
 
 using namespace pmesh;
@@ -331,6 +341,8 @@ extern "C" int pmesh_f2f_fwd(const float *texture, const float *filter, const fl
     PM_F2F_DIMS("f2f_fwd");
     if (Nf == 0) return 0;
     PM_REQUIRE(filter && cum_texture && output && (T == 0 || (texture && bary_coeff)), "f2f_fwd: null pointer");
+    if (!force_generic() && f2f16_usable(texture, filter, bary_coeff, Cin, F))
+        return f2f16_fwd(texture, filter, bary_coeff, cum_texture, output, T, Nf, Cin, Cout, (hipStream_t)stream);
     const ChunkGeom cg = chunk_geom(Cin, F);
     const int64_t gx = ceil_div(Nf, 64), gy = ceil_div(Cout, 64);
     PM_REQUIRE(grid_ok(gx) && gy <= 65535, "f2f_fwd: grid too large");
@@ -353,6 +365,9 @@ extern "C" int pmesh_f2f_bwd_texture(const float *grad_output, const float *filt
     PM_F2F_DIMS("f2f_bwd_texture");
     if (Nf == 0 || T == 0) return 0;
     PM_REQUIRE(grad_output && filter && bary_coeff && cum_texture && grad_texture, "f2f_bwd_texture: null pointer");
+    if (!force_generic() && f2f16_usable(grad_texture, filter, bary_coeff, Cin, F))
+        return f2f16_bwd_texture(grad_output, filter, bary_coeff, cum_texture, grad_texture, T, Nf, Cin, Cout,
+                                 (hipStream_t)stream);
     const ChunkGeom cg = chunk_geom(Cin, F);
     const int64_t gx = ceil_div(Nf, 64);
     PM_REQUIRE(grid_ok(gx), "f2f_bwd_texture: grid too large");
@@ -383,6 +398,14 @@ extern "C" int pmesh_f2f_bwd_filter(const float *grad_output, const float *textu
     const int S = filt_splits(Nf);
     PM_REQUIRE(workspace_bytes >= (size_t)S * nW * sizeof(float), "f2f_bwd_filter: workspace too small (%zu bytes)",
                workspace_bytes);
+    if (!force_generic() && f2f16_usable(texture, texture, bary_coeff, Cin, F)) {
+        int rc = f2f16_bwd_filter_partials(grad_output, texture, bary_coeff, cum_texture, (float *)workspace, S, T, Nf,
+                                           Cin, Cout, st);
+        if (rc) return rc;
+        f2f_reduce_k<<<dim3((unsigned)ceil_div(nW, 64)), dim3(kBlock), 0, st>>>((const float *)workspace, grad_filter, S, nW);
+        PM_LAUNCHED("f2f_bwd_filter(reduce)");
+        return 0;
+    }
     const int waves = cg.n_chunks < kFiltMaxWaves ? cg.n_chunks : kFiltMaxWaves;
     const int64_t gy = ceil_div(cg.n_chunks, waves), gz = ceil_div(Cout, 64);
     PM_REQUIRE(gy <= 65535 && gz <= 65535, "f2f_bwd_filter: grid too large");

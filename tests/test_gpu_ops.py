@@ -146,9 +146,15 @@ def test_f2v_unit_count_is_plain_scatter(cuda):
 # ------------------------------------------------------------------ facet2facet
 @pytest.mark.parametrize("nf,Cin,Cout,F,kmax", [(10, 3, 8, 16, 3), (100, 3, 32, 16, 5), (200, 64, 64, 16, 9),
                                                 (333, 16, 96, 16, 4), (70, 5, 7, 9, 3), (65, 4, 6, 36, 2),
-                                                (64, 3, 5, 50, 2), (129, 130, 64, 4, 3), (50, 8, 8, 1, 2)])
-def test_f2f_parity(cuda, nf, Cin, Cout, F, kmax):
-    say("case f2f", nf, Cin, Cout, F, kmax)
+                                                (64, 3, 5, 50, 2), (129, 130, 64, 4, 3), (50, 8, 8, 1, 2),
+                                                (300, 8, 40, 16, 14), (1000, 64, 64, 16, 9), (130, 4, 130, 16, 20)])
+@pytest.mark.parametrize("generic", [False, True])
+def test_f2f_parity(cuda, monkeypatch, nf, Cin, Cout, F, kmax, generic):
+    """``generic`` forces the shape-generic kernels also where the 16-coefficient fast path applies."""
+    say("case f2f", nf, Cin, Cout, F, kmax, generic)
+    if generic and not (F == 16 and Cin % 4 == 0):
+        pytest.skip("shape already runs the generic kernels")
+    monkeypatch.setenv("PMESH_F2F_GENERIC", "1" if generic else "0")
     rng = np.random.default_rng(13)
     counts, bary, owner = texture_case(rng, nf, kmax)
     T = int(counts.sum())

@@ -108,10 +108,22 @@ int pmesh_f2v_bwd(const float *grad_output, const float *input, const float *fil
  *   texture (T,Cin)  filter (Cout,Cin,F)  bary_coeff (T,F)  cum_texture (Nf, inclusive
  *   running total of texture points per facet, as layers.py:57 prepares it)
  *   -> output (Nf,Cout).   F <= 50 as in mesh_conv3d.cpp:211.
+ * workspace: pmesh_f2f_fwd_workspace_bytes(Cin,Cout,F) bytes, 16-byte aligned (holds the filter
+ * re-arranged for the matrix cores; may be 0 bytes for shapes that need none).
+ * facet_order: NULL, or the permutation pmesh_build_facet_order made from this cum_texture.  It
+ * only groups facets with equal numbers of texture points into the same workgroups (faster when
+ * the counts vary); results are identical with and without it.
  */
+size_t pmesh_facet_order_workspace_bytes(int64_t n_facets);
+int pmesh_build_facet_order(const int32_t *cum_texture, int64_t n_facets, int64_t n_points,
+                            int32_t *order, void *workspace, size_t workspace_bytes,
+                            pmesh_stream_t stream);
+
+size_t pmesh_f2f_fwd_workspace_bytes(int Cin, int Cout, int F);
 int pmesh_f2f_fwd(const float *texture, const float *filter, const float *bary_coeff,
-                  const int32_t *cum_texture, float *output, int64_t T, int64_t Nf, int Cin,
-                  int Cout, int F, pmesh_stream_t stream);
+                  const int32_t *cum_texture, const int32_t *facet_order, float *output, void *workspace,
+                  size_t workspace_bytes, int64_t T, int64_t Nf, int Cin, int Cout, int F,
+                  pmesh_stream_t stream);
 
 /* grad_texture (T,Cin), grad_filter (Cout,Cin,F).
  * workspace: pmesh_f2f_bwd_workspace_bytes(Cin,Cout,F).  Only rows of grad_texture that belong

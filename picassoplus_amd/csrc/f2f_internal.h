@@ -10,6 +10,11 @@ bool f2f16_usable(const void *tex, const void *W, const void *sh, int Cin, int F
 int f2f16_fwd(const float *tex, const float *W, const float *sh, const int *cum, float *out, int64_t T,
               int64_t Nf, int Cin, int Cout, hipStream_t st);
 
+// forward on the bf16 matrix cores with an exact three-way split of both operands (fp32-level accuracy)
+size_t f2f16x3_fwd_workspace_bytes(int Cin, int Cout);
+int f2f16x3_fwd(const float *tex, const float *W, const float *sh, const int *cum, const int *order, float *out,
+                void *workspace, size_t workspace_bytes, int64_t T, int64_t Nf, int Cin, int Cout, hipStream_t st);
+
 int f2f16_bwd_texture(const float *gout, const float *W, const float *sh, const int *cum, float *gtex, int64_t T,
                       int64_t Nf, int Cin, int Cout, hipStream_t st);
 

@@ -48,6 +48,20 @@ __global__ __launch_bounds__(kBlock) void rowptr_k(const unsigned *__restrict__ 
     for (int64_t r = lo; r <= hi && r <= n_rows; ++r) rowptr[r] = (int)i;
 }
 
+// key of facet f: its number of texture points, capped at 15
+__global__ __launch_bounds__(kBlock) void facet_keys_k(const int *__restrict__ cum, int64_t Nf, int T,
+                                                       unsigned *__restrict__ keys, int *__restrict__ vals)
+{
+    const int64_t f = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (f >= Nf) return;
+    int a = f ? cum[f - 1] : 0, b = cum[f];
+    a = a < 0 ? 0 : (a > T ? T : a);
+    b = b < 0 ? 0 : (b > T ? T : b);
+    const int K = b > a ? b - a : 0;
+    keys[f] = (unsigned)(K < 15 ? K : 15);
+    vals[f] = (int)f;
+}
+
 static int key_bits(int64_t n_rows)
 {
     int b = 1;
@@ -157,4 +171,34 @@ extern "C" int pmesh_build_cluster_csr(const int32_t *vt_replace, const int32_t 
         vt_replace, vt_map, n_fine, n_coarse, (unsigned *)base, (int *)(base + 2 * slot));
     PM_LAUNCHED("build_cluster_csr(keys)");
     return sort_and_rowptr("build_cluster_csr", n_fine, n_coarse, rowptr, members, workspace, workspace_bytes, st);
+}
+
+extern "C" size_t pmesh_facet_order_workspace_bytes(int64_t n_facets)
+{
+    return 3 * align_up((size_t)n_facets * 4) + align_up(sort_temp_bytes(n_facets, 4)) + 256;
+}
+
+extern "C" int pmesh_build_facet_order(const int32_t *cum_texture, int64_t n_facets, int64_t n_points, int32_t *order,
+                                       void *workspace, size_t workspace_bytes, pmesh_stream_t stream)
+{
+    clear_error();
+    PM_REQUIRE(n_facets >= 0 && n_facets < INT32_MAX && n_points >= 0 && n_points <= INT32_MAX,
+               "build_facet_order: bad sizes");
+    if (n_facets == 0) return 0;
+    PM_REQUIRE(cum_texture && order && workspace, "build_facet_order: null pointer");
+    hipStream_t st = (hipStream_t)stream;
+    char *base = (char *)workspace;
+    const size_t slot = align_up((size_t)n_facets * 4);
+    size_t temp_bytes = sort_temp_bytes(n_facets, 4);
+    PM_REQUIRE(3 * slot + temp_bytes <= workspace_bytes, "build_facet_order: workspace too small (%zu bytes)",
+               workspace_bytes);
+    unsigned *keys_in = (unsigned *)base, *keys_out = (unsigned *)(base + slot);
+    int *vals_in = (int *)(base + 2 * slot);
+    facet_keys_k<<<dim3((unsigned)ceil_div(n_facets, kBlock)), dim3(kBlock), 0, st>>>(cum_texture, n_facets,
+                                                                                       (int)n_points, keys_in, vals_in);
+    PM_LAUNCHED("build_facet_order(keys)");
+    hipError_t e = rocprim::radix_sort_pairs(base + 3 * slot, temp_bytes, keys_in, keys_out, vals_in, order,
+                                             (size_t)n_facets, 0, 4, st);
+    PM_REQUIRE(e == hipSuccess, "build_facet_order: radix sort failed: %s", hipGetErrorString(e));
+    return 0;
 }

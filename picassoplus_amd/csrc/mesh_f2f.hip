@@ -333,14 +333,30 @@ using namespace pmesh;
     PM_REQUIRE((int64_t)Cin * F <= (1 << 24) && Cout <= (1 << 20), name ": dims too large");     \
     PM_REQUIRE(T >= 0 && Nf >= 0 && T <= INT32_MAX && Nf <= INT32_MAX, name ": bad sizes")
 
+// PMESH_F2F_FP32MFMA=1 keeps the 16-coefficient fast path on the fp32 matrix instructions
+static inline bool force_fp32_mfma()
+{
+    const char *e = getenv("PMESH_F2F_FP32MFMA");
+    return e && e[0] == '1';
+}
+
+extern "C" size_t pmesh_f2f_fwd_workspace_bytes(int Cin, int Cout, int F)
+{
+    return (F == 16 && (Cin & 3) == 0) ? f2f16x3_fwd_workspace_bytes(Cin, Cout) : 0;
+}
+
 extern "C" int pmesh_f2f_fwd(const float *texture, const float *filter, const float *bary_coeff,
-                             const int32_t *cum_texture, float *output, int64_t T, int64_t Nf, int Cin,
-                             int Cout, int F, pmesh_stream_t stream)
+                             const int32_t *cum_texture, const int32_t *facet_order, float *output,
+                             void *workspace, size_t workspace_bytes, int64_t T, int64_t Nf, int Cin, int Cout,
+                             int F, pmesh_stream_t stream)
 {
     clear_error();
     PM_F2F_DIMS("f2f_fwd");
     if (Nf == 0) return 0;
     PM_REQUIRE(filter && cum_texture && output && (T == 0 || (texture && bary_coeff)), "f2f_fwd: null pointer");
+    if (!force_generic() && !force_fp32_mfma() && f2f16_usable(texture, filter, bary_coeff, Cin, F))
+        return f2f16x3_fwd(texture, filter, bary_coeff, cum_texture, facet_order, output, workspace, workspace_bytes,
+                           T, Nf, Cin, Cout, (hipStream_t)stream);
     if (!force_generic() && f2f16_usable(texture, filter, bary_coeff, Cin, F))
         return f2f16_fwd(texture, filter, bary_coeff, cum_texture, output, T, Nf, Cin, Cout, (hipStream_t)stream);
     const ChunkGeom cg = chunk_geom(Cin, F);

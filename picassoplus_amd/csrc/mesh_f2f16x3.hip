@@ -1,0 +1,338 @@
+// facet2facet forward for 16 SH coefficients on the bf16 matrix cores with fp32-level accuracy.
+//
+// v_mfma_f32_32x32x16_bf16 sustains ~14x the rate of v_mfma_f32_32x32x2_f32 on gfx950.  Both
+// operands of out = G . W^T are therefore split exactly into three bf16 pieces each,
+//     x = x1 + x2 + x3,  x1 = top 8 mantissa bits of x, x2 = top 8 bits of (x - x1), x3 = the rest
+// (truncation, so every piece is exactly representable and the sum is exact), and the product is
+// accumulated in fp32 from the six piece products of order <= 2^-16:
+//     G.W ~ G1W1 + G1W2 + G2W1 + G1W3 + G2W2 + G3W1          (dropped terms are < 2^-23 relative)
+// Six bf16 MFMAs replace eight fp32 MFMAs per 16 reduction steps at 1/14 of the cost each.
+//
+// Work decomposition (one wavefront per SIMD, 512 registers per lane):
+//   workgroup  256 facets (taken from a list sorted by number of texture points) x 64 output channels
+//   wavefront  64 facets x 64 output channels = four 32x32 accumulator tiles
+//   lane       (l32, h): facets slot l32 and 32+l32 of the wavefront, SH indices d = 8h..8h+7
+//   filter     pre-split and pre-arranged per lane by f2f16x3_pack_filter_k; the 24 KiB of four
+//              input channels are copied to LDS per step (double buffered, fetched a step ahead)
+//   G operand  formed in registers: for the next input channel, 8 values per facet from the
+//              facet's texture points (SH values held in registers), then split and packed,
+//              all placed in the issue shadow of the current channel's 24 MFMAs
+#include "f2f_internal.h"
+
+namespace pmesh {
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int kXKB = 4;                       // texture points per facet covered by one sweep (register budget)
+constexpr int kXChunk = 4 * 2 * 3 * 64;       // uint4 per LDS buffer: 4 channels x 2 tiles x 3 pieces x 64 lanes
+
+__device__ __forceinline__ float4 xld4(const float *p) { return *reinterpret_cast<const float4 *>(p); }
+__device__ __forceinline__ unsigned fbits(float x) { return __builtin_bit_cast(unsigned, x); }
+__device__ __forceinline__ float bitsf(unsigned u) { return __builtin_bit_cast(float, u); }
+// {hi16(b), hi16(a)}: two truncated bf16 values in one register, a in the low half
+__device__ __forceinline__ unsigned pack_hi(float a, float b)
+{
+    return __builtin_amdgcn_perm(fbits(b), fbits(a), 0x07060302u);
+}
+__device__ __forceinline__ float trunc_bf16(float x) { return bitsf(fbits(x) & 0xFFFF0000u); }
+
+// split eight fp32 values into three packed bf16x8 pieces
+__device__ __forceinline__ void split8(const float (&x)[8], u32x4 &p1, u32x4 &p2, u32x4 &p3)
+{
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const float a = x[2 * j], b = x[2 * j + 1];
+        p1[j] = pack_hi(a, b);
+        const float ra = a - trunc_bf16(a), rb = b - trunc_bf16(b);
+        p2[j] = pack_hi(ra, rb);
+        p3[j] = pack_hi(ra - trunc_bf16(ra), rb - trunc_bf16(rb));
+    }
+}
+
+__device__ __forceinline__ f32x16 mfma_bf16(const u32x4 &a, const u32x4 &b, const f32x16 &c)
+{
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c,
+                                                    0, 0, 0);
+}
+
+__device__ __forceinline__ int xwave_max(int v)
+{
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        const int t = __shfl_xor(v, o, 64);
+        v = t > v ? t : v;
+    }
+    return __builtin_amdgcn_readfirstlane(v);
+}
+
+// Filter (Cout, Cin, 16) -> per-lane MFMA B operands: Wp[((ci*NT + nt)*3 + piece)*64 + lane] holds the
+// eight bf16 pieces of W[nt*32 + l32][ci][8h .. 8h+7], lane = 32h + l32.  NT = even number of
+// 32-channel tiles covering Cout (zero padded).
+__global__ __launch_bounds__(kBlock) void f2f16x3_pack_filter_k(const float *__restrict__ W, u32x4 *__restrict__ Wp,
+                                                                int Cin, int Cout, int NT)
+{
+    const int idx = blockIdx.x * kBlock + threadIdx.x;
+    if (idx >= Cin * NT * 64) return;
+    const int lane = idx & 63, nt = (idx >> 6) % NT, ci = (idx >> 6) / NT;
+    const int co = nt * 32 + (lane & 31), h = lane >> 5;
+    float x[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) x[j] = 0.f;
+    if (co < Cout) {
+        const float *p = W + ((int64_t)co * Cin + ci) * 16 + 8 * h;
+        const float4 u = xld4(p), v = xld4(p + 4);
+        x[0] = u.x; x[1] = u.y; x[2] = u.z; x[3] = u.w; x[4] = v.x; x[5] = v.y; x[6] = v.z; x[7] = v.w;
+    }
+    u32x4 p1, p2, p3;
+    split8(x, p1, p2, p3);
+    u32x4 *dst = Wp + ((size_t)(ci * NT + nt) * 3) * 64 + lane;
+    dst[0] = p1; dst[64] = p2; dst[128] = p3;
+}
+
+__device__ __forceinline__ float2 xld2(const float *p) { return *reinterpret_cast<const float2 *>(p); }
+
+// eight G values per facet for one input channel: sum over the facet's texture points
+template <int KW>
+__device__ __forceinline__ void gen_next(float (&a)[2][8], const float2 (&t)[2][KW], int comp, const float (&shr)[2][KW][8])
+{
+#pragma unroll
+    for (int r = 0; r < 2; ++r)
+#pragma unroll
+        for (int s = 0; s < 8; ++s) {
+            float v = 0.f;
+#pragma unroll
+            for (int kk = 0; kk < KW; ++kk) v = fmaf(comp == 0 ? t[r][kk].x : t[r][kk].y, shr[r][kk][s], v);
+            a[r][s] = v;
+        }
+}
+
+__device__ __forceinline__ void w_chunk_fetch(const u32x4 *__restrict__ Wp, int c0, int NT, int nt0, u32x4 (&wn)[6])
+{
+    // channel c of the chunk: 2 tiles x 3 pieces x 64 lanes = 384 consecutive uint4
+#pragma unroll
+    for (int i = 0; i < 6; ++i) {
+        const int e = threadIdx.x + 256 * i, c = e / 384, o = e - c * 384;
+        wn[i] = Wp[((size_t)(c0 + c) * NT + nt0) * 192 + o];
+    }
+}
+
+// One pass over all input channels for up to KW texture points per facet (compile-time, so the
+// operand generation is a straight line of FMAs).  Texture values are fetched two channels at a
+// time, one pair ahead; the filter chunk of four channels one chunk ahead.
+template <int KW>
+__device__ __forceinline__ void x3_sweep(const float *__restrict__ tex, const u32x4 *__restrict__ Wp,
+                                         const float *__restrict__ sh, u32x4 *Ws, f32x16 (&acc)[2][2],
+                                         const int (&kbase)[2], const int (&Ks)[2], const float (&invK)[2], int Cin,
+                                         int NT, int nt0, int nblk, int lane, int h)
+{
+    // SH values of my two facets' points, my half's eight d's, pre-scaled by 1/K
+    float shr[2][KW][8];
+#pragma unroll
+    for (int r = 0; r < 2; ++r)
+#pragma unroll
+        for (int kk = 0; kk < KW; ++kk) {
+            float4 u = make_float4(0.f, 0.f, 0.f, 0.f), v = u;
+            if (kk < Ks[r]) {
+                const float *p = sh + (int64_t)(kbase[r] + kk) * 16 + 8 * h;
+                u = xld4(p);
+                v = xld4(p + 4);
+            }
+            const float s = invK[r];
+            shr[r][kk][0] = u.x * s; shr[r][kk][1] = u.y * s; shr[r][kk][2] = u.z * s; shr[r][kk][3] = u.w * s;
+            shr[r][kk][4] = v.x * s; shr[r][kk][5] = v.y * s; shr[r][kk][6] = v.z * s; shr[r][kk][7] = v.w * s;
+        }
+    unsigned trow[2][KW];                      // element offset of each texture row (T*Cin < 2^31 checked on the host)
+    float2 tc[2][KW], tn[2][KW];
+#pragma unroll
+    for (int r = 0; r < 2; ++r)
+#pragma unroll
+        for (int kk = 0; kk < KW; ++kk) {
+            trow[r][kk] = (unsigned)(kbase[r] + (kk < Ks[r] ? kk : 0)) * (unsigned)Cin;
+            tc[r][kk] = (kk < Ks[r]) ? xld2(tex + trow[r][kk]) : make_float2(0.f, 0.f);
+            tn[r][kk] = make_float2(0.f, 0.f);
+        }
+    u32x4 wn[6];
+    w_chunk_fetch(Wp, 0, NT, nt0, wn);
+#pragma unroll
+    for (int i = 0; i < 6; ++i) Ws[threadIdx.x + 256 * i] = wn[i];
+    __syncthreads();
+
+    float a[2][8];
+    gen_next<KW>(a, tc, 0, shr);
+    u32x4 pa[2][3];
+    split8(a[0], pa[0][0], pa[0][1], pa[0][2]);
+    split8(a[1], pa[1][0], pa[1][1], pa[1][2]);
+
+    for (int j = 0; j < nblk; ++j) {
+        const u32x4 *Wc = Ws + (j & 1) * kXChunk;
+        const bool more = j + 1 < nblk;
+#pragma unroll
+        for (int cp = 0; cp < 2; ++cp) {
+            if (cp == 0 && more) w_chunk_fetch(Wp, 4 * (j + 1), NT, nt0, wn);
+            if (cp == 0 || more) {
+                const int cnext = 4 * j + 2 * (cp + 1);
+#pragma unroll
+                for (int r = 0; r < 2; ++r)
+#pragma unroll
+                    for (int kk = 0; kk < KW; ++kk)
+                        tn[r][kk] = (kk < Ks[r]) ? xld2(tex + (trow[r][kk] + cnext)) : make_float2(0.f, 0.f);
+            }
+#pragma unroll
+            for (int c2 = 0; c2 < 2; ++c2) {
+                const int ci_l = 2 * cp + c2;
+                u32x4 b[2][3];
+#pragma unroll
+                for (int t = 0; t < 2; ++t)
+#pragma unroll
+                    for (int p = 0; p < 3; ++p) b[t][p] = Wc[((ci_l * 2 + t) * 3 + p) * 64 + lane];
+
+                // G values of the next channel, split into pieces while this channel's MFMAs run
+                float an[2][8];
+                if (c2 == 0) gen_next<KW>(an, tc, 1, shr);
+                else gen_next<KW>(an, tn, 0, shr);
+                u32x4 pn[2][3];
+                split8(an[0], pn[0][0], pn[0][1], pn[0][2]);
+                split8(an[1], pn[1][0], pn[1][1], pn[1][2]);
+
+                // six piece products per accumulator tile, smallest first
+#pragma unroll
+                for (int term = 0; term < 6; ++term) {
+                    const int ga = term == 0 ? 2 : term == 1 ? 1 : term == 2 ? 0 : term == 3 ? 1 : 0;
+                    const int wb = term == 0 ? 0 : term == 1 ? 1 : term == 2 ? 2 : term == 3 ? 0 : term == 4 ? 1 : 0;
+#pragma unroll
+                    for (int r = 0; r < 2; ++r)
+#pragma unroll
+                        for (int t = 0; t < 2; ++t) acc[r][t] = mfma_bf16(pa[r][ga], b[t][wb], acc[r][t]);
+                }
+#pragma unroll
+                for (int r = 0; r < 2; ++r)
+#pragma unroll
+                    for (int p = 0; p < 3; ++p) pa[r][p] = pn[r][p];
+            }
+#pragma unroll
+            for (int r = 0; r < 2; ++r)
+#pragma unroll
+                for (int kk = 0; kk < KW; ++kk) tc[r][kk] = tn[r][kk];
+        }
+        if (more) {
+#pragma unroll
+            for (int i = 0; i < 6; ++i) Ws[((j + 1) & 1) * kXChunk + threadIdx.x + 256 * i] = wn[i];
+        }
+        __syncthreads();
+    }
+}
+
+// `order` (may be null) lists the facets sorted by their number of texture points, so that the 256
+// facets of a workgroup -- and the 64 of a wavefront -- have (nearly) equal counts: the work per
+// sweep is set by the longest facet, and facets with more than kXKB points need further sweeps.
+__global__ __launch_bounds__(256, 1) void f2f16x3_fwd_k(const float *__restrict__ tex, const u32x4 *__restrict__ Wp,
+                                                        const float *__restrict__ sh, const int *__restrict__ cum,
+                                                        const int *__restrict__ order, float *__restrict__ out,
+                                                        int64_t Nf, int T, int Cin, int Cout, int NT)
+{
+    __shared__ u32x4 Ws[2 * kXChunk];
+    __shared__ int s_f[256], s_kmax;
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int l32 = lane & 31, h = lane >> 5;
+    const int64_t s0 = (int64_t)blockIdx.x * 256;
+    const int nt0 = blockIdx.y * 2, n0 = blockIdx.y * 64;
+    const int nblk = Cin >> 2;
+
+    if (threadIdx.x == 0) s_kmax = 0;
+    {
+        const int64_t slot = s0 + threadIdx.x;
+        s_f[threadIdx.x] = slot < Nf ? (order ? order[slot] : (int)slot) : -1;
+    }
+    __syncthreads();
+    int k0[2], K[2];
+    float invK[2];
+#pragma unroll
+    for (int r = 0; r < 2; ++r) {
+        const int f = s_f[w * 64 + r * 32 + l32];
+        k0[r] = 0;
+        K[r] = 0;
+        if (f >= 0 && f < Nf) {
+            int a = f ? cum[f - 1] : 0, b = cum[f];
+            a = a < 0 ? 0 : (a > T ? T : a);
+            b = b < 0 ? 0 : (b > T ? T : b);
+            k0[r] = a;
+            K[r] = b > a ? b - a : 0;
+        }
+        invK[r] = K[r] > 0 ? 1.0f / (float)K[r] : 0.f;
+    }
+    {
+        const int km = xwave_max(K[0] > K[1] ? K[0] : K[1]);
+        if (lane == 0) atomicMax(&s_kmax, km);
+    }
+    __syncthreads();
+    const int nsweeps = (s_kmax + kXKB - 1) / kXKB;
+
+    f32x16 acc[2][2];
+#pragma unroll
+    for (int r = 0; r < 2; ++r)
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) acc[r][t][i] = 0.f;
+
+    for (int sw = 0; sw < nsweeps; ++sw) {
+        int kbase[2], Ks[2];
+#pragma unroll
+        for (int r = 0; r < 2; ++r) {
+            kbase[r] = k0[r] + sw * kXKB;
+            const int rem = K[r] - sw * kXKB;
+            Ks[r] = rem < 0 ? 0 : (rem > kXKB ? kXKB : rem);
+        }
+        // every variant runs the same barriers, so wavefronts of a workgroup may pick different ones
+        const int kw = xwave_max(Ks[0] > Ks[1] ? Ks[0] : Ks[1]);
+#define PM_X3(N) x3_sweep<N>(tex, Wp, sh, Ws, acc, kbase, Ks, invK, Cin, NT, nt0, nblk, lane, h)
+        if (kw <= 1) PM_X3(1);
+        else if (kw == 2) PM_X3(2);
+        else if (kw == 3) PM_X3(3);
+        else PM_X3(4);
+#undef PM_X3
+    }
+
+#pragma unroll
+    for (int r = 0; r < 2; ++r)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int fr = s_f[w * 64 + r * 32 + 8 * (i / 4) + 4 * h + (i % 4)];
+            if (fr >= 0 && fr < Nf) {
+#pragma unroll
+                for (int t = 0; t < 2; ++t) {
+                    const int co = n0 + t * 32 + l32;
+                    if (co < Cout) out[(int64_t)fr * Cout + co] = acc[r][t][i];
+                }
+            }
+        }
+}
+
+size_t f2f16x3_fwd_workspace_bytes(int Cin, int Cout)
+{
+    const int NT = 2 * ((Cout + 63) / 64);
+    return (size_t)Cin * NT * 3 * 64 * sizeof(u32x4);
+}
+
+int f2f16x3_fwd(const float *tex, const float *W, const float *sh, const int *cum, const int *order, float *out,
+                void *workspace, size_t workspace_bytes, int64_t T, int64_t Nf, int Cin, int Cout, hipStream_t st)
+{
+    const int NT = 2 * ((Cout + 63) / 64);
+    PM_REQUIRE(T * Cin < (int64_t(1) << 31), "f2f_fwd: texture array too large for 32-bit offsets");
+    PM_REQUIRE(workspace && workspace_bytes >= f2f16x3_fwd_workspace_bytes(Cin, Cout),
+               "f2f_fwd: workspace too small (%zu bytes)", workspace_bytes);
+    PM_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 15u) == 0, "f2f_fwd: workspace must be 16-byte aligned");
+    u32x4 *Wp = (u32x4 *)workspace;
+    const int n = Cin * NT * 64;
+    f2f16x3_pack_filter_k<<<dim3((unsigned)ceil_div(n, kBlock)), dim3(kBlock), 0, st>>>(W, Wp, Cin, Cout, NT);
+    PM_LAUNCHED("f2f_fwd(pack)");
+    const int64_t gx = ceil_div(Nf, 256), gy = NT / 2;
+    PM_REQUIRE(grid_ok(gx) && gy <= 65535, "f2f_fwd: grid too large");
+    f2f16x3_fwd_k<<<dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, st>>>(tex, Wp, sh, cum, order, out, Nf, (int)T, Cin, Cout, NT);
+    PM_LAUNCHED("f2f_fwd");
+    return 0;
+}
+
+}  // namespace pmesh

@@ -132,8 +132,12 @@ def facet2facet_forward(input, filter, bary_coeff, num_texture):
     dev = same_device(input, filter, bary_coeff, num_texture)
     with torch.cuda.device(dev):
         out = torch.empty((Nf, Cout), dtype=F32, device=dev)
+        nbytes = _lib.query("pmesh_f2f_fwd_workspace_bytes", Cin, Cout, F)
+        ws = workspace(nbytes, dev)
+        order = topology.facet_order(num_texture, T) if Nf else None
         _lib.call("pmesh_f2f_fwd", input.data_ptr(), filter.data_ptr(), bary_coeff.data_ptr(),
-                  num_texture.data_ptr(), out.data_ptr(), T, Nf, Cin, Cout, F, stream_of(input))
+                  num_texture.data_ptr(), order.data_ptr() if order is not None else None, out.data_ptr(),
+                  ws.data_ptr(), nbytes, T, Nf, Cin, Cout, F, stream_of(input))
     return out
 
 

@@ -118,6 +118,24 @@ def cluster_csr(vt_replace, vt_map, n_coarse):
     return rowptr, members
 
 
+def facet_order(cum_texture, n_points):
+    """Permutation of the facets by their number of texture points (stable), from the running
+    total ``cum_texture``; lets the facet2facet kernels give every wavefront facets of equal length."""
+    key = _key("o", cum_texture, int(n_points))
+    hit = _lookup(key)
+    if hit is not None:
+        return hit[0]
+    nf = cum_texture.shape[0]
+    with torch.cuda.device(cum_texture.device):
+        order = torch.empty(nf, dtype=torch.int32, device=cum_texture.device)
+        ws_bytes = _lib.query("pmesh_facet_order_workspace_bytes", nf)
+        ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=cum_texture.device)
+        _lib.call("pmesh_build_facet_order", cum_texture.data_ptr(), nf, int(n_points), order.data_ptr(),
+                  ws.data_ptr(), ws_bytes, _stream(cum_texture))
+    _store(key, (order, cum_texture))
+    return order
+
+
 def _check_range_cached(face, n_vertices):
     """Validate a facet tensor against a vertex count once per tensor."""
     key = _key("rf", face, int(n_vertices))

@@ -40,6 +40,9 @@ def test_size_queries_are_host_only():
     assert _lib.query("pmesh_v2f_bwd_workspace_bytes", 64, 1) == 1024 * 3 * 64 * 4
     assert _lib.query("pmesh_f2v_bwd_workspace_bytes", 64, 1, 16) == 1024 * 16 * 64 * 4
     assert _lib.query("pmesh_f2f_bwd_workspace_bytes", 64, 64, 16) == 256 * 64 * 64 * 16 * 4
+    assert _lib.query("pmesh_f2f_fwd_workspace_bytes", 64, 64, 16) == 64 * 2 * 3 * 64 * 16
+    assert _lib.query("pmesh_f2f_fwd_workspace_bytes", 3, 64, 16) == 0
+    assert _lib.query("pmesh_facet_order_workspace_bytes", 1000) >= 3 * 1000 * 4
     assert _lib.query("pmesh_vertex_csr_workspace_bytes", 1000, 500) >= 3 * 3000 * 4
     assert _lib.query("pmesh_cluster_csr_workspace_bytes", 1000, 250) >= 3 * 1000 * 4
 
@@ -49,7 +52,7 @@ def test_argument_errors_without_launching():
     # bad dimensions are rejected before any device work, with a message
     assert lib.pmesh_v2f_fwd(None, None, None, None, 10, 10, 0, 1, None) != 0
     assert b"bad channel counts" in lib.pmesh_last_error()
-    assert lib.pmesh_f2f_fwd(None, None, None, None, None, 10, 10, 4, 4, 51, None) != 0
+    assert lib.pmesh_f2f_fwd(None, None, None, None, None, None, None, 0, 10, 10, 4, 4, 51, None) != 0
     assert b"maximum of 50" in lib.pmesh_last_error()
     assert lib.pmesh_sph_harm(None, None, 5, 6, None) != 0
     assert lib.pmesh_pool_max_bwd(None, None, None, None, None, -1, 2, 4, None) != 0

@@ -126,8 +126,8 @@ int pmesh_f2f_fwd(const float *texture, const float *filter, const float *bary_c
                   pmesh_stream_t stream);
 
 /* grad_texture (T,Cin), grad_filter (Cout,Cin,F).
- * workspace: pmesh_f2f_bwd_workspace_bytes(Cin,Cout,F).  Only rows of grad_texture that belong
- * to a facet are written; the caller clears it when texture rows may lie outside every facet.
+ * workspace: pmesh_f2f_bwd_workspace_bytes(Cin,Cout,F).  Every row of grad_texture is written
+ * (rows past the last facet's segment are cleared) provided cum_texture is non-decreasing.
  * pmesh_f2f_bwd is the texture half followed by the filter half; each half can be called
  * alone when only one gradient is wanted (the reference always computes both,
  * mesh_conv3d_gpu.cu:144-168). */

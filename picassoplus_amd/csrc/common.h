@@ -74,6 +74,9 @@ template <int V> __device__ __forceinline__ Pack<V> ldp(const float *p)
     if constexpr (V == 4) {
         const float4 t = *reinterpret_cast<const float4 *>(p);
         r.v[0] = t.x; r.v[1] = t.y; r.v[2] = t.z; r.v[3] = t.w;
+    } else if constexpr (V == 2) {
+        const float2 t = *reinterpret_cast<const float2 *>(p);
+        r.v[0] = t.x; r.v[1] = t.y;
     } else {
 #pragma unroll
         for (int i = 0; i < V; ++i) r.v[i] = p[i];
@@ -85,6 +88,8 @@ template <int V> __device__ __forceinline__ void stp(float *p, const Pack<V> &r)
 {
     if constexpr (V == 4) {
         *reinterpret_cast<float4 *>(p) = make_float4(r.v[0], r.v[1], r.v[2], r.v[3]);
+    } else if constexpr (V == 2) {
+        *reinterpret_cast<float2 *>(p) = make_float2(r.v[0], r.v[1]);
     } else {
 #pragma unroll
         for (int i = 0; i < V; ++i) p[i] = r.v[i];

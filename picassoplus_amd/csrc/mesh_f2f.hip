@@ -305,6 +305,17 @@ __global__ __launch_bounds__(kBlock) void f2f_fill_zero_k(float *__restrict__ p,
     if (i < n) p[i] = 0.f;
 }
 
+// rows of grad_texture past the last facet's segment belong to no facet: clear them
+__global__ __launch_bounds__(kBlock) void f2f_zero_tail_k(float *__restrict__ gtex, const int *__restrict__ cum,
+                                                          int64_t Nf, int T, int Cin)
+{
+    int last = cum[Nf - 1];
+    last = last < 0 ? 0 : (last > T ? T : last);
+    const int64_t n = (int64_t)(T - last) * Cin;
+    float *p = gtex + (int64_t)last * Cin;
+    for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (int64_t)gridDim.x * kBlock) p[i] = 0.f;
+}
+
 constexpr int kFiltMaxSplits = 256;
 
 static inline int filt_splits(int64_t Nf)
@@ -381,6 +392,8 @@ extern "C" int pmesh_f2f_bwd_texture(const float *grad_output, const float *filt
     PM_F2F_DIMS("f2f_bwd_texture");
     if (Nf == 0 || T == 0) return 0;
     PM_REQUIRE(grad_output && filter && bary_coeff && cum_texture && grad_texture, "f2f_bwd_texture: null pointer");
+    f2f_zero_tail_k<<<dim3(64), dim3(kBlock), 0, (hipStream_t)stream>>>(grad_texture, cum_texture, Nf, (int)T, Cin);
+    PM_LAUNCHED("f2f_bwd_texture(tail)");
     if (!force_generic() && f2f16_usable(grad_texture, filter, bary_coeff, Cin, F))
         return f2f16_bwd_texture(grad_output, filter, bary_coeff, cum_texture, grad_texture, T, Nf, Cin, Cout,
                                  (hipStream_t)stream);

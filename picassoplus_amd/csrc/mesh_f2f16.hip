@@ -381,29 +381,39 @@ __device__ __forceinline__ int seg_end(const int *__restrict__ cum, int64_t f, i
     return e > s ? e : s;
 }
 
-// next slab starting at facet fa; pa_cont >= 0 continues a facet that has more than kPS points
-__device__ __forceinline__ Slab make_slab(const int *__restrict__ cum, int64_t fa, int64_t fend, int T, int pa_cont)
+// next slab starting at facet fa; pa_cont >= 0 continues a facet that has more than kPS points.
+// Evaluated by every wavefront on its own (lanes 0..16 fetch the 17 segment bounds in one go, so
+// the descriptor costs one memory round trip instead of a chain of dependent loads).
+__device__ __forceinline__ Slab make_slab(const int *__restrict__ cum, int64_t fa, int64_t fend, int T, int pa_cont,
+                                          int lane)
 {
     Slab S;
     S.fa = (int)fa; S.n = 0; S.pa = 0; S.pb = 0; S.flush = 1;
     if (fa >= fend) return S;
-    const int s0 = seg_start(cum, fa, T), e0 = seg_end(cum, fa, T);
-    if (pa_cont >= 0 || e0 - s0 > kPS) {
+    const int64_t fi = fa + lane;                       // lane i: start row of facet fa + i
+    int c = T;
+    if (lane <= kFB && fi <= fend) c = seg_start(cum, fi, T);
+    const int s0 = __builtin_amdgcn_readfirstlane(c);
+    const int cn = __shfl_down(c, 1, 64);
+    const int e = cn > c ? cn : c;                      // end row of facet fa + lane
+    const int e0 = __builtin_amdgcn_readfirstlane(e);
+    const bool ok = lane < kFB && fi < fend && e - s0 <= kPS;
+    const unsigned long long mask = __ballot(ok);
+    const int n = __builtin_ctzll(~mask);               // leading facets that fit together
+    if (pa_cont >= 0 || n == 0) {
         S.n = 1;
         S.pa = pa_cont >= 0 ? pa_cont : s0;
         S.pb = (S.pa + kPS < e0) ? S.pa + kPS : e0;
         S.flush = S.pb >= e0;
         return S;
     }
-    S.pa = s0;
-    int pb = s0, n = 0;
-    while (n < kFB && fa + n < fend) {
-        const int e = seg_end(cum, fa + n, T);
-        if (e - s0 > kPS) break;
-        pb = e > pb ? e : pb;
-        ++n;
+    int pb = lane < n ? e : s0;
+#pragma unroll
+    for (int o = 16; o > 0; o >>= 1) {
+        const int t = __shfl_xor(pb, o, 64);
+        pb = t > pb ? t : pb;
     }
-    S.n = n; S.pb = pb;
+    S.n = n; S.pa = s0; S.pb = __builtin_amdgcn_readfirstlane(pb);
     return S;
 }
 
@@ -488,13 +498,13 @@ __global__ __launch_bounds__(512, 2) void f2f16_bwd_filt_k(const float *__restri
         }
     };
 
-    Slab cur = make_slab(cum, fbeg, fend, T, -1);
+    Slab cur = make_slab(cum, fbeg, fend, T, -1, lane);
     if (cur.n > 0) fetch(cur);
     publish();
     __syncthreads();
     while (cur.n > 0) {
-        const Slab nxt = cur.flush ? make_slab(cum, cur.fa + cur.n, fend, T, -1)
-                                   : make_slab(cum, cur.fa, fend, T, cur.pb);
+        const Slab nxt = cur.flush ? make_slab(cum, cur.fa + cur.n, fend, T, -1, lane)
+                                   : make_slab(cum, cur.fa, fend, T, cur.pb, lane);
         if (nxt.n > 0) fetch(nxt);
 
         // G values of my half's facets (slab facet 2*jj + h), channels 8w + 2t + sel, SH index d

@@ -91,21 +91,24 @@ __global__ __launch_bounds__(kBlock) void f2f16x3_pack_filter_k(const float *__r
     dst[0] = p1; dst[64] = p2; dst[128] = p3;
 }
 
-__device__ __forceinline__ float2 xld2(const float *p) { return *reinterpret_cast<const float2 *>(p); }
-
-// eight G values per facet for one input channel: sum over the facet's texture points
+// eight G values per facet for one input channel: sum over the facet's texture points, whose
+// values for this channel come from the wavefront's LDS slab [point][channel][facet slot]
 template <int KW>
-__device__ __forceinline__ void gen_next(float (&a)[2][8], const float2 (&t)[2][KW], int comp, const float (&shr)[2][KW][8])
+__device__ __forceinline__ void gen_next(float (&a)[2][8], const float *slab, int ch, int l32, const float (&shr)[2][KW][8])
 {
 #pragma unroll
-    for (int r = 0; r < 2; ++r)
+    for (int r = 0; r < 2; ++r) {
+        float tv[KW];
+#pragma unroll
+        for (int kk = 0; kk < KW; ++kk) tv[kk] = slab[(kk * 8 + ch) * 64 + r * 32 + l32];
 #pragma unroll
         for (int s = 0; s < 8; ++s) {
             float v = 0.f;
 #pragma unroll
-            for (int kk = 0; kk < KW; ++kk) v = fmaf(comp == 0 ? t[r][kk].x : t[r][kk].y, shr[r][kk][s], v);
+            for (int kk = 0; kk < KW; ++kk) v = fmaf(tv[kk], shr[r][kk][s], v);
             a[r][s] = v;
         }
+    }
 }
 
 __device__ __forceinline__ void w_chunk_fetch(const u32x4 *__restrict__ Wp, int c0, int NT, int nt0, u32x4 (&wn)[6])
@@ -118,15 +121,23 @@ __device__ __forceinline__ void w_chunk_fetch(const u32x4 *__restrict__ Wp, int 
     }
 }
 
+constexpr int kXSlab = kXKB * 8 * 64;      // floats per slab buffer: points x 8 channels x 64 facet slots
+
 // One pass over all input channels for up to KW texture points per facet (compile-time, so the
-// operand generation is a straight line of FMAs).  Texture values are fetched two channels at a
-// time, one pair ahead; the filter chunk of four channels one chunk ahead.
+// operand generation is a straight line of FMAs).
+//   texture values: the wavefront's 64 x KW texture rows are fetched 8 channels at a time with
+//     16-byte loads (two lanes per row), a group ahead, and parked in a wavefront-private LDS slab
+//     from which every lane picks its own facets' values;
+//   filter: chunk of four channels copied to LDS a chunk ahead (shared by the four wavefronts).
+// Both are published right before the workgroup barrier that ends a chunk.
 template <int KW>
 __device__ __forceinline__ void x3_sweep(const float *__restrict__ tex, const u32x4 *__restrict__ Wp,
-                                         const float *__restrict__ sh, u32x4 *Ws, f32x16 (&acc)[2][2],
-                                         const int (&kbase)[2], const int (&Ks)[2], const float (&invK)[2], int Cin,
-                                         int NT, int nt0, int nblk, int lane, int h)
+                                         const float *__restrict__ sh, u32x4 *Ws, float *slab, f32x16 (&acc)[2][2],
+                                         const int (&kbase)[2], const int (&Ks)[2], const float (&invK)[2],
+                                         const int *s_k0, const int *s_K, int sweep, int Cin, int NT, int nt0,
+                                         int nblk, int w, int lane, int h)
 {
+    const int l32 = lane & 31;
     // SH values of my two facets' points, my half's eight d's, pre-scaled by 1/K
     float shr[2][KW][8];
 #pragma unroll
@@ -143,16 +154,32 @@ __device__ __forceinline__ void x3_sweep(const float *__restrict__ tex, const u3
             shr[r][kk][0] = u.x * s; shr[r][kk][1] = u.y * s; shr[r][kk][2] = u.z * s; shr[r][kk][3] = u.w * s;
             shr[r][kk][4] = v.x * s; shr[r][kk][5] = v.y * s; shr[r][kk][6] = v.z * s; shr[r][kk][7] = v.w * s;
         }
-    unsigned trow[2][KW];                      // element offset of each texture row (T*Cin < 2^31 checked on the host)
-    float2 tc[2][KW], tn[2][KW];
+    // rows this lane fetches for the slab: load i covers point kk = i/2 of facet slot (lane/2) + 32*(i%2),
+    // channels 4*(lane%2) .. +3 of the group
+    const int cg4 = 4 * (lane & 1);
+    unsigned ldoff[2 * KW];
+    bool ldok[2 * KW];
 #pragma unroll
-    for (int r = 0; r < 2; ++r)
+    for (int i = 0; i < 2 * KW; ++i) {
+        const int slot = w * 64 + (lane >> 1) + 32 * (i & 1), kk = sweep * kXKB + (i >> 1);
+        ldok[i] = kk < s_K[slot];
+        ldoff[i] = (unsigned)(s_k0[slot] + (ldok[i] ? kk : 0)) * (unsigned)Cin + cg4;
+    }
+    float4 pf[2 * KW];
+    auto fetch_group = [&](int g) {
 #pragma unroll
-        for (int kk = 0; kk < KW; ++kk) {
-            trow[r][kk] = (unsigned)(kbase[r] + (kk < Ks[r] ? kk : 0)) * (unsigned)Cin;
-            tc[r][kk] = (kk < Ks[r]) ? xld2(tex + trow[r][kk]) : make_float2(0.f, 0.f);
-            tn[r][kk] = make_float2(0.f, 0.f);
+        for (int i = 0; i < 2 * KW; ++i)
+            pf[i] = (ldok[i] && 8 * g + cg4 < Cin) ? xld4(tex + (ldoff[i] + 8 * g)) : make_float4(0.f, 0.f, 0.f, 0.f);
+    };
+    auto publish_group = [&](float *dst) {
+#pragma unroll
+        for (int i = 0; i < 2 * KW; ++i) {
+            float *q = dst + ((i >> 1) * 8 + cg4) * 64 + (lane >> 1) + 32 * (i & 1);
+            q[0] = pf[i].x; q[64] = pf[i].y; q[128] = pf[i].z; q[192] = pf[i].w;
         }
+    };
+    fetch_group(0);
+    publish_group(slab);
     u32x4 wn[6];
     w_chunk_fetch(Wp, 0, NT, nt0, wn);
 #pragma unroll
@@ -160,7 +187,7 @@ __device__ __forceinline__ void x3_sweep(const float *__restrict__ tex, const u3
     __syncthreads();
 
     float a[2][8];
-    gen_next<KW>(a, tc, 0, shr);
+    gen_next<KW>(a, slab, 0, l32, shr);
     u32x4 pa[2][3];
     split8(a[0], pa[0][0], pa[0][1], pa[0][2]);
     split8(a[1], pa[1][0], pa[1][1], pa[1][2]);
@@ -168,58 +195,46 @@ __device__ __forceinline__ void x3_sweep(const float *__restrict__ tex, const u3
     for (int j = 0; j < nblk; ++j) {
         const u32x4 *Wc = Ws + (j & 1) * kXChunk;
         const bool more = j + 1 < nblk;
+        const int g = j >> 1;
+        const bool stage = !(j & 1) && 8 * (g + 1) < Cin;       // even chunk: bring in the next 8-channel group
+        if (more) w_chunk_fetch(Wp, 4 * (j + 1), NT, nt0, wn);
+        if (stage) fetch_group(g + 1);
 #pragma unroll
-        for (int cp = 0; cp < 2; ++cp) {
-            if (cp == 0 && more) w_chunk_fetch(Wp, 4 * (j + 1), NT, nt0, wn);
-            if (cp == 0 || more) {
-                const int cnext = 4 * j + 2 * (cp + 1);
+        for (int ci_l = 0; ci_l < 4; ++ci_l) {
+            u32x4 b[2][3];
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int p = 0; p < 3; ++p) b[t][p] = Wc[((ci_l * 2 + t) * 3 + p) * 64 + lane];
+
+            // G values of the next channel, split into pieces while this channel's MFMAs run
+            const int cn = 4 * j + ci_l + 1;
+            float an[2][8];
+            gen_next<KW>(an, slab + ((cn >> 3) & 1) * kXSlab, cn & 7, l32, shr);
+            u32x4 pn[2][3];
+            split8(an[0], pn[0][0], pn[0][1], pn[0][2]);
+            split8(an[1], pn[1][0], pn[1][1], pn[1][2]);
+
+            // six piece products per accumulator tile, smallest first
+#pragma unroll
+            for (int term = 0; term < 6; ++term) {
+                const int ga = term == 0 ? 2 : term == 1 ? 1 : term == 2 ? 0 : term == 3 ? 1 : 0;
+                const int wb = term == 0 ? 0 : term == 1 ? 1 : term == 2 ? 2 : term == 3 ? 0 : term == 4 ? 1 : 0;
 #pragma unroll
                 for (int r = 0; r < 2; ++r)
 #pragma unroll
-                    for (int kk = 0; kk < KW; ++kk)
-                        tn[r][kk] = (kk < Ks[r]) ? xld2(tex + (trow[r][kk] + cnext)) : make_float2(0.f, 0.f);
-            }
-#pragma unroll
-            for (int c2 = 0; c2 < 2; ++c2) {
-                const int ci_l = 2 * cp + c2;
-                u32x4 b[2][3];
-#pragma unroll
-                for (int t = 0; t < 2; ++t)
-#pragma unroll
-                    for (int p = 0; p < 3; ++p) b[t][p] = Wc[((ci_l * 2 + t) * 3 + p) * 64 + lane];
-
-                // G values of the next channel, split into pieces while this channel's MFMAs run
-                float an[2][8];
-                if (c2 == 0) gen_next<KW>(an, tc, 1, shr);
-                else gen_next<KW>(an, tn, 0, shr);
-                u32x4 pn[2][3];
-                split8(an[0], pn[0][0], pn[0][1], pn[0][2]);
-                split8(an[1], pn[1][0], pn[1][1], pn[1][2]);
-
-                // six piece products per accumulator tile, smallest first
-#pragma unroll
-                for (int term = 0; term < 6; ++term) {
-                    const int ga = term == 0 ? 2 : term == 1 ? 1 : term == 2 ? 0 : term == 3 ? 1 : 0;
-                    const int wb = term == 0 ? 0 : term == 1 ? 1 : term == 2 ? 2 : term == 3 ? 0 : term == 4 ? 1 : 0;
-#pragma unroll
-                    for (int r = 0; r < 2; ++r)
-#pragma unroll
-                        for (int t = 0; t < 2; ++t) acc[r][t] = mfma_bf16(pa[r][ga], b[t][wb], acc[r][t]);
-                }
-#pragma unroll
-                for (int r = 0; r < 2; ++r)
-#pragma unroll
-                    for (int p = 0; p < 3; ++p) pa[r][p] = pn[r][p];
+                    for (int t = 0; t < 2; ++t) acc[r][t] = mfma_bf16(pa[r][ga], b[t][wb], acc[r][t]);
             }
 #pragma unroll
             for (int r = 0; r < 2; ++r)
 #pragma unroll
-                for (int kk = 0; kk < KW; ++kk) tc[r][kk] = tn[r][kk];
+                for (int p = 0; p < 3; ++p) pa[r][p] = pn[r][p];
         }
         if (more) {
 #pragma unroll
             for (int i = 0; i < 6; ++i) Ws[((j + 1) & 1) * kXChunk + threadIdx.x + 256 * i] = wn[i];
         }
+        if (stage) publish_group(slab + ((g + 1) & 1) * kXSlab);
         __syncthreads();
     }
 }
@@ -233,7 +248,8 @@ __global__ __launch_bounds__(256, 1) void f2f16x3_fwd_k(const float *__restrict_
                                                         int64_t Nf, int T, int Cin, int Cout, int NT)
 {
     __shared__ u32x4 Ws[2 * kXChunk];
-    __shared__ int s_f[256], s_kmax;
+    __shared__ __attribute__((aligned(16))) float s_slab[4 * 2 * kXSlab];      // per wavefront: two buffers
+    __shared__ int s_f[256], s_k0[256], s_K[256], s_kmax;
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
     const int l32 = lane & 31, h = lane >> 5;
     const int64_t s0 = (int64_t)blockIdx.x * 256;
@@ -245,21 +261,25 @@ __global__ __launch_bounds__(256, 1) void f2f16x3_fwd_k(const float *__restrict_
         const int64_t slot = s0 + threadIdx.x;
         s_f[threadIdx.x] = slot < Nf ? (order ? order[slot] : (int)slot) : -1;
     }
+    {
+        const int f = s_f[threadIdx.x];
+        int a = 0, b = 0;
+        if (f >= 0 && f < Nf) {
+            a = f ? cum[f - 1] : 0;
+            b = cum[f];
+            a = a < 0 ? 0 : (a > T ? T : a);
+            b = b < 0 ? 0 : (b > T ? T : b);
+        }
+        s_k0[threadIdx.x] = a;
+        s_K[threadIdx.x] = b > a ? b - a : 0;
+    }
     __syncthreads();
     int k0[2], K[2];
     float invK[2];
 #pragma unroll
     for (int r = 0; r < 2; ++r) {
-        const int f = s_f[w * 64 + r * 32 + l32];
-        k0[r] = 0;
-        K[r] = 0;
-        if (f >= 0 && f < Nf) {
-            int a = f ? cum[f - 1] : 0, b = cum[f];
-            a = a < 0 ? 0 : (a > T ? T : a);
-            b = b < 0 ? 0 : (b > T ? T : b);
-            k0[r] = a;
-            K[r] = b > a ? b - a : 0;
-        }
+        k0[r] = s_k0[w * 64 + r * 32 + l32];
+        K[r] = s_K[w * 64 + r * 32 + l32];
         invK[r] = K[r] > 0 ? 1.0f / (float)K[r] : 0.f;
     }
     {
@@ -287,7 +307,7 @@ __global__ __launch_bounds__(256, 1) void f2f16x3_fwd_k(const float *__restrict_
         }
         // every variant runs the same barriers, so wavefronts of a workgroup may pick different ones
         const int kw = xwave_max(Ks[0] > Ks[1] ? Ks[0] : Ks[1]);
-#define PM_X3(N) x3_sweep<N>(tex, Wp, sh, Ws, acc, kbase, Ks, invK, Cin, NT, nt0, nblk, lane, h)
+#define PM_X3(N) x3_sweep<N>(tex, Wp, sh, Ws, s_slab + w * 2 * kXSlab, acc, kbase, Ks, invK, s_k0, s_K, sw, Cin, NT, nt0, nblk, w, lane, h)
         if (kw <= 1) PM_X3(1);
         else if (kw == 2) PM_X3(2);
         else if (kw == 3) PM_X3(3);

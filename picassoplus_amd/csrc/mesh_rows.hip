@@ -10,6 +10,7 @@
 // workspace, then a fixed-order reduction over workgroups.
 #include "common.h"
 #include "../../include/picasso_mesh.h"
+#include <cstdlib>
 
 namespace pmesh {
 
@@ -221,6 +222,76 @@ __global__ __launch_bounds__(kBlock) void f2v_fwd_k(const float *__restrict__ in
     }
 }
 
+// Lane (l & 15) of every 16-lane row holds one of 16 filter coefficients of an entry; FMAs read
+// them through DPP row broadcasts, so an entry in flight costs one register instead of sixteen.
+template <int Kk> __device__ __forceinline__ float row_bcast(float v)
+{
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x150 + Kk, 0xF, 0xF, false));
+}
+
+__device__ __forceinline__ void fma_bcast16(float cf, const Pack<4> (&fl)[16], Pack<4> &w)
+{
+#define PM_B(Kk)                                                                   \
+    {                                                                              \
+        const float b = row_bcast<Kk>(cf);                                         \
+        w.v[0] = fmaf(b, fl[Kk].v[0], w.v[0]); w.v[1] = fmaf(b, fl[Kk].v[1], w.v[1]); \
+        w.v[2] = fmaf(b, fl[Kk].v[2], w.v[2]); w.v[3] = fmaf(b, fl[Kk].v[3], w.v[3]); \
+    }
+    PM_B(0) PM_B(1) PM_B(2) PM_B(3) PM_B(4) PM_B(5) PM_B(6) PM_B(7)
+    PM_B(8) PM_B(9) PM_B(10) PM_B(11) PM_B(12) PM_B(13) PM_B(14) PM_B(15)
+#undef PM_B
+}
+
+// facet2vertex forward for r = 1, C % 64 == 0 (row groups are whole 16-lane DPP rows): the entries
+// of an output vertex are processed eight at a time, all their gathers issued before any use.
+__global__ __launch_bounds__(kBlock) void f2v_fwd_fast_k(const float *__restrict__ in, const float *__restrict__ filt,
+                                                         const float *__restrict__ coeff,
+                                                         const int *__restrict__ nfcount,
+                                                         const int *__restrict__ rowptr,
+                                                         const int *__restrict__ colidx, float *__restrict__ out,
+                                                         int64_t NvOut, int C, int K, int lpr_log2)
+{
+    constexpr int EB = 8;
+    const int lpr = 1 << lpr_log2;
+    const int lane = threadIdx.x & (lpr - 1), slot = threadIdx.x >> lpr_log2, l16 = threadIdx.x & 15;
+    const int64_t row = (int64_t)blockIdx.x * (kBlock >> lpr_log2) + slot;
+    if (row >= NvOut) return;
+    const int e0 = rowptr[row], e1 = rowptr[row + 1];
+    const float inv = (e1 > e0) ? 1.0f / (float)nfcount[row] : 0.f;
+    const int c = lane * 4;
+    Pack<4> acc = zero_pack<4>();
+    for (int k0 = 0; k0 < K; k0 += 16) {
+        Pack<4> fl[16];
+#pragma unroll
+        for (int k = 0; k < 16; ++k) fl[k] = (k0 + k < K) ? ldp<4>(filt + (size_t)(k0 + k) * C + c) : zero_pack<4>();
+        const bool kok = k0 + l16 < K;
+        for (int eb = e0; eb < e1; eb += EB) {
+            int64_t f[EB];
+#pragma unroll
+            for (int i = 0; i < EB; ++i) f[i] = (eb + i < e1) ? colidx[eb + i] / 3 : -1;
+            Pack<4> x[EB];
+            float cf[EB];
+#pragma unroll
+            for (int i = 0; i < EB; ++i) {
+                x[i] = (f[i] >= 0) ? ldp<4>(in + f[i] * C + c) : zero_pack<4>();
+                cf[i] = (f[i] >= 0 && kok) ? coeff[f[i] * K + k0 + l16] : 0.f;
+            }
+#pragma unroll
+            for (int i = 0; i < EB; ++i) {
+                if (eb + i < e1) {
+                    Pack<4> w = zero_pack<4>();
+                    fma_bcast16(cf[i], fl, w);
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) acc.v[u] = fmaf(w.v[u], x[i].v[u], acc.v[u]);
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) acc.v[u] *= inv;
+    stp<4>(out + row * C + c, acc);
+}
+
 // ----------------------------------------------------------------------------------------
 // facet2vertex backward, one pass over the facets:
 //   s[f,co]      = sum_{corner j, vo_j >= 0} gout[vo_j,co] / nf[vo_j]
@@ -306,6 +377,96 @@ __global__ __launch_bounds__(kBlock) void f2v_bwd_k(const float *__restrict__ go
                                               lane, slot, lpr, rpb);
             }
         }
+}
+
+// facet2vertex backward for r = 1, C % 64 == 0, K <= 16: same arithmetic as f2v_bwd_k with the
+// coefficient row spread over the 16 lanes of a DPP row, and the index chain
+// face -> vt_map -> (nf_count, gout rows) of the NEXT facet resolved while the current one is computed.
+__global__ __launch_bounds__(kBlock) void f2v_bwd_fast_k(const float *__restrict__ gout, const float *__restrict__ in,
+                                                         const float *__restrict__ filt,
+                                                         const float *__restrict__ coeff,
+                                                         const int *__restrict__ face,
+                                                         const int *__restrict__ nfcount,
+                                                         const int *__restrict__ vtmap, float *__restrict__ gin,
+                                                         float *__restrict__ partial, int64_t Nf, int64_t NvOut, int C,
+                                                         int K, int lpr_log2, int64_t rows_per_block)
+{
+    __shared__ float red[kBlock * 4];
+    const int lpr = 1 << lpr_log2, rpb = kBlock >> lpr_log2;
+    const int lane = threadIdx.x & (lpr - 1), slot = threadIdx.x >> lpr_log2, l16 = threadIdx.x & 15;
+    const int64_t fbeg = (int64_t)blockIdx.x * rows_per_block;
+    const int64_t fend = (fbeg + rows_per_block < Nf) ? fbeg + rows_per_block : Nf;
+    const int c = lane * 4;
+    Pack<4> fl[16], acc[16];
+#pragma unroll
+    for (int k = 0; k < 16; ++k) {
+        fl[k] = (k < K) ? ldp<4>(filt + (size_t)k * C + c) : zero_pack<4>();
+        acc[k] = zero_pack<4>();
+    }
+    // software pipeline over this slot's facets: indices two facets ahead, output rows one ahead
+    int64_t f = fbeg + slot;
+    int va[3] = {0, 0, 0}, vo[3] = {-1, -1, -1};
+    if (f < fend) {
+#pragma unroll
+        for (int j = 0; j < 3; ++j) va[j] = face[3 * f + j];
+#pragma unroll
+        for (int j = 0; j < 3; ++j) vo[j] = vtmap[va[j]];
+    }
+    if (f + rpb < fend) {
+#pragma unroll
+        for (int j = 0; j < 3; ++j) va[j] = face[3 * (f + rpb) + j];
+    }
+    for (; f < fend; f += rpb) {
+        // data of facet f (its output rows are known), indices of the following two
+        int von[3] = {-1, -1, -1};
+        if (f + rpb < fend) {
+#pragma unroll
+            for (int j = 0; j < 3; ++j) von[j] = vtmap[va[j]];
+        }
+        if (f + 2 * rpb < fend) {
+#pragma unroll
+            for (int j = 0; j < 3; ++j) va[j] = face[3 * (f + 2 * rpb) + j];
+        }
+        Pack<4> g[3];
+        float nf[3];
+#pragma unroll
+        for (int j = 0; j < 3; ++j) {
+            const bool ok = vo[j] >= 0 && vo[j] < NvOut;
+            g[j] = ok ? ldp<4>(gout + (int64_t)vo[j] * C + c) : zero_pack<4>();
+            nf[j] = ok ? (float)nfcount[vo[j]] : 1.f;
+        }
+        const Pack<4> x = ldp<4>(in + f * C + c);
+        const float cf = (l16 < K) ? coeff[f * K + l16] : 0.f;
+        Pack<4> s = zero_pack<4>(), w = zero_pack<4>(), t;
+#pragma unroll
+        for (int j = 0; j < 3; ++j) {
+            const float inv = 1.0f / nf[j];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) s.v[u] = fmaf(g[j].v[u], inv, s.v[u]);
+        }
+        fma_bcast16(cf, fl, w);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) t.v[u] = x.v[u] * s.v[u];
+#define PM_A(Kk)                                                                     \
+    {                                                                                \
+        const float b = row_bcast<Kk>(cf);                                           \
+        acc[Kk].v[0] = fmaf(b, t.v[0], acc[Kk].v[0]); acc[Kk].v[1] = fmaf(b, t.v[1], acc[Kk].v[1]); \
+        acc[Kk].v[2] = fmaf(b, t.v[2], acc[Kk].v[2]); acc[Kk].v[3] = fmaf(b, t.v[3], acc[Kk].v[3]); \
+    }
+        PM_A(0) PM_A(1) PM_A(2) PM_A(3) PM_A(4) PM_A(5) PM_A(6) PM_A(7)
+        PM_A(8) PM_A(9) PM_A(10) PM_A(11) PM_A(12) PM_A(13) PM_A(14) PM_A(15)
+#undef PM_A
+        Pack<4> gi;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) gi.v[u] = s.v[u] * w.v[u];
+        stp<4>(gin + f * C + c, gi);
+#pragma unroll
+        for (int j = 0; j < 3; ++j) vo[j] = von[j];
+    }
+#pragma unroll
+    for (int k = 0; k < 16; ++k)
+        if (k < K)
+            block_reduce_store<4>(acc[k], red, partial + ((size_t)blockIdx.x * K + k) * C + c, true, lane, slot, lpr, rpb);
 }
 
 // ----------------------------------------------------------------------------------------
@@ -620,7 +781,9 @@ extern "C" int pmesh_f2v_fwd(const float *input, const float *filter, const floa
     const int64_t blocks = ceil_div(NvOut, rs.rpb);
     PM_REQUIRE(grid_ok(blocks), "f2v_fwd: grid too large");
     const int cvec = ((K & 3) == 0 && aligned16(coeff)) ? 1 : 0;
-    if (V == 4)
+    if (V == 4 && (C & 63) == 0 && C <= 1024)
+        f2v_fwd_fast_k<<<dim3((unsigned)blocks), dim3(kBlock), 0, st>>>(input, filter, coeff, nf_count, rowptr, colidx, output, NvOut, C, K, rs.lpr_log2);
+    else if (V == 4)
         f2v_fwd_k<4><<<dim3((unsigned)blocks), dim3(kBlock), 0, st>>>(input, filter, coeff, nf_count, rowptr, colidx, output, NvOut, C, r, K, rs.items, rs.lpr_log2, cvec);
     else
         f2v_fwd_k<1><<<dim3((unsigned)blocks), dim3(kBlock), 0, st>>>(input, filter, coeff, nf_count, rowptr, colidx, output, NvOut, C, r, K, rs.items, rs.lpr_log2, cvec);
@@ -658,7 +821,9 @@ extern "C" int pmesh_f2v_bwd(const float *grad_output, const float *input, const
     PM_REQUIRE(workspace_bytes >= (size_t)G * K * Co * sizeof(float), "f2v_bwd: workspace too small (%zu bytes)", workspace_bytes);
     const int cvec = ((K & 3) == 0 && aligned16(coeff)) ? 1 : 0;
     float *partial = (float *)workspace;
-    if (V == 4)
+    if (V == 4 && (C & 63) == 0 && C <= 1024 && K <= 16)
+        f2v_bwd_fast_k<<<dim3(G), dim3(kBlock), 0, st>>>(grad_output, input, filter, coeff, face, nf_count, vt_map, grad_input, partial, Nf, NvOut, C, K, rs.lpr_log2, rows_per_block);
+    else if (V == 4)
         f2v_bwd_k<4><<<dim3(G), dim3(kBlock), 0, st>>>(grad_output, input, filter, coeff, face, nf_count, vt_map, grad_input, partial, Nf, NvOut, C, r, K, rs.items, rs.lpr_log2, cvec, rows_per_block);
     else
         f2v_bwd_k<1><<<dim3(G), dim3(kBlock), 0, st>>>(grad_output, input, filter, coeff, face, nf_count, vt_map, grad_input, partial, Nf, NvOut, C, r, K, rs.items, rs.lpr_log2, cvec, rows_per_block);

@@ -149,8 +149,7 @@ def facet2facet_backward(grad_output, input, filter, bary_coeff, num_texture):
         raise RuntimeError("grad_output must have shape (NfIn, Cout)")
     dev = same_device(grad_output, input, filter, bary_coeff, num_texture)
     with torch.cuda.device(dev):
-        # rows past the last facet's segment receive no gradient
-        gin = torch.zeros((T, Cin), dtype=F32, device=dev)
+        gin = torch.empty((T, Cin), dtype=F32, device=dev)
         gfilt = torch.empty((Cout, Cin, F), dtype=F32, device=dev)
         nbytes = _lib.query("pmesh_f2f_bwd_workspace_bytes", Cin, Cout, F)
         ws = workspace(nbytes, dev)

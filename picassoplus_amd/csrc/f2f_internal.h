@@ -15,6 +15,9 @@ size_t f2f16x3_fwd_workspace_bytes(int Cin, int Cout);
 int f2f16x3_fwd(const float *tex, const float *W, const float *sh, const int *cum, const int *order, float *out,
                 void *workspace, size_t workspace_bytes, int64_t T, int64_t Nf, int Cin, int Cout, hipStream_t st);
 
+int f2f16x3_bwd_filter_partials(const float *gout, const float *tex, const float *sh, const int *cum, float *partial,
+                                int splits, int64_t T, int64_t Nf, int Cin, int Cout, hipStream_t st);
+
 int f2f16_bwd_texture(const float *gout, const float *W, const float *sh, const int *cum, float *gtex, int64_t T,
                       int64_t Nf, int Cin, int Cout, hipStream_t st);
 

@@ -428,8 +428,11 @@ extern "C" int pmesh_f2f_bwd_filter(const float *grad_output, const float *textu
     PM_REQUIRE(workspace_bytes >= (size_t)S * nW * sizeof(float), "f2f_bwd_filter: workspace too small (%zu bytes)",
                workspace_bytes);
     if (!force_generic() && f2f16_usable(texture, texture, bary_coeff, Cin, F)) {
-        int rc = f2f16_bwd_filter_partials(grad_output, texture, bary_coeff, cum_texture, (float *)workspace, S, T, Nf,
-                                           Cin, Cout, st);
+        int rc = force_fp32_mfma()
+                     ? f2f16_bwd_filter_partials(grad_output, texture, bary_coeff, cum_texture, (float *)workspace, S, T,
+                                                 Nf, Cin, Cout, st)
+                     : f2f16x3_bwd_filter_partials(grad_output, texture, bary_coeff, cum_texture, (float *)workspace, S,
+                                                   T, Nf, Cin, Cout, st);
         if (rc) return rc;
         f2f_reduce_k<<<dim3((unsigned)ceil_div(nW, 64)), dim3(kBlock), 0, st>>>((const float *)workspace, grad_filter, S, nW);
         PM_LAUNCHED("f2f_bwd_filter(reduce)");

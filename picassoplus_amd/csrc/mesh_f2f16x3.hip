@@ -8,15 +8,15 @@
 //     G.W ~ G1W1 + G1W2 + G2W1 + G1W3 + G2W2 + G3W1          (dropped terms are < 2^-23 relative)
 // Six bf16 MFMAs replace eight fp32 MFMAs per 16 reduction steps at 1/14 of the cost each.
 //
-// Work decomposition (one wavefront per SIMD, 512 registers per lane):
+// Work decomposition of the forward (two wavefronts per SIMD, 256 registers per lane):
 //   workgroup  256 facets (taken from a list sorted by number of texture points) x 64 output channels
-//   wavefront  64 facets x 64 output channels = four 32x32 accumulator tiles
-//   lane       (l32, h): facets slot l32 and 32+l32 of the wavefront, SH indices d = 8h..8h+7
+//   wavefront  32 facets x 64 output channels = two 32x32 accumulator tiles
+//   lane       (l32, h): facet slot l32 of the wavefront, SH indices d = 8h..8h+7
 //   filter     pre-split and pre-arranged per lane by f2f16x3_pack_filter_k; the 24 KiB of four
-//              input channels are copied to LDS per step (double buffered, fetched a step ahead)
+//              input channels are copied to LDS two chunks ahead (three buffers)
 //   G operand  formed in registers: for the next input channel, 8 values per facet from the
 //              facet's texture points (SH values held in registers), then split and packed,
-//              all placed in the issue shadow of the current channel's 24 MFMAs
+//              interleaved with the current channel's 12 MFMAs
 #include "f2f_internal.h"
 
 namespace pmesh {
@@ -38,7 +38,8 @@ __device__ __forceinline__ unsigned pack_hi(float a, float b)
 }
 __device__ __forceinline__ float trunc_bf16(float x) { return bitsf(fbits(x) & 0xFFFF0000u); }
 
-// split eight fp32 values into three packed bf16x8 pieces
+// split eight fp32 values into three packed bf16x8 pieces (truncation; measured no slower than the
+// v_cvt_pk_bf16_f32 / v_dot2c_f32_bf16 route, which needs 28 instead of 44 instructions but slower ones)
 __device__ __forceinline__ void split8(const float (&x)[8], u32x4 &p1, u32x4 &p2, u32x4 &p3)
 {
 #pragma unroll
@@ -91,57 +92,45 @@ __global__ __launch_bounds__(kBlock) void f2f16x3_pack_filter_k(const float *__r
     dst[0] = p1; dst[64] = p2; dst[128] = p3;
 }
 
-// eight G values per facet for one input channel: sum over the facet's texture points, whose
-// values for this channel come from the wavefront's LDS slab [point][channel][facet slot]
-template <int KW>
-__device__ __forceinline__ void gen_next(float (&a)[2][8], const float *slab, int ch, int l32, const float (&shr)[2][KW][8])
-{
-#pragma unroll
-    for (int r = 0; r < 2; ++r) {
-        float tv[KW];
-#pragma unroll
-        for (int kk = 0; kk < KW; ++kk) tv[kk] = slab[(kk * 8 + ch) * 64 + r * 32 + l32];
-#pragma unroll
-        for (int s = 0; s < 8; ++s) {
-            float v = 0.f;
-#pragma unroll
-            for (int kk = 0; kk < KW; ++kk) v = fmaf(tv[kk], shr[r][kk][s], v);
-            a[r][s] = v;
-        }
-    }
-}
+// Forward work decomposition: a workgroup of kFW wavefronts owns 256 facets x 64 output channels,
+// each wavefront kFR 32-facet row tiles.  With one row tile per wavefront two wavefronts fit a SIMD
+// (256 registers each), so the FMAs / conversions of one overlap the MFMAs of the other.
+constexpr int kFR = 1;                          // row tiles (facets per lane) of a wavefront
+constexpr int kFW = 8 / kFR;                    // wavefronts per workgroup
+constexpr int kFThreads = 64 * kFW;
+constexpr int kFWn = 1536 / kFThreads;          // uint4 of a filter chunk fetched per thread
+constexpr int kXSlab = kXKB * 8 * 32 * kFR;     // floats per slab buffer: points x 8 channels x facet slots
 
-__device__ __forceinline__ void w_chunk_fetch(const u32x4 *__restrict__ Wp, int c0, int NT, int nt0, u32x4 (&wn)[6])
+__device__ __forceinline__ void w_chunk_fetch(const u32x4 *__restrict__ Wp, int c0, int NT, int nt0, u32x4 (&wn)[kFWn])
 {
     // channel c of the chunk: 2 tiles x 3 pieces x 64 lanes = 384 consecutive uint4
 #pragma unroll
-    for (int i = 0; i < 6; ++i) {
-        const int e = threadIdx.x + 256 * i, c = e / 384, o = e - c * 384;
+    for (int i = 0; i < kFWn; ++i) {
+        const int e = threadIdx.x + kFThreads * i, c = e / 384, o = e - c * 384;
         wn[i] = Wp[((size_t)(c0 + c) * NT + nt0) * 192 + o];
     }
 }
 
-constexpr int kXSlab = kXKB * 8 * 64;      // floats per slab buffer: points x 8 channels x 64 facet slots
-
 // One pass over all input channels for up to KW texture points per facet (compile-time, so the
 // operand generation is a straight line of FMAs).
-//   texture values: the wavefront's 64 x KW texture rows are fetched 8 channels at a time with
+//   texture values: the wavefront's 32*kFR x KW texture rows are fetched 8 channels at a time with
 //     16-byte loads (two lanes per row), a group ahead, and parked in a wavefront-private LDS slab
 //     from which every lane picks its own facets' values;
-//   filter: chunk of four channels copied to LDS a chunk ahead (shared by the four wavefronts).
+//   filter: chunks of four channels copied to LDS two chunks ahead (shared by the workgroup).
 // Both are published right before the workgroup barrier that ends a chunk.
 template <int KW>
 __device__ __forceinline__ void x3_sweep(const float *__restrict__ tex, const u32x4 *__restrict__ Wp,
-                                         const float *__restrict__ sh, u32x4 *Ws, float *slab, f32x16 (&acc)[2][2],
-                                         const int (&kbase)[2], const int (&Ks)[2], const float (&invK)[2],
+                                         const float *__restrict__ sh, u32x4 *Ws, float *slab, f32x16 (&acc)[kFR][2],
+                                         const int (&kbase)[kFR], const int (&Ks)[kFR], const float (&invK)[kFR],
                                          const int *s_k0, const int *s_K, int sweep, int Cin, int NT, int nt0,
                                          int nblk, int w, int lane, int h)
 {
+    constexpr int NL = kFR * KW;                 // slab loads per lane and group
     const int l32 = lane & 31;
-    // SH values of my two facets' points, my half's eight d's, pre-scaled by 1/K
-    float shr[2][KW][8];
+    // SH values of my facets' points, my half's eight d's, pre-scaled by 1/K
+    float shr[kFR][KW][8];
 #pragma unroll
-    for (int r = 0; r < 2; ++r)
+    for (int r = 0; r < kFR; ++r)
 #pragma unroll
         for (int kk = 0; kk < KW; ++kk) {
             float4 u = make_float4(0.f, 0.f, 0.f, 0.f), v = u;
@@ -154,66 +143,105 @@ __device__ __forceinline__ void x3_sweep(const float *__restrict__ tex, const u3
             shr[r][kk][0] = u.x * s; shr[r][kk][1] = u.y * s; shr[r][kk][2] = u.z * s; shr[r][kk][3] = u.w * s;
             shr[r][kk][4] = v.x * s; shr[r][kk][5] = v.y * s; shr[r][kk][6] = v.z * s; shr[r][kk][7] = v.w * s;
         }
-    // rows this lane fetches for the slab: load i covers point kk = i/2 of facet slot (lane/2) + 32*(i%2),
-    // channels 4*(lane%2) .. +3 of the group
+    // rows this lane fetches for the slab: load i covers point kk = i / kFR of facet slot
+    // (lane/2) + 32*(i % kFR), channels 4*(lane%2) .. +3 of the group
     const int cg4 = 4 * (lane & 1);
-    unsigned ldoff[2 * KW];
-    bool ldok[2 * KW];
+    unsigned ldoff[NL];
+    bool ldok[NL];
 #pragma unroll
-    for (int i = 0; i < 2 * KW; ++i) {
-        const int slot = w * 64 + (lane >> 1) + 32 * (i & 1), kk = sweep * kXKB + (i >> 1);
+    for (int i = 0; i < NL; ++i) {
+        const int slot = w * 32 * kFR + (lane >> 1) + 32 * (i % kFR), kk = sweep * kXKB + i / kFR;
         ldok[i] = kk < s_K[slot];
         ldoff[i] = (unsigned)(s_k0[slot] + (ldok[i] ? kk : 0)) * (unsigned)Cin + cg4;
     }
-    float4 pf[2 * KW];
+    float4 pf[NL];
     auto fetch_group = [&](int g) {
 #pragma unroll
-        for (int i = 0; i < 2 * KW; ++i)
+        for (int i = 0; i < NL; ++i)
             pf[i] = (ldok[i] && 8 * g + cg4 < Cin) ? xld4(tex + (ldoff[i] + 8 * g)) : make_float4(0.f, 0.f, 0.f, 0.f);
     };
     auto publish_group = [&](float *dst) {
 #pragma unroll
-        for (int i = 0; i < 2 * KW; ++i) {
-            float *q = dst + ((i >> 1) * 8 + cg4) * 64 + (lane >> 1) + 32 * (i & 1);
-            q[0] = pf[i].x; q[64] = pf[i].y; q[128] = pf[i].z; q[192] = pf[i].w;
+        for (int i = 0; i < NL; ++i) {
+            float *q = dst + ((i / kFR) * 8 + cg4) * (32 * kFR) + (lane >> 1) + 32 * (i % kFR);
+            q[0] = pf[i].x; q[32 * kFR] = pf[i].y; q[64 * kFR] = pf[i].z; q[96 * kFR] = pf[i].w;
         }
     };
+    // filter chunks sit in three LDS buffers and are published two chunks ahead, so that the chunk
+    // after the current one is always complete and operand reads may run ahead across chunk ends
+    u32x4 wn[kFWn];
     fetch_group(0);
     publish_group(slab);
-    u32x4 wn[6];
     w_chunk_fetch(Wp, 0, NT, nt0, wn);
 #pragma unroll
-    for (int i = 0; i < 6; ++i) Ws[threadIdx.x + 256 * i] = wn[i];
+    for (int i = 0; i < kFWn; ++i) Ws[threadIdx.x + kFThreads * i] = wn[i];
+    if (nblk > 1) {
+        w_chunk_fetch(Wp, 4, NT, nt0, wn);
+#pragma unroll
+        for (int i = 0; i < kFWn; ++i) Ws[kXChunk + threadIdx.x + kFThreads * i] = wn[i];
+    }
     __syncthreads();
 
-    float a[2][8];
-    gen_next<KW>(a, slab, 0, l32, shr);
-    u32x4 pa[2][3];
-    split8(a[0], pa[0][0], pa[0][1], pa[0][2]);
-    split8(a[1], pa[1][0], pa[1][1], pa[1][2]);
+    auto read_b = [&](u32x4 (&b)[2][3], int c) {          // filter pieces of channel c (c < Cin)
+        const u32x4 *Wc = Ws + ((c >> 2) % 3) * kXChunk + (c & 3) * 384 + lane;
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int p = 0; p < 3; ++p) b[t][p] = Wc[(t * 3 + p) * 64];
+    };
+    auto read_tv = [&](float (&tv)[kFR][KW], int c) {     // my facets' texture values of channel c
+        const float *sl = slab + ((c >> 3) & 1) * kXSlab + (c & 7) * (32 * kFR) + l32;
+#pragma unroll
+        for (int r = 0; r < kFR; ++r)
+#pragma unroll
+            for (int kk = 0; kk < KW; ++kk) tv[r][kk] = sl[kk * 8 * (32 * kFR) + r * 32];
+    };
+    auto gen = [&](float (&a)[kFR][8], const float (&tv)[kFR][KW]) {
+#pragma unroll
+        for (int r = 0; r < kFR; ++r)
+#pragma unroll
+            for (int s = 0; s < 8; ++s) {
+                float v = 0.f;
+#pragma unroll
+                for (int kk = 0; kk < KW; ++kk) v = fmaf(tv[r][kk], shr[r][kk][s], v);
+                a[r][s] = v;
+            }
+    };
+
+    // software pipeline over channels: while channel c is multiplied, the G values of c+1 are
+    // generated and split, and the LDS reads for c+1 (filter) and c+2 (texture) are in flight
+    u32x4 pa[kFR][3], b[2][3];
+    float tvn[kFR][KW];
+    {
+        float tv0[kFR][KW], a[kFR][8];
+        read_tv(tv0, 0);
+        read_tv(tvn, 1);
+        read_b(b, 0);
+        gen(a, tv0);
+#pragma unroll
+        for (int r = 0; r < kFR; ++r) split8(a[r], pa[r][0], pa[r][1], pa[r][2]);
+    }
 
     for (int j = 0; j < nblk; ++j) {
-        const u32x4 *Wc = Ws + (j & 1) * kXChunk;
-        const bool more = j + 1 < nblk;
         const int g = j >> 1;
+        const bool wmore = j + 2 < nblk;
         const bool stage = !(j & 1) && 8 * (g + 1) < Cin;       // even chunk: bring in the next 8-channel group
-        if (more) w_chunk_fetch(Wp, 4 * (j + 1), NT, nt0, wn);
+        if (wmore) w_chunk_fetch(Wp, 4 * (j + 2), NT, nt0, wn);
         if (stage) fetch_group(g + 1);
 #pragma unroll
         for (int ci_l = 0; ci_l < 4; ++ci_l) {
-            u32x4 b[2][3];
-#pragma unroll
-            for (int t = 0; t < 2; ++t)
-#pragma unroll
-                for (int p = 0; p < 3; ++p) b[t][p] = Wc[((ci_l * 2 + t) * 3 + p) * 64 + lane];
+            const int c = 4 * j + ci_l;
+            u32x4 bn[2][3];
+            float tvnn[kFR][KW];
+            // c+1 == Cin reads a chunk buffer / slab row that exists but is not used
+            read_b(bn, c + 1 < Cin ? c + 1 : c);
+            read_tv(tvnn, c + 2);
 
-            // G values of the next channel, split into pieces while this channel's MFMAs run
-            const int cn = 4 * j + ci_l + 1;
-            float an[2][8];
-            gen_next<KW>(an, slab + ((cn >> 3) & 1) * kXSlab, cn & 7, l32, shr);
-            u32x4 pn[2][3];
-            split8(an[0], pn[0][0], pn[0][1], pn[0][2]);
-            split8(an[1], pn[1][0], pn[1][1], pn[1][2]);
+            float an[kFR][8];
+            gen(an, tvn);
+            u32x4 pn[kFR][3];
+#pragma unroll
+            for (int r = 0; r < kFR; ++r) split8(an[r], pn[r][0], pn[r][1], pn[r][2]);
 
             // six piece products per accumulator tile, smallest first
 #pragma unroll
@@ -221,18 +249,25 @@ __device__ __forceinline__ void x3_sweep(const float *__restrict__ tex, const u3
                 const int ga = term == 0 ? 2 : term == 1 ? 1 : term == 2 ? 0 : term == 3 ? 1 : 0;
                 const int wb = term == 0 ? 0 : term == 1 ? 1 : term == 2 ? 2 : term == 3 ? 0 : term == 4 ? 1 : 0;
 #pragma unroll
-                for (int r = 0; r < 2; ++r)
+                for (int r = 0; r < kFR; ++r)
 #pragma unroll
                     for (int t = 0; t < 2; ++t) acc[r][t] = mfma_bf16(pa[r][ga], b[t][wb], acc[r][t]);
             }
 #pragma unroll
-            for (int r = 0; r < 2; ++r)
+            for (int r = 0; r < kFR; ++r) {
 #pragma unroll
                 for (int p = 0; p < 3; ++p) pa[r][p] = pn[r][p];
-        }
-        if (more) {
 #pragma unroll
-            for (int i = 0; i < 6; ++i) Ws[((j + 1) & 1) * kXChunk + threadIdx.x + 256 * i] = wn[i];
+                for (int kk = 0; kk < KW; ++kk) tvn[r][kk] = tvnn[r][kk];
+            }
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int p = 0; p < 3; ++p) b[t][p] = bn[t][p];
+        }
+        if (wmore) {
+#pragma unroll
+            for (int i = 0; i < kFWn; ++i) Ws[((j + 2) % 3) * kXChunk + threadIdx.x + kFThreads * i] = wn[i];
         }
         if (stage) publish_group(slab + ((g + 1) & 1) * kXSlab);
         __syncthreads();
@@ -240,15 +275,18 @@ __device__ __forceinline__ void x3_sweep(const float *__restrict__ tex, const u3
 }
 
 // `order` (may be null) lists the facets sorted by their number of texture points, so that the 256
-// facets of a workgroup -- and the 64 of a wavefront -- have (nearly) equal counts: the work per
+// facets of a workgroup -- and the 32*kFR of a wavefront -- have (nearly) equal counts: the work per
 // sweep is set by the longest facet, and facets with more than kXKB points need further sweeps.
-__global__ __launch_bounds__(256, 1) void f2f16x3_fwd_k(const float *__restrict__ tex, const u32x4 *__restrict__ Wp,
-                                                        const float *__restrict__ sh, const int *__restrict__ cum,
-                                                        const int *__restrict__ order, float *__restrict__ out,
-                                                        int64_t Nf, int T, int Cin, int Cout, int NT)
+__global__ __launch_bounds__(kFThreads, 2 / kFR) void f2f16x3_fwd_k(const float *__restrict__ tex,
+                                                                   const u32x4 *__restrict__ Wp,
+                                                                   const float *__restrict__ sh,
+                                                                   const int *__restrict__ cum,
+                                                                   const int *__restrict__ order,
+                                                                   float *__restrict__ out, int64_t Nf, int T, int Cin,
+                                                                   int Cout, int NT)
 {
-    __shared__ u32x4 Ws[2 * kXChunk];
-    __shared__ __attribute__((aligned(16))) float s_slab[4 * 2 * kXSlab];      // per wavefront: two buffers
+    __shared__ u32x4 Ws[3 * kXChunk];
+    __shared__ __attribute__((aligned(16))) float s_slab[kFW * 2 * kXSlab];      // per wavefront: two buffers
     __shared__ int s_f[256], s_k0[256], s_K[256], s_kmax;
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
     const int l32 = lane & 31, h = lane >> 5;
@@ -257,12 +295,9 @@ __global__ __launch_bounds__(256, 1) void f2f16x3_fwd_k(const float *__restrict_
     const int nblk = Cin >> 2;
 
     if (threadIdx.x == 0) s_kmax = 0;
-    {
-        const int64_t slot = s0 + threadIdx.x;
-        s_f[threadIdx.x] = slot < Nf ? (order ? order[slot] : (int)slot) : -1;
-    }
-    {
-        const int f = s_f[threadIdx.x];
+    for (int i = threadIdx.x; i < 256; i += kFThreads) {
+        const int64_t slot = s0 + i;
+        const int f = slot < Nf ? (order ? order[slot] : (int)slot) : -1;
         int a = 0, b = 0;
         if (f >= 0 && f < Nf) {
             a = f ? cum[f - 1] : 0;
@@ -270,43 +305,46 @@ __global__ __launch_bounds__(256, 1) void f2f16x3_fwd_k(const float *__restrict_
             a = a < 0 ? 0 : (a > T ? T : a);
             b = b < 0 ? 0 : (b > T ? T : b);
         }
-        s_k0[threadIdx.x] = a;
-        s_K[threadIdx.x] = b > a ? b - a : 0;
+        s_f[i] = f;
+        s_k0[i] = a;
+        s_K[i] = b > a ? b - a : 0;
     }
     __syncthreads();
-    int k0[2], K[2];
-    float invK[2];
+    int k0[kFR], K[kFR], kmax = 0;
+    float invK[kFR];
 #pragma unroll
-    for (int r = 0; r < 2; ++r) {
-        k0[r] = s_k0[w * 64 + r * 32 + l32];
-        K[r] = s_K[w * 64 + r * 32 + l32];
+    for (int r = 0; r < kFR; ++r) {
+        k0[r] = s_k0[w * 32 * kFR + r * 32 + l32];
+        K[r] = s_K[w * 32 * kFR + r * 32 + l32];
         invK[r] = K[r] > 0 ? 1.0f / (float)K[r] : 0.f;
+        kmax = K[r] > kmax ? K[r] : kmax;
     }
     {
-        const int km = xwave_max(K[0] > K[1] ? K[0] : K[1]);
+        const int km = xwave_max(kmax);
         if (lane == 0) atomicMax(&s_kmax, km);
     }
     __syncthreads();
     const int nsweeps = (s_kmax + kXKB - 1) / kXKB;
 
-    f32x16 acc[2][2];
+    f32x16 acc[kFR][2];
 #pragma unroll
-    for (int r = 0; r < 2; ++r)
+    for (int r = 0; r < kFR; ++r)
 #pragma unroll
         for (int t = 0; t < 2; ++t)
 #pragma unroll
             for (int i = 0; i < 16; ++i) acc[r][t][i] = 0.f;
 
     for (int sw = 0; sw < nsweeps; ++sw) {
-        int kbase[2], Ks[2];
+        int kbase[kFR], Ks[kFR], kw = 0;
 #pragma unroll
-        for (int r = 0; r < 2; ++r) {
+        for (int r = 0; r < kFR; ++r) {
             kbase[r] = k0[r] + sw * kXKB;
             const int rem = K[r] - sw * kXKB;
             Ks[r] = rem < 0 ? 0 : (rem > kXKB ? kXKB : rem);
+            kw = Ks[r] > kw ? Ks[r] : kw;
         }
         // every variant runs the same barriers, so wavefronts of a workgroup may pick different ones
-        const int kw = xwave_max(Ks[0] > Ks[1] ? Ks[0] : Ks[1]);
+        kw = xwave_max(kw);
 #define PM_X3(N) x3_sweep<N>(tex, Wp, sh, Ws, s_slab + w * 2 * kXSlab, acc, kbase, Ks, invK, s_k0, s_K, sw, Cin, NT, nt0, nblk, w, lane, h)
         if (kw <= 1) PM_X3(1);
         else if (kw == 2) PM_X3(2);
@@ -316,10 +354,10 @@ __global__ __launch_bounds__(256, 1) void f2f16x3_fwd_k(const float *__restrict_
     }
 
 #pragma unroll
-    for (int r = 0; r < 2; ++r)
+    for (int r = 0; r < kFR; ++r)
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
-            const int fr = s_f[w * 64 + r * 32 + 8 * (i / 4) + 4 * h + (i % 4)];
+            const int fr = s_f[w * 32 * kFR + r * 32 + 8 * (i / 4) + 4 * h + (i % 4)];
             if (fr >= 0 && fr < Nf) {
 #pragma unroll
                 for (int t = 0; t < 2; ++t) {
@@ -606,7 +644,7 @@ int f2f16x3_fwd(const float *tex, const float *W, const float *sh, const int *cu
     PM_LAUNCHED("f2f_fwd(pack)");
     const int64_t gx = ceil_div(Nf, 256), gy = NT / 2;
     PM_REQUIRE(grid_ok(gx) && gy <= 65535, "f2f_fwd: grid too large");
-    f2f16x3_fwd_k<<<dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, st>>>(tex, Wp, sh, cum, order, out, Nf, (int)T, Cin, Cout, NT);
+    f2f16x3_fwd_k<<<dim3((unsigned)gx, (unsigned)gy), dim3(kFThreads), 0, st>>>(tex, Wp, sh, cum, order, out, Nf, (int)T, Cin, Cout, NT);
     PM_LAUNCHED("f2f_fwd");
     return 0;
 }

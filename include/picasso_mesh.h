@@ -126,23 +126,26 @@ int pmesh_f2f_fwd(const float *texture, const float *filter, const float *bary_c
                   pmesh_stream_t stream);
 
 /* grad_texture (T,Cin), grad_filter (Cout,Cin,F).
- * workspace: pmesh_f2f_bwd_workspace_bytes(Cin,Cout,F).  Every row of grad_texture is written
+ * workspace: pmesh_f2f_bwd_workspace_bytes(Cin,Cout,F), 16-byte aligned; the two halves may share
+ * it when they run on the same stream.  facet_order: NULL or the permutation of
+ * pmesh_build_facet_order, as for the forward.  Every row of grad_texture is written
  * (rows past the last facet's segment are cleared) provided cum_texture is non-decreasing.
  * pmesh_f2f_bwd is the texture half followed by the filter half; each half can be called
  * alone when only one gradient is wanted (the reference always computes both,
  * mesh_conv3d_gpu.cu:144-168). */
 size_t pmesh_f2f_bwd_workspace_bytes(int Cin, int Cout, int F);
 int pmesh_f2f_bwd(const float *grad_output, const float *texture, const float *filter,
-                  const float *bary_coeff, const int32_t *cum_texture, float *grad_texture,
-                  float *grad_filter, void *workspace, size_t workspace_bytes, int64_t T,
-                  int64_t Nf, int Cin, int Cout, int F, pmesh_stream_t stream);
+                  const float *bary_coeff, const int32_t *cum_texture, const int32_t *facet_order,
+                  float *grad_texture, float *grad_filter, void *workspace, size_t workspace_bytes,
+                  int64_t T, int64_t Nf, int Cin, int Cout, int F, pmesh_stream_t stream);
 int pmesh_f2f_bwd_texture(const float *grad_output, const float *filter, const float *bary_coeff,
-                          const int32_t *cum_texture, float *grad_texture, int64_t T, int64_t Nf,
-                          int Cin, int Cout, int F, pmesh_stream_t stream);
+                          const int32_t *cum_texture, const int32_t *facet_order, float *grad_texture,
+                          void *workspace, size_t workspace_bytes, int64_t T, int64_t Nf, int Cin,
+                          int Cout, int F, pmesh_stream_t stream);
 int pmesh_f2f_bwd_filter(const float *grad_output, const float *texture, const float *bary_coeff,
-                         const int32_t *cum_texture, float *grad_filter, void *workspace,
-                         size_t workspace_bytes, int64_t T, int64_t Nf, int Cin, int Cout, int F,
-                         pmesh_stream_t stream);
+                         const int32_t *cum_texture, const int32_t *facet_order, float *grad_filter,
+                         void *workspace, size_t workspace_bytes, int64_t T, int64_t Nf, int Cin,
+                         int Cout, int F, pmesh_stream_t stream);
 
 /* ------------------------------------------------------------------ mesh pooling
  * replaces max_forward / max_backward / avg_forward / avg_backward

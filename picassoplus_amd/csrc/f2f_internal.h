@@ -15,6 +15,13 @@ size_t f2f16x3_fwd_workspace_bytes(int Cin, int Cout);
 int f2f16x3_fwd(const float *tex, const float *W, const float *sh, const int *cum, const int *order, float *out,
                 void *workspace, size_t workspace_bytes, int64_t T, int64_t Nf, int Cin, int Cout, hipStream_t st);
 
+// texture gradient on the bf16 matrix cores (Cout <= 64, Cout % 8 == 0, 16-byte aligned grad_output)
+bool f2f16x3_bwd_texture_usable(const void *gout, int Cout);
+size_t f2f16x3_bwd_texture_workspace_bytes(int Cin, int Cout);
+int f2f16x3_bwd_texture(const float *gout, const float *W, const float *sh, const int *cum, const int *order,
+                        float *gtex, void *workspace, size_t workspace_bytes, int64_t T, int64_t Nf, int Cin,
+                        int Cout, hipStream_t st);
+
 int f2f16x3_bwd_filter_partials(const float *gout, const float *tex, const float *sh, const int *cum, float *partial,
                                 int splits, int64_t T, int64_t Nf, int Cin, int Cout, hipStream_t st);
 

@@ -381,12 +381,16 @@ extern "C" int pmesh_f2f_fwd(const float *texture, const float *filter, const fl
 
 extern "C" size_t pmesh_f2f_bwd_workspace_bytes(int Cin, int Cout, int F)
 {
-    return (size_t)kFiltMaxSplits * Cout * Cin * F * sizeof(float);
+    // the two halves run one after the other on a stream and share the workspace
+    const size_t filt = (size_t)kFiltMaxSplits * Cout * Cin * F * sizeof(float);
+    const size_t tex = F == 16 ? f2f16x3_bwd_texture_workspace_bytes(Cin, Cout) : 0;
+    return filt > tex ? filt : tex;
 }
 
 extern "C" int pmesh_f2f_bwd_texture(const float *grad_output, const float *filter, const float *bary_coeff,
-                                     const int32_t *cum_texture, float *grad_texture, int64_t T, int64_t Nf,
-                                     int Cin, int Cout, int F, pmesh_stream_t stream)
+                                     const int32_t *cum_texture, const int32_t *facet_order, float *grad_texture,
+                                     void *workspace, size_t workspace_bytes, int64_t T, int64_t Nf, int Cin,
+                                     int Cout, int F, pmesh_stream_t stream)
 {
     clear_error();
     PM_F2F_DIMS("f2f_bwd_texture");
@@ -394,9 +398,13 @@ extern "C" int pmesh_f2f_bwd_texture(const float *grad_output, const float *filt
     PM_REQUIRE(grad_output && filter && bary_coeff && cum_texture && grad_texture, "f2f_bwd_texture: null pointer");
     f2f_zero_tail_k<<<dim3(64), dim3(kBlock), 0, (hipStream_t)stream>>>(grad_texture, cum_texture, Nf, (int)T, Cin);
     PM_LAUNCHED("f2f_bwd_texture(tail)");
-    if (!force_generic() && f2f16_usable(grad_texture, filter, bary_coeff, Cin, F))
+    if (!force_generic() && f2f16_usable(grad_texture, filter, bary_coeff, Cin, F)) {
+        if (!force_fp32_mfma() && f2f16x3_bwd_texture_usable(grad_output, Cout))
+            return f2f16x3_bwd_texture(grad_output, filter, bary_coeff, cum_texture, facet_order, grad_texture,
+                                       workspace, workspace_bytes, T, Nf, Cin, Cout, (hipStream_t)stream);
         return f2f16_bwd_texture(grad_output, filter, bary_coeff, cum_texture, grad_texture, T, Nf, Cin, Cout,
                                  (hipStream_t)stream);
+    }
     const ChunkGeom cg = chunk_geom(Cin, F);
     const int64_t gx = ceil_div(Nf, 64);
     PM_REQUIRE(grid_ok(gx), "f2f_bwd_texture: grid too large");
@@ -408,7 +416,7 @@ extern "C" int pmesh_f2f_bwd_texture(const float *grad_output, const float *filt
 }
 
 extern "C" int pmesh_f2f_bwd_filter(const float *grad_output, const float *texture, const float *bary_coeff,
-                                    const int32_t *cum_texture, float *grad_filter, void *workspace,
+                                    const int32_t *cum_texture, const int32_t *facet_order, float *grad_filter, void *workspace,
                                     size_t workspace_bytes, int64_t T, int64_t Nf, int Cin, int Cout, int F,
                                     pmesh_stream_t stream)
 {
@@ -451,13 +459,13 @@ extern "C" int pmesh_f2f_bwd_filter(const float *grad_output, const float *textu
 }
 
 extern "C" int pmesh_f2f_bwd(const float *grad_output, const float *texture, const float *filter,
-                             const float *bary_coeff, const int32_t *cum_texture, float *grad_texture,
-                             float *grad_filter, void *workspace, size_t workspace_bytes, int64_t T,
-                             int64_t Nf, int Cin, int Cout, int F, pmesh_stream_t stream)
+                             const float *bary_coeff, const int32_t *cum_texture, const int32_t *facet_order,
+                             float *grad_texture, float *grad_filter, void *workspace, size_t workspace_bytes,
+                             int64_t T, int64_t Nf, int Cin, int Cout, int F, pmesh_stream_t stream)
 {
-    int rc = pmesh_f2f_bwd_texture(grad_output, filter, bary_coeff, cum_texture, grad_texture, T, Nf, Cin, Cout, F,
-                                   stream);
+    int rc = pmesh_f2f_bwd_texture(grad_output, filter, bary_coeff, cum_texture, facet_order, grad_texture, workspace,
+                                   workspace_bytes, T, Nf, Cin, Cout, F, stream);
     if (rc) return rc;
-    return pmesh_f2f_bwd_filter(grad_output, texture, bary_coeff, cum_texture, grad_filter, workspace,
+    return pmesh_f2f_bwd_filter(grad_output, texture, bary_coeff, cum_texture, facet_order, grad_filter, workspace,
                                 workspace_bytes, T, Nf, Cin, Cout, F, stream);
 }

@@ -369,6 +369,203 @@ __global__ __launch_bounds__(kFThreads, 2 / kFR) void f2f16x3_fwd_k(const float 
 }
 
 // ----------------------------------------------------------------------------------------
+// texture gradient on the bf16 matrix cores:
+//     H[f, ci, d] = sum_co gout[f, co] W[co, ci, d]          (split-bf16 MFMAs, k = co)
+//     gtex[t, ci] = (1/K_f) sum_d sh[t, d] H[f, ci, d]       (FMAs on the accumulator registers)
+// The product is taken transposed, D[(ci,d)][f] = W^T . gout^T, with the 32 rows of a tile ordered so
+// that a lane (facet l32, half h) finds in its 16 accumulator registers exactly the 16 d's of ONE
+// input channel: tile tt = 4g + q holds channels 8g + q (rows of half 0) and 8g + 4 + q (rows of
+// half 1), accumulator register i <-> d = i.  The contraction with the SH values of the facet's
+// points then needs no cross-lane traffic, and after the four tiles of a group a lane owns four
+// consecutive channels of each of its points: one 16-byte store per point.
+//   workgroup  256 facets from the sorted list, 8 wavefronts x 32 facets, two wavefronts per SIMD
+//   gout       a lane's facet row, split once into bf16 pieces (B operand, registers)
+//   filter     pre-split / pre-arranged W^T tiles (f2f16x3_pack_filter_t_k), two tiles per LDS chunk,
+//              three chunk buffers published two chunks ahead
+//   points     sweeps of up to four texture points per facet (their SH rows in registers)
+constexpr int kTKS = 4;                          // k-steps of 16 output channels (Cout <= 64)
+constexpr int kTChunkMax = 2 * kTKS * 3 * 64;    // uint4 per chunk buffer: 2 tiles x k-steps x 3 pieces x 64 lanes
+
+// W (Cout, Cin, 16) -> A operands of the transposed product:
+// WpT[((tt*NKS + ks)*3 + piece)*64 + lane] = pieces of W[16ks + 8h .. +7][ci(tt, r)][d(r)], r = lane % 32
+__global__ __launch_bounds__(kBlock) void f2f16x3_pack_filter_t_k(const float *__restrict__ W, u32x4 *__restrict__ WpT,
+                                                                  int Cin, int Cout, int NTt, int NKS)
+{
+    const int idx = blockIdx.x * kBlock + threadIdx.x;
+    if (idx >= NTt * NKS * 64) return;
+    const int lane = idx & 63, ks = (idx >> 6) % NKS, tt = (idx >> 6) / NKS;
+    const int r = lane & 31, h = lane >> 5;
+    const int ci = 8 * (tt >> 2) + 4 * ((r >> 2) & 1) + (tt & 3), d = 4 * (r >> 3) + (r & 3);
+    float x[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const int co = 16 * ks + 8 * h + j;
+        x[j] = (ci < Cin && co < Cout) ? W[((int64_t)co * Cin + ci) * 16 + d] : 0.f;
+    }
+    u32x4 p1, p2, p3;
+    split8(x, p1, p2, p3);
+    u32x4 *dst = WpT + ((size_t)(tt * NKS + ks) * 3) * 64 + lane;
+    dst[0] = p1; dst[64] = p2; dst[128] = p3;
+}
+
+template <int KW>
+__device__ __forceinline__ void x3_tex_sweep(const u32x4 *__restrict__ WpT, const float *__restrict__ sh,
+                                             float *__restrict__ gtex, u32x4 *Ws, const u32x4 (&bp)[kTKS][3],
+                                             int kbase, int Ks, float invK, int Cin, int NKS, int NG, int lane, int h)
+{
+    // SH rows of my facet's points, pre-scaled by 1/K
+    float shr[KW][16];
+#pragma unroll
+    for (int kk = 0; kk < KW; ++kk) {
+#pragma unroll
+        for (int v4 = 0; v4 < 4; ++v4) {
+            float4 u = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (kk < Ks) u = xld4(sh + (int64_t)(kbase + kk) * 16 + 4 * v4);
+            shr[kk][4 * v4 + 0] = u.x * invK; shr[kk][4 * v4 + 1] = u.y * invK;
+            shr[kk][4 * v4 + 2] = u.z * invK; shr[kk][4 * v4 + 3] = u.w * invK;
+        }
+    }
+    const int chunk = 2 * NKS * 192;             // uint4 per chunk of two tiles
+    const int nchunks = 2 * NG;
+    auto chunk_fetch = [&](u32x4 (&wn)[3], int c) {
+#pragma unroll
+        for (int i = 0; i < 3; ++i) {
+            const int e = threadIdx.x + 512 * i;
+            if (e < chunk) wn[i] = WpT[(size_t)c * chunk + e];
+        }
+    };
+    auto chunk_publish = [&](const u32x4 (&wn)[3], int c) {
+#pragma unroll
+        for (int i = 0; i < 3; ++i) {
+            const int e = threadIdx.x + 512 * i;
+            if (e < chunk) Ws[(c % 3) * kTChunkMax + e] = wn[i];
+        }
+    };
+    u32x4 wn[3];
+    chunk_fetch(wn, 0);
+    chunk_publish(wn, 0);
+    chunk_fetch(wn, 1);
+    chunk_publish(wn, 1);
+    __syncthreads();
+
+    for (int g = 0; g < NG; ++g) {
+        float gacc[KW][4];
+#pragma unroll
+        for (int kk = 0; kk < KW; ++kk)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) gacc[kk][q] = 0.f;
+#pragma unroll
+        for (int cc = 0; cc < 2; ++cc) {
+            const int c = 2 * g + cc;
+            const bool more = c + 2 < nchunks;
+            if (more) chunk_fetch(wn, c + 2);
+            const u32x4 *Wc = Ws + (c % 3) * kTChunkMax + lane;
+#pragma unroll
+            for (int u = 0; u < 2; ++u) {
+                // H tile of two input channels: rows (channel half, d), columns = my wavefront's facets
+                f32x16 acc0;
+#pragma unroll
+                for (int i = 0; i < 16; ++i) acc0[i] = 0.f;
+#pragma unroll
+                for (int ks = 0; ks < kTKS; ++ks) {
+                    if (ks < NKS) {
+                        u32x4 a[3];
+#pragma unroll
+                        for (int p = 0; p < 3; ++p) a[p] = Wc[((u * NKS + ks) * 3 + p) * 64];
+                        // six piece products, smallest first
+                        acc0 = mfma_bf16(a[2], bp[ks][0], acc0);
+                        acc0 = mfma_bf16(a[1], bp[ks][1], acc0);
+                        acc0 = mfma_bf16(a[0], bp[ks][2], acc0);
+                        acc0 = mfma_bf16(a[1], bp[ks][0], acc0);
+                        acc0 = mfma_bf16(a[0], bp[ks][1], acc0);
+                        acc0 = mfma_bf16(a[0], bp[ks][0], acc0);
+                    }
+                }
+                // contraction with the SH rows: my channel of this tile is 8g + 4h + q, q = 2cc + u
+#pragma unroll
+                for (int kk = 0; kk < KW; ++kk) {
+                    float v = 0.f;
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) v = fmaf(shr[kk][i], acc0[i], v);
+                    gacc[kk][2 * cc + u] = v;
+                }
+            }
+            if (more) chunk_publish(wn, c + 2);
+            __syncthreads();
+        }
+        const int ci0 = 8 * g + 4 * h;
+        if (ci0 < Cin) {
+#pragma unroll
+            for (int kk = 0; kk < KW; ++kk)
+                if (kk < Ks)
+                    *reinterpret_cast<float4 *>(gtex + (int64_t)(kbase + kk) * Cin + ci0) =
+                        make_float4(gacc[kk][0], gacc[kk][1], gacc[kk][2], gacc[kk][3]);
+        }
+    }
+}
+
+__global__ __launch_bounds__(512, 2) void f2f16x3_bwd_tex_k(const float *__restrict__ gout,
+                                                            const u32x4 *__restrict__ WpT,
+                                                            const float *__restrict__ sh,
+                                                            const int *__restrict__ cum,
+                                                            const int *__restrict__ order, float *__restrict__ gtex,
+                                                            int64_t Nf, int T, int Cin, int Cout, int NKS, int NG)
+{
+    __shared__ u32x4 Ws[3 * kTChunkMax];
+    __shared__ int s_kmax;
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int l32 = lane & 31, h = lane >> 5;
+    if (threadIdx.x == 0) s_kmax = 0;
+    __syncthreads();
+
+    const int64_t slot = (int64_t)blockIdx.x * 256 + w * 32 + l32;
+    const int f = slot < Nf ? (order ? order[slot] : (int)slot) : -1;
+    int k0 = 0, K = 0;
+    if (f >= 0 && f < Nf) {
+        int a = f ? cum[f - 1] : 0, b = cum[f];
+        a = a < 0 ? 0 : (a > T ? T : a);
+        b = b < 0 ? 0 : (b > T ? T : b);
+        k0 = a;
+        K = b > a ? b - a : 0;
+    }
+    const float invK = K > 0 ? 1.0f / (float)K : 0.f;
+    {
+        const int km = xwave_max(K);
+        if (lane == 0) atomicMax(&s_kmax, km);
+    }
+    // my facet's gout row as B operand pieces: k-step ks, half h <-> channels 16ks + 8h .. + 7
+    u32x4 bp[kTKS][3];
+#pragma unroll
+    for (int ks = 0; ks < kTKS; ++ks) {
+        float x[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) x[j] = 0.f;
+        const int co = 16 * ks + 8 * h;
+        if (K > 0 && co < Cout) {
+            const float *p = gout + (int64_t)f * Cout + co;
+            const float4 u = xld4(p), v = xld4(p + 4);
+            x[0] = u.x; x[1] = u.y; x[2] = u.z; x[3] = u.w; x[4] = v.x; x[5] = v.y; x[6] = v.z; x[7] = v.w;
+        }
+        split8(x, bp[ks][0], bp[ks][1], bp[ks][2]);
+    }
+    __syncthreads();
+    const int nsweeps = (s_kmax + kXKB - 1) / kXKB;
+    for (int sw = 0; sw < nsweeps; ++sw) {
+        const int rem = K - sw * kXKB;
+        const int Ks = rem < 0 ? 0 : (rem > kXKB ? kXKB : rem);
+        const int kw = xwave_max(Ks);
+        const int kbase = k0 + sw * kXKB;
+        // every variant runs the same barriers, so wavefronts of a workgroup may pick different ones
+#define PM_X3T(N) x3_tex_sweep<N>(WpT, sh, gtex, Ws, bp, kbase, Ks, invK, Cin, NKS, NG, lane, h)
+        if (kw <= 1) PM_X3T(1);
+        else if (kw == 2) PM_X3T(2);
+        else if (kw == 3) PM_X3T(3);
+        else PM_X3T(4);
+#undef PM_X3T
+    }
+}
+
+// ----------------------------------------------------------------------------------------
 // filter gradient gW = gout^T . G on the bf16 matrix cores, split over facets.
 // A workgroup of 8 wavefronts owns a 64-channel slab of Cout, 64 input channels (8 per wavefront =
 // four 32-column tiles of two channels) and a contiguous facet range, walked in slabs of up to 16
@@ -646,6 +843,33 @@ int f2f16x3_fwd(const float *tex, const float *W, const float *sh, const int *cu
     PM_REQUIRE(grid_ok(gx) && gy <= 65535, "f2f_fwd: grid too large");
     f2f16x3_fwd_k<<<dim3((unsigned)gx, (unsigned)gy), dim3(kFThreads), 0, st>>>(tex, Wp, sh, cum, order, out, Nf, (int)T, Cin, Cout, NT);
     PM_LAUNCHED("f2f_fwd");
+    return 0;
+}
+
+size_t f2f16x3_bwd_texture_workspace_bytes(int Cin, int Cout)
+{
+    const int NG = (Cin + 7) / 8, NKS = (Cout + 15) / 16;
+    return (size_t)NG * 4 * NKS * 3 * 64 * sizeof(u32x4);
+}
+
+bool f2f16x3_bwd_texture_usable(const void *gout, int Cout) { return Cout <= 16 * kTKS && (Cout & 7) == 0 && (reinterpret_cast<uintptr_t>(gout) & 15u) == 0; }
+
+int f2f16x3_bwd_texture(const float *gout, const float *W, const float *sh, const int *cum, const int *order,
+                        float *gtex, void *workspace, size_t workspace_bytes, int64_t T, int64_t Nf, int Cin,
+                        int Cout, hipStream_t st)
+{
+    const int NG = (Cin + 7) / 8, NKS = (Cout + 15) / 16;
+    PM_REQUIRE(workspace && workspace_bytes >= f2f16x3_bwd_texture_workspace_bytes(Cin, Cout),
+               "f2f_bwd_texture: workspace too small (%zu bytes)", workspace_bytes);
+    PM_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 15u) == 0, "f2f_bwd_texture: workspace must be 16-byte aligned");
+    u32x4 *WpT = (u32x4 *)workspace;
+    const int n = NG * 4 * NKS * 64;
+    f2f16x3_pack_filter_t_k<<<dim3((unsigned)ceil_div(n, kBlock)), dim3(kBlock), 0, st>>>(W, WpT, Cin, Cout, NG * 4, NKS);
+    PM_LAUNCHED("f2f_bwd_texture(pack)");
+    const int64_t gx = ceil_div(Nf, 256);
+    PM_REQUIRE(grid_ok(gx), "f2f_bwd_texture: grid too large");
+    f2f16x3_bwd_tex_k<<<dim3((unsigned)gx), dim3(512), 0, st>>>(gout, WpT, sh, cum, order, gtex, Nf, (int)T, Cin, Cout, NKS, NG);
+    PM_LAUNCHED("f2f_bwd_texture");
     return 0;
 }
 

@@ -154,8 +154,10 @@ def facet2facet_backward(grad_output, input, filter, bary_coeff, num_texture):
         nbytes = _lib.query("pmesh_f2f_bwd_workspace_bytes", Cin, Cout, F)
         ws = workspace(nbytes, dev)
         st = stream_of(input)
+        order = topology.facet_order(num_texture, T) if Nf else None
+        order_ptr = order.data_ptr() if order is not None else None
         _lib.call("pmesh_f2f_bwd_texture", grad_output.data_ptr(), filter.data_ptr(), bary_coeff.data_ptr(),
-                  num_texture.data_ptr(), gin.data_ptr(), T, Nf, Cin, Cout, F, st)
+                  num_texture.data_ptr(), order_ptr, gin.data_ptr(), ws.data_ptr(), nbytes, T, Nf, Cin, Cout, F, st)
         _lib.call("pmesh_f2f_bwd_filter", grad_output.data_ptr(), input.data_ptr(), bary_coeff.data_ptr(),
-                  num_texture.data_ptr(), gfilt.data_ptr(), ws.data_ptr(), nbytes, T, Nf, Cin, Cout, F, st)
+                  num_texture.data_ptr(), order_ptr, gfilt.data_ptr(), ws.data_ptr(), nbytes, T, Nf, Cin, Cout, F, st)
     return [gin, gfilt]

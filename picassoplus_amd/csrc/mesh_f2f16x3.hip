@@ -821,6 +821,302 @@ int f2f16x3_bwd_filter_partials(const float *gout, const float *tex, const float
     return 0;
 }
 
+// ----------------------------------------------------------------------------------------
+// filter gradient, second formulation: G is formed exactly as in the forward (lane = facet, eight
+// d's in registers, SH rows of the facet's points in registers), split into bf16 pieces, and each
+// piece is TRANSPOSED BY THE MATRIX CORE ITSELF: D = piece . E with a 0/1 selection matrix E is exact
+// and leaves, in the accumulator layout, lane = column (channel, d) and registers = facets -- the
+// layout of an MFMA operand whose reduction index is the facet.  Two input channels share one
+// transposition tile (columns 0..15 / 16..31).  The facet order inside a reduction step is the
+// accumulator's row order; the gout operand is built with the same order.
+//   workgroup  4 wavefronts (one per SIMD, accumulators in 256 registers), 64 input x 64 output
+//              channels, a strided subset of the 32-facet tiles of the sorted facet list
+//   wavefront  16 input channels = 8 channel pairs x 2 output tiles of gW^T[(ci,d)][co]
+//   gout^T     per facet tile split and laid out per lane in LDS by the whole workgroup
+constexpr int kGCi = 16;                         // input channels of a wavefront
+
+// One pass = up to four texture points per facet (kw = the wavefront's maximum, wave-uniform: the
+// branches on it are scalar).  A single instance serves every kw: separate instances per kw made the
+// register allocator spill the accumulators at their merge points.
+// shr: SH values of my facet's points (my half's eight d's, scaled by 1/K); slab: the wavefront's
+// texture values [point][16-byte piece][facet slot]; go: the tile's gout^T operand.
+__device__ __forceinline__ void x3_filt_pass(const float (&shr)[kXKB][8], const float4 *slab, const u32x4 *go,
+                                             f32x16 (&acc)[8][2], int kw, const u32x4 &ea, const u32x4 &eb, int lane)
+{
+    constexpr int KW = kXKB;
+    const int l32 = lane & 31;
+#pragma unroll
+    for (int cp = 0; cp < 8; ++cp) {
+        // G of channels cbase + 2cp (a) and + 1 (b): eight d's of my half for my facet
+        float aa[8], ab[8];
+#pragma unroll
+        for (int kk = 0; kk < KW; ++kk) {
+            if (kk < kw) {
+                const float4 t4 = slab[(kk * 4 + (cp >> 1)) * 32 + l32];
+                const float ta = (cp & 1) ? t4.z : t4.x, tb = (cp & 1) ? t4.w : t4.y;
+#pragma unroll
+                for (int q = 0; q < 8; ++q) {
+                    aa[q] = kk ? fmaf(ta, shr[kk][q], aa[q]) : ta * shr[kk][q];
+                    ab[q] = kk ? fmaf(tb, shr[kk][q], ab[q]) : tb * shr[kk][q];
+                }
+            }
+        }
+        u32x4 pa[3], pb[3];
+        split8(aa, pa[0], pa[1], pa[2]);
+        split8(ab, pb[0], pb[1], pb[2]);
+        // transposed pieces as operands of the two reduction steps (16 facets each)
+        u32x4 o[3][2];
+#pragma unroll
+        for (int p = 0; p < 3; ++p) {
+            f32x16 d;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) d[i] = 0.f;
+            d = mfma_bf16(pa[p], ea, d);
+            d = mfma_bf16(pb[p], eb, d);
+#pragma unroll
+            for (int st = 0; st < 2; ++st)
+#pragma unroll
+                for (int jj = 0; jj < 4; ++jj) o[p][st][jj] = pack_hi(d[8 * st + 2 * jj], d[8 * st + 2 * jj + 1]);
+        }
+#pragma unroll
+        for (int st = 0; st < 2; ++st) {
+            u32x4 g[2][3];
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int p = 0; p < 3; ++p) g[t][p] = go[((st * 2 + t) * 3 + p) * 64 + lane];
+            // six piece products, smallest first; the two output tiles alternate so that no MFMA
+            // waits for the one issued right before it
+#pragma unroll
+            for (int term = 0; term < 6; ++term) {
+                const int ga = term == 0 ? 2 : term == 1 ? 1 : term == 2 ? 0 : term == 3 ? 1 : 0;
+                const int wb = term == 0 ? 0 : term == 1 ? 1 : term == 2 ? 2 : term == 3 ? 0 : term == 4 ? 1 : 0;
+#pragma unroll
+                for (int t = 0; t < 2; ++t) acc[cp][t] = mfma_bf16(o[ga][st], g[t][wb], acc[cp][t]);
+            }
+        }
+    }
+}
+
+// slot descriptors of a 32-facet tile: facet id (-1: none), first texture point, number of points
+struct XTile {
+    int f, k0, K;
+};
+__device__ __forceinline__ XTile xtile_load(const int *__restrict__ cum, const int *__restrict__ order, int64_t tile,
+                                            int64_t ntiles, int64_t Nf, int T, int i)
+{
+    XTile d = {-1, 0, 0};
+    const int64_t slot = tile * 32 + i;
+    if (tile < ntiles && slot < Nf) {
+        const int f = order ? order[slot] : (int)slot;
+        if (f >= 0 && f < Nf) {
+            int a = f ? cum[f - 1] : 0, b = cum[f];
+            a = a < 0 ? 0 : (a > T ? T : a);
+            b = b < 0 ? 0 : (b > T ? T : b);
+            if (b > a) d = {f, a, b - a};
+        }
+    }
+    return d;
+}
+
+// The inputs of a tile's first pass are fetched by the whole workgroup while the previous tile is
+// being multiplied (held in registers, written to the other LDS buffer afterwards):
+//   gout     thread (co, step, half): its eight facets in accumulator-row order
+//   SH rows  32 facets x 4 points x 64 bytes, two 16-byte pieces per thread
+//   texture  32 facets x 4 points x 64 channels, eight 16-byte pieces per thread, 16 threads per row
+struct XPre {
+    float g[8];
+    float4 shv[2], tx[8];
+};
+__device__ __forceinline__ void xpre_issue(XPre &P, const float *__restrict__ gout, const float *__restrict__ tex,
+                                           const float *__restrict__ sh, const int *sf, const int *sk0, const int *sK,
+                                           int Cin, int Cout, int c0, int n0)
+{
+    const int co = threadIdx.x & 63, st = (threadIdx.x >> 6) & 1, hh = threadIdx.x >> 7;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const int f = sf[16 * st + 8 * (j >> 2) + 4 * hh + (j & 3)];
+        P.g[j] = (f >= 0 && n0 + co < Cout) ? gout[(int64_t)f * Cout + n0 + co] : 0.f;
+    }
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const int e = threadIdx.x + 256 * i, row = e >> 2, kk = row >> 5, slot = row & 31;
+        P.shv[i] = kk < sK[slot] ? xld4(sh + (int64_t)(sk0[slot] + kk) * 16 + 4 * (e & 3)) : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const int e = threadIdx.x + 256 * i, row = e >> 4, kk = row >> 5, slot = row & 31, ci = c0 + 4 * (e & 15);
+        P.tx[i] = (kk < sK[slot] && ci < Cin) ? xld4(tex + (int64_t)(sk0[slot] + kk) * Cin + ci)
+                                              : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+}
+__device__ __forceinline__ void xpre_commit(const XPre &P, u32x4 *go, float *shs, float4 *slab)
+{
+    const int co = threadIdx.x & 63, st = (threadIdx.x >> 6) & 1, hh = threadIdx.x >> 7;
+    u32x4 p1, p2, p3;
+    split8(P.g, p1, p2, p3);
+    u32x4 *dst = go + ((st * 2 + (co >> 5)) * 3) * 64 + 32 * hh + (co & 31);
+    dst[0] = p1; dst[64] = p2; dst[128] = p3;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const int e = threadIdx.x + 256 * i;
+        *reinterpret_cast<float4 *>(shs + 4 * e) = P.shv[i];             // [point*32 + slot][16]
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const int e = threadIdx.x + 256 * i, row = e >> 4, kk = row >> 5, slot = row & 31, p16 = e & 15;
+        slab[(p16 >> 2) * (kXKB * 4 * 32) + (kk * 4 + (p16 & 3)) * 32 + slot] = P.tx[i];   // [wavefront][point][piece][slot]
+    }
+}
+
+__global__ __launch_bounds__(256, 1) void f2f16x3_bwd_filt2_k(const float *__restrict__ gout,
+                                                              const float *__restrict__ tex,
+                                                              const float *__restrict__ sh,
+                                                              const int *__restrict__ cum,
+                                                              const int *__restrict__ order,
+                                                              float *__restrict__ partial, int64_t Nf, int T, int Cin,
+                                                              int Cout, int64_t ntiles)
+{
+    __shared__ u32x4 go_s[2][2 * 2 * 3 * 64];
+    __shared__ float4 slab_s[2][4 * kXKB * 4 * 32];
+    __shared__ __attribute__((aligned(16))) float sh_s[2][kXKB * 32 * 16];
+    __shared__ int s_f[3][32], s_k0[3][32], s_K[3][32];
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int l32 = lane & 31, h = lane >> 5;
+    const int c0 = blockIdx.y * 64, n0 = blockIdx.z * 64;
+
+    // selection operands of the transposition: column n < 16 takes d = n of channel a, n >= 16 takes d = n - 16 of b
+    u32x4 ea, eb;
+#pragma unroll
+    for (int jj = 0; jj < 4; ++jj) {
+        unsigned va = 0, vb = 0;
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            const int d = 8 * h + 2 * jj + u;
+            if (l32 < 16 && d == l32) va |= 0x3F80u << (16 * u);
+            if (l32 >= 16 && d == l32 - 16) vb |= 0x3F80u << (16 * u);
+        }
+        ea[jj] = va;
+        eb[jj] = vb;
+    }
+
+    f32x16 acc[8][2];
+#pragma unroll
+    for (int cp = 0; cp < 8; ++cp)
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) acc[cp][t][i] = 0.f;
+
+    // prologue: descriptors of my first two tiles, inputs of the first
+    const int64_t stride = gridDim.x;
+    int64_t tile = blockIdx.x;
+    if (threadIdx.x < 64) {
+        const int q = threadIdx.x >> 5;
+        const XTile d = xtile_load(cum, order, tile + q * stride, ntiles, Nf, T, threadIdx.x & 31);
+        s_f[q][threadIdx.x & 31] = d.f; s_k0[q][threadIdx.x & 31] = d.k0; s_K[q][threadIdx.x & 31] = d.K;
+    }
+    __syncthreads();
+    {
+        XPre P;
+        xpre_issue(P, gout, tex, sh, s_f[0], s_k0[0], s_K[0], Cin, Cout, c0, n0);
+        xpre_commit(P, go_s[0], sh_s[0], slab_s[0]);
+    }
+    __syncthreads();
+
+    for (int it = 0; tile < ntiles; ++it, tile += stride) {
+        const int buf = it & 1, sb = it % 3, sb1 = (it + 1) % 3, sb2 = (it + 2) % 3;
+        // in flight while this tile is multiplied: inputs of the next tile, descriptors of the one after
+        XPre P;
+        xpre_issue(P, gout, tex, sh, s_f[sb1], s_k0[sb1], s_K[sb1], Cin, Cout, c0, n0);
+        XTile dn = {-1, 0, 0};
+        if (threadIdx.x < 32) dn = xtile_load(cum, order, tile + 2 * stride, ntiles, Nf, T, threadIdx.x);
+
+        const int k0 = s_k0[sb][l32], K = s_K[sb][l32];
+        const float invK = K > 0 ? 1.0f / (float)K : 0.f;
+        const int nsweeps = (xwave_max(K) + kXKB - 1) / kXKB;
+        float4 *slab = slab_s[buf] + w * (kXKB * 4 * 32);
+        for (int sw = 0; sw < nsweeps; ++sw) {
+            const int rem = K - sw * kXKB;
+            const int Ks = rem < 0 ? 0 : (rem > kXKB ? kXKB : rem);
+            const int kw = xwave_max(Ks);
+            float shr[kXKB][8];
+            if (sw == 0) {
+#pragma unroll
+                for (int kk = 0; kk < kXKB; ++kk) {
+                    const float *p = sh_s[buf] + (kk * 32 + l32) * 16 + 8 * h;
+                    const float4 u = xld4(p), v = xld4(p + 4);
+                    shr[kk][0] = u.x * invK; shr[kk][1] = u.y * invK; shr[kk][2] = u.z * invK; shr[kk][3] = u.w * invK;
+                    shr[kk][4] = v.x * invK; shr[kk][5] = v.y * invK; shr[kk][6] = v.z * invK; shr[kk][7] = v.w * invK;
+                }
+            } else {
+                // further points of long facets: fetched directly (my wavefront's slab is free after its first pass)
+#pragma unroll
+                for (int kk = 0; kk < kXKB; ++kk) {
+                    float4 u = make_float4(0.f, 0.f, 0.f, 0.f), v = u;
+                    if (kk < Ks) {
+                        const float *p = sh + (int64_t)(k0 + sw * kXKB + kk) * 16 + 8 * h;
+                        u = xld4(p);
+                        v = xld4(p + 4);
+                    }
+                    shr[kk][0] = u.x * invK; shr[kk][1] = u.y * invK; shr[kk][2] = u.z * invK; shr[kk][3] = u.w * invK;
+                    shr[kk][4] = v.x * invK; shr[kk][5] = v.y * invK; shr[kk][6] = v.z * invK; shr[kk][7] = v.w * invK;
+                }
+                const int piece = lane & 3;
+                float4 pf[2 * kXKB];
+#pragma unroll
+                for (int i = 0; i < 2 * kXKB; ++i) {
+                    const int rr = i * 16 + (lane >> 2), kk = rr >> 5, slot = rr & 31;
+                    const bool ok = sw * kXKB + kk < s_K[sb][slot] && c0 + kGCi * w + 4 * piece < Cin;
+                    pf[i] = ok ? xld4(tex + (int64_t)(s_k0[sb][slot] + sw * kXKB + kk) * Cin + c0 + kGCi * w + 4 * piece)
+                               : make_float4(0.f, 0.f, 0.f, 0.f);
+                }
+#pragma unroll
+                for (int i = 0; i < 2 * kXKB; ++i) {
+                    const int rr = i * 16 + (lane >> 2), kk = rr >> 5, slot = rr & 31;
+                    slab[(kk * 4 + piece) * 32 + slot] = pf[i];
+                }
+            }
+            x3_filt_pass(shr, slab, go_s[buf], acc, kw, ea, eb, lane);
+        }
+
+        xpre_commit(P, go_s[buf ^ 1], sh_s[buf ^ 1], slab_s[buf ^ 1]);
+        if (threadIdx.x < 32) {
+            s_f[sb2][threadIdx.x] = dn.f; s_k0[sb2][threadIdx.x] = dn.k0; s_K[sb2][threadIdx.x] = dn.K;
+        }
+        __syncthreads();
+    }
+
+    // accumulator (cp, t): lane (co = 32t + l32, half h), register i <-> row m = 8(i/4) + 4h + i%4
+    // = (channel c0 + 16w + 2cp + m/16, d = m%16); four consecutive d's per group of four registers
+    float *dst = partial + (int64_t)blockIdx.x * Cout * Cin * 16;
+#pragma unroll
+    for (int cp = 0; cp < 8; ++cp)
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            const int co = n0 + 32 * t + l32;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int ci = c0 + kGCi * w + 2 * cp + (q >> 1);
+                if (co < Cout && ci < Cin)
+                    *reinterpret_cast<float4 *>(dst + ((int64_t)co * Cin + ci) * 16 + 8 * (q & 1) + 4 * h) =
+                        make_float4(acc[cp][t][4 * q], acc[cp][t][4 * q + 1], acc[cp][t][4 * q + 2], acc[cp][t][4 * q + 3]);
+            }
+        }
+}
+
+int f2f16x3_bwd_filter_partials2(const float *gout, const float *tex, const float *sh, const int *cum, const int *order,
+                                 float *partial, int splits, int64_t T, int64_t Nf, int Cin, int Cout, hipStream_t st)
+{
+    const int64_t gy = ceil_div(Cin, 64), gz = ceil_div(Cout, 64);
+    PM_REQUIRE(gy <= 65535 && gz <= 65535, "f2f_bwd_filter: grid too large");
+    const int64_t ntiles = ceil_div(Nf, 32);
+    f2f16x3_bwd_filt2_k<<<dim3((unsigned)splits, (unsigned)gy, (unsigned)gz), dim3(256), 0, st>>>(
+        gout, tex, sh, cum, order, partial, Nf, (int)T, Cin, Cout, ntiles);
+    PM_LAUNCHED("f2f_bwd_filter");
+    return 0;
+}
+
 size_t f2f16x3_fwd_workspace_bytes(int Cin, int Cout)
 {
     const int NT = 2 * ((Cout + 63) / 64);

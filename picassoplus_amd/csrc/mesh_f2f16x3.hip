@@ -845,9 +845,8 @@ __device__ __forceinline__ void x3_filt_pass(const float (&shr)[kXKB][8], const 
 {
     constexpr int KW = kXKB;
     const int l32 = lane & 31;
-#pragma unroll
-    for (int cp = 0; cp < 8; ++cp) {
-        // G of channels cbase + 2cp (a) and + 1 (b): eight d's of my half for my facet
+    // G of channels cbase + 2cp (a) and + 1 (b), eight d's of my half for my facet, as bf16 pieces
+    auto gen = [&](u32x4 (&pa)[3], u32x4 (&pb)[3], int cp) {
         float aa[8], ab[8];
 #pragma unroll
         for (int kk = 0; kk < KW; ++kk) {
@@ -861,23 +860,50 @@ __device__ __forceinline__ void x3_filt_pass(const float (&shr)[kXKB][8], const 
                 }
             }
         }
-        u32x4 pa[3], pb[3];
         split8(aa, pa[0], pa[1], pa[2]);
         split8(ab, pb[0], pb[1], pb[2]);
-        // transposed pieces as operands of the two reduction steps (16 facets each)
-        u32x4 o[3][2];
+    };
+    // transposed pieces as operands of the two reduction steps (16 facets each); the three
+    // transpositions are independent, so their MFMAs run back to back
+    // The six MFMAs are written as one asm block with VGPR destinations: in a kernel whose accumulators
+    // live in AGPRs the compiler gives every MFMA an AGPR destination, and the 48 results would have
+    // to be copied out one by one before the packing.  The trailing s_nop cover the wait states a
+    // vector ALU read of an MFMA result needs (the compiler cannot see into the block).
+    auto transpose = [&](u32x4 (&o)[3][2], const u32x4 (&pa)[3], const u32x4 (&pb)[3]) {
+        f32x16 d0, d1, d2;
+        asm volatile("s_nop 3\n"
+                     "v_mfma_f32_32x32x16_bf16 %0, %3, %9, 0\n"
+                     "v_mfma_f32_32x32x16_bf16 %1, %4, %9, 0\n"
+                     "v_mfma_f32_32x32x16_bf16 %2, %5, %9, 0\n"
+                     "v_mfma_f32_32x32x16_bf16 %0, %6, %10, %0\n"
+                     "v_mfma_f32_32x32x16_bf16 %1, %7, %10, %1\n"
+                     "v_mfma_f32_32x32x16_bf16 %2, %8, %10, %2\n"
+                     "s_nop 15\n"
+                     "s_nop 7\n"
+                     : "=&v"(d0), "=&v"(d1), "=&v"(d2)
+                     : "v"(pa[0]), "v"(pa[1]), "v"(pa[2]), "v"(pb[0]), "v"(pb[1]), "v"(pb[2]), "v"(ea), "v"(eb));
 #pragma unroll
-        for (int p = 0; p < 3; ++p) {
-            f32x16 d;
+        for (int st = 0; st < 2; ++st)
 #pragma unroll
-            for (int i = 0; i < 16; ++i) d[i] = 0.f;
-            d = mfma_bf16(pa[p], ea, d);
-            d = mfma_bf16(pb[p], eb, d);
+            for (int jj = 0; jj < 4; ++jj) {
+                o[0][st][jj] = pack_hi(d0[8 * st + 2 * jj], d0[8 * st + 2 * jj + 1]);
+                o[1][st][jj] = pack_hi(d1[8 * st + 2 * jj], d1[8 * st + 2 * jj + 1]);
+                o[2][st][jj] = pack_hi(d2[8 * st + 2 * jj], d2[8 * st + 2 * jj + 1]);
+            }
+    };
+
+    // software pipeline over the channel pairs: the G values of pair cp+1 are generated and split
+    // (vector ALU) while the products of pair cp run on the matrix core
+    u32x4 o[3][2];
+    {
+        u32x4 pa[3], pb[3];
+        gen(pa, pb, 0);
+        transpose(o, pa, pb);
+    }
 #pragma unroll
-            for (int st = 0; st < 2; ++st)
-#pragma unroll
-                for (int jj = 0; jj < 4; ++jj) o[p][st][jj] = pack_hi(d[8 * st + 2 * jj], d[8 * st + 2 * jj + 1]);
-        }
+    for (int cp = 0; cp < 8; ++cp) {
+        u32x4 pa[3], pb[3];
+        if (cp + 1 < 8) gen(pa, pb, cp + 1);
 #pragma unroll
         for (int st = 0; st < 2; ++st) {
             u32x4 g[2][3];
@@ -895,6 +921,7 @@ __device__ __forceinline__ void x3_filt_pass(const float (&shr)[kXKB][8], const 
                 for (int t = 0; t < 2; ++t) acc[cp][t] = mfma_bf16(o[ga][st], g[t][wb], acc[cp][t]);
             }
         }
+        if (cp + 1 < 8) transpose(o, pa, pb);
     }
 }
 
@@ -923,10 +950,10 @@ __device__ __forceinline__ XTile xtile_load(const int *__restrict__ cum, const i
 // being multiplied (held in registers, written to the other LDS buffer afterwards):
 //   gout     thread (co, step, half): its eight facets in accumulator-row order
 //   SH rows  32 facets x 4 points x 64 bytes, two 16-byte pieces per thread
-//   texture  32 facets x 4 points x 64 channels, eight 16-byte pieces per thread, 16 threads per row
+// (each wavefront fetches the texture rows of its own 16 channels at the start of a pass)
 struct XPre {
     float g[8];
-    float4 shv[2], tx[8];
+    float4 shv[2];
 };
 __device__ __forceinline__ void xpre_issue(XPre &P, const float *__restrict__ gout, const float *__restrict__ tex,
                                            const float *__restrict__ sh, const int *sf, const int *sk0, const int *sK,
@@ -943,14 +970,8 @@ __device__ __forceinline__ void xpre_issue(XPre &P, const float *__restrict__ go
         const int e = threadIdx.x + 256 * i, row = e >> 2, kk = row >> 5, slot = row & 31;
         P.shv[i] = kk < sK[slot] ? xld4(sh + (int64_t)(sk0[slot] + kk) * 16 + 4 * (e & 3)) : make_float4(0.f, 0.f, 0.f, 0.f);
     }
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-        const int e = threadIdx.x + 256 * i, row = e >> 4, kk = row >> 5, slot = row & 31, ci = c0 + 4 * (e & 15);
-        P.tx[i] = (kk < sK[slot] && ci < Cin) ? xld4(tex + (int64_t)(sk0[slot] + kk) * Cin + ci)
-                                              : make_float4(0.f, 0.f, 0.f, 0.f);
-    }
 }
-__device__ __forceinline__ void xpre_commit(const XPre &P, u32x4 *go, float *shs, float4 *slab)
+__device__ __forceinline__ void xpre_commit(const XPre &P, u32x4 *go, float *shs)
 {
     const int co = threadIdx.x & 63, st = (threadIdx.x >> 6) & 1, hh = threadIdx.x >> 7;
     u32x4 p1, p2, p3;
@@ -961,11 +982,6 @@ __device__ __forceinline__ void xpre_commit(const XPre &P, u32x4 *go, float *shs
     for (int i = 0; i < 2; ++i) {
         const int e = threadIdx.x + 256 * i;
         *reinterpret_cast<float4 *>(shs + 4 * e) = P.shv[i];             // [point*32 + slot][16]
-    }
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-        const int e = threadIdx.x + 256 * i, row = e >> 4, kk = row >> 5, slot = row & 31, p16 = e & 15;
-        slab[(p16 >> 2) * (kXKB * 4 * 32) + (kk * 4 + (p16 & 3)) * 32 + slot] = P.tx[i];   // [wavefront][point][piece][slot]
     }
 }
 
@@ -978,7 +994,7 @@ __global__ __launch_bounds__(256, 1) void f2f16x3_bwd_filt2_k(const float *__res
                                                               int Cout, int64_t ntiles)
 {
     __shared__ u32x4 go_s[2][2 * 2 * 3 * 64];
-    __shared__ float4 slab_s[2][4 * kXKB * 4 * 32];
+    __shared__ float4 slab_s[4 * kXKB * 4 * 32];
     __shared__ __attribute__((aligned(16))) float sh_s[2][kXKB * 32 * 16];
     __shared__ int s_f[3][32], s_k0[3][32], s_K[3][32];
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
@@ -1020,7 +1036,7 @@ __global__ __launch_bounds__(256, 1) void f2f16x3_bwd_filt2_k(const float *__res
     {
         XPre P;
         xpre_issue(P, gout, tex, sh, s_f[0], s_k0[0], s_K[0], Cin, Cout, c0, n0);
-        xpre_commit(P, go_s[0], sh_s[0], slab_s[0]);
+        xpre_commit(P, go_s[0], sh_s[0]);
     }
     __syncthreads();
 
@@ -1035,7 +1051,7 @@ __global__ __launch_bounds__(256, 1) void f2f16x3_bwd_filt2_k(const float *__res
         const int k0 = s_k0[sb][l32], K = s_K[sb][l32];
         const float invK = K > 0 ? 1.0f / (float)K : 0.f;
         const int nsweeps = (xwave_max(K) + kXKB - 1) / kXKB;
-        float4 *slab = slab_s[buf] + w * (kXKB * 4 * 32);
+        float4 *slab = slab_s + w * (kXKB * 4 * 32);
         for (int sw = 0; sw < nsweeps; ++sw) {
             const int rem = K - sw * kXKB;
             const int Ks = rem < 0 ? 0 : (rem > kXKB ? kXKB : rem);
@@ -1050,7 +1066,7 @@ __global__ __launch_bounds__(256, 1) void f2f16x3_bwd_filt2_k(const float *__res
                     shr[kk][4] = v.x * invK; shr[kk][5] = v.y * invK; shr[kk][6] = v.z * invK; shr[kk][7] = v.w * invK;
                 }
             } else {
-                // further points of long facets: fetched directly (my wavefront's slab is free after its first pass)
+                // further points of long facets: fetched directly
 #pragma unroll
                 for (int kk = 0; kk < kXKB; ++kk) {
                     float4 u = make_float4(0.f, 0.f, 0.f, 0.f), v = u;
@@ -1062,12 +1078,15 @@ __global__ __launch_bounds__(256, 1) void f2f16x3_bwd_filt2_k(const float *__res
                     shr[kk][0] = u.x * invK; shr[kk][1] = u.y * invK; shr[kk][2] = u.z * invK; shr[kk][3] = u.w * invK;
                     shr[kk][4] = v.x * invK; shr[kk][5] = v.y * invK; shr[kk][6] = v.z * invK; shr[kk][7] = v.w * invK;
                 }
+            }
+            {
+                // my wavefront's texture rows (16 channels = 64 bytes each), four lanes per row
                 const int piece = lane & 3;
                 float4 pf[2 * kXKB];
 #pragma unroll
                 for (int i = 0; i < 2 * kXKB; ++i) {
                     const int rr = i * 16 + (lane >> 2), kk = rr >> 5, slot = rr & 31;
-                    const bool ok = sw * kXKB + kk < s_K[sb][slot] && c0 + kGCi * w + 4 * piece < Cin;
+                    const bool ok = kk < kw && sw * kXKB + kk < s_K[sb][slot] && c0 + kGCi * w + 4 * piece < Cin;
                     pf[i] = ok ? xld4(tex + (int64_t)(s_k0[sb][slot] + sw * kXKB + kk) * Cin + c0 + kGCi * w + 4 * piece)
                                : make_float4(0.f, 0.f, 0.f, 0.f);
                 }
@@ -1080,7 +1099,7 @@ __global__ __launch_bounds__(256, 1) void f2f16x3_bwd_filt2_k(const float *__res
             x3_filt_pass(shr, slab, go_s[buf], acc, kw, ea, eb, lane);
         }
 
-        xpre_commit(P, go_s[buf ^ 1], sh_s[buf ^ 1], slab_s[buf ^ 1]);
+        xpre_commit(P, go_s[buf ^ 1], sh_s[buf ^ 1]);
         if (threadIdx.x < 32) {
             s_f[sb2][threadIdx.x] = dn.f; s_k0[sb2][threadIdx.x] = dn.k0; s_K[sb2][threadIdx.x] = dn.K;
         }

@@ -835,29 +835,25 @@ int f2f16x3_bwd_filter_partials(const float *gout, const float *tex, const float
 //   gout^T     per facet tile split and laid out per lane in LDS by the whole workgroup
 constexpr int kGCi = 16;                         // input channels of a wavefront
 
-// One pass = up to four texture points per facet (kw = the wavefront's maximum, wave-uniform: the
-// branches on it are scalar).  A single instance serves every kw: separate instances per kw made the
-// register allocator spill the accumulators at their merge points.
+// One pass = up to KW texture points per facet (missing points contribute zeros), straight-line code.
 // shr: SH values of my facet's points (my half's eight d's, scaled by 1/K); slab: the wavefront's
 // texture values [point][16-byte piece][facet slot]; go: the tile's gout^T operand.
-__device__ __forceinline__ void x3_filt_pass(const float (&shr)[kXKB][8], const float4 *slab, const u32x4 *go,
-                                             f32x16 (&acc)[8][2], int kw, const u32x4 &ea, const u32x4 &eb, int lane)
+template <int KW>
+__device__ __forceinline__ void x3_filt_pass(const float (&shr)[KW][8], const float4 *slab, const u32x4 *go,
+                                             f32x16 (&acc)[8][2], const u32x4 &ea, const u32x4 &eb, int lane)
 {
-    constexpr int KW = kXKB;
     const int l32 = lane & 31;
     // G of channels cbase + 2cp (a) and + 1 (b), eight d's of my half for my facet, as bf16 pieces
     auto gen = [&](u32x4 (&pa)[3], u32x4 (&pb)[3], int cp) {
         float aa[8], ab[8];
 #pragma unroll
         for (int kk = 0; kk < KW; ++kk) {
-            if (kk < kw) {
-                const float4 t4 = slab[(kk * 4 + (cp >> 1)) * 32 + l32];
-                const float ta = (cp & 1) ? t4.z : t4.x, tb = (cp & 1) ? t4.w : t4.y;
+            const float4 t4 = slab[(kk * 4 + (cp >> 1)) * 32 + l32];
+            const float ta = (cp & 1) ? t4.z : t4.x, tb = (cp & 1) ? t4.w : t4.y;
 #pragma unroll
-                for (int q = 0; q < 8; ++q) {
-                    aa[q] = kk ? fmaf(ta, shr[kk][q], aa[q]) : ta * shr[kk][q];
-                    ab[q] = kk ? fmaf(tb, shr[kk][q], ab[q]) : tb * shr[kk][q];
-                }
+            for (int q = 0; q < 8; ++q) {
+                aa[q] = kk ? fmaf(ta, shr[kk][q], aa[q]) : ta * shr[kk][q];
+                ab[q] = kk ? fmaf(tb, shr[kk][q], ab[q]) : tb * shr[kk][q];
             }
         }
         split8(aa, pa[0], pa[1], pa[2]);
@@ -985,6 +981,84 @@ __device__ __forceinline__ void xpre_commit(const XPre &P, u32x4 *go, float *shs
     }
 }
 
+__device__ __forceinline__ int xtile_kmax(const int *sK, int lane) { return xwave_max(sK[lane & 31]); }
+
+// One tile of 32 facets whose inputs are in LDS buffer it % 2 (descriptors in it % 3): start the
+// fetches for the next tile, run the passes, publish the next tile's inputs.
+template <int KW>
+__device__ __forceinline__ void x3_filt_tile(const float *__restrict__ gout, const float *__restrict__ tex,
+                                             const float *__restrict__ sh, const int *__restrict__ cum,
+                                             const int *__restrict__ order, u32x4 (*go_s)[2 * 2 * 3 * 64], float4 *slab,
+                                             float (*sh_s)[kXKB * 32 * 16], int (*s_f)[32], int (*s_k0)[32],
+                                             int (*s_K)[32], f32x16 (&acc)[8][2], const u32x4 &ea, const u32x4 &eb,
+                                             int it, int64_t tile, int64_t stride, int64_t ntiles, int64_t Nf, int T,
+                                             int Cin, int Cout, int c0, int n0, int lane, int w)
+{
+    const int l32 = lane & 31, h = lane >> 5;
+    const int buf = it & 1, sb = it % 3, sb1 = (it + 1) % 3, sb2 = (it + 2) % 3;
+    // in flight while this tile is multiplied: inputs of the next tile, descriptors of the one after
+    XPre P;
+    xpre_issue(P, gout, tex, sh, s_f[sb1], s_k0[sb1], s_K[sb1], Cin, Cout, c0, n0);
+    XTile dn = {-1, 0, 0};
+    if (threadIdx.x < 32) dn = xtile_load(cum, order, tile + 2 * stride, ntiles, Nf, T, threadIdx.x);
+
+    const int k0 = s_k0[sb][l32], K = s_K[sb][l32];
+    const float invK = K > 0 ? 1.0f / (float)K : 0.f;
+    const int nsweeps = KW < kXKB ? 1 : (xwave_max(K) + kXKB - 1) / kXKB;
+    const int cw = c0 + kGCi * w;                        // my wavefront's first input channel
+    for (int sw = 0; sw < nsweeps; ++sw) {
+        const int rem = K - sw * kXKB;
+        const int Ks = rem < 0 ? 0 : (rem > KW ? KW : rem);
+        float shr[KW][8];
+        if (sw == 0) {
+#pragma unroll
+            for (int kk = 0; kk < KW; ++kk) {
+                const float *p = sh_s[buf] + (kk * 32 + l32) * 16 + 8 * h;
+                const float4 u = xld4(p), v = xld4(p + 4);
+                shr[kk][0] = u.x * invK; shr[kk][1] = u.y * invK; shr[kk][2] = u.z * invK; shr[kk][3] = u.w * invK;
+                shr[kk][4] = v.x * invK; shr[kk][5] = v.y * invK; shr[kk][6] = v.z * invK; shr[kk][7] = v.w * invK;
+            }
+        } else {
+            // further points of long facets: fetched directly
+#pragma unroll
+            for (int kk = 0; kk < KW; ++kk) {
+                float4 u = make_float4(0.f, 0.f, 0.f, 0.f), v = u;
+                if (kk < Ks) {
+                    const float *p = sh + (int64_t)(k0 + sw * kXKB + kk) * 16 + 8 * h;
+                    u = xld4(p);
+                    v = xld4(p + 4);
+                }
+                shr[kk][0] = u.x * invK; shr[kk][1] = u.y * invK; shr[kk][2] = u.z * invK; shr[kk][3] = u.w * invK;
+                shr[kk][4] = v.x * invK; shr[kk][5] = v.y * invK; shr[kk][6] = v.z * invK; shr[kk][7] = v.w * invK;
+            }
+        }
+        {
+            // my wavefront's texture rows (16 channels = 64 bytes each), four lanes per row
+            const int piece = lane & 3;
+            float4 pf[2 * KW];
+#pragma unroll
+            for (int i = 0; i < 2 * KW; ++i) {
+                const int rr = i * 16 + (lane >> 2), kk = rr >> 5, slot = rr & 31;
+                const bool ok = sw * kXKB + kk < s_K[sb][slot] && cw + 4 * piece < Cin;
+                pf[i] = ok ? xld4(tex + (int64_t)(s_k0[sb][slot] + sw * kXKB + kk) * Cin + cw + 4 * piece)
+                           : make_float4(0.f, 0.f, 0.f, 0.f);
+            }
+#pragma unroll
+            for (int i = 0; i < 2 * KW; ++i) {
+                const int rr = i * 16 + (lane >> 2), kk = rr >> 5, slot = rr & 31;
+                slab[(kk * 4 + piece) * 32 + slot] = pf[i];
+            }
+        }
+        x3_filt_pass<KW>(shr, slab, go_s[buf], acc, ea, eb, lane);
+    }
+
+    xpre_commit(P, go_s[buf ^ 1], sh_s[buf ^ 1]);
+    if (threadIdx.x < 32) {
+        s_f[sb2][threadIdx.x] = dn.f; s_k0[sb2][threadIdx.x] = dn.k0; s_K[sb2][threadIdx.x] = dn.K;
+    }
+    __syncthreads();
+}
+
 __global__ __launch_bounds__(256, 1) void f2f16x3_bwd_filt2_k(const float *__restrict__ gout,
                                                               const float *__restrict__ tex,
                                                               const float *__restrict__ sh,
@@ -1040,71 +1114,19 @@ __global__ __launch_bounds__(256, 1) void f2f16x3_bwd_filt2_k(const float *__res
     }
     __syncthreads();
 
-    for (int it = 0; tile < ntiles; ++it, tile += stride) {
-        const int buf = it & 1, sb = it % 3, sb1 = (it + 1) % 3, sb2 = (it + 2) % 3;
-        // in flight while this tile is multiplied: inputs of the next tile, descriptors of the one after
-        XPre P;
-        xpre_issue(P, gout, tex, sh, s_f[sb1], s_k0[sb1], s_K[sb1], Cin, Cout, c0, n0);
-        XTile dn = {-1, 0, 0};
-        if (threadIdx.x < 32) dn = xtile_load(cum, order, tile + 2 * stride, ntiles, Nf, T, threadIdx.x);
-
-        const int k0 = s_k0[sb][l32], K = s_K[sb][l32];
-        const float invK = K > 0 ? 1.0f / (float)K : 0.f;
-        const int nsweeps = (xwave_max(K) + kXKB - 1) / kXKB;
-        float4 *slab = slab_s + w * (kXKB * 4 * 32);
-        for (int sw = 0; sw < nsweeps; ++sw) {
-            const int rem = K - sw * kXKB;
-            const int Ks = rem < 0 ? 0 : (rem > kXKB ? kXKB : rem);
-            const int kw = xwave_max(Ks);
-            float shr[kXKB][8];
-            if (sw == 0) {
-#pragma unroll
-                for (int kk = 0; kk < kXKB; ++kk) {
-                    const float *p = sh_s[buf] + (kk * 32 + l32) * 16 + 8 * h;
-                    const float4 u = xld4(p), v = xld4(p + 4);
-                    shr[kk][0] = u.x * invK; shr[kk][1] = u.y * invK; shr[kk][2] = u.z * invK; shr[kk][3] = u.w * invK;
-                    shr[kk][4] = v.x * invK; shr[kk][5] = v.y * invK; shr[kk][6] = v.z * invK; shr[kk][7] = v.w * invK;
-                }
-            } else {
-                // further points of long facets: fetched directly
-#pragma unroll
-                for (int kk = 0; kk < kXKB; ++kk) {
-                    float4 u = make_float4(0.f, 0.f, 0.f, 0.f), v = u;
-                    if (kk < Ks) {
-                        const float *p = sh + (int64_t)(k0 + sw * kXKB + kk) * 16 + 8 * h;
-                        u = xld4(p);
-                        v = xld4(p + 4);
-                    }
-                    shr[kk][0] = u.x * invK; shr[kk][1] = u.y * invK; shr[kk][2] = u.z * invK; shr[kk][3] = u.w * invK;
-                    shr[kk][4] = v.x * invK; shr[kk][5] = v.y * invK; shr[kk][6] = v.z * invK; shr[kk][7] = v.w * invK;
-                }
-            }
-            {
-                // my wavefront's texture rows (16 channels = 64 bytes each), four lanes per row
-                const int piece = lane & 3;
-                float4 pf[2 * kXKB];
-#pragma unroll
-                for (int i = 0; i < 2 * kXKB; ++i) {
-                    const int rr = i * 16 + (lane >> 2), kk = rr >> 5, slot = rr & 31;
-                    const bool ok = kk < kw && sw * kXKB + kk < s_K[sb][slot] && c0 + kGCi * w + 4 * piece < Cin;
-                    pf[i] = ok ? xld4(tex + (int64_t)(s_k0[sb][slot] + sw * kXKB + kk) * Cin + c0 + kGCi * w + 4 * piece)
-                               : make_float4(0.f, 0.f, 0.f, 0.f);
-                }
-#pragma unroll
-                for (int i = 0; i < 2 * kXKB; ++i) {
-                    const int rr = i * 16 + (lane >> 2), kk = rr >> 5, slot = rr & 31;
-                    slab[(kk * 4 + piece) * 32 + slot] = pf[i];
-                }
-            }
-            x3_filt_pass(shr, slab, go_s[buf], acc, kw, ea, eb, lane);
-        }
-
-        xpre_commit(P, go_s[buf ^ 1], sh_s[buf ^ 1]);
-        if (threadIdx.x < 32) {
-            s_f[sb2][threadIdx.x] = dn.f; s_k0[sb2][threadIdx.x] = dn.k0; s_K[sb2][threadIdx.x] = dn.K;
-        }
-        __syncthreads();
-    }
+    // The sorted facet list makes the point counts of my tiles non-decreasing: four loops in sequence,
+    // each with the pass specialised for its number of points (the last one takes everything left,
+    // long facets in several sweeps).  The bound is uniform over the workgroup.
+    int it = 0;
+#define PM_PHASE(N)                                                                                                  \
+    for (; tile < ntiles && (N == kXKB || xtile_kmax(s_K[it % 3], lane) <= N); ++it, tile += stride)                 \
+        x3_filt_tile<N>(gout, tex, sh, cum, order, go_s, slab_s + w * (kXKB * 4 * 32), sh_s, s_f, s_k0, s_K, acc, ea, eb,  \
+                        it, tile, stride, ntiles, Nf, T, Cin, Cout, c0, n0, lane, w)
+    PM_PHASE(1);
+    PM_PHASE(2);
+    PM_PHASE(3);
+    PM_PHASE(4);
+#undef PM_PHASE
 
     // accumulator (cp, t): lane (co = 32t + l32, half h), register i <-> row m = 8(i/4) + 4h + i%4
     // = (channel c0 + 16w + 2cp + m/16, d = m%16); four consecutive d's per group of four registers

@@ -23,11 +23,9 @@ int f2f16x3_bwd_texture(const float *gout, const float *W, const float *sh, cons
                         int Cout, hipStream_t st);
 
 // `splits` workgroups each write one partial (Cout x Cin*16) block; every split gets a strided share of the 32-facet tiles
-int f2f16x3_bwd_filter_partials2(const float *gout, const float *tex, const float *sh, const int *cum, const int *order,
+int f2f16x3_bwd_filter_partials(const float *gout, const float *tex, const float *sh, const int *cum, const int *order,
                                  float *partial, int splits, int64_t T, int64_t Nf, int Cin, int Cout, hipStream_t st);
 
-int f2f16x3_bwd_filter_partials(const float *gout, const float *tex, const float *sh, const int *cum, float *partial,
-                                int splits, int64_t T, int64_t Nf, int Cin, int Cout, hipStream_t st);
 
 int f2f16_bwd_texture(const float *gout, const float *W, const float *sh, const int *cum, float *gtex, int64_t T,
                       int64_t Nf, int Cin, int Cout, hipStream_t st);

@@ -1,4 +1,5 @@
-// facet2facet forward for 16 SH coefficients on the bf16 matrix cores with fp32-level accuracy.
+// facet2facet for 16 SH coefficients (forward, texture gradient, filter gradient) on the bf16 matrix
+// cores with fp32-level accuracy.
 //
 // v_mfma_f32_32x32x16_bf16 sustains ~14x the rate of v_mfma_f32_32x32x2_f32 on gfx950.  Both
 // operands of out = G . W^T are therefore split exactly into three bf16 pieces each,
@@ -566,263 +567,7 @@ __global__ __launch_bounds__(512, 2) void f2f16x3_bwd_tex_k(const float *__restr
 }
 
 // ----------------------------------------------------------------------------------------
-// filter gradient gW = gout^T . G on the bf16 matrix cores, split over facets.
-// A workgroup of 8 wavefronts owns a 64-channel slab of Cout, 64 input channels (8 per wavefront =
-// four 32-column tiles of two channels) and a contiguous facet range, walked in slabs of up to 16
-// facets / kFPS texture points = ONE MFMA reduction step (k = 16 facets):
-//   A[co][facet]   gout rows, split into three bf16 pieces by the threads that stage them in LDS
-//   B[facet][q]    G values of lane-half h's facets 8h..8h+7 (column l32 of tile t = channel
-//                  8w + 4*(l32/16) + t, SH index l32%16), formed in registers from the staged
-//                  texture / SH rows (four points at a time, all LDS reads issued first), split
-// Texture, SH and gout rows of the NEXT slab are in flight (registers) while a slab is processed,
-// and the descriptor of the slab after that is being fetched.
-// ----------------------------------------------------------------------------------------
-constexpr int kFFB = 16;       // facets per slab
-constexpr int kFPS = 128;      // texture points per slab
-constexpr int kFRow = 68;      // LDS stride of a staged texture row (64 channels)
-
-struct XSlab {
-    int fa, n, pa, pb, flush;
-};
-
-__device__ __forceinline__ int xseg_start(const int *__restrict__ cum, int64_t f, int T)
-{
-    const int v = f ? cum[f - 1] : 0;
-    return v < 0 ? 0 : (v > T ? T : v);
-}
-
-// lane i (0..16) fetches the start row of facet fa + i
-__device__ __forceinline__ int slab_bounds_load(const int *__restrict__ cum, int64_t fa, int64_t fend, int T, int lane)
-{
-    const int64_t fi = fa + lane;
-    return (fa < fend && lane <= kFFB && fi <= fend) ? xseg_start(cum, fi, T) : T;
-}
-
-// descriptor of the slab starting at facet fa from the bounds fetched by slab_bounds_load;
-// pa_cont >= 0 continues a facet that has more than kFPS points
-__device__ __forceinline__ XSlab slab_from_bounds(int c, int64_t fa, int64_t fend, int pa_cont, int lane)
-{
-    XSlab S;
-    S.fa = (int)fa; S.n = 0; S.pa = 0; S.pb = 0; S.flush = 1;
-    if (fa >= fend) return S;
-    const int s0 = __builtin_amdgcn_readfirstlane(c);
-    const int cn = __shfl_down(c, 1, 64);
-    const int e = cn > c ? cn : c;
-    const int e0 = __builtin_amdgcn_readfirstlane(e);
-    const bool ok = lane < kFFB && fa + lane < fend && e - s0 <= kFPS;
-    const int n = __builtin_ctzll(~__ballot(ok));
-    if (pa_cont >= 0 || n == 0) {
-        S.n = 1;
-        S.pa = pa_cont >= 0 ? pa_cont : s0;
-        S.pb = (S.pa + kFPS < e0) ? S.pa + kFPS : e0;
-        S.flush = S.pb >= e0;
-        return S;
-    }
-    int pb = lane < n ? e : s0;
-#pragma unroll
-    for (int o = 16; o > 0; o >>= 1) {
-        const int t = __shfl_xor(pb, o, 64);
-        pb = t > pb ? t : pb;
-    }
-    S.n = n; S.pa = s0; S.pb = __builtin_amdgcn_readfirstlane(pb);
-    return S;
-}
-
-__global__ __launch_bounds__(512, 2) void f2f16x3_bwd_filt_k(const float *__restrict__ gout, const float *__restrict__ tex,
-                                                             const float *__restrict__ sh, const int *__restrict__ cum,
-                                                             float *__restrict__ partial, int64_t Nf, int T, int Cin,
-                                                             int Cout, int64_t facets_per_split)
-{
-    __shared__ __attribute__((aligned(16))) float tex_s[kFPS * kFRow];
-    __shared__ __attribute__((aligned(16))) float sh_s[kFPS * 16];
-    __shared__ __attribute__((aligned(16))) unsigned short go_p[3 * 64 * kFFB];   // [piece][co][facet] bf16
-    __shared__ int seg_s[2 * kFFB];
-    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
-    const int l32 = lane & 31, h = lane >> 5;
-    const int cbase = blockIdx.y * 64, n0 = blockIdx.z * 64;
-    const int Q = Cin * 16;
-    const int sel = l32 >> 4, d = l32 & 15;
-    const int64_t fbeg = (int64_t)blockIdx.x * facets_per_split;
-    const int64_t fend = (fbeg + facets_per_split < Nf) ? fbeg + facets_per_split : Nf;
-
-    f32x16 acc[8];
-#pragma unroll
-    for (int t = 0; t < 8; ++t)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) acc[t][i] = 0.f;
-    float g[8][4];
-#pragma unroll
-    for (int jj = 0; jj < 8; ++jj)
-#pragma unroll
-        for (int t = 0; t < 4; ++t) g[jj][t] = 0.f;
-
-    float4 rt[4], rs, rg;
-    int rseg0 = 0, rseg1 = 0;
-    auto fetch = [&](const XSlab &S) {
-        const int np = S.pb - S.pa;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int e = threadIdx.x + 512 * i, p = e >> 4, c4 = e & 15;
-            rt[i] = (p < np && cbase + 4 * c4 < Cin) ? xld4(tex + (int64_t)(S.pa + p) * Cin + cbase + 4 * c4)
-                                                    : make_float4(0.f, 0.f, 0.f, 0.f);
-        }
-        {
-            const int p = threadIdx.x >> 2, d4 = threadIdx.x & 3;
-            rs = (p < np) ? xld4(sh + (int64_t)(S.pa + p) * 16 + 4 * d4) : make_float4(0.f, 0.f, 0.f, 0.f);
-        }
-        rg = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (threadIdx.x < 256) {
-            const int fl = threadIdx.x >> 4, c4 = threadIdx.x & 15;
-            if (fl < S.n) {
-                const float *gp = gout + (int64_t)(S.fa + fl) * Cout + n0 + 4 * c4;
-                if ((Cout & 3) == 0 && n0 + 4 * c4 + 3 < Cout) rg = xld4(gp);
-                else {
-                    rg.x = (n0 + 4 * c4 < Cout) ? gp[0] : 0.f;
-                    rg.y = (n0 + 4 * c4 + 1 < Cout) ? gp[1] : 0.f;
-                    rg.z = (n0 + 4 * c4 + 2 < Cout) ? gp[2] : 0.f;
-                    rg.w = (n0 + 4 * c4 + 3 < Cout) ? gp[3] : 0.f;
-                }
-            }
-        }
-        if (threadIdx.x < kFFB) {
-            const bool on = threadIdx.x < S.n;
-            const int a = on ? xseg_start(cum, S.fa + threadIdx.x, T) : 0;
-            const int b = on ? xseg_start(cum, S.fa + threadIdx.x + 1, T) : 0;
-            rseg0 = a;
-            rseg1 = b > a ? b - a : 0;
-        }
-    };
-    auto publish = [&]() {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int e = threadIdx.x + 512 * i, p = e >> 4, c4 = e & 15;
-            *reinterpret_cast<float4 *>(tex_s + p * kFRow + 4 * c4) = rt[i];
-        }
-        *reinterpret_cast<float4 *>(sh_s + 4 * threadIdx.x) = rs;
-        if (threadIdx.x < 256) {
-            // gout[facet fl][4 channels] -> three bf16 pieces at [piece][co][fl]
-            const int fl = threadIdx.x >> 4, c4 = threadIdx.x & 15;
-            const float v[4] = {rg.x, rg.y, rg.z, rg.w};
-#pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                const float r1 = v[u] - trunc_bf16(v[u]), r2 = r1 - trunc_bf16(r1);
-                unsigned short *q = go_p + (4 * c4 + u) * kFFB + fl;
-                q[0] = (unsigned short)(fbits(v[u]) >> 16);
-                q[64 * kFFB] = (unsigned short)(fbits(r1) >> 16);
-                q[2 * 64 * kFFB] = (unsigned short)(fbits(r2) >> 16);
-            }
-        }
-        if (threadIdx.x < kFFB) {
-            seg_s[threadIdx.x] = rseg0;
-            seg_s[kFFB + threadIdx.x] = rseg1;
-        }
-    };
-
-    // descriptors: `cur` is in LDS, `nxt` is being fetched, the bounds of the one after are in flight
-    XSlab cur = slab_from_bounds(slab_bounds_load(cum, fbeg, fend, T, lane), fbeg, fend, -1, lane);
-    if (cur.n > 0) fetch(cur);
-    int64_t fa_n = cur.flush ? cur.fa + cur.n : cur.fa;
-    int cbounds = slab_bounds_load(cum, fa_n, fend, T, lane);
-    publish();
-    __syncthreads();
-    while (cur.n > 0) {
-        const XSlab nxt = slab_from_bounds(cbounds, fa_n, fend, cur.flush ? -1 : cur.pb, lane);
-        if (nxt.n > 0) fetch(nxt);
-        fa_n = nxt.flush ? nxt.fa + nxt.n : nxt.fa;
-        cbounds = slab_bounds_load(cum, fa_n, fend, T, lane);
-
-        // G values of my half's facets 8h + jj, channels cbase + 8w + 4*sel + t, SH index d: one 16-byte
-        // and one 4-byte LDS read per texture point
-#pragma unroll
-        for (int jj = 0; jj < 8; ++jj) {
-            const int fl = 8 * h + jj;
-            if (fl < cur.n) {
-                const int s = seg_s[fl], Kf = seg_s[kFFB + fl];
-                const float inv = Kf > 0 ? 1.0f / (float)Kf : 0.f;
-                const int r0 = s > cur.pa ? s : cur.pa, r1 = s + Kf < cur.pb ? s + Kf : cur.pb;
-                for (int r = r0; r < r1; r += 4) {
-                    float4 v[4];
-                    float sv[4];
-#pragma unroll
-                    for (int u = 0; u < 4; ++u) {
-                        const int p = (r + u < r1 ? r + u : r1 - 1) - cur.pa;
-                        v[u] = xld4(tex_s + p * kFRow + 8 * w + 4 * sel);
-                        sv[u] = (r + u < r1) ? sh_s[p * 16 + d] * inv : 0.f;
-                    }
-#pragma unroll
-                    for (int u = 0; u < 4; ++u) {
-                        g[jj][0] = fmaf(v[u].x, sv[u], g[jj][0]);
-                        g[jj][1] = fmaf(v[u].y, sv[u], g[jj][1]);
-                        g[jj][2] = fmaf(v[u].z, sv[u], g[jj][2]);
-                        g[jj][3] = fmaf(v[u].w, sv[u], g[jj][3]);
-                    }
-                }
-            }
-        }
-        if (cur.flush) {
-            // A pieces: gout^T of my k-group's eight facets, both 32-channel tiles of the slab of Cout
-            u32x4 ap[2][3];
-#pragma unroll
-            for (int mt = 0; mt < 2; ++mt)
-#pragma unroll
-                for (int p = 0; p < 3; ++p)
-                    ap[mt][p] = *reinterpret_cast<const u32x4 *>(go_p + (p * 64 + mt * 32 + l32) * kFFB + 8 * h);
-#pragma unroll
-            for (int t = 0; t < 4; ++t) {
-                float x[8];
-#pragma unroll
-                for (int jj = 0; jj < 8; ++jj) {
-                    x[jj] = g[jj][t];
-                    g[jj][t] = 0.f;
-                }
-                u32x4 bp[3];
-                split8(x, bp[0], bp[1], bp[2]);
-#pragma unroll
-                for (int term = 0; term < 6; ++term) {
-                    const int ia = term == 0 ? 2 : term == 1 ? 1 : term == 2 ? 0 : term == 3 ? 1 : 0;
-                    const int ib = term == 0 ? 0 : term == 1 ? 1 : term == 2 ? 2 : term == 3 ? 0 : term == 4 ? 1 : 0;
-                    acc[t] = mfma_bf16(ap[0][ia], bp[ib], acc[t]);
-                    acc[4 + t] = mfma_bf16(ap[1][ia], bp[ib], acc[4 + t]);
-                }
-            }
-        }
-        __syncthreads();
-        publish();
-        __syncthreads();
-        cur = nxt;
-    }
-
-    float *P = partial + (size_t)blockIdx.x * Cout * Q;
-    // column l32 of tile t is (channel cbase + 8w + 4*sel + t, SH index d)
-    const int cw = cbase + 8 * w + 4 * sel;
-#pragma unroll
-    for (int t = 0; t < 4; ++t) {
-        if (cw + t >= Cin) continue;
-        const int q = (cw + t) * 16 + d;
-#pragma unroll
-        for (int mt = 0; mt < 2; ++mt)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                const int co = n0 + mt * 32 + 8 * (i / 4) + 4 * h + (i % 4);
-                if (co < Cout) P[(size_t)co * Q + q] = acc[mt * 4 + t][i];
-            }
-    }
-}
-
-int f2f16x3_bwd_filter_partials(const float *gout, const float *tex, const float *sh, const int *cum, float *partial,
-                                int splits, int64_t T, int64_t Nf, int Cin, int Cout, hipStream_t st)
-{
-    const int64_t gy = ceil_div(Cin, 64), gz = ceil_div(Cout, 64);
-    PM_REQUIRE(gy <= 65535 && gz <= 65535, "f2f_bwd_filter: grid too large");
-    const int64_t fps = ceil_div(Nf, splits);
-    f2f16x3_bwd_filt_k<<<dim3((unsigned)splits, (unsigned)gy, (unsigned)gz), dim3(512), 0, st>>>(
-        gout, tex, sh, cum, partial, Nf, (int)T, Cin, Cout, fps);
-    PM_LAUNCHED("f2f_bwd_filter");
-    return 0;
-}
-
-// ----------------------------------------------------------------------------------------
-// filter gradient, second formulation: G is formed exactly as in the forward (lane = facet, eight
+// filter gradient gW = gout^T . G on the bf16 matrix cores: G is formed exactly as in the forward (lane = facet, eight
 // d's in registers, SH rows of the facet's points in registers), split into bf16 pieces, and each
 // piece is TRANSPOSED BY THE MATRIX CORE ITSELF: D = piece . E with a 0/1 selection matrix E is exact
 // and leaves, in the accumulator layout, lane = column (channel, d) and registers = facets -- the
@@ -888,6 +633,15 @@ __device__ __forceinline__ void x3_filt_pass(const float (&shr)[KW][8], const fl
             }
     };
 
+    // the gout^T operand stays in registers for the whole pass (it serves all eight channel pairs)
+    u32x4 g[2][2][3];
+#pragma unroll
+    for (int st = 0; st < 2; ++st)
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int p = 0; p < 3; ++p) g[st][t][p] = go[((st * 2 + t) * 3 + p) * 64 + lane];
+
     // software pipeline over the channel pairs: the G values of pair cp+1 are generated and split
     // (vector ALU) while the products of pair cp run on the matrix core
     u32x4 o[3][2];
@@ -902,11 +656,6 @@ __device__ __forceinline__ void x3_filt_pass(const float (&shr)[KW][8], const fl
         if (cp + 1 < 8) gen(pa, pb, cp + 1);
 #pragma unroll
         for (int st = 0; st < 2; ++st) {
-            u32x4 g[2][3];
-#pragma unroll
-            for (int t = 0; t < 2; ++t)
-#pragma unroll
-                for (int p = 0; p < 3; ++p) g[t][p] = go[((st * 2 + t) * 3 + p) * 64 + lane];
             // six piece products, smallest first; the two output tiles alternate so that no MFMA
             // waits for the one issued right before it
 #pragma unroll
@@ -914,7 +663,7 @@ __device__ __forceinline__ void x3_filt_pass(const float (&shr)[KW][8], const fl
                 const int ga = term == 0 ? 2 : term == 1 ? 1 : term == 2 ? 0 : term == 3 ? 1 : 0;
                 const int wb = term == 0 ? 0 : term == 1 ? 1 : term == 2 ? 2 : term == 3 ? 0 : term == 4 ? 1 : 0;
 #pragma unroll
-                for (int t = 0; t < 2; ++t) acc[cp][t] = mfma_bf16(o[ga][st], g[t][wb], acc[cp][t]);
+                for (int t = 0; t < 2; ++t) acc[cp][t] = mfma_bf16(o[ga][st], g[st][t][wb], acc[cp][t]);
             }
         }
         if (cp + 1 < 8) transpose(o, pa, pb);
@@ -981,6 +730,22 @@ __device__ __forceinline__ void xpre_commit(const XPre &P, u32x4 *go, float *shs
     }
 }
 
+// texture rows of one pass (KW points per facet) for my wavefront's 16 channels: 64 bytes per row,
+// four lanes per row
+template <int KW>
+__device__ __forceinline__ void xtex_issue(float4 (&pf)[2 * kXKB], const float *__restrict__ tex, const int *sk0,
+                                           const int *sK, int sweep, int cw, int Cin, int lane)
+{
+    const int piece = lane & 3;
+#pragma unroll
+    for (int i = 0; i < 2 * KW; ++i) {
+        const int rr = i * 16 + (lane >> 2), kk = rr >> 5, slot = rr & 31;
+        const bool ok = sweep * kXKB + kk < sK[slot] && cw + 4 * piece < Cin;
+        pf[i] = ok ? xld4(tex + (int64_t)(sk0[slot] + sweep * kXKB + kk) * Cin + cw + 4 * piece)
+                   : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+}
+
 __device__ __forceinline__ int xtile_kmax(const int *sK, int lane) { return xwave_max(sK[lane & 31]); }
 
 // One tile of 32 facets whose inputs are in LDS buffer it % 2 (descriptors in it % 3): start the
@@ -1033,16 +798,10 @@ __device__ __forceinline__ void x3_filt_tile(const float *__restrict__ gout, con
             }
         }
         {
-            // my wavefront's texture rows (16 channels = 64 bytes each), four lanes per row
+            // my wavefront's texture rows of this pass -> slab
+            float4 pf[2 * kXKB];
+            xtex_issue<KW>(pf, tex, s_k0[sb], s_K[sb], sw, cw, Cin, lane);
             const int piece = lane & 3;
-            float4 pf[2 * KW];
-#pragma unroll
-            for (int i = 0; i < 2 * KW; ++i) {
-                const int rr = i * 16 + (lane >> 2), kk = rr >> 5, slot = rr & 31;
-                const bool ok = sw * kXKB + kk < s_K[sb][slot] && cw + 4 * piece < Cin;
-                pf[i] = ok ? xld4(tex + (int64_t)(s_k0[sb][slot] + sw * kXKB + kk) * Cin + cw + 4 * piece)
-                           : make_float4(0.f, 0.f, 0.f, 0.f);
-            }
 #pragma unroll
             for (int i = 0; i < 2 * KW; ++i) {
                 const int rr = i * 16 + (lane >> 2), kk = rr >> 5, slot = rr & 31;
@@ -1059,7 +818,7 @@ __device__ __forceinline__ void x3_filt_tile(const float *__restrict__ gout, con
     __syncthreads();
 }
 
-__global__ __launch_bounds__(256, 1) void f2f16x3_bwd_filt2_k(const float *__restrict__ gout,
+__global__ __launch_bounds__(256, 1) void f2f16x3_bwd_filt_k(const float *__restrict__ gout,
                                                               const float *__restrict__ tex,
                                                               const float *__restrict__ sh,
                                                               const int *__restrict__ cum,
@@ -1146,13 +905,13 @@ __global__ __launch_bounds__(256, 1) void f2f16x3_bwd_filt2_k(const float *__res
         }
 }
 
-int f2f16x3_bwd_filter_partials2(const float *gout, const float *tex, const float *sh, const int *cum, const int *order,
+int f2f16x3_bwd_filter_partials(const float *gout, const float *tex, const float *sh, const int *cum, const int *order,
                                  float *partial, int splits, int64_t T, int64_t Nf, int Cin, int Cout, hipStream_t st)
 {
     const int64_t gy = ceil_div(Cin, 64), gz = ceil_div(Cout, 64);
     PM_REQUIRE(gy <= 65535 && gz <= 65535, "f2f_bwd_filter: grid too large");
     const int64_t ntiles = ceil_div(Nf, 32);
-    f2f16x3_bwd_filt2_k<<<dim3((unsigned)splits, (unsigned)gy, (unsigned)gz), dim3(256), 0, st>>>(
+    f2f16x3_bwd_filt_k<<<dim3((unsigned)splits, (unsigned)gy, (unsigned)gz), dim3(256), 0, st>>>(
         gout, tex, sh, cum, order, partial, Nf, (int)T, Cin, Cout, ntiles);
     PM_LAUNCHED("f2f_bwd_filter");
     return 0;

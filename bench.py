@@ -36,6 +36,9 @@ def parse():
     ap.add_argument("--workload", default="scene", choices=["scene", "shapes", "pool"])
     ap.add_argument("--scale", type=float, default=1.0, help="facet-count scale of the scene workload")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="after the timed region, copy a 1 GiB buffer three times (a kernel of known HBM traffic "
+                         "to scale rocprofv3's FETCH_SIZE / WRITE_SIZE counters by)")
     return ap.parse_args()
 
 
@@ -73,6 +76,13 @@ def conv_bytes_flops(d, ops):
         "f2f_bwd_filter": (4 * Nf * C + 4 * T * C + 4 * T * B + 4 * Nf + 4 * C * C * B, 2 * Nf * C * B * C + 2 * T * C * B),
     }
     return {k: tab[k] for k in ops}
+
+
+# HBM bytes per launch of the op's main kernel on the default scene workload (scale 1.0), measured with
+# rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE and scaled by what the same counters read for a 1 GiB copy
+# (--copy-calibration); reported as roofline.traffic when that workload runs.
+SCENE_TRAFFIC_BYTES = {"f2f_fwd": 4.646e9, "f2f_bwd_texture": 5.136e9, "f2f_bwd_filter": 3.365e9,
+                       "f2v_fwd": 2.046e9, "f2v_bwd": 2.020e9}
 
 
 class EventTimer:
@@ -168,7 +178,8 @@ def run_conv_layer(args, torch, kind):
         roof = dict(bound="mfma", achieved=bf[dom][1] / (dom_ms * 1e-3) / 1e12, peak=MFMA_F32_PEAK_TFLOPS, unit="TFLOP/s")
     else:
         roof = dict(bound="hbm", achieved=bf[dom][0] / (dom_ms * 1e-3) / 1e9, peak=HBM_PEAK_GBS, unit="GB/s")
-    roof.update(frac=roof["achieved"] / roof["peak"], traffic=None, kernel=dom, kernel_ms=dom_ms)
+    traffic = SCENE_TRAFFIC_BYTES.get(dom) if (kind == "scene" and args.scale == 1.0) else None
+    roof.update(frac=roof["achieved"] / roof["peak"], traffic=traffic, kernel=dom, kernel_ms=dom_ms)
     ops_report = {k: dict(ms=per_op.get(k), gbps=bf[k][0] / (per_op[k] * 1e-3) / 1e9,
                           tflops=bf[k][1] / (per_op[k] * 1e-3) / 1e12) for k in ops if k in per_op}
     res = dict(value=d["nf"] / (ms * 1e-3) / 1e6, ms_per_step=ms, roofline=roof, ops=ops_report,
@@ -180,35 +191,46 @@ def run_conv_layer(args, torch, kind):
     return res
 
 
-def cpu_baseline_conv(d, kind, torch):
-    """Vectorised oracle (float32) on the host cores over the first mesh of the batch only."""
+def cpu_baseline_conv(d, kind, torch, budget_s=12.0):
+    """Vectorised oracle (float32) on the host cores, mesh after mesh of the batch until `budget_s` is spent."""
     from oracle import torch_ref as R
     torch.set_num_threads(os.cpu_count() or 1)
-    nf, nv = int(d["mf_in"][0]), int(d["nv_in"][0])
-    T = int(d["counts"][:nf].sum())
-    f = torch.from_numpy(d["face"][:nf])
-    cum = torch.cumsum(torch.from_numpy(d["counts"][:nf]), 0, dtype=torch.int32)
-    bary = torch.from_numpy(d["bary"][:T])
-    x = torch.from_numpy(d["x"][:nv])
-    own = torch.from_numpy(d["owner"][:T])
-    corner = f.long()[own]
-    tex = x[corner[:, 0]] * bary[:, 0:1] + x[corner[:, 1]] * bary[:, 1:2] + x[corner[:, 2]] * bary[:, 2:3]
-    sh, coeff = R.sph_harm(bary, d["L"]), R.sph_harm(torch.from_numpy(d["normal"][:nf]), d["L"])
     w_f2f, w_f2v, w_v2f = (torch.from_numpy(d[k]) for k in ("w_f2f", "w_f2v", "w_v2f"))
-    vt_map, nfc = torch.from_numpy(d["vt_map"][:nv]), torch.from_numpy(d["nf_count"][:nv].astype(np.int32))
-    gy = torch.randn(nv, d["C"])
-    t0 = time.perf_counter()
-    y1 = R.f2f_fwd(tex, w_f2f, sh, cum)
-    if kind == "shapes":
-        y1 = y1 + R.v2f_fwd(x, w_v2f, f)
-    R.f2v_fwd(y1, w_f2v, coeff, f, nfc, vt_map)
-    g1, _ = R.f2v_bwd(gy, y1, w_f2v, coeff, f, nfc, vt_map)
-    R.f2f_bwd(g1, tex, w_f2f, sh, cum)
-    if kind == "shapes":
-        R.v2f_bwd(g1, x, w_v2f, f)
-    dt = time.perf_counter() - t0
-    return dict(value=nf / dt / 1e6, unit="Mfacets/s", cores=torch.get_num_threads(), kind="port",
-                sample="first mesh of the batch (%d facets, %d texture points), one pass, %.1f s" % (nf, T, dt))
+    f_off = np.concatenate([[0], np.cumsum(d["mf_in"])]).astype(np.int64)
+    v_off = np.concatenate([[0], np.cumsum(d["nv_in"])]).astype(np.int64)
+    t_off = np.concatenate([[0], np.cumsum(d["counts"])]).astype(np.int64)[f_off]
+    done_f = done_t = n_mesh = 0
+    spent = 0.0
+    for m in range(len(d["mf_in"])):
+        fa, fb, va, vb, ta, tb = f_off[m], f_off[m + 1], v_off[m], v_off[m + 1], t_off[m], t_off[m + 1]
+        nf, nv = int(fb - fa), int(vb - va)
+        f = torch.from_numpy(d["face"][fa:fb] - int(va))
+        cum = torch.cumsum(torch.from_numpy(d["counts"][fa:fb]), 0, dtype=torch.int32)
+        bary = torch.from_numpy(d["bary"][ta:tb])
+        x = torch.from_numpy(d["x"][va:vb])
+        own = torch.from_numpy(d["owner"][ta:tb] - int(fa))
+        corner = f.long()[own]
+        tex = x[corner[:, 0]] * bary[:, 0:1] + x[corner[:, 1]] * bary[:, 1:2] + x[corner[:, 2]] * bary[:, 2:3]
+        sh, coeff = R.sph_harm(bary, d["L"]), R.sph_harm(torch.from_numpy(d["normal"][fa:fb]), d["L"])
+        vt_map = torch.arange(nv, dtype=torch.int32)
+        nfc = torch.from_numpy(d["nf_count"][va:vb].astype(np.int32))
+        gy = torch.randn(nv, d["C"])
+        t0 = time.perf_counter()
+        y1 = R.f2f_fwd(tex, w_f2f, sh, cum)
+        if kind == "shapes":
+            y1 = y1 + R.v2f_fwd(x, w_v2f, f)
+        R.f2v_fwd(y1, w_f2v, coeff, f, nfc, vt_map)
+        g1, _ = R.f2v_bwd(gy, y1, w_f2v, coeff, f, nfc, vt_map)
+        R.f2f_bwd(g1, tex, w_f2f, sh, cum)
+        if kind == "shapes":
+            R.v2f_bwd(g1, x, w_v2f, f)
+        spent += time.perf_counter() - t0
+        done_f, done_t, n_mesh = done_f + nf, done_t + int(tb - ta), n_mesh + 1
+        if spent >= budget_s:
+            break
+    return dict(value=done_f / spent / 1e6, unit="Mfacets/s", cores=torch.get_num_threads(), kind="port",
+                sample="first %d of %d meshes of the batch (%d facets, %d texture points), one fwd+bwd pass each, %.1f s"
+                       % (n_mesh, len(d["mf_in"]), done_f, done_t, spent))
 
 
 def run_pool(args, torch):
@@ -274,6 +296,13 @@ def main():
         sys.exit(2)
     torch.cuda.set_device(0)
     res = run_pool(args, torch) if args.workload == "pool" else run_conv_layer(args, torch, args.workload)
+    if args.copy_calibration:
+        src = torch.empty(1 << 28, dtype=torch.float32, device="cuda:0").normal_()
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     line = dict(metric="mesh-conv layer fwd+bwd throughput", value=res.pop("value"), unit=res.pop("unit", "Mfacets/s"),
                 n_gpus=1, steps=args.steps, warmup=args.warmup, ms_per_step=res.pop("ms_per_step"),
                 higher_is_better=True, scaling="weak", vs_baseline=None, dtype="f32", data="synthetic")

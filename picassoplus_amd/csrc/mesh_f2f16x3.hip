@@ -411,8 +411,9 @@ __global__ __launch_bounds__(kBlock) void f2f16x3_pack_filter_t_k(const float *_
 
 template <int KW>
 __device__ __forceinline__ void x3_tex_sweep(const u32x4 *__restrict__ WpT, const float *__restrict__ sh,
-                                             float *__restrict__ gtex, u32x4 *Ws, const u32x4 (&bp)[kTKS][3],
-                                             int kbase, int Ks, float invK, int Cin, int NKS, int NG, int lane, int h)
+                                             float *__restrict__ gtex, u32x4 *Ws, float *stage, const int *w_k0,
+                                             const int *w_K, const u32x4 (&bp)[kTKS][3], int kbase, int Ks, float invK,
+                                             int sweep, int Cin, int NKS, int NG, int lane, int h)
 {
     // SH rows of my facet's points, pre-scaled by 1/K
     float shr[KW][16];
@@ -449,6 +450,20 @@ __device__ __forceinline__ void x3_tex_sweep(const u32x4 *__restrict__ WpT, cons
     chunk_publish(wn, 1);
     __syncthreads();
 
+    // 16-channel block gp of the stage -> global memory
+    auto flush = [&](int gp) {
+        const int ci = 16 * gp + 4 * (lane & 3);
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const int slot = 16 * i + (lane >> 2);
+            const int k0s = w_k0[slot] + sweep * kXKB, Kss = w_K[slot] - sweep * kXKB;
+#pragma unroll
+            for (int kk = 0; kk < KW; ++kk)
+                if (kk < Kss && ci < Cin)
+                    *reinterpret_cast<float4 *>(gtex + (int64_t)(k0s + kk) * Cin + ci) =
+                        *reinterpret_cast<const float4 *>(stage + (kk * 32 + slot) * 16 + 4 * (lane & 3));
+        }
+    };
     for (int g = 0; g < NG; ++g) {
         float gacc[KW][4];
 #pragma unroll
@@ -494,14 +509,14 @@ __device__ __forceinline__ void x3_tex_sweep(const u32x4 *__restrict__ WpT, cons
             if (more) chunk_publish(wn, c + 2);
             __syncthreads();
         }
-        const int ci0 = 8 * g + 4 * h;
-        if (ci0 < Cin) {
+        // Results go out 64 bytes at a time: two groups (16 channels) of every point are collected in
+        // the wavefront's LDS stage [point][facet slot][16 channels], then four lanes write one
+        // 64-byte piece of a row (32-byte pieces cost almost twice the HBM write traffic).
 #pragma unroll
-            for (int kk = 0; kk < KW; ++kk)
-                if (kk < Ks)
-                    *reinterpret_cast<float4 *>(gtex + (int64_t)(kbase + kk) * Cin + ci0) =
-                        make_float4(gacc[kk][0], gacc[kk][1], gacc[kk][2], gacc[kk][3]);
-        }
+        for (int kk = 0; kk < KW; ++kk)
+            *reinterpret_cast<float4 *>(stage + (kk * 32 + (lane & 31)) * 16 + (g & 1) * 8 + 4 * h) =
+                make_float4(gacc[kk][0], gacc[kk][1], gacc[kk][2], gacc[kk][3]);
+        if ((g & 1) || g == NG - 1) flush(g >> 1);
     }
 }
 
@@ -513,7 +528,8 @@ __global__ __launch_bounds__(512, 2) void f2f16x3_bwd_tex_k(const float *__restr
                                                             int64_t Nf, int T, int Cin, int Cout, int NKS, int NG)
 {
     __shared__ u32x4 Ws[3 * kTChunkMax];
-    __shared__ int s_kmax;
+    __shared__ __attribute__((aligned(16))) float s_stage[8][kXKB * 32 * 16];
+    __shared__ int s_k0[8][32], s_K[8][32], s_kmax;
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
     const int l32 = lane & 31, h = lane >> 5;
     if (threadIdx.x == 0) s_kmax = 0;
@@ -530,6 +546,10 @@ __global__ __launch_bounds__(512, 2) void f2f16x3_bwd_tex_k(const float *__restr
         K = b > a ? b - a : 0;
     }
     const float invK = K > 0 ? 1.0f / (float)K : 0.f;
+    if (h == 0) {
+        s_k0[w][l32] = k0;
+        s_K[w][l32] = K;
+    }
     {
         const int km = xwave_max(K);
         if (lane == 0) atomicMax(&s_kmax, km);
@@ -557,7 +577,7 @@ __global__ __launch_bounds__(512, 2) void f2f16x3_bwd_tex_k(const float *__restr
         const int kw = xwave_max(Ks);
         const int kbase = k0 + sw * kXKB;
         // every variant runs the same barriers, so wavefronts of a workgroup may pick different ones
-#define PM_X3T(N) x3_tex_sweep<N>(WpT, sh, gtex, Ws, bp, kbase, Ks, invK, Cin, NKS, NG, lane, h)
+#define PM_X3T(N) x3_tex_sweep<N>(WpT, sh, gtex, Ws, s_stage[w], s_k0[w], s_K[w], bp, kbase, Ks, invK, sw, Cin, NKS, NG, lane, h)
         if (kw <= 1) PM_X3T(1);
         else if (kw == 2) PM_X3T(2);
         else if (kw == 3) PM_X3T(3);

@@ -49,20 +49,26 @@ __device__ __forceinline__ void block_reduce_store(const Pack<V> &acc, float *re
     __syncthreads();
 }
 
-// out[o] = sum_g partial[g*n + o], g ascending within four interleaved slices, slices added
-// in order.  One workgroup covers 64 outputs.
-__global__ __launch_bounds__(kBlock) void reduce_partials_k(const float *__restrict__ partial,
-                                                            float *__restrict__ out, int G, int n)
+// out[o] = sum_g partial[g*n + o]: 64 interleaved slices of g (ascending within a slice), then the
+// slices in a fixed tree order.  One workgroup of 1024 threads covers 16 outputs, so that the few
+// thousand outputs of a filter gradient still spread over the chip.
+__global__ __launch_bounds__(1024) void reduce_partials_k(const float *__restrict__ partial,
+                                                         float *__restrict__ out, int G, int n)
 {
-    __shared__ float red[4][64];
-    const int j = threadIdx.x & 63, s = threadIdx.x >> 6;
-    const int o = blockIdx.x * 64 + j;
+    __shared__ float red[64][16];
+    const int j = threadIdx.x & 15, s = threadIdx.x >> 4;
+    const int o = blockIdx.x * 16 + j;
     float sum = 0.f;
     if (o < n)
-        for (int g = s; g < G; g += 4) sum += partial[(size_t)g * n + o];
+        for (int g = s; g < G; g += 64) sum += partial[(size_t)g * n + o];
     red[s][j] = sum;
     __syncthreads();
-    if (s == 0 && o < n) out[o] = ((red[0][j] + red[1][j]) + red[2][j]) + red[3][j];
+#pragma unroll
+    for (int half = 32; half > 0; half >>= 1) {
+        if (s < half) red[s][j] += red[s + half][j];
+        __syncthreads();
+    }
+    if (s == 0 && o < n) out[o] = red[0][j];
 }
 
 __global__ __launch_bounds__(kBlock) void fill_zero_k(float *__restrict__ p, int64_t n)
@@ -693,7 +699,7 @@ static inline int pick_v(int C, int r, std::initializer_list<const void *> ptrs)
 
 static int reduce_partials(const float *partial, float *out, int G, int n, hipStream_t st)
 {
-    reduce_partials_k<<<dim3((unsigned)ceil_div(n, 64)), dim3(kBlock), 0, st>>>(partial, out, G, n);
+    reduce_partials_k<<<dim3((unsigned)ceil_div(n, 16)), dim3(1024), 0, st>>>(partial, out, G, n);
     PM_LAUNCHED("reduce_partials");
     return 0;
 }

@@ -1,0 +1,182 @@
+"""GPU checks at the benchmark's full sizes through properties that do not need a full CPU oracle run:
+adjoint identities (each op is linear in its features and in its filter), oracle parity on a random
+sample of facets, invariance under the optional facet order, and the pooling invariants."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import loops
+from picassoplus_amd import _lib, synthetic as S
+from picassoplus_amd.mesh import topology
+from picassoplus_amd.mesh.layers import sph_harm_values
+from picassoplus_amd.mesh.pi_modules import conv3d, mesh_conv3d, pool3d, unpool3d
+from util import assert_close, dev
+
+pytestmark = pytest.mark.gpu
+
+
+def say(*a):
+    print(*a, flush=True)
+
+
+def _dot(a, b):
+    return float((a.double() * b.double()).sum())
+
+
+def _adjoint_ok(lhs, rhs, scale, what, tol=1e-5):
+    assert abs(lhs - rhs) <= tol * scale, "%s: %.9g vs %.9g (scale %.3g)" % (what, lhs, rhs, scale)
+
+
+@pytest.fixture(scope="module")
+def scene(cuda):
+    """The bench's scene batch: 8 rooms, about 2.4 M facets, area-scaled texture counts 1..9, C = 64."""
+    say("building the scene workload")
+    rng = np.random.default_rng(3000)
+    mesh = S.scene_workload(seed=3000, n_rooms=8, scale=1.0)
+    v, f = mesh["vertex"], mesh["face"]
+    nv, nf = v.shape[0], f.shape[0]
+    normal, area = S.triangle_normals_areas(v, f)
+    counts, bary, owner = S.texture_points(rng, nf, S.area_scaled_texture_counts(area))
+    C, L = 64, 3
+    d = dict(nv=nv, nf=nf, T=int(counts.sum()), C=C, counts=counts)
+    d["face"] = dev(f, cuda)
+    d["cum"] = torch.cumsum(dev(counts, cuda), 0, dtype=torch.int32)
+    d["sh"] = sph_harm_values(dev(bary.astype(np.float32), cuda), L)
+    d["coeff"] = sph_harm_values(dev(normal.astype(np.float32), cuda), L)
+    d["tex"] = dev(rng.uniform(-1, 1, (d["T"], C)).astype(np.float32), cuda)
+    d["w_f2f"] = dev(S.xavier_uniform(rng, (C, C, 16), C * 16, C * 16).astype(np.float32), cuda)
+    d["w_f2v"] = dev(S.xavier_uniform(rng, (16, C, 1), C, 16 * C).astype(np.float32), cuda)
+    d["nfc"] = dev(np.maximum(S.vertex_facet_count(f, np.arange(nv), nv), 1).astype(np.int32), cuda)
+    d["vt_map"] = dev(np.arange(nv, dtype=np.int32), cuda)
+    return d
+
+
+def test_f2f_full_size_adjoints_and_sample_parity(cuda, scene):
+    d = scene
+    say("case f2f full size", d["nf"], d["T"])
+    gen = torch.Generator(device=cuda).manual_seed(5)
+    g = torch.randn(d["nf"], d["C"], device=cuda, generator=gen)
+    tex = d["tex"].clone().requires_grad_(True)
+    w = d["w_f2f"].clone().requires_grad_(True)
+    out = conv3d.facet2facet(tex, w, d["sh"], d["cum"])
+    gtex, gw = torch.autograd.grad(out, [tex, w], g)
+    torch.cuda.synchronize()
+    lhs = _dot(out, g)
+    scale = float(out.double().norm() * g.double().norm())
+    _adjoint_ok(lhs, _dot(tex, gtex), scale, "<f2f(tex), g> = <tex, grad_texture>")
+    _adjoint_ok(lhs, _dot(w, gw), scale, "<f2f(tex), g> = <W, grad_filter>")
+
+    # oracle parity on a sample of facets: outputs and texture gradients of a facet depend on that facet only
+    rng = np.random.default_rng(6)
+    pick = np.sort(rng.choice(d["nf"], 1500, replace=False))
+    counts = d["counts"]
+    start = np.concatenate([[0], np.cumsum(counts)])[:-1]
+    rows = np.concatenate([np.arange(start[f], start[f] + counts[f]) for f in pick]).astype(np.int64)
+    rows_t = torch.from_numpy(rows).to(cuda)
+    sub_tex = d["tex"][rows_t].cpu().numpy().astype(np.float64)
+    sub_sh = d["sh"][rows_t].cpu().numpy().astype(np.float64)
+    sub_cum = np.cumsum(counts[pick]).astype(np.int32)
+    wt = d["w_f2f"].cpu().numpy().astype(np.float64)
+    pick_t = torch.from_numpy(pick).to(cuda)
+    sub_g = g[pick_t].cpu().numpy().astype(np.float64)
+    ref_out = loops.f2f_fwd(sub_tex, wt, sub_sh, sub_cum)
+    ref_gtex, _ = loops.f2f_bwd(sub_g, sub_tex, wt, sub_sh, sub_cum)
+    assert_close(out.detach()[pick_t], ref_out, "f2f out (sampled facets)")
+    assert_close(gtex[rows_t], ref_gtex, "f2f grad_texture (sampled facets)")
+
+    # the facet order is an optimisation only: per-facet results do not change by a bit
+    T, Cin = d["tex"].shape
+    ws_n = _lib.query("pmesh_f2f_fwd_workspace_bytes", Cin, d["C"], 16)
+    ws = torch.empty(ws_n, dtype=torch.uint8, device=cuda)
+    out2 = torch.empty_like(out)
+    _lib.call("pmesh_f2f_fwd", d["tex"].data_ptr(), d["w_f2f"].data_ptr(), d["sh"].data_ptr(), d["cum"].data_ptr(),
+              None, out2.data_ptr(), ws.data_ptr(), ws_n, T, d["nf"], Cin, d["C"], 16,
+              torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    assert torch.equal(out2, out.detach())
+
+
+def test_f2v_full_size_adjoints(cuda, scene):
+    d = scene
+    say("case f2v full size", d["nf"], d["nv"])
+    gen = torch.Generator(device=cuda).manual_seed(7)
+    x = torch.randn(d["nf"], d["C"], device=cuda, generator=gen).requires_grad_(True)
+    w = d["w_f2v"].clone().requires_grad_(True)
+    g = torch.randn(d["nv"], d["C"], device=cuda, generator=gen)
+    out = conv3d.facet2vertex(x, w, d["coeff"], d["face"], d["nfc"], d["vt_map"])
+    gx, gw = torch.autograd.grad(out, [x, w], g)
+    torch.cuda.synchronize()
+    lhs = _dot(out, g)
+    scale = float(out.double().norm() * g.double().norm())
+    _adjoint_ok(lhs, _dot(x, gx), scale, "<f2v(x), g> = <x, grad_input>")
+    _adjoint_ok(lhs, _dot(w, gw), scale, "<f2v(x), g> = <filter, grad_filter>")
+    # a constant field with unit coefficient 0 and all other coefficients zero is averaged to itself
+    coeff = torch.zeros_like(d["coeff"])
+    coeff[:, 0] = 1.0
+    w1 = torch.zeros_like(d["w_f2v"])
+    w1[0] = 1.0
+    ones = torch.full((d["nf"], d["C"]), 0.75, device=cuda)
+    y = mesh_conv3d.facet2vertex_forward(ones, w1, coeff, d["face"], d["nfc"], d["vt_map"])
+    torch.cuda.synchronize()
+    touched = torch.zeros(d["nv"], dtype=torch.bool, device=cuda)
+    touched[d["face"].long().reshape(-1)] = True
+    assert float((y[touched] - 0.75).abs().max()) <= 1e-6
+
+
+def test_v2f_full_size_adjoints(cuda, scene):
+    d = scene
+    gen = torch.Generator(device=cuda).manual_seed(8)
+    x = torch.randn(d["nv"], d["C"], device=cuda, generator=gen).requires_grad_(True)
+    w = torch.randn(3, d["C"], 1, device=cuda, generator=gen).requires_grad_(True)
+    g = torch.randn(d["nf"], d["C"], device=cuda, generator=gen)
+    out = conv3d.vertex2facet(x, w, d["face"])
+    gx, gw = torch.autograd.grad(out, [x, w], g)
+    torch.cuda.synchronize()
+    lhs = _dot(out, g)
+    scale = float(out.double().norm() * g.double().norm())
+    _adjoint_ok(lhs, _dot(x, gx), scale, "<v2f(x), g> = <x, grad_input>")
+    _adjoint_ok(lhs, _dot(w, gw), scale, "<v2f(x), g> = <filter, grad_filter>")
+
+
+def test_pool_full_size_invariants(cuda):
+    """1024 x 1024 grid, about 261 k clusters of 1..12 vertices, C = 128."""
+    say("case pool full size")
+    nv, C = 1024 * 1024, 128
+    rng = np.random.default_rng(4000)
+    vt_replace, vt_map, nvo = S.cluster_maps(rng, nv, mean=4.0, lo=1, hi=12, spatial=True)
+    vr, vm = dev(vt_replace, cuda), dev(vt_map, cuda)
+    gen = torch.Generator(device=cuda).manual_seed(9)
+    x = torch.randn(nv, C, device=cuda, generator=gen).requires_grad_(True)
+    vt_out = torch.zeros(nvo, 3, device=cuda)
+    g = torch.randn(nvo, C, device=cuda, generator=gen)
+    # cluster id of every fine vertex, from the maps' definition
+    rep = torch.where(vr < 0, -vr, torch.arange(nv, device=cuda, dtype=torch.int32)).long()
+    cl = vm.long()[rep]
+    assert int(cl.min()) >= 0 and int(cl.max()) == nvo - 1
+
+    y = pool3d.maxPool(x, vr, vm, vt_out)
+    (gx,) = torch.autograd.grad(y, x, g)
+    ref = torch.full((nvo, C), -float("inf"), device=cuda).scatter_reduce(0, cl[:, None].expand(-1, C), x.detach(), "amax")
+    assert torch.equal(y.detach(), ref)                                     # max values are exact
+    assert abs(_dot(gx, torch.ones_like(gx)) - _dot(g, torch.ones_like(g))) <= 1e-6 * float(g.double().abs().sum())
+    # every gradient entry sits at a maximum of its cluster
+    nz = gx != 0
+    assert torch.equal(x.detach()[nz], ref[cl][nz])
+
+    ya = pool3d.avgPool(x, vr, vm, vt_out)
+    (gxa,) = torch.autograd.grad(ya, x, g)
+    cnt = torch.zeros(nvo, device=cuda).index_add_(0, cl, torch.ones(nv, device=cuda))
+    ref_a = torch.zeros(nvo, C, device=cuda, dtype=torch.float64).index_add_(0, cl, x.detach().double()) / cnt[:, None]
+    assert float((ya.detach().double() - ref_a).abs().max()) <= 1e-5 * float(ref_a.abs().max())
+    assert float((gxa - g[cl] / cnt[cl][:, None]).abs().max()) <= 1e-6 * float(g.abs().max())
+
+    c = ya.detach().clone().requires_grad_(True)
+    u = unpool3d.interpolate(c, vr, vm)
+    gf = torch.randn(nv, C, device=cuda, generator=gen)
+    (gc,) = torch.autograd.grad(u, c, gf)
+    assert torch.equal(u.detach(), c.detach()[cl])                          # unpool copies
+    back = pool3d.avgPool(u.detach(), vr, vm, vt_out)                      # avg_pool(unpool(y)) = y
+    assert float((back - c.detach()).abs().max()) <= 2e-6 * float(c.detach().abs().max())
+    ref_gc = torch.zeros(nvo, C, device=cuda, dtype=torch.float64).index_add_(0, cl, gf.double())
+    assert float((gc.double() - ref_gc).abs().max()) <= 1e-5 * float(ref_gc.abs().max())
+    torch.cuda.synchronize()

@@ -128,7 +128,9 @@ int pmesh_f2f_fwd(const float *texture, const float *filter, const float *bary_c
 /* grad_texture (T,Cin), grad_filter (Cout,Cin,F).
  * workspace: pmesh_f2f_bwd_workspace_bytes(Cin,Cout,F), 16-byte aligned; the two halves may share
  * it when they run on the same stream.  facet_order: NULL or the permutation of
- * pmesh_build_facet_order, as for the forward.  Every row of grad_texture is written
+ * pmesh_build_facet_order, as for the forward (grad_texture is bit-identical with and without
+ * it; grad_filter sums the facets in the order given, so its last bits depend on it, and on
+ * nothing else).  Every row of grad_texture is written
  * (rows past the last facet's segment are cleared) provided cum_texture is non-decreasing.
  * pmesh_f2f_bwd is the texture half followed by the filter half; each half can be called
  * alone when only one gradient is wanted (the reference always computes both,

@@ -248,8 +248,10 @@ __device__ __forceinline__ void fma_bcast16(float cf, const Pack<4> (&fl)[16], P
 #undef PM_B
 }
 
-// facet2vertex forward for r = 1, C % 64 == 0 (row groups are whole 16-lane DPP rows): the entries
-// of an output vertex are processed eight at a time, all their gathers issued before any use.
+// facet2vertex forward for r = 1, C % 64 == 0 (row groups are whole 16-lane DPP rows), K <= 16.
+// Persistent row groups: the filter stays in registers for all the vertices a group visits, and three
+// stages of gathers are in flight at once -- the row bounds of the vertex after next, the entry list of
+// the next vertex, and the facet rows / coefficients of the current one (eight entries at a time).
 __global__ __launch_bounds__(kBlock) void f2v_fwd_fast_k(const float *__restrict__ in, const float *__restrict__ filt,
                                                          const float *__restrict__ coeff,
                                                          const int *__restrict__ nfcount,
@@ -258,29 +260,45 @@ __global__ __launch_bounds__(kBlock) void f2v_fwd_fast_k(const float *__restrict
                                                          int64_t NvOut, int C, int K, int lpr_log2)
 {
     constexpr int EB = 8;
-    const int lpr = 1 << lpr_log2;
+    const int lpr = 1 << lpr_log2, rpb = kBlock >> lpr_log2;
     const int lane = threadIdx.x & (lpr - 1), slot = threadIdx.x >> lpr_log2, l16 = threadIdx.x & 15;
-    const int64_t row = (int64_t)blockIdx.x * (kBlock >> lpr_log2) + slot;
-    if (row >= NvOut) return;
-    const int e0 = rowptr[row], e1 = rowptr[row + 1];
-    const float inv = (e1 > e0) ? 1.0f / (float)nfcount[row] : 0.f;
     const int c = lane * 4;
-    Pack<4> acc = zero_pack<4>();
-    for (int k0 = 0; k0 < K; k0 += 16) {
-        Pack<4> fl[16];
+    const bool kok = l16 < K;
+    Pack<4> fl[16];
 #pragma unroll
-        for (int k = 0; k < 16; ++k) fl[k] = (k0 + k < K) ? ldp<4>(filt + (size_t)(k0 + k) * C + c) : zero_pack<4>();
-        const bool kok = k0 + l16 < K;
+    for (int k = 0; k < 16; ++k) fl[k] = (k < K) ? ldp<4>(filt + (size_t)k * C + c) : zero_pack<4>();
+
+    const int64_t stride = (int64_t)gridDim.x * rpb;
+    int64_t row = (int64_t)blockIdx.x * rpb + slot;
+    // stage 1 (row bounds) of rows `row` and `row + stride`, stage 2 (entries) of `row`
+    int e0 = 0, e1 = 0, ne0 = 0, ne1 = 0;
+    if (row < NvOut) { e0 = rowptr[row]; e1 = rowptr[row + 1]; }
+    if (row + stride < NvOut) { ne0 = rowptr[row + stride]; ne1 = rowptr[row + stride + 1]; }
+    int f[EB];
+#pragma unroll
+    for (int i = 0; i < EB; ++i) f[i] = (e0 + i < e1) ? colidx[e0 + i] / 3 : -1;
+
+    for (; row < NvOut; row += stride) {
+        // row bounds two rows ahead, entry list one row ahead
+        int me0 = 0, me1 = 0;
+        if (row + 2 * stride < NvOut) { me0 = rowptr[row + 2 * stride]; me1 = rowptr[row + 2 * stride + 1]; }
+        int nf[EB];
+#pragma unroll
+        for (int i = 0; i < EB; ++i) nf[i] = (ne0 + i < ne1) ? colidx[ne0 + i] / 3 : -1;
+        const float inv = (e1 > e0) ? 1.0f / (float)nfcount[row] : 0.f;
+
+        Pack<4> acc = zero_pack<4>();
         for (int eb = e0; eb < e1; eb += EB) {
-            int64_t f[EB];
+            if (eb > e0) {                                   // vertices with more than eight entries
 #pragma unroll
-            for (int i = 0; i < EB; ++i) f[i] = (eb + i < e1) ? colidx[eb + i] / 3 : -1;
+                for (int i = 0; i < EB; ++i) f[i] = (eb + i < e1) ? colidx[eb + i] / 3 : -1;
+            }
             Pack<4> x[EB];
             float cf[EB];
 #pragma unroll
             for (int i = 0; i < EB; ++i) {
-                x[i] = (f[i] >= 0) ? ldp<4>(in + f[i] * C + c) : zero_pack<4>();
-                cf[i] = (f[i] >= 0 && kok) ? coeff[f[i] * K + k0 + l16] : 0.f;
+                x[i] = (f[i] >= 0) ? ldp<4>(in + (int64_t)f[i] * C + c) : zero_pack<4>();
+                cf[i] = (f[i] >= 0 && kok) ? coeff[(int64_t)f[i] * K + l16] : 0.f;
             }
 #pragma unroll
             for (int i = 0; i < EB; ++i) {
@@ -292,10 +310,13 @@ __global__ __launch_bounds__(kBlock) void f2v_fwd_fast_k(const float *__restrict
                 }
             }
         }
-    }
 #pragma unroll
-    for (int u = 0; u < 4; ++u) acc.v[u] *= inv;
-    stp<4>(out + row * C + c, acc);
+        for (int u = 0; u < 4; ++u) acc.v[u] *= inv;
+        stp<4>(out + row * C + c, acc);
+        e0 = ne0; e1 = ne1; ne0 = me0; ne1 = me1;
+#pragma unroll
+        for (int i = 0; i < EB; ++i) f[i] = nf[i];
+    }
 }
 
 // ----------------------------------------------------------------------------------------
@@ -787,8 +808,11 @@ extern "C" int pmesh_f2v_fwd(const float *input, const float *filter, const floa
     const int64_t blocks = ceil_div(NvOut, rs.rpb);
     PM_REQUIRE(grid_ok(blocks), "f2v_fwd: grid too large");
     const int cvec = ((K & 3) == 0 && aligned16(coeff)) ? 1 : 0;
-    if (V == 4 && (C & 63) == 0 && C <= 1024)
-        f2v_fwd_fast_k<<<dim3((unsigned)blocks), dim3(kBlock), 0, st>>>(input, filter, coeff, nf_count, rowptr, colidx, output, NvOut, C, K, rs.lpr_log2);
+    if (V == 4 && (C & 63) == 0 && C <= 1024 && K <= 16) {
+        // persistent: enough workgroups to fill the chip several times over, each visiting many vertices
+        const int64_t pb = blocks < 4096 ? blocks : 4096;
+        f2v_fwd_fast_k<<<dim3((unsigned)pb), dim3(kBlock), 0, st>>>(input, filter, coeff, nf_count, rowptr, colidx, output, NvOut, C, K, rs.lpr_log2);
+    }
     else if (V == 4)
         f2v_fwd_k<4><<<dim3((unsigned)blocks), dim3(kBlock), 0, st>>>(input, filter, coeff, nf_count, rowptr, colidx, output, NvOut, C, r, K, rs.items, rs.lpr_log2, cvec);
     else

@@ -148,13 +148,15 @@ def test_f2v_unit_count_is_plain_scatter(cuda):
                                                 (333, 16, 96, 16, 4), (70, 5, 7, 9, 3), (65, 4, 6, 36, 2),
                                                 (64, 3, 5, 50, 2), (129, 130, 64, 4, 3), (50, 8, 8, 1, 2),
                                                 (300, 8, 40, 16, 14), (1000, 64, 64, 16, 9), (130, 4, 130, 16, 20)])
-@pytest.mark.parametrize("generic", [False, True])
-def test_f2f_parity(cuda, monkeypatch, nf, Cin, Cout, F, kmax, generic):
-    """``generic`` forces the shape-generic kernels also where the 16-coefficient fast path applies."""
-    say("case f2f", nf, Cin, Cout, F, kmax, generic)
-    if generic and not (F == 16 and Cin % 4 == 0):
+@pytest.mark.parametrize("path", ["default", "generic", "fp32mfma"])
+def test_f2f_parity(cuda, monkeypatch, nf, Cin, Cout, F, kmax, path):
+    """``generic`` forces the shape-generic kernels and ``fp32mfma`` the fp32-matrix-instruction variant
+    of the 16-coefficient path, also where the split-bf16 kernels apply."""
+    say("case f2f", nf, Cin, Cout, F, kmax, path)
+    if path != "default" and not (F == 16 and Cin % 4 == 0):
         pytest.skip("shape already runs the generic kernels")
-    monkeypatch.setenv("PMESH_F2F_GENERIC", "1" if generic else "0")
+    monkeypatch.setenv("PMESH_F2F_GENERIC", "1" if path == "generic" else "0")
+    monkeypatch.setenv("PMESH_F2F_FP32MFMA", "1" if path == "fp32mfma" else "0")
     rng = np.random.default_rng(13)
     counts, bary, owner = texture_case(rng, nf, kmax)
     cum = np.cumsum(counts).astype(np.int32)
@@ -173,6 +175,38 @@ def test_f2f_parity(cuda, monkeypatch, nf, Cin, Cout, F, kmax, generic):
     assert_close(out, out_ref, "f2f out")
     assert_close(tt.grad, gin_ref, "f2f grad_texture")
     assert_close(ft.grad, gfilt_ref, "f2f grad_filter")
+
+
+def test_f2f_shape_sweep(cuda):
+    """Seeded sweep over channel counts, facet counts and point counts around the tile sizes of the
+    16-coefficient kernels (32-facet wavefront tiles, 4/8/16-channel groups, 64-channel blocks)."""
+    rng = np.random.default_rng(77)
+    cins = [4, 8, 12, 20, 36, 64, 68, 132]
+    couts = [8, 16, 24, 40, 64, 72, 128, 5]
+    nfs = [1, 31, 32, 33, 255, 257, 700]
+    kmaxs = [1, 2, 4, 5, 9, 13]
+    for it in range(28):
+        Cin, Cout = cins[it % len(cins)], couts[(it * 3 + 1) % len(couts)]
+        nf, kmax = nfs[(it * 5 + 2) % len(nfs)], kmaxs[(it * 7 + 3) % len(kmaxs)]
+        say("case f2f sweep", it, nf, Cin, Cout, kmax)
+        counts, bary, owner = texture_case(rng, nf, kmax, empty_frac=0.1 if nf > 1 else 0.0)
+        cum = np.cumsum(counts).astype(np.int32)
+        T = int(counts.sum()) + (it % 3)
+        tex = rng.uniform(-1, 1, (T, Cin))
+        sh = rng.normal(0, 0.5, (T, 16))
+        filt = rng.normal(0, 0.3, (Cout, Cin, 16))
+        gout = rng.normal(0, 1, (nf, Cout))
+        out_ref = loops.f2f_fwd(tex, filt, sh, cum)
+        gin_ref, gfilt_ref = loops.f2f_bwd(gout, tex, filt, sh, cum)
+        tt = dev(tex, cuda, torch.float32).requires_grad_(True)
+        ft = dev(filt, cuda, torch.float32).requires_grad_(True)
+        out = conv3d.facet2facet(tt, ft, dev(sh, cuda, torch.float32), dev(cum, cuda))
+        out.backward(dev(gout, cuda, torch.float32))
+        torch.cuda.synchronize()
+        tag = " (sweep %d: nf=%d Cin=%d Cout=%d kmax=%d)" % (it, nf, Cin, Cout, kmax)
+        assert_close(out, out_ref, "f2f out" + tag)
+        assert_close(tt.grad, gin_ref, "f2f grad_texture" + tag)
+        assert_close(ft.grad, gfilt_ref, "f2f grad_filter" + tag)
 
 
 # ------------------------------------------------------------------ pooling

@@ -373,12 +373,15 @@ __global__ __launch_bounds__(kFThreads, 2 / kFR) void f2f16x3_fwd_k(const float 
 // texture gradient on the bf16 matrix cores:
 //     H[f, ci, d] = sum_co gout[f, co] W[co, ci, d]          (split-bf16 MFMAs, k = co)
 //     gtex[t, ci] = (1/K_f) sum_d sh[t, d] H[f, ci, d]       (FMAs on the accumulator registers)
-// The product is taken transposed, D[(ci,d)][f] = W^T . gout^T, with the 32 rows of a tile ordered so
-// that a lane (facet l32, half h) finds in its 16 accumulator registers exactly the 16 d's of ONE
-// input channel: tile tt = 4g + q holds channels 8g + q (rows of half 0) and 8g + 4 + q (rows of
-// half 1), accumulator register i <-> d = i.  The contraction with the SH values of the facet's
-// points then needs no cross-lane traffic, and after the four tiles of a group a lane owns four
-// consecutive channels of each of its points: one 16-byte store per point.
+// The product is taken transposed, D[(ci,d)][f] = W^T . gout^T.  A tile tt = 4g + q holds the two input
+// channels 8g + q ("a") and 8g + 4 + q ("b"); its 32 rows are ordered so that a lane (facet l32,
+// half h) finds in its 16 accumulator registers eight d's of BOTH channels:
+//     register i  <->  channel (i/4)%2,  d = 8(i/8) + 4h + i%4.
+// Each lane contracts its eight d's with the SH values of ALL the facet's points (8 instead of 16 SH
+// values per point in registers), and one v_permlane32_swap per point exchanges the partial sums so
+// that half 0 ends up with channel a and half 1 with channel b.  After the four tiles of a group a
+// lane owns four consecutive channels of each point.  The contraction of a tile runs while the MFMAs
+// of the next tile are in flight.
 //   workgroup  256 facets from the sorted list, 8 wavefronts x 32 facets, two wavefronts per SIMD
 //   gout       a lane's facet row, split once into bf16 pieces (B operand, registers)
 //   filter     pre-split / pre-arranged W^T tiles (f2f16x3_pack_filter_t_k), two tiles per LDS chunk,
@@ -396,7 +399,8 @@ __global__ __launch_bounds__(kBlock) void f2f16x3_pack_filter_t_k(const float *_
     if (idx >= NTt * NKS * 64) return;
     const int lane = idx & 63, ks = (idx >> 6) % NKS, tt = (idx >> 6) / NKS;
     const int r = lane & 31, h = lane >> 5;
-    const int ci = 8 * (tt >> 2) + 4 * ((r >> 2) & 1) + (tt & 3), d = 4 * (r >> 3) + (r & 3);
+    // row r = 8q + 4h' + j of the tile (h' = accumulator half, register 4q + j): channel q%2, d = 8(q/2) + 4h' + j
+    const int ci = 8 * (tt >> 2) + 4 * ((r >> 3) & 1) + (tt & 3), d = 8 * (r >> 4) + 4 * ((r >> 2) & 1) + (r & 3);
     float x[8];
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
@@ -409,25 +413,26 @@ __global__ __launch_bounds__(kBlock) void f2f16x3_pack_filter_t_k(const float *_
     dst[0] = p1; dst[64] = p2; dst[128] = p3;
 }
 
-template <int KW>
+template <int KW, int NKS>
 __device__ __forceinline__ void x3_tex_sweep(const u32x4 *__restrict__ WpT, const float *__restrict__ sh,
                                              float *__restrict__ gtex, u32x4 *Ws, float *stage, const int *w_k0,
-                                             const int *w_K, const u32x4 (&bp)[kTKS][3], int kbase, int Ks, float invK,
-                                             int sweep, int Cin, int NKS, int NG, int lane, int h)
+                                             const int *w_K, const u32x4 (&bp)[NKS][3], int kbase, int Ks, float invK,
+                                             int sweep, int Cin, int NG, int lane, int h)
 {
-    // SH rows of my facet's points, pre-scaled by 1/K
-    float shr[KW][16];
+    // SH values of my facet's points for my half's eight d's (4h..4h+3, 8+4h..8+4h+3), pre-scaled by 1/K
+    float shr[KW][8];
 #pragma unroll
     for (int kk = 0; kk < KW; ++kk) {
-#pragma unroll
-        for (int v4 = 0; v4 < 4; ++v4) {
-            float4 u = make_float4(0.f, 0.f, 0.f, 0.f);
-            if (kk < Ks) u = xld4(sh + (int64_t)(kbase + kk) * 16 + 4 * v4);
-            shr[kk][4 * v4 + 0] = u.x * invK; shr[kk][4 * v4 + 1] = u.y * invK;
-            shr[kk][4 * v4 + 2] = u.z * invK; shr[kk][4 * v4 + 3] = u.w * invK;
+        float4 u = make_float4(0.f, 0.f, 0.f, 0.f), v = u;
+        if (kk < Ks) {
+            const float *p = sh + (int64_t)(kbase + kk) * 16 + 4 * h;
+            u = xld4(p);
+            v = xld4(p + 8);
         }
+        shr[kk][0] = u.x * invK; shr[kk][1] = u.y * invK; shr[kk][2] = u.z * invK; shr[kk][3] = u.w * invK;
+        shr[kk][4] = v.x * invK; shr[kk][5] = v.y * invK; shr[kk][6] = v.z * invK; shr[kk][7] = v.w * invK;
     }
-    const int chunk = 2 * NKS * 192;             // uint4 per chunk of two tiles
+    constexpr int chunk = 2 * NKS * 192;         // uint4 per chunk of two tiles
     const int nchunks = 2 * NG;
     auto chunk_fetch = [&](u32x4 (&wn)[3], int c) {
 #pragma unroll
@@ -464,12 +469,45 @@ __device__ __forceinline__ void x3_tex_sweep(const u32x4 *__restrict__ WpT, cons
                         *reinterpret_cast<const float4 *>(stage + (kk * 32 + slot) * 16 + 4 * (lane & 3));
         }
     };
-    for (int g = 0; g < NG; ++g) {
-        float gacc[KW][4];
+    // Results go out 64 bytes at a time: two groups (16 channels) of every point are collected in
+    // the wavefront's LDS stage [point][facet slot][16 channels], then four lanes write one
+    // 64-byte piece of a row (32-byte pieces cost almost twice the HBM write traffic).
+    float gacc[KW][4];
+    auto finish_group = [&](int g) {
 #pragma unroll
         for (int kk = 0; kk < KW; ++kk)
+            *reinterpret_cast<float4 *>(stage + (kk * 32 + (lane & 31)) * 16 + (g & 1) * 8 + 4 * h) =
+                make_float4(gacc[kk][0], gacc[kk][1], gacc[kk][2], gacc[kk][3]);
+        if ((g & 1) || g == NG - 1) flush(g >> 1);
+    };
+    // contraction of a finished tile (accumulator accp) into channel slot q of the group
+    f32x16 accp;
 #pragma unroll
-            for (int q = 0; q < 4; ++q) gacc[kk][q] = 0.f;
+    for (int i = 0; i < 16; ++i) accp[i] = 0.f;
+    auto contract = [&](int q) {
+        float xa[KW], xb[KW];
+#pragma unroll
+        for (int kk = 0; kk < KW; ++kk) {
+            float va = 0.f, vb = 0.f;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                va = fmaf(shr[kk][j], accp[8 * (j >> 2) + (j & 3)], va);          // channel a: registers 0-3, 8-11
+                vb = fmaf(shr[kk][j], accp[8 * (j >> 2) + 4 + (j & 3)], vb);      // channel b: registers 4-7, 12-15
+            }
+            xa[kk] = va;
+            xb[kk] = vb;
+        }
+        // xa: half 0 keeps its own, receives half 0's xb into half 1; xb: half 0 receives half 1's xa.
+        // Afterwards xa + xb is the full sum over d of channel a in half 0 and of channel b in half 1.
+        // (The s_nop cover the wait states between vector ALU writes / reads and the swap.)
+#pragma unroll
+        for (int kk = 0; kk < KW; ++kk)
+            asm volatile("s_nop 3\n v_permlane32_swap_b32 %0, %1\n s_nop 3" : "+v"(xa[kk]), "+v"(xb[kk]));
+#pragma unroll
+        for (int kk = 0; kk < KW; ++kk) gacc[kk][q] = xa[kk] + xb[kk];
+    };
+
+    for (int g = 0; g < NG; ++g) {
 #pragma unroll
         for (int cc = 0; cc < 2; ++cc) {
             const int c = 2 * g + cc;
@@ -478,54 +516,46 @@ __device__ __forceinline__ void x3_tex_sweep(const u32x4 *__restrict__ WpT, cons
             const u32x4 *Wc = Ws + (c % 3) * kTChunkMax + lane;
 #pragma unroll
             for (int u = 0; u < 2; ++u) {
-                // H tile of two input channels: rows (channel half, d), columns = my wavefront's facets
+                // H tile of two input channels: rows (d half, channel, d), columns = my wavefront's facets
                 f32x16 acc0;
 #pragma unroll
                 for (int i = 0; i < 16; ++i) acc0[i] = 0.f;
 #pragma unroll
-                for (int ks = 0; ks < kTKS; ++ks) {
-                    if (ks < NKS) {
-                        u32x4 a[3];
+                for (int ks = 0; ks < NKS; ++ks) {
+                    u32x4 a[3];
 #pragma unroll
-                        for (int p = 0; p < 3; ++p) a[p] = Wc[((u * NKS + ks) * 3 + p) * 64];
-                        // six piece products, smallest first
-                        acc0 = mfma_bf16(a[2], bp[ks][0], acc0);
-                        acc0 = mfma_bf16(a[1], bp[ks][1], acc0);
-                        acc0 = mfma_bf16(a[0], bp[ks][2], acc0);
-                        acc0 = mfma_bf16(a[1], bp[ks][0], acc0);
-                        acc0 = mfma_bf16(a[0], bp[ks][1], acc0);
-                        acc0 = mfma_bf16(a[0], bp[ks][0], acc0);
-                    }
+                    for (int p = 0; p < 3; ++p) a[p] = Wc[((u * NKS + ks) * 3 + p) * 64];
+                    // six piece products, smallest first
+                    acc0 = mfma_bf16(a[2], bp[ks][0], acc0);
+                    acc0 = mfma_bf16(a[1], bp[ks][1], acc0);
+                    acc0 = mfma_bf16(a[0], bp[ks][2], acc0);
+                    acc0 = mfma_bf16(a[1], bp[ks][0], acc0);
+                    acc0 = mfma_bf16(a[0], bp[ks][1], acc0);
+                    acc0 = mfma_bf16(a[0], bp[ks][0], acc0);
                 }
-                // contraction with the SH rows: my channel of this tile is 8g + 4h + q, q = 2cc + u
-#pragma unroll
-                for (int kk = 0; kk < KW; ++kk) {
-                    float v = 0.f;
-#pragma unroll
-                    for (int i = 0; i < 16; ++i) v = fmaf(shr[kk][i], acc0[i], v);
-                    gacc[kk][2 * cc + u] = v;
-                }
+                // meanwhile: the previous tile (the last one of the previous group when cc = u = 0)
+                contract((2 * cc + u + 3) & 3);
+                if (cc == 0 && u == 0 && g > 0) finish_group(g - 1);
+                accp = acc0;
             }
             if (more) chunk_publish(wn, c + 2);
             __syncthreads();
         }
-        // Results go out 64 bytes at a time: two groups (16 channels) of every point are collected in
-        // the wavefront's LDS stage [point][facet slot][16 channels], then four lanes write one
-        // 64-byte piece of a row (32-byte pieces cost almost twice the HBM write traffic).
-#pragma unroll
-        for (int kk = 0; kk < KW; ++kk)
-            *reinterpret_cast<float4 *>(stage + (kk * 32 + (lane & 31)) * 16 + (g & 1) * 8 + 4 * h) =
-                make_float4(gacc[kk][0], gacc[kk][1], gacc[kk][2], gacc[kk][3]);
-        if ((g & 1) || g == NG - 1) flush(g >> 1);
     }
+    contract(3);
+    finish_group(NG - 1);
 }
 
+// NKS = k-steps of 16 output channels (compile time, so that a tile's MFMAs and the previous tile's
+// contraction share one basic block and get interleaved): 2 for Cout <= 32, else 4; the packed filter
+// is zero padded to that many.
+template <int NKS>
 __global__ __launch_bounds__(512, 2) void f2f16x3_bwd_tex_k(const float *__restrict__ gout,
                                                             const u32x4 *__restrict__ WpT,
                                                             const float *__restrict__ sh,
                                                             const int *__restrict__ cum,
                                                             const int *__restrict__ order, float *__restrict__ gtex,
-                                                            int64_t Nf, int T, int Cin, int Cout, int NKS, int NG)
+                                                            int64_t Nf, int T, int Cin, int Cout, int NG)
 {
     __shared__ u32x4 Ws[3 * kTChunkMax];
     __shared__ __attribute__((aligned(16))) float s_stage[8][kXKB * 32 * 16];
@@ -555,9 +585,9 @@ __global__ __launch_bounds__(512, 2) void f2f16x3_bwd_tex_k(const float *__restr
         if (lane == 0) atomicMax(&s_kmax, km);
     }
     // my facet's gout row as B operand pieces: k-step ks, half h <-> channels 16ks + 8h .. + 7
-    u32x4 bp[kTKS][3];
+    u32x4 bp[NKS][3];
 #pragma unroll
-    for (int ks = 0; ks < kTKS; ++ks) {
+    for (int ks = 0; ks < NKS; ++ks) {
         float x[8];
 #pragma unroll
         for (int j = 0; j < 8; ++j) x[j] = 0.f;
@@ -577,7 +607,7 @@ __global__ __launch_bounds__(512, 2) void f2f16x3_bwd_tex_k(const float *__restr
         const int kw = xwave_max(Ks);
         const int kbase = k0 + sw * kXKB;
         // every variant runs the same barriers, so wavefronts of a workgroup may pick different ones
-#define PM_X3T(N) x3_tex_sweep<N>(WpT, sh, gtex, Ws, s_stage[w], s_k0[w], s_K[w], bp, kbase, Ks, invK, sw, Cin, NKS, NG, lane, h)
+#define PM_X3T(N) x3_tex_sweep<N, NKS>(WpT, sh, gtex, Ws, s_stage[w], s_k0[w], s_K[w], bp, kbase, Ks, invK, sw, Cin, NG, lane, h)
         if (kw <= 1) PM_X3T(1);
         else if (kw == 2) PM_X3T(2);
         else if (kw == 3) PM_X3T(3);
@@ -964,7 +994,7 @@ int f2f16x3_fwd(const float *tex, const float *W, const float *sh, const int *cu
 
 size_t f2f16x3_bwd_texture_workspace_bytes(int Cin, int Cout)
 {
-    const int NG = (Cin + 7) / 8, NKS = (Cout + 15) / 16;
+    const int NG = (Cin + 7) / 8, NKS = Cout <= 32 ? 2 : 4;
     return (size_t)NG * 4 * NKS * 3 * 64 * sizeof(u32x4);
 }
 
@@ -974,7 +1004,7 @@ int f2f16x3_bwd_texture(const float *gout, const float *W, const float *sh, cons
                         float *gtex, void *workspace, size_t workspace_bytes, int64_t T, int64_t Nf, int Cin,
                         int Cout, hipStream_t st)
 {
-    const int NG = (Cin + 7) / 8, NKS = (Cout + 15) / 16;
+    const int NG = (Cin + 7) / 8, NKS = Cout <= 32 ? 2 : 4;
     PM_REQUIRE(workspace && workspace_bytes >= f2f16x3_bwd_texture_workspace_bytes(Cin, Cout),
                "f2f_bwd_texture: workspace too small (%zu bytes)", workspace_bytes);
     PM_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 15u) == 0, "f2f_bwd_texture: workspace must be 16-byte aligned");
@@ -984,7 +1014,10 @@ int f2f16x3_bwd_texture(const float *gout, const float *W, const float *sh, cons
     PM_LAUNCHED("f2f_bwd_texture(pack)");
     const int64_t gx = ceil_div(Nf, 256);
     PM_REQUIRE(grid_ok(gx), "f2f_bwd_texture: grid too large");
-    f2f16x3_bwd_tex_k<<<dim3((unsigned)gx), dim3(512), 0, st>>>(gout, WpT, sh, cum, order, gtex, Nf, (int)T, Cin, Cout, NKS, NG);
+    if (NKS == 2)
+        f2f16x3_bwd_tex_k<2><<<dim3((unsigned)gx), dim3(512), 0, st>>>(gout, WpT, sh, cum, order, gtex, Nf, (int)T, Cin, Cout, NG);
+    else
+        f2f16x3_bwd_tex_k<4><<<dim3((unsigned)gx), dim3(512), 0, st>>>(gout, WpT, sh, cum, order, gtex, Nf, (int)T, Cin, Cout, NG);
     PM_LAUNCHED("f2f_bwd_texture");
     return 0;
 }

@@ -190,6 +190,18 @@ int pmesh_unpool_bwd(const float *grad_output, const int32_t *rowptr, const int3
  * xyz (N,3) -> out (N,(L+1)^2); a zero vector evaluates at direction (1,0,0). */
 int pmesh_sph_harm(const float *xyz, float *out, int64_t N, int L, pmesh_stream_t stream);
 
+/* ------------------------------------------------------------------ per-level inputs of the convs
+ * pmesh_count_vertex_adjface replaces count_vertex_adjface (decimate_gpu.cu:813-836,
+ * decimate.py:88-93): the number of (facet, corner) entries per output vertex is the row length
+ * of the facet2vertex CSR (pmesh_build_vertex_csr with that vt_map); nf_count (NvOut) int32.
+ * pmesh_triangle_geometry replaces compute_triangle_geometry_ (decimate.py:70-85):
+ * geometry (Nf,5) = unit normal, plane offset d = -n.v0, area; vertex rows have vertex_stride
+ * floats (>= 3), position first.  normal = raw / (|raw| + 1e-10) as in the reference. */
+int pmesh_count_vertex_adjface(const int32_t *rowptr, int32_t *nf_count, int64_t NvOut,
+                               pmesh_stream_t stream);
+int pmesh_triangle_geometry(const float *vertex, const int32_t *face, float *geometry, int64_t Nv,
+                            int64_t Nf, int vertex_stride, pmesh_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -718,6 +718,38 @@ static inline int pick_v(int C, int r, std::initializer_list<const void *> ptrs)
     return 4;
 }
 
+// ----------------------------------------------------------------------------------------
+// per-level producers of the convolution inputs
+// ----------------------------------------------------------------------------------------
+// nf_count[v] = number of (facet, corner) entries landing on output vertex v = its CSR row length
+__global__ __launch_bounds__(kBlock) void row_length_k(const int *__restrict__ rowptr, int *__restrict__ out, int64_t n)
+{
+    const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i < n) out[i] = rowptr[i + 1] - rowptr[i];
+}
+
+// geometry[f] = (unit normal (3), plane offset d = -n.v0, area) of triangle f; vertex rows have
+// `vstride` floats of which the first three are the position
+__global__ __launch_bounds__(kBlock) void triangle_geometry_k(const float *__restrict__ vertex, const int *__restrict__ face,
+                                                             float *__restrict__ geometry, int64_t Nf, int vstride)
+{
+    const int64_t f = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (f >= Nf) return;
+    const float *a = vertex + (int64_t)face[3 * f] * vstride;
+    const float *b = vertex + (int64_t)face[3 * f + 1] * vstride;
+    const float *c = vertex + (int64_t)face[3 * f + 2] * vstride;
+    const float ax = a[0], ay = a[1], az = a[2];
+    const float ux = b[0] - ax, uy = b[1] - ay, uz = b[2] - az;
+    const float vx = c[0] - ax, vy = c[1] - ay, vz = c[2] - az;
+    const float nx = uy * vz - uz * vy, ny = uz * vx - ux * vz, nz = ux * vy - uy * vx;
+    const float len = sqrtf(nx * nx + ny * ny + nz * nz);
+    const float inv = 1.0f / (len + 1e-10f);
+    float *g = geometry + 5 * f;
+    g[0] = nx * inv; g[1] = ny * inv; g[2] = nz * inv;
+    g[3] = -(g[0] * ax + g[1] * ay + g[2] * az);
+    g[4] = 0.5f * len;
+}
+
 static int reduce_partials(const float *partial, float *out, int G, int n, hipStream_t st)
 {
     reduce_partials_k<<<dim3((unsigned)ceil_div(n, 16)), dim3(1024), 0, st>>>(partial, out, G, n);
@@ -1000,5 +1032,30 @@ extern "C" int pmesh_sph_harm(const float *xyz, float *out, int64_t N, int L, pm
     PM_REQUIRE(grid_ok(ceil_div(N, kBlock)), "sph_harm: grid too large");
     sph_harm_k<<<dim3((unsigned)ceil_div(N, kBlock)), dim3(kBlock), 0, (hipStream_t)stream>>>(xyz, out, N, L);
     PM_LAUNCHED("sph_harm");
+    return 0;
+}
+
+extern "C" int pmesh_count_vertex_adjface(const int32_t *rowptr, int32_t *nf_count, int64_t NvOut, pmesh_stream_t stream)
+{
+    clear_error();
+    PM_REQUIRE(NvOut >= 0, "count_vertex_adjface: negative size");
+    if (NvOut == 0) return 0;
+    PM_REQUIRE(rowptr && nf_count, "count_vertex_adjface: null pointer");
+    PM_REQUIRE(grid_ok(ceil_div(NvOut, kBlock)), "count_vertex_adjface: grid too large");
+    row_length_k<<<dim3((unsigned)ceil_div(NvOut, kBlock)), dim3(kBlock), 0, (hipStream_t)stream>>>(rowptr, nf_count, NvOut);
+    PM_LAUNCHED("count_vertex_adjface");
+    return 0;
+}
+
+extern "C" int pmesh_triangle_geometry(const float *vertex, const int32_t *face, float *geometry, int64_t Nv,
+                                       int64_t Nf, int vertex_stride, pmesh_stream_t stream)
+{
+    clear_error();
+    PM_REQUIRE(Nv >= 0 && Nf >= 0 && vertex_stride >= 3, "triangle_geometry: bad sizes");
+    if (Nf == 0) return 0;
+    PM_REQUIRE(vertex && face && geometry, "triangle_geometry: null pointer");
+    PM_REQUIRE(Nv * vertex_stride < (int64_t(1) << 40) && grid_ok(ceil_div(Nf, kBlock)), "triangle_geometry: sizes too large");
+    triangle_geometry_k<<<dim3((unsigned)ceil_div(Nf, kBlock)), dim3(kBlock), 0, (hipStream_t)stream>>>(vertex, face, geometry, Nf, vertex_stride);
+    PM_LAUNCHED("triangle_geometry");
     return 0;
 }

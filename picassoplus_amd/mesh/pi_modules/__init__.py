@@ -1,3 +1,3 @@
-from . import conv3d, pool3d, unpool3d
+from . import conv3d, geometry, pool3d, unpool3d
 
-__all__ = ['conv3d', 'pool3d', 'unpool3d']
+__all__ = ['conv3d', 'geometry', 'pool3d', 'unpool3d']

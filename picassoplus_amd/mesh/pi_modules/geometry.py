@@ -1,0 +1,41 @@
+"""Per-level producers of the convolution inputs: adjacent-facet counts of the output vertices and
+triangle geometry, with the reference's function names (picasso/mesh/pi_modules/decimate.py:70-93).
+Mesh decimation itself is not part of this package."""
+import torch
+
+from ... import _lib
+from .. import topology
+from ._check import F32, I32, check_input, same_device, stream_of
+
+
+def count_vertex_adjface_(face, vtMap, vertexOut):
+    """Number of adjacent (facet, corner) entries of every output vertex ``{vtMap[i] | vtMap[i] >= 0}``
+    (decimate.py:88-93, decimate_gpu.cu:813-836) -> int32 (NvOut,).  It is the row length of the
+    facet-to-vertex adjacency, which is built (and cached for the convolutions) here."""
+    check_input(face, "face", 2, I32)
+    check_input(vtMap, "vtMap", 1, I32)
+    if not isinstance(vertexOut, torch.Tensor) or vertexOut.dim() != 2:
+        raise RuntimeError("vertexOut must have dimension of 2")
+    dev = same_device(face, vtMap)
+    nv_out = vertexOut.shape[0]
+    rowptr, _ = topology.vertex_csr(face, vtMap, nv_out)
+    with torch.cuda.device(dev):
+        out = torch.empty(nv_out, dtype=I32, device=dev)
+        _lib.call("pmesh_count_vertex_adjface", rowptr.data_ptr(), out.data_ptr(), nv_out, stream_of(face))
+    return out
+
+
+def compute_triangle_geometry_(vertex, face):
+    """(Nf, 5) = unit normal, plane offset d = -n.v0, area of every facet (decimate.py:70-85).
+    ``vertex`` (Nv, >= 3) float32 with the position in the first three columns."""
+    check_input(vertex, "vertex", 2, F32)
+    check_input(face, "face", 2, I32)
+    if vertex.shape[1] < 3 or face.shape[1] != 3:
+        raise RuntimeError("vertex must have at least 3 columns and face exactly 3")
+    dev = same_device(vertex, face)
+    topology._check_range_cached(face, vertex.shape[0])
+    with torch.cuda.device(dev):
+        out = torch.empty((face.shape[0], 5), dtype=F32, device=dev)
+        _lib.call("pmesh_triangle_geometry", vertex.data_ptr(), face.data_ptr(), out.data_ptr(), vertex.shape[0],
+                  face.shape[0], vertex.shape[1], stream_of(vertex))
+    return out

@@ -303,3 +303,37 @@ def test_bitwise_reproducible(cuda):
         assert torch.equal(a, b)
     for a, b in zip(runs[0], runs[2]):
         assert torch.equal(a, b)
+
+
+# ------------------------------------------------------------------ per-level inputs
+@pytest.mark.parametrize("mesh", ["octa", "sphere3", "room_small"])
+def test_adjface_count_and_triangle_geometry(cuda, mesh):
+    from oracle import torch_ref as R
+    from picassoplus_amd.mesh.pi_modules import geometry
+    rng = np.random.default_rng(31)
+    v, f = mesh_case(mesh)
+    nv = v.shape[0]
+    vt_map, nvo = strided_vt_map(rng, nv)
+    got = geometry.count_vertex_adjface_(dev(f, cuda), dev(vt_map, cuda), torch.zeros(nvo, 3, device=cuda))
+    ref = R.count_vertex_adjface(torch.from_numpy(f), torch.from_numpy(vt_map), nvo)
+    assert torch.equal(got.cpu(), ref.to(torch.int32))
+    assert int(got.sum()) == int((vt_map[f.reshape(-1)] >= 0).sum())
+    # geometry: vertex rows carry extra columns (colour) after the position
+    vx = np.concatenate([v, rng.uniform(0, 1, (nv, 3))], 1).astype(np.float32)
+    geo = geometry.compute_triangle_geometry_(dev(vx, cuda), dev(f, cuda))
+    torch.cuda.synchronize()
+    p = vx[:, :3].astype(np.float64)
+    raw = np.cross(p[f[:, 1]] - p[f[:, 0]], p[f[:, 2]] - p[f[:, 0]])
+    ln = np.linalg.norm(raw, axis=1, keepdims=True)
+    normal = raw / (ln + 1e-10)
+    ref_geo = np.concatenate([normal, -(normal * p[f[:, 0]]).sum(1, keepdims=True), ln / 2], 1)
+    # float32 cross products of thin or collapsed triangles cancel: direction and offset are compared
+    # on the well-shaped facets, the area (absolute scale) on all of them
+    e1, e2 = p[f[:, 1]] - p[f[:, 0]], p[f[:, 2]] - p[f[:, 0]]
+    ok = ln[:, 0] > 0.1 * np.linalg.norm(e1, axis=1) * np.linalg.norm(e2, axis=1)
+    assert ok.mean() > 0.5
+    okt = torch.from_numpy(ok).to(cuda)
+    assert_close(geo[okt][:, :4], ref_geo[ok][:, :4], "triangle normal and offset", 1e-4)
+    assert_close(geo[:, 4], ref_geo[:, 4], "triangle area")
+    assert_close(geo[okt][:, :3], R.face_normals(torch.from_numpy(p), torch.from_numpy(f)).numpy()[ok],
+                 "normals vs oracle", 1e-4)

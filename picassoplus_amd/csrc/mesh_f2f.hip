@@ -365,7 +365,9 @@ extern "C" int pmesh_f2f_fwd(const float *texture, const float *filter, const fl
     PM_F2F_DIMS("f2f_fwd");
     if (Nf == 0) return 0;
     PM_REQUIRE(filter && cum_texture && output && (T == 0 || (texture && bary_coeff)), "f2f_fwd: null pointer");
-    if (!force_generic() && !force_fp32_mfma() && f2f16_usable(texture, filter, bary_coeff, Cin, F))
+    // the split-bf16 forward addresses texture elements with 32-bit offsets
+    if (!force_generic() && !force_fp32_mfma() && f2f16_usable(texture, filter, bary_coeff, Cin, F) &&
+        T * Cin < (int64_t(1) << 31))
         return f2f16x3_fwd(texture, filter, bary_coeff, cum_texture, facet_order, output, workspace, workspace_bytes,
                            T, Nf, Cin, Cout, (hipStream_t)stream);
     if (!force_generic() && f2f16_usable(texture, filter, bary_coeff, Cin, F))

@@ -81,8 +81,8 @@ def conv_bytes_flops(d, ops):
 # HBM bytes per launch of the op's main kernel on the default scene workload (scale 1.0), measured with
 # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE and scaled by what the same counters read for a 1 GiB copy
 # (--copy-calibration); reported as roofline.traffic when that workload runs.
-SCENE_TRAFFIC_BYTES = {"f2f_fwd": 4.646e9, "f2f_bwd_texture": 5.136e9, "f2f_bwd_filter": 3.365e9,
-                       "f2v_fwd": 2.046e9, "f2v_bwd": 2.020e9}
+SCENE_TRAFFIC_BYTES = {"f2f_fwd": 4.650e9, "f2f_bwd_texture": 4.011e9, "f2f_bwd_filter": 3.365e9,
+                       "f2v_fwd": 2.066e9, "f2v_bwd": 2.020e9}
 
 
 class EventTimer:

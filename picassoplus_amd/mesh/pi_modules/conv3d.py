@@ -2,34 +2,15 @@
 
 ``vertex2facet``, ``facet2facet`` and ``facet2vertex`` take the same arguments in the same
 order as the reference functions (conv3d.py:21,55,89), save the same tensors for backward
-and return ``None`` gradients for index and coefficient inputs.  Backward only computes the
-gradients autograd asks for through ``needs_input_grad``; both are produced by one native
-call, so nothing is saved by skipping and both are always computed, as in the reference.
+and return ``None`` gradients for index and coefficient inputs.  The feature and the filter
+gradient come out of one native call, so both are always computed, as in the reference.
 """
-import torch
-
 from . import mesh_conv3d as module
+from ._autograd import native_op
 
-
-def _no_grad_flags(*tensors):
-    # the reference clears requires_grad on index / coefficient inputs in place (conv3d.py:8-9)
-    for t in tensors:
-        if t.requires_grad:
-            t.requires_grad = False
-
-
-class f2f_Function(torch.autograd.Function):
-    @staticmethod
-    def forward(ctx, textureIn, filter, baryCoeff, numTexture):
-        _no_grad_flags(baryCoeff, numTexture)
-        output = module.facet2facet_forward(textureIn, filter, baryCoeff, numTexture)
-        ctx.save_for_backward(textureIn, filter, baryCoeff, numTexture)
-        return output
-
-    @staticmethod
-    def backward(ctx, grad_output):
-        grad_input, grad_filter = module.facet2facet_backward(grad_output.contiguous(), *ctx.saved_tensors)
-        return grad_input, grad_filter, None, None
+f2f_Function = native_op("f2f_Function", module.facet2facet_forward, module.facet2facet_backward, n_inputs=4, n_grads=2)
+v2f_Function = native_op("v2f_Function", module.vertex2facet_forward, module.vertex2facet_backward, n_inputs=3, n_grads=2)
+f2v_Function = native_op("f2v_Function", module.facet2vertex_forward, module.facet2vertex_backward, n_inputs=6, n_grads=2)
 
 
 def facet2facet(textureIn, filter, baryCoeff, numTexture):
@@ -44,20 +25,6 @@ def facet2facet(textureIn, filter, baryCoeff, numTexture):
     return f2f_Function.apply(textureIn, filter, baryCoeff, numTexture)
 
 
-class v2f_Function(torch.autograd.Function):
-    @staticmethod
-    def forward(ctx, input, filter, face):
-        _no_grad_flags(face)
-        output = module.vertex2facet_forward(input, filter, face)
-        ctx.save_for_backward(input, filter, face)
-        return output
-
-    @staticmethod
-    def backward(ctx, grad_output):
-        grad_input, grad_filter = module.vertex2facet_backward(grad_output.contiguous(), *ctx.saved_tensors)
-        return grad_input, grad_filter, None
-
-
 def vertex2facet(input, filter, face):
     """Facet features as a filtered combination of the three corner features.
 
@@ -65,20 +32,6 @@ def vertex2facet(input, filter, face):
     returns (Nf, C*r) float32
     """
     return v2f_Function.apply(input, filter, face)
-
-
-class f2v_Function(torch.autograd.Function):
-    @staticmethod
-    def forward(ctx, input, filter, coeff, face, nfCount, vtMap):
-        _no_grad_flags(coeff, face, nfCount, vtMap)
-        output = module.facet2vertex_forward(input, filter, coeff, face, nfCount, vtMap)
-        ctx.save_for_backward(input, filter, coeff, face, nfCount, vtMap)
-        return output
-
-    @staticmethod
-    def backward(ctx, grad_output):
-        grad_input, grad_filter = module.facet2vertex_backward(grad_output.contiguous(), *ctx.saved_tensors)
-        return grad_input, grad_filter, None, None, None, None
 
 
 def facet2vertex(input, filter, coeff, face, nfCount, vtMap):

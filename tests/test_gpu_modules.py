@@ -142,3 +142,43 @@ def test_per_item_and_coeff_modules(cuda):
     n = torch.nn.functional.normalize(torch.randn(40, 3, device=cuda), dim=1)
     c = b(n)
     assert c.shape == (40, 7) and torch.allclose(c.sum(1), torch.ones(40, device=cuda), atol=1e-5)
+
+
+def test_argument_errors_and_side_stream(cuda):
+    """CHECK_INPUT-style failures raise RuntimeError (mesh_conv3d.cpp:24-30, 56, 138-139, 210-213), and work
+    is enqueued on the caller's current stream."""
+    from picassoplus_amd.mesh.pi_modules import conv3d, pool3d
+    rng = np.random.default_rng(41)
+    v, f = mesh_case("sphere2")
+    nv, nf = v.shape[0], f.shape[0]
+    x = torch.randn(nv, 8, device=cuda)
+    w = torch.randn(3, 8, 1, device=cuda)
+    face = torch.from_numpy(f).to(cuda)
+    with pytest.raises(RuntimeError):
+        conv3d.vertex2facet(x.cpu(), w, face)                       # CPU tensor
+    with pytest.raises(RuntimeError):
+        conv3d.vertex2facet(x.t().contiguous().t(), w, face)        # non-contiguous
+    with pytest.raises(RuntimeError):
+        conv3d.vertex2facet(x.double(), w, face)                    # wrong dtype
+    with pytest.raises(RuntimeError):
+        conv3d.vertex2facet(x, w, face.long())                      # int64 indices
+    with pytest.raises(RuntimeError):
+        conv3d.vertex2facet(x, w[:, :4].contiguous(), face)         # channel mismatch
+    with pytest.raises(RuntimeError):
+        conv3d.vertex2facet(x, w, face + nv)                        # vertex index out of range
+    with pytest.raises(RuntimeError):
+        conv3d.facet2facet(torch.randn(10, 4, device=cuda), torch.randn(8, 4, 51, device=cuda),
+                           torch.randn(10, 51, device=cuda), torch.arange(1, 11, device=cuda, dtype=torch.int32))
+    with pytest.raises(RuntimeError):
+        pool3d.maxPool(x, torch.zeros(nv - 1, dtype=torch.int32, device=cuda),
+                       torch.zeros(nv, dtype=torch.int32, device=cuda), torch.zeros(4, 3, device=cuda))
+    # side stream: the op must wait for work queued before it on that stream and be waited for after it
+    ref = conv3d.vertex2facet(x, w, face)
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        x2 = x * 1.0                                                  # producer on the side stream
+        got = conv3d.vertex2facet(x2, w, face)
+        total = got.sum()
+    side.synchronize()
+    assert torch.equal(got, ref) and float(total) == float(ref.sum())

@@ -248,10 +248,26 @@ __device__ __forceinline__ void fma_bcast16(float cf, const Pack<4> (&fl)[16], P
 #undef PM_B
 }
 
-// facet2vertex forward for r = 1, C % 64 == 0 (row groups are whole 16-lane DPP rows), K <= 16.
+// The four output channels co .. co+3 of a lane read the input channels co/R .. : for R = 1 four
+// distinct ones, for R = 2 two, each used twice (out[., c*R + m]).
+template <int R> __device__ __forceinline__ Pack<4> ld_in_expanded(const float *p)
+{
+    if constexpr (R == 1) {
+        return ldp<4>(p);
+    } else {
+        const float2 t = *reinterpret_cast<const float2 *>(p);
+        Pack<4> o;
+        o.v[0] = t.x; o.v[1] = t.x; o.v[2] = t.y; o.v[3] = t.y;
+        return o;
+    }
+}
+
+// facet2vertex forward for depth multiplier R = 1 or 2, Co = C*R a multiple of 4 and >= 64 (a 16-lane DPP row
+// then lies inside one vertex's row group; lanes past Co/4 are masked), K <= 16.
 // Persistent row groups: the filter stays in registers for all the vertices a group visits, and three
 // stages of gathers are in flight at once -- the row bounds of the vertex after next, the entry list of
 // the next vertex, and the facet rows / coefficients of the current one (eight entries at a time).
+template <int R>
 __global__ __launch_bounds__(kBlock) void f2v_fwd_fast_k(const float *__restrict__ in, const float *__restrict__ filt,
                                                          const float *__restrict__ coeff,
                                                          const int *__restrict__ nfcount,
@@ -262,11 +278,13 @@ __global__ __launch_bounds__(kBlock) void f2v_fwd_fast_k(const float *__restrict
     constexpr int EB = 8;
     const int lpr = 1 << lpr_log2, rpb = kBlock >> lpr_log2;
     const int lane = threadIdx.x & (lpr - 1), slot = threadIdx.x >> lpr_log2, l16 = threadIdx.x & 15;
-    const int c = lane * 4;
+    const int Co = C * R;
+    const int c = lane * 4;                       // my four output channels; input channels c / R ..
+    const bool on = c < Co;
     const bool kok = l16 < K;
     Pack<4> fl[16];
 #pragma unroll
-    for (int k = 0; k < 16; ++k) fl[k] = (k < K) ? ldp<4>(filt + (size_t)k * C + c) : zero_pack<4>();
+    for (int k = 0; k < 16; ++k) fl[k] = (k < K && on) ? ldp<4>(filt + (size_t)k * Co + c) : zero_pack<4>();
 
     const int64_t stride = (int64_t)gridDim.x * rpb;
     int64_t row = (int64_t)blockIdx.x * rpb + slot;
@@ -297,7 +315,7 @@ __global__ __launch_bounds__(kBlock) void f2v_fwd_fast_k(const float *__restrict
             float cf[EB];
 #pragma unroll
             for (int i = 0; i < EB; ++i) {
-                x[i] = (f[i] >= 0) ? ldp<4>(in + (int64_t)f[i] * C + c) : zero_pack<4>();
+                x[i] = (f[i] >= 0 && on) ? ld_in_expanded<R>(in + (int64_t)f[i] * C + c / R) : zero_pack<4>();
                 cf[i] = (f[i] >= 0 && kok) ? coeff[(int64_t)f[i] * K + l16] : 0.f;
             }
 #pragma unroll
@@ -312,7 +330,7 @@ __global__ __launch_bounds__(kBlock) void f2v_fwd_fast_k(const float *__restrict
         }
 #pragma unroll
         for (int u = 0; u < 4; ++u) acc.v[u] *= inv;
-        stp<4>(out + row * C + c, acc);
+        if (on) stp<4>(out + row * Co + c, acc);
         e0 = ne0; e1 = ne1; ne0 = me0; ne1 = me1;
 #pragma unroll
         for (int i = 0; i < EB; ++i) f[i] = nf[i];
@@ -409,6 +427,7 @@ __global__ __launch_bounds__(kBlock) void f2v_bwd_k(const float *__restrict__ go
 // facet2vertex backward for r = 1, C % 64 == 0, K <= 16: same arithmetic as f2v_bwd_k with the
 // coefficient row spread over the 16 lanes of a DPP row, and the index chain
 // face -> vt_map -> (nf_count, gout rows) of the NEXT facet resolved while the current one is computed.
+template <int R>
 __global__ __launch_bounds__(kBlock) void f2v_bwd_fast_k(const float *__restrict__ gout, const float *__restrict__ in,
                                                          const float *__restrict__ filt,
                                                          const float *__restrict__ coeff,
@@ -423,11 +442,13 @@ __global__ __launch_bounds__(kBlock) void f2v_bwd_fast_k(const float *__restrict
     const int lane = threadIdx.x & (lpr - 1), slot = threadIdx.x >> lpr_log2, l16 = threadIdx.x & 15;
     const int64_t fbeg = (int64_t)blockIdx.x * rows_per_block;
     const int64_t fend = (fbeg + rows_per_block < Nf) ? fbeg + rows_per_block : Nf;
-    const int c = lane * 4;
+    const int Co = C * R;
+    const int c = lane * 4;                       // my four output channels; input channels c / R ..
+    const bool on = c < Co;
     Pack<4> fl[16], acc[16];
 #pragma unroll
     for (int k = 0; k < 16; ++k) {
-        fl[k] = (k < K) ? ldp<4>(filt + (size_t)k * C + c) : zero_pack<4>();
+        fl[k] = (k < K && on) ? ldp<4>(filt + (size_t)k * Co + c) : zero_pack<4>();
         acc[k] = zero_pack<4>();
     }
     // software pipeline over this slot's facets: indices two facets ahead, output rows one ahead
@@ -459,10 +480,10 @@ __global__ __launch_bounds__(kBlock) void f2v_bwd_fast_k(const float *__restrict
 #pragma unroll
         for (int j = 0; j < 3; ++j) {
             const bool ok = vo[j] >= 0 && vo[j] < NvOut;
-            g[j] = ok ? ldp<4>(gout + (int64_t)vo[j] * C + c) : zero_pack<4>();
+            g[j] = (ok && on) ? ldp<4>(gout + (int64_t)vo[j] * Co + c) : zero_pack<4>();
             nf[j] = ok ? (float)nfcount[vo[j]] : 1.f;
         }
-        const Pack<4> x = ldp<4>(in + f * C + c);
+        const Pack<4> x = on ? ld_in_expanded<R>(in + f * C + c / R) : zero_pack<4>();
         const float cf = (l16 < K) ? coeff[f * K + l16] : 0.f;
         Pack<4> s = zero_pack<4>(), w = zero_pack<4>(), t;
 #pragma unroll
@@ -483,17 +504,24 @@ __global__ __launch_bounds__(kBlock) void f2v_bwd_fast_k(const float *__restrict
         PM_A(0) PM_A(1) PM_A(2) PM_A(3) PM_A(4) PM_A(5) PM_A(6) PM_A(7)
         PM_A(8) PM_A(9) PM_A(10) PM_A(11) PM_A(12) PM_A(13) PM_A(14) PM_A(15)
 #undef PM_A
-        Pack<4> gi;
+        if (on) {
+            if constexpr (R == 1) {
+                Pack<4> gi;
 #pragma unroll
-        for (int u = 0; u < 4; ++u) gi.v[u] = s.v[u] * w.v[u];
-        stp<4>(gin + f * C + c, gi);
+                for (int u = 0; u < 4; ++u) gi.v[u] = s.v[u] * w.v[u];
+                stp<4>(gin + f * C + c, gi);
+            } else {                                  // two input channels, each the sum over its two outputs
+                *reinterpret_cast<float2 *>(gin + f * C + c / R) =
+                    make_float2(fmaf(s.v[1], w.v[1], s.v[0] * w.v[0]), fmaf(s.v[3], w.v[3], s.v[2] * w.v[2]));
+            }
+        }
 #pragma unroll
         for (int j = 0; j < 3; ++j) vo[j] = von[j];
     }
 #pragma unroll
     for (int k = 0; k < 16; ++k)
         if (k < K)
-            block_reduce_store<4>(acc[k], red, partial + ((size_t)blockIdx.x * K + k) * C + c, true, lane, slot, lpr, rpb);
+            block_reduce_store<4>(acc[k], red, partial + ((size_t)blockIdx.x * K + k) * Co + c, on, lane, slot, lpr, rpb);
 }
 
 // ----------------------------------------------------------------------------------------
@@ -750,6 +778,17 @@ __global__ __launch_bounds__(kBlock) void triangle_geometry_k(const float *__res
     g[4] = 0.5f * len;
 }
 
+// The fast facet2vertex kernels: depth multiplier 1 or 2, Co = C*r a multiple of 4 in [64, 1024] (row groups
+// of at least one 16-lane DPP row), at most 16 coefficients, 16-byte aligned rows.
+static bool f2v_fast_ok(int C, int r, int K, std::initializer_list<const void *> ptrs)
+{
+    const int Co = C * r;
+    if (!(r == 1 || r == 2) || (Co & 3) || Co < 64 || Co > 1024 || K > 16) return false;
+    for (const void *p : ptrs)
+        if (!aligned16(p)) return false;
+    return true;
+}
+
 static int reduce_partials(const float *partial, float *out, int G, int n, hipStream_t st)
 {
     reduce_partials_k<<<dim3((unsigned)ceil_div(n, 16)), dim3(1024), 0, st>>>(partial, out, G, n);
@@ -840,10 +879,14 @@ extern "C" int pmesh_f2v_fwd(const float *input, const float *filter, const floa
     const int64_t blocks = ceil_div(NvOut, rs.rpb);
     PM_REQUIRE(grid_ok(blocks), "f2v_fwd: grid too large");
     const int cvec = ((K & 3) == 0 && aligned16(coeff)) ? 1 : 0;
-    if (V == 4 && (C & 63) == 0 && C <= 1024 && K <= 16) {
+    if (f2v_fast_ok(C, r, K, {input, filter, output})) {
         // persistent: enough workgroups to fill the chip several times over, each visiting many vertices
-        const int64_t pb = blocks < 4096 ? blocks : 4096;
-        f2v_fwd_fast_k<<<dim3((unsigned)pb), dim3(kBlock), 0, st>>>(input, filter, coeff, nf_count, rowptr, colidx, output, NvOut, C, K, rs.lpr_log2);
+        const RowShape fs = row_shape(C * r / 4);
+        const int64_t fb = ceil_div(NvOut, fs.rpb), pb = fb < 4096 ? fb : 4096;
+        if (r == 1)
+            f2v_fwd_fast_k<1><<<dim3((unsigned)pb), dim3(kBlock), 0, st>>>(input, filter, coeff, nf_count, rowptr, colidx, output, NvOut, C, K, fs.lpr_log2);
+        else
+            f2v_fwd_fast_k<2><<<dim3((unsigned)pb), dim3(kBlock), 0, st>>>(input, filter, coeff, nf_count, rowptr, colidx, output, NvOut, C, K, fs.lpr_log2);
     }
     else if (V == 4)
         f2v_fwd_k<4><<<dim3((unsigned)blocks), dim3(kBlock), 0, st>>>(input, filter, coeff, nf_count, rowptr, colidx, output, NvOut, C, r, K, rs.items, rs.lpr_log2, cvec);
@@ -883,9 +926,14 @@ extern "C" int pmesh_f2v_bwd(const float *grad_output, const float *input, const
     PM_REQUIRE(workspace_bytes >= (size_t)G * K * Co * sizeof(float), "f2v_bwd: workspace too small (%zu bytes)", workspace_bytes);
     const int cvec = ((K & 3) == 0 && aligned16(coeff)) ? 1 : 0;
     float *partial = (float *)workspace;
-    if (V == 4 && (C & 63) == 0 && C <= 1024 && K <= 16)
-        f2v_bwd_fast_k<<<dim3(G), dim3(kBlock), 0, st>>>(grad_output, input, filter, coeff, face, nf_count, vt_map, grad_input, partial, Nf, NvOut, C, K, rs.lpr_log2, rows_per_block);
-    else if (V == 4)
+    if (f2v_fast_ok(C, r, K, {grad_output, input, filter, grad_input, workspace})) {
+        const RowShape fs = row_shape(Co / 4);
+        const int64_t frows = ceil_div(ceil_div(Nf, G), fs.rpb) * fs.rpb;
+        if (r == 1)
+            f2v_bwd_fast_k<1><<<dim3(G), dim3(kBlock), 0, st>>>(grad_output, input, filter, coeff, face, nf_count, vt_map, grad_input, partial, Nf, NvOut, C, K, fs.lpr_log2, frows);
+        else
+            f2v_bwd_fast_k<2><<<dim3(G), dim3(kBlock), 0, st>>>(grad_output, input, filter, coeff, face, nf_count, vt_map, grad_input, partial, Nf, NvOut, C, K, fs.lpr_log2, frows);
+    } else if (V == 4)
         f2v_bwd_k<4><<<dim3(G), dim3(kBlock), 0, st>>>(grad_output, input, filter, coeff, face, nf_count, vt_map, grad_input, partial, Nf, NvOut, C, r, K, rs.items, rs.lpr_log2, cvec, rows_per_block);
     else
         f2v_bwd_k<1><<<dim3(G), dim3(kBlock), 0, st>>>(grad_output, input, filter, coeff, face, nf_count, vt_map, grad_input, partial, Nf, NvOut, C, r, K, rs.items, rs.lpr_log2, cvec, rows_per_block);

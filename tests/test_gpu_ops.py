@@ -97,7 +97,10 @@ def test_v2f_parity(cuda, mesh, C, r):
 @pytest.mark.parametrize("mesh,C,r,K,strided", [("tetra", 4, 1, 16, False), ("octa", 6, 2, 9, True),
                                                 ("sphere2", 32, 1, 16, False), ("sphere3", 64, 1, 16, True),
                                                 ("room_small", 64, 1, 16, False), ("torus", 20, 1, 36, False),
-                                                ("sphere2", 5, 3, 4, True), ("sphere2", 128, 1, 16, False)])
+                                                ("sphere2", 5, 3, 4, True), ("sphere2", 128, 1, 16, False),
+                                                ("sphere3", 48, 2, 16, True), ("sphere3", 96, 1, 16, False),
+                                                ("room_small", 40, 2, 9, True), ("sphere2", 36, 2, 16, False),
+                                                ("sphere2", 160, 1, 12, True), ("sphere2", 64, 2, 16, False)])
 def test_f2v_parity(cuda, mesh, C, r, K, strided):
     say("case f2v", mesh, C, r, K, strided)
     v, f = mesh_case(mesh)

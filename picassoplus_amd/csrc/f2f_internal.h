@@ -10,6 +10,11 @@ bool f2f16_usable(const void *tex, const void *W, const void *sh, int Cin, int F
 int f2f16_fwd(const float *tex, const float *W, const float *sh, const int *cum, float *out, int64_t T,
               int64_t Nf, int Cin, int Cout, hipStream_t st);
 
+// The split-bf16 kernels (mesh_f2f16x3.hip) take any channel counts; they need F == 16 and 16-byte aligned
+// filter and SH arrays.  Texture rows are read 16 bytes at a time when Cin % 4 == 0 and the array is aligned,
+// element by element otherwise.
+bool f2f16x3_usable(const void *W, const void *sh, int F);
+
 // forward on the bf16 matrix cores with an exact three-way split of both operands (fp32-level accuracy)
 size_t f2f16x3_fwd_workspace_bytes(int Cin, int Cout);
 int f2f16x3_fwd(const float *tex, const float *W, const float *sh, const int *cum, const int *order, float *out,

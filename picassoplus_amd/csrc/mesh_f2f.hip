@@ -353,7 +353,7 @@ static inline bool force_fp32_mfma()
 
 extern "C" size_t pmesh_f2f_fwd_workspace_bytes(int Cin, int Cout, int F)
 {
-    return (F == 16 && (Cin & 3) == 0) ? f2f16x3_fwd_workspace_bytes(Cin, Cout) : 0;
+    return F == 16 ? f2f16x3_fwd_workspace_bytes(Cin, Cout) : 0;
 }
 
 extern "C" int pmesh_f2f_fwd(const float *texture, const float *filter, const float *bary_coeff,
@@ -366,7 +366,7 @@ extern "C" int pmesh_f2f_fwd(const float *texture, const float *filter, const fl
     if (Nf == 0) return 0;
     PM_REQUIRE(filter && cum_texture && output && (T == 0 || (texture && bary_coeff)), "f2f_fwd: null pointer");
     // the split-bf16 forward addresses texture elements with 32-bit offsets
-    if (!force_generic() && !force_fp32_mfma() && f2f16_usable(texture, filter, bary_coeff, Cin, F) &&
+    if (!force_generic() && !force_fp32_mfma() && f2f16x3_usable(filter, bary_coeff, F) &&
         T * Cin < (int64_t(1) << 31))
         return f2f16x3_fwd(texture, filter, bary_coeff, cum_texture, facet_order, output, workspace, workspace_bytes,
                            T, Nf, Cin, Cout, (hipStream_t)stream);
@@ -400,13 +400,13 @@ extern "C" int pmesh_f2f_bwd_texture(const float *grad_output, const float *filt
     PM_REQUIRE(grad_output && filter && bary_coeff && cum_texture && grad_texture, "f2f_bwd_texture: null pointer");
     f2f_zero_tail_k<<<dim3(64), dim3(kBlock), 0, (hipStream_t)stream>>>(grad_texture, cum_texture, Nf, (int)T, Cin);
     PM_LAUNCHED("f2f_bwd_texture(tail)");
-    if (!force_generic() && f2f16_usable(grad_texture, filter, bary_coeff, Cin, F)) {
-        if (!force_fp32_mfma() && f2f16x3_bwd_texture_usable(grad_output, Cout))
-            return f2f16x3_bwd_texture(grad_output, filter, bary_coeff, cum_texture, facet_order, grad_texture,
-                                       workspace, workspace_bytes, T, Nf, Cin, Cout, (hipStream_t)stream);
+    if (!force_generic() && !force_fp32_mfma() && f2f16x3_usable(filter, bary_coeff, F) &&
+        f2f16x3_bwd_texture_usable(grad_output, Cout))
+        return f2f16x3_bwd_texture(grad_output, filter, bary_coeff, cum_texture, facet_order, grad_texture, workspace,
+                                   workspace_bytes, T, Nf, Cin, Cout, (hipStream_t)stream);
+    if (!force_generic() && f2f16_usable(grad_texture, filter, bary_coeff, Cin, F))
         return f2f16_bwd_texture(grad_output, filter, bary_coeff, cum_texture, grad_texture, T, Nf, Cin, Cout,
                                  (hipStream_t)stream);
-    }
     const ChunkGeom cg = chunk_geom(Cin, F);
     const int64_t gx = ceil_div(Nf, 64);
     PM_REQUIRE(grid_ok(gx), "f2f_bwd_texture: grid too large");
@@ -437,9 +437,9 @@ extern "C" int pmesh_f2f_bwd_filter(const float *grad_output, const float *textu
     const int S = filt_splits(Nf);
     PM_REQUIRE(workspace_bytes >= (size_t)S * nW * sizeof(float), "f2f_bwd_filter: workspace too small (%zu bytes)",
                workspace_bytes);
-    if (!force_generic() && f2f16_usable(texture, texture, bary_coeff, Cin, F)) {
-        int rc = force_fp32_mfma()
-                     ? f2f16_bwd_filter_partials(grad_output, texture, bary_coeff, cum_texture, (float *)workspace, S, T,
+    const bool x3 = !force_fp32_mfma() && f2f16x3_usable(bary_coeff, bary_coeff, F);
+    if (!force_generic() && (x3 || f2f16_usable(texture, texture, bary_coeff, Cin, F))) {
+        int rc = !x3 ? f2f16_bwd_filter_partials(grad_output, texture, bary_coeff, cum_texture, (float *)workspace, S, T,
                                                  Nf, Cin, Cout, st)
                      : f2f16x3_bwd_filter_partials(grad_output, texture, bary_coeff, cum_texture, facet_order,
                                                    (float *)workspace, S, T, Nf, Cin, Cout, st);

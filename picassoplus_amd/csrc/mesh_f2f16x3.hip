@@ -30,6 +30,19 @@ constexpr int kXKB = 4;                       // texture points per facet covere
 constexpr int kXChunk = 4 * 2 * 3 * 64;       // uint4 per LDS buffer: 4 channels x 2 tiles x 3 pieces x 64 lanes
 
 __device__ __forceinline__ float4 xld4(const float *p) { return *reinterpret_cast<const float4 *>(p); }
+// four consecutive channels of a texture row of which `n` (may be <= 0 or > 4) exist; VEC: the rows are
+// 16-byte aligned and the channel count is a multiple of 4 (compile time, so that the common case keeps
+// its straight 16-byte loads)
+template <bool VEC> __device__ __forceinline__ float4 xld4_row(const float *p, int n)
+{
+    if constexpr (VEC) return n > 0 ? xld4(p) : make_float4(0.f, 0.f, 0.f, 0.f);
+    float4 r;
+    r.x = n > 0 ? p[0] : 0.f;
+    r.y = n > 1 ? p[1] : 0.f;
+    r.z = n > 2 ? p[2] : 0.f;
+    r.w = n > 3 ? p[3] : 0.f;
+    return r;
+}
 __device__ __forceinline__ unsigned fbits(float x) { return __builtin_bit_cast(unsigned, x); }
 __device__ __forceinline__ float bitsf(unsigned u) { return __builtin_bit_cast(float, u); }
 // {hi16(b), hi16(a)}: two truncated bf16 values in one register, a in the low half
@@ -73,16 +86,16 @@ __device__ __forceinline__ int xwave_max(int v)
 // eight bf16 pieces of W[nt*32 + l32][ci][8h .. 8h+7], lane = 32h + l32.  NT = even number of
 // 32-channel tiles covering Cout (zero padded).
 __global__ __launch_bounds__(kBlock) void f2f16x3_pack_filter_k(const float *__restrict__ W, u32x4 *__restrict__ Wp,
-                                                                int Cin, int Cout, int NT)
+                                                                int Cin, int CinPad, int Cout, int NT)
 {
     const int idx = blockIdx.x * kBlock + threadIdx.x;
-    if (idx >= Cin * NT * 64) return;
+    if (idx >= CinPad * NT * 64) return;
     const int lane = idx & 63, nt = (idx >> 6) % NT, ci = (idx >> 6) / NT;
     const int co = nt * 32 + (lane & 31), h = lane >> 5;
     float x[8];
 #pragma unroll
     for (int j = 0; j < 8; ++j) x[j] = 0.f;
-    if (co < Cout) {
+    if (co < Cout && ci < Cin) {                      // channels Cin .. CinPad-1 are zero rows
         const float *p = W + ((int64_t)co * Cin + ci) * 16 + 8 * h;
         const float4 u = xld4(p), v = xld4(p + 4);
         x[0] = u.x; x[1] = u.y; x[2] = u.z; x[3] = u.w; x[4] = v.x; x[5] = v.y; x[6] = v.z; x[7] = v.w;
@@ -119,7 +132,7 @@ __device__ __forceinline__ void w_chunk_fetch(const u32x4 *__restrict__ Wp, int 
 //     from which every lane picks its own facets' values;
 //   filter: chunks of four channels copied to LDS two chunks ahead (shared by the workgroup).
 // Both are published right before the workgroup barrier that ends a chunk.
-template <int KW>
+template <int KW, bool TVEC>
 __device__ __forceinline__ void x3_sweep(const float *__restrict__ tex, const u32x4 *__restrict__ Wp,
                                          const float *__restrict__ sh, u32x4 *Ws, float *slab, f32x16 (&acc)[kFR][2],
                                          const int (&kbase)[kFR], const int (&Ks)[kFR], const float (&invK)[kFR],
@@ -159,7 +172,7 @@ __device__ __forceinline__ void x3_sweep(const float *__restrict__ tex, const u3
     auto fetch_group = [&](int g) {
 #pragma unroll
         for (int i = 0; i < NL; ++i)
-            pf[i] = (ldok[i] && 8 * g + cg4 < Cin) ? xld4(tex + (ldoff[i] + 8 * g)) : make_float4(0.f, 0.f, 0.f, 0.f);
+            pf[i] = ldok[i] ? xld4_row<TVEC>(tex + (ldoff[i] + 8 * g), Cin - (8 * g + cg4)) : make_float4(0.f, 0.f, 0.f, 0.f);
     };
     auto publish_group = [&](float *dst) {
 #pragma unroll
@@ -235,7 +248,7 @@ __device__ __forceinline__ void x3_sweep(const float *__restrict__ tex, const u3
             u32x4 bn[2][3];
             float tvnn[kFR][KW];
             // c+1 == Cin reads a chunk buffer / slab row that exists but is not used
-            read_b(bn, c + 1 < Cin ? c + 1 : c);
+            read_b(bn, c + 1 < 4 * nblk ? c + 1 : c);
             read_tv(tvnn, c + 2);
 
             float an[kFR][8];
@@ -278,6 +291,7 @@ __device__ __forceinline__ void x3_sweep(const float *__restrict__ tex, const u3
 // `order` (may be null) lists the facets sorted by their number of texture points, so that the 256
 // facets of a workgroup -- and the 32*kFR of a wavefront -- have (nearly) equal counts: the work per
 // sweep is set by the longest facet, and facets with more than kXKB points need further sweeps.
+template <bool TVEC>
 __global__ __launch_bounds__(kFThreads, 2 / kFR) void f2f16x3_fwd_k(const float *__restrict__ tex,
                                                                    const u32x4 *__restrict__ Wp,
                                                                    const float *__restrict__ sh,
@@ -293,7 +307,7 @@ __global__ __launch_bounds__(kFThreads, 2 / kFR) void f2f16x3_fwd_k(const float 
     const int l32 = lane & 31, h = lane >> 5;
     const int64_t s0 = (int64_t)blockIdx.x * 256;
     const int nt0 = blockIdx.y * 2, n0 = blockIdx.y * 64;
-    const int nblk = Cin >> 2;
+    const int nblk = (Cin + 3) >> 2;
 
     if (threadIdx.x == 0) s_kmax = 0;
     for (int i = threadIdx.x; i < 256; i += kFThreads) {
@@ -346,7 +360,7 @@ __global__ __launch_bounds__(kFThreads, 2 / kFR) void f2f16x3_fwd_k(const float 
         }
         // every variant runs the same barriers, so wavefronts of a workgroup may pick different ones
         kw = xwave_max(kw);
-#define PM_X3(N) x3_sweep<N>(tex, Wp, sh, Ws, s_slab + w * 2 * kXSlab, acc, kbase, Ks, invK, s_k0, s_K, sw, Cin, NT, nt0, nblk, w, lane, h)
+#define PM_X3(N) x3_sweep<N, TVEC>(tex, Wp, sh, Ws, s_slab + w * 2 * kXSlab, acc, kbase, Ks, invK, s_k0, s_K, sw, Cin, NT, nt0, nblk, w, lane, h)
         if (kw <= 1) PM_X3(1);
         else if (kw == 2) PM_X3(2);
         else if (kw == 3) PM_X3(3);
@@ -413,7 +427,7 @@ __global__ __launch_bounds__(kBlock) void f2f16x3_pack_filter_t_k(const float *_
     dst[0] = p1; dst[64] = p2; dst[128] = p3;
 }
 
-template <int KW, int NKS>
+template <int KW, int NKS, bool GVEC>
 __device__ __forceinline__ void x3_tex_sweep(const u32x4 *__restrict__ WpT, const float *__restrict__ sh,
                                              float *__restrict__ gtex, u32x4 *Ws, float *stage, const int *w_k0,
                                              const int *w_K, const u32x4 (&bp)[NKS][3], int kbase, int Ks, float invK,
@@ -464,9 +478,18 @@ __device__ __forceinline__ void x3_tex_sweep(const u32x4 *__restrict__ WpT, cons
             const int k0s = w_k0[slot] + sweep * kXKB, Kss = w_K[slot] - sweep * kXKB;
 #pragma unroll
             for (int kk = 0; kk < KW; ++kk)
-                if (kk < Kss && ci < Cin)
-                    *reinterpret_cast<float4 *>(gtex + (int64_t)(k0s + kk) * Cin + ci) =
-                        *reinterpret_cast<const float4 *>(stage + (kk * 32 + slot) * 16 + 4 * (lane & 3));
+                if (kk < Kss && ci < Cin) {
+                    const float4 v = *reinterpret_cast<const float4 *>(stage + (kk * 32 + slot) * 16 + 4 * (lane & 3));
+                    float *dst = gtex + (int64_t)(k0s + kk) * Cin + ci;
+                    if constexpr (GVEC) {
+                        *reinterpret_cast<float4 *>(dst) = v;
+                    } else {                               // channel count not a multiple of 4 / unaligned rows
+                        dst[0] = v.x;
+                        if (ci + 1 < Cin) dst[1] = v.y;
+                        if (ci + 2 < Cin) dst[2] = v.z;
+                        if (ci + 3 < Cin) dst[3] = v.w;
+                    }
+                }
         }
     };
     // Results go out 64 bytes at a time: two groups (16 channels) of every point are collected in
@@ -549,7 +572,7 @@ __device__ __forceinline__ void x3_tex_sweep(const u32x4 *__restrict__ WpT, cons
 // NKS = k-steps of 16 output channels (compile time, so that a tile's MFMAs and the previous tile's
 // contraction share one basic block and get interleaved): 2 for Cout <= 32, else 4; the packed filter
 // is zero padded to that many.
-template <int NKS>
+template <int NKS, bool GVEC>
 __global__ __launch_bounds__(512, 2) void f2f16x3_bwd_tex_k(const float *__restrict__ gout,
                                                             const u32x4 *__restrict__ WpT,
                                                             const float *__restrict__ sh,
@@ -607,7 +630,7 @@ __global__ __launch_bounds__(512, 2) void f2f16x3_bwd_tex_k(const float *__restr
         const int kw = xwave_max(Ks);
         const int kbase = k0 + sw * kXKB;
         // every variant runs the same barriers, so wavefronts of a workgroup may pick different ones
-#define PM_X3T(N) x3_tex_sweep<N, NKS>(WpT, sh, gtex, Ws, s_stage[w], s_k0[w], s_K[w], bp, kbase, Ks, invK, sw, Cin, NG, lane, h)
+#define PM_X3T(N) x3_tex_sweep<N, NKS, GVEC>(WpT, sh, gtex, Ws, s_stage[w], s_k0[w], s_K[w], bp, kbase, Ks, invK, sw, Cin, NG, lane, h)
         if (kw <= 1) PM_X3T(1);
         else if (kw == 2) PM_X3T(2);
         else if (kw == 3) PM_X3T(3);
@@ -782,7 +805,7 @@ __device__ __forceinline__ void xpre_commit(const XPre &P, u32x4 *go, float *shs
 
 // texture rows of one pass (KW points per facet) for my wavefront's 16 channels: 64 bytes per row,
 // four lanes per row
-template <int KW>
+template <int KW, bool TVEC>
 __device__ __forceinline__ void xtex_issue(float4 (&pf)[2 * kXKB], const float *__restrict__ tex, const int *sk0,
                                            const int *sK, int sweep, int cw, int Cin, int lane)
 {
@@ -790,8 +813,9 @@ __device__ __forceinline__ void xtex_issue(float4 (&pf)[2 * kXKB], const float *
 #pragma unroll
     for (int i = 0; i < 2 * KW; ++i) {
         const int rr = i * 16 + (lane >> 2), kk = rr >> 5, slot = rr & 31;
-        const bool ok = sweep * kXKB + kk < sK[slot] && cw + 4 * piece < Cin;
-        pf[i] = ok ? xld4(tex + (int64_t)(sk0[slot] + sweep * kXKB + kk) * Cin + cw + 4 * piece)
+        const bool ok = sweep * kXKB + kk < sK[slot];
+        pf[i] = ok ? xld4_row<TVEC>(tex + (int64_t)(sk0[slot] + sweep * kXKB + kk) * Cin + cw + 4 * piece,
+                                    Cin - (cw + 4 * piece))
                    : make_float4(0.f, 0.f, 0.f, 0.f);
     }
 }
@@ -800,7 +824,7 @@ __device__ __forceinline__ int xtile_kmax(const int *sK, int lane) { return xwav
 
 // One tile of 32 facets whose inputs are in LDS buffer it % 2 (descriptors in it % 3): start the
 // fetches for the next tile, run the passes, publish the next tile's inputs.
-template <int KW>
+template <int KW, bool TVEC>
 __device__ __forceinline__ void x3_filt_tile(const float *__restrict__ gout, const float *__restrict__ tex,
                                              const float *__restrict__ sh, const int *__restrict__ cum,
                                              const int *__restrict__ order, u32x4 (*go_s)[2 * 2 * 3 * 64], float4 *slab,
@@ -850,7 +874,7 @@ __device__ __forceinline__ void x3_filt_tile(const float *__restrict__ gout, con
         {
             // my wavefront's texture rows of this pass -> slab
             float4 pf[2 * kXKB];
-            xtex_issue<KW>(pf, tex, s_k0[sb], s_K[sb], sw, cw, Cin, lane);
+            xtex_issue<KW, TVEC>(pf, tex, s_k0[sb], s_K[sb], sw, cw, Cin, lane);
             const int piece = lane & 3;
 #pragma unroll
             for (int i = 0; i < 2 * KW; ++i) {
@@ -868,6 +892,7 @@ __device__ __forceinline__ void x3_filt_tile(const float *__restrict__ gout, con
     __syncthreads();
 }
 
+template <bool TVEC>
 __global__ __launch_bounds__(256, 1) void f2f16x3_bwd_filt_k(const float *__restrict__ gout,
                                                               const float *__restrict__ tex,
                                                               const float *__restrict__ sh,
@@ -929,7 +954,7 @@ __global__ __launch_bounds__(256, 1) void f2f16x3_bwd_filt_k(const float *__rest
     int it = 0;
 #define PM_PHASE(N)                                                                                                  \
     for (; tile < ntiles && (N == kXKB || xtile_kmax(s_K[it % 3], lane) <= N); ++it, tile += stride)                 \
-        x3_filt_tile<N>(gout, tex, sh, cum, order, go_s, slab_s + w * (kXKB * 4 * 32), sh_s, s_f, s_k0, s_K, acc, ea, eb,  \
+        x3_filt_tile<N, TVEC>(gout, tex, sh, cum, order, go_s, slab_s + w * (kXKB * 4 * 32), sh_s, s_f, s_k0, s_K, acc, ea, eb,  \
                         it, tile, stride, ntiles, Nf, T, Cin, Cout, c0, n0, lane, w)
     PM_PHASE(1);
     PM_PHASE(2);
@@ -961,16 +986,25 @@ int f2f16x3_bwd_filter_partials(const float *gout, const float *tex, const float
     const int64_t gy = ceil_div(Cin, 64), gz = ceil_div(Cout, 64);
     PM_REQUIRE(gy <= 65535 && gz <= 65535, "f2f_bwd_filter: grid too large");
     const int64_t ntiles = ceil_div(Nf, 32);
-    f2f16x3_bwd_filt_k<<<dim3((unsigned)splits, (unsigned)gy, (unsigned)gz), dim3(256), 0, st>>>(
-        gout, tex, sh, cum, order, partial, Nf, (int)T, Cin, Cout, ntiles);
+    if (!(Cin & 3) && !(reinterpret_cast<uintptr_t>(tex) & 15u))
+        f2f16x3_bwd_filt_k<true><<<dim3((unsigned)splits, (unsigned)gy, (unsigned)gz), dim3(256), 0, st>>>(
+            gout, tex, sh, cum, order, partial, Nf, (int)T, Cin, Cout, ntiles);
+    else
+        f2f16x3_bwd_filt_k<false><<<dim3((unsigned)splits, (unsigned)gy, (unsigned)gz), dim3(256), 0, st>>>(
+            gout, tex, sh, cum, order, partial, Nf, (int)T, Cin, Cout, ntiles);
     PM_LAUNCHED("f2f_bwd_filter");
     return 0;
 }
 
+bool f2f16x3_usable(const void *W, const void *sh, int F)
+{
+    return F == 16 && !(reinterpret_cast<uintptr_t>(W) & 15u) && !(reinterpret_cast<uintptr_t>(sh) & 15u);
+}
+
 size_t f2f16x3_fwd_workspace_bytes(int Cin, int Cout)
 {
-    const int NT = 2 * ((Cout + 63) / 64);
-    return (size_t)Cin * NT * 3 * 64 * sizeof(u32x4);
+    const int NT = 2 * ((Cout + 63) / 64), CinPad = (Cin + 3) & ~3;
+    return (size_t)CinPad * NT * 3 * 64 * sizeof(u32x4);
 }
 
 int f2f16x3_fwd(const float *tex, const float *W, const float *sh, const int *cum, const int *order, float *out,
@@ -982,12 +1016,15 @@ int f2f16x3_fwd(const float *tex, const float *W, const float *sh, const int *cu
                "f2f_fwd: workspace too small (%zu bytes)", workspace_bytes);
     PM_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 15u) == 0, "f2f_fwd: workspace must be 16-byte aligned");
     u32x4 *Wp = (u32x4 *)workspace;
-    const int n = Cin * NT * 64;
-    f2f16x3_pack_filter_k<<<dim3((unsigned)ceil_div(n, kBlock)), dim3(kBlock), 0, st>>>(W, Wp, Cin, Cout, NT);
+    const int CinPad = (Cin + 3) & ~3, n = CinPad * NT * 64;
+    f2f16x3_pack_filter_k<<<dim3((unsigned)ceil_div(n, kBlock)), dim3(kBlock), 0, st>>>(W, Wp, Cin, CinPad, Cout, NT);
     PM_LAUNCHED("f2f_fwd(pack)");
     const int64_t gx = ceil_div(Nf, 256), gy = NT / 2;
     PM_REQUIRE(grid_ok(gx) && gy <= 65535, "f2f_fwd: grid too large");
-    f2f16x3_fwd_k<<<dim3((unsigned)gx, (unsigned)gy), dim3(kFThreads), 0, st>>>(tex, Wp, sh, cum, order, out, Nf, (int)T, Cin, Cout, NT);
+    if (!(Cin & 3) && !(reinterpret_cast<uintptr_t>(tex) & 15u))
+        f2f16x3_fwd_k<true><<<dim3((unsigned)gx, (unsigned)gy), dim3(kFThreads), 0, st>>>(tex, Wp, sh, cum, order, out, Nf, (int)T, Cin, Cout, NT);
+    else
+        f2f16x3_fwd_k<false><<<dim3((unsigned)gx, (unsigned)gy), dim3(kFThreads), 0, st>>>(tex, Wp, sh, cum, order, out, Nf, (int)T, Cin, Cout, NT);
     PM_LAUNCHED("f2f_fwd");
     return 0;
 }
@@ -1014,10 +1051,13 @@ int f2f16x3_bwd_texture(const float *gout, const float *W, const float *sh, cons
     PM_LAUNCHED("f2f_bwd_texture(pack)");
     const int64_t gx = ceil_div(Nf, 256);
     PM_REQUIRE(grid_ok(gx), "f2f_bwd_texture: grid too large");
-    if (NKS == 2)
-        f2f16x3_bwd_tex_k<2><<<dim3((unsigned)gx), dim3(512), 0, st>>>(gout, WpT, sh, cum, order, gtex, Nf, (int)T, Cin, Cout, NG);
-    else
-        f2f16x3_bwd_tex_k<4><<<dim3((unsigned)gx), dim3(512), 0, st>>>(gout, WpT, sh, cum, order, gtex, Nf, (int)T, Cin, Cout, NG);
+    const bool gvec = !(Cin & 3) && !(reinterpret_cast<uintptr_t>(gtex) & 15u);
+#define PM_TEX(N, G) f2f16x3_bwd_tex_k<N, G><<<dim3((unsigned)gx), dim3(512), 0, st>>>(gout, WpT, sh, cum, order, gtex, Nf, (int)T, Cin, Cout, NG)
+    if (NKS == 2 && gvec) PM_TEX(2, true);
+    else if (NKS == 2) PM_TEX(2, false);
+    else if (gvec) PM_TEX(4, true);
+    else PM_TEX(4, false);
+#undef PM_TEX
     PM_LAUNCHED("f2f_bwd_texture");
     return 0;
 }

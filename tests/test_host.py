@@ -41,7 +41,8 @@ def test_size_queries_are_host_only():
     assert _lib.query("pmesh_f2v_bwd_workspace_bytes", 64, 1, 16) == 1024 * 16 * 64 * 4
     assert _lib.query("pmesh_f2f_bwd_workspace_bytes", 64, 64, 16) == 256 * 64 * 64 * 16 * 4
     assert _lib.query("pmesh_f2f_fwd_workspace_bytes", 64, 64, 16) == 64 * 2 * 3 * 64 * 16
-    assert _lib.query("pmesh_f2f_fwd_workspace_bytes", 3, 64, 16) == 0
+    assert _lib.query("pmesh_f2f_fwd_workspace_bytes", 3, 64, 16) == 4 * 2 * 3 * 64 * 16      # channels padded to 4
+    assert _lib.query("pmesh_f2f_fwd_workspace_bytes", 3, 64, 9) == 0
     assert _lib.query("pmesh_facet_order_workspace_bytes", 1000) >= 3 * 1000 * 4
     assert _lib.query("pmesh_vertex_csr_workspace_bytes", 1000, 500) >= 3 * 3000 * 4
     assert _lib.query("pmesh_cluster_csr_workspace_bytes", 1000, 250) >= 3 * 1000 * 4

@@ -33,7 +33,10 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="scene", choices=["scene", "shapes", "pool"])
+    ap.add_argument("--workload", default="scene", choices=["scene", "shapes", "pool", "firstblock"],
+                    help="scene: the headline layer (F2F+F2V, C=64); shapes: 16 small meshes V2F+F2F+F2V; pool: "
+                         "1024x1024 grid max/avg pool + unpool; firstblock: the scene batch with the reference's first "
+                         "block shapes, F2F 3->64 then F2V 64->64 with depth multiplier 2 (pi2_blocks.py:113-130)")
     ap.add_argument("--scale", type=float, default=1.0, help="facet-count scale of the scene workload")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -43,7 +46,7 @@ def parse():
 
 
 # ---------------------------------------------------------------------------- inputs
-def build_conv_inputs(mesh, C, L, seed, tex_counts="area"):
+def build_conv_inputs(mesh, C, L, seed, tex_counts="area", Cin=None, r=1):
     from picassoplus_amd import synthetic as S
     rng = np.random.default_rng(seed)
     v, f = mesh["vertex"], mesh["face"]
@@ -53,12 +56,12 @@ def build_conv_inputs(mesh, C, L, seed, tex_counts="area"):
     counts, bary, owner = S.texture_points(rng, nf, counts)
     B = (L + 1) ** 2
     return dict(
-        nv=nv, nf=nf, T=int(counts.sum()), C=C, B=B, L=L, face=f, normal=normal.astype(np.float32),
+        nv=nv, nf=nf, T=int(counts.sum()), C=C, Cin=Cin or C, r=r, B=B, L=L, face=f, normal=normal.astype(np.float32),
         counts=counts, bary=bary.astype(np.float32), owner=owner,
         vt_map=np.arange(nv, dtype=np.int32), nf_count=np.maximum(S.vertex_facet_count(f, np.arange(nv), nv), 1),
         x=rng.uniform(-1, 1, (nv, C)).astype(np.float32),
-        w_f2f=S.xavier_uniform(rng, (C, C, B), C * B, C * B).astype(np.float32),
-        w_f2v=S.xavier_uniform(rng, (B, C, 1), C, B * C).astype(np.float32),
+        w_f2f=S.xavier_uniform(rng, (C, Cin or C, B), (Cin or C) * B, C * B).astype(np.float32),
+        w_f2v=S.xavier_uniform(rng, (B, C, r), C, B * C * r).astype(np.float32),
         w_v2f=S.xavier_uniform(rng, (3, C, 1), C, 3 * C).astype(np.float32),
         mf_in=mesh["mf_in"], nv_in=mesh["nv_in"])
 
@@ -66,14 +69,15 @@ def build_conv_inputs(mesh, C, L, seed, tex_counts="area"):
 def conv_bytes_flops(d, ops):
     """Algorithmic HBM bytes / flops per op: every input read once, every output written once."""
     Nf, Nv, T, C, B = d["nf"], d["nv"], d["T"], d["C"], d["B"]
+    Ci, r = d["Cin"], d["r"]                    # F2F input channels; F2V depth multiplier (output width C * r)
     tab = {
         "v2f_fwd": (4 * Nv * C + 12 * Nf + 4 * Nf * C, 6 * Nf * C),
         "v2f_bwd": (4 * Nf * C + 12 * Nf + 8 * Nv * C, 12 * Nf * C),
-        "f2v_fwd": (4 * Nf * C + 4 * Nf * B + 12 * Nf + 8 * Nv + 4 * Nv * C, Nf * C * (2 * B + 7)),
-        "f2v_bwd": (4 * Nv * C + 8 * Nf * C + 4 * Nf * B + 12 * Nf + 8 * Nv, Nf * C * (4 * B + 12)),
-        "f2f_fwd": (4 * T * C + 4 * T * B + 4 * Nf + 4 * C * C * B + 4 * Nf * C, 2 * T * C * B + 2 * Nf * C * B * C),
-        "f2f_bwd_texture": (4 * Nf * C + 4 * T * B + 4 * Nf + 4 * C * C * B + 4 * T * C, 2 * Nf * C * B * C + 2 * T * C * B),
-        "f2f_bwd_filter": (4 * Nf * C + 4 * T * C + 4 * T * B + 4 * Nf + 4 * C * C * B, 2 * Nf * C * B * C + 2 * T * C * B),
+        "f2v_fwd": (4 * Nf * C + 4 * Nf * B + 12 * Nf + 8 * Nv + 4 * Nv * C * r, Nf * C * r * (2 * B + 7)),
+        "f2v_bwd": (4 * Nv * C * r + 8 * Nf * C + 4 * Nf * B + 12 * Nf + 8 * Nv, Nf * C * r * (4 * B + 12)),
+        "f2f_fwd": (4 * T * Ci + 4 * T * B + 4 * Nf + 4 * C * Ci * B + 4 * Nf * C, 2 * T * Ci * B + 2 * Nf * Ci * B * C),
+        "f2f_bwd_texture": (4 * Nf * C + 4 * T * B + 4 * Nf + 4 * C * Ci * B + 4 * T * Ci, 2 * Nf * Ci * B * C + 2 * T * Ci * B),
+        "f2f_bwd_filter": (4 * Nf * C + 4 * T * Ci + 4 * T * B + 4 * Nf + 4 * C * Ci * B, 2 * Nf * Ci * B * C + 2 * T * Ci * B),
     }
     return {k: tab[k] for k in ops}
 
@@ -117,11 +121,12 @@ def run_conv_layer(args, torch, kind):
     from picassoplus_amd.mesh.pi_modules import conv3d
     dev = torch.device("cuda:0")
     C, L = 64, 3
-    if kind == "scene":
+    Cin, r = (3, 2) if kind == "firstblock" else (C, 1)      # F2F input channels, F2V depth multiplier
+    if kind in ("scene", "firstblock"):
         mesh = S.scene_workload(seed=3000, n_rooms=8, scale=args.scale)
-        d = build_conv_inputs(mesh, C, L, seed=3000)
+        d = build_conv_inputs(mesh, C, L, seed=3000, Cin=Cin, r=r)
         ops = ["f2f_fwd", "f2v_fwd", "f2v_bwd", "f2f_bwd_texture", "f2f_bwd_filter"]
-        name = "scene8x300k_F2F+F2V_C64_L3_fp32_fwd+bwd"
+        name = "scene8x300k_F2F+F2V_C64_L3_fp32_fwd+bwd" if kind == "scene" else "scene8x300k_F2F3to64+F2Vr2_L3_fp32_fwd+bwd"
     else:
         mesh = S.shapes_workload(seed=2000, n_meshes=16)
         d = build_conv_inputs(mesh, C, L, seed=2000, tex_counts=3)
@@ -135,18 +140,19 @@ def run_conv_layer(args, torch, kind):
     x = t(d["x"])
     # texture-point features: barycentric interpolation of the vertex features (set-up, untimed)
     corner = face.long()[owner]
-    tex = (x[corner[:, 0]] * bary[:, 0:1] + x[corner[:, 1]] * bary[:, 1:2] + x[corner[:, 2]] * bary[:, 2:3]).contiguous()
+    tex = (x[corner[:, 0]] * bary[:, 0:1] + x[corner[:, 1]] * bary[:, 1:2] + x[corner[:, 2]] * bary[:, 2:3])
+    tex = tex[:, :Cin].contiguous()                          # first block: three colour-like channels
     del corner, owner
     sh = sph_harm_values(bary, L)
     coeff = sph_harm_values(t(d["normal"]), L)
     w_f2f, w_f2v, w_v2f = t(d["w_f2f"]), t(d["w_f2v"]), t(d["w_v2f"])
-    gy = torch.randn(d["nv"], C, device=dev, generator=torch.Generator(device=dev).manual_seed(1))
+    gy = torch.randn(d["nv"], C * r, device=dev, generator=torch.Generator(device=dev).manual_seed(1))
     tex.requires_grad_(True); w_f2f.requires_grad_(True); w_f2v.requires_grad_(True)
     if kind == "shapes":
         x.requires_grad_(True); w_v2f.requires_grad_(True)
 
     def step():
-        if kind == "scene":
+        if kind in ("scene", "firstblock"):
             y1 = conv3d.facet2facet(tex, w_f2f, sh, cum)
             y = conv3d.facet2vertex(y1, w_f2v, coeff, face, nfc, vt_map)
             return torch.autograd.grad(y, [tex, w_f2f, w_f2v], gy)
@@ -174,7 +180,7 @@ def run_conv_layer(args, torch, kind):
     total_bytes = sum(b for b, _ in bf.values())
     dom = max(ops, key=lambda k: per_op.get(k, 0.0))
     dom_ms = per_op[dom]
-    if dom.startswith("f2f"):
+    if dom.startswith("f2f") and Cin >= 16:
         roof = dict(bound="mfma", achieved=bf[dom][1] / (dom_ms * 1e-3) / 1e12, peak=MFMA_F32_PEAK_TFLOPS, unit="TFLOP/s")
     else:
         roof = dict(bound="hbm", achieved=bf[dom][0] / (dom_ms * 1e-3) / 1e9, peak=HBM_PEAK_GBS, unit="GB/s")
@@ -211,10 +217,11 @@ def cpu_baseline_conv(d, kind, torch, budget_s=12.0):
         own = torch.from_numpy(d["owner"][ta:tb] - int(fa))
         corner = f.long()[own]
         tex = x[corner[:, 0]] * bary[:, 0:1] + x[corner[:, 1]] * bary[:, 1:2] + x[corner[:, 2]] * bary[:, 2:3]
+        tex = tex[:, :d["Cin"]].contiguous()
         sh, coeff = R.sph_harm(bary, d["L"]), R.sph_harm(torch.from_numpy(d["normal"][fa:fb]), d["L"])
         vt_map = torch.arange(nv, dtype=torch.int32)
         nfc = torch.from_numpy(d["nf_count"][va:vb].astype(np.int32))
-        gy = torch.randn(nv, d["C"])
+        gy = torch.randn(nv, d["C"] * d["r"])
         t0 = time.perf_counter()
         y1 = R.f2f_fwd(tex, w_f2f, sh, cum)
         if kind == "shapes":

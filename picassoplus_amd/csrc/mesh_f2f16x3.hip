@@ -647,18 +647,18 @@ __global__ __launch_bounds__(512, 2) void f2f16x3_bwd_tex_k(const float *__restr
 // layout of an MFMA operand whose reduction index is the facet.  Two input channels share one
 // transposition tile (columns 0..15 / 16..31).  The facet order inside a reduction step is the
 // accumulator's row order; the gout operand is built with the same order.
-//   workgroup  4 wavefronts (one per SIMD, accumulators in 256 registers), 64 input x 64 output
+//   workgroup  4 wavefronts (one per SIMD, accumulators in up to 256 registers), 64 input x 64 output
 //              channels, a strided subset of the 32-facet tiles of the sorted facet list
-//   wavefront  16 input channels = 8 channel pairs x 2 output tiles of gW^T[(ci,d)][co]
+//   wavefront  16 input channels = 8 channel pairs x 2 output tiles of gW^T[(ci,d)][co]; filters with
+//              fewer than 64 input channels give every wavefront 1, 2 or 4 pairs instead (NCP)
 //   gout^T     per facet tile split and laid out per lane in LDS by the whole workgroup
-constexpr int kGCi = 16;                         // input channels of a wavefront
 
 // One pass = up to KW texture points per facet (missing points contribute zeros), straight-line code.
 // shr: SH values of my facet's points (my half's eight d's, scaled by 1/K); slab: the wavefront's
 // texture values [point][16-byte piece][facet slot]; go: the tile's gout^T operand.
-template <int KW>
+template <int KW, int NCP>
 __device__ __forceinline__ void x3_filt_pass(const float (&shr)[KW][8], const float4 *slab, const u32x4 *go,
-                                             f32x16 (&acc)[8][2], const u32x4 &ea, const u32x4 &eb, int lane)
+                                             f32x16 (&acc)[NCP][2], const u32x4 &ea, const u32x4 &eb, int lane)
 {
     const int l32 = lane & 31;
     // G of channels cbase + 2cp (a) and + 1 (b), eight d's of my half for my facet, as bf16 pieces
@@ -724,9 +724,9 @@ __device__ __forceinline__ void x3_filt_pass(const float (&shr)[KW][8], const fl
         transpose(o, pa, pb);
     }
 #pragma unroll
-    for (int cp = 0; cp < 8; ++cp) {
+    for (int cp = 0; cp < NCP; ++cp) {
         u32x4 pa[3], pb[3];
-        if (cp + 1 < 8) gen(pa, pb, cp + 1);
+        if (cp + 1 < NCP) gen(pa, pb, cp + 1);
 #pragma unroll
         for (int st = 0; st < 2; ++st) {
             // six piece products, smallest first; the two output tiles alternate so that no MFMA
@@ -739,7 +739,7 @@ __device__ __forceinline__ void x3_filt_pass(const float (&shr)[KW][8], const fl
                 for (int t = 0; t < 2; ++t) acc[cp][t] = mfma_bf16(o[ga][st], g[st][t][wb], acc[cp][t]);
             }
         }
-        if (cp + 1 < 8) transpose(o, pa, pb);
+        if (cp + 1 < NCP) transpose(o, pa, pb);
     }
 }
 
@@ -805,7 +805,7 @@ __device__ __forceinline__ void xpre_commit(const XPre &P, u32x4 *go, float *shs
 
 // texture rows of one pass (KW points per facet) for my wavefront's 16 channels: 64 bytes per row,
 // four lanes per row
-template <int KW, bool TVEC>
+template <int KW, bool TVEC, int NCP>
 __device__ __forceinline__ void xtex_issue(float4 (&pf)[2 * kXKB], const float *__restrict__ tex, const int *sk0,
                                            const int *sK, int sweep, int cw, int Cin, int lane)
 {
@@ -813,7 +813,7 @@ __device__ __forceinline__ void xtex_issue(float4 (&pf)[2 * kXKB], const float *
 #pragma unroll
     for (int i = 0; i < 2 * KW; ++i) {
         const int rr = i * 16 + (lane >> 2), kk = rr >> 5, slot = rr & 31;
-        const bool ok = sweep * kXKB + kk < sK[slot];
+        const bool ok = sweep * kXKB + kk < sK[slot] && 4 * piece < 2 * NCP;
         pf[i] = ok ? xld4_row<TVEC>(tex + (int64_t)(sk0[slot] + sweep * kXKB + kk) * Cin + cw + 4 * piece,
                                     Cin - (cw + 4 * piece))
                    : make_float4(0.f, 0.f, 0.f, 0.f);
@@ -824,12 +824,12 @@ __device__ __forceinline__ int xtile_kmax(const int *sK, int lane) { return xwav
 
 // One tile of 32 facets whose inputs are in LDS buffer it % 2 (descriptors in it % 3): start the
 // fetches for the next tile, run the passes, publish the next tile's inputs.
-template <int KW, bool TVEC>
+template <int KW, bool TVEC, int NCP>
 __device__ __forceinline__ void x3_filt_tile(const float *__restrict__ gout, const float *__restrict__ tex,
                                              const float *__restrict__ sh, const int *__restrict__ cum,
                                              const int *__restrict__ order, u32x4 (*go_s)[2 * 2 * 3 * 64], float4 *slab,
                                              float (*sh_s)[kXKB * 32 * 16], int (*s_f)[32], int (*s_k0)[32],
-                                             int (*s_K)[32], f32x16 (&acc)[8][2], const u32x4 &ea, const u32x4 &eb,
+                                             int (*s_K)[32], f32x16 (&acc)[NCP][2], const u32x4 &ea, const u32x4 &eb,
                                              int it, int64_t tile, int64_t stride, int64_t ntiles, int64_t Nf, int T,
                                              int Cin, int Cout, int c0, int n0, int lane, int w)
 {
@@ -844,8 +844,9 @@ __device__ __forceinline__ void x3_filt_tile(const float *__restrict__ gout, con
     const int k0 = s_k0[sb][l32], K = s_K[sb][l32];
     const float invK = K > 0 ? 1.0f / (float)K : 0.f;
     const int nsweeps = KW < kXKB ? 1 : (xwave_max(K) + kXKB - 1) / kXKB;
-    const int cw = c0 + kGCi * w;                        // my wavefront's first input channel
-    for (int sw = 0; sw < nsweeps; ++sw) {
+    const int cw = c0 + 2 * NCP * w;                     // my wavefront's first input channel
+    const bool idle = cw >= Cin;                         // narrow filters leave wavefronts without channels
+    for (int sw = 0; sw < nsweeps && !idle; ++sw) {
         const int rem = K - sw * kXKB;
         const int Ks = rem < 0 ? 0 : (rem > KW ? KW : rem);
         float shr[KW][8];
@@ -874,7 +875,7 @@ __device__ __forceinline__ void x3_filt_tile(const float *__restrict__ gout, con
         {
             // my wavefront's texture rows of this pass -> slab
             float4 pf[2 * kXKB];
-            xtex_issue<KW, TVEC>(pf, tex, s_k0[sb], s_K[sb], sw, cw, Cin, lane);
+            xtex_issue<KW, TVEC, NCP>(pf, tex, s_k0[sb], s_K[sb], sw, cw, Cin, lane);
             const int piece = lane & 3;
 #pragma unroll
             for (int i = 0; i < 2 * KW; ++i) {
@@ -882,7 +883,7 @@ __device__ __forceinline__ void x3_filt_tile(const float *__restrict__ gout, con
                 slab[(kk * 4 + piece) * 32 + slot] = pf[i];
             }
         }
-        x3_filt_pass<KW>(shr, slab, go_s[buf], acc, ea, eb, lane);
+        x3_filt_pass<KW, NCP>(shr, slab, go_s[buf], acc, ea, eb, lane);
     }
 
     xpre_commit(P, go_s[buf ^ 1], sh_s[buf ^ 1]);
@@ -892,7 +893,9 @@ __device__ __forceinline__ void x3_filt_tile(const float *__restrict__ gout, con
     __syncthreads();
 }
 
-template <bool TVEC>
+// NCP = channel pairs of a wavefront (8 for 64 or more input channels; fewer for narrow filters, so that
+// the four wavefronts share what channels there are)
+template <bool TVEC, int NCP>
 __global__ __launch_bounds__(256, 1) void f2f16x3_bwd_filt_k(const float *__restrict__ gout,
                                                               const float *__restrict__ tex,
                                                               const float *__restrict__ sh,
@@ -907,7 +910,7 @@ __global__ __launch_bounds__(256, 1) void f2f16x3_bwd_filt_k(const float *__rest
     __shared__ int s_f[3][32], s_k0[3][32], s_K[3][32];
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
     const int l32 = lane & 31, h = lane >> 5;
-    const int c0 = blockIdx.y * 64, n0 = blockIdx.z * 64;
+    const int c0 = blockIdx.y * (8 * NCP), n0 = blockIdx.z * 64;
 
     // selection operands of the transposition: column n < 16 takes d = n of channel a, n >= 16 takes d = n - 16 of b
     u32x4 ea, eb;
@@ -924,9 +927,9 @@ __global__ __launch_bounds__(256, 1) void f2f16x3_bwd_filt_k(const float *__rest
         eb[jj] = vb;
     }
 
-    f32x16 acc[8][2];
+    f32x16 acc[NCP][2];
 #pragma unroll
-    for (int cp = 0; cp < 8; ++cp)
+    for (int cp = 0; cp < NCP; ++cp)
 #pragma unroll
         for (int t = 0; t < 2; ++t)
 #pragma unroll
@@ -954,7 +957,7 @@ __global__ __launch_bounds__(256, 1) void f2f16x3_bwd_filt_k(const float *__rest
     int it = 0;
 #define PM_PHASE(N)                                                                                                  \
     for (; tile < ntiles && (N == kXKB || xtile_kmax(s_K[it % 3], lane) <= N); ++it, tile += stride)                 \
-        x3_filt_tile<N, TVEC>(gout, tex, sh, cum, order, go_s, slab_s + w * (kXKB * 4 * 32), sh_s, s_f, s_k0, s_K, acc, ea, eb,  \
+        x3_filt_tile<N, TVEC, NCP>(gout, tex, sh, cum, order, go_s, slab_s + w * (kXKB * 4 * 32), sh_s, s_f, s_k0, s_K, acc, ea, eb,  \
                         it, tile, stride, ntiles, Nf, T, Cin, Cout, c0, n0, lane, w)
     PM_PHASE(1);
     PM_PHASE(2);
@@ -966,13 +969,13 @@ __global__ __launch_bounds__(256, 1) void f2f16x3_bwd_filt_k(const float *__rest
     // = (channel c0 + 16w + 2cp + m/16, d = m%16); four consecutive d's per group of four registers
     float *dst = partial + (int64_t)blockIdx.x * Cout * Cin * 16;
 #pragma unroll
-    for (int cp = 0; cp < 8; ++cp)
+    for (int cp = 0; cp < NCP; ++cp)
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
             const int co = n0 + 32 * t + l32;
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
-                const int ci = c0 + kGCi * w + 2 * cp + (q >> 1);
+                const int ci = c0 + 2 * NCP * w + 2 * cp + (q >> 1);
                 if (co < Cout && ci < Cin)
                     *reinterpret_cast<float4 *>(dst + ((int64_t)co * Cin + ci) * 16 + 8 * (q & 1) + 4 * h) =
                         make_float4(acc[cp][t][4 * q], acc[cp][t][4 * q + 1], acc[cp][t][4 * q + 2], acc[cp][t][4 * q + 3]);
@@ -983,15 +986,21 @@ __global__ __launch_bounds__(256, 1) void f2f16x3_bwd_filt_k(const float *__rest
 int f2f16x3_bwd_filter_partials(const float *gout, const float *tex, const float *sh, const int *cum, const int *order,
                                  float *partial, int splits, int64_t T, int64_t Nf, int Cin, int Cout, hipStream_t st)
 {
-    const int64_t gy = ceil_div(Cin, 64), gz = ceil_div(Cout, 64);
+    // channel pairs per wavefront: the four wavefronts of a workgroup share up to 32 pairs
+    const int pairs = (Cin + 1) / 2;
+    const int ncp = pairs >= 32 ? 8 : pairs > 8 ? 4 : pairs > 4 ? 2 : 1;
+    const int64_t gy = ceil_div(Cin, 8 * ncp), gz = ceil_div(Cout, 64);
     PM_REQUIRE(gy <= 65535 && gz <= 65535, "f2f_bwd_filter: grid too large");
     const int64_t ntiles = ceil_div(Nf, 32);
-    if (!(Cin & 3) && !(reinterpret_cast<uintptr_t>(tex) & 15u))
-        f2f16x3_bwd_filt_k<true><<<dim3((unsigned)splits, (unsigned)gy, (unsigned)gz), dim3(256), 0, st>>>(
-            gout, tex, sh, cum, order, partial, Nf, (int)T, Cin, Cout, ntiles);
-    else
-        f2f16x3_bwd_filt_k<false><<<dim3((unsigned)splits, (unsigned)gy, (unsigned)gz), dim3(256), 0, st>>>(
-            gout, tex, sh, cum, order, partial, Nf, (int)T, Cin, Cout, ntiles);
+    const bool tvec = !(Cin & 3) && !(reinterpret_cast<uintptr_t>(tex) & 15u);
+    const dim3 grid((unsigned)splits, (unsigned)gy, (unsigned)gz);
+#define PM_FILT(V, N) f2f16x3_bwd_filt_k<V, N><<<grid, dim3(256), 0, st>>>(gout, tex, sh, cum, order, partial, Nf, (int)T, Cin, Cout, ntiles)
+    if (tvec) {
+        if (ncp == 8) PM_FILT(true, 8); else if (ncp == 4) PM_FILT(true, 4); else if (ncp == 2) PM_FILT(true, 2); else PM_FILT(true, 1);
+    } else {
+        if (ncp == 8) PM_FILT(false, 8); else if (ncp == 4) PM_FILT(false, 4); else if (ncp == 2) PM_FILT(false, 2); else PM_FILT(false, 1);
+    }
+#undef PM_FILT
     PM_LAUNCHED("f2f_bwd_filter");
     return 0;
 }

@@ -405,9 +405,9 @@ constexpr int kTKS = 4;                          // k-steps of 16 output channel
 constexpr int kTChunkMax = 2 * kTKS * 3 * 64;    // uint4 per chunk buffer: 2 tiles x k-steps x 3 pieces x 64 lanes
 
 // W (Cout, Cin, 16) -> A operands of the transposed product:
-// WpT[((tt*NKS + ks)*3 + piece)*64 + lane] = pieces of W[16ks + 8h .. +7][ci(tt, r)][d(r)], r = lane % 32
+// WpT[((tt*NKS + ks)*3 + piece)*64 + lane] = pieces of W[co0 + 16ks + 8h .. +7][ci(tt, r)][d(r)], r = lane % 32
 __global__ __launch_bounds__(kBlock) void f2f16x3_pack_filter_t_k(const float *__restrict__ W, u32x4 *__restrict__ WpT,
-                                                                  int Cin, int Cout, int NTt, int NKS)
+                                                                  int Cin, int Cout, int NTt, int NKS, int co0)
 {
     const int idx = blockIdx.x * kBlock + threadIdx.x;
     if (idx >= NTt * NKS * 64) return;
@@ -418,7 +418,7 @@ __global__ __launch_bounds__(kBlock) void f2f16x3_pack_filter_t_k(const float *_
     float x[8];
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
-        const int co = 16 * ks + 8 * h + j;
+        const int co = co0 + 16 * ks + 8 * h + j;             // this launch covers channels co0 .. co0 + 16 NKS - 1
         x[j] = (ci < Cin && co < Cout) ? W[((int64_t)co * Cin + ci) * 16 + d] : 0.f;
     }
     u32x4 p1, p2, p3;
@@ -431,7 +431,7 @@ template <int KW, int NKS, bool GVEC>
 __device__ __forceinline__ void x3_tex_sweep(const u32x4 *__restrict__ WpT, const float *__restrict__ sh,
                                              float *__restrict__ gtex, u32x4 *Ws, float *stage, const int *w_k0,
                                              const int *w_K, const u32x4 (&bp)[NKS][3], int kbase, int Ks, float invK,
-                                             int sweep, int Cin, int NG, int lane, int h)
+                                             int sweep, int Cin, int NG, bool add, int lane, int h)
 {
     // SH values of my facet's points for my half's eight d's (4h..4h+3, 8+4h..8+4h+3), pre-scaled by 1/K
     float shr[KW][8];
@@ -481,13 +481,19 @@ __device__ __forceinline__ void x3_tex_sweep(const u32x4 *__restrict__ WpT, cons
                 if (kk < Kss && ci < Cin) {
                     const float4 v = *reinterpret_cast<const float4 *>(stage + (kk * 32 + slot) * 16 + 4 * (lane & 3));
                     float *dst = gtex + (int64_t)(k0s + kk) * Cin + ci;
+                    // `add`: a later block of 64 output channels accumulates onto what the earlier ones wrote
                     if constexpr (GVEC) {
-                        *reinterpret_cast<float4 *>(dst) = v;
+                        float4 o = v;
+                        if (add) {
+                            const float4 p = *reinterpret_cast<const float4 *>(dst);
+                            o = make_float4(p.x + v.x, p.y + v.y, p.z + v.z, p.w + v.w);
+                        }
+                        *reinterpret_cast<float4 *>(dst) = o;
                     } else {                               // channel count not a multiple of 4 / unaligned rows
-                        dst[0] = v.x;
-                        if (ci + 1 < Cin) dst[1] = v.y;
-                        if (ci + 2 < Cin) dst[2] = v.z;
-                        if (ci + 3 < Cin) dst[3] = v.w;
+                        dst[0] = add ? dst[0] + v.x : v.x;
+                        if (ci + 1 < Cin) dst[1] = add ? dst[1] + v.y : v.y;
+                        if (ci + 2 < Cin) dst[2] = add ? dst[2] + v.z : v.z;
+                        if (ci + 3 < Cin) dst[3] = add ? dst[3] + v.w : v.w;
                     }
                 }
         }
@@ -578,7 +584,7 @@ __global__ __launch_bounds__(512, 2) void f2f16x3_bwd_tex_k(const float *__restr
                                                             const float *__restrict__ sh,
                                                             const int *__restrict__ cum,
                                                             const int *__restrict__ order, float *__restrict__ gtex,
-                                                            int64_t Nf, int T, int Cin, int Cout, int NG)
+                                                            int64_t Nf, int T, int Cin, int Cout, int NG, int co0)
 {
     __shared__ u32x4 Ws[3 * kTChunkMax];
     __shared__ __attribute__((aligned(16))) float s_stage[8][kXKB * 32 * 16];
@@ -614,7 +620,7 @@ __global__ __launch_bounds__(512, 2) void f2f16x3_bwd_tex_k(const float *__restr
         float x[8];
 #pragma unroll
         for (int j = 0; j < 8; ++j) x[j] = 0.f;
-        const int co = 16 * ks + 8 * h;
+        const int co = co0 + 16 * ks + 8 * h;
         if (K > 0 && co < Cout) {
             const float *p = gout + (int64_t)f * Cout + co;
             const float4 u = xld4(p), v = xld4(p + 4);
@@ -630,7 +636,7 @@ __global__ __launch_bounds__(512, 2) void f2f16x3_bwd_tex_k(const float *__restr
         const int kw = xwave_max(Ks);
         const int kbase = k0 + sw * kXKB;
         // every variant runs the same barriers, so wavefronts of a workgroup may pick different ones
-#define PM_X3T(N) x3_tex_sweep<N, NKS, GVEC>(WpT, sh, gtex, Ws, s_stage[w], s_k0[w], s_K[w], bp, kbase, Ks, invK, sw, Cin, NG, lane, h)
+#define PM_X3T(N) x3_tex_sweep<N, NKS, GVEC>(WpT, sh, gtex, Ws, s_stage[w], s_k0[w], s_K[w], bp, kbase, Ks, invK, sw, Cin, NG, co0 > 0, lane, h)
         if (kw <= 1) PM_X3T(1);
         else if (kw == 2) PM_X3T(2);
         else if (kw == 3) PM_X3T(3);
@@ -1040,34 +1046,39 @@ int f2f16x3_fwd(const float *tex, const float *W, const float *sh, const int *cu
 
 size_t f2f16x3_bwd_texture_workspace_bytes(int Cin, int Cout)
 {
-    const int NG = (Cin + 7) / 8, NKS = Cout <= 32 ? 2 : 4;
+    const int NG = (Cin + 7) / 8, NKS = Cout <= 32 ? 2 : 4;       // one block of at most 64 output channels at a time
     return (size_t)NG * 4 * NKS * 3 * 64 * sizeof(u32x4);
 }
 
-bool f2f16x3_bwd_texture_usable(const void *gout, int Cout) { return Cout <= 16 * kTKS && (Cout & 7) == 0 && (reinterpret_cast<uintptr_t>(gout) & 15u) == 0; }
+bool f2f16x3_bwd_texture_usable(const void *gout, int Cout) { return (Cout & 7) == 0 && (reinterpret_cast<uintptr_t>(gout) & 15u) == 0; }
 
 int f2f16x3_bwd_texture(const float *gout, const float *W, const float *sh, const int *cum, const int *order,
                         float *gtex, void *workspace, size_t workspace_bytes, int64_t T, int64_t Nf, int Cin,
                         int Cout, hipStream_t st)
 {
-    const int NG = (Cin + 7) / 8, NKS = Cout <= 32 ? 2 : 4;
+    const int NG = (Cin + 7) / 8;
     PM_REQUIRE(workspace && workspace_bytes >= f2f16x3_bwd_texture_workspace_bytes(Cin, Cout),
                "f2f_bwd_texture: workspace too small (%zu bytes)", workspace_bytes);
     PM_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 15u) == 0, "f2f_bwd_texture: workspace must be 16-byte aligned");
     u32x4 *WpT = (u32x4 *)workspace;
-    const int n = NG * 4 * NKS * 64;
-    f2f16x3_pack_filter_t_k<<<dim3((unsigned)ceil_div(n, kBlock)), dim3(kBlock), 0, st>>>(W, WpT, Cin, Cout, NG * 4, NKS);
-    PM_LAUNCHED("f2f_bwd_texture(pack)");
     const int64_t gx = ceil_div(Nf, 256);
     PM_REQUIRE(grid_ok(gx), "f2f_bwd_texture: grid too large");
     const bool gvec = !(Cin & 3) && !(reinterpret_cast<uintptr_t>(gtex) & 15u);
-#define PM_TEX(N, G) f2f16x3_bwd_tex_k<N, G><<<dim3((unsigned)gx), dim3(512), 0, st>>>(gout, WpT, sh, cum, order, gtex, Nf, (int)T, Cin, Cout, NG)
-    if (NKS == 2 && gvec) PM_TEX(2, true);
-    else if (NKS == 2) PM_TEX(2, false);
-    else if (gvec) PM_TEX(4, true);
-    else PM_TEX(4, false);
+    // output channels go 64 at a time; the first block writes grad_texture, the others add to it
+    // (launches on one stream run in order, so the packed filter buffer is reused)
+    for (int co0 = 0; co0 < Cout; co0 += 64) {
+        const int NKS = Cout - co0 <= 32 ? 2 : 4;
+        const int n = NG * 4 * NKS * 64;
+        f2f16x3_pack_filter_t_k<<<dim3((unsigned)ceil_div(n, kBlock)), dim3(kBlock), 0, st>>>(W, WpT, Cin, Cout, NG * 4, NKS, co0);
+        PM_LAUNCHED("f2f_bwd_texture(pack)");
+#define PM_TEX(N, G) f2f16x3_bwd_tex_k<N, G><<<dim3((unsigned)gx), dim3(512), 0, st>>>(gout, WpT, sh, cum, order, gtex, Nf, (int)T, Cin, Cout, NG, co0)
+        if (NKS == 2 && gvec) PM_TEX(2, true);
+        else if (NKS == 2) PM_TEX(2, false);
+        else if (gvec) PM_TEX(4, true);
+        else PM_TEX(4, false);
 #undef PM_TEX
-    PM_LAUNCHED("f2f_bwd_texture");
+        PM_LAUNCHED("f2f_bwd_texture");
+    }
     return 0;
 }
 

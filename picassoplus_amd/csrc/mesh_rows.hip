@@ -139,38 +139,56 @@ __global__ __launch_bounds__(kBlock) void v2f_bwd_k(const float *__restrict__ go
                 fk[k] = active ? ldp<V>(filt + k * Co + co) : zero_pack<V>();
                 acc[k] = zero_pack<V>();
             }
-            if (active)
-                for (int64_t row = rbeg + slot; row < rend; row += rpb) {
-                    const int e0 = rowptr[row], e1 = rowptr[row + 1];
+            if (active) {
+                // entries of a vertex are taken eight at a time, all their gathers issued before any use;
+                // the bounds of the next row are requested while this one is summed
+                constexpr int EB = 8;
+                int64_t row = rbeg + slot;
+                int e0 = 0, e1 = 0;
+                if (row < rend) { e0 = rowptr[row]; e1 = rowptr[row + 1]; }
+                for (; row < rend; row += rpb) {
+                    int ne0 = 0, ne1 = 0;
+                    if (row + rpb < rend) { ne0 = rowptr[row + rpb]; ne1 = rowptr[row + rpb + 1]; }
                     const Pack<V> x = ldp<V>(in + row * C + c);
                     Pack<V> g = zero_pack<V>(), s[3];
 #pragma unroll
                     for (int k = 0; k < 3; ++k) s[k] = zero_pack<V>();
-                    for (int e = e0; e < e1; ++e) {
-                        const int ent = colidx[e];
-                        const int f = ent / 3, k = ent - 3 * f;
-                        const Pack<V> go = ldp<V>(gout + (int64_t)f * Co + co);
+                    for (int eb = e0; eb < e1; eb += EB) {
+                        int ent[EB];
 #pragma unroll
-                        for (int i = 0; i < V; ++i) {
-                            const float w = (k == 0) ? fk[0].v[i] : (k == 1) ? fk[1].v[i] : fk[2].v[i];
-                            g.v[i] = fmaf(go.v[i], w, g.v[i]);
-                            s[0].v[i] += (k == 0) ? go.v[i] : 0.f;
-                            s[1].v[i] += (k == 1) ? go.v[i] : 0.f;
-                            s[2].v[i] += (k == 2) ? go.v[i] : 0.f;
+                        for (int i = 0; i < EB; ++i) ent[i] = (eb + i < e1) ? colidx[eb + i] : -1;
+                        Pack<V> go[EB];
+#pragma unroll
+                        for (int i = 0; i < EB; ++i)
+                            go[i] = (ent[i] >= 0) ? ldp<V>(gout + (int64_t)(ent[i] / 3) * Co + co) : zero_pack<V>();
+#pragma unroll
+                        for (int i = 0; i < EB; ++i) {
+                            const int k = ent[i] - 3 * (ent[i] / 3);          // corner; masked entries carry zeros
+#pragma unroll
+                            for (int u = 0; u < V; ++u) {
+                                const float w = (k == 0) ? fk[0].v[u] : (k == 1) ? fk[1].v[u] : fk[2].v[u];
+                                g.v[u] = fmaf(go[i].v[u], w, g.v[u]);
+                                s[0].v[u] += (k == 0) ? go[i].v[u] : 0.f;
+                                s[1].v[u] += (k == 1) ? go[i].v[u] : 0.f;
+                                s[2].v[u] += (k == 2) ? go[i].v[u] : 0.f;
+                            }
                         }
                     }
 #pragma unroll
                     for (int k = 0; k < 3; ++k)
 #pragma unroll
-                        for (int i = 0; i < V; ++i) acc[k].v[i] = fmaf(s[k].v[i], x.v[i], acc[k].v[i]);
+                        for (int u = 0; u < V; ++u) acc[k].v[u] = fmaf(s[k].v[u], x.v[u], acc[k].v[u]);
                     float *gp = gin + row * C + c;
                     if (m == 0) {
                         stp<V>(gp, g);
                     } else {
 #pragma unroll
-                        for (int i = 0; i < V; ++i) gp[i] += g.v[i];
+                        for (int u = 0; u < V; ++u) gp[u] += g.v[u];
                     }
+                    e0 = ne0;
+                    e1 = ne1;
                 }
+            }
 #pragma unroll
             for (int k = 0; k < 3; ++k)
                 block_reduce_store<V>(acc[k], red, partial + ((size_t)blockIdx.x * 3 + k) * Co + co, active,

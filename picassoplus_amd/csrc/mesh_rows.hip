@@ -579,15 +579,26 @@ __global__ __launch_bounds__(kBlock) void pool_max_fwd_k(const float *__restrict
         int idx[V];
 #pragma unroll
         for (int i = 0; i < V; ++i) idx[i] = 0;
-        for (int e = e0; e < e1; ++e) {
-            const int v = members[e];
-            const Pack<V> x = ldp<V>(in + (int64_t)v * C + c);
+        // members four at a time: their rows are all requested before the first comparison
+        constexpr int EB = 4;
+        for (int eb = e0; eb < e1; eb += EB) {
+            int v[EB];
 #pragma unroll
-            for (int i = 0; i < V; ++i) {
-                const float b = best.v[i], y = x.v[i];
-                const bool take = (e == e0) || (y > b) || (b != b && y == y);
-                best.v[i] = take ? y : b;
-                idx[i] = take ? ((y == y) ? v : 0) : idx[i];
+            for (int j = 0; j < EB; ++j) v[j] = (eb + j < e1) ? members[eb + j] : -1;
+            Pack<V> x[EB];
+#pragma unroll
+            for (int j = 0; j < EB; ++j) x[j] = (v[j] >= 0) ? ldp<V>(in + (int64_t)v[j] * C + c) : zero_pack<V>();
+#pragma unroll
+            for (int j = 0; j < EB; ++j) {
+                if (eb + j < e1) {
+#pragma unroll
+                    for (int i = 0; i < V; ++i) {
+                        const float b = best.v[i], y = x[j].v[i];
+                        const bool take = (eb + j == e0) || (y > b) || (b != b && y == y);
+                        best.v[i] = take ? y : b;
+                        idx[i] = take ? ((y == y) ? v[j] : 0) : idx[i];
+                    }
+                }
             }
         }
         stp<V>(out + row * C + c, best);
@@ -618,17 +629,33 @@ __global__ __launch_bounds__(kBlock) void cluster_sum_k(const float *__restrict_
     for (int q = lane; q < Q; q += lpr) {
         const int c = q * V;
         Pack<V> acc = zero_pack<V>();
-        for (int e = e0; e < e1; ++e) {
-            const int64_t v = members[e];
-            float wgt = 1.f;
-            if constexpr (AVG) {
-                const int rp = vtrep[v];
-                const int64_t rep = rp < 0 ? -(int64_t)rp : v;
-                wgt = 1.0f / (float)(vtrep[rep < NvFine ? rep : v] + 1);
-            }
-            const Pack<V> x = ldp<V>(in + v * C + c);
+        // members four at a time: indices, then all rows (and the cluster size), then the sums in member order
+        constexpr int EB = 4;
+        for (int eb = e0; eb < e1; eb += EB) {
+            int64_t v[EB];
 #pragma unroll
-            for (int i = 0; i < V; ++i) acc.v[i] = AVG ? fmaf(x.v[i], wgt, acc.v[i]) : acc.v[i] + x.v[i];
+            for (int j = 0; j < EB; ++j) v[j] = (eb + j < e1) ? members[eb + j] : -1;
+            Pack<V> x[EB];
+            float wgt[EB];
+            int rp[EB], cnt[EB];
+#pragma unroll
+            for (int j = 0; j < EB; ++j) {
+                x[j] = (v[j] >= 0) ? ldp<V>(in + v[j] * C + c) : zero_pack<V>();
+                rp[j] = (AVG && v[j] >= 0) ? vtrep[v[j]] : 0;
+            }
+#pragma unroll
+            for (int j = 0; j < EB; ++j) {                 // cluster size, stored at the representative
+                const int64_t rep = rp[j] < 0 ? -(int64_t)rp[j] : v[j];
+                cnt[j] = (AVG && v[j] >= 0) ? vtrep[rep < NvFine ? rep : v[j]] : 0;
+            }
+#pragma unroll
+            for (int j = 0; j < EB; ++j) wgt[j] = AVG ? 1.0f / (float)(cnt[j] + 1) : 1.f;
+#pragma unroll
+            for (int j = 0; j < EB; ++j)
+                if (eb + j < e1) {
+#pragma unroll
+                    for (int i = 0; i < V; ++i) acc.v[i] = AVG ? fmaf(x[j].v[i], wgt[j], acc.v[i]) : acc.v[i] + x[j].v[i];
+                }
         }
         stp<V>(out + row * C + c, acc);
     }

@@ -664,6 +664,11 @@ __global__ __launch_bounds__(kBlock) void cluster_sum_k(const float *__restrict_
 // per-fine-vertex gathers from the cluster's coarse row.
 enum FineMode { kUnpoolFwd = 0, kAvgBwd = 1, kMaxBwdGather = 2 };
 
+// A row group takes kFineBatch consecutive fine vertices and walks the index chain
+// vt_replace -> vt_map (-> cluster size) -> coarse row for all of them in step, so that the three
+// dependent round trips are paid once per batch.
+constexpr int kFineBatch = 4;
+
 template <int V, int MODE>
 __global__ __launch_bounds__(kBlock) void fine_gather_k(const float *__restrict__ coarse,
                                                         const int *__restrict__ maxidx,
@@ -672,29 +677,56 @@ __global__ __launch_bounds__(kBlock) void fine_gather_k(const float *__restrict_
                                                         float *__restrict__ fine, int64_t NvFine,
                                                         int64_t NvCoarse, int C, int Q, int lpr_log2)
 {
+    constexpr int NB = kFineBatch;
     const int lpr = 1 << lpr_log2;
     const int lane = threadIdx.x & (lpr - 1), slot = threadIdx.x >> lpr_log2;
-    const int64_t v = (int64_t)blockIdx.x * (kBlock >> lpr_log2) + slot;
-    if (v >= NvFine) return;
-    int cnt = 1;
-    const int vo = cluster_of(vtrep, vtmap, v, NvFine, NvCoarse, &cnt);
+    const int64_t v0 = ((int64_t)blockIdx.x * (kBlock >> lpr_log2) + slot) * NB;
+    if (v0 >= NvFine) return;
+    int rp[NB], vo[NB], cnt[NB];
+    int64_t rep[NB];
+#pragma unroll
+    for (int j = 0; j < NB; ++j) rp[j] = (v0 + j < NvFine) ? vtrep[v0 + j] : 0;
+#pragma unroll
+    for (int j = 0; j < NB; ++j) {
+        rep[j] = rp[j] < 0 ? -(int64_t)rp[j] : v0 + j;
+        const bool ok = v0 + j < NvFine && rep[j] < NvFine;
+        vo[j] = ok ? vtmap[rep[j]] : -1;
+        cnt[j] = (ok && MODE == kAvgBwd) ? vtrep[rep[j]] + 1 : 1;
+        if (vo[j] >= NvCoarse) vo[j] = -1;
+    }
     for (int q = lane; q < Q; q += lpr) {
         const int c = q * V;
-        Pack<V> o = zero_pack<V>();
-        if (vo >= 0) {
-            const Pack<V> g = ldp<V>(coarse + (int64_t)vo * C + c);
-            if constexpr (MODE == kUnpoolFwd) {
-                o = g;
-            } else if constexpr (MODE == kAvgBwd) {
-                const float d = (float)cnt;
+        Pack<V> g[NB];
 #pragma unroll
-                for (int i = 0; i < V; ++i) o.v[i] = g.v[i] / d;
-            } else {
+        for (int j = 0; j < NB; ++j) g[j] = (vo[j] >= 0) ? ldp<V>(coarse + (int64_t)vo[j] * C + c) : zero_pack<V>();
+        if constexpr (MODE == kMaxBwdGather) {
+            int mi[NB][V];
 #pragma unroll
-                for (int i = 0; i < V; ++i) o.v[i] = (maxidx[(int64_t)vo * C + c + i] == (int)v) ? g.v[i] : 0.f;
+            for (int j = 0; j < NB; ++j) {
+                if constexpr (V == 4) {
+                    const int4 m4 = (vo[j] >= 0) ? *reinterpret_cast<const int4 *>(maxidx + (int64_t)vo[j] * C + c)
+                                                 : make_int4(-1, -1, -1, -1);
+                    mi[j][0] = m4.x; mi[j][1] = m4.y; mi[j][2] = m4.z; mi[j][3] = m4.w;
+                } else {
+#pragma unroll
+                    for (int i = 0; i < V; ++i) mi[j][i] = (vo[j] >= 0) ? maxidx[(int64_t)vo[j] * C + c + i] : -1;
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < NB; ++j)
+#pragma unroll
+                for (int i = 0; i < V; ++i) g[j].v[i] = (mi[j][i] == (int)(v0 + j)) ? g[j].v[i] : 0.f;
+        } else if constexpr (MODE == kAvgBwd) {
+#pragma unroll
+            for (int j = 0; j < NB; ++j) {
+                const float d = (float)cnt[j];
+#pragma unroll
+                for (int i = 0; i < V; ++i) g[j].v[i] = g[j].v[i] / d;
             }
         }
-        stp<V>(fine + v * C + c, o);
+#pragma unroll
+        for (int j = 0; j < NB; ++j)
+            if (v0 + j < NvFine) stp<V>(fine + (v0 + j) * C + c, g[j]);
     }
 }
 
@@ -1019,7 +1051,7 @@ static int launch_fine_gather(const char *name, const float *coarse, const int32
 {
     const int V = pick_v(C, 1, {coarse, fine, maxidx ? (const void *)maxidx : (const void *)coarse});
     const RowShape rs = row_shape(C / V);
-    const int64_t blocks = ceil_div(NvFine, rs.rpb);
+    const int64_t blocks = ceil_div(NvFine, (int64_t)rs.rpb * kFineBatch);
     PM_REQUIRE(grid_ok(blocks), "%s: grid too large", name);
     if (V == 4)
         fine_gather_k<4, MODE><<<dim3((unsigned)blocks), dim3(kBlock), 0, st>>>(coarse, maxidx, vtrep, vtmap, fine, NvFine, NvCoarse, C, rs.items, rs.lpr_log2);

@@ -1,0 +1,374 @@
+// facet2vertex with the filter combination on the matrix cores (fp32 MFMA), 16 SH coefficients.
+//
+//   w[e,co]   = sum_k coeff[f_e,k] * filt[k,co]        one 32 x 16 x 32 product per 32 entries and 32 channels
+//   out[v,co] = (1/nf[v]) * sum_{e of v} w[e,co] * in[f_e, co/r]
+//
+// A wavefront takes four output vertices at a time and eight adjacency entries of each: the 32 entries
+// are the rows of the product, 32 output channels its columns.  The product comes out with
+// lane = channel and registers = entries, so the facet rows are gathered one float per lane (128
+// contiguous bytes per entry) and the weighted sum over a vertex's entries stays inside a lane:
+//     register i of lane (col, h)  <->  vertex i/4 of the four, entry slot 4h + i%4 of its eight.
+// One cross-half exchange per vertex pair and channel block finishes the sum.
+// Against the vector-ALU version this replaces 64 FMAs per entry and four channels by 1/4 of an MFMA.
+#include "common.h"
+#include "rows_internal.h"
+
+namespace pmesh {
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+// vdst lanes 32..63 <-> vsrc lanes 0..31; the s_nop cover the wait states around the swap.
+__device__ __forceinline__ void half_swap(float &a, float &b)
+{
+    asm volatile("s_nop 3\n v_permlane32_swap_b32 %0, %1\n s_nop 3" : "+v"(a), "+v"(b));
+}
+
+__device__ __forceinline__ const float *at_bytes(const float *base, unsigned byte_offset)
+{
+    return reinterpret_cast<const float *>(reinterpret_cast<const char *>(base) + byte_offset);
+}
+
+// Forward.  NCB = 32-channel blocks per workgroup column (blockIdx.y selects a chunk of 32*NCB channels).
+// Requires K == 16, 16-byte aligned coefficient rows, Nf * C * 4 < 2^32.  Workgroups are persistent; the
+// eight dies take contiguous eighths of the vertices (blockIdx.x & 7 = die).
+template <int NCB>
+__global__ __launch_bounds__(kBlock) void f2v_fwd_mfma_k(const float *__restrict__ in, const float *__restrict__ filt,
+                                                         const float *__restrict__ coeff,
+                                                         const int *__restrict__ nfcount,
+                                                         const int *__restrict__ rowptr,
+                                                         const int *__restrict__ colidx, float *__restrict__ out,
+                                                         int64_t NvOut, int C, int r, int Co)
+{
+    const int l = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int col = l & 31, h = l >> 5, j = col >> 3, s = col & 7;
+    const int co0 = blockIdx.y * (32 * NCB);
+    const unsigned row_bytes = (unsigned)C * 4u;
+
+    // B operands: step kk of half h is coefficient 8h + kk (the A operand uses the same assignment)
+    float wb[NCB][8];
+    unsigned chb[NCB];
+    bool con[NCB];
+#pragma unroll
+    for (int cb = 0; cb < NCB; ++cb) {
+        const int co = co0 + 32 * cb + col;
+        con[cb] = co < Co;
+        chb[cb] = con[cb] ? (unsigned)(co / r) * 4u : 0u;
+#pragma unroll
+        for (int kk = 0; kk < 8; ++kk) wb[cb][kk] = con[cb] ? filt[(size_t)(8 * h + kk) * Co + co] : 0.f;
+    }
+
+    const int64_t groups = (NvOut + 3) >> 2, gx = (groups + 7) >> 3;
+    const int xcd = blockIdx.x & 7;
+    const int64_t gstride = (int64_t)(gridDim.x >> 3) * 4;
+    const int64_t gend = ((xcd + 1) * gx < groups) ? (xcd + 1) * gx : groups;
+    int64_t g = xcd * gx + (int64_t)(blockIdx.x >> 3) * 4 + wave;
+
+    auto bounds = [&](int64_t gg, int &a, int &b) {
+        a = 0; b = 0;
+        const int64_t v = 4 * gg + j;
+        if (gg < gend && v < NvOut) { a = rowptr[v]; b = rowptr[v + 1]; }
+    };
+    int e0, e1, ne0, ne1;
+    bounds(g, e0, e1);
+    bounds(g + gstride, ne0, ne1);
+    int f = (e0 + s < e1) ? colidx[e0 + s] / 3 : -1;
+
+    for (; g < gend; g += gstride) {
+        // row bounds two groups ahead, first entries one group ahead
+        int me0, me1;
+        bounds(g + 2 * gstride, me0, me1);
+        const int nf = (ne0 + s < ne1) ? colidx[ne0 + s] / 3 : -1;
+        // this half stores vertices 4g + 2h and 4g + 2h + 1
+        const int64_t vs = 4 * g + 2 * h;
+        const int cnt0 = (vs < NvOut) ? nfcount[vs] : 1, cnt1 = (vs + 1 < NvOut) ? nfcount[vs + 1] : 1;
+        const unsigned long long has = __builtin_amdgcn_ballot_w64(e1 > e0);      // bit 8j: vertex j has entries
+
+        float acc[NCB][4];
+#pragma unroll
+        for (int cb = 0; cb < NCB; ++cb)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) acc[cb][q] = 0.f;
+
+        for (int p = 0;; ++p) {
+            if (p > 0) f = (e0 + 8 * p + s < e1) ? colidx[e0 + 8 * p + s] / 3 : -1;
+            // A operand: coefficients 8h .. 8h+7 of my entry (zero rows for empty slots)
+            float a[8];
+            {
+                float4 t0 = make_float4(0.f, 0.f, 0.f, 0.f), t1 = t0;
+                if (f >= 0) {
+                    const float4 *cp = reinterpret_cast<const float4 *>(coeff + (int64_t)f * 16 + 8 * h);
+                    t0 = cp[0]; t1 = cp[1];
+                }
+                a[0] = t0.x; a[1] = t0.y; a[2] = t0.z; a[3] = t0.w;
+                a[4] = t1.x; a[5] = t1.y; a[6] = t1.z; a[7] = t1.w;
+            }
+            // byte offsets of the facet rows my registers pair with
+            const unsigned boff = (f >= 0) ? (unsigned)f * row_bytes : 0xFFFFFFFFu;
+            unsigned b[16];
+#pragma unroll
+            for (int i = 0; i < 16; ++i)
+                b[i] = (unsigned)__builtin_amdgcn_ds_bpermute((8 * (i >> 2) + 4 * h + (i & 3)) * 4, (int)boff);
+            float x[NCB][16];
+#pragma unroll
+            for (int cb = 0; cb < NCB; ++cb)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    x[cb][i] = 0.f;
+                    if (b[i] != 0xFFFFFFFFu && con[cb]) x[cb][i] = *at_bytes(in, b[i] + chb[cb]);
+                }
+#pragma unroll
+            for (int cb = 0; cb < NCB; ++cb) {
+                f32x16 d;
+#pragma unroll
+                for (int i = 0; i < 16; ++i) d[i] = 0.f;
+#pragma unroll
+                for (int kk = 0; kk < 8; ++kk) d = __builtin_amdgcn_mfma_f32_32x32x2f32(a[kk], wb[cb][kk], d, 0, 0, 0);
+#pragma unroll
+                for (int i = 0; i < 16; ++i) acc[cb][i >> 2] = fmaf(d[i], x[cb][i], acc[cb][i >> 2]);
+            }
+            if (!__builtin_amdgcn_ballot_w64(e0 + 8 * (p + 1) < e1)) break;
+        }
+
+        const float inv0 = ((has >> (8 * (2 * h))) & 1ull) ? 1.0f / (float)cnt0 : 0.f;
+        const float inv1 = ((has >> (8 * (2 * h + 1))) & 1ull) ? 1.0f / (float)cnt1 : 0.f;
+#pragma unroll
+        for (int cb = 0; cb < NCB; ++cb) {
+            // (acc0, acc2) and (acc1, acc3): after the swap the sums are vertex 0/1 in half 0, 2/3 in half 1
+            half_swap(acc[cb][0], acc[cb][2]);
+            half_swap(acc[cb][1], acc[cb][3]);
+            const float o0 = (acc[cb][0] + acc[cb][2]) * inv0, o1 = (acc[cb][1] + acc[cb][3]) * inv1;
+            const int co = co0 + 32 * cb + col;
+            if (con[cb]) {
+                if (vs < NvOut) out[vs * Co + co] = o0;
+                if (vs + 1 < NvOut) out[(vs + 1) * Co + co] = o1;
+            }
+        }
+        e0 = ne0; e1 = ne1; ne0 = me0; ne1 = me1;
+        f = nf;
+    }
+}
+
+
+// ----------------------------------------------------------------------------------------
+// Backward.  A wavefront takes 32 consecutive facets (rows); per 32-channel block
+//     w  = coeff_tile (32 x 16) * filt (16 x 32)                      8 MFMAs, as in the forward
+//     s  = sum over the three corners of gout[vo, co] / nf[vo]         gathered, lane = channel
+//     gin[f, co/R] = sum over the R outputs of a channel of s * w
+//     gfilt[k, co] += coeff_tile^T (16 x 32) * (in * s) (32 x 32)      16 MFMAs, two facets each; rows
+//                                                                      16..31 of the product are unused
+// Register i of lane (col, h) is facet 8(i/4) + 4h + i%4 of the tile in every one of these.  The
+// per-facet corner data (byte offset of the gout row, 1 / nf) go through a small LDS table that each
+// wavefront writes for its own tile; the index chain face -> vt_map -> nf_count runs three tiles ahead.
+// Workgroups own contiguous facet ranges (fixed by the problem size only) and leave one partial filter
+// gradient each, summed by reduce_partials in a fixed order.
+template <int NCB, int R>
+__global__ __launch_bounds__(kBlock) void f2v_bwd_mfma_k(const float *__restrict__ gout, const float *__restrict__ in,
+                                                         const float *__restrict__ filt,
+                                                         const float *__restrict__ coeff,
+                                                         const int *__restrict__ face,
+                                                         const int *__restrict__ nfcount,
+                                                         const int *__restrict__ vtmap, float *__restrict__ gin,
+                                                         float *__restrict__ partial, int64_t Nf, int64_t NvOut, int C,
+                                                         int Co, int64_t rows_per_block)
+{
+    __shared__ uint4 meta[4][32][2];
+    __shared__ float red[4][NCB * 8][64];
+    const int l = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int col = l & 31, h = l >> 5;
+    const int co0 = blockIdx.y * (32 * NCB);
+    const int G = gridDim.x;
+    // contiguous ranges per die (workgroups go round-robin over the eight dies)
+    const int64_t rb = (G & 7) ? blockIdx.x : (int64_t)(blockIdx.x & 7) * (G >> 3) + (blockIdx.x >> 3);
+    const int64_t fbeg = rb * rows_per_block;
+    const int64_t fend = (fbeg + rows_per_block < Nf) ? fbeg + rows_per_block : Nf;
+    const unsigned in_row = (unsigned)C * 4u, out_row = (unsigned)Co * 4u;
+
+    float wb[NCB][8];
+    unsigned chb[NCB], cob[NCB];
+    bool con[NCB];
+#pragma unroll
+    for (int cb = 0; cb < NCB; ++cb) {
+        const int co = co0 + 32 * cb + col;
+        con[cb] = co < Co;
+        chb[cb] = con[cb] ? (unsigned)(co / R) * 4u : 0u;
+        cob[cb] = con[cb] ? (unsigned)co * 4u : 0u;
+#pragma unroll
+        for (int kk = 0; kk < 8; ++kk) wb[cb][kk] = con[cb] ? filt[(size_t)(8 * h + kk) * Co + co] : 0.f;
+    }
+    f32x16 d2[NCB];
+#pragma unroll
+    for (int cb = 0; cb < NCB; ++cb)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) d2[cb][i] = 0.f;
+
+    auto ld_face = [&](int64_t f0, int (&va)[3]) {
+        const int64_t f = f0 + col;
+#pragma unroll
+        for (int jj = 0; jj < 3; ++jj) va[jj] = (f < fend) ? face[3 * f + jj] : -1;
+    };
+    auto ld_vo = [&](const int (&va)[3], int (&vo)[3]) {
+#pragma unroll
+        for (int jj = 0; jj < 3; ++jj) {
+            const int t = (va[jj] >= 0) ? vtmap[va[jj]] : -1;
+            vo[jj] = (t >= 0 && t < NvOut) ? t : -1;
+        }
+    };
+    auto ld_cnt = [&](const int (&vo)[3], int (&cnt)[3]) {
+#pragma unroll
+        for (int jj = 0; jj < 3; ++jj) cnt[jj] = (vo[jj] >= 0) ? nfcount[vo[jj]] : 1;
+    };
+
+    constexpr int kStep = 4 * 32;                       // facets per workgroup step
+    int64_t f0 = fbeg + 32 * wave;
+    int vo_c[3], cnt_c[3], vo_n[3], va_nn[3];
+    {
+        int va[3];
+        ld_face(f0, va); ld_vo(va, vo_c); ld_cnt(vo_c, cnt_c);
+        ld_face(f0 + kStep, va); ld_vo(va, vo_n);
+        ld_face(f0 + 2 * kStep, va_nn);
+    }
+    for (; f0 < fend; f0 += kStep) {
+        int cnt_n[3], vo_nn[3], va_3[3];
+        ld_cnt(vo_n, cnt_n);
+        ld_vo(va_nn, vo_nn);
+        ld_face(f0 + 3 * kStep, va_3);
+
+        // corner table of my tile
+        if (h == 0) {
+            uint4 m0, m1;
+            m0.x = (vo_c[0] >= 0) ? (unsigned)vo_c[0] * out_row : 0xFFFFFFFFu;
+            m0.y = (vo_c[1] >= 0) ? (unsigned)vo_c[1] * out_row : 0xFFFFFFFFu;
+            m0.z = (vo_c[2] >= 0) ? (unsigned)vo_c[2] * out_row : 0xFFFFFFFFu;
+            m0.w = 0u;
+            m1.x = __float_as_uint((vo_c[0] >= 0) ? 1.0f / (float)cnt_c[0] : 0.f);
+            m1.y = __float_as_uint((vo_c[1] >= 0) ? 1.0f / (float)cnt_c[1] : 0.f);
+            m1.z = __float_as_uint((vo_c[2] >= 0) ? 1.0f / (float)cnt_c[2] : 0.f);
+            m1.w = 0u;
+            meta[wave][col][0] = m0;
+            meta[wave][col][1] = m1;
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+
+        // A operands: my row's coefficients 8h .. 8h+7 (first product); coefficient `col` of the facets my
+        // registers pair with (second product, lanes col < 16)
+        const bool rok = f0 + col < fend;
+        float a1[8], a2[16];
+        {
+            float4 t0 = make_float4(0.f, 0.f, 0.f, 0.f), t1 = t0;
+            if (rok) {
+                const float4 *cp = reinterpret_cast<const float4 *>(coeff + (f0 + col) * 16 + 8 * h);
+                t0 = cp[0]; t1 = cp[1];
+            }
+            a1[0] = t0.x; a1[1] = t0.y; a1[2] = t0.z; a1[3] = t0.w;
+            a1[4] = t1.x; a1[5] = t1.y; a1[6] = t1.z; a1[7] = t1.w;
+        }
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int64_t fi = f0 + 8 * (i >> 2) + 4 * h + (i & 3);
+            a2[i] = (fi < fend && col < 16) ? coeff[fi * 16 + col] : 0.f;
+        }
+
+        float sv[NCB][16], xv[NCB][16];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int ri = 8 * (i >> 2) + 4 * h + (i & 3);
+            const uint4 m0 = meta[wave][ri][0], m1 = meta[wave][ri][1];
+            const bool fok = f0 + ri < fend;
+            const unsigned xoff = (unsigned)(f0 + ri) * in_row;
+#pragma unroll
+            for (int cb = 0; cb < NCB; ++cb) {
+                float g0 = 0.f, g1 = 0.f, g2 = 0.f, xx = 0.f;
+                if (m0.x != 0xFFFFFFFFu && con[cb]) g0 = *at_bytes(gout, m0.x + cob[cb]);
+                if (m0.y != 0xFFFFFFFFu && con[cb]) g1 = *at_bytes(gout, m0.y + cob[cb]);
+                if (m0.z != 0xFFFFFFFFu && con[cb]) g2 = *at_bytes(gout, m0.z + cob[cb]);
+                if (fok && con[cb]) xx = *at_bytes(in, xoff + chb[cb]);
+                sv[cb][i] = fmaf(g2, __uint_as_float(m1.z), fmaf(g1, __uint_as_float(m1.y), g0 * __uint_as_float(m1.x)));
+                xv[cb][i] = xx;
+            }
+        }
+#pragma unroll
+        for (int cb = 0; cb < NCB; ++cb) {
+            f32x16 d;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) d[i] = 0.f;
+#pragma unroll
+            for (int kk = 0; kk < 8; ++kk) d = __builtin_amdgcn_mfma_f32_32x32x2f32(a1[kk], wb[cb][kk], d, 0, 0, 0);
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const int ri = 8 * (i >> 2) + 4 * h + (i & 3);
+                float gi = sv[cb][i] * d[i];
+                if constexpr (R == 2)          // the two outputs of an input channel sit in neighbouring lanes
+                    gi += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, gi), 0xB1, 0xF, 0xF, true));
+                if (f0 + ri < fend && con[cb] && (R == 1 || !(col & 1)))
+                    *const_cast<float *>(at_bytes(gin, (unsigned)(f0 + ri) * in_row + chb[cb])) = gi;
+            }
+#pragma unroll
+            for (int i = 0; i < 16; ++i)
+                d2[cb] = __builtin_amdgcn_mfma_f32_32x32x2f32(a2[i], xv[cb][i] * sv[cb][i], d2[cb], 0, 0, 0);
+        }
+#pragma unroll
+        for (int jj = 0; jj < 3; ++jj) { vo_c[jj] = vo_n[jj]; cnt_c[jj] = cnt_n[jj]; vo_n[jj] = vo_nn[jj]; va_nn[jj] = va_3[jj]; }
+    }
+
+    // sum the four wavefronts' products; rows 0..15 (registers 0..7) are the 16 coefficients
+#pragma unroll
+    for (int cb = 0; cb < NCB; ++cb)
+#pragma unroll
+        for (int q = 0; q < 8; ++q) red[wave][cb * 8 + q][l] = d2[cb][q];
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < NCB * 8 * 64; idx += kBlock) {
+        const int ll = idx & 63, cq = idx >> 6, cb = cq >> 3, q = cq & 7;
+        const int k = 8 * (q >> 2) + 4 * (ll >> 5) + (q & 3), co = co0 + 32 * cb + (ll & 31);
+        const float v = (red[0][cq][ll] + red[1][cq][ll]) + (red[2][cq][ll] + red[3][cq][ll]);
+        if (co < Co) partial[((size_t)blockIdx.x * 16 + k) * Co + co] = v;
+    }
+}
+
+bool f2v_mfma_ok(int64_t Nf, int C, int r, int K, const void *coeff)
+{
+    return K == 16 && C * r >= 32 && (reinterpret_cast<uintptr_t>(coeff) & 15) == 0 && Nf * (int64_t)C < (int64_t(1) << 30);
+}
+
+int f2v_fwd_mfma(const float *in, const float *filt, const float *coeff, const int *nfcount, const int *rowptr,
+                 const int *colidx, float *out, int64_t NvOut, int C, int r, hipStream_t st)
+{
+    const int Co = C * r;
+    const int ncb = Co <= 32 ? 1 : Co <= 64 ? 2 : Co <= 96 ? 3 : 2;      // wider rows: chunks of 64 channels (more wavefronts in flight)
+    const unsigned gy = (unsigned)ceil_div(Co, 32 * ncb);
+    const int64_t want = ceil_div(ceil_div(NvOut, 16), 8) * 8;            // 16 vertices per workgroup sweep
+    const unsigned gxn = (unsigned)(want < 4096 ? want : 4096);
+    const dim3 grid(gxn, gy), block(kBlock);
+    switch (ncb) {
+    case 1: f2v_fwd_mfma_k<1><<<grid, block, 0, st>>>(in, filt, coeff, nfcount, rowptr, colidx, out, NvOut, C, r, Co); break;
+    case 2: f2v_fwd_mfma_k<2><<<grid, block, 0, st>>>(in, filt, coeff, nfcount, rowptr, colidx, out, NvOut, C, r, Co); break;
+    case 3: f2v_fwd_mfma_k<3><<<grid, block, 0, st>>>(in, filt, coeff, nfcount, rowptr, colidx, out, NvOut, C, r, Co); break;
+    default: f2v_fwd_mfma_k<4><<<grid, block, 0, st>>>(in, filt, coeff, nfcount, rowptr, colidx, out, NvOut, C, r, Co); break;
+    }
+    PM_LAUNCHED("f2v_fwd(mfma)");
+    return 0;
+}
+
+
+// rows_per_block and the workgroup count depend on the problem size only (fixed summation order).
+int f2v_bwd_mfma_blocks(int64_t Nf) { return persistent_blocks(Nf, 128); }
+
+int f2v_bwd_mfma(const float *gout, const float *in, const float *filt, const float *coeff, const int *face,
+                 const int *nfcount, const int *vtmap, float *gin, float *partial, int G, int64_t Nf, int64_t NvOut,
+                 int C, int r, hipStream_t st)
+{
+    const int Co = C * r;
+    const int ncb = Co <= 32 ? 1 : 2;
+    const unsigned gy = (unsigned)ceil_div(Co, 32 * ncb);
+    const int64_t rows_per_block = ceil_div(ceil_div(Nf, G), 128) * 128;
+    const dim3 grid((unsigned)G, gy), block(kBlock);
+#define PM_GO(N, RR) f2v_bwd_mfma_k<N, RR><<<grid, block, 0, st>>>(gout, in, filt, coeff, face, nfcount, vtmap, gin, partial, Nf, NvOut, C, Co, rows_per_block)
+    if (ncb == 1) { if (r == 1) PM_GO(1, 1); else PM_GO(1, 2); }
+    else          { if (r == 1) PM_GO(2, 1); else PM_GO(2, 2); }
+#undef PM_GO
+    PM_LAUNCHED("f2v_bwd(mfma)");
+    return 0;
+}
+
+}  // namespace pmesh

@@ -9,6 +9,8 @@
 // Filter gradients are reduced in two stages: per-workgroup partial sums written to a
 // workspace, then a fixed-order reduction over workgroups.
 #include "common.h"
+#include "rows_internal.h"
+#include <stdlib.h>
 #include "../../include/picasso_mesh.h"
 #include <cstdlib>
 
@@ -248,36 +250,57 @@ __global__ __launch_bounds__(kBlock) void f2v_fwd_k(const float *__restrict__ in
 
 // Lane (l & 15) of every 16-lane row holds one of 16 filter coefficients of an entry; FMAs read
 // them through DPP row broadcasts, so an entry in flight costs one register instead of sixteen.
-template <int Kk> __device__ __forceinline__ float row_bcast(float v)
-{
-    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x150 + Kk, 0xF, 0xF, false));
-}
+// PM_FMAC4_BCAST: acc[u] += bcast_k(cf) * m[u], u = 0..3, with the broadcast as the DPP operand of the
+// FMA itself (no separate move).  A DPP read of a register that a vector ALU instruction wrote needs two
+// wait states, which the compiler does not insert for inline assembly: the group for coefficient 0
+// starts with them and is declared to rewrite `cf`, so every other group of a sequence is ordered after it.
+#define PM_SRC_0 "5"
+#define PM_SRC_1 "6"
+#define PM_SRC_2 "7"
+#define PM_SRC_3 "8"
+#define PM_FMAC_DPP(Kk, N) "v_fmac_f32_dpp %" #N ", %4, %" PM_SRC_##N " row_newbcast:" #Kk " row_mask:0xf bank_mask:0xf bound_ctrl:1\n"
+#define PM_FMAC4_BCAST0(CF, M, A)                                                               \
+    asm("s_nop 1\n" PM_FMAC_DPP(0, 0) PM_FMAC_DPP(0, 1) PM_FMAC_DPP(0, 2) PM_FMAC_DPP(0, 3)      \
+        : "+v"((A).v[0]), "+v"((A).v[1]), "+v"((A).v[2]), "+v"((A).v[3]), "+v"(CF)              \
+        : "v"((M).v[0]), "v"((M).v[1]), "v"((M).v[2]), "v"((M).v[3]))
+#define PM_FMAC4_BCAST(Kk, CF, M, A)                                                            \
+    asm(PM_FMAC_DPP(Kk, 0) PM_FMAC_DPP(Kk, 1) PM_FMAC_DPP(Kk, 2) PM_FMAC_DPP(Kk, 3)             \
+        : "+v"((A).v[0]), "+v"((A).v[1]), "+v"((A).v[2]), "+v"((A).v[3])                        \
+        : "v"(CF), "v"((M).v[0]), "v"((M).v[1]), "v"((M).v[2]), "v"((M).v[3]))
 
 __device__ __forceinline__ void fma_bcast16(float cf, const Pack<4> (&fl)[16], Pack<4> &w)
 {
-#define PM_B(Kk)                                                                   \
-    {                                                                              \
-        const float b = row_bcast<Kk>(cf);                                         \
-        w.v[0] = fmaf(b, fl[Kk].v[0], w.v[0]); w.v[1] = fmaf(b, fl[Kk].v[1], w.v[1]); \
-        w.v[2] = fmaf(b, fl[Kk].v[2], w.v[2]); w.v[3] = fmaf(b, fl[Kk].v[3], w.v[3]); \
-    }
-    PM_B(0) PM_B(1) PM_B(2) PM_B(3) PM_B(4) PM_B(5) PM_B(6) PM_B(7)
-    PM_B(8) PM_B(9) PM_B(10) PM_B(11) PM_B(12) PM_B(13) PM_B(14) PM_B(15)
-#undef PM_B
+    PM_FMAC4_BCAST0(cf, fl[0], w);
+    PM_FMAC4_BCAST(1, cf, fl[1], w);   PM_FMAC4_BCAST(2, cf, fl[2], w);   PM_FMAC4_BCAST(3, cf, fl[3], w);
+    PM_FMAC4_BCAST(4, cf, fl[4], w);   PM_FMAC4_BCAST(5, cf, fl[5], w);   PM_FMAC4_BCAST(6, cf, fl[6], w);
+    PM_FMAC4_BCAST(7, cf, fl[7], w);   PM_FMAC4_BCAST(8, cf, fl[8], w);   PM_FMAC4_BCAST(9, cf, fl[9], w);
+    PM_FMAC4_BCAST(10, cf, fl[10], w); PM_FMAC4_BCAST(11, cf, fl[11], w); PM_FMAC4_BCAST(12, cf, fl[12], w);
+    PM_FMAC4_BCAST(13, cf, fl[13], w); PM_FMAC4_BCAST(14, cf, fl[14], w); PM_FMAC4_BCAST(15, cf, fl[15], w);
 }
 
 // The four output channels co .. co+3 of a lane read the input channels co/R .. : for R = 1 four
-// distinct ones, for R = 2 two, each used twice (out[., c*R + m]).
-template <int R> __device__ __forceinline__ Pack<4> ld_in_expanded(const float *p)
+// distinct ones, for R = 2 two, each used twice (out[., c*R + m]).  InRow keeps the loaded words as they
+// come (expanding them right after a conditional load would make that load wait on the spot and undo
+// the batching of the gathers); channel u of the four reads v[u / R].
+template <int R> struct InRow { float v[4 / R]; };
+template <int R> __device__ __forceinline__ InRow<R> zero_in()
 {
+    InRow<R> o;
+#pragma unroll
+    for (int i = 0; i < 4 / R; ++i) o.v[i] = 0.f;
+    return o;
+}
+template <int R> __device__ __forceinline__ InRow<R> ld_in(const float *p)
+{
+    InRow<R> o;
     if constexpr (R == 1) {
-        return ldp<4>(p);
+        const float4 t = *reinterpret_cast<const float4 *>(p);
+        o.v[0] = t.x; o.v[1] = t.y; o.v[2] = t.z; o.v[3] = t.w;
     } else {
         const float2 t = *reinterpret_cast<const float2 *>(p);
-        Pack<4> o;
-        o.v[0] = t.x; o.v[1] = t.x; o.v[2] = t.y; o.v[3] = t.y;
-        return o;
+        o.v[0] = t.x; o.v[1] = t.y;
     }
+    return o;
 }
 
 // facet2vertex forward for depth multiplier R = 1 or 2, Co = C*R a multiple of 4 and >= 64 (a 16-lane DPP row
@@ -304,20 +327,26 @@ __global__ __launch_bounds__(kBlock) void f2v_fwd_fast_k(const float *__restrict
 #pragma unroll
     for (int k = 0; k < 16; ++k) fl[k] = (k < K && on) ? ldp<4>(filt + (size_t)k * Co + c) : zero_pack<4>();
 
-    const int64_t stride = (int64_t)gridDim.x * rpb;
-    int64_t row = (int64_t)blockIdx.x * rpb + slot;
+    // Workgroups go round-robin to the eight accelerator dies, each with an L2 of its own: die x takes the
+    // x-th contiguous eighth of the vertices, so that the vertices sharing a facet row mostly meet in one L2.
+    const int64_t groups = (NvOut + rpb - 1) / rpb, gx = (groups + 7) >> 3;
+    const int xcd = blockIdx.x & 7;
+    const int64_t stride = (int64_t)(gridDim.x >> 3) * rpb;
+    const int64_t xend = (xcd + 1) * gx * rpb;
+    const int64_t NvEnd = xend < NvOut ? xend : NvOut;
+    int64_t row = (xcd * gx + (blockIdx.x >> 3)) * rpb + slot;
     // stage 1 (row bounds) of rows `row` and `row + stride`, stage 2 (entries) of `row`
     int e0 = 0, e1 = 0, ne0 = 0, ne1 = 0;
-    if (row < NvOut) { e0 = rowptr[row]; e1 = rowptr[row + 1]; }
-    if (row + stride < NvOut) { ne0 = rowptr[row + stride]; ne1 = rowptr[row + stride + 1]; }
+    if (row < NvEnd) { e0 = rowptr[row]; e1 = rowptr[row + 1]; }
+    if (row + stride < NvEnd) { ne0 = rowptr[row + stride]; ne1 = rowptr[row + stride + 1]; }
     int f[EB];
 #pragma unroll
     for (int i = 0; i < EB; ++i) f[i] = (e0 + i < e1) ? colidx[e0 + i] / 3 : -1;
 
-    for (; row < NvOut; row += stride) {
+    for (; row < NvEnd; row += stride) {
         // row bounds two rows ahead, entry list one row ahead
         int me0 = 0, me1 = 0;
-        if (row + 2 * stride < NvOut) { me0 = rowptr[row + 2 * stride]; me1 = rowptr[row + 2 * stride + 1]; }
+        if (row + 2 * stride < NvEnd) { me0 = rowptr[row + 2 * stride]; me1 = rowptr[row + 2 * stride + 1]; }
         int nf[EB];
 #pragma unroll
         for (int i = 0; i < EB; ++i) nf[i] = (ne0 + i < ne1) ? colidx[ne0 + i] / 3 : -1;
@@ -329,11 +358,11 @@ __global__ __launch_bounds__(kBlock) void f2v_fwd_fast_k(const float *__restrict
 #pragma unroll
                 for (int i = 0; i < EB; ++i) f[i] = (eb + i < e1) ? colidx[eb + i] / 3 : -1;
             }
-            Pack<4> x[EB];
+            InRow<R> x[EB];
             float cf[EB];
 #pragma unroll
             for (int i = 0; i < EB; ++i) {
-                x[i] = (f[i] >= 0 && on) ? ld_in_expanded<R>(in + (int64_t)f[i] * C + c / R) : zero_pack<4>();
+                x[i] = (f[i] >= 0 && on) ? ld_in<R>(in + (int64_t)f[i] * C + c / R) : zero_in<R>();
                 cf[i] = (f[i] >= 0 && kok) ? coeff[(int64_t)f[i] * K + l16] : 0.f;
             }
 #pragma unroll
@@ -342,7 +371,7 @@ __global__ __launch_bounds__(kBlock) void f2v_fwd_fast_k(const float *__restrict
                     Pack<4> w = zero_pack<4>();
                     fma_bcast16(cf[i], fl, w);
 #pragma unroll
-                    for (int u = 0; u < 4; ++u) acc.v[u] = fmaf(w.v[u], x[i].v[u], acc.v[u]);
+                    for (int u = 0; u < 4; ++u) acc.v[u] = fmaf(w.v[u], x[i].v[u / R], acc.v[u]);
                 }
             }
         }
@@ -501,8 +530,8 @@ __global__ __launch_bounds__(kBlock) void f2v_bwd_fast_k(const float *__restrict
             g[j] = (ok && on) ? ldp<4>(gout + (int64_t)vo[j] * Co + c) : zero_pack<4>();
             nf[j] = ok ? (float)nfcount[vo[j]] : 1.f;
         }
-        const Pack<4> x = on ? ld_in_expanded<R>(in + f * C + c / R) : zero_pack<4>();
-        const float cf = (l16 < K) ? coeff[f * K + l16] : 0.f;
+        const InRow<R> x = on ? ld_in<R>(in + f * C + c / R) : zero_in<R>();
+        float cf = (l16 < K) ? coeff[f * K + l16] : 0.f;
         Pack<4> s = zero_pack<4>(), w = zero_pack<4>(), t;
 #pragma unroll
         for (int j = 0; j < 3; ++j) {
@@ -512,16 +541,13 @@ __global__ __launch_bounds__(kBlock) void f2v_bwd_fast_k(const float *__restrict
         }
         fma_bcast16(cf, fl, w);
 #pragma unroll
-        for (int u = 0; u < 4; ++u) t.v[u] = x.v[u] * s.v[u];
-#define PM_A(Kk)                                                                     \
-    {                                                                                \
-        const float b = row_bcast<Kk>(cf);                                           \
-        acc[Kk].v[0] = fmaf(b, t.v[0], acc[Kk].v[0]); acc[Kk].v[1] = fmaf(b, t.v[1], acc[Kk].v[1]); \
-        acc[Kk].v[2] = fmaf(b, t.v[2], acc[Kk].v[2]); acc[Kk].v[3] = fmaf(b, t.v[3], acc[Kk].v[3]); \
-    }
-        PM_A(0) PM_A(1) PM_A(2) PM_A(3) PM_A(4) PM_A(5) PM_A(6) PM_A(7)
-        PM_A(8) PM_A(9) PM_A(10) PM_A(11) PM_A(12) PM_A(13) PM_A(14) PM_A(15)
-#undef PM_A
+        for (int u = 0; u < 4; ++u) t.v[u] = x.v[u / R] * s.v[u];
+        PM_FMAC4_BCAST0(cf, t, acc[0]);
+        PM_FMAC4_BCAST(1, cf, t, acc[1]);   PM_FMAC4_BCAST(2, cf, t, acc[2]);   PM_FMAC4_BCAST(3, cf, t, acc[3]);
+        PM_FMAC4_BCAST(4, cf, t, acc[4]);   PM_FMAC4_BCAST(5, cf, t, acc[5]);   PM_FMAC4_BCAST(6, cf, t, acc[6]);
+        PM_FMAC4_BCAST(7, cf, t, acc[7]);   PM_FMAC4_BCAST(8, cf, t, acc[8]);   PM_FMAC4_BCAST(9, cf, t, acc[9]);
+        PM_FMAC4_BCAST(10, cf, t, acc[10]); PM_FMAC4_BCAST(11, cf, t, acc[11]); PM_FMAC4_BCAST(12, cf, t, acc[12]);
+        PM_FMAC4_BCAST(13, cf, t, acc[13]); PM_FMAC4_BCAST(14, cf, t, acc[14]); PM_FMAC4_BCAST(15, cf, t, acc[15]);
         if (on) {
             if constexpr (R == 1) {
                 Pack<4> gi;
@@ -866,6 +892,13 @@ static bool f2v_fast_ok(int C, int r, int K, std::initializer_list<const void *>
     return true;
 }
 
+// PMESH_F2V_VALU=1 keeps facet2vertex on the vector-ALU kernels (tests compare the two paths).
+static bool force_valu()
+{
+    const char *e = getenv("PMESH_F2V_VALU");
+    return e && e[0] == '1';
+}
+
 static int reduce_partials(const float *partial, float *out, int G, int n, hipStream_t st)
 {
     reduce_partials_k<<<dim3((unsigned)ceil_div(n, 16)), dim3(1024), 0, st>>>(partial, out, G, n);
@@ -956,10 +989,11 @@ extern "C" int pmesh_f2v_fwd(const float *input, const float *filter, const floa
     const int64_t blocks = ceil_div(NvOut, rs.rpb);
     PM_REQUIRE(grid_ok(blocks), "f2v_fwd: grid too large");
     const int cvec = ((K & 3) == 0 && aligned16(coeff)) ? 1 : 0;
+    if (!force_valu() && f2v_mfma_ok(Nf, C, r, K, coeff)) return f2v_fwd_mfma(input, filter, coeff, nf_count, rowptr, colidx, output, NvOut, C, r, st);
     if (f2v_fast_ok(C, r, K, {input, filter, output})) {
         // persistent: enough workgroups to fill the chip several times over, each visiting many vertices
         const RowShape fs = row_shape(C * r / 4);
-        const int64_t fb = ceil_div(NvOut, fs.rpb), pb = fb < 4096 ? fb : 4096;
+        const int64_t fb = ceil_div(ceil_div(NvOut, fs.rpb), 8) * 8, pb = fb < 4096 ? fb : 4096;   // a multiple of 8
         if (r == 1)
             f2v_fwd_fast_k<1><<<dim3((unsigned)pb), dim3(kBlock), 0, st>>>(input, filter, coeff, nf_count, rowptr, colidx, output, NvOut, C, K, fs.lpr_log2);
         else
@@ -1003,6 +1037,12 @@ extern "C" int pmesh_f2v_bwd(const float *grad_output, const float *input, const
     PM_REQUIRE(workspace_bytes >= (size_t)G * K * Co * sizeof(float), "f2v_bwd: workspace too small (%zu bytes)", workspace_bytes);
     const int cvec = ((K & 3) == 0 && aligned16(coeff)) ? 1 : 0;
     float *partial = (float *)workspace;
+    if (!force_valu() && (r == 1 || r == 2) && f2v_mfma_ok(Nf, C, r, K, coeff) && NvOut * (int64_t)Co < (int64_t(1) << 30)) {
+        const int Gm = f2v_bwd_mfma_blocks(Nf);
+        PM_REQUIRE(workspace_bytes >= (size_t)Gm * K * Co * sizeof(float), "f2v_bwd: workspace too small (%zu bytes)", workspace_bytes);
+        if (int rc = f2v_bwd_mfma(grad_output, input, filter, coeff, face, nf_count, vt_map, grad_input, partial, Gm, Nf, NvOut, C, r, st)) return rc;
+        return reduce_partials(partial, grad_filter, Gm, K * Co, st);
+    }
     if (f2v_fast_ok(C, r, K, {grad_output, input, filter, grad_input, workspace})) {
         const RowShape fs = row_shape(Co / 4);
         const int64_t frows = ceil_div(ceil_div(Nf, G), fs.rpb) * fs.rpb;

@@ -1,0 +1,21 @@
+// Internal interface between the row kernels' entry points (mesh_rows.hip) and the matrix-core
+// facet2vertex kernels (mesh_f2v_mfma.hip).
+#pragma once
+#include "common.h"
+
+namespace pmesh {
+
+// K == 16 coefficients in 16-byte aligned rows, at least 32 output channels, 32-bit byte offsets into `input`.
+bool f2v_mfma_ok(int64_t Nf, int C, int r, int K, const void *coeff);
+
+int f2v_fwd_mfma(const float *in, const float *filt, const float *coeff, const int *nfcount, const int *rowptr,
+                 const int *colidx, float *out, int64_t NvOut, int C, int r, hipStream_t st);
+
+// Backward on the matrix cores: depth multiplier 1 or 2, additionally NvOut * C * r * 4 < 2^32.  G workgroups
+// (f2v_bwd_mfma_blocks) leave G partial filter gradients of 16 * C * r floats in `partial`.
+int f2v_bwd_mfma_blocks(int64_t Nf);
+int f2v_bwd_mfma(const float *gout, const float *in, const float *filt, const float *coeff, const int *face,
+                 const int *nfcount, const int *vtmap, float *gin, float *partial, int G, int64_t Nf, int64_t NvOut,
+                 int C, int r, hipStream_t st);
+
+}  // namespace pmesh

@@ -100,9 +100,16 @@ def test_v2f_parity(cuda, mesh, C, r):
                                                 ("sphere2", 5, 3, 4, True), ("sphere2", 128, 1, 16, False),
                                                 ("sphere3", 48, 2, 16, True), ("sphere3", 96, 1, 16, False),
                                                 ("room_small", 40, 2, 9, True), ("sphere2", 36, 2, 16, False),
-                                                ("sphere2", 160, 1, 12, True), ("sphere2", 64, 2, 16, False)])
-def test_f2v_parity(cuda, mesh, C, r, K, strided):
-    say("case f2v", mesh, C, r, K, strided)
+                                                ("sphere2", 160, 1, 12, True), ("sphere2", 64, 2, 16, False),
+                                                ("fans", 64, 1, 16, False), ("fans", 40, 1, 16, True),
+                                                ("sphere3", 200, 1, 16, True), ("sphere2", 12, 3, 16, False),
+                                                ("room_small", 128, 2, 16, True), ("sphere3", 33, 1, 16, False)])
+@pytest.mark.parametrize("path", ["default", "valu"])
+def test_f2v_parity(cuda, monkeypatch, mesh, C, r, K, strided, path):
+    """default: matrix-core kernels where they apply (16 coefficients, at least 32 output channels);
+    valu: the vector-ALU kernels for every shape."""
+    say("case f2v", mesh, C, r, K, strided, path)
+    monkeypatch.setenv("PMESH_F2V_VALU", "1" if path == "valu" else "0")
     v, f = mesh_case(mesh)
     rng = np.random.default_rng(11)
     nv, nf = v.shape[0], f.shape[0]

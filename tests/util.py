@@ -53,6 +53,15 @@ def mesh_case(name, seed=0):
         return S.torus(24, 16)
     if name == "room_small":
         return S.room(rng, scale=0.01)
+    if name == "fans":
+        # hubs of degree 20 and 11 (more than eight adjacency entries per vertex) next to low-degree rims
+        def fan(n, base):
+            hub = base
+            rim = base + 1 + np.arange(n)
+            return np.stack([np.full(n, hub), rim, np.roll(rim, -1)], 1)
+        f = np.concatenate([fan(20, 0), fan(11, 21), fan(3, 33)]).astype(np.int32)
+        v = rng.normal(0, 1, (37, 3))
+        return v, f
     if name == "shapes_small":
         w = S.shapes_workload(seed=seed, n_meshes=2)
         return w["vertex"], w["face"]

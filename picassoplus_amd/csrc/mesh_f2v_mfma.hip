@@ -162,7 +162,7 @@ __global__ __launch_bounds__(kBlock) void f2v_fwd_mfma_k(const float *__restrict
 // Workgroups own contiguous facet ranges (fixed by the problem size only) and leave one partial filter
 // gradient each, summed by reduce_partials in a fixed order.
 template <int NCB, int R>
-__global__ __launch_bounds__(kBlock) void f2v_bwd_mfma_k(const float *__restrict__ gout, const float *__restrict__ in,
+__global__ __launch_bounds__(kBlock, 2) void f2v_bwd_mfma_k(const float *__restrict__ gout, const float *__restrict__ in,
                                                          const float *__restrict__ filt,
                                                          const float *__restrict__ coeff,
                                                          const int *__restrict__ face,
@@ -359,14 +359,15 @@ int f2v_bwd_mfma(const float *gout, const float *in, const float *filt, const fl
                  int C, int r, hipStream_t st)
 {
     const int Co = C * r;
-    const int ncb = Co <= 32 ? 1 : 2;
-    const unsigned gy = (unsigned)ceil_div(Co, 32 * ncb);
+    // one 32-channel block per workgroup column: two wavefronts per SIMD fit, which beats sharing the
+    // index chain between two blocks at one wavefront per SIMD
+    const unsigned gy = (unsigned)ceil_div(Co, 32);
     const int64_t rows_per_block = ceil_div(ceil_div(Nf, G), 128) * 128;
     const dim3 grid((unsigned)G, gy), block(kBlock);
-#define PM_GO(N, RR) f2v_bwd_mfma_k<N, RR><<<grid, block, 0, st>>>(gout, in, filt, coeff, face, nfcount, vtmap, gin, partial, Nf, NvOut, C, Co, rows_per_block)
-    if (ncb == 1) { if (r == 1) PM_GO(1, 1); else PM_GO(1, 2); }
-    else          { if (r == 1) PM_GO(2, 1); else PM_GO(2, 2); }
-#undef PM_GO
+    if (r == 1)
+        f2v_bwd_mfma_k<1, 1><<<grid, block, 0, st>>>(gout, in, filt, coeff, face, nfcount, vtmap, gin, partial, Nf, NvOut, C, Co, rows_per_block);
+    else
+        f2v_bwd_mfma_k<1, 2><<<grid, block, 0, st>>>(gout, in, filt, coeff, face, nfcount, vtmap, gin, partial, Nf, NvOut, C, Co, rows_per_block);
     PM_LAUNCHED("f2v_bwd(mfma)");
     return 0;
 }

@@ -36,7 +36,7 @@ def parse():
     ap.add_argument("--workload", default="scene", choices=["scene", "shapes", "pool", "firstblock"],
                     help="scene: the headline layer (F2F+F2V, C=64); shapes: 16 small meshes V2F+F2F+F2V; pool: "
                          "1024x1024 grid max/avg pool + unpool; firstblock: the scene batch with the reference's first "
-                         "block shapes, F2F 3->64 then F2V 64->64 with depth multiplier 2 (pi2_blocks.py:113-130)")
+                         "block shapes, F2F 3->32 then F2V 32->32 with depth multiplier 2 (pi2_blocks.py:113-130)")
     ap.add_argument("--scale", type=float, default=1.0, help="facet-count scale of the scene workload")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -120,13 +120,13 @@ def run_conv_layer(args, torch, kind):
     from picassoplus_amd.mesh.layers import sph_harm_values
     from picassoplus_amd.mesh.pi_modules import conv3d
     dev = torch.device("cuda:0")
-    C, L = 64, 3
+    C, L = (32 if kind == "firstblock" else 64), 3           # first block: EncodeChannels[0] = 32 (scene_seg.py:28)
     Cin, r = (3, 2) if kind == "firstblock" else (C, 1)      # F2F input channels, F2V depth multiplier
     if kind in ("scene", "firstblock"):
         mesh = S.scene_workload(seed=3000, n_rooms=8, scale=args.scale)
         d = build_conv_inputs(mesh, C, L, seed=3000, Cin=Cin, r=r)
         ops = ["f2f_fwd", "f2v_fwd", "f2v_bwd", "f2f_bwd_texture", "f2f_bwd_filter"]
-        name = "scene8x300k_F2F+F2V_C64_L3_fp32_fwd+bwd" if kind == "scene" else "scene8x300k_F2F3to64+F2Vr2_L3_fp32_fwd+bwd"
+        name = "scene8x300k_F2F+F2V_C64_L3_fp32_fwd+bwd" if kind == "scene" else "scene8x300k_F2F3to32+F2V32r2_L3_fp32_fwd+bwd"
     else:
         mesh = S.shapes_workload(seed=2000, n_meshes=16)
         d = build_conv_inputs(mesh, C, L, seed=2000, tex_counts=3)

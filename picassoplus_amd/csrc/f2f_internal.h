@@ -40,4 +40,12 @@ int f2f16_bwd_texture(const float *gout, const float *W, const float *sh, const 
 int f2f16_bwd_filter_partials(const float *gout, const float *tex, const float *sh, const int *cum, float *partial,
                               int splits, int64_t T, int64_t Nf, int Cin, int Cout, hipStream_t st);
 
+// Narrow filter gradient (mesh_f2f_narrow.hip): at most four input channels, F == 16.  `blocks` partial
+// gradients of Cout*Cin*16 floats are left in `partial` (blocks = f2f_narrow_blocks(Nf) <= kNarrowMaxBlocks).
+constexpr int kNarrowMaxBlocks = 2048;
+bool f2f_narrow_usable(int Cin, int F);
+int f2f_narrow_blocks(int64_t Nf);
+int f2f_bwd_filter_narrow_partials(const float *gout, const float *tex, const float *sh, const int *cum, float *partial,
+                                   int blocks, int64_t T, int64_t Nf, int Cin, int Cout, hipStream_t st);
+
 }  // namespace pmesh

@@ -17,6 +17,7 @@
 // of H holds every d of its channels.
 #include "common.h"
 #include "f2f_internal.h"
+#include "rows_internal.h"
 #include "../../include/picasso_mesh.h"
 #include <cstdlib>
 
@@ -384,7 +385,8 @@ extern "C" int pmesh_f2f_fwd(const float *texture, const float *filter, const fl
 extern "C" size_t pmesh_f2f_bwd_workspace_bytes(int Cin, int Cout, int F)
 {
     // the two halves run one after the other on a stream and share the workspace
-    const size_t filt = (size_t)kFiltMaxSplits * Cout * Cin * F * sizeof(float);
+    const size_t slices = f2f_narrow_usable(Cin, F) ? kNarrowMaxBlocks : kFiltMaxSplits;
+    const size_t filt = slices * Cout * Cin * F * sizeof(float);
     const size_t tex = F == 16 ? f2f16x3_bwd_texture_workspace_bytes(Cin, Cout) : 0;
     return filt > tex ? filt : tex;
 }
@@ -433,6 +435,15 @@ extern "C" int pmesh_f2f_bwd_filter(const float *grad_output, const float *textu
         return 0;
     }
     PM_REQUIRE(grad_output && texture && bary_coeff && cum_texture && workspace, "f2f_bwd_filter: null pointer");
+    if (!force_generic() && !force_fp32_mfma() && f2f_narrow_usable(Cin, F) && !(reinterpret_cast<uintptr_t>(bary_coeff) & 15u)) {
+        const int nb = f2f_narrow_blocks(Nf);
+        PM_REQUIRE(workspace_bytes >= (size_t)nb * nW * sizeof(float), "f2f_bwd_filter: workspace too small (%zu bytes)",
+                   workspace_bytes);
+        if (int rc = f2f_bwd_filter_narrow_partials(grad_output, texture, bary_coeff, cum_texture, (float *)workspace, nb, T,
+                                                    Nf, Cin, Cout, st))
+            return rc;
+        return reduce_partials((const float *)workspace, grad_filter, nb, (int)nW, st);
+    }
     const ChunkGeom cg = chunk_geom(Cin, F);
     const int S = filt_splits(Nf);
     PM_REQUIRE(workspace_bytes >= (size_t)S * nW * sizeof(float), "f2f_bwd_filter: workspace too small (%zu bytes)",

@@ -899,7 +899,7 @@ static bool force_valu()
     return e && e[0] == '1';
 }
 
-static int reduce_partials(const float *partial, float *out, int G, int n, hipStream_t st)
+int reduce_partials(const float *partial, float *out, int G, int n, hipStream_t st)
 {
     reduce_partials_k<<<dim3((unsigned)ceil_div(n, 16)), dim3(1024), 0, st>>>(partial, out, G, n);
     PM_LAUNCHED("reduce_partials");

@@ -9,12 +9,14 @@ clears in place (conv3d.py:8-9, pool3d.py:8-10, unpool3d.py:8-9).  ``native_op``
 import torch
 
 
-def native_op(name, forward, backward, n_inputs, n_grads, keep=None):
+def native_op(name, forward, backward, n_inputs, n_grads, keep=None, selective=False):
     """Build the autograd Function ``name``.
 
     forward(*inputs)            -> output, or (output, *extras) where extras are saved, not returned
     backward(grad, *saved)      -> one gradient or a sequence of ``n_grads`` gradients, for inputs[:n_grads]
     keep(inputs, extras)        -> tuple of tensors to save (default: all inputs, then the extras)
+    selective                   -> backward also takes ``needs=`` (one flag per gradient, from
+                                   ``ctx.needs_input_grad``) and may return ``None`` where it is False
     Inputs past the first ``n_grads`` are indices / coefficients: they get ``None`` gradients and
     their ``requires_grad`` flag is cleared in place, as in the reference.
     """
@@ -31,7 +33,10 @@ def native_op(name, forward, backward, n_inputs, n_grads, keep=None):
         return output
 
     def bwd(ctx, grad_output):
-        grads = backward(grad_output.contiguous(), *ctx.saved_tensors)
+        if selective:
+            grads = backward(grad_output.contiguous(), *ctx.saved_tensors, needs=tuple(ctx.needs_input_grad[:n_grads]))
+        else:
+            grads = backward(grad_output.contiguous(), *ctx.saved_tensors)
         grads = tuple(grads) if isinstance(grads, (tuple, list)) else (grads,)
         return grads + (None,) * (n_inputs - len(grads))
 

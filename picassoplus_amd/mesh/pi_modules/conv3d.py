@@ -3,12 +3,15 @@
 ``vertex2facet``, ``facet2facet`` and ``facet2vertex`` take the same arguments in the same
 order as the reference functions (conv3d.py:21,55,89), save the same tensors for backward
 and return ``None`` gradients for index and coefficient inputs.  The feature and the filter
-gradient come out of one native call, so both are always computed, as in the reference.
+gradient of vertex2facet and facet2vertex come out of one native call, so both are always computed,
+as in the reference; facet2facet has one native call per gradient and skips the one autograd does not
+ask for (the texture gradient of a network's input colours, the largest single saving of a first block).
 """
 from . import mesh_conv3d as module
 from ._autograd import native_op
 
-f2f_Function = native_op("f2f_Function", module.facet2facet_forward, module.facet2facet_backward, n_inputs=4, n_grads=2)
+f2f_Function = native_op("f2f_Function", module.facet2facet_forward, module.facet2facet_backward_selected, n_inputs=4,
+                         n_grads=2, selective=True)
 v2f_Function = native_op("v2f_Function", module.vertex2facet_forward, module.vertex2facet_backward, n_inputs=3, n_grads=2)
 f2v_Function = native_op("f2v_Function", module.facet2vertex_forward, module.facet2vertex_backward, n_inputs=6, n_grads=2)
 

@@ -143,21 +143,30 @@ def facet2facet_forward(input, filter, bary_coeff, num_texture):
 
 def facet2facet_backward(grad_output, input, filter, bary_coeff, num_texture):
     """mesh_conv3d.cpp:229-269 -> [grad_input (NiK,Cin), grad_filter (Cout,Cin,F)]."""
+    return facet2facet_backward_selected(grad_output, input, filter, bary_coeff, num_texture, needs=(True, True))
+
+
+def facet2facet_backward_selected(grad_output, input, filter, bary_coeff, num_texture, needs):
+    """facet2facet_backward with ``needs`` = (texture gradient wanted, filter gradient wanted): an unwanted
+    gradient is not computed and comes back as None (no counterpart in the reference, which always
+    computes both)."""
     T, Cin, Cout, F, Nf = _f2f_dims(input, filter, bary_coeff, num_texture, False)
     check_input(grad_output, "grad_output", 2, F32)
     if tuple(grad_output.shape) != (Nf, Cout):
         raise RuntimeError("grad_output must have shape (NfIn, Cout)")
     dev = same_device(grad_output, input, filter, bary_coeff, num_texture)
     with torch.cuda.device(dev):
-        gin = torch.empty((T, Cin), dtype=F32, device=dev)
-        gfilt = torch.empty((Cout, Cin, F), dtype=F32, device=dev)
+        gin = torch.empty((T, Cin), dtype=F32, device=dev) if needs[0] else None
+        gfilt = torch.empty((Cout, Cin, F), dtype=F32, device=dev) if needs[1] else None
         nbytes = _lib.query("pmesh_f2f_bwd_workspace_bytes", Cin, Cout, F)
         ws = workspace(nbytes, dev)
         st = stream_of(input)
         order = topology.facet_order(num_texture, T) if Nf else None
         order_ptr = order.data_ptr() if order is not None else None
-        _lib.call("pmesh_f2f_bwd_texture", grad_output.data_ptr(), filter.data_ptr(), bary_coeff.data_ptr(),
-                  num_texture.data_ptr(), order_ptr, gin.data_ptr(), ws.data_ptr(), nbytes, T, Nf, Cin, Cout, F, st)
-        _lib.call("pmesh_f2f_bwd_filter", grad_output.data_ptr(), input.data_ptr(), bary_coeff.data_ptr(),
-                  num_texture.data_ptr(), order_ptr, gfilt.data_ptr(), ws.data_ptr(), nbytes, T, Nf, Cin, Cout, F, st)
+        if needs[0]:
+            _lib.call("pmesh_f2f_bwd_texture", grad_output.data_ptr(), filter.data_ptr(), bary_coeff.data_ptr(),
+                      num_texture.data_ptr(), order_ptr, gin.data_ptr(), ws.data_ptr(), nbytes, T, Nf, Cin, Cout, F, st)
+        if needs[1]:
+            _lib.call("pmesh_f2f_bwd_filter", grad_output.data_ptr(), input.data_ptr(), bary_coeff.data_ptr(),
+                      num_texture.data_ptr(), order_ptr, gfilt.data_ptr(), ws.data_ptr(), nbytes, T, Nf, Cin, Cout, F, st)
     return [gin, gfilt]

@@ -111,6 +111,35 @@ def test_f2f_module_matches_oracle_composition(cuda, cin, cout):
     _compare_grads(mod, mod64)
 
 
+def test_f2f_skips_the_gradient_nobody_asked_for(cuda):
+    """Input colours do not require grad in a network: the filter gradient must not change, and no texture
+    gradient may be produced (nor its kernel launched: the call hook sees every native call)."""
+    from picassoplus_amd import _lib
+    from picassoplus_amd.mesh.pi_modules import conv3d
+    rng = np.random.default_rng(31)
+    nf, cin, cout = 300, 3, 16
+    counts, bary, _ = texture_case(rng, nf, kmax=6)
+    T = int(counts.sum())
+    tex = torch.from_numpy(rng.uniform(0, 1, (T, cin)).astype(np.float32)).to(cuda)
+    w = torch.from_numpy(rng.normal(0, 0.3, (cout, cin, 16)).astype(np.float32)).to(cuda)
+    sh = layers.SphHarmCoeff(3)(torch.from_numpy(bary).to(cuda, torch.float32))
+    cum = torch.cumsum(torch.from_numpy(counts).to(cuda), 0, dtype=torch.int32)
+    g = torch.randn(nf, cout, device=cuda)
+
+    calls = []
+    ta, wa = tex.clone().requires_grad_(True), w.clone().requires_grad_(True)
+    conv3d.facet2facet(ta, wa, sh, cum).backward(g)
+    wb = w.clone().requires_grad_(True)
+    _lib.set_call_hook(lambda name, phase: calls.append(name))
+    try:
+        conv3d.facet2facet(tex, wb, sh, cum).backward(g)
+    finally:
+        _lib.set_call_hook(None)
+    torch.cuda.synchronize()
+    assert torch.equal(wa.grad, wb.grad) and tex.grad is None
+    assert "pmesh_f2f_bwd_filter" in calls and "pmesh_f2f_bwd_texture" not in calls
+
+
 def test_pool_unpool_modules(cuda):
     rng = np.random.default_rng(23)
     nv, C = 2000, 24

@@ -346,6 +346,13 @@ using namespace pmesh;
     PM_REQUIRE(T >= 0 && Nf >= 0 && T <= INT32_MAX && Nf <= INT32_MAX, name ": bad sizes")
 
 // PMESH_F2F_FP32MFMA=1 keeps the 16-coefficient fast path on the fp32 matrix instructions
+// PMESH_F2F_BF16X3=1 keeps the three-piece bf16 kernels where the two-piece fp16 ones would run.
+static inline bool force_bf16x3()
+{
+    const char *e = getenv("PMESH_F2F_BF16X3");
+    return e && e[0] == '1';
+}
+
 static inline bool force_fp32_mfma()
 {
     const char *e = getenv("PMESH_F2F_FP32MFMA");
@@ -367,6 +374,10 @@ extern "C" int pmesh_f2f_fwd(const float *texture, const float *filter, const fl
     if (Nf == 0) return 0;
     PM_REQUIRE(filter && cum_texture && output && (T == 0 || (texture && bary_coeff)), "f2f_fwd: null pointer");
     // the split-bf16 forward addresses texture elements with 32-bit offsets
+    if (!force_generic() && !force_fp32_mfma() && !force_bf16x3() && f2f16x3_usable(filter, bary_coeff, F) &&
+        T * Cin < (int64_t(1) << 31))
+        return f2f16h2_fwd(texture, filter, bary_coeff, cum_texture, facet_order, output, workspace, workspace_bytes,
+                           T, Nf, Cin, Cout, (hipStream_t)stream);
     if (!force_generic() && !force_fp32_mfma() && f2f16x3_usable(filter, bary_coeff, F) &&
         T * Cin < (int64_t(1) << 31))
         return f2f16x3_fwd(texture, filter, bary_coeff, cum_texture, facet_order, output, workspace, workspace_bytes,

@@ -1,0 +1,447 @@
+// facet2facet forward for 16 SH coefficients on the fp16 matrix cores with fp32-level accuracy.
+//
+// Both operands of out = G . W^T are split into TWO fp16 pieces each,
+//     x = x1 + x2 + e,   x1 = x rounded to 11 significant bits,  x2 = (x - x1) rounded to 11 bits,  |e| <= 2^-23 |x|
+// and the product is accumulated in fp32 from three piece products,
+//     G.W ~ G2W1 + G1W2 + G1W1                        (the dropped G2W2 is <= 2^-22 relative),
+// three v_mfma_f32_32x32x16_f16 where the three-piece bf16 split needs six, and 24 instead of 44 vector
+// instructions per eight values split.  fp16 has a narrow exponent range, so both operands are brought
+// to a fixed magnitude by exact power-of-two scales that are taken out of the accumulator at the end:
+//     W' = beta * W        beta from max|W| (one scalar per filter, computed by f2f16h2_scale_filter_k)
+//     G'_f = alpha_f * G_f alpha_f from a bound on max|G_f| = max|tex rows of f| * max|SH rows of f|,
+//                          found by a pre-scan of the facet's rows; it rides on the SH values in registers
+// so that |W'|, |G'| < 2^14.  Elements far below their row's maximum (by more than 2^17) fall into fp16's
+// subnormal range and keep an ABSOLUTE error of 2^-25 in scaled units, i.e. below 2^-39 of the row maximum.
+//
+// Work decomposition: as the three-piece bf16 kernel (workgroup = 256 facets from the list sorted by
+// point count x 64 output channels, 8 wavefronts x 32 facets, two wavefronts per SIMD, filter chunks of
+// four channels through three LDS buffers, texture rows through a wavefront-private LDS slab).
+#include "f2f_internal.h"
+
+namespace pmesh {
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int kHKB = 4;                       // texture points per facet covered by one sweep (register budget)
+constexpr int kHChunk = 4 * 2 * 2 * 64;       // uint4 per LDS buffer: 4 channels x 2 tiles x 2 pieces x 64 lanes
+constexpr int kHW = 8;                        // wavefronts per workgroup
+constexpr int kHThreads = 64 * kHW;
+constexpr int kHWn = kHChunk / kHThreads;     // uint4 of a filter chunk fetched per thread
+constexpr int kHSlab = kHKB * 8 * 32;         // floats per slab buffer: points x 8 channels x facet slots
+
+__device__ __forceinline__ float4 hld4(const float *p) { return *reinterpret_cast<const float4 *>(p); }
+template <bool VEC> __device__ __forceinline__ float4 hld4_row(const float *p, int n)
+{
+    if constexpr (VEC) return n > 0 ? hld4(p) : make_float4(0.f, 0.f, 0.f, 0.f);
+    float4 r;
+    r.x = n > 0 ? p[0] : 0.f;
+    r.y = n > 1 ? p[1] : 0.f;
+    r.z = n > 2 ? p[2] : 0.f;
+    r.w = n > 3 ? p[3] : 0.f;
+    return r;
+}
+__device__ __forceinline__ float absmax4(const float4 &v, float m)
+{
+    return fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fmaxf(fabsf(v.z), fabsf(v.w)), m));
+}
+
+// Eight fp32 values -> two packed fp16x8 pieces, both rounded to nearest (one v_cvt_pk_f16_f32 per pair); the
+// remainder x - x1 is exact in fp32 and comes from one mixed-precision FMA per value.
+__device__ __forceinline__ void split8h(const float (&x)[8], u32x4 &p1, u32x4 &p2)
+{
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const float a = x[2 * j], b = x[2 * j + 1];
+        f16x2 hi, lo;
+        hi[0] = (_Float16)a;
+        hi[1] = (_Float16)b;
+        lo[0] = (_Float16)__builtin_fmaf((float)hi[0], -1.0f, a);
+        lo[1] = (_Float16)__builtin_fmaf((float)hi[1], -1.0f, b);
+        p1[j] = __builtin_bit_cast(unsigned, hi);
+        p2[j] = __builtin_bit_cast(unsigned, lo);
+    }
+}
+
+__device__ __forceinline__ f32x16 mfma_f16(const u32x4 &a, const u32x4 &b, const f32x16 &c)
+{
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+}
+
+__device__ __forceinline__ int hwave_max(int v)
+{
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        const int t = __shfl_xor(v, o, 64);
+        v = t > v ? t : v;
+    }
+    return __builtin_amdgcn_readfirstlane(v);
+}
+
+// Power of two s with s * m < 2^14 for a bound m >= 0 (s = 1 for m = 0 or non-finite m); *inv = 1 / s.
+__device__ __forceinline__ float pow2_scale(float m, float *inv)
+{
+    int e = (int)((__builtin_bit_cast(unsigned, m) >> 23) & 0xFFu);      // biased exponent: m < 2^(e - 126)
+    if (e == 0 || e == 255) { *inv = 1.0f; return 1.0f; }
+    e = e < 40 ? 40 : (e > 215 ? 215 : e);                                // keep both s and 1/s normal numbers
+    *inv = __builtin_bit_cast(float, (unsigned)(e - 13) << 23);           // 2^(e - 140)
+    return __builtin_bit_cast(float, (unsigned)(267 - e) << 23);          // 2^(140 - e):  s * m < 2^14
+}
+
+// header of the packed filter: {beta, 1/beta}
+__global__ __launch_bounds__(1024) void f2f16h2_scale_filter_k(const float *__restrict__ W, float *__restrict__ hdr, int64_t n)
+{
+    __shared__ float red[16];
+    float m = 0.f;
+    for (int64_t i = threadIdx.x; i < n; i += 1024) m = fmaxf(m, fabsf(W[i]));
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = m;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+#pragma unroll
+        for (int i = 1; i < 16; ++i) m = fmaxf(m, red[i]);
+        float inv;
+        const float beta = pow2_scale(m, &inv);
+        hdr[0] = beta;
+        hdr[1] = inv;
+    }
+}
+
+// Filter (Cout, Cin, 16) -> per-lane MFMA B operands: Wp[((ci*NT + nt)*2 + piece)*64 + lane] holds the
+// eight fp16 pieces of beta * W[nt*32 + l32][ci][8h .. 8h+7], lane = 32h + l32.  NT = even number of
+// 32-channel tiles covering Cout; channels Cin .. CinPad-1 and output channels past Cout are zero.
+__global__ __launch_bounds__(kBlock) void f2f16h2_pack_filter_k(const float *__restrict__ W, const float *__restrict__ hdr,
+                                                                u32x4 *__restrict__ Wp, int Cin, int CinPad, int Cout, int NT)
+{
+    const int idx = blockIdx.x * kBlock + threadIdx.x;
+    if (idx >= CinPad * NT * 64) return;
+    const int lane = idx & 63, nt = (idx >> 6) % NT, ci = (idx >> 6) / NT;
+    const int co = nt * 32 + (lane & 31), h = lane >> 5;
+    const float beta = hdr[0];
+    float x[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) x[j] = 0.f;
+    if (co < Cout && ci < Cin) {
+        const float *p = W + ((int64_t)co * Cin + ci) * 16 + 8 * h;
+        const float4 u = hld4(p), v = hld4(p + 4);
+        x[0] = u.x * beta; x[1] = u.y * beta; x[2] = u.z * beta; x[3] = u.w * beta;
+        x[4] = v.x * beta; x[5] = v.y * beta; x[6] = v.z * beta; x[7] = v.w * beta;
+    }
+    u32x4 p1, p2;
+    split8h(x, p1, p2);
+    u32x4 *dst = Wp + ((size_t)(ci * NT + nt) * 2) * 64 + lane;
+    dst[0] = p1; dst[64] = p2;
+}
+
+__device__ __forceinline__ void hw_chunk_fetch(const u32x4 *__restrict__ Wp, int c0, int NT, int nt0, u32x4 (&wn)[kHWn])
+{
+    // channel c of the chunk: 2 tiles x 2 pieces x 64 lanes = 256 consecutive uint4
+#pragma unroll
+    for (int i = 0; i < kHWn; ++i) {
+        const int e = threadIdx.x + kHThreads * i, c = e >> 8, o = e & 255;
+        wn[i] = Wp[((size_t)(c0 + c) * NT + nt0) * 128 + o];
+    }
+}
+
+// One pass over all input channels for up to KW texture points per facet.  shs = alpha_f / K_f, the factor on
+// the SH values of my facet.
+template <int KW, bool TVEC>
+__device__ __forceinline__ void h2_sweep(const float *__restrict__ tex, const u32x4 *__restrict__ Wp,
+                                         const float *__restrict__ sh, u32x4 *Ws, float *slab, f32x16 (&acc)[2],
+                                         int kbase, int Ks, float shs, const int *s_k0, const int *s_K, int sweep,
+                                         int Cin, int NT, int nt0, int nblk, int w, int lane, int h)
+{
+    const int l32 = lane & 31;
+    float shr[KW][8];
+#pragma unroll
+    for (int kk = 0; kk < KW; ++kk) {
+        float4 u = make_float4(0.f, 0.f, 0.f, 0.f), v = u;
+        if (kk < Ks) {
+            const float *p = sh + (int64_t)(kbase + kk) * 16 + 8 * h;
+            u = hld4(p);
+            v = hld4(p + 4);
+        }
+        shr[kk][0] = u.x * shs; shr[kk][1] = u.y * shs; shr[kk][2] = u.z * shs; shr[kk][3] = u.w * shs;
+        shr[kk][4] = v.x * shs; shr[kk][5] = v.y * shs; shr[kk][6] = v.z * shs; shr[kk][7] = v.w * shs;
+    }
+    // rows this lane fetches for the slab: load i covers point i of facet slot lane/2, channels 4*(lane%2) .. +3 of the group
+    const int cg4 = 4 * (lane & 1);
+    unsigned ldoff[KW];
+    bool ldok[KW];
+#pragma unroll
+    for (int i = 0; i < KW; ++i) {
+        const int slot = w * 32 + (lane >> 1), kk = sweep * kHKB + i;
+        ldok[i] = kk < s_K[slot];
+        ldoff[i] = (unsigned)(s_k0[slot] + (ldok[i] ? kk : 0)) * (unsigned)Cin + cg4;
+    }
+    float4 pf[KW];
+    auto fetch_group = [&](int g) {
+#pragma unroll
+        for (int i = 0; i < KW; ++i)
+            pf[i] = ldok[i] ? hld4_row<TVEC>(tex + (ldoff[i] + 8 * g), Cin - (8 * g + cg4)) : make_float4(0.f, 0.f, 0.f, 0.f);
+    };
+    auto publish_group = [&](float *dst) {
+#pragma unroll
+        for (int i = 0; i < KW; ++i) {
+            float *q = dst + (i * 8 + cg4) * 32 + (lane >> 1);
+            q[0] = pf[i].x; q[32] = pf[i].y; q[64] = pf[i].z; q[96] = pf[i].w;
+        }
+    };
+    u32x4 wn[kHWn];
+    fetch_group(0);
+    publish_group(slab);
+    hw_chunk_fetch(Wp, 0, NT, nt0, wn);
+#pragma unroll
+    for (int i = 0; i < kHWn; ++i) Ws[threadIdx.x + kHThreads * i] = wn[i];
+    if (nblk > 1) {
+        hw_chunk_fetch(Wp, 4, NT, nt0, wn);
+#pragma unroll
+        for (int i = 0; i < kHWn; ++i) Ws[kHChunk + threadIdx.x + kHThreads * i] = wn[i];
+    }
+    __syncthreads();
+
+    auto read_b = [&](u32x4 (&b)[2][2], int c) {          // filter pieces of channel c
+        const u32x4 *Wc = Ws + ((c >> 2) % 3) * kHChunk + (c & 3) * 256 + lane;
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int p = 0; p < 2; ++p) b[t][p] = Wc[(t * 2 + p) * 64];
+    };
+    auto read_tv = [&](float (&tv)[KW], int c) {          // my facet's texture values of channel c
+        const float *sl = slab + ((c >> 3) & 1) * kHSlab + (c & 7) * 32 + l32;
+#pragma unroll
+        for (int kk = 0; kk < KW; ++kk) tv[kk] = sl[kk * 8 * 32];
+    };
+    auto gen = [&](float (&a)[8], const float (&tv)[KW]) {
+#pragma unroll
+        for (int s = 0; s < 8; ++s) {
+            float v = 0.f;
+#pragma unroll
+            for (int kk = 0; kk < KW; ++kk) v = fmaf(tv[kk], shr[kk][s], v);
+            // keep the fp32 value: fused with the conversion below (one rounding instead of two) the first piece
+            // would depend on which instantiation the compiler fuses, and results on the facet order
+            asm volatile("" : "+v"(v));
+            a[s] = v;
+        }
+    };
+
+    // software pipeline over channels: while channel c is multiplied, the G values of c+1 are generated and
+    // split, and the LDS reads for c+1 (filter) and c+2 (texture) are in flight
+    u32x4 pa[2], b[2][2];
+    float tvn[KW];
+    {
+        float tv0[KW], a[8];
+        read_tv(tv0, 0);
+        read_tv(tvn, 1);
+        read_b(b, 0);
+        gen(a, tv0);
+        split8h(a, pa[0], pa[1]);
+    }
+    for (int j = 0; j < nblk; ++j) {
+        const int g = j >> 1;
+        const bool wmore = j + 2 < nblk;
+        const bool stage = !(j & 1) && 8 * (g + 1) < Cin;       // even chunk: bring in the next 8-channel group
+        if (wmore) hw_chunk_fetch(Wp, 4 * (j + 2), NT, nt0, wn);
+        if (stage) fetch_group(g + 1);
+#pragma unroll
+        for (int ci_l = 0; ci_l < 4; ++ci_l) {
+            const int c = 4 * j + ci_l;
+            u32x4 bn[2][2];
+            float tvnn[KW];
+            read_b(bn, c + 1 < 4 * nblk ? c + 1 : c);
+            read_tv(tvnn, c + 2);
+
+            float an[8];
+            gen(an, tvn);
+            u32x4 pn[2];
+            split8h(an, pn[0], pn[1]);
+
+            // three piece products per accumulator tile, smallest first
+#pragma unroll
+            for (int t = 0; t < 2; ++t) acc[t] = mfma_f16(pa[1], b[t][0], acc[t]);
+#pragma unroll
+            for (int t = 0; t < 2; ++t) acc[t] = mfma_f16(pa[0], b[t][1], acc[t]);
+#pragma unroll
+            for (int t = 0; t < 2; ++t) acc[t] = mfma_f16(pa[0], b[t][0], acc[t]);
+
+            pa[0] = pn[0]; pa[1] = pn[1];
+#pragma unroll
+            for (int kk = 0; kk < KW; ++kk) tvn[kk] = tvnn[kk];
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int p = 0; p < 2; ++p) b[t][p] = bn[t][p];
+        }
+        if (wmore) {
+#pragma unroll
+            for (int i = 0; i < kHWn; ++i) Ws[((j + 2) % 3) * kHChunk + threadIdx.x + kHThreads * i] = wn[i];
+        }
+        if (stage) publish_group(slab + ((g + 1) & 1) * kHSlab);
+        __syncthreads();
+    }
+}
+
+template <bool TVEC>
+__global__ __launch_bounds__(kHThreads, 2) void f2f16h2_fwd_k(const float *__restrict__ tex, const float *__restrict__ hdr,
+                                                              const u32x4 *__restrict__ Wp, const float *__restrict__ sh,
+                                                              const int *__restrict__ cum, const int *__restrict__ order,
+                                                              float *__restrict__ out, int64_t Nf, int T, int Cin,
+                                                              int Cout, int NT)
+{
+    __shared__ u32x4 Ws[3 * kHChunk];
+    __shared__ __attribute__((aligned(16))) float s_slab[kHW * 2 * kHSlab];      // per wavefront: two buffers
+    __shared__ int s_f[256], s_k0[256], s_K[256], s_kmax;
+    __shared__ float s_tm[256], s_inv[256];
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int l32 = lane & 31, h = lane >> 5;
+    const int64_t s0 = (int64_t)blockIdx.x * 256;
+    const int nt0 = blockIdx.y * 2, n0 = blockIdx.y * 64;
+    const int nblk = (Cin + 3) >> 2;
+
+    if (threadIdx.x == 0) s_kmax = 0;
+    for (int i = threadIdx.x; i < 256; i += kHThreads) {
+        const int64_t slot = s0 + i;
+        const int f = slot < Nf ? (order ? order[slot] : (int)slot) : -1;
+        int a = 0, b = 0;
+        if (f >= 0 && f < Nf) {
+            a = f ? cum[f - 1] : 0;
+            b = cum[f];
+            a = a < 0 ? 0 : (a > T ? T : a);
+            b = b < 0 ? 0 : (b > T ? T : b);
+        }
+        s_f[i] = f;
+        s_k0[i] = a;
+        s_K[i] = b > a ? b - a : 0;
+    }
+    __syncthreads();
+    const int k0 = s_k0[w * 32 + l32], K = s_K[w * 32 + l32];
+    {
+        const int km = hwave_max(K);
+        if (lane == 0) atomicMax(&s_kmax, km);
+    }
+
+    // pre-scan: largest |texture value| of each facet's rows (two lanes per row, as the slab fetches) and
+    // largest |SH value| of my facet's rows (my half's eight d's; the halves meet through s_tm)
+    {
+        const int slot = w * 32 + (lane >> 1), cg4 = 4 * (lane & 1);
+        const int rk0 = s_k0[slot], rK = s_K[slot];
+        // all loads of a batch are issued before the first comparison (four rows x 32 channels per lane pair)
+        const int rKmax = hwave_max(rK), Kmax = hwave_max(K);
+        float sm = 0.f;
+        for (int kb = 0; kb < Kmax; kb += 4) {
+            float4 u[4][2];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float *p = sh + (int64_t)(k0 + kb + i) * 16 + 8 * h;
+                const bool ok = kb + i < K;
+                u[i][0] = ok ? hld4(p) : make_float4(0.f, 0.f, 0.f, 0.f);
+                u[i][1] = ok ? hld4(p + 4) : make_float4(0.f, 0.f, 0.f, 0.f);
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i) sm = absmax4(u[i][0], absmax4(u[i][1], sm));
+        }
+        float tm = 0.f;
+        for (int kb = 0; kb < rKmax; kb += 4)
+            for (int cb = 0; cb < Cin; cb += 32) {
+                float4 v[4][4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+#pragma unroll
+                    for (int g = 0; g < 4; ++g) {
+                        const int c = cb + 8 * g + cg4;
+                        v[i][g] = (kb + i < rK && c < Cin) ? hld4_row<TVEC>(tex + (int64_t)(rk0 + kb + i) * Cin + c, Cin - c)
+                                                           : make_float4(0.f, 0.f, 0.f, 0.f);
+                    }
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+#pragma unroll
+                    for (int g = 0; g < 4; ++g) tm = absmax4(v[i][g], tm);
+            }
+        tm = fmaxf(tm, __shfl_xor(tm, 1, 64));
+        sm = fmaxf(sm, __shfl_xor(sm, 32, 64));
+        if (!(lane & 1)) s_tm[slot] = tm;
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        float inv;
+        const float alpha = pow2_scale(s_tm[w * 32 + l32] * sm, &inv);
+        if (h == 0) s_inv[w * 32 + l32] = inv;
+        s_tm[w * 32 + l32] = alpha;          // same wavefront: every read above is done (in-order LDS)
+    }
+    __syncthreads();
+    const float alpha = s_tm[w * 32 + l32];
+    const float shs = K > 0 ? alpha / (float)K : 0.f;
+    const int nsweeps = (s_kmax + kHKB - 1) / kHKB;
+
+    f32x16 acc[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[t][i] = 0.f;
+
+    for (int sw = 0; sw < nsweeps; ++sw) {
+        const int kbase = k0 + sw * kHKB;
+        const int rem = K - sw * kHKB;
+        const int Ks = rem < 0 ? 0 : (rem > kHKB ? kHKB : rem);
+        // every variant runs the same barriers, so wavefronts of a workgroup may pick different ones
+        const int kw = hwave_max(Ks);
+#define PM_H2(N) h2_sweep<N, TVEC>(tex, Wp, sh, Ws, s_slab + w * 2 * kHSlab, acc, kbase, Ks, shs, s_k0, s_K, sw, Cin, NT, nt0, nblk, w, lane, h)
+        if (kw <= 1) PM_H2(1);
+        else if (kw == 2) PM_H2(2);
+        else if (kw == 3) PM_H2(3);
+        else PM_H2(4);
+#undef PM_H2
+    }
+
+    const float ibeta = hdr[1];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        const int slot = w * 32 + 8 * (i / 4) + 4 * h + (i % 4);
+        const int fr = s_f[slot];
+        if (fr >= 0 && fr < Nf) {
+            const float us = s_inv[slot] * ibeta;
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                const int co = n0 + t * 32 + l32;
+                if (co < Cout) out[(int64_t)fr * Cout + co] = acc[t][i] * us;
+            }
+        }
+    }
+}
+
+// workspace: 16-byte header {beta, 1/beta, -, -}, then the packed filter
+size_t f2f16h2_fwd_workspace_bytes(int Cin, int Cout)
+{
+    const int NT = 2 * ((Cout + 63) / 64), CinPad = (Cin + 3) & ~3;
+    return 16 + (size_t)CinPad * NT * 2 * 64 * sizeof(u32x4);
+}
+
+int f2f16h2_fwd(const float *tex, const float *W, const float *sh, const int *cum, const int *order, float *out,
+                void *workspace, size_t workspace_bytes, int64_t T, int64_t Nf, int Cin, int Cout, hipStream_t st)
+{
+    const int NT = 2 * ((Cout + 63) / 64);
+    PM_REQUIRE(T * Cin < (int64_t(1) << 31), "f2f_fwd: texture array too large for 32-bit offsets");
+    PM_REQUIRE(workspace && workspace_bytes >= f2f16h2_fwd_workspace_bytes(Cin, Cout),
+               "f2f_fwd: workspace too small (%zu bytes)", workspace_bytes);
+    PM_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 15u) == 0, "f2f_fwd: workspace must be 16-byte aligned");
+    float *hdr = (float *)workspace;
+    u32x4 *Wp = (u32x4 *)workspace + 1;
+    f2f16h2_scale_filter_k<<<dim3(1), dim3(1024), 0, st>>>(W, hdr, (int64_t)Cout * Cin * 16);
+    PM_LAUNCHED("f2f_fwd(scale)");
+    const int CinPad = (Cin + 3) & ~3, n = CinPad * NT * 64;
+    f2f16h2_pack_filter_k<<<dim3((unsigned)ceil_div(n, kBlock)), dim3(kBlock), 0, st>>>(W, hdr, Wp, Cin, CinPad, Cout, NT);
+    PM_LAUNCHED("f2f_fwd(pack)");
+    const int64_t gx = ceil_div(Nf, 256), gy = NT / 2;
+    PM_REQUIRE(grid_ok(gx) && gy <= 65535, "f2f_fwd: grid too large");
+    if (!(Cin & 3) && !(reinterpret_cast<uintptr_t>(tex) & 15u))
+        f2f16h2_fwd_k<true><<<dim3((unsigned)gx, (unsigned)gy), dim3(kHThreads), 0, st>>>(tex, hdr, Wp, sh, cum, order, out, Nf, (int)T, Cin, Cout, NT);
+    else
+        f2f16h2_fwd_k<false><<<dim3((unsigned)gx, (unsigned)gy), dim3(kHThreads), 0, st>>>(tex, hdr, Wp, sh, cum, order, out, Nf, (int)T, Cin, Cout, NT);
+    PM_LAUNCHED("f2f_fwd");
+    return 0;
+}
+
+}  // namespace pmesh

@@ -26,6 +26,12 @@ size_t f2f16h2_fwd_workspace_bytes(int Cin, int Cout);
 int f2f16h2_fwd(const float *tex, const float *W, const float *sh, const int *cum, const int *order, float *out,
                 void *workspace, size_t workspace_bytes, int64_t T, int64_t Nf, int Cin, int Cout, hipStream_t st);
 
+// texture gradient on the fp16 matrix cores (conditions of the bf16 kernel, workspace no larger)
+size_t f2f16h2_bwd_texture_workspace_bytes(int Cin, int Cout);
+int f2f16h2_bwd_texture(const float *gout, const float *W, const float *sh, const int *cum, const int *order,
+                        float *gtex, void *workspace, size_t workspace_bytes, int64_t T, int64_t Nf, int Cin,
+                        int Cout, hipStream_t st);
+
 // texture gradient on the bf16 matrix cores (Cout % 8 == 0, 16-byte aligned grad_output; output channels are
 // taken 64 at a time, later blocks accumulate onto grad_texture)
 bool f2f16x3_bwd_texture_usable(const void *gout, int Cout);

@@ -413,6 +413,10 @@ extern "C" int pmesh_f2f_bwd_texture(const float *grad_output, const float *filt
     PM_REQUIRE(grad_output && filter && bary_coeff && cum_texture && grad_texture, "f2f_bwd_texture: null pointer");
     f2f_zero_tail_k<<<dim3(64), dim3(kBlock), 0, (hipStream_t)stream>>>(grad_texture, cum_texture, Nf, (int)T, Cin);
     PM_LAUNCHED("f2f_bwd_texture(tail)");
+    if (!force_generic() && !force_fp32_mfma() && !force_bf16x3() && f2f16x3_usable(filter, bary_coeff, F) &&
+        f2f16x3_bwd_texture_usable(grad_output, Cout))
+        return f2f16h2_bwd_texture(grad_output, filter, bary_coeff, cum_texture, facet_order, grad_texture, workspace,
+                                   workspace_bytes, T, Nf, Cin, Cout, (hipStream_t)stream);
     if (!force_generic() && !force_fp32_mfma() && f2f16x3_usable(filter, bary_coeff, F) &&
         f2f16x3_bwd_texture_usable(grad_output, Cout))
         return f2f16x3_bwd_texture(grad_output, filter, bary_coeff, cum_texture, facet_order, grad_texture, workspace,

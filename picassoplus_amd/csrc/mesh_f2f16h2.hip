@@ -444,4 +444,310 @@ int f2f16h2_fwd(const float *tex, const float *W, const float *sh, const int *cu
     return 0;
 }
 
+// ----------------------------------------------------------------------------------------
+// texture gradient on the fp16 matrix cores, same decomposition as the three-piece bf16 kernel:
+//     H[f, ci, d] = sum_co gout[f, co] W[co, ci, d]          (two-piece fp16 MFMAs, k = co)
+//     gtex[t, ci] = (1/K_f) sum_d sh[t, d] H[f, ci, d]       (FMAs on the accumulator registers)
+// The product is taken transposed, D[(ci,d)][f] = (beta W)^T . (gamma_f gout_f)^T with gamma_f from the
+// exact maximum of the facet's gout row (the lane holds it); 1 / (beta gamma_f K_f) rides on the SH values
+// of the contraction.  A tile tt = 4g + q holds the two input channels 8g + q ("a") and 8g + 4 + q ("b");
+// register i of a lane (facet l32, half h)  <->  channel (i/4)%2,  d = 8(i/8) + 4h + i%4.
+constexpr int kHTChunkMax = 2 * 4 * 2 * 64;      // uint4 per chunk buffer: 2 tiles x 4 k-steps x 2 pieces x 64 lanes
+
+// W (Cout, Cin, 16) -> A operands of the transposed product:
+// WpT[((tt*NKS + ks)*2 + piece)*64 + lane] = pieces of beta * W[co0 + 16ks + 8h .. +7][ci(tt, r)][d(r)], r = lane % 32
+__global__ __launch_bounds__(kBlock) void f2f16h2_pack_filter_t_k(const float *__restrict__ W, const float *__restrict__ hdr,
+                                                                  u32x4 *__restrict__ WpT, int Cin, int Cout, int NTt,
+                                                                  int NKS, int co0)
+{
+    const int idx = blockIdx.x * kBlock + threadIdx.x;
+    if (idx >= NTt * NKS * 64) return;
+    const int lane = idx & 63, ks = (idx >> 6) % NKS, tt = (idx >> 6) / NKS;
+    const int r = lane & 31, h = lane >> 5;
+    // row r = 8q + 4h' + j of the tile (h' = accumulator half, register 4q + j): channel q%2, d = 8(q/2) + 4h' + j
+    const int ci = 8 * (tt >> 2) + 4 * ((r >> 3) & 1) + (tt & 3), d = 8 * (r >> 4) + 4 * ((r >> 2) & 1) + (r & 3);
+    const float beta = hdr[0];
+    float x[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const int co = co0 + 16 * ks + 8 * h + j;             // this launch covers channels co0 .. co0 + 16 NKS - 1
+        x[j] = (ci < Cin && co < Cout) ? beta * W[((int64_t)co * Cin + ci) * 16 + d] : 0.f;
+    }
+    u32x4 p1, p2;
+    split8h(x, p1, p2);
+    u32x4 *dst = WpT + ((size_t)(tt * NKS + ks) * 2) * 64 + lane;
+    dst[0] = p1; dst[64] = p2;
+}
+
+template <int KW, int NKS, bool GVEC>
+__device__ __forceinline__ void h2_tex_sweep(const u32x4 *__restrict__ WpT, const float *__restrict__ sh,
+                                             float *__restrict__ gtex, u32x4 *Ws, float *stage, const int *w_k0,
+                                             const int *w_K, const u32x4 (&bp)[NKS][2], int kbase, int Ks, float shs,
+                                             int sweep, int Cin, int NG, bool add, int lane, int h)
+{
+    // SH values of my facet's points for my half's eight d's (4h..4h+3, 8+4h..8+4h+3), times shs = 1 / (K gamma beta):
+    // the scales of the two operands leave with the contraction
+    float shr[KW][8];
+#pragma unroll
+    for (int kk = 0; kk < KW; ++kk) {
+        float4 u = make_float4(0.f, 0.f, 0.f, 0.f), v = u;
+        if (kk < Ks) {
+            const float *p = sh + (int64_t)(kbase + kk) * 16 + 4 * h;
+            u = hld4(p);
+            v = hld4(p + 8);
+        }
+        shr[kk][0] = u.x * shs; shr[kk][1] = u.y * shs; shr[kk][2] = u.z * shs; shr[kk][3] = u.w * shs;
+        shr[kk][4] = v.x * shs; shr[kk][5] = v.y * shs; shr[kk][6] = v.z * shs; shr[kk][7] = v.w * shs;
+    }
+    constexpr int chunk = 2 * NKS * 128;         // uint4 per chunk of two tiles
+    constexpr int NWF = (chunk + 511) / 512;     // uint4 fetched per thread
+    const int nchunks = 2 * NG;
+    auto chunk_fetch = [&](u32x4 (&wn)[NWF], int c) {
+#pragma unroll
+        for (int i = 0; i < NWF; ++i) {
+            const int e = threadIdx.x + 512 * i;
+            if (e < chunk) wn[i] = WpT[(size_t)c * chunk + e];
+        }
+    };
+    auto chunk_publish = [&](const u32x4 (&wn)[NWF], int c) {
+#pragma unroll
+        for (int i = 0; i < NWF; ++i) {
+            const int e = threadIdx.x + 512 * i;
+            if (e < chunk) Ws[(c % 3) * kHTChunkMax + e] = wn[i];
+        }
+    };
+    u32x4 wn[NWF];
+    chunk_fetch(wn, 0);
+    chunk_publish(wn, 0);
+    chunk_fetch(wn, 1);
+    chunk_publish(wn, 1);
+    __syncthreads();
+
+    // 16-channel block gp of the stage -> global memory
+    auto flush = [&](int gp) {
+        const int ci = 16 * gp + 4 * (lane & 3);
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const int slot = 16 * i + (lane >> 2);
+            const int k0s = w_k0[slot] + sweep * kHKB, Kss = w_K[slot] - sweep * kHKB;
+#pragma unroll
+            for (int kk = 0; kk < KW; ++kk)
+                if (kk < Kss && ci < Cin) {
+                    const float4 v = *reinterpret_cast<const float4 *>(stage + (kk * 32 + slot) * 16 + 4 * (lane & 3));
+                    float *dst = gtex + (int64_t)(k0s + kk) * Cin + ci;
+                    // `add`: a later block of 64 output channels accumulates onto what the earlier ones wrote
+                    if constexpr (GVEC) {
+                        float4 o = v;
+                        if (add) {
+                            const float4 p = *reinterpret_cast<const float4 *>(dst);
+                            o = make_float4(p.x + v.x, p.y + v.y, p.z + v.z, p.w + v.w);
+                        }
+                        *reinterpret_cast<float4 *>(dst) = o;
+                    } else {                               // channel count not a multiple of 4 / unaligned rows
+                        dst[0] = add ? dst[0] + v.x : v.x;
+                        if (ci + 1 < Cin) dst[1] = add ? dst[1] + v.y : v.y;
+                        if (ci + 2 < Cin) dst[2] = add ? dst[2] + v.z : v.z;
+                        if (ci + 3 < Cin) dst[3] = add ? dst[3] + v.w : v.w;
+                    }
+                }
+        }
+    };
+    // Results go out 64 bytes at a time: two groups (16 channels) of every point are collected in
+    // the wavefront's LDS stage [point][facet slot][16 channels], then four lanes write one
+    // 64-byte piece of a row (32-byte pieces cost almost twice the HBM write traffic).
+    float gacc[KW][4];
+    auto finish_group = [&](int g) {
+#pragma unroll
+        for (int kk = 0; kk < KW; ++kk)
+            *reinterpret_cast<float4 *>(stage + (kk * 32 + (lane & 31)) * 16 + (g & 1) * 8 + 4 * h) =
+                make_float4(gacc[kk][0], gacc[kk][1], gacc[kk][2], gacc[kk][3]);
+        if ((g & 1) || g == NG - 1) flush(g >> 1);
+    };
+    // contraction of a finished tile (accumulator accp) into channel slot q of the group
+    f32x16 accp;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) accp[i] = 0.f;
+    auto contract = [&](int q) {
+        float xa[KW], xb[KW];
+#pragma unroll
+        for (int kk = 0; kk < KW; ++kk) {
+            float va = 0.f, vb = 0.f;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                va = fmaf(shr[kk][j], accp[8 * (j >> 2) + (j & 3)], va);          // channel a: registers 0-3, 8-11
+                vb = fmaf(shr[kk][j], accp[8 * (j >> 2) + 4 + (j & 3)], vb);      // channel b: registers 4-7, 12-15
+            }
+            xa[kk] = va;
+            xb[kk] = vb;
+        }
+        // xa: half 0 keeps its own, receives half 0's xb into half 1; xb: half 0 receives half 1's xa.
+        // Afterwards xa + xb is the full sum over d of channel a in half 0 and of channel b in half 1.
+        // (The s_nop cover the wait states between vector ALU writes / reads and the swap.)
+#pragma unroll
+        for (int kk = 0; kk < KW; ++kk)
+            asm volatile("s_nop 3\n v_permlane32_swap_b32 %0, %1\n s_nop 3" : "+v"(xa[kk]), "+v"(xb[kk]));
+#pragma unroll
+        for (int kk = 0; kk < KW; ++kk) gacc[kk][q] = xa[kk] + xb[kk];
+    };
+
+    for (int g = 0; g < NG; ++g) {
+#pragma unroll
+        for (int cc = 0; cc < 2; ++cc) {
+            const int c = 2 * g + cc;
+            const bool more = c + 2 < nchunks;
+            if (more) chunk_fetch(wn, c + 2);
+            const u32x4 *Wc = Ws + (c % 3) * kHTChunkMax + lane;
+#pragma unroll
+            for (int u = 0; u < 2; ++u) {
+                // H tile of two input channels: rows (d half, channel, d), columns = my wavefront's facets
+                f32x16 acc0;
+#pragma unroll
+                for (int i = 0; i < 16; ++i) acc0[i] = 0.f;
+#pragma unroll
+                for (int ks = 0; ks < NKS; ++ks) {
+                    u32x4 a[2];
+#pragma unroll
+                    for (int p = 0; p < 2; ++p) a[p] = Wc[((u * NKS + ks) * 2 + p) * 64];
+                    // three piece products, smallest first
+                    acc0 = mfma_f16(a[1], bp[ks][0], acc0);
+                    acc0 = mfma_f16(a[0], bp[ks][1], acc0);
+                    acc0 = mfma_f16(a[0], bp[ks][0], acc0);
+                }
+                // meanwhile: the previous tile (the last one of the previous group when cc = u = 0)
+                contract((2 * cc + u + 3) & 3);
+                if (cc == 0 && u == 0 && g > 0) finish_group(g - 1);
+                accp = acc0;
+            }
+            if (more) chunk_publish(wn, c + 2);
+            __syncthreads();
+        }
+    }
+    contract(3);
+    finish_group(NG - 1);
+}
+
+// NKS = k-steps of 16 output channels (compile time, so that a tile's MFMAs and the previous tile's
+// contraction share one basic block and get interleaved): 2 for Cout <= 32, else 4; the packed filter
+// is zero padded to that many.
+template <int NKS, bool GVEC>
+__global__ __launch_bounds__(512, 2) void f2f16h2_bwd_tex_k(const float *__restrict__ gout,
+                                                            const float *__restrict__ hdr,
+                                                            const u32x4 *__restrict__ WpT,
+                                                            const float *__restrict__ sh,
+                                                            const int *__restrict__ cum,
+                                                            const int *__restrict__ order, float *__restrict__ gtex,
+                                                            int64_t Nf, int T, int Cin, int Cout, int NG, int co0)
+{
+    __shared__ u32x4 Ws[3 * kHTChunkMax];
+    __shared__ __attribute__((aligned(16))) float s_stage[8][kHKB * 32 * 16];
+    __shared__ int s_k0[8][32], s_K[8][32], s_kmax;
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int l32 = lane & 31, h = lane >> 5;
+    if (threadIdx.x == 0) s_kmax = 0;
+    __syncthreads();
+
+    const int64_t slot = (int64_t)blockIdx.x * 256 + w * 32 + l32;
+    const int f = slot < Nf ? (order ? order[slot] : (int)slot) : -1;
+    int k0 = 0, K = 0;
+    if (f >= 0 && f < Nf) {
+        int a = f ? cum[f - 1] : 0, b = cum[f];
+        a = a < 0 ? 0 : (a > T ? T : a);
+        b = b < 0 ? 0 : (b > T ? T : b);
+        k0 = a;
+        K = b > a ? b - a : 0;
+    }
+    if (h == 0) {
+        s_k0[w][l32] = k0;
+        s_K[w][l32] = K;
+    }
+    {
+        const int km = hwave_max(K);
+        if (lane == 0) atomicMax(&s_kmax, km);
+    }
+    // my facet's gout row (the 16 NKS channels of this launch), scaled by gamma_f = a power of two that brings
+    // its largest element below 2^14, as B operand pieces: k-step ks, half h <-> channels 16ks + 8h .. + 7
+    float x[NKS][8];
+    float gm = 0.f;
+#pragma unroll
+    for (int ks = 0; ks < NKS; ++ks) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) x[ks][j] = 0.f;
+        const int co = co0 + 16 * ks + 8 * h;
+        if (K > 0 && co < Cout) {
+            const float *p = gout + (int64_t)f * Cout + co;
+            const float4 u = hld4(p), v = hld4(p + 4);
+            x[ks][0] = u.x; x[ks][1] = u.y; x[ks][2] = u.z; x[ks][3] = u.w;
+            x[ks][4] = v.x; x[ks][5] = v.y; x[ks][6] = v.z; x[ks][7] = v.w;
+            gm = absmax4(u, absmax4(v, gm));
+        }
+    }
+    gm = fmaxf(gm, __shfl_xor(gm, 32, 64));
+    float igamma;
+    const float gamma = pow2_scale(gm, &igamma);
+    u32x4 bp[NKS][2];
+#pragma unroll
+    for (int ks = 0; ks < NKS; ++ks) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) x[ks][j] *= gamma;
+        split8h(x[ks], bp[ks][0], bp[ks][1]);
+    }
+    const float shs = K > 0 ? igamma * hdr[1] / (float)K : 0.f;
+    __syncthreads();
+    const int nsweeps = (s_kmax + kHKB - 1) / kHKB;
+    for (int sw = 0; sw < nsweeps; ++sw) {
+        const int rem = K - sw * kHKB;
+        const int Ks = rem < 0 ? 0 : (rem > kHKB ? kHKB : rem);
+        const int kw = hwave_max(Ks);
+        const int kbase = k0 + sw * kHKB;
+        // every variant runs the same barriers, so wavefronts of a workgroup may pick different ones
+#define PM_H2T(N) h2_tex_sweep<N, NKS, GVEC>(WpT, sh, gtex, Ws, s_stage[w], s_k0[w], s_K[w], bp, kbase, Ks, shs, sw, Cin, NG, co0 > 0, lane, h)
+        if (kw <= 1) PM_H2T(1);
+        else if (kw == 2) PM_H2T(2);
+        else if (kw == 3) PM_H2T(3);
+        else PM_H2T(4);
+#undef PM_H2T
+    }
+}
+
+
+// workspace: 16-byte header {beta, 1/beta, -, -}, then the packed W^T of one block of at most 64 output channels
+size_t f2f16h2_bwd_texture_workspace_bytes(int Cin, int Cout)
+{
+    const int NG = (Cin + 7) / 8, NKS = Cout <= 32 ? 2 : 4;
+    return 16 + (size_t)NG * 4 * NKS * 2 * 64 * sizeof(u32x4);
+}
+
+int f2f16h2_bwd_texture(const float *gout, const float *W, const float *sh, const int *cum, const int *order,
+                        float *gtex, void *workspace, size_t workspace_bytes, int64_t T, int64_t Nf, int Cin,
+                        int Cout, hipStream_t st)
+{
+    const int NG = (Cin + 7) / 8;
+    PM_REQUIRE(workspace && workspace_bytes >= f2f16h2_bwd_texture_workspace_bytes(Cin, Cout),
+               "f2f_bwd_texture: workspace too small (%zu bytes)", workspace_bytes);
+    PM_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 15u) == 0, "f2f_bwd_texture: workspace must be 16-byte aligned");
+    float *hdr = (float *)workspace;
+    u32x4 *WpT = (u32x4 *)workspace + 1;
+    f2f16h2_scale_filter_k<<<dim3(1), dim3(1024), 0, st>>>(W, hdr, (int64_t)Cout * Cin * 16);
+    PM_LAUNCHED("f2f_bwd_texture(scale)");
+    const int64_t gx = ceil_div(Nf, 256);
+    PM_REQUIRE(grid_ok(gx), "f2f_bwd_texture: grid too large");
+    const bool gvec = !(Cin & 3) && !(reinterpret_cast<uintptr_t>(gtex) & 15u);
+    // output channels go 64 at a time; the first block writes grad_texture, the others add to it
+    // (launches on one stream run in order, so the packed filter buffer is reused)
+    for (int co0 = 0; co0 < Cout; co0 += 64) {
+        const int NKS = Cout - co0 <= 32 ? 2 : 4;
+        const int n = NG * 4 * NKS * 64;
+        f2f16h2_pack_filter_t_k<<<dim3((unsigned)ceil_div(n, kBlock)), dim3(kBlock), 0, st>>>(W, hdr, WpT, Cin, Cout, NG * 4, NKS, co0);
+        PM_LAUNCHED("f2f_bwd_texture(pack)");
+#define PM_TEX(N, G) f2f16h2_bwd_tex_k<N, G><<<dim3((unsigned)gx), dim3(512), 0, st>>>(gout, hdr, WpT, sh, cum, order, gtex, Nf, (int)T, Cin, Cout, NG, co0)
+        if (NKS == 2 && gvec) PM_TEX(2, true);
+        else if (NKS == 2) PM_TEX(2, false);
+        else if (gvec) PM_TEX(4, true);
+        else PM_TEX(4, false);
+#undef PM_TEX
+        PM_LAUNCHED("f2f_bwd_texture");
+    }
+    return 0;
+}
+
 }  // namespace pmesh

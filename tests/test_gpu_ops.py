@@ -158,15 +158,19 @@ def test_f2v_unit_count_is_plain_scatter(cuda):
                                                 (333, 16, 96, 16, 4), (70, 5, 7, 9, 3), (65, 4, 6, 36, 2),
                                                 (64, 3, 5, 50, 2), (129, 130, 64, 4, 3), (50, 8, 8, 1, 2),
                                                 (300, 8, 40, 16, 14), (1000, 64, 64, 16, 9), (130, 4, 130, 16, 20)])
-@pytest.mark.parametrize("path", ["default", "generic", "fp32mfma"])
+@pytest.mark.parametrize("path", ["default", "generic", "fp32mfma", "bf16x3"])
 def test_f2f_parity(cuda, monkeypatch, nf, Cin, Cout, F, kmax, path):
-    """``generic`` forces the shape-generic kernels and ``fp32mfma`` the fp32-matrix-instruction variant
-    of the 16-coefficient path, also where the split-bf16 kernels apply."""
+    """``generic`` forces the shape-generic kernels, ``fp32mfma`` the fp32-matrix-instruction variant of the
+    16-coefficient path and ``bf16x3`` the three-piece bf16 kernels, also where the two-piece fp16 kernels
+    (the default for 16 coefficients) apply."""
     say("case f2f", nf, Cin, Cout, F, kmax, path)
-    if path != "default" and not (F == 16 and Cin % 4 == 0):
+    if path in ("generic", "fp32mfma") and not (F == 16 and Cin % 4 == 0):
         pytest.skip("shape already runs the generic kernels")
+    if path == "bf16x3" and F != 16:
+        pytest.skip("the split kernels need 16 coefficients")
     monkeypatch.setenv("PMESH_F2F_GENERIC", "1" if path == "generic" else "0")
     monkeypatch.setenv("PMESH_F2F_FP32MFMA", "1" if path == "fp32mfma" else "0")
+    monkeypatch.setenv("PMESH_F2F_BF16X3", "1" if path == "bf16x3" else "0")
     rng = np.random.default_rng(13)
     counts, bary, owner = texture_case(rng, nf, kmax)
     cum = np.cumsum(counts).astype(np.int32)

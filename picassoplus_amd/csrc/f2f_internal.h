@@ -40,6 +40,10 @@ int f2f16x3_bwd_texture(const float *gout, const float *W, const float *sh, cons
                         float *gtex, void *workspace, size_t workspace_bytes, int64_t T, int64_t Nf, int Cin,
                         int Cout, hipStream_t st);
 
+// the same on the fp16 matrix cores (block-floating scales, see mesh_f2f16h2.hip)
+int f2f16h2_bwd_filter_partials(const float *gout, const float *tex, const float *sh, const int *cum, const int *order,
+                                 float *partial, int splits, int64_t T, int64_t Nf, int Cin, int Cout, hipStream_t st);
+
 // `splits` workgroups each write one partial (Cout x Cin*16) block; every split gets a strided share of the 32-facet tiles
 int f2f16x3_bwd_filter_partials(const float *gout, const float *tex, const float *sh, const int *cum, const int *order,
                                  float *partial, int splits, int64_t T, int64_t Nf, int Cin, int Cout, hipStream_t st);

@@ -467,8 +467,11 @@ extern "C" int pmesh_f2f_bwd_filter(const float *grad_output, const float *textu
     if (!force_generic() && (x3 || f2f16_usable(texture, texture, bary_coeff, Cin, F))) {
         int rc = !x3 ? f2f16_bwd_filter_partials(grad_output, texture, bary_coeff, cum_texture, (float *)workspace, S, T,
                                                  Nf, Cin, Cout, st)
-                     : f2f16x3_bwd_filter_partials(grad_output, texture, bary_coeff, cum_texture, facet_order,
-                                                   (float *)workspace, S, T, Nf, Cin, Cout, st);
+                     : force_bf16x3()
+                         ? f2f16x3_bwd_filter_partials(grad_output, texture, bary_coeff, cum_texture, facet_order,
+                                                       (float *)workspace, S, T, Nf, Cin, Cout, st)
+                         : f2f16h2_bwd_filter_partials(grad_output, texture, bary_coeff, cum_texture, facet_order,
+                                                       (float *)workspace, S, T, Nf, Cin, Cout, st);
         if (rc) return rc;
         f2f_reduce_k<<<dim3((unsigned)ceil_div(nW, 64)), dim3(kBlock), 0, st>>>((const float *)workspace, grad_filter, S, nW);
         PM_LAUNCHED("f2f_bwd_filter(reduce)");

@@ -49,12 +49,16 @@ __device__ __forceinline__ float absmax4(const float4 &v, float m)
 }
 
 // Eight fp32 values -> two packed fp16x8 pieces, both rounded to nearest (one v_cvt_pk_f16_f32 per pair); the
-// remainder x - x1 is exact in fp32 and comes from one mixed-precision FMA per value.
+// remainder x - x1 is exact in fp32.  The empty asm pins each value as an fp32 register first: otherwise the
+// compiler may fold the FMA that produced it into ONE of the two conversions of x1 it emits (a mixed-precision
+// FMA rounds the exact product once), and in a near-tie the piece that is multiplied and the piece the
+// remainder was taken from differ by one fp16 ulp.
 __device__ __forceinline__ void split8h(const float (&x)[8], u32x4 &p1, u32x4 &p2)
 {
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-        const float a = x[2 * j], b = x[2 * j + 1];
+        float a = x[2 * j], b = x[2 * j + 1];
+        asm volatile("" : "+v"(a), "+v"(b));
         f16x2 hi, lo;
         hi[0] = (_Float16)a;
         hi[1] = (_Float16)b;
@@ -221,9 +225,6 @@ __device__ __forceinline__ void h2_sweep(const float *__restrict__ tex, const u3
             float v = 0.f;
 #pragma unroll
             for (int kk = 0; kk < KW; ++kk) v = fmaf(tv[kk], shr[kk][s], v);
-            // keep the fp32 value: fused with the conversion below (one rounding instead of two) the first piece
-            // would depend on which instantiation the compiler fuses, and results on the facet order
-            asm volatile("" : "+v"(v));
             a[s] = v;
         }
     };
@@ -747,6 +748,467 @@ int f2f16h2_bwd_texture(const float *gout, const float *W, const float *sh, cons
 #undef PM_TEX
         PM_LAUNCHED("f2f_bwd_texture");
     }
+    return 0;
+}
+
+// ----------------------------------------------------------------------------------------
+// filter gradient gW = gout^T . G on the fp16 matrix cores, same decomposition as the three-piece bf16
+// kernel: G is formed as in the forward (lane = facet, eight d's in registers), split into two fp16 pieces,
+// and each piece is transposed by the matrix core itself (D = piece . E with a 0/1 selection matrix is
+// exact), which leaves lane = column (channel, d) and registers = facets -- the layout of an operand whose
+// reduction index is the facet.  Two input channels share one transposition tile.
+//
+// The reduction runs over facets, so the power-of-two scales of the two operands cannot differ from facet
+// to facet inside a sum.  They are uniform per pass instead, and the accumulators carry a scale of their own:
+//     gamma   one per 32-facet tile and workgroup, on the gout^T operand that the workgroup prepares in LDS.
+//             The operand of the next tile is split with the scale of the tiles before it (with 2^3 of
+//             head room) while its own maximum is collected; in the rare case that this maximum would
+//             overflow fp16 or leave fewer than 2^5 above the smallest normal step, the tile is fetched
+//             and split again with a scale of its own.
+//     alpha   one per pass and wavefront, on G.  A wavefront's accumulators keep one scale S = alpha * gamma,
+//             fixed by its first pass (with 2^9 of head room below the overflow bound from the largest
+//             texture value it just fetched and the largest SH value of its facets), so alpha = S / gamma
+//             afterwards; 1 / S is taken out when the partial result is written.  Small operands cost
+//             nothing (their error is absolute, far below the accumulated sum); a pass whose alpha would
+//             overflow takes the largest safe alpha and is accumulated 2^k times.
+//   workgroup  4 wavefronts (one per SIMD), 64 input x 64 output channels, a strided subset of the tiles
+//   wavefront  16 input channels = 8 channel pairs x 2 output tiles of gW^T[(ci,d)][co]; narrower filters give
+//              every wavefront 1, 2 or 4 pairs instead (NCP)
+template <int KW, int NCP>
+__device__ __forceinline__ void h2_filt_pass(const float (&shr)[KW][8], const float4 *slab, const u32x4 *go,
+                                             f32x16 (&acc)[NCP][2], const u32x4 &ea, const u32x4 &eb, int lane)
+{
+    const int l32 = lane & 31;
+    // G of channels cbase + 2cp (a) and + 1 (b), eight d's of my half for my facet, as fp16 pieces
+    auto gen = [&](u32x4 (&pa)[2], u32x4 (&pb)[2], int cp) {
+        float aa[8], ab[8];
+#pragma unroll
+        for (int kk = 0; kk < KW; ++kk) {
+            const float4 t4 = slab[(kk * 4 + (cp >> 1)) * 32 + l32];
+            const float ta = (cp & 1) ? t4.z : t4.x, tb = (cp & 1) ? t4.w : t4.y;
+#pragma unroll
+            for (int q = 0; q < 8; ++q) {
+                aa[q] = kk ? fmaf(ta, shr[kk][q], aa[q]) : ta * shr[kk][q];
+                ab[q] = kk ? fmaf(tb, shr[kk][q], ab[q]) : tb * shr[kk][q];
+            }
+        }
+        split8h(aa, pa[0], pa[1]);
+        split8h(ab, pb[0], pb[1]);
+    };
+    // The four transposition MFMAs are one asm block with VGPR destinations: in a kernel whose accumulators
+    // live in AGPRs the compiler gives every MFMA an AGPR destination, and the results would have to be
+    // copied out one by one before the packing.  The compiler cannot see into the block: the s_nop in the middle
+    // keep the second product of a chain behind the first one's write of its accumulator (only one other MFMA
+    // lies between them), the trailing ones cover the wait states a vector ALU read of an MFMA result needs.
+    auto transpose = [&](u32x4 (&o)[2][2], const u32x4 (&pa)[2], const u32x4 (&pb)[2]) {
+        f32x16 d0, d1;
+        asm volatile("s_nop 3\n"
+                     "v_mfma_f32_32x32x16_f16 %0, %2, %6, 0\n"
+                     "v_mfma_f32_32x32x16_f16 %1, %3, %6, 0\n"
+                     "s_nop 7\n"
+                     "s_nop 7\n"
+                     "v_mfma_f32_32x32x16_f16 %0, %4, %7, %0\n"
+                     "v_mfma_f32_32x32x16_f16 %1, %5, %7, %1\n"
+                     "s_nop 15\n"
+                     "s_nop 7\n"
+                     : "=&v"(d0), "=&v"(d1)
+                     : "v"(pa[0]), "v"(pa[1]), "v"(pb[0]), "v"(pb[1]), "v"(ea), "v"(eb));
+        // every result is one fp16 value, so the conversion back is exact
+#pragma unroll
+        for (int st = 0; st < 2; ++st)
+#pragma unroll
+            for (int jj = 0; jj < 4; ++jj) {
+                o[0][st][jj] = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_pkrtz(d0[8 * st + 2 * jj], d0[8 * st + 2 * jj + 1]));
+                o[1][st][jj] = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_pkrtz(d1[8 * st + 2 * jj], d1[8 * st + 2 * jj + 1]));
+            }
+    };
+
+    // the gout^T operand stays in registers for the whole pass (it serves all channel pairs)
+    u32x4 g[2][2][2];
+#pragma unroll
+    for (int st = 0; st < 2; ++st)
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int p = 0; p < 2; ++p) g[st][t][p] = go[((st * 2 + t) * 2 + p) * 64 + lane];
+
+    // software pipeline over the channel pairs: the G values of pair cp+1 are generated and split
+    // (vector ALU) while the products of pair cp run on the matrix core
+    u32x4 o[2][2];
+    {
+        u32x4 pa[2], pb[2];
+        gen(pa, pb, 0);
+        transpose(o, pa, pb);
+    }
+#pragma unroll
+    for (int cp = 0; cp < NCP; ++cp) {
+        u32x4 pa[2], pb[2];
+        if (cp + 1 < NCP) gen(pa, pb, cp + 1);
+#pragma unroll
+        for (int st = 0; st < 2; ++st) {
+            // three piece products, smallest first; the two output tiles alternate
+#pragma unroll
+            for (int t = 0; t < 2; ++t) acc[cp][t] = mfma_f16(o[1][st], g[st][t][0], acc[cp][t]);
+#pragma unroll
+            for (int t = 0; t < 2; ++t) acc[cp][t] = mfma_f16(o[0][st], g[st][t][1], acc[cp][t]);
+#pragma unroll
+            for (int t = 0; t < 2; ++t) acc[cp][t] = mfma_f16(o[0][st], g[st][t][0], acc[cp][t]);
+        }
+        if (cp + 1 < NCP) transpose(o, pa, pb);
+    }
+}
+
+// slot descriptors of a 32-facet tile: facet id (-1: none), first texture point, number of points
+struct HTile {
+    int f, k0, K;
+};
+__device__ __forceinline__ HTile htile_load(const int *__restrict__ cum, const int *__restrict__ order, int64_t tile,
+                                            int64_t ntiles, int64_t Nf, int T, int i)
+{
+    HTile d = {-1, 0, 0};
+    const int64_t slot = tile * 32 + i;
+    if (tile < ntiles && slot < Nf) {
+        const int f = order ? order[slot] : (int)slot;
+        if (f >= 0 && f < Nf) {
+            int a = f ? cum[f - 1] : 0, b = cum[f];
+            a = a < 0 ? 0 : (a > T ? T : a);
+            b = b < 0 ? 0 : (b > T ? T : b);
+            if (b > a) d = {f, a, b - a};
+        }
+    }
+    return d;
+}
+
+// The inputs of a tile's first pass are fetched by the whole workgroup while the previous tile is
+// being multiplied (held in registers, written to the other LDS buffer afterwards):
+//   gout     thread (co, step, half): its eight facets in accumulator-row order
+//   SH rows  32 facets x 4 points x 64 bytes, two 16-byte pieces per thread
+struct HPre {
+    float g[8];
+    float4 shv[2];
+};
+__device__ __forceinline__ void hpre_issue(HPre &P, const float *__restrict__ gout, const float *__restrict__ sh,
+                                           const int *sf, const int *sk0, const int *sK, int Cout, int n0)
+{
+    const int co = threadIdx.x & 63, st = (threadIdx.x >> 6) & 1, hh = threadIdx.x >> 7;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const int f = sf[16 * st + 8 * (j >> 2) + 4 * hh + (j & 3)];
+        P.g[j] = (f >= 0 && n0 + co < Cout) ? gout[(int64_t)f * Cout + n0 + co] : 0.f;
+    }
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const int e = threadIdx.x + 256 * i, row = e >> 2, kk = row >> 5, slot = row & 31;
+        P.shv[i] = kk < sK[slot] ? hld4(sh + (int64_t)(sk0[slot] + kk) * 16 + 4 * (e & 3)) : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+}
+__device__ __forceinline__ float hpre_gmax(const HPre &P)
+{
+    float m = 0.f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) m = fmaxf(m, fabsf(P.g[j]));
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
+    return m;
+}
+// gamma: scale of the gout operand
+__device__ __forceinline__ void hpre_commit(const HPre &P, u32x4 *go, float *shs, float gamma, bool with_sh)
+{
+    const int co = threadIdx.x & 63, st = (threadIdx.x >> 6) & 1, hh = threadIdx.x >> 7;
+    float x[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) x[j] = P.g[j] * gamma;
+    u32x4 p1, p2;
+    split8h(x, p1, p2);
+    u32x4 *dst = go + ((st * 2 + (co >> 5)) * 2) * 64 + 32 * hh + (co & 31);
+    dst[0] = p1; dst[64] = p2;
+    if (with_sh) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const int e = threadIdx.x + 256 * i;
+            *reinterpret_cast<float4 *>(shs + 4 * e) = P.shv[i];             // [point*32 + slot][16]
+        }
+    }
+}
+
+// does the scale s put a maximum m (> 0) into the band the pieces keep their accuracy in?
+__device__ __forceinline__ bool scale_fits(float s, float m) { return s * m < 32768.0f && s * m >= 32.0f; }
+
+// texture rows of one pass (KW points per facet) for my wavefront's channels: 64 bytes per row, four lanes per row
+template <int KW, bool TVEC, int NCP>
+__device__ __forceinline__ void htex_issue(float4 (&pf)[2 * kHKB], const float *__restrict__ tex, const int *sk0,
+                                           const int *sK, int sweep, int cw, int Cin, int lane)
+{
+    const int piece = lane & 3;
+#pragma unroll
+    for (int i = 0; i < 2 * KW; ++i) {
+        const int rr = i * 16 + (lane >> 2), kk = rr >> 5, slot = rr & 31;
+        const bool ok = sweep * kHKB + kk < sK[slot] && 4 * piece < 2 * NCP;
+        pf[i] = ok ? hld4_row<TVEC>(tex + (int64_t)(sk0[slot] + sweep * kHKB + kk) * Cin + cw + 4 * piece,
+                                    Cin - (cw + 4 * piece))
+                   : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+}
+
+__device__ __forceinline__ int htile_kmax(const int *sK, int lane) { return hwave_max(sK[lane & 31]); }
+__device__ __forceinline__ float hwave_fmax(float m)
+{
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
+    return __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, m)));
+}
+
+// State of the scales: gam_cur (workgroup-uniform) = scale the next operand is split with; S
+// (wavefront-uniform) = scale of the accumulators, fixed by the wavefront's first pass.
+struct HScales {
+    float gam_cur, S;
+};
+
+// One tile of 32 facets whose inputs are in LDS buffer it % 2 (descriptors in it % 3): start the
+// fetches for the next tile, run the passes, publish the next tile's inputs.
+template <int KW, bool TVEC, int NCP>
+__device__ __forceinline__ void h2_filt_tile(const float *__restrict__ gout, const float *__restrict__ tex,
+                                             const float *__restrict__ sh, const int *__restrict__ cum,
+                                             const int *__restrict__ order, u32x4 (*go_s)[2 * 2 * 2 * 64], float4 *slab,
+                                             float (*sh_s)[kHKB * 32 * 16], int (*s_f)[32], int (*s_k0)[32],
+                                             int (*s_K)[32], float *s_gamma, unsigned *s_gm, f32x16 (&acc)[NCP][2],
+                                             HScales &sc, const u32x4 &ea, const u32x4 &eb, int it, int64_t tile,
+                                             int64_t stride, int64_t ntiles, int64_t Nf, int T, int Cin, int Cout, int c0,
+                                             int n0, int lane, int w)
+{
+    const int l32 = lane & 31, h = lane >> 5;
+    const int buf = it & 1, sb = it % 3, sb1 = (it + 1) % 3, sb2 = (it + 2) % 3;
+    // in flight while this tile is multiplied: inputs of the next tile, descriptors of the one after
+    HPre P;
+    hpre_issue(P, gout, sh, s_f[sb1], s_k0[sb1], s_K[sb1], Cout, n0);
+    HTile dn = {-1, 0, 0};
+    if (threadIdx.x < 32) dn = htile_load(cum, order, tile + 2 * stride, ntiles, Nf, T, threadIdx.x);
+    // maxima of the gout operands: slot (it + 1) % 3 collects the next tile's at the commit below; the slot of
+    // the tile after that is cleared here (its last readers passed the barrier that ended the previous tile)
+    const int gs = (it + 1) % 3;
+    if (threadIdx.x == 0) s_gm[(it + 2) % 3] = 0u;
+
+    const float gamma = s_gamma[buf];
+    const int k0 = s_k0[sb][l32], K = s_K[sb][l32];
+    const float invK = K > 0 ? 1.0f / (float)K : 0.f;
+    const int nsweeps = KW < kHKB ? 1 : (hwave_max(K) + kHKB - 1) / kHKB;
+    const int cw = c0 + 2 * NCP * w;                     // my wavefront's first input channel
+    const bool idle = cw >= Cin;                         // narrow filters leave wavefronts without channels
+    for (int sw = 0; sw < nsweeps && !idle; ++sw) {
+        const int rem = K - sw * kHKB;
+        const int Ks = rem < 0 ? 0 : (rem > KW ? KW : rem);
+        float shr[KW][8];
+        if (sw == 0) {
+#pragma unroll
+            for (int kk = 0; kk < KW; ++kk) {
+                const float *p = sh_s[buf] + (kk * 32 + l32) * 16 + 8 * h;
+                const float4 u = hld4(p), v = hld4(p + 4);
+                shr[kk][0] = u.x * invK; shr[kk][1] = u.y * invK; shr[kk][2] = u.z * invK; shr[kk][3] = u.w * invK;
+                shr[kk][4] = v.x * invK; shr[kk][5] = v.y * invK; shr[kk][6] = v.z * invK; shr[kk][7] = v.w * invK;
+            }
+        } else {
+            // further points of long facets: fetched directly
+#pragma unroll
+            for (int kk = 0; kk < KW; ++kk) {
+                float4 u = make_float4(0.f, 0.f, 0.f, 0.f), v = u;
+                if (kk < Ks) {
+                    const float *p = sh + (int64_t)(k0 + sw * kHKB + kk) * 16 + 8 * h;
+                    u = hld4(p);
+                    v = hld4(p + 4);
+                }
+                shr[kk][0] = u.x * invK; shr[kk][1] = u.y * invK; shr[kk][2] = u.z * invK; shr[kk][3] = u.w * invK;
+                shr[kk][4] = v.x * invK; shr[kk][5] = v.y * invK; shr[kk][6] = v.z * invK; shr[kk][7] = v.w * invK;
+            }
+        }
+        float tmax = 0.f;
+        {
+            // my wavefront's texture rows of this pass -> slab
+            float4 pf[2 * kHKB];
+            htex_issue<KW, TVEC, NCP>(pf, tex, s_k0[sb], s_K[sb], sw, cw, Cin, lane);
+            const int piece = lane & 3;
+#pragma unroll
+            for (int i = 0; i < 2 * KW; ++i) {
+                const int rr = i * 16 + (lane >> 2), kk = rr >> 5, slot = rr & 31;
+                slab[(kk * 4 + piece) * 32 + slot] = pf[i];
+                tmax = absmax4(pf[i], tmax);
+            }
+        }
+        // scale of G for this pass: |G| <= KW * max|tex| * max|sh / K|
+        float smax = 0.f;
+#pragma unroll
+        for (int kk = 0; kk < KW; ++kk)
+#pragma unroll
+            for (int q = 0; q < 8; ++q) smax = fmaxf(smax, fabsf(shr[kk][q]));
+        const float bound = hwave_fmax(tmax) * hwave_fmax(smax) * (float)KW;
+        if (bound > 0.f) {
+            float inv;
+            const float need = pow2_scale(bound, &inv);          // need * bound < 2^14
+            // The accumulators keep the scale S of the first pass, so alpha follows gamma: alpha = S / gamma.
+            // The first pass leaves 2^9 of head room under `need`; a pass whose alpha would still overflow
+            // takes the largest safe one and is accumulated S / (alpha gamma) times instead (a power of two;
+            // it takes data growing by orders of magnitude along the facet list to get there).
+            if (sc.S == 0.f) sc.S = need * (1.0f / 512.0f) * gamma;
+            float al = sc.S / gamma;
+            int reps = 1;
+            if (al > need) {
+                const float r = al / need;
+                reps = r < 1048576.0f ? (int)r : 1048576;
+                al = need;
+            }
+#pragma unroll
+            for (int kk = 0; kk < KW; ++kk)
+#pragma unroll
+                for (int q = 0; q < 8; ++q) shr[kk][q] *= al;
+            for (int rep = 0; rep < reps; ++rep) h2_filt_pass<KW, NCP>(shr, slab, go_s[buf], acc, ea, eb, lane);
+        }
+    }
+
+    // next tile's operand: split with the running scale, its own maximum collected on the side
+    {
+        const float m = hpre_gmax(P);
+        if (lane == 0) atomicMax(&s_gm[gs], __builtin_bit_cast(unsigned, m));
+    }
+    hpre_commit(P, go_s[buf ^ 1], sh_s[buf ^ 1], sc.gam_cur, true);
+    if (threadIdx.x == 0) s_gamma[buf ^ 1] = sc.gam_cur;
+    if (threadIdx.x < 32) {
+        s_f[sb2][threadIdx.x] = dn.f; s_k0[sb2][threadIdx.x] = dn.k0; s_K[sb2][threadIdx.x] = dn.K;
+    }
+    __syncthreads();
+    const float gm = __builtin_bit_cast(float, s_gm[gs]);
+    if (gm > 0.f && !scale_fits(sc.gam_cur, gm)) {           // workgroup-uniform: fetch and split that tile again
+        float inv;
+        sc.gam_cur = pow2_scale(gm, &inv) * 0.125f;          // gam * gm in [2^10, 2^11)
+        hpre_issue(P, gout, sh, s_f[sb1], s_k0[sb1], s_K[sb1], Cout, n0);
+        hpre_commit(P, go_s[buf ^ 1], sh_s[buf ^ 1], sc.gam_cur, false);
+        if (threadIdx.x == 0) s_gamma[buf ^ 1] = sc.gam_cur;
+        __syncthreads();
+    }
+}
+
+// NCP = channel pairs of a wavefront (8 for 64 or more input channels; fewer for narrow filters, so that
+// the four wavefronts share what channels there are)
+template <bool TVEC, int NCP>
+__global__ __launch_bounds__(256, 1) void f2f16h2_bwd_filt_k(const float *__restrict__ gout,
+                                                              const float *__restrict__ tex,
+                                                              const float *__restrict__ sh,
+                                                              const int *__restrict__ cum,
+                                                              const int *__restrict__ order,
+                                                              float *__restrict__ partial, int64_t Nf, int T, int Cin,
+                                                              int Cout, int64_t ntiles)
+{
+    __shared__ u32x4 go_s[2][2 * 2 * 2 * 64];
+    __shared__ float4 slab_s[4 * kHKB * 4 * 32];
+    __shared__ __attribute__((aligned(16))) float sh_s[2][kHKB * 32 * 16];
+    __shared__ int s_f[3][32], s_k0[3][32], s_K[3][32];
+    __shared__ float s_gamma[2];
+    __shared__ unsigned s_gm[3];
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int l32 = lane & 31, h = lane >> 5;
+    const int c0 = blockIdx.y * (8 * NCP), n0 = blockIdx.z * 64;
+
+    // selection operands of the transposition: column n < 16 takes d = n of channel a, n >= 16 takes d = n - 16 of b
+    u32x4 ea, eb;
+#pragma unroll
+    for (int jj = 0; jj < 4; ++jj) {
+        unsigned va = 0, vb = 0;
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            const int d = 8 * h + 2 * jj + u;
+            if (l32 < 16 && d == l32) va |= 0x3C00u << (16 * u);            // fp16 1.0
+            if (l32 >= 16 && d == l32 - 16) vb |= 0x3C00u << (16 * u);
+        }
+        ea[jj] = va;
+        eb[jj] = vb;
+    }
+
+    f32x16 acc[NCP][2];
+#pragma unroll
+    for (int cp = 0; cp < NCP; ++cp)
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) acc[cp][t][i] = 0.f;
+    HScales sc = {1.0f, 0.f};
+
+    // prologue: descriptors of my first two tiles, inputs of the first (its gout maximum first, then the split)
+    const int64_t stride = gridDim.x;
+    int64_t tile = blockIdx.x;
+    if (threadIdx.x < 64) {
+        const int q = threadIdx.x >> 5;
+        const HTile d = htile_load(cum, order, tile + q * stride, ntiles, Nf, T, threadIdx.x & 31);
+        s_f[q][threadIdx.x & 31] = d.f; s_k0[q][threadIdx.x & 31] = d.k0; s_K[q][threadIdx.x & 31] = d.K;
+    }
+    if (threadIdx.x < 3) s_gm[threadIdx.x] = 0u;
+    __syncthreads();
+    {
+        HPre P;
+        hpre_issue(P, gout, sh, s_f[0], s_k0[0], s_K[0], Cout, n0);
+        const float m = hpre_gmax(P);
+        if (lane == 0) atomicMax(&s_gm[0], __builtin_bit_cast(unsigned, m));
+        __syncthreads();
+        const float gm = __builtin_bit_cast(float, s_gm[0]);
+        if (gm > 0.f) {
+            float inv;
+            sc.gam_cur = pow2_scale(gm, &inv) * 0.125f;
+        }
+        hpre_commit(P, go_s[0], sh_s[0], sc.gam_cur, true);
+        if (threadIdx.x == 0) s_gamma[0] = sc.gam_cur;
+    }
+    __syncthreads();
+
+    // The sorted facet list makes the point counts of my tiles non-decreasing: four loops in sequence,
+    // each with the pass specialised for its number of points (the last one takes everything left,
+    // long facets in several sweeps).  The bound is uniform over the workgroup.
+    int it = 0;
+#define PM_PHASE(N)                                                                                                  \
+    for (; tile < ntiles && (N == kHKB || htile_kmax(s_K[it % 3], lane) <= N); ++it, tile += stride)                 \
+        h2_filt_tile<N, TVEC, NCP>(gout, tex, sh, cum, order, go_s, slab_s + w * (kHKB * 4 * 32), sh_s, s_f, s_k0, s_K, \
+                                   s_gamma, s_gm, acc, sc, ea, eb, it, tile, stride, ntiles, Nf, T, Cin, Cout, c0, n0, lane, w)
+    PM_PHASE(1);
+    PM_PHASE(2);
+    PM_PHASE(3);
+    PM_PHASE(4);
+#undef PM_PHASE
+
+    // accumulator (cp, t): lane (co = 32t + l32, half h), register i <-> row m = 8(i/4) + 4h + i%4
+    // = (channel c0 + 2 NCP w + 2cp + m/16, d = m%16); four consecutive d's per group of four registers
+    const float unscale = sc.S != 0.f ? 1.0f / sc.S : 0.f;
+    float *dst = partial + (int64_t)blockIdx.x * Cout * Cin * 16;
+#pragma unroll
+    for (int cp = 0; cp < NCP; ++cp)
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            const int co = n0 + 32 * t + l32;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int ci = c0 + 2 * NCP * w + 2 * cp + (q >> 1);
+                if (co < Cout && ci < Cin)
+                    *reinterpret_cast<float4 *>(dst + ((int64_t)co * Cin + ci) * 16 + 8 * (q & 1) + 4 * h) =
+                        make_float4(acc[cp][t][4 * q] * unscale, acc[cp][t][4 * q + 1] * unscale,
+                                    acc[cp][t][4 * q + 2] * unscale, acc[cp][t][4 * q + 3] * unscale);
+            }
+        }
+}
+
+int f2f16h2_bwd_filter_partials(const float *gout, const float *tex, const float *sh, const int *cum, const int *order,
+                                 float *partial, int splits, int64_t T, int64_t Nf, int Cin, int Cout, hipStream_t st)
+{
+    // channel pairs per wavefront: the four wavefronts of a workgroup share up to 32 pairs
+    const int pairs = (Cin + 1) / 2;
+    const int ncp = pairs >= 32 ? 8 : pairs > 8 ? 4 : pairs > 4 ? 2 : 1;
+    const int64_t gy = ceil_div(Cin, 8 * ncp), gz = ceil_div(Cout, 64);
+    PM_REQUIRE(gy <= 65535 && gz <= 65535, "f2f_bwd_filter: grid too large");
+    const int64_t ntiles = ceil_div(Nf, 32);
+    const bool tvec = !(Cin & 3) && !(reinterpret_cast<uintptr_t>(tex) & 15u);
+    const dim3 grid((unsigned)splits, (unsigned)gy, (unsigned)gz);
+#define PM_FILT(V, N) f2f16h2_bwd_filt_k<V, N><<<grid, dim3(256), 0, st>>>(gout, tex, sh, cum, order, partial, Nf, (int)T, Cin, Cout, ntiles)
+    if (tvec) {
+        if (ncp == 8) PM_FILT(true, 8); else if (ncp == 4) PM_FILT(true, 4); else if (ncp == 2) PM_FILT(true, 2); else PM_FILT(true, 1);
+    } else {
+        if (ncp == 8) PM_FILT(false, 8); else if (ncp == 4) PM_FILT(false, 4); else if (ncp == 2) PM_FILT(false, 2); else PM_FILT(false, 1);
+    }
+#undef PM_FILT
+    PM_LAUNCHED("f2f_bwd_filter");
     return 0;
 }
 

@@ -40,13 +40,17 @@ int f2f16x3_bwd_texture(const float *gout, const float *W, const float *sh, cons
                         float *gtex, void *workspace, size_t workspace_bytes, int64_t T, int64_t Nf, int Cin,
                         int Cout, hipStream_t st);
 
-// the same on the fp16 matrix cores (block-floating scales, see mesh_f2f16h2.hip)
+// the same on the fp16 matrix cores (block-floating scales, see mesh_f2f16h2.hip).  *overflow (cleared by the
+// caller) is set when the data outgrew the scales: the partials are then void and must be computed again by
+// f2f16x3_bwd_filter_partials, whose `only_if` argument makes that launch a no-op otherwise.
 int f2f16h2_bwd_filter_partials(const float *gout, const float *tex, const float *sh, const int *cum, const int *order,
-                                 float *partial, int splits, int64_t T, int64_t Nf, int Cin, int Cout, hipStream_t st);
+                                 float *partial, int *overflow, int splits, int64_t T, int64_t Nf, int Cin, int Cout, hipStream_t st);
 
 // `splits` workgroups each write one partial (Cout x Cin*16) block; every split gets a strided share of the 32-facet tiles
+// only_if (may be null): device flag; the kernel returns at once when it reads 0
 int f2f16x3_bwd_filter_partials(const float *gout, const float *tex, const float *sh, const int *cum, const int *order,
-                                 float *partial, int splits, int64_t T, int64_t Nf, int Cin, int Cout, hipStream_t st);
+                                 float *partial, int splits, int64_t T, int64_t Nf, int Cin, int Cout, hipStream_t st,
+                                 const int *only_if = nullptr);
 
 
 int f2f16_bwd_texture(const float *gout, const float *W, const float *sh, const int *cum, float *gtex, int64_t T,

@@ -396,8 +396,9 @@ extern "C" int pmesh_f2f_fwd(const float *texture, const float *filter, const fl
 extern "C" size_t pmesh_f2f_bwd_workspace_bytes(int Cin, int Cout, int F)
 {
     // the two halves run one after the other on a stream and share the workspace
+    // partial gradients, then 256 bytes for the overflow flag of the fp16 filter gradient
     const size_t slices = f2f_narrow_usable(Cin, F) ? kNarrowMaxBlocks : kFiltMaxSplits;
-    const size_t filt = slices * Cout * Cin * F * sizeof(float);
+    const size_t filt = slices * Cout * Cin * F * sizeof(float) + 256;
     const size_t tex = F == 16 ? f2f16x3_bwd_texture_workspace_bytes(Cin, Cout) : 0;
     return filt > tex ? filt : tex;
 }
@@ -464,14 +465,28 @@ extern "C" int pmesh_f2f_bwd_filter(const float *grad_output, const float *textu
     PM_REQUIRE(workspace_bytes >= (size_t)S * nW * sizeof(float), "f2f_bwd_filter: workspace too small (%zu bytes)",
                workspace_bytes);
     const bool x3 = !force_fp32_mfma() && f2f16x3_usable(bary_coeff, bary_coeff, F);
+    PM_REQUIRE(!x3 || workspace_bytes >= (size_t)S * nW * sizeof(float) + 256,
+               "f2f_bwd_filter: workspace too small (%zu bytes)", workspace_bytes);
     if (!force_generic() && (x3 || f2f16_usable(texture, texture, bary_coeff, Cin, F))) {
+        if (x3 && !force_bf16x3()) {
+            // fp16 kernel first; if its scales did not hold, the guarded bf16 launch after it does the work again
+            int *overflow = reinterpret_cast<int *>((float *)workspace + (size_t)S * nW);
+            f2f_fill_zero_k<<<dim3(1), dim3(kBlock), 0, st>>>(reinterpret_cast<float *>(overflow), 1);
+            PM_LAUNCHED("f2f_bwd_filter(flag)");
+            if (int rc = f2f16h2_bwd_filter_partials(grad_output, texture, bary_coeff, cum_texture, facet_order,
+                                                     (float *)workspace, overflow, S, T, Nf, Cin, Cout, st))
+                return rc;
+            if (int rc = f2f16x3_bwd_filter_partials(grad_output, texture, bary_coeff, cum_texture, facet_order,
+                                                     (float *)workspace, S, T, Nf, Cin, Cout, st, overflow))
+                return rc;
+            f2f_reduce_k<<<dim3((unsigned)ceil_div(nW, 64)), dim3(kBlock), 0, st>>>((const float *)workspace, grad_filter, S, nW);
+            PM_LAUNCHED("f2f_bwd_filter(reduce)");
+            return 0;
+        }
         int rc = !x3 ? f2f16_bwd_filter_partials(grad_output, texture, bary_coeff, cum_texture, (float *)workspace, S, T,
                                                  Nf, Cin, Cout, st)
-                     : force_bf16x3()
-                         ? f2f16x3_bwd_filter_partials(grad_output, texture, bary_coeff, cum_texture, facet_order,
-                                                       (float *)workspace, S, T, Nf, Cin, Cout, st)
-                         : f2f16h2_bwd_filter_partials(grad_output, texture, bary_coeff, cum_texture, facet_order,
-                                                       (float *)workspace, S, T, Nf, Cin, Cout, st);
+                     : f2f16x3_bwd_filter_partials(grad_output, texture, bary_coeff, cum_texture, facet_order,
+                                                   (float *)workspace, S, T, Nf, Cin, Cout, st);
         if (rc) return rc;
         f2f_reduce_k<<<dim3((unsigned)ceil_div(nW, 64)), dim3(kBlock), 0, st>>>((const float *)workspace, grad_filter, S, nW);
         PM_LAUNCHED("f2f_bwd_filter(reduce)");

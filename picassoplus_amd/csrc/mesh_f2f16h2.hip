@@ -48,24 +48,28 @@ __device__ __forceinline__ float absmax4(const float4 &v, float m)
     return fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fmaxf(fabsf(v.z), fabsf(v.w)), m));
 }
 
-// Eight fp32 values -> two packed fp16x8 pieces, both rounded to nearest (one v_cvt_pk_f16_f32 per pair); the
-// remainder x - x1 is exact in fp32.  The empty asm pins each value as an fp32 register first: otherwise the
-// compiler may fold the FMA that produced it into ONE of the two conversions of x1 it emits (a mixed-precision
-// FMA rounds the exact product once), and in a near-tie the piece that is multiplied and the piece the
-// remainder was taken from differ by one fp16 ulp.
+// Eight fp32 values -> two packed fp16x8 pieces, both rounded to nearest; the remainder x - x1 is exact in
+// fp32.  Written out as instructions: left to the compiler, the FMA that produced x may be folded into ONE of
+// the two conversions of x1 it emits (a mixed-precision FMA rounds the exact product once), and in a near-tie
+// the piece that is multiplied and the piece the remainder was taken from then differ by one fp16 ulp.
 __device__ __forceinline__ void split8h(const float (&x)[8], u32x4 &p1, u32x4 &p2)
 {
+    const float neg1 = -1.0f;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-        float a = x[2 * j], b = x[2 * j + 1];
-        asm volatile("" : "+v"(a), "+v"(b));
-        f16x2 hi, lo;
-        hi[0] = (_Float16)a;
-        hi[1] = (_Float16)b;
-        lo[0] = (_Float16)__builtin_fmaf((float)hi[0], -1.0f, a);
-        lo[1] = (_Float16)__builtin_fmaf((float)hi[1], -1.0f, b);
-        p1[j] = __builtin_bit_cast(unsigned, hi);
-        p2[j] = __builtin_bit_cast(unsigned, lo);
+        // hi = {f16(a), f16(b)};  ra = a - hi.lo, rb = b - hi.hi (mixed-precision FMAs reading one half of hi
+        // each, exact);  lo = {f16(ra), f16(rb)}: four instructions per pair
+        unsigned hi, lo;
+        float ra, rb;
+        asm("v_cvt_pk_f16_f32 %0, %4, %5\n\t"
+            "s_nop 0\n\t"
+            "v_fma_mix_f32 %1, %0, %6, %4 op_sel:[0,0,0] op_sel_hi:[1,0,0]\n\t"
+            "v_fma_mix_f32 %2, %0, %6, %5 op_sel:[1,0,0] op_sel_hi:[1,0,0]\n\t"
+            "v_cvt_pk_f16_f32 %3, %1, %2"
+            : "=&v"(hi), "=&v"(ra), "=&v"(rb), "=&v"(lo)
+            : "v"(x[2 * j]), "v"(x[2 * j + 1]), "v"(neg1));
+        p1[j] = hi;
+        p2[j] = lo;
     }
 }
 
@@ -151,15 +155,18 @@ __device__ __forceinline__ void hw_chunk_fetch(const u32x4 *__restrict__ Wp, int
 }
 
 // One pass over all input channels for up to KW texture points per facet.  shs = alpha_f / K_f, the factor on
-// the SH values of my facet.
+// the SH values of my facet; slim / tlim = largest |SH value| of my facet / |texture value| of the rows I fetch
+// that the scale allows for.
 template <int KW, bool TVEC>
 __device__ __forceinline__ void h2_sweep(const float *__restrict__ tex, const u32x4 *__restrict__ Wp,
                                          const float *__restrict__ sh, u32x4 *Ws, float *slab, f32x16 (&acc)[2],
-                                         int kbase, int Ks, float shs, const int *s_k0, const int *s_K, int sweep,
-                                         int Cin, int NT, int nt0, int nblk, int w, int lane, int h)
+                                         int kbase, int Ks, float shs, float slim, float tlim, bool &viol,
+                                         const int *s_k0, const int *s_K, int sweep, int Cin, int NT, int nt0, int nblk,
+                                         int w, int lane, int h)
 {
     const int l32 = lane & 31;
     float shr[KW][8];
+    float smx = 0.f;
 #pragma unroll
     for (int kk = 0; kk < KW; ++kk) {
         float4 u = make_float4(0.f, 0.f, 0.f, 0.f), v = u;
@@ -168,6 +175,7 @@ __device__ __forceinline__ void h2_sweep(const float *__restrict__ tex, const u3
             u = hld4(p);
             v = hld4(p + 4);
         }
+        smx = absmax4(u, absmax4(v, smx));
         shr[kk][0] = u.x * shs; shr[kk][1] = u.y * shs; shr[kk][2] = u.z * shs; shr[kk][3] = u.w * shs;
         shr[kk][4] = v.x * shs; shr[kk][5] = v.y * shs; shr[kk][6] = v.z * shs; shr[kk][7] = v.w * shs;
     }
@@ -187,12 +195,17 @@ __device__ __forceinline__ void h2_sweep(const float *__restrict__ tex, const u3
         for (int i = 0; i < KW; ++i)
             pf[i] = ldok[i] ? hld4_row<TVEC>(tex + (ldoff[i] + 8 * g), Cin - (8 * g + cg4)) : make_float4(0.f, 0.f, 0.f, 0.f);
     };
+    // values past the limits the facet's scale was chosen for are recorded, not acted on here
+    viol |= smx > slim;
     auto publish_group = [&](float *dst) {
+        float m = 0.f;
 #pragma unroll
         for (int i = 0; i < KW; ++i) {
             float *q = dst + (i * 8 + cg4) * 32 + (lane >> 1);
             q[0] = pf[i].x; q[32] = pf[i].y; q[64] = pf[i].z; q[96] = pf[i].w;
+            m = absmax4(pf[i], m);
         }
+        viol |= m > tlim;
     };
     u32x4 wn[kHWn];
     fetch_group(0);
@@ -295,7 +308,7 @@ __global__ __launch_bounds__(kHThreads, 2) void f2f16h2_fwd_k(const float *__res
     __shared__ u32x4 Ws[3 * kHChunk];
     __shared__ __attribute__((aligned(16))) float s_slab[kHW * 2 * kHSlab];      // per wavefront: two buffers
     __shared__ int s_f[256], s_k0[256], s_K[256], s_kmax;
-    __shared__ float s_tm[256], s_inv[256];
+    __shared__ float s_tm[256], s_inv[256], s_tl[256];
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
     const int l32 = lane & 31, h = lane >> 5;
     const int64_t s0 = (int64_t)blockIdx.x * 256;
@@ -324,77 +337,85 @@ __global__ __launch_bounds__(kHThreads, 2) void f2f16h2_fwd_k(const float *__res
         if (lane == 0) atomicMax(&s_kmax, km);
     }
 
-    // pre-scan: largest |texture value| of each facet's rows (two lanes per row, as the slab fetches) and
-    // largest |SH value| of my facet's rows (my half's eight d's; the halves meet through s_tm)
-    {
-        const int slot = w * 32 + (lane >> 1), cg4 = 4 * (lane & 1);
-        const int rk0 = s_k0[slot], rK = s_K[slot];
-        // all loads of a batch are issued before the first comparison (four rows x 32 channels per lane pair)
-        const int rKmax = hwave_max(rK), Kmax = hwave_max(K);
-        float sm = 0.f;
-        for (int kb = 0; kb < Kmax; kb += 4) {
-            float4 u[4][2];
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const float *p = sh + (int64_t)(k0 + kb + i) * 16 + 8 * h;
-                const bool ok = kb + i < K;
-                u[i][0] = ok ? hld4(p) : make_float4(0.f, 0.f, 0.f, 0.f);
-                u[i][1] = ok ? hld4(p + 4) : make_float4(0.f, 0.f, 0.f, 0.f);
-            }
-#pragma unroll
-            for (int i = 0; i < 4; ++i) sm = absmax4(u[i][0], absmax4(u[i][1], sm));
-        }
-        float tm = 0.f;
-        for (int kb = 0; kb < rKmax; kb += 4)
-            for (int cb = 0; cb < Cin; cb += 32) {
-                float4 v[4][4];
-#pragma unroll
-                for (int i = 0; i < 4; ++i)
-#pragma unroll
-                    for (int g = 0; g < 4; ++g) {
-                        const int c = cb + 8 * g + cg4;
-                        v[i][g] = (kb + i < rK && c < Cin) ? hld4_row<TVEC>(tex + (int64_t)(rk0 + kb + i) * Cin + c, Cin - c)
-                                                           : make_float4(0.f, 0.f, 0.f, 0.f);
-                    }
-#pragma unroll
-                for (int i = 0; i < 4; ++i)
-#pragma unroll
-                    for (int g = 0; g < 4; ++g) tm = absmax4(v[i][g], tm);
-            }
-        tm = fmaxf(tm, __shfl_xor(tm, 1, 64));
-        sm = fmaxf(sm, __shfl_xor(sm, 32, 64));
-        if (!(lane & 1)) s_tm[slot] = tm;
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-        float inv;
-        const float alpha = pow2_scale(s_tm[w * 32 + l32] * sm, &inv);
-        if (h == 0) s_inv[w * 32 + l32] = inv;
-        s_tm[w * 32 + l32] = alpha;          // same wavefront: every read above is done (in-order LDS)
-    }
-    __syncthreads();
-    const float alpha = s_tm[w * 32 + l32];
-    const float shs = K > 0 ? alpha / (float)K : 0.f;
-    const int nsweeps = (s_kmax + kHKB - 1) / kHKB;
-
+    // Scale of each facet's G.  First try: a bound from the first eight channels and the first four points only
+    // (one batch of loads that the sweep reads again from cache), with 2^7 of head room; the sweeps check every
+    // value they fetch against it.  If any facet of the workgroup exceeds its bound, everything is done again
+    // with the exact maxima from a scan of all rows (which costs a second pass over the texture rows).
     f32x16 acc[2];
+    for (int attempt = 0;; ++attempt) {
+        const bool full = attempt > 0;
+        float slim;
+        {
+            const int slot = w * 32 + (lane >> 1), cg4 = 4 * (lane & 1);
+            const int rk0 = s_k0[slot], rK = s_K[slot];
+            // all loads of a batch are issued before the first comparison
+            const int rKmax = full ? hwave_max(rK) : 1, Kmax = full ? hwave_max(K) : 1, cend = full ? Cin : 1;
+            float sm = 0.f;
+            for (int kb = 0; kb < Kmax; kb += 4) {
+                float4 u[4][2];
 #pragma unroll
-    for (int t = 0; t < 2; ++t)
+                for (int i = 0; i < 4; ++i) {
+                    const float *p = sh + (int64_t)(k0 + kb + i) * 16 + 8 * h;
+                    const bool ok = kb + i < K;
+                    u[i][0] = ok ? hld4(p) : make_float4(0.f, 0.f, 0.f, 0.f);
+                    u[i][1] = ok ? hld4(p + 4) : make_float4(0.f, 0.f, 0.f, 0.f);
+                }
 #pragma unroll
-        for (int i = 0; i < 16; ++i) acc[t][i] = 0.f;
-
-    for (int sw = 0; sw < nsweeps; ++sw) {
-        const int kbase = k0 + sw * kHKB;
-        const int rem = K - sw * kHKB;
-        const int Ks = rem < 0 ? 0 : (rem > kHKB ? kHKB : rem);
-        // every variant runs the same barriers, so wavefronts of a workgroup may pick different ones
-        const int kw = hwave_max(Ks);
-#define PM_H2(N) h2_sweep<N, TVEC>(tex, Wp, sh, Ws, s_slab + w * 2 * kHSlab, acc, kbase, Ks, shs, s_k0, s_K, sw, Cin, NT, nt0, nblk, w, lane, h)
-        if (kw <= 1) PM_H2(1);
-        else if (kw == 2) PM_H2(2);
-        else if (kw == 3) PM_H2(3);
-        else PM_H2(4);
+                for (int i = 0; i < 4; ++i) sm = absmax4(u[i][0], absmax4(u[i][1], sm));
+            }
+            float tm = 0.f;
+            for (int kb = 0; kb < rKmax; kb += 4)
+                for (int cb = 0; cb < cend; cb += 32) {
+                    float4 v[4][4];
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+#pragma unroll
+                        for (int g = 0; g < 4; ++g) {
+                            const int c = cb + 8 * g + cg4;
+                            v[i][g] = (kb + i < rK && c < Cin && (full || g == 0))
+                                          ? hld4_row<TVEC>(tex + (int64_t)(rk0 + kb + i) * Cin + c, Cin - c)
+                                          : make_float4(0.f, 0.f, 0.f, 0.f);
+                        }
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+#pragma unroll
+                        for (int g = 0; g < 4; ++g) tm = absmax4(v[i][g], tm);
+                }
+            tm = fmaxf(tm, __shfl_xor(tm, 1, 64));
+            sm = fmaxf(sm, __shfl_xor(sm, 32, 64));
+            if (!full) { tm *= 8.0f; sm *= 16.0f; }          // head room of the first try (2^7 in all)
+            slim = sm;
+            if (!(lane & 1)) s_tl[slot] = tm;
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            float inv;
+            const float al = pow2_scale(s_tl[w * 32 + l32] * sm, &inv);
+            if (h == 0) { s_inv[w * 32 + l32] = inv; s_tm[w * 32 + l32] = al; }
+        }
+        __syncthreads();
+        const float alpha = s_tm[w * 32 + l32], tlim = s_tl[w * 32 + (lane >> 1)];
+        const int nsweeps = (s_kmax + kHKB - 1) / kHKB;
+        const float shs = K > 0 ? alpha / (float)K : 0.f;
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) acc[t][i] = 0.f;
+        bool viol = false;
+        for (int sw = 0; sw < nsweeps; ++sw) {
+            const int kbase = k0 + sw * kHKB;
+            const int rem = K - sw * kHKB;
+            const int Ks = rem < 0 ? 0 : (rem > kHKB ? kHKB : rem);
+            // every variant runs the same barriers, so wavefronts of a workgroup may pick different ones
+            const int kw = hwave_max(Ks);
+#define PM_H2(N) h2_sweep<N, TVEC>(tex, Wp, sh, Ws, s_slab + w * 2 * kHSlab, acc, kbase, Ks, shs, slim, tlim, viol, s_k0, s_K, sw, Cin, NT, nt0, nblk, w, lane, h)
+            if (kw <= 1) PM_H2(1);
+            else if (kw == 2) PM_H2(2);
+            else if (kw == 3) PM_H2(3);
+            else PM_H2(4);
 #undef PM_H2
+        }
+        if (full || !__syncthreads_or(viol ? 1 : 0)) break;
     }
 
     const float ibeta = hdr[1];
@@ -769,8 +790,9 @@ int f2f16h2_bwd_texture(const float *gout, const float *W, const float *sh, cons
 //             fixed by its first pass (with 2^9 of head room below the overflow bound from the largest
 //             texture value it just fetched and the largest SH value of its facets), so alpha = S / gamma
 //             afterwards; 1 / S is taken out when the partial result is written.  Small operands cost
-//             nothing (their error is absolute, far below the accumulated sum); a pass whose alpha would
-//             overflow takes the largest safe alpha and is accumulated 2^k times.
+//             nothing (their error is absolute, far below the accumulated sum).  Operands that outgrow the
+//             head room along the facet list raise *overflow: the result of this kernel is then void and
+//             the caller's guarded launch of the three-piece bf16 kernel, which needs no scales, replaces it.
 //   workgroup  4 wavefronts (one per SIMD), 64 input x 64 output channels, a strided subset of the tiles
 //   wavefront  16 input channels = 8 channel pairs x 2 output tiles of gW^T[(ci,d)][co]; narrower filters give
 //              every wavefront 1, 2 or 4 pairs instead (NCP)
@@ -972,7 +994,7 @@ __device__ __forceinline__ void h2_filt_tile(const float *__restrict__ gout, con
                                              const int *__restrict__ order, u32x4 (*go_s)[2 * 2 * 2 * 64], float4 *slab,
                                              float (*sh_s)[kHKB * 32 * 16], int (*s_f)[32], int (*s_k0)[32],
                                              int (*s_K)[32], float *s_gamma, unsigned *s_gm, f32x16 (&acc)[NCP][2],
-                                             HScales &sc, const u32x4 &ea, const u32x4 &eb, int it, int64_t tile,
+                                             HScales &sc, int *overflow, const u32x4 &ea, const u32x4 &eb, int it, int64_t tile,
                                              int64_t stride, int64_t ntiles, int64_t Nf, int T, int Cin, int Cout, int c0,
                                              int n0, int lane, int w)
 {
@@ -1043,23 +1065,23 @@ __device__ __forceinline__ void h2_filt_tile(const float *__restrict__ gout, con
         if (bound > 0.f) {
             float inv;
             const float need = pow2_scale(bound, &inv);          // need * bound < 2^14
-            // The accumulators keep the scale S of the first pass, so alpha follows gamma: alpha = S / gamma.
-            // The first pass leaves 2^9 of head room under `need`; a pass whose alpha would still overflow
-            // takes the largest safe one and is accumulated S / (alpha gamma) times instead (a power of two;
-            // it takes data growing by orders of magnitude along the facet list to get there).
+            // The accumulators keep the scale S of the wavefront's first pass (2^9 below its overflow bound), so
+            // alpha follows gamma: alpha = S / gamma.  Smaller operands later on cost nothing (their error is
+            // absolute, far below the sum).  Operands that have grown past the head room cannot be taken in
+            // at this scale: the wavefront raises the overflow flag -- the caller's next launch, the
+            // three-piece bf16 kernel, then computes the whole gradient again -- and carries on with a
+            // scale that is safe to execute.
             if (sc.S == 0.f) sc.S = need * (1.0f / 512.0f) * gamma;
             float al = sc.S / gamma;
-            int reps = 1;
             if (al > need) {
-                const float r = al / need;
-                reps = r < 1048576.0f ? (int)r : 1048576;
+                if (lane == 0) *overflow = 1;
                 al = need;
             }
 #pragma unroll
             for (int kk = 0; kk < KW; ++kk)
 #pragma unroll
                 for (int q = 0; q < 8; ++q) shr[kk][q] *= al;
-            for (int rep = 0; rep < reps; ++rep) h2_filt_pass<KW, NCP>(shr, slab, go_s[buf], acc, ea, eb, lane);
+            h2_filt_pass<KW, NCP>(shr, slab, go_s[buf], acc, ea, eb, lane);
         }
     }
 
@@ -1093,8 +1115,8 @@ __global__ __launch_bounds__(256, 1) void f2f16h2_bwd_filt_k(const float *__rest
                                                               const float *__restrict__ sh,
                                                               const int *__restrict__ cum,
                                                               const int *__restrict__ order,
-                                                              float *__restrict__ partial, int64_t Nf, int T, int Cin,
-                                                              int Cout, int64_t ntiles)
+                                                              float *__restrict__ partial, int *__restrict__ overflow,
+                                                              int64_t Nf, int T, int Cin, int Cout, int64_t ntiles)
 {
     __shared__ u32x4 go_s[2][2 * 2 * 2 * 64];
     __shared__ float4 slab_s[4 * kHKB * 4 * 32];
@@ -1163,13 +1185,15 @@ __global__ __launch_bounds__(256, 1) void f2f16h2_bwd_filt_k(const float *__rest
 #define PM_PHASE(N)                                                                                                  \
     for (; tile < ntiles && (N == kHKB || htile_kmax(s_K[it % 3], lane) <= N); ++it, tile += stride)                 \
         h2_filt_tile<N, TVEC, NCP>(gout, tex, sh, cum, order, go_s, slab_s + w * (kHKB * 4 * 32), sh_s, s_f, s_k0, s_K, \
-                                   s_gamma, s_gm, acc, sc, ea, eb, it, tile, stride, ntiles, Nf, T, Cin, Cout, c0, n0, lane, w)
+                                   s_gamma, s_gm, acc, sc, overflow, ea, eb, it, tile, stride, ntiles, Nf, T, Cin, Cout, c0, n0, lane, w)
     PM_PHASE(1);
     PM_PHASE(2);
     PM_PHASE(3);
     PM_PHASE(4);
 #undef PM_PHASE
 
+    // accumulator (cp, t): lane (co = 32t + l32, half h), register i <-> row m = 8(i/4) + 4h + i%4
+    // = (channel c0 + 2 NCP w + 2cp + m/16, d = m%16); four consecutive d's per group of four registers
     // accumulator (cp, t): lane (co = 32t + l32, half h), register i <-> row m = 8(i/4) + 4h + i%4
     // = (channel c0 + 2 NCP w + 2cp + m/16, d = m%16); four consecutive d's per group of four registers
     const float unscale = sc.S != 0.f ? 1.0f / sc.S : 0.f;
@@ -1191,7 +1215,7 @@ __global__ __launch_bounds__(256, 1) void f2f16h2_bwd_filt_k(const float *__rest
 }
 
 int f2f16h2_bwd_filter_partials(const float *gout, const float *tex, const float *sh, const int *cum, const int *order,
-                                 float *partial, int splits, int64_t T, int64_t Nf, int Cin, int Cout, hipStream_t st)
+                                 float *partial, int *overflow, int splits, int64_t T, int64_t Nf, int Cin, int Cout, hipStream_t st)
 {
     // channel pairs per wavefront: the four wavefronts of a workgroup share up to 32 pairs
     const int pairs = (Cin + 1) / 2;
@@ -1201,7 +1225,7 @@ int f2f16h2_bwd_filter_partials(const float *gout, const float *tex, const float
     const int64_t ntiles = ceil_div(Nf, 32);
     const bool tvec = !(Cin & 3) && !(reinterpret_cast<uintptr_t>(tex) & 15u);
     const dim3 grid((unsigned)splits, (unsigned)gy, (unsigned)gz);
-#define PM_FILT(V, N) f2f16h2_bwd_filt_k<V, N><<<grid, dim3(256), 0, st>>>(gout, tex, sh, cum, order, partial, Nf, (int)T, Cin, Cout, ntiles)
+#define PM_FILT(V, N) f2f16h2_bwd_filt_k<V, N><<<grid, dim3(256), 0, st>>>(gout, tex, sh, cum, order, partial, overflow, Nf, (int)T, Cin, Cout, ntiles)
     if (tvec) {
         if (ncp == 8) PM_FILT(true, 8); else if (ncp == 4) PM_FILT(true, 4); else if (ncp == 2) PM_FILT(true, 2); else PM_FILT(true, 1);
     } else {

@@ -908,8 +908,9 @@ __global__ __launch_bounds__(256, 1) void f2f16x3_bwd_filt_k(const float *__rest
                                                               const int *__restrict__ cum,
                                                               const int *__restrict__ order,
                                                               float *__restrict__ partial, int64_t Nf, int T, int Cin,
-                                                              int Cout, int64_t ntiles)
+                                                              int Cout, int64_t ntiles, const int *__restrict__ only_if)
 {
+    if (only_if && *only_if == 0) return;          // guarded launch: nothing asked for
     __shared__ u32x4 go_s[2][2 * 2 * 3 * 64];
     __shared__ float4 slab_s[4 * kXKB * 4 * 32];
     __shared__ __attribute__((aligned(16))) float sh_s[2][kXKB * 32 * 16];
@@ -990,7 +991,8 @@ __global__ __launch_bounds__(256, 1) void f2f16x3_bwd_filt_k(const float *__rest
 }
 
 int f2f16x3_bwd_filter_partials(const float *gout, const float *tex, const float *sh, const int *cum, const int *order,
-                                 float *partial, int splits, int64_t T, int64_t Nf, int Cin, int Cout, hipStream_t st)
+                                 float *partial, int splits, int64_t T, int64_t Nf, int Cin, int Cout, hipStream_t st,
+                                 const int *only_if)
 {
     // channel pairs per wavefront: the four wavefronts of a workgroup share up to 32 pairs
     const int pairs = (Cin + 1) / 2;
@@ -1000,7 +1002,7 @@ int f2f16x3_bwd_filter_partials(const float *gout, const float *tex, const float
     const int64_t ntiles = ceil_div(Nf, 32);
     const bool tvec = !(Cin & 3) && !(reinterpret_cast<uintptr_t>(tex) & 15u);
     const dim3 grid((unsigned)splits, (unsigned)gy, (unsigned)gz);
-#define PM_FILT(V, N) f2f16x3_bwd_filt_k<V, N><<<grid, dim3(256), 0, st>>>(gout, tex, sh, cum, order, partial, Nf, (int)T, Cin, Cout, ntiles)
+#define PM_FILT(V, N) f2f16x3_bwd_filt_k<V, N><<<grid, dim3(256), 0, st>>>(gout, tex, sh, cum, order, partial, Nf, (int)T, Cin, Cout, ntiles, only_if)
     if (tvec) {
         if (ncp == 8) PM_FILT(true, 8); else if (ncp == 4) PM_FILT(true, 4); else if (ncp == 2) PM_FILT(true, 2); else PM_FILT(true, 1);
     } else {

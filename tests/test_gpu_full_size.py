@@ -84,7 +84,9 @@ def test_f2f_full_size_adjoints_and_sample_parity(cuda, scene):
     assert_close(out.detach()[pick_t], ref_out, "f2f out (sampled facets)")
     assert_close(gtex[rows_t], ref_gtex, "f2f grad_texture (sampled facets)")
 
-    # the facet order is an optimisation only: per-facet results do not change by a bit
+    # the facet order is an optimisation only.  A facet's power-of-two operand scale can depend on its workgroup
+    # (all of it falls back to exact row maxima when one facet exceeds its first bound), which moves results by
+    # an ulp at most; with no such fallback, as on this data, nothing changes by a bit
     T, Cin = d["tex"].shape
     ws_n = _lib.query("pmesh_f2f_fwd_workspace_bytes", Cin, d["C"], 16)
     ws = torch.empty(ws_n, dtype=torch.uint8, device=cuda)
@@ -93,7 +95,7 @@ def test_f2f_full_size_adjoints_and_sample_parity(cuda, scene):
               None, out2.data_ptr(), ws.data_ptr(), ws_n, T, d["nf"], Cin, d["C"], 16,
               torch.cuda.current_stream().cuda_stream)
     torch.cuda.synchronize()
-    assert torch.equal(out2, out.detach())
+    assert float((out2 - out.detach()).abs().max()) <= 2e-7 * float(out.detach().abs().max())
 
 
 def test_f2v_full_size_adjoints(cuda, scene):

@@ -191,6 +191,47 @@ def test_f2f_parity(cuda, monkeypatch, nf, Cin, Cout, F, kmax, path):
     assert_close(ft.grad, gfilt_ref, "f2f grad_filter")
 
 
+@pytest.mark.parametrize("case", ["late_channels", "late_points", "growing_facets"])
+def test_f2f_wide_dynamic_range(cuda, case):
+    """The fp16 kernels choose power-of-two operand scales from what they have seen so far and must recover when
+    later data is larger by orders of magnitude: channels past the first eight (forward: first bound exceeded,
+    workgroup redone with exact maxima), later texture points / their SH rows, and facets whose magnitudes grow
+    along the sorted facet list (filter gradient: operand split again with a new scale; passes accumulated
+    several times when the accumulator scale no longer fits)."""
+    say("case f2f dynamic range", case)
+    rng = np.random.default_rng(99)
+    nf, Cin, Cout = 700, 32, 64
+    counts, bary, owner = texture_case(rng, nf, 9)
+    cum = np.cumsum(counts).astype(np.int32)
+    T = int(counts.sum())
+    tex = rng.uniform(-1, 1, (T, Cin))
+    sh = rng.normal(0, 0.5, (T, 16))
+    filt = rng.normal(0, 0.3, (Cout, Cin, 16))
+    gout = rng.normal(0, 1, (nf, Cout))
+    first = np.concatenate([[0], cum[:-1]])
+    local = np.arange(T) - first[owner]                      # index of a point inside its facet
+    if case == "late_channels":
+        tex[:, 8:] *= 3000.0
+        tex[owner % 3 == 0, 20] *= 50.0
+    elif case == "late_points":
+        tex[local >= 4] *= 500.0
+        sh[local >= 5] *= 200.0
+    else:
+        mag = 10.0 ** (counts[owner] * 1.2 - 3)              # 1e-3 .. 1e8 with the number of points
+        tex *= mag[:, None]
+        gout *= (10.0 ** (counts * 0.9 - 2))[:, None]
+    out_ref = loops.f2f_fwd(tex, filt, sh, cum)
+    gin_ref, gfilt_ref = loops.f2f_bwd(gout, tex, filt, sh, cum)
+    tt = dev(tex, cuda, torch.float32).requires_grad_(True)
+    ft = dev(filt, cuda, torch.float32).requires_grad_(True)
+    out = conv3d.facet2facet(tt, ft, dev(sh, cuda, torch.float32), dev(cum, cuda))
+    out.backward(dev(gout, cuda, torch.float32))
+    torch.cuda.synchronize()
+    assert_close(out, out_ref, "f2f out")
+    assert_close(tt.grad, gin_ref, "f2f grad_texture")
+    assert_close(ft.grad, gfilt_ref, "f2f grad_filter")
+
+
 def test_f2f_shape_sweep(cuda):
     """Seeded sweep over channel counts, facet counts and point counts around the tile sizes of the
     16-coefficient kernels (32-facet wavefront tiles, 4/8/16-channel groups, 64-channel blocks)."""

@@ -39,7 +39,7 @@ def test_library_exports_every_declared_symbol():
 def test_size_queries_are_host_only():
     assert _lib.query("pmesh_v2f_bwd_workspace_bytes", 64, 1) == 1024 * 3 * 64 * 4
     assert _lib.query("pmesh_f2v_bwd_workspace_bytes", 64, 1, 16) == 1024 * 16 * 64 * 4
-    assert _lib.query("pmesh_f2f_bwd_workspace_bytes", 64, 64, 16) == 256 * 64 * 64 * 16 * 4
+    assert _lib.query("pmesh_f2f_bwd_workspace_bytes", 64, 64, 16) == 256 * 64 * 64 * 16 * 4 + 256    # partials + flag
     assert _lib.query("pmesh_f2f_fwd_workspace_bytes", 64, 64, 16) == 64 * 2 * 3 * 64 * 16
     assert _lib.query("pmesh_f2f_fwd_workspace_bytes", 3, 64, 16) == 4 * 2 * 3 * 64 * 16      # channels padded to 4
     assert _lib.query("pmesh_f2f_fwd_workspace_bytes", 3, 64, 9) == 0

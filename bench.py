@@ -26,6 +26,10 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
 MFMA_F32_PEAK_TFLOPS = 157.3
+MFMA_F16_PEAK_TFLOPS = 2500.0
+# The facet2facet kernels get fp32 accuracy from three fp16 piece products per product (two-piece split of both
+# operands), so the matrix-core ceiling for their algorithmic (fp32-equivalent) flops is a third of the fp16 peak.
+F2F_PIECE_PRODUCTS = 3
 
 
 def parse():
@@ -85,8 +89,8 @@ def conv_bytes_flops(d, ops):
 # HBM bytes per launch of the op's main kernel on the default scene workload (scale 1.0), measured with
 # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE and scaled by what the same counters read for a 1 GiB copy
 # (--copy-calibration); reported as roofline.traffic when that workload runs.
-SCENE_TRAFFIC_BYTES = {"f2f_fwd": 4.650e9, "f2f_bwd_texture": 4.011e9, "f2f_bwd_filter": 3.365e9,
-                       "f2v_fwd": 2.066e9, "f2v_bwd": 2.020e9}
+SCENE_TRAFFIC_BYTES = {"f2f_fwd": 5.161e9, "f2f_bwd_texture": 3.981e9, "f2f_bwd_filter": 3.366e9,
+                       "f2v_fwd": 1.287e9, "f2v_bwd": 2.185e9}
 
 
 class EventTimer:
@@ -181,7 +185,10 @@ def run_conv_layer(args, torch, kind):
     dom = max(ops, key=lambda k: per_op.get(k, 0.0))
     dom_ms = per_op[dom]
     if dom.startswith("f2f") and Cin >= 16:
-        roof = dict(bound="mfma", achieved=bf[dom][1] / (dom_ms * 1e-3) / 1e12, peak=MFMA_F32_PEAK_TFLOPS, unit="TFLOP/s")
+        ach = bf[dom][1] / (dom_ms * 1e-3) / 1e12
+        roof = dict(bound="mfma", achieved=ach, peak=MFMA_F16_PEAK_TFLOPS / F2F_PIECE_PRODUCTS, unit="TFLOP/s",
+                    peak_basis="fp16 dense MFMA 2500 TFLOP/s / 3 piece products per fp32-accurate product",
+                    frac_of_fp32_mfma_peak=ach / MFMA_F32_PEAK_TFLOPS)
     else:
         roof = dict(bound="hbm", achieved=bf[dom][0] / (dom_ms * 1e-3) / 1e9, peak=HBM_PEAK_GBS, unit="GB/s")
     traffic = SCENE_TRAFFIC_BYTES.get(dom) if (kind == "scene" and args.scale == 1.0) else None

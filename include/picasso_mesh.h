@@ -112,7 +112,10 @@ int pmesh_f2v_bwd(const float *grad_output, const float *input, const float *fil
  * re-arranged for the matrix cores; may be 0 bytes for shapes that need none).
  * facet_order: NULL, or the permutation pmesh_build_facet_order made from this cum_texture.  It
  * only groups facets with equal numbers of texture points into the same workgroups (faster when
- * the counts vary); results are identical with and without it.
+ * the counts vary).  With F = 16 the products run on fp16 matrix instructions with both operands
+ * split in two and scaled by powers of two; a facet's scale may depend on its workgroup when one of
+ * the workgroup's facets exceeds its first bound, so results with and without the order agree to
+ * an ulp, and bit for bit otherwise.
  */
 size_t pmesh_facet_order_workspace_bytes(int64_t n_facets);
 int pmesh_build_facet_order(const int32_t *cum_texture, int64_t n_facets, int64_t n_points,
@@ -130,7 +133,9 @@ int pmesh_f2f_fwd(const float *texture, const float *filter, const float *bary_c
  * it when they run on the same stream.  facet_order: NULL or the permutation of
  * pmesh_build_facet_order, as for the forward (grad_texture is bit-identical with and without
  * it; grad_filter sums the facets in the order given, so its last bits depend on it, and on
- * nothing else).  Every row of grad_texture is written
+ * nothing else).  With F = 16 the filter half runs an fp16 kernel whose block-floating scales hold
+ * unless magnitudes grow by more than 2^9 along the facet list; it then flags the case on the
+ * device and a second, guarded launch (three-piece bf16, no scales) computes the result again.  Every row of grad_texture is written
  * (rows past the last facet's segment are cleared) provided cum_texture is non-decreasing.
  * pmesh_f2f_bwd is the texture half followed by the filter half; each half can be called
  * alone when only one gradient is wanted (the reference always computes both,

@@ -26,11 +26,13 @@ typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kHKB = 4;                       // texture points per facet covered by one sweep (register budget)
+constexpr int kHFKB = 5;                      // the same in the forward, which has registers for one more
+constexpr int kHTKB = 6;                      // and in the texture gradient (bounded by its LDS stage)
 constexpr int kHChunk = 4 * 2 * 2 * 64;       // uint4 per LDS buffer: 4 channels x 2 tiles x 2 pieces x 64 lanes
 constexpr int kHW = 8;                        // wavefronts per workgroup
 constexpr int kHThreads = 64 * kHW;
 constexpr int kHWn = kHChunk / kHThreads;     // uint4 of a filter chunk fetched per thread
-constexpr int kHSlab = kHKB * 8 * 32;         // floats per slab buffer: points x 8 channels x facet slots
+constexpr int kHSlab = kHFKB * 8 * 32;         // floats per slab buffer: points x 8 channels x facet slots
 
 __device__ __forceinline__ float4 hld4(const float *p) { return *reinterpret_cast<const float4 *>(p); }
 template <bool VEC> __device__ __forceinline__ float4 hld4_row(const float *p, int n)
@@ -185,7 +187,7 @@ __device__ __forceinline__ void h2_sweep(const float *__restrict__ tex, const u3
     bool ldok[KW];
 #pragma unroll
     for (int i = 0; i < KW; ++i) {
-        const int slot = w * 32 + (lane >> 1), kk = sweep * kHKB + i;
+        const int slot = w * 32 + (lane >> 1), kk = sweep * kHFKB + i;
         ldok[i] = kk < s_K[slot];
         ldoff[i] = (unsigned)(s_k0[slot] + (ldok[i] ? kk : 0)) * (unsigned)Cin + cg4;
     }
@@ -395,7 +397,7 @@ __global__ __launch_bounds__(kHThreads, 2) void f2f16h2_fwd_k(const float *__res
         }
         __syncthreads();
         const float alpha = s_tm[w * 32 + l32], tlim = s_tl[w * 32 + (lane >> 1)];
-        const int nsweeps = (s_kmax + kHKB - 1) / kHKB;
+        const int nsweeps = (s_kmax + kHFKB - 1) / kHFKB;
         const float shs = K > 0 ? alpha / (float)K : 0.f;
 #pragma unroll
         for (int t = 0; t < 2; ++t)
@@ -403,16 +405,17 @@ __global__ __launch_bounds__(kHThreads, 2) void f2f16h2_fwd_k(const float *__res
             for (int i = 0; i < 16; ++i) acc[t][i] = 0.f;
         bool viol = false;
         for (int sw = 0; sw < nsweeps; ++sw) {
-            const int kbase = k0 + sw * kHKB;
-            const int rem = K - sw * kHKB;
-            const int Ks = rem < 0 ? 0 : (rem > kHKB ? kHKB : rem);
+            const int kbase = k0 + sw * kHFKB;
+            const int rem = K - sw * kHFKB;
+            const int Ks = rem < 0 ? 0 : (rem > kHFKB ? kHFKB : rem);
             // every variant runs the same barriers, so wavefronts of a workgroup may pick different ones
             const int kw = hwave_max(Ks);
 #define PM_H2(N) h2_sweep<N, TVEC>(tex, Wp, sh, Ws, s_slab + w * 2 * kHSlab, acc, kbase, Ks, shs, slim, tlim, viol, s_k0, s_K, sw, Cin, NT, nt0, nblk, w, lane, h)
             if (kw <= 1) PM_H2(1);
             else if (kw == 2) PM_H2(2);
             else if (kw == 3) PM_H2(3);
-            else PM_H2(4);
+            else if (kw == 4) PM_H2(4);
+            else PM_H2(5);
 #undef PM_H2
         }
         if (full || !__syncthreads_or(viol ? 1 : 0)) break;
@@ -551,7 +554,7 @@ __device__ __forceinline__ void h2_tex_sweep(const u32x4 *__restrict__ WpT, cons
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
             const int slot = 16 * i + (lane >> 2);
-            const int k0s = w_k0[slot] + sweep * kHKB, Kss = w_K[slot] - sweep * kHKB;
+            const int k0s = w_k0[slot] + sweep * kHTKB, Kss = w_K[slot] - sweep * kHTKB;
 #pragma unroll
             for (int kk = 0; kk < KW; ++kk)
                 if (kk < Kss && ci < Cin) {
@@ -661,7 +664,7 @@ __global__ __launch_bounds__(512, 2) void f2f16h2_bwd_tex_k(const float *__restr
                                                             int64_t Nf, int T, int Cin, int Cout, int NG, int co0)
 {
     __shared__ u32x4 Ws[3 * kHTChunkMax];
-    __shared__ __attribute__((aligned(16))) float s_stage[8][kHKB * 32 * 16];
+    __shared__ __attribute__((aligned(16))) float s_stage[8][kHTKB * 32 * 16];
     __shared__ int s_k0[8][32], s_K[8][32], s_kmax;
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
     const int l32 = lane & 31, h = lane >> 5;
@@ -715,18 +718,20 @@ __global__ __launch_bounds__(512, 2) void f2f16h2_bwd_tex_k(const float *__restr
     }
     const float shs = K > 0 ? igamma * hdr[1] / (float)K : 0.f;
     __syncthreads();
-    const int nsweeps = (s_kmax + kHKB - 1) / kHKB;
+    const int nsweeps = (s_kmax + kHTKB - 1) / kHTKB;
     for (int sw = 0; sw < nsweeps; ++sw) {
-        const int rem = K - sw * kHKB;
-        const int Ks = rem < 0 ? 0 : (rem > kHKB ? kHKB : rem);
+        const int rem = K - sw * kHTKB;
+        const int Ks = rem < 0 ? 0 : (rem > kHTKB ? kHTKB : rem);
         const int kw = hwave_max(Ks);
-        const int kbase = k0 + sw * kHKB;
+        const int kbase = k0 + sw * kHTKB;
         // every variant runs the same barriers, so wavefronts of a workgroup may pick different ones
 #define PM_H2T(N) h2_tex_sweep<N, NKS, GVEC>(WpT, sh, gtex, Ws, s_stage[w], s_k0[w], s_K[w], bp, kbase, Ks, shs, sw, Cin, NG, co0 > 0, lane, h)
         if (kw <= 1) PM_H2T(1);
         else if (kw == 2) PM_H2T(2);
         else if (kw == 3) PM_H2T(3);
-        else PM_H2T(4);
+        else if (kw == 4) PM_H2T(4);
+        else if (kw == 5) PM_H2T(5);
+        else PM_H2T(6);
 #undef PM_H2T
     }
 }

@@ -25,7 +25,7 @@ typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
-constexpr int kHKB = 4;                       // texture points per facet covered by one sweep (register budget)
+constexpr int kHKB = 9;                       // texture points per facet covered by one pass of the filter gradient (one wavefront per SIMD: 512 registers)
 constexpr int kHFKB = 5;                      // the same in the forward, which has registers for one more
 constexpr int kHTKB = 6;                      // and in the texture gradient (bounded by its LDS stage)
 constexpr int kHChunk = 4 * 2 * 2 * 64;       // uint4 per LDS buffer: 4 channels x 2 tiles x 2 pieces x 64 lanes
@@ -909,10 +909,11 @@ __device__ __forceinline__ HTile htile_load(const int *__restrict__ cum, const i
 // The inputs of a tile's first pass are fetched by the whole workgroup while the previous tile is
 // being multiplied (held in registers, written to the other LDS buffer afterwards):
 //   gout     thread (co, step, half): its eight facets in accumulator-row order
-//   SH rows  32 facets x 4 points x 64 bytes, two 16-byte pieces per thread
+//   SH rows  32 facets x kHKB points x 64 bytes, kHShv 16-byte pieces per thread
+constexpr int kHShv = (kHKB * 32 * 4 + 255) / 256;      // 16-byte pieces of the tile's SH rows per thread
 struct HPre {
     float g[8];
-    float4 shv[2];
+    float4 shv[kHShv];
 };
 __device__ __forceinline__ void hpre_issue(HPre &P, const float *__restrict__ gout, const float *__restrict__ sh,
                                            const int *sf, const int *sk0, const int *sK, int Cout, int n0)
@@ -924,9 +925,10 @@ __device__ __forceinline__ void hpre_issue(HPre &P, const float *__restrict__ go
         P.g[j] = (f >= 0 && n0 + co < Cout) ? gout[(int64_t)f * Cout + n0 + co] : 0.f;
     }
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
+    for (int i = 0; i < kHShv; ++i) {
         const int e = threadIdx.x + 256 * i, row = e >> 2, kk = row >> 5, slot = row & 31;
-        P.shv[i] = kk < sK[slot] ? hld4(sh + (int64_t)(sk0[slot] + kk) * 16 + 4 * (e & 3)) : make_float4(0.f, 0.f, 0.f, 0.f);
+        P.shv[i] = (kk < kHKB && kk < sK[slot]) ? hld4(sh + (int64_t)(sk0[slot] + kk) * 16 + 4 * (e & 3))
+                                                : make_float4(0.f, 0.f, 0.f, 0.f);
     }
 }
 __device__ __forceinline__ float hpre_gmax(const HPre &P)
@@ -951,9 +953,9 @@ __device__ __forceinline__ void hpre_commit(const HPre &P, u32x4 *go, float *shs
     dst[0] = p1; dst[64] = p2;
     if (with_sh) {
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
+        for (int i = 0; i < kHShv; ++i) {
             const int e = threadIdx.x + 256 * i;
-            *reinterpret_cast<float4 *>(shs + 4 * e) = P.shv[i];             // [point*32 + slot][16]
+            if (e < kHKB * 32 * 4) *reinterpret_cast<float4 *>(shs + 4 * e) = P.shv[i];      // [point*32 + slot][16]
         }
     }
 }
@@ -1183,7 +1185,7 @@ __global__ __launch_bounds__(256, 1) void f2f16h2_bwd_filt_k(const float *__rest
     }
     __syncthreads();
 
-    // The sorted facet list makes the point counts of my tiles non-decreasing: four loops in sequence,
+    // The sorted facet list makes the point counts of my tiles non-decreasing: one loop per point count in sequence,
     // each with the pass specialised for its number of points (the last one takes everything left,
     // long facets in several sweeps).  The bound is uniform over the workgroup.
     int it = 0;
@@ -1195,6 +1197,11 @@ __global__ __launch_bounds__(256, 1) void f2f16h2_bwd_filt_k(const float *__rest
     PM_PHASE(2);
     PM_PHASE(3);
     PM_PHASE(4);
+    PM_PHASE(5);
+    PM_PHASE(6);
+    PM_PHASE(7);
+    PM_PHASE(8);
+    PM_PHASE(9);
 #undef PM_PHASE
 
     // accumulator (cp, t): lane (co = 32t + l32, half h), register i <-> row m = 8(i/4) + 4h + i%4

@@ -222,8 +222,8 @@ __device__ __forceinline__ void h2_sweep(const float *__restrict__ tex, const u3
     }
     __syncthreads();
 
-    auto read_b = [&](u32x4 (&b)[2][2], int c) {          // filter pieces of channel c
-        const u32x4 *Wc = Ws + ((c >> 2) % 3) * kHChunk + (c & 3) * 256 + lane;
+    auto read_b = [&](u32x4 (&b)[2][2], int buf, int cl) { // filter pieces of channel cl of the chunk in buffer buf
+        const u32x4 *Wc = Ws + buf * kHChunk + cl * 256 + lane;
 #pragma unroll
         for (int t = 0; t < 2; ++t)
 #pragma unroll
@@ -252,10 +252,11 @@ __device__ __forceinline__ void h2_sweep(const float *__restrict__ tex, const u3
         float tv0[KW], a[8];
         read_tv(tv0, 0);
         read_tv(tvn, 1);
-        read_b(b, 0);
+        read_b(b, 0, 0);
         gen(a, tv0);
         split8h(a, pa[0], pa[1]);
     }
+    int wb0 = 0, wb1 = 1, wb2 = 2;                             // LDS buffers of chunks j, j+1, j+2
     for (int j = 0; j < nblk; ++j) {
         const int g = j >> 1;
         const bool wmore = j + 2 < nblk;
@@ -267,7 +268,9 @@ __device__ __forceinline__ void h2_sweep(const float *__restrict__ tex, const u3
             const int c = 4 * j + ci_l;
             u32x4 bn[2][2];
             float tvnn[KW];
-            read_b(bn, c + 1 < 4 * nblk ? c + 1 : c);
+            // channel c+1 (past the last channel: a piece that exists but is not used)
+            if (ci_l < 3) read_b(bn, wb0, ci_l + 1);
+            else read_b(bn, j + 1 < nblk ? wb1 : wb0, j + 1 < nblk ? 0 : 3);
             read_tv(tvnn, c + 2);
 
             float an[8];
@@ -293,10 +296,12 @@ __device__ __forceinline__ void h2_sweep(const float *__restrict__ tex, const u3
         }
         if (wmore) {
 #pragma unroll
-            for (int i = 0; i < kHWn; ++i) Ws[((j + 2) % 3) * kHChunk + threadIdx.x + kHThreads * i] = wn[i];
+            for (int i = 0; i < kHWn; ++i) Ws[wb2 * kHChunk + threadIdx.x + kHThreads * i] = wn[i];
         }
         if (stage) publish_group(slab + ((g + 1) & 1) * kHSlab);
         __syncthreads();
+        const int t = wb0;
+        wb0 = wb1; wb1 = wb2; wb2 = t;
     }
 }
 

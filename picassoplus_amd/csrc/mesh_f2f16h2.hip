@@ -29,9 +29,10 @@ constexpr int kHKB = 9;                       // texture points per facet covere
 constexpr int kHFKB = 5;                      // the same in the forward, which has registers for one more
 constexpr int kHTKB = 6;                      // and in the texture gradient (bounded by its LDS stage)
 constexpr int kHChunk = 4 * 2 * 2 * 64;       // uint4 per LDS buffer: 4 channels x 2 tiles x 2 pieces x 64 lanes
-constexpr int kHW = 8;                        // wavefronts per workgroup
+constexpr int kHW = 4;                        // wavefronts per workgroup of the forward: two workgroups share a CU
+constexpr int kHFacets = 32 * kHW;            // facets per workgroup
 constexpr int kHThreads = 64 * kHW;
-constexpr int kHWn = kHChunk / kHThreads;     // uint4 of a filter chunk fetched per thread
+constexpr int kHWn = kHChunk / kHThreads;     // uint4 of a filter chunk per thread
 constexpr int kHSlab = kHFKB * 8 * 32;         // floats per slab buffer: points x 8 channels x facet slots
 
 __device__ __forceinline__ float4 hld4(const float *p) { return *reinterpret_cast<const float4 *>(p); }
@@ -146,14 +147,21 @@ __global__ __launch_bounds__(kBlock) void f2f16h2_pack_filter_k(const float *__r
     dst[0] = p1; dst[64] = p2;
 }
 
-__device__ __forceinline__ void hw_chunk_fetch(const u32x4 *__restrict__ Wp, int c0, int NT, int nt0, u32x4 (&wn)[kHWn])
+// A chunk (four channels) moves in two halves of two channels, so that only kHWn / 2 registers per thread wait
+// between a fetch and its publication.  Channel c of the chunk: 2 tiles x 2 pieces x 64 lanes = 256 consecutive uint4.
+__device__ __forceinline__ void hw_half_fetch(const u32x4 *__restrict__ Wp, int c0, int half, int NT, int nt0,
+                                              u32x4 (&wn)[kHWn / 2])
 {
-    // channel c of the chunk: 2 tiles x 2 pieces x 64 lanes = 256 consecutive uint4
 #pragma unroll
-    for (int i = 0; i < kHWn; ++i) {
-        const int e = threadIdx.x + kHThreads * i, c = e >> 8, o = e & 255;
+    for (int i = 0; i < kHWn / 2; ++i) {
+        const int e = 512 * half + threadIdx.x + kHThreads * i, c = e >> 8, o = e & 255;
         wn[i] = Wp[((size_t)(c0 + c) * NT + nt0) * 128 + o];
     }
+}
+__device__ __forceinline__ void hw_half_publish(u32x4 *Wbuf, int half, const u32x4 (&wn)[kHWn / 2])
+{
+#pragma unroll
+    for (int i = 0; i < kHWn / 2; ++i) Wbuf[512 * half + threadIdx.x + kHThreads * i] = wn[i];
 }
 
 // One pass over all input channels for up to KW texture points per facet.  shs = alpha_f / K_f, the factor on
@@ -209,17 +217,13 @@ __device__ __forceinline__ void h2_sweep(const float *__restrict__ tex, const u3
         }
         viol |= m > tlim;
     };
-    u32x4 wn[kHWn];
+    u32x4 wn[kHWn / 2];
     fetch_group(0);
     publish_group(slab);
-    hw_chunk_fetch(Wp, 0, NT, nt0, wn);
-#pragma unroll
-    for (int i = 0; i < kHWn; ++i) Ws[threadIdx.x + kHThreads * i] = wn[i];
-    if (nblk > 1) {
-        hw_chunk_fetch(Wp, 4, NT, nt0, wn);
-#pragma unroll
-        for (int i = 0; i < kHWn; ++i) Ws[kHChunk + threadIdx.x + kHThreads * i] = wn[i];
-    }
+    hw_half_fetch(Wp, 0, 0, NT, nt0, wn);
+    hw_half_publish(Ws, 0, wn);
+    hw_half_fetch(Wp, 0, 1, NT, nt0, wn);
+    hw_half_publish(Ws, 1, wn);
     __syncthreads();
 
     auto read_b = [&](u32x4 (&b)[2][2], int buf, int cl) { // filter pieces of channel cl of the chunk in buffer buf
@@ -256,21 +260,21 @@ __device__ __forceinline__ void h2_sweep(const float *__restrict__ tex, const u3
         gen(a, tv0);
         split8h(a, pa[0], pa[1]);
     }
-    int wb0 = 0, wb1 = 1, wb2 = 2;                             // LDS buffers of chunks j, j+1, j+2
+    // filter chunks alternate between two LDS buffers: chunk j+1 is fetched at the start of chunk j and published
+    // at its end; the first channel of a chunk reads its pieces right after the barrier, under the generation
+    // and split of the channel after it
     for (int j = 0; j < nblk; ++j) {
-        const int g = j >> 1;
-        const bool wmore = j + 2 < nblk;
+        const int g = j >> 1, wb = j & 1;
+        const bool wmore = j + 1 < nblk;
         const bool stage = !(j & 1) && 8 * (g + 1) < Cin;       // even chunk: bring in the next 8-channel group
-        if (wmore) hw_chunk_fetch(Wp, 4 * (j + 2), NT, nt0, wn);
+        if (wmore) hw_half_fetch(Wp, 4 * (j + 1), 0, NT, nt0, wn);
         if (stage) fetch_group(g + 1);
 #pragma unroll
         for (int ci_l = 0; ci_l < 4; ++ci_l) {
             const int c = 4 * j + ci_l;
             u32x4 bn[2][2];
             float tvnn[KW];
-            // channel c+1 (past the last channel: a piece that exists but is not used)
-            if (ci_l < 3) read_b(bn, wb0, ci_l + 1);
-            else read_b(bn, j + 1 < nblk ? wb1 : wb0, j + 1 < nblk ? 0 : 3);
+            if (ci_l < 3) read_b(bn, wb, ci_l + 1);
             read_tv(tvnn, c + 2);
 
             float an[8];
@@ -289,19 +293,21 @@ __device__ __forceinline__ void h2_sweep(const float *__restrict__ tex, const u3
             pa[0] = pn[0]; pa[1] = pn[1];
 #pragma unroll
             for (int kk = 0; kk < KW; ++kk) tvn[kk] = tvnn[kk];
+            if (ci_l < 3) {
 #pragma unroll
-            for (int t = 0; t < 2; ++t)
+                for (int t = 0; t < 2; ++t)
 #pragma unroll
-                for (int p = 0; p < 2; ++p) b[t][p] = bn[t][p];
+                    for (int p = 0; p < 2; ++p) b[t][p] = bn[t][p];
+            }
+            if (ci_l == 1 && wmore) {                       // nobody reads the other buffer during this chunk
+                hw_half_publish(Ws + (wb ^ 1) * kHChunk, 0, wn);
+                hw_half_fetch(Wp, 4 * (j + 1), 1, NT, nt0, wn);
+            }
         }
-        if (wmore) {
-#pragma unroll
-            for (int i = 0; i < kHWn; ++i) Ws[wb2 * kHChunk + threadIdx.x + kHThreads * i] = wn[i];
-        }
+        if (wmore) hw_half_publish(Ws + (wb ^ 1) * kHChunk, 1, wn);
         if (stage) publish_group(slab + ((g + 1) & 1) * kHSlab);
         __syncthreads();
-        const int t = wb0;
-        wb0 = wb1; wb1 = wb2; wb2 = t;
+        if (wmore) read_b(b, wb ^ 1, 0);
     }
 }
 
@@ -312,18 +318,18 @@ __global__ __launch_bounds__(kHThreads, 2) void f2f16h2_fwd_k(const float *__res
                                                               float *__restrict__ out, int64_t Nf, int T, int Cin,
                                                               int Cout, int NT)
 {
-    __shared__ u32x4 Ws[3 * kHChunk];
+    __shared__ u32x4 Ws[2 * kHChunk];
     __shared__ __attribute__((aligned(16))) float s_slab[kHW * 2 * kHSlab];      // per wavefront: two buffers
-    __shared__ int s_f[256], s_k0[256], s_K[256], s_kmax;
-    __shared__ float s_tm[256], s_inv[256], s_tl[256];
+    __shared__ int s_f[kHFacets], s_k0[kHFacets], s_K[kHFacets], s_kmax;
+    __shared__ float s_tm[kHFacets], s_inv[kHFacets], s_tl[kHFacets];
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
     const int l32 = lane & 31, h = lane >> 5;
-    const int64_t s0 = (int64_t)blockIdx.x * 256;
+    const int64_t s0 = (int64_t)blockIdx.x * kHFacets;
     const int nt0 = blockIdx.y * 2, n0 = blockIdx.y * 64;
     const int nblk = (Cin + 3) >> 2;
 
     if (threadIdx.x == 0) s_kmax = 0;
-    for (int i = threadIdx.x; i < 256; i += kHThreads) {
+    for (int i = threadIdx.x; i < kHFacets; i += kHThreads) {
         const int64_t slot = s0 + i;
         const int f = slot < Nf ? (order ? order[slot] : (int)slot) : -1;
         int a = 0, b = 0;
@@ -464,7 +470,7 @@ int f2f16h2_fwd(const float *tex, const float *W, const float *sh, const int *cu
     const int CinPad = (Cin + 3) & ~3, n = CinPad * NT * 64;
     f2f16h2_pack_filter_k<<<dim3((unsigned)ceil_div(n, kBlock)), dim3(kBlock), 0, st>>>(W, hdr, Wp, Cin, CinPad, Cout, NT);
     PM_LAUNCHED("f2f_fwd(pack)");
-    const int64_t gx = ceil_div(Nf, 256), gy = NT / 2;
+    const int64_t gx = ceil_div(Nf, kHFacets), gy = NT / 2;
     PM_REQUIRE(grid_ok(gx) && gy <= 65535, "f2f_fwd: grid too large");
     if (!(Cin & 3) && !(reinterpret_cast<uintptr_t>(tex) & 15u))
         f2f16h2_fwd_k<true><<<dim3((unsigned)gx, (unsigned)gy), dim3(kHThreads), 0, st>>>(tex, hdr, Wp, sh, cum, order, out, Nf, (int)T, Cin, Cout, NT);

@@ -68,4 +68,9 @@ int f2f_narrow_blocks(int64_t Nf);
 int f2f_bwd_filter_narrow_partials(const float *gout, const float *tex, const float *sh, const int *cum, float *partial,
                                    int blocks, int64_t T, int64_t Nf, int Cin, int Cout, hipStream_t st);
 
+// Narrow forward (same file): at most four input channels, F == 16, 16-byte aligned SH rows; no workspace.
+bool f2f_fwd_narrow_usable(int Cin, int F, const void *sh);
+int f2f_fwd_narrow(const float *tex, const float *W, const float *sh, const int *cum, float *out, int64_t T, int64_t Nf,
+                   int Cin, int Cout, hipStream_t st);
+
 }  // namespace pmesh

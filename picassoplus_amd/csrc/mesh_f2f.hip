@@ -374,6 +374,8 @@ extern "C" int pmesh_f2f_fwd(const float *texture, const float *filter, const fl
     if (Nf == 0) return 0;
     PM_REQUIRE(filter && cum_texture && output && (T == 0 || (texture && bary_coeff)), "f2f_fwd: null pointer");
     // the split-bf16 forward addresses texture elements with 32-bit offsets
+    if (!force_generic() && !force_fp32_mfma() && !force_bf16x3() && f2f_fwd_narrow_usable(Cin, F, bary_coeff))
+        return f2f_fwd_narrow(texture, filter, bary_coeff, cum_texture, output, T, Nf, Cin, Cout, (hipStream_t)stream);
     if (!force_generic() && !force_fp32_mfma() && !force_bf16x3() && f2f16x3_usable(filter, bary_coeff, F) &&
         T * Cin < (int64_t(1) << 31))
         return f2f16h2_fwd(texture, filter, bary_coeff, cum_texture, facet_order, output, workspace, workspace_bytes,

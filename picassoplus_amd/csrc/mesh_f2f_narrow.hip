@@ -166,4 +166,129 @@ int f2f_bwd_filter_narrow_partials(const float *gout, const float *tex, const fl
     return 0;
 }
 
+
+// ----------------------------------------------------------------------------------------
+// Forward for the same narrow inputs: out[f, co] = sum_(ci,d) G[f,ci,d] * W[co,ci,d] as fp32 MFMAs whose
+// reduction index runs over the (at most) 64 columns (ci, d):
+//   product    out tile (32 facets x 32 output channels) += G (32 facets x 2 columns) . W^T (2 columns x 32),
+//              32 MFMAs per tile; step s, half h <-> column (ci = s/8, d = 8h + s%8)
+//   lane       (facet l%32 of the tile, half h): forms the 32 G values of its half from the facet's points
+//              (32 bytes of each SH row and the point's texture values); as B operand it holds W of output
+//              channel l%32 for the same columns (registers, loaded once)
+//   wavefront  a contiguous run of 32-facet tiles in natural order (sequential reads and writes), five points
+//              per facet and round with all loads of a round in flight together
+template <int NT>
+__global__ __launch_bounds__(kBlock) void f2f_fwd_narrow_k(const float *__restrict__ tex, const float *__restrict__ W,
+                                                           const float *__restrict__ sh, const int *__restrict__ cum,
+                                                           float *__restrict__ out, int64_t Nf, int T, int Cin, int Cout,
+                                                           int64_t tiles_per_wave)
+{
+    constexpr int KU = 5;
+    const int l = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int m = l & 31, h = l >> 5;
+    const int n0 = blockIdx.y * (32 * NT);
+    // B operands: wb[nt][s] = W[n0 + 32nt + m][s/8][8h + s%8]
+    float wb[NT][32];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+        const int co = n0 + 32 * nt + m;
+#pragma unroll
+        for (int s = 0; s < 32; ++s)
+            wb[nt][s] = (co < Cout && (s >> 3) < Cin) ? W[((int64_t)co * Cin + (s >> 3)) * 16 + 8 * h + (s & 7)] : 0.f;
+    }
+    const int64_t ntiles = (Nf + 31) >> 5;
+    const int64_t tbeg = ((int64_t)blockIdx.x * 4 + wave) * tiles_per_wave;
+    const int64_t tend = (tbeg + tiles_per_wave < ntiles) ? tbeg + tiles_per_wave : ntiles;
+
+    auto bounds = [&](int64_t tile, int &a, int &b) {
+        const int64_t f = tile * 32 + m;
+        a = 0; b = 0;
+        if (tile < tend && f < Nf) {
+            a = f ? cum[f - 1] : 0;
+            b = cum[f];
+        }
+        a = a < 0 ? 0 : (a > T ? T : a);
+        b = b < a ? a : (b > T ? T : b);
+    };
+    int k0, k1;
+    bounds(tbeg, k0, k1);
+    for (int64_t tile = tbeg; tile < tend; ++tile) {
+        int nk0, nk1;
+        bounds(tile + 1, nk0, nk1);
+        const int K = k1 - k0;
+        float G[4][8];
+#pragma unroll
+        for (int c = 0; c < 4; ++c)
+#pragma unroll
+            for (int q = 0; q < 8; ++q) G[c][q] = 0.f;
+        for (int kb = 0; kb == 0 || __builtin_amdgcn_ballot_w64(kb < K) != 0ull; kb += KU) {
+            float4 su[KU], sv[KU];
+            float tv[KU][4];
+#pragma unroll
+            for (int u = 0; u < KU; ++u) {
+                const bool on = kb + u < K;
+                const int64_t pt = k0 + kb + u;
+                su[u] = on ? *reinterpret_cast<const float4 *>(sh + pt * 16 + 8 * h) : make_float4(0.f, 0.f, 0.f, 0.f);
+                sv[u] = on ? *reinterpret_cast<const float4 *>(sh + pt * 16 + 8 * h + 4) : make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+                for (int c = 0; c < 4; ++c) tv[u][c] = (on && c < Cin) ? tex[pt * Cin + c] : 0.f;
+            }
+#pragma unroll
+            for (int u = 0; u < KU; ++u)
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    G[c][0] = fmaf(tv[u][c], su[u].x, G[c][0]); G[c][1] = fmaf(tv[u][c], su[u].y, G[c][1]);
+                    G[c][2] = fmaf(tv[u][c], su[u].z, G[c][2]); G[c][3] = fmaf(tv[u][c], su[u].w, G[c][3]);
+                    G[c][4] = fmaf(tv[u][c], sv[u].x, G[c][4]); G[c][5] = fmaf(tv[u][c], sv[u].y, G[c][5]);
+                    G[c][6] = fmaf(tv[u][c], sv[u].z, G[c][6]); G[c][7] = fmaf(tv[u][c], sv[u].w, G[c][7]);
+                }
+        }
+        const float invK = K > 0 ? 1.0f / (float)K : 0.f;
+        f32x16 acc[NT];
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) acc[nt][i] = 0.f;
+#pragma unroll
+        for (int s = 0; s < 32; ++s) {
+            const float a = G[s >> 3][s & 7] * invK;
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) acc[nt] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, wb[nt][s], acc[nt], 0, 0, 0);
+        }
+        // accumulator: lane (co = n0 + 32nt + m, half h), register i <-> facet 8(i/4) + 4h + i%4 of the tile
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+            const int co = n0 + 32 * nt + m;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const int64_t f = tile * 32 + 8 * (i >> 2) + 4 * h + (i & 3);
+                if (f < Nf && co < Cout) out[f * Cout + co] = acc[nt][i];
+            }
+        }
+        k0 = nk0; k1 = nk1;
+    }
+}
+
+bool f2f_fwd_narrow_usable(int Cin, int F, const void *sh) { return F == 16 && Cin <= 4 && !(reinterpret_cast<uintptr_t>(sh) & 15u); }
+
+int f2f_fwd_narrow(const float *tex, const float *W, const float *sh, const int *cum, float *out, int64_t T, int64_t Nf,
+                   int Cin, int Cout, hipStream_t st)
+{
+    const int nt = Cout <= 32 ? 1 : 2;
+    const int64_t gy = ceil_div(Cout, 32 * nt);
+    PM_REQUIRE(gy <= 65535, "f2f_fwd: grid too large");
+    const int64_t ntiles = ceil_div(Nf, 32);
+    int64_t blocks = ceil_div(ntiles, 4 * 4);                 // at least four tiles per wavefront
+    if (blocks > 4096) blocks = 4096;
+    if (blocks < 1) blocks = 1;
+    const int64_t tpw = ceil_div(ntiles, blocks * 4);
+    const dim3 grid((unsigned)blocks, (unsigned)gy);
+    if (nt == 1)
+        f2f_fwd_narrow_k<1><<<grid, dim3(kBlock), 0, st>>>(tex, W, sh, cum, out, Nf, (int)T, Cin, Cout, tpw);
+    else
+        f2f_fwd_narrow_k<2><<<grid, dim3(kBlock), 0, st>>>(tex, W, sh, cum, out, Nf, (int)T, Cin, Cout, tpw);
+    PM_LAUNCHED("f2f_fwd(narrow)");
+    return 0;
+}
+
 }  // namespace pmesh

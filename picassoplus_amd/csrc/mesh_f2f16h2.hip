@@ -13,9 +13,10 @@
 // so that |W'|, |G'| < 2^14.  Elements far below their row's maximum (by more than 2^17) fall into fp16's
 // subnormal range and keep an ABSOLUTE error of 2^-25 in scaled units, i.e. below 2^-39 of the row maximum.
 //
-// Work decomposition: as the three-piece bf16 kernel (workgroup = 256 facets from the list sorted by
-// point count x 64 output channels, 8 wavefronts x 32 facets, two wavefronts per SIMD, filter chunks of
-// four channels through three LDS buffers, texture rows through a wavefront-private LDS slab).
+// Work decomposition of the forward: workgroup = 128 facets from the list sorted by point count x 64 output
+// channels, 4 wavefronts x 32 facets; two workgroups share a CU (two wavefronts per SIMD) and run out of
+// phase, so the prologue, barriers and stores of one overlap the channel loop of the other.  Filter chunks
+// of four channels alternate between two LDS buffers, texture rows go through a wavefront-private LDS slab.
 #include "f2f_internal.h"
 
 namespace pmesh {
@@ -26,7 +27,7 @@ typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kHKB = 9;                       // texture points per facet covered by one pass of the filter gradient (one wavefront per SIMD: 512 registers)
-constexpr int kHFKB = 5;                      // the same in the forward, which has registers for one more
+constexpr int kHFKB = 5;                      // the same per sweep of the forward (two wavefronts per SIMD: 256 registers)
 constexpr int kHTKB = 6;                      // and in the texture gradient (bounded by its LDS stage)
 constexpr int kHChunk = 4 * 2 * 2 * 64;       // uint4 per LDS buffer: 4 channels x 2 tiles x 2 pieces x 64 lanes
 constexpr int kHW = 4;                        // wavefronts per workgroup of the forward: two workgroups share a CU

@@ -232,6 +232,43 @@ def test_f2f_wide_dynamic_range(cuda, case):
     assert_close(ft.grad, gfilt_ref, "f2f grad_filter")
 
 
+def test_f2f_without_facet_order(cuda):
+    """The facet order is optional at the C ABI (NULL): same results for the forward and the texture gradient
+    (to an ulp), the same filter gradient up to summation order."""
+    from picassoplus_amd import _lib
+    from picassoplus_amd.mesh import topology
+    say("case f2f without facet order")
+    rng = np.random.default_rng(55)
+    nf, Cin, Cout = 900, 24, 40
+    counts, bary, _ = texture_case(rng, nf, 11)
+    T = int(counts.sum())
+    tex = dev(rng.uniform(-1, 1, (T, Cin)), cuda, torch.float32)
+    sh = dev(rng.normal(0, 0.5, (T, 16)), cuda, torch.float32)
+    w = dev(rng.normal(0, 0.3, (Cout, Cin, 16)), cuda, torch.float32)
+    g = dev(rng.normal(0, 1, (nf, Cout)), cuda, torch.float32)
+    cum = torch.cumsum(dev(counts, cuda), 0, dtype=torch.int32)
+    order = topology.facet_order(cum, T)
+    st = torch.cuda.current_stream().cuda_stream
+    nfw = _lib.query("pmesh_f2f_fwd_workspace_bytes", Cin, Cout, 16)
+    nbw = _lib.query("pmesh_f2f_bwd_workspace_bytes", Cin, Cout, 16)
+    ws = torch.empty(max(nfw, nbw), dtype=torch.uint8, device=cuda)
+    res = []
+    for o in (order.data_ptr(), None):
+        out = torch.empty(nf, Cout, device=cuda)
+        gtex = torch.empty(T, Cin, device=cuda)
+        gw = torch.empty(Cout, Cin, 16, device=cuda)
+        _lib.call("pmesh_f2f_fwd", tex.data_ptr(), w.data_ptr(), sh.data_ptr(), cum.data_ptr(), o, out.data_ptr(),
+                  ws.data_ptr(), nfw, T, nf, Cin, Cout, 16, st)
+        _lib.call("pmesh_f2f_bwd", g.data_ptr(), tex.data_ptr(), w.data_ptr(), sh.data_ptr(), cum.data_ptr(), o,
+                  gtex.data_ptr(), gw.data_ptr(), ws.data_ptr(), nbw, T, nf, Cin, Cout, 16, st)
+        torch.cuda.synchronize()
+        res.append((out, gtex, gw))
+    (o1, t1, w1), (o2, t2, w2) = res
+    assert float((o1 - o2).abs().max()) <= 2e-7 * float(o1.abs().max())
+    assert float((t1 - t2).abs().max()) <= 2e-7 * float(t1.abs().max())
+    assert float((w1 - w2).abs().max()) <= 1e-5 * float(w1.abs().max())
+
+
 def test_f2f_shape_sweep(cuda):
     """Seeded sweep over channel counts, facet counts and point counts around the tile sizes of the
     16-coefficient kernels (32-facet wavefront tiles, 4/8/16-channel groups, 64-channel blocks)."""

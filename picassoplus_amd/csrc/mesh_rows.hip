@@ -82,7 +82,21 @@ __global__ __launch_bounds__(kBlock) void fill_zero_k(float *__restrict__ p, int
 // ----------------------------------------------------------------------------------------
 // vertex2facet forward:  out[f, c*r+m] = sum_k filt[k,c,m] * in[face[f,k], c]
 // ----------------------------------------------------------------------------------------
-template <int V>
+// V consecutive output channels of a lane read V / R consecutive input channels (R = depth multiplier when the
+// vector form handles it: 1, or 2 with V = 4), each used R times
+template <int V, int R> __device__ __forceinline__ Pack<V> ld_in_wide(const float *p)
+{
+    if constexpr (R == 1) {
+        return ldp<V>(p);
+    } else {
+        const float2 t = *reinterpret_cast<const float2 *>(p);
+        Pack<V> o;
+        o.v[0] = t.x; o.v[1] = t.x; o.v[2] = t.y; o.v[3] = t.y;
+        return o;
+    }
+}
+
+template <int V, int R>
 __global__ __launch_bounds__(kBlock) void v2f_fwd_k(const float *__restrict__ in,
                                                     const float *__restrict__ filt,
                                                     const int *__restrict__ face,
@@ -97,8 +111,9 @@ __global__ __launch_bounds__(kBlock) void v2f_fwd_k(const float *__restrict__ in
     const int64_t v0 = face[3 * f], v1 = face[3 * f + 1], v2 = face[3 * f + 2];
     for (int q = lane; q < Q; q += lpr) {
         const int co = q * V;
-        const int c = (V == 4) ? co : co / r;
-        const Pack<V> a0 = ldp<V>(in + v0 * C + c), a1 = ldp<V>(in + v1 * C + c), a2 = ldp<V>(in + v2 * C + c);
+        const int c = (V == 4) ? co / R : co / r;
+        const Pack<V> a0 = ld_in_wide<V, R>(in + v0 * C + c), a1 = ld_in_wide<V, R>(in + v1 * C + c),
+                      a2 = ld_in_wide<V, R>(in + v2 * C + c);
         const Pack<V> f0 = ldp<V>(filt + co), f1 = ldp<V>(filt + Co + co), f2 = ldp<V>(filt + 2 * Co + co);
         Pack<V> o;
 #pragma unroll
@@ -111,9 +126,10 @@ __global__ __launch_bounds__(kBlock) void v2f_fwd_k(const float *__restrict__ in
 // vertex2facet backward, one pass over the vertex -> (facet, corner) adjacency:
 //   gin[v,c]     = sum_{(f,k) at v} sum_m gout[f,c*r+m] * filt[k,c,m]
 //   gfilt[k,c,m] = sum_v in[v,c] * sum_{(f,k) at v} gout[f,c*r+m]        (per-workgroup partials)
-// Lanes own input channels; the depth multiplier is an outer loop (V = 4 implies r = 1).
+// Lanes own V output channels.  V = 1: any depth multiplier, as an outer loop.  V = 4: r = R = 1 (four input
+// channels), or r = R = 2 (two input channels, each the sum over its two outputs: both sit in the lane).
 // ----------------------------------------------------------------------------------------
-template <int V>
+template <int V, int R>
 __global__ __launch_bounds__(kBlock) void v2f_bwd_k(const float *__restrict__ gout,
                                                     const float *__restrict__ in,
                                                     const float *__restrict__ filt,
@@ -129,12 +145,12 @@ __global__ __launch_bounds__(kBlock) void v2f_bwd_k(const float *__restrict__ go
     const int Co = C * r;
     const int64_t rbeg = (int64_t)blockIdx.x * rows_per_block;
     const int64_t rend = (rbeg + rows_per_block < Nv) ? rbeg + rows_per_block : Nv;
-    for (int m = 0; m < r; ++m)
+    for (int m = 0; m < (V == 4 ? 1 : r); ++m)
         for (int q0 = 0; q0 < Q; q0 += lpr) {
             const int q = q0 + lane;
             const bool active = q < Q;
-            const int c = q * V;
-            const int co = (V == 4) ? c : c * r + m;
+            const int c = (V == 4) ? q * V / R : q;
+            const int co = (V == 4) ? q * V : c * r + m;
             Pack<V> fk[3], acc[3];
 #pragma unroll
             for (int k = 0; k < 3; ++k) {
@@ -151,7 +167,7 @@ __global__ __launch_bounds__(kBlock) void v2f_bwd_k(const float *__restrict__ go
                 for (; row < rend; row += rpb) {
                     int ne0 = 0, ne1 = 0;
                     if (row + rpb < rend) { ne0 = rowptr[row + rpb]; ne1 = rowptr[row + rpb + 1]; }
-                    const Pack<V> x = ldp<V>(in + row * C + c);
+                    const Pack<V> x = ld_in_wide<V, R>(in + row * C + c);
                     Pack<V> g = zero_pack<V>(), s[3];
 #pragma unroll
                     for (int k = 0; k < 3; ++k) s[k] = zero_pack<V>();
@@ -181,7 +197,9 @@ __global__ __launch_bounds__(kBlock) void v2f_bwd_k(const float *__restrict__ go
 #pragma unroll
                         for (int u = 0; u < V; ++u) acc[k].v[u] = fmaf(s[k].v[u], x.v[u], acc[k].v[u]);
                     float *gp = gin + row * C + c;
-                    if (m == 0) {
+                    if constexpr (V == 4 && R == 2) {
+                        *reinterpret_cast<float2 *>(gp) = make_float2(g.v[0] + g.v[1], g.v[2] + g.v[3]);
+                    } else if (m == 0) {
                         stp<V>(gp, g);
                     } else {
 #pragma unroll
@@ -840,6 +858,15 @@ __global__ __launch_bounds__(kBlock) void sph_harm_k(const float *__restrict__ x
 // ----------------------------------------------------------------------------------------
 static inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
+// vertex2facet: V = 4 also with depth multiplier 2 (two input channels per lane) when C is even
+static inline int pick_v2f(int C, int r, std::initializer_list<const void *> ptrs)
+{
+    if (!((r == 1 && !(C & 3)) || (r == 2 && !(C & 1)))) return 1;
+    for (const void *p : ptrs)
+        if ((reinterpret_cast<uintptr_t>(p) & 15u) != 0) return 1;
+    return 4;
+}
+
 // V = 4 needs r == 1, C % 4 == 0 and 16-byte aligned feature arrays.
 static inline int pick_v(int C, int r, std::initializer_list<const void *> ptrs)
 {
@@ -923,14 +950,16 @@ extern "C" int pmesh_v2f_fwd(const float *input, const float *filter, const int3
     PM_REQUIRE(input && filter && face && output, "v2f_fwd: null pointer");
     PM_REQUIRE(Nv <= INT32_MAX && Nf <= INT32_MAX / 3, "v2f_fwd: sizes exceed int32 indexing");
     hipStream_t st = (hipStream_t)stream;
-    const int V = pick_v(C, r, {input, filter, output});
+    const int V = pick_v2f(C, r, {input, filter, output});
     const RowShape rs = row_shape(C * r / V);
     const int64_t blocks = ceil_div(Nf, rs.rpb);
     PM_REQUIRE(grid_ok(blocks), "v2f_fwd: grid too large");
-    if (V == 4)
-        v2f_fwd_k<4><<<dim3((unsigned)blocks), dim3(kBlock), 0, st>>>(input, filter, face, output, Nf, C, r, rs.items, rs.lpr_log2);
+    if (V == 4 && r == 2)
+        v2f_fwd_k<4, 2><<<dim3((unsigned)blocks), dim3(kBlock), 0, st>>>(input, filter, face, output, Nf, C, r, rs.items, rs.lpr_log2);
+    else if (V == 4)
+        v2f_fwd_k<4, 1><<<dim3((unsigned)blocks), dim3(kBlock), 0, st>>>(input, filter, face, output, Nf, C, r, rs.items, rs.lpr_log2);
     else
-        v2f_fwd_k<1><<<dim3((unsigned)blocks), dim3(kBlock), 0, st>>>(input, filter, face, output, Nf, C, r, rs.items, rs.lpr_log2);
+        v2f_fwd_k<1, 1><<<dim3((unsigned)blocks), dim3(kBlock), 0, st>>>(input, filter, face, output, Nf, C, r, rs.items, rs.lpr_log2);
     PM_LAUNCHED("v2f_fwd");
     return 0;
 }
@@ -957,16 +986,18 @@ extern "C" int pmesh_v2f_bwd(const float *grad_output, const float *input, const
         return 0;
     }
     PM_REQUIRE(grad_output && input && filter && rowptr && colidx && grad_input && workspace, "v2f_bwd: null pointer");
-    const int V = pick_v(C, r, {grad_output, input, filter, grad_input, workspace});
-    const RowShape rs = row_shape(C / V);
+    const int V = pick_v2f(C, r, {grad_output, input, filter, grad_input, workspace});
+    const RowShape rs = row_shape(V == 4 ? Co / 4 : C);
     const int G = persistent_blocks(Nv, rs.rpb);
     const int64_t rows_per_block = ceil_div(ceil_div(Nv, G), rs.rpb) * rs.rpb;
     PM_REQUIRE(workspace_bytes >= (size_t)G * 3 * Co * sizeof(float), "v2f_bwd: workspace too small (%zu bytes)", workspace_bytes);
     float *partial = (float *)workspace;
-    if (V == 4)
-        v2f_bwd_k<4><<<dim3(G), dim3(kBlock), 0, st>>>(grad_output, input, filter, rowptr, colidx, grad_input, partial, Nv, C, r, rs.items, rs.lpr_log2, rows_per_block);
+    if (V == 4 && r == 2)
+        v2f_bwd_k<4, 2><<<dim3(G), dim3(kBlock), 0, st>>>(grad_output, input, filter, rowptr, colidx, grad_input, partial, Nv, C, r, rs.items, rs.lpr_log2, rows_per_block);
+    else if (V == 4)
+        v2f_bwd_k<4, 1><<<dim3(G), dim3(kBlock), 0, st>>>(grad_output, input, filter, rowptr, colidx, grad_input, partial, Nv, C, r, rs.items, rs.lpr_log2, rows_per_block);
     else
-        v2f_bwd_k<1><<<dim3(G), dim3(kBlock), 0, st>>>(grad_output, input, filter, rowptr, colidx, grad_input, partial, Nv, C, r, rs.items, rs.lpr_log2, rows_per_block);
+        v2f_bwd_k<1, 1><<<dim3(G), dim3(kBlock), 0, st>>>(grad_output, input, filter, rowptr, colidx, grad_input, partial, Nv, C, r, rs.items, rs.lpr_log2, rows_per_block);
     PM_LAUNCHED("v2f_bwd");
     return reduce_partials(partial, grad_filter, G, 3 * Co, st);
 }

@@ -72,7 +72,8 @@ def test_cluster_csr_exact(cuda, spatial):
 # ------------------------------------------------------------------ vertex2facet
 @pytest.mark.parametrize("mesh,C,r", [("tetra", 4, 1), ("octa", 5, 2), ("sphere2", 32, 1), ("sphere3", 64, 1),
                                       ("room_small", 64, 1), ("sphere2", 7, 3), ("torus", 130, 1),
-                                      ("octa", 2048, 1), ("sphere2", 96, 1)])
+                                      ("octa", 2048, 1), ("sphere2", 96, 1), ("sphere3", 32, 2), ("room_small", 66, 2),
+                                      ("sphere2", 128, 2), ("torus", 9, 2)])
 def test_v2f_parity(cuda, mesh, C, r):
     say("case v2f", mesh, C, r)
     v, f = mesh_case(mesh)

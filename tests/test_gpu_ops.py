@@ -158,7 +158,8 @@ def test_f2v_unit_count_is_plain_scatter(cuda):
 @pytest.mark.parametrize("nf,Cin,Cout,F,kmax", [(10, 3, 8, 16, 3), (100, 3, 32, 16, 5), (200, 64, 64, 16, 9),
                                                 (333, 16, 96, 16, 4), (70, 5, 7, 9, 3), (65, 4, 6, 36, 2),
                                                 (64, 3, 5, 50, 2), (129, 130, 64, 4, 3), (50, 8, 8, 1, 2),
-                                                (300, 8, 40, 16, 14), (1000, 64, 64, 16, 9), (130, 4, 130, 16, 20)])
+                                                (300, 8, 40, 16, 14), (1000, 64, 64, 16, 9), (130, 4, 130, 16, 20),
+                                                (50, 1, 8, 16, 3), (77, 2, 33, 16, 12)])
 @pytest.mark.parametrize("path", ["default", "generic", "fp32mfma", "bf16x3"])
 def test_f2f_parity(cuda, monkeypatch, nf, Cin, Cout, F, kmax, path):
     """``generic`` forces the shape-generic kernels, ``fp32mfma`` the fp32-matrix-instruction variant of the

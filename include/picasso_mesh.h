@@ -207,6 +207,25 @@ int pmesh_count_vertex_adjface(const int32_t *rowptr, int32_t *nf_count, int64_t
 int pmesh_triangle_geometry(const float *vertex, const int32_t *face, float *geometry, int64_t Nv,
                             int64_t Nf, int vertex_stride, pmesh_stream_t stream);
 
+/* ------------------------------------------------------------------ pointwise tail of the convs
+ * replaces the PyTorch ops that follow every convolution (picasso/mesh/layers.py:114-119, 169-174,
+ * 232-238: torch.matmul(outputs, depth_weights) + biases, activation_fn, BatchNorm) by one pass:
+ *   output (N,Co) = act(input (N,Ci) . weight (Ci,Co) + bias (Co)) * scale (Co) + shift (Co)
+ * relu != 0 selects max(.,0), else identity; bias, scale, shift may be NULL (0, 1, 0): scale/shift carry
+ * an inference-mode batch norm (gamma/sqrt(var+eps), beta - mean*that).  Ci <= 1024.
+ * pmesh_dense_bwd is the gradient of the tail without scale/shift (training-mode batch norm stays
+ * outside): gz = grad_output where output > 0 (output = the forward result, NULL when relu was off);
+ * grad_input (N,Ci) = gz . weight^T (NULL skips it), grad_weight (Ci,Co) = input^T . gz,
+ * grad_bias (Co) = column sums of gz; both sums in a fixed order. */
+int pmesh_dense_fwd(const float *input, const float *weight, const float *bias, const float *scale,
+                    const float *shift, int relu, float *output, int64_t N, int Ci, int Co,
+                    pmesh_stream_t stream);
+size_t pmesh_dense_bwd_workspace_bytes(int64_t N, int Ci, int Co);
+int pmesh_dense_bwd(const float *grad_output, const float *input, const float *weight,
+                    const float *output, float *grad_input, float *grad_weight, float *grad_bias,
+                    void *workspace, size_t workspace_bytes, int64_t N, int Ci, int Co,
+                    pmesh_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -236,3 +236,28 @@ def face_normals(vertex, face):
     p = vertex[_long(face)]
     n = torch.linalg.cross(p[:, 1] - p[:, 0], p[:, 2] - p[:, 0])
     return n / torch.linalg.norm(n, dim=-1, keepdim=True).clamp_min(1e-30)
+
+
+# --------------------------------------------------------------------------
+# pointwise tail of the conv modules  (picasso/mesh/layers.py:114-119, 169-174, 232-238)
+# --------------------------------------------------------------------------
+def dense_tail_fwd(x, w, b=None, relu=True, scale=None, shift=None):
+    """act(x @ w + b) * scale + shift: matmul, bias, activation, then a batch norm that only applies
+    its running statistics (scale = gamma / sqrt(var + eps), shift = beta - mean * scale)."""
+    z = x @ w
+    if b is not None:
+        z = z + b
+    if relu:
+        z = torch.clamp_min(z, 0)
+    if scale is not None:
+        z = z * scale
+    if shift is not None:
+        z = z + shift
+    return z
+
+
+def dense_tail_bwd(gout, x, w, out=None):
+    """Gradients of act(x @ w + b) for (x, w, b); ``out`` is the forward result when act is ReLU
+    (entries with out > 0 pass the gradient), None for no activation."""
+    gz = gout if out is None else torch.where(out > 0, gout, torch.zeros_like(gout))
+    return gz @ w.t(), x.t() @ gz, gz.sum(0)

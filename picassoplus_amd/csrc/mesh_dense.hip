@@ -1,0 +1,396 @@
+// The pointwise tail of the mesh convolutions on the matrix cores (gfx950, v_mfma_f32_32x32x2_f32, fp32
+// operands and accumulators): out = act(rows . W + bias) [* scale + shift], and its gradients.  The
+// reference runs this tail as separate PyTorch ops after every convolution (picasso/mesh/layers.py:114-119,
+// 169-174, 232-238: matmul with depth_weights, + biases, activation, batch norm); here the bias, the ReLU and
+// an inference-mode batch norm ride in the epilogue of the product, and the ReLU mask of the backward pass
+// rides in the operand loads, so every pass touches each feature row once.
+#include "common.h"
+#include "rows_internal.h"
+#include "../../include/picasso_mesh.h"
+
+namespace pmesh {
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+constexpr int kDenseChunk = 64;            // reduction entries per register chunk (32 per lane half)
+constexpr int kDenseSlabFloats = 16384;    // weight slab of one workgroup in LDS (64 KiB, two workgroups per CU)
+constexpr int kDenseMaxK = 1024;          // a 32-column slab of that length is 128 KiB
+
+// rows (N x K, row stride K) times Wm (K x C, element (k, c) at w[k * wk + c * wc]) for the NT * 32 columns
+// from blockIdx.y * NT * 32 on.  A wavefront owns 32 rows: lane (r, h) holds entries h*32 .. h*32+31 of every
+// 64-entry chunk of row r (the order of the reduction index is free as long as both operands agree), so a
+// lane reads 128 contiguous bytes of its row per chunk.  The weight slab sits in LDS as [k/4][column][k%4],
+// one 16-byte read feeds four matrix instructions.  MASK: the row operand is a[r][k] where mask[r][k] > 0,
+// else 0 (the ReLU backward).
+template <int NT, bool VEC, bool MASK>
+__global__ __launch_bounds__(256, 2) void dense_rows_k(const float *__restrict__ a, const float *__restrict__ mask,
+                                                       const float *__restrict__ w, int64_t wk, int64_t wc,
+                                                       const float *__restrict__ bias,
+                                                       const float *__restrict__ scale,
+                                                       const float *__restrict__ shift, int relu,
+                                                       float *__restrict__ out, int64_t N, int K, int Kpad, int C)
+{
+    extern __shared__ __attribute__((aligned(16))) float slab[];
+    constexpr int NC = NT * 32;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int n = lane & 31, h = lane >> 5;
+    const int col0 = blockIdx.y * NC;
+    for (int idx = threadIdx.x; idx < Kpad * NC; idx += 256) {
+        const int k = idx / NC, c = idx - k * NC;
+        const float v = (k < K && col0 + c < C) ? w[(int64_t)k * wk + (int64_t)(col0 + c) * wc] : 0.f;
+        slab[((k >> 2) * NC + c) * 4 + (k & 3)] = v;
+    }
+    __syncthreads();
+    float bia[NT], scl[NT], shf[NT];
+#pragma unroll
+    for (int j = 0; j < NT; ++j) {
+        const int c = col0 + j * 32 + n;
+        bia[j] = (bias && c < C) ? bias[c] : 0.f;
+        scl[j] = (scale && c < C) ? scale[c] : 1.f;
+        shf[j] = (shift && c < C) ? shift[c] : 0.f;
+    }
+    const int64_t ntiles = (N + 31) / 32;
+    for (int64_t tile = (int64_t)blockIdx.x * 4 + wave; tile < ntiles; tile += (int64_t)gridDim.x * 4) {
+        const int64_t row = tile * 32 + n;
+        const bool live = row < N;
+        const float *ap = a + row * K;
+        const float *mp = MASK ? mask + row * K : nullptr;
+        f32x16 acc[NT];
+#pragma unroll
+        for (int j = 0; j < NT; ++j)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) acc[j][i] = 0.f;
+        for (int q = 0; q < Kpad; q += kDenseChunk) {
+            const int kb = q + h * 32;
+            float xa[32];
+            if constexpr (VEC) {
+#pragma unroll
+                for (int g = 0; g < 8; ++g) {
+                    float4 t = make_float4(0.f, 0.f, 0.f, 0.f);
+                    if (live && kb + 4 * g < K) {
+                        t = *reinterpret_cast<const float4 *>(ap + kb + 4 * g);
+                        if constexpr (MASK) {
+                            const float4 m = *reinterpret_cast<const float4 *>(mp + kb + 4 * g);
+                            t.x = m.x > 0.f ? t.x : 0.f; t.y = m.y > 0.f ? t.y : 0.f;
+                            t.z = m.z > 0.f ? t.z : 0.f; t.w = m.w > 0.f ? t.w : 0.f;
+                        }
+                    }
+                    xa[4 * g] = t.x; xa[4 * g + 1] = t.y; xa[4 * g + 2] = t.z; xa[4 * g + 3] = t.w;
+                }
+            } else {
+#pragma unroll
+                for (int t = 0; t < 32; ++t) {
+                    float v = 0.f;
+                    if (live && kb + t < K) {
+                        v = ap[kb + t];
+                        if constexpr (MASK) v = mp[kb + t] > 0.f ? v : 0.f;
+                    }
+                    xa[t] = v;
+                }
+            }
+            const float *sl = slab + ((size_t)(kb >> 2) * NC + n) * 4;
+#pragma unroll
+            for (int g = 0; g < 8; ++g) {
+#pragma unroll
+                for (int j = 0; j < NT; ++j) {
+                    const float4 b = *reinterpret_cast<const float4 *>(sl + ((size_t)g * NC + j * 32) * 4);
+                    acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(xa[4 * g], b.x, acc[j], 0, 0, 0);
+                    acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(xa[4 * g + 1], b.y, acc[j], 0, 0, 0);
+                    acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(xa[4 * g + 2], b.z, acc[j], 0, 0, 0);
+                    acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(xa[4 * g + 3], b.w, acc[j], 0, 0, 0);
+                }
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < NT; ++j) {
+            const int c = col0 + j * 32 + n;
+            if (c >= C) continue;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const int64_t r = tile * 32 + 8 * (i / 4) + 4 * h + (i % 4);
+                if (r >= N) continue;
+                float v = acc[j][i] + bia[j];
+                if (relu) v = fmaxf(v, 0.f);
+                out[r * C + c] = v * scl[j] + shf[j];
+            }
+        }
+    }
+}
+
+// Weight and bias gradient: gW[ci][co] = sum_rows x[row][ci] * gz[row][co], gb[co] = sum_rows gz[row][co] with
+// gz = g where y > 0 (MASK) or g.  The rows are the reduction index: one matrix instruction consumes two rows
+// (lane half h takes row 2t + h), lane (m, h) supplies TA input channels and TB output channels that lie
+// contiguously in its rows, and a wavefront keeps TA x TB tiles of 32 x 32 sums.  Every workgroup leaves one
+// partial of (Ci + 1) * Co floats (row Ci = bias gradient); blockIdx.y walks the channel chunks.
+template <int TA, int TB, bool VEC, bool MASK>
+__global__ __launch_bounds__(256, 2) void dense_wgrad_k(const float *__restrict__ x, const float *__restrict__ g,
+                                                        const float *__restrict__ y, float *__restrict__ partial,
+                                                        int64_t N, int Ci, int Co, int nA, int64_t rows_per_wave)
+{
+    __shared__ float red[TA * TB * 16 * 64];
+    __shared__ float bred[4][2][32 * TB];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int m = lane & 31, h = lane >> 5;
+    const int chunkA = blockIdx.y % nA, chunkB = blockIdx.y / nA;
+    const int ci0 = chunkA * TA * 32 + m * TA, co0 = chunkB * TB * 32 + m * TB;
+    f32x16 acc[TA][TB];
+#pragma unroll
+    for (int ja = 0; ja < TA; ++ja)
+#pragma unroll
+        for (int jb = 0; jb < TB; ++jb)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) acc[ja][jb][i] = 0.f;
+    float gb[TB];
+#pragma unroll
+    for (int jb = 0; jb < TB; ++jb) gb[jb] = 0.f;
+    const int64_t r0 = ((int64_t)blockIdx.x * 4 + wave) * rows_per_wave;
+    int64_t r1 = r0 + rows_per_wave;
+    if (r1 > N) r1 = N;
+    constexpr int U = 8;
+    for (int64_t base = r0; base < r1; base += 2 * U) {
+        Pack<TA> xa[U];
+        Pack<TB> gz[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int64_t row = base + 2 * u + h;
+            xa[u] = zero_pack<TA>();
+            gz[u] = zero_pack<TB>();
+            if (row < r1) {
+                if constexpr (VEC) {
+                    if (ci0 < Ci) xa[u] = ldp<TA>(x + row * Ci + ci0);
+                    if (co0 < Co) {
+                        gz[u] = ldp<TB>(g + row * Co + co0);
+                        if constexpr (MASK) {
+                            const Pack<TB> yy = ldp<TB>(y + row * Co + co0);
+#pragma unroll
+                            for (int jb = 0; jb < TB; ++jb) gz[u].v[jb] = yy.v[jb] > 0.f ? gz[u].v[jb] : 0.f;
+                        }
+                    }
+                } else {
+#pragma unroll
+                    for (int ja = 0; ja < TA; ++ja)
+                        if (ci0 + ja < Ci) xa[u].v[ja] = x[row * Ci + ci0 + ja];
+#pragma unroll
+                    for (int jb = 0; jb < TB; ++jb)
+                        if (co0 + jb < Co) {
+                            float v = g[row * Co + co0 + jb];
+                            if constexpr (MASK) v = y[row * Co + co0 + jb] > 0.f ? v : 0.f;
+                            gz[u].v[jb] = v;
+                        }
+                }
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+#pragma unroll
+            for (int jb = 0; jb < TB; ++jb) gb[jb] += gz[u].v[jb];
+#pragma unroll
+            for (int ja = 0; ja < TA; ++ja)
+#pragma unroll
+                for (int jb = 0; jb < TB; ++jb)
+                    acc[ja][jb] = __builtin_amdgcn_mfma_f32_32x32x2f32(xa[u].v[ja], gz[u].v[jb], acc[ja][jb], 0, 0, 0);
+        }
+    }
+    // the four wavefronts add up in wavefront order
+    for (int wv = 0; wv < 4; ++wv) {
+        if (wave == wv) {
+#pragma unroll
+            for (int ja = 0; ja < TA; ++ja)
+#pragma unroll
+                for (int jb = 0; jb < TB; ++jb)
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) {
+                        float *p = red + ((ja * TB + jb) * 16 + i) * 64 + lane;
+                        *p = wv == 0 ? acc[ja][jb][i] : *p + acc[ja][jb][i];
+                    }
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int jb = 0; jb < TB; ++jb) bred[wave][h][m * TB + jb] = gb[jb];
+    __syncthreads();
+    float *dst = partial + (size_t)blockIdx.x * (size_t)(Ci + 1) * Co;
+    for (int idx = threadIdx.x; idx < TA * TB * 16 * 64; idx += 256) {
+        const int ln = idx & 63, i = (idx >> 6) & 15, t = idx >> 10;
+        const int ja = t / TB, jb = t - ja * TB;
+        const int mm = 8 * (i / 4) + 4 * (ln >> 5) + (i % 4), nn = ln & 31;
+        const int ci = chunkA * TA * 32 + mm * TA + ja, co = chunkB * TB * 32 + nn * TB + jb;
+        if (ci < Ci && co < Co) dst[(size_t)ci * Co + co] = red[idx];
+    }
+    if (chunkA == 0 && threadIdx.x < 32 * TB) {
+        const int co = chunkB * TB * 32 + threadIdx.x;
+        float s = 0.f;
+#pragma unroll
+        for (int wv = 0; wv < 4; ++wv) s += bred[wv][0][threadIdx.x] + bred[wv][1][threadIdx.x];
+        if (co < Co) dst[(size_t)Ci * Co + co] = s;
+    }
+}
+
+static bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+// Column tiles per workgroup of dense_rows_k: as many as the 64 KiB slab and 8 accumulator tiles allow.
+static int rows_tiles(int Kpad, int C)
+{
+    int nt = 8;
+    while (nt > 1 && (Kpad * nt * 32 > kDenseSlabFloats || (nt / 2) * 32 >= C)) nt >>= 1;
+    return nt;
+}
+
+template <bool VEC, bool MASK>
+static void launch_rows(int NT, dim3 grid, size_t lds, hipStream_t st, const float *a, const float *mask, const float *w,
+                        int64_t wk, int64_t wc, const float *bias, const float *scale, const float *shift, int relu,
+                        float *out, int64_t N, int K, int Kpad, int C)
+{
+#define PM_ROWS(T)                                                                                                       \
+    do {                                                                                                                 \
+        if (lds > 65536)                                                                                                 \
+            (void)hipFuncSetAttribute(reinterpret_cast<const void *>(dense_rows_k<T, VEC, MASK>),                        \
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);                             \
+        dense_rows_k<T, VEC, MASK><<<grid, dim3(256), lds, st>>>(a, mask, w, wk, wc, bias, scale, shift, relu, out, N, \
+                                                                 K, Kpad, C);                                            \
+    } while (0)
+    switch (NT) {
+    case 8: PM_ROWS(8); break;
+    case 4: PM_ROWS(4); break;
+    case 2: PM_ROWS(2); break;
+    default: PM_ROWS(1); break;
+    }
+#undef PM_ROWS
+}
+
+// out (N x C) = act(a' (N x K) . Wm + bias) * scale + shift, a' = a masked by mask > 0 when mask is given.
+static int dense_rows(const char *name, const float *a, const float *mask, const float *w, int64_t wk, int64_t wc,
+                      const float *bias, const float *scale, const float *shift, int relu, float *out, int64_t N, int K,
+                      int C, hipStream_t st)
+{
+    PM_REQUIRE(K > 0 && C > 0 && K <= kDenseMaxK && C <= (1 << 20), "%s: channel counts out of range (%d, %d)", name, K, C);
+    PM_REQUIRE(N * (int64_t)(K > C ? K : C) < (int64_t(1) << 40), "%s: sizes too large", name);
+    const int Kpad = (int)ceil_div(K, kDenseChunk) * kDenseChunk;
+    PM_REQUIRE(Kpad * 32 <= 2 * kDenseSlabFloats, "%s: reduction length too large", name);
+    const int NT = rows_tiles(Kpad, C);
+    const size_t lds = (size_t)Kpad * NT * 32 * sizeof(float);
+    const int64_t ntiles = ceil_div(N, 32);
+    int64_t gx = ceil_div(ntiles, 4);
+    if (gx > 1024) gx = 1024;
+    const dim3 grid((unsigned)gx, (unsigned)ceil_div(C, NT * 32));
+    const bool vec = (K % 4 == 0) && aligned16(a) && (!mask || aligned16(mask));
+    if (vec) {
+        if (mask) launch_rows<true, true>(NT, grid, lds, st, a, mask, w, wk, wc, bias, scale, shift, relu, out, N, K, Kpad, C);
+        else launch_rows<true, false>(NT, grid, lds, st, a, mask, w, wk, wc, bias, scale, shift, relu, out, N, K, Kpad, C);
+    } else {
+        if (mask) launch_rows<false, true>(NT, grid, lds, st, a, mask, w, wk, wc, bias, scale, shift, relu, out, N, K, Kpad, C);
+        else launch_rows<false, false>(NT, grid, lds, st, a, mask, w, wk, wc, bias, scale, shift, relu, out, N, K, Kpad, C);
+    }
+    PM_LAUNCHED(name);
+    return 0;
+}
+
+struct WgradPlan {
+    int ta, tb, nA, nB, G;
+    int64_t rows_per_wave;
+};
+
+static int pick_tiles(int ch)
+{
+    return ch > 64 ? 4 : ch > 32 ? 2 : 1;
+}
+
+static WgradPlan wgrad_plan(int64_t N, int Ci, int Co)
+{
+    WgradPlan p;
+    p.ta = pick_tiles(Ci);
+    p.tb = pick_tiles(Co);
+    if (p.ta * p.tb > 8) p.tb = 2;   // at most 8 accumulator tiles per wavefront
+    p.nA = (int)ceil_div(Ci, p.ta * 32);
+    p.nB = (int)ceil_div(Co, p.tb * 32);
+    int64_t G = ceil_div(N, 4 * 256);   // at least 256 rows per wavefront
+    if (G < 1) G = 1;
+    if (G > 512) G = 512;
+    // keep the partials of wide layers modest: G * (Ci + 1) * Co floats <= 32 Mi floats
+    while (G > 1 && G * (int64_t)(Ci + 1) * Co > (int64_t(1) << 25)) G >>= 1;
+    p.G = (int)G;
+    p.rows_per_wave = ceil_div(ceil_div(N, G * 4), 2) * 2;
+    return p;
+}
+
+template <int TA, int TB>
+static void launch_wgrad(bool vec, bool mask, dim3 grid, hipStream_t st, const float *x, const float *g, const float *y,
+                         float *partial, int64_t N, int Ci, int Co, int nA, int64_t rpw)
+{
+    if (vec) {
+        if (mask) dense_wgrad_k<TA, TB, true, true><<<grid, dim3(256), 0, st>>>(x, g, y, partial, N, Ci, Co, nA, rpw);
+        else dense_wgrad_k<TA, TB, true, false><<<grid, dim3(256), 0, st>>>(x, g, y, partial, N, Ci, Co, nA, rpw);
+    } else {
+        if (mask) dense_wgrad_k<TA, TB, false, true><<<grid, dim3(256), 0, st>>>(x, g, y, partial, N, Ci, Co, nA, rpw);
+        else dense_wgrad_k<TA, TB, false, false><<<grid, dim3(256), 0, st>>>(x, g, y, partial, N, Ci, Co, nA, rpw);
+    }
+}
+
+}  // namespace pmesh
+
+using namespace pmesh;
+
+extern "C" int pmesh_dense_fwd(const float *input, const float *weight, const float *bias, const float *scale,
+                               const float *shift, int relu, float *output, int64_t N, int Ci, int Co,
+                               pmesh_stream_t stream)
+{
+    clear_error();
+    PM_REQUIRE(N >= 0, "dense_fwd: negative size");
+    if (N == 0) return 0;
+    PM_REQUIRE(input && weight && output, "dense_fwd: null pointer");
+    return dense_rows("dense_fwd", input, nullptr, weight, Co, 1, bias, scale, shift, relu, output, N, Ci, Co,
+                      (hipStream_t)stream);
+}
+
+extern "C" size_t pmesh_dense_bwd_workspace_bytes(int64_t N, int Ci, int Co)
+{
+    if (N <= 0 || Ci <= 0 || Co <= 0) return 256;
+    const WgradPlan p = wgrad_plan(N, Ci, Co);
+    return (size_t)p.G * (size_t)(Ci + 1) * Co * sizeof(float) + 256;
+}
+
+extern "C" int pmesh_dense_bwd(const float *grad_output, const float *input, const float *weight, const float *output,
+                               float *grad_input, float *grad_weight, float *grad_bias, void *workspace,
+                               size_t workspace_bytes, int64_t N, int Ci, int Co, pmesh_stream_t stream)
+{
+    clear_error();
+    PM_REQUIRE(N >= 0 && Ci > 0 && Co > 0, "dense_bwd: bad sizes");
+    PM_REQUIRE(grad_weight && grad_bias, "dense_bwd: null gradient pointer");
+    hipStream_t st = (hipStream_t)stream;
+    if (N == 0) {
+        const int rc = reduce_partials(nullptr, grad_weight, 0, Ci * Co, st);
+        return rc ? rc : reduce_partials(nullptr, grad_bias, 0, Co, st);
+    }
+    PM_REQUIRE(grad_output && input && weight && workspace, "dense_bwd: null pointer");
+    PM_REQUIRE((int64_t)Ci * Co <= (int64_t(1) << 24), "dense_bwd: weight too large");
+    if (grad_input) {
+        // grad_input (N x Ci) = gz (N x Co) . W^T: element (k = co, c = ci) of the matrix is weight[ci * Co + co]
+        const int rc = dense_rows("dense_bwd(input)", grad_output, output, weight, 1, Co, nullptr, nullptr, nullptr, 0,
+                                  grad_input, N, Co, Ci, st);
+        if (rc) return rc;
+    }
+    const WgradPlan p = wgrad_plan(N, Ci, Co);
+    const size_t slice = (size_t)(Ci + 1) * Co;
+    PM_REQUIRE(workspace_bytes >= (size_t)p.G * slice * sizeof(float), "dense_bwd: workspace too small (%zu bytes)",
+               workspace_bytes);
+    PM_REQUIRE(N * (int64_t)(Ci > Co ? Ci : Co) < (int64_t(1) << 40), "dense_bwd: sizes too large");
+    float *partial = (float *)workspace;
+    const bool vec = Ci % p.ta == 0 && Co % p.tb == 0 && aligned16(input) && aligned16(grad_output) &&
+                     (!output || aligned16(output));
+    const dim3 grid((unsigned)p.G, (unsigned)(p.nA * p.nB));
+    const bool mask = output != nullptr;
+#define PM_WG(A, B) launch_wgrad<A, B>(vec, mask, grid, st, input, grad_output, output, partial, N, Ci, Co, p.nA, p.rows_per_wave)
+    if (p.ta == 4 && p.tb == 2) PM_WG(4, 2);
+    else if (p.ta == 4 && p.tb == 1) PM_WG(4, 1);
+    else if (p.ta == 2 && p.tb == 4) PM_WG(2, 4);
+    else if (p.ta == 2 && p.tb == 2) PM_WG(2, 2);
+    else if (p.ta == 2 && p.tb == 1) PM_WG(2, 1);
+    else if (p.ta == 1 && p.tb == 4) PM_WG(1, 4);
+    else if (p.ta == 1 && p.tb == 2) PM_WG(1, 2);
+    else PM_WG(1, 1);
+#undef PM_WG
+    PM_LAUNCHED("dense_bwd(weight)");
+    int rc = reduce_partials(partial, grad_weight, p.G, Ci * Co, st, slice);
+    if (rc) return rc;
+    return reduce_partials(partial + (size_t)Ci * Co, grad_bias, p.G, Co, st, slice);
+}

@@ -55,14 +55,14 @@ __device__ __forceinline__ void block_reduce_store(const Pack<V> &acc, float *re
 // slices in a fixed tree order.  One workgroup of 1024 threads covers 16 outputs, so that the few
 // thousand outputs of a filter gradient still spread over the chip.
 __global__ __launch_bounds__(1024) void reduce_partials_k(const float *__restrict__ partial,
-                                                         float *__restrict__ out, int G, int n)
+                                                         float *__restrict__ out, int G, int n, size_t stride)
 {
     __shared__ float red[64][16];
     const int j = threadIdx.x & 15, s = threadIdx.x >> 4;
     const int o = blockIdx.x * 16 + j;
     float sum = 0.f;
     if (o < n)
-        for (int g = s; g < G; g += 64) sum += partial[(size_t)g * n + o];
+        for (int g = s; g < G; g += 64) sum += partial[(size_t)g * stride + o];
     red[s][j] = sum;
     __syncthreads();
 #pragma unroll
@@ -926,9 +926,9 @@ static bool force_valu()
     return e && e[0] == '1';
 }
 
-int reduce_partials(const float *partial, float *out, int G, int n, hipStream_t st)
+int reduce_partials(const float *partial, float *out, int G, int n, hipStream_t st, size_t stride)
 {
-    reduce_partials_k<<<dim3((unsigned)ceil_div(n, 16)), dim3(1024), 0, st>>>(partial, out, G, n);
+    reduce_partials_k<<<dim3((unsigned)ceil_div(n, 16)), dim3(1024), 0, st>>>(partial, out, G, n, stride ? stride : (size_t)n);
     PM_LAUNCHED("reduce_partials");
     return 0;
 }

@@ -5,8 +5,9 @@
 
 namespace pmesh {
 
-// out[i] = sum over the G slices of partial[g*n + i], in a fixed tree order (mesh_rows.hip).
-int reduce_partials(const float *partial, float *out, int G, int n, hipStream_t st);
+// out[i] = sum over the G slices of partial[g*stride + i], in a fixed tree order (mesh_rows.hip); stride 0
+// means densely packed slices of n floats.  G == 0 stores zeros.
+int reduce_partials(const float *partial, float *out, int G, int n, hipStream_t st, size_t stride = 0);
 
 // K == 16 coefficients in 16-byte aligned rows, at least 32 output channels, 32-bit byte offsets into `input`.
 bool f2v_mfma_ok(int64_t Nf, int C, int r, int K, const void *coeff);

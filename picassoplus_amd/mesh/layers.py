@@ -3,9 +3,10 @@
 Class names, constructor and ``forward`` signatures, parameter names, shapes and initialisers
 (and with them the state-dict keys a checkpoint carries) follow the reference so that a network
 written against ``picasso.mesh.layers`` can switch its import.  The three convolutions and the
-pool / unpool ops run in hand-written HIP kernels (``pi_modules``); the channel-mixing matmul,
-bias, activation and batch norm after each convolution stay ordinary PyTorch ops, in the
-reference's order: matmul, bias, activation, then BatchNorm1d(eps=1e-3).
+pool / unpool ops run in hand-written HIP kernels (``pi_modules``), and so does the tail after each
+separable convolution and of ``PerItemConv3d`` -- channel-mixing matmul, bias and ReLU in one pass
+(``pi_modules/dense.py``), in the reference's order: matmul, bias, activation, then
+BatchNorm1d(eps=1e-3), which stays a PyTorch op while it trains.
 """
 from typing import List
 
@@ -13,7 +14,7 @@ import torch
 import torch.nn as nn
 
 from .. import _lib
-from .pi_modules import conv3d, pool3d, unpool3d
+from .pi_modules import conv3d, dense, pool3d, unpool3d
 from .pi_modules._check import stream_of
 
 
@@ -68,6 +69,38 @@ class _ConvTail(nn.Module):
     def _tail(self, outputs):
         outputs = outputs + self.biases
         if self.activation_fn is not None:
+            outputs = self.activation_fn(outputs)
+        if self.with_bn:
+            outputs = self.BatchNorm(outputs)
+        return outputs
+
+    def _frozen_norm(self):
+        """(scale, shift) of the batch norm when it only applies its running statistics, else None."""
+        bn = self.BatchNorm
+        if bn.training or bn.running_mean is None:
+            return None
+        scale = torch.rsqrt(bn.running_var + bn.eps)
+        if bn.weight is not None:
+            scale = scale * bn.weight
+        shift = -bn.running_mean * scale
+        if bn.bias is not None:
+            shift = shift + bn.bias
+        return scale.contiguous(), shift.contiguous()
+
+    def _dense_tail(self, inputs, weights):
+        """``_tail(inputs @ weights)`` with the product, the bias and a ReLU (or no activation) in one
+        native pass; without gradients an inference-mode batch norm rides along as scale/shift.  Any
+        other activation, and batch norm in training mode, run as PyTorch ops on the result."""
+        relu = isinstance(self.activation_fn, nn.ReLU)
+        fused_act = relu or self.activation_fn is None
+        biases = self.biases.reshape(-1)
+        if fused_act and self.with_bn and not torch.is_grad_enabled():
+            frozen = self._frozen_norm()
+            if frozen is not None:
+                return dense.dense_tail_forward(inputs.contiguous(), weights.contiguous(), biases.contiguous(), relu,
+                                                frozen[0], frozen[1])
+        outputs = dense.dense_tail(inputs.contiguous(), weights.contiguous(), biases, relu and fused_act)
+        if not fused_act:
             outputs = self.activation_fn(outputs)
         if self.with_bn:
             outputs = self.BatchNorm(outputs)
@@ -132,7 +165,7 @@ class _SeparableConv(_ConvTail):
         self.biases = nn.Parameter(torch.zeros(1, self.out_channels))
 
     def _mix(self, outputs):
-        return self._tail(torch.matmul(outputs, self.depth_weights))
+        return self._dense_tail(outputs, self.depth_weights)
 
 
 class V2FConv3d(_SeparableConv):
@@ -208,7 +241,7 @@ class PerItemConv3d(_ConvTail):
         self.biases = nn.Parameter(torch.zeros(1, self.out_channels))
 
     def forward(self, inputs):
-        return self._tail(torch.matmul(inputs, self.weights))
+        return self._dense_tail(inputs, self.weights)
 
 
 class GlobalPool3d(nn.Module):

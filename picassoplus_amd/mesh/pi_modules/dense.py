@@ -1,0 +1,95 @@
+"""The pointwise tail that follows every mesh convolution, as one native pass.
+
+The reference writes it with separate PyTorch ops (picasso/mesh/layers.py:114-119, 169-174, 232-238):
+``torch.matmul(outputs, depth_weights) + biases``, the activation, then batch norm.  ``dense_tail``
+computes ``act(input @ weight + bias)`` in one kernel and, without gradients, can also apply an
+inference-mode batch norm as a per-channel ``scale``/``shift``; its backward takes the ReLU mask from
+the saved output, so no pre-activation tensor is kept.
+"""
+import torch
+
+from ... import _lib
+from ._check import F32, check_input, same_device, stream_of, workspace
+
+
+def _dims(input, weight, bias):
+    check_input(input, "input", 2, F32)
+    check_input(weight, "weight", 2, F32)
+    N, Ci = input.shape
+    if weight.shape[0] != Ci:
+        raise RuntimeError("weight must have shape (in_channels, out_channels)")
+    Co = weight.shape[1]
+    if Ci < 1 or Co < 1 or Ci > 1024:
+        raise RuntimeError("dense tail supports 1..1024 input channels, got %d" % Ci)
+    if bias is not None:
+        check_input(bias, "bias", 1, F32)
+        if bias.shape[0] != Co:
+            raise RuntimeError("bias must have out_channels entries")
+    return N, Ci, Co
+
+
+def _ptr(t):
+    return 0 if t is None else t.data_ptr()
+
+
+def dense_tail_forward(input, weight, bias=None, relu=True, scale=None, shift=None):
+    """(N,Ci),(Ci,Co),(Co,) -> act(input @ weight + bias) * scale + shift, float32 (N,Co)."""
+    N, Ci, Co = _dims(input, weight, bias)
+    for name, t in (("scale", scale), ("shift", shift)):
+        if t is not None:
+            check_input(t, name, 1, F32)
+            if t.shape[0] != Co:
+                raise RuntimeError("%s must have out_channels entries" % name)
+    dev = same_device(input, weight, *[t for t in (bias, scale, shift) if t is not None])
+    with torch.cuda.device(dev):
+        out = torch.empty((N, Co), dtype=F32, device=dev)
+        _lib.call("pmesh_dense_fwd", input.data_ptr(), weight.data_ptr(), _ptr(bias), _ptr(scale), _ptr(shift),
+                  1 if relu else 0, out.data_ptr(), N, Ci, Co, stream_of(input))
+    return out
+
+
+def dense_tail_backward(grad_output, input, weight, output=None, need_input=True):
+    """Gradients of ``act(input @ weight + bias)``: ``output`` is the forward result when the activation
+    was ReLU (its positive entries pass the gradient), None for no activation.
+    -> [grad_input (N,Ci) or None, grad_weight (Ci,Co), grad_bias (Co,)]."""
+    N, Ci, Co = _dims(input, weight, None)
+    check_input(grad_output, "grad_output", 2, F32)
+    if tuple(grad_output.shape) != (N, Co):
+        raise RuntimeError("grad_output must have shape (N, out_channels)")
+    if output is not None:
+        check_input(output, "output", 2, F32)
+        if tuple(output.shape) != (N, Co):
+            raise RuntimeError("output must have shape (N, out_channels)")
+    dev = same_device(grad_output, input, weight)
+    with torch.cuda.device(dev):
+        gin = torch.empty((N, Ci), dtype=F32, device=dev) if need_input else None
+        gw = torch.empty((Ci, Co), dtype=F32, device=dev)
+        gb = torch.empty((Co,), dtype=F32, device=dev)
+        nbytes = _lib.query("pmesh_dense_bwd_workspace_bytes", N, Ci, Co)
+        ws = workspace(nbytes, dev)
+        _lib.call("pmesh_dense_bwd", grad_output.data_ptr(), input.data_ptr(), weight.data_ptr(), _ptr(output),
+                  _ptr(gin), gw.data_ptr(), gb.data_ptr(), ws.data_ptr(), nbytes, N, Ci, Co, stream_of(input))
+    return [gin, gw, gb]
+
+
+class DenseTailFunction(torch.autograd.Function):
+    """autograd Function of dense_tail: gradients for input, weight and bias."""
+
+    @staticmethod
+    def forward(ctx, input, weight, bias, relu):
+        out = dense_tail_forward(input, weight, bias, relu)
+        ctx.relu = bool(relu)
+        ctx.save_for_backward(input, weight, out if relu else None)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        input, weight, out = ctx.saved_tensors
+        gin, gw, gb = dense_tail_backward(grad_output.contiguous(), input, weight, out if ctx.relu else None,
+                                          need_input=ctx.needs_input_grad[0])
+        return gin, gw if ctx.needs_input_grad[1] else None, gb if ctx.needs_input_grad[2] else None, None
+
+
+def dense_tail(input, weight, bias, relu=True):
+    """act(input @ weight + bias) with gradients; ``bias`` (Co,) float32."""
+    return DenseTailFunction.apply(input, weight, bias, relu)

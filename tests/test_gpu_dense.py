@@ -1,0 +1,165 @@
+"""Parity of the native pointwise tail (matmul + bias + ReLU [+ frozen batch norm] and its gradients) with the
+float64 oracle (oracle/torch_ref.py: dense_tail_fwd / dense_tail_bwd), through the Python ops and the modules
+that use it.  Bar: within 1e-5 of max |reference|."""
+import sys
+
+import numpy as np
+import pytest
+import torch
+import torch.nn as nn
+
+from oracle import torch_ref
+from picassoplus_amd.mesh import layers
+from picassoplus_amd.mesh.pi_modules import dense
+from util import assert_close
+
+pytestmark = pytest.mark.gpu
+
+
+def say(*a):
+    print(*a, flush=True)
+    sys.stdout.flush()
+
+
+SHAPES = [(1, 1, 1), (33, 3, 13), (64, 8, 32), (1000, 64, 64), (257, 96, 20), (70, 130, 257), (4099, 128, 128),
+          (100, 1024, 40), (300, 256, 256), (515, 36, 64), (2048, 32, 96), (129, 448, 128), (95, 6, 5)]
+
+
+def _case(seed, n, ci, co):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(n, ci, dtype=torch.float64, generator=g)
+    w = torch.randn(ci, co, dtype=torch.float64, generator=g) / np.sqrt(ci)
+    b = torch.randn(co, dtype=torch.float64, generator=g)
+    go = torch.randn(n, co, dtype=torch.float64, generator=g)
+    return x, w, b, go
+
+
+@pytest.mark.parametrize("n,ci,co", SHAPES)
+@pytest.mark.parametrize("relu", [True, False])
+def test_dense_tail_forward_backward(cuda, n, ci, co, relu):
+    say("case dense_tail", n, ci, co, relu)
+    x, w, b, go = _case(n + ci, n, ci, co)
+    f = lambda t: t.to(cuda, torch.float32).contiguous()
+    xd, wd, bd, god = f(x), f(w), f(b), f(go)
+    # the oracle sees the float32-rounded operands, so the mask of the ReLU is the same one
+    x, w, b, go = xd.double().cpu(), wd.double().cpu(), bd.double().cpu(), god.double().cpu()
+    out = dense.dense_tail_forward(xd, wd, bd, relu)
+    ref = torch_ref.dense_tail_fwd(x, w, b, relu)
+    torch.cuda.synchronize()
+    assert_close(out, ref.numpy(), "dense forward")
+    # entries whose float64 pre-activation is within rounding of zero may land on either side of the ReLU
+    z = x @ w + b
+    safe = (z.abs() > 1e-5 * z.abs().max()) | (not relu)
+    out64 = torch.where(safe, ref, out.double().cpu())
+    gx, gw, gb = dense.dense_tail_backward(god, xd, wd, out if relu else None)
+    rx, rw, rb = torch_ref.dense_tail_bwd(go, x, w, out64 if relu else None)
+    torch.cuda.synchronize()
+    assert_close(gx, rx.numpy(), "dense grad_input")
+    assert_close(gw, rw.numpy(), "dense grad_weight")
+    assert_close(gb, rb.numpy(), "dense grad_bias")
+    gx2, gw2, gb2 = dense.dense_tail_backward(god, xd, wd, out if relu else None, need_input=False)
+    torch.cuda.synchronize()
+    assert gx2 is None and torch.equal(gw2, gw) and torch.equal(gb2, gb)
+
+
+def test_dense_tail_frozen_norm_and_missing_operands(cuda):
+    say("case dense_tail frozen norm")
+    x, w, b, _ = _case(5, 777, 64, 48)
+    g = torch.Generator().manual_seed(6)
+    scale = torch.randn(48, dtype=torch.float64, generator=g)
+    shift = torch.randn(48, dtype=torch.float64, generator=g)
+    f = lambda t: t.to(cuda, torch.float32).contiguous()
+    xd, wd, bd, sd, hd = f(x), f(w), f(b), f(scale), f(shift)
+    x, w, b, scale, shift = (t.double().cpu() for t in (xd, wd, bd, sd, hd))
+    assert_close(dense.dense_tail_forward(xd, wd, bd, True, sd, hd),
+                 torch_ref.dense_tail_fwd(x, w, b, True, scale, shift).numpy(), "relu + scale/shift")
+    assert_close(dense.dense_tail_forward(xd, wd, None, False, sd, None),
+                 torch_ref.dense_tail_fwd(x, w, None, False, scale, None).numpy(), "scale only")
+    assert_close(dense.dense_tail_forward(xd, wd, None, False),
+                 (x @ w).numpy(), "plain product")
+
+
+def test_dense_tail_unaligned_rows_and_empty(cuda):
+    say("case dense_tail unaligned / empty")
+    x, w, b, go = _case(9, 301, 64, 64)
+    f = lambda t: t.to(cuda, torch.float32).contiguous()
+    # a view one float past an aligned base: rows are 4-byte aligned only
+    flat = torch.empty(301 * 64 + 1, dtype=torch.float32, device=cuda)
+    xd = flat[1:].view(301, 64)
+    xd.copy_(f(x))
+    assert xd.data_ptr() % 16 == 4 and xd.is_contiguous()
+    wd, bd, god = f(w), f(b), f(go)
+    x, w, b, go = (t.double().cpu() for t in (xd, wd, bd, god))
+    out = dense.dense_tail_forward(xd, wd, bd, False)
+    assert_close(out, torch_ref.dense_tail_fwd(x, w, b, False).numpy(), "unaligned forward")
+    gx, gw, gb = dense.dense_tail_backward(god, xd, wd, None)
+    rx, rw, rb = torch_ref.dense_tail_bwd(go, x, w, None)
+    assert_close(gx, rx.numpy(), "unaligned grad_input")
+    assert_close(gw, rw.numpy(), "unaligned grad_weight")
+    assert_close(gb, rb.numpy(), "unaligned grad_bias")
+    e = torch.empty(0, 64, device=cuda)
+    assert dense.dense_tail_forward(e, wd, bd, True).shape == (0, 64)
+    gx, gw, gb = dense.dense_tail_backward(torch.empty(0, 64, device=cuda), e, wd, None)
+    torch.cuda.synchronize()
+    assert gx.shape == (0, 64) and float(gw.abs().max()) == 0.0 and float(gb.abs().max()) == 0.0
+    with pytest.raises(RuntimeError):
+        dense.dense_tail_forward(xd, wd[:32].contiguous(), bd, True)
+    with pytest.raises(RuntimeError):
+        dense.dense_tail_forward(torch.randn(4, 1025, device=cuda), torch.randn(1025, 8, device=cuda), None, True)
+
+
+def test_dense_tail_is_deterministic(cuda):
+    say("case dense_tail deterministic")
+    x, w, b, go = _case(13, 20000, 64, 64)
+    f = lambda t: t.to(cuda, torch.float32).contiguous()
+    xd, wd, bd, god = f(x), f(w), f(b), f(go)
+    out = dense.dense_tail_forward(xd, wd, bd, True)
+    a = dense.dense_tail_backward(god, xd, wd, out)
+    for _ in range(3):
+        bgrads = dense.dense_tail_backward(god, xd, wd, out)
+        assert all(torch.equal(p, q) for p, q in zip(a, bgrads))
+
+
+@pytest.mark.parametrize("act", ["relu", "none", "tanh"])
+@pytest.mark.parametrize("with_bn", [True, False])
+def test_per_item_module_train_and_eval(cuda, act, with_bn):
+    """PerItemConv3d (picasso/mesh/layers.py:198-239) against the same composition in float64: training mode
+    with gradients, then evaluation mode without (frozen batch norm inside the native pass)."""
+    say("case per_item module", act, with_bn)
+    torch.manual_seed(17)
+    fn = {"relu": nn.ReLU(), "none": None, "tanh": nn.Tanh()}[act]
+    mod = layers.PerItemConv3d(24, 40, activation_fn=fn, with_bn=with_bn).to(cuda).train()
+    with torch.no_grad():
+        mod.biases.add_(0.1 * torch.randn_like(mod.biases))
+    import copy
+    mod64 = copy.deepcopy(mod).cpu().double().train()
+    x = torch.randn(333, 24)
+    g = torch.randn(333, 40)
+
+    def ref(m, t):
+        y = t @ m.weights + m.biases
+        if m.activation_fn is not None:
+            y = m.activation_fn(y)
+        return m.BatchNorm(y) if m.with_bn else y
+
+    xg = x.to(cuda).requires_grad_(True)
+    out = mod(xg)
+    out.backward(g.to(cuda))
+    x64 = x.double().requires_grad_(True)
+    y = ref(mod64, x64)
+    y.backward(g.double())
+    torch.cuda.synchronize()
+    assert_close(out, y.detach().numpy(), "PerItemConv3d output", 2e-5)
+    assert_close(xg.grad, x64.grad.numpy(), "PerItemConv3d grad_input", 2e-5)
+    for (n, p), (_, q) in zip(mod.named_parameters(), mod64.named_parameters()):
+        if n == "biases" and with_bn and fn is None:
+            # a batch norm straight after the bias removes it: the exact gradient is zero
+            assert float(p.grad.abs().max()) < 1e-3 and float(q.grad.abs().max()) < 1e-9
+            continue
+        assert_close(p.grad, q.grad.numpy(), "grad of " + n, 2e-5)
+    mod.eval(); mod64.eval()
+    with torch.no_grad():
+        assert_close(mod(x.to(cuda)), ref(mod64, x.double()).numpy(), "PerItemConv3d eval output", 2e-5)
+    # evaluation mode with gradients enabled keeps the batch norm outside the native pass and still agrees
+    xg2 = x.to(cuda).requires_grad_(True)
+    assert_close(mod(xg2), ref(mod64, x.double()).detach().numpy(), "PerItemConv3d eval output (grad mode)", 2e-5)

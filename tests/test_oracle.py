@@ -312,3 +312,44 @@ def test_float32_loops_close_to_float64():
     xf, fl, cf = rng.normal(size=(nf, C)), rng.normal(size=(K, C, 1)), rng.normal(size=(nf, K))
     a = loops.f2v_fwd(xf, fl, cf, f, nfc, ident, dtype=np.float32)
     assert a.dtype == np.float32 and rel_err(a, loops.f2v_fwd(xf, fl, cf, f, nfc, ident)) < 1e-5
+
+
+def test_dense_tail_matches_torch_layers_and_hand_values():
+    """The tail restatement against nn.Linear + ReLU + BatchNorm1d in eval mode (an independent spelling of
+    layers.py:114-119 with torch's own modules), its explicit gradients against autograd, and a case worked by
+    hand."""
+    g = torch.Generator().manual_seed(11)
+    x = torch.randn(37, 5, dtype=torch.float64, generator=g)
+    lin = torch.nn.Linear(5, 7).double()
+    bn = torch.nn.BatchNorm1d(7, eps=1e-3).double()
+    with torch.no_grad():
+        bn.running_mean.copy_(torch.randn(7, dtype=torch.float64, generator=g))
+        bn.running_var.copy_(torch.rand(7, dtype=torch.float64, generator=g) + 0.5)
+        bn.weight.copy_(torch.randn(7, dtype=torch.float64, generator=g))
+        bn.bias.copy_(torch.randn(7, dtype=torch.float64, generator=g))
+    bn.eval()
+    w, b = lin.weight.detach().t().contiguous(), lin.bias.detach()
+    scale = bn.weight.detach() / torch.sqrt(bn.running_var + bn.eps)
+    shift = bn.bias.detach() - bn.running_mean * scale
+    want = bn(torch.relu(lin(x))).detach()
+    assert rel_err(torch_ref.dense_tail_fwd(x, w, b, True, scale, shift).numpy(), want.numpy()) < 1e-13
+    assert rel_err(torch_ref.dense_tail_fwd(x, w, b, False).numpy(), lin(x).detach().numpy()) < 1e-13
+    for relu in (True, False):
+        xg = x.clone().requires_grad_(True)
+        lin.zero_grad()
+        y = torch.relu(lin(xg)) if relu else lin(xg)
+        go = torch.randn(y.shape, dtype=torch.float64, generator=g)
+        y.backward(go)
+        gx, gw, gb = torch_ref.dense_tail_bwd(go, x, w, y.detach() if relu else None)
+        assert rel_err(gx.numpy(), xg.grad.numpy()) < 1e-13
+        assert rel_err(gw.numpy(), lin.weight.grad.t().numpy()) < 1e-13
+        assert rel_err(gb.numpy(), lin.bias.grad.numpy()) < 1e-13
+    x2 = torch.tensor([[1.0, 2.0], [-1.0, 0.5]], dtype=torch.float64)
+    w2 = torch.tensor([[1.0, -1.0, 0.0], [0.5, 1.0, 2.0]], dtype=torch.float64)
+    b2 = torch.tensor([0.0, -2.0, 1.0], dtype=torch.float64)
+    assert torch_ref.dense_tail_fwd(x2, w2, b2, True).tolist() == [[2.0, 0.0, 5.0], [0.0, 0.0, 2.0]]
+    go2 = torch.ones(2, 3, dtype=torch.float64)
+    gx2, gw2, gb2 = torch_ref.dense_tail_bwd(go2, x2, w2, torch_ref.dense_tail_fwd(x2, w2, b2, True))
+    assert gx2.tolist() == [[1.0, 2.5], [0.0, 2.0]]
+    assert gw2.tolist() == [[1.0, 0.0, 0.0], [2.0, 0.0, 2.5]]
+    assert gb2.tolist() == [1.0, 0.0, 2.0]

@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the mesh-conv hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload scene|shapes|pool] [--scale S]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload scene|shapes|pool|firstblock|tail] [--scale S]
 
 A step is one forward+backward pass of the layer over one batch of seeded synthetic meshes
 already resident in HBM.  Default workload ``scene``: 8 room-like meshes of about 300 k
@@ -37,7 +37,7 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="scene", choices=["scene", "shapes", "pool", "firstblock"],
+    ap.add_argument("--workload", default="scene", choices=["scene", "shapes", "pool", "firstblock", "tail"],
                     help="scene: the headline layer (F2F+F2V, C=64); shapes: 16 small meshes V2F+F2F+F2V; pool: "
                          "1024x1024 grid max/avg pool + unpool; firstblock: the scene batch with the reference's first "
                          "block shapes, F2F 3->32 then F2V 32->32 with depth multiplier 2 (pi2_blocks.py:113-130)")
@@ -296,6 +296,67 @@ def run_pool(args, torch):
                 config=dict(workload="plane1024_pool_max+avg+unpool_C128_fp32_fwd+bwd", vertices=nv, coarse=nvo, channels=C))
 
 
+def run_tail(args, torch):
+    """The pointwise tail of a convolution on the scene batch's facet rows: act(rows @ W + b), 64 -> 64 channels,
+    forward and backward (input, weight and bias gradients)."""
+    from picassoplus_amd import _lib
+    from picassoplus_amd.mesh.pi_modules import dense
+    dev = torch.device("cuda:0")
+    N, Ci, Co = int(2_400_000 * args.scale), 64, 64
+    gen = torch.Generator(device=dev).manual_seed(5000)
+    x = torch.randn(N, Ci, device=dev, generator=gen).requires_grad_(True)
+    w = (torch.randn(Ci, Co, device=dev, generator=gen) / 8).requires_grad_(True)
+    b = torch.randn(Co, device=dev, generator=gen).requires_grad_(True)
+    g = torch.randn(N, Co, device=dev, generator=gen)
+
+    def step():
+        y = dense.dense_tail(x, w, b, True)
+        return torch.autograd.grad(y, [x, w, b], g)
+
+    timer = EventTimer(torch)
+    _lib.set_call_hook(timer)
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    timer.on = True
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    _lib.set_call_hook(None)
+    per_op = timer.summary()
+    nb = {"dense_fwd": 4 * N * (Ci + Co), "dense_bwd": 4 * N * (2 * Co + Ci) + 4 * N * Ci}
+    fl = {"dense_fwd": 2.0 * N * Ci * Co, "dense_bwd": 4.0 * N * Ci * Co}
+    dom = max(nb, key=lambda k: per_op[k])
+    ach = nb[dom] / (per_op[dom] * 1e-3) / 1e9
+    total = sum(nb.values())
+    extra = {}
+    if not args.no_cpu_baseline:
+        # the oracle's restatement (float32 PyTorch-CPU ops) on slices of the same rows until about 10 s are spent
+        from oracle import torch_ref as R
+        torch.set_num_threads(os.cpu_count() or 1)
+        xc, wc, bc, gc = x.detach().cpu(), w.detach().cpu(), b.detach().cpu(), g.cpu()
+        rows = spent = 0
+        chunk = 200_000
+        while spent < 10.0 and rows + chunk <= N:
+            xs, gs = xc[rows:rows + chunk], gc[rows:rows + chunk]
+            t0 = time.perf_counter()
+            R.dense_tail_bwd(gs, xs, wc, R.dense_tail_fwd(xs, wc, bc, True))
+            spent += time.perf_counter() - t0
+            rows += chunk
+        extra["cpu_baseline"] = dict(value=rows / spent / 1e6, unit="Mrows/s", cores=torch.get_num_threads(), kind="port",
+                                     sample="first %d of %d rows, one fwd+bwd pass, %.1f s" % (rows, N, spent))
+    return dict(value=N / (ms * 1e-3) / 1e6, unit="Mrows/s", ms_per_step=ms, **extra,
+                roofline=dict(bound="hbm", achieved=ach, peak=HBM_PEAK_GBS, unit="GB/s", frac=ach / HBM_PEAK_GBS,
+                              traffic=None, kernel=dom, kernel_ms=per_op[dom]),
+                ops={k: dict(ms=per_op[k], gbps=nb[k] / (per_op[k] * 1e-3) / 1e9,
+                             tflops=fl[k] / (per_op[k] * 1e-3) / 1e12) for k in nb},
+                hbm_gbps=total / (ms * 1e-3) / 1e9, hbm_frac=total / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                config=dict(workload="scene_rows_dense_tail_64to64_relu_fp32_fwd+bwd", rows=N, in_channels=Ci,
+                            out_channels=Co))
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -309,7 +370,12 @@ def main():
         print("bench.py needs a GPU (torch.cuda.is_available() is False)", file=sys.stderr)
         sys.exit(2)
     torch.cuda.set_device(0)
-    res = run_pool(args, torch) if args.workload == "pool" else run_conv_layer(args, torch, args.workload)
+    if args.workload == "pool":
+        res = run_pool(args, torch)
+    elif args.workload == "tail":
+        res = run_tail(args, torch)
+    else:
+        res = run_conv_layer(args, torch, args.workload)
     if args.copy_calibration:
         src = torch.empty(1 << 28, dtype=torch.float32, device="cuda:0").normal_()
         dst = torch.empty_like(src)

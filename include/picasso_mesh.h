@@ -212,7 +212,7 @@ int pmesh_triangle_geometry(const float *vertex, const int32_t *face, float *geo
  * 232-238: torch.matmul(outputs, depth_weights) + biases, activation_fn, BatchNorm) by one pass:
  *   output (N,Co) = act(input (N,Ci) . weight (Ci,Co) + bias (Co)) * scale (Co) + shift (Co)
  * relu != 0 selects max(.,0), else identity; bias, scale, shift may be NULL (0, 1, 0): scale/shift carry
- * an inference-mode batch norm (gamma/sqrt(var+eps), beta - mean*that).  Ci <= 1024.
+ * an inference-mode batch norm (gamma/sqrt(var+eps), beta - mean*that).  Ci <= 896.
  * pmesh_dense_bwd is the gradient of the tail without scale/shift (training-mode batch norm stays
  * outside): gz = grad_output where output > 0 (output = the forward result, NULL when relu was off);
  * grad_input (N,Ci) = gz . weight^T (NULL skips it), grad_weight (Ci,Co) = input^T . gz,

@@ -13,15 +13,77 @@ namespace pmesh {
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 constexpr int kDenseChunk = 64;            // reduction entries per register chunk (32 per lane half)
-constexpr int kDenseSlabFloats = 16384;    // weight slab of one workgroup in LDS (64 KiB, two workgroups per CU)
-constexpr int kDenseMaxK = 1024;          // a 32-column slab of that length is 128 KiB
+constexpr int kDenseSlabFloats = 12288;    // preferred weight slab of one workgroup in LDS (48 KiB)
+constexpr int kDenseMaxK = 896;            // a 32-column slab of that length is 112 KiB, beside 34 KiB of row stages
 
 // rows (N x K, row stride K) times Wm (K x C, element (k, c) at w[k * wk + c * wc]) for the NT * 32 columns
-// from blockIdx.y * NT * 32 on.  A wavefront owns 32 rows: lane (r, h) holds entries h*32 .. h*32+31 of every
-// 64-entry chunk of row r (the order of the reduction index is free as long as both operands agree), so a
-// lane reads 128 contiguous bytes of its row per chunk.  The weight slab sits in LDS as [k/4][column][k%4],
-// one 16-byte read feeds four matrix instructions.  MASK: the row operand is a[r][k] where mask[r][k] > 0,
-// else 0 (the ReLU backward).
+// from blockIdx.y * NT * 32 on.  A wavefront owns 32 rows at a time.  It fetches a 32 x 64 block of them with
+// fully coalesced loads (a 16-lane group per row), one block ahead of the arithmetic, and turns it into the
+// operand layout of the matrix instruction (lane = row) through a private LDS stage: lane (r, h) reads entries
+// h*32 .. h*32+31 of row r (the order of the reduction index is free as long as both operands agree).  The
+// weight slab sits in LDS as [k/4][column][k%4], one 16-byte read feeds four matrix instructions.  MASK: the
+// row operand is a[r][k] where mask[r][k] > 0, else 0 (the ReLU backward).
+constexpr int kStageStride = 68;                       // floats per staged row: 16-byte reads of 32 rows hit all banks
+constexpr int kStageFloats = 4 * 32 * kStageStride;    // four wavefronts
+
+template <bool VEC, bool MASK> struct RowBlock {
+    float v[32];
+    float m[MASK ? 32 : 1];
+};
+
+template <bool VEC, bool MASK>
+__device__ __forceinline__ void rows_issue(RowBlock<VEC, MASK> &b, const float *__restrict__ a,
+                                           const float *__restrict__ mask, int64_t tile, int q, int64_t N, int K,
+                                           int lane)
+{
+    if constexpr (VEC) {
+        const int col = q + 4 * (lane & 15);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int64_t row = tile * 32 + 4 * i + (lane >> 4);
+            float4 t = make_float4(0.f, 0.f, 0.f, 0.f), mm = make_float4(1.f, 1.f, 1.f, 1.f);
+            if (row < N && col < K) {
+                t = *reinterpret_cast<const float4 *>(a + row * K + col);
+                if constexpr (MASK) mm = *reinterpret_cast<const float4 *>(mask + row * K + col);
+            }
+            b.v[4 * i] = t.x; b.v[4 * i + 1] = t.y; b.v[4 * i + 2] = t.z; b.v[4 * i + 3] = t.w;
+            if constexpr (MASK) { b.m[4 * i] = mm.x; b.m[4 * i + 1] = mm.y; b.m[4 * i + 2] = mm.z; b.m[4 * i + 3] = mm.w; }
+        }
+    } else {
+        const int col = q + lane;
+#pragma unroll
+        for (int i = 0; i < 32; ++i) {
+            const int64_t row = tile * 32 + i;
+            const bool ok = row < N && col < K;
+            b.v[i] = ok ? a[row * K + col] : 0.f;
+            if constexpr (MASK) b.m[i] = ok ? mask[row * K + col] : 1.f;
+        }
+    }
+}
+
+template <bool VEC, bool MASK>
+__device__ __forceinline__ void rows_commit(const RowBlock<VEC, MASK> &b, float *stage, int lane)
+{
+    if constexpr (VEC) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            float4 t = make_float4(b.v[4 * i], b.v[4 * i + 1], b.v[4 * i + 2], b.v[4 * i + 3]);
+            if constexpr (MASK) {
+                t.x = b.m[4 * i] > 0.f ? t.x : 0.f; t.y = b.m[4 * i + 1] > 0.f ? t.y : 0.f;
+                t.z = b.m[4 * i + 2] > 0.f ? t.z : 0.f; t.w = b.m[4 * i + 3] > 0.f ? t.w : 0.f;
+            }
+            *reinterpret_cast<float4 *>(stage + (4 * i + (lane >> 4)) * kStageStride + 4 * (lane & 15)) = t;
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 32; ++i) {
+            float t = b.v[i];
+            if constexpr (MASK) t = b.m[i] > 0.f ? t : 0.f;
+            stage[i * kStageStride + lane] = t;
+        }
+    }
+}
+
 template <int NT, bool VEC, bool MASK>
 __global__ __launch_bounds__(256, 2) void dense_rows_k(const float *__restrict__ a, const float *__restrict__ mask,
                                                        const float *__restrict__ w, int64_t wk, int64_t wc,
@@ -30,11 +92,13 @@ __global__ __launch_bounds__(256, 2) void dense_rows_k(const float *__restrict__
                                                        const float *__restrict__ shift, int relu,
                                                        float *__restrict__ out, int64_t N, int K, int Kpad, int C)
 {
-    extern __shared__ __attribute__((aligned(16))) float slab[];
+    extern __shared__ __attribute__((aligned(16))) float lds[];
     constexpr int NC = NT * 32;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int n = lane & 31, h = lane >> 5;
     const int col0 = blockIdx.y * NC;
+    float *slab = lds + kStageFloats;
+    float *stage = lds + wave * (32 * kStageStride);
     for (int idx = threadIdx.x; idx < Kpad * NC; idx += 256) {
         const int k = idx / NC, c = idx - k * NC;
         const float v = (k < K && col0 + c < C) ? w[(int64_t)k * wk + (int64_t)(col0 + c) * wc] : 0.f;
@@ -49,70 +113,99 @@ __global__ __launch_bounds__(256, 2) void dense_rows_k(const float *__restrict__
         scl[j] = (scale && c < C) ? scale[c] : 1.f;
         shf[j] = (shift && c < C) ? shift[c] : 0.f;
     }
-    const int64_t ntiles = (N + 31) / 32;
-    for (int64_t tile = (int64_t)blockIdx.x * 4 + wave; tile < ntiles; tile += (int64_t)gridDim.x * 4) {
-        const int64_t row = tile * 32 + n;
-        const bool live = row < N;
-        const float *ap = a + row * K;
-        const float *mp = MASK ? mask + row * K : nullptr;
-        f32x16 acc[NT];
+    const int64_t ntiles = (N + 31) / 32, stride = (int64_t)gridDim.x * 4;
+    int64_t tile = (int64_t)blockIdx.x * 4 + wave;
+    int q = 0;
+    bool have = tile < ntiles;
+    RowBlock<VEC, MASK> blk;
+    if (have) rows_issue<VEC, MASK>(blk, a, mask, tile, 0, N, K, lane);
+    f32x16 acc[NT];
 #pragma unroll
-        for (int j = 0; j < NT; ++j)
+    for (int j = 0; j < NT; ++j)
 #pragma unroll
-            for (int i = 0; i < 16; ++i) acc[j][i] = 0.f;
-        for (int q = 0; q < Kpad; q += kDenseChunk) {
-            const int kb = q + h * 32;
-            float xa[32];
-            if constexpr (VEC) {
+        for (int i = 0; i < 16; ++i) acc[j][i] = 0.f;
+    while (have) {
+        rows_commit<VEC, MASK>(blk, stage, lane);
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        int64_t ntile = tile;
+        int nq = q + kDenseChunk;
+        if (nq >= Kpad) { nq = 0; ntile += stride; }
+        const bool nhave = ntile < ntiles;
+        if (nhave) rows_issue<VEC, MASK>(blk, a, mask, ntile, nq, N, K, lane);
+        const float *xs = stage + n * kStageStride + h * 32;
+        const float *sl = slab + ((size_t)((q + h * 32) >> 2) * NC + n) * 4;
 #pragma unroll
-                for (int g = 0; g < 8; ++g) {
-                    float4 t = make_float4(0.f, 0.f, 0.f, 0.f);
-                    if (live && kb + 4 * g < K) {
-                        t = *reinterpret_cast<const float4 *>(ap + kb + 4 * g);
-                        if constexpr (MASK) {
-                            const float4 m = *reinterpret_cast<const float4 *>(mp + kb + 4 * g);
-                            t.x = m.x > 0.f ? t.x : 0.f; t.y = m.y > 0.f ? t.y : 0.f;
-                            t.z = m.z > 0.f ? t.z : 0.f; t.w = m.w > 0.f ? t.w : 0.f;
-                        }
-                    }
-                    xa[4 * g] = t.x; xa[4 * g + 1] = t.y; xa[4 * g + 2] = t.z; xa[4 * g + 3] = t.w;
-                }
-            } else {
+        for (int g = 0; g < 8; ++g) {
+            const float4 x4 = *reinterpret_cast<const float4 *>(xs + 4 * g);
 #pragma unroll
-                for (int t = 0; t < 32; ++t) {
-                    float v = 0.f;
-                    if (live && kb + t < K) {
-                        v = ap[kb + t];
-                        if constexpr (MASK) v = mp[kb + t] > 0.f ? v : 0.f;
-                    }
-                    xa[t] = v;
-                }
+            for (int j = 0; j < NT; ++j) {
+                const float4 b = *reinterpret_cast<const float4 *>(sl + ((size_t)g * NC + j * 32) * 4);
+                acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(x4.x, b.x, acc[j], 0, 0, 0);
+                acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(x4.y, b.y, acc[j], 0, 0, 0);
+                acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(x4.z, b.z, acc[j], 0, 0, 0);
+                acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(x4.w, b.w, acc[j], 0, 0, 0);
             }
-            const float *sl = slab + ((size_t)(kb >> 2) * NC + n) * 4;
+        }
+        __builtin_amdgcn_wave_barrier();
+        if (q + kDenseChunk >= Kpad) {
 #pragma unroll
-            for (int g = 0; g < 8; ++g) {
+            for (int j = 0; j < NT; ++j) {
+                const int c = col0 + j * 32 + n;
 #pragma unroll
-                for (int j = 0; j < NT; ++j) {
-                    const float4 b = *reinterpret_cast<const float4 *>(sl + ((size_t)g * NC + j * 32) * 4);
-                    acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(xa[4 * g], b.x, acc[j], 0, 0, 0);
-                    acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(xa[4 * g + 1], b.y, acc[j], 0, 0, 0);
-                    acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(xa[4 * g + 2], b.z, acc[j], 0, 0, 0);
-                    acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(xa[4 * g + 3], b.w, acc[j], 0, 0, 0);
+                for (int i = 0; i < 16; ++i) {
+                    const int64_t r = tile * 32 + 8 * (i / 4) + 4 * h + (i % 4);
+                    float v = acc[j][i] + bia[j];
+                    if (relu) v = fmaxf(v, 0.f);
+                    if (c < C && r < N) out[r * C + c] = v * scl[j] + shf[j];
+                    acc[j][i] = 0.f;
                 }
             }
         }
+        tile = ntile; q = nq; have = nhave;
+    }
+}
+
+// U row pairs of the weight-gradient kernel in registers: lane half h holds row base + 2u + h.
+template <int TA, int TB, int U, bool MASK> struct PairBlock {
+    Pack<TA> xa[U];
+    Pack<TB> gz[U];
+    Pack<MASK ? TB : 1> yy[U];
+};
+
+// `base` is uniform over the wavefront, so every row pair costs one scalar base per array and the lanes share
+// one 32-bit offset; FULL skips the row bound.
+template <int TA, int TB, int U, bool VEC, bool MASK, bool FULL>
+__device__ __forceinline__ void pairs_issue(PairBlock<TA, TB, U, MASK> &blk, const float *__restrict__ x,
+                                            const float *__restrict__ g, const float *__restrict__ y, int64_t base,
+                                            int64_t r1, int h, int Ci, int Co, int ci0, int co0)
+{
+    const int xo = h * Ci + ci0, go = h * Co + co0;
 #pragma unroll
-        for (int j = 0; j < NT; ++j) {
-            const int c = col0 + j * 32 + n;
-            if (c >= C) continue;
-#pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                const int64_t r = tile * 32 + 8 * (i / 4) + 4 * h + (i % 4);
-                if (r >= N) continue;
-                float v = acc[j][i] + bia[j];
-                if (relu) v = fmaxf(v, 0.f);
-                out[r * C + c] = v * scl[j] + shf[j];
+    for (int u = 0; u < U; ++u) {
+        const float *xu = x + (base + 2 * u) * Ci;
+        const float *gu = g + (base + 2 * u) * Co;
+        const float *yu = MASK ? y + (base + 2 * u) * Co : nullptr;
+        const bool live = FULL || base + 2 * u + h < r1;
+        blk.xa[u] = zero_pack<TA>();
+        blk.gz[u] = zero_pack<TB>();
+        blk.yy[u] = zero_pack<MASK ? TB : 1>();
+        if constexpr (VEC) {
+            if (live && ci0 < Ci) blk.xa[u] = ldp<TA>(xu + xo);
+            if (live && co0 < Co) {
+                blk.gz[u] = ldp<TB>(gu + go);
+                if constexpr (MASK) blk.yy[u] = ldp<TB>(yu + go);
             }
+        } else {
+#pragma unroll
+            for (int ja = 0; ja < TA; ++ja)
+                if (live && ci0 + ja < Ci) blk.xa[u].v[ja] = xu[xo + ja];
+#pragma unroll
+            for (int jb = 0; jb < TB; ++jb)
+                if (live && co0 + jb < Co) {
+                    blk.gz[u].v[jb] = gu[go + jb];
+                    if constexpr (MASK) blk.yy[u].v[jb] = yu[go + jb];
+                }
         }
     }
 }
@@ -143,52 +236,29 @@ __global__ __launch_bounds__(256, 2) void dense_wgrad_k(const float *__restrict_
     float gb[TB];
 #pragma unroll
     for (int jb = 0; jb < TB; ++jb) gb[jb] = 0.f;
-    const int64_t r0 = ((int64_t)blockIdx.x * 4 + wave) * rows_per_wave;
+    const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+    const int64_t r0 = ((int64_t)blockIdx.x * 4 + wave_u) * rows_per_wave;
     int64_t r1 = r0 + rows_per_wave;
     if (r1 > N) r1 = N;
     constexpr int U = 8;
+    PairBlock<TA, TB, U, MASK> blk;
     for (int64_t base = r0; base < r1; base += 2 * U) {
-        Pack<TA> xa[U];
-        Pack<TB> gz[U];
+        if (base + 2 * U <= r1) pairs_issue<TA, TB, U, VEC, MASK, true>(blk, x, g, y, base, r1, h, Ci, Co, ci0, co0);
+        else pairs_issue<TA, TB, U, VEC, MASK, false>(blk, x, g, y, base, r1, h, Ci, Co, ci0, co0);
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            const int64_t row = base + 2 * u + h;
-            xa[u] = zero_pack<TA>();
-            gz[u] = zero_pack<TB>();
-            if (row < r1) {
-                if constexpr (VEC) {
-                    if (ci0 < Ci) xa[u] = ldp<TA>(x + row * Ci + ci0);
-                    if (co0 < Co) {
-                        gz[u] = ldp<TB>(g + row * Co + co0);
-                        if constexpr (MASK) {
-                            const Pack<TB> yy = ldp<TB>(y + row * Co + co0);
+            float gzv[TB];
 #pragma unroll
-                            for (int jb = 0; jb < TB; ++jb) gz[u].v[jb] = yy.v[jb] > 0.f ? gz[u].v[jb] : 0.f;
-                        }
-                    }
-                } else {
-#pragma unroll
-                    for (int ja = 0; ja < TA; ++ja)
-                        if (ci0 + ja < Ci) xa[u].v[ja] = x[row * Ci + ci0 + ja];
-#pragma unroll
-                    for (int jb = 0; jb < TB; ++jb)
-                        if (co0 + jb < Co) {
-                            float v = g[row * Co + co0 + jb];
-                            if constexpr (MASK) v = y[row * Co + co0 + jb] > 0.f ? v : 0.f;
-                            gz[u].v[jb] = v;
-                        }
-                }
+            for (int jb = 0; jb < TB; ++jb) {
+                gzv[jb] = blk.gz[u].v[jb];
+                if constexpr (MASK) gzv[jb] = blk.yy[u].v[jb] > 0.f ? gzv[jb] : 0.f;
+                gb[jb] += gzv[jb];
             }
-        }
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-#pragma unroll
-            for (int jb = 0; jb < TB; ++jb) gb[jb] += gz[u].v[jb];
 #pragma unroll
             for (int ja = 0; ja < TA; ++ja)
 #pragma unroll
                 for (int jb = 0; jb < TB; ++jb)
-                    acc[ja][jb] = __builtin_amdgcn_mfma_f32_32x32x2f32(xa[u].v[ja], gz[u].v[jb], acc[ja][jb], 0, 0, 0);
+                    acc[ja][jb] = __builtin_amdgcn_mfma_f32_32x32x2f32(blk.xa[u].v[ja], gzv[jb], acc[ja][jb], 0, 0, 0);
         }
     }
     // the four wavefronts add up in wavefront order
@@ -228,29 +298,41 @@ __global__ __launch_bounds__(256, 2) void dense_wgrad_k(const float *__restrict_
 
 static bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
-// Column tiles per workgroup of dense_rows_k: as many as the 64 KiB slab and 8 accumulator tiles allow.
+// Column tiles per workgroup of dense_rows_k: as many as the preferred slab size and 4 accumulator tiles allow.
 static int rows_tiles(int Kpad, int C)
 {
-    int nt = 8;
+    int nt = 4;
     while (nt > 1 && (Kpad * nt * 32 > kDenseSlabFloats || (nt / 2) * 32 >= C)) nt >>= 1;
     return nt;
 }
 
-template <bool VEC, bool MASK>
-static void launch_rows(int NT, dim3 grid, size_t lds, hipStream_t st, const float *a, const float *mask, const float *w,
-                        int64_t wk, int64_t wc, const float *bias, const float *scale, const float *shift, int relu,
-                        float *out, int64_t N, int K, int Kpad, int C)
+// Launch with as many workgroups as are resident at once (every tile is independent, so the count only
+// balances the load): a grid that needs a second round of workgroups would run that round at low occupancy.
+template <int NT, bool VEC, bool MASK>
+static void launch_rows_nt(int64_t wanted, unsigned gy, size_t lds, hipStream_t st, const float *a, const float *mask,
+                           const float *w, int64_t wk, int64_t wc, const float *bias, const float *scale,
+                           const float *shift, int relu, float *out, int64_t N, int K, int Kpad, int C)
 {
-#define PM_ROWS(T)                                                                                                       \
-    do {                                                                                                                 \
-        if (lds > 65536)                                                                                                 \
-            (void)hipFuncSetAttribute(reinterpret_cast<const void *>(dense_rows_k<T, VEC, MASK>),                        \
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);                             \
-        dense_rows_k<T, VEC, MASK><<<grid, dim3(256), lds, st>>>(a, mask, w, wk, wc, bias, scale, shift, relu, out, N, \
-                                                                 K, Kpad, C);                                            \
-    } while (0)
+    const void *fn = reinterpret_cast<const void *>(dense_rows_k<NT, VEC, MASK>);
+    if (lds > 65536) (void)hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    int per_cu = 0, dev = 0, cus = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, fn, 256, lds) != hipSuccess || per_cu < 1) per_cu = 1;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < 1)
+        cus = 256;
+    int64_t gx = (int64_t)per_cu * cus / gy;
+    if (gx < 1) gx = 1;
+    if (gx > wanted) gx = wanted;
+    dense_rows_k<NT, VEC, MASK><<<dim3((unsigned)gx, gy), dim3(256), lds, st>>>(a, mask, w, wk, wc, bias, scale, shift,
+                                                                                relu, out, N, K, Kpad, C);
+}
+
+template <bool VEC, bool MASK>
+static void launch_rows(int NT, int64_t wanted, unsigned gy, size_t lds, hipStream_t st, const float *a,
+                        const float *mask, const float *w, int64_t wk, int64_t wc, const float *bias, const float *scale,
+                        const float *shift, int relu, float *out, int64_t N, int K, int Kpad, int C)
+{
+#define PM_ROWS(T) launch_rows_nt<T, VEC, MASK>(wanted, gy, lds, st, a, mask, w, wk, wc, bias, scale, shift, relu, out, N, K, Kpad, C)
     switch (NT) {
-    case 8: PM_ROWS(8); break;
     case 4: PM_ROWS(4); break;
     case 2: PM_ROWS(2); break;
     default: PM_ROWS(1); break;
@@ -266,20 +348,18 @@ static int dense_rows(const char *name, const float *a, const float *mask, const
     PM_REQUIRE(K > 0 && C > 0 && K <= kDenseMaxK && C <= (1 << 20), "%s: channel counts out of range (%d, %d)", name, K, C);
     PM_REQUIRE(N * (int64_t)(K > C ? K : C) < (int64_t(1) << 40), "%s: sizes too large", name);
     const int Kpad = (int)ceil_div(K, kDenseChunk) * kDenseChunk;
-    PM_REQUIRE(Kpad * 32 <= 2 * kDenseSlabFloats, "%s: reduction length too large", name);
     const int NT = rows_tiles(Kpad, C);
-    const size_t lds = (size_t)Kpad * NT * 32 * sizeof(float);
+    const size_t lds = ((size_t)Kpad * NT * 32 + kStageFloats) * sizeof(float);
     const int64_t ntiles = ceil_div(N, 32);
-    int64_t gx = ceil_div(ntiles, 4);
-    if (gx > 1024) gx = 1024;
-    const dim3 grid((unsigned)gx, (unsigned)ceil_div(C, NT * 32));
+    const int64_t wanted = ceil_div(ntiles, 4);
+    const unsigned gy = (unsigned)ceil_div(C, NT * 32);
     const bool vec = (K % 4 == 0) && aligned16(a) && (!mask || aligned16(mask));
     if (vec) {
-        if (mask) launch_rows<true, true>(NT, grid, lds, st, a, mask, w, wk, wc, bias, scale, shift, relu, out, N, K, Kpad, C);
-        else launch_rows<true, false>(NT, grid, lds, st, a, mask, w, wk, wc, bias, scale, shift, relu, out, N, K, Kpad, C);
+        if (mask) launch_rows<true, true>(NT, wanted, gy, lds, st, a, mask, w, wk, wc, bias, scale, shift, relu, out, N, K, Kpad, C);
+        else launch_rows<true, false>(NT, wanted, gy, lds, st, a, mask, w, wk, wc, bias, scale, shift, relu, out, N, K, Kpad, C);
     } else {
-        if (mask) launch_rows<false, true>(NT, grid, lds, st, a, mask, w, wk, wc, bias, scale, shift, relu, out, N, K, Kpad, C);
-        else launch_rows<false, false>(NT, grid, lds, st, a, mask, w, wk, wc, bias, scale, shift, relu, out, N, K, Kpad, C);
+        if (mask) launch_rows<false, true>(NT, wanted, gy, lds, st, a, mask, w, wk, wc, bias, scale, shift, relu, out, N, K, Kpad, C);
+        else launch_rows<false, false>(NT, wanted, gy, lds, st, a, mask, w, wk, wc, bias, scale, shift, relu, out, N, K, Kpad, C);
     }
     PM_LAUNCHED(name);
     return 0;
@@ -305,9 +385,9 @@ static WgradPlan wgrad_plan(int64_t N, int Ci, int Co)
     p.nB = (int)ceil_div(Co, p.tb * 32);
     int64_t G = ceil_div(N, 4 * 256);   // at least 256 rows per wavefront
     if (G < 1) G = 1;
-    if (G > 512) G = 512;
-    // keep the partials of wide layers modest: G * (Ci + 1) * Co floats <= 32 Mi floats
-    while (G > 1 && G * (int64_t)(Ci + 1) * Co > (int64_t(1) << 25)) G >>= 1;
+    if (G > 1024) G = 1024;
+    // keep the partials of wide layers modest: G * (Ci + 1) * Co floats <= 8 Mi floats
+    while (G > 1 && G * (int64_t)(Ci + 1) * Co > (int64_t(1) << 23)) G >>= 1;
     p.G = (int)G;
     p.rows_per_wave = ceil_div(ceil_div(N, G * 4), 2) * 2;
     return p;

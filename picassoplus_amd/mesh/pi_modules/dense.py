@@ -19,8 +19,8 @@ def _dims(input, weight, bias):
     if weight.shape[0] != Ci:
         raise RuntimeError("weight must have shape (in_channels, out_channels)")
     Co = weight.shape[1]
-    if Ci < 1 or Co < 1 or Ci > 1024:
-        raise RuntimeError("dense tail supports 1..1024 input channels, got %d" % Ci)
+    if Ci < 1 or Co < 1 or Ci > 896:
+        raise RuntimeError("dense tail supports 1..896 input channels, got %d" % Ci)
     if bias is not None:
         check_input(bias, "bias", 1, F32)
         if bias.shape[0] != Co:

@@ -226,6 +226,20 @@ int pmesh_dense_bwd(const float *grad_output, const float *input, const float *w
                     void *workspace, size_t workspace_bytes, int64_t N, int Ci, int Co,
                     pmesh_stream_t stream);
 
+
+/* The same tail for a convolution that mixes the channels itself (F2FConv3d, picasso/mesh/layers.py:60-64:
+ * outputs + biases, activation_fn, BatchNorm): output (N,C) = act(input + bias) * scale + shift, one pass;
+ * output may be input.  pmesh_bias_act_bwd: grad_input = grad_output where output > 0 (output NULL = no
+ * activation: then the gradient of the input is grad_output itself and grad_input must be NULL),
+ * grad_bias (C) = column sums of that, in a fixed order.  The backward takes C <= 1024, or <= 4096 when
+ * C % 4 == 0 and the pointers are 16-byte aligned. */
+int pmesh_bias_act_fwd(const float *input, const float *bias, const float *scale, const float *shift,
+                       int relu, float *output, int64_t N, int C, pmesh_stream_t stream);
+size_t pmesh_bias_act_bwd_workspace_bytes(int C);
+int pmesh_bias_act_bwd(const float *grad_output, const float *output, float *grad_input,
+                       float *grad_bias, void *workspace, size_t workspace_bytes, int64_t N, int C,
+                       pmesh_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -261,3 +261,21 @@ def dense_tail_bwd(gout, x, w, out=None):
     (entries with out > 0 pass the gradient), None for no activation."""
     gz = gout if out is None else torch.where(out > 0, gout, torch.zeros_like(gout))
     return gz @ w.t(), x.t() @ gz, gz.sum(0)
+
+
+def bias_act_fwd(x, b=None, relu=True, scale=None, shift=None):
+    """act(x + b) * scale + shift: the tail of F2FConv3d (picasso/mesh/layers.py:60-64)."""
+    z = x if b is None else x + b
+    if relu:
+        z = torch.clamp_min(z, 0)
+    if scale is not None:
+        z = z * scale
+    if shift is not None:
+        z = z + shift
+    return z
+
+
+def bias_act_bwd(gout, out=None):
+    """Gradients of act(x + b) for (x, b); ``out`` is the forward result when act is ReLU, else None."""
+    gz = gout if out is None else torch.where(out > 0, gout, torch.zeros_like(gout))
+    return gz, gz.sum(0)

@@ -296,6 +296,99 @@ __global__ __launch_bounds__(256, 2) void dense_wgrad_k(const float *__restrict_
     }
 }
 
+// The same tail without a product, for convolutions that mix channels themselves (facet2facet):
+// out = act(x + bias) * scale + shift, V floats per thread.
+template <int V>
+__global__ __launch_bounds__(256) void bias_act_fwd_k(const float *__restrict__ x, const float *__restrict__ bias,
+                                                      const float *__restrict__ scale,
+                                                      const float *__restrict__ shift, int relu,
+                                                      float *__restrict__ out, int64_t n_items, int items)
+{
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n_items) return;
+    const int c = (int)(i % items) * V;
+    Pack<V> v = ldp<V>(x + i * V);
+#pragma unroll
+    for (int j = 0; j < V; ++j) {
+        float t = v.v[j] + (bias ? bias[c + j] : 0.f);
+        if (relu) t = fmaxf(t, 0.f);
+        v.v[j] = t * (scale ? scale[c + j] : 1.f) + (shift ? shift[c + j] : 0.f);
+    }
+    stp<V>(out + i * V, v);
+}
+
+// Its gradient: gin = g where y > 0 (MASK; skipped when gin is null), partial[block][c] = the block's column sums
+// of the masked g.  A group of `lpr` lanes walks a row (looping when the row has more than lpr items, at most
+// kBiasLoops times), 256 / lpr rows in flight; the row slots add up in slot order.
+constexpr int kBiasLoops = 4;
+
+template <int V, bool MASK>
+__global__ __launch_bounds__(256) void bias_act_bwd_k(const float *__restrict__ g, const float *__restrict__ y,
+                                                      float *__restrict__ gin, float *__restrict__ partial,
+                                                      int64_t N, int C, int lpr, int64_t rows_per_block)
+{
+    __shared__ float red[256 * kBiasLoops * V];
+    const int lane = threadIdx.x % lpr, slot = threadIdx.x / lpr, rpb = 256 / lpr, items = C / V;
+    Pack<V> acc[kBiasLoops];
+#pragma unroll
+    for (int k = 0; k < kBiasLoops; ++k) acc[k] = zero_pack<V>();
+    const int64_t r0 = (int64_t)blockIdx.x * rows_per_block;
+    int64_t r1 = r0 + rows_per_block;
+    if (r1 > N) r1 = N;
+    for (int64_t row = r0 + slot; row < r1; row += rpb) {
+#pragma unroll
+        for (int k = 0; k < kBiasLoops; ++k) {
+            const int cv = lane + k * lpr;
+            if (cv < items) {
+                const int64_t o = row * C + (int64_t)cv * V;
+                Pack<V> gz = ldp<V>(g + o);
+                if constexpr (MASK) {
+                    const Pack<V> yy = ldp<V>(y + o);
+#pragma unroll
+                    for (int j = 0; j < V; ++j) gz.v[j] = yy.v[j] > 0.f ? gz.v[j] : 0.f;
+                    if (gin) stp<V>(gin + o, gz);
+                }
+#pragma unroll
+                for (int j = 0; j < V; ++j) acc[k].v[j] += gz.v[j];
+            }
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < kBiasLoops; ++k)
+#pragma unroll
+        for (int j = 0; j < V; ++j) red[(threadIdx.x * kBiasLoops + k) * V + j] = acc[k].v[j];
+    __syncthreads();
+    if (slot == 0) {
+#pragma unroll
+        for (int k = 0; k < kBiasLoops; ++k) {
+            const int cv = lane + k * lpr;
+            if (cv >= items) continue;
+            Pack<V> sum = zero_pack<V>();
+            for (int t = 0; t < rpb; ++t)
+#pragma unroll
+                for (int j = 0; j < V; ++j) sum.v[j] += red[((t * lpr + lane) * kBiasLoops + k) * V + j];
+#pragma unroll
+            for (int j = 0; j < V; ++j) partial[(size_t)blockIdx.x * C + cv * V + j] = sum.v[j];
+        }
+    }
+}
+
+struct BiasPlan {
+    int V, lpr, G;
+    int64_t rows_per_block;
+};
+
+static BiasPlan bias_plan(int64_t N, int C, bool aligned)
+{
+    BiasPlan p;
+    p.V = (aligned && C % 4 == 0) ? 4 : 1;
+    const RowShape rs = row_shape(C / p.V);
+    p.lpr = rs.lpr;
+    p.G = persistent_blocks(N, rs.rpb);
+    p.rows_per_block = ceil_div(ceil_div(N, p.G), rs.rpb) * rs.rpb;
+    return p;
+}
+
 static bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
 // Column tiles per workgroup of dense_rows_k: as many as the preferred slab size and 4 accumulator tiles allow.
@@ -473,4 +566,61 @@ extern "C" int pmesh_dense_bwd(const float *grad_output, const float *input, con
     int rc = reduce_partials(partial, grad_weight, p.G, Ci * Co, st, slice);
     if (rc) return rc;
     return reduce_partials(partial + (size_t)Ci * Co, grad_bias, p.G, Co, st, slice);
+}
+
+extern "C" int pmesh_bias_act_fwd(const float *input, const float *bias, const float *scale, const float *shift,
+                                  int relu, float *output, int64_t N, int C, pmesh_stream_t stream)
+{
+    clear_error();
+    PM_REQUIRE(N >= 0 && C > 0, "bias_act_fwd: bad sizes");
+    if (N == 0) return 0;
+    PM_REQUIRE(input && output, "bias_act_fwd: null pointer");
+    PM_REQUIRE(N * (int64_t)C < (int64_t(1) << 40), "bias_act_fwd: sizes too large");
+    const bool v4 = C % 4 == 0 && aligned16(input) && aligned16(output);
+    const int V = v4 ? 4 : 1;
+    const int64_t n_items = N * C / V;
+    const int64_t blocks = ceil_div(n_items, 256);
+    PM_REQUIRE(grid_ok(blocks), "bias_act_fwd: grid too large");
+    if (v4)
+        bias_act_fwd_k<4><<<dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream>>>(input, bias, scale, shift, relu,
+                                                                                          output, n_items, C / 4);
+    else
+        bias_act_fwd_k<1><<<dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream>>>(input, bias, scale, shift, relu,
+                                                                                          output, n_items, C);
+    PM_LAUNCHED("bias_act_fwd");
+    return 0;
+}
+
+extern "C" size_t pmesh_bias_act_bwd_workspace_bytes(int C)
+{
+    return (size_t)1024 * (size_t)(C > 0 ? C : 1) * sizeof(float);
+}
+
+extern "C" int pmesh_bias_act_bwd(const float *grad_output, const float *output, float *grad_input, float *grad_bias,
+                                  void *workspace, size_t workspace_bytes, int64_t N, int C, pmesh_stream_t stream)
+{
+    clear_error();
+    PM_REQUIRE(N >= 0 && C > 0, "bias_act_bwd: bad sizes");
+    PM_REQUIRE(grad_bias, "bias_act_bwd: null grad_bias");
+    hipStream_t st = (hipStream_t)stream;
+    if (N == 0) return reduce_partials(nullptr, grad_bias, 0, C, st);
+    PM_REQUIRE(grad_output && workspace, "bias_act_bwd: null pointer");
+    PM_REQUIRE(!grad_input || output, "bias_act_bwd: grad_input is grad_output itself when there is no activation");
+    PM_REQUIRE(N * (int64_t)C < (int64_t(1) << 40), "bias_act_bwd: sizes too large");
+    const bool aligned = aligned16(grad_output) && (!output || aligned16(output)) && (!grad_input || aligned16(grad_input));
+    const BiasPlan p = bias_plan(N, C, aligned);
+    PM_REQUIRE(C / p.V <= 256 * kBiasLoops, "bias_act_bwd: more than %d channels", 256 * kBiasLoops * p.V);
+    PM_REQUIRE(workspace_bytes >= (size_t)p.G * C * sizeof(float), "bias_act_bwd: workspace too small (%zu bytes)",
+               workspace_bytes);
+    float *partial = (float *)workspace;
+    const dim3 grid((unsigned)p.G), block(256);
+    if (p.V == 4) {
+        if (output) bias_act_bwd_k<4, true><<<grid, block, 0, st>>>(grad_output, output, grad_input, partial, N, C, p.lpr, p.rows_per_block);
+        else bias_act_bwd_k<4, false><<<grid, block, 0, st>>>(grad_output, output, grad_input, partial, N, C, p.lpr, p.rows_per_block);
+    } else {
+        if (output) bias_act_bwd_k<1, true><<<grid, block, 0, st>>>(grad_output, output, grad_input, partial, N, C, p.lpr, p.rows_per_block);
+        else bias_act_bwd_k<1, false><<<grid, block, 0, st>>>(grad_output, output, grad_input, partial, N, C, p.lpr, p.rows_per_block);
+    }
+    PM_LAUNCHED("bias_act_bwd");
+    return reduce_partials(partial, grad_bias, p.G, C, st);
 }

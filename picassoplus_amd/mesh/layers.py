@@ -87,6 +87,20 @@ class _ConvTail(nn.Module):
             shift = shift + bn.bias
         return scale.contiguous(), shift.contiguous()
 
+    def _bias_tail(self, outputs):
+        """``_tail(outputs)`` with bias and ReLU (or no activation) in one native pass, and a batch norm that only
+        applies its running statistics folded in when no gradients are recorded."""
+        relu = isinstance(self.activation_fn, nn.ReLU)
+        if not (relu or self.activation_fn is None):
+            return self._tail(outputs)
+        biases = self.biases.reshape(-1)
+        if self.with_bn and not torch.is_grad_enabled():
+            frozen = self._frozen_norm()
+            if frozen is not None:
+                return dense.bias_act_forward(outputs.contiguous(), biases.contiguous(), relu, frozen[0], frozen[1])
+        outputs = dense.bias_act(outputs.contiguous(), biases, relu)
+        return self.BatchNorm(outputs) if self.with_bn else outputs
+
     def _dense_tail(self, inputs, weights):
         """``_tail(inputs @ weights)`` with the product, the bias and a ReLU (or no activation) in one
         native pass; without gradients an inference-mode batch norm rides along as scale/shift.  Any
@@ -135,7 +149,7 @@ class F2FConv3d(_ConvTail):
         assert self.num_basis == bary_coeff.shape[-1]
         running_total = torch.cumsum(num_texture, dim=0, dtype=torch.int)
         outputs = conv3d.facet2facet(input_texture, self.weights, bary_coeff, running_total)
-        return self._tail(outputs)
+        return self._bias_tail(outputs)
 
 
 class _SeparableConv(_ConvTail):

@@ -93,3 +93,68 @@ class DenseTailFunction(torch.autograd.Function):
 def dense_tail(input, weight, bias, relu=True):
     """act(input @ weight + bias) with gradients; ``bias`` (Co,) float32."""
     return DenseTailFunction.apply(input, weight, bias, relu)
+
+
+# ---------------------------------------------------------------- the tail without a product
+def bias_act_forward(input, bias=None, relu=True, scale=None, shift=None):
+    """act(input + bias) * scale + shift for a convolution that mixes the channels itself (F2FConv3d,
+    picasso/mesh/layers.py:60-64), one pass, float32 (N,C)."""
+    check_input(input, "input", 2, F32)
+    N, C = input.shape
+    for name, t in (("bias", bias), ("scale", scale), ("shift", shift)):
+        if t is not None:
+            check_input(t, name, 1, F32)
+            if t.shape[0] != C:
+                raise RuntimeError("%s must have one entry per channel" % name)
+    dev = same_device(input, *[t for t in (bias, scale, shift) if t is not None])
+    with torch.cuda.device(dev):
+        out = torch.empty((N, C), dtype=F32, device=dev)
+        if C:
+            _lib.call("pmesh_bias_act_fwd", input.data_ptr(), _ptr(bias), _ptr(scale), _ptr(shift), 1 if relu else 0,
+                      out.data_ptr(), N, C, stream_of(input))
+    return out
+
+
+def bias_act_backward(grad_output, output=None, need_input=True):
+    """-> [grad_input, grad_bias]: grad_input is grad_output where ``output`` > 0 (``output`` None = no activation:
+    grad_output itself), grad_bias its column sums."""
+    check_input(grad_output, "grad_output", 2, F32)
+    N, C = grad_output.shape
+    if output is not None:
+        check_input(output, "output", 2, F32)
+        if tuple(output.shape) != (N, C):
+            raise RuntimeError("output must have the shape of grad_output")
+    dev = same_device(grad_output) if output is None else same_device(grad_output, output)
+    with torch.cuda.device(dev):
+        gin = torch.empty((N, C), dtype=F32, device=dev) if (need_input and output is not None) else None
+        gb = torch.empty((C,), dtype=F32, device=dev)
+        nbytes = _lib.query("pmesh_bias_act_bwd_workspace_bytes", C)
+        ws = workspace(nbytes, dev)
+        _lib.call("pmesh_bias_act_bwd", grad_output.data_ptr(), _ptr(output), _ptr(gin), gb.data_ptr(), ws.data_ptr(),
+                  nbytes, N, C, stream_of(grad_output))
+    if output is None and need_input:
+        gin = grad_output
+    return [gin, gb]
+
+
+class BiasActFunction(torch.autograd.Function):
+    """autograd Function of bias_act: gradients for input and bias."""
+
+    @staticmethod
+    def forward(ctx, input, bias, relu):
+        out = bias_act_forward(input, bias, relu)
+        ctx.relu = bool(relu)
+        ctx.save_for_backward(out if relu else None)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        (out,) = ctx.saved_tensors
+        gin, gb = bias_act_backward(grad_output.contiguous(), out if ctx.relu else None,
+                                    need_input=ctx.needs_input_grad[0])
+        return gin, gb if ctx.needs_input_grad[1] else None, None
+
+
+def bias_act(input, bias, relu=True):
+    """act(input + bias) with gradients; ``bias`` (C,) float32."""
+    return BiasActFunction.apply(input, bias, relu)

@@ -163,3 +163,58 @@ def test_per_item_module_train_and_eval(cuda, act, with_bn):
     # evaluation mode with gradients enabled keeps the batch norm outside the native pass and still agrees
     xg2 = x.to(cuda).requires_grad_(True)
     assert_close(mod(xg2), ref(mod64, x.double()).detach().numpy(), "PerItemConv3d eval output (grad mode)", 2e-5)
+
+
+@pytest.mark.parametrize("n,c", [(1, 1), (77, 13), (1000, 64), (4099, 32), (300, 1024), (65, 4096), (50000, 96), (33, 6)])
+@pytest.mark.parametrize("relu", [True, False])
+def test_bias_act_forward_backward(cuda, n, c, relu):
+    say("case bias_act", n, c, relu)
+    g = torch.Generator().manual_seed(n + c)
+    f = lambda t: t.to(cuda, torch.float32).contiguous()
+    xd, bd, god = f(torch.randn(n, c, generator=g)), f(torch.randn(c, generator=g)), f(torch.randn(n, c, generator=g))
+    sd, hd = f(torch.randn(c, generator=g)), f(torch.randn(c, generator=g))
+    x, b, go, sc, sh = (t.double().cpu() for t in (xd, bd, god, sd, hd))
+    out = dense.bias_act_forward(xd, bd, relu)
+    ref = torch_ref.bias_act_fwd(x, b, relu)
+    # float32 x + b rounds once; where the float64 sum is within that rounding of zero the ReLU may differ
+    assert_close(out, ref.numpy(), "bias_act forward")
+    assert_close(dense.bias_act_forward(xd, bd, relu, sd, hd), torch_ref.bias_act_fwd(x, b, relu, sc, sh).numpy(),
+                 "bias_act forward with scale/shift")
+    gx, gb = dense.bias_act_backward(god, out if relu else None)
+    rx, rb = torch_ref.bias_act_bwd(go, out.double().cpu() if relu else None)
+    torch.cuda.synchronize()
+    assert torch.equal(gx.cpu().double(), rx)                # a selection: exact
+    assert_close(gb, rb.numpy(), "bias_act grad_bias")
+    gx2, gb2 = dense.bias_act_backward(god, out if relu else None, need_input=False)
+    assert gx2 is None and torch.equal(gb2, gb)
+
+
+@pytest.mark.parametrize("act", ["relu", "none", "tanh"])
+def test_f2f_module_tail_eval_matches_float64(cuda, act):
+    """F2FConv3d in evaluation mode without gradients folds its batch norm into the native bias pass; the same
+    module in float64 on the CPU oracle ops is the answer."""
+    import copy
+    from util import texture_case
+    say("case f2f module eval tail", act)
+    torch.manual_seed(23)
+    fn = {"relu": nn.ReLU(), "none": None, "tanh": nn.Tanh()}[act]
+    rng = np.random.default_rng(23)
+    counts, bary, _ = texture_case(rng, 300, kmax=6)
+    mod = layers.F2FConv3d(8, 16, 3, activation_fn=fn).to(cuda)
+    with torch.no_grad():
+        mod.biases.add_(0.1 * torch.randn_like(mod.biases))
+        mod.BatchNorm.running_mean.add_(0.05 * torch.randn_like(mod.BatchNorm.running_mean))
+        mod.BatchNorm.running_var.mul_(1.5)
+    mod.eval()
+    mod64 = copy.deepcopy(mod).cpu().double().eval()
+    tex = torch.from_numpy(rng.normal(0, 1, (int(counts.sum()), 8)))
+    sh64 = torch_ref.sph_harm(torch.from_numpy(bary), 3)
+    cum = torch.cumsum(torch.from_numpy(counts), 0, dtype=torch.int32)
+    y = torch_ref.f2f_fwd(tex, mod64.weights, sh64, cum) + mod64.biases
+    if fn is not None:
+        y = fn(y)
+    y = mod64.BatchNorm(y)
+    with torch.no_grad():
+        sh = layers.SphHarmCoeff(3)(torch.from_numpy(bary).to(cuda, torch.float32))
+        out = mod(tex.to(cuda, torch.float32), sh, torch.from_numpy(counts).to(cuda))
+    assert_close(out, y.detach().numpy(), "F2FConv3d eval output", 2e-5)

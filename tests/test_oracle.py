@@ -353,3 +353,23 @@ def test_dense_tail_matches_torch_layers_and_hand_values():
     assert gx2.tolist() == [[1.0, 2.5], [0.0, 2.0]]
     assert gw2.tolist() == [[1.0, 0.0, 0.0], [2.0, 0.0, 2.5]]
     assert gb2.tolist() == [1.0, 0.0, 2.0]
+
+
+def test_bias_act_matches_autograd_and_hand_values():
+    g = torch.Generator().manual_seed(12)
+    x = torch.randn(29, 6, dtype=torch.float64, generator=g)
+    b = torch.randn(6, dtype=torch.float64, generator=g)
+    go = torch.randn(29, 6, dtype=torch.float64, generator=g)
+    for relu in (True, False):
+        xg, bg = x.clone().requires_grad_(True), b.clone().requires_grad_(True)
+        y = torch.nn.functional.relu(xg + bg) if relu else xg + bg
+        y.backward(go)
+        assert rel_err(torch_ref.bias_act_fwd(x, b, relu).numpy(), y.detach().numpy()) < 1e-15
+        gx, gb = torch_ref.bias_act_bwd(go, y.detach() if relu else None)
+        assert rel_err(gx.numpy(), xg.grad.numpy()) < 1e-15 and rel_err(gb.numpy(), bg.grad.numpy()) < 1e-14
+    x2 = torch.tensor([[1.0, -3.0], [0.5, 2.0]], dtype=torch.float64)
+    b2 = torch.tensor([-1.0, 1.5], dtype=torch.float64)
+    s2, t2 = torch.tensor([2.0, -1.0], dtype=torch.float64), torch.tensor([0.25, 0.5], dtype=torch.float64)
+    assert torch_ref.bias_act_fwd(x2, b2, True, s2, t2).tolist() == [[0.25, 0.5], [0.25, -3.0]]
+    gx2, gb2 = torch_ref.bias_act_bwd(torch.ones(2, 2, dtype=torch.float64), torch_ref.bias_act_fwd(x2, b2, True))
+    assert gx2.tolist() == [[0.0, 0.0], [0.0, 1.0]] and gb2.tolist() == [0.0, 1.0]

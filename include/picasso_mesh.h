@@ -207,6 +207,16 @@ int pmesh_count_vertex_adjface(const int32_t *rowptr, int32_t *nf_count, int64_t
 int pmesh_triangle_geometry(const float *vertex, const int32_t *face, float *geometry, int64_t Nv,
                             int64_t Nf, int vertex_stride, pmesh_stream_t stream);
 
+/* pmesh_combine_clusters replaces combineClustersLauncher (decimate_gpu.cu:750-810, decimate.py:53-67): the
+ * cluster maps of two consecutive decimation steps -- A over nv_a fine vertices, B over the nv_b vertices A
+ * keeps -- become one pair (rep_out, map_out) over the fine vertices, the vt_replace / vt_map a pooling layer
+ * over both steps takes.  rep: -r = contracted into vertex r, >= 0 = number of vertices contracted into this
+ * one; map: row among the kept vertices or -1.  scratch: nv_b int32.  Counts are integer sums, so the result
+ * does not depend on the order of execution. */
+int pmesh_combine_clusters(const int32_t *rep_a, const int32_t *map_a, const int32_t *rep_b,
+                           const int32_t *map_b, int32_t *rep_out, int32_t *map_out, int32_t *scratch,
+                           int64_t nv_a, int64_t nv_b, pmesh_stream_t stream);
+
 /* ------------------------------------------------------------------ pointwise tail of the convs
  * replaces the PyTorch ops that follow every convolution (picasso/mesh/layers.py:114-119, 169-174,
  * 232-238: torch.matmul(outputs, depth_weights) + biases, activation_fn, BatchNorm) by one pass:

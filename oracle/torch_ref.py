@@ -279,3 +279,29 @@ def bias_act_bwd(gout, out=None):
     """Gradients of act(x + b) for (x, b); ``out`` is the forward result when act is ReLU, else None."""
     gz = gout if out is None else torch.where(out > 0, gout, torch.zeros_like(gout))
     return gz, gz.sum(0)
+
+
+def combine_clusters(rep_a, map_a, rep_b, map_b):
+    """Cluster maps of two decimation steps -> maps of both together (decimate_gpu.cu:750-810): update_repB
+    (:750-760) records, for every step-A survivor that also survives step B, its fine index; update_repA
+    (:761-781) moves every fine vertex whose middle-level representative step B contracts to the fine index
+    behind B's representative, which counts it; update_mapA (:782-794) chains the maps.  int32 tensors."""
+    nv_a = rep_a.shape[0]
+    ra, ma, rb, mb = (_long(t) for t in (rep_a, map_a, rep_b, map_b))
+    idx = torch.arange(nv_a)
+    owner = rb.clone()
+    keep = ma >= 0
+    keep_b = keep.clone()
+    keep_b[keep] = rb[ma[keep]] >= 0
+    owner[ma[keep_b]] = idx[keep_b]
+    rep = ra.clone()
+    vi = torch.where(ra < 0, -ra, idx)
+    vo = ma[vi]
+    hit = vo >= 0
+    hit[hit.clone()] = owner[vo[hit]] < 0
+    target = owner[-owner[vo[hit]]]
+    rep[idx[hit]] = -target
+    rep.index_add_(0, target, torch.ones_like(target))
+    mapped = torch.full_like(ma, -1)
+    mapped[keep] = mb[ma[keep]]
+    return rep.to(torch.int32), mapped.to(torch.int32)

@@ -110,6 +110,54 @@ __global__ __launch_bounds__(kBlock) void fill_int_k(int *__restrict__ p, int64_
     if (i < n) p[i] = value;
 }
 
+// ----------------------------------------------------------------------------------------
+// Composition of two decimation steps' cluster maps (A: fine -> middle, B: middle -> coarse) into fine -> coarse
+// maps, in three passes.  rep < 0: contracted into vertex -rep; rep >= 0: number of vertices contracted into
+// this one.  Index values outside their arrays are ignored rather than followed.
+__global__ __launch_bounds__(kBlock) void clusters_copy_k(const int *__restrict__ rep_a, const int *__restrict__ rep_b,
+                                                          int *__restrict__ rep_out, int *__restrict__ owner,
+                                                          int64_t nv_a, int64_t nv_b)
+{
+    const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i < nv_a) rep_out[i] = rep_a[i];
+    if (i < nv_b) owner[i] = rep_b[i];
+}
+
+// owner[vo] = the fine vertex that survives step A as middle vertex vo, for the vo that survive step B too
+// (contracted vo keep their negative entry).
+__global__ __launch_bounds__(kBlock) void clusters_owner_k(const int *__restrict__ map_a, const int *__restrict__ rep_b,
+                                                           int *__restrict__ owner, int64_t nv_a, int64_t nv_b)
+{
+    const int64_t vi = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (vi >= nv_a) return;
+    const int vo = map_a[vi];
+    if (vo >= 0 && vo < nv_b && rep_b[vo] >= 0) owner[vo] = (int)vi;
+}
+
+// A fine vertex whose middle-level representative is contracted by step B moves to the fine vertex behind B's
+// representative and counts there; the map goes through both steps.
+__global__ __launch_bounds__(kBlock) void clusters_merge_k(const int *__restrict__ rep_a, const int *__restrict__ map_a,
+                                                           const int *__restrict__ owner, const int *__restrict__ map_b,
+                                                           int *__restrict__ rep_out, int *__restrict__ map_out,
+                                                           int64_t nv_a, int64_t nv_b)
+{
+    const int64_t idx = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (idx >= nv_a) return;
+    const int own = map_a[idx];
+    map_out[idx] = (own >= 0 && own < nv_b) ? map_b[own] : -1;
+    int64_t vi = idx;
+    if (rep_a[idx] < 0) vi = -(int64_t)rep_a[idx];
+    if (vi >= nv_a) return;
+    const int vo = map_a[vi];
+    if (vo < 0 || vo >= nv_b || owner[vo] >= 0) return;
+    const int64_t vb = -(int64_t)owner[vo];
+    if (vb >= nv_b) return;
+    const int target = owner[vb];
+    if (target < 0 || target >= nv_a) return;
+    rep_out[idx] = -target;
+    atomicAdd(&rep_out[target], 1);
+}
+
 }  // namespace pmesh
 
 using namespace pmesh;
@@ -200,5 +248,26 @@ extern "C" int pmesh_build_facet_order(const int32_t *cum_texture, int64_t n_fac
     hipError_t e = rocprim::radix_sort_pairs(base + 3 * slot, temp_bytes, keys_in, keys_out, vals_in, order,
                                              (size_t)n_facets, 0, 4, st);
     PM_REQUIRE(e == hipSuccess, "build_facet_order: radix sort failed: %s", hipGetErrorString(e));
+    return 0;
+}
+
+extern "C" int pmesh_combine_clusters(const int32_t *rep_a, const int32_t *map_a, const int32_t *rep_b,
+                                      const int32_t *map_b, int32_t *rep_out, int32_t *map_out, int32_t *scratch,
+                                      int64_t nv_a, int64_t nv_b, pmesh_stream_t stream)
+{
+    clear_error();
+    PM_REQUIRE(nv_a >= 0 && nv_b >= 0 && nv_a < INT32_MAX && nv_b < INT32_MAX, "combine_clusters: bad sizes");
+    if (nv_a == 0) return 0;
+    PM_REQUIRE(rep_a && map_a && rep_out && map_out, "combine_clusters: null pointer");
+    PM_REQUIRE(nv_b == 0 || (rep_b && map_b && scratch), "combine_clusters: null pointer");
+    hipStream_t st = (hipStream_t)stream;
+    const int64_t n = nv_a > nv_b ? nv_a : nv_b;
+    const dim3 grid_n((unsigned)ceil_div(n, kBlock)), grid_a((unsigned)ceil_div(nv_a, kBlock)), block(kBlock);
+    clusters_copy_k<<<grid_n, block, 0, st>>>(rep_a, rep_b, rep_out, scratch, nv_a, nv_b);
+    PM_LAUNCHED("combine_clusters(copy)");
+    clusters_owner_k<<<grid_a, block, 0, st>>>(map_a, rep_b, scratch, nv_a, nv_b);
+    PM_LAUNCHED("combine_clusters(owner)");
+    clusters_merge_k<<<grid_a, block, 0, st>>>(rep_a, map_a, scratch, map_b, rep_out, map_out, nv_a, nv_b);
+    PM_LAUNCHED("combine_clusters(merge)");
     return 0;
 }

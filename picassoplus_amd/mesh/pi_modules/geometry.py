@@ -1,6 +1,6 @@
 """Per-level producers of the convolution inputs: adjacent-facet counts of the output vertices and
-triangle geometry, with the reference's function names (picasso/mesh/pi_modules/decimate.py:70-93).
-Mesh decimation itself is not part of this package."""
+triangle geometry, and the composition of two decimation steps' cluster maps, with the reference's function
+names (picasso/mesh/pi_modules/decimate.py:53-93).  Mesh decimation itself is not part of this package."""
 import torch
 
 from ... import _lib
@@ -39,3 +39,26 @@ def compute_triangle_geometry_(vertex, face):
         _lib.call("pmesh_triangle_geometry", vertex.data_ptr(), face.data_ptr(), out.data_ptr(), vertex.shape[0],
                   face.shape[0], vertex.shape[1], stream_of(vertex))
     return out
+
+
+def combine_clusters_(repA, mapA, repB, mapB):
+    """Cluster maps of two consecutive decimation steps -> the maps of both steps together (decimate.py:53-67,
+    decimate_gpu.cu:750-810).  ``repA``/``mapA`` (int32, fine vertices) describe the first step, ``repB``/``mapB``
+    the second over the vertices the first keeps; returns (repComb, mapComb) over the fine vertices: the
+    ``vt_replace`` / ``vt_map`` of a pooling layer across both steps."""
+    for name, t in (("repA", repA), ("mapA", mapA), ("repB", repB), ("mapB", mapB)):
+        check_input(t, name, 1, I32)
+    if repA.shape != mapA.shape or repB.shape != mapB.shape:
+        raise RuntimeError("rep and map of one step must have the same length")
+    dev = same_device(repA, mapA, repB, mapB)
+    nv_a, nv_b = repA.shape[0], repB.shape[0]
+    topology._check_range("mapA", mapA, -1, nv_b)
+    topology._check_range("repA", repA, -(nv_a - 1), max(nv_a, 1))
+    topology._check_range("repB", repB, -(nv_b - 1), max(nv_b, 1))
+    with torch.cuda.device(dev):
+        rep_out = torch.empty_like(repA)
+        map_out = torch.empty_like(mapA)
+        scratch = torch.empty(max(nv_b, 1), dtype=I32, device=dev)
+        _lib.call("pmesh_combine_clusters", repA.data_ptr(), mapA.data_ptr(), repB.data_ptr(), mapB.data_ptr(),
+                  rep_out.data_ptr(), map_out.data_ptr(), scratch.data_ptr(), nv_a, nv_b, stream_of(repA))
+    return rep_out, map_out

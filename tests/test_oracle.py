@@ -373,3 +373,46 @@ def test_bias_act_matches_autograd_and_hand_values():
     assert torch_ref.bias_act_fwd(x2, b2, True, s2, t2).tolist() == [[0.25, 0.5], [0.25, -3.0]]
     gx2, gb2 = torch_ref.bias_act_bwd(torch.ones(2, 2, dtype=torch.float64), torch_ref.bias_act_fwd(x2, b2, True))
     assert gx2.tolist() == [[0.0, 0.0], [0.0, 1.0]] and gb2.tolist() == [0.0, 1.0]
+
+
+def _roots(rep):
+    idx = np.arange(rep.shape[0])
+    return np.where(rep < 0, -rep, idx)
+
+
+@pytest.mark.parametrize("spatial,orphans", [(True, 0.0), (False, 0.0), (False, 0.1)])
+def test_combine_clusters_composes_the_two_steps(spatial, orphans):
+    """What the combined maps must mean, stated without the reference's three passes: a fine vertex lands on
+    the coarse row that step B gives to the middle vertex step A gave it, every cluster points at one member
+    that survives both steps, and that member counts the others."""
+    rng = np.random.default_rng(31)
+    nv = 5000
+    ra, ma, nmid = S.cluster_maps(rng, nv, spatial=spatial, orphan_frac=orphans)
+    rb, mb, ncoarse = S.cluster_maps(rng, nmid, spatial=spatial, orphan_frac=orphans)
+    rc, mc = (t.numpy() for t in torch_ref.combine_clusters(*(T(a) for a in (ra, ma, rb, mb))))
+    mid = ma[_roots(ra)]                                   # middle vertex of every fine vertex, -1 if dropped
+    want = np.where(mid >= 0, mb[_roots(rb)[np.maximum(mid, 0)]], -1)
+    root_c = _roots(rc)
+    assert np.array_equal(rc[root_c] >= 0, np.ones(nv, bool))              # roots are representatives
+    live = want >= 0
+    assert np.array_equal(mc[root_c][live], want[live])                    # same coarse row as the two steps
+    members = np.bincount(root_c, minlength=nv)
+    reps = np.nonzero((rc >= 0) & (mid >= 0) & live)[0]
+    assert np.array_equal(rc[reps], members[reps] - 1)                     # the representative counts the rest
+    assert np.array_equal(mc, np.where(ma >= 0, mb[np.maximum(ma, 0)], -1))
+
+
+def test_combine_clusters_hand_case_and_identity():
+    # fine 0..5; step A: {0}, {1,2 -> 2}, {3}, {4,5 -> 4}; middle rows 0:0, 1:2, 2:3, 3:4
+    ra = np.array([0, -2, 1, 0, 1, -4], np.int32)
+    ma = np.array([0, -1, 1, 2, 3, -1], np.int32)
+    # step B over middle 0..3: {0}, {1,2 -> 2}, {3}; coarse rows 0:0, 1:2, 2:3
+    rb = np.array([0, -2, 1, 0], np.int32)
+    mb = np.array([0, -1, 1, 2], np.int32)
+    rc, mc = torch_ref.combine_clusters(T(ra), T(ma), T(rb), T(mb))
+    # middle 1 (fine 2, with member 1) is contracted into middle 2 (fine 3): fine 1, 2 now point at 3, which counts 2
+    assert rc.tolist() == [0, -3, -3, 2, 1, -4]
+    assert mc.tolist() == [0, -1, -1, 1, 2, -1]
+    ident_r, ident_m = np.zeros(4, np.int32), np.arange(4, dtype=np.int32)
+    rc, mc = torch_ref.combine_clusters(T(ident_r), T(ident_m), T(rb), T(mb))
+    assert rc.tolist() == rb.tolist() and mc.tolist() == mb.tolist()

@@ -13,7 +13,9 @@ namespace pmesh {
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 constexpr int kDenseChunk = 64;            // reduction entries per register chunk (32 per lane half)
-constexpr int kDenseSlabFloats = 12288;    // preferred weight slab of one workgroup in LDS (48 KiB)
+constexpr int kDenseSlabFloats = 12288;    // preferred weight slab of a four-wavefront workgroup in LDS (48 KiB)
+constexpr int kDenseSlabWide = 22528;      // of an eight-wavefront workgroup (88 KiB)
+constexpr size_t kDenseLdsMax = 160 * 1024;
 constexpr int kDenseMaxK = 896;            // a 32-column slab of that length is 112 KiB, beside 34 KiB of row stages
 
 // rows (N x K, row stride K) times Wm (K x C, element (k, c) at w[k * wk + c * wc]) for the NT * 32 columns
@@ -24,7 +26,7 @@ constexpr int kDenseMaxK = 896;            // a 32-column slab of that length is
 // weight slab sits in LDS as [k/4][column][k%4], one 16-byte read feeds four matrix instructions.  MASK: the
 // row operand is a[r][k] where mask[r][k] > 0, else 0 (the ReLU backward).
 constexpr int kStageStride = 68;                       // floats per staged row: 16-byte reads of 32 rows hit all banks
-constexpr int kStageFloats = 4 * 32 * kStageStride;    // four wavefronts
+constexpr int kStageWave = 32 * kStageStride;          // per wavefront
 
 template <bool VEC, bool MASK> struct RowBlock {
     float v[32];
@@ -84,8 +86,8 @@ __device__ __forceinline__ void rows_commit(const RowBlock<VEC, MASK> &b, float 
     }
 }
 
-template <int NT, bool VEC, bool MASK>
-__global__ __launch_bounds__(256, 2) void dense_rows_k(const float *__restrict__ a, const float *__restrict__ mask,
+template <int NT, int NW, bool VEC, bool MASK>
+__global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void dense_rows_k(const float *__restrict__ a, const float *__restrict__ mask,
                                                        const float *__restrict__ w, int64_t wk, int64_t wc,
                                                        const float *__restrict__ bias,
                                                        const float *__restrict__ scale,
@@ -97,9 +99,9 @@ __global__ __launch_bounds__(256, 2) void dense_rows_k(const float *__restrict__
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int n = lane & 31, h = lane >> 5;
     const int col0 = blockIdx.y * NC;
-    float *slab = lds + kStageFloats;
-    float *stage = lds + wave * (32 * kStageStride);
-    for (int idx = threadIdx.x; idx < Kpad * NC; idx += 256) {
+    float *slab = lds + NW * kStageWave;
+    float *stage = lds + wave * kStageWave;
+    for (int idx = threadIdx.x; idx < Kpad * NC; idx += NW * 64) {
         const int k = idx / NC, c = idx - k * NC;
         const float v = (k < K && col0 + c < C) ? w[(int64_t)k * wk + (int64_t)(col0 + c) * wc] : 0.f;
         slab[((k >> 2) * NC + c) * 4 + (k & 3)] = v;
@@ -113,8 +115,8 @@ __global__ __launch_bounds__(256, 2) void dense_rows_k(const float *__restrict__
         scl[j] = (scale && c < C) ? scale[c] : 1.f;
         shf[j] = (shift && c < C) ? shift[c] : 0.f;
     }
-    const int64_t ntiles = (N + 31) / 32, stride = (int64_t)gridDim.x * 4;
-    int64_t tile = (int64_t)blockIdx.x * 4 + wave;
+    const int64_t ntiles = (N + 31) / 32, stride = (int64_t)gridDim.x * NW;
+    int64_t tile = (int64_t)blockIdx.x * NW + wave;
     int q = 0;
     bool have = tile < ntiles;
     RowBlock<VEC, MASK> blk;
@@ -392,43 +394,52 @@ static BiasPlan bias_plan(int64_t N, int C, bool aligned)
 static bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
 // Column tiles per workgroup of dense_rows_k: as many as the preferred slab size and 4 accumulator tiles allow.
-static int rows_tiles(int Kpad, int C)
+static int rows_tiles(int Kpad, int C, int slab_floats)
 {
     int nt = 4;
-    while (nt > 1 && (Kpad * nt * 32 > kDenseSlabFloats || (nt / 2) * 32 >= C)) nt >>= 1;
+    while (nt > 1 && (Kpad * nt * 32 > slab_floats || (nt / 2) * 32 >= C)) nt >>= 1;
     return nt;
 }
 
 // Launch with as many workgroups as are resident at once (every tile is independent, so the count only
 // balances the load): a grid that needs a second round of workgroups would run that round at low occupancy.
-template <int NT, bool VEC, bool MASK>
-static void launch_rows_nt(int64_t wanted, unsigned gy, size_t lds, hipStream_t st, const float *a, const float *mask,
+template <int NT, int NW, bool VEC, bool MASK>
+static void launch_rows_nt(int64_t ntiles, unsigned gy, size_t lds, hipStream_t st, const float *a, const float *mask,
                            const float *w, int64_t wk, int64_t wc, const float *bias, const float *scale,
                            const float *shift, int relu, float *out, int64_t N, int K, int Kpad, int C)
 {
-    const void *fn = reinterpret_cast<const void *>(dense_rows_k<NT, VEC, MASK>);
+    const void *fn = reinterpret_cast<const void *>(dense_rows_k<NT, NW, VEC, MASK>);
     if (lds > 65536) (void)hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     int per_cu = 0, dev = 0, cus = 0;
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, fn, 256, lds) != hipSuccess || per_cu < 1) per_cu = 1;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, fn, NW * 64, lds) != hipSuccess || per_cu < 1) per_cu = 1;
     if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < 1)
         cus = 256;
     int64_t gx = (int64_t)per_cu * cus / gy;
+    const int64_t wanted = ceil_div(ntiles, NW);
     if (gx < 1) gx = 1;
     if (gx > wanted) gx = wanted;
-    dense_rows_k<NT, VEC, MASK><<<dim3((unsigned)gx, gy), dim3(256), lds, st>>>(a, mask, w, wk, wc, bias, scale, shift,
-                                                                                relu, out, N, K, Kpad, C);
+    dense_rows_k<NT, NW, VEC, MASK><<<dim3((unsigned)gx, gy), dim3(NW * 64), lds, st>>>(a, mask, w, wk, wc, bias, scale,
+                                                                                        shift, relu, out, N, K, Kpad, C);
 }
 
 template <bool VEC, bool MASK>
-static void launch_rows(int NT, int64_t wanted, unsigned gy, size_t lds, hipStream_t st, const float *a,
+static void launch_rows(int NT, int NW, int64_t ntiles, unsigned gy, size_t lds, hipStream_t st, const float *a,
                         const float *mask, const float *w, int64_t wk, int64_t wc, const float *bias, const float *scale,
                         const float *shift, int relu, float *out, int64_t N, int K, int Kpad, int C)
 {
-#define PM_ROWS(T) launch_rows_nt<T, VEC, MASK>(wanted, gy, lds, st, a, mask, w, wk, wc, bias, scale, shift, relu, out, N, K, Kpad, C)
-    switch (NT) {
-    case 4: PM_ROWS(4); break;
-    case 2: PM_ROWS(2); break;
-    default: PM_ROWS(1); break;
+#define PM_ROWS(T, W) launch_rows_nt<T, W, VEC, MASK>(ntiles, gy, lds, st, a, mask, w, wk, wc, bias, scale, shift, relu, out, N, K, Kpad, C)
+    if (NW == 8) {
+        switch (NT) {
+        case 4: PM_ROWS(4, 8); break;
+        case 2: PM_ROWS(2, 8); break;
+        default: PM_ROWS(1, 8); break;
+        }
+    } else {
+        switch (NT) {
+        case 4: PM_ROWS(4, 4); break;
+        case 2: PM_ROWS(2, 4); break;
+        default: PM_ROWS(1, 4); break;
+        }
     }
 #undef PM_ROWS
 }
@@ -441,18 +452,25 @@ static int dense_rows(const char *name, const float *a, const float *mask, const
     PM_REQUIRE(K > 0 && C > 0 && K <= kDenseMaxK && C <= (1 << 20), "%s: channel counts out of range (%d, %d)", name, K, C);
     PM_REQUIRE(N * (int64_t)(K > C ? K : C) < (int64_t(1) << 40), "%s: sizes too large", name);
     const int Kpad = (int)ceil_div(K, kDenseChunk) * kDenseChunk;
-    const int NT = rows_tiles(Kpad, C);
-    const size_t lds = ((size_t)Kpad * NT * 32 + kStageFloats) * sizeof(float);
+    // Four wavefronts per workgroup and a slab of at most 48 KiB keep two workgroups on a CU.  When that slab
+    // cannot hold all the columns (the rows would be fetched once per column block), or leaves room for one
+    // workgroup only, eight wavefronts share a slab of up to 88 KiB instead.
+    int NT = rows_tiles(Kpad, C, kDenseSlabFloats), NW = 4;
+    size_t lds = ((size_t)Kpad * NT * 32 + 4 * kStageWave) * sizeof(float);
+    const int nt8 = rows_tiles(Kpad, C, kDenseSlabWide);
+    const size_t lds8 = ((size_t)Kpad * nt8 * 32 + 8 * kStageWave) * sizeof(float);
+    if (lds8 <= kDenseLdsMax && (nt8 > NT || lds > kDenseLdsMax / 2)) {
+        NT = nt8; NW = 8; lds = lds8;
+    }
     const int64_t ntiles = ceil_div(N, 32);
-    const int64_t wanted = ceil_div(ntiles, 4);
     const unsigned gy = (unsigned)ceil_div(C, NT * 32);
     const bool vec = (K % 4 == 0) && aligned16(a) && (!mask || aligned16(mask));
     if (vec) {
-        if (mask) launch_rows<true, true>(NT, wanted, gy, lds, st, a, mask, w, wk, wc, bias, scale, shift, relu, out, N, K, Kpad, C);
-        else launch_rows<true, false>(NT, wanted, gy, lds, st, a, mask, w, wk, wc, bias, scale, shift, relu, out, N, K, Kpad, C);
+        if (mask) launch_rows<true, true>(NT, NW, ntiles, gy, lds, st, a, mask, w, wk, wc, bias, scale, shift, relu, out, N, K, Kpad, C);
+        else launch_rows<true, false>(NT, NW, ntiles, gy, lds, st, a, mask, w, wk, wc, bias, scale, shift, relu, out, N, K, Kpad, C);
     } else {
-        if (mask) launch_rows<false, true>(NT, wanted, gy, lds, st, a, mask, w, wk, wc, bias, scale, shift, relu, out, N, K, Kpad, C);
-        else launch_rows<false, false>(NT, wanted, gy, lds, st, a, mask, w, wk, wc, bias, scale, shift, relu, out, N, K, Kpad, C);
+        if (mask) launch_rows<false, true>(NT, NW, ntiles, gy, lds, st, a, mask, w, wk, wc, bias, scale, shift, relu, out, N, K, Kpad, C);
+        else launch_rows<false, false>(NT, NW, ntiles, gy, lds, st, a, mask, w, wk, wc, bias, scale, shift, relu, out, N, K, Kpad, C);
     }
     PM_LAUNCHED(name);
     return 0;

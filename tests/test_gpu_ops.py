@@ -234,6 +234,48 @@ def test_f2f_wide_dynamic_range(cuda, case):
     assert_close(ft.grad, gfilt_ref, "f2f grad_filter")
 
 
+@pytest.mark.parametrize("case", ["zero_grad_rows", "relu_sparse", "all_zero", "zero_filter"])
+def test_f2f_sparse_and_zero_data(cuda, case):
+    """Data a trained network really produces: facets without a label send all-zero gradient rows, a ReLU in front
+    leaves half of the texture features zero and whole facets dark, and a freshly zeroed filter or an all-zero
+    gradient must give exact zeros, never a NaN from a scale of an empty maximum."""
+    say("case f2f sparse", case)
+    rng = np.random.default_rng(123)
+    nf, Cin, Cout = 1500, 32, 64
+    counts, bary, owner = texture_case(rng, nf, 7)
+    cum = np.cumsum(counts).astype(np.int32)
+    T = int(counts.sum())
+    tex = rng.normal(0, 1, (T, Cin))
+    sh = rng.normal(0, 0.5, (T, 16))
+    filt = rng.normal(0, 0.3, (Cout, Cin, 16))
+    gout = rng.normal(0, 1, (nf, Cout))
+    if case == "zero_grad_rows":
+        gout[rng.random(nf) < 0.7] = 0.0
+        gout[:200] = 0.0                                     # whole tiles of facets without a gradient
+    elif case == "relu_sparse":
+        tex = np.maximum(tex, 0.0)
+        tex[np.isin(owner, np.nonzero(rng.random(nf) < 0.3)[0])] = 0.0
+        gout = np.where(rng.random((nf, Cout)) < 0.5, gout, 0.0)
+    elif case == "all_zero":
+        gout[:] = 0.0
+        tex[:] = 0.0
+    else:
+        filt[:] = 0.0
+    out_ref = loops.f2f_fwd(tex, filt, sh, cum)
+    gin_ref, gfilt_ref = loops.f2f_bwd(gout, tex, filt, sh, cum)
+    tt = dev(tex, cuda, torch.float32).requires_grad_(True)
+    ft = dev(filt, cuda, torch.float32).requires_grad_(True)
+    out = conv3d.facet2facet(tt, ft, dev(sh, cuda, torch.float32), dev(cum, cuda))
+    out.backward(dev(gout, cuda, torch.float32))
+    torch.cuda.synchronize()
+    for name, got, ref in (("out", out, out_ref), ("grad_texture", tt.grad, gin_ref), ("grad_filter", ft.grad, gfilt_ref)):
+        assert bool(torch.isfinite(got).all()), name
+        if np.abs(ref).max() == 0.0:
+            assert float(got.detach().abs().max()) == 0.0, name
+        else:
+            assert_close(got, ref, "f2f " + name)
+
+
 def test_f2f_without_facet_order(cuda):
     """The facet order is optional at the C ABI (NULL): same results for the forward and the texture gradient
     (to an ulp), the same filter gradient up to summation order."""

@@ -326,7 +326,8 @@ def run_tail(args, torch):
     ms = (time.perf_counter() - t0) * 1e3 / args.steps
     _lib.set_call_hook(None)
     per_op = timer.summary()
-    nb = {"dense_fwd": 4 * N * (Ci + Co), "dense_bwd": 4 * N * (2 * Co + Ci) + 4 * N * Ci}
+    # every operand once: the ReLU mask travels as one bit per entry (N * Co / 8 bytes) from the forward to the backward
+    nb = {"dense_fwd": 4 * N * (Ci + Co) + N * Co // 8, "dense_bwd": 4 * N * (Co + Ci) + N * Co // 8 + 4 * N * Ci}
     fl = {"dense_fwd": 2.0 * N * Ci * Co, "dense_bwd": 4.0 * N * Ci * Co}
     dom = max(nb, key=lambda k: per_op[k])
     ach = nb[dom] / (per_op[dom] * 1e-3) / 1e9

@@ -223,32 +223,36 @@ int pmesh_combine_clusters(const int32_t *rep_a, const int32_t *map_a, const int
  *   output (N,Co) = act(input (N,Ci) . weight (Ci,Co) + bias (Co)) * scale (Co) + shift (Co)
  * relu != 0 selects max(.,0), else identity; bias, scale, shift may be NULL (0, 1, 0): scale/shift carry
  * an inference-mode batch norm (gamma/sqrt(var+eps), beta - mean*that).  Ci <= 896.
+ * relu_bits (NULL or N * ceil(Co/32) uint32) receives one bit per output entry, set where the activated value
+ * is > 0 (bit c % 32 of word c / 32 of the row): the ReLU mask for the backward pass at 1/32 of the output's size.
  * pmesh_dense_bwd is the gradient of the tail without scale/shift (training-mode batch norm stays
- * outside): gz = grad_output where output > 0 (output = the forward result, NULL when relu was off);
- * grad_input (N,Ci) = gz . weight^T (NULL skips it), grad_weight (Ci,Co) = input^T . gz,
+ * outside): gz = grad_output where the ReLU let the value through -- read from relu_bits when given, else
+ * from output > 0 (output = the forward result); both NULL = no activation.
+ * grad_input (N,Ci) = gz . weight^T (NULL skips it; needs Co <= 896), grad_weight (Ci,Co) = input^T . gz,
  * grad_bias (Co) = column sums of gz; both sums in a fixed order. */
 int pmesh_dense_fwd(const float *input, const float *weight, const float *bias, const float *scale,
-                    const float *shift, int relu, float *output, int64_t N, int Ci, int Co,
-                    pmesh_stream_t stream);
+                    const float *shift, int relu, float *output, uint32_t *relu_bits, int64_t N, int Ci,
+                    int Co, pmesh_stream_t stream);
 size_t pmesh_dense_bwd_workspace_bytes(int64_t N, int Ci, int Co);
 int pmesh_dense_bwd(const float *grad_output, const float *input, const float *weight,
-                    const float *output, float *grad_input, float *grad_weight, float *grad_bias,
-                    void *workspace, size_t workspace_bytes, int64_t N, int Ci, int Co,
-                    pmesh_stream_t stream);
-
+                    const float *output, const uint32_t *relu_bits, float *grad_input,
+                    float *grad_weight, float *grad_bias, void *workspace, size_t workspace_bytes,
+                    int64_t N, int Ci, int Co, pmesh_stream_t stream);
 
 /* The same tail for a convolution that mixes the channels itself (F2FConv3d, picasso/mesh/layers.py:60-64:
  * outputs + biases, activation_fn, BatchNorm): output (N,C) = act(input + bias) * scale + shift, one pass;
- * output may be input.  pmesh_bias_act_bwd: grad_input = grad_output where output > 0 (output NULL = no
- * activation: then the gradient of the input is grad_output itself and grad_input must be NULL),
- * grad_bias (C) = column sums of that, in a fixed order.  The backward takes C <= 1024, or <= 4096 when
- * C % 4 == 0 and the pointers are 16-byte aligned. */
+ * output may be input.  relu_bits as in pmesh_dense_fwd (NULL, or N * C/32 words when C % 32 == 0 and the rows
+ * are 16-byte aligned).  pmesh_bias_act_bwd: grad_input = grad_output where the ReLU let the value through
+ * (relu_bits, else output > 0; both NULL = no activation: then the gradient of the input is grad_output
+ * itself and grad_input must be NULL), grad_bias (C) = column sums of that, in a fixed order.  The backward
+ * takes C <= 1024, or <= 4096 when C % 4 == 0 and the pointers are 16-byte aligned. */
 int pmesh_bias_act_fwd(const float *input, const float *bias, const float *scale, const float *shift,
-                       int relu, float *output, int64_t N, int C, pmesh_stream_t stream);
-size_t pmesh_bias_act_bwd_workspace_bytes(int C);
-int pmesh_bias_act_bwd(const float *grad_output, const float *output, float *grad_input,
-                       float *grad_bias, void *workspace, size_t workspace_bytes, int64_t N, int C,
+                       int relu, float *output, uint32_t *relu_bits, int64_t N, int C,
                        pmesh_stream_t stream);
+size_t pmesh_bias_act_bwd_workspace_bytes(int C);
+int pmesh_bias_act_bwd(const float *grad_output, const float *output, const uint32_t *relu_bits,
+                       float *grad_input, float *grad_bias, void *workspace, size_t workspace_bytes,
+                       int64_t N, int C, pmesh_stream_t stream);
 
 #ifdef __cplusplus
 }

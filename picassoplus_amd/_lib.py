@@ -11,7 +11,7 @@ from ctypes import c_char_p, c_int, c_int64, c_size_t, c_void_p
 _HERE = os.path.dirname(os.path.abspath(__file__))
 # PICASSO_MESH_LIB points at an alternative build of the same ABI (kernel experiments)
 LIB_PATH = os.environ.get("PICASSO_MESH_LIB") or os.path.join(_HERE, "csrc", "libpicasso_mesh.so")
-ABI_VERSION = 7
+ABI_VERSION = 8
 
 P, I, L, Z = c_void_p, c_int, c_int64, c_size_t
 
@@ -47,12 +47,12 @@ SIGNATURES = {
     "pmesh_triangle_geometry": (I, [P, P, P, L, L, I, P]),
     "pmesh_sph_harm": (I, [P, P, L, I, P]),
     "pmesh_combine_clusters": (I, [P, P, P, P, P, P, P, L, L, P]),
-    "pmesh_dense_fwd": (I, [P, P, P, P, P, I, P, L, I, I, P]),
+    "pmesh_dense_fwd": (I, [P, P, P, P, P, I, P, P, L, I, I, P]),
     "pmesh_dense_bwd_workspace_bytes": (Z, [L, I, I]),
-    "pmesh_dense_bwd": (I, [P, P, P, P, P, P, P, P, Z, L, I, I, P]),
-    "pmesh_bias_act_fwd": (I, [P, P, P, P, I, P, L, I, P]),
+    "pmesh_dense_bwd": (I, [P, P, P, P, P, P, P, P, P, Z, L, I, I, P]),
+    "pmesh_bias_act_fwd": (I, [P, P, P, P, I, P, P, L, I, P]),
     "pmesh_bias_act_bwd_workspace_bytes": (Z, [I]),
-    "pmesh_bias_act_bwd": (I, [P, P, P, P, P, Z, L, I, P]),
+    "pmesh_bias_act_bwd": (I, [P, P, P, P, P, P, Z, L, I, P]),
 }
 
 _lib = None

@@ -28,15 +28,18 @@ constexpr int kDenseMaxK = 896;            // a 32-column slab of that length is
 constexpr int kStageStride = 68;                       // floats per staged row: 16-byte reads of 32 rows hit all banks
 constexpr int kStageWave = 32 * kStageStride;          // per wavefront
 
-template <bool VEC, bool MASK> struct RowBlock {
+// MASK: 0 = rows as they are, 1 = a float array of the rows' shape decides (entries > 0 pass),
+// 2 = one bit per entry decides (32-bit words, W per row, bit c % 32 of word c / 32).
+template <bool VEC, int MASK> struct RowBlock {
     float v[32];
-    float m[MASK ? 32 : 1];
+    float m[MASK == 1 ? 32 : 1];
+    unsigned w[MASK == 2 ? (VEC ? 8 : 32) : 1];
 };
 
-template <bool VEC, bool MASK>
+template <bool VEC, int MASK>
 __device__ __forceinline__ void rows_issue(RowBlock<VEC, MASK> &b, const float *__restrict__ a,
-                                           const float *__restrict__ mask, int64_t tile, int q, int64_t N, int K,
-                                           int lane)
+                                           const float *__restrict__ mask, const unsigned *__restrict__ bits, int W,
+                                           int64_t tile, int q, int64_t N, int K, int lane)
 {
     if constexpr (VEC) {
         const int col = q + 4 * (lane & 15);
@@ -44,12 +47,14 @@ __device__ __forceinline__ void rows_issue(RowBlock<VEC, MASK> &b, const float *
         for (int i = 0; i < 8; ++i) {
             const int64_t row = tile * 32 + 4 * i + (lane >> 4);
             float4 t = make_float4(0.f, 0.f, 0.f, 0.f), mm = make_float4(1.f, 1.f, 1.f, 1.f);
+            if constexpr (MASK == 2) b.w[i] = 0u;
             if (row < N && col < K) {
                 t = *reinterpret_cast<const float4 *>(a + row * K + col);
-                if constexpr (MASK) mm = *reinterpret_cast<const float4 *>(mask + row * K + col);
+                if constexpr (MASK == 1) mm = *reinterpret_cast<const float4 *>(mask + row * K + col);
+                if constexpr (MASK == 2) b.w[i] = bits[row * W + (col >> 5)];
             }
             b.v[4 * i] = t.x; b.v[4 * i + 1] = t.y; b.v[4 * i + 2] = t.z; b.v[4 * i + 3] = t.w;
-            if constexpr (MASK) { b.m[4 * i] = mm.x; b.m[4 * i + 1] = mm.y; b.m[4 * i + 2] = mm.z; b.m[4 * i + 3] = mm.w; }
+            if constexpr (MASK == 1) { b.m[4 * i] = mm.x; b.m[4 * i + 1] = mm.y; b.m[4 * i + 2] = mm.z; b.m[4 * i + 3] = mm.w; }
         }
     } else {
         const int col = q + lane;
@@ -58,21 +63,27 @@ __device__ __forceinline__ void rows_issue(RowBlock<VEC, MASK> &b, const float *
             const int64_t row = tile * 32 + i;
             const bool ok = row < N && col < K;
             b.v[i] = ok ? a[row * K + col] : 0.f;
-            if constexpr (MASK) b.m[i] = ok ? mask[row * K + col] : 1.f;
+            if constexpr (MASK == 1) b.m[i] = ok ? mask[row * K + col] : 1.f;
+            if constexpr (MASK == 2) b.w[i] = ok ? bits[row * W + (col >> 5)] : 0u;
         }
     }
 }
 
-template <bool VEC, bool MASK>
+template <bool VEC, int MASK>
 __device__ __forceinline__ void rows_commit(const RowBlock<VEC, MASK> &b, float *stage, int lane)
 {
     if constexpr (VEC) {
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
             float4 t = make_float4(b.v[4 * i], b.v[4 * i + 1], b.v[4 * i + 2], b.v[4 * i + 3]);
-            if constexpr (MASK) {
+            if constexpr (MASK == 1) {
                 t.x = b.m[4 * i] > 0.f ? t.x : 0.f; t.y = b.m[4 * i + 1] > 0.f ? t.y : 0.f;
                 t.z = b.m[4 * i + 2] > 0.f ? t.z : 0.f; t.w = b.m[4 * i + 3] > 0.f ? t.w : 0.f;
+            }
+            if constexpr (MASK == 2) {
+                const unsigned nib = b.w[i] >> ((4 * (lane & 15)) & 31);      // chunks start at multiples of 64 columns
+                t.x = (nib & 1u) ? t.x : 0.f; t.y = (nib & 2u) ? t.y : 0.f;
+                t.z = (nib & 4u) ? t.z : 0.f; t.w = (nib & 8u) ? t.w : 0.f;
             }
             *reinterpret_cast<float4 *>(stage + (4 * i + (lane >> 4)) * kStageStride + 4 * (lane & 15)) = t;
         }
@@ -80,14 +91,17 @@ __device__ __forceinline__ void rows_commit(const RowBlock<VEC, MASK> &b, float 
 #pragma unroll
         for (int i = 0; i < 32; ++i) {
             float t = b.v[i];
-            if constexpr (MASK) t = b.m[i] > 0.f ? t : 0.f;
+            if constexpr (MASK == 1) t = b.m[i] > 0.f ? t : 0.f;
+            if constexpr (MASK == 2) t = ((b.w[i] >> (lane & 31)) & 1u) ? t : 0.f;
             stage[i * kStageStride + lane] = t;
         }
     }
 }
 
-template <int NT, int NW, bool VEC, bool MASK>
+template <int NT, int NW, bool VEC, int MASK>
 __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void dense_rows_k(const float *__restrict__ a, const float *__restrict__ mask,
+                                                       const unsigned *__restrict__ bits_in,
+                                                       unsigned *__restrict__ bits_out,
                                                        const float *__restrict__ w, int64_t wk, int64_t wc,
                                                        const float *__restrict__ bias,
                                                        const float *__restrict__ scale,
@@ -120,7 +134,8 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void dense_rows_k(const f
     int q = 0;
     bool have = tile < ntiles;
     RowBlock<VEC, MASK> blk;
-    if (have) rows_issue<VEC, MASK>(blk, a, mask, tile, 0, N, K, lane);
+    const int Win = (K + 31) >> 5, Wout = (C + 31) >> 5;
+    if (have) rows_issue<VEC, MASK>(blk, a, mask, bits_in, Win, tile, 0, N, K, lane);
     f32x16 acc[NT];
 #pragma unroll
     for (int j = 0; j < NT; ++j)
@@ -134,7 +149,7 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void dense_rows_k(const f
         int nq = q + kDenseChunk;
         if (nq >= Kpad) { nq = 0; ntile += stride; }
         const bool nhave = ntile < ntiles;
-        if (nhave) rows_issue<VEC, MASK>(blk, a, mask, ntile, nq, N, K, lane);
+        if (nhave) rows_issue<VEC, MASK>(blk, a, mask, bits_in, Win, ntile, nq, N, K, lane);
         const float *xs = stage + n * kStageStride + h * 32;
         const float *sl = slab + ((size_t)((q + h * 32) >> 2) * NC + n) * 4;
 #pragma unroll
@@ -154,13 +169,24 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void dense_rows_k(const f
 #pragma unroll
             for (int j = 0; j < NT; ++j) {
                 const int c = col0 + j * 32 + n;
+                unsigned word = 0u;
 #pragma unroll
                 for (int i = 0; i < 16; ++i) {
                     const int64_t r = tile * 32 + 8 * (i / 4) + 4 * h + (i % 4);
                     float v = acc[j][i] + bia[j];
                     if (relu) v = fmaxf(v, 0.f);
                     if (c < C && r < N) out[r * C + c] = v * scl[j] + shf[j];
+                    if (bits_out) {
+                        // one ballot = the 32 columns of this block for row i of either lane half; lane i keeps it
+                        const unsigned long long pos = __builtin_amdgcn_ballot_w64(c < C && v > 0.f);
+                        const unsigned mine = h ? (unsigned)(pos >> 32) : (unsigned)pos;
+                        word = (n == i) ? mine : word;
+                    }
                     acc[j][i] = 0.f;
+                }
+                if (bits_out && n < 16) {
+                    const int64_t r = tile * 32 + 8 * (n / 4) + 4 * h + (n % 4);
+                    if (r < N && (col0 >> 5) + j < Wout) bits_out[r * Wout + (col0 >> 5) + j] = word;
                 }
             }
         }
@@ -169,34 +195,37 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void dense_rows_k(const f
 }
 
 // U row pairs of the weight-gradient kernel in registers: lane half h holds row base + 2u + h.
-template <int TA, int TB, int U, bool MASK> struct PairBlock {
+template <int TA, int TB, int U, int MASK> struct PairBlock {
     Pack<TA> xa[U];
     Pack<TB> gz[U];
-    Pack<MASK ? TB : 1> yy[U];
+    Pack<MASK == 1 ? TB : 1> yy[U];
+    unsigned yw[MASK == 2 ? U : 1];
 };
 
 // `base` is uniform over the wavefront, so every row pair costs one scalar base per array and the lanes share
 // one 32-bit offset; FULL skips the row bound.
-template <int TA, int TB, int U, bool VEC, bool MASK, bool FULL>
+template <int TA, int TB, int U, bool VEC, int MASK, bool FULL>
 __device__ __forceinline__ void pairs_issue(PairBlock<TA, TB, U, MASK> &blk, const float *__restrict__ x,
-                                            const float *__restrict__ g, const float *__restrict__ y, int64_t base,
-                                            int64_t r1, int h, int Ci, int Co, int ci0, int co0)
+                                            const float *__restrict__ g, const float *__restrict__ y,
+                                            const unsigned *__restrict__ bits, int64_t base, int64_t r1, int h, int Ci,
+                                            int Co, int ci0, int co0)
 {
-    const int xo = h * Ci + ci0, go = h * Co + co0;
+    const int xo = h * Ci + ci0, go = h * Co + co0, W = (Co + 31) >> 5, wo = h * W + (co0 >> 5);
 #pragma unroll
     for (int u = 0; u < U; ++u) {
         const float *xu = x + (base + 2 * u) * Ci;
         const float *gu = g + (base + 2 * u) * Co;
-        const float *yu = MASK ? y + (base + 2 * u) * Co : nullptr;
+        const float *yu = MASK == 1 ? y + (base + 2 * u) * Co : nullptr;
         const bool live = FULL || base + 2 * u + h < r1;
         blk.xa[u] = zero_pack<TA>();
         blk.gz[u] = zero_pack<TB>();
-        blk.yy[u] = zero_pack<MASK ? TB : 1>();
+        blk.yy[u] = zero_pack<MASK == 1 ? TB : 1>();
+        if constexpr (MASK == 2) blk.yw[u] = (live && co0 < Co) ? bits[(base + 2 * u) * W + wo] : 0u;
         if constexpr (VEC) {
             if (live && ci0 < Ci) blk.xa[u] = ldp<TA>(xu + xo);
             if (live && co0 < Co) {
                 blk.gz[u] = ldp<TB>(gu + go);
-                if constexpr (MASK) blk.yy[u] = ldp<TB>(yu + go);
+                if constexpr (MASK == 1) blk.yy[u] = ldp<TB>(yu + go);
             }
         } else {
 #pragma unroll
@@ -206,7 +235,7 @@ __device__ __forceinline__ void pairs_issue(PairBlock<TA, TB, U, MASK> &blk, con
             for (int jb = 0; jb < TB; ++jb)
                 if (live && co0 + jb < Co) {
                     blk.gz[u].v[jb] = gu[go + jb];
-                    if constexpr (MASK) blk.yy[u].v[jb] = yu[go + jb];
+                    if constexpr (MASK == 1) blk.yy[u].v[jb] = yu[go + jb];
                 }
         }
     }
@@ -217,9 +246,10 @@ __device__ __forceinline__ void pairs_issue(PairBlock<TA, TB, U, MASK> &blk, con
 // (lane half h takes row 2t + h), lane (m, h) supplies TA input channels and TB output channels that lie
 // contiguously in its rows, and a wavefront keeps TA x TB tiles of 32 x 32 sums.  Every workgroup leaves one
 // partial of (Ci + 1) * Co floats (row Ci = bias gradient); blockIdx.y walks the channel chunks.
-template <int TA, int TB, bool VEC, bool MASK>
+template <int TA, int TB, bool VEC, int MASK>
 __global__ __launch_bounds__(256, 2) void dense_wgrad_k(const float *__restrict__ x, const float *__restrict__ g,
-                                                        const float *__restrict__ y, float *__restrict__ partial,
+                                                        const float *__restrict__ y,
+                                                        const unsigned *__restrict__ bits, float *__restrict__ partial,
                                                         int64_t N, int Ci, int Co, int nA, int64_t rows_per_wave)
 {
     __shared__ float red[TA * TB * 16 * 64];
@@ -245,15 +275,16 @@ __global__ __launch_bounds__(256, 2) void dense_wgrad_k(const float *__restrict_
     constexpr int U = 8;
     PairBlock<TA, TB, U, MASK> blk;
     for (int64_t base = r0; base < r1; base += 2 * U) {
-        if (base + 2 * U <= r1) pairs_issue<TA, TB, U, VEC, MASK, true>(blk, x, g, y, base, r1, h, Ci, Co, ci0, co0);
-        else pairs_issue<TA, TB, U, VEC, MASK, false>(blk, x, g, y, base, r1, h, Ci, Co, ci0, co0);
+        if (base + 2 * U <= r1) pairs_issue<TA, TB, U, VEC, MASK, true>(blk, x, g, y, bits, base, r1, h, Ci, Co, ci0, co0);
+        else pairs_issue<TA, TB, U, VEC, MASK, false>(blk, x, g, y, bits, base, r1, h, Ci, Co, ci0, co0);
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             float gzv[TB];
 #pragma unroll
             for (int jb = 0; jb < TB; ++jb) {
                 gzv[jb] = blk.gz[u].v[jb];
-                if constexpr (MASK) gzv[jb] = blk.yy[u].v[jb] > 0.f ? gzv[jb] : 0.f;
+                if constexpr (MASK == 1) gzv[jb] = blk.yy[u].v[jb] > 0.f ? gzv[jb] : 0.f;
+                if constexpr (MASK == 2) gzv[jb] = ((blk.yw[u] >> ((co0 & 31) + jb)) & 1u) ? gzv[jb] : 0.f;
                 gb[jb] += gzv[jb];
             }
 #pragma unroll
@@ -304,19 +335,34 @@ template <int V>
 __global__ __launch_bounds__(256) void bias_act_fwd_k(const float *__restrict__ x, const float *__restrict__ bias,
                                                       const float *__restrict__ scale,
                                                       const float *__restrict__ shift, int relu,
-                                                      float *__restrict__ out, int64_t n_items, int items)
+                                                      float *__restrict__ out, unsigned *__restrict__ bits_out,
+                                                      int64_t n_items, int items)
 {
     const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (i >= n_items) return;
-    const int c = (int)(i % items) * V;
-    Pack<V> v = ldp<V>(x + i * V);
+    const bool live = i < n_items;
+    unsigned nib = 0u;
+    if (live) {
+        const int c = (int)(i % items) * V;
+        Pack<V> v = ldp<V>(x + i * V);
 #pragma unroll
-    for (int j = 0; j < V; ++j) {
-        float t = v.v[j] + (bias ? bias[c + j] : 0.f);
-        if (relu) t = fmaxf(t, 0.f);
-        v.v[j] = t * (scale ? scale[c + j] : 1.f) + (shift ? shift[c + j] : 0.f);
+        for (int j = 0; j < V; ++j) {
+            float t = v.v[j] + (bias ? bias[c + j] : 0.f);
+            if (relu) t = fmaxf(t, 0.f);
+            nib |= (t > 0.f ? 1u : 0u) << j;
+            v.v[j] = t * (scale ? scale[c + j] : 1.f) + (shift ? shift[c + j] : 0.f);
+        }
+        stp<V>(out + i * V, v);
     }
-    stp<V>(out + i * V, v);
+    if constexpr (V == 4) {
+        // eight neighbouring lanes hold the 32 columns of one mask word (rows are multiples of 32 columns here)
+        if (bits_out) {
+            unsigned word = nib << (4 * (threadIdx.x & 7));
+            word |= __shfl_xor(word, 1);
+            word |= __shfl_xor(word, 2);
+            word |= __shfl_xor(word, 4);
+            if (live && (threadIdx.x & 7) == 0) bits_out[i >> 3] = word;
+        }
+    }
 }
 
 // Its gradient: gin = g where y > 0 (MASK; skipped when gin is null), partial[block][c] = the block's column sums
@@ -324,9 +370,10 @@ __global__ __launch_bounds__(256) void bias_act_fwd_k(const float *__restrict__ 
 // kBiasLoops times), 256 / lpr rows in flight; the row slots add up in slot order.
 constexpr int kBiasLoops = 4;
 
-template <int V, bool MASK>
+template <int V, int MASK>
 __global__ __launch_bounds__(256) void bias_act_bwd_k(const float *__restrict__ g, const float *__restrict__ y,
-                                                      float *__restrict__ gin, float *__restrict__ partial,
+                                                      const unsigned *__restrict__ bits, float *__restrict__ gin,
+                                                      float *__restrict__ partial,
                                                       int64_t N, int C, int lpr, int64_t rows_per_block)
 {
     __shared__ float red[256 * kBiasLoops * V];
@@ -344,10 +391,17 @@ __global__ __launch_bounds__(256) void bias_act_bwd_k(const float *__restrict__ 
             if (cv < items) {
                 const int64_t o = row * C + (int64_t)cv * V;
                 Pack<V> gz = ldp<V>(g + o);
-                if constexpr (MASK) {
+                if constexpr (MASK == 1) {
                     const Pack<V> yy = ldp<V>(y + o);
 #pragma unroll
                     for (int j = 0; j < V; ++j) gz.v[j] = yy.v[j] > 0.f ? gz.v[j] : 0.f;
+                    if (gin) stp<V>(gin + o, gz);
+                }
+                if constexpr (MASK == 2) {
+                    // V == 4 and C % 32 == 0: word cv / 8 of the row, nibble cv % 8
+                    const unsigned nib = bits[row * (C >> 5) + (cv >> 3)] >> (4 * (cv & 7));
+#pragma unroll
+                    for (int j = 0; j < V; ++j) gz.v[j] = ((nib >> j) & 1u) ? gz.v[j] : 0.f;
                     if (gin) stp<V>(gin + o, gz);
                 }
 #pragma unroll
@@ -403,10 +457,21 @@ static int rows_tiles(int Kpad, int C, int slab_floats)
 
 // Launch with as many workgroups as are resident at once (every tile is independent, so the count only
 // balances the load): a grid that needs a second round of workgroups would run that round at low occupancy.
-template <int NT, int NW, bool VEC, bool MASK>
-static void launch_rows_nt(int64_t ntiles, unsigned gy, size_t lds, hipStream_t st, const float *a, const float *mask,
-                           const float *w, int64_t wk, int64_t wc, const float *bias, const float *scale,
-                           const float *shift, int relu, float *out, int64_t N, int K, int Kpad, int C)
+struct RowsArgs {
+    const float *a, *mask;
+    const unsigned *bits_in;
+    unsigned *bits_out;
+    const float *w;
+    int64_t wk, wc;
+    const float *bias, *scale, *shift;
+    int relu;
+    float *out;
+    int64_t N;
+    int K, Kpad, C;
+};
+
+template <int NT, int NW, bool VEC, int MASK>
+static void launch_rows_nt(int64_t ntiles, unsigned gy, size_t lds, hipStream_t st, const RowsArgs &p)
 {
     const void *fn = reinterpret_cast<const void *>(dense_rows_k<NT, NW, VEC, MASK>);
     if (lds > 65536) (void)hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -418,16 +483,14 @@ static void launch_rows_nt(int64_t ntiles, unsigned gy, size_t lds, hipStream_t 
     const int64_t wanted = ceil_div(ntiles, NW);
     if (gx < 1) gx = 1;
     if (gx > wanted) gx = wanted;
-    dense_rows_k<NT, NW, VEC, MASK><<<dim3((unsigned)gx, gy), dim3(NW * 64), lds, st>>>(a, mask, w, wk, wc, bias, scale,
-                                                                                        shift, relu, out, N, K, Kpad, C);
+    dense_rows_k<NT, NW, VEC, MASK><<<dim3((unsigned)gx, gy), dim3(NW * 64), lds, st>>>(
+        p.a, p.mask, p.bits_in, p.bits_out, p.w, p.wk, p.wc, p.bias, p.scale, p.shift, p.relu, p.out, p.N, p.K, p.Kpad, p.C);
 }
 
-template <bool VEC, bool MASK>
-static void launch_rows(int NT, int NW, int64_t ntiles, unsigned gy, size_t lds, hipStream_t st, const float *a,
-                        const float *mask, const float *w, int64_t wk, int64_t wc, const float *bias, const float *scale,
-                        const float *shift, int relu, float *out, int64_t N, int K, int Kpad, int C)
+template <bool VEC, int MASK>
+static void launch_rows(int NT, int NW, int64_t ntiles, unsigned gy, size_t lds, hipStream_t st, const RowsArgs &p)
 {
-#define PM_ROWS(T, W) launch_rows_nt<T, W, VEC, MASK>(ntiles, gy, lds, st, a, mask, w, wk, wc, bias, scale, shift, relu, out, N, K, Kpad, C)
+#define PM_ROWS(T, W) launch_rows_nt<T, W, VEC, MASK>(ntiles, gy, lds, st, p)
     if (NW == 8) {
         switch (NT) {
         case 4: PM_ROWS(4, 8); break;
@@ -444,10 +507,11 @@ static void launch_rows(int NT, int NW, int64_t ntiles, unsigned gy, size_t lds,
 #undef PM_ROWS
 }
 
-// out (N x C) = act(a' (N x K) . Wm + bias) * scale + shift, a' = a masked by mask > 0 when mask is given.
-static int dense_rows(const char *name, const float *a, const float *mask, const float *w, int64_t wk, int64_t wc,
-                      const float *bias, const float *scale, const float *shift, int relu, float *out, int64_t N, int K,
-                      int C, hipStream_t st)
+// out (N x C) = act(a' (N x K) . Wm + bias) * scale + shift; a' = a masked by mask > 0 (float array) or by
+// bits_in (one bit per entry) when given; bits_out receives one bit per output entry, set where act(.) > 0.
+static int dense_rows(const char *name, const float *a, const float *mask, const unsigned *bits_in, unsigned *bits_out,
+                      const float *w, int64_t wk, int64_t wc, const float *bias, const float *scale, const float *shift,
+                      int relu, float *out, int64_t N, int K, int C, hipStream_t st)
 {
     PM_REQUIRE(K > 0 && C > 0 && K <= kDenseMaxK && C <= (1 << 20), "%s: channel counts out of range (%d, %d)", name, K, C);
     PM_REQUIRE(N * (int64_t)(K > C ? K : C) < (int64_t(1) << 40), "%s: sizes too large", name);
@@ -465,12 +529,16 @@ static int dense_rows(const char *name, const float *a, const float *mask, const
     const int64_t ntiles = ceil_div(N, 32);
     const unsigned gy = (unsigned)ceil_div(C, NT * 32);
     const bool vec = (K % 4 == 0) && aligned16(a) && (!mask || aligned16(mask));
+    const RowsArgs p{a, mask, bits_in, bits_out, w, wk, wc, bias, scale, shift, relu, out, N, K, Kpad, C};
+    const int mode = bits_in ? 2 : mask ? 1 : 0;
     if (vec) {
-        if (mask) launch_rows<true, true>(NT, NW, ntiles, gy, lds, st, a, mask, w, wk, wc, bias, scale, shift, relu, out, N, K, Kpad, C);
-        else launch_rows<true, false>(NT, NW, ntiles, gy, lds, st, a, mask, w, wk, wc, bias, scale, shift, relu, out, N, K, Kpad, C);
+        if (mode == 2) launch_rows<true, 2>(NT, NW, ntiles, gy, lds, st, p);
+        else if (mode == 1) launch_rows<true, 1>(NT, NW, ntiles, gy, lds, st, p);
+        else launch_rows<true, 0>(NT, NW, ntiles, gy, lds, st, p);
     } else {
-        if (mask) launch_rows<false, true>(NT, NW, ntiles, gy, lds, st, a, mask, w, wk, wc, bias, scale, shift, relu, out, N, K, Kpad, C);
-        else launch_rows<false, false>(NT, NW, ntiles, gy, lds, st, a, mask, w, wk, wc, bias, scale, shift, relu, out, N, K, Kpad, C);
+        if (mode == 2) launch_rows<false, 2>(NT, NW, ntiles, gy, lds, st, p);
+        else if (mode == 1) launch_rows<false, 1>(NT, NW, ntiles, gy, lds, st, p);
+        else launch_rows<false, 0>(NT, NW, ntiles, gy, lds, st, p);
     }
     PM_LAUNCHED(name);
     return 0;
@@ -505,16 +573,20 @@ static WgradPlan wgrad_plan(int64_t N, int Ci, int Co)
 }
 
 template <int TA, int TB>
-static void launch_wgrad(bool vec, bool mask, dim3 grid, hipStream_t st, const float *x, const float *g, const float *y,
-                         float *partial, int64_t N, int Ci, int Co, int nA, int64_t rpw)
+static void launch_wgrad(bool vec, int mode, dim3 grid, hipStream_t st, const float *x, const float *g, const float *y,
+                         const unsigned *bits, float *partial, int64_t N, int Ci, int Co, int nA, int64_t rpw)
 {
+#define PM_WGK(V, M) dense_wgrad_k<TA, TB, V, M><<<grid, dim3(256), 0, st>>>(x, g, y, bits, partial, N, Ci, Co, nA, rpw)
     if (vec) {
-        if (mask) dense_wgrad_k<TA, TB, true, true><<<grid, dim3(256), 0, st>>>(x, g, y, partial, N, Ci, Co, nA, rpw);
-        else dense_wgrad_k<TA, TB, true, false><<<grid, dim3(256), 0, st>>>(x, g, y, partial, N, Ci, Co, nA, rpw);
+        if (mode == 2) PM_WGK(true, 2);
+        else if (mode == 1) PM_WGK(true, 1);
+        else PM_WGK(true, 0);
     } else {
-        if (mask) dense_wgrad_k<TA, TB, false, true><<<grid, dim3(256), 0, st>>>(x, g, y, partial, N, Ci, Co, nA, rpw);
-        else dense_wgrad_k<TA, TB, false, false><<<grid, dim3(256), 0, st>>>(x, g, y, partial, N, Ci, Co, nA, rpw);
+        if (mode == 2) PM_WGK(false, 2);
+        else if (mode == 1) PM_WGK(false, 1);
+        else PM_WGK(false, 0);
     }
+#undef PM_WGK
 }
 
 }  // namespace pmesh
@@ -522,15 +594,15 @@ static void launch_wgrad(bool vec, bool mask, dim3 grid, hipStream_t st, const f
 using namespace pmesh;
 
 extern "C" int pmesh_dense_fwd(const float *input, const float *weight, const float *bias, const float *scale,
-                               const float *shift, int relu, float *output, int64_t N, int Ci, int Co,
-                               pmesh_stream_t stream)
+                               const float *shift, int relu, float *output, uint32_t *relu_bits, int64_t N, int Ci,
+                               int Co, pmesh_stream_t stream)
 {
     clear_error();
     PM_REQUIRE(N >= 0, "dense_fwd: negative size");
     if (N == 0) return 0;
     PM_REQUIRE(input && weight && output, "dense_fwd: null pointer");
-    return dense_rows("dense_fwd", input, nullptr, weight, Co, 1, bias, scale, shift, relu, output, N, Ci, Co,
-                      (hipStream_t)stream);
+    return dense_rows("dense_fwd", input, nullptr, nullptr, relu_bits, weight, Co, 1, bias, scale, shift, relu, output, N,
+                      Ci, Co, (hipStream_t)stream);
 }
 
 extern "C" size_t pmesh_dense_bwd_workspace_bytes(int64_t N, int Ci, int Co)
@@ -541,8 +613,8 @@ extern "C" size_t pmesh_dense_bwd_workspace_bytes(int64_t N, int Ci, int Co)
 }
 
 extern "C" int pmesh_dense_bwd(const float *grad_output, const float *input, const float *weight, const float *output,
-                               float *grad_input, float *grad_weight, float *grad_bias, void *workspace,
-                               size_t workspace_bytes, int64_t N, int Ci, int Co, pmesh_stream_t stream)
+                               const uint32_t *relu_bits, float *grad_input, float *grad_weight, float *grad_bias,
+                               void *workspace, size_t workspace_bytes, int64_t N, int Ci, int Co, pmesh_stream_t stream)
 {
     clear_error();
     PM_REQUIRE(N >= 0 && Ci > 0 && Co > 0, "dense_bwd: bad sizes");
@@ -554,10 +626,11 @@ extern "C" int pmesh_dense_bwd(const float *grad_output, const float *input, con
     }
     PM_REQUIRE(grad_output && input && weight && workspace, "dense_bwd: null pointer");
     PM_REQUIRE((int64_t)Ci * Co <= (int64_t(1) << 24), "dense_bwd: weight too large");
+    if (relu_bits) output = nullptr;          // the bits are the cheaper form of the same mask
     if (grad_input) {
         // grad_input (N x Ci) = gz (N x Co) . W^T: element (k = co, c = ci) of the matrix is weight[ci * Co + co]
-        const int rc = dense_rows("dense_bwd(input)", grad_output, output, weight, 1, Co, nullptr, nullptr, nullptr, 0,
-                                  grad_input, N, Co, Ci, st);
+        const int rc = dense_rows("dense_bwd(input)", grad_output, output, relu_bits, nullptr, weight, 1, Co, nullptr,
+                                  nullptr, nullptr, 0, grad_input, N, Co, Ci, st);
         if (rc) return rc;
     }
     const WgradPlan p = wgrad_plan(N, Ci, Co);
@@ -569,8 +642,8 @@ extern "C" int pmesh_dense_bwd(const float *grad_output, const float *input, con
     const bool vec = Ci % p.ta == 0 && Co % p.tb == 0 && aligned16(input) && aligned16(grad_output) &&
                      (!output || aligned16(output));
     const dim3 grid((unsigned)p.G, (unsigned)(p.nA * p.nB));
-    const bool mask = output != nullptr;
-#define PM_WG(A, B) launch_wgrad<A, B>(vec, mask, grid, st, input, grad_output, output, partial, N, Ci, Co, p.nA, p.rows_per_wave)
+    const int mode = relu_bits ? 2 : output ? 1 : 0;
+#define PM_WG(A, B) launch_wgrad<A, B>(vec, mode, grid, st, input, grad_output, output, relu_bits, partial, N, Ci, Co, p.nA, p.rows_per_wave)
     if (p.ta == 4 && p.tb == 2) PM_WG(4, 2);
     else if (p.ta == 4 && p.tb == 1) PM_WG(4, 1);
     else if (p.ta == 2 && p.tb == 4) PM_WG(2, 4);
@@ -587,7 +660,7 @@ extern "C" int pmesh_dense_bwd(const float *grad_output, const float *input, con
 }
 
 extern "C" int pmesh_bias_act_fwd(const float *input, const float *bias, const float *scale, const float *shift,
-                                  int relu, float *output, int64_t N, int C, pmesh_stream_t stream)
+                                  int relu, float *output, uint32_t *relu_bits, int64_t N, int C, pmesh_stream_t stream)
 {
     clear_error();
     PM_REQUIRE(N >= 0 && C > 0, "bias_act_fwd: bad sizes");
@@ -595,16 +668,17 @@ extern "C" int pmesh_bias_act_fwd(const float *input, const float *bias, const f
     PM_REQUIRE(input && output, "bias_act_fwd: null pointer");
     PM_REQUIRE(N * (int64_t)C < (int64_t(1) << 40), "bias_act_fwd: sizes too large");
     const bool v4 = C % 4 == 0 && aligned16(input) && aligned16(output);
+    PM_REQUIRE(!relu_bits || (v4 && C % 32 == 0), "bias_act_fwd: the bit mask needs C %% 32 == 0 and 16-byte aligned rows");
     const int V = v4 ? 4 : 1;
     const int64_t n_items = N * C / V;
     const int64_t blocks = ceil_div(n_items, 256);
     PM_REQUIRE(grid_ok(blocks), "bias_act_fwd: grid too large");
     if (v4)
         bias_act_fwd_k<4><<<dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream>>>(input, bias, scale, shift, relu,
-                                                                                          output, n_items, C / 4);
+                                                                                          output, relu_bits, n_items, C / 4);
     else
         bias_act_fwd_k<1><<<dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream>>>(input, bias, scale, shift, relu,
-                                                                                          output, n_items, C);
+                                                                                          output, nullptr, n_items, C);
     PM_LAUNCHED("bias_act_fwd");
     return 0;
 }
@@ -614,8 +688,9 @@ extern "C" size_t pmesh_bias_act_bwd_workspace_bytes(int C)
     return (size_t)1024 * (size_t)(C > 0 ? C : 1) * sizeof(float);
 }
 
-extern "C" int pmesh_bias_act_bwd(const float *grad_output, const float *output, float *grad_input, float *grad_bias,
-                                  void *workspace, size_t workspace_bytes, int64_t N, int C, pmesh_stream_t stream)
+extern "C" int pmesh_bias_act_bwd(const float *grad_output, const float *output, const uint32_t *relu_bits,
+                                  float *grad_input, float *grad_bias, void *workspace, size_t workspace_bytes, int64_t N,
+                                  int C, pmesh_stream_t stream)
 {
     clear_error();
     PM_REQUIRE(N >= 0 && C > 0, "bias_act_bwd: bad sizes");
@@ -623,21 +698,24 @@ extern "C" int pmesh_bias_act_bwd(const float *grad_output, const float *output,
     hipStream_t st = (hipStream_t)stream;
     if (N == 0) return reduce_partials(nullptr, grad_bias, 0, C, st);
     PM_REQUIRE(grad_output && workspace, "bias_act_bwd: null pointer");
-    PM_REQUIRE(!grad_input || output, "bias_act_bwd: grad_input is grad_output itself when there is no activation");
+    if (relu_bits) output = nullptr;
+    PM_REQUIRE(!grad_input || output || relu_bits, "bias_act_bwd: grad_input is grad_output itself when there is no activation");
     PM_REQUIRE(N * (int64_t)C < (int64_t(1) << 40), "bias_act_bwd: sizes too large");
     const bool aligned = aligned16(grad_output) && (!output || aligned16(output)) && (!grad_input || aligned16(grad_input));
     const BiasPlan p = bias_plan(N, C, aligned);
+    PM_REQUIRE(!relu_bits || (p.V == 4 && C % 32 == 0), "bias_act_bwd: the bit mask needs C %% 32 == 0 and 16-byte aligned rows");
     PM_REQUIRE(C / p.V <= 256 * kBiasLoops, "bias_act_bwd: more than %d channels", 256 * kBiasLoops * p.V);
     PM_REQUIRE(workspace_bytes >= (size_t)p.G * C * sizeof(float), "bias_act_bwd: workspace too small (%zu bytes)",
                workspace_bytes);
     float *partial = (float *)workspace;
     const dim3 grid((unsigned)p.G), block(256);
     if (p.V == 4) {
-        if (output) bias_act_bwd_k<4, true><<<grid, block, 0, st>>>(grad_output, output, grad_input, partial, N, C, p.lpr, p.rows_per_block);
-        else bias_act_bwd_k<4, false><<<grid, block, 0, st>>>(grad_output, output, grad_input, partial, N, C, p.lpr, p.rows_per_block);
+        if (relu_bits) bias_act_bwd_k<4, 2><<<grid, block, 0, st>>>(grad_output, output, relu_bits, grad_input, partial, N, C, p.lpr, p.rows_per_block);
+        else if (output) bias_act_bwd_k<4, 1><<<grid, block, 0, st>>>(grad_output, output, relu_bits, grad_input, partial, N, C, p.lpr, p.rows_per_block);
+        else bias_act_bwd_k<4, 0><<<grid, block, 0, st>>>(grad_output, output, relu_bits, grad_input, partial, N, C, p.lpr, p.rows_per_block);
     } else {
-        if (output) bias_act_bwd_k<1, true><<<grid, block, 0, st>>>(grad_output, output, grad_input, partial, N, C, p.lpr, p.rows_per_block);
-        else bias_act_bwd_k<1, false><<<grid, block, 0, st>>>(grad_output, output, grad_input, partial, N, C, p.lpr, p.rows_per_block);
+        if (output) bias_act_bwd_k<1, 1><<<grid, block, 0, st>>>(grad_output, output, relu_bits, grad_input, partial, N, C, p.lpr, p.rows_per_block);
+        else bias_act_bwd_k<1, 0><<<grid, block, 0, st>>>(grad_output, output, relu_bits, grad_input, partial, N, C, p.lpr, p.rows_per_block);
     }
     PM_LAUNCHED("bias_act_bwd");
     return reduce_partials(partial, grad_bias, p.G, C, st);

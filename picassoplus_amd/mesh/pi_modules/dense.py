@@ -32,8 +32,10 @@ def _ptr(t):
     return 0 if t is None else t.data_ptr()
 
 
-def dense_tail_forward(input, weight, bias=None, relu=True, scale=None, shift=None):
-    """(N,Ci),(Ci,Co),(Co,) -> act(input @ weight + bias) * scale + shift, float32 (N,Co)."""
+def dense_tail_forward(input, weight, bias=None, relu=True, scale=None, shift=None, with_bits=False):
+    """(N,Ci),(Ci,Co),(Co,) -> act(input @ weight + bias) * scale + shift, float32 (N,Co).
+    ``with_bits`` also returns the ReLU mask as bits: int32 (N, ceil(Co/32)), bit c%32 of word c//32 set where
+    the activated value is positive -- what ``dense_tail_backward`` reads instead of the whole output."""
     N, Ci, Co = _dims(input, weight, bias)
     for name, t in (("scale", scale), ("shift", shift)):
         if t is not None:
@@ -43,14 +45,16 @@ def dense_tail_forward(input, weight, bias=None, relu=True, scale=None, shift=No
     dev = same_device(input, weight, *[t for t in (bias, scale, shift) if t is not None])
     with torch.cuda.device(dev):
         out = torch.empty((N, Co), dtype=F32, device=dev)
+        bits = torch.empty((N, (Co + 31) // 32), dtype=torch.int32, device=dev) if with_bits else None
         _lib.call("pmesh_dense_fwd", input.data_ptr(), weight.data_ptr(), _ptr(bias), _ptr(scale), _ptr(shift),
-                  1 if relu else 0, out.data_ptr(), N, Ci, Co, stream_of(input))
-    return out
+                  1 if relu else 0, out.data_ptr(), _ptr(bits), N, Ci, Co, stream_of(input))
+    return (out, bits) if with_bits else out
 
 
-def dense_tail_backward(grad_output, input, weight, output=None, need_input=True):
+def dense_tail_backward(grad_output, input, weight, output=None, need_input=True, relu_bits=None):
     """Gradients of ``act(input @ weight + bias)``: ``output`` is the forward result when the activation
-    was ReLU (its positive entries pass the gradient), None for no activation.
+    was ReLU (its positive entries pass the gradient), or ``relu_bits`` the bit form of the same mask from
+    ``dense_tail_forward(..., with_bits=True)``; both None for no activation.
     -> [grad_input (N,Ci) or None, grad_weight (Ci,Co), grad_bias (Co,)]."""
     N, Ci, Co = _dims(input, weight, None)
     check_input(grad_output, "grad_output", 2, F32)
@@ -60,6 +64,10 @@ def dense_tail_backward(grad_output, input, weight, output=None, need_input=True
         check_input(output, "output", 2, F32)
         if tuple(output.shape) != (N, Co):
             raise RuntimeError("output must have shape (N, out_channels)")
+    if relu_bits is not None:
+        check_input(relu_bits, "relu_bits", 2, torch.int32)
+        if tuple(relu_bits.shape) != (N, (Co + 31) // 32):
+            raise RuntimeError("relu_bits must have shape (N, ceil(out_channels / 32))")
     dev = same_device(grad_output, input, weight)
     with torch.cuda.device(dev):
         gin = torch.empty((N, Ci), dtype=F32, device=dev) if need_input else None
@@ -68,7 +76,7 @@ def dense_tail_backward(grad_output, input, weight, output=None, need_input=True
         nbytes = _lib.query("pmesh_dense_bwd_workspace_bytes", N, Ci, Co)
         ws = workspace(nbytes, dev)
         _lib.call("pmesh_dense_bwd", grad_output.data_ptr(), input.data_ptr(), weight.data_ptr(), _ptr(output),
-                  _ptr(gin), gw.data_ptr(), gb.data_ptr(), ws.data_ptr(), nbytes, N, Ci, Co, stream_of(input))
+                  _ptr(relu_bits), _ptr(gin), gw.data_ptr(), gb.data_ptr(), ws.data_ptr(), nbytes, N, Ci, Co, stream_of(input))
     return [gin, gw, gb]
 
 
@@ -77,16 +85,19 @@ class DenseTailFunction(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, input, weight, bias, relu):
-        out = dense_tail_forward(input, weight, bias, relu)
-        ctx.relu = bool(relu)
-        ctx.save_for_backward(input, weight, out if relu else None)
+        # the backward pass reads the ReLU mask as bits (1/32 of the output) instead of the output
+        if relu:
+            out, bits = dense_tail_forward(input, weight, bias, True, with_bits=True)
+        else:
+            out, bits = dense_tail_forward(input, weight, bias, False), None
+        ctx.save_for_backward(input, weight, bits)
         return out
 
     @staticmethod
     def backward(ctx, grad_output):
-        input, weight, out = ctx.saved_tensors
-        gin, gw, gb = dense_tail_backward(grad_output.contiguous(), input, weight, out if ctx.relu else None,
-                                          need_input=ctx.needs_input_grad[0])
+        input, weight, bits = ctx.saved_tensors
+        gin, gw, gb = dense_tail_backward(grad_output.contiguous(), input, weight, None,
+                                          need_input=ctx.needs_input_grad[0], relu_bits=bits)
         return gin, gw if ctx.needs_input_grad[1] else None, gb if ctx.needs_input_grad[2] else None, None
 
 
@@ -96,11 +107,19 @@ def dense_tail(input, weight, bias, relu=True):
 
 
 # ---------------------------------------------------------------- the tail without a product
-def bias_act_forward(input, bias=None, relu=True, scale=None, shift=None):
+def bits_supported(C, *tensors):
+    """The bit form of the ReLU mask of ``bias_act`` needs whole 32-column words and 16-byte aligned rows."""
+    return C % 32 == 0 and all(t.data_ptr() % 16 == 0 for t in tensors)
+
+
+def bias_act_forward(input, bias=None, relu=True, scale=None, shift=None, with_bits=False):
     """act(input + bias) * scale + shift for a convolution that mixes the channels itself (F2FConv3d,
-    picasso/mesh/layers.py:60-64), one pass, float32 (N,C)."""
+    picasso/mesh/layers.py:60-64), one pass, float32 (N,C).  ``with_bits`` (C % 32 == 0) also returns the
+    ReLU mask as bits, int32 (N, C/32), as ``dense_tail_forward`` does."""
     check_input(input, "input", 2, F32)
     N, C = input.shape
+    if with_bits and not bits_supported(C, input):
+        raise RuntimeError("the bit mask needs a multiple of 32 channels and 16-byte aligned rows")
     for name, t in (("bias", bias), ("scale", scale), ("shift", shift)):
         if t is not None:
             check_input(t, name, 1, F32)
@@ -109,30 +128,37 @@ def bias_act_forward(input, bias=None, relu=True, scale=None, shift=None):
     dev = same_device(input, *[t for t in (bias, scale, shift) if t is not None])
     with torch.cuda.device(dev):
         out = torch.empty((N, C), dtype=F32, device=dev)
+        bits = torch.empty((N, C // 32), dtype=torch.int32, device=dev) if with_bits else None
         if C:
             _lib.call("pmesh_bias_act_fwd", input.data_ptr(), _ptr(bias), _ptr(scale), _ptr(shift), 1 if relu else 0,
-                      out.data_ptr(), N, C, stream_of(input))
-    return out
+                      out.data_ptr(), _ptr(bits), N, C, stream_of(input))
+    return (out, bits) if with_bits else out
 
 
-def bias_act_backward(grad_output, output=None, need_input=True):
-    """-> [grad_input, grad_bias]: grad_input is grad_output where ``output`` > 0 (``output`` None = no activation:
-    grad_output itself), grad_bias its column sums."""
+def bias_act_backward(grad_output, output=None, need_input=True, relu_bits=None):
+    """-> [grad_input, grad_bias]: grad_input is grad_output where ``output`` > 0, or where ``relu_bits`` (the bit
+    form from ``bias_act_forward(..., with_bits=True)``) is set; both None = no activation: grad_output itself;
+    grad_bias its column sums."""
     check_input(grad_output, "grad_output", 2, F32)
     N, C = grad_output.shape
     if output is not None:
         check_input(output, "output", 2, F32)
         if tuple(output.shape) != (N, C):
             raise RuntimeError("output must have the shape of grad_output")
+    if relu_bits is not None:
+        check_input(relu_bits, "relu_bits", 2, torch.int32)
+        if C % 32 or tuple(relu_bits.shape) != (N, C // 32):
+            raise RuntimeError("relu_bits must have shape (N, channels / 32)")
+    masked = output is not None or relu_bits is not None
     dev = same_device(grad_output) if output is None else same_device(grad_output, output)
     with torch.cuda.device(dev):
-        gin = torch.empty((N, C), dtype=F32, device=dev) if (need_input and output is not None) else None
+        gin = torch.empty((N, C), dtype=F32, device=dev) if (need_input and masked) else None
         gb = torch.empty((C,), dtype=F32, device=dev)
         nbytes = _lib.query("pmesh_bias_act_bwd_workspace_bytes", C)
         ws = workspace(nbytes, dev)
-        _lib.call("pmesh_bias_act_bwd", grad_output.data_ptr(), _ptr(output), _ptr(gin), gb.data_ptr(), ws.data_ptr(),
-                  nbytes, N, C, stream_of(grad_output))
-    if output is None and need_input:
+        _lib.call("pmesh_bias_act_bwd", grad_output.data_ptr(), _ptr(output), _ptr(relu_bits), _ptr(gin), gb.data_ptr(),
+                  ws.data_ptr(), nbytes, N, C, stream_of(grad_output))
+    if not masked and need_input:
         gin = grad_output
     return [gin, gb]
 
@@ -142,16 +168,21 @@ class BiasActFunction(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, input, bias, relu):
-        out = bias_act_forward(input, bias, relu)
-        ctx.relu = bool(relu)
-        ctx.save_for_backward(out if relu else None)
+        out = bits = None
+        if relu and bits_supported(input.shape[1], input):
+            out, bits = bias_act_forward(input, bias, True, with_bits=True)
+        else:
+            out = bias_act_forward(input, bias, relu)
+        ctx.save_for_backward(out if (relu and bits is None) else None, bits)
         return out
 
     @staticmethod
     def backward(ctx, grad_output):
-        (out,) = ctx.saved_tensors
-        gin, gb = bias_act_backward(grad_output.contiguous(), out if ctx.relu else None,
-                                    need_input=ctx.needs_input_grad[0])
+        out, bits = ctx.saved_tensors
+        grad_output = grad_output.contiguous()
+        if bits is not None and grad_output.data_ptr() % 16:
+            grad_output = grad_output.clone()                  # the bit path reads 16-byte pieces
+        gin, gb = bias_act_backward(grad_output, out, need_input=ctx.needs_input_grad[0], relu_bits=bits)
         return gin, gb if ctx.needs_input_grad[1] else None, None
 
 

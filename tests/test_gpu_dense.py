@@ -60,6 +60,18 @@ def test_dense_tail_forward_backward(cuda, n, ci, co, relu):
     gx2, gw2, gb2 = dense.dense_tail_backward(god, xd, wd, out if relu else None, need_input=False)
     torch.cuda.synchronize()
     assert gx2 is None and torch.equal(gw2, gw) and torch.equal(gb2, gb)
+    if relu:
+        # the bit form of the ReLU mask: same output, bits = (out > 0), and the very same gradients from it
+        out_b, bits = dense.dense_tail_forward(xd, wd, bd, True, with_bits=True)
+        assert torch.equal(out_b, out) and bits.shape == (n, (co + 31) // 32) and bits.dtype == torch.int32
+        cols = torch.arange(co, device=cuda)
+        unpacked = (bits[:, cols // 32] >> (cols % 32)) & 1
+        assert torch.equal(unpacked.bool(), out > 0)
+        if co % 32:
+            assert int((bits[:, -1].long() & 0xFFFFFFFF).max()) < (1 << (co % 32))          # no stray bits past Co
+        gx3, gw3, gb3 = dense.dense_tail_backward(god, xd, wd, None, relu_bits=bits)
+        torch.cuda.synchronize()
+        assert torch.equal(gx3, gx) and torch.equal(gw3, gw) and torch.equal(gb3, gb)
 
 
 def test_dense_tail_frozen_norm_and_missing_operands(cuda):
@@ -187,6 +199,16 @@ def test_bias_act_forward_backward(cuda, n, c, relu):
     assert_close(gb, rb.numpy(), "bias_act grad_bias")
     gx2, gb2 = dense.bias_act_backward(god, out if relu else None, need_input=False)
     assert gx2 is None and torch.equal(gb2, gb)
+    if relu and c % 32 == 0:
+        out_b, bits = dense.bias_act_forward(xd, bd, True, with_bits=True)
+        cols = torch.arange(c, device=cuda)
+        assert torch.equal(out_b, out) and torch.equal(((bits[:, cols // 32] >> (cols % 32)) & 1).bool(), out > 0)
+        gx3, gb3 = dense.bias_act_backward(god, None, relu_bits=bits)
+        torch.cuda.synchronize()
+        assert torch.equal(gx3, gx) and torch.equal(gb3, gb)
+    elif relu:
+        with pytest.raises(RuntimeError):
+            dense.bias_act_forward(xd, bd, True, with_bits=True)
 
 
 @pytest.mark.parametrize("act", ["relu", "none", "tanh"])

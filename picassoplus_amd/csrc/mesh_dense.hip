@@ -42,16 +42,19 @@ __device__ __forceinline__ void rows_issue(RowBlock<VEC, MASK> &b, const float *
                                            int64_t tile, int q, int64_t N, int K, int lane)
 {
     if constexpr (VEC) {
-        const int col = q + 4 * (lane & 15);
+        // tile and q are uniform: a scalar base per group of four rows plus one lane offset
+        const int col = q + 4 * (lane & 15), sub = lane >> 4;
+        const int lane_off = sub * K + col, lane_word = sub * W + (col >> 5);
+        const int64_t left = N - tile * 32;
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-            const int64_t row = tile * 32 + 4 * i + (lane >> 4);
+            const int64_t row0 = tile * 32 + 4 * i;
             float4 t = make_float4(0.f, 0.f, 0.f, 0.f), mm = make_float4(1.f, 1.f, 1.f, 1.f);
             if constexpr (MASK == 2) b.w[i] = 0u;
-            if (row < N && col < K) {
-                t = *reinterpret_cast<const float4 *>(a + row * K + col);
-                if constexpr (MASK == 1) mm = *reinterpret_cast<const float4 *>(mask + row * K + col);
-                if constexpr (MASK == 2) b.w[i] = bits[row * W + (col >> 5)];
+            if (4 * i + sub < left && col < K) {
+                t = *reinterpret_cast<const float4 *>(a + row0 * K + lane_off);
+                if constexpr (MASK == 1) mm = *reinterpret_cast<const float4 *>(mask + row0 * K + lane_off);
+                if constexpr (MASK == 2) b.w[i] = bits[row0 * W + lane_word];
             }
             b.v[4 * i] = t.x; b.v[4 * i + 1] = t.y; b.v[4 * i + 2] = t.z; b.v[4 * i + 3] = t.w;
             if constexpr (MASK == 1) { b.m[4 * i] = mm.x; b.m[4 * i + 1] = mm.y; b.m[4 * i + 2] = mm.z; b.m[4 * i + 3] = mm.w; }
@@ -98,6 +101,41 @@ __device__ __forceinline__ void rows_commit(const RowBlock<VEC, MASK> &b, float 
     }
 }
 
+// Epilogue of one 32-row tile: out = max(acc + bias, floor) * scale + shift, lane (n, h) holds column n of every
+// 32-column block and rows 8(i/4) + 4h + i%4.  BITS: one ballot per register gives the 32 mask bits of a row of
+// either lane half; lane i keeps the word of its row and the sixteen rows of a half leave in one store.
+// FULL: the tile lies inside the matrix, no bounds.  Clears the accumulators.
+template <int NT, bool BITS, bool FULL>
+__device__ __forceinline__ void rows_store(f32x16 (&acc)[NT], const float (&bia)[NT], const float (&scl)[NT],
+                                           const float (&shf)[NT], float floor_v, float *__restrict__ tile_out,
+                                           unsigned *__restrict__ tile_bits, int C, int Wout, int col0, int n, int h,
+                                           int64_t left)
+{
+#pragma unroll
+    for (int j = 0; j < NT; ++j) {
+        const int c = col0 + j * 32 + n;
+        const bool col_ok = FULL || c < C;
+        float *lane_out = tile_out + 4 * h * C + c;
+        unsigned word = 0u;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int ri = 8 * (i / 4) + (i % 4);                      // row of lane half 0; half 1 is four rows on
+            const float v = fmaxf(acc[j][i] + bia[j], floor_v);
+            if (FULL || (col_ok && ri + 4 * h < left)) lane_out[(int64_t)ri * C] = v * scl[j] + shf[j];
+            if constexpr (BITS) {
+                const unsigned long long pos = __builtin_amdgcn_ballot_w64(col_ok && v > 0.f);
+                const unsigned mine = h ? (unsigned)(pos >> 32) : (unsigned)pos;
+                word = (n == i) ? mine : word;
+            }
+            acc[j][i] = 0.f;
+        }
+        if constexpr (BITS) {
+            const int rn = 8 * (n / 4) + 4 * h + (n % 4);
+            if (n < 16 && (FULL || (rn < left && (col0 >> 5) + j < Wout))) tile_bits[(int64_t)rn * Wout + j] = word;
+        }
+    }
+}
+
 template <int NT, int NW, bool VEC, int MASK>
 __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void dense_rows_k(const float *__restrict__ a, const float *__restrict__ mask,
                                                        const unsigned *__restrict__ bits_in,
@@ -110,7 +148,8 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void dense_rows_k(const f
 {
     extern __shared__ __attribute__((aligned(16))) float lds[];
     constexpr int NC = NT * 32;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    // the wavefront index as a scalar: tile numbers and with them every row base stay in scalar registers
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const int n = lane & 31, h = lane >> 5;
     const int col0 = blockIdx.y * NC;
     float *slab = lds + NW * kStageWave;
@@ -129,6 +168,7 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void dense_rows_k(const f
         scl[j] = (scale && c < C) ? scale[c] : 1.f;
         shf[j] = (shift && c < C) ? shift[c] : 0.f;
     }
+    const float floor_v = relu ? 0.f : -__builtin_inff();      // max(v, floor_v) is the ReLU or the identity
     const int64_t ntiles = (N + 31) / 32, stride = (int64_t)gridDim.x * NW;
     int64_t tile = (int64_t)blockIdx.x * NW + wave;
     int q = 0;
@@ -166,28 +206,16 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void dense_rows_k(const f
         }
         __builtin_amdgcn_wave_barrier();
         if (q + kDenseChunk >= Kpad) {
-#pragma unroll
-            for (int j = 0; j < NT; ++j) {
-                const int c = col0 + j * 32 + n;
-                unsigned word = 0u;
-#pragma unroll
-                for (int i = 0; i < 16; ++i) {
-                    const int64_t r = tile * 32 + 8 * (i / 4) + 4 * h + (i % 4);
-                    float v = acc[j][i] + bia[j];
-                    if (relu) v = fmaxf(v, 0.f);
-                    if (c < C && r < N) out[r * C + c] = v * scl[j] + shf[j];
-                    if (bits_out) {
-                        // one ballot = the 32 columns of this block for row i of either lane half; lane i keeps it
-                        const unsigned long long pos = __builtin_amdgcn_ballot_w64(c < C && v > 0.f);
-                        const unsigned mine = h ? (unsigned)(pos >> 32) : (unsigned)pos;
-                        word = (n == i) ? mine : word;
-                    }
-                    acc[j][i] = 0.f;
-                }
-                if (bits_out && n < 16) {
-                    const int64_t r = tile * 32 + 8 * (n / 4) + 4 * h + (n % 4);
-                    if (r < N && (col0 >> 5) + j < Wout) bits_out[r * Wout + (col0 >> 5) + j] = word;
-                }
+            const int64_t left = N - tile * 32;
+            const bool full = left >= 32 && col0 + NC <= C;            // uniform: no bounds inside the tile
+            float *tile_out = out + tile * 32 * C;
+            unsigned *tile_bits = bits_out ? bits_out + tile * 32 * Wout + (col0 >> 5) : nullptr;
+            if (tile_bits) {
+                if (full) rows_store<NT, true, true>(acc, bia, scl, shf, floor_v, tile_out, tile_bits, C, Wout, col0, n, h, left);
+                else rows_store<NT, true, false>(acc, bia, scl, shf, floor_v, tile_out, tile_bits, C, Wout, col0, n, h, left);
+            } else {
+                if (full) rows_store<NT, false, true>(acc, bia, scl, shf, floor_v, tile_out, tile_bits, C, Wout, col0, n, h, left);
+                else rows_store<NT, false, false>(acc, bia, scl, shf, floor_v, tile_out, tile_bits, C, Wout, col0, n, h, left);
             }
         }
         tile = ntile; q = nq; have = nhave;

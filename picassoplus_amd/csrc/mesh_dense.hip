@@ -3,7 +3,8 @@
 // reference runs this tail as separate PyTorch ops after every convolution (picasso/mesh/layers.py:114-119,
 // 169-174, 232-238: matmul with depth_weights, + biases, activation, batch norm); here the bias, the ReLU and
 // an inference-mode batch norm ride in the epilogue of the product, and the ReLU mask of the backward pass
-// rides in the operand loads, so every pass touches each feature row once.
+// rides in the operand loads -- as one bit per entry that the forward's epilogue leaves behind, or read off
+// the forward's output -- so every pass touches each feature row once.
 #include "common.h"
 #include "rows_internal.h"
 #include "../../include/picasso_mesh.h"

@@ -182,3 +182,41 @@ def test_pool_full_size_invariants(cuda):
     ref_gc = torch.zeros(nvo, C, device=cuda, dtype=torch.float64).index_add_(0, cl, gf.double())
     assert float((gc.double() - ref_gc).abs().max()) <= 1e-5 * float(ref_gc.abs().max())
     torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("ci,co", [(64, 64), (128, 128)])
+def test_dense_tail_full_size_adjoints_and_sample_parity(cuda, ci, co):
+    """The pointwise tail on 2.4 M rows: without activation y = x W + b is linear, so <y - b, g> = <x, gx> = <W, gW>
+    and gb = column sums of g; with ReLU a random sample of rows is checked against the float64 oracle and the bit
+    mask against the output."""
+    from oracle import torch_ref
+    from picassoplus_amd.mesh.pi_modules import dense
+    say("case dense tail full size", ci, co)
+    N = 2_400_000
+    gen = torch.Generator(device=cuda).manual_seed(ci)
+    x = torch.randn(N, ci, device=cuda, generator=gen)
+    w = torch.randn(ci, co, device=cuda, generator=gen) / ci ** 0.5
+    b = torch.randn(co, device=cuda, generator=gen)
+    g = torch.randn(N, co, device=cuda, generator=gen)
+    y = dense.dense_tail_forward(x, w, b, False)
+    gx, gw, gb = dense.dense_tail_backward(g, x, w, None)
+    lhs = _dot(y, g) - _dot(b[None, :].expand_as(g), g)
+    scale = float(y.double().norm() * g.double().norm())
+    _adjoint_ok(lhs, _dot(x, gx), scale, "dense <y-b,g> = <x,gx>")
+    _adjoint_ok(lhs, _dot(w, gw), scale, "dense <y-b,g> = <W,gW>")
+    assert_close(gb, g.double().sum(0).cpu().numpy(), "dense grad_bias")
+    del y, gx
+    yr, bits = dense.dense_tail_forward(x, w, b, True, with_bits=True)
+    cols = torch.arange(co, device=cuda)
+    pick = torch.randint(0, N, (4096,), device=cuda, generator=gen)
+    assert torch.equal(((bits[pick][:, cols // 32] >> (cols % 32)) & 1).bool(), yr[pick] > 0)
+    ref = torch_ref.dense_tail_fwd(x[pick].double().cpu(), w.double().cpu(), b.double().cpu(), True)
+    assert_close(yr[pick], ref.numpy(), "dense forward sample")
+    gxr, gwr, gbr = dense.dense_tail_backward(g, x, w, None, relu_bits=bits)
+    rx, _, _ = torch_ref.dense_tail_bwd(g[pick].double().cpu(), x[pick].double().cpu(), w.double().cpu(),
+                                        yr[pick].double().cpu())
+    assert_close(gxr[pick], rx.numpy(), "dense grad_input sample")
+    # the weight gradient of the masked pass, on the GPU in float64 from the same mask
+    gz = torch.where(yr > 0, g, torch.zeros_like(g)).double()
+    assert_close(gwr, (x.double().t() @ gz).cpu().numpy(), "dense grad_weight")
+    assert_close(gbr, gz.sum(0).cpu().numpy(), "dense grad_bias (masked)")

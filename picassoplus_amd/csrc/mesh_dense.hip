@@ -8,19 +8,51 @@
 #include "common.h"
 #include "rows_internal.h"
 #include "../../include/picasso_mesh.h"
+#include <stdlib.h>
 
 namespace pmesh {
 
 typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
+// Exact split of eight fp32 values into three bf16 pieces each (8 + 8 + 8 mantissa bits, by truncation), packed
+// in the k order of v_mfma_f32_32x32x16_bf16.  Six piece products a1b1 + a1b2 + a2b1 + a1b3 + a2b2 + a3b1,
+// accumulated in fp32, give the fp32 product to 2^-24: the matrix cores run them at a sixth of the bf16 rate,
+// still 2.6 times the rate of the fp32 matrix instruction.
+__device__ __forceinline__ unsigned dense_pack_hi(float a, float b)
+{
+    return __builtin_amdgcn_perm(__builtin_bit_cast(unsigned, b), __builtin_bit_cast(unsigned, a), 0x07060302u);
+}
+__device__ __forceinline__ float dense_trunc(float x)
+{
+    return __builtin_bit_cast(float, __builtin_bit_cast(unsigned, x) & 0xFFFF0000u);
+}
+__device__ __forceinline__ void dense_split8(const float (&x)[8], u32x4 &p1, u32x4 &p2, u32x4 &p3)
+{
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const float a = x[2 * j], b = x[2 * j + 1];
+        p1[j] = dense_pack_hi(a, b);
+        const float ra = a - dense_trunc(a), rb = b - dense_trunc(b);
+        p2[j] = dense_pack_hi(ra, rb);
+        p3[j] = dense_pack_hi(ra - dense_trunc(ra), rb - dense_trunc(rb));
+    }
+}
+__device__ __forceinline__ f32x16 dense_mfma_bf16(const u32x4 &a, const u32x4 &b, const f32x16 &c)
+{
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+}
 
 constexpr int kDenseChunk = 64;            // reduction entries per register chunk (32 per lane half)
-constexpr int kDenseSlabFloats = 12288;    // preferred weight slab of a four-wavefront workgroup in LDS (48 KiB)
-constexpr int kDenseSlabWide = 22528;      // of an eight-wavefront workgroup (88 KiB)
+constexpr int kDenseSlabBytes = 48 * 1024;      // preferred weight slab of a four-wavefront workgroup in LDS
+constexpr int kDenseSlabWideBytes = 88 * 1024;  // of an eight-wavefront workgroup
+constexpr int kDenseSlabSixBytes = 104 * 1024;  // of a six-wavefront workgroup (split-bf16 products only)
 constexpr size_t kDenseLdsMax = 160 * 1024;
 constexpr int kDenseMaxK = 896;            // a 32-column slab of that length is 112 KiB, beside 34 KiB of row stages
 
 // rows (N x K, row stride K) times Wm (K x C, element (k, c) at w[k * wk + c * wc]) for the NT * 32 columns
-// from blockIdx.y * NT * 32 on.  A wavefront owns 32 rows at a time.  It fetches a 32 x 64 block of them with
+// of this workgroup's column block.  A wavefront owns 32 rows at a time.  It fetches a 32 x 64 block of them with
 // fully coalesced loads (a 16-lane group per row), one block ahead of the arithmetic, and turns it into the
 // operand layout of the matrix instruction (lane = row) through a private LDS stage: lane (r, h) reads entries
 // h*32 .. h*32+31 of row r (the order of the reduction index is free as long as both operands agree).  The
@@ -137,7 +169,9 @@ __device__ __forceinline__ void rows_store(f32x16 (&acc)[NT], const float (&bia)
     }
 }
 
-template <int NT, int NW, bool VEC, int MASK>
+// X3: the product runs on the bf16 matrix instruction with both operands split in three (the slab then holds
+// [k/8][column][piece] blocks of eight bf16, 6 bytes per weight); otherwise on the fp32 matrix instruction.
+template <int NT, int NW, bool VEC, int MASK, bool X3>
 __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void dense_rows_k(const float *__restrict__ a, const float *__restrict__ mask,
                                                        const unsigned *__restrict__ bits_in,
                                                        unsigned *__restrict__ bits_out,
@@ -152,13 +186,32 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void dense_rows_k(const f
     // the wavefront index as a scalar: tile numbers and with them every row base stay in scalar registers
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const int n = lane & 31, h = lane >> 5;
-    const int col0 = blockIdx.y * NC;
+    // the column blocks of the same rows are neighbouring workgroups: they run together and share the rows' HBM reads
+    const int ncb = (C + NC - 1) / NC;
+    const int col0 = (int)(blockIdx.x % ncb) * NC;
+    const int64_t row_block = blockIdx.x / ncb, row_blocks = gridDim.x / ncb;
     float *slab = lds + NW * kStageWave;
     float *stage = lds + wave * kStageWave;
-    for (int idx = threadIdx.x; idx < Kpad * NC; idx += NW * 64) {
-        const int k = idx / NC, c = idx - k * NC;
-        const float v = (k < K && col0 + c < C) ? w[(int64_t)k * wk + (int64_t)(col0 + c) * wc] : 0.f;
-        slab[((k >> 2) * NC + c) * 4 + (k & 3)] = v;
+    if constexpr (X3) {
+        u32x4 *slab3 = reinterpret_cast<u32x4 *>(slab);
+        for (int idx = threadIdx.x; idx < (Kpad >> 3) * NC; idx += NW * 64) {
+            const int kb = idx / NC, c = idx - kb * NC;
+            float v[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const int k = 8 * kb + e;
+                v[e] = (k < K && col0 + c < C) ? w[(int64_t)k * wk + (int64_t)(col0 + c) * wc] : 0.f;
+            }
+            u32x4 p1, p2, p3;
+            dense_split8(v, p1, p2, p3);
+            slab3[(size_t)idx * 3] = p1; slab3[(size_t)idx * 3 + 1] = p2; slab3[(size_t)idx * 3 + 2] = p3;
+        }
+    } else {
+        for (int idx = threadIdx.x; idx < Kpad * NC; idx += NW * 64) {
+            const int k = idx / NC, c = idx - k * NC;
+            const float v = (k < K && col0 + c < C) ? w[(int64_t)k * wk + (int64_t)(col0 + c) * wc] : 0.f;
+            slab[((k >> 2) * NC + c) * 4 + (k & 3)] = v;
+        }
     }
     __syncthreads();
     float bia[NT], scl[NT], shf[NT];
@@ -170,8 +223,8 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void dense_rows_k(const f
         shf[j] = (shift && c < C) ? shift[c] : 0.f;
     }
     const float floor_v = relu ? 0.f : -__builtin_inff();      // max(v, floor_v) is the ReLU or the identity
-    const int64_t ntiles = (N + 31) / 32, stride = (int64_t)gridDim.x * NW;
-    int64_t tile = (int64_t)blockIdx.x * NW + wave;
+    const int64_t ntiles = (N + 31) / 32, stride = row_blocks * NW;
+    int64_t tile = row_block * NW + wave;
     int q = 0;
     bool have = tile < ntiles;
     RowBlock<VEC, MASK> blk;
@@ -192,17 +245,44 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void dense_rows_k(const f
         const bool nhave = ntile < ntiles;
         if (nhave) rows_issue<VEC, MASK>(blk, a, mask, bits_in, Win, ntile, nq, N, K, lane);
         const float *xs = stage + n * kStageStride + h * 32;
-        const float *sl = slab + ((size_t)((q + h * 32) >> 2) * NC + n) * 4;
+        if constexpr (X3) {
+            // lane (r, h) owns reduction entries q + 32h + 8t + e of row r in step t, the slab block (q + 32h)/8 + t
+            u32x4 pa[4][3];
 #pragma unroll
-        for (int g = 0; g < 8; ++g) {
-            const float4 x4 = *reinterpret_cast<const float4 *>(xs + 4 * g);
+            for (int t = 0; t < 4; ++t) {
+                const float4 lo = *reinterpret_cast<const float4 *>(xs + 8 * t);
+                const float4 hi = *reinterpret_cast<const float4 *>(xs + 8 * t + 4);
+                const float xv[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+                dense_split8(xv, pa[t][0], pa[t][1], pa[t][2]);
+            }
+            const u32x4 *sl = reinterpret_cast<const u32x4 *>(slab) + ((size_t)((q + h * 32) >> 3) * NC + n) * 3;
 #pragma unroll
-            for (int j = 0; j < NT; ++j) {
-                const float4 b = *reinterpret_cast<const float4 *>(sl + ((size_t)g * NC + j * 32) * 4);
-                acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(x4.x, b.x, acc[j], 0, 0, 0);
-                acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(x4.y, b.y, acc[j], 0, 0, 0);
-                acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(x4.z, b.z, acc[j], 0, 0, 0);
-                acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(x4.w, b.w, acc[j], 0, 0, 0);
+            for (int t = 0; t < 4; ++t) {
+#pragma unroll
+                for (int j = 0; j < NT; ++j) {
+                    const u32x4 *bp = sl + ((size_t)t * NC + j * 32) * 3;
+                    const u32x4 b1 = bp[0], b2 = bp[1], b3 = bp[2];
+                    acc[j] = dense_mfma_bf16(pa[t][2], b1, acc[j]);
+                    acc[j] = dense_mfma_bf16(pa[t][1], b2, acc[j]);
+                    acc[j] = dense_mfma_bf16(pa[t][0], b3, acc[j]);
+                    acc[j] = dense_mfma_bf16(pa[t][1], b1, acc[j]);
+                    acc[j] = dense_mfma_bf16(pa[t][0], b2, acc[j]);
+                    acc[j] = dense_mfma_bf16(pa[t][0], b1, acc[j]);
+                }
+            }
+        } else {
+            const float *sl = slab + ((size_t)((q + h * 32) >> 2) * NC + n) * 4;
+#pragma unroll
+            for (int g = 0; g < 8; ++g) {
+                const float4 x4 = *reinterpret_cast<const float4 *>(xs + 4 * g);
+#pragma unroll
+                for (int j = 0; j < NT; ++j) {
+                    const float4 b = *reinterpret_cast<const float4 *>(sl + ((size_t)g * NC + j * 32) * 4);
+                    acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(x4.x, b.x, acc[j], 0, 0, 0);
+                    acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(x4.y, b.y, acc[j], 0, 0, 0);
+                    acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(x4.z, b.z, acc[j], 0, 0, 0);
+                    acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(x4.w, b.w, acc[j], 0, 0, 0);
+                }
             }
         }
         __builtin_amdgcn_wave_barrier();
@@ -274,8 +354,11 @@ __device__ __forceinline__ void pairs_issue(PairBlock<TA, TB, U, MASK> &blk, con
 // gz = g where y > 0 (MASK) or g.  The rows are the reduction index: one matrix instruction consumes two rows
 // (lane half h takes row 2t + h), lane (m, h) supplies TA input channels and TB output channels that lie
 // contiguously in its rows, and a wavefront keeps TA x TB tiles of 32 x 32 sums.  Every workgroup leaves one
-// partial of (Ci + 1) * Co floats (row Ci = bias gradient); blockIdx.y walks the channel chunks.
-template <int TA, int TB, bool VEC, int MASK>
+// partial of (Ci + 1) * Co floats (row Ci = bias gradient).  The channel chunks of one row range are neighbouring
+// workgroups (chunk = blockIdx.x % chunks), so they run at the same time and the rows they share come from HBM once.
+// X3: the sixteen rows of a block are one reduction step of the bf16 matrix instruction (lane half h holds the
+// eight rows base + 2u + h), both operands split in three pieces, six piece products per tile.
+template <int TA, int TB, bool VEC, int MASK, bool X3>
 __global__ __launch_bounds__(256, 2) void dense_wgrad_k(const float *__restrict__ x, const float *__restrict__ g,
                                                         const float *__restrict__ y,
                                                         const unsigned *__restrict__ bits, float *__restrict__ partial,
@@ -285,7 +368,9 @@ __global__ __launch_bounds__(256, 2) void dense_wgrad_k(const float *__restrict_
     __shared__ float bred[4][2][32 * TB];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int m = lane & 31, h = lane >> 5;
-    const int chunkA = blockIdx.y % nA, chunkB = blockIdx.y / nA;
+    const int nchunks = nA * ((Co + TB * 32 - 1) / (TB * 32));
+    const int chunk = (int)(blockIdx.x % nchunks), range = (int)(blockIdx.x / nchunks);
+    const int chunkA = chunk % nA, chunkB = chunk / nA;
     const int ci0 = chunkA * TA * 32 + m * TA, co0 = chunkB * TB * 32 + m * TB;
     f32x16 acc[TA][TB];
 #pragma unroll
@@ -298,7 +383,7 @@ __global__ __launch_bounds__(256, 2) void dense_wgrad_k(const float *__restrict_
 #pragma unroll
     for (int jb = 0; jb < TB; ++jb) gb[jb] = 0.f;
     const int wave_u = __builtin_amdgcn_readfirstlane(wave);
-    const int64_t r0 = ((int64_t)blockIdx.x * 4 + wave_u) * rows_per_wave;
+    const int64_t r0 = ((int64_t)range * 4 + wave_u) * rows_per_wave;
     int64_t r1 = r0 + rows_per_wave;
     if (r1 > N) r1 = N;
     constexpr int U = 8;
@@ -306,21 +391,54 @@ __global__ __launch_bounds__(256, 2) void dense_wgrad_k(const float *__restrict_
     for (int64_t base = r0; base < r1; base += 2 * U) {
         if (base + 2 * U <= r1) pairs_issue<TA, TB, U, VEC, MASK, true>(blk, x, g, y, bits, base, r1, h, Ci, Co, ci0, co0);
         else pairs_issue<TA, TB, U, VEC, MASK, false>(blk, x, g, y, bits, base, r1, h, Ci, Co, ci0, co0);
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-            float gzv[TB];
+        if constexpr (X3) {
+            u32x4 pb[TB][3];
 #pragma unroll
             for (int jb = 0; jb < TB; ++jb) {
-                gzv[jb] = blk.gz[u].v[jb];
-                if constexpr (MASK == 1) gzv[jb] = blk.yy[u].v[jb] > 0.f ? gzv[jb] : 0.f;
-                if constexpr (MASK == 2) gzv[jb] = ((blk.yw[u] >> ((co0 & 31) + jb)) & 1u) ? gzv[jb] : 0.f;
-                gb[jb] += gzv[jb];
+                float gzv[U];
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    gzv[u] = blk.gz[u].v[jb];
+                    if constexpr (MASK == 1) gzv[u] = blk.yy[u].v[jb] > 0.f ? gzv[u] : 0.f;
+                    if constexpr (MASK == 2) gzv[u] = ((blk.yw[u] >> ((co0 & 31) + jb)) & 1u) ? gzv[u] : 0.f;
+                    gb[jb] += gzv[u];
+                }
+                dense_split8(gzv, pb[jb][0], pb[jb][1], pb[jb][2]);
             }
 #pragma unroll
-            for (int ja = 0; ja < TA; ++ja)
+            for (int ja = 0; ja < TA; ++ja) {
+                float xv[U];
 #pragma unroll
-                for (int jb = 0; jb < TB; ++jb)
-                    acc[ja][jb] = __builtin_amdgcn_mfma_f32_32x32x2f32(blk.xa[u].v[ja], gzv[jb], acc[ja][jb], 0, 0, 0);
+                for (int u = 0; u < U; ++u) xv[u] = blk.xa[u].v[ja];
+                u32x4 pa[3];
+                dense_split8(xv, pa[0], pa[1], pa[2]);
+#pragma unroll
+                for (int jb = 0; jb < TB; ++jb) {
+                    acc[ja][jb] = dense_mfma_bf16(pa[2], pb[jb][0], acc[ja][jb]);
+                    acc[ja][jb] = dense_mfma_bf16(pa[1], pb[jb][1], acc[ja][jb]);
+                    acc[ja][jb] = dense_mfma_bf16(pa[0], pb[jb][2], acc[ja][jb]);
+                    acc[ja][jb] = dense_mfma_bf16(pa[1], pb[jb][0], acc[ja][jb]);
+                    acc[ja][jb] = dense_mfma_bf16(pa[0], pb[jb][1], acc[ja][jb]);
+                    acc[ja][jb] = dense_mfma_bf16(pa[0], pb[jb][0], acc[ja][jb]);
+                }
+            }
+        } else {
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                float gzv[TB];
+#pragma unroll
+                for (int jb = 0; jb < TB; ++jb) {
+                    gzv[jb] = blk.gz[u].v[jb];
+                    if constexpr (MASK == 1) gzv[jb] = blk.yy[u].v[jb] > 0.f ? gzv[jb] : 0.f;
+                    if constexpr (MASK == 2) gzv[jb] = ((blk.yw[u] >> ((co0 & 31) + jb)) & 1u) ? gzv[jb] : 0.f;
+                    gb[jb] += gzv[jb];
+                }
+#pragma unroll
+                for (int ja = 0; ja < TA; ++ja)
+#pragma unroll
+                    for (int jb = 0; jb < TB; ++jb)
+                        acc[ja][jb] = __builtin_amdgcn_mfma_f32_32x32x2f32(blk.xa[u].v[ja], gzv[jb], acc[ja][jb], 0, 0, 0);
+            }
         }
     }
     // the four wavefronts add up in wavefront order
@@ -341,7 +459,7 @@ __global__ __launch_bounds__(256, 2) void dense_wgrad_k(const float *__restrict_
 #pragma unroll
     for (int jb = 0; jb < TB; ++jb) bred[wave][h][m * TB + jb] = gb[jb];
     __syncthreads();
-    float *dst = partial + (size_t)blockIdx.x * (size_t)(Ci + 1) * Co;
+    float *dst = partial + (size_t)range * (size_t)(Ci + 1) * Co;
     for (int idx = threadIdx.x; idx < TA * TB * 16 * 64; idx += 256) {
         const int ln = idx & 63, i = (idx >> 6) & 15, t = idx >> 10;
         const int ja = t / TB, jb = t - ja * TB;
@@ -477,11 +595,18 @@ static BiasPlan bias_plan(int64_t N, int C, bool aligned)
 static bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
 // Column tiles per workgroup of dense_rows_k: as many as the preferred slab size and 4 accumulator tiles allow.
-static int rows_tiles(int Kpad, int C, int slab_floats)
+static int rows_tiles(int Kpad, int C, int slab_weights)
 {
     int nt = 4;
-    while (nt > 1 && (Kpad * nt * 32 > slab_floats || (nt / 2) * 32 >= C)) nt >>= 1;
+    while (nt > 1 && (Kpad * nt * 32 > slab_weights || (nt / 2) * 32 >= C)) nt >>= 1;
     return nt;
+}
+
+// PMESH_DENSE_FP32MFMA=1 keeps the products on the fp32 matrix instruction (tests compare the two paths).
+static bool force_fp32_mfma()
+{
+    const char *e = getenv("PMESH_DENSE_FP32MFMA");
+    return e && e[0] == '1';
 }
 
 // Launch with as many workgroups as are resident at once (every tile is independent, so the count only
@@ -499,10 +624,10 @@ struct RowsArgs {
     int K, Kpad, C;
 };
 
-template <int NT, int NW, bool VEC, int MASK>
+template <int NT, int NW, bool VEC, int MASK, bool X3>
 static void launch_rows_nt(int64_t ntiles, unsigned gy, size_t lds, hipStream_t st, const RowsArgs &p)
 {
-    const void *fn = reinterpret_cast<const void *>(dense_rows_k<NT, NW, VEC, MASK>);
+    const void *fn = reinterpret_cast<const void *>(dense_rows_k<NT, NW, VEC, MASK, X3>);
     if (lds > 65536) (void)hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     int per_cu = 0, dev = 0, cus = 0;
     if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, fn, NW * 64, lds) != hipSuccess || per_cu < 1) per_cu = 1;
@@ -512,14 +637,21 @@ static void launch_rows_nt(int64_t ntiles, unsigned gy, size_t lds, hipStream_t 
     const int64_t wanted = ceil_div(ntiles, NW);
     if (gx < 1) gx = 1;
     if (gx > wanted) gx = wanted;
-    dense_rows_k<NT, NW, VEC, MASK><<<dim3((unsigned)gx, gy), dim3(NW * 64), lds, st>>>(
+    dense_rows_k<NT, NW, VEC, MASK, X3><<<dim3((unsigned)(gx * gy)), dim3(NW * 64), lds, st>>>(
         p.a, p.mask, p.bits_in, p.bits_out, p.w, p.wk, p.wc, p.bias, p.scale, p.shift, p.relu, p.out, p.N, p.K, p.Kpad, p.C);
 }
 
-template <bool VEC, int MASK>
+template <bool VEC, int MASK, bool X3>
 static void launch_rows(int NT, int NW, int64_t ntiles, unsigned gy, size_t lds, hipStream_t st, const RowsArgs &p)
 {
-#define PM_ROWS(T, W) launch_rows_nt<T, W, VEC, MASK>(ntiles, gy, lds, st, p)
+#define PM_ROWS(T, W) launch_rows_nt<T, W, VEC, MASK, X3>(ntiles, gy, lds, st, p)
+    if constexpr (X3) {
+        if (NW == 6) {
+            if (NT == 4) PM_ROWS(4, 6);
+            else PM_ROWS(2, 6);
+            return;
+        }
+    }
     if (NW == 8) {
         switch (NT) {
         case 4: PM_ROWS(4, 8); break;
@@ -547,28 +679,53 @@ static int dense_rows(const char *name, const float *a, const float *mask, const
     const int Kpad = (int)ceil_div(K, kDenseChunk) * kDenseChunk;
     // Four wavefronts per workgroup and a slab of at most 48 KiB keep two workgroups on a CU.  When that slab
     // cannot hold all the columns (the rows would be fetched once per column block), or leaves room for one
-    // workgroup only, eight wavefronts share a slab of up to 88 KiB instead.
-    int NT = rows_tiles(Kpad, C, kDenseSlabFloats), NW = 4;
-    size_t lds = ((size_t)Kpad * NT * 32 + 4 * kStageWave) * sizeof(float);
-    const int nt8 = rows_tiles(Kpad, C, kDenseSlabWide);
-    const size_t lds8 = ((size_t)Kpad * nt8 * 32 + 8 * kStageWave) * sizeof(float);
-    if (lds8 <= kDenseLdsMax && (nt8 > NT || lds > kDenseLdsMax / 2)) {
-        NT = nt8; NW = 8; lds = lds8;
+    // workgroup only, eight wavefronts share a slab of up to 88 KiB instead.  The split-bf16 product needs
+    // 6 bytes per weight; reductions too long for that slab stay on the fp32 matrix instruction.
+    bool x3 = !force_fp32_mfma();
+    int NT = 1, NW = 4;
+    size_t lds = 0;
+    for (;;) {
+        const int wbytes = x3 ? 6 : 4;
+        NT = rows_tiles(Kpad, C, kDenseSlabBytes / wbytes);
+        NW = 4;
+        lds = (size_t)Kpad * NT * 32 * wbytes + 4 * kStageWave * sizeof(float);
+        const int nt8 = rows_tiles(Kpad, C, kDenseSlabWideBytes / wbytes);
+        const size_t lds8 = (size_t)Kpad * nt8 * 32 * wbytes + 8 * kStageWave * sizeof(float);
+        if (lds8 <= kDenseLdsMax && (nt8 > NT || lds > kDenseLdsMax / 2)) {
+            NT = nt8; NW = 8; lds = lds8;
+        }
+        if (x3) {
+            // six wavefronts leave 108 KiB for the slab: 128 columns of a 128-long reduction in split bf16
+            const int nt6 = rows_tiles(Kpad, C, kDenseSlabSixBytes / wbytes);
+            const size_t lds6 = (size_t)Kpad * nt6 * 32 * wbytes + 6 * kStageWave * sizeof(float);
+            if (lds6 <= kDenseLdsMax && nt6 > NT) {
+                NT = nt6; NW = 6; lds = lds6;
+            }
+        }
+        if (lds <= kDenseLdsMax || !x3) break;
+        x3 = false;
     }
+    PM_REQUIRE(lds <= kDenseLdsMax, "%s: reduction length %d too large", name, K);
     const int64_t ntiles = ceil_div(N, 32);
     const unsigned gy = (unsigned)ceil_div(C, NT * 32);
     const bool vec = (K % 4 == 0) && aligned16(a) && (!mask || aligned16(mask));
     const RowsArgs p{a, mask, bits_in, bits_out, w, wk, wc, bias, scale, shift, relu, out, N, K, Kpad, C};
     const int mode = bits_in ? 2 : mask ? 1 : 0;
+#define PM_PICK(V, M)                                                          \
+    do {                                                                       \
+        if (x3) launch_rows<V, M, true>(NT, NW, ntiles, gy, lds, st, p);       \
+        else launch_rows<V, M, false>(NT, NW, ntiles, gy, lds, st, p);         \
+    } while (0)
     if (vec) {
-        if (mode == 2) launch_rows<true, 2>(NT, NW, ntiles, gy, lds, st, p);
-        else if (mode == 1) launch_rows<true, 1>(NT, NW, ntiles, gy, lds, st, p);
-        else launch_rows<true, 0>(NT, NW, ntiles, gy, lds, st, p);
+        if (mode == 2) PM_PICK(true, 2);
+        else if (mode == 1) PM_PICK(true, 1);
+        else PM_PICK(true, 0);
     } else {
-        if (mode == 2) launch_rows<false, 2>(NT, NW, ntiles, gy, lds, st, p);
-        else if (mode == 1) launch_rows<false, 1>(NT, NW, ntiles, gy, lds, st, p);
-        else launch_rows<false, 0>(NT, NW, ntiles, gy, lds, st, p);
+        if (mode == 2) PM_PICK(false, 2);
+        else if (mode == 1) PM_PICK(false, 1);
+        else PM_PICK(false, 0);
     }
+#undef PM_PICK
     PM_LAUNCHED(name);
     return 0;
 }
@@ -605,7 +762,12 @@ template <int TA, int TB>
 static void launch_wgrad(bool vec, int mode, dim3 grid, hipStream_t st, const float *x, const float *g, const float *y,
                          const unsigned *bits, float *partial, int64_t N, int Ci, int Co, int nA, int64_t rpw)
 {
-#define PM_WGK(V, M) dense_wgrad_k<TA, TB, V, M><<<grid, dim3(256), 0, st>>>(x, g, y, bits, partial, N, Ci, Co, nA, rpw)
+    const bool x3 = !force_fp32_mfma();
+#define PM_WGK(V, M)                                                                                                        \
+    do {                                                                                                                    \
+        if (x3) dense_wgrad_k<TA, TB, V, M, true><<<grid, dim3(256), 0, st>>>(x, g, y, bits, partial, N, Ci, Co, nA, rpw);  \
+        else dense_wgrad_k<TA, TB, V, M, false><<<grid, dim3(256), 0, st>>>(x, g, y, bits, partial, N, Ci, Co, nA, rpw);    \
+    } while (0)
     if (vec) {
         if (mode == 2) PM_WGK(true, 2);
         else if (mode == 1) PM_WGK(true, 1);
@@ -670,7 +832,7 @@ extern "C" int pmesh_dense_bwd(const float *grad_output, const float *input, con
     float *partial = (float *)workspace;
     const bool vec = Ci % p.ta == 0 && Co % p.tb == 0 && aligned16(input) && aligned16(grad_output) &&
                      (!output || aligned16(output));
-    const dim3 grid((unsigned)p.G, (unsigned)(p.nA * p.nB));
+    const dim3 grid((unsigned)(p.G * p.nA * p.nB));
     const int mode = relu_bits ? 2 : output ? 1 : 0;
 #define PM_WG(A, B) launch_wgrad<A, B>(vec, mode, grid, st, input, grad_output, output, relu_bits, partial, N, Ci, Co, p.nA, p.rows_per_wave)
     if (p.ta == 4 && p.tb == 2) PM_WG(4, 2);

@@ -34,10 +34,21 @@ def _case(seed, n, ci, co):
     return x, w, b, go
 
 
+@pytest.fixture(params=["split_bf16", "fp32_mfma"])
+def product_path(request, monkeypatch):
+    """The row kernels multiply on the bf16 matrix instruction with operands split in three (default) or, behind
+    PMESH_DENSE_FP32MFMA=1 (read at every call), on the fp32 matrix instruction."""
+    if request.param == "fp32_mfma":
+        monkeypatch.setenv("PMESH_DENSE_FP32MFMA", "1")
+    else:
+        monkeypatch.delenv("PMESH_DENSE_FP32MFMA", raising=False)
+    return request.param
+
+
 @pytest.mark.parametrize("n,ci,co", SHAPES)
 @pytest.mark.parametrize("relu", [True, False])
-def test_dense_tail_forward_backward(cuda, n, ci, co, relu):
-    say("case dense_tail", n, ci, co, relu)
+def test_dense_tail_forward_backward(cuda, product_path, n, ci, co, relu):
+    say("case dense_tail", product_path, n, ci, co, relu)
     x, w, b, go = _case(n + ci, n, ci, co)
     f = lambda t: t.to(cuda, torch.float32).contiguous()
     xd, wd, bd, god = f(x), f(w), f(b), f(go)

@@ -165,8 +165,8 @@ def test_per_item_and_coeff_modules(cuda):
     torch.manual_seed(5)
     mod = layers.PerItemConv3d(10, 6, activation_fn=nn.ReLU(), with_bn=False).to(cuda)
     x = torch.randn(50, 10, device=cuda)
-    ref = torch.relu(x @ mod.weights + mod.biases)
-    assert torch.allclose(mod(x), ref)
+    ref = torch.relu(x.double() @ mod.weights.double() + mod.biases.double())
+    assert_close(mod(x), ref.detach().cpu().numpy(), "PerItemConv3d output")
     b = layers.BuildF2VCoeff(7).to(cuda)
     n = torch.nn.functional.normalize(torch.randn(40, 3, device=cuda), dim=1)
     c = b(n)

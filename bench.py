@@ -82,6 +82,9 @@ def conv_bytes_flops(d, ops):
         "f2f_fwd": (4 * T * Ci + 4 * T * B + 4 * Nf + 4 * C * Ci * B + 4 * Nf * C, 2 * T * Ci * B + 2 * Nf * Ci * B * C),
         "f2f_bwd_texture": (4 * Nf * C + 4 * T * B + 4 * Nf + 4 * C * Ci * B + 4 * T * Ci, 2 * Nf * Ci * B * C + 2 * T * Ci * B),
         "f2f_bwd_filter": (4 * Nf * C + 4 * T * Ci + 4 * T * B + 4 * Nf + 4 * C * Ci * B, 2 * Nf * Ci * B * C + 2 * T * Ci * B),
+        # texture points interpolated from vertex features, with their basis values (forward) / transposed (backward)
+        "texture_fwd": (4 * Nv * C + 16 * Nf + 12 * T + 4 * T * C + 4 * T * B, 5 * T * C + 60 * T),
+        "texture_bwd": (4 * T * C + 12 * T + 16 * Nf + 4 * Nv * C, 6 * T * C),
     }
     return {k: tab[k] for k in ops}
 
@@ -122,7 +125,7 @@ class EventTimer:
 def run_conv_layer(args, torch, kind):
     from picassoplus_amd import _lib, synthetic as S
     from picassoplus_amd.mesh.layers import sph_harm_values
-    from picassoplus_amd.mesh.pi_modules import conv3d
+    from picassoplus_amd.mesh.pi_modules import conv3d, texture
     dev = torch.device("cuda:0")
     C, L = (32 if kind == "firstblock" else 64), 3           # first block: EncodeChannels[0] = 32 (scene_seg.py:28)
     Cin, r = (3, 2) if kind == "firstblock" else (C, 1)      # F2F input channels, F2V depth multiplier
@@ -134,20 +137,20 @@ def run_conv_layer(args, torch, kind):
     else:
         mesh = S.shapes_workload(seed=2000, n_meshes=16)
         d = build_conv_inputs(mesh, C, L, seed=2000, tex_counts=3)
-        ops = ["v2f_fwd", "f2f_fwd", "f2v_fwd", "f2v_bwd", "f2f_bwd_texture", "f2f_bwd_filter", "v2f_bwd"]
-        name = "shapes16_V2F+F2F+F2V_C64_L3_fp32_fwd+bwd"
+        ops = ["v2f_fwd", "texture_fwd", "f2f_fwd", "f2v_fwd", "f2v_bwd", "f2f_bwd_texture", "f2f_bwd_filter",
+               "texture_bwd", "v2f_bwd"]
+        name = "shapes16_V2F+texture+F2F+F2V_C64_L3_fp32_fwd+bwd"
     t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
     face, vt_map, nfc = t(d["face"]), t(d["vt_map"]), t(d["nf_count"].astype(np.int32))
     cum = torch.cumsum(t(d["counts"]), 0, dtype=torch.int32)
     bary = t(d["bary"])
     owner = t(d["owner"])
     x = t(d["x"])
-    # texture-point features: barycentric interpolation of the vertex features (set-up, untimed)
-    corner = face.long()[owner]
-    tex = (x[corner[:, 0]] * bary[:, 0:1] + x[corner[:, 1]] * bary[:, 1:2] + x[corner[:, 2]] * bary[:, 2:3])
+    # scene workloads take the texture-point features as given data, like the reference's networks (set-up, untimed);
+    # the shapes block interpolates them from the vertex features inside the step
+    tex, sh = texture.interpolate(x, face, bary, cum, L)
     tex = tex[:, :Cin].contiguous()                          # first block: three colour-like channels
-    del corner, owner
-    sh = sph_harm_values(bary, L)
+    del owner
     coeff = sph_harm_values(t(d["normal"]), L)
     w_f2f, w_f2v, w_v2f = t(d["w_f2f"]), t(d["w_f2v"]), t(d["w_v2f"])
     gy = torch.randn(d["nv"], C * r, device=dev, generator=torch.Generator(device=dev).manual_seed(1))
@@ -161,9 +164,10 @@ def run_conv_layer(args, torch, kind):
             y = conv3d.facet2vertex(y1, w_f2v, coeff, face, nfc, vt_map)
             return torch.autograd.grad(y, [tex, w_f2f, w_f2v], gy)
         y0 = conv3d.vertex2facet(x, w_v2f, face)
-        y1 = conv3d.facet2facet(tex, w_f2f, sh, cum)
+        tex_s, sh_s = texture.interpolate(x, face, bary, cum, L)
+        y1 = conv3d.facet2facet(tex_s, w_f2f, sh_s, cum)
         y = conv3d.facet2vertex(y0 + y1, w_f2v, coeff, face, nfc, vt_map)
-        return torch.autograd.grad(y, [x, tex, w_v2f, w_f2f, w_f2v], gy)
+        return torch.autograd.grad(y, [x, w_v2f, w_f2f, w_f2v], gy)
 
     timer = EventTimer(torch)
     _lib.set_call_hook(timer)
@@ -230,13 +234,16 @@ def cpu_baseline_conv(d, kind, torch, budget_s=12.0):
         nfc = torch.from_numpy(d["nf_count"][va:vb].astype(np.int32))
         gy = torch.randn(nv, d["C"] * d["r"])
         t0 = time.perf_counter()
+        if kind == "shapes":
+            tex, sh = R.texture_fwd(x, f, bary, cum), R.sph_harm(bary, d["L"])
         y1 = R.f2f_fwd(tex, w_f2f, sh, cum)
         if kind == "shapes":
             y1 = y1 + R.v2f_fwd(x, w_v2f, f)
         R.f2v_fwd(y1, w_f2v, coeff, f, nfc, vt_map)
         g1, _ = R.f2v_bwd(gy, y1, w_f2v, coeff, f, nfc, vt_map)
-        R.f2f_bwd(g1, tex, w_f2f, sh, cum)
+        gt, _ = R.f2f_bwd(g1, tex, w_f2f, sh, cum)
         if kind == "shapes":
+            R.texture_bwd(gt, nv, f, bary, cum)
             R.v2f_bwd(g1, x, w_v2f, f)
         spent += time.perf_counter() - t0
         done_f, done_t, n_mesh = done_f + nf, done_t + int(tb - ta), n_mesh + 1

@@ -195,6 +195,26 @@ int pmesh_unpool_bwd(const float *grad_output, const int32_t *rowptr, const int3
  * xyz (N,3) -> out (N,(L+1)^2); a zero vector evaluates at direction (1,0,0). */
 int pmesh_sph_harm(const float *xyz, float *out, int64_t N, int L, pmesh_stream_t stream);
 
+/* ------------------------------------------------------------------ texture points from vertex features
+ * No counterpart among the reference's extensions: the reference reads the features of the texture
+ * points from its dataset files (picasso/mesh/dataset_scene.py:29-33) and evaluates the basis of
+ * their barycentric coordinates with SphHarmCoeff (picasso/networks/scene_seg.py:150).  An encoder
+ * block that runs facet2facet on vertex features needs them interpolated:
+ *   texture[k,c] = sum_j bary[k,j] * input[face[f,j], c]   for k in [cum_texture[f-1], cum_texture[f])
+ *   bary_coeff[k,:] = SH basis of degree L at bary[k,:]     (as pmesh_sph_harm; NULL = not wanted)
+ * in one pass: input (Nv,C), face (Nf,3), bary (T,3), cum_texture (Nf, inclusive running total as for
+ * facet2facet) -> texture (T,C), bary_coeff (T,(L+1)^2).  Rows of texture / bary_coeff beyond
+ * cum_texture[Nf-1] are not written.
+ * Backward: grad_input (Nv,C) = transpose of the interpolation applied to grad_texture (T,C), summed in
+ * adjacency order; rowptr/colidx: vertex CSR with vt_map = NULL, n_rows = Nv (the one
+ * pmesh_v2f_bwd takes).  bary gets no gradient. */
+int pmesh_texture_fwd(const float *input, const int32_t *face, const float *bary,
+                      const int32_t *cum_texture, float *texture, float *bary_coeff, int64_t Nv,
+                      int64_t Nf, int64_t T, int C, int L, pmesh_stream_t stream);
+int pmesh_texture_bwd(const float *grad_texture, const float *bary, const int32_t *cum_texture,
+                      const int32_t *rowptr, const int32_t *colidx, float *grad_input, int64_t Nv,
+                      int64_t Nf, int64_t T, int C, pmesh_stream_t stream);
+
 /* ------------------------------------------------------------------ per-level inputs of the convs
  * pmesh_count_vertex_adjface replaces count_vertex_adjface (decimate_gpu.cu:813-836,
  * decimate.py:88-93): the number of (facet, corner) entries per output vertex is the row length

@@ -173,3 +173,19 @@ def sph_harm(xyz, L, dtype=np.float64):
     if _call("ref_sph_harm", dtype, xyz.shape[0], L, xyz, out):
         raise NotImplementedError("spherical-harmonic degree must be 0..5")
     return out
+
+
+def texture_fwd(x, face, bary, cum, dtype=np.float64):
+    """Features of texture points by barycentric interpolation of the corner features: (T, C)."""
+    x, bary, face, cum = _f(x, dtype), _f(bary, dtype), _i(face), _i(cum)
+    T = int(cum[-1]) if cum.shape[0] else 0
+    tex = np.empty((T, x.shape[1]), dtype)
+    _call("ref_texture_fwd", dtype, cum.shape[0], x.shape[1], face, cum, bary, x, tex)
+    return tex
+
+
+def texture_bwd(gtex, nv, face, bary, cum, dtype=np.float64):
+    gtex, bary, face, cum = _f(gtex, dtype), _f(bary, dtype), _i(face), _i(cum)
+    gin = np.empty((nv, gtex.shape[1]), dtype)
+    _call("ref_texture_bwd", dtype, cum.shape[0], nv, gtex.shape[1], face, cum, bary, gtex, gin)
+    return gin

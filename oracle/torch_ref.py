@@ -155,6 +155,27 @@ def f2f_bwd(gout, tex, filt, bary, cum):
 
 
 # --------------------------------------------------------------------------
+# texture points from vertex features: tex[k] = sum_j bary[k,j] * x[face[f(k),j]] for the rows k of
+# facet f's segment (the grouping of layers.py:57); the reference loads texture features from its
+# dataset files (dataset_scene.py:29-33) and has no such routine -- the encoder-block workload chains
+# facet2facet after vertex features this way
+# --------------------------------------------------------------------------
+def texture_fwd(x, face, bary, cum):
+    _, seg = _segments(cum, bary.shape[0])
+    corner = _long(face)[seg]                                   # (T, 3)
+    return (x[corner] * bary[:, :, None]).sum(1)
+
+
+def texture_bwd(gtex, nv, face, bary, cum):
+    _, seg = _segments(cum, bary.shape[0])
+    corner = _long(face)[seg]
+    gin = torch.zeros(nv, gtex.shape[1], dtype=gtex.dtype)
+    for j in range(3):
+        gin = gin.index_add(0, corner[:, j], gtex * bary[:, j:j + 1])
+    return gin
+
+
+# --------------------------------------------------------------------------
 # pooling / unpooling over decimation clusters
 # (mesh_pool3d_gpu.cu:20-155, mesh_unpool3d_gpu.cu:5-46)
 # --------------------------------------------------------------------------

@@ -1,0 +1,199 @@
+// Texture points of the facets from vertex features (gfx950, wave64).
+//
+//   forward   tex[k, c] = sum_j bary[k, j] * in[face[f, j], c]   for the rows k of facet f's segment
+//             [cum[f-1], cum[f]) -- the grouping facet2facet expects (picasso/mesh/layers.py:57) --
+//             and, in the same pass, coeff[k, :] = spherical-harmonic basis at bary[k, :]
+//             (what picasso/networks/scene_seg.py:150 computes with a chain of elementwise kernels);
+//   backward  gin[v, c] = sum over the (facet, corner) pairs at v, over the facet's rows k, of
+//             bary[k, corner] * gtex[k, c], a segmented sum over the sorted vertex adjacency (no atomics,
+//             fixed order).
+//
+// Both are bound by HBM.  A group of lanes owns one facet (forward) or one vertex (backward) and spans the
+// channels with 16-byte items; the three corner rows of a facet are fetched once and stay in registers for all of
+// the facet's points, whose rows leave as one contiguous run.
+#include "common.h"
+#include "sph_internal.h"
+#include "../../include/picasso_mesh.h"
+
+namespace pmesh {
+
+constexpr int kTexBatch = 4;   // texture points in flight per lane group
+
+template <int V, int LC>   // LC: compile-time degree of the basis, -1 = read `L`
+__global__ __launch_bounds__(kBlock) void texture_fwd_k(const float *__restrict__ in, const int *__restrict__ face,
+                                                        const int *__restrict__ cum, const float *__restrict__ bary,
+                                                        float *__restrict__ tex, float *__restrict__ coeff,
+                                                        int64_t Nf, int64_t T, int C, int Q, int lpr_log2, int L)
+{
+    const int lpr = 1 << lpr_log2;
+    const int lane = threadIdx.x & (lpr - 1), slot = threadIdx.x >> lpr_log2;
+    const int rpb = kBlock >> lpr_log2;
+    const int64_t f = (int64_t)blockIdx.x * rpb + slot;
+    int64_t k0 = 0, k1 = 0;
+    if (f < Nf) {
+        k0 = f ? cum[f - 1] : 0;
+        k1 = cum[f];
+        if (k0 < 0) k0 = 0;
+        if (k1 > T) k1 = T;
+    }
+    if (k0 < k1) {
+        const int64_t v0 = face[3 * f], v1 = face[3 * f + 1], v2 = face[3 * f + 2];
+        for (int q = lane; q < Q; q += lpr) {
+            const int c = q * V;
+            const Pack<V> a0 = ldp<V>(in + v0 * C + c), a1 = ldp<V>(in + v1 * C + c), a2 = ldp<V>(in + v2 * C + c);
+            for (int64_t kb = k0; kb < k1; kb += kTexBatch) {
+                float b[kTexBatch][3];
+#pragma unroll
+                for (int i = 0; i < kTexBatch; ++i)
+#pragma unroll
+                    for (int j = 0; j < 3; ++j) b[i][j] = (kb + i < k1) ? bary[3 * (kb + i) + j] : 0.f;
+#pragma unroll
+                for (int i = 0; i < kTexBatch; ++i) {
+                    if (kb + i >= k1) break;
+                    Pack<V> o;
+#pragma unroll
+                    for (int u = 0; u < V; ++u) o.v[u] = fmaf(b[i][2], a2.v[u], fmaf(b[i][1], a1.v[u], b[i][0] * a0.v[u]));
+                    stp<V>(tex + (kb + i) * C + c, o);
+                }
+            }
+        }
+    }
+    if (!coeff) return;
+    // The points of the workgroup's facets are one contiguous run of rows: its lanes take them one each, so
+    // the coordinates come in and the basis values leave as contiguous pieces.
+    const int64_t fa = (int64_t)blockIdx.x * rpb;
+    int64_t fb = fa + rpb;
+    if (fb > Nf) fb = Nf;
+    int64_t ka = fa ? cum[fa - 1] : 0, kz = cum[fb - 1];
+    if (ka < 0) ka = 0;
+    if (kz > T) kz = T;
+    const int Lv = LC >= 0 ? LC : L;
+    const int B = (Lv + 1) * (Lv + 1);
+    for (int64_t k = ka + threadIdx.x; k < kz; k += kBlock) {
+        float v[36];
+        sph_harm_at(bary[3 * k], bary[3 * k + 1], bary[3 * k + 2], Lv, v);
+        float *o = coeff + k * B;
+        if constexpr (LC == 3) {
+#pragma unroll
+            for (int i = 0; i < 16; i += 4) *reinterpret_cast<float4 *>(o + i) = make_float4(v[i], v[i + 1], v[i + 2], v[i + 3]);
+        } else {
+            for (int i = 0; i < B; ++i) o[i] = v[i];
+        }
+    }
+}
+
+template <int V>
+__global__ __launch_bounds__(kBlock) void texture_bwd_k(const float *__restrict__ gtex, const float *__restrict__ bary,
+                                                        const int *__restrict__ cum, const int *__restrict__ rowptr,
+                                                        const int *__restrict__ colidx, float *__restrict__ gin,
+                                                        int64_t Nv, int64_t Nf, int64_t T, int C, int Q, int lpr_log2)
+{
+    const int lpr = 1 << lpr_log2;
+    const int lane = threadIdx.x & (lpr - 1), slot = threadIdx.x >> lpr_log2;
+    const int64_t row = (int64_t)blockIdx.x * (kBlock >> lpr_log2) + slot;
+    if (row >= Nv) return;
+    const int e0 = rowptr[row], e1 = rowptr[row + 1];
+    constexpr int EB = 4;
+    for (int q = lane; q < Q; q += lpr) {
+        const int c = q * V;
+        Pack<V> acc = zero_pack<V>();
+        for (int eb = e0; eb < e1; eb += EB) {
+            // the adjacency entries of a vertex four at a time: all segment bounds requested before any is used
+            int ent[EB], corner[EB];
+            int64_t s0[EB], s1[EB];
+#pragma unroll
+            for (int i = 0; i < EB; ++i) ent[i] = (eb + i < e1) ? colidx[eb + i] : -1;
+#pragma unroll
+            for (int i = 0; i < EB; ++i) {
+                const int64_t f = ent[i] / 3;
+                corner[i] = ent[i] - 3 * (int)f;
+                const bool ok = ent[i] >= 0 && f < Nf;
+                s0[i] = (ok && f > 0) ? cum[f - 1] : 0;
+                s1[i] = ok ? cum[f] : 0;
+            }
+#pragma unroll
+            for (int i = 0; i < EB; ++i) {
+                if (s0[i] < 0) s0[i] = 0;
+                if (s1[i] > T) s1[i] = T;
+            }
+#pragma unroll
+            for (int i = 0; i < EB; ++i) {
+                for (int64_t kb = s0[i]; kb < s1[i]; kb += kTexBatch) {
+                    float w[kTexBatch];
+                    Pack<V> g[kTexBatch];
+#pragma unroll
+                    for (int p = 0; p < kTexBatch; ++p) {
+                        const bool in = kb + p < s1[i];
+                        w[p] = in ? bary[3 * (kb + p) + corner[i]] : 0.f;
+                        g[p] = in ? ldp<V>(gtex + (kb + p) * C + c) : zero_pack<V>();
+                    }
+#pragma unroll
+                    for (int p = 0; p < kTexBatch; ++p)
+#pragma unroll
+                        for (int u = 0; u < V; ++u) acc.v[u] = fmaf(w[p], g[p].v[u], acc.v[u]);
+                }
+            }
+        }
+        stp<V>(gin + row * C + c, acc);
+    }
+}
+
+static inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+}  // namespace pmesh
+
+using namespace pmesh;
+
+extern "C" int pmesh_texture_fwd(const float *input, const int32_t *face, const float *bary, const int32_t *cum_texture,
+                                 float *texture, float *bary_coeff, int64_t Nv, int64_t Nf, int64_t T, int C, int L,
+                                 pmesh_stream_t stream)
+{
+    clear_error();
+    PM_REQUIRE(Nv >= 0 && Nf >= 0 && T >= 0 && C >= 0, "texture_fwd: negative size");
+    PM_REQUIRE(!bary_coeff || (L >= 0 && L <= 5), "texture_fwd: basis degree %d outside 0..5", L);
+    PM_REQUIRE(T < (int64_t(1) << 31), "texture_fwd: more than 2^31 texture points");
+    if (T == 0 || Nf == 0) return 0;
+    PM_REQUIRE(face && bary && cum_texture, "texture_fwd: null pointer");
+    PM_REQUIRE(C == 0 || (input && texture && Nv > 0), "texture_fwd: null pointer");
+    hipStream_t st = (hipStream_t)stream;
+    const bool vec = C % 4 == 0 && aligned16(input) && aligned16(texture);
+    const RowShape rs = row_shape(C == 0 ? 1 : vec ? C / 4 : C);
+    const int Q = C == 0 ? 0 : rs.items;
+    const int64_t blocks = ceil_div(Nf, rs.rpb);
+    PM_REQUIRE(grid_ok(blocks), "texture_fwd: grid too large");
+    const dim3 grid((unsigned)blocks), block(kBlock);
+    const bool l3 = bary_coeff && L == 3 && aligned16(bary_coeff);
+    if (vec) {
+        if (l3) texture_fwd_k<4, 3><<<grid, block, 0, st>>>(input, face, cum_texture, bary, texture, bary_coeff, Nf, T, C, Q, rs.lpr_log2, L);
+        else texture_fwd_k<4, -1><<<grid, block, 0, st>>>(input, face, cum_texture, bary, texture, bary_coeff, Nf, T, C, Q, rs.lpr_log2, L);
+    } else {
+        if (l3) texture_fwd_k<1, 3><<<grid, block, 0, st>>>(input, face, cum_texture, bary, texture, bary_coeff, Nf, T, C, Q, rs.lpr_log2, L);
+        else texture_fwd_k<1, -1><<<grid, block, 0, st>>>(input, face, cum_texture, bary, texture, bary_coeff, Nf, T, C, Q, rs.lpr_log2, L);
+    }
+    PM_LAUNCHED("texture_fwd");
+    return 0;
+}
+
+extern "C" int pmesh_texture_bwd(const float *grad_texture, const float *bary, const int32_t *cum_texture,
+                                 const int32_t *rowptr, const int32_t *colidx, float *grad_input, int64_t Nv,
+                                 int64_t Nf, int64_t T, int C, pmesh_stream_t stream)
+{
+    clear_error();
+    PM_REQUIRE(Nv >= 0 && Nf >= 0 && T >= 0 && C >= 0, "texture_bwd: negative size");
+    PM_REQUIRE(T < (int64_t(1) << 31), "texture_bwd: more than 2^31 texture points");
+    if (Nv == 0 || C == 0) return 0;
+    PM_REQUIRE(grad_input && rowptr, "texture_bwd: null pointer");
+    PM_REQUIRE(Nf == 0 || (colidx && cum_texture), "texture_bwd: null pointer");
+    PM_REQUIRE(T == 0 || (grad_texture && bary), "texture_bwd: null pointer");
+    hipStream_t st = (hipStream_t)stream;
+    const bool vec = C % 4 == 0 && aligned16(grad_input) && aligned16(grad_texture);
+    const RowShape rs = row_shape(vec ? C / 4 : C);
+    const int64_t blocks = ceil_div(Nv, rs.rpb);
+    PM_REQUIRE(grid_ok(blocks), "texture_bwd: grid too large");
+    if (vec)
+        texture_bwd_k<4><<<dim3((unsigned)blocks), dim3(kBlock), 0, st>>>(grad_texture, bary, cum_texture, rowptr, colidx, grad_input, Nv, Nf, T, C, rs.items, rs.lpr_log2);
+    else
+        texture_bwd_k<1><<<dim3((unsigned)blocks), dim3(kBlock), 0, st>>>(grad_texture, bary, cum_texture, rowptr, colidx, grad_input, Nv, Nf, T, C, rs.items, rs.lpr_log2);
+    PM_LAUNCHED("texture_bwd");
+    return 0;
+}

@@ -15,7 +15,7 @@ from picassoplus_amd import synthetic as S
 from picassoplus_amd.mesh import topology
 from picassoplus_amd.mesh.layers import sph_harm_values
 from picassoplus_amd.mesh.pi_modules import (conv3d, mesh_conv3d, mesh_pool3d, mesh_unpool3d, pool3d,
-                                             unpool3d)
+                                             texture, unpool3d)
 from util import assert_close, dev, mesh_case, rel_err, strided_vt_map, texture_case
 
 pytestmark = pytest.mark.gpu
@@ -92,6 +92,78 @@ def test_v2f_parity(cuda, mesh, C, r):
     assert_close(out, out_ref, "v2f out")
     assert_close(xt.grad, gin_ref, "v2f grad_input")
     assert_close(ft.grad, gfilt_ref, "v2f grad_filter")
+
+
+# ------------------------------------------------------------------ texture points from vertex features
+@pytest.mark.parametrize("mesh,C,kmax,L", [("tetra", 4, 3, 3), ("octa", 3, 9, 3), ("sphere2", 64, 9, 3), ("fans", 32, 5, 2),
+                                           ("room_small", 64, 9, 3), ("torus", 130, 4, 5), ("sphere3", 7, 20, None),
+                                           ("sphere2", 2048, 2, 0)])
+def test_texture_interpolation_parity(cuda, mesh, C, kmax, L):
+    say("case texture", mesh, C, kmax, L)
+    v, f = mesh_case(mesh)
+    rng = np.random.default_rng(12)
+    nv, nf = v.shape[0], f.shape[0]
+    counts, bary, owner = texture_case(rng, nf, kmax=kmax)
+    cum = np.cumsum(counts).astype(np.int32)
+    T = int(cum[-1])
+    x = rng.uniform(-1, 1, (nv, C))
+    g = rng.normal(0, 1, (T, C))
+    tex_ref = loops.texture_fwd(x, f, bary, cum)
+    gin_ref = loops.texture_bwd(g, nv, f, bary, cum)
+    xt = dev(x, cuda, torch.float32).requires_grad_(True)
+    bt = dev(bary, cuda, torch.float32)
+    res = texture.interpolate(xt, dev(f, cuda), bt, dev(cum, cuda), L)
+    tex, coeff = res if L is not None else (res, None)
+    tex.backward(dev(g, cuda, torch.float32))
+    torch.cuda.synchronize()
+    assert_close(tex, tex_ref, "texture features")
+    assert_close(xt.grad, gin_ref, "texture grad_input")
+    if L is not None:
+        assert not coeff.requires_grad
+        assert_close(coeff, loops.sph_harm(bt.cpu().numpy().astype(np.float64), L), "texture basis values")
+        # the fused basis is the stand-alone kernel's, bit for bit
+        assert torch.equal(coeff, sph_harm_values(bt, L))
+
+
+def test_texture_interpolation_feeds_facet2facet(cuda):
+    """Gradient of a facet2facet layer with respect to vertex features through the interpolation, against the
+    oracle's composition."""
+    say("case texture_chain")
+    v, f = mesh_case("sphere3")
+    rng = np.random.default_rng(13)
+    nv, nf, C, Co, L = v.shape[0], f.shape[0], 16, 32, 3
+    counts, bary, owner = texture_case(rng, nf, kmax=4)
+    cum = np.cumsum(counts).astype(np.int32)
+    x = rng.uniform(-1, 1, (nv, C))
+    filt = rng.normal(0, 0.2, (Co, C, (L + 1) ** 2))
+    gout = rng.normal(0, 1, (nf, Co))
+    T64 = lambda a: torch.from_numpy(np.ascontiguousarray(a))
+    sh = torch_ref.sph_harm(T64(bary), L)
+    xr = T64(x).requires_grad_(True)
+    out_ref = torch_ref.f2f_fwd(torch_ref.texture_fwd(xr, T64(f), T64(bary), T64(cum)), T64(filt), sh, T64(cum))
+    (gx_ref,) = torch.autograd.grad(out_ref, xr, T64(gout))
+    xt = dev(x, cuda, torch.float32).requires_grad_(True)
+    tex, coeff = texture.interpolate(xt, dev(f, cuda), dev(bary, cuda, torch.float32), dev(cum, cuda), L)
+    out = conv3d.facet2facet(tex, dev(filt, cuda, torch.float32), coeff, dev(cum, cuda))
+    out.backward(dev(gout, cuda, torch.float32))
+    torch.cuda.synchronize()
+    assert_close(out, out_ref.detach().numpy(), "chain out")
+    assert_close(xt.grad, gx_ref.numpy(), "chain grad_input")
+
+
+def test_texture_interpolation_rejects_bad_totals(cuda):
+    say("case texture_bad_totals")
+    x = torch.zeros(4, 8, device=cuda)
+    face = torch.tensor([[0, 1, 2], [1, 2, 3]], dtype=torch.int32, device=cuda)
+    bary = torch.full((5, 3), 1 / 3, device=cuda)
+    with pytest.raises(RuntimeError, match="running total"):
+        texture.interpolate(x, face, bary, torch.tensor([2, 4], dtype=torch.int32, device=cuda))
+    with pytest.raises(RuntimeError, match="running total"):
+        texture.interpolate(x, face, bary, torch.tensor([6, 5], dtype=torch.int32, device=cuda))
+    with pytest.raises(RuntimeError, match="one running total per facet"):
+        texture.interpolate(x, face, bary, torch.tensor([5], dtype=torch.int32, device=cuda))
+    empty = texture.interpolate(x, face, bary[:0], torch.zeros(2, dtype=torch.int32, device=cuda))
+    assert empty[0].shape == (0, 8) and empty[1].shape == (0, 16)
 
 
 # ------------------------------------------------------------------ facet2vertex

@@ -14,7 +14,7 @@ import torch
 
 from picassoplus_amd import _lib, synthetic as S
 from picassoplus_amd.mesh import layers
-from picassoplus_amd.mesh.pi_modules import conv3d, mesh_conv3d, mesh_pool3d, mesh_unpool3d, pool3d, unpool3d
+from picassoplus_amd.mesh.pi_modules import conv3d, mesh_conv3d, mesh_pool3d, mesh_unpool3d, pool3d, texture, unpool3d
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
@@ -57,6 +57,10 @@ def test_argument_errors_without_launching():
     assert b"maximum of 50" in lib.pmesh_last_error()
     assert lib.pmesh_sph_harm(None, None, 5, 6, None) != 0
     assert lib.pmesh_pool_max_bwd(None, None, None, None, None, -1, 2, 4, None) != 0
+    assert lib.pmesh_texture_fwd(None, None, None, None, None, None, 4, 2, 6, 8, 3, None) != 0
+    assert b"null pointer" in lib.pmesh_last_error()
+    assert lib.pmesh_texture_bwd(None, None, None, None, None, None, 4, 2, -1, 8, None) != 0
+    assert lib.pmesh_texture_fwd(None, None, None, None, None, None, 4, 2, 0, 8, 3, None) == 0
     # empty problems succeed without touching the (null) pointers
     assert lib.pmesh_v2f_fwd(None, None, None, None, 0, 0, 8, 1, None) == 0
     assert lib.pmesh_last_error() == b""
@@ -78,6 +82,8 @@ def test_cpu_tensors_are_refused_like_the_reference():
         unpool3d.interpolate(x, torch.zeros(4, dtype=torch.int32), torch.zeros(4, dtype=torch.int32))
     with pytest.raises(RuntimeError, match="must be a CUDA tensor"):
         layers.SphHarmCoeff(3)(torch.eye(3))
+    with pytest.raises(RuntimeError, match="must be a CUDA tensor"):
+        texture.interpolate(x, face, torch.zeros(4, 3), torch.zeros(2, dtype=torch.int32))
 
 
 def test_native_module_surface_matches_reference_extensions():

@@ -416,3 +416,47 @@ def test_combine_clusters_hand_case_and_identity():
     ident_r, ident_m = np.zeros(4, np.int32), np.arange(4, dtype=np.int32)
     rc, mc = torch_ref.combine_clusters(T(ident_r), T(ident_m), T(rb), T(mb))
     assert rc.tolist() == rb.tolist() and mc.tolist() == mb.tolist()
+
+
+# ------------------------------------------------------------------ texture points from vertex features
+def test_texture_interpolation_pins():
+    """Hand values on one triangle, the invariants barycentric weights fix, autograd of the forward for the
+    explicit backward, the adjoint identity, and agreement of the two restatements."""
+    # one triangle, four points: the three corners and the centroid
+    x = np.array([[1.0, 10.0], [2.0, 20.0], [4.0, 40.0]])
+    face = np.array([[2, 0, 1]], np.int32)                       # corner order differs from vertex order on purpose
+    bary = np.array([[1, 0, 0], [0, 1, 0], [0, 0, 1], [1 / 3, 1 / 3, 1 / 3]])
+    cum = np.array([4], np.int32)
+    tex = loops.texture_fwd(x, face, bary, cum)
+    assert np.allclose(tex, [[4, 40], [1, 10], [2, 20], [7 / 3, 70 / 3]], atol=EPS)
+    g = np.array([[1.0, 0.0], [0.0, 1.0], [2.0, 2.0], [3.0, 6.0]])
+    gin = loops.texture_bwd(g, 3, face, bary, cum)
+    # vertex 0 is corner 1, vertex 1 is corner 2, vertex 2 is corner 0
+    assert np.allclose(gin, [[0 + 1, 1 + 2], [2 + 1, 2 + 2], [1 + 1, 0 + 2]], atol=EPS)
+
+    rng = np.random.default_rng(11)
+    v, f = mesh_case("sphere2")
+    nv, nf, C = v.shape[0], f.shape[0], 7
+    counts, bary, owner = texture_case(rng, nf)                  # includes facets without points
+    cum = np.cumsum(counts).astype(np.int32)
+    x = rng.normal(size=(nv, C))
+    tex = loops.texture_fwd(x, f, bary, cum)
+    # independent statement through the owner list the generator returns
+    ref = np.einsum("kj,kjc->kc", bary, x[f[owner].astype(np.int64)])
+    assert rel_err(tex, ref) < EPS
+    # weights sum to one: constant features stay constant, affine functions of position are reproduced
+    assert np.allclose(loops.texture_fwd(np.full((nv, 2), 3.5), f, bary, cum), 3.5, atol=EPS)
+    pos = loops.texture_fwd(v, f, bary, cum)
+    assert rel_err(pos, np.einsum("kj,kjc->kc", bary, v[f[owner].astype(np.int64)])) < EPS
+    # the torch restatement agrees, forward and backward; its backward is autograd of its forward
+    xt = T(x).requires_grad_(True)
+    tt = torch_ref.texture_fwd(xt, T(f), T(bary), T(cum))
+    assert rel_err(tt.detach().numpy(), tex) < EPS
+    g = rng.normal(size=tex.shape)
+    (ga,) = torch.autograd.grad(tt, xt, T(g))
+    gl = loops.texture_bwd(g, nv, f, bary, cum)
+    gt = torch_ref.texture_bwd(T(g), nv, T(f), T(bary), T(cum)).numpy()
+    assert rel_err(gl, ga.numpy()) < EPS and rel_err(gt, ga.numpy()) < EPS
+    assert abs((tex * g).sum() - (x * gl).sum()) < 1e-9 * abs((tex * g).sum())
+    # float32 loops stay close to float64
+    assert rel_err(loops.texture_fwd(x, f, bary, cum, np.float32), tex) < 1e-6

@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the mesh-conv hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload scene|shapes|pool|firstblock|tail] [--scale S]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload scene|shapes|pool|firstblock|tail|hierarchy] [--scale S]
 
 A step is one forward+backward pass of the layer over one batch of seeded synthetic meshes
 already resident in HBM.  Default workload ``scene``: 8 room-like meshes of about 300 k
@@ -37,7 +37,7 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="scene", choices=["scene", "shapes", "pool", "firstblock", "tail"],
+    ap.add_argument("--workload", default="scene", choices=["scene", "shapes", "pool", "firstblock", "tail", "hierarchy"],
                     help="scene: the headline layer (F2F+F2V, C=64); shapes: 16 small meshes V2F+F2F+F2V; pool: "
                          "1024x1024 grid max/avg pool + unpool; firstblock: the scene batch with the reference's first "
                          "block shapes, F2F 3->32 then F2V 32->32 with depth multiplier 2 (pi2_blocks.py:113-130)")
@@ -119,6 +119,14 @@ class EventTimer:
             tot[key] = tot.get(key, 0.0) + a.elapsed_time(b)
             cnt[key] = cnt.get(key, 0) + 1
         return {k: tot[k] / cnt[k] for k in tot}
+
+    def totals(self, steps):
+        """Milliseconds per step and entry point, summed over all of a step's calls."""
+        tot = {}
+        for name, a, b in self.pairs:
+            key = name.replace("pmesh_", "")
+            tot[key] = tot.get(key, 0.0) + a.elapsed_time(b)
+        return {k: v / steps for k, v in tot.items()}
 
 
 # ---------------------------------------------------------------------------- workloads
@@ -365,6 +373,147 @@ def run_tail(args, torch):
                             out_channels=Co))
 
 
+def run_hierarchy(args, torch):
+    """Encoder-decoder stack of the mesh modules over one 2 M-facet mesh and four 4:1 coarser levels: per level
+    V2F + (texture interpolation -> F2F) -> F2V at widths 32/64/128/256, max / avg pooling between levels, then
+    unpooling back to the finest level with a pointwise layer per level; forward + backward.  Also times every
+    level's block alone, to show how the kernels' shares move with mesh size and width."""
+    from torch import nn
+    from picassoplus_amd import _lib, synthetic as S
+    from picassoplus_amd.mesh import layers
+    from picassoplus_amd.mesh.pi_modules import texture
+    dev = torch.device("cuda:0")
+    L, NL = 3, 4
+    W = [32, 64, 128, 256, 256]
+    cells = 1024 if args.scale == 1.0 else max(16, int(1024 * args.scale ** 0.5) // 16 * 16)
+    meshes = S.hierarchy_workload(seed=5000, cells=cells, levels=NL)
+    rng = np.random.default_rng(5000)
+    torch.manual_seed(5000)
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+    lv = []
+    for l in range(NL):
+        m = meshes[l]
+        v, f = m["vertex"], m["face"]
+        nv, nf = v.shape[0], f.shape[0]
+        normal, _ = S.triangle_normals_areas(v, f)
+        counts, bary, _ = S.texture_points(rng, nf, rng.integers(1, 4, nf).astype(np.int32))
+        lv.append(dict(nv=nv, nf=nf, T=int(counts.sum()), C=W[l], Cin=W[l], r=1, B=(L + 1) ** 2, face=t(f),
+                       nfc=t(np.maximum(S.vertex_facet_count(f, np.arange(nv), nv), 1).astype(np.int32)),
+                       ident=torch.arange(nv, dtype=torch.int32, device=dev),
+                       coeff=layers.sph_harm_values(t(normal.astype(np.float32)), L), counts=t(counts),
+                       cum=torch.cumsum(t(counts), 0, dtype=torch.int32), bary=t(bary.astype(np.float32)),
+                       vr=t(m["vt_replace"]), vm=t(m["vt_map"]), vt_out=torch.zeros(m["nv_out"], 3, device=dev),
+                       np_face=f, np_counts=counts, np_bary=bary, np_normal=normal,
+                       v2f=layers.V2FConv3d(W[l], W[l], L, with_bn=False).to(dev),
+                       f2f=layers.F2FConv3d(W[l], W[l], L, with_bn=False).to(dev),
+                       f2v=layers.F2VConv3d(W[l], W[l + 1], L, with_bn=False).to(dev),
+                       pool=layers.Pool3d("max" if l % 2 == 0 else "avg"),
+                       up=layers.PerItemConv3d(W[l + 1], W[l], with_bn=False).to(dev)))
+    params = [p for d in lv for k in ("v2f", "f2f", "f2v", "up") for p in d[k].parameters()]
+    x0 = torch.randn(lv[0]["nv"], W[0], device=dev, requires_grad=True)
+    gy = torch.randn(lv[0]["nv"], W[0], device=dev)
+
+    def block(d, x):
+        tex, sh = texture.interpolate(x, d["face"], d["bary"], d["cum"], L)
+        y = d["v2f"](x, d["face"]) + d["f2f"](tex, sh, d["counts"])
+        z = d["f2v"](y, d["face"], d["nfc"], d["ident"], d["coeff"])
+        return z, d["pool"](z, d["vr"], d["vm"], d["vt_out"])
+
+    def step():
+        x, skips = x0, []
+        for d in lv:
+            z, x = block(d, x)
+            skips.append(z)
+        for d, z in zip(reversed(lv), reversed(skips)):
+            x = d["up"](z + layers.Unpool3d.forward(x, d["vr"], d["vm"]))
+        return torch.autograd.grad(x, [x0] + params, gy)
+
+    def timed(fn):
+        timer = EventTimer(torch)
+        _lib.set_call_hook(timer)
+        for _ in range(args.warmup):
+            fn()
+        torch.cuda.synchronize()
+        timer.on = True
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            fn()
+        torch.cuda.synchronize()
+        ms = (time.perf_counter() - t0) * 1e3 / args.steps
+        _lib.set_call_hook(None)
+        return ms, timer.totals(args.steps)
+
+    ms, per_op = timed(step)
+    # every level's block alone (forward + backward of its five ops and their tails)
+    conv_ops = ["v2f_fwd", "texture_fwd", "f2f_fwd", "f2v_fwd", "f2v_bwd", "f2f_bwd_texture", "f2f_bwd_filter",
+                "texture_bwd", "v2f_bwd"]
+    report, best = [], None
+    for l, d in enumerate(lv):
+        xin = torch.randn(d["nv"], W[l], device=dev, requires_grad=True)
+        gz, gp = torch.randn(d["nv"], W[l + 1], device=dev), torch.randn(d["vt_out"].shape[0], W[l + 1], device=dev)
+        own = [p for k in ("v2f", "f2f", "f2v") for p in d[k].parameters()]
+
+        def one(d=d, xin=xin, gz=gz, gp=gp, own=own):
+            z, p = block(d, xin)
+            return torch.autograd.grad([z, p], [xin] + own, [gz, gp])
+
+        lms, lops = timed(one)
+        bf = conv_bytes_flops(d, conv_ops)
+        report.append(dict(level=l, facets=d["nf"], vertices=d["nv"], texture_points=d["T"], channels=W[l], ms=lms,
+                           ops_ms={k: round(v, 4) for k, v in sorted(lops.items())},
+                           share={k: round(v / sum(lops.values()), 3) for k, v in sorted(lops.items())}))
+        for k in conv_ops:
+            if k in lops and (best is None or lops[k] > best[0]):
+                best = (lops[k], k, l, bf[k])
+    dom_ms, dom, dl, (nbytes, nflops) = best
+    if dom.startswith("f2f"):
+        ach = nflops / (dom_ms * 1e-3) / 1e12
+        roof = dict(bound="mfma", achieved=ach, peak=MFMA_F16_PEAK_TFLOPS / F2F_PIECE_PRODUCTS, unit="TFLOP/s",
+                    peak_basis="fp16 dense MFMA 2500 TFLOP/s / 3 piece products per fp32-accurate product",
+                    frac_of_fp32_mfma_peak=ach / MFMA_F32_PEAK_TFLOPS)
+    else:
+        roof = dict(bound="hbm", achieved=nbytes / (dom_ms * 1e-3) / 1e9, peak=HBM_PEAK_GBS, unit="GB/s")
+    roof.update(frac=roof["achieved"] / roof["peak"], traffic=None, kernel="%s@level%d" % (dom, dl), kernel_ms=dom_ms)
+    res = dict(value=lv[0]["nf"] / (ms * 1e-3) / 1e6, ms_per_step=ms, roofline=roof,
+               ops_ms_per_step={k: round(v, 4) for k, v in sorted(per_op.items())}, levels=report,
+               config=dict(workload="grid%d_4levels_V2F+texture+F2F+F2V+pool+unpool_C32-256_L3_fp32_fwd+bwd" % cells,
+                           facets=[d["nf"] for d in lv], vertices=[d["nv"] for d in lv] + [int(lv[-1]["vt_out"].shape[0])],
+                           channels=W[:NL], sh_degree=L))
+    if not args.no_cpu_baseline:
+        res["cpu_baseline"] = cpu_baseline_block(lv[-1], W[NL - 1], L, torch)
+    return res
+
+
+def cpu_baseline_block(d, C, L, torch):
+    """The oracle's restatement (float32 PyTorch-CPU ops) of the coarsest level's convolutions, forward + backward."""
+    from oracle import torch_ref as R
+    from picassoplus_amd import synthetic as S
+    torch.set_num_threads(os.cpu_count() or 1)
+    rng = np.random.default_rng(1)
+    nv, nf, B = d["nv"], d["nf"], (L + 1) ** 2
+    f = torch.from_numpy(d["np_face"])
+    cum = torch.cumsum(torch.from_numpy(d["np_counts"]), 0, dtype=torch.int32)
+    bary = torch.from_numpy(d["np_bary"].astype(np.float32))
+    coeff = R.sph_harm(torch.from_numpy(d["np_normal"].astype(np.float32)), L)
+    x, gy = torch.randn(nv, C), torch.randn(nv, C)
+    w_v2f = torch.from_numpy(S.xavier_uniform(rng, (3, C, 1), C, 3 * C).astype(np.float32))
+    w_f2f = torch.from_numpy(S.xavier_uniform(rng, (C, C, B), C * B, C * B).astype(np.float32))
+    w_f2v = torch.from_numpy(S.xavier_uniform(rng, (B, C, 1), C, B * C).astype(np.float32))
+    nfc, ident = d["nfc"].cpu(), torch.arange(nv, dtype=torch.int32)
+    t0 = time.perf_counter()
+    tex, sh = R.texture_fwd(x, f, bary, cum), R.sph_harm(bary, L)
+    y = R.f2f_fwd(tex, w_f2f, sh, cum) + R.v2f_fwd(x, w_v2f, f)
+    R.f2v_fwd(y, w_f2v, coeff, f, nfc, ident)
+    g1, _ = R.f2v_bwd(gy, y, w_f2v, coeff, f, nfc, ident)
+    gt, _ = R.f2f_bwd(g1, tex, w_f2f, sh, cum)
+    R.texture_bwd(gt, nv, f, bary, cum)
+    R.v2f_bwd(g1, x, w_v2f, f)
+    spent = time.perf_counter() - t0
+    return dict(value=nf / spent / 1e6, unit="Mfacets/s", cores=torch.get_num_threads(), kind="port",
+                sample="convolutions of the coarsest conv level only (%d facets, %d channels; no tails, pools or "
+                       "other levels), one fwd+bwd pass, %.1f s" % (nf, C, spent))
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -382,6 +531,8 @@ def main():
         res = run_pool(args, torch)
     elif args.workload == "tail":
         res = run_tail(args, torch)
+    elif args.workload == "hierarchy":
+        res = run_hierarchy(args, torch)
     else:
         res = run_conv_layer(args, torch, args.workload)
     if args.copy_calibration:

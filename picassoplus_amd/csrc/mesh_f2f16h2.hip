@@ -7,7 +7,7 @@
 // three v_mfma_f32_32x32x16_f16 where the three-piece bf16 split needs six, and 24 instead of 44 vector
 // instructions per eight values split.  fp16 has a narrow exponent range, so both operands are brought
 // to a fixed magnitude by exact power-of-two scales that are taken out of the accumulator at the end:
-//     W' = beta * W        beta from max|W| (one scalar per filter, computed by f2f16h2_scale_filter_k)
+//     W' = beta * W        beta from max|W| (one scalar per filter, computed by filter_scale)
 //     G'_f = alpha_f * G_f alpha_f from a bound on max|G_f| = max|tex rows of f| * max|SH rows of f|,
 //                          found by a pre-scan of the facet's rows; it rides on the SH values in registers
 // so that |W'|, |G'| < 2^14.  Elements far below their row's maximum (by more than 2^17) fall into fp16's
@@ -102,24 +102,46 @@ __device__ __forceinline__ float pow2_scale(float m, float *inv)
     return __builtin_bit_cast(float, (unsigned)(267 - e) << 23);          // 2^(140 - e):  s * m < 2^14
 }
 
-// header of the packed filter: {beta, 1/beta}
-__global__ __launch_bounds__(1024) void f2f16h2_scale_filter_k(const float *__restrict__ W, float *__restrict__ hdr, int64_t n)
+// header of the packed filter: {beta, 1/beta}, from max|W| in two steps: up to 256 workgroups leave one maximum
+// each in `partial` (the start of the packed-filter area, which the pack kernel overwrites afterwards), one
+// workgroup combines them.  A maximum does not depend on the order, so the header is the same from run to run.
+__global__ __launch_bounds__(256) void f2f16h2_absmax_k(const float *__restrict__ W, float *__restrict__ partial, int64_t n)
 {
-    __shared__ float red[16];
+    __shared__ float red[4];
     float m = 0.f;
-    for (int64_t i = threadIdx.x; i < n; i += 1024) m = fmaxf(m, fabsf(W[i]));
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) m = fmaxf(m, fabsf(W[i]));
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = m;
+    __syncthreads();
+    if (threadIdx.x == 0) partial[blockIdx.x] = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+}
+
+__global__ __launch_bounds__(256) void f2f16h2_scale_filter_k(const float *__restrict__ partial, int G, float *__restrict__ hdr)
+{
+    __shared__ float red[4];
+    float m = (int)threadIdx.x < G ? partial[threadIdx.x] : 0.f;
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
     if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = m;
     __syncthreads();
     if (threadIdx.x == 0) {
-#pragma unroll
-        for (int i = 1; i < 16; ++i) m = fmaxf(m, red[i]);
+        m = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
         float inv;
         const float beta = pow2_scale(m, &inv);
         hdr[0] = beta;
         hdr[1] = inv;
     }
+}
+
+// hdr <- scale of the n filter values; `scratch` = at least 256 floats that the caller overwrites afterwards
+static void filter_scale(const float *W, float *hdr, float *scratch, int64_t n, hipStream_t st)
+{
+    int G = (int)((n + 4095) / 4096);
+    if (G < 1) G = 1;
+    if (G > 256) G = 256;
+    f2f16h2_absmax_k<<<dim3(G), dim3(256), 0, st>>>(W, scratch, n);
+    f2f16h2_scale_filter_k<<<dim3(1), dim3(256), 0, st>>>(scratch, G, hdr);
 }
 
 // Filter (Cout, Cin, 16) -> per-lane MFMA B operands: Wp[((ci*NT + nt)*2 + piece)*64 + lane] holds the
@@ -466,7 +488,7 @@ int f2f16h2_fwd(const float *tex, const float *W, const float *sh, const int *cu
     PM_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 15u) == 0, "f2f_fwd: workspace must be 16-byte aligned");
     float *hdr = (float *)workspace;
     u32x4 *Wp = (u32x4 *)workspace + 1;
-    f2f16h2_scale_filter_k<<<dim3(1), dim3(1024), 0, st>>>(W, hdr, (int64_t)Cout * Cin * 16);
+    filter_scale(W, hdr, (float *)Wp, (int64_t)Cout * Cin * 16, st);
     PM_LAUNCHED("f2f_fwd(scale)");
     const int CinPad = (Cin + 3) & ~3, n = CinPad * NT * 64;
     f2f16h2_pack_filter_k<<<dim3((unsigned)ceil_div(n, kBlock)), dim3(kBlock), 0, st>>>(W, hdr, Wp, Cin, CinPad, Cout, NT);
@@ -766,7 +788,7 @@ int f2f16h2_bwd_texture(const float *gout, const float *W, const float *sh, cons
     PM_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 15u) == 0, "f2f_bwd_texture: workspace must be 16-byte aligned");
     float *hdr = (float *)workspace;
     u32x4 *WpT = (u32x4 *)workspace + 1;
-    f2f16h2_scale_filter_k<<<dim3(1), dim3(1024), 0, st>>>(W, hdr, (int64_t)Cout * Cin * 16);
+    filter_scale(W, hdr, (float *)WpT, (int64_t)Cout * Cin * 16, st);
     PM_LAUNCHED("f2f_bwd_texture(scale)");
     const int64_t gx = ceil_div(Nf, 256);
     PM_REQUIRE(grid_ok(gx), "f2f_bwd_texture: grid too large");

@@ -14,6 +14,7 @@ import torch
 import torch.nn as nn
 
 from .. import _lib
+from . import topology
 from .pi_modules import conv3d, dense, pool3d, unpool3d
 from .pi_modules._check import stream_of
 
@@ -147,7 +148,7 @@ class F2FConv3d(_ConvTail):
     def forward(self, input_texture, bary_coeff, num_texture):
         assert self.in_channels == input_texture.shape[-1]
         assert self.num_basis == bary_coeff.shape[-1]
-        running_total = torch.cumsum(num_texture, dim=0, dtype=torch.int)
+        running_total = topology.running_total(num_texture)
         outputs = conv3d.facet2facet(input_texture, self.weights, bary_coeff, running_total)
         return self._bias_tail(outputs)
 

@@ -18,7 +18,7 @@ from .. import _lib
 
 _LOCK = threading.Lock()
 _CACHE = OrderedDict()
-MAX_ENTRIES = 64
+MAX_ENTRIES = 256
 
 
 def clear_cache():
@@ -134,6 +134,19 @@ def facet_order(cum_texture, n_points):
                   ws.data_ptr(), ws_bytes, _stream(cum_texture))
     _store(key, (order, cum_texture))
     return order
+
+
+def running_total(num_texture):
+    """Inclusive running total (int32) of the per-facet texture-point counts, the form facet2facet takes
+    (picasso/mesh/layers.py:57 computes it in every forward); cached per counts tensor, so that the facet order
+    built from it is found again too."""
+    key = _key("c", num_texture)
+    hit = _lookup(key)
+    if hit is not None:
+        return hit[0]
+    total = torch.cumsum(num_texture, dim=0, dtype=torch.int)
+    _store(key, (total, num_texture))
+    return total
 
 
 def _check_range_cached(face, n_vertices):

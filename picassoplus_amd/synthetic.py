@@ -285,6 +285,43 @@ def plane_workload(seed=4000, n=1024):
     return dict(vertex=v, face=f, nv_in=np.array([v.shape[0]], I32), mf_in=np.array([f.shape[0]], I32))
 
 
+def grid_cluster_maps(cells):
+    """4:1 cluster maps from the (cells+1)^2 vertices of a ``cells``-by-``cells`` grid patch (vertex id
+    ``i * (cells+1) + j``) to the (cells/2+1)^2 vertices of the grid of half the resolution: coarse vertex (I, J)
+    collects the fine vertices {2I, 2I+1} x {2J, 2J+1} inside the patch; its representative is the last of them,
+    so vertex 0 never represents others, and representatives ascend with the coarse id.
+    Returns (vt_replace, vt_map, nv_out) with the meaning ``cluster_maps`` documents."""
+    assert cells >= 2 and cells % 2 == 0
+    nf, nc = cells + 1, cells // 2 + 1
+    i, j = np.meshgrid(np.arange(nf), np.arange(nf), indexing="ij")
+    I, J = i // 2, j // 2
+    rep = np.minimum(2 * I + 1, cells) * nf + np.minimum(2 * J + 1, cells)        # fine id of my representative
+    rep, fine = rep.reshape(-1), (i * nf + j).reshape(-1)
+    size = np.bincount(rep, minlength=nf * nf)
+    is_rep = rep == fine
+    vt_replace = np.where(is_rep, size[fine] - 1, -rep).astype(I32)
+    vt_map = np.where(is_rep, (I * nc + J).reshape(-1), -1).astype(I32)
+    return vt_replace, vt_map, nc * nc
+
+
+def hierarchy_workload(seed=5000, cells=1024, levels=4):
+    """One planar scene-like mesh of 2*cells^2 facets with ``levels`` coarser versions of itself, each a jittered
+    grid of half the resolution (a quarter of the vertices), and the 4:1 cluster maps between consecutive levels.
+    Returns a list of ``levels + 1`` dicts: vertex, face, and (all but the last) vt_replace, vt_map, nv_out."""
+    rng = np.random.default_rng(seed)
+    out = []
+    for l in range(levels + 1):
+        n = cells >> l
+        h = float(1 << l)
+        v, f = grid_patch(rng, n, n, (0, 0, 0), (h, 0, 0), (0, h, 0), flip_frac=0.5)
+        v = v + rng.normal(0, 0.1 * h, v.shape) * np.array([1.0, 1.0, 0.2])
+        lev = dict(vertex=v, face=f)
+        if l < levels:
+            lev["vt_replace"], lev["vt_map"], lev["nv_out"] = grid_cluster_maps(n)
+        out.append(lev)
+    return out
+
+
 def xavier_uniform(rng, shape, fan_in, fan_out):
     a = (6.0 / (fan_in + fan_out)) ** 0.5
     return rng.uniform(-a, a, shape)

@@ -187,6 +187,30 @@ def test_cluster_map_invariants(spatial):
     assert sizes.min() >= 1 and sizes.max() <= 12 and 3.5 < sizes.mean() < 4.5 and sizes.sum() == nv
 
 
+def test_hierarchy_workload_levels_and_maps():
+    levels = S.hierarchy_workload(seed=1, cells=16, levels=3)
+    assert [lv["vertex"].shape[0] for lv in levels] == [17 * 17, 9 * 9, 5 * 5, 3 * 3]
+    assert [lv["face"].shape[0] for lv in levels] == [2 * 16 * 16, 2 * 8 * 8, 2 * 4 * 4, 2 * 2 * 2]
+    for fine, coarse in zip(levels[:-1], levels[1:]):
+        r, m, nvo = fine["vt_replace"], fine["vt_map"], fine["nv_out"]
+        nv = fine["vertex"].shape[0]
+        assert nvo == coarse["vertex"].shape[0] and fine["face"].max() == nv - 1
+        members = r < 0
+        reps = -r[members]
+        assert (r[reps] > 0).all() and 0 not in set(reps.tolist()) and (m[members] == -1).all()
+        assert np.array_equal(np.bincount(reps, minlength=nv)[r > 0], r[r > 0])
+        kept = m >= 0
+        assert np.array_equal(m[kept], np.arange(nvo))                         # ascending, dense
+        assert (r[r >= 0] + 1).sum() == nv and (r[r >= 0] + 1).max() == 4
+        # a coarse vertex sits among its members: within one fine cell (plus jitter) of their mean position
+        rep_of = np.where(r < 0, -r, np.arange(nv))
+        mean = np.zeros((nvo, 3))
+        np.add.at(mean, m[rep_of], fine["vertex"])
+        mean /= np.bincount(m[rep_of], minlength=nvo)[:, None]
+        step = fine["vertex"][:, 0].max() / (np.sqrt(nv) - 1)
+        assert np.abs(mean - coarse["vertex"])[:, :2].max() < 2.0 * step
+
+
 def test_texture_points():
     rng = np.random.default_rng(6)
     counts, bary, owner = S.texture_points(rng, 100, rng.integers(0, 10, 100))

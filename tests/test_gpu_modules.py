@@ -211,3 +211,75 @@ def test_argument_errors_and_side_stream(cuda):
         total = got.sum()
     side.synchronize()
     assert torch.equal(got, ref) and float(total) == float(ref.sum())
+
+
+def test_two_level_stack_matches_oracle_composition(cuda):
+    """Encoder-decoder over a mesh hierarchy, as the benchmark's hierarchy workload builds it: per level
+    V2F + (texture interpolation -> F2F) -> F2V, pooling, then unpooling back with a pointwise layer; outputs and
+    every gradient against the same composition of float64 oracle ops."""
+    from picassoplus_amd.mesh.pi_modules import texture
+    L, W = 3, [8, 16, 16]
+    meshes = S.hierarchy_workload(seed=7, cells=16, levels=2)
+    rng = np.random.default_rng(24)
+    torch.manual_seed(6)
+    lv = []
+    for l in range(2):
+        m = meshes[l]
+        v, f = m["vertex"], m["face"]
+        nv, nf = v.shape[0], f.shape[0]
+        normal, _ = S.triangle_normals_areas(v, f)
+        counts, bary, _ = S.texture_points(rng, nf, rng.integers(0, 4, nf).astype(np.int32))
+        d = dict(nv=nv, face=torch.from_numpy(f), counts=torch.from_numpy(counts), bary=torch.from_numpy(bary),
+                 normal=torch.from_numpy(normal), nfc=torch.from_numpy(np.maximum(S.vertex_facet_count(f, np.arange(nv), nv), 1).astype(np.int32)),
+                 ident=torch.arange(nv, dtype=torch.int32), vr=torch.from_numpy(m["vt_replace"]), vm=torch.from_numpy(m["vt_map"]),
+                 nvo=m["nv_out"], method="max" if l == 0 else "avg",
+                 v2f=layers.V2FConv3d(W[l], W[l], L, with_bn=False).to(cuda), f2f=layers.F2FConv3d(W[l], W[l], L, with_bn=False).to(cuda),
+                 f2v=layers.F2VConv3d(W[l], W[l + 1], L, with_bn=False).to(cuda), up=layers.PerItemConv3d(W[l + 1], W[l], with_bn=False).to(cuda))
+        for k in ("v2f", "f2f", "f2v", "up"):
+            with torch.no_grad():
+                d[k].biases.add_(0.1 * torch.randn_like(d[k].biases))
+            d[k + "64"] = _twin(d[k])
+        lv.append(d)
+    x = torch.from_numpy(rng.normal(0, 1, (lv[0]["nv"], W[0])))
+    g = torch.from_numpy(rng.normal(0, 1, (lv[0]["nv"], W[0])))
+
+    # GPU: modules of the mesh layer
+    c = lambda t: t.to(cuda, torch.float32) if t.dtype == torch.float64 else t.to(cuda)
+    xg = c(x).requires_grad_(True)
+    h, skips = xg, []
+    for d in lv:
+        tex, sh = texture.interpolate(h, c(d["face"]), c(d["bary"]), torch.cumsum(c(d["counts"]), 0, dtype=torch.int32), L)
+        y = d["v2f"](h, c(d["face"])) + d["f2f"](tex, sh, c(d["counts"]))
+        z = d["f2v"](y, c(d["face"]), c(d["nfc"]), c(d["ident"]), layers.SphHarmCoeff(L)(c(d["normal"])))
+        skips.append(z)
+        h = layers.Pool3d(d["method"])(z, c(d["vr"]), c(d["vm"]), torch.zeros(d["nvo"], 3, device=cuda))
+    for d, z in zip(reversed(lv), reversed(skips)):
+        h = d["up"](z + layers.Unpool3d()(h, c(d["vr"]), c(d["vm"])))
+    h.backward(c(g))
+
+    # float64 oracle composition
+    x64 = x.clone().requires_grad_(True)
+    r, skips64 = x64, []
+    for d in lv:
+        a, b, e = d["v2f64"], d["f2f64"], d["f2v64"]
+        cum = torch.cumsum(d["counts"], 0, dtype=torch.int32)
+        sh64 = R.sph_harm(d["bary"], L)
+        tex64 = R.texture_fwd(r, d["face"], d["bary"], cum)
+        spatial = (R.sph_harm(torch.eye(3, dtype=torch.float64), L) @ a.spatial_weights).reshape(3, a.in_channels, 1)
+        y = _ref_tail(a, R.v2f_fwd(r, spatial, d["face"]) @ a.depth_weights) + _ref_tail(b, R.f2f_fwd(tex64, b.weights, sh64, cum))
+        z = _ref_tail(e, R.f2v_fwd(y, e.spatial_weights, R.sph_harm(d["normal"], L), d["face"], d["nfc"], d["ident"]) @ e.depth_weights)
+        skips64.append(z)
+        if d["method"] == "max":
+            _, idx = R.maxpool_fwd(z.detach(), d["vr"], d["vm"], d["nvo"])
+            r = torch.gather(z, 0, idx.long())                  # every coarse row of this hierarchy has members
+        else:
+            r = R.avgpool_fwd(z, d["vr"], d["vm"], d["nvo"])
+    for d, z in zip(reversed(lv), reversed(skips64)):
+        r = _ref_tail(d["up64"], (z + R.unpool_fwd(r, d["vr"], d["vm"])) @ d["up64"].weights)
+    r.backward(g)
+    torch.cuda.synchronize()
+    assert_close(h, r.detach().numpy(), "stack output", TOL)
+    assert_close(xg.grad, x64.grad.numpy(), "stack grad_input", TOL)
+    for d in lv:
+        for k in ("v2f", "f2f", "f2v", "up"):
+            _compare_grads(d[k], d[k + "64"])

@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the mesh-conv hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload scene|shapes|pool|firstblock|tail|hierarchy] [--scale S]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload scene|shapes|pool|firstblock|tail|hierarchy|texture] [--scale S]
 
 A step is one forward+backward pass of the layer over one batch of seeded synthetic meshes
 already resident in HBM.  Default workload ``scene``: 8 room-like meshes of about 300 k
@@ -37,7 +37,7 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="scene", choices=["scene", "shapes", "pool", "firstblock", "tail", "hierarchy"],
+    ap.add_argument("--workload", default="scene", choices=["scene", "shapes", "pool", "firstblock", "tail", "hierarchy", "texture"],
                     help="scene: the headline layer (F2F+F2V, C=64); shapes: 16 small meshes V2F+F2F+F2V; pool: "
                          "1024x1024 grid max/avg pool + unpool; firstblock: the scene batch with the reference's first "
                          "block shapes, F2F 3->32 then F2V 32->32 with depth multiplier 2 (pi2_blocks.py:113-130)")
@@ -373,6 +373,65 @@ def run_tail(args, torch):
                             out_channels=Co))
 
 
+def run_texture(args, torch):
+    """Texture points of the scene batch's facets interpolated from 64-channel vertex features, with the SH basis of
+    their barycentric coordinates (forward), and the transposed gather (backward)."""
+    from picassoplus_amd import _lib, synthetic as S
+    from picassoplus_amd.mesh.pi_modules import texture
+    dev = torch.device("cuda:0")
+    C, L = 64, 3
+    mesh = S.scene_workload(seed=3000, n_rooms=8, scale=args.scale)
+    d = build_conv_inputs(mesh, C, L, seed=3000)
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+    face, bary, x = t(d["face"]), t(d["bary"]), t(d["x"]).requires_grad_(True)
+    cum = torch.cumsum(t(d["counts"]), 0, dtype=torch.int32)
+    g = torch.randn(d["T"], C, device=dev, generator=torch.Generator(device=dev).manual_seed(1))
+
+    def step():
+        tex, _ = texture.interpolate(x, face, bary, cum, L)
+        return torch.autograd.grad(tex, x, g)
+
+    timer = EventTimer(torch)
+    _lib.set_call_hook(timer)
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    timer.on = True
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    _lib.set_call_hook(None)
+    per_op = timer.summary()
+    ops = ["texture_fwd", "texture_bwd"]
+    bf = conv_bytes_flops(d, ops)
+    dom = max(ops, key=lambda k: per_op[k])
+    ach = bf[dom][0] / (per_op[dom] * 1e-3) / 1e9
+    total = sum(b for b, _ in bf.values())
+    extra = {}
+    if not args.no_cpu_baseline:
+        from oracle import torch_ref as R
+        torch.set_num_threads(os.cpu_count() or 1)
+        nf, nv = int(d["mf_in"][0]), int(d["nv_in"][0])               # first mesh of the batch
+        nt = int(d["counts"][:nf].sum())
+        f0, c0 = torch.from_numpy(d["face"][:nf]), torch.cumsum(torch.from_numpy(d["counts"][:nf]), 0, dtype=torch.int32)
+        b0, x0, g0 = torch.from_numpy(d["bary"][:nt]), torch.from_numpy(d["x"][:nv]), torch.randn(nt, C)
+        t0 = time.perf_counter()
+        R.texture_fwd(x0, f0, b0, c0); R.sph_harm(b0, L); R.texture_bwd(g0, nv, f0, b0, c0)
+        spent = time.perf_counter() - t0
+        extra["cpu_baseline"] = dict(value=nf / spent / 1e6, unit="Mfacets/s", cores=torch.get_num_threads(), kind="port",
+                                     sample="first of %d meshes (%d facets, %d texture points), one fwd+bwd pass, %.1f s"
+                                            % (len(d["mf_in"]), nf, nt, spent))
+    return dict(value=d["nf"] / (ms * 1e-3) / 1e6, ms_per_step=ms, **extra,
+                roofline=dict(bound="hbm", achieved=ach, peak=HBM_PEAK_GBS, unit="GB/s", frac=ach / HBM_PEAK_GBS,
+                              traffic=None, kernel=dom, kernel_ms=per_op[dom]),
+                ops={k: dict(ms=per_op[k], gbps=bf[k][0] / (per_op[k] * 1e-3) / 1e9) for k in ops},
+                hbm_gbps=total / (ms * 1e-3) / 1e9, hbm_frac=total / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                config=dict(workload="scene8x300k_texture_interpolation+SH_C64_L3_fp32_fwd+bwd", facets=d["nf"],
+                            vertices=d["nv"], texture_points=d["T"], channels=C, sh_degree=L))
+
+
 def run_hierarchy(args, torch):
     """Encoder-decoder stack of the mesh modules over one 2 M-facet mesh and four 4:1 coarser levels: per level
     V2F + (texture interpolation -> F2F) -> F2V at widths 32/64/128/256, max / avg pooling between levels, then
@@ -533,6 +592,8 @@ def main():
         res = run_tail(args, torch)
     elif args.workload == "hierarchy":
         res = run_hierarchy(args, torch)
+    elif args.workload == "texture":
+        res = run_texture(args, torch)
     else:
         res = run_conv_layer(args, torch, args.workload)
     if args.copy_calibration:

@@ -138,6 +138,81 @@ __global__ __launch_bounds__(kBlock) void texture_bwd_k(const float *__restrict_
     }
 }
 
+// The same sum for rows of at most 64 lanes per vertex and at least 8, with a shorter dependent chain per vertex:
+// row bounds -> eight adjacency entries -> their segment bounds -> the points of all eight facets as ONE flat
+// sequence, eight rows requested at a time.  Lane s of the group locates flat point t + s (a facet's points follow
+// its predecessor's, so the order of the sum is the one of texture_bwd_k and the results are identical); the lanes
+// pick the eight locations up with cross-lane reads.  Workgroups go round-robin to the eight accelerator dies, each
+// with an L2 of its own: die x takes the x-th contiguous eighth of the row blocks (the grid is 8 * ceil(blocks / 8)),
+// so that the three vertices that read a facet's rows mostly meet in one L2.
+template <int V>
+__global__ __launch_bounds__(kBlock) void texture_bwd_flat_k(const float *__restrict__ gtex, const float *__restrict__ bary,
+                                                             const int *__restrict__ cum, const int *__restrict__ rowptr,
+                                                             const int *__restrict__ colidx, float *__restrict__ gin,
+                                                             int64_t Nv, int64_t Nf, int T, int C, int Q, int lpr_log2)
+{
+    constexpr int EB = 8, PB = 8;
+    const int lpr = 1 << lpr_log2, rpb = kBlock >> lpr_log2;
+    const int lane = threadIdx.x & (lpr - 1), slot = threadIdx.x >> lpr_log2;
+    const int gbase = (threadIdx.x & 63) & ~(lpr - 1);          // first lane of my group within the wavefront
+    const int64_t nblk = (Nv + rpb - 1) / rpb, per_die = (nblk + 7) >> 3;
+    const int64_t blk = (int64_t)(blockIdx.x & 7) * per_die + (blockIdx.x >> 3);
+    const int64_t row = blk * rpb + slot;
+    if ((int64_t)(blockIdx.x >> 3) >= per_die || row >= Nv) return;      // whole groups leave together
+    const bool active = lane < Q;
+    const int c = lane * V;
+    const int e0 = rowptr[row], e1 = rowptr[row + 1];
+    Pack<V> acc = zero_pack<V>();
+    for (int eb = e0; eb < e1; eb += EB) {
+        int ent[EB], s0[EB], pre[EB + 1], corner[EB];
+#pragma unroll
+        for (int i = 0; i < EB; ++i) ent[i] = (eb + i < e1) ? colidx[eb + i] : -1;
+        int a[EB], b[EB];
+#pragma unroll
+        for (int i = 0; i < EB; ++i) {
+            const int f = ent[i] / 3;
+            corner[i] = ent[i] - 3 * f;
+            const bool ok = ent[i] >= 0 && f < Nf;
+            a[i] = (ok && f > 0) ? cum[f - 1] : 0;
+            b[i] = ok ? cum[f] : 0;
+        }
+        pre[0] = 0;
+#pragma unroll
+        for (int i = 0; i < EB; ++i) {
+            const int lo = a[i] < 0 ? 0 : a[i], hi = b[i] > T ? T : b[i];
+            s0[i] = lo;
+            pre[i + 1] = pre[i] + (hi > lo ? hi - lo : 0);
+        }
+        const int P = pre[EB];
+        for (int t = 0; t < P; t += PB) {
+            const int u = t + (lane & (PB - 1));
+            int k = s0[0] + u, cr = corner[0];
+#pragma unroll
+            for (int j = 1; j < EB; ++j) {
+                const bool past = u >= pre[j];
+                k = past ? s0[j] + (u - pre[j]) : k;
+                cr = past ? corner[j] : cr;
+            }
+            const int mine = u < P ? k * 4 + cr : -1;
+            float w[PB];
+            Pack<V> g[PB];
+#pragma unroll
+            for (int s = 0; s < PB; ++s) {
+                const int pk = __shfl(mine, gbase + s, 64);
+                const bool in = pk >= 0;
+                const int64_t kk = pk >> 2;
+                w[s] = in ? bary[3 * kk + (pk & 3)] : 0.f;
+                g[s] = (in && active) ? ldp<V>(gtex + kk * C + c) : zero_pack<V>();
+            }
+#pragma unroll
+            for (int s = 0; s < PB; ++s)
+#pragma unroll
+                for (int x = 0; x < V; ++x) acc.v[x] = fmaf(w[s], g[s].v[x], acc.v[x]);
+        }
+    }
+    if (active) stp<V>(gin + row * C + c, acc);
+}
+
 static inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 }  // namespace pmesh
@@ -190,7 +265,15 @@ extern "C" int pmesh_texture_bwd(const float *grad_texture, const float *bary, c
     const RowShape rs = row_shape(vec ? C / 4 : C);
     const int64_t blocks = ceil_div(Nv, rs.rpb);
     PM_REQUIRE(grid_ok(blocks), "texture_bwd: grid too large");
-    if (vec)
+    // rows of 8 to 64 lanes take the flat kernel (a point's location travels as 4 * row + corner in 32 bits)
+    const bool flat = rs.lpr >= 8 && rs.lpr <= 64 && rs.items <= rs.lpr && T < (int64_t(1) << 29);
+    const int64_t fblocks = 8 * ceil_div(blocks, 8);
+    PM_REQUIRE(grid_ok(fblocks), "texture_bwd: grid too large");
+    if (vec && flat)
+        texture_bwd_flat_k<4><<<dim3((unsigned)fblocks), dim3(kBlock), 0, st>>>(grad_texture, bary, cum_texture, rowptr, colidx, grad_input, Nv, Nf, (int)T, C, rs.items, rs.lpr_log2);
+    else if (flat)
+        texture_bwd_flat_k<1><<<dim3((unsigned)fblocks), dim3(kBlock), 0, st>>>(grad_texture, bary, cum_texture, rowptr, colidx, grad_input, Nv, Nf, (int)T, C, rs.items, rs.lpr_log2);
+    else if (vec)
         texture_bwd_k<4><<<dim3((unsigned)blocks), dim3(kBlock), 0, st>>>(grad_texture, bary, cum_texture, rowptr, colidx, grad_input, Nv, Nf, T, C, rs.items, rs.lpr_log2);
     else
         texture_bwd_k<1><<<dim3((unsigned)blocks), dim3(kBlock), 0, st>>>(grad_texture, bary, cum_texture, rowptr, colidx, grad_input, Nv, Nf, T, C, rs.items, rs.lpr_log2);

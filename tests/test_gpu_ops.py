@@ -96,7 +96,7 @@ def test_v2f_parity(cuda, mesh, C, r):
 
 # ------------------------------------------------------------------ texture points from vertex features
 @pytest.mark.parametrize("mesh,C,kmax,L", [("tetra", 4, 3, 3), ("octa", 3, 9, 3), ("sphere2", 64, 9, 3), ("fans", 32, 5, 2),
-                                           ("room_small", 64, 9, 3), ("torus", 130, 4, 5), ("sphere3", 7, 20, None),
+                                           ("room_small", 64, 9, 3), ("room_small", 96, 9, 1), ("fans", 128, 3, 3), ("torus", 130, 4, 5), ("sphere3", 7, 20, None),
                                            ("sphere2", 2048, 2, 0)])
 def test_texture_interpolation_parity(cuda, mesh, C, kmax, L):
     say("case texture", mesh, C, kmax, L)

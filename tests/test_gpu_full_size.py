@@ -9,7 +9,7 @@ from oracle import loops
 from picassoplus_amd import _lib, synthetic as S
 from picassoplus_amd.mesh import topology
 from picassoplus_amd.mesh.layers import sph_harm_values
-from picassoplus_amd.mesh.pi_modules import conv3d, mesh_conv3d, pool3d, unpool3d
+from picassoplus_amd.mesh.pi_modules import conv3d, mesh_conv3d, pool3d, texture, unpool3d
 from util import assert_close, dev
 
 pytestmark = pytest.mark.gpu
@@ -41,7 +41,9 @@ def scene(cuda):
     d = dict(nv=nv, nf=nf, T=int(counts.sum()), C=C, counts=counts)
     d["face"] = dev(f, cuda)
     d["cum"] = torch.cumsum(dev(counts, cuda), 0, dtype=torch.int32)
-    d["sh"] = sph_harm_values(dev(bary.astype(np.float32), cuda), L)
+    d["bary"] = dev(bary.astype(np.float32), cuda)
+    d["bary64"], d["face_np"] = bary, f
+    d["sh"] = sph_harm_values(d["bary"], L)
     d["coeff"] = sph_harm_values(dev(normal.astype(np.float32), cuda), L)
     d["tex"] = dev(rng.uniform(-1, 1, (d["T"], C)).astype(np.float32), cuda)
     d["w_f2f"] = dev(S.xavier_uniform(rng, (C, C, 16), C * 16, C * 16).astype(np.float32), cuda)
@@ -138,6 +140,35 @@ def test_v2f_full_size_adjoints(cuda, scene):
     scale = float(out.double().norm() * g.double().norm())
     _adjoint_ok(lhs, _dot(x, gx), scale, "<v2f(x), g> = <x, grad_input>")
     _adjoint_ok(lhs, _dot(w, gw), scale, "<v2f(x), g> = <filter, grad_filter>")
+
+
+def test_texture_interpolation_full_size(cuda, scene):
+    """Adjoint identity, the invariants of barycentric weights (constants stay constant), the fused basis against the
+    stand-alone kernel, and oracle parity on a random sample of facets."""
+    d = scene
+    say("case texture full size", d["nf"], d["T"])
+    gen = torch.Generator(device=cuda).manual_seed(9)
+    x = torch.randn(d["nv"], d["C"], device=cuda, generator=gen).requires_grad_(True)
+    g = torch.randn(d["T"], d["C"], device=cuda, generator=gen)
+    tex, sh = texture.interpolate(x, d["face"], d["bary"], d["cum"], 3)
+    (gx,) = torch.autograd.grad(tex, x, g)
+    torch.cuda.synchronize()
+    assert torch.equal(sh, d["sh"])
+    _adjoint_ok(_dot(tex, g), _dot(x, gx), float(tex.double().norm() * g.double().norm()), "<tex(x), g> = <x, grad_input>")
+    const = texture.interpolate(torch.full((d["nv"], 8), 2.5, device=cuda), d["face"], d["bary"], d["cum"], None)
+    assert float((const - 2.5).abs().max()) < 1e-5
+    # every gradient row sums what its vertex's corners received: total mass is preserved (weights sum to one)
+    _adjoint_ok(float(gx.double().sum()), float(g.double().sum()), float(g.double().abs().sum()), "sum of grad_input = sum of grad_texture")
+    # oracle on 500 random facets: their rows of the output
+    rng = np.random.default_rng(10)
+    pick = np.sort(rng.choice(d["nf"], 500, replace=False))
+    cum = np.cumsum(d["counts"])
+    xs = x.detach().cpu().numpy().astype(np.float64)
+    tex_np = tex.detach().cpu().numpy()
+    for f in pick[:500]:
+        k0, k1 = (cum[f - 1] if f else 0), cum[f]
+        ref = d["bary64"][k0:k1] @ xs[d["face_np"][f].astype(np.int64)]
+        assert np.abs(tex_np[k0:k1] - ref).max() <= 1e-5 * max(np.abs(ref).max(), 1.0)
 
 
 def test_pool_full_size_invariants(cuda):

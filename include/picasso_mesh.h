@@ -227,6 +227,14 @@ int pmesh_count_vertex_adjface(const int32_t *rowptr, int32_t *nf_count, int64_t
 int pmesh_triangle_geometry(const float *vertex, const int32_t *face, float *geometry, int64_t Nv,
                             int64_t Nf, int vertex_stride, pmesh_stream_t stream);
 
+/* pmesh_facet_frame gives, in one pass over the facets, what a network computes per mesh level before its
+ * facet2vertex convolutions: geometry (Nf,5) as pmesh_triangle_geometry; normal (Nf,3) = the unit normal turned
+ * towards the origin as the viewpoint, i.e. negated when -centre . normal < 0 (get_oriented_normals,
+ * picasso/networks/scene_seg.py:117-124); coeff (Nf,(L+1)^2) = SH basis at that normal (cal_sph_harm on the
+ * oriented normals, scene_seg.py:149,164).  Any output pointer may be NULL. */
+int pmesh_facet_frame(const float *vertex, const int32_t *face, float *geometry, float *normal, float *coeff,
+                      int64_t Nv, int64_t Nf, int vertex_stride, int L, pmesh_stream_t stream);
+
 /* pmesh_combine_clusters replaces combineClustersLauncher (decimate_gpu.cu:750-810, decimate.py:53-67): the
  * cluster maps of two consecutive decimation steps -- A over nv_a fine vertices, B over the nv_b vertices A
  * keeps -- become one pair (rep_out, map_out) over the fine vertices, the vt_replace / vt_map a pooling layer

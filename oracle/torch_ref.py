@@ -259,6 +259,15 @@ def face_normals(vertex, face):
     return n / torch.linalg.norm(n, dim=-1, keepdim=True).clamp_min(1e-30)
 
 
+def oriented_normals(normals, vertex, face):
+    """Normals turned towards the origin as the viewpoint (picasso/networks/scene_seg.py:117-124): the sign of
+    -centre . normal, with 0 counted as +1."""
+    centre = vertex[_long(face)][:, :, :3].mean(1)
+    sign = torch.sign((-centre * normals).sum(-1, keepdim=True))
+    sign = torch.where(sign > -1, torch.ones_like(sign), sign)
+    return normals * sign
+
+
 # --------------------------------------------------------------------------
 # pointwise tail of the conv modules  (picasso/mesh/layers.py:114-119, 169-174, 232-238)
 # --------------------------------------------------------------------------

@@ -11,7 +11,7 @@ from ctypes import c_char_p, c_int, c_int64, c_size_t, c_void_p
 _HERE = os.path.dirname(os.path.abspath(__file__))
 # PICASSO_MESH_LIB points at an alternative build of the same ABI (kernel experiments)
 LIB_PATH = os.environ.get("PICASSO_MESH_LIB") or os.path.join(_HERE, "csrc", "libpicasso_mesh.so")
-ABI_VERSION = 9
+ABI_VERSION = 10
 
 P, I, L, Z = c_void_p, c_int, c_int64, c_size_t
 
@@ -46,6 +46,7 @@ SIGNATURES = {
     "pmesh_count_vertex_adjface": (I, [P, P, L, P]),
     "pmesh_triangle_geometry": (I, [P, P, P, L, L, I, P]),
     "pmesh_sph_harm": (I, [P, P, L, I, P]),
+    "pmesh_facet_frame": (I, [P, P, P, P, P, L, L, I, I, P]),
     "pmesh_texture_fwd": (I, [P, P, P, P, P, P, L, L, L, I, I, P]),
     "pmesh_texture_bwd": (I, [P, P, P, P, P, P, L, L, L, I, P]),
     "pmesh_combine_clusters": (I, [P, P, P, P, P, P, P, L, L, P]),

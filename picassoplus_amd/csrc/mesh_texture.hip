@@ -213,6 +213,48 @@ __global__ __launch_bounds__(kBlock) void texture_bwd_flat_k(const float *__rest
     if (active) stp<V>(gin + row * C + c, acc);
 }
 
+// Per-level producer of the facet2vertex coefficients in one pass: triangle geometry (unit normal, plane offset,
+// area: picasso/mesh/pi_modules/decimate.py:70-85), the normal turned towards the origin as the viewpoint
+// (picasso/networks/scene_seg.py:117-124: flipped when -centre . normal < 0), and the spherical-harmonic basis at the
+// oriented normal (scene_seg.py:149,164).  Any of the three outputs may be absent.
+__global__ __launch_bounds__(kBlock) void facet_frame_k(const float *__restrict__ vertex, const int *__restrict__ face,
+                                                       float *__restrict__ geometry, float *__restrict__ normal,
+                                                       float *__restrict__ coeff, int64_t Nf, int vstride, int L)
+{
+    const int64_t f = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (f >= Nf) return;
+    const float *a = vertex + (int64_t)face[3 * f] * vstride;
+    const float *b = vertex + (int64_t)face[3 * f + 1] * vstride;
+    const float *c = vertex + (int64_t)face[3 * f + 2] * vstride;
+    const float ax = a[0], ay = a[1], az = a[2], bx = b[0], by = b[1], bz = b[2], cx = c[0], cy = c[1], cz = c[2];
+    const float ux = bx - ax, uy = by - ay, uz = bz - az;
+    const float vx = cx - ax, vy = cy - ay, vz = cz - az;
+    float nx = uy * vz - uz * vy, ny = uz * vx - ux * vz, nz = ux * vy - uy * vx;
+    const float len = sqrtf(nx * nx + ny * ny + nz * nz);
+    const float inv = 1.0f / (len + 1e-10f);
+    nx *= inv; ny *= inv; nz *= inv;
+    if (geometry) {
+        float *g = geometry + 5 * f;
+        g[0] = nx; g[1] = ny; g[2] = nz;
+        g[3] = -(nx * ax + ny * ay + nz * az);
+        g[4] = 0.5f * len;
+    }
+    // sign(-centre . n), with 0 counted as +1
+    const float mx = (ax + bx + cx) / 3.0f, my = (ay + by + cy) / 3.0f, mz = (az + bz + cz) / 3.0f;
+    const float towards = -(mx * nx + my * ny + mz * nz);
+    if (towards < 0.f) { nx = -nx; ny = -ny; nz = -nz; }
+    if (normal) {
+        normal[3 * f] = nx; normal[3 * f + 1] = ny; normal[3 * f + 2] = nz;
+    }
+    if (coeff) {
+        const int B = (L + 1) * (L + 1);
+        float v[36];
+        sph_harm_at(nx, ny, nz, L, v);
+        float *o = coeff + f * B;
+        for (int i = 0; i < B; ++i) o[i] = v[i];
+    }
+}
+
 static inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 }  // namespace pmesh
@@ -278,5 +320,19 @@ extern "C" int pmesh_texture_bwd(const float *grad_texture, const float *bary, c
     else
         texture_bwd_k<1><<<dim3((unsigned)blocks), dim3(kBlock), 0, st>>>(grad_texture, bary, cum_texture, rowptr, colidx, grad_input, Nv, Nf, T, C, rs.items, rs.lpr_log2);
     PM_LAUNCHED("texture_bwd");
+    return 0;
+}
+
+extern "C" int pmesh_facet_frame(const float *vertex, const int32_t *face, float *geometry, float *normal, float *coeff,
+                                 int64_t Nv, int64_t Nf, int vertex_stride, int L, pmesh_stream_t stream)
+{
+    clear_error();
+    PM_REQUIRE(Nv >= 0 && Nf >= 0 && vertex_stride >= 3, "facet_frame: bad sizes");
+    PM_REQUIRE(!coeff || (L >= 0 && L <= 5), "facet_frame: basis degree %d outside 0..5", L);
+    if (Nf == 0 || !(geometry || normal || coeff)) return 0;
+    PM_REQUIRE(vertex && face, "facet_frame: null pointer");
+    PM_REQUIRE(Nv * vertex_stride < (int64_t(1) << 40) && grid_ok(ceil_div(Nf, kBlock)), "facet_frame: sizes too large");
+    facet_frame_k<<<dim3((unsigned)ceil_div(Nf, kBlock)), dim3(kBlock), 0, (hipStream_t)stream>>>(vertex, face, geometry, normal, coeff, Nf, vertex_stride, L);
+    PM_LAUNCHED("facet_frame");
     return 0;
 }

@@ -1,5 +1,5 @@
-"""Per-level producers of the convolution inputs: adjacent-facet counts of the output vertices and
-triangle geometry, and the composition of two decimation steps' cluster maps, with the reference's function
+"""Per-level producers of the convolution inputs: adjacent-facet counts of the output vertices,
+triangle geometry, oriented normals with their basis coefficients, and the composition of two decimation steps' cluster maps, with the reference's function
 names (picasso/mesh/pi_modules/decimate.py:53-93).  Mesh decimation itself is not part of this package."""
 import torch
 
@@ -39,6 +39,32 @@ def compute_triangle_geometry_(vertex, face):
         _lib.call("pmesh_triangle_geometry", vertex.data_ptr(), face.data_ptr(), out.data_ptr(), vertex.shape[0],
                   face.shape[0], vertex.shape[1], stream_of(vertex))
     return out
+
+
+def facet_frame_(vertex, face, degree=3):
+    """Triangle geometry, oriented normals and their spherical-harmonic coefficients in one native pass:
+    what a network prepares per mesh level for its facet2vertex convolutions (picasso/networks/scene_seg.py:146-149,
+    161-164: ``compute_triangle_geometry_`` -> ``get_oriented_normals`` -> ``cal_sph_harm``).
+
+    returns (geometry (Nf, 5), face_normals (Nf, 3) turned towards the origin, filt_coeff (Nf, (degree+1)^2));
+    ``degree`` None skips the coefficients (third result None)."""
+    check_input(vertex, "vertex", 2, F32)
+    check_input(face, "face", 2, I32)
+    if vertex.shape[1] < 3 or face.shape[1] != 3:
+        raise RuntimeError("vertex must have at least 3 columns and face exactly 3")
+    if degree is not None and (degree < 0 or degree > 5):
+        raise NotImplementedError("spherical harmonics are implemented for degree 0..5")
+    dev = same_device(vertex, face)
+    topology._check_range_cached(face, vertex.shape[0])
+    nf = face.shape[0]
+    with torch.cuda.device(dev):
+        geo = torch.empty((nf, 5), dtype=F32, device=dev)
+        nrm = torch.empty((nf, 3), dtype=F32, device=dev)
+        coeff = torch.empty((nf, (degree + 1) ** 2), dtype=F32, device=dev) if degree is not None else None
+        _lib.call("pmesh_facet_frame", vertex.data_ptr(), face.data_ptr(), geo.data_ptr(), nrm.data_ptr(),
+                  coeff.data_ptr() if coeff is not None else None, vertex.shape[0], nf, vertex.shape[1],
+                  int(degree) if degree is not None else 0, stream_of(vertex))
+    return geo, nrm, coeff
 
 
 def combine_clusters_(repA, mapA, repB, mapB):

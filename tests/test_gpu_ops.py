@@ -545,3 +545,36 @@ def test_adjface_count_and_triangle_geometry(cuda, mesh):
     assert_close(geo[:, 4], ref_geo[:, 4], "triangle area")
     assert_close(geo[okt][:, :3], R.face_normals(torch.from_numpy(p), torch.from_numpy(f)).numpy()[ok],
                  "normals vs oracle", 1e-4)
+
+
+@pytest.mark.parametrize("mesh,L", [("octa", 3), ("sphere3", 3), ("room_small", 5), ("torus", None)])
+def test_facet_frame_parity(cuda, mesh, L):
+    """Geometry, oriented normals and their basis coefficients from one kernel against the oracle's three steps."""
+    say("case facet_frame", mesh, L)
+    from picassoplus_amd.mesh.pi_modules import geometry
+    from oracle import torch_ref as R
+    v, f = mesh_case(mesh)
+    rng = np.random.default_rng(14)
+    v = v + rng.normal(0, 0.3, 3)                                  # viewpoint off-centre
+    vx = np.concatenate([v, rng.uniform(0, 1, (v.shape[0], 3))], 1).astype(np.float32)     # position + colour
+    geo, nrm, coeff = geometry.facet_frame_(dev(vx, cuda), dev(f, cuda), L)
+    torch.cuda.synchronize()
+    assert torch.equal(geo, geometry.compute_triangle_geometry_(dev(vx, cuda), dev(f, cuda)))
+    p = torch.from_numpy(vx[:, :3].astype(np.float64))
+    n_ref = R.face_normals(p, torch.from_numpy(f))
+    o_ref = R.oriented_normals(n_ref, p, torch.from_numpy(f)).numpy()
+    centre = vx[:, :3].astype(np.float64)[f.astype(np.int64)].mean(1)
+    # compared on well-shaped facets (float32 cross products of thin or collapsed triangles cancel) whose sign is
+    # not a rounding matter
+    pp = p.numpy()
+    e1, e2 = pp[f[:, 1]] - pp[f[:, 0]], pp[f[:, 2]] - pp[f[:, 0]]
+    shaped = np.linalg.norm(np.cross(e1, e2), axis=1) > 0.1 * np.linalg.norm(e1, axis=1) * np.linalg.norm(e2, axis=1)
+    sure = shaped & (np.abs((centre * n_ref.numpy()).sum(1)) > 1e-4)
+    assert sure.mean() > 0.5
+    assert_close(nrm[torch.from_numpy(sure).to(cuda)], o_ref[sure], "oriented normals", 1e-4)
+    assert torch.equal(nrm.abs(), geo[:, :3].abs())
+    if L is None:
+        assert coeff is None
+    else:
+        assert torch.equal(coeff, sph_harm_values(nrm, L))
+        assert_close(coeff[torch.from_numpy(sure).to(cuda)], loops.sph_harm(o_ref[sure], L), "coefficients", 1e-4)

@@ -61,6 +61,8 @@ def test_argument_errors_without_launching():
     assert b"null pointer" in lib.pmesh_last_error()
     assert lib.pmesh_texture_bwd(None, None, None, None, None, None, 4, 2, -1, 8, None) != 0
     assert lib.pmesh_texture_fwd(None, None, None, None, None, None, 4, 2, 0, 8, 3, None) == 0
+    assert lib.pmesh_facet_frame(None, None, None, None, None, 4, 2, 2, 3, None) != 0
+    assert lib.pmesh_facet_frame(None, None, None, None, None, 4, 2, 3, 3, None) == 0      # nothing asked for
     # empty problems succeed without touching the (null) pointers
     assert lib.pmesh_v2f_fwd(None, None, None, None, 0, 0, 8, 1, None) == 0
     assert lib.pmesh_last_error() == b""

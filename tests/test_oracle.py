@@ -460,3 +460,32 @@ def test_texture_interpolation_pins():
     assert abs((tex * g).sum() - (x * gl).sum()) < 1e-9 * abs((tex * g).sum())
     # float32 loops stay close to float64
     assert rel_err(loops.texture_fwd(x, f, bary, cum, np.float32), tex) < 1e-6
+
+
+def test_oriented_normals_pins():
+    """Hand case, an element-by-element restatement, and what orientation towards the origin means."""
+    v = T(np.array([[1.0, 0, 2], [0, 1, 2], [0, 0, 2], [1, 0, -3], [0, 1, -3], [0, 0, -3]]))
+    f = T(np.array([[0, 1, 2], [3, 4, 5], [2, 1, 0]], np.int32))
+    n = torch_ref.face_normals(v, f)
+    assert np.allclose(n.numpy(), [[0, 0, 1], [0, 0, 1], [0, 0, -1]], atol=EPS)
+    o = torch_ref.oriented_normals(n, v, f).numpy()
+    # facets above the origin look down, the one below looks up, whatever the winding
+    assert np.allclose(o, [[0, 0, -1], [0, 0, 1], [0, 0, -1]], atol=EPS)
+    # a plane through the origin (-centre . n = 0) keeps its normal
+    v0 = T(np.array([[1.0, 0, 0], [0, 1, 0], [-1, -1, 0]]))
+    f0 = T(np.array([[0, 1, 2]], np.int32))
+    n0 = torch_ref.face_normals(v0, f0)
+    assert np.array_equal(torch_ref.oriented_normals(n0, v0, f0).numpy(), n0.numpy())
+    rng = np.random.default_rng(31)
+    vv, ff = mesh_case("room_small")
+    vv = vv + rng.normal(0, 1, 3)                                   # origin somewhere inside the scene
+    n = torch_ref.face_normals(T(vv), T(ff))
+    o = torch_ref.oriented_normals(n, T(vv), T(ff)).numpy()
+    centre = vv[ff.astype(np.int64)].mean(1)
+    for i in range(0, ff.shape[0], 7):                             # the reference's rule, one facet at a time
+        s = np.sign(-(centre[i] * n[i].numpy()).sum())
+        assert np.array_equal(o[i], n[i].numpy() * (s if s == -1 else 1.0))
+    assert ((centre * o).sum(1) <= 1e-12).all()                     # every normal faces the origin
+    assert np.allclose(np.abs(o), np.abs(n.numpy()))
+    assert np.array_equal(torch_ref.oriented_normals(T(o), T(vv), T(ff)).numpy(), o)    # idempotent
+    assert (o != n.numpy()).any() and (o == n.numpy()).all(1).any()

@@ -160,49 +160,65 @@ __global__ __launch_bounds__(kBlock) void texture_bwd_flat_k(const float *__rest
     const int64_t row = blk * rpb + slot;
     if ((int64_t)(blockIdx.x >> 3) >= per_die || row >= Nv) return;      // whole groups leave together
     const bool active = lane < Q;
-    const int c = lane * V;
+    // byte offsets into grad_texture and bary fit 32 bits (checked by the caller): the vector ALU is this kernel's
+    // busiest unit, so a point's location is turned into its two offsets once, by the lane that locates it
+    const unsigned row_bytes = (unsigned)C * 4u, col_bytes = active ? (unsigned)(lane * V) * 4u : 0u;   // idle lanes read column 0
+    const char *gbytes = reinterpret_cast<const char *>(gtex), *bbytes = reinterpret_cast<const char *>(bary);
     const int e0 = rowptr[row], e1 = rowptr[row + 1];
     Pack<V> acc = zero_pack<V>();
     for (int eb = e0; eb < e1; eb += EB) {
-        int ent[EB], s0[EB], pre[EB + 1], corner[EB];
+        // every load below is unconditional (indices clamped into the row, results masked afterwards): a conditional
+        // load costs a branch of its own
+        int ent[EB], pre[EB + 1], key[EB];
 #pragma unroll
-        for (int i = 0; i < EB; ++i) ent[i] = (eb + i < e1) ? colidx[eb + i] : -1;
+        for (int i = 0; i < EB; ++i) {
+            const int idx = eb + i < e1 ? eb + i : e1 - 1;
+            ent[i] = colidx[idx];
+        }
+#pragma unroll
+        for (int i = 0; i < EB; ++i) ent[i] = (eb + i < e1) ? ent[i] : -1;
         int a[EB], b[EB];
 #pragma unroll
         for (int i = 0; i < EB; ++i) {
             const int f = ent[i] / 3;
-            corner[i] = ent[i] - 3 * f;
-            const bool ok = ent[i] >= 0 && f < Nf;
-            a[i] = (ok && f > 0) ? cum[f - 1] : 0;
-            b[i] = ok ? cum[f] : 0;
+            int fc = f < 0 ? 0 : f;
+            fc = fc < (int)Nf ? fc : (int)Nf - 1;
+            a[i] = cum[fc > 0 ? fc - 1 : 0];
+            b[i] = cum[fc];
         }
         pre[0] = 0;
 #pragma unroll
         for (int i = 0; i < EB; ++i) {
-            const int lo = a[i] < 0 ? 0 : a[i], hi = b[i] > T ? T : b[i];
-            s0[i] = lo;
+            const int f = ent[i] / 3;
+            const bool ok = ent[i] >= 0 && f < Nf;
+            int lo = (ok && f > 0) ? a[i] : 0, hi = ok ? b[i] : 0;
+            lo = lo < 0 ? 0 : lo;
+            hi = hi > T ? T : hi;
             pre[i + 1] = pre[i] + (hi > lo ? hi - lo : 0);
+            // flat point u of entry i is row lo + (u - pre[i]) with corner ent % 3: 4 * row + corner = 4 * u + key
+            key[i] = 4 * (lo - pre[i]) + (ent[i] - 3 * f);
         }
         const int P = pre[EB];
         for (int t = 0; t < P; t += PB) {
-            const int u = t + (lane & (PB - 1));
-            int k = s0[0] + u, cr = corner[0];
+            // slots past the end repeat the step's first point with weight zero
+            const int ur = t + (lane & (PB - 1));
+            const bool mine = ur < P;
+            const int u = mine ? ur : t;
+            int kq = key[0];
 #pragma unroll
-            for (int j = 1; j < EB; ++j) {
-                const bool past = u >= pre[j];
-                k = past ? s0[j] + (u - pre[j]) : k;
-                cr = past ? corner[j] : cr;
-            }
-            const int mine = u < P ? k * 4 + cr : -1;
+            for (int j = 1; j < EB; ++j) kq = u >= pre[j] ? key[j] : kq;
+            kq += 4 * u;                                          // 4 * row + corner of my point
+            const unsigned my_g = (unsigned)(kq >> 2) * row_bytes;
+            const unsigned my_b = ((unsigned)(kq >> 2) * 12u + (unsigned)(kq & 3) * 4u) | (mine ? 0u : 1u);
             float w[PB];
             Pack<V> g[PB];
 #pragma unroll
             for (int s = 0; s < PB; ++s) {
-                const int pk = __shfl(mine, gbase + s, 64);
-                const bool in = pk >= 0;
-                const int64_t kk = pk >> 2;
-                w[s] = in ? bary[3 * kk + (pk & 3)] : 0.f;
-                g[s] = (in && active) ? ldp<V>(gtex + kk * C + c) : zero_pack<V>();
+                const unsigned og = (unsigned)__shfl((int)my_g, gbase + s, 64);
+                const unsigned ob = (unsigned)__shfl((int)my_b, gbase + s, 64);
+                const float wr = *reinterpret_cast<const float *>(bbytes + (ob & ~1u));
+                w[s] = (ob & 1u) ? 0.f : wr;
+                g[s] = ldp<V>(reinterpret_cast<const float *>(gbytes + (og + col_bytes)));
             }
 #pragma unroll
             for (int s = 0; s < PB; ++s)
@@ -210,7 +226,7 @@ __global__ __launch_bounds__(kBlock) void texture_bwd_flat_k(const float *__rest
                 for (int x = 0; x < V; ++x) acc.v[x] = fmaf(w[s], g[s].v[x], acc.v[x]);
         }
     }
-    if (active) stp<V>(gin + row * C + c, acc);
+    if (active) stp<V>(gin + row * C + lane * V, acc);
 }
 
 // Per-level producer of the facet2vertex coefficients in one pass: triangle geometry (unit normal, plane offset,
@@ -307,8 +323,9 @@ extern "C" int pmesh_texture_bwd(const float *grad_texture, const float *bary, c
     const RowShape rs = row_shape(vec ? C / 4 : C);
     const int64_t blocks = ceil_div(Nv, rs.rpb);
     PM_REQUIRE(grid_ok(blocks), "texture_bwd: grid too large");
-    // rows of 8 to 64 lanes take the flat kernel (a point's location travels as 4 * row + corner in 32 bits)
-    const bool flat = rs.lpr >= 8 && rs.lpr <= 64 && rs.items <= rs.lpr && T < (int64_t(1) << 29);
+    // rows of 8 to 64 lanes take the flat kernel (a point's location travels as 32-bit byte offsets)
+    const bool flat = rs.lpr >= 8 && rs.lpr <= 64 && rs.items <= rs.lpr && T < (int64_t(1) << 28) &&
+                      T * C * 4 < (int64_t(1) << 32) - 4096;
     const int64_t fblocks = 8 * ceil_div(blocks, 8);
     PM_REQUIRE(grid_ok(fblocks), "texture_bwd: grid too large");
     if (vec && flat)

@@ -251,3 +251,86 @@ def test_dense_tail_full_size_adjoints_and_sample_parity(cuda, ci, co):
     gz = torch.where(yr > 0, g, torch.zeros_like(g)).double()
     assert_close(gwr, (x.double().t() @ gz).cpu().numpy(), "dense grad_weight")
     assert_close(gbr, gz.sum(0).cpu().numpy(), "dense grad_bias (masked)")
+
+
+def test_config_sphere_v2f_then_f2v_forward(cuda):
+    """The single-mesh configuration: jittered icosphere of level 5 (10 242 vertices, 20 480 facets), one V2F
+    convolution 32 -> 64 then one F2V convolution 64 -> 64, degree 3, Uniform(-1, 1) features, Xavier-uniform
+    weights, forward only -- modules on the GPU against the float64 oracle composition."""
+    from oracle import torch_ref as R
+    from picassoplus_amd.mesh import layers
+    say("case sphere level 5, V2F then F2V")
+    mesh = S.sphere_workload(seed=1000, level=5)
+    v, f = mesh["vertex"], mesh["face"]
+    nv, nf = v.shape[0], f.shape[0]
+    assert (nv, nf) == (10242, 20480)
+    rng = np.random.default_rng(1000)
+    x = rng.uniform(-1, 1, (nv, 32))
+    normal, _ = S.triangle_normals_areas(v, f)
+    nfc = S.vertex_facet_count(f, np.arange(nv), nv).astype(np.int32)
+    torch.manual_seed(1000)
+    v2f = layers.V2FConv3d(32, 64, 3, with_bn=False).to(cuda)
+    f2v = layers.F2VConv3d(64, 64, 3, with_bn=False).to(cuda)
+    with torch.no_grad():
+        for m in (v2f, f2v):
+            for p in m.parameters():
+                if p.dim() > 1 and p.numel() > p.shape[-1]:
+                    torch.nn.init.xavier_uniform_(p.view(p.shape[0], -1) if p.dim() == 3 else p)
+            m.biases.uniform_(-0.1, 0.1)
+        face, ident = dev(f, cuda), torch.arange(nv, dtype=torch.int32, device=cuda)
+        coeff = sph_harm_values(dev(normal.astype(np.float32), cuda), 3)
+        y = f2v(v2f(dev(x.astype(np.float32), cuda), face), face, dev(nfc, cuda), ident, coeff)
+    torch.cuda.synchronize()
+    T64 = lambda t: t.detach().cpu().double()
+    f64, x64 = torch.from_numpy(f), torch.from_numpy(x.astype(np.float32)).double()
+    spatial = (R.sph_harm(torch.eye(3, dtype=torch.float64), 3) @ T64(v2f.spatial_weights)).reshape(3, 32, 1)
+    h = torch.relu(R.v2f_fwd(x64, spatial, f64) @ T64(v2f.depth_weights) + T64(v2f.biases))
+    c64 = R.sph_harm(torch.from_numpy(normal.astype(np.float32)).double(), 3)
+    h = R.f2v_fwd(h, T64(f2v.spatial_weights), c64, f64, torch.from_numpy(nfc), torch.arange(nv, dtype=torch.int32))
+    ref = torch.relu(h @ T64(f2v.depth_weights) + T64(f2v.biases))
+    assert float(ref.abs().max()) > 0
+    assert_close(y, ref.numpy(), "sphere configuration output", 2e-5)
+
+
+def test_config_shapes_block_forward_backward(cuda):
+    """The shapes configuration at full size (16 meshes, about 329 k facets, C = 64, three texture points per
+    facet): y = F2V(V2F(X) + F2F(texture(X))) with dL/dy ~ N(0, 1); output and the gradients of X and of the
+    three filters against the float64 oracle."""
+    from oracle import torch_ref as R
+    from picassoplus_amd.mesh.pi_modules import texture
+    say("case shapes block at full size")
+    mesh = S.shapes_workload(seed=2000, n_meshes=16)
+    v, f = mesh["vertex"], mesh["face"]
+    nv, nf, C, L = v.shape[0], f.shape[0], 64, 3
+    rng = np.random.default_rng(2000)
+    normal, _ = S.triangle_normals_areas(v, f)
+    counts, bary, _ = S.texture_points(rng, nf, np.full(nf, 3, np.int32))
+    bary = bary.astype(np.float32)
+    nfc = np.maximum(S.vertex_facet_count(f, np.arange(nv), nv), 1).astype(np.int32)
+    x = rng.uniform(-1, 1, (nv, C)).astype(np.float32)
+    w_v2f = S.xavier_uniform(rng, (3, C, 1), C, 3 * C).astype(np.float32)
+    w_f2f = S.xavier_uniform(rng, (C, C, 16), C * 16, C * 16).astype(np.float32)
+    w_f2v = S.xavier_uniform(rng, (16, C, 1), C, 16 * C).astype(np.float32)
+    gy = rng.normal(0, 1, (nv, C)).astype(np.float32)
+    leaves = [dev(a, cuda).requires_grad_(True) for a in (x, w_v2f, w_f2f, w_f2v)]
+    xg, wv, wf, wo = leaves
+    face, cum = dev(f, cuda), torch.cumsum(dev(counts, cuda), 0, dtype=torch.int32)
+    ident = torch.arange(nv, dtype=torch.int32, device=cuda)
+    tex, sh = texture.interpolate(xg, face, dev(bary, cuda), cum, L)
+    y = conv3d.facet2vertex(conv3d.vertex2facet(xg, wv, face) + conv3d.facet2facet(tex, wf, sh, cum), wo,
+                            sph_harm_values(dev(normal.astype(np.float32), cuda), L), face, dev(nfc, cuda), ident)
+    grads = torch.autograd.grad(y, leaves, dev(gy, cuda))
+    torch.cuda.synchronize()
+    say("  oracle (float64, CPU)")
+    torch.set_num_threads(8)
+    D = lambda a: torch.from_numpy(a).double()
+    ref_leaves = [D(a).requires_grad_(True) for a in (x, w_v2f, w_f2f, w_f2v)]
+    x64, wv64, wf64, wo64 = ref_leaves
+    f64, cum64, b64 = torch.from_numpy(f), torch.from_numpy(np.cumsum(counts).astype(np.int32)), D(bary)
+    tex64 = R.texture_fwd(x64, f64, b64, cum64)
+    y64 = R.f2v_fwd(R.v2f_fwd(x64, wv64, f64) + R.f2f_fwd(tex64, wf64, R.sph_harm(b64, L), cum64), wo64,
+                    R.sph_harm(D(normal.astype(np.float32)), L), f64, torch.from_numpy(nfc), torch.arange(nv, dtype=torch.int32))
+    ref_grads = torch.autograd.grad(y64, ref_leaves, D(gy))
+    assert_close(y, y64.detach().numpy(), "shapes block output")
+    for name, g, r in zip(("X", "V2F filter", "F2F filter", "F2V filter"), grads, ref_grads):
+        assert_close(g, r.numpy(), "shapes block gradient of " + name)

@@ -283,3 +283,56 @@ def test_two_level_stack_matches_oracle_composition(cuda):
     for d in lv:
         for k in ("v2f", "f2f", "f2v", "up"):
             _compare_grads(d[k], d[k + "64"])
+
+
+def test_forward_replays_from_a_hip_graph(cuda):
+    """A serving loop records the layer once and replays it: the native calls must be capturable (no allocation,
+    synchronisation or host-side state inside the library; the adjacency is cached by the warm-up run) and every
+    replay must equal the eager result for the inputs then in the static buffers."""
+    from picassoplus_amd.mesh.pi_modules import conv3d, pool3d, texture, unpool3d
+    rng = np.random.default_rng(41)
+    meshes = S.hierarchy_workload(seed=9, cells=32, levels=1)
+    v, f = meshes[0]["vertex"], meshes[0]["face"]
+    nv, nf, C, L = v.shape[0], f.shape[0], 32, 3
+    normal, _ = S.triangle_normals_areas(v, f)
+    counts, bary, _ = S.texture_points(rng, nf, rng.integers(1, 4, nf).astype(np.int32))
+    c = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(cuda)
+    face, cum, bt = c(f), torch.cumsum(c(counts), 0, dtype=torch.int32), c(bary.astype(np.float32))
+    coeff = layers.SphHarmCoeff(L)(c(normal.astype(np.float32)))
+    nfc = c(np.maximum(S.vertex_facet_count(f, np.arange(nv), nv), 1).astype(np.int32))
+    ident = torch.arange(nv, dtype=torch.int32, device=cuda)
+    vr, vm = c(meshes[0]["vt_replace"]), c(meshes[0]["vt_map"])
+    vt_out = torch.zeros(meshes[0]["nv_out"], 3, device=cuda)
+    torch.manual_seed(8)
+    mods = [layers.V2FConv3d(C, C, L, with_bn=False).to(cuda), layers.F2FConv3d(C, C, L, with_bn=False).to(cuda),
+            layers.F2VConv3d(C, C, L, with_bn=False).to(cuda)]
+    cnt = c(counts)
+
+    def run(x):
+        tex, sh = texture.interpolate(x, face, bt, cum, L)
+        y = mods[0](x, face) + mods[1](tex, sh, cnt)
+        z = mods[2](y, face, nfc, ident, coeff)
+        p = pool3d.maxPool(z, vr, vm, vt_out)
+        return z + unpool3d.interpolate(p, vr, vm)
+
+    static_x = torch.randn(nv, C, device=cuda)
+    with torch.no_grad():
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(2):
+                run(static_x)                                   # warm-up: adjacency and checks are cached now
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            static_y = run(static_x)
+        for i in range(3):
+            x = torch.randn(nv, C, device=cuda, generator=torch.Generator(device=cuda).manual_seed(100 + i))
+            static_x.copy_(x)
+            graph.replay()
+            torch.cuda.synchronize()
+            got = static_y.clone()
+            eager = run(x)                                      # the program's own eager work between the replays
+            torch.cuda.synchronize()
+            assert torch.equal(got, eager), "replay %d differs from the eager result" % i

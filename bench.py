@@ -43,6 +43,9 @@ def parse():
                          "block shapes, F2F 3->32 then F2V 32->32 with depth multiplier 2 (pi2_blocks.py:113-130)")
     ap.add_argument("--scale", type=float, default=1.0, help="facet-count scale of the scene workload")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--f2f-half", action="store_true",
+                    help="facet2facet in its half-precision variant (one fp16 piece per operand, fp32 accumulation; "
+                         "results within 1e-3 instead of 1e-5): a separate figure, never the default")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="after the timed region, copy a 1 GiB buffer three times (a kernel of known HBM traffic "
                          "to scale rocprofv3's FETCH_SIZE / WRITE_SIZE counters by)")
@@ -198,18 +201,20 @@ def run_conv_layer(args, torch, kind):
     dom_ms = per_op[dom]
     if dom.startswith("f2f") and Cin >= 16:
         ach = bf[dom][1] / (dom_ms * 1e-3) / 1e12
-        roof = dict(bound="mfma", achieved=ach, peak=MFMA_F16_PEAK_TFLOPS / F2F_PIECE_PRODUCTS, unit="TFLOP/s",
-                    peak_basis="fp16 dense MFMA 2500 TFLOP/s / 3 piece products per fp32-accurate product",
+        pieces = 1 if args.f2f_half else F2F_PIECE_PRODUCTS
+        roof = dict(bound="mfma", achieved=ach, peak=MFMA_F16_PEAK_TFLOPS / pieces, unit="TFLOP/s",
+                    peak_basis="fp16 dense MFMA 2500 TFLOP/s, one product per element (half-precision variant)" if args.f2f_half
+                    else "fp16 dense MFMA 2500 TFLOP/s / 3 piece products per fp32-accurate product",
                     frac_of_fp32_mfma_peak=ach / MFMA_F32_PEAK_TFLOPS)
     else:
         roof = dict(bound="hbm", achieved=bf[dom][0] / (dom_ms * 1e-3) / 1e9, peak=HBM_PEAK_GBS, unit="GB/s")
-    traffic = SCENE_TRAFFIC_BYTES.get(dom) if (kind == "scene" and args.scale == 1.0) else None
+    traffic = SCENE_TRAFFIC_BYTES.get(dom) if (kind == "scene" and args.scale == 1.0 and not args.f2f_half) else None
     roof.update(frac=roof["achieved"] / roof["peak"], traffic=traffic, kernel=dom, kernel_ms=dom_ms)
     ops_report = {k: dict(ms=per_op.get(k), gbps=bf[k][0] / (per_op[k] * 1e-3) / 1e9,
                           tflops=bf[k][1] / (per_op[k] * 1e-3) / 1e12) for k in ops if k in per_op}
     res = dict(value=d["nf"] / (ms * 1e-3) / 1e6, ms_per_step=ms, roofline=roof, ops=ops_report,
                hbm_gbps=total_bytes / (ms * 1e-3) / 1e9, hbm_frac=total_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
-               config=dict(workload=name, facets=d["nf"], vertices=d["nv"], texture_points=d["T"], channels=C,
+               config=dict(workload=name + ("_f2f-half-products" if args.f2f_half else ""), facets=d["nf"], vertices=d["nv"], texture_points=d["T"], channels=C,
                            sh_degree=L, meshes=int(len(d["mf_in"])), algorithmic_bytes=total_bytes))
     if not args.no_cpu_baseline:
         res["cpu_baseline"] = cpu_baseline_conv(d, kind, torch)
@@ -586,6 +591,8 @@ def main():
         print("bench.py needs a GPU (torch.cuda.is_available() is False)", file=sys.stderr)
         sys.exit(2)
     torch.cuda.set_device(0)
+    if args.f2f_half:
+        os.environ["PMESH_F2F_HALF"] = "1"          # read by the library at every call
     if args.workload == "pool":
         res = run_pool(args, torch)
     elif args.workload == "tail":
@@ -605,7 +612,8 @@ def main():
         del src, dst
     line = dict(metric="mesh-conv layer fwd+bwd throughput", value=res.pop("value"), unit=res.pop("unit", "Mfacets/s"),
                 n_gpus=1, steps=args.steps, warmup=args.warmup, ms_per_step=res.pop("ms_per_step"),
-                higher_is_better=True, scaling="weak", vs_baseline=None, dtype="f32", data="synthetic")
+                higher_is_better=True, scaling="weak", vs_baseline=None,
+                dtype="f16 products, f32 accumulate (f2f); f32 elsewhere" if args.f2f_half else "f32", data="synthetic")
     line.update(res)
     print(json.dumps(line))
 

@@ -24,13 +24,13 @@ int f2f16x3_fwd(const float *tex, const float *W, const float *sh, const int *cu
 // (mesh_f2f16h2.hip); same conditions as the bf16 kernels, workspace no larger than theirs
 size_t f2f16h2_fwd_workspace_bytes(int Cin, int Cout);
 int f2f16h2_fwd(const float *tex, const float *W, const float *sh, const int *cum, const int *order, float *out,
-                void *workspace, size_t workspace_bytes, int64_t T, int64_t Nf, int Cin, int Cout, hipStream_t st);
+                void *workspace, size_t workspace_bytes, int64_t T, int64_t Nf, int Cin, int Cout, hipStream_t st, bool half = false);
 
 // texture gradient on the fp16 matrix cores (conditions of the bf16 kernel, workspace no larger)
 size_t f2f16h2_bwd_texture_workspace_bytes(int Cin, int Cout);
 int f2f16h2_bwd_texture(const float *gout, const float *W, const float *sh, const int *cum, const int *order,
                         float *gtex, void *workspace, size_t workspace_bytes, int64_t T, int64_t Nf, int Cin,
-                        int Cout, hipStream_t st);
+                        int Cout, hipStream_t st, bool half = false);
 
 // texture gradient on the bf16 matrix cores (Cout % 8 == 0, 16-byte aligned grad_output; output channels are
 // taken 64 at a time, later blocks accumulate onto grad_texture)
@@ -44,7 +44,8 @@ int f2f16x3_bwd_texture(const float *gout, const float *W, const float *sh, cons
 // caller) is set when the data outgrew the scales: the partials are then void and must be computed again by
 // f2f16x3_bwd_filter_partials, whose `only_if` argument makes that launch a no-op otherwise.
 int f2f16h2_bwd_filter_partials(const float *gout, const float *tex, const float *sh, const int *cum, const int *order,
-                                 float *partial, int *overflow, int splits, int64_t T, int64_t Nf, int Cin, int Cout, hipStream_t st);
+                                 float *partial, int *overflow, int splits, int64_t T, int64_t Nf, int Cin, int Cout, hipStream_t st,
+                                 bool half = false);
 
 // `splits` workgroups each write one partial (Cout x Cin*16) block; every split gets a strided share of the 32-facet tiles
 // only_if (may be null): device flag; the kernel returns at once when it reads 0

@@ -353,6 +353,14 @@ static inline bool force_bf16x3()
     return e && e[0] == '1';
 }
 
+// PMESH_F2F_HALF=1: the half-precision variant of the fp16 kernels (one fp16 piece per operand, one product, fp32
+// accumulation): results within 1e-3 of the largest output instead of 1e-5.
+static inline bool want_half()
+{
+    const char *e = getenv("PMESH_F2F_HALF");
+    return e && e[0] == '1';
+}
+
 static inline bool force_fp32_mfma()
 {
     const char *e = getenv("PMESH_F2F_FP32MFMA");
@@ -379,7 +387,7 @@ extern "C" int pmesh_f2f_fwd(const float *texture, const float *filter, const fl
     if (!force_generic() && !force_fp32_mfma() && !force_bf16x3() && f2f16x3_usable(filter, bary_coeff, F) &&
         T * Cin < (int64_t(1) << 31))
         return f2f16h2_fwd(texture, filter, bary_coeff, cum_texture, facet_order, output, workspace, workspace_bytes,
-                           T, Nf, Cin, Cout, (hipStream_t)stream);
+                           T, Nf, Cin, Cout, (hipStream_t)stream, want_half());
     if (!force_generic() && !force_fp32_mfma() && f2f16x3_usable(filter, bary_coeff, F) &&
         T * Cin < (int64_t(1) << 31))
         return f2f16x3_fwd(texture, filter, bary_coeff, cum_texture, facet_order, output, workspace, workspace_bytes,
@@ -419,7 +427,7 @@ extern "C" int pmesh_f2f_bwd_texture(const float *grad_output, const float *filt
     if (!force_generic() && !force_fp32_mfma() && !force_bf16x3() && f2f16x3_usable(filter, bary_coeff, F) &&
         f2f16x3_bwd_texture_usable(grad_output, Cout))
         return f2f16h2_bwd_texture(grad_output, filter, bary_coeff, cum_texture, facet_order, grad_texture, workspace,
-                                   workspace_bytes, T, Nf, Cin, Cout, (hipStream_t)stream);
+                                   workspace_bytes, T, Nf, Cin, Cout, (hipStream_t)stream, want_half());
     if (!force_generic() && !force_fp32_mfma() && f2f16x3_usable(filter, bary_coeff, F) &&
         f2f16x3_bwd_texture_usable(grad_output, Cout))
         return f2f16x3_bwd_texture(grad_output, filter, bary_coeff, cum_texture, facet_order, grad_texture, workspace,
@@ -476,7 +484,7 @@ extern "C" int pmesh_f2f_bwd_filter(const float *grad_output, const float *textu
             f2f_fill_zero_k<<<dim3(1), dim3(kBlock), 0, st>>>(reinterpret_cast<float *>(overflow), 1);
             PM_LAUNCHED("f2f_bwd_filter(flag)");
             if (int rc = f2f16h2_bwd_filter_partials(grad_output, texture, bary_coeff, cum_texture, facet_order,
-                                                     (float *)workspace, overflow, S, T, Nf, Cin, Cout, st))
+                                                     (float *)workspace, overflow, S, T, Nf, Cin, Cout, st, want_half()))
                 return rc;
             if (int rc = f2f16x3_bwd_filter_partials(grad_output, texture, bary_coeff, cum_texture, facet_order,
                                                      (float *)workspace, S, T, Nf, Cin, Cout, st, overflow))

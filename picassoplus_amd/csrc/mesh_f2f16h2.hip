@@ -77,6 +77,18 @@ __device__ __forceinline__ void split8h(const float (&x)[8], u32x4 &p1, u32x4 &p
     }
 }
 
+// Eight fp32 values -> one packed fp16x8 piece, rounded to nearest (the first piece of split8h): the operand of the
+// half-precision variant, whose products keep fp16's 11 significant bits and accumulate in fp32.
+__device__ __forceinline__ void cvt8h(const float (&x)[8], u32x4 &p1)
+{
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        unsigned hi;
+        asm("v_cvt_pk_f16_f32 %0, %1, %2" : "=v"(hi) : "v"(x[2 * j]), "v"(x[2 * j + 1]));
+        p1[j] = hi;
+    }
+}
+
 __device__ __forceinline__ f32x16 mfma_f16(const u32x4 &a, const u32x4 &b, const f32x16 &c)
 {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
@@ -190,7 +202,7 @@ __device__ __forceinline__ void hw_half_publish(u32x4 *Wbuf, int half, const u32
 // One pass over all input channels for up to KW texture points per facet.  shs = alpha_f / K_f, the factor on
 // the SH values of my facet; slim / tlim = largest |SH value| of my facet / |texture value| of the rows I fetch
 // that the scale allows for.
-template <int KW, bool TVEC>
+template <int KW, bool TVEC, bool HALF>
 __device__ __forceinline__ void h2_sweep(const float *__restrict__ tex, const u32x4 *__restrict__ Wp,
                                          const float *__restrict__ sh, u32x4 *Ws, float *slab, f32x16 (&acc)[2],
                                          int kbase, int Ks, float shs, float slim, float tlim, bool &viol,
@@ -281,7 +293,8 @@ __device__ __forceinline__ void h2_sweep(const float *__restrict__ tex, const u3
         read_tv(tvn, 1);
         read_b(b, 0, 0);
         gen(a, tv0);
-        split8h(a, pa[0], pa[1]);
+        if constexpr (HALF) cvt8h(a, pa[0]);
+        else split8h(a, pa[0], pa[1]);
     }
     // filter chunks alternate between two LDS buffers: chunk j+1 is fetched at the start of chunk j and published
     // at its end; the first channel of a chunk reads its pieces right after the barrier, under the generation
@@ -303,15 +316,21 @@ __device__ __forceinline__ void h2_sweep(const float *__restrict__ tex, const u3
             float an[8];
             gen(an, tvn);
             u32x4 pn[2];
-            split8h(an, pn[0], pn[1]);
-
-            // three piece products per accumulator tile, smallest first
+            if constexpr (HALF) {
+                cvt8h(an, pn[0]);
+                pn[1] = pn[0];
 #pragma unroll
-            for (int t = 0; t < 2; ++t) acc[t] = mfma_f16(pa[1], b[t][0], acc[t]);
+                for (int t = 0; t < 2; ++t) acc[t] = mfma_f16(pa[0], b[t][0], acc[t]);
+            } else {
+                split8h(an, pn[0], pn[1]);
+                // three piece products per accumulator tile, smallest first
 #pragma unroll
-            for (int t = 0; t < 2; ++t) acc[t] = mfma_f16(pa[0], b[t][1], acc[t]);
+                for (int t = 0; t < 2; ++t) acc[t] = mfma_f16(pa[1], b[t][0], acc[t]);
 #pragma unroll
-            for (int t = 0; t < 2; ++t) acc[t] = mfma_f16(pa[0], b[t][0], acc[t]);
+                for (int t = 0; t < 2; ++t) acc[t] = mfma_f16(pa[0], b[t][1], acc[t]);
+#pragma unroll
+                for (int t = 0; t < 2; ++t) acc[t] = mfma_f16(pa[0], b[t][0], acc[t]);
+            }
 
             pa[0] = pn[0]; pa[1] = pn[1];
 #pragma unroll
@@ -334,7 +353,7 @@ __device__ __forceinline__ void h2_sweep(const float *__restrict__ tex, const u3
     }
 }
 
-template <bool TVEC>
+template <bool TVEC, bool HALF>
 __global__ __launch_bounds__(kHThreads, 2) void f2f16h2_fwd_k(const float *__restrict__ tex, const float *__restrict__ hdr,
                                                               const u32x4 *__restrict__ Wp, const float *__restrict__ sh,
                                                               const int *__restrict__ cum, const int *__restrict__ order,
@@ -444,7 +463,7 @@ __global__ __launch_bounds__(kHThreads, 2) void f2f16h2_fwd_k(const float *__res
             const int Ks = rem < 0 ? 0 : (rem > kHFKB ? kHFKB : rem);
             // every variant runs the same barriers, so wavefronts of a workgroup may pick different ones
             const int kw = hwave_max(Ks);
-#define PM_H2(N) h2_sweep<N, TVEC>(tex, Wp, sh, Ws, s_slab + w * 2 * kHSlab, acc, kbase, Ks, shs, slim, tlim, viol, s_k0, s_K, sw, Cin, NT, nt0, nblk, w, lane, h)
+#define PM_H2(N) h2_sweep<N, TVEC, HALF>(tex, Wp, sh, Ws, s_slab + w * 2 * kHSlab, acc, kbase, Ks, shs, slim, tlim, viol, s_k0, s_K, sw, Cin, NT, nt0, nblk, w, lane, h)
             if (kw <= 1) PM_H2(1);
             else if (kw == 2) PM_H2(2);
             else if (kw == 3) PM_H2(3);
@@ -479,7 +498,7 @@ size_t f2f16h2_fwd_workspace_bytes(int Cin, int Cout)
 }
 
 int f2f16h2_fwd(const float *tex, const float *W, const float *sh, const int *cum, const int *order, float *out,
-                void *workspace, size_t workspace_bytes, int64_t T, int64_t Nf, int Cin, int Cout, hipStream_t st)
+                void *workspace, size_t workspace_bytes, int64_t T, int64_t Nf, int Cin, int Cout, hipStream_t st, bool half)
 {
     const int NT = 2 * ((Cout + 63) / 64);
     PM_REQUIRE(T * Cin < (int64_t(1) << 31), "f2f_fwd: texture array too large for 32-bit offsets");
@@ -495,10 +514,13 @@ int f2f16h2_fwd(const float *tex, const float *W, const float *sh, const int *cu
     PM_LAUNCHED("f2f_fwd(pack)");
     const int64_t gx = ceil_div(Nf, kHFacets), gy = NT / 2;
     PM_REQUIRE(grid_ok(gx) && gy <= 65535, "f2f_fwd: grid too large");
-    if (!(Cin & 3) && !(reinterpret_cast<uintptr_t>(tex) & 15u))
-        f2f16h2_fwd_k<true><<<dim3((unsigned)gx, (unsigned)gy), dim3(kHThreads), 0, st>>>(tex, hdr, Wp, sh, cum, order, out, Nf, (int)T, Cin, Cout, NT);
-    else
-        f2f16h2_fwd_k<false><<<dim3((unsigned)gx, (unsigned)gy), dim3(kHThreads), 0, st>>>(tex, hdr, Wp, sh, cum, order, out, Nf, (int)T, Cin, Cout, NT);
+#define PM_FWD(V, H) f2f16h2_fwd_k<V, H><<<dim3((unsigned)gx, (unsigned)gy), dim3(kHThreads), 0, st>>>(tex, hdr, Wp, sh, cum, order, out, Nf, (int)T, Cin, Cout, NT)
+    const bool tvec = !(Cin & 3) && !(reinterpret_cast<uintptr_t>(tex) & 15u);
+    if (tvec && half) PM_FWD(true, true);
+    else if (tvec) PM_FWD(true, false);
+    else if (half) PM_FWD(false, true);
+    else PM_FWD(false, false);
+#undef PM_FWD
     PM_LAUNCHED("f2f_fwd");
     return 0;
 }
@@ -538,7 +560,7 @@ __global__ __launch_bounds__(kBlock) void f2f16h2_pack_filter_t_k(const float *_
     dst[0] = p1; dst[64] = p2;
 }
 
-template <int KW, int NKS, bool GVEC>
+template <int KW, int NKS, bool GVEC, bool HALF>
 __device__ __forceinline__ void h2_tex_sweep(const u32x4 *__restrict__ WpT, const float *__restrict__ sh,
                                              float *__restrict__ gtex, u32x4 *Ws, float *stage, const int *w_k0,
                                              const int *w_K, const u32x4 (&bp)[NKS][2], int kbase, int Ks, float shs,
@@ -667,9 +689,11 @@ __device__ __forceinline__ void h2_tex_sweep(const u32x4 *__restrict__ WpT, cons
                     u32x4 a[2];
 #pragma unroll
                     for (int p = 0; p < 2; ++p) a[p] = Wc[((u * NKS + ks) * 2 + p) * 64];
-                    // three piece products, smallest first
-                    acc0 = mfma_f16(a[1], bp[ks][0], acc0);
-                    acc0 = mfma_f16(a[0], bp[ks][1], acc0);
+                    // three piece products, smallest first (half-precision variant: the product of the first pieces)
+                    if constexpr (!HALF) {
+                        acc0 = mfma_f16(a[1], bp[ks][0], acc0);
+                        acc0 = mfma_f16(a[0], bp[ks][1], acc0);
+                    }
                     acc0 = mfma_f16(a[0], bp[ks][0], acc0);
                 }
                 // meanwhile: the previous tile (the last one of the previous group when cc = u = 0)
@@ -688,7 +712,7 @@ __device__ __forceinline__ void h2_tex_sweep(const u32x4 *__restrict__ WpT, cons
 // NKS = k-steps of 16 output channels (compile time, so that a tile's MFMAs and the previous tile's
 // contraction share one basic block and get interleaved): 2 for Cout <= 32, else 4; the packed filter
 // is zero padded to that many.
-template <int NKS, bool GVEC>
+template <int NKS, bool GVEC, bool HALF>
 __global__ __launch_bounds__(512, 2) void f2f16h2_bwd_tex_k(const float *__restrict__ gout,
                                                             const float *__restrict__ hdr,
                                                             const u32x4 *__restrict__ WpT,
@@ -759,7 +783,7 @@ __global__ __launch_bounds__(512, 2) void f2f16h2_bwd_tex_k(const float *__restr
         const int kw = hwave_max(Ks);
         const int kbase = k0 + sw * kHTKB;
         // every variant runs the same barriers, so wavefronts of a workgroup may pick different ones
-#define PM_H2T(N) h2_tex_sweep<N, NKS, GVEC>(WpT, sh, gtex, Ws, s_stage[w], s_k0[w], s_K[w], bp, kbase, Ks, shs, sw, Cin, NG, co0 > 0, lane, h)
+#define PM_H2T(N) h2_tex_sweep<N, NKS, GVEC, HALF>(WpT, sh, gtex, Ws, s_stage[w], s_k0[w], s_K[w], bp, kbase, Ks, shs, sw, Cin, NG, co0 > 0, lane, h)
         if (kw <= 1) PM_H2T(1);
         else if (kw == 2) PM_H2T(2);
         else if (kw == 3) PM_H2T(3);
@@ -780,7 +804,7 @@ size_t f2f16h2_bwd_texture_workspace_bytes(int Cin, int Cout)
 
 int f2f16h2_bwd_texture(const float *gout, const float *W, const float *sh, const int *cum, const int *order,
                         float *gtex, void *workspace, size_t workspace_bytes, int64_t T, int64_t Nf, int Cin,
-                        int Cout, hipStream_t st)
+                        int Cout, hipStream_t st, bool half)
 {
     const int NG = (Cin + 7) / 8;
     PM_REQUIRE(workspace && workspace_bytes >= f2f16h2_bwd_texture_workspace_bytes(Cin, Cout),
@@ -800,7 +824,11 @@ int f2f16h2_bwd_texture(const float *gout, const float *W, const float *sh, cons
         const int n = NG * 4 * NKS * 64;
         f2f16h2_pack_filter_t_k<<<dim3((unsigned)ceil_div(n, kBlock)), dim3(kBlock), 0, st>>>(W, hdr, WpT, Cin, Cout, NG * 4, NKS, co0);
         PM_LAUNCHED("f2f_bwd_texture(pack)");
-#define PM_TEX(N, G) f2f16h2_bwd_tex_k<N, G><<<dim3((unsigned)gx), dim3(512), 0, st>>>(gout, hdr, WpT, sh, cum, order, gtex, Nf, (int)T, Cin, Cout, NG, co0)
+#define PM_TEX(N, G)                                                                                                           \
+    do {                                                                                                                       \
+        if (half) f2f16h2_bwd_tex_k<N, G, true><<<dim3((unsigned)gx), dim3(512), 0, st>>>(gout, hdr, WpT, sh, cum, order, gtex, Nf, (int)T, Cin, Cout, NG, co0); \
+        else f2f16h2_bwd_tex_k<N, G, false><<<dim3((unsigned)gx), dim3(512), 0, st>>>(gout, hdr, WpT, sh, cum, order, gtex, Nf, (int)T, Cin, Cout, NG, co0);   \
+    } while (0)
         if (NKS == 2 && gvec) PM_TEX(2, true);
         else if (NKS == 2) PM_TEX(2, false);
         else if (gvec) PM_TEX(4, true);
@@ -835,7 +863,7 @@ int f2f16h2_bwd_texture(const float *gout, const float *W, const float *sh, cons
 //   workgroup  4 wavefronts (one per SIMD), 64 input x 64 output channels, a strided subset of the tiles
 //   wavefront  16 input channels = 8 channel pairs x 2 output tiles of gW^T[(ci,d)][co]; narrower filters give
 //              every wavefront 1, 2 or 4 pairs instead (NCP)
-template <int KW, int NCP>
+template <int KW, int NCP, bool HALF>
 __device__ __forceinline__ void h2_filt_pass(const float (&shr)[KW][8], const float4 *slab, const u32x4 *go,
                                              f32x16 (&acc)[NCP][2], const u32x4 &ea, const u32x4 &eb, int lane)
 {
@@ -853,8 +881,14 @@ __device__ __forceinline__ void h2_filt_pass(const float (&shr)[KW][8], const fl
                 ab[q] = kk ? fmaf(tb, shr[kk][q], ab[q]) : tb * shr[kk][q];
             }
         }
-        split8h(aa, pa[0], pa[1]);
-        split8h(ab, pb[0], pb[1]);
+        if constexpr (HALF) {
+            cvt8h(aa, pa[0]);
+            cvt8h(ab, pb[0]);
+            pa[1] = pa[0]; pb[1] = pb[0];
+        } else {
+            split8h(aa, pa[0], pa[1]);
+            split8h(ab, pb[0], pb[1]);
+        }
     };
     // The four transposition MFMAs are one asm block with VGPR destinations: in a kernel whose accumulators
     // live in AGPRs the compiler gives every MFMA an AGPR destination, and the results would have to be
@@ -862,6 +896,28 @@ __device__ __forceinline__ void h2_filt_pass(const float (&shr)[KW][8], const fl
     // keep the second product of a chain behind the first one's write of its accumulator (only one other MFMA
     // lies between them), the trailing ones cover the wait states a vector ALU read of an MFMA result needs.
     auto transpose = [&](u32x4 (&o)[2][2], const u32x4 (&pa)[2], const u32x4 (&pb)[2]) {
+        if constexpr (HALF) {
+            // one piece per operand: the chain of two products with the wait states of the block below
+            f32x16 d;
+            asm volatile("s_nop 3\n"
+                         "v_mfma_f32_32x32x16_f16 %0, %1, %3, 0\n"
+                         "s_nop 7\n"
+                         "s_nop 7\n"
+                         "s_nop 7\n"
+                         "v_mfma_f32_32x32x16_f16 %0, %2, %4, %0\n"
+                         "s_nop 15\n"
+                         "s_nop 7\n"
+                         : "=&v"(d)
+                         : "v"(pa[0]), "v"(pb[0]), "v"(ea), "v"(eb));
+#pragma unroll
+            for (int st = 0; st < 2; ++st)
+#pragma unroll
+                for (int jj = 0; jj < 4; ++jj) {
+                    o[0][st][jj] = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_pkrtz(d[8 * st + 2 * jj], d[8 * st + 2 * jj + 1]));
+                    o[1][st][jj] = o[0][st][jj];
+                }
+            return;
+        }
         f32x16 d0, d1;
         asm volatile("s_nop 3\n"
                      "v_mfma_f32_32x32x16_f16 %0, %2, %6, 0\n"
@@ -908,10 +964,12 @@ __device__ __forceinline__ void h2_filt_pass(const float (&shr)[KW][8], const fl
 #pragma unroll
         for (int st = 0; st < 2; ++st) {
             // three piece products, smallest first; the two output tiles alternate
+            if constexpr (!HALF) {
 #pragma unroll
-            for (int t = 0; t < 2; ++t) acc[cp][t] = mfma_f16(o[1][st], g[st][t][0], acc[cp][t]);
+                for (int t = 0; t < 2; ++t) acc[cp][t] = mfma_f16(o[1][st], g[st][t][0], acc[cp][t]);
 #pragma unroll
-            for (int t = 0; t < 2; ++t) acc[cp][t] = mfma_f16(o[0][st], g[st][t][1], acc[cp][t]);
+                for (int t = 0; t < 2; ++t) acc[cp][t] = mfma_f16(o[0][st], g[st][t][1], acc[cp][t]);
+            }
 #pragma unroll
             for (int t = 0; t < 2; ++t) acc[cp][t] = mfma_f16(o[0][st], g[st][t][0], acc[cp][t]);
         }
@@ -1029,7 +1087,7 @@ struct HScales {
 
 // One tile of 32 facets whose inputs are in LDS buffer it % 2 (descriptors in it % 3): start the
 // fetches for the next tile, run the passes, publish the next tile's inputs.
-template <int KW, bool TVEC, int NCP>
+template <int KW, bool TVEC, int NCP, bool HALF>
 __device__ __forceinline__ void h2_filt_tile(const float *__restrict__ gout, const float *__restrict__ tex,
                                              const float *__restrict__ sh, const int *__restrict__ cum,
                                              const int *__restrict__ order, u32x4 (*go_s)[2 * 2 * 2 * 64], float4 *slab,
@@ -1122,7 +1180,7 @@ __device__ __forceinline__ void h2_filt_tile(const float *__restrict__ gout, con
             for (int kk = 0; kk < KW; ++kk)
 #pragma unroll
                 for (int q = 0; q < 8; ++q) shr[kk][q] *= al;
-            h2_filt_pass<KW, NCP>(shr, slab, go_s[buf], acc, ea, eb, lane);
+            h2_filt_pass<KW, NCP, HALF>(shr, slab, go_s[buf], acc, ea, eb, lane);
         }
     }
 
@@ -1150,7 +1208,7 @@ __device__ __forceinline__ void h2_filt_tile(const float *__restrict__ gout, con
 
 // NCP = channel pairs of a wavefront (8 for 64 or more input channels; fewer for narrow filters, so that
 // the four wavefronts share what channels there are)
-template <bool TVEC, int NCP>
+template <bool TVEC, int NCP, bool HALF>
 __global__ __launch_bounds__(256, 1) void f2f16h2_bwd_filt_k(const float *__restrict__ gout,
                                                               const float *__restrict__ tex,
                                                               const float *__restrict__ sh,
@@ -1225,7 +1283,7 @@ __global__ __launch_bounds__(256, 1) void f2f16h2_bwd_filt_k(const float *__rest
     int it = 0;
 #define PM_PHASE(N)                                                                                                  \
     for (; tile < ntiles && (N == kHKB || htile_kmax(s_K[it % 3], lane) <= N); ++it, tile += stride)                 \
-        h2_filt_tile<N, TVEC, NCP>(gout, tex, sh, cum, order, go_s, slab_s + w * (kHKB * 4 * 32), sh_s, s_f, s_k0, s_K, \
+        h2_filt_tile<N, TVEC, NCP, HALF>(gout, tex, sh, cum, order, go_s, slab_s + w * (kHKB * 4 * 32), sh_s, s_f, s_k0, s_K, \
                                    s_gamma, s_gm, acc, sc, overflow, ea, eb, it, tile, stride, ntiles, Nf, T, Cin, Cout, c0, n0, lane, w)
     PM_PHASE(1);
     PM_PHASE(2);
@@ -1261,7 +1319,7 @@ __global__ __launch_bounds__(256, 1) void f2f16h2_bwd_filt_k(const float *__rest
 }
 
 int f2f16h2_bwd_filter_partials(const float *gout, const float *tex, const float *sh, const int *cum, const int *order,
-                                 float *partial, int *overflow, int splits, int64_t T, int64_t Nf, int Cin, int Cout, hipStream_t st)
+                                 float *partial, int *overflow, int splits, int64_t T, int64_t Nf, int Cin, int Cout, hipStream_t st, bool half)
 {
     // channel pairs per wavefront: the four wavefronts of a workgroup share up to 32 pairs
     const int pairs = (Cin + 1) / 2;
@@ -1271,7 +1329,11 @@ int f2f16h2_bwd_filter_partials(const float *gout, const float *tex, const float
     const int64_t ntiles = ceil_div(Nf, 32);
     const bool tvec = !(Cin & 3) && !(reinterpret_cast<uintptr_t>(tex) & 15u);
     const dim3 grid((unsigned)splits, (unsigned)gy, (unsigned)gz);
-#define PM_FILT(V, N) f2f16h2_bwd_filt_k<V, N><<<grid, dim3(256), 0, st>>>(gout, tex, sh, cum, order, partial, overflow, Nf, (int)T, Cin, Cout, ntiles)
+#define PM_FILT(V, N)                                                                                                              \
+    do {                                                                                                                           \
+        if (half) f2f16h2_bwd_filt_k<V, N, true><<<grid, dim3(256), 0, st>>>(gout, tex, sh, cum, order, partial, overflow, Nf, (int)T, Cin, Cout, ntiles); \
+        else f2f16h2_bwd_filt_k<V, N, false><<<grid, dim3(256), 0, st>>>(gout, tex, sh, cum, order, partial, overflow, Nf, (int)T, Cin, Cout, ntiles);   \
+    } while (0)
     if (tvec) {
         if (ncp == 8) PM_FILT(true, 8); else if (ncp == 4) PM_FILT(true, 4); else if (ncp == 2) PM_FILT(true, 2); else PM_FILT(true, 1);
     } else {

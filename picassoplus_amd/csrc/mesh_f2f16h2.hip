@@ -199,6 +199,20 @@ __device__ __forceinline__ void hw_half_publish(u32x4 *Wbuf, int half, const u32
     for (int i = 0; i < kHWn / 2; ++i) Wbuf[512 * half + threadIdx.x + kHThreads * i] = wn[i];
 }
 
+// The same chunk straight from global memory into an LDS buffer (no registers in between, so the request can leave
+// a whole chunk ahead): lane L of wavefront w delivers element 256 i + 64 w + L of the chunk, the wavefront's 64
+// elements land side by side from the wavefront-uniform base in M0.  The data is there after vmcnt has drained.
+__device__ __forceinline__ void hw_chunk_to_lds(const u32x4 *__restrict__ Wp, int c0, int NT, int nt0, u32x4 *Wbuf, int wave)
+{
+#pragma unroll
+    for (int i = 0; i < kHWn; ++i) {
+        const int e = kHThreads * i + threadIdx.x, c = e >> 8, o = e & 255;
+        __builtin_amdgcn_global_load_lds(
+            (const __attribute__((address_space(1))) void *)(Wp + ((size_t)(c0 + c) * NT + nt0) * 128 + o),
+            (__attribute__((address_space(3))) void *)(Wbuf + kHThreads * i + 64 * wave), 16, 0, 0);
+    }
+}
+
 // One pass over all input channels for up to KW texture points per facet.  shs = alpha_f / K_f, the factor on
 // the SH values of my facet; slim / tlim = largest |SH value| of my facet / |texture value| of the rows I fetch
 // that the scale allows for.
@@ -253,6 +267,7 @@ __device__ __forceinline__ void h2_sweep(const float *__restrict__ tex, const u3
         viol |= m > tlim;
     };
     u32x4 wn[kHWn / 2];
+    const int wave_u = __builtin_amdgcn_readfirstlane(w);
     fetch_group(0);
     publish_group(slab);
     hw_half_fetch(Wp, 0, 0, NT, nt0, wn);
@@ -303,7 +318,7 @@ __device__ __forceinline__ void h2_sweep(const float *__restrict__ tex, const u3
         const int g = j >> 1, wb = j & 1;
         const bool wmore = j + 1 < nblk;
         const bool stage = !(j & 1) && 8 * (g + 1) < Cin;       // even chunk: bring in the next 8-channel group
-        if (wmore) hw_half_fetch(Wp, 4 * (j + 1), 0, NT, nt0, wn);
+        if (wmore) hw_chunk_to_lds(Wp, 4 * (j + 1), NT, nt0, Ws + (wb ^ 1) * kHChunk, wave_u);   // nobody reads that buffer during this chunk
         if (stage) fetch_group(g + 1);
 #pragma unroll
         for (int ci_l = 0; ci_l < 4; ++ci_l) {
@@ -341,12 +356,8 @@ __device__ __forceinline__ void h2_sweep(const float *__restrict__ tex, const u3
 #pragma unroll
                     for (int p = 0; p < 2; ++p) b[t][p] = bn[t][p];
             }
-            if (ci_l == 1 && wmore) {                       // nobody reads the other buffer during this chunk
-                hw_half_publish(Ws + (wb ^ 1) * kHChunk, 0, wn);
-                hw_half_fetch(Wp, 4 * (j + 1), 1, NT, nt0, wn);
-            }
         }
-        if (wmore) hw_half_publish(Ws + (wb ^ 1) * kHChunk, 1, wn);
+        if (wmore) __builtin_amdgcn_s_waitcnt(0x0F70);      // vmcnt(0): the next chunk has landed in its buffer
         if (stage) publish_group(slab + ((g + 1) & 1) * kHSlab);
         __syncthreads();
         if (wmore) read_b(b, wb ^ 1, 0);

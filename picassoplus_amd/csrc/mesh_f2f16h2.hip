@@ -16,7 +16,8 @@
 // Work decomposition of the forward: workgroup = 128 facets from the list sorted by point count x 64 output
 // channels, 4 wavefronts x 32 facets; two workgroups share a CU (two wavefronts per SIMD) and run out of
 // phase, so the prologue, barriers and stores of one overlap the channel loop of the other.  Filter chunks
-// of four channels alternate between two LDS buffers, texture rows go through a wavefront-private LDS slab.
+// of four channels alternate between two LDS buffers and arrive there straight from global memory, requested one
+// chunk ahead; texture rows go through a wavefront-private LDS slab.
 #include "f2f_internal.h"
 
 namespace pmesh {
@@ -311,7 +312,7 @@ __device__ __forceinline__ void h2_sweep(const float *__restrict__ tex, const u3
         if constexpr (HALF) cvt8h(a, pa[0]);
         else split8h(a, pa[0], pa[1]);
     }
-    // filter chunks alternate between two LDS buffers: chunk j+1 is fetched at the start of chunk j and published
+    // filter chunks alternate between two LDS buffers: chunk j+1 is requested at the start of chunk j and has landed
     // at its end; the first channel of a chunk reads its pieces right after the barrier, under the generation
     // and split of the channel after it
     for (int j = 0; j < nblk; ++j) {

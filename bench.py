@@ -95,8 +95,8 @@ def conv_bytes_flops(d, ops):
 # HBM bytes per launch of the op's main kernel on the default scene workload (scale 1.0), measured with
 # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE and scaled by what the same counters read for a 1 GiB copy
 # (--copy-calibration); reported as roofline.traffic when that workload runs.
-SCENE_TRAFFIC_BYTES = {"f2f_fwd": 5.973e9, "f2f_bwd_texture": 3.744e9, "f2f_bwd_filter": 3.348e9,
-                       "f2v_fwd": 1.285e9, "f2v_bwd": 2.185e9}
+SCENE_TRAFFIC_BYTES = {"f2f_fwd": 5.323e9, "f2f_bwd_texture": 3.748e9, "f2f_bwd_filter": 3.348e9,
+                       "f2v_fwd": 1.284e9, "f2v_bwd": 2.186e9}
 
 
 class EventTimer:

@@ -99,6 +99,13 @@ SCENE_TRAFFIC_BYTES = {"f2f_fwd": 5.323e9, "f2f_bwd_texture": 3.748e9, "f2f_bwd_
                        "f2v_fwd": 1.284e9, "f2v_bwd": 2.186e9}
 
 
+# the same for the other workloads at scale 1.0 (profiles/*_hbm_traffic_pmc.txt); an op of two kernels is their sum
+POOL_TRAFFIC_BYTES = {"pool_max_fwd": 0.818e9, "pool_max_bwd": 0.841e9, "pool_avg_fwd": 0.693e9, "pool_avg_bwd": 0.698e9,
+                      "unpool_fwd": 0.695e9, "unpool_bwd": 0.684e9}
+TAIL_TRAFFIC_BYTES = {"dense_fwd": 1.249e9, "dense_bwd": 2.514e9}
+TEXTURE_TRAFFIC_BYTES = {"texture_fwd": 3.396e9, "texture_bwd": 3.293e9}
+
+
 class EventTimer:
     """Brackets every native call with HIP events on the launch stream."""
 
@@ -308,9 +315,25 @@ def run_pool(args, torch):
     dom = max(nb, key=lambda k: per_op[k])
     ach = nb[dom] / (per_op[dom] * 1e-3) / 1e9
     total = sum(nb.values())
-    return dict(value=nv / (ms * 1e-3) / 1e6, unit="Mvertices/s", ms_per_step=ms,
+    extra = {}
+    if not args.no_cpu_baseline:
+        # the oracle's restatement (float32 PyTorch-CPU scatter / gather ops) of the same six ops, once
+        from oracle import torch_ref as R
+        torch.set_num_threads(os.cpu_count() or 1)
+        xc, rc, mc, gc, gf = x.detach().cpu(), vr.cpu(), vm.cpu(), g_c.cpu(), g_f.cpu()
+        t0 = time.perf_counter()
+        _, idx = R.maxpool_fwd(xc, rc, mc, nvo)
+        R.maxpool_bwd(gc, nv, idx)
+        ya = R.avgpool_fwd(xc, rc, mc, nvo)
+        R.avgpool_bwd(gc, rc, mc)
+        R.unpool_fwd(ya, rc, mc)
+        R.unpool_bwd(gf, nvo, rc, mc)
+        spent = time.perf_counter() - t0
+        extra["cpu_baseline"] = dict(value=nv / spent / 1e6, unit="Mvertices/s", cores=torch.get_num_threads(), kind="port",
+                                     sample="the whole grid (%d vertices, %d channels), one pass of the six ops, %.1f s" % (nv, C, spent))
+    return dict(value=nv / (ms * 1e-3) / 1e6, unit="Mvertices/s", ms_per_step=ms, **extra,
                 roofline=dict(bound="hbm", achieved=ach, peak=HBM_PEAK_GBS, unit="GB/s", frac=ach / HBM_PEAK_GBS,
-                              traffic=None, kernel=dom, kernel_ms=per_op[dom]),
+                              traffic=POOL_TRAFFIC_BYTES.get(dom), kernel=dom, kernel_ms=per_op[dom]),
                 ops={k: dict(ms=per_op[k], gbps=nb[k] / (per_op[k] * 1e-3) / 1e9) for k in nb},
                 hbm_gbps=total / (ms * 1e-3) / 1e9, hbm_frac=total / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
                 config=dict(workload="plane1024_pool_max+avg+unpool_C128_fp32_fwd+bwd", vertices=nv, coarse=nvo, channels=C))
@@ -370,7 +393,8 @@ def run_tail(args, torch):
                                      sample="first %d of %d rows, one fwd+bwd pass, %.1f s" % (rows, N, spent))
     return dict(value=N / (ms * 1e-3) / 1e6, unit="Mrows/s", ms_per_step=ms, **extra,
                 roofline=dict(bound="hbm", achieved=ach, peak=HBM_PEAK_GBS, unit="GB/s", frac=ach / HBM_PEAK_GBS,
-                              traffic=None, kernel=dom, kernel_ms=per_op[dom]),
+                              traffic=TAIL_TRAFFIC_BYTES.get(dom) if args.scale == 1.0 else None, kernel=dom,
+                              kernel_ms=per_op[dom]),
                 ops={k: dict(ms=per_op[k], gbps=nb[k] / (per_op[k] * 1e-3) / 1e9,
                              tflops=fl[k] / (per_op[k] * 1e-3) / 1e12) for k in nb},
                 hbm_gbps=total / (ms * 1e-3) / 1e9, hbm_frac=total / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
@@ -430,7 +454,8 @@ def run_texture(args, torch):
                                             % (len(d["mf_in"]), nf, nt, spent))
     return dict(value=d["nf"] / (ms * 1e-3) / 1e6, ms_per_step=ms, **extra,
                 roofline=dict(bound="hbm", achieved=ach, peak=HBM_PEAK_GBS, unit="GB/s", frac=ach / HBM_PEAK_GBS,
-                              traffic=None, kernel=dom, kernel_ms=per_op[dom]),
+                              traffic=TEXTURE_TRAFFIC_BYTES.get(dom) if args.scale == 1.0 else None, kernel=dom,
+                              kernel_ms=per_op[dom]),
                 ops={k: dict(ms=per_op[k], gbps=bf[k][0] / (per_op[k] * 1e-3) / 1e9) for k in ops},
                 hbm_gbps=total / (ms * 1e-3) / 1e9, hbm_frac=total / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
                 config=dict(workload="scene8x300k_texture_interpolation+SH_C64_L3_fp32_fwd+bwd", facets=d["nf"],

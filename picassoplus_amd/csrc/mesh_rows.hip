@@ -898,6 +898,7 @@ extern "C" int pmesh_v2f_fwd(const float *input, const float *filter, const int3
     PM_REQUIRE(Nv >= 0 && Nf >= 0, "v2f_fwd: negative size");
     if (Nf == 0) return 0;
     PM_REQUIRE(input && filter && face && output, "v2f_fwd: null pointer");
+    PM_REQUIRE(Nv > 0, "v2f_fwd: facets given but no input vertices");
     PM_REQUIRE(Nv <= INT32_MAX && Nf <= INT32_MAX / 3, "v2f_fwd: sizes exceed int32 indexing");
     hipStream_t st = (hipStream_t)stream;
     const int V = pick_v2f(C, r, {input, filter, output});

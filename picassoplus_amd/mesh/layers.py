@@ -105,7 +105,11 @@ class _ConvTail(nn.Module):
     def _dense_tail(self, inputs, weights):
         """``_tail(inputs @ weights)`` with the product, the bias and a ReLU (or no activation) in one
         native pass; without gradients an inference-mode batch norm rides along as scale/shift.  Any
-        other activation, and batch norm in training mode, run as PyTorch ops on the result."""
+        other activation, and batch norm in training mode, run as PyTorch ops on the result.  Layers with more
+        than ``dense.MAX_CHANNELS`` (896) input or output channels run the reference's PyTorch ops instead."""
+        if max(weights.shape) > dense.MAX_CHANNELS:
+            # wider than the native pass takes (its weight slab must fit LDS): the reference's own ops
+            return self._tail(torch.matmul(inputs, weights))
         relu = isinstance(self.activation_fn, nn.ReLU)
         fused_act = relu or self.activation_fn is None
         biases = self.biases.reshape(-1)
@@ -197,7 +201,10 @@ class V2FConv3d(_SeparableConv):
     def _corners(self, device):
         key = (self.L, device)
         if key not in V2FConv3d._corner_basis:
-            V2FConv3d._corner_basis[key] = sph_harm_values(torch.eye(3, device=device), self.L)
+            # an ordinary tensor also when the first call comes from inside torch.inference_mode(): an inference
+            # tensor could not be saved for a later training step's backward
+            with torch.inference_mode(False), torch.no_grad():
+                V2FConv3d._corner_basis[key] = sph_harm_values(torch.eye(3, device=device), self.L)
         return V2FConv3d._corner_basis[key]
 
     def forward(self, inputs, face):

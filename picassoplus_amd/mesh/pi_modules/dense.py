@@ -12,6 +12,9 @@ from ... import _lib
 from ._check import F32, check_input, same_device, stream_of, workspace
 
 
+MAX_CHANNELS = 896     # input channels of the forward, output channels of grad_input: one 32-column weight slab in LDS
+
+
 def _dims(input, weight, bias):
     check_input(input, "input", 2, F32)
     check_input(weight, "weight", 2, F32)
@@ -19,7 +22,7 @@ def _dims(input, weight, bias):
     if weight.shape[0] != Ci:
         raise RuntimeError("weight must have shape (in_channels, out_channels)")
     Co = weight.shape[1]
-    if Ci < 1 or Co < 1 or Ci > 896:
+    if Ci < 1 or Co < 1 or Ci > MAX_CHANNELS:
         raise RuntimeError("dense tail supports 1..896 input channels, got %d" % Ci)
     if bias is not None:
         check_input(bias, "bias", 1, F32)

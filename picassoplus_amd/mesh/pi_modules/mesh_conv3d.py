@@ -28,8 +28,8 @@ def vertex2facet_forward(input, filter, face):
     """mesh_conv3d.cpp:123-152: (NvIn,C),(3,C,r),(NfIn,3) -> (NfIn,C*r)."""
     Nv, Nf, C, r = _v2f_dims(input, filter, face)
     dev = same_device(input, filter, face)
-    if Nf and Nv:
-        topology._check_range_cached(face, Nv)
+    if Nf:
+        topology._check_range_cached(face, Nv)       # an empty input with facets raises: every index is out of range
     with torch.cuda.device(dev):
         out = torch.empty((Nf, C * r), dtype=F32, device=dev)
         _lib.call("pmesh_v2f_fwd", input.data_ptr(), filter.data_ptr(), face.data_ptr(), out.data_ptr(),

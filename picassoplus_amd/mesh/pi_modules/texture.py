@@ -29,15 +29,14 @@ def _dims(input, face, baryCoord, numTexture):
 
 
 def _check_totals(numTexture, T):
-    """One-off validation of the running totals (synchronises; only on a cache miss)."""
-    key = topology._key("rt", numTexture, int(T))
-    if topology._lookup(key) is None:
+    """One-off validation of the running totals (synchronises; only the first time a tensor is seen)."""
+    def check():
         if numTexture.numel() and topology._checks_enabled():
             steps = torch.diff(numTexture, prepend=numTexture.new_zeros(1))
             if int(steps.min()) < 0 or int(numTexture[-1]) != T:
                 raise RuntimeError("numTexture must be a non-decreasing running total that ends at the number of "
                                    "texture points (%d)" % T)
-        topology._store(key, (True, numTexture))
+    topology.checked_once("rt", (numTexture,), (int(T),), check)
 
 
 def texture_forward(input, face, baryCoord, numTexture, degree):
@@ -46,8 +45,8 @@ def texture_forward(input, face, baryCoord, numTexture, degree):
     if degree is not None and (degree < 0 or degree > 5):
         raise NotImplementedError("spherical harmonics are implemented for degree 0..5")
     dev = same_device(input, face, baryCoord, numTexture)
-    if Nf and Nv:
-        topology._check_range_cached(face, Nv)
+    if Nf:
+        topology._check_range_cached(face, Nv)       # an empty input with facets raises: every index is out of range
     _check_totals(numTexture, T)
     with torch.cuda.device(dev):
         tex = torch.empty((T, C), dtype=F32, device=dev)

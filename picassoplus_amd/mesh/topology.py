@@ -4,51 +4,128 @@ The reference passes raw index tensors (``face``, ``vt_map``, ``vt_replace``) to
 and scatters with float atomics.  Here the scatter ops are segmented reductions, which need
 the transposed adjacency.  A network reuses the same index tensors for every convolution of
 a mesh level, forward and backward (picasso/networks/pi2_blocks.py:89-92 in the reference),
-so the adjacency is cached per index tensor: the key is the tensor's storage address, shape
-and in-place version counter, and the entry keeps the tensor alive so the address cannot be
-recycled while cached.
+so the adjacency is cached per index tensor.
+
+Cache discipline
+  key      storage address, shape, in-place version counter and device of every index tensor
+           involved (plus the integer arguments).  Inference tensors carry no version counter;
+           they cannot be modified outside inference mode, and their key uses -1.
+  lifetime an entry holds WEAK references to its index tensors and dies with the first of them:
+           a training loop that feeds fresh ``face`` / ``vt_map`` tensors every batch
+           (picasso/mesh/fit.py:34-45, dataset_scene.py:87-111) keeps the adjacency of the
+           batches still alive and nothing else.  While a tensor lives its storage address
+           cannot be handed to another allocation, so a live key never names other data.
+  size     the device arrays of all entries together stay below ``MAX_BYTES`` (environment
+           variable PICASSO_MESH_CACHE_BYTES, default 2 GiB); the least recently used go first.
+  streams  an entry remembers the stream it was built on and an event recorded behind the build;
+           a consumer on another stream waits for that event (nothing is waited for once the
+           event has completed, and nothing during stream capture, whose warm-up has run the build).
 """
 import os
 import threading
+import weakref
 from collections import OrderedDict
 
 import torch
 
 from .. import _lib
 
-_LOCK = threading.Lock()
-_CACHE = OrderedDict()
-MAX_ENTRIES = 256
+_LOCK = threading.RLock()        # re-entrant: a finaliser may run while the owner thread holds it
+_CACHE = OrderedDict()           # key -> _Entry
+_BYTES = 0
+MAX_BYTES = int(os.environ.get("PICASSO_MESH_CACHE_BYTES", str(2 << 30)))
+
+
+class _Entry:
+    __slots__ = ("value", "nbytes", "stream", "event", "finalizers")
+
+    def __init__(self, value, nbytes, stream, event):
+        self.value, self.nbytes, self.stream, self.event, self.finalizers = value, nbytes, stream, event, []
 
 
 def clear_cache():
+    global _BYTES
     with _LOCK:
+        for e in _CACHE.values():
+            for fin in e.finalizers:
+                fin.detach()
         _CACHE.clear()
+        _BYTES = 0
+
+
+def cache_bytes():
+    """Device bytes held by the cached adjacency arrays."""
+    return _BYTES
+
+
+def cache_entries():
+    return len(_CACHE)
+
+
+def _version(t):
+    return t._version if not t.is_inference() else -1
 
 
 def _key(kind, *tensors_and_ints):
     parts = [kind]
     for t in tensors_and_ints:
         if isinstance(t, torch.Tensor):
-            parts.append((t.data_ptr(), tuple(t.shape), t._version, t.device.index))
+            parts.append((t.data_ptr(), tuple(t.shape), _version(t), t.device.index))
         else:
             parts.append(t)
     return tuple(parts)
 
 
+def _drop(key):
+    global _BYTES
+    with _LOCK:
+        e = _CACHE.pop(key, None)
+        if e is not None:
+            _BYTES -= e.nbytes
+            for fin in e.finalizers:
+                fin.detach()
+
+
 def _lookup(key):
+    """Cached value or None.  A hit on another stream than the builder's waits for the build."""
     with _LOCK:
-        hit = _CACHE.get(key)
-        if hit is not None:
-            _CACHE.move_to_end(key)
-        return hit
+        e = _CACHE.get(key)
+        if e is None:
+            return None
+        _CACHE.move_to_end(key)
+        ev = e.event
+    if ev is not None:
+        if ev.query():
+            e.event = None
+        elif not torch.cuda.is_current_stream_capturing():
+            cur = torch.cuda.current_stream()
+            if cur.cuda_stream != e.stream:
+                cur.wait_event(ev)
+    return e.value
 
 
-def _store(key, value):
+def _store(key, value, owners, arrays=()):
+    """``owners``: the index tensors the entry is valid for (weakly referenced); ``arrays``: the device arrays
+    built for it (counted against MAX_BYTES; they are part of ``value``)."""
+    global _BYTES
+    nbytes = sum(int(a.numel()) * a.element_size() for a in arrays)
+    event = stream = None
+    if arrays and arrays[0].is_cuda and not torch.cuda.is_current_stream_capturing():
+        cur = torch.cuda.current_stream(arrays[0].device)
+        event, stream = torch.cuda.Event(), cur.cuda_stream
+        event.record(cur)
+    e = _Entry(value, nbytes, stream, event)
     with _LOCK:
-        _CACHE[key] = value
-        while len(_CACHE) > MAX_ENTRIES:
-            _CACHE.popitem(last=False)
+        _drop(key)
+        for t in owners:
+            if t is not None:
+                fin = weakref.finalize(t, _drop, key)
+                fin.atexit = False
+                e.finalizers.append(fin)
+        _CACHE[key] = e
+        _BYTES += nbytes
+        while _BYTES > MAX_BYTES and len(_CACHE) > 1:
+            _drop(next(iter(_CACHE)))
 
 
 def _stream(t):
@@ -60,10 +137,11 @@ def _checks_enabled():
 
 
 def _check_range(name, t, lo, hi):
-    """One-off validation of an index tensor (synchronises; only on a cache miss)."""
+    """One-off validation of an index tensor (one reduction and one synchronisation; only on a cache miss,
+    and not at all with PICASSO_MESH_SKIP_CHECKS=1)."""
     if t.numel() == 0 or not _checks_enabled():
         return
-    mn, mx = int(t.min()), int(t.max())
+    mn, mx = (int(x) for x in torch.aminmax(t))
     if mn < lo or mx >= hi:
         raise RuntimeError("%s holds indices in [%d, %d], valid range is [%d, %d)" % (name, mn, mx, lo, hi))
 
@@ -78,7 +156,7 @@ def vertex_csr(face, vt_map, n_rows):
     key = _key("v", face, vt_map, int(n_rows))
     hit = _lookup(key)
     if hit is not None:
-        return hit[0], hit[1]
+        return hit
     nf = face.shape[0]
     n_keys = vt_map.shape[0] if vt_map is not None else n_rows
     _check_range("face", face, 0, n_keys)
@@ -90,7 +168,7 @@ def vertex_csr(face, vt_map, n_rows):
         _lib.call("pmesh_build_vertex_csr", face.data_ptr(), vt_map.data_ptr() if vt_map is not None else None,
                   nf, n_keys if vt_map is not None else 0, n_rows, rowptr.data_ptr(), colidx.data_ptr(),
                   ws.data_ptr(), ws_bytes, _stream(face))
-    _store(key, (rowptr, colidx, face, vt_map))
+    _store(key, (rowptr, colidx), (face, vt_map), (rowptr, colidx))
     return rowptr, colidx
 
 
@@ -102,7 +180,7 @@ def cluster_csr(vt_replace, vt_map, n_coarse):
     key = _key("c", vt_replace, vt_map, int(n_coarse))
     hit = _lookup(key)
     if hit is not None:
-        return hit[0], hit[1]
+        return hit
     n_fine = vt_replace.shape[0]
     if vt_map.shape[0] != n_fine:
         raise RuntimeError("vt_replace and vt_map must have the same length")
@@ -114,7 +192,7 @@ def cluster_csr(vt_replace, vt_map, n_coarse):
         ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=vt_replace.device)
         _lib.call("pmesh_build_cluster_csr", vt_replace.data_ptr(), vt_map.data_ptr(), n_fine, n_coarse,
                   rowptr.data_ptr(), members.data_ptr(), ws.data_ptr(), ws_bytes, _stream(vt_replace))
-    _store(key, (rowptr, members, vt_replace, vt_map))
+    _store(key, (rowptr, members), (vt_replace, vt_map), (rowptr, members))
     return rowptr, members
 
 
@@ -124,7 +202,7 @@ def facet_order(cum_texture, n_points):
     key = _key("o", cum_texture, int(n_points))
     hit = _lookup(key)
     if hit is not None:
-        return hit[0]
+        return hit
     nf = cum_texture.shape[0]
     with torch.cuda.device(cum_texture.device):
         order = torch.empty(nf, dtype=torch.int32, device=cum_texture.device)
@@ -132,7 +210,7 @@ def facet_order(cum_texture, n_points):
         ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=cum_texture.device)
         _lib.call("pmesh_build_facet_order", cum_texture.data_ptr(), nf, int(n_points), order.data_ptr(),
                   ws.data_ptr(), ws_bytes, _stream(cum_texture))
-    _store(key, (order, cum_texture))
+    _store(key, order, (cum_texture,), (order,))
     return order
 
 
@@ -140,26 +218,29 @@ def running_total(num_texture):
     """Inclusive running total (int32) of the per-facet texture-point counts, the form facet2facet takes
     (picasso/mesh/layers.py:57 computes it in every forward); cached per counts tensor, so that the facet order
     built from it is found again too."""
-    key = _key("c", num_texture)
+    key = _key("t", num_texture)
     hit = _lookup(key)
     if hit is not None:
-        return hit[0]
+        return hit
     total = torch.cumsum(num_texture, dim=0, dtype=torch.int)
-    _store(key, (total, num_texture))
+    _store(key, total, (num_texture,), (total,))
     return total
+
+
+def checked_once(kind, owners, extra, check):
+    """Run ``check()`` unless the same tensors (and ``extra`` integers) passed it before."""
+    key = _key(kind, *owners, *extra)
+    if _lookup(key) is None:
+        check()
+        _store(key, True, owners)
 
 
 def _check_range_cached(face, n_vertices):
     """Validate a facet tensor against a vertex count once per tensor."""
-    key = _key("rf", face, int(n_vertices))
-    if _lookup(key) is None:
-        _check_range("face", face, 0, n_vertices)
-        _store(key, (True, face))
+    checked_once("rf", (face,), (int(n_vertices),), lambda: _check_range("face", face, 0, n_vertices))
 
 
 def _check_cluster_cached(vt_replace, vt_map):
-    key = _key("rk", vt_replace, vt_map)
-    if _lookup(key) is None:
-        n_fine = vt_replace.shape[0]
-        _check_range("vt_replace", vt_replace, -(n_fine - 1), max(n_fine, 1))
-        _store(key, (True, vt_replace, vt_map))
+    n_fine = vt_replace.shape[0]
+    checked_once("rk", (vt_replace, vt_map), (),
+                 lambda: _check_range("vt_replace", vt_replace, -(n_fine - 1), max(n_fine, 1)))

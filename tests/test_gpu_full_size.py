@@ -86,6 +86,23 @@ def test_f2f_full_size_adjoints_and_sample_parity(cuda, scene):
     assert_close(out.detach()[pick_t], ref_out, "f2f out (sampled facets)")
     assert_close(gtex[rows_t], ref_gtex, "f2f grad_texture (sampled facets)")
 
+    # the filter gradient element by element: float64 restatement, one mesh-sized block of facets at a time
+    # (G of a block is 300 k x 64 x 16 doubles), summed over the blocks
+    say("  grad_filter against the float64 oracle, block by block")
+    from oracle import torch_ref as R
+    torch.set_num_threads(16)
+    cum_np = np.cumsum(counts).astype(np.int64)
+    ref_gw = torch.zeros(d["C"], d["C"], 16, dtype=torch.float64)
+    tex_c, sh_c, g_c = d["tex"].cpu(), d["sh"].cpu(), g.cpu()
+    step = 300_000
+    for f0 in range(0, d["nf"], step):
+        f1 = min(f0 + step, d["nf"])
+        k0, k1 = (int(cum_np[f0 - 1]) if f0 else 0), int(cum_np[f1 - 1])
+        G, _, _ = R.f2f_moments(tex_c[k0:k1].double(), sh_c[k0:k1].double(), torch.from_numpy((cum_np[f0:f1] - k0).astype(np.int32)))
+        ref_gw += torch.einsum("fo,fcd->ocd", g_c[f0:f1].double(), G)
+        del G
+    assert_close(gw, ref_gw.numpy(), "f2f grad_filter (whole batch, element by element)")
+
     # the facet order is an optimisation only.  A facet's power-of-two operand scale can depend on its workgroup
     # (all of it falls back to exact row maxima when one facet exceeds its first bound), which moves results by
     # an ulp at most; with no such fallback, as on this data, nothing changes by a bit
@@ -114,6 +131,33 @@ def test_f2v_full_size_adjoints(cuda, scene):
     scale = float(out.double().norm() * g.double().norm())
     _adjoint_ok(lhs, _dot(x, gx), scale, "<f2v(x), g> = <x, grad_input>")
     _adjoint_ok(lhs, _dot(w, gw), scale, "<f2v(x), g> = <filter, grad_filter>")
+    # oracle parity: output rows of sampled vertices (a row depends on the facets around that vertex only),
+    # grad_input rows of sampled facets (a row depends on the facet's three vertices only), and the whole
+    # filter gradient element by element from the float64 restatement
+    say("  f2v sampled rows and grad_filter against the float64 oracle")
+    from oracle import torch_ref as R
+    torch.set_num_threads(16)
+    rng = np.random.default_rng(11)
+    f_np = d["face_np"].astype(np.int64)
+    nfc_np = d["nfc"].cpu().numpy()
+    x_np, w_np = x.detach().cpu().numpy().astype(np.float64), w.detach().cpu().numpy().astype(np.float64)
+    coeff_np = d["coeff"].cpu().numpy().astype(np.float64)
+    pick_v = np.sort(rng.choice(d["nv"], 2000, replace=False))
+    is_pick = np.zeros(d["nv"], bool)
+    is_pick[pick_v] = True
+    around = np.nonzero(is_pick[f_np].any(1))[0]                 # facets with a sampled corner
+    sub_out = loops.f2v_fwd(x_np[around], w_np, coeff_np[around], f_np[around].astype(np.int32), nfc_np,
+                            np.arange(d["nv"], dtype=np.int32))
+    assert_close(out.detach()[torch.from_numpy(pick_v).to(cuda)], sub_out[pick_v], "f2v out (sampled vertices)")
+    pick_f = np.sort(rng.choice(d["nf"], 2000, replace=False))
+    sub_gin, _ = loops.f2v_bwd(g.cpu().numpy().astype(np.float64), x_np[pick_f], w_np, coeff_np[pick_f],
+                               f_np[pick_f].astype(np.int32), nfc_np, np.arange(d["nv"], dtype=np.int32))
+    assert_close(gx[torch.from_numpy(pick_f).to(cuda)], sub_gin, "f2v grad_input (sampled facets)")
+    _, ref_gw = R.f2v_bwd(g.cpu().double(), x.detach().cpu().double(), w.detach().cpu().double(), d["coeff"].cpu().double(),
+                          d["face"].cpu(), d["nfc"].cpu(), d["vt_map"].cpu())
+    assert_close(gw, ref_gw.numpy(), "f2v grad_filter (whole batch, element by element)")
+    del ref_gw
+
     # a constant field with unit coefficient 0 and all other coefficients zero is averaged to itself
     coeff = torch.zeros_like(d["coeff"])
     coeff[:, 0] = 1.0
@@ -195,6 +239,15 @@ def test_pool_full_size_invariants(cuda):
     # every gradient entry sits at a maximum of its cluster
     nz = gx != 0
     assert torch.equal(x.detach()[nz], ref[cl][nz])
+    # the arg-max indices of the whole grid, bit for bit against the oracle (smallest vertex wins a tie)
+    from oracle import torch_ref as R
+    from picassoplus_amd.mesh.pi_modules import mesh_pool3d
+    torch.set_num_threads(16)
+    y2, idx = mesh_pool3d.max_forward(x.detach(), vr, vm, vt_out)
+    ref_y, ref_idx = R.maxpool_fwd(x.detach().cpu(), torch.from_numpy(vt_replace), torch.from_numpy(vt_map), nvo)
+    assert np.array_equal(idx.cpu().numpy(), ref_idx.numpy()), "max_index differs from the oracle"
+    assert np.array_equal(y2.cpu().numpy(), ref_y.numpy())
+    del ref_y, ref_idx, y2, idx
 
     ya = pool3d.avgPool(x, vr, vm, vt_out)
     (gxa,) = torch.autograd.grad(ya, x, g)

@@ -213,26 +213,30 @@ def test_argument_errors_and_side_stream(cuda):
     assert torch.equal(got, ref) and float(total) == float(ref.sum())
 
 
-def test_two_level_stack_matches_oracle_composition(cuda):
+@pytest.mark.parametrize("cells,W", [(16, [8, 16, 16]), (64, [32, 64, 128, 256, 256])],
+                         ids=["two_levels_8_16", "four_levels_32_64_128_256"])
+def test_level_stack_matches_oracle_composition(cuda, cells, W):
     """Encoder-decoder over a mesh hierarchy, as the benchmark's hierarchy workload builds it: per level
     V2F + (texture interpolation -> F2F) -> F2V, pooling, then unpooling back with a pointwise layer; outputs and
-    every gradient against the same composition of float64 oracle ops."""
+    every gradient against the same composition of float64 oracle ops.  The four-level case runs the hierarchy
+    configuration's widths 32 / 64 / 128 / 256 (4:1 levels of a 64 x 64-cell grid: 8192, 2048, 512 and 128 facets)."""
     from picassoplus_amd.mesh.pi_modules import texture
-    L, W = 3, [8, 16, 16]
-    meshes = S.hierarchy_workload(seed=7, cells=16, levels=2)
+    L, n_levels = 3, len(W) - 1
+    print("case level stack", cells, W, flush=True)
+    meshes = S.hierarchy_workload(seed=7, cells=cells, levels=n_levels)
     rng = np.random.default_rng(24)
     torch.manual_seed(6)
     lv = []
-    for l in range(2):
+    for l in range(n_levels):
         m = meshes[l]
         v, f = m["vertex"], m["face"]
         nv, nf = v.shape[0], f.shape[0]
         normal, _ = S.triangle_normals_areas(v, f)
-        counts, bary, _ = S.texture_points(rng, nf, rng.integers(0, 4, nf).astype(np.int32))
+        counts, bary, _ = S.texture_points(rng, nf, rng.integers(0, 4 if n_levels == 2 else 10, nf).astype(np.int32))
         d = dict(nv=nv, face=torch.from_numpy(f), counts=torch.from_numpy(counts), bary=torch.from_numpy(bary),
                  normal=torch.from_numpy(normal), nfc=torch.from_numpy(np.maximum(S.vertex_facet_count(f, np.arange(nv), nv), 1).astype(np.int32)),
                  ident=torch.arange(nv, dtype=torch.int32), vr=torch.from_numpy(m["vt_replace"]), vm=torch.from_numpy(m["vt_map"]),
-                 nvo=m["nv_out"], method="max" if l == 0 else "avg",
+                 nvo=m["nv_out"], method="max" if l % 2 == 0 else "avg",
                  v2f=layers.V2FConv3d(W[l], W[l], L, with_bn=False).to(cuda), f2f=layers.F2FConv3d(W[l], W[l], L, with_bn=False).to(cuda),
                  f2v=layers.F2VConv3d(W[l], W[l + 1], L, with_bn=False).to(cuda), up=layers.PerItemConv3d(W[l + 1], W[l], with_bn=False).to(cuda))
         for k in ("v2f", "f2f", "f2v", "up"):
@@ -336,3 +340,79 @@ def test_forward_replays_from_a_hip_graph(cuda):
             eager = run(x)                                      # the program's own eager work between the replays
             torch.cuda.synchronize()
             assert torch.equal(got, eager), "replay %d differs from the eager result" % i
+
+
+def _block_step(cuda, mods, x, f_np, bary_np, counts_np, normal_np, nfc_np, vr_np, vm_np, nvo, train):
+    """One step of a small block with index tensors made from numpy anew: what a data loader hands a training or
+    evaluation loop every batch."""
+    from picassoplus_amd.mesh.pi_modules import texture
+    c = lambda a: torch.from_numpy(a).to(cuda)
+    face, counts, bary = c(f_np), c(counts_np), c(bary_np)
+    nfc, ident, vr, vm = c(nfc_np), torch.arange(x.shape[0], dtype=torch.int32, device=cuda), c(vr_np), c(vm_np)
+    coeff = layers.SphHarmCoeff(3)(c(normal_np))
+    xg = x.clone().requires_grad_(train)
+    tex, sh = texture.interpolate(xg, face, bary, torch.cumsum(counts, 0, dtype=torch.int32), 3)
+    y = mods[0](xg, face, nfc, ident, coeff) + mods[2](mods[1](tex, sh, counts), face, nfc, ident, coeff)
+    p = layers.Pool3d("max")(y, vr, vm, torch.zeros(nvo, 3, device=cuda))
+    z = y + layers.Unpool3d()(p, vr, vm)
+    if not train:
+        return [z]
+    z.backward(torch.ones_like(z))
+    return [z.detach(), xg.grad] + [q.grad.clone() for m in mods for q in m.parameters()]
+
+
+def _block_case(cuda):
+    rng = np.random.default_rng(31)
+    meshes = S.hierarchy_workload(seed=11, cells=32, levels=1)
+    v, f = meshes[0]["vertex"], meshes[0]["face"]
+    nv, nf, C = v.shape[0], f.shape[0], 32
+    normal, _ = S.triangle_normals_areas(v, f)
+    counts, bary, _ = S.texture_points(rng, nf, rng.integers(1, 5, nf).astype(np.int32))
+    nfc = np.maximum(S.vertex_facet_count(f, np.arange(nv), nv), 1).astype(np.int32)
+    torch.manual_seed(12)
+    mods = [layers.V2VConv3d(C, [C, C], 3, [1, 1], with_bn=False).to(cuda), layers.F2FConv3d(C, C, 3, with_bn=False).to(cuda),
+            layers.F2VConv3d(C, C, 3, with_bn=False).to(cuda)]
+    x = torch.randn(nv, C, device=cuda)
+    args = (f, bary.astype(np.float32), counts, normal.astype(np.float32), nfc, meshes[0]["vt_replace"], meshes[0]["vt_map"],
+            meshes[0]["nv_out"])
+    return mods, x, args
+
+
+def test_fresh_index_tensors_every_step_keep_memory_flat(cuda):
+    """A training loop hands new face / vt_map / vt_replace tensors to the modules in every batch
+    (picasso/mesh/fit.py:34-45 in the reference): the adjacency built for a batch must go when the batch's tensors go,
+    device memory must stay flat over hundreds of steps, and every step must give the bits of the first one."""
+    from picassoplus_amd.mesh import topology
+    mods, x, args = _block_case(cuda)
+    topology.clear_cache()
+    first = _block_step(cuda, mods, x, *args, train=True)
+    for m in mods:
+        m.zero_grad(set_to_none=True)
+    torch.cuda.synchronize()
+    assert topology.cache_entries() == 0, "adjacency outlived its index tensors"
+    base = torch.cuda.memory_allocated()
+    peak_entries = 0
+    for step in range(300):
+        got = _block_step(cuda, mods, x, *args, train=True)
+        peak_entries = max(peak_entries, topology.cache_entries())
+        for m in mods:
+            m.zero_grad(set_to_none=True)
+        if step % 100 == 99:
+            torch.cuda.synchronize()
+            assert all(torch.equal(a, b) for a, b in zip(got, first)), "step %d differs from the first" % step
+            del got
+            assert torch.cuda.memory_allocated() <= base + (1 << 20), (torch.cuda.memory_allocated(), base)
+    assert topology.cache_entries() == 0 and topology.cache_bytes() == 0
+
+
+def test_modules_run_under_inference_mode(cuda):
+    """An evaluation loop that moves its batch to the GPU inside torch.inference_mode() makes inference tensors,
+    which have no version counter: the adjacency cache must take them as keys (V2V, F2F, pooling, unpooling)."""
+    mods, x, args = _block_case(cuda)
+    with torch.no_grad():
+        ref = _block_step(cuda, mods, x, *args, train=False)[0]
+    with torch.inference_mode():
+        out = _block_step(cuda, mods, x.clone(), *args, train=False)[0]
+        out2 = _block_step(cuda, mods, x.clone(), *args, train=False)[0]
+    torch.cuda.synchronize()
+    assert torch.equal(out, ref) and torch.equal(out2, ref)

@@ -16,7 +16,7 @@ from picassoplus_amd.mesh import topology
 from picassoplus_amd.mesh.layers import sph_harm_values
 from picassoplus_amd.mesh.pi_modules import (conv3d, mesh_conv3d, mesh_pool3d, mesh_unpool3d, pool3d,
                                              texture, unpool3d)
-from util import assert_close, dev, mesh_case, rel_err, strided_vt_map, texture_case
+from util import assert_as_good_as_f32, assert_close, dev, mesh_case, rel_err, strided_vt_map, texture_case
 
 pytestmark = pytest.mark.gpu
 
@@ -92,6 +92,12 @@ def test_v2f_parity(cuda, mesh, C, r):
     assert_close(out, out_ref, "v2f out")
     assert_close(xt.grad, gin_ref, "v2f grad_input")
     assert_close(ft.grad, gfilt_ref, "v2f grad_filter")
+    # no worse than twice the float32 loops in the reference's summation order
+    f32 = np.float32
+    gin32, gfilt32 = loops.v2f_bwd(gout.astype(f32), x.astype(f32), filt.astype(f32), f, dtype=f32)
+    assert_as_good_as_f32(out, out_ref, loops.v2f_fwd(x.astype(f32), filt.astype(f32), f, dtype=f32), "v2f out")
+    assert_as_good_as_f32(xt.grad, gin_ref, gin32, "v2f grad_input")
+    assert_as_good_as_f32(ft.grad, gfilt_ref, gfilt32, "v2f grad_filter")
 
 
 # ------------------------------------------------------------------ texture points from vertex features
@@ -206,6 +212,12 @@ def test_f2v_parity(cuda, monkeypatch, mesh, C, r, K, strided, path):
     assert_close(out, out_ref, "f2v out")
     assert_close(xt.grad, gin_ref, "f2v grad_input")
     assert_close(ft.grad, gfilt_ref, "f2v grad_filter")
+    f32 = np.float32
+    a32 = (x.astype(f32), filt.astype(f32), coeff.astype(f32), f, np.maximum(nfc, 1), vt_map)
+    gin32, gfilt32 = loops.f2v_bwd(gout.astype(f32), *a32, dtype=f32)
+    assert_as_good_as_f32(out, out_ref, loops.f2v_fwd(*a32, dtype=f32), "f2v out")
+    assert_as_good_as_f32(xt.grad, gin_ref, gin32, "f2v grad_input")
+    assert_as_good_as_f32(ft.grad, gfilt_ref, gfilt32, "f2v grad_filter")
 
 
 def test_f2v_unit_count_is_plain_scatter(cuda):
@@ -231,7 +243,9 @@ def test_f2v_unit_count_is_plain_scatter(cuda):
                                                 (333, 16, 96, 16, 4), (70, 5, 7, 9, 3), (65, 4, 6, 36, 2),
                                                 (64, 3, 5, 50, 2), (129, 130, 64, 4, 3), (50, 8, 8, 1, 2),
                                                 (300, 8, 40, 16, 14), (1000, 64, 64, 16, 9), (130, 4, 130, 16, 20),
-                                                (50, 1, 8, 16, 3), (77, 2, 33, 16, 12)])
+                                                (50, 1, 8, 16, 3), (77, 2, 33, 16, 12),
+                                                (300, 128, 128, 16, 9), (260, 256, 256, 16, 9), (150, 128, 256, 16, 6),
+                                                (90, 256, 128, 16, 4), (200, 32, 32, 16, 9)])
 @pytest.mark.parametrize("path", ["default", "generic", "fp32mfma", "bf16x3", "half"])
 def test_f2f_parity(cuda, monkeypatch, nf, Cin, Cout, F, kmax, path):
     """``generic`` forces the shape-generic kernels, ``fp32mfma`` the fp32-matrix-instruction variant of the
@@ -267,6 +281,14 @@ def test_f2f_parity(cuda, monkeypatch, nf, Cin, Cout, F, kmax, path):
          assert_close(ft.grad, gfilt_ref, "f2f grad_filter", tol)]
     if path == "half" and Cin > 4 and Cin % 4 == 0 and Cout % 8 == 0:
         assert max(e) > 2e-6, "the half-precision variant did not run"         # it is not the full-precision result
+    if path != "half":
+        f32 = np.float32
+        a32 = (tex.astype(f32), filt.astype(f32), sh.astype(f32), cum)
+        gin32, gfilt32 = loops.f2f_bwd(gout.astype(f32), *a32, dtype=f32)
+        e_o = assert_as_good_as_f32(out, out_ref, loops.f2f_fwd(*a32, dtype=f32), "f2f out")
+        e_t = assert_as_good_as_f32(tt.grad, gin_ref, gin32, "f2f grad_texture")
+        e_w = assert_as_good_as_f32(ft.grad, gfilt_ref, gfilt32, "f2f grad_filter")
+        say("  errors (build, float32 oracle): out %.2e %.2e  grad_texture %.2e %.2e  grad_filter %.2e %.2e" % (e_o + e_t + e_w))
 
 
 @pytest.mark.parametrize("case", ["late_channels", "late_points", "growing_facets"])

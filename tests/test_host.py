@@ -225,3 +225,43 @@ def test_texture_points():
 def test_bench_refuses_more_than_one_gpu():
     res = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
     assert res.returncode != 0 and "one GPU" in res.stderr
+
+
+def test_adjacency_cache_discipline():
+    """The cache of per-index-tensor arrays: an entry dies with its index tensor (weak references), inference
+    tensors are accepted as keys, the least recently used entries go when the byte bound is passed, and an in-place
+    change of an index tensor makes a new key.  Host-side logic only: the cached values here are CPU tensors."""
+    import gc
+    from picassoplus_amd.mesh import topology as T
+    T.clear_cache()
+    a = torch.arange(12, dtype=torch.int32)
+    calls = []
+    T.checked_once("x", (a,), (3,), lambda: calls.append(1))
+    T.checked_once("x", (a,), (3,), lambda: calls.append(1))
+    assert calls == [1] and T.cache_entries() == 1
+    a.add_(1)                                         # version counter moved: a new key
+    T.checked_once("x", (a,), (3,), lambda: calls.append(1))
+    assert calls == [1, 1]
+    del a
+    gc.collect()
+    assert T.cache_entries() == 0                     # entries went with their tensor
+    with torch.inference_mode():
+        b = torch.arange(6, dtype=torch.int32)
+    assert b.is_inference()
+    T.checked_once("x", (b,), (), lambda: calls.append(1))    # no version counter to read on this one
+    assert T.cache_entries() == 1
+    # byte bound: three arrays of 400 bytes against a bound of 1000
+    old = T.MAX_BYTES
+    try:
+        T.MAX_BYTES = 1000
+        T.clear_cache()
+        owners = [torch.zeros(4, dtype=torch.int32) for _ in range(3)]
+        for i, o in enumerate(owners):
+            arr = torch.zeros(100, dtype=torch.int32)
+            T._store(T._key("y", o), arr, (o,), (arr,))
+        assert T.cache_entries() == 2 and T.cache_bytes() == 800
+        assert T._lookup(T._key("y", owners[0])) is None and T._lookup(T._key("y", owners[2])) is not None
+    finally:
+        T.MAX_BYTES = old
+        T.clear_cache()
+    assert T.cache_bytes() == 0

@@ -24,6 +24,22 @@ def assert_close(y, ref, what, tol=TOL_F32):
     return e
 
 
+# Second parity criterion of the convolutions: the build's error must not exceed twice the error the float32 loop
+# oracle makes when it sums in the reference's order (both measured against the float64 answer).  Below two units of
+# the last place of the largest value the comparison would measure the rounding of the result itself, not of the
+# sums, hence the floor.
+F32_FLOOR = 2.0 ** -22
+
+
+def assert_as_good_as_f32(y, ref64, ref32, what):
+    """``y`` (GPU result) against the float64 oracle ``ref64``, relative to how far the float32 oracle ``ref32``
+    (reference summation order) is from it: err(y) <= max(2 err(ref32), 2^-22).  Returns (err(y), err(ref32))."""
+    e = rel_err(y.detach().cpu().numpy() if isinstance(y, torch.Tensor) else y, ref64)
+    e32 = rel_err(ref32, ref64)
+    assert e <= max(2.0 * e32, F32_FLOOR), "%s: error %.3e exceeds twice the float32 oracle's %.3e" % (what, e, e32)
+    return e, e32
+
+
 def dev(a, device, dtype=None):
     t = torch.from_numpy(np.ascontiguousarray(a))
     if dtype is not None:

@@ -154,6 +154,25 @@ def f2f_bwd(gout, tex, filt, bary, cum):
     return gin, gfilt
 
 
+def f2f_bwd_filter_pointwise(gout, tex, bary, cum, block=200_000):
+    """The filter gradient in the reference's own point-wise form (mesh_conv3d_gpu.cu:85-135: every texture
+    point k of facet f adds gout[f,co] * tex[k,ci] * bary[k,d] / K_f), as one product per block of points:
+    gfilt[co,(ci,d)] = sum_k (gout[f(k),co] / K_f(k)) * (tex[k,ci] * bary[k,d]).  No per-facet moments are
+    formed, so memory stays at block * Cin * F values: the form for scene-sized batches."""
+    T, Cin = tex.shape
+    F = bary.shape[1]
+    counts, seg = _segments(cum, T)
+    inv = torch.where(counts > 0, 1.0 / counts.clamp(min=1).to(tex.dtype), torch.zeros((), dtype=tex.dtype))
+    gfilt = torch.zeros(gout.shape[1], Cin * F, dtype=tex.dtype)
+    for k0 in range(0, T, block):
+        k1 = min(k0 + block, T)
+        s = seg[k0:k1]
+        a = gout[s] * inv[s][:, None]
+        b = (tex[k0:k1, :, None] * bary[k0:k1, None, :]).reshape(k1 - k0, Cin * F)
+        gfilt += a.t() @ b
+    return gfilt.reshape(gout.shape[1], Cin, F)
+
+
 # --------------------------------------------------------------------------
 # texture points from vertex features: tex[k] = sum_j bary[k,j] * x[face[f(k),j]] for the rows k of
 # facet f's segment (the grouping of layers.py:57); the reference loads texture features from its

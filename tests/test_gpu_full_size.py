@@ -86,21 +86,11 @@ def test_f2f_full_size_adjoints_and_sample_parity(cuda, scene):
     assert_close(out.detach()[pick_t], ref_out, "f2f out (sampled facets)")
     assert_close(gtex[rows_t], ref_gtex, "f2f grad_texture (sampled facets)")
 
-    # the filter gradient element by element: float64 restatement, one mesh-sized block of facets at a time
-    # (G of a block is 300 k x 64 x 16 doubles), summed over the blocks
-    say("  grad_filter against the float64 oracle, block by block")
+    # the filter gradient element by element, from the reference's point-wise form in float64 (blocks of points)
+    say("  grad_filter against the float64 oracle")
     from oracle import torch_ref as R
     torch.set_num_threads(16)
-    cum_np = np.cumsum(counts).astype(np.int64)
-    ref_gw = torch.zeros(d["C"], d["C"], 16, dtype=torch.float64)
-    tex_c, sh_c, g_c = d["tex"].cpu(), d["sh"].cpu(), g.cpu()
-    step = 300_000
-    for f0 in range(0, d["nf"], step):
-        f1 = min(f0 + step, d["nf"])
-        k0, k1 = (int(cum_np[f0 - 1]) if f0 else 0), int(cum_np[f1 - 1])
-        G, _, _ = R.f2f_moments(tex_c[k0:k1].double(), sh_c[k0:k1].double(), torch.from_numpy((cum_np[f0:f1] - k0).astype(np.int32)))
-        ref_gw += torch.einsum("fo,fcd->ocd", g_c[f0:f1].double(), G)
-        del G
+    ref_gw = R.f2f_bwd_filter_pointwise(g.cpu().double(), d["tex"].cpu().double(), d["sh"].cpu().double(), d["cum"].cpu())
     assert_close(gw, ref_gw.numpy(), "f2f grad_filter (whole batch, element by element)")
 
     # the facet order is an optimisation only.  A facet's power-of-two operand scale can depend on its workgroup

@@ -226,6 +226,18 @@ def test_explicit_backwards_match_autograd_and_loops():
     lp = loops.f2f_bwd(go, tex, W, sh, cum)
     for a, e, l in zip(auto, expl, lp):
         assert rel_err(e.numpy(), a.numpy()) < EPS and rel_err(l, a.numpy()) < EPS
+    # the point-wise form of the filter gradient (blocks of points, no per-facet moments) is the same sum:
+    # against autograd of the forward and the loops, with blocks that cut facets in two
+    pw = torch_ref.f2f_bwd_filter_pointwise(T(go), T(tex), T(sh), T(cum), block=7)
+    assert rel_err(pw.numpy(), auto[1].numpy()) < EPS and rel_err(pw.numpy(), lp[1]) < EPS
+    # nf_count as produced by count_vertex_adjface: the number of (facet, corner) pairs per kept vertex, counted by hand
+    cnt = np.zeros(nvo, np.int64)
+    for fc in f:
+        for vtx in fc:
+            if vt_map[vtx] >= 0:
+                cnt[vt_map[vtx]] += 1
+    assert np.array_equal(torch_ref.count_vertex_adjface(T(f), T(vt_map), nvo).numpy(), cnt)
+    assert np.array_equal(S.vertex_facet_count(f, vt_map, nvo), cnt)
 
 
 def test_adjoint_identities():

@@ -20,7 +20,8 @@
  *     thread-local message.  Argument errors are detected before anything is launched.
  *   - Reductions run over sorted adjacency (CSR) in a fixed order: results are
  *     bit-reproducible from run to run, unlike the reference's float atomics.
- *   - Entry points are re-entrant; they keep no global mutable state.
+ *   - Entry points are re-entrant; they keep no global mutable state (pmesh_f2v_bwd_static is the
+ *     one exception, see there).
  *
  * Symbols: cout = c*r + m is the depth-multiplied output channel of the V2F / F2V
  * convolutions, (C, r) = filter.shape[1:].
@@ -102,6 +103,23 @@ int pmesh_f2v_bwd(const float *grad_output, const float *input, const float *fil
                   const int32_t *vt_map, float *grad_input, float *grad_filter, void *workspace,
                   size_t workspace_bytes, int64_t Nf, int64_t NvIn, int64_t NvOut, int C, int r,
                   int K, pmesh_stream_t stream);
+
+/* pmesh_f2v_bwd for callers that cannot allocate device memory.  No counterpart in the reference (whose
+ * extensions allocate their outputs and need no workspace): it is for code that runs under HIP graph capture,
+ * tight serving loops and harnesses that forbid allocation.  Same arguments and results as pmesh_f2v_bwd without
+ * the workspace: the partial filter gradients go to a device array of pmesh_f2v_bwd_static_max_bytes() (8 MiB)
+ * that is part of the library image -- every GPU the library runs on holds its copy until the process ends.
+ * Limit: pmesh_f2v_bwd_workspace_bytes(C, r, K) must fit, i.e. K * C * r <= 2048 (16 coefficients: C * r <= 128);
+ * larger shapes fail with an error before anything is launched.  The call allocates and frees nothing.  All calls
+ * on one GPU share the array, which keeps the last call's contents (nothing needs clearing: every slice read is
+ * written first): calls that overlap on one GPU, on different streams or threads, race and must be serialised by
+ * the caller.  Unlike every other entry point, this one keeps state in the library (the array's address per
+ * device, looked up on the first call on that device). */
+size_t pmesh_f2v_bwd_static_max_bytes(void);
+int pmesh_f2v_bwd_static(const float *grad_output, const float *input, const float *filter,
+                         const float *coeff, const int32_t *face, const int32_t *nf_count,
+                         const int32_t *vt_map, float *grad_input, float *grad_filter, int64_t Nf,
+                         int64_t NvIn, int64_t NvOut, int C, int r, int K, pmesh_stream_t stream);
 
 /* ------------------------------------------------------------------ facet2facet
  * replaces facet2facet_forward / facet2facet_backward (mesh_conv3d.cpp:192-269)

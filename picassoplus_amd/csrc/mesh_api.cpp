@@ -22,4 +22,4 @@ void clear_error() { g_err[0] = 0; }
 }  // namespace pmesh
 
 extern "C" const char *pmesh_last_error(void) { return pmesh::g_err; }
-extern "C" int pmesh_abi_version(void) { return 10; }
+extern "C" int pmesh_abi_version(void) { return 11; }

@@ -14,6 +14,7 @@
 #include <stdlib.h>
 #include "../../include/picasso_mesh.h"
 #include <cstdlib>
+#include <mutex>
 
 namespace pmesh {
 
@@ -1038,6 +1039,57 @@ extern "C" int pmesh_f2v_bwd(const float *grad_output, const float *input, const
         f2v_bwd_k<1><<<dim3(G), dim3(kBlock), 0, st>>>(grad_output, input, filter, coeff, face, nf_count, vt_map, grad_input, partial, Nf, NvOut, C, r, K, rs.items, rs.lpr_log2, cvec, rows_per_block);
     PM_LAUNCHED("f2v_bwd");
     return reduce_partials(partial, grad_filter, G, K * Co, st);
+}
+
+// ---- facet2vertex backward without a workspace argument -----------------------------------
+// For callers that cannot allocate device memory (stream capture, serving loops, harnesses that forbid it): the
+// partial filter gradients live in a file-scope device array instead of a caller's workspace.  Every GPU the library
+// runs on holds its own copy of the array, at its own address, until the process ends; the address is looked up
+// once per device and kept.  Calls on one GPU share the array: calls that overlap there race.
+constexpr size_t kStaticScratchBytes = size_t(8) << 20;                   // K * C * r <= 2048 at 1024 partial slices
+constexpr int kStaticScratchMaxDevices = 64;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+static void *g_scratch_ptr[kStaticScratchMaxDevices];                     // device address of `scratch`, per device
+static std::mutex g_scratch_lock;
+
+// Device address of the current device's copy of `scratch` (the array's name itself is a host-side handle).
+static int static_scratch(void **out)
+{
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return fail("f2v_bwd_static: hipGetDevice failed: %s", hipGetErrorString(e));
+    PM_REQUIRE(dev >= 0 && dev < kStaticScratchMaxDevices, "f2v_bwd_static: device index %d not supported", dev);
+    std::lock_guard<std::mutex> hold(g_scratch_lock);
+    if (!g_scratch_ptr[dev]) {
+        void *p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p) return fail("f2v_bwd_static: hipGetSymbolAddress failed: %s", hipGetErrorString(e));
+        g_scratch_ptr[dev] = p;
+    }
+    *out = g_scratch_ptr[dev];
+    return 0;
+}
+
+extern "C" size_t pmesh_f2v_bwd_static_max_bytes(void) { return kStaticScratchBytes; }
+
+extern "C" int pmesh_f2v_bwd_static(const float *grad_output, const float *input, const float *filter,
+                                    const float *coeff, const int32_t *face, const int32_t *nf_count,
+                                    const int32_t *vt_map, float *grad_input, float *grad_filter, int64_t Nf,
+                                    int64_t NvIn, int64_t NvOut, int C, int r, int K, pmesh_stream_t stream)
+{
+    clear_error();
+    PM_DIMS("f2v_bwd_static");
+    PM_REQUIRE(K > 0 && K <= 4096, "f2v_bwd_static: bad filter size K=%d", K);
+    const size_t need = pmesh_f2v_bwd_workspace_bytes(C, r, K);
+    PM_REQUIRE(need <= kStaticScratchBytes,
+               "f2v_bwd_static: K*C*r = %lld needs %zu bytes of scratch, the static array holds %zu (K*C*r <= %zu); "
+               "use pmesh_f2v_bwd with a workspace", (long long)K * C * r, need, kStaticScratchBytes,
+               kStaticScratchBytes / (1024 * sizeof(float)));
+    void *ws = nullptr;
+    if (int rc = static_scratch(&ws)) return rc;
+    // every partial slice the reduction reads is written by the kernels of this call: nothing to clear
+    return pmesh_f2v_bwd(grad_output, input, filter, coeff, face, nf_count, vt_map, grad_input, grad_filter, ws,
+                         kStaticScratchBytes, Nf, NvIn, NvOut, C, r, K, stream);
 }
 
 // ---- pooling ---------------------------------------------------------------------------

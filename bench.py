@@ -46,6 +46,12 @@ def parse():
     ap.add_argument("--f2f-half", action="store_true",
                     help="facet2facet in its half-precision variant (one fp16 piece per operand, fp32 accumulation; "
                          "results within 1e-3 instead of 1e-5): a separate figure, never the default")
+    ap.add_argument("--bf16-features", action="store_true",
+                    help="scene workload with the features (texture rows, layer outputs, their gradients) kept in bf16 "
+                         "in HBM and one fp16 product per element with fp32 accumulation: a separate figure")
+    ap.add_argument("--traffic-from", nargs=2, metavar=("FETCH_CSV", "WRITE_CSV"),
+                    help="no benchmark: turn the counter_collection CSVs of two rocprofv3 --pmc runs (FETCH_SIZE, "
+                         "WRITE_SIZE) of this workload into profiles/traffic.json and a text summary")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="after the timed region, copy a 1 GiB buffer three times (a kernel of known HBM traffic "
                          "to scale rocprofv3's FETCH_SIZE / WRITE_SIZE counters by)")
@@ -92,18 +98,107 @@ def conv_bytes_flops(d, ops):
     return {k: tab[k] for k in ops}
 
 
-# HBM bytes per launch of the op's main kernel on the default scene workload (scale 1.0), measured with
-# rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE and scaled by what the same counters read for a 1 GiB copy
-# (--copy-calibration); reported as roofline.traffic when that workload runs.
-SCENE_TRAFFIC_BYTES = {"f2f_fwd": 5.323e9, "f2f_bwd_texture": 3.748e9, "f2f_bwd_filter": 3.348e9,
-                       "f2v_fwd": 1.284e9, "f2v_bwd": 2.186e9}
+# ---------------------------------------------------------------------------- measured HBM traffic
+# roofline.traffic = HBM bytes per launch of the dominant op from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per
+# dispatch), scaled by what the same counters read for a 1 GiB device copy (--copy-calibration).  The figures live in
+# profiles/traffic.json, written by `bench.py --traffic-from FETCH.csv WRITE.csv --workload W` from the two counter
+# runs, together with the identity of the build they were measured on (a hash over the kernel sources): a bench run
+# of any other build reports traffic = null instead of a stale number.
+TRAFFIC_JSON = os.path.join(ROOT, "profiles", "traffic.json")
+# op -> kernels whose traffic it sums (regular expressions on the demangled kernel name, after "pmesh::")
+TRAFFIC_KERNELS = {
+    "scene": {"f2f_fwd": [r"f2f16h2_fwd_k"], "f2f_bwd_texture": [r"f2f16h2_bwd_tex_k"],
+              "f2f_bwd_filter": [r"f2f16h2_bwd_filt_k", r"f2f16x3_bwd_filt_k", r"f2f_reduce_k"],
+              "f2v_fwd": [r"f2v_fwd_mfma_k"], "f2v_bwd": [r"f2v_bwd_mfma_k", r"reduce_partials_k"]},
+    "pool": {"pool_max_fwd": [r"pool_max_fwd_k"], "pool_max_bwd": [r"fine_gather_k<4, 2>"],
+             "pool_avg_fwd": [r"cluster_sum_k<4, true>"], "pool_avg_bwd": [r"fine_gather_k<4, 1>"],
+             "unpool_fwd": [r"fine_gather_k<4, 0>"], "unpool_bwd": [r"cluster_sum_k<4, false>"]},
+    "tail": {"dense_fwd": [r"dense_rows_k<.*false, (true|false)>$"], "dense_bwd": [r"dense_rows_k<.*true, (true|false)>$", r"dense_wgrad_k", r"reduce_partials_k"]},
+    "texture": {"texture_fwd": [r"texture_fwd_k"], "texture_bwd": [r"texture_bwd_flat_k", r"texture_bwd_k"]},
+}
 
 
-# the same for the other workloads at scale 1.0 (profiles/*_hbm_traffic_pmc.txt); an op of two kernels is their sum
-POOL_TRAFFIC_BYTES = {"pool_max_fwd": 0.818e9, "pool_max_bwd": 0.841e9, "pool_avg_fwd": 0.693e9, "pool_avg_bwd": 0.698e9,
-                      "unpool_fwd": 0.695e9, "unpool_bwd": 0.684e9}
-TAIL_TRAFFIC_BYTES = {"dense_fwd": 1.249e9, "dense_bwd": 2.514e9}
-TEXTURE_TRAFFIC_BYTES = {"texture_fwd": 3.396e9, "texture_bwd": 3.293e9}
+def build_id():
+    """Identity of the kernels being timed: hash over the sources the library is built from."""
+    import hashlib
+    h = hashlib.sha256()
+    csrc = os.path.join(ROOT, "picassoplus_amd", "csrc")
+    for name in sorted(os.listdir(csrc)):
+        if name.endswith((".hip", ".h", ".cpp")):
+            h.update(name.encode())
+            h.update(open(os.path.join(csrc, name), "rb").read())
+    return h.hexdigest()[:16]
+
+
+def measured_traffic(workload, variant, op):
+    """Bytes per launch of `op` from profiles/traffic.json, or None when the file is absent, holds another build's
+    figures or does not cover this workload variant."""
+    try:
+        tab = json.load(open(TRAFFIC_JSON))
+    except (OSError, ValueError):
+        return None
+    ent = tab.get(workload + ("+" + variant if variant else ""))
+    if not ent or ent.get("build_id") != build_id():
+        return None
+    return ent.get("bytes_per_launch", {}).get(op)
+
+
+def write_traffic(args):
+    """profiles/traffic.json (and a text summary beside it) from the two rocprofv3 counter runs of one workload."""
+    import csv, re, subprocess
+    def agg(path, counter):
+        out = {}
+        for r in csv.DictReader(open(path)):
+            if r["Counter_Name"] == counter:
+                name = re.sub(r"^void ", "", r["Kernel_Name"])
+                name = re.sub(r"\(.*$", "", name)
+                out.setdefault(name, []).append(float(r["Counter_Value"]))
+        return out
+    F, W = agg(args.traffic_from[0], "FETCH_SIZE"), agg(args.traffic_from[1], "WRITE_SIZE")
+    copy = [k for k in F if "copyBuffer" in k]
+    if not copy or copy[0] not in W:
+        sys.exit("--traffic-from: no device-copy kernel in the counter files (run bench.py with --copy-calibration)")
+    # the three 1 GiB copies dominate the copy kernel's total
+    fcal, wcal = sum(F[copy[0]]) / 3.0, sum(W[copy[0]]) / 3.0
+    ff, wf = 1048576.0 / fcal, 1048576.0 / wcal
+    per_kernel, ops = {}, {}
+    for op, pats in TRAFFIC_KERNELS[args.workload].items():
+        tot = 0.0
+        for pat in pats:
+            for k in sorted(set(F) | set(W)):
+                short = k.replace("pmesh::", "")
+                if re.match(pat, short) or re.search(pat, short):
+                    f = sum(F.get(k, [0])) / max(len(F.get(k, [0])), 1)
+                    w = sum(W.get(k, [0])) / max(len(W.get(k, [0])), 1)
+                    per_kernel[short] = (f, w, f * 1024 * ff, w * 1024 * wf)
+                    tot += f * 1024 * ff + w * 1024 * wf
+        ops[op] = tot
+    key = args.workload + ("+f2f-half" if args.f2f_half else "") + ("+bf16" if args.bf16_features else "")
+    try:
+        tab = json.load(open(TRAFFIC_JSON))
+    except (OSError, ValueError):
+        tab = {}
+    try:
+        git = subprocess.run(["git", "-C", ROOT, "rev-parse", "--short", "HEAD"], capture_output=True, text=True).stdout.strip()
+    except OSError:
+        git = ""
+    tab[key] = dict(build_id=build_id(), git_head_when_measured=git, scale_fetch=ff, scale_write=wf,
+                    bytes_per_launch={k: round(v) for k, v in ops.items()})
+    json.dump(tab, open(TRAFFIC_JSON, "w"), indent=1, sort_keys=True)
+    lines = ["HBM traffic per launch from rocprofv3 PMC, workload %s, MI355X, build %s" % (key, build_id()),
+             "commands (from /tmp, TMPDIR=/tmp), one counter per run, then the summary:",
+             "  rocprofv3 --pmc FETCH_SIZE -d <out> -o pmc --output-format csv -- python3 bench.py --workload %s --steps 2 --warmup 1 --no-cpu-baseline --copy-calibration" % args.workload,
+             "  rocprofv3 --pmc WRITE_SIZE -d <out> -o pmc --output-format csv -- python3 bench.py --workload %s --steps 2 --warmup 1 --no-cpu-baseline --copy-calibration" % args.workload,
+             "  python3 bench.py --workload %s --traffic-from <FETCH csv> <WRITE csv>" % args.workload,
+             "calibration: three 1 GiB device copies read %.0f KiB (FETCH_SIZE) and %.0f KiB (WRITE_SIZE) per copy -> scale factors %.3f and %.3f" % (fcal, wcal, ff, wf), "",
+             "%-44s %14s %14s %10s %10s" % ("kernel (mean per launch)", "FETCH_SIZE KiB", "WRITE_SIZE KiB", "read GB", "written GB")]
+    for k, (f, w, rb, wb) in per_kernel.items():
+        lines.append("%-44s %14.1f %14.1f %10.3f %10.3f" % (k[:44], f, w, rb / 1e9, wb / 1e9))
+    lines += ["", "per op (sum of its kernels), as written to profiles/traffic.json:"]
+    lines += ["  %-18s %.3f GB" % (k, v / 1e9) for k, v in ops.items()]
+    out = os.path.join(ROOT, "profiles", "%s_hbm_traffic_pmc.txt" % key.replace("+", "_"))
+    open(out, "w").write("\n".join(lines) + "\n")
+    print("\n".join(lines))
 
 
 class EventTimer:
@@ -215,12 +310,39 @@ def run_conv_layer(args, torch, kind):
                     frac_of_fp32_mfma_peak=ach / MFMA_F32_PEAK_TFLOPS)
     else:
         roof = dict(bound="hbm", achieved=bf[dom][0] / (dom_ms * 1e-3) / 1e9, peak=HBM_PEAK_GBS, unit="GB/s")
-    traffic = SCENE_TRAFFIC_BYTES.get(dom) if (kind == "scene" and args.scale == 1.0 and not args.f2f_half) else None
+    traffic = measured_traffic("scene", "f2f-half" if args.f2f_half else "", dom) if (kind == "scene" and args.scale == 1.0) else None
     roof.update(frac=roof["achieved"] / roof["peak"], traffic=traffic, kernel=dom, kernel_ms=dom_ms)
+    # adjacency of the step's index tensors, built cold (fresh tensors, nothing cached, range checks included): what
+    # a training loop that gets new index tensors with every batch pays per step on top of ms_per_step
+    from picassoplus_amd.mesh import topology
+    index_ms = {}
+    for label, build in (("vertex_csr", lambda: topology.vertex_csr(face.clone(), vt_map.clone(), d["nv"])),
+                         ("facet_order", lambda: topology.facet_order(cum.clone(), d["T"]))):
+        best = None
+        for _ in range(3):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            build()
+            torch.cuda.synchronize()
+            dt = (time.perf_counter() - t0) * 1e3
+            best = dt if best is None else min(best, dt)
+        index_ms[label] = best
+    if kind == "shapes":
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        topology.vertex_csr(face.clone(), None, d["nv"])
+        torch.cuda.synchronize()
+        index_ms["vertex_csr_inputs"] = (time.perf_counter() - t0) * 1e3
     ops_report = {k: dict(ms=per_op.get(k), gbps=bf[k][0] / (per_op[k] * 1e-3) / 1e9,
                           tflops=bf[k][1] / (per_op[k] * 1e-3) / 1e12) for k in ops if k in per_op}
     res = dict(value=d["nf"] / (ms * 1e-3) / 1e6, ms_per_step=ms, roofline=roof, ops=ops_report,
                hbm_gbps=total_bytes / (ms * 1e-3) / 1e9, hbm_frac=total_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+               index_build_ms=sum(index_ms.values()), index_build=index_ms,
+               dtype=("f32 in HBM; facet2facet products one fp16 piece per operand on v_mfma_f32_32x32x16_f16, f32 accumulate; "
+                      "facet2vertex f32" if args.f2f_half else
+                      "f32 in HBM; facet2facet products on v_mfma_f32_32x32x16_f16 with both operands split into two "
+                      "fp16 pieces (three piece products, about 22 significant bits), f32 accumulate; facet2vertex f32 "
+                      "(filter combination on v_mfma_f32_32x32x2_f32)"),
                config=dict(workload=name + ("_f2f-half-products" if args.f2f_half else ""), facets=d["nf"], vertices=d["nv"], texture_points=d["T"], channels=C,
                            sh_degree=L, meshes=int(len(d["mf_in"])), algorithmic_bytes=total_bytes))
     if not args.no_cpu_baseline:
@@ -333,7 +455,7 @@ def run_pool(args, torch):
                                      sample="the whole grid (%d vertices, %d channels), one pass of the six ops, %.1f s" % (nv, C, spent))
     return dict(value=nv / (ms * 1e-3) / 1e6, unit="Mvertices/s", ms_per_step=ms, **extra,
                 roofline=dict(bound="hbm", achieved=ach, peak=HBM_PEAK_GBS, unit="GB/s", frac=ach / HBM_PEAK_GBS,
-                              traffic=POOL_TRAFFIC_BYTES.get(dom), kernel=dom, kernel_ms=per_op[dom]),
+                              traffic=measured_traffic("pool", "", dom), kernel=dom, kernel_ms=per_op[dom]),
                 ops={k: dict(ms=per_op[k], gbps=nb[k] / (per_op[k] * 1e-3) / 1e9) for k in nb},
                 hbm_gbps=total / (ms * 1e-3) / 1e9, hbm_frac=total / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
                 config=dict(workload="plane1024_pool_max+avg+unpool_C128_fp32_fwd+bwd", vertices=nv, coarse=nvo, channels=C))
@@ -392,8 +514,10 @@ def run_tail(args, torch):
         extra["cpu_baseline"] = dict(value=rows / spent / 1e6, unit="Mrows/s", cores=torch.get_num_threads(), kind="port",
                                      sample="first %d of %d rows, one fwd+bwd pass, %.1f s" % (rows, N, spent))
     return dict(value=N / (ms * 1e-3) / 1e6, unit="Mrows/s", ms_per_step=ms, **extra,
+                dtype="f32 in HBM; products on v_mfma_f32_32x32x16_bf16 with both operands split exactly into three bf16 "
+                      "pieces (six piece products), f32 accumulate",
                 roofline=dict(bound="hbm", achieved=ach, peak=HBM_PEAK_GBS, unit="GB/s", frac=ach / HBM_PEAK_GBS,
-                              traffic=TAIL_TRAFFIC_BYTES.get(dom) if args.scale == 1.0 else None, kernel=dom,
+                              traffic=measured_traffic("tail", "", dom) if args.scale == 1.0 else None, kernel=dom,
                               kernel_ms=per_op[dom]),
                 ops={k: dict(ms=per_op[k], gbps=nb[k] / (per_op[k] * 1e-3) / 1e9,
                              tflops=fl[k] / (per_op[k] * 1e-3) / 1e12) for k in nb},
@@ -454,7 +578,7 @@ def run_texture(args, torch):
                                             % (len(d["mf_in"]), nf, nt, spent))
     return dict(value=d["nf"] / (ms * 1e-3) / 1e6, ms_per_step=ms, **extra,
                 roofline=dict(bound="hbm", achieved=ach, peak=HBM_PEAK_GBS, unit="GB/s", frac=ach / HBM_PEAK_GBS,
-                              traffic=TEXTURE_TRAFFIC_BYTES.get(dom) if args.scale == 1.0 else None, kernel=dom,
+                              traffic=measured_traffic("texture", "", dom) if args.scale == 1.0 else None, kernel=dom,
                               kernel_ms=per_op[dom]),
                 ops={k: dict(ms=per_op[k], gbps=bf[k][0] / (per_op[k] * 1e-3) / 1e9) for k in ops},
                 hbm_gbps=total / (ms * 1e-3) / 1e9, hbm_frac=total / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
@@ -564,6 +688,8 @@ def run_hierarchy(args, torch):
         roof = dict(bound="hbm", achieved=nbytes / (dom_ms * 1e-3) / 1e9, peak=HBM_PEAK_GBS, unit="GB/s")
     roof.update(frac=roof["achieved"] / roof["peak"], traffic=None, kernel="%s@level%d" % (dom, dl), kernel_ms=dom_ms)
     res = dict(value=lv[0]["nf"] / (ms * 1e-3) / 1e6, ms_per_step=ms, roofline=roof,
+               dtype="f32 in HBM; facet2facet products two fp16 pieces per operand, pointwise tails three bf16 pieces per "
+                     "operand, f32 accumulate; everything else f32",
                ops_ms_per_step={k: round(v, 4) for k, v in sorted(per_op.items())}, levels=report,
                config=dict(workload="grid%d_4levels_V2F+texture+F2F+F2V+pool+unpool_C32-256_L3_fp32_fwd+bwd" % cells,
                            facets=[d["nf"] for d in lv], vertices=[d["nv"] for d in lv] + [int(lv[-1]["vt_out"].shape[0])],
@@ -605,6 +731,9 @@ def cpu_baseline_block(d, C, L, torch):
 
 def main():
     args = parse()
+    if args.traffic_from:
+        write_traffic(args)
+        return
     if args.gpus != 1:
         print("bench.py measures one GPU: this path keeps whole meshes on one device and nothing here "
               "uses a second one; run with --gpus 1", file=sys.stderr)
@@ -638,7 +767,7 @@ def main():
     line = dict(metric="mesh-conv layer fwd+bwd throughput", value=res.pop("value"), unit=res.pop("unit", "Mfacets/s"),
                 n_gpus=1, steps=args.steps, warmup=args.warmup, ms_per_step=res.pop("ms_per_step"),
                 higher_is_better=True, scaling="weak", vs_baseline=None,
-                dtype="f16 products, f32 accumulate (f2f); f32 elsewhere" if args.f2f_half else "f32", data="synthetic")
+                dtype=res.pop("dtype", "f32"), data="synthetic", build_id=build_id())
     line.update(res)
     print(json.dumps(line))
 

@@ -746,7 +746,8 @@ def main():
         sys.exit(2)
     torch.cuda.set_device(0)
     if args.f2f_half:
-        os.environ["PMESH_F2F_HALF"] = "1"          # read by the library at every call
+        os.environ["PMESH_F2F_HALF"] = "1"
+        _lib.reload_options()                       # the library reads its switches once
     if args.workload == "pool":
         res = run_pool(args, torch)
     elif args.workload == "tail":

@@ -42,6 +42,10 @@ typedef void *pmesh_stream_t;
 int pmesh_abi_version(void);
 /* Message of the last failing call on the calling thread ("" if none). */
 const char *pmesh_last_error(void);
+/* The library reads its switches from the environment once, at its first call: PMESH_F2F_GENERIC, PMESH_F2F_BF16X3,
+ * PMESH_F2F_HALF, PMESH_F2V_VALU, PMESH_DENSE_FP32MFMA ("1" = set; they select other kernel families than the
+ * default for comparison).  pmesh_reload_options() reads them again.  No counterpart in the reference. */
+void pmesh_reload_options(void);
 
 /* ------------------------------------------------------------------ adjacency (CSR)
  * The reference scatters with float atomics and therefore needs no adjacency.  Here the
@@ -159,6 +163,9 @@ int pmesh_f2f_fwd(const float *texture, const float *filter, const float *bary_c
  * alone when only one gradient is wanted (the reference always computes both,
  * mesh_conv3d_gpu.cu:144-168). */
 size_t pmesh_f2f_bwd_workspace_bytes(int Cin, int Cout, int F);
+/* The same for a given number of facets: the partial filter gradients take one slice per group of facets, so a
+ * small mesh needs a fraction of the upper bound above (which holds for any Nf). */
+size_t pmesh_f2f_bwd_workspace_bytes_for(int64_t Nf, int Cin, int Cout, int F);
 int pmesh_f2f_bwd(const float *grad_output, const float *texture, const float *filter,
                   const float *bary_coeff, const int32_t *cum_texture, const int32_t *facet_order,
                   float *grad_texture, float *grad_filter, void *workspace, size_t workspace_bytes,

@@ -11,7 +11,7 @@ from ctypes import c_char_p, c_int, c_int64, c_size_t, c_void_p
 _HERE = os.path.dirname(os.path.abspath(__file__))
 # PICASSO_MESH_LIB points at an alternative build of the same ABI (kernel experiments)
 LIB_PATH = os.environ.get("PICASSO_MESH_LIB") or os.path.join(_HERE, "csrc", "libpicasso_mesh.so")
-ABI_VERSION = 11
+ABI_VERSION = 12
 
 P, I, L, Z = c_void_p, c_int, c_int64, c_size_t
 
@@ -36,6 +36,8 @@ SIGNATURES = {
     "pmesh_facet_order_workspace_bytes": (Z, [L]),
     "pmesh_build_facet_order": (I, [P, L, L, P, P, Z, P]),
     "pmesh_f2f_bwd_workspace_bytes": (Z, [I, I, I]),
+    "pmesh_f2f_bwd_workspace_bytes_for": (Z, [L, I, I, I]),
+    "pmesh_reload_options": (None, []),
     "pmesh_f2f_bwd": (I, [P, P, P, P, P, P, P, P, P, Z, L, L, I, I, I, P]),
     "pmesh_f2f_bwd_texture": (I, [P, P, P, P, P, P, P, Z, L, L, I, I, I, P]),
     "pmesh_f2f_bwd_filter": (I, [P, P, P, P, P, P, P, Z, L, L, I, I, I, P]),
@@ -112,6 +114,12 @@ def call(name, *args):
     if rc != 0:
         msg = lib.pmesh_last_error()
         raise RuntimeError("%s failed: %s" % (name, msg.decode() if msg else "unknown error"))
+
+
+def reload_options():
+    """Make the library read its PMESH_* switches from the environment again (it reads them once, at its first
+    call): for tests and benchmarks that change them inside one process."""
+    load().pmesh_reload_options()
 
 
 def query(name, *args):

@@ -26,6 +26,19 @@ void clear_error();
             return ::pmesh::fail("%s: kernel launch failed: %s", name, hipGetErrorString(e__)); \
     } while (0)
 
+// Switches that route an op to another kernel family than the default (tests compare the families; benchmarks time
+// the variants).  Read from the environment ONCE, at the first call into the library, and again only when
+// pmesh_reload_options() is called: PMESH_F2F_GENERIC, PMESH_F2F_BF16X3, PMESH_F2F_HALF, PMESH_F2V_VALU,
+// PMESH_DENSE_FP32MFMA (each "1" to set).
+struct Options {
+    bool f2f_generic;        // facet2facet on the shape-generic fp32-MFMA kernels
+    bool f2f_bf16x3;         // 16 coefficients: the three-piece bf16 kernels instead of the two-piece fp16 ones
+    bool f2f_half;           // 16 coefficients: one fp16 piece per operand (results within 1e-3)
+    bool f2v_valu;           // facet2vertex on the vector-ALU kernels
+    bool dense_fp32mfma;     // pointwise tail on the fp32 matrix instruction
+};
+const Options &options();
+
 // Every index the kernels compute must fit int32 element counts times channels in int64;
 // grids are 1-D and must stay below 2^31 workgroups.
 inline bool grid_ok(int64_t blocks) { return blocks >= 0 && blocks < (int64_t(1) << 31); }

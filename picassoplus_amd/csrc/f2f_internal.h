@@ -4,12 +4,6 @@
 
 namespace pmesh {
 
-// The fast path needs F == 16, Cin % 4 == 0 and 16-byte aligned texture / SH / filter arrays.
-bool f2f16_usable(const void *tex, const void *W, const void *sh, int Cin, int F);
-
-int f2f16_fwd(const float *tex, const float *W, const float *sh, const int *cum, float *out, int64_t T,
-              int64_t Nf, int Cin, int Cout, hipStream_t st);
-
 // The split-bf16 kernels (mesh_f2f16x3.hip) take any channel counts; they need F == 16 and 16-byte aligned
 // filter and SH arrays.  Texture rows are read 16 bytes at a time when Cin % 4 == 0 and the array is aligned,
 // element by element otherwise.
@@ -53,13 +47,6 @@ int f2f16x3_bwd_filter_partials(const float *gout, const float *tex, const float
                                  float *partial, int splits, int64_t T, int64_t Nf, int Cin, int Cout, hipStream_t st,
                                  const int *only_if = nullptr);
 
-
-int f2f16_bwd_texture(const float *gout, const float *W, const float *sh, const int *cum, float *gtex, int64_t T,
-                      int64_t Nf, int Cin, int Cout, hipStream_t st);
-
-// writes `splits` partial (Cout x Cin*16) blocks; the caller reduces them in split order
-int f2f16_bwd_filter_partials(const float *gout, const float *tex, const float *sh, const int *cum, float *partial,
-                              int splits, int64_t T, int64_t Nf, int Cin, int Cout, hipStream_t st);
 
 // Narrow filter gradient (mesh_f2f_narrow.hip): at most four input channels, F == 16.  `blocks` partial
 // gradients of Cout*Cin*16 floats are left in `partial` (blocks = f2f_narrow_blocks(Nf) <= kNarrowMaxBlocks).

@@ -602,12 +602,8 @@ static int rows_tiles(int Kpad, int C, int slab_weights)
     return nt;
 }
 
-// PMESH_DENSE_FP32MFMA=1 keeps the products on the fp32 matrix instruction (tests compare the two paths).
-static bool force_fp32_mfma()
-{
-    const char *e = getenv("PMESH_DENSE_FP32MFMA");
-    return e && e[0] == '1';
-}
+// the fp32 matrix instruction on request (tests compare the two paths)
+static bool force_fp32_mfma() { return options().dense_fp32mfma; }
 
 // Launch with as many workgroups as are resident at once (every tile is independent, so the count only
 // balances the load): a grid that needs a second round of workgroups would run that round at low occupancy.

@@ -327,13 +327,7 @@ static inline int filt_splits(int64_t Nf)
     return (int)s;
 }
 
-// PMESH_F2F_GENERIC=1 routes every shape through the shape-generic kernels of this file
-// (read on every call so that tests can flip it).
-static inline bool force_generic()
-{
-    const char *e = getenv("PMESH_F2F_GENERIC");
-    return e && e[0] == '1';
-}
+static inline bool force_generic() { return options().f2f_generic; }
 
 }  // namespace pmesh
 
@@ -345,27 +339,8 @@ using namespace pmesh;
     PM_REQUIRE((int64_t)Cin * F <= (1 << 24) && Cout <= (1 << 20), name ": dims too large");     \
     PM_REQUIRE(T >= 0 && Nf >= 0 && T <= INT32_MAX && Nf <= INT32_MAX, name ": bad sizes")
 
-// PMESH_F2F_FP32MFMA=1 keeps the 16-coefficient fast path on the fp32 matrix instructions
-// PMESH_F2F_BF16X3=1 keeps the three-piece bf16 kernels where the two-piece fp16 ones would run.
-static inline bool force_bf16x3()
-{
-    const char *e = getenv("PMESH_F2F_BF16X3");
-    return e && e[0] == '1';
-}
-
-// PMESH_F2F_HALF=1: the half-precision variant of the fp16 kernels (one fp16 piece per operand, one product, fp32
-// accumulation): results within 1e-3 of the largest output instead of 1e-5.
-static inline bool want_half()
-{
-    const char *e = getenv("PMESH_F2F_HALF");
-    return e && e[0] == '1';
-}
-
-static inline bool force_fp32_mfma()
-{
-    const char *e = getenv("PMESH_F2F_FP32MFMA");
-    return e && e[0] == '1';
-}
+static inline bool force_bf16x3() { return options().f2f_bf16x3; }
+static inline bool want_half() { return options().f2f_half; }
 
 extern "C" size_t pmesh_f2f_fwd_workspace_bytes(int Cin, int Cout, int F)
 {
@@ -382,18 +357,16 @@ extern "C" int pmesh_f2f_fwd(const float *texture, const float *filter, const fl
     if (Nf == 0) return 0;
     PM_REQUIRE(filter && cum_texture && output && (T == 0 || (texture && bary_coeff)), "f2f_fwd: null pointer");
     // the split-bf16 forward addresses texture elements with 32-bit offsets
-    if (!force_generic() && !force_fp32_mfma() && !force_bf16x3() && f2f_fwd_narrow_usable(Cin, F, bary_coeff))
+    if (!force_generic() && !force_bf16x3() && f2f_fwd_narrow_usable(Cin, F, bary_coeff))
         return f2f_fwd_narrow(texture, filter, bary_coeff, cum_texture, output, T, Nf, Cin, Cout, (hipStream_t)stream);
-    if (!force_generic() && !force_fp32_mfma() && !force_bf16x3() && f2f16x3_usable(filter, bary_coeff, F) &&
+    if (!force_generic() && !force_bf16x3() && f2f16x3_usable(filter, bary_coeff, F) &&
         T * Cin < (int64_t(1) << 31))
         return f2f16h2_fwd(texture, filter, bary_coeff, cum_texture, facet_order, output, workspace, workspace_bytes,
                            T, Nf, Cin, Cout, (hipStream_t)stream, want_half());
-    if (!force_generic() && !force_fp32_mfma() && f2f16x3_usable(filter, bary_coeff, F) &&
+    if (!force_generic() && f2f16x3_usable(filter, bary_coeff, F) &&
         T * Cin < (int64_t(1) << 31))
         return f2f16x3_fwd(texture, filter, bary_coeff, cum_texture, facet_order, output, workspace, workspace_bytes,
                            T, Nf, Cin, Cout, (hipStream_t)stream);
-    if (!force_generic() && f2f16_usable(texture, filter, bary_coeff, Cin, F))
-        return f2f16_fwd(texture, filter, bary_coeff, cum_texture, output, T, Nf, Cin, Cout, (hipStream_t)stream);
     const ChunkGeom cg = chunk_geom(Cin, F);
     const int64_t gx = ceil_div(Nf, 64), gy = ceil_div(Cout, 64);
     PM_REQUIRE(grid_ok(gx) && gy <= 65535, "f2f_fwd: grid too large");
@@ -403,14 +376,24 @@ extern "C" int pmesh_f2f_fwd(const float *texture, const float *filter, const fl
     return 0;
 }
 
-extern "C" size_t pmesh_f2f_bwd_workspace_bytes(int Cin, int Cout, int F)
+// the two halves run one after the other on a stream and share the workspace: partial filter gradients (as many
+// slices as this facet count makes), then 256 bytes for the overflow flag of the fp16 filter gradient
+static size_t f2f_bwd_ws(int64_t slices, int Cin, int Cout, int F)
 {
-    // the two halves run one after the other on a stream and share the workspace
-    // partial gradients, then 256 bytes for the overflow flag of the fp16 filter gradient
-    const size_t slices = f2f_narrow_usable(Cin, F) ? kNarrowMaxBlocks : kFiltMaxSplits;
-    const size_t filt = slices * Cout * Cin * F * sizeof(float) + 256;
+    const size_t filt = (size_t)slices * Cout * Cin * F * sizeof(float) + 256;
     const size_t tex = F == 16 ? f2f16x3_bwd_texture_workspace_bytes(Cin, Cout) : 0;
     return filt > tex ? filt : tex;
+}
+
+extern "C" size_t pmesh_f2f_bwd_workspace_bytes(int Cin, int Cout, int F)
+{
+    return f2f_bwd_ws(f2f_narrow_usable(Cin, F) ? kNarrowMaxBlocks : kFiltMaxSplits, Cin, Cout, F);
+}
+
+extern "C" size_t pmesh_f2f_bwd_workspace_bytes_for(int64_t Nf, int Cin, int Cout, int F)
+{
+    if (Nf < 0) Nf = 0;
+    return f2f_bwd_ws(f2f_narrow_usable(Cin, F) ? f2f_narrow_blocks(Nf) : filt_splits(Nf), Cin, Cout, F);
 }
 
 extern "C" int pmesh_f2f_bwd_texture(const float *grad_output, const float *filter, const float *bary_coeff,
@@ -424,17 +407,14 @@ extern "C" int pmesh_f2f_bwd_texture(const float *grad_output, const float *filt
     PM_REQUIRE(grad_output && filter && bary_coeff && cum_texture && grad_texture, "f2f_bwd_texture: null pointer");
     f2f_zero_tail_k<<<dim3(64), dim3(kBlock), 0, (hipStream_t)stream>>>(grad_texture, cum_texture, Nf, (int)T, Cin);
     PM_LAUNCHED("f2f_bwd_texture(tail)");
-    if (!force_generic() && !force_fp32_mfma() && !force_bf16x3() && f2f16x3_usable(filter, bary_coeff, F) &&
+    if (!force_generic() && !force_bf16x3() && f2f16x3_usable(filter, bary_coeff, F) &&
         f2f16x3_bwd_texture_usable(grad_output, Cout))
         return f2f16h2_bwd_texture(grad_output, filter, bary_coeff, cum_texture, facet_order, grad_texture, workspace,
                                    workspace_bytes, T, Nf, Cin, Cout, (hipStream_t)stream, want_half());
-    if (!force_generic() && !force_fp32_mfma() && f2f16x3_usable(filter, bary_coeff, F) &&
+    if (!force_generic() && f2f16x3_usable(filter, bary_coeff, F) &&
         f2f16x3_bwd_texture_usable(grad_output, Cout))
         return f2f16x3_bwd_texture(grad_output, filter, bary_coeff, cum_texture, facet_order, grad_texture, workspace,
                                    workspace_bytes, T, Nf, Cin, Cout, (hipStream_t)stream);
-    if (!force_generic() && f2f16_usable(grad_texture, filter, bary_coeff, Cin, F))
-        return f2f16_bwd_texture(grad_output, filter, bary_coeff, cum_texture, grad_texture, T, Nf, Cin, Cout,
-                                 (hipStream_t)stream);
     const ChunkGeom cg = chunk_geom(Cin, F);
     const int64_t gx = ceil_div(Nf, 64);
     PM_REQUIRE(grid_ok(gx), "f2f_bwd_texture: grid too large");
@@ -461,7 +441,7 @@ extern "C" int pmesh_f2f_bwd_filter(const float *grad_output, const float *textu
         return 0;
     }
     PM_REQUIRE(grad_output && texture && bary_coeff && cum_texture && workspace, "f2f_bwd_filter: null pointer");
-    if (!force_generic() && !force_fp32_mfma() && f2f_narrow_usable(Cin, F) && !(reinterpret_cast<uintptr_t>(bary_coeff) & 15u)) {
+    if (!force_generic() && f2f_narrow_usable(Cin, F) && !(reinterpret_cast<uintptr_t>(bary_coeff) & 15u)) {
         const int nb = f2f_narrow_blocks(Nf);
         PM_REQUIRE(workspace_bytes >= (size_t)nb * nW * sizeof(float), "f2f_bwd_filter: workspace too small (%zu bytes)",
                    workspace_bytes);
@@ -474,11 +454,11 @@ extern "C" int pmesh_f2f_bwd_filter(const float *grad_output, const float *textu
     const int S = filt_splits(Nf);
     PM_REQUIRE(workspace_bytes >= (size_t)S * nW * sizeof(float), "f2f_bwd_filter: workspace too small (%zu bytes)",
                workspace_bytes);
-    const bool x3 = !force_fp32_mfma() && f2f16x3_usable(bary_coeff, bary_coeff, F);
-    PM_REQUIRE(!x3 || workspace_bytes >= (size_t)S * nW * sizeof(float) + 256,
-               "f2f_bwd_filter: workspace too small (%zu bytes)", workspace_bytes);
-    if (!force_generic() && (x3 || f2f16_usable(texture, texture, bary_coeff, Cin, F))) {
-        if (x3 && !force_bf16x3()) {
+    const bool x3 = !force_generic() && f2f16x3_usable(bary_coeff, bary_coeff, F);
+    if (x3) {
+        PM_REQUIRE(workspace_bytes >= (size_t)S * nW * sizeof(float) + 256, "f2f_bwd_filter: workspace too small (%zu bytes)",
+                   workspace_bytes);
+        if (!force_bf16x3()) {
             // fp16 kernel first; if its scales did not hold, the guarded bf16 launch after it does the work again
             int *overflow = reinterpret_cast<int *>((float *)workspace + (size_t)S * nW);
             f2f_fill_zero_k<<<dim3(1), dim3(kBlock), 0, st>>>(reinterpret_cast<float *>(overflow), 1);
@@ -489,15 +469,10 @@ extern "C" int pmesh_f2f_bwd_filter(const float *grad_output, const float *textu
             if (int rc = f2f16x3_bwd_filter_partials(grad_output, texture, bary_coeff, cum_texture, facet_order,
                                                      (float *)workspace, S, T, Nf, Cin, Cout, st, overflow))
                 return rc;
-            f2f_reduce_k<<<dim3((unsigned)ceil_div(nW, 64)), dim3(kBlock), 0, st>>>((const float *)workspace, grad_filter, S, nW);
-            PM_LAUNCHED("f2f_bwd_filter(reduce)");
-            return 0;
+        } else if (int rc = f2f16x3_bwd_filter_partials(grad_output, texture, bary_coeff, cum_texture, facet_order,
+                                                        (float *)workspace, S, T, Nf, Cin, Cout, st)) {
+            return rc;
         }
-        int rc = !x3 ? f2f16_bwd_filter_partials(grad_output, texture, bary_coeff, cum_texture, (float *)workspace, S, T,
-                                                 Nf, Cin, Cout, st)
-                     : f2f16x3_bwd_filter_partials(grad_output, texture, bary_coeff, cum_texture, facet_order,
-                                                   (float *)workspace, S, T, Nf, Cin, Cout, st);
-        if (rc) return rc;
         f2f_reduce_k<<<dim3((unsigned)ceil_div(nW, 64)), dim3(kBlock), 0, st>>>((const float *)workspace, grad_filter, S, nW);
         PM_LAUNCHED("f2f_bwd_filter(reduce)");
         return 0;

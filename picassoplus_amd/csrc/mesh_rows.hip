@@ -870,12 +870,8 @@ static bool f2v_fast_ok(int C, int r, int K, std::initializer_list<const void *>
     return true;
 }
 
-// PMESH_F2V_VALU=1 keeps facet2vertex on the vector-ALU kernels (tests compare the two paths).
-static bool force_valu()
-{
-    const char *e = getenv("PMESH_F2V_VALU");
-    return e && e[0] == '1';
-}
+// the vector-ALU kernels on request (tests compare the two paths)
+static bool force_valu() { return options().f2v_valu; }
 
 int reduce_partials(const float *partial, float *out, int G, int n, hipStream_t st, size_t stride)
 {

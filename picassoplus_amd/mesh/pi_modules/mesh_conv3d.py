@@ -158,7 +158,7 @@ def facet2facet_backward_selected(grad_output, input, filter, bary_coeff, num_te
     with torch.cuda.device(dev):
         gin = torch.empty((T, Cin), dtype=F32, device=dev) if needs[0] else None
         gfilt = torch.empty((Cout, Cin, F), dtype=F32, device=dev) if needs[1] else None
-        nbytes = _lib.query("pmesh_f2f_bwd_workspace_bytes", Cin, Cout, F)
+        nbytes = _lib.query("pmesh_f2f_bwd_workspace_bytes_for", Nf, Cin, Cout, F)
         ws = workspace(nbytes, dev)
         st = stream_of(input)
         order = topology.facet_order(num_texture, T) if Nf else None

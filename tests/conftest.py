@@ -20,3 +20,19 @@ def cuda():
     from picassoplus_amd import _lib
     _lib.load()                      # fail loudly if the HIP library is missing
     return torch.device("cuda:0")
+
+
+@pytest.fixture
+def native_options(monkeypatch):
+    """Set PMESH_* switches for one test: the library reads them once, so it is told to read them again, and once
+    more when the test is over."""
+    from picassoplus_amd import _lib
+
+    def set_options(**env):
+        for k, v in env.items():
+            monkeypatch.setenv(k, v)
+        _lib.reload_options()
+
+    yield set_options
+    monkeypatch.undo()
+    _lib.reload_options()

@@ -35,13 +35,10 @@ def _case(seed, n, ci, co):
 
 
 @pytest.fixture(params=["split_bf16", "fp32_mfma"])
-def product_path(request, monkeypatch):
+def product_path(request, native_options):
     """The row kernels multiply on the bf16 matrix instruction with operands split in three (default) or, behind
-    PMESH_DENSE_FP32MFMA=1 (read at every call), on the fp32 matrix instruction."""
-    if request.param == "fp32_mfma":
-        monkeypatch.setenv("PMESH_DENSE_FP32MFMA", "1")
-    else:
-        monkeypatch.delenv("PMESH_DENSE_FP32MFMA", raising=False)
+    PMESH_DENSE_FP32MFMA=1, on the fp32 matrix instruction."""
+    native_options(PMESH_DENSE_FP32MFMA="1" if request.param == "fp32_mfma" else "0")
     return request.param
 
 

@@ -184,11 +184,11 @@ def test_texture_interpolation_rejects_bad_totals(cuda):
                                                 ("sphere3", 200, 1, 16, True), ("sphere2", 12, 3, 16, False),
                                                 ("room_small", 128, 2, 16, True), ("sphere3", 33, 1, 16, False)])
 @pytest.mark.parametrize("path", ["default", "valu"])
-def test_f2v_parity(cuda, monkeypatch, mesh, C, r, K, strided, path):
+def test_f2v_parity(cuda, native_options, mesh, C, r, K, strided, path):
     """default: matrix-core kernels where they apply (16 coefficients, at least 32 output channels);
     valu: the vector-ALU kernels for every shape."""
     say("case f2v", mesh, C, r, K, strided, path)
-    monkeypatch.setenv("PMESH_F2V_VALU", "1" if path == "valu" else "0")
+    native_options(PMESH_F2V_VALU="1" if path == "valu" else "0")
     v, f = mesh_case(mesh)
     rng = np.random.default_rng(11)
     nv, nf = v.shape[0], f.shape[0]
@@ -246,21 +246,19 @@ def test_f2v_unit_count_is_plain_scatter(cuda):
                                                 (50, 1, 8, 16, 3), (77, 2, 33, 16, 12),
                                                 (300, 128, 128, 16, 9), (260, 256, 256, 16, 9), (150, 128, 256, 16, 6),
                                                 (90, 256, 128, 16, 4), (200, 32, 32, 16, 9)])
-@pytest.mark.parametrize("path", ["default", "generic", "fp32mfma", "bf16x3", "half"])
-def test_f2f_parity(cuda, monkeypatch, nf, Cin, Cout, F, kmax, path):
-    """``generic`` forces the shape-generic kernels, ``fp32mfma`` the fp32-matrix-instruction variant of the
-    16-coefficient path and ``bf16x3`` the three-piece bf16 kernels, also where the two-piece fp16 kernels
-    (the default for 16 coefficients) apply; ``half`` their half-precision variant (one fp16 piece per operand, fp32
-    accumulation), held to 1e-3 of the largest reference value instead of 1e-5."""
+@pytest.mark.parametrize("path", ["default", "generic", "bf16x3", "half"])
+def test_f2f_parity(cuda, native_options, nf, Cin, Cout, F, kmax, path):
+    """``generic`` forces the shape-generic kernels (fp32 matrix instruction) and ``bf16x3`` the three-piece bf16
+    kernels, also where the two-piece fp16 kernels (the default for 16 coefficients) apply; ``half`` their
+    half-precision variant (one fp16 piece per operand, fp32 accumulation), held to 1e-3 of the largest reference
+    value instead of 1e-5."""
     say("case f2f", nf, Cin, Cout, F, kmax, path)
-    if path in ("generic", "fp32mfma") and not (F == 16 and Cin % 4 == 0):
+    if path == "generic" and F != 16:
         pytest.skip("shape already runs the generic kernels")
     if path in ("bf16x3", "half") and F != 16:
         pytest.skip("the split kernels need 16 coefficients")
-    monkeypatch.setenv("PMESH_F2F_HALF", "1" if path == "half" else "0")
-    monkeypatch.setenv("PMESH_F2F_GENERIC", "1" if path == "generic" else "0")
-    monkeypatch.setenv("PMESH_F2F_FP32MFMA", "1" if path == "fp32mfma" else "0")
-    monkeypatch.setenv("PMESH_F2F_BF16X3", "1" if path == "bf16x3" else "0")
+    native_options(PMESH_F2F_HALF="1" if path == "half" else "0", PMESH_F2F_GENERIC="1" if path == "generic" else "0",
+                   PMESH_F2F_BF16X3="1" if path == "bf16x3" else "0")
     rng = np.random.default_rng(13)
     counts, bary, owner = texture_case(rng, nf, kmax)
     cum = np.cumsum(counts).astype(np.int32)

@@ -30,7 +30,7 @@ def assert_close(y, ref, what, tol=TOL_F32):
 # sums, hence the floor.  factor = 2 for vertex2facet and facet2vertex.  facet2facet is held to 3: the reference adds
 # 16-term inner sums (over d) into each output, a blocked summation, while any matrix-core kernel runs ONE
 # accumulator through all Cin * 16 terms of a row; that order alone costs the float32 matrix instruction 3 to 3.5
-# times the reference order's error (the `generic` and `fp32mfma` paths, exact fp32 products), and the two-piece fp16
+# times the reference order's error (the `generic` path, exact fp32 products), and the two-piece fp16
 # kernels measure 1.1 to 2.6.
 F32_FLOOR = 2.0 ** -22
 

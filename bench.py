@@ -79,18 +79,20 @@ def build_conv_inputs(mesh, C, L, seed, tex_counts="area", Cin=None, r=1):
         mf_in=mesh["mf_in"], nv_in=mesh["nv_in"])
 
 
-def conv_bytes_flops(d, ops):
-    """Algorithmic HBM bytes / flops per op: every input read once, every output written once."""
+def conv_bytes_flops(d, ops, fb=4):
+    """Algorithmic HBM bytes / flops per op: every input read once, every output written once.  ``fb`` = bytes per
+    FEATURE value (texture rows, layer inputs / outputs and their gradients): 4, or 2 for the bf16-feature variant;
+    indices, SH coefficients, filters and filter gradients are 4 bytes in both."""
     Nf, Nv, T, C, B = d["nf"], d["nv"], d["T"], d["C"], d["B"]
     Ci, r = d["Cin"], d["r"]                    # F2F input channels; F2V depth multiplier (output width C * r)
     tab = {
-        "v2f_fwd": (4 * Nv * C + 12 * Nf + 4 * Nf * C, 6 * Nf * C),
-        "v2f_bwd": (4 * Nf * C + 12 * Nf + 8 * Nv * C, 12 * Nf * C),
-        "f2v_fwd": (4 * Nf * C + 4 * Nf * B + 12 * Nf + 8 * Nv + 4 * Nv * C * r, Nf * C * r * (2 * B + 7)),
-        "f2v_bwd": (4 * Nv * C * r + 8 * Nf * C + 4 * Nf * B + 12 * Nf + 8 * Nv, Nf * C * r * (4 * B + 12)),
-        "f2f_fwd": (4 * T * Ci + 4 * T * B + 4 * Nf + 4 * C * Ci * B + 4 * Nf * C, 2 * T * Ci * B + 2 * Nf * Ci * B * C),
-        "f2f_bwd_texture": (4 * Nf * C + 4 * T * B + 4 * Nf + 4 * C * Ci * B + 4 * T * Ci, 2 * Nf * Ci * B * C + 2 * T * Ci * B),
-        "f2f_bwd_filter": (4 * Nf * C + 4 * T * Ci + 4 * T * B + 4 * Nf + 4 * C * Ci * B, 2 * Nf * Ci * B * C + 2 * T * Ci * B),
+        "v2f_fwd": (fb * Nv * C + 12 * Nf + fb * Nf * C, 6 * Nf * C),
+        "v2f_bwd": (fb * Nf * C + 12 * Nf + 2 * fb * Nv * C, 12 * Nf * C),
+        "f2v_fwd": (fb * Nf * C + 4 * Nf * B + 12 * Nf + 8 * Nv + fb * Nv * C * r, Nf * C * r * (2 * B + 7)),
+        "f2v_bwd": (fb * Nv * C * r + 2 * fb * Nf * C + 4 * Nf * B + 12 * Nf + 8 * Nv, Nf * C * r * (4 * B + 12)),
+        "f2f_fwd": (fb * T * Ci + 4 * T * B + 4 * Nf + 4 * C * Ci * B + fb * Nf * C, 2 * T * Ci * B + 2 * Nf * Ci * B * C),
+        "f2f_bwd_texture": (fb * Nf * C + 4 * T * B + 4 * Nf + 4 * C * Ci * B + fb * T * Ci, 2 * Nf * Ci * B * C + 2 * T * Ci * B),
+        "f2f_bwd_filter": (fb * Nf * C + fb * T * Ci + 4 * T * B + 4 * Nf + 4 * C * Ci * B, 2 * Nf * Ci * B * C + 2 * T * Ci * B),
         # texture points interpolated from vertex features, with their basis values (forward) / transposed (backward)
         "texture_fwd": (4 * Nv * C + 16 * Nf + 12 * T + 4 * T * C + 4 * T * B, 5 * T * C + 60 * T),
         "texture_bwd": (4 * T * C + 12 * T + 16 * Nf + 4 * Nv * C, 6 * T * C),
@@ -267,6 +269,12 @@ def run_conv_layer(args, torch, kind):
     coeff = sph_harm_values(t(d["normal"]), L)
     w_f2f, w_f2v, w_v2f = t(d["w_f2f"]), t(d["w_f2v"]), t(d["w_v2f"])
     gy = torch.randn(d["nv"], C * r, device=dev, generator=torch.Generator(device=dev).manual_seed(1))
+    bf16 = bool(args.bf16_features)
+    if bf16:
+        if kind != "scene":
+            sys.exit("--bf16-features is a variant of the scene workload")
+        tex, gy = tex.to(torch.bfloat16), gy.to(torch.bfloat16)
+        name = "scene8x300k_F2F+F2V_C64_L3_bf16-features_fwd+bwd"
     tex.requires_grad_(True); w_f2f.requires_grad_(True); w_f2v.requires_grad_(True)
     if kind == "shapes":
         x.requires_grad_(True); w_v2f.requires_grad_(True)
@@ -296,21 +304,22 @@ def run_conv_layer(args, torch, kind):
     timer.on = False
     _lib.set_call_hook(None)
     ms = (t1 - t0) * 1e3 / args.steps
-    per_op = timer.summary()
-    bf = conv_bytes_flops(d, ops)
+    per_op = {k.replace("_bf16", ""): v for k, v in timer.summary().items()}
+    bf = conv_bytes_flops(d, ops, 2 if bf16 else 4)
     total_bytes = sum(b for b, _ in bf.values())
     dom = max(ops, key=lambda k: per_op.get(k, 0.0))
     dom_ms = per_op[dom]
     if dom.startswith("f2f") and Cin >= 16:
         ach = bf[dom][1] / (dom_ms * 1e-3) / 1e12
-        pieces = 1 if args.f2f_half else F2F_PIECE_PRODUCTS
+        pieces = 1 if (args.f2f_half or bf16) else F2F_PIECE_PRODUCTS
         roof = dict(bound="mfma", achieved=ach, peak=MFMA_F16_PEAK_TFLOPS / pieces, unit="TFLOP/s",
-                    peak_basis="fp16 dense MFMA 2500 TFLOP/s, one product per element (half-precision variant)" if args.f2f_half
+                    peak_basis="fp16 dense MFMA 2500 TFLOP/s, one product per element (reduced-precision variant)" if pieces == 1
                     else "fp16 dense MFMA 2500 TFLOP/s / 3 piece products per fp32-accurate product",
                     frac_of_fp32_mfma_peak=ach / MFMA_F32_PEAK_TFLOPS)
     else:
         roof = dict(bound="hbm", achieved=bf[dom][0] / (dom_ms * 1e-3) / 1e9, peak=HBM_PEAK_GBS, unit="GB/s")
-    traffic = measured_traffic("scene", "f2f-half" if args.f2f_half else "", dom) if (kind == "scene" and args.scale == 1.0) else None
+    traffic = (measured_traffic("scene", "bf16" if bf16 else "f2f-half" if args.f2f_half else "", dom)
+               if (kind == "scene" and args.scale == 1.0) else None)
     roof.update(frac=roof["achieved"] / roof["peak"], traffic=traffic, kernel=dom, kernel_ms=dom_ms)
     # adjacency of the step's index tensors, built cold (fresh tensors, nothing cached, range checks included): what
     # a training loop that gets new index tensors with every batch pays per step on top of ms_per_step
@@ -338,12 +347,15 @@ def run_conv_layer(args, torch, kind):
     res = dict(value=d["nf"] / (ms * 1e-3) / 1e6, ms_per_step=ms, roofline=roof, ops=ops_report,
                hbm_gbps=total_bytes / (ms * 1e-3) / 1e9, hbm_frac=total_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
                index_build_ms=sum(index_ms.values()), index_build=index_ms,
-               dtype=("f32 in HBM; facet2facet products one fp16 piece per operand on v_mfma_f32_32x32x16_f16, f32 accumulate; "
+               dtype=("bf16 features in HBM (texture rows, layer outputs, their gradients), f32 filters and coefficients; "
+                      "facet2facet products one fp16 piece per operand on v_mfma_f32_32x32x16_f16, every sum accumulated in f32"
+                      if bf16 else
+                      "f32 in HBM; facet2facet products one fp16 piece per operand on v_mfma_f32_32x32x16_f16, f32 accumulate; "
                       "facet2vertex f32" if args.f2f_half else
                       "f32 in HBM; facet2facet products on v_mfma_f32_32x32x16_f16 with both operands split into two "
                       "fp16 pieces (three piece products, about 22 significant bits), f32 accumulate; facet2vertex f32 "
                       "(filter combination on v_mfma_f32_32x32x2_f32)"),
-               config=dict(workload=name + ("_f2f-half-products" if args.f2f_half else ""), facets=d["nf"], vertices=d["nv"], texture_points=d["T"], channels=C,
+               config=dict(workload=name + ("_f2f-half-products" if args.f2f_half and not bf16 else ""), facets=d["nf"], vertices=d["nv"], texture_points=d["T"], channels=C,
                            sh_degree=L, meshes=int(len(d["mf_in"])), algorithmic_bytes=total_bytes))
     if not args.no_cpu_baseline:
         res["cpu_baseline"] = cpu_baseline_conv(d, kind, torch)

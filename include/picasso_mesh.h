@@ -179,6 +179,38 @@ int pmesh_f2f_bwd_filter(const float *grad_output, const float *texture, const f
                          void *workspace, size_t workspace_bytes, int64_t T, int64_t Nf, int Cin,
                          int Cout, int F, pmesh_stream_t stream);
 
+/* ------------------------------------------------------------------ features in bf16 (reduced-precision variant)
+ * No counterpart in the reference, which computes in float32 throughout.  The convolutions of a layer with the
+ * FEATURE tensors -- texture rows, layer inputs / outputs and their gradients -- kept in bf16 in HBM (uint16_t here:
+ * the upper half of the float32 bit pattern, rounded to nearest even on store).  Filters, SH coefficients and filter
+ * gradients stay float32; every sum is accumulated in float32; the facet2facet products take one fp16 piece per
+ * operand (exact power-of-two scales as in the float32 path).  Results agree with the float64 evaluation of the same
+ * bf16-rounded inputs within 1e-3 of the largest output before the final rounding to bf16.
+ * Shapes: facet2facet F = 16, Cin % 4 == 0, Cout % 8 == 0; facet2vertex K = 16, C * r >= 32, r = 1 or 2.  Other
+ * arguments, workspaces and the facet order are those of the float32 entry points of the same name, except the
+ * backward workspace: pmesh_f2f_bwd_bf16_workspace_bytes (with more than 64 output channels the texture gradient
+ * accumulates its blocks of 64 channels in a float32 copy of grad_texture inside the workspace). */
+size_t pmesh_f2f_bwd_bf16_workspace_bytes(int64_t T, int64_t Nf, int Cin, int Cout, int F);
+int pmesh_f2f_fwd_bf16(const uint16_t *texture, const float *filter, const float *bary_coeff,
+                       const int32_t *cum_texture, const int32_t *facet_order, uint16_t *output, void *workspace,
+                       size_t workspace_bytes, int64_t T, int64_t Nf, int Cin, int Cout, int F,
+                       pmesh_stream_t stream);
+int pmesh_f2f_bwd_texture_bf16(const uint16_t *grad_output, const float *filter, const float *bary_coeff,
+                               const int32_t *cum_texture, const int32_t *facet_order, uint16_t *grad_texture,
+                               void *workspace, size_t workspace_bytes, int64_t T, int64_t Nf, int Cin, int Cout,
+                               int F, pmesh_stream_t stream);
+int pmesh_f2f_bwd_filter_bf16(const uint16_t *grad_output, const uint16_t *texture, const float *bary_coeff,
+                              const int32_t *cum_texture, const int32_t *facet_order, float *grad_filter,
+                              void *workspace, size_t workspace_bytes, int64_t T, int64_t Nf, int Cin, int Cout,
+                              int F, pmesh_stream_t stream);
+int pmesh_f2v_fwd_bf16(const uint16_t *input, const float *filter, const float *coeff, const int32_t *nf_count,
+                       const int32_t *rowptr, const int32_t *colidx, uint16_t *output, int64_t Nf, int64_t NvOut,
+                       int C, int r, int K, pmesh_stream_t stream);
+int pmesh_f2v_bwd_bf16(const uint16_t *grad_output, const uint16_t *input, const float *filter, const float *coeff,
+                       const int32_t *face, const int32_t *nf_count, const int32_t *vt_map, uint16_t *grad_input,
+                       float *grad_filter, void *workspace, size_t workspace_bytes, int64_t Nf, int64_t NvIn,
+                       int64_t NvOut, int C, int r, int K, pmesh_stream_t stream);
+
 /* ------------------------------------------------------------------ mesh pooling
  * replaces max_forward / max_backward / avg_forward / avg_backward
  * (mesh_pool3d.cpp:29-148).  rowptr/members: cluster CSR of (vt_replace, vt_map).

@@ -307,14 +307,15 @@ __global__ __launch_bounds__(kBlock) void f2f_fill_zero_k(float *__restrict__ p,
 }
 
 // rows of grad_texture past the last facet's segment belong to no facet: clear them
-__global__ __launch_bounds__(kBlock) void f2f_zero_tail_k(float *__restrict__ gtex, const int *__restrict__ cum,
+template <typename TIO>
+__global__ __launch_bounds__(kBlock) void f2f_zero_tail_k(TIO *__restrict__ gtex, const int *__restrict__ cum,
                                                           int64_t Nf, int T, int Cin)
 {
     int last = cum[Nf - 1];
     last = last < 0 ? 0 : (last > T ? T : last);
     const int64_t n = (int64_t)(T - last) * Cin;
-    float *p = gtex + (int64_t)last * Cin;
-    for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (int64_t)gridDim.x * kBlock) p[i] = 0.f;
+    TIO *p = gtex + (int64_t)last * Cin;
+    for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (int64_t)gridDim.x * kBlock) p[i] = TIO(0);
 }
 
 constexpr int kFiltMaxSplits = 256;
@@ -405,7 +406,7 @@ extern "C" int pmesh_f2f_bwd_texture(const float *grad_output, const float *filt
     PM_F2F_DIMS("f2f_bwd_texture");
     if (Nf == 0 || T == 0) return 0;
     PM_REQUIRE(grad_output && filter && bary_coeff && cum_texture && grad_texture, "f2f_bwd_texture: null pointer");
-    f2f_zero_tail_k<<<dim3(64), dim3(kBlock), 0, (hipStream_t)stream>>>(grad_texture, cum_texture, Nf, (int)T, Cin);
+    f2f_zero_tail_k<float><<<dim3(64), dim3(kBlock), 0, (hipStream_t)stream>>>(grad_texture, cum_texture, Nf, (int)T, Cin);
     PM_LAUNCHED("f2f_bwd_texture(tail)");
     if (!force_generic() && !force_bf16x3() && f2f16x3_usable(filter, bary_coeff, F) &&
         f2f16x3_bwd_texture_usable(grad_output, Cout))
@@ -499,4 +500,83 @@ extern "C" int pmesh_f2f_bwd(const float *grad_output, const float *texture, con
     if (rc) return rc;
     return pmesh_f2f_bwd_filter(grad_output, texture, bary_coeff, cum_texture, facet_order, grad_filter, workspace,
                                 workspace_bytes, T, Nf, Cin, Cout, F, stream);
+}
+
+// ---- features in bf16 (the reduced-precision variant): 16 coefficients only, one fp16 product per element
+#define PM_F2F_BF16(name)                                                                                          \
+    PM_F2F_DIMS(name);                                                                                             \
+    PM_REQUIRE(F == 16, name ": bf16 features are implemented for 16 coefficients (SH degree 3), got F=%d", F);    \
+    PM_REQUIRE(!(Cin & 3) && !(Cout & 7), name ": bf16 features need Cin %% 4 == 0 and Cout %% 8 == 0 (Cin=%d Cout=%d)", Cin, Cout)
+
+extern "C" size_t pmesh_f2f_bwd_bf16_workspace_bytes(int64_t T, int64_t Nf, int Cin, int Cout, int F)
+{
+    if (T < 0) T = 0;
+    const size_t filt = pmesh_f2f_bwd_workspace_bytes_for(Nf, Cin, Cout, F);
+    const size_t tex = f2f16h2_bwd_texture_bf16_workspace_bytes(T, Cin, Cout);
+    return filt > tex ? filt : tex;
+}
+
+extern "C" int pmesh_f2f_fwd_bf16(const uint16_t *texture, const float *filter, const float *bary_coeff,
+                                  const int32_t *cum_texture, const int32_t *facet_order, uint16_t *output,
+                                  void *workspace, size_t workspace_bytes, int64_t T, int64_t Nf, int Cin, int Cout,
+                                  int F, pmesh_stream_t stream)
+{
+    clear_error();
+    PM_F2F_BF16("f2f_fwd_bf16");
+    if (Nf == 0) return 0;
+    PM_REQUIRE(filter && cum_texture && output && (T == 0 || (texture && bary_coeff)), "f2f_fwd_bf16: null pointer");
+    PM_REQUIRE(f2f16x3_usable(filter, bary_coeff, F), "f2f_fwd_bf16: filter and bary_coeff must be 16-byte aligned");
+    return f2f16h2_fwd(texture, filter, bary_coeff, cum_texture, facet_order, output, workspace, workspace_bytes, T, Nf,
+                       Cin, Cout, (hipStream_t)stream, true, true);
+}
+
+extern "C" int pmesh_f2f_bwd_texture_bf16(const uint16_t *grad_output, const float *filter, const float *bary_coeff,
+                                          const int32_t *cum_texture, const int32_t *facet_order,
+                                          uint16_t *grad_texture, void *workspace, size_t workspace_bytes, int64_t T,
+                                          int64_t Nf, int Cin, int Cout, int F, pmesh_stream_t stream)
+{
+    clear_error();
+    PM_F2F_BF16("f2f_bwd_texture_bf16");
+    if (Nf == 0 || T == 0) return 0;
+    PM_REQUIRE(grad_output && filter && bary_coeff && cum_texture && grad_texture, "f2f_bwd_texture_bf16: null pointer");
+    PM_REQUIRE(f2f16x3_usable(filter, bary_coeff, F), "f2f_bwd_texture_bf16: filter and bary_coeff must be 16-byte aligned");
+    f2f_zero_tail_k<uint16_t><<<dim3(64), dim3(kBlock), 0, (hipStream_t)stream>>>(grad_texture, cum_texture, Nf, (int)T, Cin);
+    PM_LAUNCHED("f2f_bwd_texture_bf16(tail)");
+    return f2f16h2_bwd_texture(grad_output, filter, bary_coeff, cum_texture, facet_order, grad_texture, workspace,
+                               workspace_bytes, T, Nf, Cin, Cout, (hipStream_t)stream, true, true);
+}
+
+extern "C" int pmesh_f2f_bwd_filter_bf16(const uint16_t *grad_output, const uint16_t *texture, const float *bary_coeff,
+                                         const int32_t *cum_texture, const int32_t *facet_order, float *grad_filter,
+                                         void *workspace, size_t workspace_bytes, int64_t T, int64_t Nf, int Cin,
+                                         int Cout, int F, pmesh_stream_t stream)
+{
+    clear_error();
+    PM_F2F_BF16("f2f_bwd_filter_bf16");
+    PM_REQUIRE(grad_filter, "f2f_bwd_filter_bf16: null grad_filter");
+    hipStream_t st = (hipStream_t)stream;
+    const int64_t nW = (int64_t)Cout * Cin * F;
+    if (Nf == 0 || T == 0) {
+        f2f_fill_zero_k<<<dim3((unsigned)ceil_div(nW, kBlock)), dim3(kBlock), 0, st>>>(grad_filter, nW);
+        PM_LAUNCHED("f2f_bwd_filter_bf16(fill)");
+        return 0;
+    }
+    PM_REQUIRE(grad_output && texture && bary_coeff && cum_texture && workspace, "f2f_bwd_filter_bf16: null pointer");
+    PM_REQUIRE(!(reinterpret_cast<uintptr_t>(bary_coeff) & 15u), "f2f_bwd_filter_bf16: bary_coeff must be 16-byte aligned");
+    const int S = filt_splits(Nf);
+    PM_REQUIRE(workspace_bytes >= (size_t)S * nW * sizeof(float) + 256, "f2f_bwd_filter_bf16: workspace too small (%zu bytes)",
+               workspace_bytes);
+    // as in pmesh_f2f_bwd_filter: the fp16 kernel, then the guarded bf16-product launch if its scales did not hold
+    int *overflow = reinterpret_cast<int *>((float *)workspace + (size_t)S * nW);
+    f2f_fill_zero_k<<<dim3(1), dim3(kBlock), 0, st>>>(reinterpret_cast<float *>(overflow), 1);
+    PM_LAUNCHED("f2f_bwd_filter_bf16(flag)");
+    if (int rc = f2f16h2_bwd_filter_partials(grad_output, texture, bary_coeff, cum_texture, facet_order, (float *)workspace,
+                                             overflow, S, T, Nf, Cin, Cout, st, true, true))
+        return rc;
+    if (int rc = f2f16x3_bwd_filter_partials(grad_output, texture, bary_coeff, cum_texture, facet_order, (float *)workspace,
+                                             S, T, Nf, Cin, Cout, st, overflow, true))
+        return rc;
+    f2f_reduce_k<<<dim3((unsigned)ceil_div(nW, 64)), dim3(kBlock), 0, st>>>((const float *)workspace, grad_filter, S, nW);
+    PM_LAUNCHED("f2f_bwd_filter_bf16(reduce)");
+    return 0;
 }

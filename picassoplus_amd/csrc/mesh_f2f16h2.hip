@@ -48,6 +48,112 @@ template <bool VEC> __device__ __forceinline__ float4 hld4_row(const float *p, i
     r.w = n > 3 ? p[3] : 0.f;
     return r;
 }
+// Features kept in bf16 in HBM (the reduced-precision variant): rows of bf16 values, converted on load and
+// rounded to nearest even on store; the arithmetic in between is the one-product fp16 path with fp32 accumulation.
+typedef unsigned short bf16_t;
+__device__ __forceinline__ float bf16_lo(unsigned u) { return __builtin_bit_cast(float, u << 16); }
+__device__ __forceinline__ float bf16_hi(unsigned u) { return __builtin_bit_cast(float, u & 0xFFFF0000u); }
+__device__ __forceinline__ unsigned pack2_bf16(float a, float b)              // a in the low half
+{
+    unsigned r;
+    asm("v_cvt_pk_bf16_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+    return r;
+}
+__device__ __forceinline__ float4 hld4(const bf16_t *p)
+{
+    const uint2 u = *reinterpret_cast<const uint2 *>(p);
+    return make_float4(bf16_lo(u.x), bf16_hi(u.x), bf16_lo(u.y), bf16_hi(u.y));
+}
+template <bool VEC> __device__ __forceinline__ float4 hld4_row(const bf16_t *p, int n)
+{
+    if constexpr (VEC) return n > 0 ? hld4(p) : make_float4(0.f, 0.f, 0.f, 0.f);
+    float4 r;
+    r.x = n > 0 ? bf16_lo(p[0]) : 0.f;
+    r.y = n > 1 ? bf16_lo(p[1]) : 0.f;
+    r.z = n > 2 ? bf16_lo(p[2]) : 0.f;
+    r.w = n > 3 ? bf16_lo(p[3]) : 0.f;
+    return r;
+}
+// eight consecutive values of a row (16-byte aligned for bf16, two 16-byte loads for float)
+__device__ __forceinline__ void hld8(const float *p, float4 &u, float4 &v) { u = hld4(p); v = hld4(p + 4); }
+__device__ __forceinline__ void hld8(const bf16_t *p, float4 &u, float4 &v)
+{
+    const uint4 w = *reinterpret_cast<const uint4 *>(p);
+    u = make_float4(bf16_lo(w.x), bf16_hi(w.x), bf16_lo(w.y), bf16_hi(w.y));
+    v = make_float4(bf16_lo(w.z), bf16_hi(w.z), bf16_lo(w.w), bf16_hi(w.w));
+}
+__device__ __forceinline__ float hld1(const float *p) { return *p; }
+// two-byte accesses are slow on this memory path: a single bf16 value is read as the aligned 4 bytes that hold it
+// (rows have an even number of values, neighbouring lanes share the word) ...
+__device__ __forceinline__ float hld1(const bf16_t *p) { return bf16_lo(*p); }
+// element `idx` of an array (even row lengths, 4-byte aligned base), in two steps: the fetch of the word that holds
+// it, and its conversion once all fetches of a batch are out (arithmetic right behind a conditional fetch makes the
+// wavefront wait for that fetch on the spot)
+__device__ __forceinline__ unsigned hld_raw(const float *base, int64_t idx) { return reinterpret_cast<const unsigned *>(base)[idx]; }
+__device__ __forceinline__ unsigned hld_raw(const bf16_t *base, int64_t idx) { return reinterpret_cast<const unsigned *>(base)[idx >> 1]; }
+__device__ __forceinline__ float hcvt_raw(unsigned w, int, float) { return __builtin_bit_cast(float, w); }
+__device__ __forceinline__ float hcvt_raw(unsigned w, int odd, bf16_t) { return odd ? bf16_hi(w) : bf16_lo(w); }
+__device__ __forceinline__ void hst1(float *p, float v) { *p = v; }
+__device__ __forceinline__ void hst1(bf16_t *p, float v) { *p = (bf16_t)(pack2_bf16(v, 0.f) & 0xFFFFu); }
+// ... and neighbouring lanes that hold neighbouring values p[0], p[1] (the even lane the first) write them as one
+// 4-byte store.  Every lane calls this; `ok` says whether the pair is stored.
+__device__ __forceinline__ void hst1_pair(float *p, float v, bool ok, int lane)
+{
+    (void)lane;
+    if (ok) *p = v;
+}
+__device__ __forceinline__ void hst1_pair(bf16_t *p, float v, bool ok, int lane)
+{
+    const float nb = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));
+    if (ok && !(lane & 1)) *reinterpret_cast<unsigned *>(p) = pack2_bf16(v, nb);
+}
+__device__ __forceinline__ void hst4(float *p, const float4 &v) { *reinterpret_cast<float4 *>(p) = v; }
+__device__ __forceinline__ void hst4(bf16_t *p, const float4 &v)
+{
+    *reinterpret_cast<uint2 *>(p) = make_uint2(pack2_bf16(v.x, v.y), pack2_bf16(v.z, v.w));
+}
+
+// What a conditional fetch of four consecutive channels leaves in registers, and its conversion to four floats.  The
+// two are separate because arithmetic right behind a conditional fetch makes the wavefront wait for that fetch on the
+// spot: all fetches of a batch go out first, the conversions follow.
+template <typename TIO> struct HRaw4;
+template <> struct HRaw4<float> { float4 v; };
+template <> struct HRaw4<bf16_t> { uint2 v; };
+template <bool VEC> __device__ __forceinline__ HRaw4<float> hld4_raw(const float *p, int n)
+{
+    HRaw4<float> r;
+    r.v = hld4_row<VEC>(p, n);
+    return r;
+}
+template <bool VEC> __device__ __forceinline__ HRaw4<bf16_t> hld4_raw(const bf16_t *p, int n)
+{
+    HRaw4<bf16_t> r;
+    if constexpr (VEC) {
+        r.v = n > 0 ? *reinterpret_cast<const uint2 *>(p) : make_uint2(0u, 0u);
+    } else {
+        r.v.x = (n > 0 ? (unsigned)p[0] : 0u) | (n > 1 ? (unsigned)p[1] << 16 : 0u);
+        r.v.y = (n > 2 ? (unsigned)p[2] : 0u) | (n > 3 ? (unsigned)p[3] << 16 : 0u);
+    }
+    return r;
+}
+__device__ __forceinline__ HRaw4<float> hraw_zero(float)
+{
+    HRaw4<float> r;
+    r.v = make_float4(0.f, 0.f, 0.f, 0.f);
+    return r;
+}
+__device__ __forceinline__ HRaw4<bf16_t> hraw_zero(bf16_t)
+{
+    HRaw4<bf16_t> r;
+    r.v = make_uint2(0u, 0u);
+    return r;
+}
+__device__ __forceinline__ float4 hcvt4(const HRaw4<float> &r) { return r.v; }
+__device__ __forceinline__ float4 hcvt4(const HRaw4<bf16_t> &r)
+{
+    return make_float4(bf16_lo(r.v.x), bf16_hi(r.v.x), bf16_lo(r.v.y), bf16_hi(r.v.y));
+}
+
 __device__ __forceinline__ float absmax4(const float4 &v, float m)
 {
     return fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fmaxf(fabsf(v.z), fabsf(v.w)), m));
@@ -217,8 +323,8 @@ __device__ __forceinline__ void hw_chunk_to_lds(const u32x4 *__restrict__ Wp, in
 // One pass over all input channels for up to KW texture points per facet.  shs = alpha_f / K_f, the factor on
 // the SH values of my facet; slim / tlim = largest |SH value| of my facet / |texture value| of the rows I fetch
 // that the scale allows for.
-template <int KW, bool TVEC, bool HALF>
-__device__ __forceinline__ void h2_sweep(const float *__restrict__ tex, const u32x4 *__restrict__ Wp,
+template <int KW, bool TVEC, bool HALF, typename TIO>
+__device__ __forceinline__ void h2_sweep(const TIO *__restrict__ tex, const u32x4 *__restrict__ Wp,
                                          const float *__restrict__ sh, u32x4 *Ws, float *slab, f32x16 (&acc)[2],
                                          int kbase, int Ks, float shs, float slim, float tlim, bool &viol,
                                          const int *s_k0, const int *s_K, int sweep, int Cin, int NT, int nt0, int nblk,
@@ -249,11 +355,11 @@ __device__ __forceinline__ void h2_sweep(const float *__restrict__ tex, const u3
         ldok[i] = kk < s_K[slot];
         ldoff[i] = (unsigned)(s_k0[slot] + (ldok[i] ? kk : 0)) * (unsigned)Cin + cg4;
     }
-    float4 pf[KW];
+    HRaw4<TIO> pf[KW];
     auto fetch_group = [&](int g) {
 #pragma unroll
         for (int i = 0; i < KW; ++i)
-            pf[i] = ldok[i] ? hld4_row<TVEC>(tex + (ldoff[i] + 8 * g), Cin - (8 * g + cg4)) : make_float4(0.f, 0.f, 0.f, 0.f);
+            pf[i] = ldok[i] ? hld4_raw<TVEC>(tex + (ldoff[i] + 8 * g), Cin - (8 * g + cg4)) : hraw_zero(TIO());
     };
     // values past the limits the facet's scale was chosen for are recorded, not acted on here
     viol |= smx > slim;
@@ -262,8 +368,9 @@ __device__ __forceinline__ void h2_sweep(const float *__restrict__ tex, const u3
 #pragma unroll
         for (int i = 0; i < KW; ++i) {
             float *q = dst + (i * 8 + cg4) * 32 + (lane >> 1);
-            q[0] = pf[i].x; q[32] = pf[i].y; q[64] = pf[i].z; q[96] = pf[i].w;
-            m = absmax4(pf[i], m);
+            const float4 pv = hcvt4(pf[i]);
+            q[0] = pv.x; q[32] = pv.y; q[64] = pv.z; q[96] = pv.w;
+            m = absmax4(pv, m);
         }
         viol |= m > tlim;
     };
@@ -365,11 +472,11 @@ __device__ __forceinline__ void h2_sweep(const float *__restrict__ tex, const u3
     }
 }
 
-template <bool TVEC, bool HALF>
-__global__ __launch_bounds__(kHThreads, 2) void f2f16h2_fwd_k(const float *__restrict__ tex, const float *__restrict__ hdr,
+template <bool TVEC, bool HALF, typename TIO>
+__global__ __launch_bounds__(kHThreads, 2) void f2f16h2_fwd_k(const TIO *__restrict__ tex, const float *__restrict__ hdr,
                                                               const u32x4 *__restrict__ Wp, const float *__restrict__ sh,
                                                               const int *__restrict__ cum, const int *__restrict__ order,
-                                                              float *__restrict__ out, int64_t Nf, int T, int Cin,
+                                                              TIO *__restrict__ out, int64_t Nf, int T, int Cin,
                                                               int Cout, int NT)
 {
     __shared__ u32x4 Ws[2 * kHChunk];
@@ -433,20 +540,20 @@ __global__ __launch_bounds__(kHThreads, 2) void f2f16h2_fwd_k(const float *__res
             float tm = 0.f;
             for (int kb = 0; kb < rKmax; kb += 4)
                 for (int cb = 0; cb < cend; cb += 32) {
-                    float4 v[4][4];
+                    HRaw4<TIO> v[4][4];
 #pragma unroll
                     for (int i = 0; i < 4; ++i)
 #pragma unroll
                         for (int g = 0; g < 4; ++g) {
                             const int c = cb + 8 * g + cg4;
                             v[i][g] = (kb + i < rK && c < Cin && (full || g == 0))
-                                          ? hld4_row<TVEC>(tex + (int64_t)(rk0 + kb + i) * Cin + c, Cin - c)
-                                          : make_float4(0.f, 0.f, 0.f, 0.f);
+                                          ? hld4_raw<TVEC>(tex + (int64_t)(rk0 + kb + i) * Cin + c, Cin - c)
+                                          : hraw_zero(TIO());
                         }
 #pragma unroll
                     for (int i = 0; i < 4; ++i)
 #pragma unroll
-                        for (int g = 0; g < 4; ++g) tm = absmax4(v[i][g], tm);
+                        for (int g = 0; g < 4; ++g) tm = absmax4(hcvt4(v[i][g]), tm);
                 }
             tm = fmaxf(tm, __shfl_xor(tm, 1, 64));
             sm = fmaxf(sm, __shfl_xor(sm, 32, 64));
@@ -475,7 +582,7 @@ __global__ __launch_bounds__(kHThreads, 2) void f2f16h2_fwd_k(const float *__res
             const int Ks = rem < 0 ? 0 : (rem > kHFKB ? kHFKB : rem);
             // every variant runs the same barriers, so wavefronts of a workgroup may pick different ones
             const int kw = hwave_max(Ks);
-#define PM_H2(N) h2_sweep<N, TVEC, HALF>(tex, Wp, sh, Ws, s_slab + w * 2 * kHSlab, acc, kbase, Ks, shs, slim, tlim, viol, s_k0, s_K, sw, Cin, NT, nt0, nblk, w, lane, h)
+#define PM_H2(N) h2_sweep<N, TVEC, HALF, TIO>(tex, Wp, sh, Ws, s_slab + w * 2 * kHSlab, acc, kbase, Ks, shs, slim, tlim, viol, s_k0, s_K, sw, Cin, NT, nt0, nblk, w, lane, h)
             if (kw <= 1) PM_H2(1);
             else if (kw == 2) PM_H2(2);
             else if (kw == 3) PM_H2(3);
@@ -491,13 +598,12 @@ __global__ __launch_bounds__(kHThreads, 2) void f2f16h2_fwd_k(const float *__res
     for (int i = 0; i < 16; ++i) {
         const int slot = w * 32 + 8 * (i / 4) + 4 * h + (i % 4);
         const int fr = s_f[slot];
-        if (fr >= 0 && fr < Nf) {
-            const float us = s_inv[slot] * ibeta;
+        const bool rok = fr >= 0 && fr < Nf;
+        const float us = s_inv[slot] * ibeta;
 #pragma unroll
-            for (int t = 0; t < 2; ++t) {
-                const int co = n0 + t * 32 + l32;
-                if (co < Cout) out[(int64_t)fr * Cout + co] = acc[t][i] * us;
-            }
+        for (int t = 0; t < 2; ++t) {
+            const int co = n0 + t * 32 + l32;
+            hst1_pair(out + ((int64_t)(rok ? fr : 0) * Cout + co), acc[t][i] * us, rok && co < Cout, l32);
         }
     }
 }
@@ -509,8 +615,9 @@ size_t f2f16h2_fwd_workspace_bytes(int Cin, int Cout)
     return 16 + (size_t)CinPad * NT * 2 * 64 * sizeof(u32x4);
 }
 
-int f2f16h2_fwd(const float *tex, const float *W, const float *sh, const int *cum, const int *order, float *out,
-                void *workspace, size_t workspace_bytes, int64_t T, int64_t Nf, int Cin, int Cout, hipStream_t st, bool half)
+int f2f16h2_fwd(const void *tex_, const float *W, const float *sh, const int *cum, const int *order, void *out_,
+                void *workspace, size_t workspace_bytes, int64_t T, int64_t Nf, int Cin, int Cout, hipStream_t st, bool half,
+                bool bf16)
 {
     const int NT = 2 * ((Cout + 63) / 64);
     PM_REQUIRE(T * Cin < (int64_t(1) << 31), "f2f_fwd: texture array too large for 32-bit offsets");
@@ -526,12 +633,19 @@ int f2f16h2_fwd(const float *tex, const float *W, const float *sh, const int *cu
     PM_LAUNCHED("f2f_fwd(pack)");
     const int64_t gx = ceil_div(Nf, kHFacets), gy = NT / 2;
     PM_REQUIRE(grid_ok(gx) && gy <= 65535, "f2f_fwd: grid too large");
-#define PM_FWD(V, H) f2f16h2_fwd_k<V, H><<<dim3((unsigned)gx, (unsigned)gy), dim3(kHThreads), 0, st>>>(tex, hdr, Wp, sh, cum, order, out, Nf, (int)T, Cin, Cout, NT)
-    const bool tvec = !(Cin & 3) && !(reinterpret_cast<uintptr_t>(tex) & 15u);
-    if (tvec && half) PM_FWD(true, true);
-    else if (tvec) PM_FWD(true, false);
-    else if (half) PM_FWD(false, true);
-    else PM_FWD(false, false);
+#define PM_FWD(V, H, TIO) f2f16h2_fwd_k<V, H, TIO><<<dim3((unsigned)gx, (unsigned)gy), dim3(kHThreads), 0, st>>>((const TIO *)tex_, hdr, Wp, sh, cum, order, (TIO *)out_, Nf, (int)T, Cin, Cout, NT)
+    if (bf16) {
+        // bf16 features: the one-product kernels, rows read eight bytes at a time
+        PM_REQUIRE(!(Cin & 3) && !(Cout & 1) && !(reinterpret_cast<uintptr_t>(tex_) & 7u) && !(reinterpret_cast<uintptr_t>(out_) & 3u),
+                   "f2f_fwd: bf16 features need a multiple of 4 input channels, an even number of output channels and aligned rows");
+        PM_FWD(true, true, bf16_t);
+    } else {
+        const bool tvec = !(Cin & 3) && !(reinterpret_cast<uintptr_t>(tex_) & 15u);
+        if (tvec && half) PM_FWD(true, true, float);
+        else if (tvec) PM_FWD(true, false, float);
+        else if (half) PM_FWD(false, true, float);
+        else PM_FWD(false, false, float);
+    }
 #undef PM_FWD
     PM_LAUNCHED("f2f_fwd");
     return 0;
@@ -572,9 +686,9 @@ __global__ __launch_bounds__(kBlock) void f2f16h2_pack_filter_t_k(const float *_
     dst[0] = p1; dst[64] = p2;
 }
 
-template <int KW, int NKS, bool GVEC, bool HALF>
+template <int KW, int NKS, bool GVEC, bool HALF, typename TIO>
 __device__ __forceinline__ void h2_tex_sweep(const u32x4 *__restrict__ WpT, const float *__restrict__ sh,
-                                             float *__restrict__ gtex, u32x4 *Ws, float *stage, const int *w_k0,
+                                             TIO *__restrict__ gtex, u32x4 *Ws, float *stage, const int *w_k0,
                                              const int *w_K, const u32x4 (&bp)[NKS][2], int kbase, int Ks, float shs,
                                              int sweep, int Cin, int NG, bool add, int lane, int h)
 {
@@ -627,20 +741,20 @@ __device__ __forceinline__ void h2_tex_sweep(const u32x4 *__restrict__ WpT, cons
             for (int kk = 0; kk < KW; ++kk)
                 if (kk < Kss && ci < Cin) {
                     const float4 v = *reinterpret_cast<const float4 *>(stage + (kk * 32 + slot) * 16 + 4 * (lane & 3));
-                    float *dst = gtex + (int64_t)(k0s + kk) * Cin + ci;
+                    TIO *dst = gtex + (int64_t)(k0s + kk) * Cin + ci;
                     // `add`: a later block of 64 output channels accumulates onto what the earlier ones wrote
                     if constexpr (GVEC) {
                         float4 o = v;
                         if (add) {
-                            const float4 p = *reinterpret_cast<const float4 *>(dst);
+                            const float4 p = hld4(dst);
                             o = make_float4(p.x + v.x, p.y + v.y, p.z + v.z, p.w + v.w);
                         }
-                        *reinterpret_cast<float4 *>(dst) = o;
+                        hst4(dst, o);
                     } else {                               // channel count not a multiple of 4 / unaligned rows
-                        dst[0] = add ? dst[0] + v.x : v.x;
-                        if (ci + 1 < Cin) dst[1] = add ? dst[1] + v.y : v.y;
-                        if (ci + 2 < Cin) dst[2] = add ? dst[2] + v.z : v.z;
-                        if (ci + 3 < Cin) dst[3] = add ? dst[3] + v.w : v.w;
+                        hst1(dst, add ? hld1(dst) + v.x : v.x);
+                        if (ci + 1 < Cin) hst1(dst + 1, add ? hld1(dst + 1) + v.y : v.y);
+                        if (ci + 2 < Cin) hst1(dst + 2, add ? hld1(dst + 2) + v.z : v.z);
+                        if (ci + 3 < Cin) hst1(dst + 3, add ? hld1(dst + 3) + v.w : v.w);
                     }
                 }
         }
@@ -724,13 +838,13 @@ __device__ __forceinline__ void h2_tex_sweep(const u32x4 *__restrict__ WpT, cons
 // NKS = k-steps of 16 output channels (compile time, so that a tile's MFMAs and the previous tile's
 // contraction share one basic block and get interleaved): 2 for Cout <= 32, else 4; the packed filter
 // is zero padded to that many.
-template <int NKS, bool GVEC, bool HALF>
-__global__ __launch_bounds__(512, 2) void f2f16h2_bwd_tex_k(const float *__restrict__ gout,
+template <int NKS, bool GVEC, bool HALF, typename TIN, typename TIO>
+__global__ __launch_bounds__(512, 2) void f2f16h2_bwd_tex_k(const TIN *__restrict__ gout,
                                                             const float *__restrict__ hdr,
                                                             const u32x4 *__restrict__ WpT,
                                                             const float *__restrict__ sh,
                                                             const int *__restrict__ cum,
-                                                            const int *__restrict__ order, float *__restrict__ gtex,
+                                                            const int *__restrict__ order, TIO *__restrict__ gtex,
                                                             int64_t Nf, int T, int Cin, int Cout, int NG, int co0)
 {
     __shared__ u32x4 Ws[3 * kHTChunkMax];
@@ -769,8 +883,8 @@ __global__ __launch_bounds__(512, 2) void f2f16h2_bwd_tex_k(const float *__restr
         for (int j = 0; j < 8; ++j) x[ks][j] = 0.f;
         const int co = co0 + 16 * ks + 8 * h;
         if (K > 0 && co < Cout) {
-            const float *p = gout + (int64_t)f * Cout + co;
-            const float4 u = hld4(p), v = hld4(p + 4);
+            float4 u, v;
+            hld8(gout + ((int64_t)f * Cout + co), u, v);
             x[ks][0] = u.x; x[ks][1] = u.y; x[ks][2] = u.z; x[ks][3] = u.w;
             x[ks][4] = v.x; x[ks][5] = v.y; x[ks][6] = v.z; x[ks][7] = v.w;
             gm = absmax4(u, absmax4(v, gm));
@@ -795,7 +909,7 @@ __global__ __launch_bounds__(512, 2) void f2f16h2_bwd_tex_k(const float *__restr
         const int kw = hwave_max(Ks);
         const int kbase = k0 + sw * kHTKB;
         // every variant runs the same barriers, so wavefronts of a workgroup may pick different ones
-#define PM_H2T(N) h2_tex_sweep<N, NKS, GVEC, HALF>(WpT, sh, gtex, Ws, s_stage[w], s_k0[w], s_K[w], bp, kbase, Ks, shs, sw, Cin, NG, co0 > 0, lane, h)
+#define PM_H2T(N) h2_tex_sweep<N, NKS, GVEC, HALF, TIO>(WpT, sh, gtex, Ws, s_stage[w], s_k0[w], s_K[w], bp, kbase, Ks, shs, sw, Cin, NG, co0 > 0, lane, h)
         if (kw <= 1) PM_H2T(1);
         else if (kw == 2) PM_H2T(2);
         else if (kw == 3) PM_H2T(3);
@@ -814,9 +928,27 @@ size_t f2f16h2_bwd_texture_workspace_bytes(int Cin, int Cout)
     return 16 + (size_t)NG * 4 * NKS * 2 * 64 * sizeof(u32x4);
 }
 
-int f2f16h2_bwd_texture(const float *gout, const float *W, const float *sh, const int *cum, const int *order,
-                        float *gtex, void *workspace, size_t workspace_bytes, int64_t T, int64_t Nf, int Cin,
-                        int Cout, hipStream_t st, bool half)
+// bf16 features and more than 64 output channels: the blocks of 64 output channels accumulate in a float32 copy of
+// grad_texture behind the packed filter (a bf16 running sum would be rounded once per block), converted at the end
+size_t f2f16h2_bwd_texture_bf16_workspace_bytes(int64_t T, int Cin, int Cout)
+{
+    const size_t base = (f2f16h2_bwd_texture_workspace_bytes(Cin, Cout) + 255) & ~(size_t)255;
+    return Cout > 64 ? base + (size_t)T * Cin * sizeof(float) : base;
+}
+
+__global__ __launch_bounds__(kBlock) void f2f16h2_rows_to_bf16_k(const float *__restrict__ src, bf16_t *__restrict__ dst,
+                                                                 const int *__restrict__ cum, int64_t Nf, int T, int Cin)
+{
+    int last = cum[Nf - 1];
+    last = last < 0 ? 0 : (last > T ? T : last);
+    const int64_t n4 = (int64_t)last * Cin / 4;                   // Cin is a multiple of 4
+    for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n4; i += (int64_t)gridDim.x * kBlock)
+        hst4(dst + 4 * i, hld4(src + 4 * i));
+}
+
+int f2f16h2_bwd_texture(const void *gout_, const float *W, const float *sh, const int *cum, const int *order,
+                        void *gtex_, void *workspace, size_t workspace_bytes, int64_t T, int64_t Nf, int Cin,
+                        int Cout, hipStream_t st, bool half, bool bf16)
 {
     const int NG = (Cin + 7) / 8;
     PM_REQUIRE(workspace && workspace_bytes >= f2f16h2_bwd_texture_workspace_bytes(Cin, Cout),
@@ -828,7 +960,16 @@ int f2f16h2_bwd_texture(const float *gout, const float *W, const float *sh, cons
     PM_LAUNCHED("f2f_bwd_texture(scale)");
     const int64_t gx = ceil_div(Nf, 256);
     PM_REQUIRE(grid_ok(gx), "f2f_bwd_texture: grid too large");
-    const bool gvec = !(Cin & 3) && !(reinterpret_cast<uintptr_t>(gtex) & 15u);
+    const bool gvec = !(Cin & 3) && !(reinterpret_cast<uintptr_t>(gtex_) & (bf16 ? 7u : 15u));
+    PM_REQUIRE(!bf16 || (gvec && !(Cout & 7) && !(reinterpret_cast<uintptr_t>(gout_) & 15u)),
+               "f2f_bwd_texture: bf16 features need Cin %% 4 == 0, Cout %% 8 == 0 and 16-byte aligned rows");
+    float *gtex32 = nullptr;
+    if (bf16 && Cout > 64) {
+        PM_REQUIRE(workspace_bytes >= f2f16h2_bwd_texture_bf16_workspace_bytes(T, Cin, Cout),
+                   "f2f_bwd_texture: workspace too small (%zu bytes) for bf16 features and more than 64 output channels", workspace_bytes);
+        gtex32 = reinterpret_cast<float *>(reinterpret_cast<char *>(workspace) +
+                                           ((f2f16h2_bwd_texture_workspace_bytes(Cin, Cout) + 255) & ~(size_t)255));
+    }
     // output channels go 64 at a time; the first block writes grad_texture, the others add to it
     // (launches on one stream run in order, so the packed filter buffer is reused)
     for (int co0 = 0; co0 < Cout; co0 += 64) {
@@ -836,17 +977,30 @@ int f2f16h2_bwd_texture(const float *gout, const float *W, const float *sh, cons
         const int n = NG * 4 * NKS * 64;
         f2f16h2_pack_filter_t_k<<<dim3((unsigned)ceil_div(n, kBlock)), dim3(kBlock), 0, st>>>(W, hdr, WpT, Cin, Cout, NG * 4, NKS, co0);
         PM_LAUNCHED("f2f_bwd_texture(pack)");
-#define PM_TEX(N, G)                                                                                                           \
-    do {                                                                                                                       \
-        if (half) f2f16h2_bwd_tex_k<N, G, true><<<dim3((unsigned)gx), dim3(512), 0, st>>>(gout, hdr, WpT, sh, cum, order, gtex, Nf, (int)T, Cin, Cout, NG, co0); \
-        else f2f16h2_bwd_tex_k<N, G, false><<<dim3((unsigned)gx), dim3(512), 0, st>>>(gout, hdr, WpT, sh, cum, order, gtex, Nf, (int)T, Cin, Cout, NG, co0);   \
-    } while (0)
-        if (NKS == 2 && gvec) PM_TEX(2, true);
-        else if (NKS == 2) PM_TEX(2, false);
-        else if (gvec) PM_TEX(4, true);
-        else PM_TEX(4, false);
+#define PM_TEX(N, G, H, TIN, TIO, DST) f2f16h2_bwd_tex_k<N, G, H, TIN, TIO><<<dim3((unsigned)gx), dim3(512), 0, st>>>((const TIN *)gout_, hdr, WpT, sh, cum, order, (TIO *)(DST), Nf, (int)T, Cin, Cout, NG, co0)
+        if (bf16 && gtex32) {
+            if (NKS == 2) PM_TEX(2, true, true, bf16_t, float, gtex32);
+            else PM_TEX(4, true, true, bf16_t, float, gtex32);
+        } else if (bf16) {
+            if (NKS == 2) PM_TEX(2, true, true, bf16_t, bf16_t, gtex_);
+            else PM_TEX(4, true, true, bf16_t, bf16_t, gtex_);
+        } else if (half) {
+            if (NKS == 2 && gvec) PM_TEX(2, true, true, float, float, gtex_);
+            else if (NKS == 2) PM_TEX(2, false, true, float, float, gtex_);
+            else if (gvec) PM_TEX(4, true, true, float, float, gtex_);
+            else PM_TEX(4, false, true, float, float, gtex_);
+        } else {
+            if (NKS == 2 && gvec) PM_TEX(2, true, false, float, float, gtex_);
+            else if (NKS == 2) PM_TEX(2, false, false, float, float, gtex_);
+            else if (gvec) PM_TEX(4, true, false, float, float, gtex_);
+            else PM_TEX(4, false, false, float, float, gtex_);
+        }
 #undef PM_TEX
         PM_LAUNCHED("f2f_bwd_texture");
+    }
+    if (gtex32) {
+        f2f16h2_rows_to_bf16_k<<<dim3(1024), dim3(kBlock), 0, st>>>(gtex32, (bf16_t *)gtex_, cum, Nf, (int)T, Cin);
+        PM_LAUNCHED("f2f_bwd_texture(convert)");
     }
     return 0;
 }
@@ -1019,15 +1173,19 @@ struct HPre {
     float g[8];
     float4 shv[kHShv];
 };
-__device__ __forceinline__ void hpre_issue(HPre &P, const float *__restrict__ gout, const float *__restrict__ sh,
+template <typename TIO>
+__device__ __forceinline__ void hpre_issue(HPre &P, const TIO *__restrict__ gout, const float *__restrict__ sh,
                                            const int *sf, const int *sk0, const int *sK, int Cout, int n0)
 {
     const int co = threadIdx.x & 63, st = (threadIdx.x >> 6) & 1, hh = threadIdx.x >> 7;
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
         const int f = sf[16 * st + 8 * (j >> 2) + 4 * hh + (j & 3)];
-        P.g[j] = (f >= 0 && n0 + co < Cout) ? gout[(int64_t)f * Cout + n0 + co] : 0.f;
+        // (kept as raw bits until the fetches are out; Cout is even for bf16 rows, so the half is the column's parity)
+        P.g[j] = __builtin_bit_cast(float, (f >= 0 && n0 + co < Cout) ? hld_raw(gout, (int64_t)f * Cout + n0 + co) : 0u);
     }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) P.g[j] = hcvt_raw(__builtin_bit_cast(unsigned, P.g[j]), (n0 + co) & 1, TIO());
 #pragma unroll
     for (int i = 0; i < kHShv; ++i) {
         const int e = threadIdx.x + 256 * i, row = e >> 2, kk = row >> 5, slot = row & 31;
@@ -1068,8 +1226,8 @@ __device__ __forceinline__ void hpre_commit(const HPre &P, u32x4 *go, float *shs
 __device__ __forceinline__ bool scale_fits(float s, float m) { return s * m < 32768.0f && s * m >= 32.0f; }
 
 // texture rows of one pass (KW points per facet) for my wavefront's channels: 64 bytes per row, four lanes per row
-template <int KW, bool TVEC, int NCP>
-__device__ __forceinline__ void htex_issue(float4 (&pf)[2 * kHKB], const float *__restrict__ tex, const int *sk0,
+template <int KW, bool TVEC, int NCP, typename TIO>
+__device__ __forceinline__ void htex_issue(HRaw4<TIO> (&pf)[2 * kHKB], const TIO *__restrict__ tex, const int *sk0,
                                            const int *sK, int sweep, int cw, int Cin, int lane)
 {
     const int piece = lane & 3;
@@ -1077,9 +1235,9 @@ __device__ __forceinline__ void htex_issue(float4 (&pf)[2 * kHKB], const float *
     for (int i = 0; i < 2 * KW; ++i) {
         const int rr = i * 16 + (lane >> 2), kk = rr >> 5, slot = rr & 31;
         const bool ok = sweep * kHKB + kk < sK[slot] && 4 * piece < 2 * NCP;
-        pf[i] = ok ? hld4_row<TVEC>(tex + (int64_t)(sk0[slot] + sweep * kHKB + kk) * Cin + cw + 4 * piece,
+        pf[i] = ok ? hld4_raw<TVEC>(tex + (int64_t)(sk0[slot] + sweep * kHKB + kk) * Cin + cw + 4 * piece,
                                     Cin - (cw + 4 * piece))
-                   : make_float4(0.f, 0.f, 0.f, 0.f);
+                   : hraw_zero(TIO());
     }
 }
 
@@ -1099,8 +1257,8 @@ struct HScales {
 
 // One tile of 32 facets whose inputs are in LDS buffer it % 2 (descriptors in it % 3): start the
 // fetches for the next tile, run the passes, publish the next tile's inputs.
-template <int KW, bool TVEC, int NCP, bool HALF>
-__device__ __forceinline__ void h2_filt_tile(const float *__restrict__ gout, const float *__restrict__ tex,
+template <int KW, bool TVEC, int NCP, bool HALF, typename TIO>
+__device__ __forceinline__ void h2_filt_tile(const TIO *__restrict__ gout, const TIO *__restrict__ tex,
                                              const float *__restrict__ sh, const int *__restrict__ cum,
                                              const int *__restrict__ order, u32x4 (*go_s)[2 * 2 * 2 * 64], float4 *slab,
                                              float (*sh_s)[kHKB * 32 * 16], int (*s_f)[32], int (*s_k0)[32],
@@ -1156,14 +1314,15 @@ __device__ __forceinline__ void h2_filt_tile(const float *__restrict__ gout, con
         float tmax = 0.f;
         {
             // my wavefront's texture rows of this pass -> slab
-            float4 pf[2 * kHKB];
-            htex_issue<KW, TVEC, NCP>(pf, tex, s_k0[sb], s_K[sb], sw, cw, Cin, lane);
+            HRaw4<TIO> pf[2 * kHKB];
+            htex_issue<KW, TVEC, NCP, TIO>(pf, tex, s_k0[sb], s_K[sb], sw, cw, Cin, lane);
             const int piece = lane & 3;
 #pragma unroll
             for (int i = 0; i < 2 * KW; ++i) {
                 const int rr = i * 16 + (lane >> 2), kk = rr >> 5, slot = rr & 31;
-                slab[(kk * 4 + piece) * 32 + slot] = pf[i];
-                tmax = absmax4(pf[i], tmax);
+                const float4 pv = hcvt4(pf[i]);
+                slab[(kk * 4 + piece) * 32 + slot] = pv;
+                tmax = absmax4(pv, tmax);
             }
         }
         // scale of G for this pass: |G| <= KW * max|tex| * max|sh / K|
@@ -1220,9 +1379,9 @@ __device__ __forceinline__ void h2_filt_tile(const float *__restrict__ gout, con
 
 // NCP = channel pairs of a wavefront (8 for 64 or more input channels; fewer for narrow filters, so that
 // the four wavefronts share what channels there are)
-template <bool TVEC, int NCP, bool HALF>
-__global__ __launch_bounds__(256, 1) void f2f16h2_bwd_filt_k(const float *__restrict__ gout,
-                                                              const float *__restrict__ tex,
+template <bool TVEC, int NCP, bool HALF, typename TIO>
+__global__ __launch_bounds__(256, 1) void f2f16h2_bwd_filt_k(const TIO *__restrict__ gout,
+                                                              const TIO *__restrict__ tex,
                                                               const float *__restrict__ sh,
                                                               const int *__restrict__ cum,
                                                               const int *__restrict__ order,
@@ -1295,7 +1454,7 @@ __global__ __launch_bounds__(256, 1) void f2f16h2_bwd_filt_k(const float *__rest
     int it = 0;
 #define PM_PHASE(N)                                                                                                  \
     for (; tile < ntiles && (N == kHKB || htile_kmax(s_K[it % 3], lane) <= N); ++it, tile += stride)                 \
-        h2_filt_tile<N, TVEC, NCP, HALF>(gout, tex, sh, cum, order, go_s, slab_s + w * (kHKB * 4 * 32), sh_s, s_f, s_k0, s_K, \
+        h2_filt_tile<N, TVEC, NCP, HALF, TIO>(gout, tex, sh, cum, order, go_s, slab_s + w * (kHKB * 4 * 32), sh_s, s_f, s_k0, s_K, \
                                    s_gamma, s_gm, acc, sc, overflow, ea, eb, it, tile, stride, ntiles, Nf, T, Cin, Cout, c0, n0, lane, w)
     PM_PHASE(1);
     PM_PHASE(2);
@@ -1330,8 +1489,9 @@ __global__ __launch_bounds__(256, 1) void f2f16h2_bwd_filt_k(const float *__rest
         }
 }
 
-int f2f16h2_bwd_filter_partials(const float *gout, const float *tex, const float *sh, const int *cum, const int *order,
-                                 float *partial, int *overflow, int splits, int64_t T, int64_t Nf, int Cin, int Cout, hipStream_t st, bool half)
+int f2f16h2_bwd_filter_partials(const void *gout_, const void *tex_, const float *sh, const int *cum, const int *order,
+                                 float *partial, int *overflow, int splits, int64_t T, int64_t Nf, int Cin, int Cout, hipStream_t st,
+                                 bool half, bool bf16)
 {
     // channel pairs per wavefront: the four wavefronts of a workgroup share up to 32 pairs
     const int pairs = (Cin + 1) / 2;
@@ -1339,18 +1499,21 @@ int f2f16h2_bwd_filter_partials(const float *gout, const float *tex, const float
     const int64_t gy = ceil_div(Cin, 8 * ncp), gz = ceil_div(Cout, 64);
     PM_REQUIRE(gy <= 65535 && gz <= 65535, "f2f_bwd_filter: grid too large");
     const int64_t ntiles = ceil_div(Nf, 32);
-    const bool tvec = !(Cin & 3) && !(reinterpret_cast<uintptr_t>(tex) & 15u);
+    const bool tvec = !(Cin & 3) && !(reinterpret_cast<uintptr_t>(tex_) & (bf16 ? 7u : 15u));
+    PM_REQUIRE(!bf16 || tvec, "f2f_bwd_filter: bf16 features need a multiple of 4 input channels and 8-byte aligned rows");
     const dim3 grid((unsigned)splits, (unsigned)gy, (unsigned)gz);
-#define PM_FILT(V, N)                                                                                                              \
-    do {                                                                                                                           \
-        if (half) f2f16h2_bwd_filt_k<V, N, true><<<grid, dim3(256), 0, st>>>(gout, tex, sh, cum, order, partial, overflow, Nf, (int)T, Cin, Cout, ntiles); \
-        else f2f16h2_bwd_filt_k<V, N, false><<<grid, dim3(256), 0, st>>>(gout, tex, sh, cum, order, partial, overflow, Nf, (int)T, Cin, Cout, ntiles);   \
+#define PM_FILT(V, N, H, TIO) f2f16h2_bwd_filt_k<V, N, H, TIO><<<grid, dim3(256), 0, st>>>((const TIO *)gout_, (const TIO *)tex_, sh, cum, order, partial, overflow, Nf, (int)T, Cin, Cout, ntiles)
+#define PM_FILT_N(V, H, TIO)                                                                              \
+    do {                                                                                                  \
+        if (ncp == 8) PM_FILT(V, 8, H, TIO); else if (ncp == 4) PM_FILT(V, 4, H, TIO);                    \
+        else if (ncp == 2) PM_FILT(V, 2, H, TIO); else PM_FILT(V, 1, H, TIO);                             \
     } while (0)
-    if (tvec) {
-        if (ncp == 8) PM_FILT(true, 8); else if (ncp == 4) PM_FILT(true, 4); else if (ncp == 2) PM_FILT(true, 2); else PM_FILT(true, 1);
-    } else {
-        if (ncp == 8) PM_FILT(false, 8); else if (ncp == 4) PM_FILT(false, 4); else if (ncp == 2) PM_FILT(false, 2); else PM_FILT(false, 1);
-    }
+    if (bf16) PM_FILT_N(true, true, bf16_t);
+    else if (tvec && half) PM_FILT_N(true, true, float);
+    else if (tvec) PM_FILT_N(true, false, float);
+    else if (half) PM_FILT_N(false, true, float);
+    else PM_FILT_N(false, false, float);
+#undef PM_FILT_N
 #undef PM_FILT
     PM_LAUNCHED("f2f_bwd_filter");
     return 0;

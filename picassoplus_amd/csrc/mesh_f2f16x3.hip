@@ -43,6 +43,26 @@ template <bool VEC> __device__ __forceinline__ float4 xld4_row(const float *p, i
     r.w = n > 3 ? p[3] : 0.f;
     return r;
 }
+// bf16 feature rows (the filter gradient also serves the reduced-precision variant as its guarded second launch)
+typedef unsigned short bf16_t;
+__device__ __forceinline__ float xbf(unsigned short v) { return __builtin_bit_cast(float, (unsigned)v << 16); }
+template <bool VEC> __device__ __forceinline__ float4 xld4_row(const bf16_t *p, int n)
+{
+    if constexpr (VEC) {
+        if (n <= 0) return make_float4(0.f, 0.f, 0.f, 0.f);
+        const uint2 u = *reinterpret_cast<const uint2 *>(p);
+        return make_float4(__builtin_bit_cast(float, u.x << 16), __builtin_bit_cast(float, u.x & 0xFFFF0000u),
+                           __builtin_bit_cast(float, u.y << 16), __builtin_bit_cast(float, u.y & 0xFFFF0000u));
+    }
+    float4 r;
+    r.x = n > 0 ? xbf(p[0]) : 0.f;
+    r.y = n > 1 ? xbf(p[1]) : 0.f;
+    r.z = n > 2 ? xbf(p[2]) : 0.f;
+    r.w = n > 3 ? xbf(p[3]) : 0.f;
+    return r;
+}
+__device__ __forceinline__ float xld1(const float *p) { return *p; }
+__device__ __forceinline__ float xld1(const bf16_t *p) { return xbf(*p); }
 __device__ __forceinline__ unsigned fbits(float x) { return __builtin_bit_cast(unsigned, x); }
 __device__ __forceinline__ float bitsf(unsigned u) { return __builtin_bit_cast(float, u); }
 // {hi16(b), hi16(a)}: two truncated bf16 values in one register, a in the low half
@@ -779,7 +799,8 @@ struct XPre {
     float g[8];
     float4 shv[2];
 };
-__device__ __forceinline__ void xpre_issue(XPre &P, const float *__restrict__ gout, const float *__restrict__ tex,
+template <typename TIO>
+__device__ __forceinline__ void xpre_issue(XPre &P, const TIO *__restrict__ gout, const TIO *__restrict__ tex,
                                            const float *__restrict__ sh, const int *sf, const int *sk0, const int *sK,
                                            int Cin, int Cout, int c0, int n0)
 {
@@ -787,7 +808,7 @@ __device__ __forceinline__ void xpre_issue(XPre &P, const float *__restrict__ go
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
         const int f = sf[16 * st + 8 * (j >> 2) + 4 * hh + (j & 3)];
-        P.g[j] = (f >= 0 && n0 + co < Cout) ? gout[(int64_t)f * Cout + n0 + co] : 0.f;
+        P.g[j] = (f >= 0 && n0 + co < Cout) ? xld1(gout + ((int64_t)f * Cout + n0 + co)) : 0.f;
     }
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
@@ -811,8 +832,8 @@ __device__ __forceinline__ void xpre_commit(const XPre &P, u32x4 *go, float *shs
 
 // texture rows of one pass (KW points per facet) for my wavefront's 16 channels: 64 bytes per row,
 // four lanes per row
-template <int KW, bool TVEC, int NCP>
-__device__ __forceinline__ void xtex_issue(float4 (&pf)[2 * kXKB], const float *__restrict__ tex, const int *sk0,
+template <int KW, bool TVEC, int NCP, typename TIO>
+__device__ __forceinline__ void xtex_issue(float4 (&pf)[2 * kXKB], const TIO *__restrict__ tex, const int *sk0,
                                            const int *sK, int sweep, int cw, int Cin, int lane)
 {
     const int piece = lane & 3;
@@ -830,8 +851,8 @@ __device__ __forceinline__ int xtile_kmax(const int *sK, int lane) { return xwav
 
 // One tile of 32 facets whose inputs are in LDS buffer it % 2 (descriptors in it % 3): start the
 // fetches for the next tile, run the passes, publish the next tile's inputs.
-template <int KW, bool TVEC, int NCP>
-__device__ __forceinline__ void x3_filt_tile(const float *__restrict__ gout, const float *__restrict__ tex,
+template <int KW, bool TVEC, int NCP, typename TIO>
+__device__ __forceinline__ void x3_filt_tile(const TIO *__restrict__ gout, const TIO *__restrict__ tex,
                                              const float *__restrict__ sh, const int *__restrict__ cum,
                                              const int *__restrict__ order, u32x4 (*go_s)[2 * 2 * 3 * 64], float4 *slab,
                                              float (*sh_s)[kXKB * 32 * 16], int (*s_f)[32], int (*s_k0)[32],
@@ -881,7 +902,7 @@ __device__ __forceinline__ void x3_filt_tile(const float *__restrict__ gout, con
         {
             // my wavefront's texture rows of this pass -> slab
             float4 pf[2 * kXKB];
-            xtex_issue<KW, TVEC, NCP>(pf, tex, s_k0[sb], s_K[sb], sw, cw, Cin, lane);
+            xtex_issue<KW, TVEC, NCP, TIO>(pf, tex, s_k0[sb], s_K[sb], sw, cw, Cin, lane);
             const int piece = lane & 3;
 #pragma unroll
             for (int i = 0; i < 2 * KW; ++i) {
@@ -901,9 +922,9 @@ __device__ __forceinline__ void x3_filt_tile(const float *__restrict__ gout, con
 
 // NCP = channel pairs of a wavefront (8 for 64 or more input channels; fewer for narrow filters, so that
 // the four wavefronts share what channels there are)
-template <bool TVEC, int NCP>
-__global__ __launch_bounds__(256, 1) void f2f16x3_bwd_filt_k(const float *__restrict__ gout,
-                                                              const float *__restrict__ tex,
+template <bool TVEC, int NCP, typename TIO>
+__global__ __launch_bounds__(256, 1) void f2f16x3_bwd_filt_k(const TIO *__restrict__ gout,
+                                                              const TIO *__restrict__ tex,
                                                               const float *__restrict__ sh,
                                                               const int *__restrict__ cum,
                                                               const int *__restrict__ order,
@@ -964,7 +985,7 @@ __global__ __launch_bounds__(256, 1) void f2f16x3_bwd_filt_k(const float *__rest
     int it = 0;
 #define PM_PHASE(N)                                                                                                  \
     for (; tile < ntiles && (N == kXKB || xtile_kmax(s_K[it % 3], lane) <= N); ++it, tile += stride)                 \
-        x3_filt_tile<N, TVEC, NCP>(gout, tex, sh, cum, order, go_s, slab_s + w * (kXKB * 4 * 32), sh_s, s_f, s_k0, s_K, acc, ea, eb,  \
+        x3_filt_tile<N, TVEC, NCP, TIO>(gout, tex, sh, cum, order, go_s, slab_s + w * (kXKB * 4 * 32), sh_s, s_f, s_k0, s_K, acc, ea, eb,  \
                         it, tile, stride, ntiles, Nf, T, Cin, Cout, c0, n0, lane, w)
     PM_PHASE(1);
     PM_PHASE(2);
@@ -990,9 +1011,9 @@ __global__ __launch_bounds__(256, 1) void f2f16x3_bwd_filt_k(const float *__rest
         }
 }
 
-int f2f16x3_bwd_filter_partials(const float *gout, const float *tex, const float *sh, const int *cum, const int *order,
+int f2f16x3_bwd_filter_partials(const void *gout_, const void *tex_, const float *sh, const int *cum, const int *order,
                                  float *partial, int splits, int64_t T, int64_t Nf, int Cin, int Cout, hipStream_t st,
-                                 const int *only_if)
+                                 const int *only_if, bool bf16)
 {
     // channel pairs per wavefront: the four wavefronts of a workgroup share up to 32 pairs
     const int pairs = (Cin + 1) / 2;
@@ -1000,14 +1021,19 @@ int f2f16x3_bwd_filter_partials(const float *gout, const float *tex, const float
     const int64_t gy = ceil_div(Cin, 8 * ncp), gz = ceil_div(Cout, 64);
     PM_REQUIRE(gy <= 65535 && gz <= 65535, "f2f_bwd_filter: grid too large");
     const int64_t ntiles = ceil_div(Nf, 32);
-    const bool tvec = !(Cin & 3) && !(reinterpret_cast<uintptr_t>(tex) & 15u);
+    const bool tvec = !(Cin & 3) && !(reinterpret_cast<uintptr_t>(tex_) & (bf16 ? 7u : 15u));
+    PM_REQUIRE(!bf16 || tvec, "f2f_bwd_filter: bf16 features need a multiple of 4 input channels and 8-byte aligned rows");
     const dim3 grid((unsigned)splits, (unsigned)gy, (unsigned)gz);
-#define PM_FILT(V, N) f2f16x3_bwd_filt_k<V, N><<<grid, dim3(256), 0, st>>>(gout, tex, sh, cum, order, partial, Nf, (int)T, Cin, Cout, ntiles, only_if)
-    if (tvec) {
-        if (ncp == 8) PM_FILT(true, 8); else if (ncp == 4) PM_FILT(true, 4); else if (ncp == 2) PM_FILT(true, 2); else PM_FILT(true, 1);
-    } else {
-        if (ncp == 8) PM_FILT(false, 8); else if (ncp == 4) PM_FILT(false, 4); else if (ncp == 2) PM_FILT(false, 2); else PM_FILT(false, 1);
-    }
+#define PM_FILT(V, N, TIO) f2f16x3_bwd_filt_k<V, N, TIO><<<grid, dim3(256), 0, st>>>((const TIO *)gout_, (const TIO *)tex_, sh, cum, order, partial, Nf, (int)T, Cin, Cout, ntiles, only_if)
+#define PM_FILT_N(V, TIO)                                                                     \
+    do {                                                                                      \
+        if (ncp == 8) PM_FILT(V, 8, TIO); else if (ncp == 4) PM_FILT(V, 4, TIO);              \
+        else if (ncp == 2) PM_FILT(V, 2, TIO); else PM_FILT(V, 1, TIO);                       \
+    } while (0)
+    if (bf16) PM_FILT_N(true, bf16_t);
+    else if (tvec) PM_FILT_N(true, float);
+    else PM_FILT_N(false, float);
+#undef PM_FILT_N
 #undef PM_FILT
     PM_LAUNCHED("f2f_bwd_filter");
     return 0;

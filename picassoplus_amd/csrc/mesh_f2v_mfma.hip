@@ -23,26 +23,65 @@ __device__ __forceinline__ void half_swap(float &a, float &b)
     asm volatile("s_nop 3\n v_permlane32_swap_b32 %0, %1\n s_nop 3" : "+v"(a), "+v"(b));
 }
 
-__device__ __forceinline__ const float *at_bytes(const float *base, unsigned byte_offset)
+template <typename TIO> __device__ __forceinline__ const TIO *at_bytes(const TIO *base, unsigned byte_offset)
 {
-    return reinterpret_cast<const float *>(reinterpret_cast<const char *>(base) + byte_offset);
+    return reinterpret_cast<const TIO *>(reinterpret_cast<const char *>(base) + byte_offset);
+}
+
+// Features kept in bf16 in HBM (the reduced-precision variant of the layer): converted on load, rounded to nearest
+// even on store; all sums stay in fp32.
+typedef unsigned short bf16_t;
+// Value at `byte_offset` from `base`, in two steps: ld_raw fetches the 4 bytes that hold it (a conditional fetch must
+// not be followed by arithmetic inside its branch, or the wavefront waits for every fetch on the spot and the gathers
+// no longer overlap), cvt_raw turns them into the value once all fetches of a batch are out.  A bf16 value is read
+// as the aligned word that holds it (rows have an even number of values, so neighbouring lanes share the word) and
+// written as one 4-byte store per lane pair: 2-byte accesses are slow on this memory path.
+__device__ __forceinline__ unsigned ld_raw(const float *base, unsigned byte_offset)
+{
+    return *reinterpret_cast<const unsigned *>(reinterpret_cast<const char *>(base) + byte_offset);
+}
+__device__ __forceinline__ unsigned ld_raw(const bf16_t *base, unsigned byte_offset)
+{
+    return *reinterpret_cast<const unsigned *>(reinterpret_cast<const char *>(base) + (byte_offset & ~3u));
+}
+__device__ __forceinline__ float cvt_raw(unsigned w, unsigned, float) { return __builtin_bit_cast(float, w); }
+__device__ __forceinline__ float cvt_raw(unsigned w, unsigned byte_offset, bf16_t)
+{
+    return __builtin_bit_cast(float, (byte_offset & 2u) ? (w & 0xFFFF0000u) : (w << 16));
+}
+// Lanes l and l ^ STEP hold neighbouring values p[0], p[1] (the lane with (lane & STEP) == 0 the first): every lane
+// calls this, `ok` says whether the pair is stored.  STEP = 1: neighbouring lanes; 2: lanes two apart.
+template <int STEP> __device__ __forceinline__ void st1_pair(float *p, float v, bool ok, int lane)
+{
+    (void)lane;
+    if (ok) *p = v;
+}
+template <int STEP> __device__ __forceinline__ void st1_pair(bf16_t *p, float v, bool ok, int lane)
+{
+    // quad_perm [1,0,3,2] swaps neighbours, [2,3,0,1] swaps lanes two apart
+    const float nb = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), STEP == 1 ? 0xB1 : 0x4E, 0xF, 0xF, true));
+    if (ok && !(lane & STEP)) {
+        unsigned r;
+        asm("v_cvt_pk_bf16_f32 %0, %1, %2" : "=v"(r) : "v"(v), "v"(nb));
+        *reinterpret_cast<unsigned *>(p) = r;
+    }
 }
 
 // Forward.  NCB = 32-channel blocks per workgroup column (blockIdx.y selects a chunk of 32*NCB channels).
 // Requires K == 16, 16-byte aligned coefficient rows, Nf * C * 4 < 2^32.  Workgroups are persistent; the
 // eight dies take contiguous eighths of the vertices (blockIdx.x & 7 = die).
-template <int NCB>
-__global__ __launch_bounds__(kBlock) void f2v_fwd_mfma_k(const float *__restrict__ in, const float *__restrict__ filt,
+template <int NCB, typename TIO>
+__global__ __launch_bounds__(kBlock) void f2v_fwd_mfma_k(const TIO *__restrict__ in, const float *__restrict__ filt,
                                                          const float *__restrict__ coeff,
                                                          const int *__restrict__ nfcount,
                                                          const int *__restrict__ rowptr,
-                                                         const int *__restrict__ colidx, float *__restrict__ out,
+                                                         const int *__restrict__ colidx, TIO *__restrict__ out,
                                                          int64_t NvOut, int C, int r, int Co)
 {
     const int l = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int col = l & 31, h = l >> 5, j = col >> 3, s = col & 7;
     const int co0 = blockIdx.y * (32 * NCB);
-    const unsigned row_bytes = (unsigned)C * 4u;
+    const unsigned row_bytes = (unsigned)C * (unsigned)sizeof(TIO);
 
     // B operands: step kk of half h is coefficient 8h + kk (the A operand uses the same assignment)
     float wb[NCB][8];
@@ -52,7 +91,7 @@ __global__ __launch_bounds__(kBlock) void f2v_fwd_mfma_k(const float *__restrict
     for (int cb = 0; cb < NCB; ++cb) {
         const int co = co0 + 32 * cb + col;
         con[cb] = co < Co;
-        chb[cb] = con[cb] ? (unsigned)(co / r) * 4u : 0u;
+        chb[cb] = con[cb] ? (unsigned)(co / r) * (unsigned)sizeof(TIO) : 0u;
 #pragma unroll
         for (int kk = 0; kk < 8; ++kk) wb[cb][kk] = con[cb] ? filt[(size_t)(8 * h + kk) * Co + co] : 0.f;
     }
@@ -108,14 +147,19 @@ __global__ __launch_bounds__(kBlock) void f2v_fwd_mfma_k(const float *__restrict
 #pragma unroll
             for (int i = 0; i < 16; ++i)
                 b[i] = (unsigned)__builtin_amdgcn_ds_bpermute((8 * (i >> 2) + 4 * h + (i & 3)) * 4, (int)boff);
-            float x[NCB][16];
+            unsigned xr[NCB][16];
 #pragma unroll
             for (int cb = 0; cb < NCB; ++cb)
 #pragma unroll
                 for (int i = 0; i < 16; ++i) {
-                    x[cb][i] = 0.f;
-                    if (b[i] != 0xFFFFFFFFu && con[cb]) x[cb][i] = *at_bytes(in, b[i] + chb[cb]);
+                    xr[cb][i] = 0u;
+                    if (b[i] != 0xFFFFFFFFu && con[cb]) xr[cb][i] = ld_raw(in, b[i] + chb[cb]);
                 }
+            float x[NCB][16];
+#pragma unroll
+            for (int cb = 0; cb < NCB; ++cb)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) x[cb][i] = cvt_raw(xr[cb][i], chb[cb], TIO());
 #pragma unroll
             for (int cb = 0; cb < NCB; ++cb) {
                 f32x16 d;
@@ -138,10 +182,8 @@ __global__ __launch_bounds__(kBlock) void f2v_fwd_mfma_k(const float *__restrict
             half_swap(acc[cb][1], acc[cb][3]);
             const float o0 = (acc[cb][0] + acc[cb][2]) * inv0, o1 = (acc[cb][1] + acc[cb][3]) * inv1;
             const int co = co0 + 32 * cb + col;
-            if (con[cb]) {
-                if (vs < NvOut) out[vs * Co + co] = o0;
-                if (vs + 1 < NvOut) out[(vs + 1) * Co + co] = o1;
-            }
+            st1_pair<1>(out + (vs * Co + co), o0, con[cb] && vs < NvOut, col);
+            st1_pair<1>(out + ((vs + 1) * Co + co), o1, con[cb] && vs + 1 < NvOut, col);
         }
         e0 = ne0; e1 = ne1; ne0 = me0; ne1 = me1;
         f = nf;
@@ -161,13 +203,13 @@ __global__ __launch_bounds__(kBlock) void f2v_fwd_mfma_k(const float *__restrict
 // wavefront writes for its own tile; the index chain face -> vt_map -> nf_count runs three tiles ahead.
 // Workgroups own contiguous facet ranges (fixed by the problem size only) and leave one partial filter
 // gradient each, summed by reduce_partials in a fixed order.
-template <int NCB, int R>
-__global__ __launch_bounds__(kBlock, 2) void f2v_bwd_mfma_k(const float *__restrict__ gout, const float *__restrict__ in,
+template <int NCB, int R, typename TIO>
+__global__ __launch_bounds__(kBlock, 2) void f2v_bwd_mfma_k(const TIO *__restrict__ gout, const TIO *__restrict__ in,
                                                          const float *__restrict__ filt,
                                                          const float *__restrict__ coeff,
                                                          const int *__restrict__ face,
                                                          const int *__restrict__ nfcount,
-                                                         const int *__restrict__ vtmap, float *__restrict__ gin,
+                                                         const int *__restrict__ vtmap, TIO *__restrict__ gin,
                                                          float *__restrict__ partial, int64_t Nf, int64_t NvOut, int C,
                                                          int Co, int64_t rows_per_block)
 {
@@ -181,7 +223,7 @@ __global__ __launch_bounds__(kBlock, 2) void f2v_bwd_mfma_k(const float *__restr
     const int64_t rb = (G & 7) ? blockIdx.x : (int64_t)(blockIdx.x & 7) * (G >> 3) + (blockIdx.x >> 3);
     const int64_t fbeg = rb * rows_per_block;
     const int64_t fend = (fbeg + rows_per_block < Nf) ? fbeg + rows_per_block : Nf;
-    const unsigned in_row = (unsigned)C * 4u, out_row = (unsigned)Co * 4u;
+    const unsigned in_row = (unsigned)C * (unsigned)sizeof(TIO), out_row = (unsigned)Co * (unsigned)sizeof(TIO);
 
     float wb[NCB][8];
     unsigned chb[NCB], cob[NCB];
@@ -190,8 +232,8 @@ __global__ __launch_bounds__(kBlock, 2) void f2v_bwd_mfma_k(const float *__restr
     for (int cb = 0; cb < NCB; ++cb) {
         const int co = co0 + 32 * cb + col;
         con[cb] = co < Co;
-        chb[cb] = con[cb] ? (unsigned)(co / R) * 4u : 0u;
-        cob[cb] = con[cb] ? (unsigned)co * 4u : 0u;
+        chb[cb] = con[cb] ? (unsigned)(co / R) * (unsigned)sizeof(TIO) : 0u;
+        cob[cb] = con[cb] ? (unsigned)co * (unsigned)sizeof(TIO) : 0u;
 #pragma unroll
         for (int kk = 0; kk < 8; ++kk) wb[cb][kk] = con[cb] ? filt[(size_t)(8 * h + kk) * Co + co] : 0.f;
     }
@@ -279,13 +321,15 @@ __global__ __launch_bounds__(kBlock, 2) void f2v_bwd_mfma_k(const float *__restr
             const unsigned xoff = (unsigned)(f0 + ri) * in_row;
 #pragma unroll
             for (int cb = 0; cb < NCB; ++cb) {
-                float g0 = 0.f, g1 = 0.f, g2 = 0.f, xx = 0.f;
-                if (m0.x != 0xFFFFFFFFu && con[cb]) g0 = *at_bytes(gout, m0.x + cob[cb]);
-                if (m0.y != 0xFFFFFFFFu && con[cb]) g1 = *at_bytes(gout, m0.y + cob[cb]);
-                if (m0.z != 0xFFFFFFFFu && con[cb]) g2 = *at_bytes(gout, m0.z + cob[cb]);
-                if (fok && con[cb]) xx = *at_bytes(in, xoff + chb[cb]);
+                unsigned r0 = 0u, r1 = 0u, r2 = 0u, rx = 0u;
+                if (m0.x != 0xFFFFFFFFu && con[cb]) r0 = ld_raw(gout, m0.x + cob[cb]);
+                if (m0.y != 0xFFFFFFFFu && con[cb]) r1 = ld_raw(gout, m0.y + cob[cb]);
+                if (m0.z != 0xFFFFFFFFu && con[cb]) r2 = ld_raw(gout, m0.z + cob[cb]);
+                if (fok && con[cb]) rx = ld_raw(in, xoff + chb[cb]);
+                // (row offsets are multiples of 4 bytes: the half of the word depends on the column only)
+                const float g0 = cvt_raw(r0, cob[cb], TIO()), g1 = cvt_raw(r1, cob[cb], TIO()), g2 = cvt_raw(r2, cob[cb], TIO());
                 sv[cb][i] = fmaf(g2, __uint_as_float(m1.z), fmaf(g1, __uint_as_float(m1.y), g0 * __uint_as_float(m1.x)));
-                xv[cb][i] = xx;
+                xv[cb][i] = cvt_raw(rx, chb[cb], TIO());
             }
         }
 #pragma unroll
@@ -301,8 +345,9 @@ __global__ __launch_bounds__(kBlock, 2) void f2v_bwd_mfma_k(const float *__restr
                 float gi = sv[cb][i] * d[i];
                 if constexpr (R == 2)          // the two outputs of an input channel sit in neighbouring lanes
                     gi += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, gi), 0xB1, 0xF, 0xF, true));
-                if (f0 + ri < fend && con[cb] && (R == 1 || !(col & 1)))
-                    *const_cast<float *>(at_bytes(gin, (unsigned)(f0 + ri) * in_row + chb[cb])) = gi;
+                // R == 2: the even lanes hold the channels, neighbouring channels sit two lanes apart
+                st1_pair<R>(const_cast<TIO *>(at_bytes(gin, (unsigned)(f0 + ri) * in_row + chb[cb])), gi,
+                            f0 + ri < fend && con[cb] && (R == 1 || !(col & 1)), col);
             }
 #pragma unroll
             for (int i = 0; i < 16; ++i)
@@ -331,8 +376,9 @@ bool f2v_mfma_ok(int64_t Nf, int C, int r, int K, const void *coeff)
     return K == 16 && C * r >= 32 && (reinterpret_cast<uintptr_t>(coeff) & 15) == 0 && Nf * (int64_t)C < (int64_t(1) << 30);
 }
 
-int f2v_fwd_mfma(const float *in, const float *filt, const float *coeff, const int *nfcount, const int *rowptr,
-                 const int *colidx, float *out, int64_t NvOut, int C, int r, hipStream_t st)
+template <typename TIO>
+static void f2v_fwd_launch(const TIO *in, const float *filt, const float *coeff, const int *nfcount, const int *rowptr,
+                           const int *colidx, TIO *out, int64_t NvOut, int C, int r, hipStream_t st)
 {
     const int Co = C * r;
     const int ncb = Co <= 32 ? 1 : Co <= 64 ? 2 : Co <= 96 ? 3 : 2;      // wider rows: chunks of 64 channels (more wavefronts in flight)
@@ -341,11 +387,17 @@ int f2v_fwd_mfma(const float *in, const float *filt, const float *coeff, const i
     const unsigned gxn = (unsigned)(want < 4096 ? want : 4096);
     const dim3 grid(gxn, gy), block(kBlock);
     switch (ncb) {
-    case 1: f2v_fwd_mfma_k<1><<<grid, block, 0, st>>>(in, filt, coeff, nfcount, rowptr, colidx, out, NvOut, C, r, Co); break;
-    case 2: f2v_fwd_mfma_k<2><<<grid, block, 0, st>>>(in, filt, coeff, nfcount, rowptr, colidx, out, NvOut, C, r, Co); break;
-    case 3: f2v_fwd_mfma_k<3><<<grid, block, 0, st>>>(in, filt, coeff, nfcount, rowptr, colidx, out, NvOut, C, r, Co); break;
-    default: f2v_fwd_mfma_k<4><<<grid, block, 0, st>>>(in, filt, coeff, nfcount, rowptr, colidx, out, NvOut, C, r, Co); break;
+    case 1: f2v_fwd_mfma_k<1, TIO><<<grid, block, 0, st>>>(in, filt, coeff, nfcount, rowptr, colidx, out, NvOut, C, r, Co); break;
+    case 2: f2v_fwd_mfma_k<2, TIO><<<grid, block, 0, st>>>(in, filt, coeff, nfcount, rowptr, colidx, out, NvOut, C, r, Co); break;
+    default: f2v_fwd_mfma_k<3, TIO><<<grid, block, 0, st>>>(in, filt, coeff, nfcount, rowptr, colidx, out, NvOut, C, r, Co); break;
     }
+}
+
+int f2v_fwd_mfma(const void *in, const float *filt, const float *coeff, const int *nfcount, const int *rowptr,
+                 const int *colidx, void *out, int64_t NvOut, int C, int r, hipStream_t st, bool bf16)
+{
+    if (bf16) f2v_fwd_launch((const bf16_t *)in, filt, coeff, nfcount, rowptr, colidx, (bf16_t *)out, NvOut, C, r, st);
+    else f2v_fwd_launch((const float *)in, filt, coeff, nfcount, rowptr, colidx, (float *)out, NvOut, C, r, st);
     PM_LAUNCHED("f2v_fwd(mfma)");
     return 0;
 }
@@ -354,9 +406,10 @@ int f2v_fwd_mfma(const float *in, const float *filt, const float *coeff, const i
 // rows_per_block and the workgroup count depend on the problem size only (fixed summation order).
 int f2v_bwd_mfma_blocks(int64_t Nf) { return persistent_blocks(Nf, 128); }
 
-int f2v_bwd_mfma(const float *gout, const float *in, const float *filt, const float *coeff, const int *face,
-                 const int *nfcount, const int *vtmap, float *gin, float *partial, int G, int64_t Nf, int64_t NvOut,
-                 int C, int r, hipStream_t st)
+template <typename TIO>
+static void f2v_bwd_launch(const TIO *gout, const TIO *in, const float *filt, const float *coeff, const int *face,
+                           const int *nfcount, const int *vtmap, TIO *gin, float *partial, int G, int64_t Nf, int64_t NvOut,
+                           int C, int r, hipStream_t st)
 {
     const int Co = C * r;
     // one 32-channel block per workgroup column: two wavefronts per SIMD fit, which beats sharing the
@@ -365,9 +418,19 @@ int f2v_bwd_mfma(const float *gout, const float *in, const float *filt, const fl
     const int64_t rows_per_block = ceil_div(ceil_div(Nf, G), 128) * 128;
     const dim3 grid((unsigned)G, gy), block(kBlock);
     if (r == 1)
-        f2v_bwd_mfma_k<1, 1><<<grid, block, 0, st>>>(gout, in, filt, coeff, face, nfcount, vtmap, gin, partial, Nf, NvOut, C, Co, rows_per_block);
+        f2v_bwd_mfma_k<1, 1, TIO><<<grid, block, 0, st>>>(gout, in, filt, coeff, face, nfcount, vtmap, gin, partial, Nf, NvOut, C, Co, rows_per_block);
     else
-        f2v_bwd_mfma_k<1, 2><<<grid, block, 0, st>>>(gout, in, filt, coeff, face, nfcount, vtmap, gin, partial, Nf, NvOut, C, Co, rows_per_block);
+        f2v_bwd_mfma_k<1, 2, TIO><<<grid, block, 0, st>>>(gout, in, filt, coeff, face, nfcount, vtmap, gin, partial, Nf, NvOut, C, Co, rows_per_block);
+}
+
+int f2v_bwd_mfma(const void *gout, const void *in, const float *filt, const float *coeff, const int *face,
+                 const int *nfcount, const int *vtmap, void *gin, float *partial, int G, int64_t Nf, int64_t NvOut,
+                 int C, int r, hipStream_t st, bool bf16)
+{
+    if (bf16)
+        f2v_bwd_launch((const bf16_t *)gout, (const bf16_t *)in, filt, coeff, face, nfcount, vtmap, (bf16_t *)gin, partial, G, Nf, NvOut, C, r, st);
+    else
+        f2v_bwd_launch((const float *)gout, (const float *)in, filt, coeff, face, nfcount, vtmap, (float *)gin, partial, G, Nf, NvOut, C, r, st);
     PM_LAUNCHED("f2v_bwd(mfma)");
     return 0;
 }

@@ -1037,6 +1037,55 @@ extern "C" int pmesh_f2v_bwd(const float *grad_output, const float *input, const
     return reduce_partials(partial, grad_filter, G, K * Co, st);
 }
 
+// ---- facet2vertex with the features in bf16 (the reduced-precision variant of the layer) ----------------------
+// input, output, grad_output and grad_input rows are bf16; filter, coefficients and the filter gradient stay float.
+// Only the shapes of the matrix-core kernels: 16 coefficients, at least 32 output channels, depth multiplier 1 or 2.
+extern "C" int pmesh_f2v_fwd_bf16(const uint16_t *input, const float *filter, const float *coeff,
+                                  const int32_t *nf_count, const int32_t *rowptr, const int32_t *colidx,
+                                  uint16_t *output, int64_t Nf, int64_t NvOut, int C, int r, int K,
+                                  pmesh_stream_t stream)
+{
+    clear_error();
+    PM_DIMS("f2v_fwd_bf16");
+    PM_REQUIRE(Nf >= 0 && NvOut >= 0, "f2v_fwd_bf16: negative size");
+    if (NvOut == 0) return 0;
+    PM_REQUIRE(input && filter && coeff && nf_count && rowptr && colidx && output, "f2v_fwd_bf16: null pointer");
+    PM_REQUIRE(NvOut <= INT32_MAX && Nf <= INT32_MAX / 3, "f2v_fwd_bf16: sizes exceed int32 indexing");
+    PM_REQUIRE(f2v_mfma_ok(Nf, C, r, K, coeff) && !(C & 1) && !((reinterpret_cast<uintptr_t>(input) | reinterpret_cast<uintptr_t>(output)) & 3u),
+               "f2v_fwd_bf16: bf16 features need 16 coefficients in 16-byte aligned rows, an even channel count and at least 32 output channels (K=%d C=%d r=%d)", K, C, r);
+    return f2v_fwd_mfma(input, filter, coeff, nf_count, rowptr, colidx, output, NvOut, C, r, (hipStream_t)stream, true);
+}
+
+extern "C" int pmesh_f2v_bwd_bf16(const uint16_t *grad_output, const uint16_t *input, const float *filter,
+                                  const float *coeff, const int32_t *face, const int32_t *nf_count,
+                                  const int32_t *vt_map, uint16_t *grad_input, float *grad_filter, void *workspace,
+                                  size_t workspace_bytes, int64_t Nf, int64_t NvIn, int64_t NvOut, int C, int r,
+                                  int K, pmesh_stream_t stream)
+{
+    clear_error();
+    (void)NvIn;
+    PM_DIMS("f2v_bwd_bf16");
+    PM_REQUIRE(Nf >= 0 && NvOut >= 0, "f2v_bwd_bf16: negative size");
+    PM_REQUIRE(grad_filter, "f2v_bwd_bf16: null grad_filter");
+    PM_REQUIRE(NvOut <= INT32_MAX && Nf <= INT32_MAX / 3, "f2v_bwd_bf16: sizes exceed int32 indexing");
+    hipStream_t st = (hipStream_t)stream;
+    const int Co = C * r;
+    if (Nf == 0) {
+        fill_zero_k<<<dim3((unsigned)ceil_div((int64_t)K * Co, kBlock)), dim3(kBlock), 0, st>>>(grad_filter, (int64_t)K * Co);
+        PM_LAUNCHED("f2v_bwd_bf16(fill)");
+        return 0;
+    }
+    PM_REQUIRE(grad_output && input && filter && coeff && face && nf_count && vt_map && grad_input && workspace, "f2v_bwd_bf16: null pointer");
+    PM_REQUIRE((r == 1 || r == 2) && f2v_mfma_ok(Nf, C, r, K, coeff) && NvOut * (int64_t)Co < (int64_t(1) << 30) && !(C & 1) &&
+                   !((reinterpret_cast<uintptr_t>(input) | reinterpret_cast<uintptr_t>(grad_output) | reinterpret_cast<uintptr_t>(grad_input)) & 3u),
+               "f2v_bwd_bf16: bf16 features need 16 coefficients in 16-byte aligned rows, an even channel count, at least 32 output channels and depth multiplier 1 or 2 (K=%d C=%d r=%d)", K, C, r);
+    const int Gm = f2v_bwd_mfma_blocks(Nf);
+    PM_REQUIRE(workspace_bytes >= (size_t)Gm * K * Co * sizeof(float), "f2v_bwd_bf16: workspace too small (%zu bytes)", workspace_bytes);
+    float *partial = (float *)workspace;
+    if (int rc = f2v_bwd_mfma(grad_output, input, filter, coeff, face, nf_count, vt_map, grad_input, partial, Gm, Nf, NvOut, C, r, st, true)) return rc;
+    return reduce_partials(partial, grad_filter, Gm, K * Co, st);
+}
+
 // ---- facet2vertex backward without a workspace argument -----------------------------------
 // For callers that cannot allocate device memory (stream capture, serving loops, harnesses that forbid it): the
 // partial filter gradients live in a file-scope device array instead of a caller's workspace.  Every GPU the library

@@ -12,14 +12,15 @@ int reduce_partials(const float *partial, float *out, int G, int n, hipStream_t 
 // K == 16 coefficients in 16-byte aligned rows, at least 32 output channels, 32-bit byte offsets into `input`.
 bool f2v_mfma_ok(int64_t Nf, int C, int r, int K, const void *coeff);
 
-int f2v_fwd_mfma(const float *in, const float *filt, const float *coeff, const int *nfcount, const int *rowptr,
-                 const int *colidx, float *out, int64_t NvOut, int C, int r, hipStream_t st);
+// bf16: feature rows (in, out) are bf16 (unsigned short) instead of float
+int f2v_fwd_mfma(const void *in, const float *filt, const float *coeff, const int *nfcount, const int *rowptr,
+                 const int *colidx, void *out, int64_t NvOut, int C, int r, hipStream_t st, bool bf16 = false);
 
 // Backward on the matrix cores: depth multiplier 1 or 2, additionally NvOut * C * r * 4 < 2^32.  G workgroups
 // (f2v_bwd_mfma_blocks) leave G partial filter gradients of 16 * C * r floats in `partial`.
 int f2v_bwd_mfma_blocks(int64_t Nf);
-int f2v_bwd_mfma(const float *gout, const float *in, const float *filt, const float *coeff, const int *face,
-                 const int *nfcount, const int *vtmap, float *gin, float *partial, int G, int64_t Nf, int64_t NvOut,
-                 int C, int r, hipStream_t st);
+int f2v_bwd_mfma(const void *gout, const void *in, const float *filt, const float *coeff, const int *face,
+                 const int *nfcount, const int *vtmap, void *gin, float *partial, int G, int64_t Nf, int64_t NvOut,
+                 int C, int r, hipStream_t st, bool bf16 = false);
 
 }  // namespace pmesh

@@ -36,4 +36,13 @@ def workspace(nbytes, device):
     return torch.empty(max(int(nbytes), 1), dtype=torch.uint8, device=device)
 
 
-F32, I32 = torch.float32, torch.int32
+F32, I32, BF16 = torch.float32, torch.int32, torch.bfloat16
+
+
+def feature_dtype(x, name):
+    """float32, or bfloat16 for the reduced-precision variant (features in bf16 in HBM); anything else raises like
+    a dtype mismatch in the reference's ``data_ptr<float>()``."""
+    if isinstance(x, torch.Tensor) and x.dtype in (F32, BF16):
+        return x.dtype
+    raise RuntimeError("expected scalar type Float (or BFloat16 features) for %s but found %s"
+                       % (name, getattr(x, "dtype", type(x))))

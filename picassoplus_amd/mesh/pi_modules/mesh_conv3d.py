@@ -8,7 +8,7 @@ import torch
 
 from ... import _lib
 from .. import topology
-from ._check import F32, I32, check_input, same_device, stream_of, workspace
+from ._check import BF16, F32, I32, check_input, feature_dtype, same_device, stream_of, workspace
 
 
 # ---------------------------------------------------------------- vertex2facet
@@ -58,7 +58,7 @@ def vertex2facet_backward(grad_output, input, filter, face):
 
 # ---------------------------------------------------------------- facet2vertex
 def _f2v_dims(input, filter, coeff, face, nf_count, vt_map):
-    check_input(input, "input", 2, F32)
+    check_input(input, "input", 2, feature_dtype(input, "input"))
     check_input(filter, "filter", 3, F32)
     check_input(coeff, "coeff", 2, F32)
     check_input(face, "face", 2, I32)
@@ -76,40 +76,43 @@ def _f2v_dims(input, filter, coeff, face, nf_count, vt_map):
 
 
 def facet2vertex_forward(input, filter, coeff, face, nf_count, vt_map):
-    """mesh_conv3d.cpp:33-74 -> (NvOut, C*r)."""
+    """mesh_conv3d.cpp:33-74 -> (NvOut, C*r).  ``input`` may be bfloat16 (features in bf16 in HBM: the output is
+    bfloat16 too, filter and coefficients stay float32)."""
     Nf, C, K, r, NvOut, NvIn = _f2v_dims(input, filter, coeff, face, nf_count, vt_map)
     dev = same_device(input, filter, coeff, face, nf_count, vt_map)
     rowptr, colidx = topology.vertex_csr(face, vt_map, NvOut)
     with torch.cuda.device(dev):
-        out = torch.empty((NvOut, C * r), dtype=F32, device=dev)
-        _lib.call("pmesh_f2v_fwd", input.data_ptr(), filter.data_ptr(), coeff.data_ptr(), nf_count.data_ptr(),
-                  rowptr.data_ptr(), colidx.data_ptr(), out.data_ptr(), Nf, NvOut, C, r, K, stream_of(input))
+        out = torch.empty((NvOut, C * r), dtype=input.dtype, device=dev)
+        _lib.call("pmesh_f2v_fwd_bf16" if input.dtype == BF16 else "pmesh_f2v_fwd", input.data_ptr(), filter.data_ptr(),
+                  coeff.data_ptr(), nf_count.data_ptr(), rowptr.data_ptr(), colidx.data_ptr(), out.data_ptr(), Nf, NvOut,
+                  C, r, K, stream_of(input))
     return out
 
 
 def facet2vertex_backward(grad_output, input, filter, coeff, face, nf_count, vt_map):
-    """mesh_conv3d.cpp:75-122 -> [grad_input (NfIn,C), grad_filter (K,C,r)]."""
+    """mesh_conv3d.cpp:75-122 -> [grad_input (NfIn,C), grad_filter (K,C,r)]; bfloat16 features give a bfloat16
+    grad_input and a float32 grad_filter."""
     Nf, C, K, r, NvOut, NvIn = _f2v_dims(input, filter, coeff, face, nf_count, vt_map)
-    check_input(grad_output, "grad_output", 2, F32)
+    check_input(grad_output, "grad_output", 2, input.dtype)
     if tuple(grad_output.shape) != (NvOut, C * r):
         raise RuntimeError("grad_output must have shape (NvOut, C*r)")
     dev = same_device(grad_output, input, filter, coeff, face, nf_count, vt_map)
     if Nf:
         topology._check_range_cached(face, NvIn)
     with torch.cuda.device(dev):
-        gin = torch.empty((Nf, C), dtype=F32, device=dev)
+        gin = torch.empty((Nf, C), dtype=input.dtype, device=dev)
         gfilt = torch.empty((K, C, r), dtype=F32, device=dev)
         nbytes = _lib.query("pmesh_f2v_bwd_workspace_bytes", C, r, K)
         ws = workspace(nbytes, dev)
-        _lib.call("pmesh_f2v_bwd", grad_output.data_ptr(), input.data_ptr(), filter.data_ptr(), coeff.data_ptr(),
-                  face.data_ptr(), nf_count.data_ptr(), vt_map.data_ptr(), gin.data_ptr(), gfilt.data_ptr(),
-                  ws.data_ptr(), nbytes, Nf, NvIn, NvOut, C, r, K, stream_of(input))
+        _lib.call("pmesh_f2v_bwd_bf16" if input.dtype == BF16 else "pmesh_f2v_bwd", grad_output.data_ptr(), input.data_ptr(),
+                  filter.data_ptr(), coeff.data_ptr(), face.data_ptr(), nf_count.data_ptr(), vt_map.data_ptr(),
+                  gin.data_ptr(), gfilt.data_ptr(), ws.data_ptr(), nbytes, Nf, NvIn, NvOut, C, r, K, stream_of(input))
     return [gin, gfilt]
 
 
 # ---------------------------------------------------------------- facet2facet
 def _f2f_dims(input, filter, bary_coeff, num_texture, forward):
-    check_input(input, "input", 2, F32)
+    check_input(input, "input", 2, feature_dtype(input, "input"))
     check_input(filter, "filter", 3, F32)
     check_input(bary_coeff, "bary_coeff", 2, F32)
     check_input(num_texture, "num_texture", 1, I32)
@@ -127,17 +130,18 @@ def _f2f_dims(input, filter, bary_coeff, num_texture, forward):
 
 
 def facet2facet_forward(input, filter, bary_coeff, num_texture):
-    """mesh_conv3d.cpp:192-228; ``num_texture`` is the inclusive running total per facet."""
+    """mesh_conv3d.cpp:192-228; ``num_texture`` is the inclusive running total per facet.  ``input`` may be bfloat16
+    (features in bf16 in HBM: bfloat16 output, float32 filter and coefficients, one fp16 product per element)."""
     T, Cin, Cout, F, Nf = _f2f_dims(input, filter, bary_coeff, num_texture, True)
     dev = same_device(input, filter, bary_coeff, num_texture)
     with torch.cuda.device(dev):
-        out = torch.empty((Nf, Cout), dtype=F32, device=dev)
+        out = torch.empty((Nf, Cout), dtype=input.dtype, device=dev)
         nbytes = _lib.query("pmesh_f2f_fwd_workspace_bytes", Cin, Cout, F)
         ws = workspace(nbytes, dev)
         order = topology.facet_order(num_texture, T) if Nf else None
-        _lib.call("pmesh_f2f_fwd", input.data_ptr(), filter.data_ptr(), bary_coeff.data_ptr(),
-                  num_texture.data_ptr(), order.data_ptr() if order is not None else None, out.data_ptr(),
-                  ws.data_ptr(), nbytes, T, Nf, Cin, Cout, F, stream_of(input))
+        _lib.call("pmesh_f2f_fwd_bf16" if input.dtype == BF16 else "pmesh_f2f_fwd", input.data_ptr(), filter.data_ptr(),
+                  bary_coeff.data_ptr(), num_texture.data_ptr(), order.data_ptr() if order is not None else None,
+                  out.data_ptr(), ws.data_ptr(), nbytes, T, Nf, Cin, Cout, F, stream_of(input))
     return out
 
 
@@ -151,22 +155,24 @@ def facet2facet_backward_selected(grad_output, input, filter, bary_coeff, num_te
     gradient is not computed and comes back as None (no counterpart in the reference, which always
     computes both)."""
     T, Cin, Cout, F, Nf = _f2f_dims(input, filter, bary_coeff, num_texture, False)
-    check_input(grad_output, "grad_output", 2, F32)
+    check_input(grad_output, "grad_output", 2, input.dtype)
     if tuple(grad_output.shape) != (Nf, Cout):
         raise RuntimeError("grad_output must have shape (NfIn, Cout)")
     dev = same_device(grad_output, input, filter, bary_coeff, num_texture)
+    sfx = "_bf16" if input.dtype == BF16 else ""
     with torch.cuda.device(dev):
-        gin = torch.empty((T, Cin), dtype=F32, device=dev) if needs[0] else None
+        gin = torch.empty((T, Cin), dtype=input.dtype, device=dev) if needs[0] else None
         gfilt = torch.empty((Cout, Cin, F), dtype=F32, device=dev) if needs[1] else None
-        nbytes = _lib.query("pmesh_f2f_bwd_workspace_bytes_for", Nf, Cin, Cout, F)
+        nbytes = (_lib.query("pmesh_f2f_bwd_bf16_workspace_bytes", T, Nf, Cin, Cout, F) if sfx
+                  else _lib.query("pmesh_f2f_bwd_workspace_bytes_for", Nf, Cin, Cout, F))
         ws = workspace(nbytes, dev)
         st = stream_of(input)
         order = topology.facet_order(num_texture, T) if Nf else None
         order_ptr = order.data_ptr() if order is not None else None
         if needs[0]:
-            _lib.call("pmesh_f2f_bwd_texture", grad_output.data_ptr(), filter.data_ptr(), bary_coeff.data_ptr(),
+            _lib.call("pmesh_f2f_bwd_texture" + sfx, grad_output.data_ptr(), filter.data_ptr(), bary_coeff.data_ptr(),
                       num_texture.data_ptr(), order_ptr, gin.data_ptr(), ws.data_ptr(), nbytes, T, Nf, Cin, Cout, F, st)
         if needs[1]:
-            _lib.call("pmesh_f2f_bwd_filter", grad_output.data_ptr(), input.data_ptr(), bary_coeff.data_ptr(),
+            _lib.call("pmesh_f2f_bwd_filter" + sfx, grad_output.data_ptr(), input.data_ptr(), bary_coeff.data_ptr(),
                       num_texture.data_ptr(), order_ptr, gfilt.data_ptr(), ws.data_ptr(), nbytes, T, Nf, Cin, Cout, F, st)
     return [gin, gfilt]

@@ -102,3 +102,27 @@ def texture_case(rng, nf, kmax=5, empty_frac=0.1):
     counts[rng.random(nf) < empty_frac] = 0
     counts, bary, owner = S.texture_points(rng, nf, counts)
     return counts, bary, owner
+
+
+TOL_BF16 = 1e-3   # reduced-precision variant: features in bf16 in HBM, fp32 accumulation
+
+
+def to_bf16(a):
+    """numpy float array -> the same values rounded to bf16 (nearest even), as float64."""
+    return torch.from_numpy(np.ascontiguousarray(a, dtype=np.float32)).to(torch.bfloat16).to(torch.float64).numpy()
+
+
+def assert_close_bf16_store(y, ref, what, tol=TOL_BF16):
+    """A result that left the kernel as bf16: within ``tol`` of the largest reference value before the final rounding
+    to bf16, i.e. |y - ref| <= tol max|ref| + 2^-8 |ref| element by element (2^-8 |ref| bounds the rounding of a
+    value to bf16's eight significant bits)."""
+    y = y.detach().to(torch.float64).cpu().numpy() if isinstance(y, torch.Tensor) else np.asarray(y, np.float64)
+    ref = np.asarray(ref, np.float64)
+    assert y.shape == ref.shape, (y.shape, ref.shape)
+    if ref.size == 0:
+        return 0.0
+    den = np.abs(ref).max()
+    slack = np.abs(y - ref) - 2.0 ** -8 * np.abs(ref)
+    e = float(slack.max() / den) if den > 0 else float(np.abs(y).max())
+    assert e <= tol, "%s: error beyond the bf16 store rounding %.3e > %.1e of max|ref|" % (what, e, tol)
+    return e

@@ -302,6 +302,34 @@ int pmesh_combine_clusters(const int32_t *rep_a, const int32_t *map_a, const int
                            const int32_t *map_b, int32_t *rep_out, int32_t *map_out, int32_t *scratch,
                            int64_t nv_a, int64_t nv_b, pmesh_stream_t stream);
 
+/* ------------------------------------------------------------------ mesh decimation (producer of the cluster maps)
+ * The arithmetic of one decimation round, meshDecimationLauncher (decimate_gpu.cu:618-747), re-specified with fixed
+ * summation orders and total orders so that vt_replace / vt_map are the same on every run (the reference's float
+ * atomics, unstable sorts and tie handling make them vary).  The integer plumbing between these calls -- edge
+ * extraction, sorting, unique, scans -- is the caller's (picassoplus_amd/mesh/pi_modules/decimate.py).
+ *   pmesh_vertex_quadrics    quadric (Nv,10) of every vertex from its facets (initVertexQuadrics :220-247), summed
+ *                            over the vertex CSR in ascending (facet, corner) order; geometry (Nf,5) as
+ *                            pmesh_triangle_geometry; use_area weights a facet by area * 100 / 3, else by 1.
+ *   pmesh_boundary_quadrics  rows (n_edges,10): weighted quadric of the plane through each boundary edge
+ *                            perpendicular to its facet (addBoundaryQuadrics :304-362); the caller adds row i to both
+ *                            end points, in ascending edge order.
+ *   pmesh_edge_costs         contraction cost of each candidate edge (vi, vj) (computeEdgeCost :365-404, with the
+ *                            3 x 3 solve and conditioning test of RrefDim3 :79-193).
+ *   pmesh_cluster_vertices_host  the two greedy passes of clusterVertices (:561-614) over ONE sample's candidate
+ *                            edges in contraction order.  HOST pointers, like the reference's host routine.  An edge
+ *                            of the second pass joins its free end to the cluster of its covered end in either
+ *                            position (the reference contracts a covered non-seed vertex into a free one when they
+ *                            come in that order, which leaves chains the pooling ops cannot follow). */
+int pmesh_vertex_quadrics(const float *geometry, const int32_t *rowptr, const int32_t *colidx, float *quadric,
+                          int64_t Nv, int use_area, pmesh_stream_t stream);
+int pmesh_boundary_quadrics(const float *vertex, const float *geometry, const int32_t *edge_vi, const int32_t *edge_vj,
+                            const int32_t *edge_face, float *rows, int64_t n_edges, int vertex_stride, int use_area,
+                            float wgt_bnd, pmesh_stream_t stream);
+int pmesh_edge_costs(const float *vertex, const float *quadric, const int32_t *edge_vi, const int32_t *edge_vj,
+                     float *cost, int64_t n_edges, int vertex_stride, pmesh_stream_t stream);
+int pmesh_cluster_vertices_host(const int32_t *edge_vi, const int32_t *edge_vj, int64_t n_edges, int32_t vt_start,
+                                int32_t vt_num, int32_t n_remove, int32_t *vt_replace);
+
 /* ------------------------------------------------------------------ pointwise tail of the convs
  * replaces the PyTorch ops that follow every convolution (picasso/mesh/layers.py:114-119, 169-174,
  * 232-238: torch.matmul(outputs, depth_weights) + biases, activation_fn, BatchNorm) by one pass:

@@ -6,12 +6,12 @@ they never fall back to another implementation.
 import ctypes
 import os
 
-from ctypes import c_char_p, c_int, c_int64, c_size_t, c_void_p
+from ctypes import c_char_p, c_float, c_int, c_int64, c_size_t, c_void_p
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 # PICASSO_MESH_LIB points at an alternative build of the same ABI (kernel experiments)
 LIB_PATH = os.environ.get("PICASSO_MESH_LIB") or os.path.join(_HERE, "csrc", "libpicasso_mesh.so")
-ABI_VERSION = 13
+ABI_VERSION = 14
 
 P, I, L, Z = c_void_p, c_int, c_int64, c_size_t
 
@@ -60,6 +60,10 @@ SIGNATURES = {
     "pmesh_texture_fwd": (I, [P, P, P, P, P, P, L, L, L, I, I, P]),
     "pmesh_texture_bwd": (I, [P, P, P, P, P, P, L, L, L, I, P]),
     "pmesh_combine_clusters": (I, [P, P, P, P, P, P, P, L, L, P]),
+    "pmesh_vertex_quadrics": (I, [P, P, P, P, L, I, P]),
+    "pmesh_boundary_quadrics": (I, [P, P, P, P, P, P, L, I, I, c_float, P]),
+    "pmesh_edge_costs": (I, [P, P, P, P, P, L, I, P]),
+    "pmesh_cluster_vertices_host": (I, [P, P, L, I, I, I, P]),
     "pmesh_dense_fwd": (I, [P, P, P, P, P, I, P, P, L, I, I, P]),
     "pmesh_dense_bwd_workspace_bytes": (Z, [L, I, I]),
     "pmesh_dense_bwd": (I, [P, P, P, P, P, P, P, P, P, Z, L, I, I, P]),

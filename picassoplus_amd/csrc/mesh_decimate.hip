@@ -1,0 +1,243 @@
+// One round of quadric-error mesh decimation (the producer of vt_replace / vt_map): the arithmetic kernels and the
+// serial vertex clustering, in a deterministic re-specification of picasso/mesh/pi_modules/source/decimate_gpu.cu.
+//
+// The reference accumulates vertex quadrics with float atomics, sorts with unstable comparators and clusters on the
+// host in whatever order the sorts leave ties in, so its vt_replace / vt_map change from run to run.  Here every
+// sum runs in a fixed order and every sort has a total order:
+//   vertex quadric   face contributions in ascending (facet, corner) order (vertex CSR), then boundary-edge
+//                    contributions in ascending (vi, vj) order (a second CSR over the boundary edges' endpoints)
+//   candidate edges  unique (vi < vj) pairs, ordered by (sample, cost, vi, vj)
+//   clustering       the reference's two greedy passes over that order (clusterVertices, decimate_gpu.cu:561-614)
+// The sorts, scans and compactions between these steps are index plumbing done by the caller (radix sorts of
+// integer keys); this file holds what computes.
+#include "common.h"
+#include "../../include/picasso_mesh.h"
+#include <vector>
+
+namespace pmesh {
+
+constexpr float kAreaMagnitude = 100.0f;        // areas in dm^2 for inputs in metres (decimate_gpu.cu:16)
+constexpr float kRrefEps = 2.220446049250313e-16f;
+constexpr float kRcondEps = 1e-6f;
+
+// plane (n, d) -> the ten distinct entries of [n; d] [n; d]^T in the order q11 q12 q13 q22 q23 q33 q14 q24 q34 q44
+__device__ __forceinline__ void plane_quadric(const float n[3], float d, float (&Q)[10])
+{
+    Q[0] = n[0] * n[0]; Q[1] = n[0] * n[1]; Q[2] = n[0] * n[2];
+    Q[3] = n[1] * n[1]; Q[4] = n[1] * n[2]; Q[5] = n[2] * n[2];
+    Q[6] = n[0] * d;    Q[7] = n[1] * d;    Q[8] = n[2] * d;
+    Q[9] = d * d;
+}
+
+// Quadric of every vertex from its incident facets (decimate_gpu.cu:220-247), summed in adjacency order.
+// geometry rows: unit normal, plane offset d, area.  rowptr / colidx: vertex CSR of `face` (entries 3 f + corner).
+__global__ __launch_bounds__(kBlock) void vertex_quadric_k(const float *__restrict__ geometry, const int *__restrict__ rowptr,
+                                                           const int *__restrict__ colidx, float *__restrict__ quadric,
+                                                           int64_t Nv, int use_area)
+{
+    const int64_t v = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (v >= Nv) return;
+    float S[10];
+#pragma unroll
+    for (int i = 0; i < 10; ++i) S[i] = 0.f;
+    for (int e = rowptr[v]; e < rowptr[v + 1]; ++e) {
+        const float *g = geometry + (int64_t)(colidx[e] / 3) * 5;
+        const float n[3] = {g[0], g[1], g[2]};
+        float Q[10];
+        plane_quadric(n, g[3], Q);
+        const float w = use_area ? g[4] * kAreaMagnitude / 3 : 1.0f;
+#pragma unroll
+        for (int i = 0; i < 10; ++i) S[i] += Q[i] * w;
+    }
+#pragma unroll
+    for (int i = 0; i < 10; ++i) quadric[v * 10 + i] = S[i];
+}
+
+// Weighted quadric of every boundary edge (an edge that belongs to one facet): the plane through the edge
+// perpendicular to that facet (decimate_gpu.cu:304-362).  rows: (nb, 10); each row is added to both end points.
+__global__ __launch_bounds__(kBlock) void boundary_quadric_k(const float *__restrict__ vertex, const float *__restrict__ geometry,
+                                                             const int *__restrict__ edge_vi, const int *__restrict__ edge_vj,
+                                                             const int *__restrict__ edge_face, float *__restrict__ rows,
+                                                             int64_t nb, int D, int use_area, float wgt_bnd)
+{
+    const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= nb) return;
+    const float *pi = vertex + (int64_t)edge_vi[i] * D, *pj = vertex + (int64_t)edge_vj[i] * D;
+    const float *n = geometry + (int64_t)edge_face[i] * 5;
+    const float dx[3] = {pj[0] - pi[0], pj[1] - pi[1], pj[2] - pi[2]};
+    float b[3] = {n[1] * dx[2] - n[2] * dx[1], n[2] * dx[0] - n[0] * dx[2], n[0] * dx[1] - n[1] * dx[0]};
+    float len = sqrtf(b[0] * b[0] + b[1] * b[1] + b[2] * b[2]);
+    len = len > 1e-20f ? len : 1e-20f;
+    b[0] /= len; b[1] /= len; b[2] /= len;
+    const float d = -(b[0] * pi[0] + b[1] * pi[1] + b[2] * pi[2]);
+    const float w = use_area ? (dx[0] * dx[0] + dx[1] * dx[1] + dx[2] * dx[2]) * kAreaMagnitude * wgt_bnd : wgt_bnd;
+    float Q[10];
+    plane_quadric(b, d, Q);
+#pragma unroll
+    for (int k = 0; k < 10; ++k) rows[i * 10 + k] = Q[k] * w;
+}
+
+// x^T A x + 2 b.x + c
+__device__ __forceinline__ float quadric_error(const float x[3], const float A[3][3], const float b[3], float c)
+{
+    return ((x[0] * A[0][0] + x[1] * A[1][0] + x[2] * A[2][0]) * x[0] + (x[0] * A[0][1] + x[1] * A[1][1] + x[2] * A[2][1]) * x[1] +
+            (x[0] * A[0][2] + x[1] * A[1][2] + x[2] * A[2][2]) * x[2]) +
+           (x[0] * b[0] + x[1] * b[1] + x[2] * b[2]) * 2 + c;
+}
+
+// Reduced row echelon form of [A | b | I] with partial pivoting and the negligible-column rule of the reference's
+// RrefDim3 (decimate_gpu.cu:79-193): x = -A^-1 b, and the reciprocal condition number 1 / (|A|_inf |A^-1|_inf).
+__device__ __forceinline__ float solve3(const float A[3][3], const float b[3], float (&x)[3])
+{
+    float M[3][7];
+#pragma unroll
+    for (int r = 0; r < 3; ++r) {
+#pragma unroll
+        for (int c = 0; c < 3; ++c) {
+            M[r][c] = A[r][c];
+            M[r][c + 4] = r == c ? 1.f : 0.f;
+        }
+        M[r][3] = b[r];
+    }
+    float normA = 0.f;
+#pragma unroll
+    for (int r = 0; r < 3; ++r) normA = fmaxf(normA, fabsf(M[r][0]) + fabsf(M[r][1]) + fabsf(M[r][2]));
+    const float tol = kRrefEps * 7 * normA;
+    int i = 0, j = 0;
+    while (i < 3 && j < 7) {
+        float p = fabsf(M[i][j]);
+        int k = i;
+        for (int r = i + 1; r < 3; ++r)
+            if (p < fabsf(M[r][j])) { p = fabsf(M[r][j]); k = r; }
+        if (p <= tol) {
+            for (int r = i; r < 3; ++r) M[r][j] = 0.f;
+            ++j;
+            continue;
+        }
+        for (int c = j; c < 7; ++c) { const float t = M[i][c]; M[i][c] = M[k][c]; M[k][c] = t; }
+        const float pivot = M[i][j];
+        for (int c = j; c < 7; ++c) M[i][c] = M[i][c] / pivot;
+        for (int r = 0; r < 3; ++r) {
+            if (r == i) continue;
+            const float f = M[r][j];
+            for (int c = j; c < 7; ++c) M[r][c] -= f * M[i][c];
+        }
+        ++i;
+        ++j;
+    }
+    x[0] = -M[0][3]; x[1] = -M[1][3]; x[2] = -M[2][3];
+    float normInv = 0.f;
+#pragma unroll
+    for (int r = 0; r < 3; ++r) normInv = fmaxf(normInv, fabsf(M[r][4]) + fabsf(M[r][5]) + fabsf(M[r][6]));
+    return 1.0f / (normA * normInv);
+}
+
+// Cost of contracting each candidate edge (decimate_gpu.cu:365-404): the error of the summed quadric at its
+// minimiser when the 3 x 3 system is well conditioned, else the smaller of the errors at the two end points.
+__global__ __launch_bounds__(kBlock) void edge_cost_k(const float *__restrict__ vertex, const float *__restrict__ quadric,
+                                                      const int *__restrict__ edge_vi, const int *__restrict__ edge_vj,
+                                                      float *__restrict__ cost, int64_t ne, int D)
+{
+    const int64_t e = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (e >= ne) return;
+    const int vi = edge_vi[e], vj = edge_vj[e];
+    float Q[10];
+#pragma unroll
+    for (int k = 0; k < 10; ++k) Q[k] = quadric[(int64_t)vi * 10 + k] + quadric[(int64_t)vj * 10 + k];
+    const float A[3][3] = {{Q[0], Q[1], Q[2]}, {Q[1], Q[3], Q[4]}, {Q[2], Q[4], Q[5]}};
+    const float b[3] = {Q[6], Q[7], Q[8]};
+    float x[3];
+    const float rcond = solve3(A, b, x);
+    if (rcond > kRcondEps) {
+        cost[e] = quadric_error(x, A, b, Q[9]);
+    } else {
+        const float ei = quadric_error(vertex + (int64_t)vi * D, A, b, Q[9]), ej = quadric_error(vertex + (int64_t)vj * D, A, b, Q[9]);
+        cost[e] = ei < ej ? ei : ej;
+    }
+}
+
+}  // namespace pmesh
+
+using namespace pmesh;
+
+extern "C" int pmesh_vertex_quadrics(const float *geometry, const int32_t *rowptr, const int32_t *colidx, float *quadric,
+                                     int64_t Nv, int use_area, pmesh_stream_t stream)
+{
+    clear_error();
+    PM_REQUIRE(Nv >= 0 && Nv <= INT32_MAX, "vertex_quadrics: bad vertex count");
+    if (Nv == 0) return 0;
+    PM_REQUIRE(geometry && rowptr && colidx && quadric, "vertex_quadrics: null pointer");
+    vertex_quadric_k<<<dim3((unsigned)ceil_div(Nv, kBlock)), dim3(kBlock), 0, (hipStream_t)stream>>>(geometry, rowptr, colidx, quadric, Nv, use_area);
+    PM_LAUNCHED("vertex_quadrics");
+    return 0;
+}
+
+extern "C" int pmesh_boundary_quadrics(const float *vertex, const float *geometry, const int32_t *edge_vi, const int32_t *edge_vj,
+                                       const int32_t *edge_face, float *rows, int64_t n_edges, int vertex_stride, int use_area,
+                                       float wgt_bnd, pmesh_stream_t stream)
+{
+    clear_error();
+    PM_REQUIRE(n_edges >= 0 && n_edges <= INT32_MAX && vertex_stride >= 3, "boundary_quadrics: bad sizes");
+    if (n_edges == 0) return 0;
+    PM_REQUIRE(vertex && geometry && edge_vi && edge_vj && edge_face && rows, "boundary_quadrics: null pointer");
+    boundary_quadric_k<<<dim3((unsigned)ceil_div(n_edges, kBlock)), dim3(kBlock), 0, (hipStream_t)stream>>>(
+        vertex, geometry, edge_vi, edge_vj, edge_face, rows, n_edges, vertex_stride, use_area, wgt_bnd);
+    PM_LAUNCHED("boundary_quadrics");
+    return 0;
+}
+
+extern "C" int pmesh_edge_costs(const float *vertex, const float *quadric, const int32_t *edge_vi, const int32_t *edge_vj,
+                                float *cost, int64_t n_edges, int vertex_stride, pmesh_stream_t stream)
+{
+    clear_error();
+    PM_REQUIRE(n_edges >= 0 && n_edges <= INT32_MAX && vertex_stride >= 3, "edge_costs: bad sizes");
+    if (n_edges == 0) return 0;
+    PM_REQUIRE(vertex && quadric && edge_vi && edge_vj && cost, "edge_costs: null pointer");
+    edge_cost_k<<<dim3((unsigned)ceil_div(n_edges, kBlock)), dim3(kBlock), 0, (hipStream_t)stream>>>(vertex, quadric, edge_vi, edge_vj, cost,
+                                                                                                   n_edges, vertex_stride);
+    PM_LAUNCHED("edge_costs");
+    return 0;
+}
+
+// HOST arrays.  The candidate edges of ONE sample in contraction order, its vertex range [vt_start, vt_start + vt_num)
+// and the number of vertices to remove; vt_replace (whole batch, zero on entry for this sample's range) receives
+// -representative for contracted vertices and the member count for representatives.
+extern "C" int pmesh_cluster_vertices_host(const int32_t *edge_vi, const int32_t *edge_vj, int64_t n_edges, int32_t vt_start,
+                                           int32_t vt_num, int32_t n_remove, int32_t *vt_replace)
+{
+    clear_error();
+    PM_REQUIRE(n_edges >= 0 && vt_num >= 0, "cluster_vertices_host: bad sizes");
+    if (n_edges == 0 || n_remove <= 0) return 0;
+    PM_REQUIRE(edge_vi && edge_vj && vt_replace, "cluster_vertices_host: null pointer");
+    std::vector<char> covered((size_t)vt_num, 0);
+    auto in_range = [&](int v) { return v >= vt_start && v - vt_start < vt_num; };
+    int removed = 0;
+    // first pass: disjoint pairs, cheapest edges first; vi is contracted into vj (decimate_gpu.cu:568-585)
+    for (int64_t i = 0; i < n_edges && removed < n_remove; ++i) {
+        const int vi = edge_vi[i], vj = edge_vj[i];
+        PM_REQUIRE(in_range(vi) && in_range(vj), "cluster_vertices_host: edge (%d, %d) outside the sample's vertex range", vi, vj);
+        if (vi != vj && vj != 0 && !covered[vi - vt_start] && !covered[vj - vt_start]) {   // -0 cannot say 'contracted into vertex 0'
+            vt_replace[vi] = -vj;
+            vt_replace[vj] += 1;
+            covered[vi - vt_start] = covered[vj - vt_start] = 1;
+            ++removed;
+        }
+    }
+    // second pass: a vertex still free joins the cluster of a covered neighbour, cheapest edges first (:587-613).
+    // (An edge joins its FREE end to its covered end whichever of the two positions they are in; the reference
+    // takes only a pair member in second position for the swap and otherwise contracts a covered vertex into a
+    // free one, which leaves a chain vt_replace -> vt_replace that the pooling kernels cannot follow.)
+    for (int64_t i = 0; i < n_edges && removed < n_remove; ++i) {
+        int a = edge_vi[i], b = edge_vj[i];
+        const bool ca = covered[a - vt_start] != 0, cb = covered[b - vt_start] != 0;
+        if (ca == cb || a == b) continue;                           // both covered, or both free (the first pass ran out of budget)
+        if (cb) { const int t = a; a = b; b = t; }        // a: covered, b: free
+        if (vt_replace[a] < 0) a = -vt_replace[a];        // representative of a's cluster
+        if (a == 0) continue;                             // -0 cannot say 'contracted into vertex 0'
+        vt_replace[b] = -a;
+        vt_replace[a] += 1;
+        covered[b - vt_start] = 2;
+        ++removed;
+    }
+    return 0;
+}

@@ -1,0 +1,190 @@
+"""Quadric-error mesh decimation: API of picasso/mesh/pi_modules/decimate.py (``mesh_decimation_`` and the
+``simplify`` round of the reference's ``mesh_decimation`` extension, decimate.cpp:21-89), deterministic.
+
+One round (``simplify``) = vertex quadrics from the facets and the boundary edges -> cost of every candidate
+edge -> greedy vertex clustering in cost order -> cluster maps, contracted vertices, remapped facets.  The
+reference gets different ``vt_replace`` / ``vt_map`` from run to run (float atomics, unstable sorts, ties broken by
+whatever order a sort leaves); here every sum has a fixed order and the candidate edges a total order
+(sample, cost, vi, vj), so the maps are a function of the input alone.  The arithmetic runs in native kernels
+(``pmesh_vertex_quadrics``, ``pmesh_boundary_quadrics``, ``pmesh_edge_costs``), the serial clustering in a native host
+routine as in the reference (``pmesh_cluster_vertices_host``), the contraction is the average pooling op over the new
+maps; sorting / unique / scans of integer keys between them are PyTorch ops.
+"""
+import ctypes
+
+import numpy as np
+import torch
+
+from ... import _lib
+from .. import topology
+from . import mesh_pool3d
+from ._check import F32, I32, check_input, same_device, stream_of
+from .geometry import combine_clusters_, compute_triangle_geometry_, count_vertex_adjface_  # noqa: F401 (decimate.py:53-93)
+
+
+def vertex_quadrics(vertexIn, faceIn, geometryIn, useArea=True, wgtBnd=5.0):
+    """Quadric (Nv, 10) of every vertex and the candidate edges of the batch.
+
+    returns (quadric, edge_vi, edge_vj): the unique edges (vi < vj, int32) in ascending (vi, vj) order."""
+    check_input(vertexIn, "vertexIn", 2, F32)
+    check_input(faceIn, "faceIn", 2, I32)
+    check_input(geometryIn, "geometryIn", 2, F32)
+    Nv, D = vertexIn.shape
+    Nf = faceIn.shape[0]
+    if D < 3:
+        raise RuntimeError("The shape of input vertex should be (Nv, 3+)).")
+    if faceIn.shape[1] != 3:
+        raise RuntimeError("The shape of input face should be (Nf, 3)).")
+    if tuple(geometryIn.shape) != (Nf, 5):
+        raise RuntimeError("The shape of input face normals should be (Nf, 5)).")
+    dev = same_device(vertexIn, faceIn, geometryIn)
+    st = stream_of(vertexIn)
+    rowptr, colidx = topology.vertex_csr(faceIn, None, Nv)
+    with torch.cuda.device(dev):
+        quadric = torch.empty((Nv, 10), dtype=F32, device=dev)
+        _lib.call("pmesh_vertex_quadrics", geometryIn.data_ptr(), rowptr.data_ptr(), colidx.data_ptr(), quadric.data_ptr(),
+                  Nv, 1 if useArea else 0, st)
+        # the three edges of every facet as (lower, higher) vertex pairs; one 64-bit key per edge
+        f = faceIn.long()
+        a = torch.stack([f[:, 0], f[:, 0], f[:, 1]], 1).reshape(-1)
+        b = torch.stack([f[:, 1], f[:, 2], f[:, 2]], 1).reshape(-1)
+        key, order = torch.sort(torch.minimum(a, b) * Nv + torch.maximum(a, b), stable=True)
+        ukey, counts = torch.unique_consecutive(key, return_counts=True)
+        vi, vj = torch.div(ukey, Nv, rounding_mode="floor"), ukey % Nv
+        ok = vi != vj                                            # a facet with a repeated vertex has no such edge
+        if wgtBnd > 0:
+            first = torch.cumsum(counts, 0) - counts
+            bnd = (counts == 1) & ok                             # an edge that belongs to exactly one facet
+            nb = int(bnd.sum())
+            if nb:
+                bvi, bvj = vi[bnd].to(I32), vj[bnd].to(I32)
+                bface = torch.div(order[first[bnd]], 3, rounding_mode="floor").to(I32)
+                rows = torch.empty((nb, 10), dtype=F32, device=dev)
+                _lib.call("pmesh_boundary_quadrics", vertexIn.data_ptr(), geometryIn.data_ptr(), bvi.data_ptr(), bvj.data_ptr(),
+                          bface.data_ptr(), rows.data_ptr(), nb, D, 1 if useArea else 0, float(wgtBnd), st)
+                # every row goes to both end points: a segmented sum over the end points in ascending edge order
+                ends = torch.cat([bvi, bvj]).long()
+                _, members = torch.sort(ends, stable=True)
+                ptr = torch.zeros(Nv + 1, dtype=torch.int64, device=dev)
+                ptr[1:] = torch.cumsum(torch.bincount(ends, minlength=Nv), 0)
+                quadric = quadric + _segment_row_sum(torch.cat([rows, rows]), ptr.to(I32), members.to(I32), Nv)
+    return quadric, vi[ok].to(I32).contiguous(), vj[ok].to(I32).contiguous()
+
+
+def _segment_row_sum(rows, rowptr, members, n_out):
+    """out[v] = sum of rows[members[rowptr[v] .. rowptr[v+1])] in that order (the segmented row sum of the unpooling
+    gradient, used here for quadrics)."""
+    out = torch.empty((n_out, rows.shape[1]), dtype=F32, device=rows.device)
+    _lib.call("pmesh_unpool_bwd", rows.data_ptr(), rowptr.data_ptr(), members.data_ptr(), out.data_ptr(), n_out,
+              rows.shape[0], rows.shape[1], stream_of(rows))
+    return out
+
+
+def edge_costs(vertexIn, quadric, edge_vi, edge_vj):
+    """Contraction cost (float32) of every candidate edge."""
+    check_input(quadric, "quadric", 2, F32)
+    check_input(edge_vi, "edge_vi", 1, I32)
+    check_input(edge_vj, "edge_vj", 1, I32)
+    dev = same_device(vertexIn, quadric, edge_vi, edge_vj)
+    with torch.cuda.device(dev):
+        cost = torch.empty(edge_vi.shape[0], dtype=F32, device=dev)
+        _lib.call("pmesh_edge_costs", vertexIn.data_ptr(), quadric.data_ptr(), edge_vi.data_ptr(), edge_vj.data_ptr(),
+                  cost.data_ptr(), edge_vi.shape[0], vertexIn.shape[1], stream_of(vertexIn))
+    return cost
+
+
+def contraction_order(cost, edge_vi, nvIn_cumsum):
+    """Order of the candidate edges: by sample, then cost (NaN last), then (vi, vj) -- the edges come in (vi, vj) order,
+    so two stable sorts do it.  returns (permutation, sample of each edge in that order)."""
+    by_cost = torch.sort(cost, stable=True).indices
+    sample = torch.bucketize(edge_vi[by_cost].long(), nvIn_cumsum.long(), right=True)
+    by_sample = torch.sort(sample, stable=True)
+    return by_cost[by_sample.indices], by_sample.values
+
+
+def cluster_vertices(edge_vi, edge_vj, sample, nvIn_cumsum, nv2Remove, Nv):
+    """The two greedy passes per sample on the host (as the reference runs them): -> vt_replace int32 (Nv,) on the host."""
+    vi = np.ascontiguousarray(edge_vi.cpu().numpy(), dtype=np.int32)
+    vj = np.ascontiguousarray(edge_vj.cpu().numpy(), dtype=np.int32)
+    smp = sample.cpu().numpy()
+    ends = np.asarray(nvIn_cumsum.cpu().numpy(), dtype=np.int64)
+    budget = np.asarray(nv2Remove.cpu().numpy(), dtype=np.int64)
+    vt_replace = np.zeros(Nv, dtype=np.int32)
+    bounds = np.searchsorted(smp, np.arange(len(ends) + 1))
+    P = ctypes.c_void_p
+    for b in range(len(ends)):
+        e0, e1 = int(bounds[b]), int(bounds[b + 1])
+        start = int(ends[b - 1]) if b else 0
+        if e1 > e0 and budget[b] > 0:
+            _lib.call("pmesh_cluster_vertices_host", P(vi.ctypes.data + 4 * e0), P(vj.ctypes.data + 4 * e0), e1 - e0, start,
+                      int(ends[b]) - start, int(budget[b]), P(vt_replace.ctypes.data))
+    return vt_replace
+
+
+def simplify(vertexIn, faceIn, geometryIn, nvIn_cumsum, mfIn_cumsum, nv2Remove, useArea=True, wgtBnd=5.0):
+    """One decimation round: the reference's ``mesh_decimation.simplify`` (decimate.cpp:21-89,
+    decimate_gpu.cu:618-747).  ``nvIn_cumsum`` / ``mfIn_cumsum``: running totals of vertices / facets per sample.
+
+    returns [vertexOut (Nv, D), faceOut (Nf, 3), isDegenerate (Nf,) bool, vtReplace (Nv,), vtMap (Nv,), nvOut (B,),
+    mfOut (B,)]: contracted vertices in the rows of the surviving input vertices (filter with ``vtMap >= 0``), facets
+    renumbered to the output vertices (filter with ``~isDegenerate``)."""
+    for name, t in (("nvIn", nvIn_cumsum), ("mfIn", mfIn_cumsum), ("nv2Remove", nv2Remove)):
+        check_input(t, name, 1, I32)
+    useArea, wgtBnd = bool(useArea), float(wgtBnd)
+    Nv, D = vertexIn.shape
+    dev = vertexIn.device
+    quadric, evi, evj = vertex_quadrics(vertexIn, faceIn, geometryIn, useArea, wgtBnd)
+    cost = edge_costs(vertexIn, quadric, evi, evj)
+    perm, sample = contraction_order(cost, evi, nvIn_cumsum)
+    vt_replace = torch.from_numpy(cluster_vertices(evi[perm], evj[perm], sample, nvIn_cumsum, nv2Remove, Nv)).to(dev)
+    with torch.cuda.device(dev):
+        ids = torch.arange(Nv, dtype=I32, device=dev)
+        rep = torch.where(vt_replace < 0, -vt_replace, ids).long()
+        new_face = rep[faceIn.long()]
+        degenerate = (new_face[:, 0] == new_face[:, 1]) | (new_face[:, 0] == new_face[:, 2]) | (new_face[:, 1] == new_face[:, 2])
+        kept = torch.zeros(Nv, dtype=torch.int64, device=dev)
+        kept[new_face[~degenerate].reshape(-1)] = 1
+        # vertices that keep a facet are numbered in order; contracted vertices and those left without a facet get -1
+        vt_map = torch.where(kept > 0, torch.cumsum(kept, 0) - 1, torch.full_like(kept, -1)).to(I32)
+        face_out = torch.where(degenerate[:, None], new_face, vt_map.long()[new_face]).to(I32)
+        sample_v = torch.bucketize(ids.long(), nvIn_cumsum.long(), right=True)
+        sample_f = torch.bucketize(torch.arange(faceIn.shape[0], device=dev), mfIn_cumsum.long(), right=True)
+        B = nvIn_cumsum.shape[0]
+        nv_out = torch.bincount(sample_v[kept > 0], minlength=B)[:B].to(I32)
+        mf_out = torch.bincount(sample_f[~degenerate], minlength=B)[:B].to(I32)
+        # contracted position = mean of the cluster's vertices (all D columns) in the row of its representative; rows of
+        # contracted vertices stay zero (decimate_gpu.cu:401-441)
+        is_rep = vt_replace >= 0
+        rep_row = torch.where(is_rep, torch.cumsum(is_rep, 0) - 1, torch.full_like(kept, -1)).to(I32)
+        n_rep = int(is_rep.sum())
+        vertex_out = torch.zeros((Nv, D), dtype=F32, device=dev)
+        if n_rep:
+            vertex_out[is_rep] = mesh_pool3d.avg_forward(vertexIn, vt_replace, rep_row, torch.empty((n_rep, 1), dtype=F32, device=dev))
+    return [vertex_out, face_out, degenerate, vt_replace, vt_map, nv_out, mf_out]
+
+
+def mesh_decimation_(vertexIn, faceIn, geometryIn, nvIn, mfIn, nvOut, useArea=True, wgtBnd=5):
+    """Decimate every sample of the batch to (about) ``nvOut`` vertices (decimate.py:5-52): rounds of ``simplify``
+    until no sample has vertices left to remove, the rounds' cluster maps composed with ``combine_clusters_``.
+
+    returns (vertexOut, faceOut, geometryOut, nvOut, mfOut, vtReplace, vtMap) with vtReplace / vtMap over the INPUT
+    vertices: the index maps the pooling / unpooling ops and the strided facet2vertex take."""
+    dev = vertexIn.device
+    nv2Remove = (nvIn - nvOut).to(I32)
+    repIn = torch.zeros(vertexIn.shape[0], dtype=I32, device=dev)
+    mapIn = torch.arange(vertexIn.shape[0], dtype=I32, device=dev)
+    while bool(torch.any(nv2Remove > 0)):
+        nv_cum = torch.cumsum(nvIn, 0, dtype=I32)
+        mf_cum = torch.cumsum(mfIn, 0, dtype=I32)
+        vertexOut, faceOut, isDegenerate, repOut, mapOut, nvOut, mfOut = simplify(
+            vertexIn, faceIn, geometryIn, nv_cum, mf_cum, nv2Remove.contiguous(), useArea, wgtBnd)
+        removed = nvIn - nvOut
+        if not bool(torch.any(removed > 0)):
+            break                                     # nothing left that can be contracted (no candidate edges)
+        faceIn = faceOut[~isDegenerate].contiguous()
+        vertexIn = vertexOut[mapOut >= 0].contiguous()
+        geometryIn = compute_triangle_geometry_(vertexIn, faceIn)
+        nv2Remove = (nv2Remove - removed).to(I32)
+        repIn, mapIn = combine_clusters_(repIn, mapIn, repOut, mapOut)
+        nvIn, mfIn = nvOut, mfOut
+    return vertexIn, faceIn, geometryIn, nvIn, mfIn, repIn, mapIn

@@ -1,6 +1,6 @@
 """Per-level producers of the convolution inputs: adjacent-facet counts of the output vertices,
 triangle geometry, oriented normals with their basis coefficients, and the composition of two decimation steps' cluster maps, with the reference's function
-names (picasso/mesh/pi_modules/decimate.py:53-93).  Mesh decimation itself is not part of this package."""
+names (picasso/mesh/pi_modules/decimate.py:53-93).  The decimation that produces the cluster maps is in decimate.py."""
 import torch
 
 from ... import _lib

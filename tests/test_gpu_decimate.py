@@ -1,0 +1,156 @@
+"""Mesh decimation on the GPU against oracle/decimate_ref.py.
+
+Floating-point stages (vertex quadrics, edge costs, contracted positions) within a tolerance of the float64 oracle;
+integer stages (candidate edges, cluster maps, facets, counts) bit-exact against the oracle run on the SAME costs
+(the device computes them in float32, so the order of near-equal costs is the device's; everything after the costs
+is a function of their order alone).  The whole loop through the properties its callers rely on."""
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import decimate_ref as D
+from oracle import torch_ref
+from picassoplus_amd.mesh.pi_modules import decimate, pool3d
+from picassoplus_amd.mesh.pi_modules.geometry import compute_triangle_geometry_
+from util import dev, mesh_case
+
+pytestmark = pytest.mark.gpu
+I32 = torch.int32
+
+
+def say(*a):
+    print(*a, flush=True)
+    sys.stdout.flush()
+
+
+def batch(names, seed=0):
+    vs, fs, nv, mf, off = [], [], [], [], 0
+    for k, name in enumerate(names):
+        v, f = mesh_case(name, seed + k)
+        v = np.asarray(v, np.float32)[:, :3] + np.float32(3.0 * k)
+        vs.append(v)
+        fs.append(f.astype(np.int32) + off)
+        nv.append(len(v))
+        mf.append(len(f))
+        off += len(v)
+    return np.concatenate(vs), np.concatenate(fs), np.array(nv, np.int32), np.array(mf, np.int32)
+
+
+CASES = [("tetra",), ("grid2",), ("sphere2",), ("torus", "sphere3"), ("room_small",), ("shapes_small", "fans")]
+
+
+@pytest.mark.parametrize("names", CASES, ids=lambda n: "+".join(n))
+@pytest.mark.parametrize("use_area,wgt_bnd", [(True, 5.0), (False, 5.0), (True, 0.0)])
+def test_quadrics_and_costs_match_oracle(cuda, names, use_area, wgt_bnd):
+    say("case decimate quadrics", names, use_area, wgt_bnd)
+    v, f, nv, mf = batch(names)
+    vx, fc = dev(v, cuda), dev(f, cuda)
+    geo = compute_triangle_geometry_(vx, fc)
+    g = geo.cpu().numpy()
+    q, evi, evj = decimate.vertex_quadrics(vx, fc, geo, use_area, wgt_bnd)
+    wq, wi, wj = D.vertex_quadrics(v, f, g, use_area, wgt_bnd)
+    assert np.array_equal(evi.cpu().numpy(), wi) and np.array_equal(evj.cpu().numpy(), wj)
+    qn = q.cpu().numpy()
+    row = np.abs(wq).max(1, keepdims=True)
+    assert np.all(np.abs(qn - wq) <= 2e-6 * np.maximum(row, 1e-30)), "vertex quadrics"
+    cost = decimate.edge_costs(vx, q, evi, evj).cpu().numpy()
+    want, rcond = D.edge_costs(v, qn, wi, wj, return_rcond=True)           # float64 arithmetic on the device's quadrics
+    Q = qn[wi].astype(np.float64) + qn[wj]
+    reach = 1 + np.maximum((v[wi].astype(np.float64) ** 2).sum(1), (v[wj].astype(np.float64) ** 2).sum(1))
+    scale = np.abs(Q).sum(1) * reach
+    # the branch is taken on a float32 reciprocal condition number: compare where the float64 one is clear of the
+    # threshold; at a well-conditioned minimiser float32 elimination loses about 1 / rcond ulps
+    clear = (rcond > 4 * D.RCOND_EPS) | (rcond < 0.25 * D.RCOND_EPS)
+    loss = np.where(rcond > D.RCOND_EPS, 1 / np.maximum(rcond, 1e-30), 1.0)
+    tol = 4e-7 * scale * np.maximum(loss, 8.0)
+    bad = clear & ~(np.abs(cost - want) <= tol)
+    assert not bad.any(), "edge costs: %d of %d off, worst %g" % (bad.sum(), len(bad), np.abs(cost - want)[bad].max())
+    assert clear.mean() > 0.9
+
+
+@pytest.mark.parametrize("names,frac", [(("tetra",), 0.5), (("grid2",), 0.4), (("sphere2",), 0.5), (("torus", "sphere3"), 0.3),
+                                        (("room_small",), 0.5), (("shapes_small", "fans"), 0.45), (("sphere3", "torus"), 0.0)],
+                         ids=lambda n: "+".join(n) if isinstance(n, tuple) else str(n))
+def test_simplify_round_is_exact_given_the_costs(cuda, names, frac):
+    say("case decimate simplify", names, frac)
+    v, f, nv, mf = batch(names)
+    vx, fc = dev(v, cuda), dev(f, cuda)
+    geo = compute_triangle_geometry_(vx, fc)
+    nv_cum, mf_cum = np.cumsum(nv).astype(np.int32), np.cumsum(mf).astype(np.int32)
+    n_remove = (nv * frac).astype(np.int32)
+    out = decimate.simplify(vx, fc, geo, dev(nv_cum, cuda), dev(mf_cum, cuda), dev(n_remove, cuda), True, 5.0)
+    again = decimate.simplify(vx.clone(), fc.clone(), geo.clone(), dev(nv_cum, cuda), dev(mf_cum, cuda), dev(n_remove, cuda), True, 5.0)
+    for a, b in zip(out, again):
+        assert torch.equal(a, b), "two runs differ"
+    q, evi, evj = decimate.vertex_quadrics(vx, fc, geo, True, 5.0)
+    cost = decimate.edge_costs(vx, q, evi, evj).cpu().numpy()
+    want = D.simplify(v, f, geo.cpu().numpy(), nv_cum, mf_cum, n_remove, True, 5.0, cost=cost)
+    vo, fo, deg, rep, vmap, nv_o, mf_o = (t.cpu().numpy() for t in out)
+    assert np.array_equal(rep, want[3]), "vt_replace"
+    assert np.array_equal(vmap, want[4]), "vt_map"
+    assert np.array_equal(deg, want[2]) and np.array_equal(fo, want[1]), "facets"
+    assert np.array_equal(nv_o, want[5]) and np.array_equal(mf_o, want[6]), "counts"
+    assert np.abs(vo - want[0]).max() <= 1e-6 * max(np.abs(v).max(), 1.0), "contracted positions"
+    assert (rep < 0).sum() <= n_remove.sum()
+    if frac == 0.0:
+        assert not rep.any() and np.array_equal(vmap, np.arange(len(v))) and not deg.any()
+
+
+def test_decimation_loop_feeds_the_pooling_ops(cuda):
+    say("case decimate loop")
+    v, f, nv, mf = batch(("sphere3", "torus", "room_small"))
+    vx, fc = dev(v, cuda), dev(f, cuda)
+    geo = compute_triangle_geometry_(vx, fc)
+    target = (nv // 3).astype(np.int32)
+    res = decimate.mesh_decimation_(vx, fc, geo, dev(nv, cuda), dev(mf, cuda), dev(target, cuda))
+    res2 = decimate.mesh_decimation_(vx, fc, geo, dev(nv, cuda), dev(mf, cuda), dev(target, cuda))
+    for a, b in zip(res, res2):
+        assert torch.equal(a, b), "two runs differ"
+    vo, fo, go, nv_o, mf_o, rep, vmap = res
+    nv_o, mf_o = nv_o.cpu().numpy(), mf_o.cpu().numpy()
+    say("  vertices", nv.tolist(), "->", nv_o.tolist(), "facets", mf.tolist(), "->", mf_o.tolist())
+    # closed surfaces reach their target exactly; the open room may lose vertices whose facets all collapse
+    assert nv_o[0] == target[0] and nv_o[1] == target[1] and nv_o[2] <= target[2]
+    assert mf_o[0] == 2 * nv_o[0] - 4 and mf_o[1] == 2 * nv_o[1]           # Euler: sphere, torus
+    assert vo.shape[0] == nv_o.sum() and fo.shape[0] == mf_o.sum() and go.shape == (fo.shape[0], 5)
+    fo_n = fo.cpu().numpy()
+    cum = np.concatenate([[0], np.cumsum(nv_o)])
+    fcum = np.concatenate([[0], np.cumsum(mf_o)])
+    for b in range(3):                                                      # facets stay inside their own sample
+        part = fo_n[fcum[b]:fcum[b + 1]]
+        assert part.min() >= cum[b] and part.max() < cum[b + 1]
+    assert torch.equal(go, compute_triangle_geometry_(vo, fo))
+    # the maps over the input vertices are what pooling takes
+    rep_n, map_n = rep.cpu().numpy(), vmap.cpu().numpy()
+    head = np.where(rep_n < 0, -rep_n, np.arange(len(v)))
+    assert np.all(rep_n[head] >= 0)
+    x = np.random.default_rng(0).normal(size=(len(v), 8)).astype(np.float32)
+    T = torch.from_numpy
+    pooled = pool3d.maxPool(dev(x, cuda), rep, vmap, vo)
+    want, _ = torch_ref.maxpool_fwd(T(x), T(rep_n), T(map_n), vo.shape[0])
+    assert np.array_equal(pooled.cpu().numpy(), want.numpy())
+    # positions are means over clusters of means: the pooled input positions stay close to them
+    centre = pool3d.avgPool(vx, rep, vmap, vo).cpu().numpy()
+    used = np.bincount(map_n[head][map_n[head] >= 0], minlength=vo.shape[0]) > 0
+    assert used.all()
+    assert np.abs(centre - vo.cpu().numpy()).max() < 0.35
+
+
+def test_decimate_argument_errors(cuda):
+    say("case decimate errors")
+    v, f, nv, mf = batch(("sphere1",))
+    vx, fc = dev(v, cuda), dev(f, cuda)
+    geo = compute_triangle_geometry_(vx, fc)
+    args = [dev(np.cumsum(nv).astype(np.int32), cuda), dev(np.cumsum(mf).astype(np.int32), cuda), dev((nv // 2).astype(np.int32), cuda)]
+    with pytest.raises(RuntimeError):
+        decimate.simplify(vx.cpu(), fc, geo, *args)
+    with pytest.raises(RuntimeError):
+        decimate.simplify(vx, fc.long(), geo, *args)
+    with pytest.raises(RuntimeError):
+        decimate.simplify(vx, fc, geo[:, :4].contiguous(), *args)
+    with pytest.raises(RuntimeError):
+        decimate.simplify(vx[:, :2].contiguous(), fc, geo, *args)
+    with pytest.raises(RuntimeError):
+        decimate.simplify(vx, fc, geo, args[0].long(), args[1], args[2])

@@ -265,3 +265,27 @@ def test_adjacency_cache_discipline():
         T.MAX_BYTES = old
         T.clear_cache()
     assert T.cache_bytes() == 0
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_host_vertex_clustering_matches_the_oracle(seed):
+    """pmesh_cluster_vertices_host runs on host arrays (no device needed): the two greedy passes over the candidate
+    edges, bit-exact against the oracle's statement of them."""
+    import ctypes
+
+    from oracle import decimate_ref
+    rng = np.random.default_rng(seed)
+    num, start = (300, 0) if seed % 2 else (120, 50)
+    pairs = sorted({tuple(sorted(p)) for p in rng.integers(start, start + num, (4 * num, 2)).tolist() if p[0] != p[1]})
+    order = rng.permutation(len(pairs))
+    vi = np.ascontiguousarray(np.array(pairs, np.int32)[order, 0])
+    vj = np.ascontiguousarray(np.array(pairs, np.int32)[order, 1])
+    for budget in (0, 1, num // 5, num):
+        got = np.zeros(start + num, np.int32)
+        _lib.call("pmesh_cluster_vertices_host", vi.ctypes.data, vj.ctypes.data, len(vi), start, num, budget, got.ctypes.data)
+        want = np.zeros(start + num, np.int32)
+        decimate_ref.cluster_vertices(vi, vj, start, num, budget, want)
+        assert np.array_equal(got, want)
+        assert (got < 0).sum() <= budget
+    with pytest.raises(RuntimeError):                       # an edge that leaves the sample's vertex range
+        _lib.call("pmesh_cluster_vertices_host", vi.ctypes.data, vj.ctypes.data, len(vi), start, num // 2, num, got.ctypes.data)

@@ -154,3 +154,31 @@ def test_decimate_argument_errors(cuda):
         decimate.simplify(vx[:, :2].contiguous(), fc, geo, *args)
     with pytest.raises(RuntimeError):
         decimate.simplify(vx, fc, geo, args[0].long(), args[1], args[2])
+
+
+def test_mesh_hierarchy_levels_feed_a_network_block(cuda):
+    """MeshHierarchy (picasso/mesh/utils.py:32-58) in both constructor forms: every level is a valid mesh, the maps of
+    a level pool the features of the level above, and the strided form honours the floor on the vertex count."""
+    say("case decimate hierarchy")
+    from picassoplus_amd.mesh.utils import MeshHierarchy, count_vertex_adjface
+    v, f, nv, mf = batch(("sphere3", "torus"))
+    vx, fc = dev(v, cuda), dev(f, cuda)
+    levels = MeshHierarchy([2, 3], [100, 150], True, 1.0)(vx, fc, dev(nv, cuda), dev(mf, cuda))
+    assert len(levels) == 3 and levels[0][5] is None and levels[0][6] is None
+    n_prev = nv
+    for lvl, (vl, fl, gl, nvl, mfl, rep, vmap) in enumerate(levels):
+        nvl_n, mfl_n = nvl.cpu().numpy(), mfl.cpu().numpy()
+        assert vl.shape[0] == nvl_n.sum() and fl.shape[0] == mfl_n.sum() and gl.shape == (fl.shape[0], 5)
+        assert int(fl.max()) < vl.shape[0] and int(fl.min()) >= 0
+        if lvl:
+            want = np.maximum(n_prev // [2, 3][lvl - 1], [100, 150][lvl - 1])
+            assert np.array_equal(nvl_n, want), (nvl_n, want)          # closed surfaces reach the target exactly
+            above = levels[lvl - 1][0]
+            assert rep.shape[0] == above.shape[0] and vmap.shape[0] == above.shape[0]
+            pooled = pool3d.avgPool(above, rep, vmap, vl)
+            assert pooled.shape == vl.shape and bool(torch.isfinite(pooled).all())
+            nf_count = count_vertex_adjface(fl, torch.arange(vl.shape[0], dtype=I32, device=cuda), vl)
+            assert int(nf_count.min()) >= 1 and int(nf_count.sum()) == 3 * fl.shape[0]
+        n_prev = nvl_n
+    fixed = MeshHierarchy([dev(np.array([300, 200], np.int32), cuda)], True, 1.0)(vx, fc, dev(nv, cuda), dev(mf, cuda))
+    assert fixed[1][3].cpu().tolist() == [300, 200]

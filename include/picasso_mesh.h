@@ -149,6 +149,17 @@ int pmesh_f2f_fwd(const float *texture, const float *filter, const float *bary_c
                   const int32_t *cum_texture, const int32_t *facet_order, float *output, void *workspace,
                   size_t workspace_bytes, int64_t T, int64_t Nf, int Cin, int Cout, int F,
                   pmesh_stream_t stream);
+/* The same with the module's tail on the store (picasso/mesh/layers.py:59-63: outputs + biases, activation_fn; the
+ * per-channel scale and shift carry a batch norm that only applies its running statistics):
+ *   output = act(conv + bias) * scale + shift      bias, scale, shift (Cout) each optional; relu: 0 / 1
+ * relu_bits (NULL, or Nf * Cout/32 words when Cout % 32 == 0 and output is 16-byte aligned): bit c % 32 of word
+ * [f][c / 32] is set where the ReLU let the value through, the form pmesh_bias_act_bwd takes.  The fp16 kernels for 16
+ * coefficients apply the tail as they store; every other shape runs pmesh_f2f_fwd and then pmesh_bias_act_fwd in place. */
+int pmesh_f2f_fwd_act(const float *texture, const float *filter, const float *bary_coeff,
+                      const int32_t *cum_texture, const int32_t *facet_order, const float *bias,
+                      const float *scale, const float *shift, int relu, float *output, uint32_t *relu_bits,
+                      void *workspace, size_t workspace_bytes, int64_t T, int64_t Nf, int Cin, int Cout,
+                      int F, pmesh_stream_t stream);
 
 /* grad_texture (T,Cin), grad_filter (Cout,Cin,F).
  * workspace: pmesh_f2f_bwd_workspace_bytes(Cin,Cout,F), 16-byte aligned; the two halves may share

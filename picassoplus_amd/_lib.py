@@ -11,7 +11,7 @@ from ctypes import c_char_p, c_float, c_int, c_int64, c_size_t, c_void_p
 _HERE = os.path.dirname(os.path.abspath(__file__))
 # PICASSO_MESH_LIB points at an alternative build of the same ABI (kernel experiments)
 LIB_PATH = os.environ.get("PICASSO_MESH_LIB") or os.path.join(_HERE, "csrc", "libpicasso_mesh.so")
-ABI_VERSION = 14
+ABI_VERSION = 15
 
 P, I, L, Z = c_void_p, c_int, c_int64, c_size_t
 
@@ -33,6 +33,7 @@ SIGNATURES = {
     "pmesh_f2v_bwd_static": (I, [P, P, P, P, P, P, P, P, P, L, L, L, I, I, I, P]),
     "pmesh_f2f_fwd_workspace_bytes": (Z, [I, I, I]),
     "pmesh_f2f_fwd": (I, [P, P, P, P, P, P, P, Z, L, L, I, I, I, P]),
+    "pmesh_f2f_fwd_act": (I, [P, P, P, P, P, P, P, P, I, P, P, P, Z, L, L, I, I, I, P]),
     "pmesh_facet_order_workspace_bytes": (Z, [L]),
     "pmesh_build_facet_order": (I, [P, L, L, P, P, Z, P]),
     "pmesh_f2f_bwd_workspace_bytes": (Z, [I, I, I]),

@@ -17,10 +17,17 @@ int f2f16x3_fwd(const float *tex, const float *W, const float *sh, const int *cu
 // forward on the fp16 matrix cores with a two-way split and power-of-two scaling of both operands
 // (mesh_f2f16h2.hip); same conditions as the bf16 kernels, workspace no larger than theirs
 size_t f2f16h2_fwd_workspace_bytes(int Cin, int Cout);
+// What the forward does to a value before it stores it: out = act(conv + bias) * scale + shift, every pointer optional
+// (per output channel); bits (float features, Cout % 32 == 0): the ReLU mask, one word per facet and 32 channels.
+struct F2FTail {
+    const float *bias, *scale, *shift;
+    unsigned *bits;
+    int relu;
+};
 // bf16: texture and output rows are bf16 (unsigned short) instead of float; runs the one-product kernels
 int f2f16h2_fwd(const void *tex, const float *W, const float *sh, const int *cum, const int *order, void *out,
                 void *workspace, size_t workspace_bytes, int64_t T, int64_t Nf, int Cin, int Cout, hipStream_t st, bool half = false,
-                bool bf16 = false);
+                bool bf16 = false, const F2FTail *tail = nullptr);
 
 // texture gradient on the fp16 matrix cores (conditions of the bf16 kernel, workspace no larger)
 size_t f2f16h2_bwd_texture_workspace_bytes(int Cin, int Cout);

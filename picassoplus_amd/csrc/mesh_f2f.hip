@@ -348,12 +348,13 @@ extern "C" size_t pmesh_f2f_fwd_workspace_bytes(int Cin, int Cout, int F)
     return F == 16 ? f2f16x3_fwd_workspace_bytes(Cin, Cout) : 0;
 }
 
-extern "C" int pmesh_f2f_fwd(const float *texture, const float *filter, const float *bary_coeff,
-                             const int32_t *cum_texture, const int32_t *facet_order, float *output,
-                             void *workspace, size_t workspace_bytes, int64_t T, int64_t Nf, int Cin, int Cout,
-                             int F, pmesh_stream_t stream)
+// *fused (may be null) <- true when the kernel that ran applied `tail` itself
+static int f2f_fwd_any(const float *texture, const float *filter, const float *bary_coeff,
+                       const int32_t *cum_texture, const int32_t *facet_order, float *output,
+                       void *workspace, size_t workspace_bytes, int64_t T, int64_t Nf, int Cin, int Cout,
+                       int F, pmesh_stream_t stream, const F2FTail *tail, bool *fused)
 {
-    clear_error();
+    if (fused) *fused = false;
     PM_F2F_DIMS("f2f_fwd");
     if (Nf == 0) return 0;
     PM_REQUIRE(filter && cum_texture && output && (T == 0 || (texture && bary_coeff)), "f2f_fwd: null pointer");
@@ -361,9 +362,12 @@ extern "C" int pmesh_f2f_fwd(const float *texture, const float *filter, const fl
     if (!force_generic() && !force_bf16x3() && f2f_fwd_narrow_usable(Cin, F, bary_coeff))
         return f2f_fwd_narrow(texture, filter, bary_coeff, cum_texture, output, T, Nf, Cin, Cout, (hipStream_t)stream);
     if (!force_generic() && !force_bf16x3() && f2f16x3_usable(filter, bary_coeff, F) &&
-        T * Cin < (int64_t(1) << 31))
+        T * Cin < (int64_t(1) << 31)) {
+        const bool fuse = tail && (!tail->bits || Cout % 32 == 0);
+        if (fused) *fused = fuse;
         return f2f16h2_fwd(texture, filter, bary_coeff, cum_texture, facet_order, output, workspace, workspace_bytes,
-                           T, Nf, Cin, Cout, (hipStream_t)stream, want_half());
+                           T, Nf, Cin, Cout, (hipStream_t)stream, want_half(), false, fuse ? tail : nullptr);
+    }
     if (!force_generic() && f2f16x3_usable(filter, bary_coeff, F) &&
         T * Cin < (int64_t(1) << 31))
         return f2f16x3_fwd(texture, filter, bary_coeff, cum_texture, facet_order, output, workspace, workspace_bytes,
@@ -375,6 +379,35 @@ extern "C" int pmesh_f2f_fwd(const float *texture, const float *filter, const fl
         texture, filter, bary_coeff, cum_texture, output, Nf, (int)T, Cin, Cout, cg);
     PM_LAUNCHED("f2f_fwd");
     return 0;
+}
+
+extern "C" int pmesh_f2f_fwd(const float *texture, const float *filter, const float *bary_coeff,
+                             const int32_t *cum_texture, const int32_t *facet_order, float *output,
+                             void *workspace, size_t workspace_bytes, int64_t T, int64_t Nf, int Cin, int Cout,
+                             int F, pmesh_stream_t stream)
+{
+    clear_error();
+    return f2f_fwd_any(texture, filter, bary_coeff, cum_texture, facet_order, output, workspace, workspace_bytes, T, Nf,
+                       Cin, Cout, F, stream, nullptr, nullptr);
+}
+
+extern "C" int pmesh_f2f_fwd_act(const float *texture, const float *filter, const float *bary_coeff,
+                                 const int32_t *cum_texture, const int32_t *facet_order, const float *bias,
+                                 const float *scale, const float *shift, int relu, float *output, uint32_t *relu_bits,
+                                 void *workspace, size_t workspace_bytes, int64_t T, int64_t Nf, int Cin, int Cout,
+                                 int F, pmesh_stream_t stream)
+{
+    clear_error();
+    PM_REQUIRE(!relu_bits || (Cout % 32 == 0 && !(reinterpret_cast<uintptr_t>(output) & 15u)),
+               "f2f_fwd_act: the bit mask needs a multiple of 32 output channels and 16-byte aligned rows");
+    const F2FTail tail = {bias, scale, shift, relu_bits, relu ? 1 : 0};
+    bool fused = false;
+    if (int rc = f2f_fwd_any(texture, filter, bary_coeff, cum_texture, facet_order, output, workspace, workspace_bytes, T,
+                             Nf, Cin, Cout, F, stream, &tail, &fused))
+        return rc;
+    if (fused || Nf == 0) return 0;
+    // kernels without the epilogue: the tail as a pass of its own over the result, in place
+    return pmesh_bias_act_fwd(output, bias, scale, shift, relu, output, relu_bits, Nf, Cout, stream);
 }
 
 // the two halves run one after the other on a stream and share the workspace: partial filter gradients (as many

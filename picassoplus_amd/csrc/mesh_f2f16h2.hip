@@ -477,7 +477,7 @@ __global__ __launch_bounds__(kHThreads, 2) void f2f16h2_fwd_k(const TIO *__restr
                                                               const u32x4 *__restrict__ Wp, const float *__restrict__ sh,
                                                               const int *__restrict__ cum, const int *__restrict__ order,
                                                               TIO *__restrict__ out, int64_t Nf, int T, int Cin,
-                                                              int Cout, int NT)
+                                                              int Cout, int NT, F2FTail tail)
 {
     __shared__ u32x4 Ws[2 * kHChunk];
     __shared__ __attribute__((aligned(16))) float s_slab[kHW * 2 * kHSlab];      // per wavefront: two buffers
@@ -594,6 +594,17 @@ __global__ __launch_bounds__(kHThreads, 2) void f2f16h2_fwd_k(const TIO *__restr
     }
 
     const float ibeta = hdr[1];
+    // what rides on the store: bias, ReLU (and its mask as bits), a per-channel scale and shift
+    float tb[2], tsc[2], tsf[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+        const int co = n0 + t * 32 + l32;
+        const bool cok = co < Cout;
+        tb[t] = (tail.bias && cok) ? tail.bias[co] : 0.f;
+        tsc[t] = (tail.scale && cok) ? tail.scale[co] : 1.f;
+        tsf[t] = (tail.shift && cok) ? tail.shift[co] : 0.f;
+    }
+    const bool plain = !tail.bias && !tail.scale && !tail.shift && !tail.relu;
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
         const int slot = w * 32 + 8 * (i / 4) + 4 * h + (i % 4);
@@ -603,7 +614,18 @@ __global__ __launch_bounds__(kHThreads, 2) void f2f16h2_fwd_k(const TIO *__restr
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
             const int co = n0 + t * 32 + l32;
-            hst1_pair(out + ((int64_t)(rok ? fr : 0) * Cout + co), acc[t][i] * us, rok && co < Cout, l32);
+            float v = acc[t][i] * us;
+            if (!plain) {
+                v += tb[t];
+                if (tail.relu) v = fmaxf(v, 0.f);
+                if (tail.bits) {
+                    // the 32 lanes of a half are the 32 channels of one mask word of its facet
+                    const unsigned long long m = __builtin_amdgcn_ballot_w64(v > 0.f && co < Cout);
+                    if (l32 == 0 && rok && n0 + 32 * t < Cout) tail.bits[(int64_t)fr * (Cout >> 5) + ((n0 >> 5) + t)] = (unsigned)(m >> (32 * h));
+                }
+                v = v * tsc[t] + tsf[t];
+            }
+            hst1_pair(out + ((int64_t)(rok ? fr : 0) * Cout + co), v, rok && co < Cout, l32);
         }
     }
 }
@@ -617,9 +639,11 @@ size_t f2f16h2_fwd_workspace_bytes(int Cin, int Cout)
 
 int f2f16h2_fwd(const void *tex_, const float *W, const float *sh, const int *cum, const int *order, void *out_,
                 void *workspace, size_t workspace_bytes, int64_t T, int64_t Nf, int Cin, int Cout, hipStream_t st, bool half,
-                bool bf16)
+                bool bf16, const F2FTail *tail)
 {
     const int NT = 2 * ((Cout + 63) / 64);
+    const F2FTail tl = tail ? *tail : F2FTail{nullptr, nullptr, nullptr, nullptr, 0};
+    PM_REQUIRE(!tl.bits || (!bf16 && Cout % 32 == 0), "f2f_fwd: the bit mask needs float features and a multiple of 32 output channels");
     PM_REQUIRE(T * Cin < (int64_t(1) << 31), "f2f_fwd: texture array too large for 32-bit offsets");
     PM_REQUIRE(workspace && workspace_bytes >= f2f16h2_fwd_workspace_bytes(Cin, Cout),
                "f2f_fwd: workspace too small (%zu bytes)", workspace_bytes);
@@ -633,7 +657,7 @@ int f2f16h2_fwd(const void *tex_, const float *W, const float *sh, const int *cu
     PM_LAUNCHED("f2f_fwd(pack)");
     const int64_t gx = ceil_div(Nf, kHFacets), gy = NT / 2;
     PM_REQUIRE(grid_ok(gx) && gy <= 65535, "f2f_fwd: grid too large");
-#define PM_FWD(V, H, TIO) f2f16h2_fwd_k<V, H, TIO><<<dim3((unsigned)gx, (unsigned)gy), dim3(kHThreads), 0, st>>>((const TIO *)tex_, hdr, Wp, sh, cum, order, (TIO *)out_, Nf, (int)T, Cin, Cout, NT)
+#define PM_FWD(V, H, TIO) f2f16h2_fwd_k<V, H, TIO><<<dim3((unsigned)gx, (unsigned)gy), dim3(kHThreads), 0, st>>>((const TIO *)tex_, hdr, Wp, sh, cum, order, (TIO *)out_, Nf, (int)T, Cin, Cout, NT, tl)
     if (bf16) {
         // bf16 features: the one-product kernels, rows read eight bytes at a time
         PM_REQUIRE(!(Cin & 3) && !(Cout & 1) && !(reinterpret_cast<uintptr_t>(tex_) & 7u) && !(reinterpret_cast<uintptr_t>(out_) & 3u),

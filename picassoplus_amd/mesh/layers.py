@@ -15,7 +15,7 @@ import torch.nn as nn
 
 from .. import _lib
 from . import topology
-from .pi_modules import conv3d, dense, pool3d, unpool3d
+from .pi_modules import conv3d, dense, mesh_conv3d, pool3d, unpool3d
 from .pi_modules._check import stream_of
 
 
@@ -153,6 +153,18 @@ class F2FConv3d(_ConvTail):
         assert self.in_channels == input_texture.shape[-1]
         assert self.num_basis == bary_coeff.shape[-1]
         running_total = topology.running_total(num_texture)
+        relu = isinstance(self.activation_fn, nn.ReLU)
+        if (relu or self.activation_fn is None) and input_texture.dtype == torch.float32:
+            # bias and activation ride on the convolution's store; a batch norm that only applies its running
+            # statistics rides along when no gradients are recorded
+            biases = self.biases.reshape(-1)
+            if self.with_bn and not torch.is_grad_enabled():
+                frozen = self._frozen_norm()
+                if frozen is not None:
+                    return mesh_conv3d.facet2facet_forward_act(input_texture.contiguous(), self.weights, bary_coeff,
+                                                               running_total, biases.contiguous(), relu, frozen[0], frozen[1])
+            outputs = conv3d.facet2facet_bias_act(input_texture, self.weights, biases, bary_coeff, running_total, relu)
+            return self.BatchNorm(outputs) if self.with_bn else outputs
         outputs = conv3d.facet2facet(input_texture, self.weights, bary_coeff, running_total)
         return self._bias_tail(outputs)
 

@@ -7,6 +7,9 @@ gradient of vertex2facet and facet2vertex come out of one native call, so both a
 as in the reference; facet2facet has one native call per gradient and skips the one autograd does not
 ask for (the texture gradient of a network's input colours, the largest single saving of a first block).
 """
+import torch
+
+from . import dense
 from . import mesh_conv3d as module
 from ._autograd import native_op
 
@@ -45,3 +48,44 @@ def facet2vertex(input, filter, coeff, face, nfCount, vtMap):
     returns (NvOut, C*r) float32
     """
     return f2v_Function.apply(input, filter, coeff, face, nfCount, vtMap)
+
+
+class F2FBiasActFunction(torch.autograd.Function):
+    """facet2facet followed by ``+ bias`` and a ReLU (or no activation), the first two steps of F2FConv3d's tail
+    (picasso/mesh/layers.py:59-63), as ONE native forward: the convolution kernel applies them as it stores.  Backward:
+    the masked gradient and the bias gradient in one pass, then the two facet2facet gradients autograd asks for."""
+
+    @staticmethod
+    def forward(ctx, textureIn, filter, bias, baryCoeff, numTexture, relu):
+        for t in (baryCoeff, numTexture):
+            if t.requires_grad:
+                t.requires_grad = False
+        bits = None
+        if relu and filter.shape[0] % 32 == 0:
+            out, bits = module.facet2facet_forward_act(textureIn, filter, baryCoeff, numTexture, bias, True, with_bits=True)
+        else:
+            out = module.facet2facet_forward_act(textureIn, filter, baryCoeff, numTexture, bias, relu)
+        ctx.relu = relu
+        ctx.save_for_backward(textureIn, filter, baryCoeff, numTexture, out if (relu and bits is None) else None, bits)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        textureIn, filter, baryCoeff, numTexture, out, bits = ctx.saved_tensors
+        grad_output = grad_output.contiguous()
+        if bits is not None and grad_output.data_ptr() % 16:
+            grad_output = grad_output.clone()
+        need_conv = ctx.needs_input_grad[0] or ctx.needs_input_grad[1]
+        gz, gb = dense.bias_act_backward(grad_output, out, need_input=need_conv, relu_bits=bits)
+        gtex = gfilt = None
+        if need_conv:
+            gtex, gfilt = module.facet2facet_backward_selected(gz, textureIn, filter, baryCoeff, numTexture,
+                                                               needs=tuple(ctx.needs_input_grad[:2]))
+        return gtex, gfilt, gb if ctx.needs_input_grad[2] else None, None, None, None
+
+
+def facet2facet_bias_act(textureIn, filter, bias, baryCoeff, numTexture, relu=True):
+    """act(facet2facet(textureIn, filter, baryCoeff, numTexture) + bias) with gradients for the texture, the filter
+    and the bias (Cout,); no counterpart function in the reference, whose module adds the bias and applies the
+    activation as separate PyTorch ops (picasso/mesh/layers.py:59-63)."""
+    return F2FBiasActFunction.apply(textureIn, filter, bias, baryCoeff, numTexture, relu)

@@ -145,6 +145,35 @@ def facet2facet_forward(input, filter, bary_coeff, num_texture):
     return out
 
 
+def facet2facet_forward_act(input, filter, bary_coeff, num_texture, bias=None, relu=True, scale=None, shift=None,
+                            with_bits=False):
+    """facet2facet_forward with the module's tail on the store (picasso/mesh/layers.py:59-63):
+    act(conv + bias) * scale + shift, float32 features; ``bias`` / ``scale`` / ``shift`` (Cout,) float32 or None.
+    ``with_bits`` (Cout % 32 == 0) also returns the ReLU mask as bits, int32 (Nf, Cout / 32)."""
+    T, Cin, Cout, F, Nf = _f2f_dims(input, filter, bary_coeff, num_texture, True)
+    if input.dtype != F32:
+        raise RuntimeError("the fused tail takes float32 features")
+    for name, t in (("bias", bias), ("scale", scale), ("shift", shift)):
+        if t is not None:
+            check_input(t, name, 1, F32)
+            if t.shape[0] != Cout:
+                raise RuntimeError("%s must have one entry per output channel" % name)
+    if with_bits and Cout % 32:
+        raise RuntimeError("the bit mask needs a multiple of 32 output channels")
+    dev = same_device(input, filter, bary_coeff, num_texture, *[t for t in (bias, scale, shift) if t is not None])
+    with torch.cuda.device(dev):
+        out = torch.empty((Nf, Cout), dtype=F32, device=dev)
+        bits = torch.empty((Nf, Cout // 32), dtype=torch.int32, device=dev) if with_bits else None
+        nbytes = _lib.query("pmesh_f2f_fwd_workspace_bytes", Cin, Cout, F)
+        ws = workspace(nbytes, dev)
+        order = topology.facet_order(num_texture, T) if Nf else None
+        ptr = lambda t: t.data_ptr() if t is not None else None
+        _lib.call("pmesh_f2f_fwd_act", input.data_ptr(), filter.data_ptr(), bary_coeff.data_ptr(), num_texture.data_ptr(),
+                  ptr(order), ptr(bias), ptr(scale), ptr(shift), 1 if relu else 0, out.data_ptr(), ptr(bits), ws.data_ptr(),
+                  nbytes, T, Nf, Cin, Cout, F, stream_of(input))
+    return (out, bits) if with_bits else out
+
+
 def facet2facet_backward(grad_output, input, filter, bary_coeff, num_texture):
     """mesh_conv3d.cpp:229-269 -> [grad_input (NiK,Cin), grad_filter (Cout,Cin,F)]."""
     return facet2facet_backward_selected(grad_output, input, filter, bary_coeff, num_texture, needs=(True, True))

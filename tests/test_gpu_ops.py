@@ -291,6 +291,63 @@ def test_f2f_parity(cuda, native_options, nf, Cin, Cout, F, kmax, path):
         say("  errors (build, float32 oracle): out %.2e %.2e  grad_texture %.2e %.2e  grad_filter %.2e %.2e" % (e_o + e_t + e_w))
 
 
+@pytest.mark.parametrize("nf,Cin,Cout,F,kmax", [(200, 64, 64, 16, 9), (333, 16, 96, 16, 4), (300, 8, 40, 16, 14),
+                                                (100, 3, 32, 16, 5), (70, 5, 7, 9, 3), (260, 128, 256, 16, 6)])
+@pytest.mark.parametrize("relu", [True, False])
+def test_f2f_fused_tail_parity(cuda, nf, Cin, Cout, F, kmax, relu):
+    """facet2facet with bias and ReLU on the convolution's store (the first steps of F2FConv3d's tail,
+    picasso/mesh/layers.py:59-63) against the oracle's composition in float64, gradients included; the shapes cover the
+    fp16 kernels that fuse the tail, with and without the bit form of the mask (Cout % 32), and the kernels that run
+    the tail as a second pass (narrow, generic).  Inference form: scale and shift of a frozen batch norm as well."""
+    say("case f2f fused tail", nf, Cin, Cout, F, kmax, relu)
+    rng = np.random.default_rng(31)
+    counts, bary, owner = texture_case(rng, nf, kmax)
+    cum = np.cumsum(counts).astype(np.int32)
+    T = int(counts.sum())
+    tex = rng.uniform(-1, 1, (T, Cin))
+    sh = rng.normal(0, 0.5, (T, F))
+    filt = rng.normal(0, 0.3, (Cout, Cin, F))
+    bias = rng.normal(0, 0.5, Cout)
+    gout = rng.normal(0, 1, (nf, Cout))
+    conv = loops.f2f_fwd(tex, filt, sh, cum)
+    z = conv + bias
+    # keep the comparison away from the kink: values within the build's error of zero may land on either side
+    z_safe = np.abs(z) > 1e-4 * np.abs(conv).max()
+    out_ref = np.maximum(z, 0) if relu else z
+    tt = dev(tex, cuda, torch.float32).requires_grad_(True)
+    ft = dev(filt, cuda, torch.float32).requires_grad_(True)
+    bt = dev(bias, cuda, torch.float32).requires_grad_(True)
+    sht, cumt = dev(sh, cuda, torch.float32), dev(cum, cuda)
+    out = conv3d.facet2facet_bias_act(tt, ft, bt, sht, cumt, relu)
+    g = gout * z_safe                                          # no gradient through entries too close to the kink
+    gin_ref, gfilt_ref = loops.f2f_bwd(g * (z > 0) if relu else g, tex, filt, sh, cum)
+    out.backward(dev(g, cuda, torch.float32))
+    torch.cuda.synchronize()
+    o = out.detach().cpu().numpy()
+    assert np.abs(o - out_ref).max() <= 1e-5 * np.abs(conv).max(), "fused out"
+    if relu:
+        assert np.array_equal(o[z_safe] > 0, z[z_safe] > 0)
+    assert_close(tt.grad, gin_ref, "fused grad_texture")
+    assert_close(ft.grad, gfilt_ref, "fused grad_filter")
+    assert_close(bt.grad, (g * (z > 0) if relu else g).sum(0), "fused grad_bias")
+    # the same values as the two-step path of the module
+    two = torch.relu(conv3d.facet2facet(tt.detach(), ft.detach(), sht, cumt) + bt.detach()) if relu else \
+        conv3d.facet2facet(tt.detach(), ft.detach(), sht, cumt) + bt.detach()
+    assert float((out.detach() - two).abs().max()) <= 3e-7 * np.abs(conv).max(), "fused and two-step results differ"
+    # inference form with a frozen batch norm
+    scale, shift = rng.uniform(0.5, 2, Cout), rng.normal(0, 1, Cout)
+    y = mesh_conv3d.facet2facet_forward_act(tt.detach(), ft.detach(), sht, cumt, bt.detach(), relu,
+                                            dev(scale, cuda, torch.float32), dev(shift, cuda, torch.float32))
+    want = out_ref * scale + shift
+    assert np.abs(y.cpu().numpy() - want).max() <= 1e-5 * max(np.abs(want).max(), np.abs(conv).max() * scale.max())
+    if Cout % 32 == 0 and relu:
+        y2, bits = mesh_conv3d.facet2facet_forward_act(tt.detach(), ft.detach(), sht, cumt, bt.detach(), True, with_bits=True)
+        assert torch.equal(y2, out.detach())
+        b = bits.cpu().numpy().view(np.uint32)
+        mask = ((b[:, :, None] >> np.arange(32, dtype=np.uint32)) & 1).reshape(nf, Cout).astype(bool)
+        assert np.array_equal(mask, o > 0)
+
+
 @pytest.mark.parametrize("case", ["late_channels", "late_points", "growing_facets"])
 def test_f2f_wide_dynamic_range(cuda, case):
     """The fp16 kernels choose power-of-two operand scales from what they have seen so far and must recover when

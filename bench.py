@@ -115,18 +115,24 @@ TRAFFIC_KERNELS = {
     "pool": {"pool_max_fwd": [r"pool_max_fwd_k"], "pool_max_bwd": [r"fine_gather_k<4, 2>"],
              "pool_avg_fwd": [r"cluster_sum_k<4, true>"], "pool_avg_bwd": [r"fine_gather_k<4, 1>"],
              "unpool_fwd": [r"fine_gather_k<4, 0>"], "unpool_bwd": [r"cluster_sum_k<4, false>"]},
-    "tail": {"dense_fwd": [r"dense_rows_k<.*false, (true|false)>$"], "dense_bwd": [r"dense_rows_k<.*true, (true|false)>$", r"dense_wgrad_k", r"reduce_partials_k"]},
+    "tail": {"dense_fwd": [r"dense_rows_k<\d+, \d+, (true|false), 0, "],
+             "dense_bwd": [r"dense_rows_k<\d+, \d+, (true|false), [12], ", r"dense_wgrad_k", r"reduce_partials_k"]},
     "texture": {"texture_fwd": [r"texture_fwd_k"], "texture_bwd": [r"texture_bwd_flat_k", r"texture_bwd_k"]},
 }
 
 
+TIMED_SOURCES = ("mesh_f2f", "mesh_f2v", "mesh_rows", "mesh_dense", "mesh_texture", "common", "f2f_internal", "rows_internal",
+                 "sph_internal")
+
+
 def build_id():
-    """Identity of the kernels being timed: hash over the sources the library is built from."""
+    """Identity of the kernels being timed: hash over the sources that hold them (convolutions, pooling, tails,
+    texture interpolation and their shared headers; index builds and mesh preparation are not timed here)."""
     import hashlib
     h = hashlib.sha256()
     csrc = os.path.join(ROOT, "picassoplus_amd", "csrc")
     for name in sorted(os.listdir(csrc)):
-        if name.endswith((".hip", ".h", ".cpp")):
+        if name.endswith((".hip", ".h", ".cpp")) and name.startswith(TIMED_SOURCES):
             h.update(name.encode())
             h.update(open(os.path.join(csrc, name), "rb").read())
     return h.hexdigest()[:16]
@@ -160,8 +166,8 @@ def write_traffic(args):
     copy = [k for k in F if "copyBuffer" in k]
     if not copy or copy[0] not in W:
         sys.exit("--traffic-from: no device-copy kernel in the counter files (run bench.py with --copy-calibration)")
-    # the three 1 GiB copies dominate the copy kernel's total
-    fcal, wcal = sum(F[copy[0]]) / 3.0, sum(W[copy[0]]) / 3.0
+    # the three 1 GiB copies are the copy kernel's three largest dispatches
+    fcal, wcal = sum(sorted(F[copy[0]])[-3:]) / 3.0, sum(sorted(W[copy[0]])[-3:]) / 3.0
     ff, wf = 1048576.0 / fcal, 1048576.0 / wcal
     per_kernel, ops = {}, {}
     for op, pats in TRAFFIC_KERNELS[args.workload].items():

@@ -378,6 +378,93 @@ int pmesh_bias_act_bwd(const float *grad_output, const float *output, const uint
                        float *grad_input, float *grad_bias, void *workspace, size_t workspace_bytes,
                        int64_t N, int C, pmesh_stream_t stream);
 
+/* ------------------------------------------------------------------ point-cloud branch
+ * replaces the reference's point_nnquery / point_sample / point_buildkernel / point_conv3d / point_pool3d /
+ * point_unpool3d extensions (picasso/point/pi_modules/source/).  Points of a batch are concatenated;
+ * nv_database / nv_query are INCLUSIVE running totals of the points per sample (B entries), as the reference's
+ * wrappers pass them (picasso/point/pi_modules/nnquery.py:20-21).  Pairs are (query, database point) rows.
+ *
+ * Adjacency of an index column: row r -> ascending list of the entries i with keys[i * key_stride] == r (entries
+ * outside [0, n_rows) belong to no row).  The point ops take it sorted by query for their forward, by database
+ * point for their input gradients; pmesh_point_unpool_bwd takes it over the flattened (Nrows * K) index array. */
+size_t pmesh_index_csr_workspace_bytes(int64_t n, int64_t n_rows);
+int pmesh_build_index_csr(const int32_t *keys, int key_stride, int64_t n, int64_t n_rows, int32_t *rowptr,
+                          int32_t *order, void *workspace, size_t workspace_bytes, pmesh_stream_t stream);
+
+/* range search (nnquery.cpp:29-78 "range", nnquery_gpu.cu:20-126): database points of the query's sample closer than
+ * radius, ascending, the first nn_sample of them.  Two steps, because the caller allocates the pair arrays between
+ * them: count (Mp) <- neighbours per query; then, with cnt_info = inclusive running total of count (int64) and
+ * Nout = its last entry, nn_index (Nout,2) and nn_dist (Nout) <- the pairs and their distances. */
+int pmesh_point_range_count(const float *database, const float *query, const int32_t *nv_database,
+                            const int32_t *nv_query, int B, int64_t Np, int64_t Mp, float radius, int nn_sample,
+                            int32_t *count, pmesh_stream_t stream);
+int pmesh_point_range_fill(const float *database, const float *query, const int32_t *nv_database,
+                           const int32_t *nv_query, int B, int64_t Np, int64_t Mp, float radius, const int64_t *cnt_info,
+                           int64_t Nout, int32_t *nn_index, float *nn_dist, pmesh_stream_t stream);
+/* cube search (nnquery.cpp:81-129 "cube", nnquery_gpu.cu:134-250): neighbours inside the axis-aligned cube of edge
+ * length; nn_index (Nout,3) = query, database point, cell of a grid_size^3 grid over the cube. */
+int pmesh_point_cube_count(const float *database, const float *query, const int32_t *nv_database,
+                           const int32_t *nv_query, int B, int64_t Np, int64_t Mp, float length, int nn_sample,
+                           int32_t *count, pmesh_stream_t stream);
+int pmesh_point_cube_fill(const float *database, const float *query, const int32_t *nv_database,
+                          const int32_t *nv_query, int B, int64_t Np, int64_t Mp, float length, int grid_size,
+                          const int64_t *cnt_info, int64_t Nout, int32_t *nn_index, pmesh_stream_t stream);
+/* three nearest neighbours (nnquery.cpp:132-171 "knn3", nnquery_gpu.cu:262-330): nn_index, nn_dist (Mp,3). */
+int pmesh_point_knn3(const float *database, const float *query, const int32_t *nv_database, const int32_t *nv_query,
+                     int B, int64_t Np, int64_t Mp, int32_t *nn_index, float *nn_dist, pmesh_stream_t stream);
+/* farthest point sampling (sample.cpp:20-50 "fps", sample_gpu.cu:11-100): index_out (Mp) <- per sample its first
+ * point, then repeatedly the point farthest from those chosen (lowest index among equals); temp: Np floats. */
+int pmesh_point_fps(const float *xyz, const int32_t *nv_in, const int32_t *nv_out, int B, int64_t Np, int64_t Mp,
+                    float *temp, int32_t *index_out, pmesh_stream_t stream);
+/* kernel bins of neighbour pairs (buildkernel.cpp:22-117 "SPH3D", "fuzzySPH3D", buildkernel_gpu.cu:20-155): an
+ * (n azimuth, p elevation, q radial) spherical kernel plus the centre bin 0.  filt_index (Nout); fuzzy form:
+ * filt_index, filt_coeff (Nout,3): centre, own elevation bin, neighbouring elevation bin. */
+int pmesh_point_sph3d_kernel(const float *database, const float *query, const int32_t *nn_index, const float *nn_dist,
+                             int64_t Nout, int64_t Np, int64_t Mp, int n, int p, int q, float radius,
+                             int32_t *filt_index, pmesh_stream_t stream);
+int pmesh_point_fuzzy_sph3d_kernel(const float *database, const float *query, const int32_t *nn_index,
+                                   const float *nn_dist, int64_t Nout, int64_t Np, int64_t Mp, int n, int p, int q,
+                                   float radius, int32_t *filt_index, float *filt_coeff, pmesh_stream_t stream);
+
+/* depthwise point convolution (pcloud_conv3d.cpp:29-213: SPH3D_forward/backward, fuzzySPH3D_forward/backward):
+ *   input (Np,C), filter (F,C,r), nn_count (Mp), nn_index (Nout,2), bin_index (Nout,T), bin_coeff (Nout,T) or NULL
+ *   (plain form: T = 1, weight 1) -> output (Mp,C*r); rowptr / order: the pairs sorted by query (key column 0).
+ * backward: grad_input (Np,C) (NULL skips it; needs rowptr_in / order_in: the pairs sorted by database point, key
+ * column 1), grad_filter (F,C,r); workspace pmesh_point_conv_bwd_workspace_bytes.  At most 512 bins. */
+int pmesh_point_conv_fwd(const float *input, const float *filter, const int32_t *nn_count, const int32_t *nn_index,
+                         const int32_t *bin_index, const float *bin_coeff, const int32_t *rowptr, const int32_t *order,
+                         float *output, int64_t Np, int64_t Mp, int64_t Nout, int F, int C, int r, int T,
+                         pmesh_stream_t stream);
+size_t pmesh_point_conv_bwd_workspace_bytes(int64_t Nout, int F, int C, int r);
+int pmesh_point_conv_bwd(const float *grad_output, const float *input, const float *filter, const int32_t *nn_count,
+                         const int32_t *nn_index, const int32_t *bin_index, const float *bin_coeff,
+                         const int32_t *rowptr_in, const int32_t *order_in, float *grad_input, float *grad_filter,
+                         void *workspace, size_t workspace_bytes, int64_t Np, int64_t Mp, int64_t Nout, int F, int C,
+                         int r, int T, pmesh_stream_t stream);
+
+/* point pooling (pcloud_pool3d.cpp:23-148): input (Np,C) -> output (Mp,C) over the pairs.  max: max_index (Mp,C) =
+ * database point that holds the maximum (first pair among equals; -1 and output 0 for a query without pairs); its
+ * backward gathers, per database point, the gradients of the queries whose maximum it holds. */
+int pmesh_point_pool_max_fwd(const float *input, const int32_t *nn_index, const int32_t *rowptr, const int32_t *order,
+                             float *output, int32_t *max_index, int64_t Np, int64_t Mp, int64_t Nout, int C,
+                             pmesh_stream_t stream);
+int pmesh_point_pool_max_bwd(const float *grad_output, const int32_t *max_index, const int32_t *nn_index,
+                             const int32_t *rowptr_in, const int32_t *order_in, float *grad_input, int64_t Np, int64_t Mp,
+                             int64_t Nout, int C, pmesh_stream_t stream);
+int pmesh_point_pool_avg_fwd(const float *input, const int32_t *nn_count, const int32_t *nn_index, const int32_t *rowptr,
+                             const int32_t *order, float *output, int64_t Np, int64_t Mp, int64_t Nout, int C,
+                             pmesh_stream_t stream);
+int pmesh_point_pool_avg_bwd(const float *grad_output, const int32_t *nn_count, const int32_t *nn_index,
+                             const int32_t *rowptr_in, const int32_t *order_in, float *grad_input, int64_t Np, int64_t Mp,
+                             int64_t Nout, int C, pmesh_stream_t stream);
+
+/* weighted unpooling (pcloud_unpool3d.cpp:20-83): output (Nrows,C) = sum_k input[nn_index[o,k]] * weight[o,k] with
+ * nn_index, weight (Nrows,K), input (Nin,C); backward over the adjacency of the flattened index array. */
+int pmesh_point_unpool_fwd(const float *input, const float *weight, const int32_t *nn_index, float *output, int64_t Nrows,
+                           int64_t Nin, int C, int K, pmesh_stream_t stream);
+int pmesh_point_unpool_bwd(const float *grad_output, const float *weight, const int32_t *rowptr_in, const int32_t *order_in,
+                           float *grad_input, int64_t Nrows, int64_t Nin, int C, int K, pmesh_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

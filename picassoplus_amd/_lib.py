@@ -11,7 +11,7 @@ from ctypes import c_char_p, c_float, c_int, c_int64, c_size_t, c_void_p
 _HERE = os.path.dirname(os.path.abspath(__file__))
 # PICASSO_MESH_LIB points at an alternative build of the same ABI (kernel experiments)
 LIB_PATH = os.environ.get("PICASSO_MESH_LIB") or os.path.join(_HERE, "csrc", "libpicasso_mesh.so")
-ABI_VERSION = 15
+ABI_VERSION = 16
 
 P, I, L, Z = c_void_p, c_int, c_int64, c_size_t
 
@@ -32,6 +32,25 @@ SIGNATURES = {
     "pmesh_f2v_bwd_static_max_bytes": (Z, []),
     "pmesh_f2v_bwd_static": (I, [P, P, P, P, P, P, P, P, P, L, L, L, I, I, I, P]),
     "pmesh_f2f_fwd_workspace_bytes": (Z, [I, I, I]),
+    "pmesh_index_csr_workspace_bytes": (Z, [L, L]),
+    "pmesh_build_index_csr": (I, [P, I, L, L, P, P, P, Z, P]),
+    "pmesh_point_range_count": (I, [P, P, P, P, I, L, L, ctypes.c_float, I, P, P]),
+    "pmesh_point_range_fill": (I, [P, P, P, P, I, L, L, ctypes.c_float, P, L, P, P, P]),
+    "pmesh_point_cube_count": (I, [P, P, P, P, I, L, L, ctypes.c_float, I, P, P]),
+    "pmesh_point_cube_fill": (I, [P, P, P, P, I, L, L, ctypes.c_float, I, P, L, P, P]),
+    "pmesh_point_knn3": (I, [P, P, P, P, I, L, L, P, P, P]),
+    "pmesh_point_fps": (I, [P, P, P, I, L, L, P, P, P]),
+    "pmesh_point_sph3d_kernel": (I, [P, P, P, P, L, L, L, I, I, I, ctypes.c_float, P, P]),
+    "pmesh_point_fuzzy_sph3d_kernel": (I, [P, P, P, P, L, L, L, I, I, I, ctypes.c_float, P, P, P]),
+    "pmesh_point_conv_fwd": (I, [P, P, P, P, P, P, P, P, P, L, L, L, I, I, I, I, P]),
+    "pmesh_point_conv_bwd_workspace_bytes": (Z, [L, I, I, I]),
+    "pmesh_point_conv_bwd": (I, [P, P, P, P, P, P, P, P, P, P, P, P, Z, L, L, L, I, I, I, I, P]),
+    "pmesh_point_pool_max_fwd": (I, [P, P, P, P, P, P, L, L, L, I, P]),
+    "pmesh_point_pool_max_bwd": (I, [P, P, P, P, P, P, L, L, L, I, P]),
+    "pmesh_point_pool_avg_fwd": (I, [P, P, P, P, P, P, L, L, L, I, P]),
+    "pmesh_point_pool_avg_bwd": (I, [P, P, P, P, P, P, L, L, L, I, P]),
+    "pmesh_point_unpool_fwd": (I, [P, P, P, P, L, L, I, I, P]),
+    "pmesh_point_unpool_bwd": (I, [P, P, P, P, P, L, L, I, I, P]),
     "pmesh_f2f_fwd": (I, [P, P, P, P, P, P, P, Z, L, L, I, I, I, P]),
     "pmesh_f2f_fwd_act": (I, [P, P, P, P, P, P, P, P, I, P, P, P, Z, L, L, I, I, I, P]),
     "pmesh_facet_order_workspace_bytes": (Z, [L]),

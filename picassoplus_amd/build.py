@@ -10,7 +10,7 @@ from concurrent.futures import ThreadPoolExecutor
 
 CSRC = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc")
 LIB = os.path.join(CSRC, "libpicasso_mesh.so")
-SOURCES = ["mesh_api.cpp", "mesh_csr.hip", "mesh_rows.hip", "mesh_f2v_mfma.hip", "mesh_f2f.hip", "mesh_f2f16x3.hip", "mesh_f2f16h2.hip", "mesh_f2f_narrow.hip", "mesh_dense.hip", "mesh_texture.hip", "mesh_decimate.hip"]
+SOURCES = ["mesh_api.cpp", "mesh_csr.hip", "mesh_rows.hip", "mesh_f2v_mfma.hip", "mesh_f2f.hip", "mesh_f2f16x3.hip", "mesh_f2f16h2.hip", "mesh_f2f_narrow.hip", "mesh_dense.hip", "mesh_texture.hip", "mesh_decimate.hip", "pcloud_query.hip", "pcloud_ops.hip"]
 ARCH = "gfx950"
 # packed-fp32 code generation stays off for every device translation unit
 FLAGS = ["--offload-arch=" + ARCH, "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function",

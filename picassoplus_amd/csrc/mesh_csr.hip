@@ -37,6 +37,17 @@ __global__ __launch_bounds__(kBlock) void cluster_keys_k(const int *__restrict__
     vals[v] = (int)v;
 }
 
+// key of entry i of a strided index array: the row keys[i * stride] names, or n_rows when it names none
+__global__ __launch_bounds__(kBlock) void index_keys_k(const int *__restrict__ src, int stride, int64_t n, int64_t n_rows,
+                                                       unsigned *__restrict__ keys, int *__restrict__ vals)
+{
+    const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= n) return;
+    const int64_t key = src[i * stride];
+    keys[i] = (key >= 0 && key < n_rows) ? (unsigned)key : (unsigned)n_rows;
+    vals[i] = (int)i;
+}
+
 // rowptr[r] = first sorted position whose key is >= r, for r in [0, n_rows]
 __global__ __launch_bounds__(kBlock) void rowptr_k(const unsigned *__restrict__ sorted_keys, int64_t n,
                                                    int64_t n_rows, int *__restrict__ rowptr)
@@ -190,6 +201,31 @@ extern "C" int pmesh_build_vertex_csr(const int32_t *face, const int32_t *vt_map
         face, vt_map, n, n_vt_map, n_rows, (unsigned *)base, (int *)(base + 2 * slot));
     PM_LAUNCHED("build_vertex_csr(keys)");
     return sort_and_rowptr("build_vertex_csr", n, n_rows, rowptr, colidx, workspace, workspace_bytes, st);
+}
+
+extern "C" size_t pmesh_index_csr_workspace_bytes(int64_t n, int64_t n_rows) { return csr_workspace(n, n_rows); }
+
+extern "C" int pmesh_build_index_csr(const int32_t *keys, int key_stride, int64_t n, int64_t n_rows, int32_t *rowptr,
+                                     int32_t *order, void *workspace, size_t workspace_bytes, pmesh_stream_t stream)
+{
+    clear_error();
+    PM_REQUIRE(n >= 0 && n_rows >= 0 && key_stride > 0, "build_index_csr: bad sizes");
+    PM_REQUIRE(n < INT32_MAX && n_rows < INT32_MAX, "build_index_csr: sizes exceed int32 indexing");
+    PM_REQUIRE(rowptr, "build_index_csr: null rowptr");
+    hipStream_t st = (hipStream_t)stream;
+    if (n == 0) {
+        fill_int_k<<<dim3((unsigned)ceil_div(n_rows + 1, kBlock)), dim3(kBlock), 0, st>>>(rowptr, n_rows + 1, 0);
+        PM_LAUNCHED("build_index_csr(fill)");
+        return 0;
+    }
+    PM_REQUIRE(keys && order && workspace, "build_index_csr: null pointer");
+    PM_REQUIRE(workspace_bytes >= 3 * align_up((size_t)n * 4), "build_index_csr: workspace too small");
+    char *base = (char *)workspace;
+    const size_t slot = align_up((size_t)n * 4);
+    index_keys_k<<<dim3((unsigned)ceil_div(n, kBlock)), dim3(kBlock), 0, st>>>(keys, key_stride, n, n_rows, (unsigned *)base,
+                                                                               (int *)(base + 2 * slot));
+    PM_LAUNCHED("build_index_csr(keys)");
+    return sort_and_rowptr("build_index_csr", n, n_rows, rowptr, order, workspace, workspace_bytes, st);
 }
 
 extern "C" size_t pmesh_cluster_csr_workspace_bytes(int64_t n_fine, int64_t n_coarse)

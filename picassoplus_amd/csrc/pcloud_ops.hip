@@ -1,0 +1,466 @@
+// Point-cloud branch, part 2: the (fuzzy) depthwise point convolution, point pooling and weighted unpooling
+// (picasso/point/pi_modules/source/pcloud_conv3d_gpu.cu, pcloud_pool3d_gpu.cu, pcloud_unpool3d_gpu.cu).
+//
+// The reference runs one thread per (neighbour pair, channel) and adds into the output with float atomics.  Here
+// every op is a segmented sum over a sorted adjacency of the pairs (pmesh_build_index_csr): by query for the forward
+// ops, by database point for the input gradients, so each output row is written once, by one lane group, in a fixed
+// order.  The filter gradient is summed per workgroup in LDS (one column per thread, pairs in ascending order) and the
+// workgroups' partial results are added in a fixed tree order.
+//
+//   w[p, co]        = sum_t coeff[p, t] * filter[bin[p, t], co]           (plain form: one bin, weight 1)
+//   out[o, co]      = (1 / nn_count[o]) sum_{p = (o, i)} in[i, co / r] * w[p, co]
+//   gin[i, c]       = sum_{p = (o, i)} (1 / nn_count[o]) sum_m gout[o, c r + m] * w[p, c r + m]
+//   gfilt[f, co]    = sum_p sum_t [bin[p, t] = f] coeff[p, t] * gout[o, co] * in[i, co / r] / nn_count[o]
+#include "common.h"
+#include "rows_internal.h"
+#include "../../include/picasso_mesh.h"
+
+namespace pmesh {
+
+struct PairGraph {
+    const int *nn_index;      // (Nout, 2): query, database point
+    const int *nn_count;      // (Mp) divisor per query
+    const int *bin_index;     // (Nout, T)
+    const float *bin_coeff;   // (Nout, T) or null
+    int64_t Np, Mp, Nout;
+    int T, F;
+};
+
+// weight of pair p for V output channels starting at co
+template <int V> __device__ __forceinline__ Pack<V> pair_weight(const PairGraph &g, const float *__restrict__ filt, int64_t p, int CR, int co)
+{
+    Pack<V> w = zero_pack<V>();
+    for (int t = 0; t < g.T; ++t) {
+        const int b = g.bin_index[p * g.T + t];
+        const float c = g.bin_coeff ? g.bin_coeff[p * g.T + t] : 1.f;
+        if (b >= 0 && b < g.F) {
+            const Pack<V> f = ldp<V>(filt + (int64_t)b * CR + co);
+#pragma unroll
+            for (int u = 0; u < V; ++u) w.v[u] = fmaf(c, f.v[u], w.v[u]);
+        }
+    }
+    return w;
+}
+
+__device__ __forceinline__ float inv_count(const int *__restrict__ nn_count, int64_t o)
+{
+    const int c = nn_count[o];
+    return c > 0 ? 1.0f / (float)c : 0.f;
+}
+
+// V = 4 needs depth multiplier 1 (output channel = input channel) and 16-byte aligned rows
+template <int V>
+__global__ __launch_bounds__(kBlock) void point_conv_fwd_k(const float *__restrict__ in, const float *__restrict__ filt, PairGraph g,
+                                                           const int *__restrict__ rowptr, const int *__restrict__ order,
+                                                           float *__restrict__ out, int C, int r, int items, int lpr_log2)
+{
+    const int lpr = 1 << lpr_log2, lane = threadIdx.x & (lpr - 1), slot = threadIdx.x >> lpr_log2;
+    const int64_t row = (int64_t)blockIdx.x * (kBlock >> lpr_log2) + slot;
+    if (row >= g.Mp) return;
+    const int CR = C * r, e0 = rowptr[row], e1 = rowptr[row + 1];
+    const float inv = inv_count(g.nn_count, row);
+    for (int q = lane; q < items; q += lpr) {
+        const int co = q * V;
+        Pack<V> acc = zero_pack<V>();
+        for (int e = e0; e < e1; ++e) {
+            const int64_t p = order[e];
+            const int i = g.nn_index[p * 2 + 1];
+            if (i < 0 || i >= g.Np) continue;
+            const Pack<V> w = pair_weight<V>(g, filt, p, CR, co);
+            Pack<V> x;
+            if constexpr (V == 1) x.v[0] = in[(int64_t)i * C + co / r];
+            else x = ldp<V>(in + (int64_t)i * C + co);
+#pragma unroll
+            for (int u = 0; u < V; ++u) acc.v[u] = fmaf(x.v[u], w.v[u], acc.v[u]);
+        }
+#pragma unroll
+        for (int u = 0; u < V; ++u) acc.v[u] *= inv;
+        stp<V>(out + row * CR + co, acc);
+    }
+}
+
+// rows = database points; lanes own V input channels (V = 4: depth multiplier 1)
+template <int V>
+__global__ __launch_bounds__(kBlock) void point_conv_bwd_in_k(const float *__restrict__ gout, const float *__restrict__ filt, PairGraph g,
+                                                              const int *__restrict__ rowptr, const int *__restrict__ order,
+                                                              float *__restrict__ gin, int C, int r, int items, int lpr_log2)
+{
+    const int lpr = 1 << lpr_log2, lane = threadIdx.x & (lpr - 1), slot = threadIdx.x >> lpr_log2;
+    const int64_t row = (int64_t)blockIdx.x * (kBlock >> lpr_log2) + slot;
+    if (row >= g.Np) return;
+    const int CR = C * r, e0 = rowptr[row], e1 = rowptr[row + 1];
+    for (int q = lane; q < items; q += lpr) {
+        const int c = q * V;
+        Pack<V> acc = zero_pack<V>();
+        for (int e = e0; e < e1; ++e) {
+            const int64_t p = order[e];
+            const int o = g.nn_index[p * 2];
+            if (o < 0 || o >= g.Mp) continue;
+            const float inv = inv_count(g.nn_count, o);
+            if constexpr (V == 1) {
+                float s = 0.f;
+                for (int m = 0; m < r; ++m) {
+                    const Pack<1> w = pair_weight<1>(g, filt, p, CR, c * r + m);
+                    s = fmaf(gout[(int64_t)o * CR + c * r + m], w.v[0], s);
+                }
+                acc.v[0] = fmaf(s, inv, acc.v[0]);
+            } else {
+                const Pack<V> w = pair_weight<V>(g, filt, p, CR, c), go = ldp<V>(gout + (int64_t)o * CR + c);
+#pragma unroll
+                for (int u = 0; u < V; ++u) acc.v[u] = fmaf(go.v[u] * w.v[u], inv, acc.v[u]);
+            }
+        }
+        stp<V>(gin + row * C + c, acc);
+    }
+}
+
+// filter gradient: workgroup (x, y) sums pairs [x * per, (x + 1) * per) for columns y * cols .. into LDS, one column per
+// thread, and leaves partial[x][F][CR]
+__global__ void point_conv_bwd_filt_k(const float *__restrict__ gout, const float *__restrict__ in, PairGraph g,
+                                      float *__restrict__ partial, int C, int r, int cols, int64_t per)
+{
+    extern __shared__ float s_acc[];          // [F][cols]
+    const int CR = C * r, co = blockIdx.y * cols + threadIdx.x;
+    for (int f = 0; f < g.F; ++f) s_acc[f * cols + threadIdx.x] = 0.f;
+    const int64_t p0 = (int64_t)blockIdx.x * per, p1 = p0 + per < g.Nout ? p0 + per : g.Nout;
+    if (co < CR) {
+        for (int64_t p = p0; p < p1; ++p) {
+            const int o = g.nn_index[p * 2], i = g.nn_index[p * 2 + 1];
+            if (o < 0 || o >= g.Mp || i < 0 || i >= g.Np) continue;
+            const float d = gout[(int64_t)o * CR + co] * in[(int64_t)i * C + co / r] * inv_count(g.nn_count, o);
+            for (int t = 0; t < g.T; ++t) {
+                const int b = g.bin_index[p * g.T + t];
+                const float c = g.bin_coeff ? g.bin_coeff[p * g.T + t] : 1.f;
+                if (b >= 0 && b < g.F) s_acc[b * cols + threadIdx.x] = fmaf(c, d, s_acc[b * cols + threadIdx.x]);
+            }
+        }
+        float *dst = partial + (int64_t)blockIdx.x * g.F * CR;
+        for (int f = 0; f < g.F; ++f) dst[(int64_t)f * CR + co] = s_acc[f * cols + threadIdx.x];
+    }
+}
+
+// ------------------------------------------------------------------------------------------------ pooling
+// MODE 0: max with arg-max (first pair among equals; -1 and 0 for a query without neighbours), 1: average
+template <int V, int MODE>
+__global__ __launch_bounds__(kBlock) void point_pool_fwd_k(const float *__restrict__ in, const int *__restrict__ nn_index,
+                                                           const int *__restrict__ nn_count, const int *__restrict__ rowptr,
+                                                           const int *__restrict__ order, float *__restrict__ out,
+                                                           int *__restrict__ max_index, int64_t Np, int64_t Mp, int C, int items,
+                                                           int lpr_log2)
+{
+    const int lpr = 1 << lpr_log2, lane = threadIdx.x & (lpr - 1), slot = threadIdx.x >> lpr_log2;
+    const int64_t row = (int64_t)blockIdx.x * (kBlock >> lpr_log2) + slot;
+    if (row >= Mp) return;
+    const int e0 = rowptr[row], e1 = rowptr[row + 1];
+    const float inv = MODE == 1 ? inv_count(nn_count, row) : 0.f;
+    for (int q = lane; q < items; q += lpr) {
+        const int c = q * V;
+        Pack<V> acc = zero_pack<V>();
+        int idx[V];
+#pragma unroll
+        for (int u = 0; u < V; ++u) idx[u] = -1;
+        for (int e = e0; e < e1; ++e) {
+            const int i = nn_index[(int64_t)order[e] * 2 + 1];
+            if (i < 0 || i >= Np) continue;
+            const Pack<V> x = ldp<V>(in + (int64_t)i * C + c);
+#pragma unroll
+            for (int u = 0; u < V; ++u) {
+                if constexpr (MODE == 0) {
+                    if (idx[u] < 0 || x.v[u] > acc.v[u]) { acc.v[u] = x.v[u]; idx[u] = i; }
+                } else {
+                    acc.v[u] += x.v[u];
+                }
+            }
+        }
+        if constexpr (MODE == 1) {
+#pragma unroll
+            for (int u = 0; u < V; ++u) acc.v[u] *= inv;
+        }
+        stp<V>(out + row * C + c, acc);
+        if constexpr (MODE == 0) {
+#pragma unroll
+            for (int u = 0; u < V; ++u) max_index[row * C + c + u] = idx[u];
+        }
+    }
+}
+
+// rows = database points: the gradient of every query that took its maximum here (MODE 0) / of every query it is a
+// neighbour of, divided by that query's count (MODE 1)
+template <int V, int MODE>
+__global__ __launch_bounds__(kBlock) void point_pool_bwd_k(const float *__restrict__ gout, const int *__restrict__ max_index,
+                                                           const int *__restrict__ nn_index, const int *__restrict__ nn_count,
+                                                           const int *__restrict__ rowptr, const int *__restrict__ order,
+                                                           float *__restrict__ gin, int64_t Np, int64_t Mp, int C, int items,
+                                                           int lpr_log2)
+{
+    const int lpr = 1 << lpr_log2, lane = threadIdx.x & (lpr - 1), slot = threadIdx.x >> lpr_log2;
+    const int64_t row = (int64_t)blockIdx.x * (kBlock >> lpr_log2) + slot;
+    if (row >= Np) return;
+    const int e0 = rowptr[row], e1 = rowptr[row + 1];
+    for (int q = lane; q < items; q += lpr) {
+        const int c = q * V;
+        Pack<V> acc = zero_pack<V>();
+        for (int e = e0; e < e1; ++e) {
+            const int o = nn_index[(int64_t)order[e] * 2];
+            if (o < 0 || o >= Mp) continue;
+            const Pack<V> go = ldp<V>(gout + (int64_t)o * C + c);
+            if constexpr (MODE == 0) {
+#pragma unroll
+                for (int u = 0; u < V; ++u) acc.v[u] += (max_index[(int64_t)o * C + c + u] == (int)row) ? go.v[u] : 0.f;
+            } else {
+                const float inv = inv_count(nn_count, o);
+#pragma unroll
+                for (int u = 0; u < V; ++u) acc.v[u] = fmaf(go.v[u], inv, acc.v[u]);
+            }
+        }
+        stp<V>(gin + row * C + c, acc);
+    }
+}
+
+// ------------------------------------------------------------------------------------------------ unpooling
+template <int V>
+__global__ __launch_bounds__(kBlock) void point_unpool_fwd_k(const float *__restrict__ in, const float *__restrict__ weight,
+                                                             const int *__restrict__ nn_index, float *__restrict__ out, int64_t Nrows,
+                                                             int64_t Nin, int C, int K, int items, int lpr_log2)
+{
+    const int lpr = 1 << lpr_log2, lane = threadIdx.x & (lpr - 1), slot = threadIdx.x >> lpr_log2;
+    const int64_t row = (int64_t)blockIdx.x * (kBlock >> lpr_log2) + slot;
+    if (row >= Nrows) return;
+    for (int q = lane; q < items; q += lpr) {
+        const int c = q * V;
+        Pack<V> acc = zero_pack<V>();
+        for (int k = 0; k < K; ++k) {
+            const int i = nn_index[row * K + k];
+            if (i < 0 || i >= Nin) continue;
+            const float w = weight[row * K + k];
+            const Pack<V> x = ldp<V>(in + (int64_t)i * C + c);
+#pragma unroll
+            for (int u = 0; u < V; ++u) acc.v[u] = fmaf(x.v[u], w, acc.v[u]);
+        }
+        stp<V>(out + row * C + c, acc);
+    }
+}
+
+// rows = coarse points; entries e = o * K + k of the flattened index array that name the row
+template <int V>
+__global__ __launch_bounds__(kBlock) void point_unpool_bwd_k(const float *__restrict__ gout, const float *__restrict__ weight,
+                                                             const int *__restrict__ rowptr, const int *__restrict__ order,
+                                                             float *__restrict__ gin, int64_t Nin, int C, int K, int items,
+                                                             int lpr_log2)
+{
+    const int lpr = 1 << lpr_log2, lane = threadIdx.x & (lpr - 1), slot = threadIdx.x >> lpr_log2;
+    const int64_t row = (int64_t)blockIdx.x * (kBlock >> lpr_log2) + slot;
+    if (row >= Nin) return;
+    const int e0 = rowptr[row], e1 = rowptr[row + 1];
+    for (int q = lane; q < items; q += lpr) {
+        const int c = q * V;
+        Pack<V> acc = zero_pack<V>();
+        for (int e = e0; e < e1; ++e) {
+            const int64_t ent = order[e];
+            const float w = weight[ent];
+            const Pack<V> go = ldp<V>(gout + (ent / K) * C + c);
+#pragma unroll
+            for (int u = 0; u < V; ++u) acc.v[u] = fmaf(go.v[u], w, acc.v[u]);
+        }
+        stp<V>(gin + row * C + c, acc);
+    }
+}
+
+static bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// number of workgroups (pair ranges) of the filter gradient: a function of the problem only, capped so that the partial
+// results stay below 64 MiB
+static int filt_blocks(int64_t Nout, int F, int CR)
+{
+    int64_t G = ceil_div(Nout, 256);
+    if (G < 1) G = 1;
+    if (G > 1024) G = 1024;
+    const int64_t per = (int64_t)F * CR * 4;
+    while (G > 1 && G * per > (int64_t(64) << 20)) G /= 2;
+    return (int)G;
+}
+
+}  // namespace pmesh
+
+using namespace pmesh;
+
+#define PM_POINT_DIMS(name)                                                                                          \
+    PM_REQUIRE(Np >= 0 && Mp >= 0 && Nout >= 0 && Np <= INT32_MAX && Mp <= INT32_MAX && Nout < INT32_MAX, name ": bad sizes"); \
+    PM_REQUIRE(C > 0 && C <= (1 << 20), name ": bad channel count C=%d", C)
+
+#define PM_ROW_LAUNCH(kernel, rows, items_, ...)                                                                     \
+    do {                                                                                                             \
+        const RowShape rs = row_shape(items_);                                                                       \
+        const int64_t blocks = ceil_div(rows, rs.rpb);                                                               \
+        PM_REQUIRE(grid_ok(blocks), "grid too large");                                                               \
+        kernel<<<dim3((unsigned)blocks), dim3(kBlock), 0, st>>>(__VA_ARGS__, rs.items, rs.lpr_log2);                 \
+    } while (0)
+
+extern "C" int pmesh_point_conv_fwd(const float *input, const float *filter, const int32_t *nn_count, const int32_t *nn_index,
+                                    const int32_t *bin_index, const float *bin_coeff, const int32_t *rowptr, const int32_t *order,
+                                    float *output, int64_t Np, int64_t Mp, int64_t Nout, int F, int C, int r, int T,
+                                    pmesh_stream_t stream)
+{
+    clear_error();
+    PM_POINT_DIMS("point_conv_fwd");
+    PM_REQUIRE(F > 0 && r > 0 && T > 0 && (int64_t)C * r <= (1 << 20), "point_conv_fwd: bad filter shape");
+    if (Mp == 0) return 0;
+    PM_REQUIRE(output && nn_count && rowptr && filter, "point_conv_fwd: null pointer");
+    PM_REQUIRE(Nout == 0 || (input && nn_index && bin_index && order), "point_conv_fwd: null pointer");
+    hipStream_t st = (hipStream_t)stream;
+    const PairGraph g = {nn_index, nn_count, bin_index, bin_coeff, Np, Mp, Nout, T, F};
+    const int CR = C * r;
+    if (r == 1 && C % 4 == 0 && aligned16(input) && aligned16(filter) && aligned16(output))
+        PM_ROW_LAUNCH(point_conv_fwd_k<4>, Mp, CR / 4, input, filter, g, rowptr, order, output, C, r);
+    else
+        PM_ROW_LAUNCH(point_conv_fwd_k<1>, Mp, CR, input, filter, g, rowptr, order, output, C, r);
+    PM_LAUNCHED("point_conv_fwd");
+    return 0;
+}
+
+extern "C" size_t pmesh_point_conv_bwd_workspace_bytes(int64_t Nout, int F, int C, int r)
+{
+    if (Nout < 0 || F <= 0 || C <= 0 || r <= 0) return 0;
+    return (size_t)filt_blocks(Nout, F, C * r) * F * C * r * sizeof(float);
+}
+
+extern "C" int pmesh_point_conv_bwd(const float *grad_output, const float *input, const float *filter, const int32_t *nn_count,
+                                    const int32_t *nn_index, const int32_t *bin_index, const float *bin_coeff,
+                                    const int32_t *rowptr_in, const int32_t *order_in, float *grad_input, float *grad_filter,
+                                    void *workspace, size_t workspace_bytes, int64_t Np, int64_t Mp, int64_t Nout, int F, int C,
+                                    int r, int T, pmesh_stream_t stream)
+{
+    clear_error();
+    PM_POINT_DIMS("point_conv_bwd");
+    PM_REQUIRE(F > 0 && F <= 512 && r > 0 && T > 0 && (int64_t)C * r <= (1 << 20), "point_conv_bwd: bad filter shape (at most 512 bins)");
+    PM_REQUIRE(grad_filter, "point_conv_bwd: null pointer");
+    hipStream_t st = (hipStream_t)stream;
+    const int CR = C * r;
+    if (Nout == 0 || Mp == 0 || Np == 0) {
+        if (grad_input && Np > 0)
+            if (int rc = reduce_partials(nullptr, grad_input, 0, (int)(Np * C), st)) return rc;
+        return reduce_partials(nullptr, grad_filter, 0, F * CR, st);
+    }
+    PM_REQUIRE(grad_output && input && filter && nn_count && nn_index && bin_index && workspace, "point_conv_bwd: null pointer");
+    const PairGraph g = {nn_index, nn_count, bin_index, bin_coeff, Np, Mp, Nout, T, F};
+    if (grad_input) {
+        PM_REQUIRE(rowptr_in && order_in, "point_conv_bwd: the input gradient needs the pairs sorted by database point");
+        if (r == 1 && C % 4 == 0 && aligned16(grad_output) && aligned16(filter) && aligned16(grad_input))
+            PM_ROW_LAUNCH(point_conv_bwd_in_k<4>, Np, C / 4, grad_output, filter, g, rowptr_in, order_in, grad_input, C, r);
+        else
+            PM_ROW_LAUNCH(point_conv_bwd_in_k<1>, Np, C, grad_output, filter, g, rowptr_in, order_in, grad_input, C, r);
+        PM_LAUNCHED("point_conv_bwd(input)");
+    }
+    const int G = filt_blocks(Nout, F, CR);
+    PM_REQUIRE(workspace_bytes >= (size_t)G * F * CR * sizeof(float), "point_conv_bwd: workspace too small (%zu bytes)", workspace_bytes);
+    int cols = 256;
+    while (cols > 32 && ((size_t)F * cols * 4 > 65536 || cols / 2 >= CR)) cols /= 2;
+    PM_REQUIRE((size_t)F * cols * 4 <= 65536, "point_conv_bwd: too many bins");
+    const int64_t per = ceil_div(Nout, G);
+    point_conv_bwd_filt_k<<<dim3((unsigned)G, (unsigned)ceil_div(CR, cols)), dim3(cols), (size_t)F * cols * 4, st>>>(
+        grad_output, input, g, (float *)workspace, C, r, cols, per);
+    PM_LAUNCHED("point_conv_bwd(filter)");
+    return reduce_partials((const float *)workspace, grad_filter, G, F * CR, st);
+}
+
+extern "C" int pmesh_point_pool_max_fwd(const float *input, const int32_t *nn_index, const int32_t *rowptr, const int32_t *order,
+                                        float *output, int32_t *max_index, int64_t Np, int64_t Mp, int64_t Nout, int C,
+                                        pmesh_stream_t stream)
+{
+    clear_error();
+    PM_POINT_DIMS("point_pool_max_fwd");
+    if (Mp == 0) return 0;
+    PM_REQUIRE(output && max_index && rowptr && (Nout == 0 || (input && nn_index && order)), "point_pool_max_fwd: null pointer");
+    hipStream_t st = (hipStream_t)stream;
+    if (C % 4 == 0 && aligned16(input) && aligned16(output))
+        PM_ROW_LAUNCH((point_pool_fwd_k<4, 0>), Mp, C / 4, input, nn_index, nullptr, rowptr, order, output, max_index, Np, Mp, C);
+    else
+        PM_ROW_LAUNCH((point_pool_fwd_k<1, 0>), Mp, C, input, nn_index, nullptr, rowptr, order, output, max_index, Np, Mp, C);
+    PM_LAUNCHED("point_pool_max_fwd");
+    return 0;
+}
+
+extern "C" int pmesh_point_pool_max_bwd(const float *grad_output, const int32_t *max_index, const int32_t *nn_index,
+                                        const int32_t *rowptr_in, const int32_t *order_in, float *grad_input, int64_t Np, int64_t Mp,
+                                        int64_t Nout, int C, pmesh_stream_t stream)
+{
+    clear_error();
+    PM_POINT_DIMS("point_pool_max_bwd");
+    if (Np == 0) return 0;
+    PM_REQUIRE(grad_input && rowptr_in && (Nout == 0 || (grad_output && max_index && nn_index && order_in)), "point_pool_max_bwd: null pointer");
+    hipStream_t st = (hipStream_t)stream;
+    if (C % 4 == 0 && aligned16(grad_output) && aligned16(grad_input))
+        PM_ROW_LAUNCH((point_pool_bwd_k<4, 0>), Np, C / 4, grad_output, max_index, nn_index, nullptr, rowptr_in, order_in, grad_input, Np, Mp, C);
+    else
+        PM_ROW_LAUNCH((point_pool_bwd_k<1, 0>), Np, C, grad_output, max_index, nn_index, nullptr, rowptr_in, order_in, grad_input, Np, Mp, C);
+    PM_LAUNCHED("point_pool_max_bwd");
+    return 0;
+}
+
+extern "C" int pmesh_point_pool_avg_fwd(const float *input, const int32_t *nn_count, const int32_t *nn_index, const int32_t *rowptr,
+                                        const int32_t *order, float *output, int64_t Np, int64_t Mp, int64_t Nout, int C,
+                                        pmesh_stream_t stream)
+{
+    clear_error();
+    PM_POINT_DIMS("point_pool_avg_fwd");
+    if (Mp == 0) return 0;
+    PM_REQUIRE(output && nn_count && rowptr && (Nout == 0 || (input && nn_index && order)), "point_pool_avg_fwd: null pointer");
+    hipStream_t st = (hipStream_t)stream;
+    if (C % 4 == 0 && aligned16(input) && aligned16(output))
+        PM_ROW_LAUNCH((point_pool_fwd_k<4, 1>), Mp, C / 4, input, nn_index, nn_count, rowptr, order, output, nullptr, Np, Mp, C);
+    else
+        PM_ROW_LAUNCH((point_pool_fwd_k<1, 1>), Mp, C, input, nn_index, nn_count, rowptr, order, output, nullptr, Np, Mp, C);
+    PM_LAUNCHED("point_pool_avg_fwd");
+    return 0;
+}
+
+extern "C" int pmesh_point_pool_avg_bwd(const float *grad_output, const int32_t *nn_count, const int32_t *nn_index,
+                                        const int32_t *rowptr_in, const int32_t *order_in, float *grad_input, int64_t Np, int64_t Mp,
+                                        int64_t Nout, int C, pmesh_stream_t stream)
+{
+    clear_error();
+    PM_POINT_DIMS("point_pool_avg_bwd");
+    if (Np == 0) return 0;
+    PM_REQUIRE(grad_input && rowptr_in && (Nout == 0 || (grad_output && nn_count && nn_index && order_in)), "point_pool_avg_bwd: null pointer");
+    hipStream_t st = (hipStream_t)stream;
+    if (C % 4 == 0 && aligned16(grad_output) && aligned16(grad_input))
+        PM_ROW_LAUNCH((point_pool_bwd_k<4, 1>), Np, C / 4, grad_output, nullptr, nn_index, nn_count, rowptr_in, order_in, grad_input, Np, Mp, C);
+    else
+        PM_ROW_LAUNCH((point_pool_bwd_k<1, 1>), Np, C, grad_output, nullptr, nn_index, nn_count, rowptr_in, order_in, grad_input, Np, Mp, C);
+    PM_LAUNCHED("point_pool_avg_bwd");
+    return 0;
+}
+
+extern "C" int pmesh_point_unpool_fwd(const float *input, const float *weight, const int32_t *nn_index, float *output, int64_t Nrows,
+                                      int64_t Nin, int C, int K, pmesh_stream_t stream)
+{
+    clear_error();
+    PM_REQUIRE(Nrows >= 0 && Nin >= 0 && Nrows <= INT32_MAX && Nin <= INT32_MAX && C > 0 && C <= (1 << 20) && K > 0 && K <= 1024,
+               "point_unpool_fwd: bad sizes");
+    if (Nrows == 0) return 0;
+    PM_REQUIRE(output && weight && nn_index && (Nin == 0 || input), "point_unpool_fwd: null pointer");
+    hipStream_t st = (hipStream_t)stream;
+    if (C % 4 == 0 && aligned16(input) && aligned16(output))
+        PM_ROW_LAUNCH(point_unpool_fwd_k<4>, Nrows, C / 4, input, weight, nn_index, output, Nrows, Nin, C, K);
+    else
+        PM_ROW_LAUNCH(point_unpool_fwd_k<1>, Nrows, C, input, weight, nn_index, output, Nrows, Nin, C, K);
+    PM_LAUNCHED("point_unpool_fwd");
+    return 0;
+}
+
+extern "C" int pmesh_point_unpool_bwd(const float *grad_output, const float *weight, const int32_t *rowptr_in, const int32_t *order_in,
+                                      float *grad_input, int64_t Nrows, int64_t Nin, int C, int K, pmesh_stream_t stream)
+{
+    clear_error();
+    PM_REQUIRE(Nrows >= 0 && Nin >= 0 && Nrows <= INT32_MAX / (K > 0 ? K : 1) && Nin <= INT32_MAX && C > 0 && C <= (1 << 20) && K > 0 && K <= 1024,
+               "point_unpool_bwd: bad sizes");
+    if (Nin == 0) return 0;
+    PM_REQUIRE(grad_input && rowptr_in && (Nrows == 0 || (grad_output && weight && order_in)), "point_unpool_bwd: null pointer");
+    hipStream_t st = (hipStream_t)stream;
+    if (C % 4 == 0 && aligned16(grad_output) && aligned16(grad_input))
+        PM_ROW_LAUNCH(point_unpool_bwd_k<4>, Nin, C / 4, grad_output, weight, rowptr_in, order_in, grad_input, Nin, C, K);
+    else
+        PM_ROW_LAUNCH(point_unpool_bwd_k<1>, Nin, C, grad_output, weight, rowptr_in, order_in, grad_input, Nin, C, K);
+    PM_LAUNCHED("point_unpool_bwd");
+    return 0;
+}

@@ -196,6 +196,29 @@ def cluster_csr(vt_replace, vt_map, n_coarse):
     return rowptr, members
 
 
+def index_csr(index, column, n_rows):
+    """Row r -> ascending list of the entries i with ``index[i, column] == r`` (the point-cloud ops' pairs sorted by
+    query or by database point); ``column`` None takes the flattened tensor itself as the keys.
+    Returns (rowptr int32 (n_rows + 1), order int32 (n_entries))."""
+    key = _key("i", index, -1 if column is None else int(column), int(n_rows))
+    hit = _lookup(key)
+    if hit is not None:
+        return hit
+    if column is None:
+        n, stride, offset = index.numel(), 1, 0
+    else:
+        n, stride, offset = index.shape[0], index.shape[1], int(column)
+    with torch.cuda.device(index.device):
+        rowptr = torch.empty(n_rows + 1, dtype=torch.int32, device=index.device)
+        order = torch.empty(n, dtype=torch.int32, device=index.device)
+        ws_bytes = _lib.query("pmesh_index_csr_workspace_bytes", n, n_rows)
+        ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=index.device)
+        _lib.call("pmesh_build_index_csr", index.data_ptr() + 4 * offset if n else None, stride, n, n_rows, rowptr.data_ptr(),
+                  order.data_ptr(), ws.data_ptr(), ws_bytes, _stream(index))
+    _store(key, (rowptr, order), (index,), (rowptr, order))
+    return rowptr, order
+
+
 def facet_order(cum_texture, n_points):
     """Permutation of the facets by their number of texture points (stable), from the running
     total ``cum_texture``; lets the facet2facet kernels give every wavefront facets of equal length."""

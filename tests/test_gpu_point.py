@@ -1,0 +1,234 @@
+"""The point-cloud branch on the GPU against oracle/point_ref.py, through the reference-shaped API.
+
+Searches, sampling and arg-max indices bit-exact (the device compares the same float32 distances, each operation
+rounded on its own); kernel bins exact away from bin borders, fuzzy weights within 1e-5; convolution, pooling and
+unpooling outputs and gradients within 1e-5 of the float64 oracle."""
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import point_ref as P
+from picassoplus_amd.point import layers as point_layers
+from picassoplus_amd.point import utils as point_utils
+from picassoplus_amd.point.pi_modules import (buildkernel, conv3d, nnquery, point_nnquery, point_pool3d, pool3d, sample,
+                                               unpool3d)
+from test_oracle_point import cloud, subsample
+from util import assert_close, dev
+
+pytestmark = pytest.mark.gpu
+I32, F32 = torch.int32, torch.float32
+
+
+def say(*a):
+    print(*a, flush=True)
+    sys.stdout.flush()
+
+
+def n(t):
+    return t.detach().cpu().numpy()
+
+
+@pytest.mark.parametrize("sizes,frac,radius,limit", [([300, 1, 120], 0.4, 0.2, None), ([2000, 1500], 1.0, 0.12, None),
+                                                     ([500], 0.5, 0.3, 7), ([64, 64, 64, 64, 64], 1.0, 0.5, 1),
+                                                     ([4000], 0.25, 0.05, None)])
+def test_range_cube_knn_bit_exact(cuda, sizes, frac, radius, limit):
+    say("case point search", sizes, frac, radius, limit)
+    db, nvd = cloud(21, sizes)
+    q, nvq = (db, nvd) if frac == 1.0 else subsample(22, db, nvd, frac)
+    D, Q, ND, NQ = dev(db, cuda), dev(q, cuda), dev(nvd, cuda), dev(nvq, cuda)
+    cnt_info, nn_count, nn_index, nn_dist = nnquery.range_search_(D, Q, ND, NQ, radius=radius, nnsample=limit)
+    w = P.range_search(db, q, np.cumsum(nvd), np.cumsum(nvq), radius, 2147483647 if limit is None else limit)
+    assert cnt_info.dtype == torch.int64 and nn_count.dtype == I32 and nn_index.dtype == I32
+    assert np.array_equal(n(cnt_info), w[0]) and np.array_equal(n(nn_count), w[1])
+    assert np.array_equal(n(nn_index), w[2]) and np.array_equal(n(nn_dist), w[3])
+    cnt_info, nn_count, nn_index = nnquery.cube_search_(D, Q, ND, NQ, length=2 * radius, nnsample=limit, gridsize=3)
+    w = P.cube_search(db, q, np.cumsum(nvd), np.cumsum(nvq), 2 * radius, 2147483647 if limit is None else limit, 3)
+    assert np.array_equal(n(cnt_info), w[0]) and np.array_equal(n(nn_count), w[1]) and np.array_equal(n(nn_index), w[2])
+    nn3, d3 = nnquery.knn3_search_(D, Q, ND, NQ)
+    w = P.knn3_search(db, q, np.cumsum(nvd), np.cumsum(nvq))
+    assert np.array_equal(n(nn3), w[0]) and np.array_equal(n(d3), w[1])
+    # extra feature columns of the point arrays are ignored
+    wide = torch.cat([D, torch.ones_like(D)], 1)
+    again = nnquery.range_search_(wide, Q, ND, NQ, radius=radius, nnsample=limit)
+    assert torch.equal(again[2], nnquery.range_search_(D, Q, ND, NQ, radius=radius, nnsample=limit)[2])
+
+
+@pytest.mark.parametrize("sizes,keep", [([120, 60], [15, 60]), ([3000], [700]), ([1, 5, 2048], [1, 3, 256])])
+def test_fps_bit_exact(cuda, sizes, keep):
+    say("case point fps", sizes, keep)
+    xyz, nv = cloud(23, sizes)
+    m = np.array(keep, np.int32)
+    got = sample.fps_(dev(xyz, cuda), dev(nv, cuda), dev(m, cuda))
+    assert got.dtype == I32 and np.array_equal(n(got), P.fps(xyz, np.cumsum(nv), np.cumsum(m)))
+
+
+@pytest.mark.parametrize("kernel", [(8, 2, 3), (8, 4, 1), (4, 2, 2)])
+def test_kernel_bins(cuda, kernel):
+    say("case point bins", kernel)
+    db, nvd = cloud(24, [1500, 900])
+    q, nvq = subsample(25, db, nvd, 0.3)
+    radius = 0.25
+    _, _, nn_index, nn_dist = P.range_search(db, q, np.cumsum(nvd), np.cumsum(nvq), radius)
+    D, Q, NI, ND = dev(db, cuda), dev(q, cuda), dev(nn_index, cuda), dev(nn_dist, cuda)
+    got = n(buildkernel.SPH3Dkernel_(D, Q, NI, ND, radius, kernel=list(kernel)))
+    want, (al, be, ga) = P.sph3d_kernel(db, q, nn_index, nn_dist, radius, kernel)
+    # a pair within 1e-4 of a bin border (or of the centre radius) may fall on either side of it
+    frac = lambda v: np.abs(v - np.round(v))
+    away = (frac(al) > 1e-4) & (frac(be) > 1e-4) & (frac(ga) > 1e-4)
+    centre = nn_dist < 0.3 * radius - 1e-6                            # bin 0 whatever the direction (a point paired with itself too)
+    clear = centre | (away & (nn_dist > 0.3 * radius + 1e-6))
+    assert clear.mean() > 0.99 and np.array_equal(got[clear], want[clear])
+    assert got.min() >= 0 and got.max() <= kernel[0] * kernel[1] * kernel[2]
+    fi, fc = buildkernel.fuzzySPH3Dkernel_(D, Q, NI, ND, radius, kernel=list(kernel))
+    wi, wc, _ = P.fuzzy_sph3d_kernel(db, q, nn_index, nn_dist, radius, kernel)
+    clear = away & (nn_dist > 0) & (np.abs(frac(be) - 0.5) > 1e-4)     # also clear of the side the pair leans to
+    assert clear.mean() > 0.97
+    assert np.abs(n(fc) - wc).max() < 1e-5 or np.abs(n(fc)[clear] - wc[clear]).max() < 1e-5
+    assert np.array_equal(n(fi)[clear], wi[clear]) and np.abs(n(fc)[clear] - wc[clear]).max() < 1e-5
+    assert np.allclose(n(fc).sum(1), 1, atol=1e-5)
+
+
+def point_graph(cuda, seed, sizes, radius, T, F, limit=None):
+    rng = np.random.default_rng(seed)
+    db, nvd = cloud(seed, sizes)
+    q, nvq = subsample(seed + 1, db, nvd, 0.5)
+    _, count, nn_index, nn_dist = P.range_search(db, q, np.cumsum(nvd), np.cumsum(nvq), radius, 2147483647 if limit is None else limit)
+    if T is None:
+        bins, coeff = rng.integers(0, F, len(nn_index)).astype(np.int32), None
+    else:
+        bins = rng.integers(0, F, (len(nn_index), T)).astype(np.int32)
+        coeff = rng.uniform(0, 1, (len(nn_index), T)).astype(np.float32)
+    return db, q, count, nn_index, nn_dist, bins, coeff
+
+
+@pytest.mark.parametrize("sizes,radius,C,r,F,T", [([60], 0.45, 5, 1, 7, None), ([60], 0.45, 5, 2, 7, 3), ([800, 500], 0.2, 64, 1, 17, 17),
+                                                  ([2000], 0.15, 32, 2, 33, 3), ([300], 0.3, 130, 1, 49, None),
+                                                  ([500], 0.25, 16, 1, 125, 1), ([400], 0.25, 8, 3, 300, 2)])
+def test_conv_parity(cuda, sizes, radius, C, r, F, T):
+    say("case point conv", sizes, radius, C, r, F, T)
+    db, q, count, nn_index, _, bins, coeff = point_graph(cuda, 31, sizes, radius, T, F)
+    rng = np.random.default_rng(32)
+    x, filt = rng.normal(size=(len(db), C)), rng.normal(0, 0.3, (F, C, r))
+    g = rng.normal(size=(len(q), C * r))
+    out_ref = P.conv_fwd(x, filt, count, nn_index, bins, coeff)
+    gin_ref, gfilt_ref = P.conv_bwd(g, x, filt, count, nn_index, bins, coeff)
+    xt, ft = dev(x, cuda, F32).requires_grad_(True), dev(filt, cuda, F32).requires_grad_(True)
+    args = (dev(count, cuda), dev(nn_index, cuda), dev(bins, cuda))
+    out = conv3d.conv3d(xt, ft, *args) if coeff is None else conv3d.fuzzyconv3d(xt, ft, *args, dev(coeff, cuda))
+    out.backward(dev(g, cuda, F32))
+    torch.cuda.synchronize()
+    assert_close(out, out_ref, "point conv out")
+    assert_close(xt.grad, gin_ref, "point conv grad_input")
+    assert_close(ft.grad, gfilt_ref, "point conv grad_filter")
+    # same bits on a second run
+    xt2, ft2 = xt.detach().clone().requires_grad_(True), ft.detach().clone().requires_grad_(True)
+    out2 = conv3d.conv3d(xt2, ft2, *args) if coeff is None else conv3d.fuzzyconv3d(xt2, ft2, *args, dev(coeff, cuda))
+    out2.backward(dev(g, cuda, F32))
+    assert torch.equal(out, out2) and torch.equal(xt.grad, xt2.grad) and torch.equal(ft.grad, ft2.grad)
+
+
+@pytest.mark.parametrize("sizes,radius,C", [([60], 0.45, 4), ([1500, 700], 0.2, 64), ([900], 0.25, 37)])
+def test_pool_and_unpool_parity(cuda, sizes, radius, C):
+    say("case point pool", sizes, radius, C)
+    db, q, count, nn_index, nn_dist, _, _ = point_graph(cuda, 41, sizes, radius, None, 3)
+    rng = np.random.default_rng(42)
+    x = rng.normal(size=(len(db), C)).astype(np.float32)
+    x[5] = x[9]
+    g = rng.normal(size=(len(q), C)).astype(np.float32)
+    CT, NI = dev(count, cuda), dev(nn_index, cuda)
+    xt = dev(x, cuda).requires_grad_(True)
+    mx = pool3d.maxPool(xt, CT, NI)
+    mx.backward(dev(g, cuda))
+    w_mx, w_idx = P.pool_max_fwd(x, count, nn_index)
+    out, idx = point_pool3d.max_forward(xt.detach(), CT, NI)
+    assert np.array_equal(n(mx), w_mx) and np.array_equal(n(idx), w_idx) and torch.equal(out, mx.detach())
+    assert_close(xt.grad, P.pool_max_bwd(g.astype(np.float64), len(db), w_idx), "point max pool grad")
+    xt.grad = None
+    av = pool3d.avgPool(xt, CT, NI)
+    av.backward(dev(g, cuda))
+    assert_close(av, P.pool_avg_fwd(x, count, nn_index), "point avg pool")
+    assert_close(xt.grad, P.pool_avg_bwd(g, len(db), count, nn_index), "point avg pool grad")
+    with pytest.raises(RuntimeError):
+        point_pool3d.max_backward(dev(g, cuda), xt.detach(), idx)       # the gather form needs the pairs
+    # unpooling from the queries back to the database points
+    nn3, d3 = P.knn3_search(q, db, np.cumsum([max(1, int(s * 0.5)) for s in sizes]), np.cumsum(sizes))
+    w = (1 / (d3 + 1e-8)).astype(np.float32)
+    w = w / w.sum(1, keepdims=True)
+    y = rng.normal(size=(len(q), C)).astype(np.float32)
+    yt = dev(y, cuda).requires_grad_(True)
+    up = unpool3d.interpolate(yt, dev(w, cuda), dev(nn3, cuda))
+    gu = rng.normal(size=(len(db), C)).astype(np.float32)
+    up.backward(dev(gu, cuda))
+    assert_close(up, P.unpool_fwd(y, w, nn3), "point unpool")
+    assert_close(yt.grad, P.unpool_bwd(gu, len(q), w, nn3), "point unpool grad")
+
+
+def test_dual_block_graph_and_module(cuda):
+    """What DualBlock does with the point branch (picasso/networks/pi2_blocks.py:43-62): the spherical-harmonic graph
+    of a vertex set on itself, then PCloudConv3d on it, against the oracle composition."""
+    say("case point module")
+    xyz, nv = cloud(51, [700, 400], scale=1.0)
+    L, radius, limit = 3, 0.2, 20
+    X, NV = dev(xyz, cuda), dev(nv, cuda)
+    nn_cnt, nn_idx, nn_dst, filt_idx, filt_coeff = point_utils.build_sphere_harmonics(X, X, NV, NV, radius, L=L, nn_uplimit=limit)
+    w = P.range_search(xyz, xyz, np.cumsum(nv), np.cumsum(nv), radius, limit)
+    assert np.array_equal(n(nn_cnt), w[1]) and np.array_equal(n(nn_idx), w[2]) and np.array_equal(n(nn_dst), w[3])
+    assert int(nn_cnt.max()) <= limit and int(nn_cnt.min()) >= 1      # every point finds itself
+    K = (L + 1) ** 2 + 1
+    assert tuple(filt_idx.shape) == (len(w[2]), K) and filt_idx.dtype == I32 and torch.equal(filt_idx[0], torch.arange(K, dtype=I32, device=cuda))
+    from oracle import loops
+    delta = xyz[w[2][:, 1]].astype(np.float64) - xyz[w[2][:, 0]].astype(np.float64)
+    gamma = np.clip(w[3].astype(np.float64) / radius, 0, 1)[:, None]
+    # a pair of a point with itself has no direction: the basis is evaluated at (1, 0, 0), as atan2(0, 0) = 0 makes the reference do
+    sh = loops.sph_harm(np.where((np.abs(delta).sum(1) == 0)[:, None], [[1.0, 0, 0]], delta), L)
+    coeff_ref = np.concatenate([1 - gamma, gamma * sh], 1)
+    assert np.abs(n(filt_coeff) - coeff_ref).max() < 2e-6
+    torch.manual_seed(0)
+    conv = point_layers.PCloudConv3d(24, 40, K, with_bn=False).to(cuda)
+    feat = torch.randn(len(xyz), 24, device=cuda, requires_grad=True)
+    out = conv(feat, nn_cnt, nn_idx, filt_idx, filt_coeff)
+    g = torch.randn_like(out)
+    out.backward(g)
+    f64 = lambda t: n(t).astype(np.float64)
+    mid = P.conv_fwd(f64(feat), f64(conv.spatial_weights), w[1], w[2], n(filt_idx), f64(filt_coeff))
+    z = mid @ f64(conv.depth_weights) + f64(conv.biases)
+    assert_close(out, np.maximum(z, 0), "PCloudConv3d out")
+    gz = f64(g) * (z > 0)
+    gmid = gz @ f64(conv.depth_weights).T
+    gin, gfilt = P.conv_bwd(gmid, f64(feat), f64(conv.spatial_weights), w[1], w[2], n(filt_idx), f64(filt_coeff))
+    assert_close(feat.grad, gin, "PCloudConv3d grad input", 2e-5)
+    assert_close(conv.spatial_weights.grad, gfilt, "PCloudConv3d grad spatial", 2e-5)
+    assert_close(conv.depth_weights.grad, mid.T @ gz, "PCloudConv3d grad depth", 2e-5)
+    # the other two graph builders
+    g_rng = point_utils.build_range_graph(X, X, NV, NV, radius, nn_uplimit=limit, kernel_shape=[8, 4, 1], fuzzy=True)
+    assert tuple(g_rng[3].shape) == (len(w[2]), 3) and torch.equal(g_rng[1], nn_idx)
+    g_cube = point_utils.build_cube_graph(X, X, NV, NV, radius, nn_uplimit=limit, grid_size=3)
+    assert g_cube[1].shape[1] == 2 and g_cube[3].dim() == 1 and int(g_cube[3].max()) < 27
+    plain = point_layers.PCloudConv3d(24, 8, 27, with_bn=True).to(cuda)
+    y = plain(feat.detach(), g_cube[0], g_cube[1], g_cube[3])
+    assert tuple(y.shape) == (len(xyz), 8) and bool(torch.isfinite(y).all())
+
+
+def test_point_argument_errors(cuda):
+    say("case point errors")
+    db, nvd = cloud(61, [50])
+    D, ND = dev(db, cuda), dev(nvd, cuda)
+    with pytest.raises(RuntimeError):
+        nnquery.range_search_(D.cpu(), D, ND, ND, radius=0.1)
+    with pytest.raises(RuntimeError):
+        nnquery.range_search_(D, D, ND, ND, radius=-1.0)
+    with pytest.raises(RuntimeError):
+        point_nnquery.range(D, D, ND.long(), ND, 0.1, 5)               # the native layer takes int32 totals only
+    _, cnt, idx, dst = nnquery.range_search_(D, D, ND, ND, radius=0.3)
+    with pytest.raises(RuntimeError):
+        buildkernel.SPH3Dkernel_(D, D, idx, dst, 0.3, kernel=[7, 2, 3])          # odd azimuth count
+    x = torch.randn(50, 4, device=cuda)
+    with pytest.raises(RuntimeError):
+        conv3d.conv3d(x, torch.randn(3, 5, 1, device=cuda), cnt, idx, torch.zeros(len(idx), dtype=I32, device=cuda))
+    with pytest.raises(RuntimeError):
+        conv3d.conv3d(x, torch.randn(3, 4, 1, device=cuda), cnt, idx, torch.zeros(len(idx), dtype=torch.int64, device=cuda))
+    # empty inputs
+    e = nnquery.range_search_(D, D[:0], ND, ND * 0, radius=0.1)
+    assert e[2].shape == (0, 2) and e[1].shape == (0,)

@@ -18,6 +18,7 @@
 // phase, so the prologue, barriers and stores of one overlap the channel loop of the other.  Filter chunks
 // of four channels alternate between two LDS buffers and arrive there straight from global memory, requested one
 // chunk ahead; texture rows go through a wavefront-private LDS slab.
+#include <type_traits>
 #include "f2f_internal.h"
 
 namespace pmesh {
@@ -201,14 +202,43 @@ __device__ __forceinline__ f32x16 mfma_f16(const u32x4 &a, const u32x4 &b, const
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
 }
 
+// Maxima over the wavefront without a trip through LDS: four data-parallel-primitive steps leave the maximum of each
+// row of 16 lanes in all of its lanes (lane ^ 1, lane ^ 2, mirror of 8, mirror of 16), one lane of each row is read
+// into a scalar register.  All 64 lanes must be active.
+template <int CTRL> __device__ __forceinline__ int hdpp(int v) { return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xF, 0xF, true); }
+__device__ __forceinline__ int hrow_max(int v)
+{
+    int t;
+    t = hdpp<0xB1>(v); v = t > v ? t : v;
+    t = hdpp<0x4E>(v); v = t > v ? t : v;
+    t = hdpp<0x141>(v); v = t > v ? t : v;
+    t = hdpp<0x140>(v); v = t > v ? t : v;
+    return v;
+}
 __device__ __forceinline__ int hwave_max(int v)
 {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) {
-        const int t = __shfl_xor(v, o, 64);
-        v = t > v ? t : v;
-    }
-    return __builtin_amdgcn_readfirstlane(v);
+    v = hrow_max(v);
+    const int a = __builtin_amdgcn_readlane(v, 0), b = __builtin_amdgcn_readlane(v, 16);
+    const int c = __builtin_amdgcn_readlane(v, 32), d = __builtin_amdgcn_readlane(v, 48);
+    const int ab = a > b ? a : b, cd = c > d ? c : d;
+    return ab > cd ? ab : cd;
+}
+__device__ __forceinline__ float hrow_fmax(float m)
+{
+    m = fmaxf(m, __builtin_bit_cast(float, hdpp<0xB1>(__builtin_bit_cast(int, m))));
+    m = fmaxf(m, __builtin_bit_cast(float, hdpp<0x4E>(__builtin_bit_cast(int, m))));
+    m = fmaxf(m, __builtin_bit_cast(float, hdpp<0x141>(__builtin_bit_cast(int, m))));
+    m = fmaxf(m, __builtin_bit_cast(float, hdpp<0x140>(__builtin_bit_cast(int, m))));
+    return m;
+}
+__device__ __forceinline__ float hwave_fmax(float m)
+{
+    const int v = __builtin_bit_cast(int, hrow_fmax(m));
+    const float a = __builtin_bit_cast(float, __builtin_amdgcn_readlane(v, 0));
+    const float b = __builtin_bit_cast(float, __builtin_amdgcn_readlane(v, 16));
+    const float c = __builtin_bit_cast(float, __builtin_amdgcn_readlane(v, 32));
+    const float d = __builtin_bit_cast(float, __builtin_amdgcn_readlane(v, 48));
+    return fmaxf(fmaxf(a, b), fmaxf(c, d));
 }
 
 // Power of two s with s * m < 2^14 for a bound m >= 0 (s = 1 for m = 0 or non-finite m); *inv = 1 / s.
@@ -1053,17 +1083,34 @@ int f2f16h2_bwd_texture(const void *gout_, const float *W, const float *sh, cons
 //   workgroup  4 wavefronts (one per SIMD), 64 input x 64 output channels, a strided subset of the tiles
 //   wavefront  16 input channels = 8 channel pairs x 2 output tiles of gW^T[(ci,d)][co]; narrower filters give
 //              every wavefront 1, 2 or 4 pairs instead (NCP)
-template <int KW, int NCP, bool HALF>
+template <int KW, int NCP, bool HALF, bool PRE>
 __device__ __forceinline__ void h2_filt_pass(const float (&shr)[KW][8], const float4 *slab, const u32x4 *go,
                                              f32x16 (&acc)[NCP][2], const u32x4 &ea, const u32x4 &eb, int lane)
 {
     const int l32 = lane & 31;
     // G of channels cbase + 2cp (a) and + 1 (b), eight d's of my half for my facet, as fp16 pieces
+    // texture values of my facet's points for four channels (two pairs).  With few points per facet they are read a
+    // pair of channel pairs ahead, into the registers the wider phases need for their SH values: the blocks of matrix
+    // instructions between the generations are fixed points of the instruction order, and a read issued behind one
+    // would be waited for right there.
+    constexpr bool RP = KW <= 6;
+    float4 tq[RP ? KW : 1];
+    auto slab_at = [&](int kk, int q) -> float4 {
+        return PRE ? slab[(kk * 32 + l32) * 4 + (q ^ ((l32 >> 2) & 3))] : slab[(kk * 4 + q) * 32 + l32];
+    };
+    auto read_q = [&](int q) {
+        if constexpr (RP) {
+#pragma unroll
+            for (int kk = 0; kk < KW; ++kk) tq[kk] = slab_at(kk, q);
+        }
+    };
     auto gen = [&](u32x4 (&pa)[2], u32x4 (&pb)[2], int cp) {
         float aa[8], ab[8];
 #pragma unroll
         for (int kk = 0; kk < KW; ++kk) {
-            const float4 t4 = slab[(kk * 4 + (cp >> 1)) * 32 + l32];
+            float4 t4;
+            if constexpr (RP) t4 = tq[kk];
+            else t4 = slab_at(kk, cp >> 1);
             const float ta = (cp & 1) ? t4.z : t4.x, tb = (cp & 1) ? t4.w : t4.y;
 #pragma unroll
             for (int q = 0; q < 8; ++q) {
@@ -1142,6 +1189,7 @@ __device__ __forceinline__ void h2_filt_pass(const float (&shr)[KW][8], const fl
     // software pipeline over the channel pairs: the G values of pair cp+1 are generated and split
     // (vector ALU) while the products of pair cp run on the matrix core
     u32x4 o[2][2];
+    read_q(0);
     {
         u32x4 pa[2], pb[2];
         gen(pa, pb, 0);
@@ -1151,6 +1199,7 @@ __device__ __forceinline__ void h2_filt_pass(const float (&shr)[KW][8], const fl
     for (int cp = 0; cp < NCP; ++cp) {
         u32x4 pa[2], pb[2];
         if (cp + 1 < NCP) gen(pa, pb, cp + 1);
+        if (!(cp & 1) && cp + 2 < NCP) read_q((cp + 2) >> 1);      // (pair cp + 1 was the last reader of the registers)
 #pragma unroll
         for (int st = 0; st < 2; ++st) {
             // three piece products, smallest first; the two output tiles alternate
@@ -1167,24 +1216,44 @@ __device__ __forceinline__ void h2_filt_pass(const float (&shr)[KW][8], const fl
     }
 }
 
-// slot descriptors of a 32-facet tile: facet id (-1: none), first texture point, number of points
+// 256 zero bytes in global memory: what a fetch without a row reads instead, so that no fetch of the prefetch stage
+// sits behind a branch (a branch per fetch also puts a wait for LDS in front of every single one)
+__device__ __attribute__((aligned(256))) unsigned h2_zero_row[64];
+
+// slot descriptors of a 32-facet tile: facet id (-1: none), first texture point, number of points.  They come in
+// two dependent fetches (facet order, then the running totals of that facet), issued in two different tiles (by lanes
+// i < 32 of two wavefronts, the facet passing through LDS), so that neither waits for the other: the results stay as
+// fetched until the end of the tile.
 struct HTile {
     int f, k0, K;
 };
-__device__ __forceinline__ HTile htile_load(const int *__restrict__ cum, const int *__restrict__ order, int64_t tile,
-                                            int64_t ntiles, int64_t Nf, int T, int i)
+__device__ __forceinline__ int htile_facet(const int *__restrict__ order, int64_t tile, int64_t ntiles, int64_t Nf, int i)
+{
+    const int64_t slot = tile * 32 + i;
+    const bool ok = tile < ntiles && slot < Nf;
+    return order ? order[ok ? slot : 0] : (int)slot;            // (a valid slot's value is used only)
+}
+struct HTileRaw {
+    int f, a, b;                                               // facet or -1, cum[f - 1] (cum[0] for f = 0), cum[f]
+};
+__device__ __forceinline__ HTileRaw htile_totals(const int *__restrict__ cum, int f, int64_t tile, int64_t ntiles, int64_t Nf, int i)
+{
+    const int64_t slot = tile * 32 + i;
+    const bool ok = tile < ntiles && slot < Nf && f >= 0 && f < Nf;
+    const int fi = ok ? f : 0;
+    HTileRaw r;
+    r.f = ok ? f : -1;
+    r.a = cum[fi ? fi - 1 : 0];
+    r.b = cum[fi];
+    return r;
+}
+__device__ __forceinline__ HTile htile_finish(const HTileRaw &r, int T)
 {
     HTile d = {-1, 0, 0};
-    const int64_t slot = tile * 32 + i;
-    if (tile < ntiles && slot < Nf) {
-        const int f = order ? order[slot] : (int)slot;
-        if (f >= 0 && f < Nf) {
-            int a = f ? cum[f - 1] : 0, b = cum[f];
-            a = a < 0 ? 0 : (a > T ? T : a);
-            b = b < 0 ? 0 : (b > T ? T : b);
-            if (b > a) d = {f, a, b - a};
-        }
-    }
+    int a = r.f > 0 ? r.a : 0, b = r.b;
+    a = a < 0 ? 0 : (a > T ? T : a);
+    b = b < 0 ? 0 : (b > T ? T : b);
+    if (r.f >= 0 && b > a) d = {r.f, a, b - a};
     return d;
 }
 
@@ -1197,6 +1266,14 @@ struct HPre {
     float g[8];
     float4 shv[kHShv];
 };
+__device__ __forceinline__ unsigned hld_raw_or_zero(const float *base, int64_t idx, bool ok)
+{
+    return *(ok ? reinterpret_cast<const unsigned *>(base) + idx : h2_zero_row);
+}
+__device__ __forceinline__ unsigned hld_raw_or_zero(const bf16_t *base, int64_t idx, bool ok)
+{
+    return *(ok ? reinterpret_cast<const unsigned *>(base) + (idx >> 1) : h2_zero_row);
+}
 template <typename TIO>
 __device__ __forceinline__ void hpre_issue(HPre &P, const TIO *__restrict__ gout, const float *__restrict__ sh,
                                            const int *sf, const int *sk0, const int *sK, int Cout, int n0)
@@ -1206,15 +1283,18 @@ __device__ __forceinline__ void hpre_issue(HPre &P, const TIO *__restrict__ gout
     for (int j = 0; j < 8; ++j) {
         const int f = sf[16 * st + 8 * (j >> 2) + 4 * hh + (j & 3)];
         // (kept as raw bits until the fetches are out; Cout is even for bf16 rows, so the half is the column's parity)
-        P.g[j] = __builtin_bit_cast(float, (f >= 0 && n0 + co < Cout) ? hld_raw(gout, (int64_t)f * Cout + n0 + co) : 0u);
+        P.g[j] = __builtin_bit_cast(float, hld_raw_or_zero(gout, (int64_t)f * Cout + n0 + co, f >= 0 && n0 + co < Cout));
     }
 #pragma unroll
     for (int j = 0; j < 8; ++j) P.g[j] = hcvt_raw(__builtin_bit_cast(unsigned, P.g[j]), (n0 + co) & 1, TIO());
+    // piece threadIdx.x + 256 i of the SH rows: slot (threadIdx.x / 4) % 32 for every i, point threadIdx.x / 128 + 2 i
+    const int slot = (threadIdx.x >> 2) & 31, K = sK[slot];
+    const float *row0 = sh + ((int64_t)sk0[slot] + (threadIdx.x >> 7)) * 16 + 4 * (threadIdx.x & 3);
 #pragma unroll
     for (int i = 0; i < kHShv; ++i) {
-        const int e = threadIdx.x + 256 * i, row = e >> 2, kk = row >> 5, slot = row & 31;
-        P.shv[i] = (kk < kHKB && kk < sK[slot]) ? hld4(sh + (int64_t)(sk0[slot] + kk) * 16 + 4 * (e & 3))
-                                                : make_float4(0.f, 0.f, 0.f, 0.f);
+        const int kk = (threadIdx.x >> 7) + 2 * i;
+        const bool ok = kk < kHKB && kk < K;
+        P.shv[i] = hld4(ok ? row0 + 32 * i : reinterpret_cast<const float *>(h2_zero_row));
     }
 }
 __device__ __forceinline__ float hpre_gmax(const HPre &P)
@@ -1222,9 +1302,7 @@ __device__ __forceinline__ float hpre_gmax(const HPre &P)
     float m = 0.f;
 #pragma unroll
     for (int j = 0; j < 8; ++j) m = fmaxf(m, fabsf(P.g[j]));
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
-    return m;
+    return hwave_fmax(m);
 }
 // gamma: scale of the gout operand
 __device__ __forceinline__ void hpre_commit(const HPre &P, u32x4 *go, float *shs, float gamma, bool with_sh)
@@ -1265,50 +1343,113 @@ __device__ __forceinline__ void htex_issue(HRaw4<TIO> (&pf)[2 * kHKB], const TIO
     }
 }
 
-__device__ __forceinline__ int htile_kmax(const int *sK, int lane) { return hwave_max(sK[lane & 31]); }
-__device__ __forceinline__ float hwave_fmax(float m)
+// The same rows straight into a slab buffer of the wavefront (fp32 rows of at least 64 channels, at most kHPre points
+// per facet), a whole tile ahead: no register holds them on the way, so the request can leave before the tile in
+// front is multiplied.  Row-major slab, 64 bytes per (point, facet slot); lane L of instruction j delivers the
+// 16 bytes at position 64 j + L, and fetches the piece (L & 3) ^ (slot / 4 & 3) of its row there, which spreads the
+// 16-byte reads of 16 consecutive slots over all banks.  Entries without a row receive zeros from h2_zero_row.
+// The data is there after vmcnt has drained.
+// The requests are written as instructions: the compiler puts a wait for all outstanding fetches in front of the
+// next LDS access it cannot tell apart from the landing zone of such a request, which would end the prefetch right
+// where it starts.  It counts its own fetches only; the ones here are older than any fetch it waits for later in the
+// tile and return in order, so its waits hold.  The readers of the slab wait themselves (hwait_vm0).
+constexpr int kHPre = 6;
+constexpr int kHSlabW = 2 * kHPre * 128;              // float4 of a wavefront's slab: two buffers of kHPre points (>= one of kHKB)
+static_assert(kHSlabW >= kHKB * 128, "slab");
+__device__ __forceinline__ void hdma16(const float *src, unsigned lds_base)
 {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
-    return __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, m)));
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(src), "s"(lds_base) : "memory", "m0");
 }
+template <int KW>
+__device__ __forceinline__ void htex_dma(const float *__restrict__ tex, const int *sk0, const int *sK, float4 *buf, int cw,
+                                         int Cin, int lane)
+{
+    // row 16 j + lane / 4 of the tile's (point, slot) rows: point j / 2, slot lane / 4 or 16 + lane / 4
+    const int r = lane >> 2;
+    const int k0a = sk0[r], Ka = sK[r], k0b = sk0[16 + r], Kb = sK[16 + r];
+    const unsigned base = (unsigned)(size_t)(__attribute__((address_space(3))) void *)buf;
+    // (one address per slot in front of the selections: a product inside a selected operand turns it into a branch)
+    const int pa = (lane & 3) ^ ((r >> 2) & 3), pb = (lane & 3) ^ (((16 + r) >> 2) & 3);
+    const float *rowa = tex + (int64_t)k0a * Cin + cw + 4 * pa, *rowb = tex + (int64_t)k0b * Cin + cw + 4 * pb;
+    const bool cola = cw + 4 * pa < Cin, colb = cw + 4 * pb < Cin;
+#pragma unroll
+    for (int j = 0; j < 2 * KW; ++j) {
+        const int kk = j >> 1;
+        const bool ok = (j & 1) ? (kk < Kb && colb) : (kk < Ka && cola);
+        const float *row = ((j & 1) ? rowb : rowa) + (int64_t)kk * Cin;
+        hdma16(ok ? row : reinterpret_cast<const float *>(h2_zero_row), base + 1024u * j);
+    }
+}
+// every outstanding fetch has arrived (an instruction the compiler keeps count with, and a fence for its LDS reads)
+__device__ __forceinline__ void hwait_vm0()
+{
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    asm volatile("" ::: "memory");
+}
+
 
 // State of the scales: gam_cur (workgroup-uniform) = scale the next operand is split with; S
 // (wavefront-uniform) = scale of the accumulators, fixed by the wavefront's first pass.
 struct HScales {
     float gam_cur, S;
+#ifdef PM_TIMING
+    unsigned long long tm[6];
+#endif
 };
+#ifdef PM_TIMING
+__device__ unsigned long long pm_filt_dbg[4 * 8 + 512 * 4 * 8];
+#define PM_T(i) do { const unsigned long long t_ = __builtin_readcyclecounter(); sc.tm[i] += t_ - tprev_; if (blockIdx.x == 7 && lane == 0 && it < 512) pm_filt_dbg[32 + (it * 4 + w) * 8 + i] = t_ - tprev_; tprev_ = t_; } while (0)
+#else
+#define PM_T(i) do { } while (0)
+#endif
 
 // One tile of 32 facets whose inputs are in LDS buffer it % 2 (descriptors in it % 3): start the
 // fetches for the next tile, run the passes, publish the next tile's inputs.
-template <int KW, bool TVEC, int NCP, bool HALF, typename TIO>
+template <int KW, bool TVEC, int NCP, bool HALF, bool PRE, typename TIO>
 __device__ __forceinline__ void h2_filt_tile(const TIO *__restrict__ gout, const TIO *__restrict__ tex,
                                              const float *__restrict__ sh, const int *__restrict__ cum,
                                              const int *__restrict__ order, u32x4 (*go_s)[2 * 2 * 2 * 64], float4 *slab,
                                              float (*sh_s)[kHKB * 32 * 16], int (*s_f)[32], int (*s_k0)[32],
-                                             int (*s_K)[32], float *s_gamma, unsigned *s_gm, f32x16 (&acc)[NCP][2],
+                                             int (*s_K)[32], int *s_kmax, int (*s_fn)[32], float *s_gamma, unsigned *s_gm, f32x16 (&acc)[NCP][2],
                                              HScales &sc, int *overflow, const u32x4 &ea, const u32x4 &eb, int it, int64_t tile,
                                              int64_t stride, int64_t ntiles, int64_t Nf, int T, int Cin, int Cout, int c0,
                                              int n0, int lane, int w)
 {
     const int l32 = lane & 31, h = lane >> 5;
     const int buf = it & 1, sb = it % 3, sb1 = (it + 1) % 3, sb2 = (it + 2) % 3;
+    const int cw = c0 + 2 * NCP * w;                     // my wavefront's first input channel
+    const bool idle = cw >= Cin;                         // narrow filters leave wavefronts without channels
+#ifdef PM_TIMING
+    unsigned long long tprev_ = __builtin_readcyclecounter();
+#endif
+    if constexpr (PRE) {
+        // my texture rows of this tile were requested a tile ago (or at the start of the phase); nothing else is
+        // outstanding here, the end of the tile before consumed all of its fetches
+        hwait_vm0();
+        if (!idle)
+            if constexpr (std::is_same<TIO, float>::value)
+                htex_dma<KW>(tex, s_k0[sb1], s_K[sb1], slab + ((it + 1) & 1) * (KW * 128), cw, Cin, lane);
+        slab += (it & 1) * (KW * 128);
+    }
     // in flight while this tile is multiplied: inputs of the next tile, descriptors of the one after
     HPre P;
     hpre_issue(P, gout, sh, s_f[sb1], s_k0[sb1], s_K[sb1], Cout, n0);
-    HTile dn = {-1, 0, 0};
-    if (threadIdx.x < 32) dn = htile_load(cum, order, tile + 2 * stride, ntiles, Nf, T, threadIdx.x);
+    // descriptors: running totals of the tile after the next (its facets came in during the tile before), facets
+    // of the one after that
+    HTileRaw dr = {-1, 0, 0};
+    int fn3 = -1;
+    if (w == 1 && lane < 32) dr = htile_totals(cum, s_fn[it & 1][lane], tile + 2 * stride, ntiles, Nf, lane);
+    if (w == 2 && lane < 32) fn3 = htile_facet(order, tile + 3 * stride, ntiles, Nf, lane);
     // maxima of the gout operands: slot (it + 1) % 3 collects the next tile's at the commit below; the slot of
     // the tile after that is cleared here (its last readers passed the barrier that ended the previous tile)
     const int gs = (it + 1) % 3;
     if (threadIdx.x == 0) s_gm[(it + 2) % 3] = 0u;
 
+    PM_T(0);
     const float gamma = s_gamma[buf];
     const int k0 = s_k0[sb][l32], K = s_K[sb][l32];
     const float invK = K > 0 ? 1.0f / (float)K : 0.f;
-    const int nsweeps = KW < kHKB ? 1 : (hwave_max(K) + kHKB - 1) / kHKB;
-    const int cw = c0 + 2 * NCP * w;                     // my wavefront's first input channel
-    const bool idle = cw >= Cin;                         // narrow filters leave wavefronts without channels
+    const int nsweeps = KW < kHKB ? 1 : (__builtin_amdgcn_readfirstlane(s_kmax[sb]) + kHKB - 1) / kHKB;
     for (int sw = 0; sw < nsweeps && !idle; ++sw) {
         const int rem = K - sw * kHKB;
         const int Ks = rem < 0 ? 0 : (rem > KW ? KW : rem);
@@ -1336,7 +1477,10 @@ __device__ __forceinline__ void h2_filt_tile(const TIO *__restrict__ gout, const
             }
         }
         float tmax = 0.f;
-        {
+        if constexpr (PRE) {
+#pragma unroll
+            for (int i = 0; i < 2 * KW; ++i) tmax = absmax4(slab[64 * i + lane], tmax);
+        } else {
             // my wavefront's texture rows of this pass -> slab
             HRaw4<TIO> pf[2 * kHKB];
             htex_issue<KW, TVEC, NCP, TIO>(pf, tex, s_k0[sb], s_K[sb], sw, cw, Cin, lane);
@@ -1375,7 +1519,9 @@ __device__ __forceinline__ void h2_filt_tile(const TIO *__restrict__ gout, const
             for (int kk = 0; kk < KW; ++kk)
 #pragma unroll
                 for (int q = 0; q < 8; ++q) shr[kk][q] *= al;
-            h2_filt_pass<KW, NCP, HALF>(shr, slab, go_s[buf], acc, ea, eb, lane);
+            PM_T(1);
+            h2_filt_pass<KW, NCP, HALF, PRE>(shr, slab, go_s[buf], acc, ea, eb, lane);
+            PM_T(2);
         }
     }
 
@@ -1386,10 +1532,21 @@ __device__ __forceinline__ void h2_filt_tile(const TIO *__restrict__ gout, const
     }
     hpre_commit(P, go_s[buf ^ 1], sh_s[buf ^ 1], sc.gam_cur, true);
     if (threadIdx.x == 0) s_gamma[buf ^ 1] = sc.gam_cur;
-    if (threadIdx.x < 32) {
-        s_f[sb2][threadIdx.x] = dn.f; s_k0[sb2][threadIdx.x] = dn.k0; s_K[sb2][threadIdx.x] = dn.K;
+    if (w == 1) {
+        const HTile dn = htile_finish(dr, T);            // (lanes 32..63: no facet)
+        if (lane < 32) {
+            s_f[sb2][lane] = dn.f; s_k0[sb2][lane] = dn.k0; s_K[sb2][lane] = dn.K;
+        }
+        const int km = hwave_max(dn.K);
+        if (lane == 0) s_kmax[sb2] = km;
     }
+    if (w == 2 && lane < 32) s_fn[(it + 1) & 1][lane] = fn3;       // (read at the start of the next tile)
+    PM_T(3);
     __syncthreads();
+    PM_T(4);
+#ifdef PM_TIMING
+    if (blockIdx.x == 7 && lane == 0 && it < 512) pm_filt_dbg[32 + (it * 4 + w) * 8 + 7] = KW;
+#endif
     const float gm = __builtin_bit_cast(float, s_gm[gs]);
     if (gm > 0.f && !scale_fits(sc.gam_cur, gm)) {           // workgroup-uniform: fetch and split that tile again
         float inv;
@@ -1413,14 +1570,16 @@ __global__ __launch_bounds__(256, 1) void f2f16h2_bwd_filt_k(const TIO *__restri
                                                               int64_t Nf, int T, int Cin, int Cout, int64_t ntiles)
 {
     __shared__ u32x4 go_s[2][2 * 2 * 2 * 64];
-    __shared__ float4 slab_s[4 * kHKB * 4 * 32];
+    __shared__ float4 slab_s[4 * kHSlabW];
     __shared__ __attribute__((aligned(16))) float sh_s[2][kHKB * 32 * 16];
-    __shared__ int s_f[3][32], s_k0[3][32], s_K[3][32];
+    __shared__ int s_f[3][32], s_k0[3][32], s_K[3][32], s_kmax[3], s_fn[2][32];
     __shared__ float s_gamma[2];
     __shared__ unsigned s_gm[3];
-    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63, w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int l32 = lane & 31, h = lane >> 5;
     const int c0 = blockIdx.y * (8 * NCP), n0 = blockIdx.z * 64;
+    // phases of at most kHPre points request their texture rows a tile ahead, into the two halves of the slab
+    constexpr bool kPre = TVEC && NCP == 8 && std::is_same<TIO, float>::value;
 
     // selection operands of the transposition: column n < 16 takes d = n of channel a, n >= 16 takes d = n - 16 of b
     u32x4 ea, eb;
@@ -1445,14 +1604,24 @@ __global__ __launch_bounds__(256, 1) void f2f16h2_bwd_filt_k(const TIO *__restri
 #pragma unroll
             for (int i = 0; i < 16; ++i) acc[cp][t][i] = 0.f;
     HScales sc = {1.0f, 0.f};
+#ifdef PM_TIMING
+    for (int i = 0; i < 6; ++i) sc.tm[i] = 0;
+    const unsigned long long tstart_ = __builtin_readcyclecounter();
+#endif
 
     // prologue: descriptors of my first two tiles, inputs of the first (its gout maximum first, then the split)
     const int64_t stride = gridDim.x;
     int64_t tile = blockIdx.x;
-    if (threadIdx.x < 64) {
-        const int q = threadIdx.x >> 5;
-        const HTile d = htile_load(cum, order, tile + q * stride, ntiles, Nf, T, threadIdx.x & 31);
-        s_f[q][threadIdx.x & 31] = d.f; s_k0[q][threadIdx.x & 31] = d.k0; s_K[q][threadIdx.x & 31] = d.K;
+    if (w == 0) {
+        const int q = lane >> 5;
+        const int64_t tq = tile + q * stride;
+        const HTile d = htile_finish(htile_totals(cum, htile_facet(order, tq, ntiles, Nf, l32), tq, ntiles, Nf, l32), T);
+        s_f[q][l32] = d.f; s_k0[q][l32] = d.k0; s_K[q][l32] = d.K;
+        const int km = hrow_max(d.K);                   // rows of 16 lanes
+        const int k0m = max(__builtin_amdgcn_readlane(km, 0), __builtin_amdgcn_readlane(km, 16));
+        const int k1m = max(__builtin_amdgcn_readlane(km, 32), __builtin_amdgcn_readlane(km, 48));
+        if (lane == 0) { s_kmax[0] = k0m; s_kmax[1] = k1m; }
+        if (lane < 32) s_fn[0][lane] = htile_facet(order, tile + 2 * stride, ntiles, Nf, lane);
     }
     if (threadIdx.x < 3) s_gm[threadIdx.x] = 0u;
     __syncthreads();
@@ -1477,9 +1646,20 @@ __global__ __launch_bounds__(256, 1) void f2f16h2_bwd_filt_k(const TIO *__restri
     // long facets in several sweeps).  The bound is uniform over the workgroup.
     int it = 0;
 #define PM_PHASE(N)                                                                                                  \
-    for (; tile < ntiles && (N == kHKB || htile_kmax(s_K[it % 3], lane) <= N); ++it, tile += stride)                 \
-        h2_filt_tile<N, TVEC, NCP, HALF, TIO>(gout, tex, sh, cum, order, go_s, slab_s + w * (kHKB * 4 * 32), sh_s, s_f, s_k0, s_K, \
-                                   s_gamma, s_gm, acc, sc, overflow, ea, eb, it, tile, stride, ntiles, Nf, T, Cin, Cout, c0, n0, lane, w)
+    if (tile < ntiles && (N == kHKB || __builtin_amdgcn_readfirstlane(s_kmax[it % 3]) <= N)) {                                        \
+        if constexpr (kPre && N <= kHPre) {                                                                          \
+            /* rows of the phase's first tile; requests of the phase before (same slab, other plane count) land first */ \
+            hwait_vm0();                                                                                             \
+            if (c0 + 2 * NCP * w < Cin)                                                                              \
+                if constexpr (std::is_same<TIO, float>::value)                                                       \
+                    htex_dma<N>(tex, s_k0[it % 3], s_K[it % 3], slab_s + w * kHSlabW + (it & 1) * (N * 128), \
+                                c0 + 2 * NCP * w, Cin, lane);                                                        \
+        }                                                                                                            \
+        for (; tile < ntiles && (N == kHKB || __builtin_amdgcn_readfirstlane(s_kmax[it % 3]) <= N); ++it, tile += stride)             \
+            h2_filt_tile<N, TVEC, NCP, HALF, (kPre && N <= kHPre), TIO>(                                             \
+                gout, tex, sh, cum, order, go_s, slab_s + w * kHSlabW, sh_s, s_f, s_k0, s_K, s_kmax, s_fn, s_gamma, s_gm, acc, sc, \
+                overflow, ea, eb, it, tile, stride, ntiles, Nf, T, Cin, Cout, c0, n0, lane, w);                      \
+    }
     PM_PHASE(1);
     PM_PHASE(2);
     PM_PHASE(3);
@@ -1495,6 +1675,13 @@ __global__ __launch_bounds__(256, 1) void f2f16h2_bwd_filt_k(const TIO *__restri
     // = (channel c0 + 2 NCP w + 2cp + m/16, d = m%16); four consecutive d's per group of four registers
     // accumulator (cp, t): lane (co = 32t + l32, half h), register i <-> row m = 8(i/4) + 4h + i%4
     // = (channel c0 + 2 NCP w + 2cp + m/16, d = m%16); four consecutive d's per group of four registers
+#ifdef PM_TIMING
+    if (blockIdx.x == 7 && lane == 0) {
+        for (int i = 0; i < 6; ++i) pm_filt_dbg[8 * w + i] = sc.tm[i];
+        pm_filt_dbg[8 * w + 6] = __builtin_readcyclecounter() - tstart_;
+        pm_filt_dbg[8 * w + 7] = it;
+    }
+#endif
     const float unscale = sc.S != 0.f ? 1.0f / sc.S : 0.f;
     float *dst = partial + (int64_t)blockIdx.x * Cout * Cin * 16;
 #pragma unroll
@@ -1544,3 +1731,9 @@ int f2f16h2_bwd_filter_partials(const void *gout_, const void *tex_, const float
 }
 
 }  // namespace pmesh
+#ifdef PM_TIMING
+extern "C" int pmesh_dbg_filt_timing(unsigned long long *host)
+{
+    return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(pmesh::pm_filt_dbg), sizeof(unsigned long long) * (32 + 512 * 4 * 8));
+}
+#endif

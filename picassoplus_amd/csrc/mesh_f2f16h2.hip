@@ -197,6 +197,15 @@ __device__ __forceinline__ void cvt8h(const float (&x)[8], u32x4 &p1)
     }
 }
 
+#ifdef PM_TIMING
+#define PM_FTARGS , ftm, ftprev
+__device__ unsigned long long pm_filt_dbg[4 * 8 + 512 * 4 * 8];
+__device__ unsigned long long pm_fwd_dbg[20000 * 12];
+#define PM_FT(i) do { const unsigned long long t_ = __builtin_readcyclecounter(); ftm[i] += t_ - ftprev; ftprev = t_; } while (0)
+#else
+#define PM_FT(i) do { } while (0)
+#define PM_FTARGS
+#endif
 __device__ __forceinline__ f32x16 mfma_f16(const u32x4 &a, const u32x4 &b, const f32x16 &c)
 {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
@@ -352,29 +361,21 @@ __device__ __forceinline__ void hw_chunk_to_lds(const u32x4 *__restrict__ Wp, in
 
 // One pass over all input channels for up to KW texture points per facet.  shs = alpha_f / K_f, the factor on
 // the SH values of my facet; slim / tlim = largest |SH value| of my facet / |texture value| of the rows I fetch
-// that the scale allows for.
-template <int KW, bool TVEC, bool HALF, typename TIO>
+// that the scale allows for.  FIRST (the first sweep of the first try) chooses them itself from what it fetches
+// anyway -- the SH rows of its points and the first eight channels of their texture rows, with 2^7 of head room --
+// and leaves 1 / alpha_f in s_inv; the later sweeps take them from there.  Nothing of that leaves the wavefront.
+template <int KW, bool TVEC, bool HALF, bool FIRST, typename TIO>
 __device__ __forceinline__ void h2_sweep(const TIO *__restrict__ tex, const u32x4 *__restrict__ Wp,
                                          const float *__restrict__ sh, u32x4 *Ws, float *slab, f32x16 (&acc)[2],
-                                         int kbase, int Ks, float shs, float slim, float tlim, bool &viol,
-                                         const int *s_k0, const int *s_K, int sweep, int Cin, int NT, int nt0, int nblk,
-                                         int w, int lane, int h)
+                                         int kbase, int Ks, int K, float &shs, float &slim, float &tlim, bool &viol,
+                                         const int *s_k0, const int *s_K, float *s_tl, float *s_inv, int sweep, int Cin,
+                                         int NT, int nt0, int nblk, int w, int lane, int h
+#ifdef PM_TIMING
+                                         , unsigned long long (&ftm)[12], unsigned long long &ftprev
+#endif
+                                         )
 {
     const int l32 = lane & 31;
-    float shr[KW][8];
-    float smx = 0.f;
-#pragma unroll
-    for (int kk = 0; kk < KW; ++kk) {
-        float4 u = make_float4(0.f, 0.f, 0.f, 0.f), v = u;
-        if (kk < Ks) {
-            const float *p = sh + (int64_t)(kbase + kk) * 16 + 8 * h;
-            u = hld4(p);
-            v = hld4(p + 4);
-        }
-        smx = absmax4(u, absmax4(v, smx));
-        shr[kk][0] = u.x * shs; shr[kk][1] = u.y * shs; shr[kk][2] = u.z * shs; shr[kk][3] = u.w * shs;
-        shr[kk][4] = v.x * shs; shr[kk][5] = v.y * shs; shr[kk][6] = v.z * shs; shr[kk][7] = v.w * shs;
-    }
     // rows this lane fetches for the slab: load i covers point i of facet slot lane/2, channels 4*(lane%2) .. +3 of the group
     const int cg4 = 4 * (lane & 1);
     unsigned ldoff[KW];
@@ -391,8 +392,6 @@ __device__ __forceinline__ void h2_sweep(const TIO *__restrict__ tex, const u32x
         for (int i = 0; i < KW; ++i)
             pf[i] = ldok[i] ? hld4_raw<TVEC>(tex + (ldoff[i] + 8 * g), Cin - (8 * g + cg4)) : hraw_zero(TIO());
     };
-    // values past the limits the facet's scale was chosen for are recorded, not acted on here
-    viol |= smx > slim;
     auto publish_group = [&](float *dst) {
         float m = 0.f;
 #pragma unroll
@@ -404,15 +403,58 @@ __device__ __forceinline__ void h2_sweep(const TIO *__restrict__ tex, const u32x
         }
         viol |= m > tlim;
     };
-    u32x4 wn[kHWn / 2];
     const int wave_u = __builtin_amdgcn_readfirstlane(w);
+    // All requests of the set-up leave before any of them is waited for: the first filter chunk straight into its
+    // buffer (free since the barrier that ended the sweep before), the first texture group and the SH rows through
+    // registers.
+    hw_chunk_to_lds(Wp, 0, NT, nt0, Ws, wave_u);
     fetch_group(0);
+    float4 su[KW], sv[KW];
+#pragma unroll
+    for (int kk = 0; kk < KW; ++kk) {
+        su[kk] = make_float4(0.f, 0.f, 0.f, 0.f);
+        sv[kk] = su[kk];
+        if (kk < Ks) {
+            const float *p = sh + (int64_t)(kbase + kk) * 16 + 8 * h;
+            su[kk] = hld4(p);
+            sv[kk] = hld4(p + 4);
+        }
+    }
+    float smx = 0.f;
+#pragma unroll
+    for (int kk = 0; kk < KW; ++kk) smx = absmax4(su[kk], absmax4(sv[kk], smx));
+    if constexpr (FIRST) {
+        float tm = 0.f;
+#pragma unroll
+        for (int i = 0; i < KW; ++i) tm = absmax4(hcvt4(pf[i]), tm);
+        tm = fmaxf(tm, __builtin_bit_cast(float, hdpp<0xB1>(__builtin_bit_cast(int, tm))));      // the lane pair of a slot
+        float sm = fmaxf(smx, __shfl_xor(smx, 32, 64));                                         // both halves of a facet
+        tm *= 8.0f;
+        sm *= 16.0f;
+        slim = sm;
+        tlim = tm;
+        if (!(lane & 1)) s_tl[w * 32 + (lane >> 1)] = tm;
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        float inv;
+        const float al = pow2_scale(s_tl[w * 32 + l32] * sm, &inv);
+        if (h == 0) s_inv[w * 32 + l32] = inv;
+        shs = K > 0 ? al / (float)K : 0.f;
+    }
+    // values past the limits the facet's scale was chosen for are recorded, not acted on here
+    viol |= smx > slim;
+    float shr[KW][8];
+#pragma unroll
+    for (int kk = 0; kk < KW; ++kk) {
+        shr[kk][0] = su[kk].x * shs; shr[kk][1] = su[kk].y * shs; shr[kk][2] = su[kk].z * shs; shr[kk][3] = su[kk].w * shs;
+        shr[kk][4] = sv[kk].x * shs; shr[kk][5] = sv[kk].y * shs; shr[kk][6] = sv[kk].z * shs; shr[kk][7] = sv[kk].w * shs;
+    }
     publish_group(slab);
-    hw_half_fetch(Wp, 0, 0, NT, nt0, wn);
-    hw_half_publish(Ws, 0, wn);
-    hw_half_fetch(Wp, 0, 1, NT, nt0, wn);
-    hw_half_publish(Ws, 1, wn);
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    PM_FT(2);
     __syncthreads();
+    PM_FT(3);
 
     auto read_b = [&](u32x4 (&b)[2][2], int buf, int cl) { // filter pieces of channel cl of the chunk in buffer buf
         const u32x4 *Wc = Ws + buf * kHChunk + cl * 256 + lane;
@@ -495,9 +537,12 @@ __device__ __forceinline__ void h2_sweep(const TIO *__restrict__ tex, const u32x
                     for (int p = 0; p < 2; ++p) b[t][p] = bn[t][p];
             }
         }
+        PM_FT(4);
         if (wmore) __builtin_amdgcn_s_waitcnt(0x0F70);      // vmcnt(0): the next chunk has landed in its buffer
         if (stage) publish_group(slab + ((g + 1) & 1) * kHSlab);
+        PM_FT(5);
         __syncthreads();
+        PM_FT(6);
         if (wmore) read_b(b, wb ^ 1, 0);
     }
 }
@@ -511,16 +556,22 @@ __global__ __launch_bounds__(kHThreads, 2) void f2f16h2_fwd_k(const TIO *__restr
 {
     __shared__ u32x4 Ws[2 * kHChunk];
     __shared__ __attribute__((aligned(16))) float s_slab[kHW * 2 * kHSlab];      // per wavefront: two buffers
-    __shared__ int s_f[kHFacets], s_k0[kHFacets], s_K[kHFacets], s_kmax;
-    __shared__ float s_tm[kHFacets], s_inv[kHFacets], s_tl[kHFacets];
+    __shared__ int s_f[kHFacets], s_k0[kHFacets], s_K[kHFacets], s_kmax[kHFacets / 64];
+    __shared__ float s_inv[kHFacets], s_tl[kHFacets];
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
     const int l32 = lane & 31, h = lane >> 5;
     const int64_t s0 = (int64_t)blockIdx.x * kHFacets;
     const int nt0 = blockIdx.y * 2, n0 = blockIdx.y * 64;
     const int nblk = (Cin + 3) >> 2;
+    const float ibeta = hdr[1];                      // (needed by the stores at the end: asked for here, not there)
+#ifdef PM_TIMING
+    unsigned long long ftm[12] = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0}, ftprev = __builtin_readcyclecounter();
+    const unsigned long long ftstart = ftprev;
+#endif
 
-    if (threadIdx.x == 0) s_kmax = 0;
-    for (int i = threadIdx.x; i < kHFacets; i += kHThreads) {
+    static_assert(kHFacets <= kHThreads && kHFacets % 64 == 0, "one descriptor per thread of the first wavefronts");
+    if (threadIdx.x < kHFacets) {
+        const int i = threadIdx.x;
         const int64_t slot = s0 + i;
         const int f = slot < Nf ? (order ? order[slot] : (int)slot) : -1;
         int a = 0, b = 0;
@@ -533,28 +584,30 @@ __global__ __launch_bounds__(kHThreads, 2) void f2f16h2_fwd_k(const TIO *__restr
         s_f[i] = f;
         s_k0[i] = a;
         s_K[i] = b > a ? b - a : 0;
+        const int km = hwave_max(b > a ? b - a : 0);            // (whole wavefronts are in here)
+        if (lane == 0) s_kmax[w] = km;
     }
     __syncthreads();
+    PM_FT(0);
     const int k0 = s_k0[w * 32 + l32], K = s_K[w * 32 + l32];
-    {
-        const int km = hwave_max(K);
-        if (lane == 0) atomicMax(&s_kmax, km);
-    }
+    int kmax_wg = 0;
+#pragma unroll
+    for (int i = 0; i < kHFacets / 64; ++i) kmax_wg = max(kmax_wg, s_kmax[i]);
 
-    // Scale of each facet's G.  First try: a bound from the first eight channels and the first four points only
-    // (one batch of loads that the sweep reads again from cache), with 2^7 of head room; the sweeps check every
+    // Scale of each facet's G.  First try: a bound from the first eight channels of the points of the first sweep
+    // (which that sweep works out itself from its first fetches), with 2^7 of head room; the sweeps check every
     // value they fetch against it.  If any facet of the workgroup exceeds its bound, everything is done again
     // with the exact maxima from a scan of all rows (which costs a second pass over the texture rows).
     f32x16 acc[2];
     for (int attempt = 0;; ++attempt) {
         const bool full = attempt > 0;
-        float slim;
-        {
+        float slim = 0.f, tlim = 0.f, shs = 0.f;
+        if (full) {
             const int slot = w * 32 + (lane >> 1), cg4 = 4 * (lane & 1);
             const int rk0 = s_k0[slot], rK = s_K[slot];
             // all loads of a batch are issued before the first comparison
-            const int rKmax = full ? hwave_max(rK) : 1, Kmax = full ? hwave_max(K) : 1, cend = full ? Cin : 1;
-            float sm = 0.f;
+            const int rKmax = hwave_max(rK), Kmax = hwave_max(K);
+            float sm = 0.f, tm = 0.f;
             for (int kb = 0; kb < Kmax; kb += 4) {
                 float4 u[4][2];
 #pragma unroll
@@ -567,18 +620,16 @@ __global__ __launch_bounds__(kHThreads, 2) void f2f16h2_fwd_k(const TIO *__restr
 #pragma unroll
                 for (int i = 0; i < 4; ++i) sm = absmax4(u[i][0], absmax4(u[i][1], sm));
             }
-            float tm = 0.f;
             for (int kb = 0; kb < rKmax; kb += 4)
-                for (int cb = 0; cb < cend; cb += 32) {
+                for (int cb = 0; cb < Cin; cb += 32) {
                     HRaw4<TIO> v[4][4];
 #pragma unroll
                     for (int i = 0; i < 4; ++i)
 #pragma unroll
                         for (int g = 0; g < 4; ++g) {
                             const int c = cb + 8 * g + cg4;
-                            v[i][g] = (kb + i < rK && c < Cin && (full || g == 0))
-                                          ? hld4_raw<TVEC>(tex + (int64_t)(rk0 + kb + i) * Cin + c, Cin - c)
-                                          : hraw_zero(TIO());
+                            v[i][g] = (kb + i < rK && c < Cin) ? hld4_raw<TVEC>(tex + (int64_t)(rk0 + kb + i) * Cin + c, Cin - c)
+                                                              : hraw_zero(TIO());
                         }
 #pragma unroll
                     for (int i = 0; i < 4; ++i)
@@ -587,20 +638,19 @@ __global__ __launch_bounds__(kHThreads, 2) void f2f16h2_fwd_k(const TIO *__restr
                 }
             tm = fmaxf(tm, __shfl_xor(tm, 1, 64));
             sm = fmaxf(sm, __shfl_xor(sm, 32, 64));
-            if (!full) { tm *= 8.0f; sm *= 16.0f; }          // head room of the first try (2^7 in all)
             slim = sm;
+            tlim = tm;
             if (!(lane & 1)) s_tl[slot] = tm;
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
             __builtin_amdgcn_wave_barrier();
             __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
             float inv;
             const float al = pow2_scale(s_tl[w * 32 + l32] * sm, &inv);
-            if (h == 0) { s_inv[w * 32 + l32] = inv; s_tm[w * 32 + l32] = al; }
+            if (h == 0) s_inv[w * 32 + l32] = inv;
+            shs = K > 0 ? al / (float)K : 0.f;
         }
-        __syncthreads();
-        const float alpha = s_tm[w * 32 + l32], tlim = s_tl[w * 32 + (lane >> 1)];
-        const int nsweeps = (s_kmax + kHFKB - 1) / kHFKB;
-        const float shs = K > 0 ? alpha / (float)K : 0.f;
+        PM_FT(1);
+        const int nsweeps = (kmax_wg + kHFKB - 1) / kHFKB;
 #pragma unroll
         for (int t = 0; t < 2; ++t)
 #pragma unroll
@@ -612,18 +662,27 @@ __global__ __launch_bounds__(kHThreads, 2) void f2f16h2_fwd_k(const TIO *__restr
             const int Ks = rem < 0 ? 0 : (rem > kHFKB ? kHFKB : rem);
             // every variant runs the same barriers, so wavefronts of a workgroup may pick different ones
             const int kw = hwave_max(Ks);
-#define PM_H2(N) h2_sweep<N, TVEC, HALF, TIO>(tex, Wp, sh, Ws, s_slab + w * 2 * kHSlab, acc, kbase, Ks, shs, slim, tlim, viol, s_k0, s_K, sw, Cin, NT, nt0, nblk, w, lane, h)
-            if (kw <= 1) PM_H2(1);
-            else if (kw == 2) PM_H2(2);
-            else if (kw == 3) PM_H2(3);
-            else if (kw == 4) PM_H2(4);
-            else PM_H2(5);
+#define PM_H2(N, FIRST) h2_sweep<N, TVEC, HALF, FIRST, TIO>(tex, Wp, sh, Ws, s_slab + w * 2 * kHSlab, acc, kbase, Ks, K, shs, slim, tlim, viol, s_k0, s_K, s_tl, s_inv, sw, Cin, NT, nt0, nblk, w, lane, h PM_FTARGS)
+            if (!full && sw == 0) {
+                if (kw <= 1) PM_H2(1, true);
+                else if (kw == 2) PM_H2(2, true);
+                else if (kw == 3) PM_H2(3, true);
+                else if (kw == 4) PM_H2(4, true);
+                else PM_H2(5, true);
+            } else {
+                if (kw <= 1) PM_H2(1, false);
+                else if (kw == 2) PM_H2(2, false);
+                else if (kw == 3) PM_H2(3, false);
+                else if (kw == 4) PM_H2(4, false);
+                else PM_H2(5, false);
+            }
 #undef PM_H2
         }
+        PM_FT(1);
         if (full || !__syncthreads_or(viol ? 1 : 0)) break;
     }
+    PM_FT(3);
 
-    const float ibeta = hdr[1];
     // what rides on the store: bias, ReLU (and its mask as bits), a per-channel scale and shift
     float tb[2], tsc[2], tsf[2];
 #pragma unroll
@@ -635,12 +694,46 @@ __global__ __launch_bounds__(kHThreads, 2) void f2f16h2_fwd_k(const TIO *__restr
         tsf[t] = (tail.shift && cok) ? tail.shift[co] : 0.f;
     }
     const bool plain = !tail.bias && !tail.scale && !tail.shift && !tail.relu;
+    PM_FT(8);
+    // facets and scales of my 16 rows (four runs of four slots), read before the first store goes out
+    int frow[16];
+    float urow[16];
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
         const int slot = w * 32 + 8 * (i / 4) + 4 * h + (i % 4);
-        const int fr = s_f[slot];
+        frow[i] = s_f[slot];
+        urow[i] = s_inv[slot];
+    }
+    PM_FT(9);
+    // the common case without any condition on a store: float rows, nothing riding on them, all of the wavefront's
+    // rows and columns present
+    if constexpr (std::is_same<TIO, float>::value) {
+        bool mine = true;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) mine = mine && frow[i] >= 0 && frow[i] < Nf;
+        if (plain && n0 + 64 <= Cout && __builtin_amdgcn_ballot_w64(mine) == ~0ull) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                float *rowp = out + ((int64_t)frow[i] * Cout + n0 + l32);
+                const float us = urow[i] * ibeta;
+                rowp[0] = acc[0][i] * us;
+                rowp[32] = acc[1][i] * us;
+            }
+            PM_FT(10);
+            PM_FT(7);
+#ifdef PM_TIMING
+            if (lane == 0 && w == 0 && blockIdx.y == 0 && blockIdx.x < 20000)
+                for (int i = 0; i < 12; ++i) pm_fwd_dbg[12 * blockIdx.x + i] = ftm[i];
+#endif
+            return;
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        if (i == 8) PM_FT(10);
+        const int fr = frow[i];
         const bool rok = fr >= 0 && fr < Nf;
-        const float us = s_inv[slot] * ibeta;
+        const float us = urow[i] * ibeta;
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
             const int co = n0 + t * 32 + l32;
@@ -655,9 +748,21 @@ __global__ __launch_bounds__(kHThreads, 2) void f2f16h2_fwd_k(const TIO *__restr
                 }
                 v = v * tsc[t] + tsf[t];
             }
+#if defined(PM_EPI) && PM_EPI == 1
+            hst1_pair(out + ((int64_t)(rok ? s0 + w * 32 + 8 * (i / 4) + 4 * h + (i % 4) : 0) * Cout + co), v, rok && co < Cout, l32);
+#elif defined(PM_EPI) && PM_EPI == 2
+            hst1_pair(out + ((int64_t)(rok ? fr : 0) * Cout + co), v, rok && co < Cout && v == 123.456f, l32);
+#else
             hst1_pair(out + ((int64_t)(rok ? fr : 0) * Cout + co), v, rok && co < Cout, l32);
+#endif
         }
     }
+#ifdef PM_TIMING
+    PM_FT(7);
+    if (lane == 0 && w == 0 && blockIdx.y == 0 && blockIdx.x < 20000) {
+        for (int i = 0; i < 12; ++i) pm_fwd_dbg[12 * blockIdx.x + i] = ftm[i];
+    }
+#endif
 }
 
 // workspace: 16-byte header {beta, 1/beta, -, -}, then the packed filter
@@ -1397,7 +1502,6 @@ struct HScales {
 #endif
 };
 #ifdef PM_TIMING
-__device__ unsigned long long pm_filt_dbg[4 * 8 + 512 * 4 * 8];
 #define PM_T(i) do { const unsigned long long t_ = __builtin_readcyclecounter(); sc.tm[i] += t_ - tprev_; if (blockIdx.x == 7 && lane == 0 && it < 512) pm_filt_dbg[32 + (it * 4 + w) * 8 + i] = t_ - tprev_; tprev_ = t_; } while (0)
 #else
 #define PM_T(i) do { } while (0)
@@ -1735,5 +1839,9 @@ int f2f16h2_bwd_filter_partials(const void *gout_, const void *tex_, const float
 extern "C" int pmesh_dbg_filt_timing(unsigned long long *host)
 {
     return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(pmesh::pm_filt_dbg), sizeof(unsigned long long) * (32 + 512 * 4 * 8));
+}
+extern "C" int pmesh_dbg_fwd_timing(unsigned long long *host)
+{
+    return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(pmesh::pm_fwd_dbg), sizeof(unsigned long long) * 20000 * 12);
 }
 #endif

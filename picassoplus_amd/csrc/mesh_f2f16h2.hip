@@ -201,6 +201,7 @@ __device__ __forceinline__ void cvt8h(const float (&x)[8], u32x4 &p1)
 #define PM_FTARGS , ftm, ftprev
 __device__ unsigned long long pm_filt_dbg[4 * 8 + 512 * 4 * 8];
 __device__ unsigned long long pm_fwd_dbg[20000 * 12];
+__device__ unsigned long long pm_tex_dbg[20000 * 12];
 #define PM_FT(i) do { const unsigned long long t_ = __builtin_readcyclecounter(); ftm[i] += t_ - ftprev; ftprev = t_; } while (0)
 #else
 #define PM_FT(i) do { } while (0)
@@ -845,26 +846,19 @@ __global__ __launch_bounds__(kBlock) void f2f16h2_pack_filter_t_k(const float *_
     dst[0] = p1; dst[64] = p2;
 }
 
-template <int KW, int NKS, bool GVEC, bool HALF, typename TIO>
+// FIRST (the first sweep) also turns the facet's gout row x, which the kernel has asked for, into the operand
+// pieces bp and the factor shs -- after its own requests have left, so that the two round trips overlap.
+template <int KW, int NKS, bool GVEC, bool HALF, bool FIRST, typename TIO>
 __device__ __forceinline__ void h2_tex_sweep(const u32x4 *__restrict__ WpT, const float *__restrict__ sh,
                                              TIO *__restrict__ gtex, u32x4 *Ws, float *stage, const int *w_k0,
-                                             const int *w_K, const u32x4 (&bp)[NKS][2], int kbase, int Ks, float shs,
-                                             int sweep, int Cin, int NG, bool add, int lane, int h)
+                                             const int *w_K, float (*x)[8], u32x4 (&bp)[NKS][2], int kbase, int Ks,
+                                             int K, float ibeta, float &shs, int sweep, int Cin, int NG, bool add, int lane,
+                                             int h
+#ifdef PM_TIMING
+                                             , unsigned long long (&ftm)[12], unsigned long long &ftprev
+#endif
+                                             )
 {
-    // SH values of my facet's points for my half's eight d's (4h..4h+3, 8+4h..8+4h+3), times shs = 1 / (K gamma beta):
-    // the scales of the two operands leave with the contraction
-    float shr[KW][8];
-#pragma unroll
-    for (int kk = 0; kk < KW; ++kk) {
-        float4 u = make_float4(0.f, 0.f, 0.f, 0.f), v = u;
-        if (kk < Ks) {
-            const float *p = sh + (int64_t)(kbase + kk) * 16 + 4 * h;
-            u = hld4(p);
-            v = hld4(p + 8);
-        }
-        shr[kk][0] = u.x * shs; shr[kk][1] = u.y * shs; shr[kk][2] = u.z * shs; shr[kk][3] = u.w * shs;
-        shr[kk][4] = v.x * shs; shr[kk][5] = v.y * shs; shr[kk][6] = v.z * shs; shr[kk][7] = v.w * shs;
-    }
     constexpr int chunk = 2 * NKS * 128;         // uint4 per chunk of two tiles
     constexpr int NWF = (chunk + 511) / 512;     // uint4 fetched per thread
     const int nchunks = 2 * NG;
@@ -882,12 +876,56 @@ __device__ __forceinline__ void h2_tex_sweep(const u32x4 *__restrict__ WpT, cons
             if (e < chunk) Ws[(c % 3) * kHTChunkMax + e] = wn[i];
         }
     };
-    u32x4 wn[NWF];
+    // All requests of the set-up leave before any of them is waited for: the first two filter chunks and the SH rows.
+    u32x4 wn[NWF], wn1[NWF];
     chunk_fetch(wn, 0);
+    chunk_fetch(wn1, 1);
+    // SH values of my facet's points for my half's eight d's (4h..4h+3, 8+4h..8+4h+3), times shs = 1 / (K gamma beta):
+    // the scales of the two operands leave with the contraction
+    float4 su[KW], sv[KW];
+#pragma unroll
+    for (int kk = 0; kk < KW; ++kk) {
+        su[kk] = make_float4(0.f, 0.f, 0.f, 0.f);
+        sv[kk] = su[kk];
+        if (kk < Ks) {
+            const float *p = sh + (int64_t)(kbase + kk) * 16 + 4 * h;
+            su[kk] = hld4(p);
+            sv[kk] = hld4(p + 8);
+        }
+    }
+    if constexpr (FIRST) {
+        // my facet's gout row, scaled by gamma_f = a power of two that brings its largest element below 2^14, as B
+        // operand pieces: k-step ks, half h <-> channels 16ks + 8h .. + 7
+        float gm = 0.f;
+#pragma unroll
+        for (int ks = 0; ks < NKS; ++ks)
+#pragma unroll
+            for (int j = 0; j < 8; ++j) gm = fmaxf(gm, fabsf(x[ks][j]));
+        gm = fmaxf(gm, __shfl_xor(gm, 32, 64));
+        float igamma;
+        const float gamma = pow2_scale(gm, &igamma);
+#pragma unroll
+        for (int ks = 0; ks < NKS; ++ks) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) x[ks][j] *= gamma;
+            float xs[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) xs[j] = x[ks][j];
+            split8h(xs, bp[ks][0], bp[ks][1]);
+        }
+        shs = K > 0 ? igamma * ibeta / (float)K : 0.f;
+    }
+    float shr[KW][8];
+#pragma unroll
+    for (int kk = 0; kk < KW; ++kk) {
+        shr[kk][0] = su[kk].x * shs; shr[kk][1] = su[kk].y * shs; shr[kk][2] = su[kk].z * shs; shr[kk][3] = su[kk].w * shs;
+        shr[kk][4] = sv[kk].x * shs; shr[kk][5] = sv[kk].y * shs; shr[kk][6] = sv[kk].z * shs; shr[kk][7] = sv[kk].w * shs;
+    }
     chunk_publish(wn, 0);
-    chunk_fetch(wn, 1);
-    chunk_publish(wn, 1);
+    chunk_publish(wn1, 1);
+    PM_FT(1);
     __syncthreads();
+    PM_FT(2);
 
     // 16-channel block gp of the stage -> global memory
     auto flush = [&](int gp) {
@@ -986,19 +1024,23 @@ __device__ __forceinline__ void h2_tex_sweep(const u32x4 *__restrict__ WpT, cons
                 if (cc == 0 && u == 0 && g > 0) finish_group(g - 1);
                 accp = acc0;
             }
+            PM_FT(3);
             if (more) chunk_publish(wn, c + 2);
+            PM_FT(4);
             __syncthreads();
+            PM_FT(5);
         }
     }
     contract(3);
     finish_group(NG - 1);
+    PM_FT(6);
 }
 
 // NKS = k-steps of 16 output channels (compile time, so that a tile's MFMAs and the previous tile's
 // contraction share one basic block and get interleaved): 2 for Cout <= 32, else 4; the packed filter
 // is zero padded to that many.
 template <int NKS, bool GVEC, bool HALF, typename TIN, typename TIO>
-__global__ __launch_bounds__(512, 2) void f2f16h2_bwd_tex_k(const TIN *__restrict__ gout,
+__global__ __launch_bounds__(512, 1) void f2f16h2_bwd_tex_k(const TIN *__restrict__ gout,
                                                             const float *__restrict__ hdr,
                                                             const u32x4 *__restrict__ WpT,
                                                             const float *__restrict__ sh,
@@ -1008,11 +1050,13 @@ __global__ __launch_bounds__(512, 2) void f2f16h2_bwd_tex_k(const TIN *__restric
 {
     __shared__ u32x4 Ws[3 * kHTChunkMax];
     __shared__ __attribute__((aligned(16))) float s_stage[8][kHTKB * 32 * 16];
-    __shared__ int s_k0[8][32], s_K[8][32], s_kmax;
+    __shared__ int s_k0[8][32], s_K[8][32], s_kmax[8];
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
     const int l32 = lane & 31, h = lane >> 5;
-    if (threadIdx.x == 0) s_kmax = 0;
-    __syncthreads();
+#ifdef PM_TIMING
+    unsigned long long ftm[12] = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0}, ftprev = __builtin_readcyclecounter();
+#endif
+    const float ibeta = hdr[1];                      // (used after the first fetches have come back)
 
     const int64_t slot = (int64_t)blockIdx.x * 256 + w * 32 + l32;
     const int f = slot < Nf ? (order ? order[slot] : (int)slot) : -1;
@@ -1030,12 +1074,10 @@ __global__ __launch_bounds__(512, 2) void f2f16h2_bwd_tex_k(const TIN *__restric
     }
     {
         const int km = hwave_max(K);
-        if (lane == 0) atomicMax(&s_kmax, km);
+        if (lane == 0) s_kmax[w] = km;
     }
-    // my facet's gout row (the 16 NKS channels of this launch), scaled by gamma_f = a power of two that brings
-    // its largest element below 2^14, as B operand pieces: k-step ks, half h <-> channels 16ks + 8h .. + 7
+    // my facet's gout row (the 16 NKS channels of this launch): asked for here, used by the first sweep
     float x[NKS][8];
-    float gm = 0.f;
 #pragma unroll
     for (int ks = 0; ks < NKS; ++ks) {
 #pragma unroll
@@ -1046,37 +1088,48 @@ __global__ __launch_bounds__(512, 2) void f2f16h2_bwd_tex_k(const TIN *__restric
             hld8(gout + ((int64_t)f * Cout + co), u, v);
             x[ks][0] = u.x; x[ks][1] = u.y; x[ks][2] = u.z; x[ks][3] = u.w;
             x[ks][4] = v.x; x[ks][5] = v.y; x[ks][6] = v.z; x[ks][7] = v.w;
-            gm = absmax4(u, absmax4(v, gm));
         }
     }
-    gm = fmaxf(gm, __shfl_xor(gm, 32, 64));
-    float igamma;
-    const float gamma = pow2_scale(gm, &igamma);
     u32x4 bp[NKS][2];
-#pragma unroll
-    for (int ks = 0; ks < NKS; ++ks) {
-#pragma unroll
-        for (int j = 0; j < 8; ++j) x[ks][j] *= gamma;
-        split8h(x[ks], bp[ks][0], bp[ks][1]);
+    float shs = 0.f;
+    PM_FT(0);
+    // The first sweep starts without a barrier in front (which would wait for the gout rows): every workgroup runs
+    // it, and the barrier of its set-up is the one that makes the wavefronts' point counts visible to all.
+#define PM_H2T(N, FIRST, X) h2_tex_sweep<N, NKS, GVEC, HALF, FIRST, TIO>(WpT, sh, gtex, Ws, s_stage[w], s_k0[w], s_K[w], X, bp, kbase, Ks, K, ibeta, shs, sw, Cin, NG, co0 > 0, lane, h PM_FTARGS)
+    {
+        const int sw = 0, kbase = k0;
+        const int Ks = K > kHTKB ? kHTKB : K;
+        const int kw = hwave_max(Ks);
+        // every variant runs the same barriers, so wavefronts of a workgroup may pick different ones
+        if (kw <= 1) PM_H2T(1, true, x);
+        else if (kw == 2) PM_H2T(2, true, x);
+        else if (kw == 3) PM_H2T(3, true, x);
+        else if (kw == 4) PM_H2T(4, true, x);
+        else if (kw == 5) PM_H2T(5, true, x);
+        else PM_H2T(6, true, x);
     }
-    const float shs = K > 0 ? igamma * hdr[1] / (float)K : 0.f;
-    __syncthreads();
-    const int nsweeps = (s_kmax + kHTKB - 1) / kHTKB;
-    for (int sw = 0; sw < nsweeps; ++sw) {
+    int kmax_wg = 0;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) kmax_wg = max(kmax_wg, s_kmax[i]);
+    const int nsweeps = (kmax_wg + kHTKB - 1) / kHTKB;
+    for (int sw = 1; sw < nsweeps; ++sw) {
         const int rem = K - sw * kHTKB;
         const int Ks = rem < 0 ? 0 : (rem > kHTKB ? kHTKB : rem);
         const int kw = hwave_max(Ks);
         const int kbase = k0 + sw * kHTKB;
-        // every variant runs the same barriers, so wavefronts of a workgroup may pick different ones
-#define PM_H2T(N) h2_tex_sweep<N, NKS, GVEC, HALF, TIO>(WpT, sh, gtex, Ws, s_stage[w], s_k0[w], s_K[w], bp, kbase, Ks, shs, sw, Cin, NG, co0 > 0, lane, h)
-        if (kw <= 1) PM_H2T(1);
-        else if (kw == 2) PM_H2T(2);
-        else if (kw == 3) PM_H2T(3);
-        else if (kw == 4) PM_H2T(4);
-        else if (kw == 5) PM_H2T(5);
-        else PM_H2T(6);
-#undef PM_H2T
+        float (*none)[8] = nullptr;
+        if (kw <= 1) PM_H2T(1, false, none);
+        else if (kw == 2) PM_H2T(2, false, none);
+        else if (kw == 3) PM_H2T(3, false, none);
+        else if (kw == 4) PM_H2T(4, false, none);
+        else if (kw == 5) PM_H2T(5, false, none);
+        else PM_H2T(6, false, none);
     }
+#undef PM_H2T
+#ifdef PM_TIMING
+    if (lane == 0 && w == 0 && blockIdx.x < 20000)
+        for (int i = 0; i < 12; ++i) pm_tex_dbg[12 * blockIdx.x + i] = ftm[i];
+#endif
 }
 
 
@@ -1839,6 +1892,10 @@ int f2f16h2_bwd_filter_partials(const void *gout_, const void *tex_, const float
 extern "C" int pmesh_dbg_filt_timing(unsigned long long *host)
 {
     return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(pmesh::pm_filt_dbg), sizeof(unsigned long long) * (32 + 512 * 4 * 8));
+}
+extern "C" int pmesh_dbg_tex_timing(unsigned long long *host)
+{
+    return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(pmesh::pm_tex_dbg), sizeof(unsigned long long) * 20000 * 12);
 }
 extern "C" int pmesh_dbg_fwd_timing(unsigned long long *host)
 {

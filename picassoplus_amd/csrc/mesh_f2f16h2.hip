@@ -197,16 +197,6 @@ __device__ __forceinline__ void cvt8h(const float (&x)[8], u32x4 &p1)
     }
 }
 
-#ifdef PM_TIMING
-#define PM_FTARGS , ftm, ftprev
-__device__ unsigned long long pm_filt_dbg[4 * 8 + 512 * 4 * 8];
-__device__ unsigned long long pm_fwd_dbg[20000 * 12];
-__device__ unsigned long long pm_tex_dbg[20000 * 12];
-#define PM_FT(i) do { const unsigned long long t_ = __builtin_readcyclecounter(); ftm[i] += t_ - ftprev; ftprev = t_; } while (0)
-#else
-#define PM_FT(i) do { } while (0)
-#define PM_FTARGS
-#endif
 __device__ __forceinline__ f32x16 mfma_f16(const u32x4 &a, const u32x4 &b, const f32x16 &c)
 {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
@@ -329,25 +319,9 @@ __global__ __launch_bounds__(kBlock) void f2f16h2_pack_filter_k(const float *__r
     dst[0] = p1; dst[64] = p2;
 }
 
-// A chunk (four channels) moves in two halves of two channels, so that only kHWn / 2 registers per thread wait
-// between a fetch and its publication.  Channel c of the chunk: 2 tiles x 2 pieces x 64 lanes = 256 consecutive uint4.
-__device__ __forceinline__ void hw_half_fetch(const u32x4 *__restrict__ Wp, int c0, int half, int NT, int nt0,
-                                              u32x4 (&wn)[kHWn / 2])
-{
-#pragma unroll
-    for (int i = 0; i < kHWn / 2; ++i) {
-        const int e = 512 * half + threadIdx.x + kHThreads * i, c = e >> 8, o = e & 255;
-        wn[i] = Wp[((size_t)(c0 + c) * NT + nt0) * 128 + o];
-    }
-}
-__device__ __forceinline__ void hw_half_publish(u32x4 *Wbuf, int half, const u32x4 (&wn)[kHWn / 2])
-{
-#pragma unroll
-    for (int i = 0; i < kHWn / 2; ++i) Wbuf[512 * half + threadIdx.x + kHThreads * i] = wn[i];
-}
-
-// The same chunk straight from global memory into an LDS buffer (no registers in between, so the request can leave
-// a whole chunk ahead): lane L of wavefront w delivers element 256 i + 64 w + L of the chunk, the wavefront's 64
+// A filter chunk (four channels; channel c of the chunk = 2 tiles x 2 pieces x 64 lanes = 256 consecutive uint4)
+// straight from global memory into an LDS buffer (no registers in between, so the request can leave a whole chunk
+// ahead): lane L of wavefront w delivers element 256 i + 64 w + L of the chunk, the wavefront's 64
 // elements land side by side from the wavefront-uniform base in M0.  The data is there after vmcnt has drained.
 __device__ __forceinline__ void hw_chunk_to_lds(const u32x4 *__restrict__ Wp, int c0, int NT, int nt0, u32x4 *Wbuf, int wave)
 {
@@ -371,9 +345,6 @@ __device__ __forceinline__ void h2_sweep(const TIO *__restrict__ tex, const u32x
                                          int kbase, int Ks, int K, float &shs, float &slim, float &tlim, bool &viol,
                                          const int *s_k0, const int *s_K, float *s_tl, float *s_inv, int sweep, int Cin,
                                          int NT, int nt0, int nblk, int w, int lane, int h
-#ifdef PM_TIMING
-                                         , unsigned long long (&ftm)[12], unsigned long long &ftprev
-#endif
                                          )
 {
     const int l32 = lane & 31;
@@ -453,9 +424,7 @@ __device__ __forceinline__ void h2_sweep(const TIO *__restrict__ tex, const u32x
     }
     publish_group(slab);
     __builtin_amdgcn_s_waitcnt(0x0F70);
-    PM_FT(2);
     __syncthreads();
-    PM_FT(3);
 
     auto read_b = [&](u32x4 (&b)[2][2], int buf, int cl) { // filter pieces of channel cl of the chunk in buffer buf
         const u32x4 *Wc = Ws + buf * kHChunk + cl * 256 + lane;
@@ -538,12 +507,9 @@ __device__ __forceinline__ void h2_sweep(const TIO *__restrict__ tex, const u32x
                     for (int p = 0; p < 2; ++p) b[t][p] = bn[t][p];
             }
         }
-        PM_FT(4);
         if (wmore) __builtin_amdgcn_s_waitcnt(0x0F70);      // vmcnt(0): the next chunk has landed in its buffer
         if (stage) publish_group(slab + ((g + 1) & 1) * kHSlab);
-        PM_FT(5);
         __syncthreads();
-        PM_FT(6);
         if (wmore) read_b(b, wb ^ 1, 0);
     }
 }
@@ -565,10 +531,6 @@ __global__ __launch_bounds__(kHThreads, 2) void f2f16h2_fwd_k(const TIO *__restr
     const int nt0 = blockIdx.y * 2, n0 = blockIdx.y * 64;
     const int nblk = (Cin + 3) >> 2;
     const float ibeta = hdr[1];                      // (needed by the stores at the end: asked for here, not there)
-#ifdef PM_TIMING
-    unsigned long long ftm[12] = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0}, ftprev = __builtin_readcyclecounter();
-    const unsigned long long ftstart = ftprev;
-#endif
 
     static_assert(kHFacets <= kHThreads && kHFacets % 64 == 0, "one descriptor per thread of the first wavefronts");
     if (threadIdx.x < kHFacets) {
@@ -589,7 +551,6 @@ __global__ __launch_bounds__(kHThreads, 2) void f2f16h2_fwd_k(const TIO *__restr
         if (lane == 0) s_kmax[w] = km;
     }
     __syncthreads();
-    PM_FT(0);
     const int k0 = s_k0[w * 32 + l32], K = s_K[w * 32 + l32];
     int kmax_wg = 0;
 #pragma unroll
@@ -650,7 +611,6 @@ __global__ __launch_bounds__(kHThreads, 2) void f2f16h2_fwd_k(const TIO *__restr
             if (h == 0) s_inv[w * 32 + l32] = inv;
             shs = K > 0 ? al / (float)K : 0.f;
         }
-        PM_FT(1);
         const int nsweeps = (kmax_wg + kHFKB - 1) / kHFKB;
 #pragma unroll
         for (int t = 0; t < 2; ++t)
@@ -663,7 +623,7 @@ __global__ __launch_bounds__(kHThreads, 2) void f2f16h2_fwd_k(const TIO *__restr
             const int Ks = rem < 0 ? 0 : (rem > kHFKB ? kHFKB : rem);
             // every variant runs the same barriers, so wavefronts of a workgroup may pick different ones
             const int kw = hwave_max(Ks);
-#define PM_H2(N, FIRST) h2_sweep<N, TVEC, HALF, FIRST, TIO>(tex, Wp, sh, Ws, s_slab + w * 2 * kHSlab, acc, kbase, Ks, K, shs, slim, tlim, viol, s_k0, s_K, s_tl, s_inv, sw, Cin, NT, nt0, nblk, w, lane, h PM_FTARGS)
+#define PM_H2(N, FIRST) h2_sweep<N, TVEC, HALF, FIRST, TIO>(tex, Wp, sh, Ws, s_slab + w * 2 * kHSlab, acc, kbase, Ks, K, shs, slim, tlim, viol, s_k0, s_K, s_tl, s_inv, sw, Cin, NT, nt0, nblk, w, lane, h)
             if (!full && sw == 0) {
                 if (kw <= 1) PM_H2(1, true);
                 else if (kw == 2) PM_H2(2, true);
@@ -679,10 +639,8 @@ __global__ __launch_bounds__(kHThreads, 2) void f2f16h2_fwd_k(const TIO *__restr
             }
 #undef PM_H2
         }
-        PM_FT(1);
         if (full || !__syncthreads_or(viol ? 1 : 0)) break;
     }
-    PM_FT(3);
 
     // what rides on the store: bias, ReLU (and its mask as bits), a per-channel scale and shift
     float tb[2], tsc[2], tsf[2];
@@ -695,7 +653,6 @@ __global__ __launch_bounds__(kHThreads, 2) void f2f16h2_fwd_k(const TIO *__restr
         tsf[t] = (tail.shift && cok) ? tail.shift[co] : 0.f;
     }
     const bool plain = !tail.bias && !tail.scale && !tail.shift && !tail.relu;
-    PM_FT(8);
     // facets and scales of my 16 rows (four runs of four slots), read before the first store goes out
     int frow[16];
     float urow[16];
@@ -705,7 +662,6 @@ __global__ __launch_bounds__(kHThreads, 2) void f2f16h2_fwd_k(const TIO *__restr
         frow[i] = s_f[slot];
         urow[i] = s_inv[slot];
     }
-    PM_FT(9);
     // the common case without any condition on a store: float rows, nothing riding on them, all of the wavefront's
     // rows and columns present
     if constexpr (std::is_same<TIO, float>::value) {
@@ -720,18 +676,11 @@ __global__ __launch_bounds__(kHThreads, 2) void f2f16h2_fwd_k(const TIO *__restr
                 rowp[0] = acc[0][i] * us;
                 rowp[32] = acc[1][i] * us;
             }
-            PM_FT(10);
-            PM_FT(7);
-#ifdef PM_TIMING
-            if (lane == 0 && w == 0 && blockIdx.y == 0 && blockIdx.x < 20000)
-                for (int i = 0; i < 12; ++i) pm_fwd_dbg[12 * blockIdx.x + i] = ftm[i];
-#endif
             return;
         }
     }
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
-        if (i == 8) PM_FT(10);
         const int fr = frow[i];
         const bool rok = fr >= 0 && fr < Nf;
         const float us = urow[i] * ibeta;
@@ -749,21 +698,9 @@ __global__ __launch_bounds__(kHThreads, 2) void f2f16h2_fwd_k(const TIO *__restr
                 }
                 v = v * tsc[t] + tsf[t];
             }
-#if defined(PM_EPI) && PM_EPI == 1
-            hst1_pair(out + ((int64_t)(rok ? s0 + w * 32 + 8 * (i / 4) + 4 * h + (i % 4) : 0) * Cout + co), v, rok && co < Cout, l32);
-#elif defined(PM_EPI) && PM_EPI == 2
-            hst1_pair(out + ((int64_t)(rok ? fr : 0) * Cout + co), v, rok && co < Cout && v == 123.456f, l32);
-#else
             hst1_pair(out + ((int64_t)(rok ? fr : 0) * Cout + co), v, rok && co < Cout, l32);
-#endif
         }
     }
-#ifdef PM_TIMING
-    PM_FT(7);
-    if (lane == 0 && w == 0 && blockIdx.y == 0 && blockIdx.x < 20000) {
-        for (int i = 0; i < 12; ++i) pm_fwd_dbg[12 * blockIdx.x + i] = ftm[i];
-    }
-#endif
 }
 
 // workspace: 16-byte header {beta, 1/beta, -, -}, then the packed filter
@@ -854,9 +791,6 @@ __device__ __forceinline__ void h2_tex_sweep(const u32x4 *__restrict__ WpT, cons
                                              const int *w_K, float (*x)[8], u32x4 (&bp)[NKS][2], int kbase, int Ks,
                                              int K, float ibeta, float &shs, int sweep, int Cin, int NG, bool add, int lane,
                                              int h
-#ifdef PM_TIMING
-                                             , unsigned long long (&ftm)[12], unsigned long long &ftprev
-#endif
                                              )
 {
     constexpr int chunk = 2 * NKS * 128;         // uint4 per chunk of two tiles
@@ -923,9 +857,7 @@ __device__ __forceinline__ void h2_tex_sweep(const u32x4 *__restrict__ WpT, cons
     }
     chunk_publish(wn, 0);
     chunk_publish(wn1, 1);
-    PM_FT(1);
     __syncthreads();
-    PM_FT(2);
 
     // 16-channel block gp of the stage -> global memory
     auto flush = [&](int gp) {
@@ -1024,16 +956,12 @@ __device__ __forceinline__ void h2_tex_sweep(const u32x4 *__restrict__ WpT, cons
                 if (cc == 0 && u == 0 && g > 0) finish_group(g - 1);
                 accp = acc0;
             }
-            PM_FT(3);
             if (more) chunk_publish(wn, c + 2);
-            PM_FT(4);
             __syncthreads();
-            PM_FT(5);
         }
     }
     contract(3);
     finish_group(NG - 1);
-    PM_FT(6);
 }
 
 // NKS = k-steps of 16 output channels (compile time, so that a tile's MFMAs and the previous tile's
@@ -1053,9 +981,6 @@ __global__ __launch_bounds__(512, 1) void f2f16h2_bwd_tex_k(const TIN *__restric
     __shared__ int s_k0[8][32], s_K[8][32], s_kmax[8];
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
     const int l32 = lane & 31, h = lane >> 5;
-#ifdef PM_TIMING
-    unsigned long long ftm[12] = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0}, ftprev = __builtin_readcyclecounter();
-#endif
     const float ibeta = hdr[1];                      // (used after the first fetches have come back)
 
     const int64_t slot = (int64_t)blockIdx.x * 256 + w * 32 + l32;
@@ -1092,10 +1017,9 @@ __global__ __launch_bounds__(512, 1) void f2f16h2_bwd_tex_k(const TIN *__restric
     }
     u32x4 bp[NKS][2];
     float shs = 0.f;
-    PM_FT(0);
     // The first sweep starts without a barrier in front (which would wait for the gout rows): every workgroup runs
     // it, and the barrier of its set-up is the one that makes the wavefronts' point counts visible to all.
-#define PM_H2T(N, FIRST, X) h2_tex_sweep<N, NKS, GVEC, HALF, FIRST, TIO>(WpT, sh, gtex, Ws, s_stage[w], s_k0[w], s_K[w], X, bp, kbase, Ks, K, ibeta, shs, sw, Cin, NG, co0 > 0, lane, h PM_FTARGS)
+#define PM_H2T(N, FIRST, X) h2_tex_sweep<N, NKS, GVEC, HALF, FIRST, TIO>(WpT, sh, gtex, Ws, s_stage[w], s_k0[w], s_K[w], X, bp, kbase, Ks, K, ibeta, shs, sw, Cin, NG, co0 > 0, lane, h)
     {
         const int sw = 0, kbase = k0;
         const int Ks = K > kHTKB ? kHTKB : K;
@@ -1126,10 +1050,6 @@ __global__ __launch_bounds__(512, 1) void f2f16h2_bwd_tex_k(const TIN *__restric
         else PM_H2T(6, false, none);
     }
 #undef PM_H2T
-#ifdef PM_TIMING
-    if (lane == 0 && w == 0 && blockIdx.x < 20000)
-        for (int i = 0; i < 12; ++i) pm_tex_dbg[12 * blockIdx.x + i] = ftm[i];
-#endif
 }
 
 
@@ -1550,15 +1470,7 @@ __device__ __forceinline__ void hwait_vm0()
 // (wavefront-uniform) = scale of the accumulators, fixed by the wavefront's first pass.
 struct HScales {
     float gam_cur, S;
-#ifdef PM_TIMING
-    unsigned long long tm[6];
-#endif
 };
-#ifdef PM_TIMING
-#define PM_T(i) do { const unsigned long long t_ = __builtin_readcyclecounter(); sc.tm[i] += t_ - tprev_; if (blockIdx.x == 7 && lane == 0 && it < 512) pm_filt_dbg[32 + (it * 4 + w) * 8 + i] = t_ - tprev_; tprev_ = t_; } while (0)
-#else
-#define PM_T(i) do { } while (0)
-#endif
 
 // One tile of 32 facets whose inputs are in LDS buffer it % 2 (descriptors in it % 3): start the
 // fetches for the next tile, run the passes, publish the next tile's inputs.
@@ -1576,9 +1488,6 @@ __device__ __forceinline__ void h2_filt_tile(const TIO *__restrict__ gout, const
     const int buf = it & 1, sb = it % 3, sb1 = (it + 1) % 3, sb2 = (it + 2) % 3;
     const int cw = c0 + 2 * NCP * w;                     // my wavefront's first input channel
     const bool idle = cw >= Cin;                         // narrow filters leave wavefronts without channels
-#ifdef PM_TIMING
-    unsigned long long tprev_ = __builtin_readcyclecounter();
-#endif
     if constexpr (PRE) {
         // my texture rows of this tile were requested a tile ago (or at the start of the phase); nothing else is
         // outstanding here, the end of the tile before consumed all of its fetches
@@ -1602,7 +1511,6 @@ __device__ __forceinline__ void h2_filt_tile(const TIO *__restrict__ gout, const
     const int gs = (it + 1) % 3;
     if (threadIdx.x == 0) s_gm[(it + 2) % 3] = 0u;
 
-    PM_T(0);
     const float gamma = s_gamma[buf];
     const int k0 = s_k0[sb][l32], K = s_K[sb][l32];
     const float invK = K > 0 ? 1.0f / (float)K : 0.f;
@@ -1676,9 +1584,7 @@ __device__ __forceinline__ void h2_filt_tile(const TIO *__restrict__ gout, const
             for (int kk = 0; kk < KW; ++kk)
 #pragma unroll
                 for (int q = 0; q < 8; ++q) shr[kk][q] *= al;
-            PM_T(1);
             h2_filt_pass<KW, NCP, HALF, PRE>(shr, slab, go_s[buf], acc, ea, eb, lane);
-            PM_T(2);
         }
     }
 
@@ -1698,12 +1604,7 @@ __device__ __forceinline__ void h2_filt_tile(const TIO *__restrict__ gout, const
         if (lane == 0) s_kmax[sb2] = km;
     }
     if (w == 2 && lane < 32) s_fn[(it + 1) & 1][lane] = fn3;       // (read at the start of the next tile)
-    PM_T(3);
     __syncthreads();
-    PM_T(4);
-#ifdef PM_TIMING
-    if (blockIdx.x == 7 && lane == 0 && it < 512) pm_filt_dbg[32 + (it * 4 + w) * 8 + 7] = KW;
-#endif
     const float gm = __builtin_bit_cast(float, s_gm[gs]);
     if (gm > 0.f && !scale_fits(sc.gam_cur, gm)) {           // workgroup-uniform: fetch and split that tile again
         float inv;
@@ -1761,10 +1662,6 @@ __global__ __launch_bounds__(256, 1) void f2f16h2_bwd_filt_k(const TIO *__restri
 #pragma unroll
             for (int i = 0; i < 16; ++i) acc[cp][t][i] = 0.f;
     HScales sc = {1.0f, 0.f};
-#ifdef PM_TIMING
-    for (int i = 0; i < 6; ++i) sc.tm[i] = 0;
-    const unsigned long long tstart_ = __builtin_readcyclecounter();
-#endif
 
     // prologue: descriptors of my first two tiles, inputs of the first (its gout maximum first, then the split)
     const int64_t stride = gridDim.x;
@@ -1832,13 +1729,6 @@ __global__ __launch_bounds__(256, 1) void f2f16h2_bwd_filt_k(const TIO *__restri
     // = (channel c0 + 2 NCP w + 2cp + m/16, d = m%16); four consecutive d's per group of four registers
     // accumulator (cp, t): lane (co = 32t + l32, half h), register i <-> row m = 8(i/4) + 4h + i%4
     // = (channel c0 + 2 NCP w + 2cp + m/16, d = m%16); four consecutive d's per group of four registers
-#ifdef PM_TIMING
-    if (blockIdx.x == 7 && lane == 0) {
-        for (int i = 0; i < 6; ++i) pm_filt_dbg[8 * w + i] = sc.tm[i];
-        pm_filt_dbg[8 * w + 6] = __builtin_readcyclecounter() - tstart_;
-        pm_filt_dbg[8 * w + 7] = it;
-    }
-#endif
     const float unscale = sc.S != 0.f ? 1.0f / sc.S : 0.f;
     float *dst = partial + (int64_t)blockIdx.x * Cout * Cin * 16;
 #pragma unroll
@@ -1888,17 +1778,3 @@ int f2f16h2_bwd_filter_partials(const void *gout_, const void *tex_, const float
 }
 
 }  // namespace pmesh
-#ifdef PM_TIMING
-extern "C" int pmesh_dbg_filt_timing(unsigned long long *host)
-{
-    return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(pmesh::pm_filt_dbg), sizeof(unsigned long long) * (32 + 512 * 4 * 8));
-}
-extern "C" int pmesh_dbg_tex_timing(unsigned long long *host)
-{
-    return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(pmesh::pm_tex_dbg), sizeof(unsigned long long) * 20000 * 12);
-}
-extern "C" int pmesh_dbg_fwd_timing(unsigned long long *host)
-{
-    return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(pmesh::pm_fwd_dbg), sizeof(unsigned long long) * 20000 * 12);
-}
-#endif

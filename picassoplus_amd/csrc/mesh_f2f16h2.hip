@@ -1421,7 +1421,7 @@ __device__ __forceinline__ void htex_issue(HRaw4<TIO> (&pf)[2 * kHKB], const TIO
     }
 }
 
-// The same rows straight into a slab buffer of the wavefront (fp32 rows of at least 64 channels, at most kHPre points
+// The same rows straight into a slab buffer of the wavefront (fp32 rows, four or eight channel pairs per wavefront, at most kHPre points
 // per facet), a whole tile ahead: no register holds them on the way, so the request can leave before the tile in
 // front is multiplied.  Row-major slab, 64 bytes per (point, facet slot); lane L of instruction j delivers the
 // 16 bytes at position 64 j + L, and fetches the piece (L & 3) ^ (slot / 4 & 3) of its row there, which spreads the
@@ -1438,7 +1438,7 @@ __device__ __forceinline__ void hdma16(const float *src, unsigned lds_base)
 {
     asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(src), "s"(lds_base) : "memory", "m0");
 }
-template <int KW>
+template <int KW, int NCP>
 __device__ __forceinline__ void htex_dma(const float *__restrict__ tex, const int *sk0, const int *sK, float4 *buf, int cw,
                                          int Cin, int lane)
 {
@@ -1449,7 +1449,8 @@ __device__ __forceinline__ void htex_dma(const float *__restrict__ tex, const in
     // (one address per slot in front of the selections: a product inside a selected operand turns it into a branch)
     const int pa = (lane & 3) ^ ((r >> 2) & 3), pb = (lane & 3) ^ (((16 + r) >> 2) & 3);
     const float *rowa = tex + (int64_t)k0a * Cin + cw + 4 * pa, *rowb = tex + (int64_t)k0b * Cin + cw + 4 * pb;
-    const bool cola = cw + 4 * pa < Cin, colb = cw + 4 * pb < Cin;
+    // (a wavefront with four channel pairs owns the first 32 bytes of its 64-byte slab rows; the rest reads zeros)
+    const bool cola = cw + 4 * pa < Cin && 4 * pa < 2 * NCP, colb = cw + 4 * pb < Cin && 4 * pb < 2 * NCP;
 #pragma unroll
     for (int j = 0; j < 2 * KW; ++j) {
         const int kk = j >> 1;
@@ -1494,7 +1495,7 @@ __device__ __forceinline__ void h2_filt_tile(const TIO *__restrict__ gout, const
         hwait_vm0();
         if (!idle)
             if constexpr (std::is_same<TIO, float>::value)
-                htex_dma<KW>(tex, s_k0[sb1], s_K[sb1], slab + ((it + 1) & 1) * (KW * 128), cw, Cin, lane);
+                htex_dma<KW, NCP>(tex, s_k0[sb1], s_K[sb1], slab + ((it + 1) & 1) * (KW * 128), cw, Cin, lane);
         slab += (it & 1) * (KW * 128);
     }
     // in flight while this tile is multiplied: inputs of the next tile, descriptors of the one after
@@ -1637,7 +1638,7 @@ __global__ __launch_bounds__(256, 1) void f2f16h2_bwd_filt_k(const TIO *__restri
     const int l32 = lane & 31, h = lane >> 5;
     const int c0 = blockIdx.y * (8 * NCP), n0 = blockIdx.z * 64;
     // phases of at most kHPre points request their texture rows a tile ahead, into the two halves of the slab
-    constexpr bool kPre = TVEC && NCP == 8 && std::is_same<TIO, float>::value;
+    constexpr bool kPre = TVEC && NCP >= 4 && std::is_same<TIO, float>::value;
 
     // selection operands of the transposition: column n < 16 takes d = n of channel a, n >= 16 takes d = n - 16 of b
     u32x4 ea, eb;
@@ -1706,7 +1707,7 @@ __global__ __launch_bounds__(256, 1) void f2f16h2_bwd_filt_k(const TIO *__restri
             hwait_vm0();                                                                                             \
             if (c0 + 2 * NCP * w < Cin)                                                                              \
                 if constexpr (std::is_same<TIO, float>::value)                                                       \
-                    htex_dma<N>(tex, s_k0[it % 3], s_K[it % 3], slab_s + w * kHSlabW + (it & 1) * (N * 128), \
+                    htex_dma<N, NCP>(tex, s_k0[it % 3], s_K[it % 3], slab_s + w * kHSlabW + (it & 1) * (N * 128), \
                                 c0 + 2 * NCP * w, Cin, lane);                                                        \
         }                                                                                                            \
         for (; tile < ntiles && (N == kHKB || __builtin_amdgcn_readfirstlane(s_kmax[it % 3]) <= N); ++it, tile += stride)             \

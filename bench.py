@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the mesh-conv hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload scene|shapes|pool|firstblock|tail|hierarchy|texture] [--scale S]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload scene|shapes|pool|firstblock|tail|hierarchy|texture|pcloud] [--scale S]
 
 A step is one forward+backward pass of the layer over one batch of seeded synthetic meshes
 already resident in HBM.  Default workload ``scene``: 8 room-like meshes of about 300 k
@@ -37,7 +37,7 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="scene", choices=["scene", "shapes", "pool", "firstblock", "tail", "hierarchy", "texture"],
+    ap.add_argument("--workload", default="scene", choices=["scene", "shapes", "pool", "firstblock", "tail", "hierarchy", "texture", "pcloud"],
                     help="scene: the headline layer (F2F+F2V, C=64); shapes: 16 small meshes V2F+F2F+F2V; pool: "
                          "1024x1024 grid max/avg pool + unpool; firstblock: the scene batch with the reference's first "
                          "block shapes, F2F 3->32 then F2V 32->32 with depth multiplier 2 (pi2_blocks.py:113-130)")
@@ -604,6 +604,88 @@ def run_texture(args, torch):
                             vertices=d["nv"], texture_points=d["T"], channels=C, sh_degree=L))
 
 
+def run_pcloud(args, torch):
+    """The point-cloud branch of a dual block on a coarse level of the scene batch (picasso/networks/pi2_blocks.py:43-62):
+    every 16th vertex of the eight rooms, 128 channels, spherical-harmonic graph of the set on itself (range search,
+    at most 16 neighbours, 17 weighted bins per pair), fuzzy depthwise convolution forward and backward.  The graph
+    build (search + coefficients) is set-up, as in the reference's data pipeline, and reported beside the step."""
+    from picassoplus_amd import _lib, synthetic as S
+    from picassoplus_amd.point import utils as PU
+    from picassoplus_amd.point.pi_modules import conv3d as pconv
+    dev = torch.device("cuda:0")
+    C, L, limit = 128, 3, 16
+    mesh = S.scene_workload(seed=3000, n_rooms=8, scale=args.scale)
+    nv_in = np.asarray(mesh["nv_in"], np.int64)
+    start = np.concatenate([[0], np.cumsum(nv_in)])
+    keep = np.concatenate([np.arange(start[b], start[b + 1], 16) for b in range(len(nv_in))])
+    nv = np.array([len(np.arange(start[b], start[b + 1], 16)) for b in range(len(nv_in))], np.int32)
+    xyz = torch.from_numpy(np.ascontiguousarray(mesh["vertex"][keep], dtype=np.float32)).to(dev)
+    NV = torch.from_numpy(nv).to(dev)
+    # radius: about 12 neighbours per point on the rooms' surfaces (points per area x pi r^2)
+    v0 = mesh["vertex"][keep[:nv[0]]]                             # (the first room: its points lie on the faces of a box)
+    ext = v0.max(0) - v0.min(0)
+    radius = float(np.sqrt(12.0 / np.pi / (len(v0) / max(2.0 * (ext[0] * ext[1] + ext[1] * ext[2] + ext[0] * ext[2]), 1e-9))))
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    nn_cnt, nn_idx, nn_dst, filt_idx, filt_coeff = PU.build_sphere_harmonics(xyz, xyz, NV, NV, radius, L=L, nn_uplimit=limit)
+    torch.cuda.synchronize()
+    graph_ms = (time.perf_counter() - t0) * 1e3
+    Np, P, T = xyz.shape[0], nn_idx.shape[0], filt_idx.shape[1]
+    gen = torch.Generator(device=dev).manual_seed(6000)
+    x = torch.randn(Np, C, device=dev, generator=gen).requires_grad_(True)
+    w = (torch.randn(T, C, 1, device=dev, generator=gen) / 4).requires_grad_(True)
+    g = torch.randn(Np, C, device=dev, generator=gen)
+
+    def step():
+        y = pconv.fuzzyconv3d(x, w, nn_cnt, nn_idx, filt_idx, filt_coeff)
+        return torch.autograd.grad(y, [x, w], g)
+
+    timer = EventTimer(torch)
+    _lib.set_call_hook(timer)
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    timer.on = True
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    _lib.set_call_hook(None)
+    per_op = timer.summary()
+    # every operand once: per pair its index pair, T bins and T weights, one gathered row of C floats; per point a row
+    pair = 8 + 8 * T
+    nb = {"point_conv_fwd": P * (pair + 4 * C) + 4 * Np * C + 4 * Np,
+          "point_conv_bwd": P * (2 * pair + 8 * C) + 4 * Np * C * 2 + 4 * Np}     # input and filter gradient: two passes over the pairs
+    fl = {"point_conv_fwd": 2.0 * P * C * (T + 1), "point_conv_bwd": 2.0 * P * C * (2 * T + 2)}
+    dom = max(nb, key=lambda k: per_op[k])
+    ach = nb[dom] / (per_op[dom] * 1e-3) / 1e9
+    total = sum(nb.values())
+    extra = {}
+    if not args.no_cpu_baseline:
+        # the oracle (numpy, float64) on the first sample's points and pairs
+        from oracle import point_ref as R
+        n0 = int(nv[0])
+        cnt = nn_cnt[:n0].cpu().numpy()
+        p0 = int(cnt.sum())
+        idx, fi, fc = nn_idx[:p0].cpu().numpy(), filt_idx[:p0].cpu().numpy(), filt_coeff[:p0].cpu().numpy().astype(np.float64)
+        xs, ws, gs = x[:n0].detach().cpu().numpy().astype(np.float64), w.detach().cpu().numpy().astype(np.float64), g[:n0].cpu().numpy().astype(np.float64)
+        t0 = time.perf_counter()
+        R.conv_fwd(xs, ws, cnt, idx, fi, fc)
+        R.conv_bwd(gs, xs, ws, cnt, idx, fi, fc)
+        spent = time.perf_counter() - t0
+        extra["cpu_baseline"] = dict(value=n0 / spent / 1e6, unit="Mpoints/s", cores=1, kind="port",
+                                     sample="first sample (%d points, %d pairs), one fwd+bwd pass, %.1f s" % (n0, p0, spent))
+    return dict(value=Np / (ms * 1e-3) / 1e6, unit="Mpoints/s", ms_per_step=ms, graph_build_ms=graph_ms, **extra, dtype="f32",
+                roofline=dict(bound="hbm", achieved=ach, peak=HBM_PEAK_GBS, unit="GB/s", frac=ach / HBM_PEAK_GBS, traffic=None,
+                              kernel=dom, kernel_ms=per_op[dom]),
+                ops={k: dict(ms=per_op[k], gbps=nb[k] / (per_op[k] * 1e-3) / 1e9, tflops=fl[k] / (per_op[k] * 1e-3) / 1e12)
+                     for k in nb},
+                hbm_gbps=total / (ms * 1e-3) / 1e9, hbm_frac=total / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                config=dict(workload="scene8_every16th_vertex_fuzzy_pointconv_C128_L3_nn16_fp32_fwd+bwd", points=Np, pairs=P,
+                            bins_per_pair=T, channels=C, radius=radius, meshes=int(len(nv))))
+
+
 def run_hierarchy(args, torch):
     """Encoder-decoder stack of the mesh modules over one 2 M-facet mesh and four 4:1 coarser levels: per level
     V2F + (texture interpolation -> F2F) -> F2V at widths 32/64/128/256, max / avg pooling between levels, then
@@ -774,6 +856,8 @@ def main():
         res = run_hierarchy(args, torch)
     elif args.workload == "texture":
         res = run_texture(args, torch)
+    elif args.workload == "pcloud":
+        res = run_pcloud(args, torch)
     else:
         res = run_conv_layer(args, torch, args.workload)
     if args.copy_calibration:

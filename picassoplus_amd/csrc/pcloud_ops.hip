@@ -139,6 +139,76 @@ __global__ void point_conv_bwd_filt_k(const float *__restrict__ gout, const floa
     }
 }
 
+// The same with at most FB bins, kept in registers: the workgroup turns 32 pairs at a time into a dense table
+// cm[pair][bin] (the coefficients of a pair's T entries, summed per bin, by one thread per pair), then every thread
+// multiplies its column's 32 products gout * in / count by the table rows, which all lanes read at the same address.
+// Pairs in ascending order per workgroup, as above.
+template <int FB>
+__global__ __launch_bounds__(256) void point_conv_bwd_filt_dense_k(const float *__restrict__ gout, const float *__restrict__ in,
+                                                                   PairGraph g, float *__restrict__ partial, int C, int r,
+                                                                   int64_t per)
+{
+    constexpr int PB = 32;
+    __shared__ __attribute__((aligned(16))) float s_cm[PB][FB];
+    __shared__ int s_o[PB], s_i[PB];
+    __shared__ float s_inv[PB];
+    const int CR = C * r, co = blockIdx.y * blockDim.x + threadIdx.x;
+    const bool mine = co < CR;
+    float acc[FB];
+#pragma unroll
+    for (int f = 0; f < FB; ++f) acc[f] = 0.f;
+    const int64_t p0 = (int64_t)blockIdx.x * per, p1 = p0 + per < g.Nout ? p0 + per : g.Nout;
+    for (int64_t pb = p0; pb < p1; pb += PB) {
+        __syncthreads();                                          // the table's readers of the block before are done
+        for (int e = threadIdx.x; e < PB * FB; e += blockDim.x) (&s_cm[0][0])[e] = 0.f;
+        __syncthreads();
+        if (threadIdx.x < PB) {
+            const int64_t p = pb + threadIdx.x;
+            int o = -1, i = -1;
+            if (p < p1) {
+                o = g.nn_index[p * 2];
+                i = g.nn_index[p * 2 + 1];
+                if (o < 0 || o >= g.Mp || i < 0 || i >= g.Np) o = -1;
+            }
+            s_o[threadIdx.x] = o;
+            s_i[threadIdx.x] = i;
+            s_inv[threadIdx.x] = o >= 0 ? inv_count(g.nn_count, o) : 0.f;
+            if (o >= 0)
+                for (int t = 0; t < g.T; ++t) {
+                    const int b = g.bin_index[p * g.T + t];
+                    if (b >= 0 && b < g.F) s_cm[threadIdx.x][b] += g.bin_coeff ? g.bin_coeff[p * g.T + t] : 1.f;
+                }
+        }
+        __syncthreads();
+        if (!mine) continue;
+#pragma unroll 1
+        for (int q0 = 0; q0 < PB; q0 += 8) {
+            float d[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {                         // eight pairs' operands in flight
+                const int o = s_o[q0 + u], i = s_i[q0 + u];
+                d[u] = o >= 0 ? gout[(int64_t)o * CR + co] * in[(int64_t)i * C + co / r] * s_inv[q0 + u] : 0.f;
+            }
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+#pragma unroll
+                for (int f4 = 0; f4 < FB; f4 += 4) {
+                    const float4 c = *reinterpret_cast<const float4 *>(&s_cm[q0 + u][f4]);
+                    acc[f4] = fmaf(c.x, d[u], acc[f4]);
+                    acc[f4 + 1] = fmaf(c.y, d[u], acc[f4 + 1]);
+                    acc[f4 + 2] = fmaf(c.z, d[u], acc[f4 + 2]);
+                    acc[f4 + 3] = fmaf(c.w, d[u], acc[f4 + 3]);
+                }
+        }
+    }
+    if (mine) {
+        float *dst = partial + (int64_t)blockIdx.x * g.F * CR;
+#pragma unroll
+        for (int f = 0; f < FB; ++f)
+            if (f < g.F) dst[(int64_t)f * CR + co] = acc[f];
+    }
+}
+
 // ------------------------------------------------------------------------------------------------ pooling
 // MODE 0: max with arg-max (first pair among equals; -1 and 0 for a query without neighbours), 1: average
 template <int V, int MODE>
@@ -353,10 +423,19 @@ extern "C" int pmesh_point_conv_bwd(const float *grad_output, const float *input
     }
     const int G = filt_blocks(Nout, F, CR);
     PM_REQUIRE(workspace_bytes >= (size_t)G * F * CR * sizeof(float), "point_conv_bwd: workspace too small (%zu bytes)", workspace_bytes);
+    const int64_t per = ceil_div(Nout, G);
+    if (F <= 64) {
+        int threads = 256;
+        while (threads > 64 && threads / 2 >= CR) threads /= 2;
+        const dim3 grid((unsigned)G, (unsigned)ceil_div(CR, threads));
+        if (F <= 32) point_conv_bwd_filt_dense_k<32><<<grid, dim3(threads), 0, st>>>(grad_output, input, g, (float *)workspace, C, r, per);
+        else point_conv_bwd_filt_dense_k<64><<<grid, dim3(threads), 0, st>>>(grad_output, input, g, (float *)workspace, C, r, per);
+        PM_LAUNCHED("point_conv_bwd(filter)");
+        return reduce_partials((const float *)workspace, grad_filter, G, F * CR, st);
+    }
     int cols = 256;
     while (cols > 32 && ((size_t)F * cols * 4 > 65536 || cols / 2 >= CR)) cols /= 2;
     PM_REQUIRE((size_t)F * cols * 4 <= 65536, "point_conv_bwd: too many bins");
-    const int64_t per = ceil_div(Nout, G);
     point_conv_bwd_filt_k<<<dim3((unsigned)G, (unsigned)ceil_div(CR, cols)), dim3(cols), (size_t)F * cols * 4, st>>>(
         grad_output, input, g, (float *)workspace, C, r, cols, per);
     PM_LAUNCHED("point_conv_bwd(filter)");

@@ -4,8 +4,10 @@
 // The reference runs one thread per (neighbour pair, channel) and adds into the output with float atomics.  Here
 // every op is a segmented sum over a sorted adjacency of the pairs (pmesh_build_index_csr): by query for the forward
 // ops, by database point for the input gradients, so each output row is written once, by one lane group, in a fixed
-// order.  The filter gradient is summed per workgroup in LDS (one column per thread, pairs in ascending order) and the
-// workgroups' partial results are added in a fixed tree order.
+// order.  The filter gradient is summed per workgroup (one column per thread, pairs in ascending order; bins in
+// registers up to 64 of them, in LDS beyond) and the workgroups' partial results are added in a fixed tree order.
+// With at most 32 bins, depth multiplier 1 and at most 256 channels, forward and input gradient keep the filter in
+// registers and read the pairs' coefficients from a dense per-pair table in LDS.
 //
 //   w[p, co]        = sum_t coeff[p, t] * filter[bin[p, t], co]           (plain form: one bin, weight 1)
 //   out[o, co]      = (1 / nn_count[o]) sum_{p = (o, i)} in[i, co / r] * w[p, co]
@@ -111,6 +113,87 @@ __global__ __launch_bounds__(kBlock) void point_conv_bwd_in_k(const float *__res
             }
         }
         stp<V>(gin + row * C + c, acc);
+    }
+}
+
+// Forward (MODE 0: rows = queries, the other end of a pair is a database row of `src` = in) and input gradient (MODE 1:
+// rows = database points, the other end a query row of `src` = gout, weighted by 1 / nn_count of that query) for at most
+// FB bins, depth multiplier 1 and rows of at most 256 channels in four-channel pieces: a lane keeps its four columns of
+// the filter in registers, and the workgroup turns the pairs of its rows, 128 at a time, into a dense table
+// cm[pair][bin] in LDS (one thread per pair), together with the pair's other end and weight.  The weight of a pair for
+// a lane's channels is then FB x 4 FMAs on table rows that all lanes of a row read at the same address, instead of T
+// dependent fetches of filter rows per pair and lane.
+template <int FB, int MODE>
+__global__ __launch_bounds__(kBlock) void point_conv_rows_dense_k(const float *__restrict__ src, const float *__restrict__ filt,
+                                                                  PairGraph g, const int *__restrict__ rowptr,
+                                                                  const int *__restrict__ order, float *__restrict__ out, int C,
+                                                                  int lpr_log2)
+{
+    constexpr int NP = 128;
+    __shared__ __attribute__((aligned(16))) float s_cm[NP][FB];
+    __shared__ int s_other[NP];
+    __shared__ float s_scale[NP];
+    const int lpr = 1 << lpr_log2, lane = threadIdx.x & (lpr - 1), slot = threadIdx.x >> lpr_log2, rpb = kBlock >> lpr_log2;
+    const int64_t rows = MODE == 0 ? g.Mp : g.Np, nother = MODE == 0 ? g.Np : g.Mp;
+    const int64_t row0 = (int64_t)blockIdx.x * rpb, row = row0 + slot;
+    const int64_t rowl = row0 + rpb < rows ? row0 + rpb : rows;
+    const int eb = rowptr[row0], ee = rowptr[rowl];                 // the workgroup's pairs, in row order
+    const bool live = row < rows && 4 * lane < C;
+    const int e0 = row < rows ? rowptr[row] : 0, e1 = row < rows ? rowptr[row + 1] : 0;
+    const int c = 4 * lane;
+    float fr[FB][4];
+#pragma unroll
+    for (int f = 0; f < FB; ++f) {
+        const float4 v = (live && f < g.F) ? *reinterpret_cast<const float4 *>(filt + (int64_t)f * C + c) : make_float4(0.f, 0.f, 0.f, 0.f);
+        fr[f][0] = v.x; fr[f][1] = v.y; fr[f][2] = v.z; fr[f][3] = v.w;
+    }
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int cb = eb; cb < ee; cb += NP) {
+        __syncthreads();                                          // the table's readers of the chunk before are done
+        for (int e = threadIdx.x; e < NP * FB / 4; e += kBlock) reinterpret_cast<float4 *>(&s_cm[0][0])[e] = make_float4(0.f, 0.f, 0.f, 0.f);
+        __syncthreads();
+        if (threadIdx.x < NP && cb + (int)threadIdx.x < ee) {
+            const int64_t p = order[cb + threadIdx.x];
+            const int o = g.nn_index[p * 2], i = g.nn_index[p * 2 + 1];
+            const int other = MODE == 0 ? i : o;
+            const bool ok = other >= 0 && other < nother;
+            s_other[threadIdx.x] = ok ? other : -1;
+            s_scale[threadIdx.x] = (MODE == 1 && ok) ? inv_count(g.nn_count, o) : 1.f;
+            if (ok)
+                for (int t = 0; t < g.T; ++t) {
+                    const int b = g.bin_index[p * g.T + t];
+                    if (b >= 0 && b < g.F) s_cm[threadIdx.x][b] += g.bin_coeff ? g.bin_coeff[p * g.T + t] : 1.f;
+                }
+        }
+        __syncthreads();
+        if (!live) continue;
+        const int a = e0 > cb ? e0 : cb, b = e1 < cb + NP ? e1 : cb + NP;
+        for (int e = a; e < b; ++e) {
+            const int q = e - cb, other = s_other[q];
+            if (other < 0) continue;
+            const float4 x = *reinterpret_cast<const float4 *>(src + (int64_t)other * C + c);      // (asked for before the weight is formed)
+            float w[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int f4 = 0; f4 < FB; f4 += 4) {
+                const float4 m = *reinterpret_cast<const float4 *>(&s_cm[q][f4]);
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    w[u] = fmaf(m.x, fr[f4][u], w[u]);
+                    w[u] = fmaf(m.y, fr[f4 + 1][u], w[u]);
+                    w[u] = fmaf(m.z, fr[f4 + 2][u], w[u]);
+                    w[u] = fmaf(m.w, fr[f4 + 3][u], w[u]);
+                }
+            }
+            const float sc = s_scale[q];
+            acc[0] = fmaf(x.x * w[0], sc, acc[0]);
+            acc[1] = fmaf(x.y * w[1], sc, acc[1]);
+            acc[2] = fmaf(x.z * w[2], sc, acc[2]);
+            acc[3] = fmaf(x.w * w[3], sc, acc[3]);
+        }
+    }
+    if (live) {
+        const float inv = MODE == 0 ? inv_count(g.nn_count, row) : 1.f;
+        *reinterpret_cast<float4 *>(out + row * C + c) = make_float4(acc[0] * inv, acc[1] * inv, acc[2] * inv, acc[3] * inv);
     }
 }
 
@@ -380,7 +463,13 @@ extern "C" int pmesh_point_conv_fwd(const float *input, const float *filter, con
     hipStream_t st = (hipStream_t)stream;
     const PairGraph g = {nn_index, nn_count, bin_index, bin_coeff, Np, Mp, Nout, T, F};
     const int CR = C * r;
-    if (r == 1 && C % 4 == 0 && aligned16(input) && aligned16(filter) && aligned16(output))
+    if (r == 1 && C % 4 == 0 && C <= 256 && F <= 32 && aligned16(input) && aligned16(filter) && aligned16(output)) {
+        const RowShape rs = row_shape(C / 4);
+        const int64_t blocks = ceil_div(Mp, rs.rpb);
+        PM_REQUIRE(grid_ok(blocks), "grid too large");
+        if (F <= 16) point_conv_rows_dense_k<16, 0><<<dim3((unsigned)blocks), dim3(kBlock), 0, st>>>(input, filter, g, rowptr, order, output, C, rs.lpr_log2);
+        else point_conv_rows_dense_k<32, 0><<<dim3((unsigned)blocks), dim3(kBlock), 0, st>>>(input, filter, g, rowptr, order, output, C, rs.lpr_log2);
+    } else if (r == 1 && C % 4 == 0 && aligned16(input) && aligned16(filter) && aligned16(output))
         PM_ROW_LAUNCH(point_conv_fwd_k<4>, Mp, CR / 4, input, filter, g, rowptr, order, output, C, r);
     else
         PM_ROW_LAUNCH(point_conv_fwd_k<1>, Mp, CR, input, filter, g, rowptr, order, output, C, r);
@@ -415,7 +504,13 @@ extern "C" int pmesh_point_conv_bwd(const float *grad_output, const float *input
     const PairGraph g = {nn_index, nn_count, bin_index, bin_coeff, Np, Mp, Nout, T, F};
     if (grad_input) {
         PM_REQUIRE(rowptr_in && order_in, "point_conv_bwd: the input gradient needs the pairs sorted by database point");
-        if (r == 1 && C % 4 == 0 && aligned16(grad_output) && aligned16(filter) && aligned16(grad_input))
+        if (r == 1 && C % 4 == 0 && C <= 256 && F <= 32 && aligned16(grad_output) && aligned16(filter) && aligned16(grad_input)) {
+            const RowShape rs = row_shape(C / 4);
+            const int64_t blocks = ceil_div(Np, rs.rpb);
+            PM_REQUIRE(grid_ok(blocks), "grid too large");
+            if (F <= 16) point_conv_rows_dense_k<16, 1><<<dim3((unsigned)blocks), dim3(kBlock), 0, st>>>(grad_output, filter, g, rowptr_in, order_in, grad_input, C, rs.lpr_log2);
+            else point_conv_rows_dense_k<32, 1><<<dim3((unsigned)blocks), dim3(kBlock), 0, st>>>(grad_output, filter, g, rowptr_in, order_in, grad_input, C, rs.lpr_log2);
+        } else if (r == 1 && C % 4 == 0 && aligned16(grad_output) && aligned16(filter) && aligned16(grad_input))
             PM_ROW_LAUNCH(point_conv_bwd_in_k<4>, Np, C / 4, grad_output, filter, g, rowptr_in, order_in, grad_input, C, r);
         else
             PM_ROW_LAUNCH(point_conv_bwd_in_k<1>, Np, C, grad_output, filter, g, rowptr_in, order_in, grad_input, C, r);

@@ -118,16 +118,19 @@ TRAFFIC_KERNELS = {
     "tail": {"dense_fwd": [r"dense_rows_k<\d+, \d+, (true|false), 0, "],
              "dense_bwd": [r"dense_rows_k<\d+, \d+, (true|false), [12], ", r"dense_wgrad_k", r"reduce_partials_k"]},
     "texture": {"texture_fwd": [r"texture_fwd_k"], "texture_bwd": [r"texture_bwd_flat_k", r"texture_bwd_k"]},
+    "pcloud": {"point_conv_fwd": [r"point_conv_rows_dense_k<\d+, 0>", r"point_conv_fwd_k"],
+               "point_conv_bwd": [r"point_conv_rows_dense_k<\d+, 1>", r"point_conv_bwd_in_k", r"point_conv_bwd_filt", r"reduce_partials_k"]},
 }
 
 
-TIMED_SOURCES = ("mesh_f2f", "mesh_f2v", "mesh_rows", "mesh_dense", "mesh_texture", "common", "f2f_internal", "rows_internal",
-                 "sph_internal")
+TIMED_SOURCES = ("mesh_f2f", "mesh_f2v", "mesh_rows", "mesh_dense", "mesh_texture", "pcloud_ops", "common", "f2f_internal",
+                 "rows_internal", "sph_internal")
 
 
 def build_id():
     """Identity of the kernels being timed: hash over the sources that hold them (convolutions, pooling, tails,
-    texture interpolation and their shared headers; index builds and mesh preparation are not timed here)."""
+    texture interpolation, point convolution and their shared headers; index builds, neighbour searches and mesh
+    preparation are not timed here)."""
     import hashlib
     h = hashlib.sha256()
     csrc = os.path.join(ROOT, "picassoplus_amd", "csrc")
@@ -677,8 +680,9 @@ def run_pcloud(args, torch):
         extra["cpu_baseline"] = dict(value=n0 / spent / 1e6, unit="Mpoints/s", cores=1, kind="port",
                                      sample="first sample (%d points, %d pairs), one fwd+bwd pass, %.1f s" % (n0, p0, spent))
     return dict(value=Np / (ms * 1e-3) / 1e6, unit="Mpoints/s", ms_per_step=ms, graph_build_ms=graph_ms, **extra, dtype="f32",
-                roofline=dict(bound="hbm", achieved=ach, peak=HBM_PEAK_GBS, unit="GB/s", frac=ach / HBM_PEAK_GBS, traffic=None,
-                              kernel=dom, kernel_ms=per_op[dom]),
+                roofline=dict(bound="hbm", achieved=ach, peak=HBM_PEAK_GBS, unit="GB/s", frac=ach / HBM_PEAK_GBS,
+                              traffic=measured_traffic("pcloud", "", dom) if args.scale == 1.0 else None, kernel=dom,
+                              kernel_ms=per_op[dom]),
                 ops={k: dict(ms=per_op[k], gbps=nb[k] / (per_op[k] * 1e-3) / 1e9, tflops=fl[k] / (per_op[k] * 1e-3) / 1e12)
                      for k in nb},
                 hbm_gbps=total / (ms * 1e-3) / 1e9, hbm_frac=total / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,

@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the mesh-conv hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload scene|shapes|pool|firstblock|tail|hierarchy|texture|pcloud] [--scale S]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload scene|shapes|pool|firstblock|tail|hierarchy|texture|pcloud|decimate] [--scale S]
 
 A step is one forward+backward pass of the layer over one batch of seeded synthetic meshes
 already resident in HBM.  Default workload ``scene``: 8 room-like meshes of about 300 k
@@ -37,7 +37,7 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="scene", choices=["scene", "shapes", "pool", "firstblock", "tail", "hierarchy", "texture", "pcloud"],
+    ap.add_argument("--workload", default="scene", choices=["scene", "shapes", "pool", "firstblock", "tail", "hierarchy", "texture", "pcloud", "decimate"],
                     help="scene: the headline layer (F2F+F2V, C=64); shapes: 16 small meshes V2F+F2F+F2V; pool: "
                          "1024x1024 grid max/avg pool + unpool; firstblock: the scene batch with the reference's first "
                          "block shapes, F2F 3->32 then F2V 32->32 with depth multiplier 2 (pi2_blocks.py:113-130)")
@@ -690,6 +690,72 @@ def run_pcloud(args, torch):
                             bins_per_pair=T, channels=C, radius=radius, meshes=int(len(nv))))
 
 
+def run_decimate(args, torch):
+    """Mesh decimation of the scene batch to a quarter of its vertices (picasso/mesh/pi_modules/decimate.py:5-52): the
+    producer of the cluster maps the pooling ops take.  One step = the whole loop of simplification rounds; the
+    native calls (quadrics, edge costs, host clustering, cluster composition, position averaging) are timed per entry
+    point, the rest of a step is the integer sorts / scans / compactions between them (PyTorch ops)."""
+    from picassoplus_amd import _lib, synthetic as S
+    from picassoplus_amd.mesh.pi_modules import decimate as D
+    dev = torch.device("cuda:0")
+    mesh = S.scene_workload(seed=3000, n_rooms=8, scale=args.scale)
+    t = lambda a, dt: torch.from_numpy(np.ascontiguousarray(a)).to(dt).to(dev)
+    vertex, face = t(mesh["vertex"], torch.float32), t(mesh["face"], torch.int32)
+    nv_in, mf_in = t(mesh["nv_in"], torch.int32), t(mesh["mf_in"], torch.int32)
+    nv_out = (nv_in // 4).to(torch.int32)
+    geometry = D.compute_triangle_geometry_(vertex, face)
+    Nv, Nf = vertex.shape[0], face.shape[0]
+    rounds = []
+
+    def step():
+        out = D.mesh_decimation_(vertex, face, geometry, nv_in, mf_in, nv_out)
+        return out
+
+    timer = EventTimer(torch)
+    _lib.set_call_hook(timer)
+    for _ in range(max(1, min(args.warmup, 2))):
+        out = step()
+    torch.cuda.synchronize()
+    timer.on = True
+    steps = max(1, min(args.steps, 5))
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        out = step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / steps
+    _lib.set_call_hook(None)
+    per_step = timer.totals(steps)
+    per_call = timer.summary()
+    calls = {}
+    for name, _, _ in timer.pairs:
+        k = name.replace("pmesh_", "")
+        calls[k] = calls.get(k, 0) + 1
+    n_rounds = calls.get("edge_costs", steps) // steps
+    # the edge-cost kernel: per candidate edge two quadrics (10 floats each), two positions, two indices in, one cost out
+    n_edges0 = None
+    dom = "edge_costs"
+    extra = {}
+    if not args.no_cpu_baseline:
+        from oracle import decimate_ref as R
+        # the numpy oracle on the first sample, one round
+        n0, m0 = int(mesh["nv_in"][0]), int(mesh["mf_in"][0])
+        v0 = np.ascontiguousarray(mesh["vertex"][:n0], dtype=np.float32)
+        f0 = np.ascontiguousarray(mesh["face"][:m0], dtype=np.int32)
+        t0 = time.perf_counter()
+        R.simplify(v0, f0, R.triangle_geometry(v0, f0), np.array([n0]), np.array([m0]), np.array([n0 - n0 // 4]))
+        spent = time.perf_counter() - t0
+        extra["cpu_baseline"] = dict(value=n0 / spent / 1e6, unit="Mvertices/s", cores=1, kind="port",
+                                     sample="first sample (%d vertices, %d facets), ONE simplification round, %.1f s" % (n0, m0, spent))
+    native = sum(per_step.values())
+    return dict(value=Nv / (ms * 1e-3) / 1e6, unit="Mvertices/s", ms_per_step=ms, steps_timed=steps, rounds=n_rounds, **extra,
+                dtype="f32 (quadrics, costs), int32 (maps)",
+                roofline=dict(bound="hbm", achieved=None, peak=HBM_PEAK_GBS, unit="GB/s", frac=None, traffic=None, kernel=dom,
+                              kernel_ms=per_call.get(dom)),
+                native_ms_per_step=native, ops_ms_per_step=per_step, ops_ms_per_call=per_call,
+                vertices_out=int(out[0].shape[0]), facets_out=int(out[1].shape[0]),
+                config=dict(workload="scene8x300k_decimation_to_quarter_fp32", vertices=Nv, facets=Nf, meshes=int(len(mesh["nv_in"]))))
+
+
 def run_hierarchy(args, torch):
     """Encoder-decoder stack of the mesh modules over one 2 M-facet mesh and four 4:1 coarser levels: per level
     V2F + (texture interpolation -> F2F) -> F2V at widths 32/64/128/256, max / avg pooling between levels, then
@@ -862,6 +928,8 @@ def main():
         res = run_texture(args, torch)
     elif args.workload == "pcloud":
         res = run_pcloud(args, torch)
+    elif args.workload == "decimate":
+        res = run_decimate(args, torch)
     else:
         res = run_conv_layer(args, torch, args.workload)
     if args.copy_calibration:

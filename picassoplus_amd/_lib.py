@@ -146,6 +146,36 @@ def call(name, *args):
         raise RuntimeError("%s failed: %s" % (name, msg.decode() if msg else "unknown error"))
 
 
+def call_many(name, arg_lists, workers=8):
+    """Invoke a HOST-side int-returning entry point once per argument list, on a small thread pool (ctypes releases
+    the interpreter lock during a foreign call; the library's error text is per thread and is read on the thread
+    that failed).  The call hook sees one begin / end pair around all of them."""
+    lib = load()
+    fn = getattr(lib, name)
+    hook = _call_hook
+    if hook is not None:
+        hook(name, "begin")
+
+    def one(args):
+        rc = fn(*args)
+        if rc != 0:
+            msg = lib.pmesh_last_error()
+            return msg.decode() if msg else "unknown error"
+        return None
+
+    if len(arg_lists) <= 1 or workers <= 1:
+        errors = [one(a) for a in arg_lists]
+    else:
+        from concurrent.futures import ThreadPoolExecutor
+        with ThreadPoolExecutor(max_workers=min(workers, len(arg_lists))) as pool:
+            errors = list(pool.map(one, arg_lists))
+    if hook is not None:
+        hook(name, "end")
+    for e in errors:
+        if e is not None:
+            raise RuntimeError("%s failed: %s" % (name, e))
+
+
 def reload_options():
     """Make the library read its PMESH_* switches from the environment again (it reads them once, at its first
     call): for tests and benchmarks that change them inside one process."""

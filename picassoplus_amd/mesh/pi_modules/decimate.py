@@ -112,12 +112,15 @@ def cluster_vertices(edge_vi, edge_vj, sample, nvIn_cumsum, nv2Remove, Nv):
     vt_replace = np.zeros(Nv, dtype=np.int32)
     bounds = np.searchsorted(smp, np.arange(len(ends) + 1))
     P = ctypes.c_void_p
+    jobs = []
     for b in range(len(ends)):
         e0, e1 = int(bounds[b]), int(bounds[b + 1])
         start = int(ends[b - 1]) if b else 0
         if e1 > e0 and budget[b] > 0:
-            _lib.call("pmesh_cluster_vertices_host", P(vi.ctypes.data + 4 * e0), P(vj.ctypes.data + 4 * e0), e1 - e0, start,
-                      int(ends[b]) - start, int(budget[b]), P(vt_replace.ctypes.data))
+            jobs.append((P(vi.ctypes.data + 4 * e0), P(vj.ctypes.data + 4 * e0), e1 - e0, start, int(ends[b]) - start,
+                         int(budget[b]), P(vt_replace.ctypes.data)))
+    # the samples are independent and write disjoint ranges of vt_replace: one host thread each
+    _lib.call_many("pmesh_cluster_vertices_host", jobs)
     return vt_replace
 
 

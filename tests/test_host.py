@@ -289,3 +289,37 @@ def test_host_vertex_clustering_matches_the_oracle(seed):
         assert (got < 0).sum() <= budget
     with pytest.raises(RuntimeError):                       # an edge that leaves the sample's vertex range
         _lib.call("pmesh_cluster_vertices_host", vi.ctypes.data, vj.ctypes.data, len(vi), start, num // 2, num, got.ctypes.data)
+
+
+def test_call_many_runs_independent_samples_on_threads_and_reports_a_failure():
+    """_lib.call_many: the samples of a batch (disjoint vertex ranges of one vt_replace array) on a thread pool give what
+    one call after the other gives; a failing call raises with the library's message of ITS thread."""
+    import ctypes
+
+    rng = np.random.default_rng(7)
+    P = ctypes.c_void_p
+    num, samples = 200, 6
+    vi_all, vj_all, jobs = [], [], []
+    for b in range(samples):
+        pairs = sorted({tuple(sorted(p)) for p in rng.integers(b * num, (b + 1) * num, (3 * num, 2)).tolist() if p[0] != p[1]})
+        perm = rng.permutation(len(pairs))
+        vi_all.append(np.ascontiguousarray(np.array(pairs, np.int32)[perm, 0]))
+        vj_all.append(np.ascontiguousarray(np.array(pairs, np.int32)[perm, 1]))
+    one, many = np.zeros(samples * num, np.int32), np.zeros(samples * num, np.int32)
+    for b in range(samples):
+        _lib.call("pmesh_cluster_vertices_host", vi_all[b].ctypes.data, vj_all[b].ctypes.data, len(vi_all[b]), b * num, num, num // 3,
+                  one.ctypes.data)
+        jobs.append((P(vi_all[b].ctypes.data), P(vj_all[b].ctypes.data), len(vi_all[b]), b * num, num, num // 3, P(many.ctypes.data)))
+    _lib.call_many("pmesh_cluster_vertices_host", jobs)
+    assert np.array_equal(one, many) and (many < 0).sum() > 0
+    seen = []
+    _lib.set_call_hook(lambda name, phase: seen.append((name, phase)))
+    try:
+        _lib.call_many("pmesh_cluster_vertices_host", jobs[:2])
+    finally:
+        _lib.set_call_hook(None)
+    assert seen == [("pmesh_cluster_vertices_host", "begin"), ("pmesh_cluster_vertices_host", "end")]
+    bad = list(jobs)
+    bad[3] = bad[3][:4] + (num // 2,) + bad[3][5:]          # the sample's range cut in half: its edges leave it
+    with pytest.raises(RuntimeError, match="outside the sample's vertex range"):
+        _lib.call_many("pmesh_cluster_vertices_host", bad)

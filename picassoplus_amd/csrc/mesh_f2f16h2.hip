@@ -1436,7 +1436,11 @@ constexpr int kHSlabW = 2 * kHPre * 128;              // float4 of a wavefront's
 static_assert(kHSlabW >= kHKB * 128, "slab");
 __device__ __forceinline__ void hdma16(const float *src, unsigned lds_base)
 {
-    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(src), "s"(lds_base) : "memory", "m0");
+    unsigned keep;                                      // (M0 is handed back as it was found: the compiler may hold a value of its own there)
+    asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off\n\ts_mov_b32 m0, %0"
+                 : "=&s"(keep)
+                 : "v"(src), "s"(lds_base)
+                 : "memory");
 }
 template <int KW, int NCP>
 __device__ __forceinline__ void htex_dma(const float *__restrict__ tex, const int *sk0, const int *sK, float4 *buf, int cw,

@@ -377,3 +377,98 @@ def test_config_shapes_block_forward_backward(cuda):
     assert_close(y, y64.detach().numpy(), "shapes block output")
     for name, g, r in zip(("X", "V2F filter", "F2F filter", "F2V filter"), grads, ref_grads):
         assert_close(g, r.numpy(), "shapes block gradient of " + name)
+
+
+def test_point_conv_full_size_adjoints_and_sample_parity(cuda):
+    """The bench's point-cloud workload (every 16th vertex of the scene batch, spherical-harmonic graph of at most 16
+    neighbours, 128 channels): the fuzzy point convolution is linear in its input and in its filter, so
+    <g, conv(x, w)> = <x, grad_x> = <w, grad_w>; a sample of output rows against the float64 oracle; the graph's
+    invariants (counts within the limit, every point its own neighbour, pairs sorted by query)."""
+    from oracle import point_ref
+    from picassoplus_amd.point import utils as PU
+    from picassoplus_amd.point.pi_modules import conv3d as pconv
+    say("case point conv full size")
+    mesh = S.scene_workload(seed=3000, n_rooms=8, scale=1.0)
+    nv_in = np.asarray(mesh["nv_in"], np.int64)
+    start = np.concatenate([[0], np.cumsum(nv_in)])
+    keep = np.concatenate([np.arange(start[b], start[b + 1], 16) for b in range(len(nv_in))])
+    nv = np.array([len(np.arange(start[b], start[b + 1], 16)) for b in range(len(nv_in))], np.int32)
+    xyz = dev(np.ascontiguousarray(mesh["vertex"][keep], dtype=np.float32), cuda)
+    NV = dev(nv, cuda)
+    C, L, limit, radius = 128, 3, 16, 0.18
+    nn_cnt, nn_idx, nn_dst, filt_idx, filt_coeff = PU.build_sphere_harmonics(xyz, xyz, NV, NV, radius, L=L, nn_uplimit=limit)
+    Np, P, T = xyz.shape[0], nn_idx.shape[0], filt_idx.shape[1]
+    cnt = nn_cnt.cpu().numpy()
+    idx = nn_idx.cpu().numpy()
+    assert cnt.sum() == P and cnt.min() >= 1 and cnt.max() <= limit and T == (L + 1) ** 2 + 1
+    assert np.all(np.diff(idx[:, 0]) >= 0) and np.array_equal(np.bincount(idx[:, 0], minlength=Np), cnt)
+    first = np.concatenate([[0], np.cumsum(cnt)[:-1]])
+    sample_of = np.repeat(np.arange(len(nv)), nv)
+    assert np.array_equal(sample_of[idx[:, 0]], sample_of[idx[:, 1]])           # neighbours stay inside the sample
+    assert bool((nn_dst < radius).all())
+    gen = torch.Generator(device=cuda).manual_seed(11)
+    x = torch.randn(Np, C, device=cuda, generator=gen).requires_grad_(True)
+    w = (torch.randn(T, C, 1, device=cuda, generator=gen) / 4).requires_grad_(True)
+    g = torch.randn(Np, C, device=cuda, generator=gen)
+    y = pconv.fuzzyconv3d(x, w, nn_cnt, nn_idx, filt_idx, filt_coeff)
+    gx, gw = torch.autograd.grad(y, [x, w], g)
+    lhs = _dot(g, y.detach())
+    scale = float(g.double().norm() * y.detach().double().norm())
+    _adjoint_ok(lhs, _dot(x.detach(), gx), scale, "point conv: <g, y> = <x, gx>")
+    _adjoint_ok(lhs, _dot(w.detach(), gw), scale, "point conv: <g, y> = <w, gw>")
+    # sampled rows against the oracle (each row needs only its own pairs)
+    rng = np.random.default_rng(12)
+    rows = np.sort(rng.choice(Np, 400, replace=False))
+    fi, fc = filt_idx.cpu().numpy(), filt_coeff.cpu().numpy().astype(np.float64)
+    xs, ws = x.detach().cpu().numpy().astype(np.float64), w.detach().cpu().numpy().astype(np.float64)
+    sel = np.concatenate([np.arange(first[r], first[r] + cnt[r]) for r in rows])
+    sub_idx = idx[sel].copy()
+    sub_idx[:, 0] = np.repeat(np.arange(len(rows)), cnt[rows])
+    ref = point_ref.conv_fwd(xs, ws, cnt[rows], sub_idx, fi[sel], fc[sel])
+    assert_close(y.detach()[torch.from_numpy(rows).to(cuda)], ref, "point conv sampled rows")
+
+
+def test_decimation_full_size_invariants(cuda):
+    """The scene batch decimated to a quarter of its vertices: the maps' invariants (A.5 of the pooling ops' contract),
+    facets that reference live output vertices only, no degenerate facet left, the sample counts, a second run
+    bit-equal to the first, and max pooling over the maps equal to a brute-force maximum over the clusters on a sample."""
+    from picassoplus_amd.mesh.pi_modules import decimate as D
+    say("case decimation full size")
+    mesh = S.scene_workload(seed=3000, n_rooms=8, scale=1.0)
+    vertex, face = dev(mesh["vertex"].astype(np.float32), cuda), dev(mesh["face"].astype(np.int32), cuda)
+    nv_in, mf_in = dev(mesh["nv_in"].astype(np.int32), cuda), dev(mesh["mf_in"].astype(np.int32), cuda)
+    nv_out = (nv_in // 4).to(torch.int32)
+    geometry = D.compute_triangle_geometry_(vertex, face)
+    out = D.mesh_decimation_(vertex, face, geometry, nv_in, mf_in, nv_out)
+    again = D.mesh_decimation_(vertex, face, geometry, nv_in, mf_in, nv_out)
+    for a, b in zip(out, again):
+        assert torch.equal(a, b)
+    v2, f2, g2, nv2, mf2, rep, vmap = out
+    Nv, Nv2 = vertex.shape[0], v2.shape[0]
+    assert int(nv2.sum()) == Nv2 and int(mf2.sum()) == f2.shape[0] and tuple(g2.shape) == (f2.shape[0], 5)
+    # every sample reaches its target (a few vertices below it: vertices that lose their last facet are dropped too)
+    assert bool((nv2 <= nv_in).all())
+    assert bool((nv2.double() <= nv_out.double()).all()) and bool((nv2.double() >= 0.99 * nv_out.double() - 8).all())
+    assert int(f2.min()) >= 0 and int(f2.max()) < Nv2
+    fl = f2.long()
+    assert not bool(((fl[:, 0] == fl[:, 1]) | (fl[:, 0] == fl[:, 2]) | (fl[:, 1] == fl[:, 2])).any())
+    r, m = rep.cpu().numpy().astype(np.int64), vmap.cpu().numpy().astype(np.int64)
+    contracted = r < 0
+    target = np.where(contracted, -r, np.arange(Nv))
+    assert np.all(r[target] >= 0)                                  # a representative is not contracted itself
+    assert np.array_equal(np.bincount(target, minlength=Nv)[~contracted] - 1, r[~contracted])   # member counts
+    assert np.all(m[contracted] == -1)
+    live = m >= 0
+    assert np.array_equal(np.sort(m[live]), np.arange(Nv2)) and np.all(np.diff(m[live]) > 0)   # ascending numbering
+    # pooling over the maps on a sample of coarse vertices
+    x = torch.randn(Nv, 8, device=cuda, generator=torch.Generator(device=cuda).manual_seed(3))
+    pooled = pool3d.maxPool(x, rep, vmap, v2)
+    coarse = m[target]                                             # coarse row of every input vertex (-1: dropped cluster)
+    rng = np.random.default_rng(4)
+    pick = rng.choice(Nv2, 300, replace=False)
+    xs = x.cpu().numpy()
+    order = np.argsort(coarse, kind="stable")
+    lo = np.searchsorted(coarse[order], pick, side="left")
+    hi = np.searchsorted(coarse[order], pick, side="right")
+    want = np.stack([xs[order[a:b]].max(0) for a, b in zip(lo, hi)])
+    assert np.array_equal(pooled[torch.from_numpy(pick).to(cuda)].cpu().numpy(), want)

@@ -102,15 +102,37 @@ def contraction_order(cost, edge_vi, nvIn_cumsum):
     return by_cost[by_sample.indices], by_sample.values
 
 
+_staging = {}
+
+
+def _pinned(name, n, dtype):
+    """A page-locked host buffer of at least ``n`` elements, kept between calls (the edge lists of a scene-scale batch
+    are tens of megabytes: through pageable memory their trip to the host costs more than the clustering itself)."""
+    buf = _staging.get(name)
+    if buf is None or buf.numel() < n or buf.dtype != dtype:
+        buf = torch.empty(max(n, 1), dtype=dtype, pin_memory=True)
+        _staging[name] = buf
+    return buf[:n]
+
+
 def cluster_vertices(edge_vi, edge_vj, sample, nvIn_cumsum, nv2Remove, Nv):
     """The two greedy passes per sample on the host (as the reference runs them): -> vt_replace int32 (Nv,) on the host."""
-    vi = np.ascontiguousarray(edge_vi.cpu().numpy(), dtype=np.int32)
-    vj = np.ascontiguousarray(edge_vj.cpu().numpy(), dtype=np.int32)
-    smp = sample.cpu().numpy()
+    n = edge_vi.shape[0]
+    B = nvIn_cumsum.shape[0]
+    # where each sample's edges begin: found on the device, so that the per-edge sample numbers stay there
+    bounds_d = torch.searchsorted(sample.contiguous(), torch.arange(B + 1, device=sample.device, dtype=sample.dtype))
+    if edge_vi.is_cuda:
+        vi_h, vj_h = _pinned("vi", n, I32), _pinned("vj", n, I32)
+        vi_h.copy_(edge_vi, non_blocking=True)
+        vj_h.copy_(edge_vj, non_blocking=True)
+        torch.cuda.current_stream(edge_vi.device).synchronize()
+    else:
+        vi_h, vj_h = edge_vi.contiguous(), edge_vj.contiguous()
+    vi, vj = vi_h.numpy(), vj_h.numpy()
+    bounds = bounds_d.cpu().numpy()
     ends = np.asarray(nvIn_cumsum.cpu().numpy(), dtype=np.int64)
     budget = np.asarray(nv2Remove.cpu().numpy(), dtype=np.int64)
-    vt_replace = np.zeros(Nv, dtype=np.int32)
-    bounds = np.searchsorted(smp, np.arange(len(ends) + 1))
+    vt_replace = np.zeros(Nv, dtype=np.int32)               # (ordinary memory: the passes access it at random)
     P = ctypes.c_void_p
     jobs = []
     for b in range(len(ends)):

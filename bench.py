@@ -628,11 +628,16 @@ def run_pcloud(args, torch):
     v0 = mesh["vertex"][keep[:nv[0]]]                             # (the first room: its points lie on the faces of a box)
     ext = v0.max(0) - v0.min(0)
     radius = float(np.sqrt(12.0 / np.pi / (len(v0) / max(2.0 * (ext[0] * ext[1] + ext[1] * ext[2] + ext[0] * ext[2]), 1e-9))))
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    nn_cnt, nn_idx, nn_dst, filt_idx, filt_coeff = PU.build_sphere_harmonics(xyz, xyz, NV, NV, radius, L=L, nn_uplimit=limit)
-    torch.cuda.synchronize()
-    graph_ms = (time.perf_counter() - t0) * 1e3
+    # the graph build (range search + kernel bins): the first call carries one-time costs, the median of five more is
+    # what a data pipeline pays per batch
+    graph_times = []
+    for _ in range(6):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        nn_cnt, nn_idx, nn_dst, filt_idx, filt_coeff = PU.build_sphere_harmonics(xyz, xyz, NV, NV, radius, L=L, nn_uplimit=limit)
+        torch.cuda.synchronize()
+        graph_times.append((time.perf_counter() - t0) * 1e3)
+    graph_cold_ms, graph_ms = graph_times[0], float(np.median(graph_times[1:]))
     Np, P, T = xyz.shape[0], nn_idx.shape[0], filt_idx.shape[1]
     gen = torch.Generator(device=dev).manual_seed(6000)
     x = torch.randn(Np, C, device=dev, generator=gen).requires_grad_(True)
@@ -679,7 +684,7 @@ def run_pcloud(args, torch):
         spent = time.perf_counter() - t0
         extra["cpu_baseline"] = dict(value=n0 / spent / 1e6, unit="Mpoints/s", cores=1, kind="port",
                                      sample="first sample (%d points, %d pairs), one fwd+bwd pass, %.1f s" % (n0, p0, spent))
-    return dict(value=Np / (ms * 1e-3) / 1e6, unit="Mpoints/s", ms_per_step=ms, graph_build_ms=graph_ms, **extra, dtype="f32",
+    return dict(value=Np / (ms * 1e-3) / 1e6, unit="Mpoints/s", ms_per_step=ms, graph_build_ms=graph_ms, graph_build_first_ms=graph_cold_ms, **extra, dtype="f32",
                 roofline=dict(bound="hbm", achieved=ach, peak=HBM_PEAK_GBS, unit="GB/s", frac=ach / HBM_PEAK_GBS,
                               traffic=measured_traffic("pcloud", "", dom) if args.scale == 1.0 else None, kernel=dom,
                               kernel_ms=per_op[dom]),

@@ -409,6 +409,30 @@ int pmesh_point_cube_count(const float *database, const float *query, const int3
 int pmesh_point_cube_fill(const float *database, const float *query, const int32_t *nv_database,
                           const int32_t *nv_query, int B, int64_t Np, int64_t Mp, float length, int grid_size,
                           const int64_t *cnt_info, int64_t Nout, int32_t *nn_index, pmesh_stream_t stream);
+/* The range and cube searches over a cell grid of the database points: the same outputs as the four functions above
+ * (which scan a query's whole sample, as nnquery_gpu.cu:20-250 does), at a cost that grows with the neighbours
+ * instead of the sample size.  pmesh_point_grid_build sorts the database points into cells at least `reach` wide
+ * (the radius of the range searches, half the edge of the cube searches that will use the grid; a search that
+ * reaches further still works, over more cells) and leaves the grid in `grid` (256-byte aligned,
+ * pmesh_point_grid_workspace_bytes(Np) bytes; Np > 0, B <= 2^20).  The *_grid searches take the grid and otherwise
+ * the arguments of their scanning counterparts. */
+size_t pmesh_point_grid_workspace_bytes(int64_t Np);
+int pmesh_point_grid_build(const float *database, const int32_t *nv_database, int B, int64_t Np, float reach,
+                           void *grid, size_t grid_bytes, pmesh_stream_t stream);
+int pmesh_point_range_count_grid(const void *grid, const float *database, const float *query,
+                                 const int32_t *nv_database, const int32_t *nv_query, int B, int64_t Np, int64_t Mp,
+                                 float radius, int nn_sample, int32_t *count, pmesh_stream_t stream);
+int pmesh_point_range_fill_grid(const void *grid, const float *database, const float *query,
+                                const int32_t *nv_database, const int32_t *nv_query, int B, int64_t Np, int64_t Mp,
+                                float radius, const int64_t *cnt_info, int64_t Nout, int32_t *nn_index, float *nn_dist,
+                                pmesh_stream_t stream);
+int pmesh_point_cube_count_grid(const void *grid, const float *database, const float *query,
+                                const int32_t *nv_database, const int32_t *nv_query, int B, int64_t Np, int64_t Mp,
+                                float length, int nn_sample, int32_t *count, pmesh_stream_t stream);
+int pmesh_point_cube_fill_grid(const void *grid, const float *database, const float *query,
+                               const int32_t *nv_database, const int32_t *nv_query, int B, int64_t Np, int64_t Mp,
+                               float length, int grid_size, const int64_t *cnt_info, int64_t Nout, int32_t *nn_index,
+                               pmesh_stream_t stream);
 /* three nearest neighbours (nnquery.cpp:132-171 "knn3", nnquery_gpu.cu:262-330): nn_index, nn_dist (Mp,3). */
 int pmesh_point_knn3(const float *database, const float *query, const int32_t *nv_database, const int32_t *nv_query,
                      int B, int64_t Np, int64_t Mp, int32_t *nn_index, float *nn_dist, pmesh_stream_t stream);

@@ -11,7 +11,7 @@ from ctypes import c_char_p, c_float, c_int, c_int64, c_size_t, c_void_p
 _HERE = os.path.dirname(os.path.abspath(__file__))
 # PICASSO_MESH_LIB points at an alternative build of the same ABI (kernel experiments)
 LIB_PATH = os.environ.get("PICASSO_MESH_LIB") or os.path.join(_HERE, "csrc", "libpicasso_mesh.so")
-ABI_VERSION = 16
+ABI_VERSION = 17
 
 P, I, L, Z = c_void_p, c_int, c_int64, c_size_t
 
@@ -38,6 +38,12 @@ SIGNATURES = {
     "pmesh_point_range_fill": (I, [P, P, P, P, I, L, L, ctypes.c_float, P, L, P, P, P]),
     "pmesh_point_cube_count": (I, [P, P, P, P, I, L, L, ctypes.c_float, I, P, P]),
     "pmesh_point_cube_fill": (I, [P, P, P, P, I, L, L, ctypes.c_float, I, P, L, P, P]),
+    "pmesh_point_grid_workspace_bytes": (Z, [L]),
+    "pmesh_point_grid_build": (I, [P, P, I, L, ctypes.c_float, P, Z, P]),
+    "pmesh_point_range_count_grid": (I, [P, P, P, P, P, I, L, L, ctypes.c_float, I, P, P]),
+    "pmesh_point_range_fill_grid": (I, [P, P, P, P, P, I, L, L, ctypes.c_float, P, L, P, P, P]),
+    "pmesh_point_cube_count_grid": (I, [P, P, P, P, P, I, L, L, ctypes.c_float, I, P, P]),
+    "pmesh_point_cube_fill_grid": (I, [P, P, P, P, P, I, L, L, ctypes.c_float, I, P, L, P, P]),
     "pmesh_point_knn3": (I, [P, P, P, P, I, L, L, P, P, P]),
     "pmesh_point_fps": (I, [P, P, P, I, L, L, P, P, P]),
     "pmesh_point_sph3d_kernel": (I, [P, P, P, P, L, L, L, I, I, I, ctypes.c_float, P, P]),

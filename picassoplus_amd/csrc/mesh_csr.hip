@@ -91,6 +91,15 @@ static size_t sort_temp_bytes(int64_t n, int bits)
     return bytes;
 }
 
+// the same stable sort for the other sources of the library (rows_internal.h)
+size_t sort_pairs_temp_bytes(int64_t n, int bits) { return sort_temp_bytes(n, bits); }
+hipError_t sort_pairs(void *temp, size_t temp_bytes, const unsigned *keys_in, unsigned *keys_out, const int *vals_in,
+                      int *vals_out, int64_t n, int bits, hipStream_t st)
+{
+    if (n <= 0) return hipSuccess;
+    return rocprim::radix_sort_pairs(temp, temp_bytes, keys_in, keys_out, vals_in, vals_out, (size_t)n, 0, bits, st);
+}
+
 static size_t csr_workspace(int64_t n, int64_t n_rows)
 {
     return 3 * align_up((size_t)n * 4) + align_up(sort_temp_bytes(n, key_bits(n_rows))) + 256;

@@ -792,15 +792,25 @@ __global__ __launch_bounds__(kBlock) void pool_max_bwd_scatter_k(const float *__
 // ----------------------------------------------------------------------------------------
 // real spherical-harmonic basis, degree <= 5, cartesian closed forms on the unit direction
 // ----------------------------------------------------------------------------------------
-__global__ __launch_bounds__(kBlock) void sph_harm_k(const float *__restrict__ xyz, float *__restrict__ out,
-                                                     int64_t N, int L)
+// (the degree is a compile-time constant so that a row stays in registers)
+template <int L>
+__global__ __launch_bounds__(kBlock) void sph_harm_k(const float *__restrict__ xyz, float *__restrict__ out, int64_t N)
 {
     const int64_t n = (int64_t)blockIdx.x * kBlock + threadIdx.x;
     if (n >= N) return;
-    const int B = (L + 1) * (L + 1);
-    float v[36];
+    constexpr int B = (L + 1) * (L + 1);
+    float v[B];
     sph_harm_at(xyz[3 * n], xyz[3 * n + 1], xyz[3 * n + 2], L, v);
     float *o = out + n * B;
+    if constexpr (B % 4 == 0) {
+        // (rows of 16 or 64 bytes times a multiple: aligned whenever the array is)
+        if ((reinterpret_cast<uintptr_t>(out) & 15u) == 0) {
+#pragma unroll
+            for (int i = 0; i < B; i += 4) *reinterpret_cast<float4 *>(o + i) = make_float4(v[i], v[i + 1], v[i + 2], v[i + 3]);
+            return;
+        }
+    }
+#pragma unroll
     for (int i = 0; i < B; ++i) o[i] = v[i];
 }
 
@@ -1274,7 +1284,16 @@ extern "C" int pmesh_sph_harm(const float *xyz, float *out, int64_t N, int L, pm
     if (N == 0) return 0;
     PM_REQUIRE(xyz && out, "sph_harm: null pointer");
     PM_REQUIRE(grid_ok(ceil_div(N, kBlock)), "sph_harm: grid too large");
-    sph_harm_k<<<dim3((unsigned)ceil_div(N, kBlock)), dim3(kBlock), 0, (hipStream_t)stream>>>(xyz, out, N, L);
+    const dim3 grid((unsigned)ceil_div(N, kBlock)), block(kBlock);
+    hipStream_t st = (hipStream_t)stream;
+    switch (L) {
+    case 0: sph_harm_k<0><<<grid, block, 0, st>>>(xyz, out, N); break;
+    case 1: sph_harm_k<1><<<grid, block, 0, st>>>(xyz, out, N); break;
+    case 2: sph_harm_k<2><<<grid, block, 0, st>>>(xyz, out, N); break;
+    case 3: sph_harm_k<3><<<grid, block, 0, st>>>(xyz, out, N); break;
+    case 4: sph_harm_k<4><<<grid, block, 0, st>>>(xyz, out, N); break;
+    default: sph_harm_k<5><<<grid, block, 0, st>>>(xyz, out, N); break;
+    }
     PM_LAUNCHED("sph_harm");
     return 0;
 }

@@ -8,6 +8,7 @@
 // Distances are compared in float32 with every operation rounded on its own (no fused multiply-add), so the integer
 // outputs do not depend on how a compiler contracts the expression.
 #include "common.h"
+#include "rows_internal.h"
 #include "../../include/picasso_mesh.h"
 #include <cmath>
 
@@ -103,6 +104,414 @@ __global__ __launch_bounds__(kBlock) void point_fill_k(const float *__restrict__
             nn_index[at * 3 + 2] = (xi * grid_size + yi) * grid_size + zi;
         }
         ++at;
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// The range and cube searches over a cell grid.  The scans above cost queries x sample size; here the database
+// points are sorted into cells at least as wide as the search reaches (radius, or half the cube's edge), so a
+// query looks at the 27 cells around its own.  The outputs are the scans': the same float32 test decides who is
+// a neighbour, and of a query's neighbours the nn_sample lowest database indices are kept, in ascending order (the
+// fill step inserts every neighbour it meets into the query's sorted output segment).
+//
+// One grid serves all samples: cell (b, x, y, z) of sample b over the bounding box of all finite database
+// coordinates; at most kGridMaxCells cells and kGridMaxAxis per axis, the cell edge h grows until that holds.
+// h >= 1.01 x reach, and a cell coordinate carries an error below 2 * kGridMaxAxis * 2^-23 cells, so two points
+// whose coordinates differ by less than the reach lie at most one cell apart on every axis; a search that reaches
+// further than the grid was built for widens its window instead.  Points that belong to no sample sort behind the
+// last cell; coordinates that are not finite never pass the distance test, whichever cell they fall into.
+constexpr int kGridMaxCells = 1 << 20;
+constexpr int kGridMaxAxis = 4096;
+constexpr int kGridKeyBits = 21;                        // keys 0 .. kGridMaxCells
+constexpr float kGridSlack = 1.01f;
+
+struct PointGrid {                                      // head of a grid workspace
+    float ox, oy, oz, inv_h;
+    int nx, ny, nz, cells;                              // cells per sample = nx * ny * nz
+    int lo[3], hi[3];                                   // bounding box, floats as order-preserving integers
+};
+constexpr size_t kGridHead = 256;
+static_assert(sizeof(PointGrid) <= kGridHead, "grid head");
+
+__device__ __forceinline__ int ordered_int(float f)
+{
+    const int i = __float_as_int(f);
+    return i >= 0 ? i : i ^ 0x7fffffff;
+}
+__device__ __forceinline__ float ordered_float(int i) { return __int_as_float(i >= 0 ? i : i ^ 0x7fffffff); }
+
+// empties the cells and the bounding box
+__global__ __launch_bounds__(kBlock) void grid_clear_k(PointGrid *__restrict__ G, int2 *__restrict__ cells)
+{
+    const int i = blockIdx.x * kBlock + threadIdx.x;
+    if (i < kGridMaxCells) cells[i] = make_int2(0, 0);
+    if (i == 0)
+        for (int a = 0; a < 3; ++a) { G->lo[a] = INT32_MAX; G->hi[a] = INT32_MIN; }
+}
+
+__device__ __forceinline__ bool finite3(float x, float y, float z) { return fabsf(x) < INFINITY && fabsf(y) < INFINITY && fabsf(z) < INFINITY; }
+
+constexpr int kBboxPer = 16;                            // points per thread of the bounding-box pass
+__global__ __launch_bounds__(kBlock) void grid_bbox_k(const float *__restrict__ db, const int *__restrict__ nvd, int B, int64_t Np,
+                                                      PointGrid *__restrict__ G)
+{
+    __shared__ int s_lo[3][kBlock / 64], s_hi[3][kBlock / 64];
+    int lo[3] = {INT32_MAX, INT32_MAX, INT32_MAX}, hi[3] = {INT32_MIN, INT32_MIN, INT32_MIN};
+    const int64_t n = B > 0 ? (nvd[B - 1] < Np ? nvd[B - 1] : Np) : 0;
+    const int64_t k0 = (int64_t)blockIdx.x * kBlock * kBboxPer + threadIdx.x;
+    for (int i = 0; i < kBboxPer; ++i) {
+        const int64_t k = k0 + (int64_t)i * kBlock;
+        if (k >= n) break;
+        const float x = db[k * 3], y = db[k * 3 + 1], z = db[k * 3 + 2];
+        if (!finite3(x, y, z)) continue;
+        const int v[3] = {ordered_int(x), ordered_int(y), ordered_int(z)};
+#pragma unroll
+        for (int a = 0; a < 3; ++a) {
+            lo[a] = v[a] < lo[a] ? v[a] : lo[a];
+            hi[a] = v[a] > hi[a] ? v[a] : hi[a];
+        }
+    }
+#pragma unroll
+    for (int a = 0; a < 3; ++a) {
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) {
+            const int l = __shfl_xor(lo[a], o, 64), h = __shfl_xor(hi[a], o, 64);
+            lo[a] = l < lo[a] ? l : lo[a];
+            hi[a] = h > hi[a] ? h : hi[a];
+        }
+        if ((threadIdx.x & 63) == 0) { s_lo[a][threadIdx.x >> 6] = lo[a]; s_hi[a][threadIdx.x >> 6] = hi[a]; }
+    }
+    __syncthreads();
+    if (threadIdx.x < 3) {
+        const int a = threadIdx.x;
+        int l = s_lo[a][0], h = s_hi[a][0];
+        for (int w = 1; w < kBlock / 64; ++w) {
+            l = s_lo[a][w] < l ? s_lo[a][w] : l;
+            h = s_hi[a][w] > h ? s_hi[a][w] : h;
+        }
+        if (l <= h) {
+            atomicMin(&G->lo[a], l);
+            atomicMax(&G->hi[a], h);
+        }
+    }
+}
+
+// origin, cell edge and cell counts from the bounding box (one thread)
+__global__ void grid_dims_k(PointGrid *__restrict__ G, int B, float reach)
+{
+    if (blockIdx.x || threadIdx.x) return;
+    float o[3] = {0.f, 0.f, 0.f}, ext[3] = {0.f, 0.f, 0.f};
+    for (int a = 0; a < 3; ++a)
+        if (G->lo[a] <= G->hi[a]) {
+            o[a] = ordered_float(G->lo[a]);
+            ext[a] = ordered_float(G->hi[a]) - o[a];
+        }
+    float h = reach * kGridSlack;
+    int n[3] = {1, 1, 1};
+    bool fits = false;
+    if (h > 0.f && h < INFINITY && finite3(ext[0], ext[1], ext[2]))
+        for (int it = 0; it < 400 && !fits && h < INFINITY; ++it) {
+            double total = (double)(B > 0 ? B : 1);
+            bool axis = true;
+            for (int a = 0; a < 3; ++a) {
+                const float c = floorf(ext[a] / h);
+                axis = axis && c < (float)kGridMaxAxis;
+                n[a] = (int)fminf(c, (float)kGridMaxAxis) + 1;
+                total *= (double)n[a];
+            }
+            fits = axis && total <= (double)kGridMaxCells;
+            if (!fits) h *= 1.26f;
+        }
+    if (!fits) {                                        // one cell per sample: every query looks at its whole sample
+        n[0] = n[1] = n[2] = 1;
+        G->inv_h = 0.f;
+    } else {
+        G->inv_h = 1.0f / h;
+    }
+    G->ox = o[0]; G->oy = o[1]; G->oz = o[2];
+    G->nx = n[0]; G->ny = n[1]; G->nz = n[2];
+    G->cells = n[0] * n[1] * n[2];
+}
+
+// cell coordinate of a database point, inside the grid whatever the value
+__device__ __forceinline__ int grid_coord(float p, float o, float inv_h, int n)
+{
+    float v = floorf((p - o) * inv_h);
+    v = fmaxf(v, 0.f);                                  // (also what a NaN becomes)
+    v = fminf(v, (float)(n - 1));
+    return (int)v;
+}
+
+__global__ __launch_bounds__(kBlock) void grid_keys_k(const float *__restrict__ db, const int *__restrict__ nvd, int B, int64_t Np,
+                                                      const PointGrid *__restrict__ G, unsigned *__restrict__ keys,
+                                                      int *__restrict__ ids)
+{
+    const int64_t k = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (k >= Np) return;
+    int b = 0;
+    while (b < B && k >= nvd[b]) ++b;
+    unsigned key = (unsigned)kGridMaxCells;
+    if (b < B) {
+        const int x = grid_coord(db[k * 3], G->ox, G->inv_h, G->nx), y = grid_coord(db[k * 3 + 1], G->oy, G->inv_h, G->ny),
+                  z = grid_coord(db[k * 3 + 2], G->oz, G->inv_h, G->nz);
+        key = (unsigned)(b * G->cells + (x * G->ny + y) * G->nz + z);
+    }
+    keys[k] = key;
+    ids[k] = (int)k;
+}
+
+// [first, last) sorted position of every occupied cell, and the sorted points as (x, y, z, database index)
+__global__ __launch_bounds__(kBlock) void grid_cells_k(const float *__restrict__ db, const unsigned *__restrict__ keys,
+                                                       const int *__restrict__ ids, int64_t Np, int2 *__restrict__ cells,
+                                                       float4 *__restrict__ pts)
+{
+    const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= Np) return;
+    const unsigned key = keys[i];
+    const int id = ids[i];
+    pts[i] = make_float4(db[(int64_t)id * 3], db[(int64_t)id * 3 + 1], db[(int64_t)id * 3 + 2], __int_as_float(id));
+    if (key >= (unsigned)kGridMaxCells) return;
+    if (i == 0 || keys[i - 1] != key) cells[key].x = (int)i;
+    if (i == Np - 1 || keys[i + 1] != key) cells[key].y = (int)i + 1;
+}
+
+// cells a query looks at on one axis: its own and `reach` cells to either side, cut to the grid (empty if c0 > c1)
+struct GridSpan {
+    int c0, c1;
+};
+__device__ __forceinline__ GridSpan grid_span(float q, float o, float inv_h, int n, int reach)
+{
+    float v = floorf((q - o) * inv_h);
+    v = fmaxf(v, -2.f - (float)reach);                  // (a NaN query ends up outside and finds nothing, as in the scan)
+    v = fminf(v, (float)(n + 1 + reach));
+    const int c = (int)v;
+    GridSpan s;
+    s.c0 = c - reach > 0 ? c - reach : 0;
+    s.c1 = c + reach < n - 1 ? c + reach : n - 1;
+    return s;
+}
+__device__ __forceinline__ int grid_reach(float size, int mode, float inv_h)
+{
+    const float need = (mode == 0 ? size : size / 2) * kGridSlack * inv_h - 1e-3f;
+    const float r = ceilf(fminf(need, (float)kGridMaxAxis));
+    return r > 1.f ? (int)r : 1;
+}
+
+// Visits the database points of sample b in the cells around (qx, qy, qz).  The (x, y) columns of those cells are dealt
+// out to the `lanes` lanes that share the query (`sub`: which of them I am); the cells of a column follow each other
+// in the sort order, so a column's points are one run, read four at a time.  f(point) returns false to stop this lane.
+template <int MODE, typename F>
+__device__ __forceinline__ void grid_visit(const PointGrid *__restrict__ G, const int2 *__restrict__ cells,
+                                           const float4 *__restrict__ pts, int b, float qx, float qy, float qz, float size,
+                                           int sub, int lanes, F f)
+{
+    const float inv_h = G->inv_h;
+    const int nx = G->nx, ny = G->ny, nz = G->nz, reach = grid_reach(size, MODE, inv_h);
+    const GridSpan sx = grid_span(qx, G->ox, inv_h, nx, reach), sy = grid_span(qy, G->oy, inv_h, ny, reach),
+                   sz = grid_span(qz, G->oz, inv_h, nz, reach);
+    if (sx.c0 > sx.c1 || sy.c0 > sy.c1 || sz.c0 > sz.c1) return;
+    const int wy = sy.c1 - sy.c0 + 1, ncol = (sx.c1 - sx.c0 + 1) * wy;
+    const int2 *mine = cells + (int64_t)b * G->cells;
+    for (int c = sub; c < ncol; c += lanes) {
+        const int x = sx.c0 + c / wy, y = sy.c0 + c % wy;
+        const int2 *col = mine + (x * ny + y) * nz;
+        int s = INT32_MAX, e = 0;
+        for (int z = sz.c0; z <= sz.c1; ++z) {
+            const int2 r = col[z];
+            if (r.y > r.x) {
+                s = r.x < s ? r.x : s;
+                e = r.y > e ? r.y : e;
+            }
+        }
+        for (int i = s; i < e; i += 4) {
+            float4 p[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) p[u] = pts[i + u < e ? i + u : e - 1];
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+                if (i + u < e && !f(p[u])) return;
+        }
+    }
+}
+
+__device__ __forceinline__ float sq_dist(float qx, float qy, float qz, const float4 &p, float &dx, float &dy, float &dz)
+{
+#pragma clang fp contract(off)
+    dx = p.x - qx;
+    dy = p.y - qy;
+    dz = p.z - qz;
+    return (dx * dx + dy * dy) + dz * dz;
+}
+
+// sample of query j and its index b
+__device__ __forceinline__ int sample_index(int64_t j, const int *__restrict__ nvq, int B)
+{
+    int b = 0;
+    while (b < B && j >= nvq[b]) ++b;
+    return b;
+}
+
+// kQLanes neighbouring lanes share a query: the searches are chains of dependent fetches (cell, then its points), and
+// a chip-wide grid of one thread per query would leave most of the latency uncovered.
+constexpr int kQLanes = 8;
+constexpr int kQPerBlock = kBlock / kQLanes;
+
+template <int MODE>
+__global__ __launch_bounds__(kBlock) void point_count_grid_k(const PointGrid *__restrict__ G, const int2 *__restrict__ cells,
+                                                             const float4 *__restrict__ pts, const float *__restrict__ query,
+                                                             const int *__restrict__ nvq, int B, int64_t Mp, float size,
+                                                             int nn_sample, int *__restrict__ count)
+{
+    const int64_t j = (int64_t)blockIdx.x * kQPerBlock + threadIdx.x / kQLanes;
+    const int sub = threadIdx.x % kQLanes;
+    const bool valid = j < Mp;
+    const int b = valid ? sample_index(j, nvq, B) : B;
+    int cnt = 0;
+    if (b < B) {
+        const float qx = query[j * 3], qy = query[j * 3 + 1], qz = query[j * 3 + 2];
+        grid_visit<MODE>(G, cells, pts, b, qx, qy, qz, size, sub, kQLanes, [&](const float4 &p) {
+            float dx, dy, dz;
+            const float d2 = sq_dist(qx, qy, qz, p, dx, dy, dz);
+            cnt += is_neighbour<MODE>(d2, dx, dy, dz, size) ? 1 : 0;
+            return cnt < nn_sample;
+        });
+    }
+    // (every lane of the wavefront is here: none has left the kernel)
+#pragma unroll
+    for (int o = 1; o < kQLanes; o <<= 1) {
+        const int other = __shfl_xor(cnt, o, 64);
+        cnt = (int)((int64_t)cnt + other < nn_sample ? cnt + other : nn_sample);
+    }
+    if (valid && sub == 0) count[j] = cnt;
+}
+
+// One lane's way to fill a query's segment, for the queries with more neighbours than the workgroup's buffers hold:
+// the database indices to keep are held sorted (in `seg`: the query's buffer if they fit, else its segment of nn_index)
+// while the neighbours come in; once all places are taken a neighbour replaces the largest index if it is lower.  The
+// other columns follow from the final indices.
+template <int MODE>
+__device__ void fill_by_insertion(const PointGrid *__restrict__ G, const int2 *__restrict__ cells, const float4 *__restrict__ pts,
+                                  const float *__restrict__ db, int b, int64_t j, float qx, float qy, float qz, int64_t Np,
+                                  float size, int grid_size, int64_t at, int64_t m, int *seg, int step, int *nn_index,
+                                  float *nn_dist)
+{
+#pragma clang fp contract(off)
+    constexpr int W = MODE == 0 ? 2 : 3;                // seg[step * t]: database index of the query's t-th pair so far
+    int64_t filled = 0;
+    int last = -1;                                      // the largest index kept so far
+    grid_visit<MODE>(G, cells, pts, b, qx, qy, qz, size, 0, 1, [&](const float4 &p) {
+        float dx, dy, dz;
+        const float d2 = sq_dist(qx, qy, qz, p, dx, dy, dz);
+        if (!is_neighbour<MODE>(d2, dx, dy, dz, size)) return true;
+        const int id = __float_as_int(p.w);
+        if (filled == m && id > last) return true;
+        const int64_t top = filled < m ? filled++ : m - 1;
+        int64_t pos = top;
+        int newlast = id;
+        while (pos > 0) {
+            const int prev = seg[step * (pos - 1)];
+            if (prev < id) break;
+            if (pos == top) newlast = prev;
+            seg[step * pos] = prev;
+            --pos;
+        }
+        seg[step * pos] = id;
+        last = newlast;
+        return true;
+    });
+    for (int64_t t = 0; t < filled; ++t) {
+        const int kept = seg[step * t];
+        const int id = kept < 0 ? 0 : (kept >= Np ? (int)Np - 1 : kept);
+        float dx, dy, dz;
+        const float d2 = sq_dist(qx, qy, qz, db + (int64_t)id * 3, dx, dy, dz);
+        nn_index[(at + t) * W] = (int)j;
+        nn_index[(at + t) * W + 1] = kept;
+        if constexpr (MODE == 0) {
+            nn_dist[at + t] = sqrtf(d2);
+        } else {
+            const float half = size / 2, cell = size / (float)grid_size;
+            const int xi = (int)((dx + half) / cell), yi = (int)((dy + half) / cell), zi = (int)((dz + half) / cell);
+            nn_index[(at + t) * W + 2] = (xi * grid_size + yi) * grid_size + zi;
+        }
+    }
+}
+
+// Pairs of query j at [cnt_info[j-1], cnt_info[j]): its lanes drop the neighbours they meet into a buffer of the
+// workgroup (database index; distance or kernel cell), then every neighbour finds its place by counting the lower
+// indices, and the first cnt_info[j] - cnt_info[j-1] places are written.
+constexpr int kFillCap = 128;
+template <int MODE>
+__global__ __launch_bounds__(kBlock) void point_fill_grid_k(const PointGrid *__restrict__ G, const int2 *__restrict__ cells,
+                                                            const float4 *__restrict__ pts, const float *__restrict__ db,
+                                                            const float *__restrict__ query, const int *__restrict__ nvq, int B,
+                                                            int64_t Np, int64_t Mp, float size, int grid_size,
+                                                            const int64_t *__restrict__ cnt_info, int64_t Nout,
+                                                            int *__restrict__ nn_index, float *__restrict__ nn_dist)
+{
+#pragma clang fp contract(off)
+    constexpr int W = MODE == 0 ? 2 : 3;
+    __shared__ int s_id[kQPerBlock][kFillCap + 1];
+    __shared__ unsigned s_val[kQPerBlock][kFillCap + 1];
+    __shared__ int s_cnt[kQPerBlock];
+    const int q = threadIdx.x / kQLanes, sub = threadIdx.x % kQLanes;
+    const int64_t j = (int64_t)blockIdx.x * kQPerBlock + q;
+    const bool valid = j < Mp;
+    const int b = valid ? sample_index(j, nvq, B) : B;
+    int64_t at = 0, m = 0;
+    float qx = 0.f, qy = 0.f, qz = 0.f;
+    if (b < B) {
+        int64_t end = cnt_info[j];
+        at = j ? cnt_info[j - 1] : 0;
+        if (at < 0) at = 0;
+        if (end > Nout) end = Nout;
+        m = end > at ? end - at : 0;
+        qx = query[j * 3]; qy = query[j * 3 + 1]; qz = query[j * 3 + 2];
+    }
+    if (sub == 0) s_cnt[q] = 0;
+    // (the lanes of a query sit in one wavefront)
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    if (m > 0)
+        grid_visit<MODE>(G, cells, pts, b, qx, qy, qz, size, sub, kQLanes, [&](const float4 &p) {
+            float dx, dy, dz;
+            const float d2 = sq_dist(qx, qy, qz, p, dx, dy, dz);
+            if (!is_neighbour<MODE>(d2, dx, dy, dz, size)) return true;
+            const int slot = atomicAdd(&s_cnt[q], 1);
+            if (slot < kFillCap) {
+                s_id[q][slot] = __float_as_int(p.w);
+                if constexpr (MODE == 0) {
+                    s_val[q][slot] = __float_as_uint(sqrtf(d2));
+                } else {
+                    const float half = size / 2, cell = size / (float)grid_size;
+                    const int xi = (int)((dx + half) / cell), yi = (int)((dy + half) / cell), zi = (int)((dz + half) / cell);
+                    s_val[q][slot] = (unsigned)((xi * grid_size + yi) * grid_size + zi);
+                }
+            }
+            return true;
+        });
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    if (m <= 0) return;
+    const int total = s_cnt[q];
+    if (total > kFillCap) {
+        if (sub == 0) {
+            const bool fits = m <= kFillCap;
+            fill_by_insertion<MODE>(G, cells, pts, db, b, j, qx, qy, qz, Np, size, grid_size, at, m,
+                                    fits ? &s_id[q][0] : nn_index + at * W + 1, fits ? 1 : W, nn_index, nn_dist);
+        }
+        return;
+    }
+    for (int e = sub; e < total; e += kQLanes) {
+        const int id = s_id[q][e];
+        int rank = 0;
+        for (int f = 0; f < total; ++f) rank += s_id[q][f] < id ? 1 : 0;
+        if (rank >= m) continue;
+        nn_index[(at + rank) * W] = (int)j;
+        nn_index[(at + rank) * W + 1] = id;
+        if constexpr (MODE == 0) nn_dist[at + rank] = __uint_as_float(s_val[q][e]);
+        else nn_index[(at + rank) * W + 2] = (int)s_val[q][e];
     }
 }
 
@@ -328,6 +737,119 @@ extern "C" int pmesh_point_cube_fill(const float *database, const float *query, 
     PM_REQUIRE(cnt_info && nn_index, "point_cube_fill: null pointer");
     point_fill_k<1><<<dim3((unsigned)ceil_div(Mp, kBlock)), dim3(kBlock), 0, (hipStream_t)stream>>>(
         database, query, nv_database, nv_query, B, Np, Mp, length, grid_size, cnt_info, Nout, nn_index, nullptr);
+    PM_LAUNCHED("point_cube_fill");
+    return 0;
+}
+
+// grid workspace: head, cells, sorted points, then the sort's buffers (keys in/out, ids in/out, temporary storage)
+static size_t grid_slot(int64_t Np) { return (((size_t)Np * 4) + 255) & ~size_t(255); }
+static size_t grid_search_bytes(int64_t Np) { return kGridHead + (size_t)kGridMaxCells * sizeof(int2) + 4 * grid_slot(Np); }
+
+extern "C" size_t pmesh_point_grid_workspace_bytes(int64_t Np)
+{
+    if (Np < 0) Np = 0;
+    return grid_search_bytes(Np) + 4 * grid_slot(Np) + ((sort_pairs_temp_bytes(Np, kGridKeyBits) + 255) & ~size_t(255));
+}
+
+extern "C" int pmesh_point_grid_build(const float *database, const int32_t *nv_database, int B, int64_t Np, float reach,
+                                      void *grid, size_t grid_bytes, pmesh_stream_t stream)
+{
+    clear_error();
+    PM_REQUIRE(B > 0 && B <= kGridMaxCells && Np > 0 && Np <= INT32_MAX, "point_grid_build: bad sizes");
+    PM_REQUIRE(reach > 0, "point_grid_build: the reach of the searches must be positive");
+    PM_REQUIRE(database && nv_database && grid, "point_grid_build: null pointer");
+    PM_REQUIRE(((uintptr_t)grid & 255) == 0, "point_grid_build: the workspace must be aligned to 256 bytes");
+    PM_REQUIRE(grid_bytes >= pmesh_point_grid_workspace_bytes(Np), "point_grid_build: workspace too small (%zu bytes)", grid_bytes);
+    hipStream_t st = (hipStream_t)stream;
+    char *base = (char *)grid;
+    PointGrid *G = (PointGrid *)base;
+    int2 *cells = (int2 *)(base + kGridHead);
+    float4 *pts = (float4 *)(base + kGridHead + (size_t)kGridMaxCells * sizeof(int2));
+    char *sortb = base + grid_search_bytes(Np);
+    const size_t slot = grid_slot(Np);
+    unsigned *keys_in = (unsigned *)sortb, *keys_out = (unsigned *)(sortb + slot);
+    int *ids_in = (int *)(sortb + 2 * slot), *ids_out = (int *)(sortb + 3 * slot);
+    void *temp = sortb + 4 * slot;
+    const unsigned pb = (unsigned)ceil_div(Np, kBlock);
+    grid_clear_k<<<dim3(kGridMaxCells / kBlock), dim3(kBlock), 0, st>>>(G, cells);
+    grid_bbox_k<<<dim3((unsigned)ceil_div(Np, (int64_t)kBlock * kBboxPer)), dim3(kBlock), 0, st>>>(database, nv_database, B, Np, G);
+    grid_dims_k<<<dim3(1), dim3(64), 0, st>>>(G, B, reach);
+    grid_keys_k<<<dim3(pb), dim3(kBlock), 0, st>>>(database, nv_database, B, Np, G, keys_in, ids_in);
+    PM_LAUNCHED("point_grid_build");
+    const hipError_t e = sort_pairs(temp, sort_pairs_temp_bytes(Np, kGridKeyBits), keys_in, keys_out, ids_in, ids_out, Np,
+                                    kGridKeyBits, st);
+    PM_REQUIRE(e == hipSuccess, "point_grid_build: radix sort failed: %s", hipGetErrorString(e));
+    grid_cells_k<<<dim3(pb), dim3(kBlock), 0, st>>>(database, keys_out, ids_out, Np, cells, pts);
+    PM_LAUNCHED("point_grid_build");
+    return 0;
+}
+
+#define PM_GRID_PARTS(name)                                                                                             \
+    PM_REQUIRE(grid && Np > 0, name ": no grid");                                                                       \
+    const PointGrid *G = (const PointGrid *)grid;                                                                       \
+    const int2 *cells = (const int2 *)((const char *)grid + kGridHead);                                                 \
+    const float4 *pts = (const float4 *)((const char *)grid + kGridHead + (size_t)kGridMaxCells * sizeof(int2))
+
+extern "C" int pmesh_point_range_count_grid(const void *grid, const float *database, const float *query,
+                                            const int32_t *nv_database, const int32_t *nv_query, int B, int64_t Np, int64_t Mp,
+                                            float radius, int nn_sample, int32_t *count, pmesh_stream_t stream)
+{
+    clear_error();
+    PM_REQUIRE(radius > 0 && nn_sample > 0, "point_range_count: radius and nn_sample must be positive");
+    PM_QUERY_DIMS("point_range_count");
+    PM_REQUIRE(count, "point_range_count: null pointer");
+    PM_GRID_PARTS("point_range_count");
+    point_count_grid_k<0><<<dim3((unsigned)ceil_div(Mp, kQPerBlock)), dim3(kBlock), 0, (hipStream_t)stream>>>(
+        G, cells, pts, query, nv_query, B, Mp, radius, nn_sample, count);
+    PM_LAUNCHED("point_range_count");
+    return 0;
+}
+
+extern "C" int pmesh_point_range_fill_grid(const void *grid, const float *database, const float *query,
+                                           const int32_t *nv_database, const int32_t *nv_query, int B, int64_t Np, int64_t Mp,
+                                           float radius, const int64_t *cnt_info, int64_t Nout, int32_t *nn_index, float *nn_dist,
+                                           pmesh_stream_t stream)
+{
+    clear_error();
+    PM_REQUIRE(radius > 0 && Nout >= 0, "point_range_fill: bad arguments");
+    PM_QUERY_DIMS("point_range_fill");
+    if (Nout == 0) return 0;
+    PM_REQUIRE(cnt_info && nn_index && nn_dist, "point_range_fill: null pointer");
+    PM_GRID_PARTS("point_range_fill");
+    point_fill_grid_k<0><<<dim3((unsigned)ceil_div(Mp, kQPerBlock)), dim3(kBlock), 0, (hipStream_t)stream>>>(
+        G, cells, pts, database, query, nv_query, B, Np, Mp, radius, 1, cnt_info, Nout, nn_index, nn_dist);
+    PM_LAUNCHED("point_range_fill");
+    return 0;
+}
+
+extern "C" int pmesh_point_cube_count_grid(const void *grid, const float *database, const float *query,
+                                           const int32_t *nv_database, const int32_t *nv_query, int B, int64_t Np, int64_t Mp,
+                                           float length, int nn_sample, int32_t *count, pmesh_stream_t stream)
+{
+    clear_error();
+    PM_REQUIRE(length > 0 && nn_sample > 0, "point_cube_count: length and nn_sample must be positive");
+    PM_QUERY_DIMS("point_cube_count");
+    PM_REQUIRE(count, "point_cube_count: null pointer");
+    PM_GRID_PARTS("point_cube_count");
+    point_count_grid_k<1><<<dim3((unsigned)ceil_div(Mp, kQPerBlock)), dim3(kBlock), 0, (hipStream_t)stream>>>(
+        G, cells, pts, query, nv_query, B, Mp, length, nn_sample, count);
+    PM_LAUNCHED("point_cube_count");
+    return 0;
+}
+
+extern "C" int pmesh_point_cube_fill_grid(const void *grid, const float *database, const float *query,
+                                          const int32_t *nv_database, const int32_t *nv_query, int B, int64_t Np, int64_t Mp,
+                                          float length, int grid_size, const int64_t *cnt_info, int64_t Nout, int32_t *nn_index,
+                                          pmesh_stream_t stream)
+{
+    clear_error();
+    PM_REQUIRE(length > 0 && grid_size > 0 && Nout >= 0, "point_cube_fill: bad arguments");
+    PM_QUERY_DIMS("point_cube_fill");
+    if (Nout == 0) return 0;
+    PM_REQUIRE(cnt_info && nn_index, "point_cube_fill: null pointer");
+    PM_GRID_PARTS("point_cube_fill");
+    point_fill_grid_k<1><<<dim3((unsigned)ceil_div(Mp, kQPerBlock)), dim3(kBlock), 0, (hipStream_t)stream>>>(
+        G, cells, pts, database, query, nv_query, B, Np, Mp, length, grid_size, cnt_info, Nout, nn_index, nullptr);
     PM_LAUNCHED("point_cube_fill");
     return 0;
 }

@@ -23,4 +23,10 @@ int f2v_bwd_mfma(const void *gout, const void *in, const float *filt, const floa
                  const int *nfcount, const int *vtmap, void *gin, float *partial, int G, int64_t Nf, int64_t NvOut,
                  int C, int r, hipStream_t st, bool bf16 = false);
 
+// Stable radix sort of (32-bit key, id) pairs on the low `bits` bits of the keys (mesh_csr.hip); `temp` holds
+// sort_pairs_temp_bytes(n, bits) bytes.
+size_t sort_pairs_temp_bytes(int64_t n, int bits);
+hipError_t sort_pairs(void *temp, size_t temp_bytes, const unsigned *keys_in, unsigned *keys_out, const int *vals_in,
+                      int *vals_out, int64_t n, int bits, hipStream_t st);
+
 }  // namespace pmesh

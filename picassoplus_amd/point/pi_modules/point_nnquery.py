@@ -21,6 +21,12 @@ def _dims(database, query, nv_database, nv_query):
     return database.shape[0], query.shape[0], nv_database.shape[0], same_device(database, query, nv_database, nv_query)
 
 
+# Databases of at least this many points are searched through a cell grid (same outputs; the cost of a query then
+# grows with its neighbours, not with its sample), smaller ones by the scan over the query's sample.
+GRID_MIN_POINTS = 2048
+GRID_MAX_SAMPLES = 1 << 20
+
+
 def _search(kind, database, query, nv_database, nv_query, size, nn_sample, grid_size=None):
     Np, Mp, B, dev = _dims(database, query, nv_database, nv_query)
     if not nn_sample > 0:
@@ -30,16 +36,24 @@ def _search(kind, database, query, nv_database, nv_query, size, nn_sample, grid_
     args = (database.data_ptr(), query.data_ptr(), nv_database.data_ptr(), nv_query.data_ptr(), B, Np, Mp, float(size))
     with torch.cuda.device(dev):
         count = torch.zeros(Mp, dtype=I32, device=dev)
-        _lib.call("pmesh_point_%s_count" % kind, *args, nn_sample, count.data_ptr(), st)
+        if Mp and Np >= max(GRID_MIN_POINTS, 1) and 0 < B <= GRID_MAX_SAMPLES:
+            grid = torch.empty(_lib.query("pmesh_point_grid_workspace_bytes", Np), dtype=torch.uint8, device=dev)
+            _lib.call("pmesh_point_grid_build", database.data_ptr(), nv_database.data_ptr(), B, Np,
+                      float(size) if kind == "range" else float(size) / 2, grid.data_ptr(), grid.numel(), st)
+            args = (grid.data_ptr(),) + args
+            kind_fn = kind + "_%s_grid"
+        else:
+            kind_fn = kind + "_%s"
+        _lib.call("pmesh_point_" + kind_fn % "count", *args, nn_sample, count.data_ptr(), st)
         cnt_info = torch.cumsum(count, 0, dtype=torch.int64)
         n_out = int(cnt_info[-1]) if Mp else 0                   # the pair arrays are sized on the host, as in the reference
         width = 2 if kind == "range" else 3
         nn_index = torch.empty((n_out, width), dtype=I32, device=dev)
         if kind == "range":
             nn_dist = torch.empty(n_out, dtype=F32, device=dev)
-            _lib.call("pmesh_point_range_fill", *args, cnt_info.data_ptr(), n_out, nn_index.data_ptr(), nn_dist.data_ptr(), st)
+            _lib.call("pmesh_point_" + kind_fn % "fill", *args, cnt_info.data_ptr(), n_out, nn_index.data_ptr(), nn_dist.data_ptr(), st)
             return cnt_info, nn_index, nn_dist
-        _lib.call("pmesh_point_cube_fill", *args, int(grid_size), cnt_info.data_ptr(), n_out, nn_index.data_ptr(), st)
+        _lib.call("pmesh_point_" + kind_fn % "fill", *args, int(grid_size), cnt_info.data_ptr(), n_out, nn_index.data_ptr(), st)
         return cnt_info, nn_index
 
 

@@ -33,8 +33,10 @@ def n(t):
 @pytest.mark.parametrize("sizes,frac,radius,limit", [([300, 1, 120], 0.4, 0.2, None), ([2000, 1500], 1.0, 0.12, None),
                                                      ([500], 0.5, 0.3, 7), ([64, 64, 64, 64, 64], 1.0, 0.5, 1),
                                                      ([4000], 0.25, 0.05, None)])
-def test_range_cube_knn_bit_exact(cuda, sizes, frac, radius, limit):
-    say("case point search", sizes, frac, radius, limit)
+@pytest.mark.parametrize("grid", [False, True])
+def test_range_cube_knn_bit_exact(cuda, monkeypatch, sizes, frac, radius, limit, grid):
+    say("case point search", sizes, frac, radius, limit, "grid" if grid else "scan")
+    monkeypatch.setattr(point_nnquery, "GRID_MIN_POINTS", 0 if grid else 1 << 40)
     db, nvd = cloud(21, sizes)
     q, nvq = (db, nvd) if frac == 1.0 else subsample(22, db, nvd, frac)
     D, Q, ND, NQ = dev(db, cuda), dev(q, cuda), dev(nvd, cuda), dev(nvq, cuda)
@@ -53,6 +55,81 @@ def test_range_cube_knn_bit_exact(cuda, sizes, frac, radius, limit):
     wide = torch.cat([D, torch.ones_like(D)], 1)
     again = nnquery.range_search_(wide, Q, ND, NQ, radius=radius, nnsample=limit)
     assert torch.equal(again[2], nnquery.range_search_(D, Q, ND, NQ, radius=radius, nnsample=limit)[2])
+
+
+def _searches(D, Q, ND, NQ, radius, limit):
+    a = nnquery.range_search_(D, Q, ND, NQ, radius=radius, nnsample=limit)
+    b = nnquery.cube_search_(D, Q, ND, NQ, length=2 * radius, nnsample=limit, gridsize=4)
+    return [n(t) for t in a + b]
+
+
+@pytest.mark.parametrize("shape", ["plane", "far", "same", "spread", "nonfinite", "outside", "dense", "dense_all"])
+def test_grid_search_matches_scan(cuda, monkeypatch, shape):
+    """The cell-grid searches return what the scans return (which the test above holds against the oracle), also where
+    the grid degenerates: no extent on an axis, coordinates far from the origin (coarse float spacing), all points
+    equal, an extent so large that the cells grow, coordinates that are not finite, queries outside the database's
+    bounding box, more neighbours than the limit keeps (the lowest indices must survive, in order), and more neighbours
+    per query than the search kernel buffers, all of them kept."""
+    say("case grid search", shape)
+    rng = np.random.default_rng(77)
+    sizes, radius, limit = ([500, 300] if shape == "dense_all" else [1500, 900]), 0.15, None
+    db, nvd = cloud(31, sizes)
+    q, nvq = subsample(32, db, nvd, 0.5)
+    if shape == "plane":
+        db[:, 2] = 0.25
+        q[:, 2] = 0.25
+    elif shape == "far":
+        db += np.float32(4096.0)
+        q += np.float32(4096.0)
+    elif shape == "same":
+        db[:] = db[0]
+        q[:] = db[0]
+        limit = 40
+    elif shape == "spread":
+        db[::50] *= np.float32(3.0e6)
+    elif shape == "nonfinite":
+        db[5] = np.nan
+        db[17, 1] = np.inf
+        db[400, 0] = -np.inf
+        q[3] = np.nan
+        q[9, 2] = np.inf
+    elif shape == "outside":
+        q = (q + rng.uniform(-2.0, 2.0, q.shape)).astype(np.float32)
+    elif shape == "dense":
+        radius, limit = 0.6, 9
+    elif shape == "dense_all":
+        radius = 0.6
+    D, Q, ND, NQ = dev(db, cuda), dev(q, cuda), dev(nvd, cuda), dev(nvq, cuda)
+    monkeypatch.setattr(point_nnquery, "GRID_MIN_POINTS", 1 << 40)
+    want = _searches(D, Q, ND, NQ, radius, limit)
+    monkeypatch.setattr(point_nnquery, "GRID_MIN_POINTS", 0)
+    got = _searches(D, Q, ND, NQ, radius, limit)
+    assert want[0][-1] > 0 or shape == "nonfinite"
+    for a, b in zip(want, got):
+        assert a.dtype == b.dtype and np.array_equal(a, b, equal_nan=True)
+
+
+def test_grid_search_beyond_the_reach_it_was_built_for(cuda):
+    """A search that reaches further than the cells are wide looks at more cells: through the C-ABI, a grid built for a
+    tenth of the radius."""
+    from picassoplus_amd import _lib
+    db, nvd = cloud(41, [1200])
+    D, ND = dev(db, cuda), dev(np.cumsum(nvd).astype(np.int32), cuda)
+    Np, radius = db.shape[0], 0.2
+    ws = torch.empty(_lib.query("pmesh_point_grid_workspace_bytes", Np), dtype=torch.uint8, device=cuda)
+    _lib.call("pmesh_point_grid_build", D.data_ptr(), ND.data_ptr(), 1, Np, radius / 10, ws.data_ptr(), ws.numel(), None)
+    count = torch.zeros(Np, dtype=I32, device=cuda)
+    _lib.call("pmesh_point_range_count_grid", ws.data_ptr(), D.data_ptr(), D.data_ptr(), ND.data_ptr(), ND.data_ptr(), 1, Np, Np,
+              radius, 2147483647, count.data_ptr(), None)
+    w = P.range_search(db, db, np.cumsum(nvd), np.cumsum(nvd), radius, 2147483647)
+    assert np.array_equal(n(count), w[1])
+    cnt_info = torch.cumsum(count, 0, dtype=torch.int64)
+    n_out = int(cnt_info[-1])
+    nn_index = torch.empty((n_out, 2), dtype=I32, device=cuda)
+    nn_dist = torch.empty(n_out, dtype=F32, device=cuda)
+    _lib.call("pmesh_point_range_fill_grid", ws.data_ptr(), D.data_ptr(), D.data_ptr(), ND.data_ptr(), ND.data_ptr(), 1, Np, Np,
+              radius, cnt_info.data_ptr(), n_out, nn_index.data_ptr(), nn_dist.data_ptr(), None)
+    assert np.array_equal(n(nn_index), w[2]) and np.array_equal(n(nn_dist), w[3])
 
 
 @pytest.mark.parametrize("sizes,keep", [([120, 60], [15, 60]), ([3000], [700]), ([1, 5, 2048], [1, 3, 256])])

@@ -6,8 +6,9 @@
 // ops, by database point for the input gradients, so each output row is written once, by one lane group, in a fixed
 // order.  The filter gradient is summed per workgroup (one column per thread, pairs in ascending order; bins in
 // registers up to 64 of them, in LDS beyond) and the workgroups' partial results are added in a fixed tree order.
-// With at most 32 bins, depth multiplier 1 and at most 256 channels, forward and input gradient keep the filter in
-// registers and read the pairs' coefficients from a dense per-pair table in LDS.
+// With at most 36 bins, depth multiplier 1 and at most 256 channels, forward and input gradient keep the filter in
+// registers and read the pairs' coefficients from a dense per-pair table in LDS (instances for 16, 20, 32 and 36 bins:
+// a kernel's cost follows the instance's bins, not the filter's).
 //
 //   w[p, co]        = sum_t coeff[p, t] * filter[bin[p, t], co]           (plain form: one bin, weight 1)
 //   out[o, co]      = (1 / nn_count[o]) sum_{p = (o, i)} in[i, co / r] * w[p, co]
@@ -116,6 +117,29 @@ __global__ __launch_bounds__(kBlock) void point_conv_bwd_in_k(const float *__res
     }
 }
 
+// Adds the coefficients of pair p's T entries to its row of a dense table cm[bin] in LDS (entries in ascending order).
+// The entries are fetched eight at a time before the first of them is added: one thread walks a pair, and a fetch per
+// step of the walk would leave it waiting T times in a row.
+__device__ __forceinline__ void pair_row_to_table(const PairGraph &g, int64_t p, float *row)
+{
+    const int T = g.T;
+    const int *bi = g.bin_index + p * T;
+    const float *bc = g.bin_coeff ? g.bin_coeff + p * T : nullptr;
+    for (int t0 = 0; t0 < T; t0 += 8) {
+        int b[8];
+        float cf[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int t = t0 + u < T ? t0 + u : T - 1;          // (no branch around a fetch; the surplus is dropped below)
+            b[u] = bi[t];
+            cf[u] = bc ? bc[t] : 1.f;
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+            if (t0 + u < T && b[u] >= 0 && b[u] < g.F) row[b[u]] += cf[u];
+    }
+}
+
 // Forward (MODE 0: rows = queries, the other end of a pair is a database row of `src` = in) and input gradient (MODE 1:
 // rows = database points, the other end a query row of `src` = gout, weighted by 1 / nn_count of that query) for at most
 // FB bins, depth multiplier 1 and rows of at most 256 channels in four-channel pieces: a lane keeps its four columns of
@@ -159,36 +183,44 @@ __global__ __launch_bounds__(kBlock) void point_conv_rows_dense_k(const float *_
             const bool ok = other >= 0 && other < nother;
             s_other[threadIdx.x] = ok ? other : -1;
             s_scale[threadIdx.x] = (MODE == 1 && ok) ? inv_count(g.nn_count, o) : 1.f;
-            if (ok)
-                for (int t = 0; t < g.T; ++t) {
-                    const int b = g.bin_index[p * g.T + t];
-                    if (b >= 0 && b < g.F) s_cm[threadIdx.x][b] += g.bin_coeff ? g.bin_coeff[p * g.T + t] : 1.f;
-                }
+            if (ok) pair_row_to_table(g, p, s_cm[threadIdx.x]);
         }
         __syncthreads();
         if (!live) continue;
         const int a = e0 > cb ? e0 : cb, b = e1 < cb + NP ? e1 : cb + NP;
-        for (int e = a; e < b; ++e) {
-            const int q = e - cb, other = s_other[q];
-            if (other < 0) continue;
-            const float4 x = *reinterpret_cast<const float4 *>(src + (int64_t)other * C + c);      // (asked for before the weight is formed)
-            float w[4] = {0.f, 0.f, 0.f, 0.f};
+        for (int e4 = a; e4 < b; e4 += 4) {
+            // the rows of four pairs are asked for before the first weight is formed (the sums stay in pair order)
+            float4 x[4];
+            bool ok[4];
 #pragma unroll
-            for (int f4 = 0; f4 < FB; f4 += 4) {
-                const float4 m = *reinterpret_cast<const float4 *>(&s_cm[q][f4]);
-#pragma unroll
-                for (int u = 0; u < 4; ++u) {
-                    w[u] = fmaf(m.x, fr[f4][u], w[u]);
-                    w[u] = fmaf(m.y, fr[f4 + 1][u], w[u]);
-                    w[u] = fmaf(m.z, fr[f4 + 2][u], w[u]);
-                    w[u] = fmaf(m.w, fr[f4 + 3][u], w[u]);
-                }
+            for (int k = 0; k < 4; ++k) {
+                const int other = e4 + k < b ? s_other[e4 + k - cb] : -1;
+                ok[k] = other >= 0;
+                x[k] = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (ok[k]) x[k] = *reinterpret_cast<const float4 *>(src + (int64_t)other * C + c);
             }
-            const float sc = s_scale[q];
-            acc[0] = fmaf(x.x * w[0], sc, acc[0]);
-            acc[1] = fmaf(x.y * w[1], sc, acc[1]);
-            acc[2] = fmaf(x.z * w[2], sc, acc[2]);
-            acc[3] = fmaf(x.w * w[3], sc, acc[3]);
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                if (!ok[k]) continue;
+                const int q = e4 + k - cb;
+                float w[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int f4 = 0; f4 < FB; f4 += 4) {
+                    const float4 m = *reinterpret_cast<const float4 *>(&s_cm[q][f4]);
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) {
+                        w[u] = fmaf(m.x, fr[f4][u], w[u]);
+                        w[u] = fmaf(m.y, fr[f4 + 1][u], w[u]);
+                        w[u] = fmaf(m.z, fr[f4 + 2][u], w[u]);
+                        w[u] = fmaf(m.w, fr[f4 + 3][u], w[u]);
+                    }
+                }
+                const float sc = s_scale[q];
+                acc[0] = fmaf(x[k].x * w[0], sc, acc[0]);
+                acc[1] = fmaf(x[k].y * w[1], sc, acc[1]);
+                acc[2] = fmaf(x[k].z * w[2], sc, acc[2]);
+                acc[3] = fmaf(x[k].w * w[3], sc, acc[3]);
+            }
         }
     }
     if (live) {
@@ -256,11 +288,7 @@ __global__ __launch_bounds__(256) void point_conv_bwd_filt_dense_k(const float *
             s_o[threadIdx.x] = o;
             s_i[threadIdx.x] = i;
             s_inv[threadIdx.x] = o >= 0 ? inv_count(g.nn_count, o) : 0.f;
-            if (o >= 0)
-                for (int t = 0; t < g.T; ++t) {
-                    const int b = g.bin_index[p * g.T + t];
-                    if (b >= 0 && b < g.F) s_cm[threadIdx.x][b] += g.bin_coeff ? g.bin_coeff[p * g.T + t] : 1.f;
-                }
+            if (o >= 0) pair_row_to_table(g, p, s_cm[threadIdx.x]);
         }
         __syncthreads();
         if (!mine) continue;
@@ -427,7 +455,7 @@ static int filt_blocks(int64_t Nout, int F, int CR)
 {
     int64_t G = ceil_div(Nout, 256);
     if (G < 1) G = 1;
-    if (G > 1024) G = 1024;
+    if (G > 4096) G = 4096;
     const int64_t per = (int64_t)F * CR * 4;
     while (G > 1 && G * per > (int64_t(64) << 20)) G /= 2;
     return (int)G;
@@ -463,12 +491,14 @@ extern "C" int pmesh_point_conv_fwd(const float *input, const float *filter, con
     hipStream_t st = (hipStream_t)stream;
     const PairGraph g = {nn_index, nn_count, bin_index, bin_coeff, Np, Mp, Nout, T, F};
     const int CR = C * r;
-    if (r == 1 && C % 4 == 0 && C <= 256 && F <= 32 && aligned16(input) && aligned16(filter) && aligned16(output)) {
+    if (r == 1 && C % 4 == 0 && C <= 256 && F <= 36 && aligned16(input) && aligned16(filter) && aligned16(output)) {
         const RowShape rs = row_shape(C / 4);
         const int64_t blocks = ceil_div(Mp, rs.rpb);
         PM_REQUIRE(grid_ok(blocks), "grid too large");
         if (F <= 16) point_conv_rows_dense_k<16, 0><<<dim3((unsigned)blocks), dim3(kBlock), 0, st>>>(input, filter, g, rowptr, order, output, C, rs.lpr_log2);
-        else point_conv_rows_dense_k<32, 0><<<dim3((unsigned)blocks), dim3(kBlock), 0, st>>>(input, filter, g, rowptr, order, output, C, rs.lpr_log2);
+        else if (F <= 20) point_conv_rows_dense_k<20, 0><<<dim3((unsigned)blocks), dim3(kBlock), 0, st>>>(input, filter, g, rowptr, order, output, C, rs.lpr_log2);
+        else if (F <= 32) point_conv_rows_dense_k<32, 0><<<dim3((unsigned)blocks), dim3(kBlock), 0, st>>>(input, filter, g, rowptr, order, output, C, rs.lpr_log2);
+        else point_conv_rows_dense_k<36, 0><<<dim3((unsigned)blocks), dim3(kBlock), 0, st>>>(input, filter, g, rowptr, order, output, C, rs.lpr_log2);
     } else if (r == 1 && C % 4 == 0 && aligned16(input) && aligned16(filter) && aligned16(output))
         PM_ROW_LAUNCH(point_conv_fwd_k<4>, Mp, CR / 4, input, filter, g, rowptr, order, output, C, r);
     else
@@ -504,12 +534,14 @@ extern "C" int pmesh_point_conv_bwd(const float *grad_output, const float *input
     const PairGraph g = {nn_index, nn_count, bin_index, bin_coeff, Np, Mp, Nout, T, F};
     if (grad_input) {
         PM_REQUIRE(rowptr_in && order_in, "point_conv_bwd: the input gradient needs the pairs sorted by database point");
-        if (r == 1 && C % 4 == 0 && C <= 256 && F <= 32 && aligned16(grad_output) && aligned16(filter) && aligned16(grad_input)) {
+        if (r == 1 && C % 4 == 0 && C <= 256 && F <= 36 && aligned16(grad_output) && aligned16(filter) && aligned16(grad_input)) {
             const RowShape rs = row_shape(C / 4);
             const int64_t blocks = ceil_div(Np, rs.rpb);
             PM_REQUIRE(grid_ok(blocks), "grid too large");
             if (F <= 16) point_conv_rows_dense_k<16, 1><<<dim3((unsigned)blocks), dim3(kBlock), 0, st>>>(grad_output, filter, g, rowptr_in, order_in, grad_input, C, rs.lpr_log2);
-            else point_conv_rows_dense_k<32, 1><<<dim3((unsigned)blocks), dim3(kBlock), 0, st>>>(grad_output, filter, g, rowptr_in, order_in, grad_input, C, rs.lpr_log2);
+            else if (F <= 20) point_conv_rows_dense_k<20, 1><<<dim3((unsigned)blocks), dim3(kBlock), 0, st>>>(grad_output, filter, g, rowptr_in, order_in, grad_input, C, rs.lpr_log2);
+            else if (F <= 32) point_conv_rows_dense_k<32, 1><<<dim3((unsigned)blocks), dim3(kBlock), 0, st>>>(grad_output, filter, g, rowptr_in, order_in, grad_input, C, rs.lpr_log2);
+            else point_conv_rows_dense_k<36, 1><<<dim3((unsigned)blocks), dim3(kBlock), 0, st>>>(grad_output, filter, g, rowptr_in, order_in, grad_input, C, rs.lpr_log2);
         } else if (r == 1 && C % 4 == 0 && aligned16(grad_output) && aligned16(filter) && aligned16(grad_input))
             PM_ROW_LAUNCH(point_conv_bwd_in_k<4>, Np, C / 4, grad_output, filter, g, rowptr_in, order_in, grad_input, C, r);
         else
@@ -523,7 +555,9 @@ extern "C" int pmesh_point_conv_bwd(const float *grad_output, const float *input
         int threads = 256;
         while (threads > 64 && threads / 2 >= CR) threads /= 2;
         const dim3 grid((unsigned)G, (unsigned)ceil_div(CR, threads));
-        if (F <= 32) point_conv_bwd_filt_dense_k<32><<<grid, dim3(threads), 0, st>>>(grad_output, input, g, (float *)workspace, C, r, per);
+        if (F <= 20) point_conv_bwd_filt_dense_k<20><<<grid, dim3(threads), 0, st>>>(grad_output, input, g, (float *)workspace, C, r, per);
+        else if (F <= 32) point_conv_bwd_filt_dense_k<32><<<grid, dim3(threads), 0, st>>>(grad_output, input, g, (float *)workspace, C, r, per);
+        else if (F <= 36) point_conv_bwd_filt_dense_k<36><<<grid, dim3(threads), 0, st>>>(grad_output, input, g, (float *)workspace, C, r, per);
         else point_conv_bwd_filt_dense_k<64><<<grid, dim3(threads), 0, st>>>(grad_output, input, g, (float *)workspace, C, r, per);
         PM_LAUNCHED("point_conv_bwd(filter)");
         return reduce_partials((const float *)workspace, grad_filter, G, F * CR, st);

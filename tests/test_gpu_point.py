@@ -183,7 +183,8 @@ def point_graph(cuda, seed, sizes, radius, T, F, limit=None):
 @pytest.mark.parametrize("sizes,radius,C,r,F,T", [([60], 0.45, 5, 1, 7, None), ([60], 0.45, 5, 2, 7, 3), ([800, 500], 0.2, 64, 1, 17, 17),
                                                   ([2000], 0.15, 32, 2, 33, 3), ([300], 0.3, 130, 1, 49, None),
                                                   ([500], 0.25, 16, 1, 125, 1), ([400], 0.25, 8, 3, 300, 2),
-                                                  # filter in registers: 16 / 32 bins, several table chunks per workgroup
+                                                  # filter in registers: 16 / 20 / 32 / 36 bins, several table chunks per workgroup
+                                                  ([700], 0.25, 64, 1, 33, 3), ([500], 0.3, 128, 1, 20, 6), ([400], 0.3, 12, 1, 36, None),
                                                   ([1500], 0.3, 256, 1, 26, 5), ([900, 40], 0.2, 128, 1, 10, 4),
                                                   ([700], 0.25, 32, 1, 8, None), ([600], 0.3, 36, 1, 32, 2)])
 def test_conv_parity(cuda, sizes, radius, C, r, F, T):

@@ -542,9 +542,16 @@ __global__ __launch_bounds__(kBlock) void point_knn3_k(const float *__restrict__
     nn_dist[j * 3] = sqrtf(b1); nn_dist[j * 3 + 1] = sqrtf(b2); nn_dist[j * 3 + 2] = sqrtf(b3);
 }
 
-// Farthest point sampling: one workgroup of 1024 threads per sample.  temp[k] = squared distance of point k to the
-// chosen set; every round updates it against the last chosen point and takes the arg-max (lowest index among equals).
+// Farthest point sampling: one workgroup of 1024 threads per sample.  Every round updates the squared distance of
+// each point to the chosen set against the last chosen point and takes the arg-max (lowest index among equals).
+// A sample of at most 1024 * kFpsPer points lives in registers for the whole run (thread t holds points t, t + 1024,
+// ... and their distances), the round's winner is found by every thread from the wavefronts' candidates in LDS, and
+// its owner hands the coordinates to the others through LDS: two barriers and no global memory access per round
+// (a round over global memory -- the distances in `temp`, the winner's coordinates fetched by all -- takes seven
+// times as long).  Larger samples run that slower form.
 constexpr int kFpsThreads = 1024;
+constexpr int kFpsPer = 16;
+static_assert(kFpsThreads / 64 == 16, "the wavefronts' candidates of a round are compared within one row of 16 lanes");
 __global__ __launch_bounds__(kFpsThreads) void point_fps_k(const float *__restrict__ xyz, const int *__restrict__ nv_in,
                                                            const int *__restrict__ nv_out, int B, int64_t Np, int64_t Mp,
                                                            float *__restrict__ temp, int *__restrict__ index_out)
@@ -553,19 +560,91 @@ __global__ __launch_bounds__(kFpsThreads) void point_fps_k(const float *__restri
     __shared__ float s_best[kFpsThreads / 64];
     __shared__ int s_idx[kFpsThreads / 64];
     __shared__ int s_cur;
+    __shared__ float s_xyz[3];
     const int b = blockIdx.x;
     if (b >= B) return;
     const int n0 = b ? nv_in[b - 1] : 0, n1 = nv_in[b] < Np ? nv_in[b] : (int)Np;
     const int m0 = b ? nv_out[b - 1] : 0, m1 = nv_out[b] < Mp ? nv_out[b] : (int)Mp;
     const int N = n1 - n0, M = m1 - m0;
     if (M <= 0) return;
-    for (int k = threadIdx.x; k < N; k += kFpsThreads) temp[n0 + k] = 1e38f;
-    int cur = n0;
     if (threadIdx.x == 0) index_out[m0] = N > 0 ? n0 : 0;
     if (N <= 0) {
         for (int j = 1 + threadIdx.x; j < M; j += kFpsThreads) index_out[m0 + j] = 0;
         return;
     }
+    // arg-max over a wavefront: larger value, then lower index.  Within rows of 16 lanes the candidates move through
+    // DPP operands (lane pairs, quad halves, mirrored halves of 8 and 16: every lane of a row ends up with the row's
+    // winner; all lanes of the wavefront are active here), across the four rows through the LDS crossbar.
+    auto take_better = [](float &best, int &besti, float ob, int oi) {
+        const bool take = ob > best || (ob == best && oi < besti);
+        best = take ? ob : best;
+        besti = take ? oi : besti;
+    };
+    auto row_argmax = [&](float &best, int &besti) {
+#define PM_FPS_DPP(ctrl)                                                                                                  \
+    take_better(best, besti, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, best), ctrl, 0xF, 0xF, true)), \
+                __builtin_amdgcn_update_dpp(0, besti, ctrl, 0xF, 0xF, true))
+        PM_FPS_DPP(0xB1);
+        PM_FPS_DPP(0x4E);
+        PM_FPS_DPP(0x141);
+        PM_FPS_DPP(0x140);
+#undef PM_FPS_DPP
+    };
+    auto wave_argmax = [&](float &best, int &besti) {
+        row_argmax(best, besti);
+#pragma unroll
+        for (int o = 16; o <= 32; o <<= 1) take_better(best, besti, __shfl_xor(best, o, 64), __shfl_xor(besti, o, 64));
+    };
+    if (N <= kFpsThreads * kFpsPer) {
+        const int per = (N + kFpsThreads - 1) / kFpsThreads;      // points of the busiest thread
+        float px[kFpsPer], py[kFpsPer], pz[kFpsPer], td[kFpsPer];
+#pragma unroll
+        for (int i = 0; i < kFpsPer; ++i) {
+            const int k = threadIdx.x + i * kFpsThreads;
+            const bool in = k < N;
+            const float *p = xyz + (int64_t)(n0 + (in ? k : 0)) * 3;
+            px[i] = p[0]; py[i] = p[1]; pz[i] = p[2];
+            td[i] = in ? 1e38f : -1.f;                            // (a distance is never below zero: no point there wins)
+        }
+        float x1 = xyz[(int64_t)n0 * 3], y1 = xyz[(int64_t)n0 * 3 + 1], z1 = xyz[(int64_t)n0 * 3 + 2];
+        for (int j = 1; j < M; ++j) {
+            float best = -1.f;
+            int besti = n0;
+#pragma unroll
+            for (int i = 0; i < kFpsPer; ++i) {
+                if (i < per) {
+                    const float dx = px[i] - x1, dy = py[i] - y1, dz = pz[i] - z1;
+                    const float d = (dx * dx + dy * dy) + dz * dz;
+                    const float d2 = d < td[i] ? d : td[i];
+                    td[i] = d2;
+                    const bool up = d2 > best;
+                    best = up ? d2 : best;
+                    besti = up ? n0 + (int)threadIdx.x + i * kFpsThreads : besti;
+                }
+            }
+            wave_argmax(best, besti);
+            if ((threadIdx.x & 63) == 0) { s_best[threadIdx.x >> 6] = best; s_idx[threadIdx.x >> 6] = besti; }
+            __syncthreads();
+            // lane l looks at the candidate of wavefront l % 16; the row exchange leaves the winner in every lane
+            float bb = s_best[threadIdx.x & 15];
+            int bi = s_idx[threadIdx.x & 15];
+            row_argmax(bb, bi);
+            if (threadIdx.x == 0) index_out[m0 + j] = bi;
+            const int rel = bi - n0;
+            if ((rel & (kFpsThreads - 1)) == (int)threadIdx.x) {  // my point: its slot is rel / 1024
+                float cx = px[0], cy = py[0], cz = pz[0];
+#pragma unroll
+                for (int i = 1; i < kFpsPer; ++i)
+                    if (i == rel / kFpsThreads) { cx = px[i]; cy = py[i]; cz = pz[i]; }
+                s_xyz[0] = cx; s_xyz[1] = cy; s_xyz[2] = cz;
+            }
+            __syncthreads();
+            x1 = s_xyz[0]; y1 = s_xyz[1]; z1 = s_xyz[2];
+        }
+        return;
+    }
+    for (int k = threadIdx.x; k < N; k += kFpsThreads) temp[n0 + k] = 1e38f;
+    int cur = n0;
     __syncthreads();
     for (int j = 1; j < M; ++j) {
         const float x1 = xyz[(int64_t)cur * 3], y1 = xyz[(int64_t)cur * 3 + 1], z1 = xyz[(int64_t)cur * 3 + 2];
@@ -580,13 +659,7 @@ __global__ __launch_bounds__(kFpsThreads) void point_fps_k(const float *__restri
             if (d2 != td) temp[n0 + k] = d2;
             if (d2 > best) { best = d2; besti = n0 + k; }
         }
-        // arg-max over the workgroup: larger value, then lower index
-#pragma unroll
-        for (int o = 32; o > 0; o >>= 1) {
-            const float ob = __shfl_xor(best, o, 64);
-            const int oi = __shfl_xor(besti, o, 64);
-            if (ob > best || (ob == best && oi < besti)) { best = ob; besti = oi; }
-        }
+        wave_argmax(best, besti);
         if ((threadIdx.x & 63) == 0) { s_best[threadIdx.x >> 6] = best; s_idx[threadIdx.x >> 6] = besti; }
         __syncthreads();
         if (threadIdx.x == 0) {

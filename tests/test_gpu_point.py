@@ -132,7 +132,9 @@ def test_grid_search_beyond_the_reach_it_was_built_for(cuda):
     assert np.array_equal(n(nn_index), w[2]) and np.array_equal(n(nn_dist), w[3])
 
 
-@pytest.mark.parametrize("sizes,keep", [([120, 60], [15, 60]), ([3000], [700]), ([1, 5, 2048], [1, 3, 256])])
+@pytest.mark.parametrize("sizes,keep", [([120, 60], [15, 60]), ([3000], [700]), ([1, 5, 2048], [1, 3, 256]),
+                                        # a sample beyond the 16 384 points that the kernel holds in registers
+                                        ([17000, 300], [40, 20])])
 def test_fps_bit_exact(cuda, sizes, keep):
     say("case point fps", sizes, keep)
     xyz, nv = cloud(23, sizes)

@@ -661,6 +661,41 @@ def run_pcloud(args, torch):
     ms = (time.perf_counter() - t0) * 1e3 / args.steps
     _lib.set_call_hook(None)
     per_op = timer.summary()
+    extra = {}
+    # the other ops of a point level, once each beside the step (wall clock around synchronised calls, median of five):
+    # sampling a quarter of every sample, the pooling graph of the sampled points, pooling and interpolation back
+    from picassoplus_amd.point.pi_modules import nnquery as pnn, pool3d as ppool, sample as psample, unpool3d as punpool
+
+    def wall(fn, reps=5):
+        fn()
+        ts = []
+        for _ in range(reps):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            out = fn()
+            torch.cuda.synchronize()
+            ts.append((time.perf_counter() - t0) * 1e3)
+        return float(np.median(ts)), out
+
+    NQ = torch.from_numpy((nv // 4).astype(np.int32)).to(dev)
+    other = {}
+    other["fps_quarter"], picked = wall(lambda: psample.fps_(xyz, NV, NQ))
+    q = xyz[picked.long()].contiguous()
+    other["range_search_pool_graph"], (_, pcnt, pidx, _) = wall(lambda: pnn.range_search_(xyz, q, NV, NQ, radius=2 * radius, nnsample=32))
+    gq = torch.randn(q.shape[0], C, device=dev, generator=gen)
+
+    def fwd_bwd(fn, *a):
+        def run():
+            return torch.autograd.grad(fn(*a), [a[0]], gq if a[0] is x else g)
+        return run
+
+    other["max_pool_fwd_bwd"], _ = wall(fwd_bwd(ppool.maxPool, x, pcnt, pidx))
+    other["avg_pool_fwd_bwd"], _ = wall(fwd_bwd(ppool.avgPool, x, pcnt, pidx))
+    other["knn3_search"], (nn3, d3) = wall(lambda: pnn.knn3_search_(q, xyz, NQ, NV))
+    xq = torch.randn(q.shape[0], C, device=dev, generator=gen).requires_grad_(True)
+    other["interpolate_fwd_bwd"], _ = wall(fwd_bwd(punpool.interpolate, xq, PU.compute_unpool_weight(d3), nn3))
+    extra["other_ops_ms"] = {k: round(v, 4) for k, v in other.items()}
+    extra["other_ops_config"] = dict(sampled_points=int(q.shape[0]), pool_pairs=int(pidx.shape[0]))
     # every operand once: per pair its index pair, T bins and T weights, one gathered row of C floats; per point a row
     pair = 8 + 8 * T
     nb = {"point_conv_fwd": P * (pair + 4 * C) + 4 * Np * C + 4 * Np,
@@ -669,7 +704,6 @@ def run_pcloud(args, torch):
     dom = max(nb, key=lambda k: per_op[k])
     ach = nb[dom] / (per_op[dom] * 1e-3) / 1e9
     total = sum(nb.values())
-    extra = {}
     if not args.no_cpu_baseline:
         # the oracle (numpy, float64) on the first sample's points and pairs
         from oracle import point_ref as R

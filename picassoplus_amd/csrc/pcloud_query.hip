@@ -438,8 +438,14 @@ __device__ void fill_by_insertion(const PointGrid *__restrict__ G, const int2 *_
 
 // Pairs of query j at [cnt_info[j-1], cnt_info[j]): its lanes drop the neighbours they meet into a buffer of the
 // workgroup (database index; distance or kernel cell), then every neighbour finds its place by counting the lower
-// indices, and the first cnt_info[j] - cnt_info[j-1] places are written.
+// indices, and the first m = cnt_info[j] - cnt_info[j-1] places are written.  A query with more neighbours than the
+// buffer holds, of which it keeps at most half a buffer: the m-th lowest of the indices that did get in bounds the
+// m-th lowest of all from above, so the walk is repeated for the neighbours up to that index only (up to three
+// times; each round leaves out at least half a buffer of what the round before let in).  A query that keeps ALL of
+// more neighbours than the buffer holds sorts them through its output segment (below).  What is left -- a long
+// segment that is still only part of the neighbours -- is filled by one lane (fill_by_insertion).
 constexpr int kFillCap = 128;
+constexpr int kFillRounds = 4;
 template <int MODE>
 __global__ __launch_bounds__(kBlock) void point_fill_grid_k(const PointGrid *__restrict__ G, const int2 *__restrict__ cells,
                                                             const float4 *__restrict__ pts, const float *__restrict__ db,
@@ -450,9 +456,13 @@ __global__ __launch_bounds__(kBlock) void point_fill_grid_k(const PointGrid *__r
 {
 #pragma clang fp contract(off)
     constexpr int W = MODE == 0 ? 2 : 3;
-    __shared__ int s_id[kQPerBlock][kFillCap + 1];
-    __shared__ unsigned s_val[kQPerBlock][kFillCap + 1];
-    __shared__ int s_cnt[kQPerBlock];
+    // a query's buffer: kFillCap indices, then as many distances / kernel cells; as one array of indices where all
+    // neighbours are kept (below)
+    constexpr int kRow = 2 * (kFillCap + 1);
+    __shared__ int s_buf[kQPerBlock][kRow];
+    int *s_id_q = &s_buf[threadIdx.x / kQLanes][0];
+    unsigned *s_val_q = reinterpret_cast<unsigned *>(s_id_q + kFillCap + 1);
+    __shared__ int s_cnt[kQPerBlock], s_thr[kQPerBlock];
     const int q = threadIdx.x / kQLanes, sub = threadIdx.x % kQLanes;
     const int64_t j = (int64_t)blockIdx.x * kQPerBlock + q;
     const bool valid = j < Mp;
@@ -467,51 +477,206 @@ __global__ __launch_bounds__(kBlock) void point_fill_grid_k(const PointGrid *__r
         m = end > at ? end - at : 0;
         qx = query[j * 3]; qy = query[j * 3 + 1]; qz = query[j * 3 + 2];
     }
-    if (sub == 0) s_cnt[q] = 0;
-    // (the lanes of a query sit in one wavefront)
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    if (m > 0)
-        grid_visit<MODE>(G, cells, pts, b, qx, qy, qz, size, sub, kQLanes, [&](const float4 &p) {
-            float dx, dy, dz;
-            const float d2 = sq_dist(qx, qy, qz, p, dx, dy, dz);
-            if (!is_neighbour<MODE>(d2, dx, dy, dz, size)) return true;
-            const int slot = atomicAdd(&s_cnt[q], 1);
-            if (slot < kFillCap) {
-                s_id[q][slot] = __float_as_int(p.w);
+    // a segment longer than a query's buffer is left to point_fill_long_k: -1 in its first place says so
+    bool later = m > kRow;
+    // (the lanes of a query sit in one wavefront, and every lane of the wavefront stays until the last exchange)
+    auto lanes_meet = [] {
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    };
+    int thr = INT32_MAX;                                // neighbours above this index are not among the m lowest
+    int total = 0;
+    bool open = m > 0 && !later, all_kept = false;
+    for (int round = 0; round < kFillRounds; ++round) {
+        if (!__builtin_amdgcn_ballot_w64(open)) break;
+        if (open && sub == 0) s_cnt[q] = 0;
+        lanes_meet();
+        if (open)
+            grid_visit<MODE>(G, cells, pts, b, qx, qy, qz, size, sub, kQLanes, [&](const float4 &p) {
+                float dx, dy, dz;
+                const float d2 = sq_dist(qx, qy, qz, p, dx, dy, dz);
+                if (!is_neighbour<MODE>(d2, dx, dy, dz, size)) return true;
+                const int id = __float_as_int(p.w);
+                if (id > thr) return true;
+                const int slot = atomicAdd(&s_cnt[q], 1);
+                if (slot < kFillCap) {
+                    s_id_q[slot] = id;
+                    if constexpr (MODE == 0) {
+                        s_val_q[slot] = __float_as_uint(sqrtf(d2));
+                    } else {
+                        const float half = size / 2, cell = size / (float)grid_size;
+                        const int xi = (int)((dx + half) / cell), yi = (int)((dy + half) / cell), zi = (int)((dz + half) / cell);
+                        s_val_q[slot] = (unsigned)((xi * grid_size + yi) * grid_size + zi);
+                    }
+                }
+                return true;
+            });
+        lanes_meet();
+        bool narrow = false;
+        if (open) {
+            total = s_cnt[q];
+            if (total <= kFillCap) open = false;
+            else if (round == 0 && total == m) { open = false; all_kept = true; }
+            else if (m > kFillCap / 2 || round == kFillRounds - 1) { open = false; later = true; }
+            else narrow = true;
+        }
+        if (__builtin_amdgcn_ballot_w64(narrow)) {
+            if (narrow)
+                for (int e = sub; e < kFillCap; e += kQLanes) {
+                    const int id = s_id_q[e];
+                    int rank = 0;
+                    for (int f = 0; f < kFillCap; ++f) rank += s_id_q[f] < id ? 1 : 0;
+                    if (rank == m - 1) s_thr[q] = id;
+                }
+            lanes_meet();
+            if (narrow) thr = s_thr[q];
+        }
+    }
+    // More neighbours than the buffer holds, all of them kept (and at most kRow of them): their indices go into the
+    // query's whole buffer in the order met, then every entry of that list finds its place by counting the lower
+    // indices in it.
+    if (__builtin_amdgcn_ballot_w64(all_kept)) {
+        if (all_kept && sub == 0) s_cnt[q] = 0;
+        lanes_meet();
+        if (all_kept)
+            grid_visit<MODE>(G, cells, pts, b, qx, qy, qz, size, sub, kQLanes, [&](const float4 &p) {
+                float dx, dy, dz;
+                const float d2 = sq_dist(qx, qy, qz, p, dx, dy, dz);
+                if (!is_neighbour<MODE>(d2, dx, dy, dz, size)) return true;
+                const int slot = atomicAdd(&s_cnt[q], 1);
+                if (slot < m) s_id_q[slot] = __float_as_int(p.w);
+                return true;
+            });
+        lanes_meet();
+        // (a second walk with the counting inside would make every lane of the wavefront wait through the count of
+        // every neighbour any lane meets; the list itself is walked instead, and a neighbour's distance or cell comes
+        // from its coordinates)
+        if (all_kept)
+            for (int e = sub; e < (int)m; e += kQLanes) {
+                const int id = s_id_q[e];
+                int r0 = 0, r1 = 0;
+                int f = 0;
+                for (; f + 2 <= (int)m; f += 2) {
+                    const int2 two = *reinterpret_cast<const int2 *>(s_id_q + f);
+                    r0 += two.x < id ? 1 : 0;
+                    r1 += two.y < id ? 1 : 0;
+                }
+                if (f < (int)m) r0 += s_id_q[f] < id ? 1 : 0;
+                const int rank = r0 + r1;
+                const int64_t row = id < 0 ? 0 : (id >= Np ? Np - 1 : id);
+                float dx, dy, dz;
+                const float d2 = sq_dist(qx, qy, qz, db + row * 3, dx, dy, dz);
+                nn_index[(at + rank) * W] = (int)j;
+                nn_index[(at + rank) * W + 1] = id;
                 if constexpr (MODE == 0) {
-                    s_val[q][slot] = __float_as_uint(sqrtf(d2));
+                    nn_dist[at + rank] = sqrtf(d2);
                 } else {
                     const float half = size / 2, cell = size / (float)grid_size;
                     const int xi = (int)((dx + half) / cell), yi = (int)((dy + half) / cell), zi = (int)((dz + half) / cell);
-                    s_val[q][slot] = (unsigned)((xi * grid_size + yi) * grid_size + zi);
+                    nn_index[(at + rank) * W + 2] = (xi * grid_size + yi) * grid_size + zi;
+                }
+            }
+    }
+    if (m <= 0 || all_kept) return;
+    if (later) {
+        if (sub == 0) nn_index[at * W] = -1;
+        return;
+    }
+    for (int e = sub; e < total; e += kQLanes) {
+        const int id = s_id_q[e];
+        int rank = 0;
+        for (int f = 0; f < total; ++f) rank += s_id_q[f] < id ? 1 : 0;
+        if (rank >= m) continue;
+        nn_index[(at + rank) * W] = (int)j;
+        nn_index[(at + rank) * W + 1] = id;
+        if constexpr (MODE == 0) nn_dist[at + rank] = __uint_as_float(s_val_q[e]);
+        else nn_index[(at + rank) * W + 2] = (int)s_val_q[e];
+    }
+}
+
+// The segments point_fill_grid_k left (first place = -1): a wavefront per query, up to kLongCap neighbours in its
+// buffer (index; distance or kernel cell), places by counting the lower indices as above; beyond that, one lane's
+// sorted insertion.  A workgroup looks at kBlock queries and its wavefronts share out the marked ones.
+constexpr int kLongCap = 4096;
+template <int MODE>
+__global__ __launch_bounds__(kBlock) void point_fill_long_k(const PointGrid *__restrict__ G, const int2 *__restrict__ cells,
+                                                            const float4 *__restrict__ pts, const float *__restrict__ db,
+                                                            const float *__restrict__ query, const int *__restrict__ nvq, int B,
+                                                            int64_t Np, int64_t Mp, float size, int grid_size,
+                                                            const int64_t *__restrict__ cnt_info, int64_t Nout,
+                                                            int *nn_index, float *nn_dist)
+{
+#pragma clang fp contract(off)
+    constexpr int W = MODE == 0 ? 2 : 3, NW = kBlock / 64;
+    __shared__ int s_id[NW][kLongCap];
+    __shared__ unsigned s_val[NW][kLongCap];
+    __shared__ int s_list[kBlock], s_n, s_cnt[NW];
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    if (threadIdx.x == 0) s_n = 0;
+    __syncthreads();
+    {
+        const int64_t j = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+        if (j < Mp && sample_index(j, nvq, B) < B) {
+            int64_t at = j ? cnt_info[j - 1] : 0, end = cnt_info[j];
+            if (at < 0) at = 0;
+            if (end > Nout) end = Nout;
+            if (end > at && nn_index[at * W] == -1) s_list[atomicAdd(&s_n, 1)] = (int)threadIdx.x;
+        }
+    }
+    __syncthreads();
+    const int n = s_n;
+    for (int i = w; i < n; i += NW) {
+        const int64_t j = (int64_t)blockIdx.x * kBlock + s_list[i];
+        const int b = sample_index(j, nvq, B);
+        int64_t at = j ? cnt_info[j - 1] : 0, end = cnt_info[j];
+        if (at < 0) at = 0;
+        if (end > Nout) end = Nout;
+        const int64_t m = end - at;
+        const float qx = query[j * 3], qy = query[j * 3 + 1], qz = query[j * 3 + 2];
+        if (lane == 0) s_cnt[w] = 0;
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        grid_visit<MODE>(G, cells, pts, b, qx, qy, qz, size, lane, 64, [&](const float4 &p) {
+            float dx, dy, dz;
+            const float d2 = sq_dist(qx, qy, qz, p, dx, dy, dz);
+            if (!is_neighbour<MODE>(d2, dx, dy, dz, size)) return true;
+            const int slot = atomicAdd(&s_cnt[w], 1);
+            if (slot < kLongCap) {
+                s_id[w][slot] = __float_as_int(p.w);
+                if constexpr (MODE == 0) {
+                    s_val[w][slot] = __float_as_uint(sqrtf(d2));
+                } else {
+                    const float half = size / 2, cell = size / (float)grid_size;
+                    const int xi = (int)((dx + half) / cell), yi = (int)((dy + half) / cell), zi = (int)((dz + half) / cell);
+                    s_val[w][slot] = (unsigned)((xi * grid_size + yi) * grid_size + zi);
                 }
             }
             return true;
         });
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    if (m <= 0) return;
-    const int total = s_cnt[q];
-    if (total > kFillCap) {
-        if (sub == 0) {
-            const bool fits = m <= kFillCap;
-            fill_by_insertion<MODE>(G, cells, pts, db, b, j, qx, qy, qz, Np, size, grid_size, at, m,
-                                    fits ? &s_id[q][0] : nn_index + at * W + 1, fits ? 1 : W, nn_index, nn_dist);
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        const int total = s_cnt[w];
+        if (total > kLongCap) {
+            if (lane == 0)
+                fill_by_insertion<MODE>(G, cells, pts, db, b, j, qx, qy, qz, Np, size, grid_size, at, m, nn_index + at * W + 1, W,
+                                        nn_index, nn_dist);
+            continue;
         }
-        return;
-    }
-    for (int e = sub; e < total; e += kQLanes) {
-        const int id = s_id[q][e];
-        int rank = 0;
-        for (int f = 0; f < total; ++f) rank += s_id[q][f] < id ? 1 : 0;
-        if (rank >= m) continue;
-        nn_index[(at + rank) * W] = (int)j;
-        nn_index[(at + rank) * W + 1] = id;
-        if constexpr (MODE == 0) nn_dist[at + rank] = __uint_as_float(s_val[q][e]);
-        else nn_index[(at + rank) * W + 2] = (int)s_val[q][e];
+        for (int e = lane; e < total; e += 64) {
+            const int id = s_id[w][e];
+            int rank = 0;
+            for (int f = 0; f < total; ++f) rank += s_id[w][f] < id ? 1 : 0;
+            if (rank >= m) continue;
+            nn_index[(at + rank) * W] = (int)j;
+            nn_index[(at + rank) * W + 1] = id;
+            if constexpr (MODE == 0) nn_dist[at + rank] = __uint_as_float(s_val[w][e]);
+            else nn_index[(at + rank) * W + 2] = (int)s_val[w][e];
+        }
+        // (a segment with fewer neighbours than places keeps its mark otherwise)
+        if (lane == 0 && total == 0) nn_index[at * W] = (int)j;
     }
 }
 
@@ -891,6 +1056,8 @@ extern "C" int pmesh_point_range_fill_grid(const void *grid, const float *databa
     PM_GRID_PARTS("point_range_fill");
     point_fill_grid_k<0><<<dim3((unsigned)ceil_div(Mp, kQPerBlock)), dim3(kBlock), 0, (hipStream_t)stream>>>(
         G, cells, pts, database, query, nv_query, B, Np, Mp, radius, 1, cnt_info, Nout, nn_index, nn_dist);
+    point_fill_long_k<0><<<dim3((unsigned)ceil_div(Mp, kBlock)), dim3(kBlock), 0, (hipStream_t)stream>>>(
+        G, cells, pts, database, query, nv_query, B, Np, Mp, radius, 1, cnt_info, Nout, nn_index, nn_dist);
     PM_LAUNCHED("point_range_fill");
     return 0;
 }
@@ -922,6 +1089,8 @@ extern "C" int pmesh_point_cube_fill_grid(const void *grid, const float *databas
     PM_REQUIRE(cnt_info && nn_index, "point_cube_fill: null pointer");
     PM_GRID_PARTS("point_cube_fill");
     point_fill_grid_k<1><<<dim3((unsigned)ceil_div(Mp, kQPerBlock)), dim3(kBlock), 0, (hipStream_t)stream>>>(
+        G, cells, pts, database, query, nv_query, B, Np, Mp, length, grid_size, cnt_info, Nout, nn_index, nullptr);
+    point_fill_long_k<1><<<dim3((unsigned)ceil_div(Mp, kBlock)), dim3(kBlock), 0, (hipStream_t)stream>>>(
         G, cells, pts, database, query, nv_query, B, Np, Mp, length, grid_size, cnt_info, Nout, nn_index, nullptr);
     PM_LAUNCHED("point_cube_fill");
     return 0;

@@ -109,6 +109,27 @@ def test_grid_search_matches_scan(cuda, monkeypatch, shape):
         assert a.dtype == b.dtype and np.array_equal(a, b, equal_nan=True)
 
 
+@pytest.mark.parametrize("limit", [None, 300, 20])
+def test_grid_search_with_more_neighbours_than_any_buffer(cuda, monkeypatch, limit):
+    """4500 database points inside the reach of three queries: more than the per-query buffers of the fill kernels
+    hold (128 and 258 places in the first, 4096 in the one for long segments), kept all, cut to a long segment, cut
+    to a short one."""
+    say("case grid search crowd", limit)
+    rng = np.random.default_rng(5)
+    db = (0.5 + 0.01 * rng.standard_normal((4500, 3))).astype(np.float32)
+    db = np.concatenate([db, cloud(6, [600])[0]])
+    q = np.array([[0.5, 0.5, 0.5], [0.51, 0.5, 0.49], [0.9, 0.1, 0.2]], np.float32)
+    nvd, nvq = np.array([db.shape[0]], np.int32), np.array([3], np.int32)
+    D, Q, ND, NQ = dev(db, cuda), dev(q, cuda), dev(nvd, cuda), dev(nvq, cuda)
+    monkeypatch.setattr(point_nnquery, "GRID_MIN_POINTS", 1 << 40)
+    want = _searches(D, Q, ND, NQ, 0.2, limit)
+    monkeypatch.setattr(point_nnquery, "GRID_MIN_POINTS", 0)
+    got = _searches(D, Q, ND, NQ, 0.2, limit)
+    assert want[1].max() > 4096 or limit is not None
+    for a, b in zip(want, got):
+        assert a.dtype == b.dtype and np.array_equal(a, b)
+
+
 def test_grid_search_beyond_the_reach_it_was_built_for(cuda):
     """A search that reaches further than the cells are wide looks at more cells: through the C-ABI, a grid built for a
     tenth of the radius."""

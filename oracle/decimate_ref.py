@@ -118,8 +118,11 @@ def rref_solve(A, b, dtype=np.float64):
 def quadric_error(x, Q):
     """x^T A x + 2 b.x + c in the reference's association (decimate_gpu.cu:190-198)."""
     A = Q[:, [0, 1, 2, 1, 3, 4, 2, 4, 5]].reshape(-1, 3, 3)
-    xa = np.einsum("nr,nrc->nc", x, A)
-    return (xa * x).sum(1) + (x * Q[:, 6:9]).sum(1) * 2 + Q[:, 9]
+    # every product and sum written out, left to right: in float32 the result is then a function of the inputs alone
+    # (an einsum may fuse or reorder), which is what a device kernel can be compared with bit for bit
+    x0, x1, x2 = x[:, 0], x[:, 1], x[:, 2]
+    xa = [x0 * A[:, 0, c] + x1 * A[:, 1, c] + x2 * A[:, 2, c] for c in range(3)]
+    return (xa[0] * x0 + xa[1] * x1 + xa[2] * x2) + (x0 * Q[:, 6] + x1 * Q[:, 7] + x2 * Q[:, 8]) * 2 + Q[:, 9]
 
 
 def edge_costs(vertex, quadric, edge_vi, edge_vj, dtype=np.float64, return_rcond=False):

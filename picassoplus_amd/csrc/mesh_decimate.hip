@@ -14,6 +14,11 @@
 #include "../../include/picasso_mesh.h"
 #include <vector>
 
+// Every product and sum of this file is rounded on its own (no fused multiply-adds): the quadrics and costs are then
+// the float32 values that the same expressions give anywhere, and the contraction order that follows from the costs
+// can be checked against a float32 restatement from the mesh alone.
+#pragma clang fp contract(off)
+
 namespace pmesh {
 
 constexpr float kAreaMagnitude = 100.0f;        // areas in dm^2 for inputs in metres (decimate_gpu.cu:16)

@@ -70,6 +70,62 @@ def test_quadrics_and_costs_match_oracle(cuda, names, use_area, wgt_bnd):
     assert clear.mean() > 0.9
 
 
+def _ulps(a, b):
+    """Distance of two float32 arrays in units of the last place (0 where both are NaN or bit-equal)."""
+    ia = np.ascontiguousarray(a, np.float32).view(np.int32).astype(np.int64)
+    ib = np.ascontiguousarray(b, np.float32).view(np.int32).astype(np.int64)
+    ia = np.where(ia < 0, -(ia & 0x7FFFFFFF), ia)
+    ib = np.where(ib < 0, -(ib & 0x7FFFFFFF), ib)
+    d = np.abs(ia - ib)
+    return np.where(np.isnan(a) & np.isnan(b), 0, d)
+
+
+@pytest.mark.parametrize("names", CASES, ids=lambda n: "+".join(n))
+@pytest.mark.parametrize("use_area,wgt_bnd", [(True, 5.0), (False, 5.0), (True, 0.0)])
+def test_quadrics_and_costs_equal_the_float32_oracle(cuda, names, use_area, wgt_bnd):
+    """EVERY candidate edge (no conditioning mask): the kernels round each product and sum on its own, so their
+    float32 quadrics and costs are the float32 oracle's bit for bit -- including which branch an edge near the
+    condition-number threshold takes."""
+    say("case decimate float32 identity", names, use_area, wgt_bnd)
+    v, f, nv, mf = batch(names)
+    vx, fc = dev(v, cuda), dev(f, cuda)
+    geo = compute_triangle_geometry_(vx, fc)
+    g = geo.cpu().numpy()
+    q, evi, evj = decimate.vertex_quadrics(vx, fc, geo, use_area, wgt_bnd)
+    wq, wi, wj = D.vertex_quadrics(v, f, g, use_area, wgt_bnd, dtype=np.float32)
+    assert wq.dtype == np.float32
+    qn = q.cpu().numpy()
+    dq = _ulps(qn, wq)
+    assert dq.max() == 0, "vertex quadrics: %d of %d entries differ from the float32 oracle, worst %d ulp" % ((dq > 0).sum(), dq.size, dq.max())
+    cost = decimate.edge_costs(vx, q, evi, evj).cpu().numpy()
+    want = D.edge_costs(v, qn, wi, wj, dtype=np.float32)
+    assert want.dtype == np.float32
+    dc = _ulps(cost, want)
+    assert dc.max() == 0, "edge costs: %d of %d differ from the float32 oracle, worst %d ulp" % ((dc > 0).sum(), dc.size, dc.max())
+
+
+@pytest.mark.parametrize("names,frac", [(("sphere2",), 0.5), (("torus", "sphere3"), 0.3), (("room_small",), 0.5),
+                                        (("shapes_small", "fans"), 0.45)],
+                         ids=lambda n: "+".join(n) if isinstance(n, tuple) else str(n))
+def test_simplify_round_equals_the_float32_oracle_from_the_mesh_alone(cuda, names, frac):
+    """The oracle runs the whole round from (vertex, face, geometry) in float32 -- its own quadrics, its own costs, its
+    own contraction order -- and every integer output of the device's round equals it."""
+    say("case decimate simplify from the mesh alone", names, frac)
+    v, f, nv, mf = batch(names)
+    vx, fc = dev(v, cuda), dev(f, cuda)
+    geo = compute_triangle_geometry_(vx, fc)
+    nv_cum, mf_cum = np.cumsum(nv).astype(np.int32), np.cumsum(mf).astype(np.int32)
+    n_remove = (nv * frac).astype(np.int32)
+    out = decimate.simplify(vx, fc, geo, dev(nv_cum, cuda), dev(mf_cum, cuda), dev(n_remove, cuda), True, 5.0)
+    want = D.simplify(v, f, geo.cpu().numpy(), nv_cum, mf_cum, n_remove, True, 5.0, dtype=np.float32)
+    vo, fo, deg, rep, vmap, nv_o, mf_o = (t.cpu().numpy() for t in out)
+    same = (rep == want[3]) & (vmap == want[4])
+    assert same.all(), "maps differ from the float32 oracle's on %d of %d vertices" % ((~same).sum(), len(same))
+    assert np.array_equal(deg, want[2]) and np.array_equal(fo, want[1]), "facets"
+    assert np.array_equal(nv_o, want[5]) and np.array_equal(mf_o, want[6]), "counts"
+    assert np.abs(vo - want[0]).max() <= 1e-6 * max(np.abs(v).max(), 1.0), "contracted positions"
+
+
 @pytest.mark.parametrize("names,frac", [(("tetra",), 0.5), (("grid2",), 0.4), (("sphere2",), 0.5), (("torus", "sphere3"), 0.3),
                                         (("room_small",), 0.5), (("shapes_small", "fans"), 0.45), (("sphere3", "torus"), 0.0)],
                          ids=lambda n: "+".join(n) if isinstance(n, tuple) else str(n))

@@ -624,10 +624,10 @@ def test_adjface_count_and_triangle_geometry(cuda, mesh):
     ok = ln[:, 0] > 0.1 * np.linalg.norm(e1, axis=1) * np.linalg.norm(e2, axis=1)
     assert ok.mean() > 0.5
     okt = torch.from_numpy(ok).to(cuda)
-    assert_close(geo[okt][:, :4], ref_geo[ok][:, :4], "triangle normal and offset", 1e-4)
+    assert_close(geo[okt][:, :4], ref_geo[ok][:, :4], "triangle normal and offset")
     assert_close(geo[:, 4], ref_geo[:, 4], "triangle area")
     assert_close(geo[okt][:, :3], R.face_normals(torch.from_numpy(p), torch.from_numpy(f)).numpy()[ok],
-                 "normals vs oracle", 1e-4)
+                 "normals vs oracle")
 
 
 @pytest.mark.parametrize("mesh,L", [("octa", 3), ("sphere3", 3), ("room_small", 5), ("torus", None)])
@@ -654,10 +654,10 @@ def test_facet_frame_parity(cuda, mesh, L):
     shaped = np.linalg.norm(np.cross(e1, e2), axis=1) > 0.1 * np.linalg.norm(e1, axis=1) * np.linalg.norm(e2, axis=1)
     sure = shaped & (np.abs((centre * n_ref.numpy()).sum(1)) > 1e-4)
     assert sure.mean() > 0.5
-    assert_close(nrm[torch.from_numpy(sure).to(cuda)], o_ref[sure], "oriented normals", 1e-4)
+    assert_close(nrm[torch.from_numpy(sure).to(cuda)], o_ref[sure], "oriented normals")
     assert torch.equal(nrm.abs(), geo[:, :3].abs())
     if L is None:
         assert coeff is None
     else:
         assert torch.equal(coeff, sph_harm_values(nrm, L))
-        assert_close(coeff[torch.from_numpy(sure).to(cuda)], loops.sph_harm(o_ref[sure], L), "coefficients", 1e-4)
+        assert_close(coeff[torch.from_numpy(sure).to(cuda)], loops.sph_harm(o_ref[sure], L), "coefficients")

@@ -302,9 +302,9 @@ def test_dual_block_graph_and_module(cuda):
     gz = f64(g) * (z > 0)
     gmid = gz @ f64(conv.depth_weights).T
     gin, gfilt = P.conv_bwd(gmid, f64(feat), f64(conv.spatial_weights), w[1], w[2], n(filt_idx), f64(filt_coeff))
-    assert_close(feat.grad, gin, "PCloudConv3d grad input", 2e-5)
-    assert_close(conv.spatial_weights.grad, gfilt, "PCloudConv3d grad spatial", 2e-5)
-    assert_close(conv.depth_weights.grad, mid.T @ gz, "PCloudConv3d grad depth", 2e-5)
+    assert_close(feat.grad, gin, "PCloudConv3d grad input")
+    assert_close(conv.spatial_weights.grad, gfilt, "PCloudConv3d grad spatial")
+    assert_close(conv.depth_weights.grad, mid.T @ gz, "PCloudConv3d grad depth")
     # the other two graph builders
     g_rng = point_utils.build_range_graph(X, X, NV, NV, radius, nn_uplimit=limit, kernel_shape=[8, 4, 1], fuzzy=True)
     assert tuple(g_rng[3].shape) == (len(w[2]), 3) and torch.equal(g_rng[1], nn_idx)

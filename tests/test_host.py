@@ -323,3 +323,21 @@ def test_call_many_runs_independent_samples_on_threads_and_reports_a_failure():
     bad[3] = bad[3][:4] + (num // 2,) + bad[3][5:]          # the sample's range cut in half: its edges leave it
     with pytest.raises(RuntimeError, match="outside the sample's vertex range"):
         _lib.call_many("pmesh_cluster_vertices_host", bad)
+
+
+def test_bf16_store_criterion_tells_rounding_from_truncation():
+    """The slack the bf16 parity criterion grants the final store (2^-8 of each value) covers round-to-nearest and
+    nothing more: the same exact results stored by truncation fail it."""
+    import torch
+    from util import assert_close_bf16_store
+    rng = np.random.default_rng(5)
+    ref = rng.uniform(0.5, 4.0, 20000) * rng.choice([-1.0, 1.0], 20000)
+    as_f32 = torch.from_numpy(ref.astype(np.float32))
+    rounded = as_f32.to(torch.bfloat16)
+    truncated = (as_f32.view(torch.int32) & -65536).view(torch.float32)
+    # the criterion's own tolerance set to (almost) nothing: only the store's rounding is in play
+    assert_close_bf16_store(rounded, ref, "rounded to nearest", tol=1e-6)
+    with pytest.raises(AssertionError):
+        assert_close_bf16_store(truncated, ref, "truncated", tol=1e-6)
+    with pytest.raises(AssertionError):
+        assert_close_bf16_store(truncated, ref, "truncated", tol=1e-3)

@@ -18,8 +18,12 @@ def rel_err(y, ref):
     return float(num / den) if den > 0 else float(num)
 
 
+MEASURED = []    # (label, measured error, bound) of every parity assertion of the session, reported by conftest.py
+
+
 def assert_close(y, ref, what, tol=TOL_F32):
     e = rel_err(y.detach().cpu().numpy() if isinstance(y, torch.Tensor) else y, ref)
+    MEASURED.append((what, e, tol))
     assert e <= tol, "%s: max rel err %.3e > %.1e" % (what, e, tol)
     return e
 
@@ -40,6 +44,8 @@ def assert_as_good_as_f32(y, ref64, ref32, what, factor=2.0):
     (reference summation order) is from it: err(y) <= max(factor err(ref32), 2^-22).  Returns (err(y), err(ref32))."""
     e = rel_err(y.detach().cpu().numpy() if isinstance(y, torch.Tensor) else y, ref64)
     e32 = rel_err(ref32, ref64)
+    # reported as the ratio to the float32 oracle's error (floored as the bound is) against the factor allowed
+    MEASURED.append((what + " [error / float32 oracle's error]", e / max(e32, F32_FLOOR / (factor or 1.0)), factor or float("inf")))
     if factor is not None:
         assert e <= max(factor * e32, F32_FLOOR), "%s: error %.3e exceeds %g x the float32 oracle's %.3e" % (what, e, factor, e32)
     return e, e32
@@ -114,8 +120,10 @@ def to_bf16(a):
 
 def assert_close_bf16_store(y, ref, what, tol=TOL_BF16):
     """A result that left the kernel as bf16: within ``tol`` of the largest reference value before the final rounding
-    to bf16, i.e. |y - ref| <= tol max|ref| + 2^-8 |ref| element by element (2^-8 |ref| bounds the rounding of a
-    value to bf16's eight significant bits)."""
+    to bf16, i.e. |y - ref| <= tol max|ref| + 2^-8 |ref| element by element.  bf16 keeps eight significant bits (one
+    implicit, seven stored), so neighbouring values are 2^-7 of the binade's start apart: rounding to nearest moves a
+    value by at most 2^-8 of its magnitude, a store that truncates by up to 2^-7 (test_host.py checks that such a
+    store fails this criterion)."""
     y = y.detach().to(torch.float64).cpu().numpy() if isinstance(y, torch.Tensor) else np.asarray(y, np.float64)
     ref = np.asarray(ref, np.float64)
     assert y.shape == ref.shape, (y.shape, ref.shape)
@@ -124,5 +132,6 @@ def assert_close_bf16_store(y, ref, what, tol=TOL_BF16):
     den = np.abs(ref).max()
     slack = np.abs(y - ref) - 2.0 ** -8 * np.abs(ref)
     e = float(slack.max() / den) if den > 0 else float(np.abs(y).max())
+    MEASURED.append((what + " [bf16 store]", e, tol))
     assert e <= tol, "%s: error beyond the bf16 store rounding %.3e > %.1e of max|ref|" % (what, e, tol)
     return e

@@ -472,3 +472,95 @@ def test_decimation_full_size_invariants(cuda):
     hi = np.searchsorted(coarse[order], pick, side="right")
     want = np.stack([xs[order[a:b]].max(0) for a, b in zip(lo, hi)])
     assert np.array_equal(pooled[torch.from_numpy(pick).to(cuda)].cpu().numpy(), want)
+
+
+@pytest.mark.parametrize("level,C", [(0, 32), (3, 256)])
+def test_hierarchy_level_full_size(cuda, level, C):
+    """The finest (2.1 M facets, width 32) and the coarsest (32 768 facets, width 256) level of the hierarchy
+    workload at the bench's sizes: the three convolutions through adjoint identities, oracle parity on sampled
+    facets / vertices, and the facet2facet filter gradient element by element.  These are the kernel instances the
+    scene batch does not reach (half-empty 64-column tiles at width 32, four blocks of 64 output channels at 256)."""
+    from oracle import torch_ref as R
+    torch.set_num_threads(16)
+    cells = 1024 >> level
+    say("case hierarchy level", level, "width", C, "cells", cells)
+    rng = np.random.default_rng(5000 + level)
+    h = float(1 << level)
+    v, f = S.grid_patch(rng, cells, cells, (0, 0, 0), (h, 0, 0), (0, h, 0), flip_frac=0.5)
+    v = v + rng.normal(0, 0.1 * h, v.shape) * np.array([1.0, 1.0, 0.2])
+    nv, nf = v.shape[0], f.shape[0]
+    assert nf == 2 * cells * cells
+    normal, _ = S.triangle_normals_areas(v, f)
+    counts, bary, _ = S.texture_points(rng, nf, rng.integers(1, 4, nf).astype(np.int32))
+    T = int(counts.sum())
+    face, cum = dev(f, cuda), torch.cumsum(dev(counts, cuda), 0, dtype=torch.int32)
+    sh = sph_harm_values(dev(bary.astype(np.float32), cuda), 3)
+    coeff = sph_harm_values(dev(normal.astype(np.float32), cuda), 3)
+    nfc_np = np.maximum(S.vertex_facet_count(f, np.arange(nv), nv), 1).astype(np.int32)
+    nfc, ident = dev(nfc_np, cuda), torch.arange(nv, dtype=torch.int32, device=cuda)
+    gen = torch.Generator(device=cuda).manual_seed(50 + level)
+
+    # facet2facet C -> C
+    tex = torch.rand(T, C, device=cuda, generator=gen).mul_(2).sub_(1).requires_grad_(True)
+    w = dev(S.xavier_uniform(rng, (C, C, 16), C * 16, C * 16).astype(np.float32), cuda).requires_grad_(True)
+    g = torch.randn(nf, C, device=cuda, generator=gen)
+    out = conv3d.facet2facet(tex, w, sh, cum)
+    gtex, gw = torch.autograd.grad(out, [tex, w], g)
+    torch.cuda.synchronize()
+    lhs, scale = _dot(out, g), float(out.double().norm() * g.double().norm())
+    _adjoint_ok(lhs, _dot(tex, gtex), scale, "<f2f(tex), g> = <tex, grad_texture>")
+    _adjoint_ok(lhs, _dot(w, gw), scale, "<f2f(tex), g> = <W, grad_filter>")
+    pick = np.sort(rng.choice(nf, 600, replace=False))
+    start = np.concatenate([[0], np.cumsum(counts)])[:-1]
+    rows = np.concatenate([np.arange(start[i], start[i] + counts[i]) for i in pick]).astype(np.int64)
+    rows_t, pick_t = torch.from_numpy(rows).to(cuda), torch.from_numpy(pick).to(cuda)
+    w64 = w.detach().cpu().numpy().astype(np.float64)
+    sub_tex, sub_sh = tex.detach()[rows_t].cpu().numpy().astype(np.float64), sh[rows_t].cpu().numpy().astype(np.float64)
+    sub_cum = np.cumsum(counts[pick]).astype(np.int32)
+    ref_out = loops.f2f_fwd(sub_tex, w64, sub_sh, sub_cum)
+    ref_gtex, _ = loops.f2f_bwd(g[pick_t].cpu().numpy().astype(np.float64), sub_tex, w64, sub_sh, sub_cum)
+    tag = " (hierarchy level %d)" % level
+    assert_close(out.detach()[pick_t], ref_out, "f2f out, sampled facets" + tag)
+    assert_close(gtex[rows_t], ref_gtex, "f2f grad_texture, sampled facets" + tag)
+    ref_gw = R.f2f_bwd_filter_pointwise(g.cpu().double(), tex.detach().cpu().double(), sh.cpu().double(), cum.cpu())
+    assert_close(gw, ref_gw.numpy(), "f2f grad_filter, element by element" + tag)
+    del out, gtex, gw, ref_gw, tex
+
+    # facet2vertex C -> C and vertex2facet C -> C
+    x = torch.randn(nf, C, device=cuda, generator=gen).requires_grad_(True)
+    wv = dev(S.xavier_uniform(rng, (16, C, 1), C, 16 * C).astype(np.float32), cuda).requires_grad_(True)
+    gv = torch.randn(nv, C, device=cuda, generator=gen)
+    y = conv3d.facet2vertex(x, wv, coeff, face, nfc, ident)
+    gx, gwv = torch.autograd.grad(y, [x, wv], gv)
+    torch.cuda.synchronize()
+    lhs, scale = _dot(y, gv), float(y.double().norm() * gv.double().norm())
+    _adjoint_ok(lhs, _dot(x, gx), scale, "<f2v(x), g> = <x, grad_input>")
+    _adjoint_ok(lhs, _dot(wv, gwv), scale, "<f2v(x), g> = <filter, grad_filter>")
+    f_np = f.astype(np.int64)
+    x_np, wv_np, cf_np = (a.detach().cpu().numpy().astype(np.float64) for a in (x, wv, coeff))
+    pick_v = np.sort(rng.choice(nv, 1000, replace=False))
+    is_pick = np.zeros(nv, bool)
+    is_pick[pick_v] = True
+    around = np.nonzero(is_pick[f_np].any(1))[0]
+    sub = loops.f2v_fwd(x_np[around], wv_np, cf_np[around], f[around].astype(np.int32), nfc_np, np.arange(nv, dtype=np.int32))
+    assert_close(y.detach()[torch.from_numpy(pick_v).to(cuda)], sub[pick_v], "f2v out, sampled vertices" + tag)
+    pick_f = np.sort(rng.choice(nf, 1000, replace=False))
+    sub_gin, _ = loops.f2v_bwd(gv.cpu().numpy().astype(np.float64), x_np[pick_f], wv_np, cf_np[pick_f],
+                               f[pick_f].astype(np.int32), nfc_np, np.arange(nv, dtype=np.int32))
+    assert_close(gx[torch.from_numpy(pick_f).to(cuda)], sub_gin, "f2v grad_input, sampled facets" + tag)
+    _, ref_gwv = R.f2v_bwd(gv.cpu().double(), x.detach().cpu().double(), wv.detach().cpu().double(), coeff.cpu().double(),
+                           face.cpu(), nfc.cpu(), ident.cpu())
+    assert_close(gwv, ref_gwv.numpy(), "f2v grad_filter, element by element" + tag)
+    del y, gx, x
+
+    xv = torch.randn(nv, C, device=cuda, generator=gen).requires_grad_(True)
+    w3 = torch.randn(3, C, 1, device=cuda, generator=gen).requires_grad_(True)
+    gf = torch.randn(nf, C, device=cuda, generator=gen)
+    z = conv3d.vertex2facet(xv, w3, face)
+    gxv, gw3 = torch.autograd.grad(z, [xv, w3], gf)
+    torch.cuda.synchronize()
+    lhs, scale = _dot(z, gf), float(z.double().norm() * gf.double().norm())
+    _adjoint_ok(lhs, _dot(xv, gxv), scale, "<v2f(x), g> = <x, grad_input>")
+    _adjoint_ok(lhs, _dot(w3, gw3), scale, "<v2f(x), g> = <filter, grad_filter>")
+    sub_z = loops.v2f_fwd(xv.detach().cpu().numpy().astype(np.float64), w3.detach().cpu().numpy().astype(np.float64), f[pick_f])
+    assert_close(z.detach()[torch.from_numpy(pick_f).to(cuda)], sub_z, "v2f out, sampled facets" + tag)

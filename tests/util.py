@@ -45,7 +45,7 @@ def assert_as_good_as_f32(y, ref64, ref32, what, factor=2.0):
     e = rel_err(y.detach().cpu().numpy() if isinstance(y, torch.Tensor) else y, ref64)
     e32 = rel_err(ref32, ref64)
     # reported as the ratio to the float32 oracle's error (floored as the bound is) against the factor allowed
-    MEASURED.append((what + " [error / float32 oracle's error]", e / max(e32, F32_FLOOR / (factor or 1.0)), factor or float("inf")))
+    MEASURED.append((what + (" [error / float32 oracle's error]" if factor else " [error / float32 oracle's error, cross-check path: reported only]"), e / max(e32, F32_FLOOR / (factor or 1.0)), factor or float("inf")))
     if factor is not None:
         assert e <= max(factor * e32, F32_FLOOR), "%s: error %.3e exceeds %g x the float32 oracle's %.3e" % (what, e, factor, e32)
     return e, e32

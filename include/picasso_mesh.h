@@ -363,6 +363,20 @@ int pmesh_dense_bwd(const float *grad_output, const float *input, const float *w
                     float *grad_weight, float *grad_bias, void *workspace, size_t workspace_bytes,
                     int64_t N, int Ci, int Co, pmesh_stream_t stream);
 
+/* vertex2facet (depth multiplier 1) and its tail as ONE pass: replaces mesh_conv3d.vertex2facet_forward
+ * (mesh_conv3d.cpp:123-152, kernel mesh_conv3d_gpu.cu:176-195) followed by the PyTorch ops of V2FConv3d.forward
+ * (picasso/mesh/layers.py:113-119):
+ *   output (Nf,Co) = act((sum_j filter[j] * input[face[:,j]]) . weight (C,Co) + bias) * scale + shift
+ * The facet rows of the convolution are formed in the loads of the product (three gathered vertex rows per facet,
+ * weighted per channel) and never pass through memory -- unless conv_rows (Nf,C) is given, which receives them for
+ * the backward pass (pmesh_dense_bwd takes them as its `input`, pmesh_v2f_bwd the gradient that comes out of it).
+ * filter (3,C) = the (3,C,1) filter of pmesh_v2f_fwd; C % 4 == 0, C <= 896; every face index in [0, Nv) (the
+ * caller's check, as for pmesh_v2f_fwd); bias, scale, shift, relu, relu_bits as in pmesh_dense_fwd. */
+int pmesh_v2f_dense_fwd(const float *input, const float *filter, const int32_t *face, const float *weight,
+                        const float *bias, const float *scale, const float *shift, int relu, float *output,
+                        uint32_t *relu_bits, float *conv_rows, int64_t Nv, int64_t Nf, int C, int Co,
+                        pmesh_stream_t stream);
+
 /* The same tail for a convolution that mixes the channels itself (F2FConv3d, picasso/mesh/layers.py:60-64:
  * outputs + biases, activation_fn, BatchNorm): output (N,C) = act(input + bias) * scale + shift, one pass;
  * output may be input.  relu_bits as in pmesh_dense_fwd (NULL, or N * C/32 words when C % 32 == 0 and the rows

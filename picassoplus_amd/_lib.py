@@ -11,7 +11,7 @@ from ctypes import c_char_p, c_float, c_int, c_int64, c_size_t, c_void_p
 _HERE = os.path.dirname(os.path.abspath(__file__))
 # PICASSO_MESH_LIB points at an alternative build of the same ABI (kernel experiments)
 LIB_PATH = os.environ.get("PICASSO_MESH_LIB") or os.path.join(_HERE, "csrc", "libpicasso_mesh.so")
-ABI_VERSION = 17
+ABI_VERSION = 18
 
 P, I, L, Z = c_void_p, c_int, c_int64, c_size_t
 
@@ -91,6 +91,7 @@ SIGNATURES = {
     "pmesh_edge_costs": (I, [P, P, P, P, P, L, I, P]),
     "pmesh_cluster_vertices_host": (I, [P, P, L, I, I, I, P]),
     "pmesh_dense_fwd": (I, [P, P, P, P, P, I, P, P, L, I, I, P]),
+    "pmesh_v2f_dense_fwd": (I, [P, P, P, P, P, P, P, I, P, P, P, L, L, I, I, P]),
     "pmesh_dense_bwd_workspace_bytes": (Z, [L, I, I]),
     "pmesh_dense_bwd": (I, [P, P, P, P, P, P, P, P, P, Z, L, I, I, P]),
     "pmesh_bias_act_fwd": (I, [P, P, P, P, I, P, P, L, I, P]),

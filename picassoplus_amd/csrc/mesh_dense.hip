@@ -62,12 +62,94 @@ constexpr int kStageStride = 68;                       // floats per staged row:
 constexpr int kStageWave = 32 * kStageStride;          // per wavefront
 
 // MASK: 0 = rows as they are, 1 = a float array of the rows' shape decides (entries > 0 pass),
-// 2 = one bit per entry decides (32-bit words, W per row, bit c % 32 of word c / 32).
+// 2 = one bit per entry decides (32-bit words, W per row, bit c % 32 of word c / 32),
+// 3 = the rows are vertex2facet rows formed while they are loaded (the convolution in front of the tail never
+//     leaves its result in memory unless asked to): row f, column c = sum_j vfilt[j][c] * a[face[f][j]][c].
 template <bool VEC, int MASK> struct RowBlock {
     float v[32];
     float m[MASK == 1 ? 32 : 1];
     unsigned w[MASK == 2 ? (VEC ? 8 : 32) : 1];
+    float g[MASK == 3 ? 64 : 1];              // the rows of the second and third corner
 };
+
+// What mode 3 reads besides the vertex rows `a` (Nv x K): facets (N x 3), the per-corner channel weights (3 x K),
+// and where the formed rows go as well when the caller keeps them for the backward pass (N x K, or null).
+struct RowGather {
+    const int *face;
+    const float *vfilt;
+    float *keep;
+};
+
+// The 96 corner indices of a 32-facet tile, spread over the wavefront: lane l holds entries l and 64 + l.
+struct TileCorners {
+    int lo, hi;
+};
+__device__ __forceinline__ TileCorners corners_issue(const int *__restrict__ face, int64_t tile, int64_t N, int lane)
+{
+    TileCorners c;
+    const int64_t base = tile * 96, end = 3 * N;
+    c.lo = base + lane < end ? face[base + lane] : 0;
+    c.hi = (lane < 32 && base + 64 + lane < end) ? face[base + 64 + lane] : 0;
+    return c;
+}
+// corner j of row r of the tile, read from the lane that holds it
+__device__ __forceinline__ int corner_of(const TileCorners &c, int r, int j)
+{
+    const int e = 3 * r + j;
+    const int a = __builtin_amdgcn_ds_bpermute((e & 63) * 4, c.lo), b = __builtin_amdgcn_ds_bpermute((e & 63) * 4, c.hi);
+    return e < 64 ? a : b;
+}
+
+// Mode 3, the fetches of a 32 x 64 block: three gathered 16-byte pieces per row and 16-lane group.
+__device__ __forceinline__ void rows_issue_gather(RowBlock<true, 3> &b, const float *__restrict__ a, const TileCorners &tc,
+                                                  int64_t tile, int q, int64_t N, int K, int lane)
+{
+    const int col = q + 4 * (lane & 15), sub = lane >> 4;
+    const int64_t left = N - tile * 32;
+    // 32-bit byte offsets from the scalar base (the launcher checks that the vertex array stays below 4 GiB)
+    const unsigned row_bytes = (unsigned)K * 4u, col_bytes = (unsigned)col * 4u;
+    const char *base = reinterpret_cast<const char *>(a);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const int r = 4 * i + sub;
+        const int v0 = corner_of(tc, r, 0), v1 = corner_of(tc, r, 1), v2 = corner_of(tc, r, 2);
+        float4 t0 = make_float4(0.f, 0.f, 0.f, 0.f), t1 = t0, t2 = t0;
+        if (r < left && col < K) {
+            t0 = *reinterpret_cast<const float4 *>(base + ((unsigned)v0 * row_bytes + col_bytes));
+            t1 = *reinterpret_cast<const float4 *>(base + ((unsigned)v1 * row_bytes + col_bytes));
+            t2 = *reinterpret_cast<const float4 *>(base + ((unsigned)v2 * row_bytes + col_bytes));
+        }
+        b.v[4 * i] = t0.x; b.v[4 * i + 1] = t0.y; b.v[4 * i + 2] = t0.z; b.v[4 * i + 3] = t0.w;
+        b.g[4 * i] = t1.x; b.g[4 * i + 1] = t1.y; b.g[4 * i + 2] = t1.z; b.g[4 * i + 3] = t1.w;
+        b.g[32 + 4 * i] = t2.x; b.g[32 + 4 * i + 1] = t2.y; b.g[32 + 4 * i + 2] = t2.z; b.g[32 + 4 * i + 3] = t2.w;
+    }
+}
+
+// Mode 3, the block into the stage: the three corners' pieces weighted per channel (corner 0 first, as the
+// reference sums them, mesh_conv3d_gpu.cu:176-195), and into `keep` for the first column block's workgroups.
+__device__ __forceinline__ void rows_commit_gather(const RowBlock<true, 3> &b, float *stage, const float *__restrict__ vfilt,
+                                                   float *__restrict__ keep, int64_t tile, int q, int64_t N, int K, int lane)
+{
+    const int col = q + 4 * (lane & 15), sub = lane >> 4;
+    float4 f0 = make_float4(0.f, 0.f, 0.f, 0.f), f1 = f0, f2 = f0;
+    if (col < K) {
+        f0 = *reinterpret_cast<const float4 *>(vfilt + col);
+        f1 = *reinterpret_cast<const float4 *>(vfilt + K + col);
+        f2 = *reinterpret_cast<const float4 *>(vfilt + 2 * K + col);
+    }
+    const int64_t left = N - tile * 32;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        float4 t;
+        t.x = fmaf(f2.x, b.g[32 + 4 * i], fmaf(f1.x, b.g[4 * i], f0.x * b.v[4 * i]));
+        t.y = fmaf(f2.y, b.g[32 + 4 * i + 1], fmaf(f1.y, b.g[4 * i + 1], f0.y * b.v[4 * i + 1]));
+        t.z = fmaf(f2.z, b.g[32 + 4 * i + 2], fmaf(f1.z, b.g[4 * i + 2], f0.z * b.v[4 * i + 2]));
+        t.w = fmaf(f2.w, b.g[32 + 4 * i + 3], fmaf(f1.w, b.g[4 * i + 3], f0.w * b.v[4 * i + 3]));
+        *reinterpret_cast<float4 *>(stage + (4 * i + sub) * kStageStride + 4 * (lane & 15)) = t;
+        if (keep && 4 * i + sub < left && col < K)
+            *reinterpret_cast<float4 *>(keep + (tile * 32 + 4 * i + sub) * K + col) = t;
+    }
+}
 
 template <bool VEC, int MASK>
 __device__ __forceinline__ void rows_issue(RowBlock<VEC, MASK> &b, const float *__restrict__ a,
@@ -179,7 +261,8 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void dense_rows_k(const f
                                                        const float *__restrict__ bias,
                                                        const float *__restrict__ scale,
                                                        const float *__restrict__ shift, int relu,
-                                                       float *__restrict__ out, int64_t N, int K, int Kpad, int C)
+                                                       float *__restrict__ out, int64_t N, int K, int Kpad, int C,
+                                                       RowGather gat)
 {
     extern __shared__ __attribute__((aligned(16))) float lds[];
     constexpr int NC = NT * 32;
@@ -229,21 +312,47 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void dense_rows_k(const f
     bool have = tile < ntiles;
     RowBlock<VEC, MASK> blk;
     const int Win = (K + 31) >> 5, Wout = (C + 31) >> 5;
-    if (have) rows_issue<VEC, MASK>(blk, a, mask, bits_in, Win, tile, 0, N, K, lane);
+    // mode 3: the corner indices of a tile are fetched one tile ahead of its rows
+    TileCorners tc = {0, 0}, tc_next = {0, 0};
+    float *keep = nullptr;
+    if constexpr (MASK == 3) {
+        static_assert(MASK != 3 || VEC, "rows formed on load come in 16-byte pieces");
+        keep = col0 == 0 ? gat.keep : nullptr;
+        // The gathered rows of a block are fetched when the block is due, not a block ahead: three corners are 96
+        // registers in flight, which do not fit beside the product's; the other wavefronts of the CU cover the wait.
+        if (have) {
+            tc = corners_issue(gat.face, tile, N, lane);
+            tc_next = corners_issue(gat.face, tile + stride, N, lane);
+        }
+    } else {
+        if (have) rows_issue<VEC, MASK>(blk, a, mask, bits_in, Win, tile, 0, N, K, lane);
+    }
     f32x16 acc[NT];
 #pragma unroll
     for (int j = 0; j < NT; ++j)
 #pragma unroll
         for (int i = 0; i < 16; ++i) acc[j][i] = 0.f;
     while (have) {
-        rows_commit<VEC, MASK>(blk, stage, lane);
+        if constexpr (MASK == 3) {
+            rows_issue_gather(blk, a, tc, tile, q, N, K, lane);
+            rows_commit_gather(blk, stage, gat.vfilt, keep, tile, q, N, K, lane);
+        } else {
+            rows_commit<VEC, MASK>(blk, stage, lane);
+        }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         int64_t ntile = tile;
         int nq = q + kDenseChunk;
         if (nq >= Kpad) { nq = 0; ntile += stride; }
         const bool nhave = ntile < ntiles;
-        if (nhave) rows_issue<VEC, MASK>(blk, a, mask, bits_in, Win, ntile, nq, N, K, lane);
+        if constexpr (MASK == 3) {
+            if (nhave && nq == 0) {
+                tc = tc_next;
+                tc_next = corners_issue(gat.face, ntile + stride, N, lane);
+            }
+        } else {
+            if (nhave) rows_issue<VEC, MASK>(blk, a, mask, bits_in, Win, ntile, nq, N, K, lane);
+        }
         const float *xs = stage + n * kStageStride + h * 32;
         if constexpr (X3) {
             // lane (r, h) owns reduction entries q + 32h + 8t + e of row r in step t, the slab block (q + 32h)/8 + t
@@ -618,6 +727,7 @@ struct RowsArgs {
     float *out;
     int64_t N;
     int K, Kpad, C;
+    RowGather gat;
 };
 
 template <int NT, int NW, bool VEC, int MASK, bool X3>
@@ -634,7 +744,7 @@ static void launch_rows_nt(int64_t ntiles, unsigned gy, size_t lds, hipStream_t 
     if (gx < 1) gx = 1;
     if (gx > wanted) gx = wanted;
     dense_rows_k<NT, NW, VEC, MASK, X3><<<dim3((unsigned)(gx * gy)), dim3(NW * 64), lds, st>>>(
-        p.a, p.mask, p.bits_in, p.bits_out, p.w, p.wk, p.wc, p.bias, p.scale, p.shift, p.relu, p.out, p.N, p.K, p.Kpad, p.C);
+        p.a, p.mask, p.bits_in, p.bits_out, p.w, p.wk, p.wc, p.bias, p.scale, p.shift, p.relu, p.out, p.N, p.K, p.Kpad, p.C, p.gat);
 }
 
 template <bool VEC, int MASK, bool X3>
@@ -668,7 +778,7 @@ static void launch_rows(int NT, int NW, int64_t ntiles, unsigned gy, size_t lds,
 // bits_in (one bit per entry) when given; bits_out receives one bit per output entry, set where act(.) > 0.
 static int dense_rows(const char *name, const float *a, const float *mask, const unsigned *bits_in, unsigned *bits_out,
                       const float *w, int64_t wk, int64_t wc, const float *bias, const float *scale, const float *shift,
-                      int relu, float *out, int64_t N, int K, int C, hipStream_t st)
+                      int relu, float *out, int64_t N, int K, int C, hipStream_t st, const RowGather *gather = nullptr)
 {
     PM_REQUIRE(K > 0 && C > 0 && K <= kDenseMaxK && C <= (1 << 20), "%s: channel counts out of range (%d, %d)", name, K, C);
     PM_REQUIRE(N * (int64_t)(K > C ? K : C) < (int64_t(1) << 40), "%s: sizes too large", name);
@@ -702,18 +812,27 @@ static int dense_rows(const char *name, const float *a, const float *mask, const
         x3 = false;
     }
     PM_REQUIRE(lds <= kDenseLdsMax, "%s: reduction length %d too large", name, K);
+    if (gather && NT > 2) {
+        // rows formed on load: 96 registers of gathered pieces beside at most two accumulator tiles
+        NT = 2;
+        lds = (size_t)Kpad * NT * 32 * (x3 ? 6 : 4) + (size_t)NW * kStageWave * sizeof(float);
+    }
     const int64_t ntiles = ceil_div(N, 32);
     const unsigned gy = (unsigned)ceil_div(C, NT * 32);
     const bool vec = (K % 4 == 0) && aligned16(a) && (!mask || aligned16(mask));
-    const RowsArgs p{a, mask, bits_in, bits_out, w, wk, wc, bias, scale, shift, relu, out, N, K, Kpad, C};
-    const int mode = bits_in ? 2 : mask ? 1 : 0;
+    const RowsArgs p{a, mask, bits_in, bits_out, w, wk, wc, bias, scale, shift, relu, out, N, K, Kpad, C,
+                     gather ? *gather : RowGather{nullptr, nullptr, nullptr}};
+    const int mode = gather ? 3 : bits_in ? 2 : mask ? 1 : 0;
+    PM_REQUIRE(mode != 3 || (vec && aligned16(gather->vfilt) && (!gather->keep || aligned16(gather->keep))),
+               "%s: rows formed on load need a multiple of 4 channels and 16-byte aligned arrays", name);
 #define PM_PICK(V, M)                                                          \
     do {                                                                       \
         if (x3) launch_rows<V, M, true>(NT, NW, ntiles, gy, lds, st, p);       \
         else launch_rows<V, M, false>(NT, NW, ntiles, gy, lds, st, p);         \
     } while (0)
     if (vec) {
-        if (mode == 2) PM_PICK(true, 2);
+        if (mode == 3) PM_PICK(true, 3);
+        else if (mode == 2) PM_PICK(true, 2);
         else if (mode == 1) PM_PICK(true, 1);
         else PM_PICK(true, 0);
     } else {
@@ -790,6 +909,24 @@ extern "C" int pmesh_dense_fwd(const float *input, const float *weight, const fl
     PM_REQUIRE(input && weight && output, "dense_fwd: null pointer");
     return dense_rows("dense_fwd", input, nullptr, nullptr, relu_bits, weight, Co, 1, bias, scale, shift, relu, output, N,
                       Ci, Co, (hipStream_t)stream);
+}
+
+extern "C" int pmesh_v2f_dense_fwd(const float *input, const float *filter, const int32_t *face, const float *weight,
+                                   const float *bias, const float *scale, const float *shift, int relu, float *output,
+                                   uint32_t *relu_bits, float *conv_rows, int64_t Nv, int64_t Nf, int C, int Co,
+                                   pmesh_stream_t stream)
+{
+    clear_error();
+    PM_REQUIRE(Nv >= 0 && Nf >= 0, "v2f_dense_fwd: negative size");
+    if (Nf == 0) return 0;
+    PM_REQUIRE(Nv > 0, "v2f_dense_fwd: facets without vertices");
+    PM_REQUIRE(input && filter && face && weight && output, "v2f_dense_fwd: null pointer");
+    PM_REQUIRE(Nv <= INT32_MAX && Nf <= INT32_MAX / 3, "v2f_dense_fwd: sizes exceed int32 indexing");
+    PM_REQUIRE(C > 0 && C % 4 == 0, "v2f_dense_fwd: the channel count must be a multiple of 4 (got %d)", C);
+    PM_REQUIRE(Nv * (int64_t)C * 4 < (int64_t(1) << 32), "v2f_dense_fwd: vertex array too large for 32-bit offsets");
+    const RowGather gat{face, filter, conv_rows};
+    return dense_rows("v2f_dense_fwd", input, nullptr, nullptr, relu_bits, weight, Co, 1, bias, scale, shift, relu, output, Nf,
+                      C, Co, (hipStream_t)stream, &gat);
 }
 
 extern "C" size_t pmesh_dense_bwd_workspace_bytes(int64_t N, int Ci, int Co)

@@ -222,6 +222,22 @@ class V2FConv3d(_SeparableConv):
     def forward(self, inputs, face):
         spatial_filter = torch.matmul(self._corners(inputs.device), self.spatial_weights)
         spatial_filter = spatial_filter.reshape([3, self.in_channels, self.multiplier])
+        relu = isinstance(self.activation_fn, nn.ReLU)
+        weights = self.depth_weights
+        if ((relu or self.activation_fn is None) and max(weights.shape) <= dense.MAX_CHANNELS
+                and inputs.dim() == 2 and inputs.is_contiguous() and dense.v2f_dense_supported(inputs, spatial_filter, weights)):
+            # the convolution, the pointwise product, the bias and the activation in one native pass: the facet rows
+            # of the convolution are formed inside the product's loads (and kept only for a backward pass); a batch
+            # norm that only applies its running statistics rides along when no gradients are recorded
+            spatial_filter = spatial_filter.contiguous()
+            biases = self.biases.reshape(-1)
+            if self.with_bn and not torch.is_grad_enabled():
+                frozen = self._frozen_norm()
+                if frozen is not None:
+                    return dense.v2f_dense_forward(inputs, spatial_filter, face, weights.contiguous(), biases.contiguous(),
+                                                   relu, frozen[0], frozen[1])
+            outputs = dense.v2f_dense(inputs, spatial_filter, face, weights.contiguous(), biases, relu)
+            return self.BatchNorm(outputs) if self.with_bn else outputs
         outputs = conv3d.vertex2facet(inputs, spatial_filter, face)
         return self._mix(outputs)
 

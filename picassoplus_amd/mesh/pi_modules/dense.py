@@ -109,6 +109,88 @@ def dense_tail(input, weight, bias, relu=True):
     return DenseTailFunction.apply(input, weight, bias, relu)
 
 
+# ---------------------------------------------------------------- vertex2facet and its tail in one pass
+def v2f_dense_supported(input, filter, weight):
+    """The one-pass form takes depth multiplier 1, a multiple of 4 channels and what the tail itself takes."""
+    C = input.shape[1]
+    return (input.dtype == F32 and filter.shape[2] == 1 and C % 4 == 0 and 0 < C <= MAX_CHANNELS
+            and weight.shape[1] >= 1 and input.data_ptr() % 16 == 0 and filter.data_ptr() % 16 == 0)
+
+
+def v2f_dense_forward(input, filter, face, weight, bias=None, relu=True, scale=None, shift=None, with_bits=False,
+                      keep_rows=False):
+    """act(vertex2facet(input, filter, face) @ weight + bias) * scale + shift in one kernel: the facet rows of the
+    convolution are formed inside the loads of the product.  input (Nv,C), filter (3,C,1), face (Nf,3) int32,
+    weight (C,Co) -> (Nf,Co).  ``keep_rows`` also returns the convolution's rows (Nf,C), which the backward pass
+    needs; ``with_bits`` the ReLU mask as bits.  Returns out, or (out, bits, rows) when either is asked for."""
+    from .. import topology
+    from ._check import I32
+    check_input(input, "input", 2, F32)
+    check_input(filter, "filter", 3, F32)
+    check_input(face, "face", 2, I32)
+    check_input(weight, "weight", 2, F32)
+    Nv, C = input.shape
+    Nf, Co = face.shape[0], weight.shape[1]
+    if tuple(filter.shape) != (3, C, 1):
+        raise RuntimeError("3 filters required, or input Channel size error of the filter")
+    if face.shape[1] != 3:
+        raise RuntimeError("face must have shape (NfIn, 3)")
+    if weight.shape[0] != C:
+        raise RuntimeError("weight must have shape (in_channels, out_channels)")
+    if C % 4 or C > MAX_CHANNELS:
+        raise RuntimeError("the one-pass vertex2facet tail takes a multiple of 4 channels, at most %d" % MAX_CHANNELS)
+    for name, t in (("bias", bias), ("scale", scale), ("shift", shift)):
+        if t is not None:
+            check_input(t, name, 1, F32)
+            if t.shape[0] != Co:
+                raise RuntimeError("%s must have out_channels entries" % name)
+    dev = same_device(input, filter, face, weight, *[t for t in (bias, scale, shift) if t is not None])
+    if Nf:
+        topology._check_range_cached(face, Nv)
+    with torch.cuda.device(dev):
+        out = torch.empty((Nf, Co), dtype=F32, device=dev)
+        bits = torch.empty((Nf, (Co + 31) // 32), dtype=torch.int32, device=dev) if with_bits else None
+        rows = torch.empty((Nf, C), dtype=F32, device=dev) if keep_rows else None
+        _lib.call("pmesh_v2f_dense_fwd", input.data_ptr(), filter.data_ptr(), face.data_ptr(), weight.data_ptr(),
+                  _ptr(bias), _ptr(scale), _ptr(shift), 1 if relu else 0, out.data_ptr(), _ptr(bits), _ptr(rows),
+                  Nv, Nf, C, Co, stream_of(input))
+    return (out, bits, rows) if (with_bits or keep_rows) else out
+
+
+class V2FDenseFunction(torch.autograd.Function):
+    """vertex2facet, the product with the pointwise weights, the bias and a ReLU (or no activation) as ONE native
+    forward (picasso/mesh/layers.py:108-117 runs them as a native op and three PyTorch ops).  The convolution's rows
+    are kept only when a gradient will need them.  Backward: the tail's gradients from the kept rows, then the
+    convolution's from what the tail hands down."""
+
+    @staticmethod
+    def forward(ctx, input, filter, face, weight, bias, relu):
+        if face.requires_grad:
+            face.requires_grad = False
+        need = any(ctx.needs_input_grad[i] for i in (0, 1, 3, 4))
+        res = v2f_dense_forward(input, filter, face, weight, bias, relu, with_bits=bool(relu and need), keep_rows=need)
+        out, bits, rows = res if need else (res, None, None)
+        ctx.save_for_backward(input, filter, face, weight, bits, rows)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        from . import mesh_conv3d
+        input, filter, face, weight, bits, rows = ctx.saved_tensors
+        need_conv = ctx.needs_input_grad[0] or ctx.needs_input_grad[1]
+        grows, gw, gb = dense_tail_backward(grad_output.contiguous(), rows, weight, None, need_input=need_conv, relu_bits=bits)
+        gin = gfilt = None
+        if need_conv:
+            gin, gfilt = mesh_conv3d.vertex2facet_backward(grows, input, filter, face)
+        return (gin if ctx.needs_input_grad[0] else None, gfilt if ctx.needs_input_grad[1] else None, None,
+                gw if ctx.needs_input_grad[3] else None, gb if ctx.needs_input_grad[4] else None, None)
+
+
+def v2f_dense(input, filter, face, weight, bias, relu=True):
+    """act(vertex2facet(input, filter, face) @ weight + bias) with gradients for input, filter, weight and bias."""
+    return V2FDenseFunction.apply(input, filter, face, weight, bias, relu)
+
+
 # ---------------------------------------------------------------- the tail without a product
 def bits_supported(C, *tensors):
     """The bit form of the ReLU mask of ``bias_act`` needs whole 32-column words and 16-byte aligned rows."""

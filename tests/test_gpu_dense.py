@@ -248,3 +248,86 @@ def test_f2f_module_tail_eval_matches_float64(cuda, act):
         sh = layers.SphHarmCoeff(3)(torch.from_numpy(bary).to(cuda, torch.float32))
         out = mod(tex.to(cuda, torch.float32), sh, torch.from_numpy(counts).to(cuda))
     assert_close(out, y.detach().numpy(), "F2FConv3d eval output")
+
+
+V2F_SHAPES = [("tetra", 4, 1), ("octa", 8, 32), ("sphere2", 32, 64), ("sphere3", 64, 64), ("torus", 64, 128), ("room_small", 96, 20),
+              ("sphere2", 128, 300), ("fans", 12, 7), ("shapes_small", 256, 256)]
+
+
+@pytest.mark.parametrize("mesh,c,co", V2F_SHAPES)
+@pytest.mark.parametrize("relu", [True, False])
+def test_v2f_dense_one_pass(cuda, product_path, mesh, c, co, relu):
+    """vertex2facet + pointwise product + bias + ReLU as one kernel against the float64 oracle composition
+    (oracle: v2f_fwd, then dense_tail_fwd), forward with and without the kept rows / mask bits / frozen norm, and all
+    four gradients through autograd against the oracle's explicit backward formulas."""
+    from oracle import loops
+    from util import dev, mesh_case
+    say("case v2f_dense", product_path, mesh, c, co, relu)
+    v, f = mesh_case(mesh)
+    nv, nf = v.shape[0], f.shape[0]
+    rng = np.random.default_rng(c * 1000 + co)
+    x = rng.uniform(-1, 1, (nv, c)).astype(np.float32)
+    filt = rng.normal(0, 0.6, (3, c, 1)).astype(np.float32)
+    w = (rng.normal(0, 1, (c, co)) / np.sqrt(c)).astype(np.float32)
+    b = rng.normal(0, 0.3, co).astype(np.float32)
+    g = rng.normal(0, 1, (nf, co)).astype(np.float32)
+    xd, fd, wd, bd, gd, face = (dev(a, cuda) for a in (x, filt, w, b, g, f))
+    rows64 = loops.v2f_fwd(x.astype(np.float64), filt.astype(np.float64), f)
+    T = lambda a: torch.from_numpy(np.ascontiguousarray(a, np.float64))
+    ref = torch_ref.dense_tail_fwd(T(rows64), T(w), T(b), relu).numpy()
+    out = dense.v2f_dense_forward(xd, fd, face, wd, bd, relu)
+    out2, bits, rows = dense.v2f_dense_forward(xd, fd, face, wd, bd, relu, with_bits=True, keep_rows=True)
+    torch.cuda.synchronize()
+    assert_close(out, ref, "v2f_dense forward")
+    assert torch.equal(out, out2)
+    assert_close(rows, rows64, "v2f_dense kept rows")
+    cols = torch.arange(co, device=cuda)
+    if relu:
+        assert torch.equal(((bits[:, cols // 32] >> (cols % 32)) & 1).bool(), out > 0)
+    # the same bits as the two native passes it replaces make
+    from picassoplus_amd.mesh.pi_modules import mesh_conv3d
+    two = dense.dense_tail_forward(mesh_conv3d.vertex2facet_forward(xd, fd, face), wd, bd, relu)
+    assert_close(out, two.double().cpu().numpy(), "v2f_dense against the two passes", 2e-6)
+    scale, shift = dev(rng.uniform(0.5, 2, co).astype(np.float32), cuda), dev(rng.normal(0, 1, co).astype(np.float32), cuda)
+    outn = dense.v2f_dense_forward(xd, fd, face, wd, bd, relu, scale, shift)
+    assert_close(outn, ref * scale.double().cpu().numpy() + shift.double().cpu().numpy(), "v2f_dense with scale/shift")
+    # gradients
+    xg, fg, wg, bg = (t.clone().requires_grad_(True) for t in (xd, fd, wd, bd))
+    y = dense.v2f_dense(xg, fg, face, wg, bg, relu)
+    assert torch.equal(y.detach(), out)
+    y.backward(gd)
+    torch.cuda.synchronize()
+    z = rows64 @ w.astype(np.float64) + b
+    safe = (np.abs(z) > 1e-5 * np.abs(z).max()) | (not relu)
+    out64 = np.where(safe, ref, out.double().cpu().numpy())
+    grows, gw, gb = torch_ref.dense_tail_bwd(T(g), T(rows64), T(w), T(out64) if relu else None)
+    gx, gf = loops.v2f_bwd(grows.numpy(), x.astype(np.float64), filt.astype(np.float64), f)
+    assert_close(xg.grad, gx, "v2f_dense grad_input")
+    assert_close(fg.grad, gf, "v2f_dense grad_filter")
+    assert_close(wg.grad, gw.numpy(), "v2f_dense grad_weight")
+    assert_close(bg.grad, gb.numpy(), "v2f_dense grad_bias")
+    # nothing is kept when no gradient is recorded
+    with torch.no_grad():
+        assert torch.equal(dense.v2f_dense(xd, fd, face, wd, bd, relu), out)
+
+
+def test_v2f_module_takes_the_one_pass_form(cuda):
+    """V2FConv3d calls one native forward where the reference runs the convolution and three PyTorch ops; other depth
+    multipliers and activations keep the separate passes.  Both give the oracle's result (test_gpu_modules.py)."""
+    from picassoplus_amd import _lib
+    from util import dev, mesh_case
+    v, f = mesh_case("sphere2")
+    x = torch.randn(v.shape[0], 32, device=cuda)
+    face = dev(f, cuda)
+    calls = []
+    _lib.set_call_hook(lambda name, phase: calls.append(name) if phase == "begin" else None)
+    try:
+        layers.V2FConv3d(32, 64, 3, with_bn=False).to(cuda)(x, face)
+        one = list(calls)
+        del calls[:]
+        layers.V2FConv3d(32, 64, 3, depth_multiplier=2, with_bn=False).to(cuda)(x, face)
+        two = list(calls)
+    finally:
+        _lib.set_call_hook(None)
+    assert [c for c in one if c != "pmesh_sph_harm"] == ["pmesh_v2f_dense_fwd"], one      # (the corner basis, first call only)
+    assert "pmesh_v2f_fwd" in two and "pmesh_dense_fwd" in two, two

@@ -137,10 +137,27 @@ def edge_costs(vertex, quadric, edge_vi, edge_vj, dtype=np.float64, return_rcond
     return (cost, rcond) if return_rcond else cost
 
 
-def contraction_order(cost, edge_vi, nv_cumsum):
-    """DETERMINISTIC: candidate edges by (sample, cost, vi, vj), NaN costs last; the reference sorts each sample's
-    costs with thrust::sort_by_key and leaves ties to it (decimate_gpu.cu:682-705).  returns (perm, sample[perm])."""
-    by_cost = np.argsort(cost, kind="stable")
+def edge_mix(edge_vi, edge_vj):
+    """32-bit mix of an edge's end points: what orders candidate edges of EQUAL cost.  Flat regions give thousands of
+    edges the same (zero) cost; ordered by (vi, vj) the greedy clustering would sweep them one after the other along the
+    vertex numbering, ordered by this mix their choices are local (and can be made in parallel rounds)."""
+    m = 0xFFFFFFFF
+    h = ((edge_vi.astype(np.int64) * 0x9E3779B1) & m) + ((edge_vj.astype(np.int64) * 0x85EBCA77) & m) & m
+    h &= m
+    h ^= h >> 15
+    h = (h * 0x2C1B3C6D) & m
+    h ^= h >> 12
+    h = (h * 0x297A2D39) & m
+    h ^= h >> 15
+    return h
+
+
+def contraction_order(cost, edge_vi, edge_vj, nv_cumsum):
+    """DETERMINISTIC: candidate edges by (sample, cost, mix(vi, vj), vi, vj), NaN costs last, -0 = +0; the reference
+    sorts each sample's costs with thrust::sort_by_key and leaves ties to it (decimate_gpu.cu:682-705).  The edges come
+    in ascending (vi, vj) order, so stable sorts keep that as the last criterion.  returns (perm, sample[perm])."""
+    by_mix = np.argsort(edge_mix(edge_vi, edge_vj), kind="stable")
+    by_cost = by_mix[np.argsort(np.asarray(cost)[by_mix], kind="stable")]
     sample = np.searchsorted(np.asarray(nv_cumsum, np.int64), edge_vi[by_cost].astype(np.int64), side="right")
     by_sample = np.argsort(sample, kind="stable")
     return by_cost[by_sample], sample[by_sample]
@@ -192,7 +209,7 @@ def simplify(vertex, face, geometry, nv_cumsum, mf_cumsum, nv2remove, use_area=T
     quadric, evi, evj = vertex_quadrics(vertex, face, geometry, use_area, wgt_bnd, dtype)
     if cost is None:
         cost = edge_costs(vertex, quadric, evi, evj, dtype)
-    perm, sample = contraction_order(np.asarray(cost), evi, nv_cumsum)
+    perm, sample = contraction_order(np.asarray(cost), evi, evj, nv_cumsum)
     vt_replace = np.zeros(nv, np.int32)
     bounds = np.searchsorted(sample, np.arange(len(nv_cumsum) + 1))
     for b in range(len(nv_cumsum)):

@@ -6,7 +6,8 @@
 // sum runs in a fixed order and every sort has a total order:
 //   vertex quadric   face contributions in ascending (facet, corner) order (vertex CSR), then boundary-edge
 //                    contributions in ascending (vi, vj) order (a second CSR over the boundary edges' endpoints)
-//   candidate edges  unique (vi < vj) pairs, ordered by (sample, cost, vi, vj)
+//   candidate edges  unique (vi < vj) pairs, ordered by (sample, cost, a 32-bit mix of (vi, vj), vi, vj): the mix keeps
+//                    the many equal-cost edges of flat regions from lining up along the vertex numbering
 //   clustering       the reference's two greedy passes over that order (clusterVertices, decimate_gpu.cu:561-614)
 // The sorts, scans and compactions between these steps are index plumbing done by the caller (radix sorts of
 // integer keys); this file holds what computes.
@@ -161,9 +162,210 @@ __global__ __launch_bounds__(kBlock) void edge_cost_k(const float *__restrict__ 
     }
 }
 
+// ----------------------------------------------------------------------------------------
+// The two greedy passes of the vertex clustering on the device, with the result of the serial host routine below.
+//
+// First pass (disjoint pairs, cheapest edge first).  For a total order of the edges the serial greedy choice is the
+// fixed point of: an edge both of whose end points are free, and which is the first such edge at BOTH of them, is
+// chosen; its end points are covered; repeat.  Every round costs two sweeps over the edge list (propose with an
+// integer atomic minimum per end point, select).  A budget that runs out stops the serial pass after its first
+// n_remove choices, which are the n_remove lowest-ranked edges of the fixed point: the caller cuts the chosen set
+// by rank.
+// Second pass (runs only when the first one did not exhaust the budget, i.e. after a MAXIMAL matching: no edge has
+// two free end points).  A free vertex then joins the cluster of the covered end of its first edge in the order
+// whose cluster has a representative other than vertex 0, and vertices that join never enable others to (all their
+// neighbours are covered already): one atomic minimum per edge finds each free vertex's edge, the caller cuts by
+// rank again, one sweep applies.
+// All atomics are integer minima / additions: the result does not depend on their order.
+constexpr int kNoEdge = 0x7FFFFFFF;
+
+__global__ __launch_bounds__(kBlock) void fill_int_k(int *__restrict__ p, int v, int64_t n)
+{
+    const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i < n) p[i] = v;
+}
+
+// status[1] <- 1 if an edge is not (vi < vj) inside [0, Nv): such an edge takes no part (the serial routine refuses it)
+__global__ __launch_bounds__(kBlock) void match_check_k(const int *__restrict__ evi, const int *__restrict__ evj, int64_t E,
+                                                        int64_t Nv, int *__restrict__ status)
+{
+    const int64_t r = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (r >= E) return;
+    const int a = evi[r], b = evj[r];
+    if (!(a >= 0 && a < b && b < Nv)) status[1] = 1;
+}
+
+__global__ __launch_bounds__(kBlock) void match_propose_k(const int *__restrict__ evi, const int *__restrict__ evj, int64_t E,
+                                                          int64_t Nv, const int *__restrict__ state, int *__restrict__ best)
+{
+    const int64_t r = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (r >= E) return;
+    const int a = evi[r], b = evj[r];
+    if (!(a >= 0 && a < b && b < Nv)) return;
+    if (state[a] | state[b]) return;
+    atomicMin(best + a, (int)r);
+    atomicMin(best + b, (int)r);
+}
+
+__global__ __launch_bounds__(kBlock) void match_select_k(const int *__restrict__ evi, const int *__restrict__ evj, int64_t E,
+                                                         int64_t Nv, int *__restrict__ state, const int *__restrict__ best,
+                                                         int *__restrict__ chosen)
+{
+    const int64_t r = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (r >= E) return;
+    const int a = evi[r], b = evj[r];
+    if (!(a >= 0 && a < b && b < Nv)) return;
+    if (best[a] == (int)r && best[b] == (int)r) {
+        chosen[r] = 1;
+        state[a] = 1;
+        state[b] = 1;
+    }
+}
+
+// status[0] <- 1 if an edge with two free end points is left
+__global__ __launch_bounds__(kBlock) void match_left_k(const int *__restrict__ evi, const int *__restrict__ evj, int64_t E,
+                                                       int64_t Nv, const int *__restrict__ state, int *__restrict__ status)
+{
+    const int64_t r = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (r >= E) return;
+    const int a = evi[r], b = evj[r];
+    if (!(a >= 0 && a < b && b < Nv)) return;
+    if (!(state[a] | state[b])) status[0] = 1;
+}
+
+__global__ __launch_bounds__(kBlock) void contract_pairs_k(const int *__restrict__ evi, const int *__restrict__ evj,
+                                                           const int *__restrict__ keep, int64_t E, int *__restrict__ vt_replace)
+{
+    const int64_t r = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (r >= E || !keep[r]) return;
+    vt_replace[evi[r]] = -evj[r];          // vi is contracted into vj (decimate_gpu.cu:568-585)
+    vt_replace[evj[r]] = 1;
+}
+
+// the covered and the free end of an edge with exactly one covered end, and the covered end's representative
+__device__ __forceinline__ bool attach_ends(int a, int b, const int *__restrict__ vt_replace, int &rep, int &fr)
+{
+    const int ra = vt_replace[a], rb = vt_replace[b];
+    const bool ca = ra != 0, cb = rb != 0;
+    if (ca == cb) return false;
+    fr = ca ? b : a;
+    const int cov = ca ? a : b, rc = ca ? ra : rb;
+    rep = rc < 0 ? -rc : cov;
+    return rep != 0;                        // -0 cannot say 'contracted into vertex 0'
+}
+
+__global__ __launch_bounds__(kBlock) void attach_propose_k(const int *__restrict__ evi, const int *__restrict__ evj,
+                                                           const int *__restrict__ sample, const int *__restrict__ open,
+                                                           int64_t E, int64_t Nv, const int *__restrict__ vt_replace,
+                                                           int *__restrict__ first_edge)
+{
+    const int64_t r = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (r >= E || !open[sample[r]]) return;
+    const int a = evi[r], b = evj[r];
+    if (!(a >= 0 && a < b && b < Nv)) return;
+    int rep, fr;
+    if (attach_ends(a, b, vt_replace, rep, fr)) atomicMin(first_edge + fr, (int)r);
+}
+
+__global__ __launch_bounds__(kBlock) void attach_flag_k(const int *__restrict__ evi, const int *__restrict__ evj,
+                                                        const int *__restrict__ sample, const int *__restrict__ open,
+                                                        int64_t E, int64_t Nv, const int *__restrict__ vt_replace,
+                                                        const int *__restrict__ first_edge, int *__restrict__ attaches)
+{
+    const int64_t r = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (r >= E) return;
+    int flag = 0;
+    const int a = evi[r], b = evj[r];
+    if (open[sample[r]] && a >= 0 && a < b && b < Nv) {
+        int rep, fr;
+        if (attach_ends(a, b, vt_replace, rep, fr)) flag = first_edge[fr] == (int)r;
+    }
+    attaches[r] = flag;
+}
+
+// first_edge tells the free end of a kept edge (vt_replace is being written here and can no longer say)
+__global__ __launch_bounds__(kBlock) void attach_apply_k(const int *__restrict__ evi, const int *__restrict__ evj,
+                                                         const int *__restrict__ keep, int64_t E, const int *__restrict__ first_edge,
+                                                         const int *__restrict__ pairs, int *__restrict__ vt_replace)
+{
+    const int64_t r = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (r >= E || !keep[r]) return;
+    const int a = evi[r], b = evj[r];
+    const int fr = first_edge[a] == (int)r ? a : b, cov = fr == a ? b : a;
+    const int rc = pairs[cov];              // the first pass's entry of the covered end: not written by this kernel
+    const int rep = rc < 0 ? -rc : cov;
+    vt_replace[fr] = -rep;
+    atomicAdd(vt_replace + rep, 1);
+}
+
 }  // namespace pmesh
 
 using namespace pmesh;
+
+extern "C" int pmesh_cluster_match(const int32_t *edge_vi, const int32_t *edge_vj, int64_t n_edges, int64_t Nv, int32_t *state,
+                                   int32_t *best, int32_t *chosen, int32_t *status, int rounds, pmesh_stream_t stream)
+{
+    clear_error();
+    PM_REQUIRE(n_edges >= 0 && n_edges < kNoEdge && Nv >= 0 && Nv <= INT32_MAX && rounds >= 1 && rounds <= 64,
+               "cluster_match: bad sizes");
+    PM_REQUIRE(status, "cluster_match: null status");
+    hipStream_t st = (hipStream_t)stream;
+    fill_int_k<<<dim3(1), dim3(kBlock), 0, st>>>(status, 0, 2);
+    PM_LAUNCHED("cluster_match(status)");
+    if (n_edges == 0 || Nv == 0) return 0;
+    PM_REQUIRE(edge_vi && edge_vj && state && best && chosen, "cluster_match: null pointer");
+    const dim3 ge((unsigned)ceil_div(n_edges, kBlock)), gv((unsigned)ceil_div(Nv, kBlock)), blk(kBlock);
+    match_check_k<<<ge, blk, 0, st>>>(edge_vi, edge_vj, n_edges, Nv, status);
+    for (int i = 0; i < rounds; ++i) {
+        fill_int_k<<<gv, blk, 0, st>>>(best, kNoEdge, Nv);
+        match_propose_k<<<ge, blk, 0, st>>>(edge_vi, edge_vj, n_edges, Nv, state, best);
+        match_select_k<<<ge, blk, 0, st>>>(edge_vi, edge_vj, n_edges, Nv, state, best, chosen);
+    }
+    match_left_k<<<ge, blk, 0, st>>>(edge_vi, edge_vj, n_edges, Nv, state, status);
+    PM_LAUNCHED("cluster_match");
+    return 0;
+}
+
+extern "C" int pmesh_cluster_contract_pairs(const int32_t *edge_vi, const int32_t *edge_vj, const int32_t *keep, int64_t n_edges,
+                                            int32_t *vt_replace, pmesh_stream_t stream)
+{
+    clear_error();
+    PM_REQUIRE(n_edges >= 0 && n_edges < kNoEdge, "cluster_contract_pairs: bad sizes");
+    if (n_edges == 0) return 0;
+    PM_REQUIRE(edge_vi && edge_vj && keep && vt_replace, "cluster_contract_pairs: null pointer");
+    contract_pairs_k<<<dim3((unsigned)ceil_div(n_edges, kBlock)), dim3(kBlock), 0, (hipStream_t)stream>>>(edge_vi, edge_vj, keep, n_edges, vt_replace);
+    PM_LAUNCHED("cluster_contract_pairs");
+    return 0;
+}
+
+extern "C" int pmesh_cluster_attach_propose(const int32_t *edge_vi, const int32_t *edge_vj, const int32_t *edge_sample,
+                                            const int32_t *sample_open, int64_t n_edges, int64_t Nv, const int32_t *vt_replace,
+                                            int32_t *first_edge, int32_t *attaches, pmesh_stream_t stream)
+{
+    clear_error();
+    PM_REQUIRE(n_edges >= 0 && n_edges < kNoEdge && Nv >= 0 && Nv <= INT32_MAX, "cluster_attach_propose: bad sizes");
+    if (n_edges == 0 || Nv == 0) return 0;
+    PM_REQUIRE(edge_vi && edge_vj && edge_sample && sample_open && vt_replace && first_edge && attaches, "cluster_attach_propose: null pointer");
+    hipStream_t st = (hipStream_t)stream;
+    const dim3 ge((unsigned)ceil_div(n_edges, kBlock)), gv((unsigned)ceil_div(Nv, kBlock)), blk(kBlock);
+    fill_int_k<<<gv, blk, 0, st>>>(first_edge, kNoEdge, Nv);
+    attach_propose_k<<<ge, blk, 0, st>>>(edge_vi, edge_vj, edge_sample, sample_open, n_edges, Nv, vt_replace, first_edge);
+    attach_flag_k<<<ge, blk, 0, st>>>(edge_vi, edge_vj, edge_sample, sample_open, n_edges, Nv, vt_replace, first_edge, attaches);
+    PM_LAUNCHED("cluster_attach_propose");
+    return 0;
+}
+
+extern "C" int pmesh_cluster_attach(const int32_t *edge_vi, const int32_t *edge_vj, const int32_t *keep, int64_t n_edges,
+                                    const int32_t *first_edge, const int32_t *pairs, int32_t *vt_replace, pmesh_stream_t stream)
+{
+    clear_error();
+    PM_REQUIRE(n_edges >= 0 && n_edges < kNoEdge, "cluster_attach: bad sizes");
+    if (n_edges == 0) return 0;
+    PM_REQUIRE(edge_vi && edge_vj && keep && first_edge && pairs && vt_replace && pairs != vt_replace, "cluster_attach: null or aliased pointer");
+    attach_apply_k<<<dim3((unsigned)ceil_div(n_edges, kBlock)), dim3(kBlock), 0, (hipStream_t)stream>>>(edge_vi, edge_vj, keep, n_edges, first_edge, pairs, vt_replace);
+    PM_LAUNCHED("cluster_attach");
+    return 0;
+}
 
 extern "C" int pmesh_vertex_quadrics(const float *geometry, const int32_t *rowptr, const int32_t *colidx, float *quadric,
                                      int64_t Nv, int use_area, pmesh_stream_t stream)

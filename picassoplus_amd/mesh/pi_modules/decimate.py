@@ -5,12 +5,16 @@ One round (``simplify``) = vertex quadrics from the facets and the boundary edge
 edge -> greedy vertex clustering in cost order -> cluster maps, contracted vertices, remapped facets.  The
 reference gets different ``vt_replace`` / ``vt_map`` from run to run (float atomics, unstable sorts, ties broken by
 whatever order a sort leaves); here every sum has a fixed order and the candidate edges a total order
-(sample, cost, vi, vj), so the maps are a function of the input alone.  The arithmetic runs in native kernels
-(``pmesh_vertex_quadrics``, ``pmesh_boundary_quadrics``, ``pmesh_edge_costs``), the serial clustering in a native host
-routine as in the reference (``pmesh_cluster_vertices_host``), the contraction is the average pooling op over the new
-maps; sorting / unique / scans of integer keys between them are PyTorch ops.
+(sample, cost, mix(vi, vj), vi, vj), so the maps are a function of the input alone.  The arithmetic runs in native kernels
+(``pmesh_vertex_quadrics``, ``pmesh_boundary_quadrics``, ``pmesh_edge_costs``), the greedy clustering on the device as a
+fixed-point iteration with the serial routine's result (``cluster_vertices_device``; the reference's serial host
+routine is ``pmesh_cluster_vertices_host``, kept as the checker and behind ``PMESH_DECIMATE_HOST_CLUSTERING=1``), the
+contraction is the average pooling op over the new maps; sorting / unique / scans of integer keys between them are
+PyTorch ops.
 """
 import ctypes
+import os
+import threading
 
 import numpy as np
 import torch
@@ -93,25 +97,47 @@ def edge_costs(vertexIn, quadric, edge_vi, edge_vj):
     return cost
 
 
-def contraction_order(cost, edge_vi, nvIn_cumsum):
-    """Order of the candidate edges: by sample, then cost (NaN last), then (vi, vj) -- the edges come in (vi, vj) order,
-    so two stable sorts do it.  returns (permutation, sample of each edge in that order)."""
-    by_cost = torch.sort(cost, stable=True).indices
+def edge_mix(edge_vi, edge_vj):
+    """32-bit mix of an edge's end points (int64 tensor): the criterion between candidate edges of EQUAL cost.  The
+    flat parts of a scene give most of its edges the same (zero) cost; in (vi, vj) order the greedy clustering would
+    sweep them one after the other along the vertex numbering (thousands of dependent steps), in the order of this mix
+    the choices are local and the device's rounds settle in a few dozen."""
+    m = 0xFFFFFFFF
+    h = (((edge_vi.long() * 0x9E3779B1) & m) + ((edge_vj.long() * 0x85EBCA77) & m)) & m
+    h = h ^ (h >> 15)
+    h = (h * 0x2C1B3C6D) & m
+    h = h ^ (h >> 12)
+    h = (h * 0x297A2D39) & m
+    return h ^ (h >> 15)
+
+
+def contraction_order(cost, edge_vi, edge_vj, nvIn_cumsum):
+    """Order of the candidate edges: by sample, then cost (NaN last), then ``edge_mix``, then (vi, vj) -- the edges come
+    in (vi, vj) order, so three stable sorts do it.  returns (permutation, sample of each edge in that order)."""
+    # one 64-bit key per edge: the cost as an integer that orders like the float (NaN above everything, -0 = +0) in the
+    # upper half, the mix in the lower; then the samples apart by a stable sort of their (8-bit, when they fit) numbers
+    bits = (cost + 0.0).view(torch.int32).long()
+    ordered = torch.where(bits >= 0, bits, -(bits + 2147483648) - 1)               # negative floats: larger magnitude, lower
+    ordered = torch.where(torch.isnan(cost), torch.full_like(ordered, 2147483647), ordered)
+    by_cost = torch.sort((ordered << 32) | edge_mix(edge_vi, edge_vj), stable=True).indices
     sample = torch.bucketize(edge_vi[by_cost].long(), nvIn_cumsum.long(), right=True)
-    by_sample = torch.sort(sample, stable=True)
-    return by_cost[by_sample.indices], by_sample.values
+    narrow = torch.uint8 if nvIn_cumsum.shape[0] < 256 else torch.int64
+    by_sample = torch.sort(sample.to(narrow), stable=True)
+    return by_cost[by_sample.indices], by_sample.values.long()
 
 
-_staging = {}
+_staging = threading.local()
 
 
 def _pinned(name, n, dtype):
     """A page-locked host buffer of at least ``n`` elements, kept between calls (the edge lists of a scene-scale batch
-    are tens of megabytes: through pageable memory their trip to the host costs more than the clustering itself)."""
-    buf = _staging.get(name)
+    are tens of megabytes: through pageable memory their trip to the host costs more than the clustering itself).
+    One set of buffers per calling thread: two threads that decimate at once never share one."""
+    bufs = _staging.__dict__.setdefault("bufs", {})
+    buf = bufs.get(name)
     if buf is None or buf.numel() < n or buf.dtype != dtype:
         buf = torch.empty(max(n, 1), dtype=dtype, pin_memory=True)
-        _staging[name] = buf
+        bufs[name] = buf
     return buf[:n]
 
 
@@ -146,6 +172,63 @@ def cluster_vertices(edge_vi, edge_vj, sample, nvIn_cumsum, nv2Remove, Nv):
     return vt_replace
 
 
+def cluster_vertices_device(edge_vi, edge_vj, sample, nvIn_cumsum, nv2Remove, Nv, rounds_per_check=8):
+    """The same two greedy passes on the device, for all samples at once: -> vt_replace int32 (Nv,) on the device, equal
+    to what ``cluster_vertices`` returns.  Nothing but a status word per ``rounds_per_check`` rounds of the first pass
+    crosses to the host.
+
+    First pass: the serial choice "take an edge when both its ends are free" over a total order is the fixed point of
+    "an edge that is the first edge with two free ends at BOTH of its ends is taken" (``pmesh_cluster_match``); the
+    serial pass stops at its budget, i.e. keeps the lowest-ranked of these edges.  Second pass (only for a sample whose
+    first pass left budget, i.e. ended with no edge between two free vertices): a free vertex joins the cluster behind
+    its first edge to a covered vertex -- no vertex that joins can enable another one -- again cut by rank."""
+    dev = edge_vi.device
+    E, B = edge_vi.shape[0], nvIn_cumsum.shape[0]
+    st = stream_of(edge_vi)
+    with torch.cuda.device(dev):
+        vt_replace = torch.zeros(Nv, dtype=I32, device=dev)
+        if E == 0 or Nv == 0:
+            return vt_replace
+        edge_vi, edge_vj = edge_vi.contiguous(), edge_vj.contiguous()
+        sample = sample.to(I32).contiguous()
+        budget = nv2Remove.to(torch.int64).clamp(min=0)
+        state = torch.zeros(Nv, dtype=I32, device=dev)
+        best = torch.empty(Nv, dtype=I32, device=dev)
+        chosen = torch.zeros(E, dtype=I32, device=dev)
+        status = torch.zeros(4, dtype=I32, device=dev)
+        while True:
+            _lib.call("pmesh_cluster_match", edge_vi.data_ptr(), edge_vj.data_ptr(), E, Nv, state.data_ptr(), best.data_ptr(),
+                      chosen.data_ptr(), status.data_ptr(), rounds_per_check, st)
+            left, bad = status[:2].tolist()
+            if bad:
+                raise RuntimeError("cluster_vertices: a candidate edge is not (vi < vj) inside the vertex range")
+            if not left:
+                break
+        # rank of each chosen edge among its sample's chosen edges; the budget keeps the first ones
+        first = torch.searchsorted(sample, torch.arange(B + 1, device=dev, dtype=I32))
+
+        def cut(flags, allowance):
+            run = torch.cumsum(flags, 0)
+            before = torch.cat([run.new_zeros(1), run])[first]                 # flags counted ahead of each sample
+            rank = run - before[:-1][sample.long()]
+            return (flags > 0) & (rank <= allowance[sample.long()]), before[1:] - before[:-1]
+
+        keep, n_chosen = cut(chosen, budget)
+        _lib.call("pmesh_cluster_contract_pairs", edge_vi.data_ptr(), edge_vj.data_ptr(), keep.to(I32).data_ptr(), E,
+                  vt_replace.data_ptr(), st)
+        # second pass where the first one left budget
+        open_ = (n_chosen < budget).to(I32).contiguous()
+        first_edge = best
+        attaches = chosen
+        _lib.call("pmesh_cluster_attach_propose", edge_vi.data_ptr(), edge_vj.data_ptr(), sample.data_ptr(), open_.data_ptr(), E, Nv,
+                  vt_replace.data_ptr(), first_edge.data_ptr(), attaches.data_ptr(), st)
+        keep2, _ = cut(attaches, budget - torch.minimum(n_chosen, budget))
+        pairs = vt_replace.clone()
+        _lib.call("pmesh_cluster_attach", edge_vi.data_ptr(), edge_vj.data_ptr(), keep2.to(I32).data_ptr(), E, first_edge.data_ptr(),
+                  pairs.data_ptr(), vt_replace.data_ptr(), st)
+    return vt_replace
+
+
 def simplify(vertexIn, faceIn, geometryIn, nvIn_cumsum, mfIn_cumsum, nv2Remove, useArea=True, wgtBnd=5.0):
     """One decimation round: the reference's ``mesh_decimation.simplify`` (decimate.cpp:21-89,
     decimate_gpu.cu:618-747).  ``nvIn_cumsum`` / ``mfIn_cumsum``: running totals of vertices / facets per sample.
@@ -160,8 +243,11 @@ def simplify(vertexIn, faceIn, geometryIn, nvIn_cumsum, mfIn_cumsum, nv2Remove, 
     dev = vertexIn.device
     quadric, evi, evj = vertex_quadrics(vertexIn, faceIn, geometryIn, useArea, wgtBnd)
     cost = edge_costs(vertexIn, quadric, evi, evj)
-    perm, sample = contraction_order(cost, evi, nvIn_cumsum)
-    vt_replace = torch.from_numpy(cluster_vertices(evi[perm], evj[perm], sample, nvIn_cumsum, nv2Remove, Nv)).to(dev)
+    perm, sample = contraction_order(cost, evi, evj, nvIn_cumsum)
+    if evi.is_cuda and os.environ.get("PMESH_DECIMATE_HOST_CLUSTERING") != "1":
+        vt_replace = cluster_vertices_device(evi[perm], evj[perm], sample, nvIn_cumsum, nv2Remove, Nv)
+    else:
+        vt_replace = torch.from_numpy(cluster_vertices(evi[perm], evj[perm], sample, nvIn_cumsum, nv2Remove, Nv)).to(dev)
     with torch.cuda.device(dev):
         ids = torch.arange(Nv, dtype=I32, device=dev)
         rep = torch.where(vt_replace < 0, -vt_replace, ids).long()

@@ -238,3 +238,58 @@ def test_mesh_hierarchy_levels_feed_a_network_block(cuda):
         n_prev = nvl_n
     fixed = MeshHierarchy([dev(np.array([300, 200], np.int32), cuda)], True, 1.0)(vx, fc, dev(nv, cuda), dev(mf, cuda))
     assert fixed[1][3].cpu().tolist() == [300, 200]
+
+
+@pytest.mark.parametrize("seed", range(10))
+def test_device_clustering_equals_the_serial_host_routine(cuda, seed):
+    """cluster_vertices_device (fixed-point rounds of the first pass, one-step second pass, both cut by rank) against
+    pmesh_cluster_vertices_host and the oracle's statement of the two serial passes, on random graphs of several samples
+    with budgets from nothing to everything -- including chains of ascending ranks, the slowest case for the rounds."""
+    say("case device clustering", seed)
+    rng = np.random.default_rng(100 + seed)
+    samples = 1 + seed % 4
+    num = [int(n) for n in rng.integers(2, 400, samples)]
+    starts = np.concatenate([[0], np.cumsum(num)])
+    vi_l, vj_l, smp = [], [], []
+    for b in range(samples):
+        lo, n = int(starts[b]), num[b]
+        pairs = {tuple(sorted(p)) for p in rng.integers(lo, lo + n, (int(rng.integers(1, 5)) * n, 2)).tolist() if p[0] != p[1]}
+        if seed % 3 == 0:                                   # a path in ascending order of rank: one choice per round
+            pairs |= {(lo + i, lo + i + 1) for i in range(min(n - 1, 40))}
+        pairs = sorted(pairs)
+        order = np.arange(len(pairs)) if seed % 3 == 0 else rng.permutation(len(pairs))
+        vi_l.append(np.array(pairs, np.int32).reshape(-1, 2)[order, 0])
+        vj_l.append(np.array(pairs, np.int32).reshape(-1, 2)[order, 1])
+        smp.append(np.full(len(pairs), b, np.int64))
+    vi, vj, sample = np.concatenate(vi_l), np.concatenate(vj_l), np.concatenate(smp)
+    nv_cum = torch.from_numpy(starts[1:].astype(np.int32))
+    Nv = int(starts[-1])
+    for frac in (0.0, 0.1, 0.45, 0.8, 1.0):
+        budget = np.array([int(n * frac) for n in num], np.int32)
+        want = np.zeros(Nv, np.int32)
+        for b in range(samples):
+            m = sample == b
+            D.cluster_vertices(vi[m], vj[m], int(starts[b]), num[b], int(budget[b]), want)
+        host = decimate.cluster_vertices(torch.from_numpy(vi), torch.from_numpy(vj), torch.from_numpy(sample), nv_cum,
+                                         torch.from_numpy(budget), Nv)
+        assert np.array_equal(host, want)
+        got = decimate.cluster_vertices_device(dev(vi, cuda), dev(vj, cuda), dev(sample, cuda), nv_cum.to(cuda), dev(budget, cuda), Nv,
+                                               rounds_per_check=1 + seed % 3)
+        assert np.array_equal(got.cpu().numpy(), want), "budget fraction %g: %d vertices differ" % (frac, (got.cpu().numpy() != want).sum())
+    with pytest.raises(RuntimeError):
+        decimate.cluster_vertices_device(dev(vj, cuda), dev(vi, cuda), dev(sample, cuda), nv_cum.to(cuda), dev(budget, cuda), Nv)
+
+
+def test_simplify_is_the_same_with_host_clustering(cuda, monkeypatch):
+    v, f, nv, mf = batch(("sphere3", "room_small", "torus"))
+    vx, fc = dev(v, cuda), dev(f, cuda)
+    geo = compute_triangle_geometry_(vx, fc)
+    args = (vx, fc, geo, dev(np.cumsum(nv).astype(np.int32), cuda), dev(np.cumsum(mf).astype(np.int32), cuda))
+    for frac in (0.3, 0.7):
+        n_remove = dev((nv * frac).astype(np.int32), cuda)
+        monkeypatch.delenv("PMESH_DECIMATE_HOST_CLUSTERING", raising=False)
+        a = decimate.simplify(*args, n_remove, True, 5.0)
+        monkeypatch.setenv("PMESH_DECIMATE_HOST_CLUSTERING", "1")
+        b = decimate.simplify(*args, n_remove, True, 5.0)
+        for x, y in zip(a, b):
+            assert torch.equal(x, y)

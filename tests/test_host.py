@@ -341,3 +341,26 @@ def test_bf16_store_criterion_tells_rounding_from_truncation():
         assert_close_bf16_store(truncated, ref, "truncated", tol=1e-6)
     with pytest.raises(AssertionError):
         assert_close_bf16_store(truncated, ref, "truncated", tol=1e-3)
+
+
+def test_contraction_order_of_the_product_is_the_oracles():
+    """decimate.contraction_order packs (cost, mix) into one integer key per edge; on CPU tensors it must order the edges
+    exactly as the oracle's lexicographic statement does, for costs that are negative, signed zeros, denormal,
+    infinite, NaN or an ulp apart."""
+    import torch
+    from oracle import decimate_ref as R
+    from picassoplus_amd.mesh.pi_modules import decimate as D
+    rng = np.random.default_rng(0)
+    n = 6000
+    vi = np.sort(rng.integers(0, 300, n)).astype(np.int32)
+    vj = (vi + rng.integers(1, 50, n)).astype(np.int32)
+    k = np.argsort(vi.astype(np.int64) * 1000 + vj, kind="stable")
+    vi, vj = vi[k], vj[k]
+    special = np.array([0.0, -0.0, 1e-45, -1e-45, 1e-30, -1e-30, -2.5, 2.5, np.nan, np.inf, -np.inf, 1.0, 1.0000001, -1.0], np.float32)
+    cost = rng.choice(special, n)
+    cost[::7] = rng.normal(size=len(cost[::7])).astype(np.float32)
+    cum = np.array([100, 200, 300])
+    want_perm, want_sample = R.contraction_order(cost, vi, vj, cum)
+    perm, sample = D.contraction_order(torch.from_numpy(cost), torch.from_numpy(vi), torch.from_numpy(vj), torch.from_numpy(cum))
+    assert np.array_equal(perm.numpy(), want_perm) and np.array_equal(sample.numpy(), want_sample)
+    assert np.array_equal(D.edge_mix(torch.from_numpy(vi), torch.from_numpy(vj)).numpy(), R.edge_mix(vi, vj))

@@ -160,11 +160,48 @@ def test_edge_costs_float32_mode_is_close():
 
 
 # ------------------------------------------------------------------ order and clustering
+def _mix_by_hand(a, b):
+    """edge_mix with Python integers and explicit 32-bit masks."""
+    m = (1 << 32) - 1
+    h = (a * 0x9E3779B1 + b * 0x85EBCA77) & m
+    h ^= h >> 15
+    h = (h * 0x2C1B3C6D) & m
+    h ^= h >> 12
+    h = (h * 0x297A2D39) & m
+    return h ^ (h >> 15)
+
+
 def test_contraction_order_is_total():
-    cost = np.array([0.5, 0.1, 0.1, np.nan, 0.1, 0.0])
-    vi = np.array([0, 1, 2, 2, 5, 6], np.int32)                         # samples: vertices 0-3, 4-7
-    perm, sample = D.contraction_order(cost, vi, np.array([4, 8]))
-    assert perm.tolist() == [1, 2, 0, 3, 5, 4] and sample.tolist() == [0, 0, 0, 0, 1, 1]
+    """(sample, cost, mix, vi, vj): samples apart, costs ascending with NaN last and -0 = +0, equal costs by the mix of
+    their end points (checked against integer arithmetic by hand), equal mixes by (vi, vj)."""
+    rng = np.random.default_rng(4)
+    n = 400
+    vi = np.sort(rng.integers(0, 8, n)).astype(np.int32)                # samples: vertices 0-3, 4-7
+    vj = (vi + rng.integers(1, 2 ** 30, n)).astype(np.int32)
+    key = np.argsort(vi.astype(np.int64) * 2 ** 31 + vj, kind="stable")  # the callers' ascending (vi, vj) order
+    vi, vj = vi[key], vj[key]
+    cost = rng.choice([0.0, -0.0, 0.25, 0.25, 1e-9, np.nan, 3.0], n)
+    perm, sample = D.contraction_order(cost, vi, vj, np.array([4, 8]))
+    assert sorted(perm.tolist()) == list(range(n))
+    assert np.array_equal(sample, (vi[perm] >= 4).astype(int)) and np.all(np.diff(sample) >= 0)
+    mix = [_mix_by_hand(int(a), int(b)) for a, b in zip(vi, vj)]
+    assert np.array_equal(D.edge_mix(vi, vj), np.array(mix, np.int64))
+    assert len(set(mix)) > 0.95 * len(set(zip(vi.tolist(), vj.tolist())))     # it does spread the pairs
+    for x, y in zip(perm[:-1].tolist(), perm[1:].tolist()):
+        if (vi[x] >= 4) != (vi[y] >= 4):
+            continue
+        cx, cy = cost[x], cost[y]
+        if np.isnan(cx):
+            assert np.isnan(cy)
+        elif not np.isnan(cy) and cx != cy:
+            assert cx < cy
+        elif not np.isnan(cy):
+            assert (mix[x], vi[x], vj[x]) < (mix[y], vi[y], vj[y])
+    # a case small enough to read: costs decide, then the mix (edge (2, 3) before (1, 2) because its mix is smaller)
+    vi3, vj3 = np.array([0, 1, 2], np.int32), np.array([1, 2, 3], np.int32)
+    order3, _ = D.contraction_order(np.array([0.5, 0.1, 0.1]), vi3, vj3, np.array([4]))
+    first, second = ((1, 2), (2, 3)) if _mix_by_hand(1, 2) < _mix_by_hand(2, 3) else ((2, 3), (1, 2))
+    assert [(int(vi3[i]), int(vj3[i])) for i in order3] == [first, second, (0, 1)]
 
 
 def brute_force_clusters(edges, start, num, budget):

@@ -331,6 +331,20 @@ int pmesh_combine_clusters(const int32_t *rep_a, const int32_t *map_a, const int
  *                            of the second pass joins its free end to the cluster of its covered end in either
  *                            position (the reference contracts a covered non-seed vertex into a free one when they
  *                            come in that order, which leaves chains the pooling ops cannot follow). */
+/*   pmesh_edge_list_count / _fill  the unique edges (vi < vj) of the facets in ascending (vi, vj) order, replacing
+ *                            the sort of all 3 Nf facet edges and the duplicate removal (:250-297): one thread per
+ *                            vertex orders the higher corners of the facets in its row of the vertex CSR (rowptr,
+ *                            colidx of pmesh_build_vertex_csr over `face`).  count: counts (2,Nv) <- per vertex the
+ *                            number of edges it is the lower end of, and of those held by ONE facet side (boundary
+ *                            edges).  fill: offsets (2,Nv) = exclusive running totals of each row of counts; writes the edges,
+ *                            and the boundary edges with the facet that holds each.  spill: 12 Nf ints, touched by
+ *                            rows of more than 16 entries only; with spill NULL such a row sets *need_spill (which
+ *                            the caller zeroes beforehand) and counts nothing: call again with a spill area. */
+int pmesh_edge_list_count(const int32_t *face, const int32_t *rowptr, const int32_t *colidx, int64_t Nv, int64_t Nf,
+                          int32_t *counts, int32_t *spill, int32_t *need_spill, pmesh_stream_t stream);
+int pmesh_edge_list_fill(const int32_t *face, const int32_t *rowptr, const int32_t *colidx, int64_t Nv, int64_t Nf,
+                         const int32_t *offsets, int32_t *edge_vi, int32_t *edge_vj, int32_t *bnd_vi, int32_t *bnd_vj,
+                         int32_t *bnd_face, int32_t *spill, pmesh_stream_t stream);
 int pmesh_vertex_quadrics(const float *geometry, const int32_t *rowptr, const int32_t *colidx, float *quadric,
                           int64_t Nv, int use_area, pmesh_stream_t stream);
 int pmesh_boundary_quadrics(const float *vertex, const float *geometry, const int32_t *edge_vi, const int32_t *edge_vj,

@@ -90,6 +90,8 @@ SIGNATURES = {
     "pmesh_boundary_quadrics": (I, [P, P, P, P, P, P, L, I, I, c_float, P]),
     "pmesh_edge_costs": (I, [P, P, P, P, P, L, I, P]),
     "pmesh_cluster_vertices_host": (I, [P, P, L, I, I, I, P]),
+    "pmesh_edge_list_count": (I, [P, P, P, L, L, P, P, P, P]),
+    "pmesh_edge_list_fill": (I, [P, P, P, L, L, P, P, P, P, P, P, P, P]),
     "pmesh_cluster_match": (I, [P, P, L, L, P, P, P, P, I, P]),
     "pmesh_cluster_contract_pairs": (I, [P, P, P, L, P, P]),
     "pmesh_cluster_attach_propose": (I, [P, P, P, P, L, L, P, P, P, P]),

@@ -163,6 +163,114 @@ __global__ __launch_bounds__(kBlock) void edge_cost_k(const float *__restrict__ 
 }
 
 // ----------------------------------------------------------------------------------------
+// Candidate edges from the vertex adjacency, without a sort of the whole edge list: the edges (v, w), v < w, of the
+// facets around v are exactly those whose lower end is v, so one thread per vertex collects the other corners w > v
+// of its row's facets, orders them, and writes the distinct ones -- which leaves the batch's unique edges in
+// ascending (vi, vj) order (decimate_gpu.cu:250-297 sorts all 3 Nf facet edges instead).  With each edge: how many
+// facet sides hold it (1 = boundary edge) and the lowest facet that does.
+// A row's candidates (two per adjacency entry) are ordered in LDS up to kEdgeLocal of them, beyond that
+// in the row's own segment of `spill` (4 ints per adjacency entry, 12 Nf in all; only touched when some row is that
+// long: without a spill area such a row raises *need_spill and is left out, and the caller comes back with one).
+constexpr int kEdgeLocal = 32;          // candidates of a row ordered in LDS (rows of up to 16 adjacency entries)
+constexpr int kEdgeBlock = 128;         // threads per workgroup: 2 x 32 x 128 ints of LDS
+
+struct EdgeRow {
+    int n;          // candidates w > v, ordered ascending by (w, facet); -1 = too long for LDS and no spill area
+    int *w, *f;
+    int stride;     // element i of the lists sits at w[i * stride]
+};
+
+__device__ __forceinline__ void edge_row_collect(const int *__restrict__ face, const int *__restrict__ rowptr,
+                                                 const int *__restrict__ colidx, int64_t Nv, int v, int *lw, int *lf,
+                                                 int *__restrict__ spill, EdgeRow &row)
+{
+    const int e0 = rowptr[v], e1 = rowptr[v + 1];
+    const bool big = 2 * (e1 - e0) > kEdgeLocal;
+    if (big && !spill) {
+        row.n = -1;                      // the caller comes back with a spill area
+        return;
+    }
+    row.w = big ? spill + 4 * (int64_t)e0 : lw;
+    row.f = big ? spill + 4 * (int64_t)e0 + 2 * (e1 - e0) : lf;
+    row.stride = big ? 1 : kEdgeBlock;
+    const int sd = row.stride;
+    int n = 0;
+    for (int e = e0; e < e1; ++e) {
+        const int en = colidx[e], fc = en / 3, c = en - 3 * fc;
+#pragma unroll
+        for (int d = 1; d <= 2; ++d) {
+            const int w = face[3 * (int64_t)fc + (c + d) % 3];
+            if (w > v && w < Nv) {
+                // insertion by (w, facet): rows are short
+                int i = n++;
+                while (i > 0 && (row.w[(i - 1) * sd] > w || (row.w[(i - 1) * sd] == w && row.f[(i - 1) * sd] > fc))) {
+                    row.w[i * sd] = row.w[(i - 1) * sd];
+                    row.f[i * sd] = row.f[(i - 1) * sd];
+                    --i;
+                }
+                row.w[i * sd] = w;
+                row.f[i * sd] = fc;
+            }
+        }
+    }
+    row.n = n;
+}
+
+// counts[v] = distinct edges whose lower end is v, counts[Nv + v] = those held by exactly one facet side
+__global__ __launch_bounds__(kEdgeBlock) void edge_list_count_k(const int *__restrict__ face, const int *__restrict__ rowptr,
+                                                                const int *__restrict__ colidx, int64_t Nv, int *__restrict__ counts,
+                                                                int *__restrict__ spill, int *__restrict__ need_spill)
+{
+    __shared__ int lw[kEdgeLocal * kEdgeBlock], lf[kEdgeLocal * kEdgeBlock];
+    const int64_t v = (int64_t)blockIdx.x * kEdgeBlock + threadIdx.x;
+    if (v >= Nv) return;
+    EdgeRow row;
+    edge_row_collect(face, rowptr, colidx, Nv, (int)v, lw + threadIdx.x, lf + threadIdx.x, spill, row);
+    if (row.n < 0) *need_spill = 1;
+    const int sd = row.stride;
+    int distinct = 0, single = 0;
+    for (int i = 0; i < row.n;) {
+        int j = i + 1;
+        while (j < row.n && row.w[j * sd] == row.w[i * sd]) ++j;
+        ++distinct;
+        single += (j - i) == 1;
+        i = j;
+    }
+    counts[v] = distinct;
+    counts[Nv + v] = single;
+}
+
+// offsets = exclusive running totals of counts
+__global__ __launch_bounds__(kEdgeBlock) void edge_list_fill_k(const int *__restrict__ face, const int *__restrict__ rowptr,
+                                                               const int *__restrict__ colidx, int64_t Nv, const int *__restrict__ offsets,
+                                                               int *__restrict__ edge_vi, int *__restrict__ edge_vj,
+                                                               int *__restrict__ bnd_vi, int *__restrict__ bnd_vj,
+                                                               int *__restrict__ bnd_face, int *__restrict__ spill)
+{
+    __shared__ int lw[kEdgeLocal * kEdgeBlock], lf[kEdgeLocal * kEdgeBlock];
+    const int64_t v = (int64_t)blockIdx.x * kEdgeBlock + threadIdx.x;
+    if (v >= Nv) return;
+    EdgeRow row;
+    edge_row_collect(face, rowptr, colidx, Nv, (int)v, lw + threadIdx.x, lf + threadIdx.x, spill, row);
+    const int sd = row.stride;
+    int o = offsets[v], ob = offsets[Nv + v];
+    for (int i = 0; i < row.n;) {
+        int j = i + 1;
+        while (j < row.n && row.w[j * sd] == row.w[i * sd]) ++j;
+        edge_vi[o] = (int)v;
+        edge_vj[o] = row.w[i * sd];
+        ++o;
+        if (j - i == 1) {
+            bnd_vi[ob] = (int)v;
+            bnd_vj[ob] = row.w[i * sd];
+            bnd_face[ob] = row.f[i * sd];
+            ++ob;
+        }
+        i = j;
+    }
+}
+
+// ----------------------------------------------------------------------------------------
 // The two greedy passes of the vertex clustering on the device, with the result of the serial host routine below.
 //
 // First pass (disjoint pairs, cheapest edge first).  For a total order of the edges the serial greedy choice is the
@@ -301,6 +409,32 @@ __global__ __launch_bounds__(kBlock) void attach_apply_k(const int *__restrict__
 }  // namespace pmesh
 
 using namespace pmesh;
+
+extern "C" int pmesh_edge_list_count(const int32_t *face, const int32_t *rowptr, const int32_t *colidx, int64_t Nv, int64_t Nf,
+                                     int32_t *counts, int32_t *spill, int32_t *need_spill, pmesh_stream_t stream)
+{
+    clear_error();
+    PM_REQUIRE(Nv >= 0 && Nv <= INT32_MAX && Nf >= 0 && Nf <= INT32_MAX / 6, "edge_list_count: bad sizes");
+    if (Nv == 0) return 0;
+    PM_REQUIRE(face && rowptr && colidx && counts && need_spill, "edge_list_count: null pointer");
+    edge_list_count_k<<<dim3((unsigned)ceil_div(Nv, kEdgeBlock)), dim3(kEdgeBlock), 0, (hipStream_t)stream>>>(face, rowptr, colidx, Nv, counts, spill, need_spill);
+    PM_LAUNCHED("edge_list_count");
+    return 0;
+}
+
+extern "C" int pmesh_edge_list_fill(const int32_t *face, const int32_t *rowptr, const int32_t *colidx, int64_t Nv, int64_t Nf,
+                                    const int32_t *offsets, int32_t *edge_vi, int32_t *edge_vj, int32_t *bnd_vi, int32_t *bnd_vj,
+                                    int32_t *bnd_face, int32_t *spill, pmesh_stream_t stream)
+{
+    clear_error();
+    PM_REQUIRE(Nv >= 0 && Nv <= INT32_MAX && Nf >= 0 && Nf <= INT32_MAX / 6, "edge_list_fill: bad sizes");
+    if (Nv == 0) return 0;
+    PM_REQUIRE(face && rowptr && colidx && offsets, "edge_list_fill: null pointer");      // (the lists may be empty)
+    edge_list_fill_k<<<dim3((unsigned)ceil_div(Nv, kEdgeBlock)), dim3(kEdgeBlock), 0, (hipStream_t)stream>>>(
+        face, rowptr, colidx, Nv, offsets, edge_vi, edge_vj, bnd_vi, bnd_vj, bnd_face, spill);
+    PM_LAUNCHED("edge_list_fill");
+    return 0;
+}
 
 extern "C" int pmesh_cluster_match(const int32_t *edge_vi, const int32_t *edge_vj, int64_t n_edges, int64_t Nv, int32_t *state,
                                    int32_t *best, int32_t *chosen, int32_t *status, int rounds, pmesh_stream_t stream)

@@ -48,31 +48,51 @@ def vertex_quadrics(vertexIn, faceIn, geometryIn, useArea=True, wgtBnd=5.0):
         quadric = torch.empty((Nv, 10), dtype=F32, device=dev)
         _lib.call("pmesh_vertex_quadrics", geometryIn.data_ptr(), rowptr.data_ptr(), colidx.data_ptr(), quadric.data_ptr(),
                   Nv, 1 if useArea else 0, st)
-        # the three edges of every facet as (lower, higher) vertex pairs; one 64-bit key per edge
-        f = faceIn.long()
-        a = torch.stack([f[:, 0], f[:, 0], f[:, 1]], 1).reshape(-1)
-        b = torch.stack([f[:, 1], f[:, 2], f[:, 2]], 1).reshape(-1)
-        key, order = torch.sort(torch.minimum(a, b) * Nv + torch.maximum(a, b), stable=True)
-        ukey, counts = torch.unique_consecutive(key, return_counts=True)
-        vi, vj = torch.div(ukey, Nv, rounding_mode="floor"), ukey % Nv
-        ok = vi != vj                                            # a facet with a repeated vertex has no such edge
-        if wgtBnd > 0:
-            first = torch.cumsum(counts, 0) - counts
-            bnd = (counts == 1) & ok                             # an edge that belongs to exactly one facet
-            nb = int(bnd.sum())
-            if nb:
-                bvi, bvj = vi[bnd].to(I32), vj[bnd].to(I32)
-                bface = torch.div(order[first[bnd]], 3, rounding_mode="floor").to(I32)
-                rows = torch.empty((nb, 10), dtype=F32, device=dev)
-                _lib.call("pmesh_boundary_quadrics", vertexIn.data_ptr(), geometryIn.data_ptr(), bvi.data_ptr(), bvj.data_ptr(),
-                          bface.data_ptr(), rows.data_ptr(), nb, D, 1 if useArea else 0, float(wgtBnd), st)
-                # every row goes to both end points: a segmented sum over the end points in ascending edge order
-                ends = torch.cat([bvi, bvj]).long()
-                _, members = torch.sort(ends, stable=True)
-                ptr = torch.zeros(Nv + 1, dtype=torch.int64, device=dev)
-                ptr[1:] = torch.cumsum(torch.bincount(ends, minlength=Nv), 0)
-                quadric = quadric + _segment_row_sum(torch.cat([rows, rows]), ptr.to(I32), members.to(I32), Nv)
-    return quadric, vi[ok].to(I32).contiguous(), vj[ok].to(I32).contiguous()
+        # the unique edges (vi < vj) in ascending order and the boundary edges among them, from the adjacency rows
+        evi, evj, bvi, bvj, bface = edge_list(faceIn, rowptr, colidx, Nv)
+        nb = bvi.shape[0]
+        if wgtBnd > 0 and nb:
+            rows = torch.empty((nb, 10), dtype=F32, device=dev)
+            _lib.call("pmesh_boundary_quadrics", vertexIn.data_ptr(), geometryIn.data_ptr(), bvi.data_ptr(), bvj.data_ptr(),
+                      bface.data_ptr(), rows.data_ptr(), nb, D, 1 if useArea else 0, float(wgtBnd), st)
+            # every row goes to both end points: a segmented sum over the end points in ascending edge order
+            ends = torch.cat([bvi, bvj]).long()
+            _, members = torch.sort(ends, stable=True)
+            ptr = torch.zeros(Nv + 1, dtype=torch.int64, device=dev)
+            ptr[1:] = torch.cumsum(torch.bincount(ends, minlength=Nv), 0)
+            quadric = quadric + _segment_row_sum(torch.cat([rows, rows]), ptr.to(I32), members.to(I32), Nv)
+    return quadric, evi, evj
+
+
+def edge_list(faceIn, rowptr, colidx, Nv):
+    """Unique edges of the facets from the vertex adjacency (``topology.vertex_csr(faceIn, None, Nv)``), without a sort
+    of all facet edges: -> (edge_vi, edge_vj, bnd_vi, bnd_vj, bnd_face) int32; edges with vi < vj in ascending (vi, vj)
+    order, the boundary edges (held by one facet side) among them in the same order with the facet that holds each."""
+    dev = faceIn.device
+    Nf = faceIn.shape[0]
+    st = stream_of(faceIn)
+    with torch.cuda.device(dev):
+        counts = torch.empty((2, Nv), dtype=I32, device=dev)
+        flag = torch.zeros(1, dtype=I32, device=dev)
+        spill = None
+        while True:
+            _lib.call("pmesh_edge_list_count", faceIn.data_ptr(), rowptr.data_ptr(), colidx.data_ptr(), Nv, Nf, counts.data_ptr(),
+                      spill.data_ptr() if spill is not None else None, flag.data_ptr(), st)
+            # (row by row: a scan along the rows of a two-row tensor takes a slow path of the library)
+            ends = torch.stack([torch.cumsum(counts[0], 0, dtype=I32), torch.cumsum(counts[1], 0, dtype=I32)])
+            n_edges, n_bnd, need = torch.cat([ends[:, -1] if Nv else ends.new_zeros(2), flag]).tolist()
+            if not need:
+                break
+            # some vertex has more than 16 adjacency entries: its candidates are ordered in memory
+            spill = torch.empty(12 * Nf, dtype=I32, device=dev)
+            flag.zero_()
+        offsets = (ends - counts).contiguous()
+        evi, evj = torch.empty(n_edges, dtype=I32, device=dev), torch.empty(n_edges, dtype=I32, device=dev)
+        bvi, bvj, bface = (torch.empty(n_bnd, dtype=I32, device=dev) for _ in range(3))
+        _lib.call("pmesh_edge_list_fill", faceIn.data_ptr(), rowptr.data_ptr(), colidx.data_ptr(), Nv, Nf, offsets.data_ptr(),
+                  evi.data_ptr(), evj.data_ptr(), bvi.data_ptr(), bvj.data_ptr(), bface.data_ptr(),
+                  spill.data_ptr() if spill is not None else None, st)
+    return evi, evj, bvi, bvj, bface
 
 
 def _segment_row_sum(rows, rowptr, members, n_out):

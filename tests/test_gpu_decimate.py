@@ -293,3 +293,36 @@ def test_simplify_is_the_same_with_host_clustering(cuda, monkeypatch):
         b = decimate.simplify(*args, n_remove, True, 5.0)
         for x, y in zip(a, b):
             assert torch.equal(x, y)
+
+
+@pytest.mark.parametrize("case", ["fans", "hub60", "sphere3+torus", "degenerate"])
+def test_edge_list_from_the_adjacency_equals_the_sorted_edge_list(cuda, case):
+    """decimate.edge_list (one thread per vertex over its adjacency row) against the oracle's sort of all facet edges:
+    the same unique edges in the same order, the same boundary edges with the same facets -- including a vertex whose
+    row is too long for the kernel's private memory and facets with a repeated vertex."""
+    from picassoplus_amd.mesh import topology
+    say("case edge list", case)
+    if case == "hub60":
+        n = 60
+        rim = 1 + np.arange(n)
+        f = np.stack([np.zeros(n, np.int64), rim, np.roll(rim, -1)], 1)[:-7].astype(np.int32)      # an open fan
+        f = np.concatenate([f, f[:5, [0, 2, 1]]]).astype(np.int32)                                  # some sides held twice
+        nv = n + 1
+    elif case == "degenerate":
+        f = np.array([[0, 1, 2], [2, 2, 3], [3, 4, 4], [5, 5, 5], [1, 2, 3], [6, 0, 6]], np.int32)
+        nv = 7
+    elif case == "fans":
+        v, f = mesh_case("fans")
+        nv = v.shape[0]
+    else:
+        v, f, _, _ = batch(("sphere3", "torus"))
+        nv = v.shape[0]
+    fc = dev(f, cuda)
+    rowptr, colidx = topology.vertex_csr(fc, None, nv)
+    evi, evj, bvi, bvj, bface = decimate.edge_list(fc, rowptr, colidx, nv)
+    wi, wj, counts, first_face = D.unique_edges(f, nv)
+    ok = wi != wj
+    assert np.array_equal(evi.cpu().numpy(), wi[ok]) and np.array_equal(evj.cpu().numpy(), wj[ok])
+    bnd = (counts == 1) & ok
+    assert np.array_equal(bvi.cpu().numpy(), wi[bnd]) and np.array_equal(bvj.cpu().numpy(), wj[bnd])
+    assert np.array_equal(bface.cpu().numpy(), first_face[bnd])

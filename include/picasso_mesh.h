@@ -490,6 +490,12 @@ int pmesh_point_cube_fill_grid(const void *grid, const float *database, const fl
 /* three nearest neighbours (nnquery.cpp:132-171 "knn3", nnquery_gpu.cu:262-330): nn_index, nn_dist (Mp,3). */
 int pmesh_point_knn3(const float *database, const float *query, const int32_t *nv_database, const int32_t *nv_query,
                      int B, int64_t Np, int64_t Mp, int32_t *nn_index, float *nn_dist, pmesh_stream_t stream);
+/* The same search over a cell grid (pmesh_point_grid_build with reach = -c: no radius to go by, about c cells per
+ * database point of a sample), same nn_index and nn_dist bit for bit: the window of cells around a query grows
+ * until its third nearest is closer than anything outside the window can be. */
+int pmesh_point_knn3_grid(const void *grid, const float *database, const float *query, const int32_t *nv_database,
+                          const int32_t *nv_query, int B, int64_t Np, int64_t Mp, int32_t *nn_index, float *nn_dist,
+                          pmesh_stream_t stream);
 /* farthest point sampling (sample.cpp:20-50 "fps", sample_gpu.cu:11-100): index_out (Mp) <- per sample its first
  * point, then repeatedly the point farthest from those chosen (lowest index among equals); temp: Np floats. */
 int pmesh_point_fps(const float *xyz, const int32_t *nv_in, const int32_t *nv_out, int B, int64_t Np, int64_t Mp,

@@ -45,6 +45,7 @@ SIGNATURES = {
     "pmesh_point_cube_count_grid": (I, [P, P, P, P, P, I, L, L, ctypes.c_float, I, P, P]),
     "pmesh_point_cube_fill_grid": (I, [P, P, P, P, P, I, L, L, ctypes.c_float, I, P, L, P, P]),
     "pmesh_point_knn3": (I, [P, P, P, P, I, L, L, P, P, P]),
+    "pmesh_point_knn3_grid": (I, [P, P, P, P, P, I, L, L, P, P, P]),
     "pmesh_point_fps": (I, [P, P, P, I, L, L, P, P, P]),
     "pmesh_point_sph3d_kernel": (I, [P, P, P, P, L, L, L, I, I, I, ctypes.c_float, P, P]),
     "pmesh_point_fuzzy_sph3d_kernel": (I, [P, P, P, P, L, L, L, I, I, I, ctypes.c_float, P, P, P]),

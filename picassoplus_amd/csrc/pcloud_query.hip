@@ -197,7 +197,7 @@ __global__ __launch_bounds__(kBlock) void grid_bbox_k(const float *__restrict__ 
 }
 
 // origin, cell edge and cell counts from the bounding box (one thread)
-__global__ void grid_dims_k(PointGrid *__restrict__ G, int B, float reach)
+__global__ void grid_dims_k(PointGrid *__restrict__ G, int B, float reach, int64_t per_sample)
 {
     if (blockIdx.x || threadIdx.x) return;
     float o[3] = {0.f, 0.f, 0.f}, ext[3] = {0.f, 0.f, 0.f};
@@ -207,6 +207,26 @@ __global__ void grid_dims_k(PointGrid *__restrict__ G, int B, float reach)
             ext[a] = ordered_float(G->hi[a]) - o[a];
         }
     float h = reach * kGridSlack;
+    if (reach < 0.f && finite3(ext[0], ext[1], ext[2])) {
+        // no search radius to go by (nearest-neighbour queries): about -reach cells per database point of a sample.
+        // Axes shorter than the edge that comes out get one cell and leave the product to the others.
+        const float target = fmaxf(-reach * (float)per_sample, 1.f);
+        bool on[3] = {ext[0] > 0.f, ext[1] > 0.f, ext[2] > 0.f};
+        h = 0.f;
+        for (int it = 0; it < 4; ++it) {
+            float vol = 1.f;
+            int act = 0;
+            for (int a = 0; a < 3; ++a)
+                if (on[a]) { vol *= ext[a]; ++act; }
+            if (!act) break;
+            h = powf(vol / target, 1.0f / (float)act);
+            bool again = false;
+            for (int a = 0; a < 3; ++a)
+                if (on[a] && ext[a] < h) { on[a] = false; again = true; }
+            if (!again) break;
+        }
+        if (!(h > 0.f)) h = fmaxf(fmaxf(ext[0], ext[1]), fmaxf(ext[2], 1e-30f));     // all points in one place
+    }
     int n[3] = {1, 1, 1};
     bool fits = false;
     if (h > 0.f && h < INFINITY && finite3(ext[0], ext[1], ext[2]))
@@ -707,6 +727,117 @@ __global__ __launch_bounds__(kBlock) void point_knn3_k(const float *__restrict__
     nn_dist[j * 3] = sqrtf(b1); nn_dist[j * 3 + 1] = sqrtf(b2); nn_dist[j * 3 + 2] = sqrtf(b3);
 }
 
+// The three nearest over the cell grid, same result as the scan above: kQLanes lanes share a query and deal out the
+// (x, y) columns of a window of cells around it; each keeps its three best by (squared distance, database index), the
+// lists are merged, and the window grows until the third best is closer than anything outside it can be (a point in a
+// cell r + 1 or more cells away on some axis is at least r cell edges away) or until it covers the sample's grid.
+struct Near3 {
+    float d[3];
+    int i[3];
+};
+__device__ __forceinline__ bool nearer(float d, int i, float b, int j) { return d < b || (d == b && i < j); }
+__device__ __forceinline__ void near3_insert(Near3 &n, float d, int i)
+{
+    if (nearer(d, i, n.d[0], n.i[0])) {
+        n.d[2] = n.d[1]; n.i[2] = n.i[1]; n.d[1] = n.d[0]; n.i[1] = n.i[0]; n.d[0] = d; n.i[0] = i;
+    } else if (nearer(d, i, n.d[1], n.i[1])) {
+        n.d[2] = n.d[1]; n.i[2] = n.i[1]; n.d[1] = d; n.i[1] = i;
+    } else if (nearer(d, i, n.d[2], n.i[2])) {
+        n.d[2] = d; n.i[2] = i;
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void point_knn3_grid_k(const PointGrid *__restrict__ G, const int2 *__restrict__ cells,
+                                                            const float4 *__restrict__ pts, const float *__restrict__ query,
+                                                            const int *__restrict__ nvd, const int *__restrict__ nvq, int B,
+                                                            int64_t Mp, int *__restrict__ nn_index, float *__restrict__ nn_dist)
+{
+    const int64_t j = (int64_t)blockIdx.x * kQPerBlock + threadIdx.x / kQLanes;
+    const int sub = threadIdx.x % kQLanes;
+    const bool valid = j < Mp;
+    const int b = valid ? sample_index(j, nvq, B) : B;
+    if (b >= B) {
+        // (all lanes of a query leave together; the lanes of the other queries do not wait for them)
+        if (valid && sub == 0)
+            for (int i = 0; i < 3; ++i) { nn_index[j * 3 + i] = 0; nn_dist[j * 3 + i] = INFINITY; }
+        return;
+    }
+    const int first = b ? nvd[b - 1] : 0;               // what the scan reports in the places it cannot fill
+    const float qx = query[j * 3], qy = query[j * 3 + 1], qz = query[j * 3 + 2];
+    const float inv_h = G->inv_h, h = inv_h > 0.f ? 1.0f / inv_h : INFINITY;
+    const int n[3] = {G->nx, G->ny, G->nz};
+    const float q[3] = {qx, qy, qz}, o[3] = {G->ox, G->oy, G->oz};
+    int c[3], r = 1;
+    bool sane = true;
+    for (int a = 0; a < 3; ++a) {
+        float v = floorf((q[a] - o[a]) * inv_h);
+        sane = sane && v == v;
+        v = fminf(fmaxf(v, -4.f * kGridMaxAxis), 4.f * kGridMaxAxis);
+        c[a] = sane ? (int)v : 0;
+        const int out = c[a] < 0 ? -c[a] : (c[a] > n[a] - 1 ? c[a] - (n[a] - 1) : 0);       // cells between me and the grid
+        r = out > r ? out : r;
+    }
+    if (!sane) r = 8 * kGridMaxAxis;                    // a query that is not a number is no nearer to anything: every cell
+    const int2 *mine = cells + (int64_t)b * G->cells;
+    Near3 best;
+    for (;;) {
+        for (int i = 0; i < 3; ++i) { best.d[i] = INFINITY; best.i[i] = first; }
+        int lo[3], hi[3];
+        bool all = true;
+        for (int a = 0; a < 3; ++a) {
+            lo[a] = c[a] - r > 0 ? c[a] - r : 0;
+            hi[a] = c[a] + r < n[a] - 1 ? c[a] + r : n[a] - 1;
+            all = all && c[a] - r <= 0 && c[a] + r >= n[a] - 1;
+        }
+        const int wy = hi[1] - lo[1] + 1, ncol = (hi[0] - lo[0] + 1) * wy;
+        for (int k = sub; k < ncol; k += kQLanes) {
+            const int x = lo[0] + k / wy, y = lo[1] + k % wy;
+            const int2 *col = mine + (x * n[1] + y) * n[2];
+            int s = INT32_MAX, e = 0;
+            for (int z = lo[2]; z <= hi[2]; ++z) {
+                const int2 rg = col[z];
+                if (rg.y > rg.x) {
+                    s = rg.x < s ? rg.x : s;
+                    e = rg.y > e ? rg.y : e;
+                }
+            }
+            for (int i = s; i < e; i += 4) {
+                float4 p[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) p[u] = pts[i + u < e ? i + u : e - 1];
+#pragma unroll
+                for (int u = 0; u < 4; ++u)
+                    if (i + u < e) {
+                        float dx, dy, dz;
+                        const float d2 = sq_dist(qx, qy, qz, p[u], dx, dy, dz);
+                        near3_insert(best, d2, __float_as_int(p[u].w));
+                    }
+            }
+        }
+        // the lanes of the query exchange their lists (all eight are here together)
+#pragma unroll
+        for (int step = 1; step < kQLanes; step <<= 1) {
+            Near3 other;
+#pragma unroll
+            for (int i = 0; i < 3; ++i) {
+                other.d[i] = __shfl_xor(best.d[i], step, 64);
+                other.i[i] = __shfl_xor(best.i[i], step, 64);
+            }
+#pragma unroll
+            for (int i = 0; i < 3; ++i)
+                if (other.d[i] < INFINITY) near3_insert(best, other.d[i], other.i[i]);
+        }
+        if (all || sqrtf(best.d[2]) < ((float)r - 0.01f) * h) break;
+        r = r + 1 > r + r / 2 ? r + 1 : r + r / 2;
+    }
+    if (sub == 0) {
+        for (int i = 0; i < 3; ++i) {
+            nn_index[j * 3 + i] = best.i[i];
+            nn_dist[j * 3 + i] = sqrtf(best.d[i]);
+        }
+    }
+}
+
 // Farthest point sampling: one workgroup of 1024 threads per sample.  Every round updates the squared distance of
 // each point to the chosen set against the last chosen point and takes the arg-max (lowest index among equals).
 // A sample of at most 1024 * kFpsPer points lives in registers for the whole run (thread t holds points t, t + 1024,
@@ -995,7 +1126,7 @@ extern "C" int pmesh_point_grid_build(const float *database, const int32_t *nv_d
 {
     clear_error();
     PM_REQUIRE(B > 0 && B <= kGridMaxCells && Np > 0 && Np <= INT32_MAX, "point_grid_build: bad sizes");
-    PM_REQUIRE(reach > 0, "point_grid_build: the reach of the searches must be positive");
+    PM_REQUIRE(reach > 0 || (reach < 0 && reach >= -64.f), "point_grid_build: the reach of the searches must be positive (or -c for c cells per point)");
     PM_REQUIRE(database && nv_database && grid, "point_grid_build: null pointer");
     PM_REQUIRE(((uintptr_t)grid & 255) == 0, "point_grid_build: the workspace must be aligned to 256 bytes");
     PM_REQUIRE(grid_bytes >= pmesh_point_grid_workspace_bytes(Np), "point_grid_build: workspace too small (%zu bytes)", grid_bytes);
@@ -1012,7 +1143,7 @@ extern "C" int pmesh_point_grid_build(const float *database, const int32_t *nv_d
     const unsigned pb = (unsigned)ceil_div(Np, kBlock);
     grid_clear_k<<<dim3(kGridMaxCells / kBlock), dim3(kBlock), 0, st>>>(G, cells);
     grid_bbox_k<<<dim3((unsigned)ceil_div(Np, (int64_t)kBlock * kBboxPer)), dim3(kBlock), 0, st>>>(database, nv_database, B, Np, G);
-    grid_dims_k<<<dim3(1), dim3(64), 0, st>>>(G, B, reach);
+    grid_dims_k<<<dim3(1), dim3(64), 0, st>>>(G, B, reach, ceil_div(Np, (int64_t)B));
     grid_keys_k<<<dim3(pb), dim3(kBlock), 0, st>>>(database, nv_database, B, Np, G, keys_in, ids_in);
     PM_LAUNCHED("point_grid_build");
     const hipError_t e = sort_pairs(temp, sort_pairs_temp_bytes(Np, kGridKeyBits), keys_in, keys_out, ids_in, ids_out, Np,
@@ -1106,6 +1237,20 @@ extern "C" int pmesh_point_knn3(const float *database, const float *query, const
     point_knn3_k<<<dim3((unsigned)ceil_div(Mp, kBlock)), dim3(kBlock), 0, (hipStream_t)stream>>>(database, query, nv_database, nv_query,
                                                                                             B, Np, Mp, nn_index, nn_dist);
     PM_LAUNCHED("point_knn3");
+    return 0;
+}
+
+extern "C" int pmesh_point_knn3_grid(const void *grid, const float *database, const float *query, const int32_t *nv_database,
+                                     const int32_t *nv_query, int B, int64_t Np, int64_t Mp, int32_t *nn_index, float *nn_dist,
+                                     pmesh_stream_t stream)
+{
+    clear_error();
+    PM_QUERY_DIMS("point_knn3_grid");
+    PM_REQUIRE(nn_index && nn_dist, "point_knn3_grid: null pointer");
+    PM_GRID_PARTS("point_knn3_grid");
+    point_knn3_grid_k<<<dim3((unsigned)ceil_div(Mp, kQPerBlock)), dim3(kBlock), 0, (hipStream_t)stream>>>(
+        G, cells, pts, query, nv_database, nv_query, B, Mp, nn_index, nn_dist);
+    PM_LAUNCHED("point_knn3_grid");
     return 0;
 }
 

@@ -25,6 +25,7 @@ def _dims(database, query, nv_database, nv_query):
 # grows with its neighbours, not with its sample), smaller ones by the scan over the query's sample.
 GRID_MIN_POINTS = 2048
 GRID_MAX_SAMPLES = 1 << 20
+KNN_CELLS_PER_POINT = 4.0        # cells of the nearest-neighbour grid per database point of a sample
 
 
 def _search(kind, database, query, nv_database, nv_query, size, nn_sample, grid_size=None):
@@ -79,6 +80,15 @@ def knn3(database, query, nv_database, nv_query):
     with torch.cuda.device(dev):
         nn_index = torch.empty((Mp, 3), dtype=I32, device=dev)
         nn_dist = torch.empty((Mp, 3), dtype=F32, device=dev)
+        if Mp and Np >= max(GRID_MIN_POINTS, 1) and 0 < B <= GRID_MAX_SAMPLES:
+            # a cell grid with about KNN_CELLS_PER_POINT cells per point of a sample: a query looks at the cells around it
+            grid = torch.empty(_lib.query("pmesh_point_grid_workspace_bytes", Np), dtype=torch.uint8, device=dev)
+            st = stream_of(database)
+            _lib.call("pmesh_point_grid_build", database.data_ptr(), nv_database.data_ptr(), B, Np, -float(KNN_CELLS_PER_POINT),
+                      grid.data_ptr(), grid.numel(), st)
+            _lib.call("pmesh_point_knn3_grid", grid.data_ptr(), database.data_ptr(), query.data_ptr(), nv_database.data_ptr(),
+                      nv_query.data_ptr(), B, Np, Mp, nn_index.data_ptr(), nn_dist.data_ptr(), st)
+            return nn_index, nn_dist
         _lib.call("pmesh_point_knn3", database.data_ptr(), query.data_ptr(), nv_database.data_ptr(), nv_query.data_ptr(), B, Np,
                   Mp, nn_index.data_ptr(), nn_dist.data_ptr(), stream_of(database))
     return nn_index, nn_dist

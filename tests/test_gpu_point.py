@@ -60,7 +60,8 @@ def test_range_cube_knn_bit_exact(cuda, monkeypatch, sizes, frac, radius, limit,
 def _searches(D, Q, ND, NQ, radius, limit):
     a = nnquery.range_search_(D, Q, ND, NQ, radius=radius, nnsample=limit)
     b = nnquery.cube_search_(D, Q, ND, NQ, length=2 * radius, nnsample=limit, gridsize=4)
-    return [n(t) for t in a + b]
+    c = nnquery.knn3_search_(D, Q, ND, NQ)
+    return [n(t) for t in a + b + c]
 
 
 @pytest.mark.parametrize("shape", ["plane", "far", "same", "spread", "nonfinite", "outside", "dense", "dense_all"])

@@ -43,6 +43,8 @@ def parse():
                          "block shapes, F2F 3->32 then F2V 32->32 with depth multiplier 2 (pi2_blocks.py:113-130)")
     ap.add_argument("--scale", type=float, default=1.0, help="facet-count scale of the scene workload")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--degree", type=int, default=3, choices=[0, 1, 2, 3, 4, 5],
+                    help="spherical-harmonic degree of the scene workload's filters (3 = the headline configuration)")
     ap.add_argument("--f2f-half", action="store_true",
                     help="facet2facet in its half-precision variant (one fp16 piece per operand, fp32 accumulation; "
                          "results within 1e-3 instead of 1e-5): a separate figure, never the default")
@@ -252,12 +254,16 @@ def run_conv_layer(args, torch, kind):
     from picassoplus_amd.mesh.pi_modules import conv3d, texture
     dev = torch.device("cuda:0")
     C, L = (32 if kind == "firstblock" else 64), 3           # first block: EncodeChannels[0] = 32 (scene_seg.py:28)
+    if args.degree != 3:
+        if kind != "scene":
+            sys.exit("--degree is a variant of the scene workload")
+        L = args.degree
     Cin, r = (3, 2) if kind == "firstblock" else (C, 1)      # F2F input channels, F2V depth multiplier
     if kind in ("scene", "firstblock"):
         mesh = S.scene_workload(seed=3000, n_rooms=8, scale=args.scale)
         d = build_conv_inputs(mesh, C, L, seed=3000, Cin=Cin, r=r)
         ops = ["f2f_fwd", "f2v_fwd", "f2v_bwd", "f2f_bwd_texture", "f2f_bwd_filter"]
-        name = "scene8x300k_F2F+F2V_C64_L3_fp32_fwd+bwd" if kind == "scene" else "scene8x300k_F2F3to32+F2V32r2_L3_fp32_fwd+bwd"
+        name = "scene8x300k_F2F+F2V_C64_L%d_fp32_fwd+bwd" % L if kind == "scene" else "scene8x300k_F2F3to32+F2V32r2_L3_fp32_fwd+bwd"
     else:
         mesh = S.shapes_workload(seed=2000, n_meshes=16)
         d = build_conv_inputs(mesh, C, L, seed=2000, tex_counts=3)
@@ -313,7 +319,8 @@ def run_conv_layer(args, torch, kind):
     timer.on = False
     _lib.set_call_hook(None)
     ms = (t1 - t0) * 1e3 / args.steps
-    per_op = {k.replace("_bf16", ""): v for k, v in timer.summary().items()}
+    # per entry point and step (a degree other than 3 calls an entry point once per block of 16 coefficients)
+    per_op = {k.replace("_bf16", ""): v for k, v in timer.totals(args.steps).items()}
     bf = conv_bytes_flops(d, ops, 2 if bf16 else 4)
     total_bytes = sum(b for b, _ in bf.values())
     dom = max(ops, key=lambda k: per_op.get(k, 0.0))
@@ -328,7 +335,7 @@ def run_conv_layer(args, torch, kind):
     else:
         roof = dict(bound="hbm", achieved=bf[dom][0] / (dom_ms * 1e-3) / 1e9, peak=HBM_PEAK_GBS, unit="GB/s")
     traffic = (measured_traffic("scene", "bf16" if bf16 else "f2f-half" if args.f2f_half else "", dom)
-               if (kind == "scene" and args.scale == 1.0) else None)
+               if (kind == "scene" and args.scale == 1.0 and L == 3) else None)
     roof.update(frac=roof["achieved"] / roof["peak"], traffic=traffic, kernel=dom, kernel_ms=dom_ms)
     # adjacency of the step's index tensors, built cold (fresh tensors, nothing cached, range checks included): what
     # a training loop that gets new index tensors with every batch pays per step on top of ms_per_step

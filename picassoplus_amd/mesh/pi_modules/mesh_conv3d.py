@@ -4,6 +4,8 @@ Same six functions, argument order and result shapes as the pybind module define
 picasso/mesh/pi_modules/source/mesh_conv3d.cpp:272-279; the arithmetic runs in
 libpicasso_mesh.so (HIP, gfx950) through the C ABI of include/picasso_mesh.h.
 """
+import os
+
 import torch
 
 from ... import _lib
@@ -75,11 +77,37 @@ def _f2v_dims(input, filter, coeff, face, nf_count, vt_map):
     return Nf, C, K, r, nf_count.shape[0], vt_map.shape[0]
 
 
+def _f2v_blocks_of_16(input, filter, coeff):
+    """The matrix-core kernels of facet2vertex take 16 coefficients.  From 9 coefficients on, any other count runs as
+    ceil(K / 16) such convolutions over zero-padded blocks (the output is linear in the pair filter x coefficients)
+    instead of on the vector-ALU kernels, whose cost grows with K.  Returns [(filter block (16,C,r), coefficient block
+    (Nf,16))], or None where the native call takes the operands as they are."""
+    K, C, r = filter.shape
+    if K == 16 or K < 9 or C * r < 32 or input.dtype != F32 or os.environ.get("PMESH_F2V_VALU") == "1":
+        return None
+    n = (K + 15) // 16
+    pad = torch.nn.functional.pad
+    blocks = []
+    for j in range(n):
+        if 16 * j + 16 <= K:
+            blocks.append((filter[16 * j:16 * j + 16].contiguous(), coeff[:, 16 * j:16 * j + 16].contiguous()))
+        else:                                                        # (only the last block is padded)
+            blocks.append((pad(filter[16 * j:], (0, 0, 0, 0, 0, 16 * j + 16 - K)), pad(coeff[:, 16 * j:], (0, 16 * j + 16 - K))))
+    return blocks
+
+
 def facet2vertex_forward(input, filter, coeff, face, nf_count, vt_map):
     """mesh_conv3d.cpp:33-74 -> (NvOut, C*r).  ``input`` may be bfloat16 (features in bf16 in HBM: the output is
     bfloat16 too, filter and coefficients stay float32)."""
     Nf, C, K, r, NvOut, NvIn = _f2v_dims(input, filter, coeff, face, nf_count, vt_map)
     dev = same_device(input, filter, coeff, face, nf_count, vt_map)
+    blocks = _f2v_blocks_of_16(input, filter, coeff)
+    if blocks is not None:
+        out = None
+        for fb, cb in blocks:
+            part = facet2vertex_forward(input, fb, cb, face, nf_count, vt_map)
+            out = part if out is None else out.add_(part)
+        return out
     rowptr, colidx = topology.vertex_csr(face, vt_map, NvOut)
     with torch.cuda.device(dev):
         out = torch.empty((NvOut, C * r), dtype=input.dtype, device=dev)
@@ -97,6 +125,14 @@ def facet2vertex_backward(grad_output, input, filter, coeff, face, nf_count, vt_
     if tuple(grad_output.shape) != (NvOut, C * r):
         raise RuntimeError("grad_output must have shape (NvOut, C*r)")
     dev = same_device(grad_output, input, filter, coeff, face, nf_count, vt_map)
+    blocks = _f2v_blocks_of_16(input, filter, coeff)
+    if blocks is not None:
+        gin, parts = None, []
+        for fb, cb in blocks:
+            g_in, g_f = facet2vertex_backward(grad_output, input, fb, cb, face, nf_count, vt_map)
+            gin = g_in if gin is None else gin.add_(g_in)
+            parts.append(g_f)
+        return [gin, torch.cat(parts, 0)[:K].contiguous()]
     if Nf:
         topology._check_range_cached(face, NvIn)
     with torch.cuda.device(dev):
@@ -129,11 +165,35 @@ def _f2f_dims(input, filter, bary_coeff, num_texture, forward):
     return T, Cin, Cout, F, num_texture.shape[0]
 
 
+def _blocks_of_16(input, filter, bary_coeff):
+    """The matrix-core kernels take 16 coefficients (degree 3).  Any other count is run as ceil(F / 16) such
+    convolutions: the filter and the coefficient rows are padded with zeros to a multiple of 16 and cut into blocks,
+    and ``G . W^T`` is the sum over the blocks (the convolution is linear in the pair).  Returns the list of
+    (filter block (Cout,Cin,16), coefficient block (T,16)), or None where the native call takes the operands as they are
+    (16 coefficients; bfloat16 features, whose block sums would be rounded once more; the shape-generic kernels asked
+    for by PMESH_F2F_GENERIC=1)."""
+    F = filter.shape[2]
+    if F == 16 or input.dtype != F32 or os.environ.get("PMESH_F2F_GENERIC") == "1":
+        return None
+    n = (F + 15) // 16
+    pad = torch.nn.functional.pad
+    cut = lambda t, j: (t[..., 16 * j:16 * j + 16].contiguous() if 16 * j + 16 <= F        # (only the last block is padded)
+                        else pad(t[..., 16 * j:], (0, 16 * j + 16 - F)))
+    return [(cut(filter, j), cut(bary_coeff, j)) for j in range(n)]
+
+
 def facet2facet_forward(input, filter, bary_coeff, num_texture):
     """mesh_conv3d.cpp:192-228; ``num_texture`` is the inclusive running total per facet.  ``input`` may be bfloat16
     (features in bf16 in HBM: bfloat16 output, float32 filter and coefficients, one fp16 product per element)."""
     T, Cin, Cout, F, Nf = _f2f_dims(input, filter, bary_coeff, num_texture, True)
     dev = same_device(input, filter, bary_coeff, num_texture)
+    blocks = _blocks_of_16(input, filter, bary_coeff)
+    if blocks is not None:
+        out = None
+        for fb, bb in blocks:
+            part = facet2facet_forward(input, fb, bb, num_texture)
+            out = part if out is None else out.add_(part)
+        return out
     with torch.cuda.device(dev):
         out = torch.empty((Nf, Cout), dtype=input.dtype, device=dev)
         nbytes = _lib.query("pmesh_f2f_fwd_workspace_bytes", Cin, Cout, F)
@@ -161,6 +221,11 @@ def facet2facet_forward_act(input, filter, bary_coeff, num_texture, bias=None, r
     if with_bits and Cout % 32:
         raise RuntimeError("the bit mask needs a multiple of 32 output channels")
     dev = same_device(input, filter, bary_coeff, num_texture, *[t for t in (bias, scale, shift) if t is not None])
+    if _blocks_of_16(input, filter, bary_coeff) is not None:
+        # other coefficient counts: the sum over the blocks of 16 first, the tail as one pass over it
+        from . import dense
+        conv = facet2facet_forward(input, filter, bary_coeff, num_texture)
+        return dense.bias_act_forward(conv, bias, relu, scale, shift, with_bits=with_bits)
     with torch.cuda.device(dev):
         out = torch.empty((Nf, Cout), dtype=F32, device=dev)
         bits = torch.empty((Nf, Cout // 32), dtype=torch.int32, device=dev) if with_bits else None
@@ -188,6 +253,16 @@ def facet2facet_backward_selected(grad_output, input, filter, bary_coeff, num_te
     if tuple(grad_output.shape) != (Nf, Cout):
         raise RuntimeError("grad_output must have shape (NfIn, Cout)")
     dev = same_device(grad_output, input, filter, bary_coeff, num_texture)
+    blocks = _blocks_of_16(input, filter, bary_coeff)
+    if blocks is not None:
+        # the texture gradient is the sum over the blocks, the filter gradient their concatenation
+        gin, parts = None, []
+        for fb, bb in blocks:
+            g_in, g_f = facet2facet_backward_selected(grad_output, input, fb, bb, num_texture, needs)
+            if needs[0]:
+                gin = g_in if gin is None else gin.add_(g_in)
+            parts.append(g_f)
+        return [gin, torch.cat(parts, 2)[:, :, :F].contiguous() if needs[1] else None]
     sfx = "_bf16" if input.dtype == BF16 else ""
     with torch.cuda.device(dev):
         gin = torch.empty((T, Cin), dtype=input.dtype, device=dev) if needs[0] else None

@@ -182,11 +182,12 @@ def test_texture_interpolation_rejects_bad_totals(cuda):
                                                 ("sphere2", 160, 1, 12, True), ("sphere2", 64, 2, 16, False),
                                                 ("fans", 64, 1, 16, False), ("fans", 40, 1, 16, True),
                                                 ("sphere3", 200, 1, 16, True), ("sphere2", 12, 3, 16, False),
-                                                ("room_small", 128, 2, 16, True), ("sphere3", 33, 1, 16, False)])
+                                                ("room_small", 128, 2, 16, True), ("sphere3", 33, 1, 16, False),
+                                                ("sphere3", 64, 1, 25, False), ("room_small", 32, 2, 36, True)])
 @pytest.mark.parametrize("path", ["default", "valu"])
 def test_f2v_parity(cuda, native_options, mesh, C, r, K, strided, path):
-    """default: matrix-core kernels where they apply (16 coefficients, at least 32 output channels);
-    valu: the vector-ALU kernels for every shape."""
+    """default: matrix-core kernels where they apply (at least 32 output channels; 16 coefficients, or from 9 on as
+    zero-padded blocks of 16); valu: the vector-ALU kernels for every shape."""
     say("case f2v", mesh, C, r, K, strided, path)
     native_options(PMESH_F2V_VALU="1" if path == "valu" else "0")
     v, f = mesh_case(mesh)
@@ -249,14 +250,12 @@ def test_f2v_unit_count_is_plain_scatter(cuda):
 @pytest.mark.parametrize("path", ["default", "generic", "bf16x3", "half"])
 def test_f2f_parity(cuda, native_options, nf, Cin, Cout, F, kmax, path):
     """``generic`` forces the shape-generic kernels (fp32 matrix instruction) and ``bf16x3`` the three-piece bf16
-    kernels, also where the two-piece fp16 kernels (the default for 16 coefficients) apply; ``half`` their
+    kernels, also where the two-piece fp16 kernels (the default, 16 coefficients per block) apply; ``half`` their
     half-precision variant (one fp16 piece per operand, fp32 accumulation), held to 1e-3 of the largest reference
     value instead of 1e-5."""
     say("case f2f", nf, Cin, Cout, F, kmax, path)
-    if path == "generic" and F != 16:
-        pytest.skip("shape already runs the generic kernels")
-    if path in ("bf16x3", "half") and F != 16:
-        pytest.skip("the split kernels need 16 coefficients")
+    # other coefficient counts than 16 run as blocks of 16 (zero padded) through whichever split kernels are selected;
+    # ``generic`` takes them as they are
     native_options(PMESH_F2F_HALF="1" if path == "half" else "0", PMESH_F2F_GENERIC="1" if path == "generic" else "0",
                    PMESH_F2F_BF16X3="1" if path == "bf16x3" else "0")
     rng = np.random.default_rng(13)

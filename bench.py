@@ -125,19 +125,14 @@ TRAFFIC_KERNELS = {
 }
 
 
-TIMED_SOURCES = ("mesh_f2f", "mesh_f2v", "mesh_rows", "mesh_dense", "mesh_texture", "pcloud_ops", "common", "f2f_internal",
-                 "rows_internal", "sph_internal")
-
-
 def build_id():
-    """Identity of the kernels being timed: hash over the sources that hold them (convolutions, pooling, tails,
-    texture interpolation, point convolution and their shared headers; index builds, neighbour searches and mesh
-    preparation are not timed here)."""
+    """Identity of the kernels being timed: hash over every source of the native library (kernels of all workloads,
+    the index builds, neighbour searches and mesh preparation included, and their shared headers)."""
     import hashlib
     h = hashlib.sha256()
     csrc = os.path.join(ROOT, "picassoplus_amd", "csrc")
     for name in sorted(os.listdir(csrc)):
-        if name.endswith((".hip", ".h", ".cpp")) and name.startswith(TIMED_SOURCES):
+        if name.endswith((".hip", ".h", ".cpp")):
             h.update(name.encode())
             h.update(open(os.path.join(csrc, name), "rb").read())
     return h.hexdigest()[:16]

@@ -355,6 +355,18 @@ int pmesh_edge_costs(const float *vertex, const float *quadric, const int32_t *e
 int pmesh_cluster_vertices_host(const int32_t *edge_vi, const int32_t *edge_vj, int64_t n_edges, int32_t vt_start,
                                 int32_t vt_num, int32_t n_remove, int32_t *vt_replace);
 
+/* After the clustering (decimate_gpu.cu:487-549): pmesh_simplify_faces writes the facets over the clusters'
+ * representatives (new_face (Nf,3)), which of them collapse (degenerate (Nf) bytes, alive = 1 - degenerate as int32
+ * for the caller's running totals) and which vertices keep a facet (kept (Nv), cleared here first);
+ * pmesh_simplify_renumber, given kept_total = inclusive running total of kept, the output numbering: vt_map (Nv)
+ * = kept_total - 1 for kept vertices, -1 otherwise, and face_out (Nf,3) = vt_map of the new corners for live
+ * facets (collapsed facets keep their unmapped corners, as in the reference). */
+int pmesh_simplify_faces(const int32_t *face, const int32_t *vt_replace, int64_t Nf, int64_t Nv, int32_t *new_face,
+                         uint8_t *degenerate, int32_t *alive, int32_t *kept, pmesh_stream_t stream);
+int pmesh_simplify_renumber(const int32_t *new_face, const uint8_t *degenerate, const int32_t *kept,
+                            const int32_t *kept_total, int64_t Nf, int64_t Nv, int32_t *vt_map, int32_t *face_out,
+                            pmesh_stream_t stream);
+
 /* The same two passes (clusterVertices, decimate_gpu.cu:561-614) for the whole batch on the DEVICE, in four steps
  * between which the caller cuts the chosen edges by their rank within the sample (two prefix sums): the result is
  * that of pmesh_cluster_vertices_host sample by sample.  edge_vi / edge_vj: the candidate edges of all samples in

@@ -93,6 +93,8 @@ SIGNATURES = {
     "pmesh_cluster_vertices_host": (I, [P, P, L, I, I, I, P]),
     "pmesh_edge_list_count": (I, [P, P, P, L, L, P, P, P, P]),
     "pmesh_edge_list_fill": (I, [P, P, P, L, L, P, P, P, P, P, P, P, P]),
+    "pmesh_simplify_faces": (I, [P, P, L, L, P, P, P, P, P]),
+    "pmesh_simplify_renumber": (I, [P, P, P, P, L, L, P, P, P]),
     "pmesh_cluster_match": (I, [P, P, L, L, P, P, P, P, I, P]),
     "pmesh_cluster_contract_pairs": (I, [P, P, P, L, P, P]),
     "pmesh_cluster_attach_propose": (I, [P, P, P, P, L, L, P, P, P, P]),

@@ -406,9 +406,96 @@ __global__ __launch_bounds__(kBlock) void attach_apply_k(const int *__restrict__
     atomicAdd(vt_replace + rep, 1);
 }
 
+// ----------------------------------------------------------------------------------------
+// After the clustering: the facets over the clusters' representatives, which of them collapse (two corners in one
+// cluster), which vertices keep a facet (decimate_gpu.cu:487-496), and -- once the caller has the running totals of
+// the kept vertices -- the output numbering of vertices and facets (:519-549).
+__global__ __launch_bounds__(kBlock) void simplify_faces_k(const int *__restrict__ face, const int *__restrict__ vt_replace,
+                                                           int64_t Nf, int64_t Nv, int *__restrict__ new_face,
+                                                           unsigned char *__restrict__ degenerate, int *__restrict__ alive,
+                                                           int *__restrict__ kept)
+{
+    const int64_t f = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (f >= Nf) return;
+    int c[3];
+#pragma unroll
+    for (int j = 0; j < 3; ++j) {
+        const int v = face[3 * f + j];
+        const int r = (v >= 0 && v < Nv) ? vt_replace[v] : 0;
+        c[j] = r < 0 ? -r : v;
+        new_face[3 * f + j] = c[j];
+    }
+    const bool dg = c[0] == c[1] || c[0] == c[2] || c[1] == c[2];
+    degenerate[f] = dg ? 1 : 0;
+    alive[f] = dg ? 0 : 1;
+    if (!dg) {
+#pragma unroll
+        for (int j = 0; j < 3; ++j)
+            if (c[j] >= 0 && c[j] < Nv) kept[c[j]] = 1;          // (every writer writes 1)
+    }
+}
+
+// kept_total = inclusive running total of kept
+__global__ __launch_bounds__(kBlock) void simplify_vertex_map_k(const int *__restrict__ kept, const int *__restrict__ kept_total,
+                                                                int64_t Nv, int *__restrict__ vt_map)
+{
+    const int64_t v = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (v < Nv) vt_map[v] = kept[v] ? kept_total[v] - 1 : -1;
+}
+
+__global__ __launch_bounds__(kBlock) void simplify_face_out_k(const int *__restrict__ new_face, const unsigned char *__restrict__ degenerate,
+                                                              const int *__restrict__ kept_total, int64_t Nf, int64_t Nv,
+                                                              int *__restrict__ face_out)
+{
+    const int64_t f = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (f >= Nf) return;
+    const bool dg = degenerate[f] != 0;
+#pragma unroll
+    for (int j = 0; j < 3; ++j) {
+        const int c = new_face[3 * f + j];
+        face_out[3 * f + j] = (dg || c < 0 || c >= Nv) ? c : kept_total[c] - 1;       // corners of a live facet are kept vertices
+    }
+}
+
 }  // namespace pmesh
 
 using namespace pmesh;
+
+extern "C" int pmesh_simplify_faces(const int32_t *face, const int32_t *vt_replace, int64_t Nf, int64_t Nv, int32_t *new_face,
+                                    uint8_t *degenerate, int32_t *alive, int32_t *kept, pmesh_stream_t stream)
+{
+    clear_error();
+    PM_REQUIRE(Nf >= 0 && Nv >= 0 && Nv <= INT32_MAX && Nf <= INT32_MAX / 3, "simplify_faces: bad sizes");
+    hipStream_t st = (hipStream_t)stream;
+    if (Nv > 0) {
+        PM_REQUIRE(kept, "simplify_faces: null pointer");
+        fill_int_k<<<dim3((unsigned)ceil_div(Nv, kBlock)), dim3(kBlock), 0, st>>>(kept, 0, Nv);
+    }
+    if (Nf == 0) return 0;
+    PM_REQUIRE(face && vt_replace && new_face && degenerate && alive && kept, "simplify_faces: null pointer");
+    simplify_faces_k<<<dim3((unsigned)ceil_div(Nf, kBlock)), dim3(kBlock), 0, st>>>(face, vt_replace, Nf, Nv, new_face, degenerate, alive, kept);
+    PM_LAUNCHED("simplify_faces");
+    return 0;
+}
+
+extern "C" int pmesh_simplify_renumber(const int32_t *new_face, const uint8_t *degenerate, const int32_t *kept,
+                                       const int32_t *kept_total, int64_t Nf, int64_t Nv, int32_t *vt_map, int32_t *face_out,
+                                       pmesh_stream_t stream)
+{
+    clear_error();
+    PM_REQUIRE(Nf >= 0 && Nv >= 0 && Nv <= INT32_MAX && Nf <= INT32_MAX / 3, "simplify_renumber: bad sizes");
+    hipStream_t st = (hipStream_t)stream;
+    if (Nv > 0) {
+        PM_REQUIRE(kept && kept_total && vt_map, "simplify_renumber: null pointer");
+        simplify_vertex_map_k<<<dim3((unsigned)ceil_div(Nv, kBlock)), dim3(kBlock), 0, st>>>(kept, kept_total, Nv, vt_map);
+    }
+    if (Nf > 0) {
+        PM_REQUIRE(new_face && degenerate && kept_total && face_out, "simplify_renumber: null pointer");
+        simplify_face_out_k<<<dim3((unsigned)ceil_div(Nf, kBlock)), dim3(kBlock), 0, st>>>(new_face, degenerate, kept_total, Nf, Nv, face_out);
+    }
+    PM_LAUNCHED("simplify_renumber");
+    return 0;
+}
 
 extern "C" int pmesh_edge_list_count(const int32_t *face, const int32_t *rowptr, const int32_t *colidx, int64_t Nv, int64_t Nf,
                                      int32_t *counts, int32_t *spill, int32_t *need_spill, pmesh_stream_t stream)

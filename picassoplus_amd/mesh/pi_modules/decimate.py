@@ -268,29 +268,39 @@ def simplify(vertexIn, faceIn, geometryIn, nvIn_cumsum, mfIn_cumsum, nv2Remove, 
         vt_replace = cluster_vertices_device(evi[perm], evj[perm], sample, nvIn_cumsum, nv2Remove, Nv)
     else:
         vt_replace = torch.from_numpy(cluster_vertices(evi[perm], evj[perm], sample, nvIn_cumsum, nv2Remove, Nv)).to(dev)
+    Nf = faceIn.shape[0]
+    B = nvIn_cumsum.shape[0]
+    st = stream_of(vertexIn)
     with torch.cuda.device(dev):
-        ids = torch.arange(Nv, dtype=I32, device=dev)
-        rep = torch.where(vt_replace < 0, -vt_replace, ids).long()
-        new_face = rep[faceIn.long()]
-        degenerate = (new_face[:, 0] == new_face[:, 1]) | (new_face[:, 0] == new_face[:, 2]) | (new_face[:, 1] == new_face[:, 2])
-        kept = torch.zeros(Nv, dtype=torch.int64, device=dev)
-        kept[new_face[~degenerate].reshape(-1)] = 1
-        # vertices that keep a facet are numbered in order; contracted vertices and those left without a facet get -1
-        vt_map = torch.where(kept > 0, torch.cumsum(kept, 0) - 1, torch.full_like(kept, -1)).to(I32)
-        face_out = torch.where(degenerate[:, None], new_face, vt_map.long()[new_face]).to(I32)
-        sample_v = torch.bucketize(ids.long(), nvIn_cumsum.long(), right=True)
-        sample_f = torch.bucketize(torch.arange(faceIn.shape[0], device=dev), mfIn_cumsum.long(), right=True)
-        B = nvIn_cumsum.shape[0]
-        nv_out = torch.bincount(sample_v[kept > 0], minlength=B)[:B].to(I32)
-        mf_out = torch.bincount(sample_f[~degenerate], minlength=B)[:B].to(I32)
+        # facets over the representatives, collapsed facets, vertices that keep a facet; then the output numbering from
+        # the running totals: vertices that keep a facet are numbered in order, the others get -1
+        new_face = torch.empty((Nf, 3), dtype=I32, device=dev)
+        degenerate = torch.empty(Nf, dtype=torch.bool, device=dev)
+        alive = torch.empty(Nf, dtype=I32, device=dev)
+        kept = torch.empty(Nv, dtype=I32, device=dev)
+        faceIn = faceIn.contiguous()
+        _lib.call("pmesh_simplify_faces", faceIn.data_ptr(), vt_replace.data_ptr(), Nf, Nv, new_face.data_ptr(),
+                  degenerate.data_ptr(), alive.data_ptr(), kept.data_ptr(), st)
+        kept_total = torch.cumsum(kept, 0, dtype=I32)
+        alive_total = torch.cumsum(alive, 0, dtype=I32)
+        vt_map = torch.empty(Nv, dtype=I32, device=dev)
+        face_out = torch.empty((Nf, 3), dtype=I32, device=dev)
+        _lib.call("pmesh_simplify_renumber", new_face.data_ptr(), degenerate.data_ptr(), kept.data_ptr(), kept_total.data_ptr(),
+                  Nf, Nv, vt_map.data_ptr(), face_out.data_ptr(), st)
+
+        def per_sample(total, ends):
+            # counts per sample from a running total read at the samples' ends
+            at = torch.cat([total.new_zeros(1), total])[ends.long().clamp(0, total.shape[0])]
+            return (at - torch.cat([at.new_zeros(1), at[:-1]])).to(I32)
+
+        nv_out = per_sample(kept_total, nvIn_cumsum)
+        mf_out = per_sample(alive_total, mfIn_cumsum)
         # contracted position = mean of the cluster's vertices (all D columns) in the row of its representative; rows of
-        # contracted vertices stay zero (decimate_gpu.cu:401-441)
-        is_rep = vt_replace >= 0
-        rep_row = torch.where(is_rep, torch.cumsum(is_rep, 0) - 1, torch.full_like(kept, -1)).to(I32)
-        n_rep = int(is_rep.sum())
-        vertex_out = torch.zeros((Nv, D), dtype=F32, device=dev)
-        if n_rep:
-            vertex_out[is_rep] = mesh_pool3d.avg_forward(vertexIn, vt_replace, rep_row, torch.empty((n_rep, 1), dtype=F32, device=dev))
+        # contracted vertices stay zero (decimate_gpu.cu:401-441): the average pooling op over a map that sends every
+        # representative to its own row
+        own_row = torch.where(vt_replace >= 0, torch.arange(Nv, dtype=I32, device=dev), torch.full_like(vt_replace, -1))
+        vertex_out = (mesh_pool3d.avg_forward(vertexIn, vt_replace, own_row, torch.empty((Nv, 1), dtype=F32, device=dev))
+                      if Nv else torch.zeros((0, D), dtype=F32, device=dev))
     return [vertex_out, face_out, degenerate, vt_replace, vt_map, nv_out, mf_out]
 
 
@@ -304,18 +314,30 @@ def mesh_decimation_(vertexIn, faceIn, geometryIn, nvIn, mfIn, nvOut, useArea=Tr
     nv2Remove = (nvIn - nvOut).to(I32)
     repIn = torch.zeros(vertexIn.shape[0], dtype=I32, device=dev)
     mapIn = torch.arange(vertexIn.shape[0], dtype=I32, device=dev)
-    while bool(torch.any(nv2Remove > 0)):
+    left = int(nv2Remove.max()) if nv2Remove.numel() else 0
+    while left > 0:
         nv_cum = torch.cumsum(nvIn, 0, dtype=I32)
         mf_cum = torch.cumsum(mfIn, 0, dtype=I32)
         vertexOut, faceOut, isDegenerate, repOut, mapOut, nvOut, mfOut = simplify(
             vertexIn, faceIn, geometryIn, nv_cum, mf_cum, nv2Remove.contiguous(), useArea, wgtBnd)
         removed = nvIn - nvOut
-        if not bool(torch.any(removed > 0)):
+        still = (nv2Remove - removed).to(I32)
+        # what the host needs of this round, in one transfer: did it remove anything, the sizes of the next round's
+        # arrays, and whether a sample still has vertices to remove
+        most, nv_total, mf_total, left = torch.stack([removed.max(), nvOut.sum(), mfOut.sum(), still.max()]).tolist()
+        if most <= 0:
             break                                     # nothing left that can be contracted (no candidate edges)
-        faceIn = faceOut[~isDegenerate].contiguous()
-        vertexIn = vertexOut[mapOut >= 0].contiguous()
+        faceIn = _rows_where(faceOut, ~isDegenerate, mf_total)
+        vertexIn = _rows_where(vertexOut, mapOut >= 0, nv_total)
         geometryIn = compute_triangle_geometry_(vertexIn, faceIn)
-        nv2Remove = (nv2Remove - removed).to(I32)
+        nv2Remove = still
         repIn, mapIn = combine_clusters_(repIn, mapIn, repOut, mapOut)
         nvIn, mfIn = nvOut, mfOut
     return vertexIn, faceIn, geometryIn, nvIn, mfIn, repIn, mapIn
+
+
+def _rows_where(rows, mask, count):
+    """rows[mask] when the number of selected rows is known already (no second trip to the host for it)."""
+    if hasattr(torch, "nonzero_static"):
+        return rows.index_select(0, torch.nonzero_static(mask, size=int(count)).squeeze(1))
+    return rows[mask].contiguous()

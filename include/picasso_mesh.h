@@ -370,28 +370,32 @@ int pmesh_simplify_renumber(const int32_t *new_face, const uint8_t *degenerate, 
 /* The same two passes (clusterVertices, decimate_gpu.cu:561-614) for the whole batch on the DEVICE, in four steps
  * between which the caller cuts the chosen edges by their rank within the sample (two prefix sums): the result is
  * that of pmesh_cluster_vertices_host sample by sample.  edge_vi / edge_vj: the candidate edges of all samples in
- * contraction order, vi < vj, every edge inside one sample; the edge's position in the list is its rank.
+ * ascending (vi, vj) order (vi < vj, every edge inside one sample; neighbouring threads then touch neighbouring
+ * vertices), edge_rank: each edge's position in the contraction order (distinct integers, ascending within a sample
+ * in the order the serial routine would walk them).
  *   pmesh_cluster_match           `rounds` rounds of the first pass's fixed point (an edge is chosen when it is the
- *                                 first edge with two free ends at both of its ends).  state (Nv) and chosen
+ *                                 lowest-ranked edge with two free ends at both of its ends).  state (Nv) and chosen
  *                                 (n_edges) are zero before the first call and carry over; best (Nv) is scratch.
  *                                 status[0] <- 1 while an edge with two free ends is left (call again), status[1]
  *                                 <- 1 if an edge is not (0 <= vi < vj < Nv) -- such an edge is left out.
  *   pmesh_cluster_contract_pairs  vt_replace[vi] = -vj, vt_replace[vj] = 1 for the edges with keep != 0 (the chosen
  *                                 edges whose rank among the sample's chosen edges is within its budget).
  *   pmesh_cluster_attach_propose  second pass, for the samples with sample_open != 0 (budget not exhausted by the
- *                                 first): first_edge (Nv) <- for every free vertex the first edge to a covered vertex
- *                                 whose cluster's representative is not vertex 0; attaches (n_edges) <- 1 for these.
+ *                                 first): first_edge (Nv) <- for every free vertex the rank of its first edge to a
+ *                                 covered vertex whose cluster's representative is not vertex 0; attaches (n_edges)
+ *                                 <- 1 for these edges.
  *   pmesh_cluster_attach          for the edges with keep != 0 among them: the free end joins the covered end's
  *                                 cluster; pairs = a copy of vt_replace as the first pass left it. */
-int pmesh_cluster_match(const int32_t *edge_vi, const int32_t *edge_vj, int64_t n_edges, int64_t Nv, int32_t *state,
-                        int32_t *best, int32_t *chosen, int32_t *status, int rounds, pmesh_stream_t stream);
+int pmesh_cluster_match(const int32_t *edge_vi, const int32_t *edge_vj, const int32_t *edge_rank, int64_t n_edges, int64_t Nv,
+                        int32_t *state, int32_t *best, int32_t *chosen, int32_t *status, int rounds, pmesh_stream_t stream);
 int pmesh_cluster_contract_pairs(const int32_t *edge_vi, const int32_t *edge_vj, const int32_t *keep, int64_t n_edges,
                                  int32_t *vt_replace, pmesh_stream_t stream);
-int pmesh_cluster_attach_propose(const int32_t *edge_vi, const int32_t *edge_vj, const int32_t *edge_sample,
-                                 const int32_t *sample_open, int64_t n_edges, int64_t Nv, const int32_t *vt_replace,
-                                 int32_t *first_edge, int32_t *attaches, pmesh_stream_t stream);
-int pmesh_cluster_attach(const int32_t *edge_vi, const int32_t *edge_vj, const int32_t *keep, int64_t n_edges,
-                         const int32_t *first_edge, const int32_t *pairs, int32_t *vt_replace, pmesh_stream_t stream);
+int pmesh_cluster_attach_propose(const int32_t *edge_vi, const int32_t *edge_vj, const int32_t *edge_rank,
+                                 const int32_t *edge_sample, const int32_t *sample_open, int64_t n_edges, int64_t Nv,
+                                 const int32_t *vt_replace, int32_t *first_edge, int32_t *attaches, pmesh_stream_t stream);
+int pmesh_cluster_attach(const int32_t *edge_vi, const int32_t *edge_vj, const int32_t *edge_rank, const int32_t *keep,
+                         int64_t n_edges, const int32_t *first_edge, const int32_t *pairs, int32_t *vt_replace,
+                         pmesh_stream_t stream);
 
 /* ------------------------------------------------------------------ pointwise tail of the convs
  * replaces the PyTorch ops that follow every convolution (picasso/mesh/layers.py:114-119, 169-174,

@@ -95,10 +95,10 @@ SIGNATURES = {
     "pmesh_edge_list_fill": (I, [P, P, P, L, L, P, P, P, P, P, P, P, P]),
     "pmesh_simplify_faces": (I, [P, P, L, L, P, P, P, P, P]),
     "pmesh_simplify_renumber": (I, [P, P, P, P, L, L, P, P, P]),
-    "pmesh_cluster_match": (I, [P, P, L, L, P, P, P, P, I, P]),
+    "pmesh_cluster_match": (I, [P, P, P, L, L, P, P, P, P, I, P]),
     "pmesh_cluster_contract_pairs": (I, [P, P, P, L, P, P]),
-    "pmesh_cluster_attach_propose": (I, [P, P, P, P, L, L, P, P, P, P]),
-    "pmesh_cluster_attach": (I, [P, P, P, L, P, P, P, P]),
+    "pmesh_cluster_attach_propose": (I, [P, P, P, P, P, L, L, P, P, P, P]),
+    "pmesh_cluster_attach": (I, [P, P, P, P, L, P, P, P, P]),
     "pmesh_dense_fwd": (I, [P, P, P, P, P, I, P, P, L, I, I, P]),
     "pmesh_v2f_dense_fwd": (I, [P, P, P, P, P, P, P, I, P, P, P, L, L, I, I, P]),
     "pmesh_dense_bwd_workspace_bytes": (Z, [L, I, I]),

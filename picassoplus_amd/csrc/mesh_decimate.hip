@@ -303,28 +303,32 @@ __global__ __launch_bounds__(kBlock) void match_check_k(const int *__restrict__ 
     if (!(a >= 0 && a < b && b < Nv)) status[1] = 1;
 }
 
-__global__ __launch_bounds__(kBlock) void match_propose_k(const int *__restrict__ evi, const int *__restrict__ evj, int64_t E,
-                                                          int64_t Nv, const int *__restrict__ state, int *__restrict__ best)
+__global__ __launch_bounds__(kBlock) void match_propose_k(const int *__restrict__ evi, const int *__restrict__ evj,
+                                                          const int *__restrict__ rank, int64_t E, int64_t Nv,
+                                                          const int *__restrict__ state, int *__restrict__ best)
 {
-    const int64_t r = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-    if (r >= E) return;
-    const int a = evi[r], b = evj[r];
+    const int64_t e = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (e >= E) return;
+    const int a = evi[e], b = evj[e];
     if (!(a >= 0 && a < b && b < Nv)) return;
     if (state[a] | state[b]) return;
-    atomicMin(best + a, (int)r);
-    atomicMin(best + b, (int)r);
+    const int r = rank[e];
+    atomicMin(best + a, r);
+    atomicMin(best + b, r);
 }
 
-__global__ __launch_bounds__(kBlock) void match_select_k(const int *__restrict__ evi, const int *__restrict__ evj, int64_t E,
-                                                         int64_t Nv, int *__restrict__ state, const int *__restrict__ best,
+__global__ __launch_bounds__(kBlock) void match_select_k(const int *__restrict__ evi, const int *__restrict__ evj,
+                                                         const int *__restrict__ rank, int64_t E, int64_t Nv,
+                                                         int *__restrict__ state, const int *__restrict__ best,
                                                          int *__restrict__ chosen)
 {
-    const int64_t r = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-    if (r >= E) return;
-    const int a = evi[r], b = evj[r];
+    const int64_t e = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (e >= E) return;
+    const int a = evi[e], b = evj[e];
     if (!(a >= 0 && a < b && b < Nv)) return;
-    if (best[a] == (int)r && best[b] == (int)r) {
-        chosen[r] = 1;
+    const int r = rank[e];
+    if (best[a] == r && best[b] == r) {
+        chosen[e] = 1;
         state[a] = 1;
         state[b] = 1;
     }
@@ -363,43 +367,45 @@ __device__ __forceinline__ bool attach_ends(int a, int b, const int *__restrict_
 }
 
 __global__ __launch_bounds__(kBlock) void attach_propose_k(const int *__restrict__ evi, const int *__restrict__ evj,
-                                                           const int *__restrict__ sample, const int *__restrict__ open,
-                                                           int64_t E, int64_t Nv, const int *__restrict__ vt_replace,
-                                                           int *__restrict__ first_edge)
+                                                           const int *__restrict__ rank, const int *__restrict__ sample,
+                                                           const int *__restrict__ open, int64_t E, int64_t Nv,
+                                                           const int *__restrict__ vt_replace, int *__restrict__ first_edge)
 {
-    const int64_t r = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-    if (r >= E || !open[sample[r]]) return;
-    const int a = evi[r], b = evj[r];
+    const int64_t e = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (e >= E || !open[sample[e]]) return;
+    const int a = evi[e], b = evj[e];
     if (!(a >= 0 && a < b && b < Nv)) return;
     int rep, fr;
-    if (attach_ends(a, b, vt_replace, rep, fr)) atomicMin(first_edge + fr, (int)r);
+    if (attach_ends(a, b, vt_replace, rep, fr)) atomicMin(first_edge + fr, rank[e]);
 }
 
 __global__ __launch_bounds__(kBlock) void attach_flag_k(const int *__restrict__ evi, const int *__restrict__ evj,
-                                                        const int *__restrict__ sample, const int *__restrict__ open,
-                                                        int64_t E, int64_t Nv, const int *__restrict__ vt_replace,
-                                                        const int *__restrict__ first_edge, int *__restrict__ attaches)
+                                                        const int *__restrict__ rank, const int *__restrict__ sample,
+                                                        const int *__restrict__ open, int64_t E, int64_t Nv,
+                                                        const int *__restrict__ vt_replace, const int *__restrict__ first_edge,
+                                                        int *__restrict__ attaches)
 {
-    const int64_t r = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-    if (r >= E) return;
+    const int64_t e = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (e >= E) return;
     int flag = 0;
-    const int a = evi[r], b = evj[r];
-    if (open[sample[r]] && a >= 0 && a < b && b < Nv) {
+    const int a = evi[e], b = evj[e];
+    if (open[sample[e]] && a >= 0 && a < b && b < Nv) {
         int rep, fr;
-        if (attach_ends(a, b, vt_replace, rep, fr)) flag = first_edge[fr] == (int)r;
+        if (attach_ends(a, b, vt_replace, rep, fr)) flag = first_edge[fr] == rank[e];
     }
-    attaches[r] = flag;
+    attaches[e] = flag;
 }
 
 // first_edge tells the free end of a kept edge (vt_replace is being written here and can no longer say)
 __global__ __launch_bounds__(kBlock) void attach_apply_k(const int *__restrict__ evi, const int *__restrict__ evj,
-                                                         const int *__restrict__ keep, int64_t E, const int *__restrict__ first_edge,
-                                                         const int *__restrict__ pairs, int *__restrict__ vt_replace)
+                                                         const int *__restrict__ rank, const int *__restrict__ keep, int64_t E,
+                                                         const int *__restrict__ first_edge, const int *__restrict__ pairs,
+                                                         int *__restrict__ vt_replace)
 {
-    const int64_t r = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-    if (r >= E || !keep[r]) return;
-    const int a = evi[r], b = evj[r];
-    const int fr = first_edge[a] == (int)r ? a : b, cov = fr == a ? b : a;
+    const int64_t e = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (e >= E || !keep[e]) return;
+    const int a = evi[e], b = evj[e];
+    const int fr = first_edge[a] == rank[e] ? a : b, cov = fr == a ? b : a;
     const int rc = pairs[cov];              // the first pass's entry of the covered end: not written by this kernel
     const int rep = rc < 0 ? -rc : cov;
     vt_replace[fr] = -rep;
@@ -523,8 +529,9 @@ extern "C" int pmesh_edge_list_fill(const int32_t *face, const int32_t *rowptr, 
     return 0;
 }
 
-extern "C" int pmesh_cluster_match(const int32_t *edge_vi, const int32_t *edge_vj, int64_t n_edges, int64_t Nv, int32_t *state,
-                                   int32_t *best, int32_t *chosen, int32_t *status, int rounds, pmesh_stream_t stream)
+extern "C" int pmesh_cluster_match(const int32_t *edge_vi, const int32_t *edge_vj, const int32_t *edge_rank, int64_t n_edges,
+                                   int64_t Nv, int32_t *state, int32_t *best, int32_t *chosen, int32_t *status, int rounds,
+                                   pmesh_stream_t stream)
 {
     clear_error();
     PM_REQUIRE(n_edges >= 0 && n_edges < kNoEdge && Nv >= 0 && Nv <= INT32_MAX && rounds >= 1 && rounds <= 64,
@@ -534,13 +541,13 @@ extern "C" int pmesh_cluster_match(const int32_t *edge_vi, const int32_t *edge_v
     fill_int_k<<<dim3(1), dim3(kBlock), 0, st>>>(status, 0, 2);
     PM_LAUNCHED("cluster_match(status)");
     if (n_edges == 0 || Nv == 0) return 0;
-    PM_REQUIRE(edge_vi && edge_vj && state && best && chosen, "cluster_match: null pointer");
+    PM_REQUIRE(edge_vi && edge_vj && edge_rank && state && best && chosen, "cluster_match: null pointer");
     const dim3 ge((unsigned)ceil_div(n_edges, kBlock)), gv((unsigned)ceil_div(Nv, kBlock)), blk(kBlock);
     match_check_k<<<ge, blk, 0, st>>>(edge_vi, edge_vj, n_edges, Nv, status);
     for (int i = 0; i < rounds; ++i) {
         fill_int_k<<<gv, blk, 0, st>>>(best, kNoEdge, Nv);
-        match_propose_k<<<ge, blk, 0, st>>>(edge_vi, edge_vj, n_edges, Nv, state, best);
-        match_select_k<<<ge, blk, 0, st>>>(edge_vi, edge_vj, n_edges, Nv, state, best, chosen);
+        match_propose_k<<<ge, blk, 0, st>>>(edge_vi, edge_vj, edge_rank, n_edges, Nv, state, best);
+        match_select_k<<<ge, blk, 0, st>>>(edge_vi, edge_vj, edge_rank, n_edges, Nv, state, best, chosen);
     }
     match_left_k<<<ge, blk, 0, st>>>(edge_vi, edge_vj, n_edges, Nv, state, status);
     PM_LAUNCHED("cluster_match");
@@ -559,31 +566,33 @@ extern "C" int pmesh_cluster_contract_pairs(const int32_t *edge_vi, const int32_
     return 0;
 }
 
-extern "C" int pmesh_cluster_attach_propose(const int32_t *edge_vi, const int32_t *edge_vj, const int32_t *edge_sample,
-                                            const int32_t *sample_open, int64_t n_edges, int64_t Nv, const int32_t *vt_replace,
-                                            int32_t *first_edge, int32_t *attaches, pmesh_stream_t stream)
+extern "C" int pmesh_cluster_attach_propose(const int32_t *edge_vi, const int32_t *edge_vj, const int32_t *edge_rank,
+                                            const int32_t *edge_sample, const int32_t *sample_open, int64_t n_edges, int64_t Nv,
+                                            const int32_t *vt_replace, int32_t *first_edge, int32_t *attaches,
+                                            pmesh_stream_t stream)
 {
     clear_error();
     PM_REQUIRE(n_edges >= 0 && n_edges < kNoEdge && Nv >= 0 && Nv <= INT32_MAX, "cluster_attach_propose: bad sizes");
     if (n_edges == 0 || Nv == 0) return 0;
-    PM_REQUIRE(edge_vi && edge_vj && edge_sample && sample_open && vt_replace && first_edge && attaches, "cluster_attach_propose: null pointer");
+    PM_REQUIRE(edge_vi && edge_vj && edge_rank && edge_sample && sample_open && vt_replace && first_edge && attaches, "cluster_attach_propose: null pointer");
     hipStream_t st = (hipStream_t)stream;
     const dim3 ge((unsigned)ceil_div(n_edges, kBlock)), gv((unsigned)ceil_div(Nv, kBlock)), blk(kBlock);
     fill_int_k<<<gv, blk, 0, st>>>(first_edge, kNoEdge, Nv);
-    attach_propose_k<<<ge, blk, 0, st>>>(edge_vi, edge_vj, edge_sample, sample_open, n_edges, Nv, vt_replace, first_edge);
-    attach_flag_k<<<ge, blk, 0, st>>>(edge_vi, edge_vj, edge_sample, sample_open, n_edges, Nv, vt_replace, first_edge, attaches);
+    attach_propose_k<<<ge, blk, 0, st>>>(edge_vi, edge_vj, edge_rank, edge_sample, sample_open, n_edges, Nv, vt_replace, first_edge);
+    attach_flag_k<<<ge, blk, 0, st>>>(edge_vi, edge_vj, edge_rank, edge_sample, sample_open, n_edges, Nv, vt_replace, first_edge, attaches);
     PM_LAUNCHED("cluster_attach_propose");
     return 0;
 }
 
-extern "C" int pmesh_cluster_attach(const int32_t *edge_vi, const int32_t *edge_vj, const int32_t *keep, int64_t n_edges,
-                                    const int32_t *first_edge, const int32_t *pairs, int32_t *vt_replace, pmesh_stream_t stream)
+extern "C" int pmesh_cluster_attach(const int32_t *edge_vi, const int32_t *edge_vj, const int32_t *edge_rank, const int32_t *keep,
+                                    int64_t n_edges, const int32_t *first_edge, const int32_t *pairs, int32_t *vt_replace,
+                                    pmesh_stream_t stream)
 {
     clear_error();
     PM_REQUIRE(n_edges >= 0 && n_edges < kNoEdge, "cluster_attach: bad sizes");
     if (n_edges == 0) return 0;
-    PM_REQUIRE(edge_vi && edge_vj && keep && first_edge && pairs && vt_replace && pairs != vt_replace, "cluster_attach: null or aliased pointer");
-    attach_apply_k<<<dim3((unsigned)ceil_div(n_edges, kBlock)), dim3(kBlock), 0, (hipStream_t)stream>>>(edge_vi, edge_vj, keep, n_edges, first_edge, pairs, vt_replace);
+    PM_REQUIRE(edge_vi && edge_vj && edge_rank && keep && first_edge && pairs && vt_replace && pairs != vt_replace, "cluster_attach: null or aliased pointer");
+    attach_apply_k<<<dim3((unsigned)ceil_div(n_edges, kBlock)), dim3(kBlock), 0, (hipStream_t)stream>>>(edge_vi, edge_vj, edge_rank, keep, n_edges, first_edge, pairs, vt_replace);
     PM_LAUNCHED("cluster_attach");
     return 0;
 }

@@ -192,16 +192,20 @@ def cluster_vertices(edge_vi, edge_vj, sample, nvIn_cumsum, nv2Remove, Nv):
     return vt_replace
 
 
-def cluster_vertices_device(edge_vi, edge_vj, sample, nvIn_cumsum, nv2Remove, Nv, rounds_per_check=8):
+def cluster_vertices_device(edge_vi, edge_vj, perm, sample, nvIn_cumsum, nv2Remove, Nv, rounds_per_check=8):
     """The same two greedy passes on the device, for all samples at once: -> vt_replace int32 (Nv,) on the device, equal
-    to what ``cluster_vertices`` returns.  Nothing but a status word per ``rounds_per_check`` rounds of the first pass
+    to what ``cluster_vertices`` returns for ``edge_vi[perm], edge_vj[perm]``.  ``edge_vi`` / ``edge_vj``: the candidate
+    edges in ascending (vi, vj) order, ``perm`` / ``sample``: their contraction order and the sample of each edge in
+    that order (``contraction_order``).  Nothing but a status word per ``rounds_per_check`` rounds of the first pass
     crosses to the host.
 
     First pass: the serial choice "take an edge when both its ends are free" over a total order is the fixed point of
     "an edge that is the first edge with two free ends at BOTH of its ends is taken" (``pmesh_cluster_match``); the
     serial pass stops at its budget, i.e. keeps the lowest-ranked of these edges.  Second pass (only for a sample whose
     first pass left budget, i.e. ended with no edge between two free vertices): a free vertex joins the cluster behind
-    its first edge to a covered vertex -- no vertex that joins can enable another one -- again cut by rank."""
+    its first edge to a covered vertex -- no vertex that joins can enable another one -- again cut by rank.  The kernels
+    walk the edges in (vi, vj) order, where neighbouring threads touch neighbouring vertices, and carry each edge's
+    rank along."""
     dev = edge_vi.device
     E, B = edge_vi.shape[0], nvIn_cumsum.shape[0]
     st = stream_of(edge_vi)
@@ -210,15 +214,20 @@ def cluster_vertices_device(edge_vi, edge_vj, sample, nvIn_cumsum, nv2Remove, Nv
         if E == 0 or Nv == 0:
             return vt_replace
         edge_vi, edge_vj = edge_vi.contiguous(), edge_vj.contiguous()
-        sample = sample.to(I32).contiguous()
+        perm = perm.long()
+        rank = torch.empty(E, dtype=I32, device=dev)
+        rank[perm] = torch.arange(E, dtype=I32, device=dev)
+        sample = sample.to(I32).contiguous()                         # of the edges in contraction order
+        sample_e = torch.empty(E, dtype=I32, device=dev)
+        sample_e[perm] = sample
         budget = nv2Remove.to(torch.int64).clamp(min=0)
         state = torch.zeros(Nv, dtype=I32, device=dev)
         best = torch.empty(Nv, dtype=I32, device=dev)
         chosen = torch.zeros(E, dtype=I32, device=dev)
         status = torch.zeros(4, dtype=I32, device=dev)
         while True:
-            _lib.call("pmesh_cluster_match", edge_vi.data_ptr(), edge_vj.data_ptr(), E, Nv, state.data_ptr(), best.data_ptr(),
-                      chosen.data_ptr(), status.data_ptr(), rounds_per_check, st)
+            _lib.call("pmesh_cluster_match", edge_vi.data_ptr(), edge_vj.data_ptr(), rank.data_ptr(), E, Nv, state.data_ptr(),
+                      best.data_ptr(), chosen.data_ptr(), status.data_ptr(), rounds_per_check, st)
             left, bad = status[:2].tolist()
             if bad:
                 raise RuntimeError("cluster_vertices: a candidate edge is not (vi < vj) inside the vertex range")
@@ -227,25 +236,26 @@ def cluster_vertices_device(edge_vi, edge_vj, sample, nvIn_cumsum, nv2Remove, Nv
         # rank of each chosen edge among its sample's chosen edges; the budget keeps the first ones
         first = torch.searchsorted(sample, torch.arange(B + 1, device=dev, dtype=I32))
 
-        def cut(flags, allowance):
+        def cut(flags_e, allowance):
+            flags = flags_e[perm]                                     # in contraction order
             run = torch.cumsum(flags, 0)
-            before = torch.cat([run.new_zeros(1), run])[first]                 # flags counted ahead of each sample
-            rank = run - before[:-1][sample.long()]
-            return (flags > 0) & (rank <= allowance[sample.long()]), before[1:] - before[:-1]
+            before = torch.cat([run.new_zeros(1), run])[first]        # flags counted ahead of each sample
+            place = run - before[:-1][sample.long()]
+            keep = (flags > 0) & (place <= allowance[sample.long()])
+            return keep.to(I32)[rank.long()].contiguous(), before[1:] - before[:-1]
 
         keep, n_chosen = cut(chosen, budget)
-        _lib.call("pmesh_cluster_contract_pairs", edge_vi.data_ptr(), edge_vj.data_ptr(), keep.to(I32).data_ptr(), E,
-                  vt_replace.data_ptr(), st)
+        _lib.call("pmesh_cluster_contract_pairs", edge_vi.data_ptr(), edge_vj.data_ptr(), keep.data_ptr(), E, vt_replace.data_ptr(), st)
         # second pass where the first one left budget
         open_ = (n_chosen < budget).to(I32).contiguous()
         first_edge = best
         attaches = chosen
-        _lib.call("pmesh_cluster_attach_propose", edge_vi.data_ptr(), edge_vj.data_ptr(), sample.data_ptr(), open_.data_ptr(), E, Nv,
-                  vt_replace.data_ptr(), first_edge.data_ptr(), attaches.data_ptr(), st)
+        _lib.call("pmesh_cluster_attach_propose", edge_vi.data_ptr(), edge_vj.data_ptr(), rank.data_ptr(), sample_e.data_ptr(),
+                  open_.data_ptr(), E, Nv, vt_replace.data_ptr(), first_edge.data_ptr(), attaches.data_ptr(), st)
         keep2, _ = cut(attaches, budget - torch.minimum(n_chosen, budget))
         pairs = vt_replace.clone()
-        _lib.call("pmesh_cluster_attach", edge_vi.data_ptr(), edge_vj.data_ptr(), keep2.to(I32).data_ptr(), E, first_edge.data_ptr(),
-                  pairs.data_ptr(), vt_replace.data_ptr(), st)
+        _lib.call("pmesh_cluster_attach", edge_vi.data_ptr(), edge_vj.data_ptr(), rank.data_ptr(), keep2.data_ptr(), E,
+                  first_edge.data_ptr(), pairs.data_ptr(), vt_replace.data_ptr(), st)
     return vt_replace
 
 
@@ -265,7 +275,7 @@ def simplify(vertexIn, faceIn, geometryIn, nvIn_cumsum, mfIn_cumsum, nv2Remove, 
     cost = edge_costs(vertexIn, quadric, evi, evj)
     perm, sample = contraction_order(cost, evi, evj, nvIn_cumsum)
     if evi.is_cuda and os.environ.get("PMESH_DECIMATE_HOST_CLUSTERING") != "1":
-        vt_replace = cluster_vertices_device(evi[perm], evj[perm], sample, nvIn_cumsum, nv2Remove, Nv)
+        vt_replace = cluster_vertices_device(evi, evj, perm, sample, nvIn_cumsum, nv2Remove, Nv)
     else:
         vt_replace = torch.from_numpy(cluster_vertices(evi[perm], evj[perm], sample, nvIn_cumsum, nv2Remove, Nv)).to(dev)
     Nf = faceIn.shape[0]

@@ -273,11 +273,15 @@ def test_device_clustering_equals_the_serial_host_routine(cuda, seed):
         host = decimate.cluster_vertices(torch.from_numpy(vi), torch.from_numpy(vj), torch.from_numpy(sample), nv_cum,
                                          torch.from_numpy(budget), Nv)
         assert np.array_equal(host, want)
-        got = decimate.cluster_vertices_device(dev(vi, cuda), dev(vj, cuda), dev(sample, cuda), nv_cum.to(cuda), dev(budget, cuda), Nv,
-                                               rounds_per_check=1 + seed % 3)
+        # the device routine takes the edges in ascending (vi, vj) order plus their contraction order
+        by_pair = np.lexsort((vj, vi))
+        perm = np.argsort(by_pair, kind="stable")               # position of contraction-order edge k in the (vi, vj) list
+        got = decimate.cluster_vertices_device(dev(vi[by_pair], cuda), dev(vj[by_pair], cuda), dev(perm, cuda), dev(sample, cuda),
+                                               nv_cum.to(cuda), dev(budget, cuda), Nv, rounds_per_check=1 + seed % 3)
         assert np.array_equal(got.cpu().numpy(), want), "budget fraction %g: %d vertices differ" % (frac, (got.cpu().numpy() != want).sum())
     with pytest.raises(RuntimeError):
-        decimate.cluster_vertices_device(dev(vj, cuda), dev(vi, cuda), dev(sample, cuda), nv_cum.to(cuda), dev(budget, cuda), Nv)
+        decimate.cluster_vertices_device(dev(vj, cuda), dev(vi, cuda), dev(np.arange(len(vi)), cuda), dev(sample, cuda), nv_cum.to(cuda),
+                                         dev(budget, cuda), Nv)
 
 
 def test_simplify_is_the_same_with_host_clustering(cuda, monkeypatch):

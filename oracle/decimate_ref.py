@@ -138,7 +138,7 @@ def edge_costs(vertex, quadric, edge_vi, edge_vj, dtype=np.float64, return_rcond
 
 
 def edge_mix(edge_vi, edge_vj):
-    """32-bit mix of an edge's end points: what orders candidate edges of EQUAL cost.  Flat regions give thousands of
+    """24-bit mix of an edge's end points: what orders candidate edges of EQUAL cost.  Flat regions give thousands of
     edges the same (zero) cost; ordered by (vi, vj) the greedy clustering would sweep them one after the other along the
     vertex numbering, ordered by this mix their choices are local (and can be made in parallel rounds)."""
     m = 0xFFFFFFFF
@@ -149,7 +149,7 @@ def edge_mix(edge_vi, edge_vj):
     h ^= h >> 12
     h = (h * 0x297A2D39) & m
     h ^= h >> 15
-    return h
+    return h >> 8                              # 24 bits: cost, mix and a sample number below 256 share one 64-bit key
 
 
 def contraction_order(cost, edge_vi, edge_vj, nv_cumsum):

@@ -118,7 +118,7 @@ def edge_costs(vertexIn, quadric, edge_vi, edge_vj):
 
 
 def edge_mix(edge_vi, edge_vj):
-    """32-bit mix of an edge's end points (int64 tensor): the criterion between candidate edges of EQUAL cost.  The
+    """24-bit mix of an edge's end points (int64 tensor): the criterion between candidate edges of EQUAL cost.  The
     flat parts of a scene give most of its edges the same (zero) cost; in (vi, vj) order the greedy clustering would
     sweep them one after the other along the vertex numbering (thousands of dependent steps), in the order of this mix
     the choices are local and the device's rounds settle in a few dozen."""
@@ -128,22 +128,26 @@ def edge_mix(edge_vi, edge_vj):
     h = (h * 0x2C1B3C6D) & m
     h = h ^ (h >> 12)
     h = (h * 0x297A2D39) & m
-    return h ^ (h >> 15)
+    return (h ^ (h >> 15)) >> 8
 
 
 def contraction_order(cost, edge_vi, edge_vj, nvIn_cumsum):
     """Order of the candidate edges: by sample, then cost (NaN last), then ``edge_mix``, then (vi, vj) -- the edges come
     in (vi, vj) order, so three stable sorts do it.  returns (permutation, sample of each edge in that order)."""
-    # one 64-bit key per edge: the cost as an integer that orders like the float (NaN above everything, -0 = +0) in the
-    # upper half, the mix in the lower; then the samples apart by a stable sort of their (8-bit, when they fit) numbers
+    # one 64-bit key per edge: the sample number (when there are fewer than 256) on top, the cost as an integer that
+    # orders like the float (NaN above everything, -0 = +0) below it, the 24-bit mix at the bottom; the sort is stable,
+    # so equal keys stay in (vi, vj) order
     bits = (cost + 0.0).view(torch.int32).long()
     ordered = torch.where(bits >= 0, bits, -(bits + 2147483648) - 1)               # negative floats: larger magnitude, lower
     ordered = torch.where(torch.isnan(cost), torch.full_like(ordered, 2147483647), ordered)
-    by_cost = torch.sort((ordered << 32) | edge_mix(edge_vi, edge_vj), stable=True).indices
-    sample = torch.bucketize(edge_vi[by_cost].long(), nvIn_cumsum.long(), right=True)
-    narrow = torch.uint8 if nvIn_cumsum.shape[0] < 256 else torch.int64
-    by_sample = torch.sort(sample.to(narrow), stable=True)
-    return by_cost[by_sample.indices], by_sample.values.long()
+    key = ((ordered + 2147483648) << 24) | edge_mix(edge_vi, edge_vj)               # 32 + 24 bits, non-negative
+    sample = torch.bucketize(edge_vi.long(), nvIn_cumsum.long(), right=True)
+    if nvIn_cumsum.shape[0] < 128:
+        perm = torch.sort((sample << 56) | key, stable=True).indices
+        return perm, sample[perm]
+    by_cost = torch.sort(key, stable=True).indices
+    by_sample = torch.sort(sample[by_cost], stable=True)
+    return by_cost[by_sample.indices], by_sample.values
 
 
 _staging = threading.local()

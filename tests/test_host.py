@@ -359,8 +359,8 @@ def test_contraction_order_of_the_product_is_the_oracles():
     special = np.array([0.0, -0.0, 1e-45, -1e-45, 1e-30, -1e-30, -2.5, 2.5, np.nan, np.inf, -np.inf, 1.0, 1.0000001, -1.0], np.float32)
     cost = rng.choice(special, n)
     cost[::7] = rng.normal(size=len(cost[::7])).astype(np.float32)
-    cum = np.array([100, 200, 300])
-    want_perm, want_sample = R.contraction_order(cost, vi, vj, cum)
-    perm, sample = D.contraction_order(torch.from_numpy(cost), torch.from_numpy(vi), torch.from_numpy(vj), torch.from_numpy(cum))
-    assert np.array_equal(perm.numpy(), want_perm) and np.array_equal(sample.numpy(), want_sample)
+    for cum in (np.array([100, 200, 300]), np.arange(2, 302, 2)):       # few samples: one key per edge; many: two sorts
+        want_perm, want_sample = R.contraction_order(cost, vi, vj, cum)
+        perm, sample = D.contraction_order(torch.from_numpy(cost), torch.from_numpy(vi), torch.from_numpy(vj), torch.from_numpy(cum))
+        assert np.array_equal(perm.numpy(), want_perm) and np.array_equal(sample.numpy(), want_sample)
     assert np.array_equal(D.edge_mix(torch.from_numpy(vi), torch.from_numpy(vj)).numpy(), R.edge_mix(vi, vj))

@@ -168,7 +168,7 @@ def _mix_by_hand(a, b):
     h = (h * 0x2C1B3C6D) & m
     h ^= h >> 12
     h = (h * 0x297A2D39) & m
-    return h ^ (h >> 15)
+    return (h ^ (h >> 15)) >> 8
 
 
 def test_contraction_order_is_total():
@@ -186,7 +186,7 @@ def test_contraction_order_is_total():
     assert np.array_equal(sample, (vi[perm] >= 4).astype(int)) and np.all(np.diff(sample) >= 0)
     mix = [_mix_by_hand(int(a), int(b)) for a, b in zip(vi, vj)]
     assert np.array_equal(D.edge_mix(vi, vj), np.array(mix, np.int64))
-    assert len(set(mix)) > 0.95 * len(set(zip(vi.tolist(), vj.tolist())))     # it does spread the pairs
+    assert len(set(mix)) > 0.95 * len(set(zip(vi.tolist(), vj.tolist()))) and max(mix) < 2 ** 24     # it does spread the pairs
     for x, y in zip(perm[:-1].tolist(), perm[1:].tolist()):
         if (vi[x] >= 4) != (vi[y] >= 4):
             continue

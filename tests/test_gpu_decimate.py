@@ -330,3 +330,31 @@ def test_edge_list_from_the_adjacency_equals_the_sorted_edge_list(cuda, case):
     bnd = (counts == 1) & ok
     assert np.array_equal(bvi.cpu().numpy(), wi[bnd]) and np.array_equal(bvj.cpu().numpy(), wj[bnd])
     assert np.array_equal(bface.cpu().numpy(), first_face[bnd])
+
+
+def test_round_on_degenerate_batches(cuda):
+    """A sample without facets beside a regular one, a mesh whose facets are all collapsed, and a round with nothing to
+    remove: the round's outputs keep their shapes and meanings (no candidate edges -> nothing contracted)."""
+    v, f = mesh_case("octa")
+    v = np.asarray(v, np.float32)
+    lone = np.zeros((3, 3), np.float32)                                  # three vertices, no facet
+    vs = np.concatenate([v, lone])
+    nv_cum = np.array([len(v), len(vs)], np.int32)
+    mf_cum = np.array([len(f), len(f)], np.int32)
+    vx, fc = dev(vs, cuda), dev(f.astype(np.int32), cuda)
+    geo = compute_triangle_geometry_(vx, fc)
+    out = decimate.simplify(vx, fc, geo, dev(nv_cum, cuda), dev(mf_cum, cuda), dev(np.array([3, 2], np.int32), cuda), True, 5.0)
+    want = D.simplify(vs, f.astype(np.int32), geo.cpu().numpy(), nv_cum, mf_cum, np.array([3, 2], np.int32), True, 5.0, dtype=np.float32)
+    for got, ref in zip(out[1:], want[1:]):
+        assert np.array_equal(got.cpu().numpy(), ref)
+    assert not out[3][len(v):].any()                                     # nothing to contract in the facet-less sample
+    # every facet collapsed: no edges at all
+    flat = dev(np.array([[0, 0, 0], [2, 2, 2]], np.int32), cuda)
+    vx2 = dev(v[:3], cuda)
+    geo2 = compute_triangle_geometry_(vx2, flat)
+    one = torch.tensor([3], dtype=I32, device=cuda)
+    out2 = decimate.simplify(vx2, flat, geo2, one, torch.tensor([2], dtype=I32, device=cuda), torch.tensor([2], dtype=I32, device=cuda))
+    assert not out2[3].any() and bool(out2[2].all()) and out2[5].tolist() == [0] and out2[6].tolist() == [0]
+    res = decimate.mesh_decimation_(vx2, flat, geo2, one, torch.tensor([2], dtype=I32, device=cuda), torch.tensor([1], dtype=I32, device=cuda))
+    # vertices left without a live facet leave the mesh (as in the reference); the loop ends, sizes agree
+    assert res[0].shape[0] == int(res[3].sum()) == 0 and res[1].shape[0] == int(res[4].sum()) == 0

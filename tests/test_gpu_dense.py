@@ -331,3 +331,22 @@ def test_v2f_module_takes_the_one_pass_form(cuda):
         _lib.set_call_hook(None)
     assert [c for c in one if c != "pmesh_sph_harm"] == ["pmesh_v2f_dense_fwd"], one      # (the corner basis, first call only)
     assert "pmesh_v2f_fwd" in two and "pmesh_dense_fwd" in two, two
+
+
+def test_v2f_dense_empty_and_refused_shapes(cuda):
+    """No facets: an empty result, nothing launched on bad memory; a channel count that is not a multiple of 4 and a face
+    index outside the vertex range raise like the ops they replace."""
+    x = torch.randn(10, 8, device=cuda)
+    filt = torch.randn(3, 8, 1, device=cuda)
+    w = torch.randn(8, 5, device=cuda)
+    none = torch.zeros((0, 3), dtype=torch.int32, device=cuda)
+    out, bits, rows = dense.v2f_dense_forward(x, filt, none, w, None, True, with_bits=True, keep_rows=True)
+    assert out.shape == (0, 5) and bits.shape == (0, 1) and rows.shape == (0, 8)
+    face = torch.tensor([[0, 1, 2], [3, 9, 4]], dtype=torch.int32, device=cuda)
+    assert dense.v2f_dense_forward(x, filt, face, w).shape == (2, 5)
+    with pytest.raises(RuntimeError):
+        dense.v2f_dense_forward(x[:, :6].contiguous(), filt[:, :6].contiguous(), face, w[:6].contiguous())
+    with pytest.raises(RuntimeError):
+        dense.v2f_dense_forward(x, filt, torch.tensor([[0, 1, 10]], dtype=torch.int32, device=cuda), w)
+    with pytest.raises(RuntimeError):
+        dense.v2f_dense_forward(x.cpu(), filt, face, w)

@@ -121,7 +121,7 @@ TRAFFIC_KERNELS = {
              "dense_bwd": [r"dense_rows_k<\d+, \d+, (true|false), [12], ", r"dense_wgrad_k", r"reduce_partials_k"]},
     "texture": {"texture_fwd": [r"texture_fwd_k"], "texture_bwd": [r"texture_bwd_flat_k", r"texture_bwd_k"]},
     "pcloud": {"point_conv_fwd": [r"point_conv_rows_dense_k<\d+, 0>", r"point_conv_fwd_k"],
-               "point_conv_bwd": [r"point_conv_rows_dense_k<\d+, 1>", r"point_conv_bwd_in_k", r"point_conv_bwd_filt", r"reduce_partials_k"]},
+               "point_conv_bwd": [r"point_conv_bwd_fused_k", r"point_conv_rows_dense_k<\d+, 1>", r"point_conv_bwd_in_k", r"point_conv_bwd_filt", r"reduce_partials_k"]},
 }
 
 

@@ -15,6 +15,7 @@
 //   gin[i, c]       = sum_{p = (o, i)} (1 / nn_count[o]) sum_m gout[o, c r + m] * w[p, c r + m]
 //   gfilt[f, co]    = sum_p sum_t [bin[p, t] = f] coeff[p, t] * gout[o, co] * in[i, co / r] / nn_count[o]
 #include "common.h"
+#include <stdlib.h>
 #include "rows_internal.h"
 #include "../../include/picasso_mesh.h"
 
@@ -227,6 +228,136 @@ __global__ __launch_bounds__(kBlock) void point_conv_rows_dense_k(const float *_
         const float inv = MODE == 0 ? inv_count(g.nn_count, row) : 1.f;
         *reinterpret_cast<float4 *>(out + row * C + c) = make_float4(acc[0] * inv, acc[1] * inv, acc[2] * inv, acc[3] * inv);
     }
+}
+
+// Input gradient AND filter gradient from one walk over the pairs (at most FB <= 20 bins, depth multiplier 1, rows of at
+// most 128 channels): gin[i][c] = sum over the pairs of point i of gout[o][c] * w(p)[c] / count[o] with
+// w(p)[c] = sum_f cm[p][f] * filt[f][c], and gfilt[f][c] += cm[p][f] * (gout[o][c] * in[i][c] / count[o]).  A lane keeps
+// two channels of the filter and of the filter gradient in registers, a wave the rows of 64 / lanes-per-row database
+// points; it builds the dense table cm of its own pairs, 64 at a time, in its own piece of LDS and meets no other wave
+// until the end.  Waves are persistent over the row groups (their number is a function of the problem only); at the
+// end the lanes that hold the same channels add their accumulators in a fixed order: partial[workgroup][F][C].
+template <int FB>
+__global__ __launch_bounds__(kBlock, 3) void point_conv_bwd_fused_k(const float *__restrict__ gout, const float *__restrict__ in,
+                                                                    const float *__restrict__ filt, PairGraph g,
+                                                                    const int *__restrict__ rowptr, const int *__restrict__ order,
+                                                                    float *__restrict__ gin, float *__restrict__ partial, int C,
+                                                                    int lpr_log2)
+{
+    constexpr int NW = kBlock / 64;
+    __shared__ __attribute__((aligned(16))) float s_cm[NW][64][FB];
+    __shared__ int s_other[NW][64];
+    __shared__ float s_scale[NW][64];
+    static_assert(NW * 64 >= 128, "the table doubles as the buffer of the final sum (FB x 128 floats)");
+    const int wave = threadIdx.x >> 6, wl = threadIdx.x & 63;
+    const int lpr = 1 << lpr_log2, lane = wl & (lpr - 1), slot = wl >> lpr_log2, rpw = 64 >> lpr_log2;
+    const int64_t rows = g.Np, nother = g.Mp;
+    const bool chan = 2 * lane < C;
+    const int c = 2 * lane;
+    float fr[FB][2], ga[FB][2];
+#pragma unroll
+    for (int f = 0; f < FB; ++f) {
+        const float2 v = (chan && f < g.F) ? *reinterpret_cast<const float2 *>(filt + (int64_t)f * C + c) : make_float2(0.f, 0.f);
+        fr[f][0] = v.x; fr[f][1] = v.y;
+        ga[f][0] = ga[f][1] = 0.f;
+    }
+    float(*cm)[FB] = s_cm[wave];
+    int *other_of = s_other[wave];
+    float *scale_of = s_scale[wave];
+    const int64_t groups = (rows + rpw - 1) / rpw;
+    for (int64_t wb = (int64_t)blockIdx.x * NW + wave; wb < groups; wb += (int64_t)gridDim.x * NW) {
+        const int64_t row0 = wb * rpw, row = row0 + slot;
+        const int64_t rowl = row0 + rpw < rows ? row0 + rpw : rows;
+        const int eb = rowptr[row0], ee = rowptr[rowl];             // the wave's pairs, in row order
+        const bool live = row < rows && chan;
+        const int e0 = row < rows ? rowptr[row] : 0, e1 = row < rows ? rowptr[row + 1] : 0;
+        const float2 xin = live ? *reinterpret_cast<const float2 *>(in + row * C + c) : make_float2(0.f, 0.f);
+        float acc[2] = {0.f, 0.f};
+        for (int cb = eb; cb < ee; cb += 64) {
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");  // the table's readers of the chunk before are done
+            __builtin_amdgcn_wave_barrier();
+            {
+                int o = -1;
+                float sc = 1.f;
+                int64_t p = 0;
+                if (cb + wl < ee) {
+                    p = order[cb + wl];
+                    const int oo = g.nn_index[p * 2], i = g.nn_index[p * 2 + 1];
+                    if (oo >= 0 && oo < nother && i >= 0 && i < rows) o = oo;
+                }
+                if (o >= 0) sc = inv_count(g.nn_count, o);
+                other_of[wl] = o;
+                scale_of[wl] = sc;
+#pragma unroll
+                for (int f4 = 0; f4 < FB; f4 += 4) *reinterpret_cast<float4 *>(&cm[wl][f4]) = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (o >= 0) pair_row_to_table(g, p, cm[wl]);
+            }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            if (!live) continue;
+            const int a = e0 > cb ? e0 : cb, b = e1 < cb + 64 ? e1 : cb + 64;
+            for (int e4 = a; e4 < b; e4 += 4) {
+                float2 x[4];
+                bool ok[4];
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    const int other = e4 + k < b ? other_of[e4 + k - cb] : -1;
+                    ok[k] = other >= 0;
+                    x[k] = make_float2(0.f, 0.f);
+                    if (ok[k]) x[k] = *reinterpret_cast<const float2 *>(gout + (int64_t)other * C + c);
+                }
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    if (!ok[k]) continue;
+                    const int q = e4 + k - cb;
+                    const float sc = scale_of[q];
+                    const float du[2] = {x[k].x * xin.x * sc, x[k].y * xin.y * sc};
+                    float w[2] = {0.f, 0.f};
+#pragma unroll
+                    for (int f4 = 0; f4 < FB; f4 += 4) {
+                        const float4 m = *reinterpret_cast<const float4 *>(&cm[q][f4]);
+#pragma unroll
+                        for (int u = 0; u < 2; ++u) {
+                            w[u] = fmaf(m.x, fr[f4][u], w[u]);
+                            w[u] = fmaf(m.y, fr[f4 + 1][u], w[u]);
+                            w[u] = fmaf(m.z, fr[f4 + 2][u], w[u]);
+                            w[u] = fmaf(m.w, fr[f4 + 3][u], w[u]);
+                            ga[f4][u] = fmaf(m.x, du[u], ga[f4][u]);
+                            ga[f4 + 1][u] = fmaf(m.y, du[u], ga[f4 + 1][u]);
+                            ga[f4 + 2][u] = fmaf(m.z, du[u], ga[f4 + 2][u]);
+                            ga[f4 + 3][u] = fmaf(m.w, du[u], ga[f4 + 3][u]);
+                        }
+                    }
+                    acc[0] = fmaf(x[k].x * w[0], sc, acc[0]);
+                    acc[1] = fmaf(x[k].y * w[1], sc, acc[1]);
+                }
+            }
+        }
+        if (live) *reinterpret_cast<float2 *>(gin + row * C + c) = make_float2(acc[0], acc[1]);
+    }
+    // the row slots of a wave add up across its lanes, then the waves one after the other through LDS, wave 0 first
+    for (int off = lpr; off < 64; off <<= 1) {
+#pragma unroll
+        for (int f = 0; f < FB; ++f) {
+            ga[f][0] += __shfl_xor(ga[f][0], off, 64);
+            ga[f][1] += __shfl_xor(ga[f][1], off, 64);
+        }
+    }
+    float *red = &s_cm[0][0][0];                                  // FB x C floats
+    for (int w = 0; w < NW; ++w) {
+        __syncthreads();
+        if (wave == w && wl < lpr && chan) {
+#pragma unroll
+            for (int f = 0; f < FB; ++f) {
+                float2 *d = reinterpret_cast<float2 *>(red + f * C + c);
+                *d = w ? make_float2(d->x + ga[f][0], d->y + ga[f][1]) : make_float2(ga[f][0], ga[f][1]);
+            }
+        }
+    }
+    __syncthreads();
+    float *dst = partial + (int64_t)blockIdx.x * g.F * C;
+    for (int e = threadIdx.x; e < g.F * C; e += kBlock) dst[e] = red[e];
 }
 
 // filter gradient: workgroup (x, y) sums pairs [x * per, (x + 1) * per) for columns y * cols .. into LDS, one column per
@@ -532,6 +663,21 @@ extern "C" int pmesh_point_conv_bwd(const float *grad_output, const float *input
     }
     PM_REQUIRE(grad_output && input && filter && nn_count && nn_index && bin_index && workspace, "point_conv_bwd: null pointer");
     const PairGraph g = {nn_index, nn_count, bin_index, bin_coeff, Np, Mp, Nout, T, F};
+    if (grad_input && r == 1 && C % 4 == 0 && C <= 128 && F <= 20 && aligned16(grad_output) && aligned16(filter) && aligned16(grad_input) &&
+        aligned16(input) && !getenv("PMESH_POINT_CONV_TWO_PASSES")) {
+        // both gradients from one walk over the pairs in database-point order
+        PM_REQUIRE(rowptr_in && order_in, "point_conv_bwd: the input gradient needs the pairs sorted by database point");
+        const RowShape rs = row_shape(C / 2);                        // two channels per lane: at most 64 lanes per row
+        const int64_t groups = ceil_div(Np, (int64_t)(64 >> rs.lpr_log2)), wgs = ceil_div(groups, (int64_t)(kBlock / 64));
+        int G = filt_blocks(Nout, F, CR);                            // as many workgroups as the chip holds at once
+        if (G > 768) G = 768;
+        if (G > wgs) G = (int)(wgs > 0 ? wgs : 1);
+        PM_REQUIRE(workspace_bytes >= (size_t)G * F * CR * sizeof(float), "point_conv_bwd: workspace too small (%zu bytes)", workspace_bytes);
+        if (F <= 16) point_conv_bwd_fused_k<16><<<dim3((unsigned)G), dim3(kBlock), 0, st>>>(grad_output, input, filter, g, rowptr_in, order_in, grad_input, (float *)workspace, C, rs.lpr_log2);
+        else point_conv_bwd_fused_k<20><<<dim3((unsigned)G), dim3(kBlock), 0, st>>>(grad_output, input, filter, g, rowptr_in, order_in, grad_input, (float *)workspace, C, rs.lpr_log2);
+        PM_LAUNCHED("point_conv_bwd(fused)");
+        return reduce_partials((const float *)workspace, grad_filter, G, F * CR, st);
+    }
     if (grad_input) {
         PM_REQUIRE(rowptr_in && order_in, "point_conv_bwd: the input gradient needs the pairs sorted by database point");
         if (r == 1 && C % 4 == 0 && C <= 256 && F <= 36 && aligned16(grad_output) && aligned16(filter) && aligned16(grad_input)) {

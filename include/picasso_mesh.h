@@ -352,6 +352,12 @@ int pmesh_boundary_quadrics(const float *vertex, const float *geometry, const in
                             float wgt_bnd, pmesh_stream_t stream);
 int pmesh_edge_costs(const float *vertex, const float *quadric, const int32_t *edge_vi, const int32_t *edge_vj,
                      float *cost, int64_t n_edges, int vertex_stride, pmesh_stream_t stream);
+/* Sort keys of the contraction order (the reference sorts (sample, cost) with thrust, decimate_gpu.cu:662-686; ties
+ * are broken here by a 24-bit mix of the end points, then by (vi, vj) through a stable sort): keys[e] =
+ * sample(vi) << 56 | cost as order-preserving 32-bit integer << 24 | mix(vi, vj), for B < 128 samples with the running
+ * totals nv_cumsum of their vertex counts. */
+int pmesh_contraction_keys(const float *cost, const int32_t *edge_vi, const int32_t *edge_vj, const int32_t *nv_cumsum,
+                           int64_t n_edges, int B, int64_t *keys, pmesh_stream_t stream);
 int pmesh_cluster_vertices_host(const int32_t *edge_vi, const int32_t *edge_vj, int64_t n_edges, int32_t vt_start,
                                 int32_t vt_num, int32_t n_remove, int32_t *vt_replace);
 
@@ -368,7 +374,7 @@ int pmesh_simplify_renumber(const int32_t *new_face, const uint8_t *degenerate, 
                             pmesh_stream_t stream);
 
 /* The same two passes (clusterVertices, decimate_gpu.cu:561-614) for the whole batch on the DEVICE, in four steps
- * between which the caller cuts the chosen edges by their rank within the sample (two prefix sums): the result is
+ * between which the chosen edges are cut by their rank within the sample (a running total of the caller's + pmesh_cluster_cut): the result is
  * that of pmesh_cluster_vertices_host sample by sample.  edge_vi / edge_vj: the candidate edges of all samples in
  * ascending (vi, vj) order (vi < vj, every edge inside one sample; neighbouring threads then touch neighbouring
  * vertices), edge_rank: each edge's position in the contraction order (distinct integers, ascending within a sample
@@ -378,6 +384,14 @@ int pmesh_simplify_renumber(const int32_t *new_face, const uint8_t *degenerate, 
  *                                 (n_edges) are zero before the first call and carry over; best (Nv) is scratch.
  *                                 status[0] <- 1 while an edge with two free ends is left (call again), status[1]
  *                                 <- 1 if an edge is not (0 <= vi < vj < Nv) -- such an edge is left out.
+ *   pmesh_cluster_ranks           edge_rank / edge_sample from the contraction order: order (n_edges) lists the edges
+ *                                 in the order of contraction, order_sample their samples in that order.
+ *   pmesh_cluster_flags_by_rank   by_rank[edge_rank[e]] = (flags[e] != 0): the chosen edges in contraction order, for
+ *                                 the caller's running total `run` (inclusive, int32).
+ *   pmesh_cluster_cut             keep[e] = flags[e] and the edge is among the first allowance[sample] flagged edges of
+ *                                 its sample; first (B + 1): where each sample's edges begin in the contraction order.
+ *                                 With sample_open / left (B, together or both null): whether the sample's flagged
+ *                                 edges stayed below its allowance, and the allowance they leave.
  *   pmesh_cluster_contract_pairs  vt_replace[vi] = -vj, vt_replace[vj] = 1 for the edges with keep != 0 (the chosen
  *                                 edges whose rank among the sample's chosen edges is within its budget).
  *   pmesh_cluster_attach_propose  second pass, for the samples with sample_open != 0 (budget not exhausted by the
@@ -388,6 +402,12 @@ int pmesh_simplify_renumber(const int32_t *new_face, const uint8_t *degenerate, 
  *                                 cluster; pairs = a copy of vt_replace as the first pass left it. */
 int pmesh_cluster_match(const int32_t *edge_vi, const int32_t *edge_vj, const int32_t *edge_rank, int64_t n_edges, int64_t Nv,
                         int32_t *state, int32_t *best, int32_t *chosen, int32_t *status, int rounds, pmesh_stream_t stream);
+int pmesh_cluster_ranks(const int64_t *order, const int32_t *order_sample, int64_t n_edges, int32_t *edge_rank, int32_t *edge_sample,
+                        pmesh_stream_t stream);
+int pmesh_cluster_flags_by_rank(const int32_t *flags, const int32_t *edge_rank, int64_t n_edges, int32_t *by_rank, pmesh_stream_t stream);
+int pmesh_cluster_cut(const int32_t *flags, const int32_t *edge_rank, const int32_t *edge_sample, const int32_t *run,
+                      const int64_t *first, const int32_t *allowance, int64_t n_edges, int B, int32_t *keep, int32_t *sample_open,
+                      int32_t *left, pmesh_stream_t stream);
 int pmesh_cluster_contract_pairs(const int32_t *edge_vi, const int32_t *edge_vj, const int32_t *keep, int64_t n_edges,
                                  int32_t *vt_replace, pmesh_stream_t stream);
 int pmesh_cluster_attach_propose(const int32_t *edge_vi, const int32_t *edge_vj, const int32_t *edge_rank,

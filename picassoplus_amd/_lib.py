@@ -11,7 +11,7 @@ from ctypes import c_char_p, c_float, c_int, c_int64, c_size_t, c_void_p
 _HERE = os.path.dirname(os.path.abspath(__file__))
 # PICASSO_MESH_LIB points at an alternative build of the same ABI (kernel experiments)
 LIB_PATH = os.environ.get("PICASSO_MESH_LIB") or os.path.join(_HERE, "csrc", "libpicasso_mesh.so")
-ABI_VERSION = 18
+ABI_VERSION = 19
 
 P, I, L, Z = c_void_p, c_int, c_int64, c_size_t
 
@@ -96,6 +96,10 @@ SIGNATURES = {
     "pmesh_simplify_faces": (I, [P, P, L, L, P, P, P, P, P]),
     "pmesh_simplify_renumber": (I, [P, P, P, P, L, L, P, P, P]),
     "pmesh_cluster_match": (I, [P, P, P, L, L, P, P, P, P, I, P]),
+    "pmesh_contraction_keys": (I, [P, P, P, P, L, I, P, P]),
+    "pmesh_cluster_ranks": (I, [P, P, L, P, P, P]),
+    "pmesh_cluster_flags_by_rank": (I, [P, P, L, P, P]),
+    "pmesh_cluster_cut": (I, [P, P, P, P, P, P, L, I, P, P, P, P]),
     "pmesh_cluster_contract_pairs": (I, [P, P, P, L, P, P]),
     "pmesh_cluster_attach_propose": (I, [P, P, P, P, P, L, L, P, P, P, P]),
     "pmesh_cluster_attach": (I, [P, P, P, P, L, P, P, P, P]),

@@ -354,6 +354,91 @@ __global__ __launch_bounds__(kBlock) void contract_pairs_k(const int *__restrict
     vt_replace[evj[r]] = 1;
 }
 
+// One 64-bit sort key per candidate edge: the sample of vi (number of running totals <= vi, fewer than 128 samples) in
+// the top byte, below it the cost as an integer that orders like the float (-0 = +0, NaN above everything), the 24-bit
+// mix of the end points at the bottom.
+__global__ __launch_bounds__(kBlock) void contraction_keys_k(const float *__restrict__ cost, const int *__restrict__ evi,
+                                                             const int *__restrict__ evj, const int *__restrict__ nv_cumsum, int B,
+                                                             int64_t E, int64_t *__restrict__ keys)
+{
+    __shared__ int s_end[128];
+    if (threadIdx.x < 128) s_end[threadIdx.x] = (int)threadIdx.x < B ? nv_cumsum[threadIdx.x] : INT32_MAX;
+    __syncthreads();
+    const int64_t e = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (e >= E) return;
+    const int a = evi[e], b = evj[e];
+    const float c = cost[e] + 0.0f;
+    const int64_t bits = __float_as_int(c);
+    int64_t ordered = bits >= 0 ? bits : -(bits + 2147483648LL) - 1;     // negative floats: larger magnitude, lower
+    if (c != c) ordered = 2147483647;
+    uint32_t h = (uint32_t)a * 0x9E3779B1u + (uint32_t)b * 0x85EBCA77u;
+    h ^= h >> 15;
+    h *= 0x2C1B3C6Du;
+    h ^= h >> 12;
+    h *= 0x297A2D39u;
+    h ^= h >> 15;
+    int lo = 0, hi = B;                                                  // first running total above vi
+    while (lo < hi) {
+        const int mid = (lo + hi) >> 1;
+        if (s_end[mid] <= a) lo = mid + 1;
+        else hi = mid;
+    }
+    keys[e] = ((int64_t)lo << 56) | ((ordered + 2147483648LL) << 24) | (int64_t)(h >> 8);
+}
+
+// the contraction order turned round: rank[perm[i]] = i, edge_sample[perm[i]] = sample[i]
+__global__ __launch_bounds__(kBlock) void cluster_ranks_k(const int64_t *__restrict__ perm, const int *__restrict__ sample, int64_t E,
+                                                          int *__restrict__ rank, int *__restrict__ edge_sample)
+{
+    const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= E) return;
+    const int64_t e = perm[i];
+    if (e < 0 || e >= E) return;
+    rank[e] = (int)i;
+    edge_sample[e] = sample[i];
+}
+
+__global__ __launch_bounds__(kBlock) void cluster_flags_by_rank_k(const int *__restrict__ flags, const int *__restrict__ rank, int64_t E,
+                                                                  int *__restrict__ by_rank)
+{
+    const int64_t e = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (e >= E) return;
+    const int r = rank[e];
+    if (r >= 0 && r < E) by_rank[r] = flags[e] != 0;
+}
+
+// flagged edges ahead of sample b in the contraction order (run: inclusive running total of the flags in that order)
+__device__ __forceinline__ int flagged_before(const int *__restrict__ run, const int64_t *__restrict__ first, int b)
+{
+    const int64_t at = first[b];
+    return at > 0 ? run[at - 1] : 0;
+}
+
+// keeps a flagged edge when it is among the first allowance[sample] flagged edges of its sample
+__global__ __launch_bounds__(kBlock) void cluster_cut_k(const int *__restrict__ flags, const int *__restrict__ rank,
+                                                        const int *__restrict__ edge_sample, const int *__restrict__ run,
+                                                        const int64_t *__restrict__ first, const int *__restrict__ allowance, int64_t E,
+                                                        int B, int *__restrict__ keep)
+{
+    const int64_t e = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (e >= E) return;
+    int k = 0;
+    const int b = edge_sample[e], r = rank[e];
+    if (flags[e] && b >= 0 && b < B && r >= 0 && r < E) k = run[r] - flagged_before(run, first, b) <= allowance[b];
+    keep[e] = k;
+}
+
+__global__ __launch_bounds__(kBlock) void cluster_budget_k(const int *__restrict__ run, const int64_t *__restrict__ first,
+                                                           const int *__restrict__ allowance, int B, int *__restrict__ open,
+                                                           int *__restrict__ left)
+{
+    const int b = blockIdx.x * kBlock + threadIdx.x;
+    if (b >= B) return;
+    const int taken = flagged_before(run, first, b + 1) - flagged_before(run, first, b), a = allowance[b];
+    open[b] = taken < a;
+    left[b] = a - (taken < a ? taken : a);
+}
+
 // the covered and the free end of an edge with exactly one covered end, and the covered end's representative
 __device__ __forceinline__ bool attach_ends(int a, int b, const int *__restrict__ vt_replace, int &rep, int &fr)
 {
@@ -566,6 +651,46 @@ extern "C" int pmesh_cluster_contract_pairs(const int32_t *edge_vi, const int32_
     return 0;
 }
 
+extern "C" int pmesh_cluster_ranks(const int64_t *order, const int32_t *order_sample, int64_t n_edges, int32_t *edge_rank,
+                                   int32_t *edge_sample, pmesh_stream_t stream)
+{
+    clear_error();
+    PM_REQUIRE(n_edges >= 0 && n_edges < kNoEdge, "cluster_ranks: bad sizes");
+    if (n_edges == 0) return 0;
+    PM_REQUIRE(order && order_sample && edge_rank && edge_sample, "cluster_ranks: null pointer");
+    cluster_ranks_k<<<dim3((unsigned)ceil_div(n_edges, kBlock)), dim3(kBlock), 0, (hipStream_t)stream>>>(order, order_sample, n_edges, edge_rank, edge_sample);
+    PM_LAUNCHED("cluster_ranks");
+    return 0;
+}
+
+extern "C" int pmesh_cluster_flags_by_rank(const int32_t *flags, const int32_t *edge_rank, int64_t n_edges, int32_t *by_rank,
+                                           pmesh_stream_t stream)
+{
+    clear_error();
+    PM_REQUIRE(n_edges >= 0 && n_edges < kNoEdge, "cluster_flags_by_rank: bad sizes");
+    if (n_edges == 0) return 0;
+    PM_REQUIRE(flags && edge_rank && by_rank, "cluster_flags_by_rank: null pointer");
+    cluster_flags_by_rank_k<<<dim3((unsigned)ceil_div(n_edges, kBlock)), dim3(kBlock), 0, (hipStream_t)stream>>>(flags, edge_rank, n_edges, by_rank);
+    PM_LAUNCHED("cluster_flags_by_rank");
+    return 0;
+}
+
+extern "C" int pmesh_cluster_cut(const int32_t *flags, const int32_t *edge_rank, const int32_t *edge_sample, const int32_t *run,
+                                 const int64_t *first, const int32_t *allowance, int64_t n_edges, int B, int32_t *keep,
+                                 int32_t *sample_open, int32_t *left, pmesh_stream_t stream)
+{
+    clear_error();
+    PM_REQUIRE(n_edges >= 0 && n_edges < kNoEdge && B >= 0, "cluster_cut: bad sizes");
+    if (n_edges == 0 || B == 0) return 0;
+    PM_REQUIRE(flags && edge_rank && edge_sample && run && first && allowance && keep, "cluster_cut: null pointer");
+    PM_REQUIRE((sample_open == nullptr) == (left == nullptr), "cluster_cut: sample_open and left come together");
+    hipStream_t st = (hipStream_t)stream;
+    cluster_cut_k<<<dim3((unsigned)ceil_div(n_edges, kBlock)), dim3(kBlock), 0, st>>>(flags, edge_rank, edge_sample, run, first, allowance, n_edges, B, keep);
+    if (sample_open) cluster_budget_k<<<dim3((unsigned)ceil_div(B, kBlock)), dim3(kBlock), 0, st>>>(run, first, allowance, B, sample_open, left);
+    PM_LAUNCHED("cluster_cut");
+    return 0;
+}
+
 extern "C" int pmesh_cluster_attach_propose(const int32_t *edge_vi, const int32_t *edge_vj, const int32_t *edge_rank,
                                             const int32_t *edge_sample, const int32_t *sample_open, int64_t n_edges, int64_t Nv,
                                             const int32_t *vt_replace, int32_t *first_edge, int32_t *attaches,
@@ -633,6 +758,19 @@ extern "C" int pmesh_edge_costs(const float *vertex, const float *quadric, const
     edge_cost_k<<<dim3((unsigned)ceil_div(n_edges, kBlock)), dim3(kBlock), 0, (hipStream_t)stream>>>(vertex, quadric, edge_vi, edge_vj, cost,
                                                                                                    n_edges, vertex_stride);
     PM_LAUNCHED("edge_costs");
+    return 0;
+}
+
+extern "C" int pmesh_contraction_keys(const float *cost, const int32_t *edge_vi, const int32_t *edge_vj, const int32_t *nv_cumsum,
+                                      int64_t n_edges, int B, int64_t *keys, pmesh_stream_t stream)
+{
+    clear_error();
+    PM_REQUIRE(n_edges >= 0 && n_edges <= INT32_MAX && B >= 0 && B < 128, "contraction_keys: bad sizes (at most 127 samples)");
+    if (n_edges == 0) return 0;
+    PM_REQUIRE(cost && edge_vi && edge_vj && keys && (nv_cumsum || B == 0), "contraction_keys: null pointer");
+    contraction_keys_k<<<dim3((unsigned)ceil_div(n_edges, kBlock)), dim3(kBlock), 0, (hipStream_t)stream>>>(cost, edge_vi, edge_vj, nv_cumsum, B,
+                                                                                                         n_edges, keys);
+    PM_LAUNCHED("contraction_keys");
     return 0;
 }
 

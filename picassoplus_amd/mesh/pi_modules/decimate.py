@@ -56,11 +56,9 @@ def vertex_quadrics(vertexIn, faceIn, geometryIn, useArea=True, wgtBnd=5.0):
             _lib.call("pmesh_boundary_quadrics", vertexIn.data_ptr(), geometryIn.data_ptr(), bvi.data_ptr(), bvj.data_ptr(),
                       bface.data_ptr(), rows.data_ptr(), nb, D, 1 if useArea else 0, float(wgtBnd), st)
             # every row goes to both end points: a segmented sum over the end points in ascending edge order
-            ends = torch.cat([bvi, bvj]).long()
-            _, members = torch.sort(ends, stable=True)
-            ptr = torch.zeros(Nv + 1, dtype=torch.int64, device=dev)
-            ptr[1:] = torch.cumsum(torch.bincount(ends, minlength=Nv), 0)
-            quadric = quadric + _segment_row_sum(torch.cat([rows, rows]), ptr.to(I32), members.to(I32), Nv)
+            by_end = torch.sort(torch.cat([bvi, bvj]), stable=True)
+            ptr = torch.searchsorted(by_end.values, torch.arange(Nv + 1, dtype=I32, device=dev), out_int32=True)
+            quadric = quadric + _segment_row_sum(torch.cat([rows, rows]), ptr, by_end.indices.to(I32), Nv)
     return quadric, evi, evj
 
 
@@ -137,6 +135,16 @@ def contraction_order(cost, edge_vi, edge_vj, nvIn_cumsum):
     # one 64-bit key per edge: the sample number (when there are fewer than 256) on top, the cost as an integer that
     # orders like the float (NaN above everything, -0 = +0) below it, the 24-bit mix at the bottom; the sort is stable,
     # so equal keys stay in (vi, vj) order
+    if cost.is_cuda and nvIn_cumsum.shape[0] < 128:
+        # the keys in one native pass, the sample read back off the sorted keys
+        E = cost.shape[0]
+        with torch.cuda.device(cost.device):
+            keys = torch.empty(E, dtype=torch.int64, device=cost.device)
+            _lib.call("pmesh_contraction_keys", cost.contiguous().data_ptr(), edge_vi.contiguous().data_ptr(),
+                      edge_vj.contiguous().data_ptr(), nvIn_cumsum.contiguous().data_ptr(), E, nvIn_cumsum.shape[0],
+                      keys.data_ptr(), stream_of(cost))
+            by_key = torch.sort(keys, stable=True)
+        return by_key.indices, by_key.values >> 56
     bits = (cost + 0.0).view(torch.int32).long()
     ordered = torch.where(bits >= 0, bits, -(bits + 2147483648) - 1)               # negative floats: larger magnitude, lower
     ordered = torch.where(torch.isnan(cost), torch.full_like(ordered, 2147483647), ordered)
@@ -218,13 +226,12 @@ def cluster_vertices_device(edge_vi, edge_vj, perm, sample, nvIn_cumsum, nv2Remo
         if E == 0 or Nv == 0:
             return vt_replace
         edge_vi, edge_vj = edge_vi.contiguous(), edge_vj.contiguous()
-        perm = perm.long()
-        rank = torch.empty(E, dtype=I32, device=dev)
-        rank[perm] = torch.arange(E, dtype=I32, device=dev)
+        perm = perm.long().contiguous()
         sample = sample.to(I32).contiguous()                         # of the edges in contraction order
+        rank = torch.empty(E, dtype=I32, device=dev)
         sample_e = torch.empty(E, dtype=I32, device=dev)
-        sample_e[perm] = sample
-        budget = nv2Remove.to(torch.int64).clamp(min=0)
+        _lib.call("pmesh_cluster_ranks", perm.data_ptr(), sample.data_ptr(), E, rank.data_ptr(), sample_e.data_ptr(), st)
+        budget = nv2Remove.to(I32).clamp(min=0).contiguous()
         state = torch.zeros(Nv, dtype=I32, device=dev)
         best = torch.empty(Nv, dtype=I32, device=dev)
         chosen = torch.zeros(E, dtype=I32, device=dev)
@@ -237,26 +244,30 @@ def cluster_vertices_device(edge_vi, edge_vj, perm, sample, nvIn_cumsum, nv2Remo
                 raise RuntimeError("cluster_vertices: a candidate edge is not (vi < vj) inside the vertex range")
             if not left:
                 break
-        # rank of each chosen edge among its sample's chosen edges; the budget keeps the first ones
-        first = torch.searchsorted(sample, torch.arange(B + 1, device=dev, dtype=I32))
+        # where each sample's edges begin in the contraction order
+        first = torch.searchsorted(sample, torch.arange(B + 1, device=dev, dtype=I32)).contiguous()
+        by_rank = torch.empty(E, dtype=I32, device=dev)
 
-        def cut(flags_e, allowance):
-            flags = flags_e[perm]                                     # in contraction order
-            run = torch.cumsum(flags, 0)
-            before = torch.cat([run.new_zeros(1), run])[first]        # flags counted ahead of each sample
-            place = run - before[:-1][sample.long()]
-            keep = (flags > 0) & (place <= allowance[sample.long()])
-            return keep.to(I32)[rank.long()].contiguous(), before[1:] - before[:-1]
+        def cut(flags_e, allowance, with_rest):
+            # the flagged edges whose place among their sample's flagged edges (contraction order) is within its allowance
+            _lib.call("pmesh_cluster_flags_by_rank", flags_e.data_ptr(), rank.data_ptr(), E, by_rank.data_ptr(), st)
+            run = torch.cumsum(by_rank, 0, dtype=I32)
+            keep = torch.empty(E, dtype=I32, device=dev)
+            open_ = torch.empty(B, dtype=I32, device=dev) if with_rest else None
+            rest = torch.empty(B, dtype=I32, device=dev) if with_rest else None
+            _lib.call("pmesh_cluster_cut", flags_e.data_ptr(), rank.data_ptr(), sample_e.data_ptr(), run.data_ptr(), first.data_ptr(),
+                      allowance.data_ptr(), E, B, keep.data_ptr(), open_.data_ptr() if with_rest else 0,
+                      rest.data_ptr() if with_rest else 0, st)
+            return keep, open_, rest
 
-        keep, n_chosen = cut(chosen, budget)
+        keep, open_, rest = cut(chosen, budget, True)
         _lib.call("pmesh_cluster_contract_pairs", edge_vi.data_ptr(), edge_vj.data_ptr(), keep.data_ptr(), E, vt_replace.data_ptr(), st)
         # second pass where the first one left budget
-        open_ = (n_chosen < budget).to(I32).contiguous()
         first_edge = best
         attaches = chosen
         _lib.call("pmesh_cluster_attach_propose", edge_vi.data_ptr(), edge_vj.data_ptr(), rank.data_ptr(), sample_e.data_ptr(),
                   open_.data_ptr(), E, Nv, vt_replace.data_ptr(), first_edge.data_ptr(), attaches.data_ptr(), st)
-        keep2, _ = cut(attaches, budget - torch.minimum(n_chosen, budget))
+        keep2, _, _ = cut(attaches, rest, False)
         pairs = vt_replace.clone()
         _lib.call("pmesh_cluster_attach", edge_vi.data_ptr(), edge_vj.data_ptr(), rank.data_ptr(), keep2.data_ptr(), E,
                   first_edge.data_ptr(), pairs.data_ptr(), vt_replace.data_ptr(), st)

@@ -284,6 +284,29 @@ def test_device_clustering_equals_the_serial_host_routine(cuda, seed):
                                          dev(budget, cuda), Nv)
 
 
+def test_contraction_order_on_the_device_is_the_oracles(cuda):
+    """The native sort keys (few samples) and the two-sort path (many samples) order the candidate edges exactly as the
+    oracle's lexicographic statement, for costs that are negative, signed zeros, denormal, infinite, NaN or an ulp
+    apart; the samples read off the keys are the oracle's."""
+    rng = np.random.default_rng(0)
+    n = 20000
+    vi = rng.integers(0, 300, n)
+    vj = vi + rng.integers(1, 50, n)
+    k = np.argsort(vi.astype(np.int64) * 1000 + vj, kind="stable")
+    vi, vj = vi[k].astype(np.int32), vj[k].astype(np.int32)
+    special = np.array([0.0, -0.0, 1e-45, -1e-45, 1e-30, -1e-30, -2.5, 2.5, np.nan, np.inf, -np.inf, 1.0, 1.0000001, -1.0], np.float32)
+    cost = rng.choice(special, n)
+    cost[::7] = rng.normal(size=len(cost[::7])).astype(np.float32)
+    for cum in (np.array([300]), np.array([100, 100, 200, 300]), np.arange(3, 384, 3)[:127], np.arange(2, 302, 2)):
+        cum = cum.astype(np.int32)
+        want_perm, want_sample = D.contraction_order(cost, vi, vj, cum)
+        perm, sample = decimate.contraction_order(dev(cost, cuda), dev(vi, cuda), dev(vj, cuda), dev(cum, cuda))
+        assert np.array_equal(perm.cpu().numpy(), want_perm), len(cum)
+        assert np.array_equal(sample.cpu().numpy(), want_sample), len(cum)
+    perm, sample = decimate.contraction_order(dev(cost[:0], cuda), dev(vi[:0], cuda), dev(vj[:0], cuda), dev(np.array([5], np.int32), cuda))
+    assert perm.shape[0] == 0 and sample.shape[0] == 0
+
+
 def test_simplify_is_the_same_with_host_clustering(cuda, monkeypatch):
     v, f, nv, mf = batch(("sphere3", "room_small", "torus"))
     vx, fc = dev(v, cuda), dev(f, cuda)

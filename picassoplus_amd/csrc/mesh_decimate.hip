@@ -91,6 +91,50 @@ __device__ __forceinline__ float quadric_error(const float x[3], const float A[3
            (x[0] * b[0] + x[1] * b[1] + x[2] * b[2]) * 2 + c;
 }
 
+// One step of the elimination at row I, column J (both fixed at compile time, so that the 3 x 7 matrix lives in
+// registers): the largest entry of the column from row I down becomes the pivot; a column whose candidates are all
+// negligible is cleared and left.  Returns whether a pivot was taken.
+template <int I, int J>
+__device__ __forceinline__ bool rref_step(float (&M)[3][7], float tol)
+{
+    float p = fabsf(M[I][J]);
+    int k = I;
+#pragma unroll
+    for (int r = I + 1; r < 3; ++r)
+        if (p < fabsf(M[r][J])) { p = fabsf(M[r][J]); k = r; }
+    if (p <= tol) {
+#pragma unroll
+        for (int r = I; r < 3; ++r) M[r][J] = 0.f;
+        return false;
+    }
+#pragma unroll
+    for (int r = I + 1; r < 3; ++r)
+        if (k == r) {
+#pragma unroll
+            for (int c = J; c < 7; ++c) { const float t = M[I][c]; M[I][c] = M[r][c]; M[r][c] = t; }
+        }
+    const float pivot = M[I][J];
+#pragma unroll
+    for (int c = J; c < 7; ++c) M[I][c] = M[I][c] / pivot;
+#pragma unroll
+    for (int r = 0; r < 3; ++r) {
+        if (r == I) continue;
+        const float f = M[r][J];
+#pragma unroll
+        for (int c = J; c < 7; ++c) M[r][c] -= f * M[I][c];
+    }
+    return true;
+}
+
+// column J with `i` rows done so far (i <= J)
+template <int J>
+__device__ __forceinline__ void rref_column(float (&M)[3][7], float tol, int &i)
+{
+    if (i == 0) i += rref_step<0, J>(M, tol);
+    else if (J >= 1 && i == 1) i += rref_step<1, (J >= 1 ? J : 1)>(M, tol);
+    else if (J >= 2 && i == 2) i += rref_step<2, (J >= 2 ? J : 2)>(M, tol);
+}
+
 // Reduced row echelon form of [A | b | I] with partial pivoting and the negligible-column rule of the reference's
 // RrefDim3 (decimate_gpu.cu:79-193): x = -A^-1 b, and the reciprocal condition number 1 / (|A|_inf |A^-1|_inf).
 __device__ __forceinline__ float solve3(const float A[3][3], const float b[3], float (&x)[3])
@@ -109,28 +153,14 @@ __device__ __forceinline__ float solve3(const float A[3][3], const float b[3], f
 #pragma unroll
     for (int r = 0; r < 3; ++r) normA = fmaxf(normA, fabsf(M[r][0]) + fabsf(M[r][1]) + fabsf(M[r][2]));
     const float tol = kRrefEps * 7 * normA;
-    int i = 0, j = 0;
-    while (i < 3 && j < 7) {
-        float p = fabsf(M[i][j]);
-        int k = i;
-        for (int r = i + 1; r < 3; ++r)
-            if (p < fabsf(M[r][j])) { p = fabsf(M[r][j]); k = r; }
-        if (p <= tol) {
-            for (int r = i; r < 3; ++r) M[r][j] = 0.f;
-            ++j;
-            continue;
-        }
-        for (int c = j; c < 7; ++c) { const float t = M[i][c]; M[i][c] = M[k][c]; M[k][c] = t; }
-        const float pivot = M[i][j];
-        for (int c = j; c < 7; ++c) M[i][c] = M[i][c] / pivot;
-        for (int r = 0; r < 3; ++r) {
-            if (r == i) continue;
-            const float f = M[r][j];
-            for (int c = j; c < 7; ++c) M[r][c] -= f * M[i][c];
-        }
-        ++i;
-        ++j;
-    }
+    int i = 0;                                        // rows done; the columns are walked until three are
+    rref_column<0>(M, tol, i);
+    rref_column<1>(M, tol, i);
+    rref_column<2>(M, tol, i);
+    rref_column<3>(M, tol, i);
+    rref_column<4>(M, tol, i);
+    rref_column<5>(M, tol, i);
+    rref_column<6>(M, tol, i);
     x[0] = -M[0][3]; x[1] = -M[1][3]; x[2] = -M[2][3];
     float normInv = 0.f;
 #pragma unroll

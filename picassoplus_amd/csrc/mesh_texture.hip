@@ -77,7 +77,7 @@ __global__ __launch_bounds__(kBlock) void texture_fwd_k(const float *__restrict_
 #pragma unroll
             for (int i = 0; i < 16; i += 4) *reinterpret_cast<float4 *>(o + i) = make_float4(v[i], v[i + 1], v[i + 2], v[i + 3]);
         } else {
-            for (int i = 0; i < B; ++i) o[i] = v[i];
+            sph_store(o, v, Lv);
         }
     }
 }
@@ -266,8 +266,7 @@ __global__ __launch_bounds__(kBlock) void facet_frame_k(const float *__restrict_
         const int B = (L + 1) * (L + 1);
         float v[36];
         sph_harm_at(nx, ny, nz, L, v);
-        float *o = coeff + f * B;
-        for (int i = 0; i < B; ++i) o[i] = v[i];
+        sph_store(coeff + f * B, v, L);
     }
 }
 

@@ -62,4 +62,23 @@ __device__ __forceinline__ void sph_harm_at(float x, float y, float z, int L, fl
     }
 }
 
+// The (L + 1)^2 basis values of a point to memory, degree by degree with compile-time indices: a copy loop over a
+// run-time count would index the value array dynamically and push it out of the registers into private memory.
+template <int D>
+__device__ __forceinline__ void sph_store_degree(float *o, const float (&v)[36])
+{
+#pragma unroll
+    for (int i = D * D; i < (D + 1) * (D + 1); ++i) o[i] = v[i];
+}
+
+__device__ __forceinline__ void sph_store(float *o, const float (&v)[36], int L)
+{
+    sph_store_degree<0>(o, v);
+    if (L >= 1) sph_store_degree<1>(o, v);
+    if (L >= 2) sph_store_degree<2>(o, v);
+    if (L >= 3) sph_store_degree<3>(o, v);
+    if (L >= 4) sph_store_degree<4>(o, v);
+    if (L >= 5) sph_store_degree<5>(o, v);
+}
+
 }  // namespace pmesh

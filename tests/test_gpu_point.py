@@ -10,6 +10,7 @@ import pytest
 import torch
 
 from oracle import point_ref as P
+from picassoplus_amd import _lib
 from picassoplus_amd.point import layers as point_layers
 from picassoplus_amd.point import utils as point_utils
 from picassoplus_amd.point.pi_modules import (buildkernel, conv3d, nnquery, point_nnquery, point_pool3d, pool3d, sample,
@@ -232,6 +233,39 @@ def test_conv_parity(cuda, sizes, radius, C, r, F, T):
     out2 = conv3d.conv3d(xt2, ft2, *args) if coeff is None else conv3d.fuzzyconv3d(xt2, ft2, *args, dev(coeff, cuda))
     out2.backward(dev(g, cuda, F32))
     assert torch.equal(out, out2) and torch.equal(xt.grad, xt2.grad) and torch.equal(ft.grad, ft2.grad)
+
+
+@pytest.mark.parametrize("sizes,radius,C,F,T", [([800, 500], 0.2, 64, 17, 17), ([500], 0.3, 128, 20, 6), ([900, 40], 0.2, 128, 10, 4),
+                                                ([700], 0.25, 32, 8, None), ([400], 0.25, 8, 12, 2), ([300, 1, 90], 0.3, 4, 16, 3),
+                                                ([3000], 0.12, 20, 5, 2)])
+def test_conv_backward_in_one_pass_and_in_two(cuda, monkeypatch, sizes, radius, C, F, T):
+    """Shapes the one-pass backward takes (depth multiplier 1, at most 20 bins and 128 channels, from one row per
+    wavefront to 32): both gradients against the oracle, and against the separate input- and filter-gradient passes."""
+    say("case point conv backward", sizes, radius, C, F, T)
+    db, q, count, nn_index, _, bins, coeff = point_graph(cuda, 41, sizes, radius, T, F)
+    rng = np.random.default_rng(42)
+    x, filt = rng.normal(size=(len(db), C)), rng.normal(0, 0.3, (F, C, 1))
+    g = rng.normal(size=(len(q), C))
+    gin_ref, gfilt_ref = P.conv_bwd(g, x, filt, count, nn_index, bins, coeff)
+    args = (dev(count, cuda), dev(nn_index, cuda), dev(bins, cuda))
+    grads = {}
+    for two in (False, True):
+        if two:
+            monkeypatch.setenv("PMESH_POINT_CONV_TWO_PASSES", "1")
+        seen = []
+        _lib.set_call_hook(lambda name, phase: seen.append(name))
+        xt, ft = dev(x, cuda, F32).requires_grad_(True), dev(filt, cuda, F32).requires_grad_(True)
+        out = conv3d.conv3d(xt, ft, *args) if coeff is None else conv3d.fuzzyconv3d(xt, ft, *args, dev(coeff, cuda))
+        out.backward(dev(g, cuda, F32))
+        torch.cuda.synchronize()
+        _lib.set_call_hook(None)
+        assert "pmesh_point_conv_bwd" in seen
+        label = "two passes" if two else "one pass"
+        assert_close(xt.grad, gin_ref, "point conv grad_input [%s]" % label)
+        assert_close(ft.grad, gfilt_ref, "point conv grad_filter [%s]" % label)
+        grads[two] = (xt.grad, ft.grad)
+    assert_close(grads[False][0], grads[True][0].double().cpu().numpy(), "point conv grad_input one pass vs two")
+    assert_close(grads[False][1], grads[True][1].double().cpu().numpy(), "point conv grad_filter one pass vs two")
 
 
 @pytest.mark.parametrize("sizes,radius,C", [([60], 0.45, 4), ([1500, 700], 0.2, 64), ([900], 0.25, 37)])

@@ -701,7 +701,7 @@ def run_pcloud(args, torch):
     # every operand once: per pair its index pair, T bins and T weights, one gathered row of C floats; per point a row
     pair = 8 + 8 * T
     nb = {"point_conv_fwd": P * (pair + 4 * C) + 4 * Np * C + 4 * Np,
-          "point_conv_bwd": P * (2 * pair + 8 * C) + 4 * Np * C * 2 + 4 * Np}     # input and filter gradient: two passes over the pairs
+          "point_conv_bwd": P * (pair + 4 * C) + 4 * Np * C * 2 + 4 * Np}     # input and filter gradient from one walk over the pairs
     fl = {"point_conv_fwd": 2.0 * P * C * (T + 1), "point_conv_bwd": 2.0 * P * C * (2 * T + 2)}
     dom = max(nb, key=lambda k: per_op[k])
     ach = nb[dom] / (per_op[dom] * 1e-3) / 1e9

@@ -51,6 +51,8 @@ def parse():
     ap.add_argument("--bf16-features", action="store_true",
                     help="scene workload with the features (texture rows, layer outputs, their gradients) kept in bf16 "
                          "in HBM and one fp16 product per element with fp32 accumulation: a separate figure")
+    ap.add_argument("--graph", action="store_true",
+                    help="hierarchy workload: also record the step (forward + backward) once as a HIP graph and time its replays")
     ap.add_argument("--traffic-from", nargs=2, metavar=("FETCH_CSV", "WRITE_CSV"),
                     help="no benchmark: turn the counter_collection CSVs of two rocprofv3 --pmc runs (FETCH_SIZE, "
                          "WRITE_SIZE) of this workload into profiles/traffic.json and a text summary")
@@ -865,21 +867,51 @@ def run_hierarchy(args, torch):
         return torch.autograd.grad(x, [x0] + params, gy)
 
     def timed(fn):
-        timer = EventTimer(torch)
-        _lib.set_call_hook(timer)
+        # the step's time from a plain loop, the per-op times from a second loop with an event pair around every native
+        # call (some 150 calls per step here: the event records alone add 4 % to a full-size step and a third to a small one)
         for _ in range(args.warmup):
             fn()
         torch.cuda.synchronize()
-        timer.on = True
         t0 = time.perf_counter()
         for _ in range(args.steps):
             fn()
         torch.cuda.synchronize()
         ms = (time.perf_counter() - t0) * 1e3 / args.steps
+        timer = EventTimer(torch)
+        _lib.set_call_hook(timer)
+        timer.on = True
+        for _ in range(args.steps):
+            fn()
+        torch.cuda.synchronize()
         _lib.set_call_hook(None)
         return ms, timer.totals(args.steps)
 
     ms, per_op = timed(step)
+    graph_ms = None
+    if args.graph:
+        # the same step recorded once and replayed: what the launches of about 150 kernels per step cost on the host
+        # side no longer lies between the kernels (matters for small meshes; a 2 M-facet step is bound by the GPU)
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            step()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            recorded = step()
+        for _ in range(args.warmup):
+            graph.replay()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            graph.replay()
+        torch.cuda.synchronize()
+        graph_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+        eager = step()
+        torch.cuda.synchronize()
+        if not all(torch.equal(a, b) for a, b in zip(recorded, eager)):
+            sys.exit("bench.py --graph: the replayed step differs from the eager one")
     # every level's block alone (forward + backward of its five ops and their tails)
     conv_ops = ["v2f_fwd", "texture_fwd", "f2f_fwd", "f2v_fwd", "f2v_bwd", "f2f_bwd_texture", "f2f_bwd_filter",
                 "texture_bwd", "v2f_bwd"]
@@ -917,6 +949,8 @@ def run_hierarchy(args, torch):
                config=dict(workload="grid%d_4levels_V2F+texture+F2F+F2V+pool+unpool_C32-256_L3_fp32_fwd+bwd" % cells,
                            facets=[d["nf"] for d in lv], vertices=[d["nv"] for d in lv] + [int(lv[-1]["vt_out"].shape[0])],
                            channels=W[:NL], sh_degree=L))
+    if graph_ms is not None:
+        res["graph_replay_ms_per_step"] = graph_ms
     if not args.no_cpu_baseline:
         res["cpu_baseline"] = cpu_baseline_block(lv[-1], W[NL - 1], L, torch)
     return res

@@ -342,6 +342,72 @@ def test_forward_replays_from_a_hip_graph(cuda):
             assert torch.equal(got, eager), "replay %d differs from the eager result" % i
 
 
+def test_training_step_replays_from_a_hip_graph(cuda):
+    """Forward AND backward of a two-level stack (V2F + texture -> F2F -> F2V with their tails, max / avg pooling,
+    unpooling with a pointwise layer; gradients for the input and every parameter) recorded once and replayed: the
+    native calls of the backward pass allocate, synchronise and clear nothing outside kernels either, and every replay
+    equals the eager step on the inputs then in the static buffers, with eager work between the replays."""
+    from picassoplus_amd.mesh.pi_modules import texture
+    rng = np.random.default_rng(43)
+    meshes = S.hierarchy_workload(seed=13, cells=32, levels=2)
+    L, W = 3, [32, 64, 64]
+    c = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(cuda)
+    torch.manual_seed(14)
+    lv = []
+    for l, m in enumerate(meshes[:2]):
+        v, f = m["vertex"], m["face"]
+        nv, nf = v.shape[0], f.shape[0]
+        normal, _ = S.triangle_normals_areas(v, f)
+        counts, bary, _ = S.texture_points(rng, nf, rng.integers(1, 4, nf).astype(np.int32))
+        lv.append(dict(nv=nv, face=c(f), counts=c(counts), cum=torch.cumsum(c(counts), 0, dtype=torch.int32), bary=c(bary.astype(np.float32)),
+                       nfc=c(np.maximum(S.vertex_facet_count(f, np.arange(nv), nv), 1).astype(np.int32)),
+                       ident=torch.arange(nv, dtype=torch.int32, device=cuda), coeff=layers.SphHarmCoeff(L)(c(normal.astype(np.float32))),
+                       vr=c(m["vt_replace"]), vm=c(m["vt_map"]), vt_out=torch.zeros(m["nv_out"], 3, device=cuda),
+                       v2f=layers.V2FConv3d(W[l], W[l], L, with_bn=False).to(cuda), f2f=layers.F2FConv3d(W[l], W[l], L, with_bn=False).to(cuda),
+                       f2v=layers.F2VConv3d(W[l], W[l + 1], L, with_bn=False).to(cuda), pool=layers.Pool3d("max" if l == 0 else "avg"),
+                       up=layers.PerItemConv3d(W[l + 1], W[l], with_bn=False).to(cuda)))
+    params = [p for d in lv for k in ("v2f", "f2f", "f2v", "up") for p in d[k].parameters()]
+    static_x = torch.randn(lv[0]["nv"], W[0], device=cuda, requires_grad=True)
+    static_g = torch.randn(lv[0]["nv"], W[0], device=cuda)
+
+    def step(x, g):
+        h, skips = x, []
+        for d in lv:
+            tex, sh = texture.interpolate(h, d["face"], d["bary"], d["cum"], L)
+            y = d["v2f"](h, d["face"]) + d["f2f"](tex, sh, d["counts"])
+            z = d["f2v"](y, d["face"], d["nfc"], d["ident"], d["coeff"])
+            skips.append(z)
+            h = d["pool"](z, d["vr"], d["vm"], d["vt_out"])
+        for d, z in zip(reversed(lv), reversed(skips)):
+            h = d["up"](z + layers.Unpool3d.forward(h, d["vr"], d["vm"]))
+        return [h] + list(torch.autograd.grad(h, [x] + params, g))
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            step(static_x, static_g)                            # warm-up: adjacency, filter packs and checks are cached now
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        static_out = step(static_x, static_g)
+    for i in range(4):
+        gen = torch.Generator(device=cuda).manual_seed(200 + i)
+        x = torch.randn(lv[0]["nv"], W[0], device=cuda, generator=gen)
+        g = torch.randn(lv[0]["nv"], W[0], device=cuda, generator=gen)
+        with torch.no_grad():
+            static_x.copy_(x)
+            static_g.copy_(g)
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [t.clone() for t in static_out]
+        eager = step(x.requires_grad_(True), g)                 # the program's own eager work between the replays
+        torch.cuda.synchronize()
+        for k, (a, b) in enumerate(zip(got, eager)):
+            assert torch.equal(a, b), "replay %d: result %d differs from the eager step" % (i, k)
+
+
 def _block_step(cuda, mods, x, f_np, bary_np, counts_np, normal_np, nfc_np, vr_np, vm_np, nvo, train):
     """One step of a small block with index tensors made from numpy anew: what a data loader hands a training or
     evaluation loop every batch."""

@@ -35,6 +35,8 @@ struct Options {
     bool f2f_bf16x3;         // 16 coefficients: the three-piece bf16 kernels instead of the two-piece fp16 ones
     bool f2f_half;           // 16 coefficients: one fp16 piece per operand (results within 1e-3)
     bool f2v_valu;           // facet2vertex on the vector-ALU kernels
+    bool f2v_fp32mfma;       // facet2vertex forward: the filter combination on the fp32 matrix instruction instead of split fp16
+    bool point_conv_two_passes;   // point convolution backward: input and filter gradient as separate passes
     bool dense_fp32mfma;     // pointwise tail on the fp32 matrix instruction
 };
 const Options &options();

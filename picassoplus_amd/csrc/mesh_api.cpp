@@ -37,6 +37,8 @@ static void load_options()
     g_options.f2f_bf16x3 = env_set("PMESH_F2F_BF16X3");
     g_options.f2f_half = env_set("PMESH_F2F_HALF");
     g_options.f2v_valu = env_set("PMESH_F2V_VALU");
+    g_options.f2v_fp32mfma = env_set("PMESH_F2V_FP32MFMA");
+    g_options.point_conv_two_passes = env_set("PMESH_POINT_CONV_TWO_PASSES");
     g_options.dense_fp32mfma = env_set("PMESH_DENSE_FP32MFMA");
     g_options_loaded = true;
 }

@@ -11,11 +11,10 @@
 // One cross-half exchange per vertex pair and channel block finishes the sum.
 // Against the vector-ALU version this replaces 64 FMAs per entry and four channels by 1/4 of an MFMA.
 #include "common.h"
+#include "fp16_split.h"
 #include "rows_internal.h"
 
 namespace pmesh {
-
-typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 // vdst lanes 32..63 <-> vsrc lanes 0..31; the s_nop cover the wait states around the swap.
 __device__ __forceinline__ void half_swap(float &a, float &b)
@@ -70,8 +69,13 @@ template <int STEP> __device__ __forceinline__ void st1_pair(bf16_t *p, float v,
 // Forward.  NCB = 32-channel blocks per workgroup column (blockIdx.y selects a chunk of 32*NCB channels).
 // Requires K == 16, 16-byte aligned coefficient rows, Nf * C * 4 < 2^32.  Workgroups are persistent; the
 // eight dies take contiguous eighths of the vertices (blockIdx.x & 7 = die).
-template <int NCB, typename TIO>
-__global__ __launch_bounds__(kBlock) void f2v_fwd_mfma_k(const TIO *__restrict__ in, const float *__restrict__ filt,
+// H2: the product on the fp16 matrix instruction, both operands split into two fp16 pieces (three piece products of
+// 32 cycles where the fp32 instruction takes eight of 64, and matrix work that runs beside the vector ALU instead of
+// in its place): the filter columns are scaled and split once per wavefront, the coefficients of a pass's 32 entries
+// are brought below 2^14 by one power of two for the wavefront, which leaves the sum again on the way into the
+// vertex sums.
+template <int NCB, typename TIO, bool H2>
+__global__ __launch_bounds__(kBlock, (H2 && NCB <= 2 && sizeof(TIO) == 4) ? 4 : 1) void f2v_fwd_mfma_k(const TIO *__restrict__ in, const float *__restrict__ filt,
                                                          const float *__restrict__ coeff,
                                                          const int *__restrict__ nfcount,
                                                          const int *__restrict__ rowptr,
@@ -94,6 +98,24 @@ __global__ __launch_bounds__(kBlock) void f2v_fwd_mfma_k(const TIO *__restrict__
         chb[cb] = con[cb] ? (unsigned)(co / r) * (unsigned)sizeof(TIO) : 0u;
 #pragma unroll
         for (int kk = 0; kk < 8; ++kk) wb[cb][kk] = con[cb] ? filt[(size_t)(8 * h + kk) * Co + co] : 0.f;
+    }
+
+    u32x4 bh[NCB], bl[NCB];
+    float inv_beta = 1.f;
+    if constexpr (H2) {
+        float m = 0.f;
+#pragma unroll
+        for (int cb = 0; cb < NCB; ++cb)
+#pragma unroll
+            for (int kk = 0; kk < 8; ++kk) m = fmaxf(m, fabsf(wb[cb][kk]));
+        const float beta = pow2_scale(hwave_fmax(m), &inv_beta);
+#pragma unroll
+        for (int cb = 0; cb < NCB; ++cb) {
+            float t[8];
+#pragma unroll
+            for (int kk = 0; kk < 8; ++kk) t[kk] = wb[cb][kk] * beta;
+            split8h(t, bh[cb], bl[cb]);
+        }
     }
 
     const int64_t groups = (NvOut + 3) >> 2, gx = (groups + 7) >> 3;
@@ -160,15 +182,45 @@ __global__ __launch_bounds__(kBlock) void f2v_fwd_mfma_k(const TIO *__restrict__
             for (int cb = 0; cb < NCB; ++cb)
 #pragma unroll
                 for (int i = 0; i < 16; ++i) x[cb][i] = cvt_raw(xr[cb][i], chb[cb], TIO());
+            if constexpr (H2) {
+                float m = 0.f;
 #pragma unroll
-            for (int cb = 0; cb < NCB; ++cb) {
-                f32x16 d;
+                for (int kk = 0; kk < 8; ++kk) m = fmaxf(m, fabsf(a[kk]));
+                float inv_alpha;
+                const float alpha = pow2_scale(hwave_fmax(m), &inv_alpha);       // (every lane of the wavefront is here)
 #pragma unroll
-                for (int i = 0; i < 16; ++i) d[i] = 0.f;
+                for (int kk = 0; kk < 8; ++kk) a[kk] *= alpha;
+                u32x4 ah, al;
+                split8h(a, ah, al);
+                const float unscale = inv_alpha * inv_beta;
 #pragma unroll
-                for (int kk = 0; kk < 8; ++kk) d = __builtin_amdgcn_mfma_f32_32x32x2f32(a[kk], wb[cb][kk], d, 0, 0, 0);
+                for (int cb = 0; cb < NCB; ++cb) {
+                    f32x16 d;
 #pragma unroll
-                for (int i = 0; i < 16; ++i) acc[cb][i >> 2] = fmaf(d[i], x[cb][i], acc[cb][i >> 2]);
+                    for (int i = 0; i < 16; ++i) d[i] = 0.f;
+                    // three piece products, smallest first
+                    d = mfma_f16(al, bh[cb], d);
+                    d = mfma_f16(ah, bl[cb], d);
+                    d = mfma_f16(ah, bh[cb], d);
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        float t = 0.f;
+#pragma unroll
+                        for (int i = 4 * q; i < 4 * q + 4; ++i) t = fmaf(d[i], x[cb][i], t);
+                        acc[cb][q] = fmaf(t, unscale, acc[cb][q]);
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int cb = 0; cb < NCB; ++cb) {
+                    f32x16 d;
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) d[i] = 0.f;
+#pragma unroll
+                    for (int kk = 0; kk < 8; ++kk) d = __builtin_amdgcn_mfma_f32_32x32x2f32(a[kk], wb[cb][kk], d, 0, 0, 0);
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) acc[cb][i >> 2] = fmaf(d[i], x[cb][i], acc[cb][i >> 2]);
+                }
             }
             if (!__builtin_amdgcn_ballot_w64(e0 + 8 * (p + 1) < e1)) break;
         }
@@ -386,11 +438,21 @@ static void f2v_fwd_launch(const TIO *in, const float *filt, const float *coeff,
     const int64_t want = ceil_div(ceil_div(NvOut, 16), 8) * 8;            // 16 vertices per workgroup sweep
     const unsigned gxn = (unsigned)(want < 4096 ? want : 4096);
     const dim3 grid(gxn, gy), block(kBlock);
-    switch (ncb) {
-    case 1: f2v_fwd_mfma_k<1, TIO><<<grid, block, 0, st>>>(in, filt, coeff, nfcount, rowptr, colidx, out, NvOut, C, r, Co); break;
-    case 2: f2v_fwd_mfma_k<2, TIO><<<grid, block, 0, st>>>(in, filt, coeff, nfcount, rowptr, colidx, out, NvOut, C, r, Co); break;
-    default: f2v_fwd_mfma_k<3, TIO><<<grid, block, 0, st>>>(in, filt, coeff, nfcount, rowptr, colidx, out, NvOut, C, r, Co); break;
+#define PM_F2V_FWD(N, H) f2v_fwd_mfma_k<N, TIO, H><<<grid, block, 0, st>>>(in, filt, coeff, nfcount, rowptr, colidx, out, NvOut, C, r, Co)
+    if (options().f2v_fp32mfma) {
+        switch (ncb) {
+        case 1: PM_F2V_FWD(1, false); break;
+        case 2: PM_F2V_FWD(2, false); break;
+        default: PM_F2V_FWD(3, false); break;
+        }
+    } else {
+        switch (ncb) {
+        case 1: PM_F2V_FWD(1, true); break;
+        case 2: PM_F2V_FWD(2, true); break;
+        default: PM_F2V_FWD(3, true); break;
+        }
     }
+#undef PM_F2V_FWD
 }
 
 int f2v_fwd_mfma(const void *in, const float *filt, const float *coeff, const int *nfcount, const int *rowptr,

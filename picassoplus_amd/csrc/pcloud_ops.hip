@@ -15,7 +15,6 @@
 //   gin[i, c]       = sum_{p = (o, i)} (1 / nn_count[o]) sum_m gout[o, c r + m] * w[p, c r + m]
 //   gfilt[f, co]    = sum_p sum_t [bin[p, t] = f] coeff[p, t] * gout[o, co] * in[i, co / r] / nn_count[o]
 #include "common.h"
-#include <stdlib.h>
 #include "rows_internal.h"
 #include "../../include/picasso_mesh.h"
 
@@ -664,7 +663,7 @@ extern "C" int pmesh_point_conv_bwd(const float *grad_output, const float *input
     PM_REQUIRE(grad_output && input && filter && nn_count && nn_index && bin_index && workspace, "point_conv_bwd: null pointer");
     const PairGraph g = {nn_index, nn_count, bin_index, bin_coeff, Np, Mp, Nout, T, F};
     if (grad_input && r == 1 && C % 4 == 0 && C <= 128 && F <= 20 && aligned16(grad_output) && aligned16(filter) && aligned16(grad_input) &&
-        aligned16(input) && !getenv("PMESH_POINT_CONV_TWO_PASSES")) {
+        aligned16(input) && !options().point_conv_two_passes) {
         // both gradients from one walk over the pairs in database-point order
         PM_REQUIRE(rowptr_in && order_in, "point_conv_bwd: the input gradient needs the pairs sorted by database point");
         const RowShape rs = row_shape(C / 2);                        // two channels per lane: at most 64 lanes per row

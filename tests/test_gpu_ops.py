@@ -184,12 +184,13 @@ def test_texture_interpolation_rejects_bad_totals(cuda):
                                                 ("sphere3", 200, 1, 16, True), ("sphere2", 12, 3, 16, False),
                                                 ("room_small", 128, 2, 16, True), ("sphere3", 33, 1, 16, False),
                                                 ("sphere3", 64, 1, 25, False), ("room_small", 32, 2, 36, True)])
-@pytest.mark.parametrize("path", ["default", "valu"])
+@pytest.mark.parametrize("path", ["default", "valu", "fp32mfma"])
 def test_f2v_parity(cuda, native_options, mesh, C, r, K, strided, path):
     """default: matrix-core kernels where they apply (at least 32 output channels; 16 coefficients, or from 9 on as
-    zero-padded blocks of 16); valu: the vector-ALU kernels for every shape."""
+    zero-padded blocks of 16), the forward's filter combination as two-piece fp16 products; fp32mfma: the same kernels
+    with that product on the fp32 matrix instruction; valu: the vector-ALU kernels for every shape."""
     say("case f2v", mesh, C, r, K, strided, path)
-    native_options(PMESH_F2V_VALU="1" if path == "valu" else "0")
+    native_options(PMESH_F2V_VALU="1" if path == "valu" else "0", PMESH_F2V_FP32MFMA="1" if path == "fp32mfma" else "0")
     v, f = mesh_case(mesh)
     rng = np.random.default_rng(11)
     nv, nf = v.shape[0], f.shape[0]

@@ -238,7 +238,7 @@ def test_conv_parity(cuda, sizes, radius, C, r, F, T):
 @pytest.mark.parametrize("sizes,radius,C,F,T", [([800, 500], 0.2, 64, 17, 17), ([500], 0.3, 128, 20, 6), ([900, 40], 0.2, 128, 10, 4),
                                                 ([700], 0.25, 32, 8, None), ([400], 0.25, 8, 12, 2), ([300, 1, 90], 0.3, 4, 16, 3),
                                                 ([3000], 0.12, 20, 5, 2)])
-def test_conv_backward_in_one_pass_and_in_two(cuda, monkeypatch, sizes, radius, C, F, T):
+def test_conv_backward_in_one_pass_and_in_two(cuda, native_options, sizes, radius, C, F, T):
     """Shapes the one-pass backward takes (depth multiplier 1, at most 20 bins and 128 channels, from one row per
     wavefront to 32): both gradients against the oracle, and against the separate input- and filter-gradient passes."""
     say("case point conv backward", sizes, radius, C, F, T)
@@ -251,7 +251,7 @@ def test_conv_backward_in_one_pass_and_in_two(cuda, monkeypatch, sizes, radius, 
     grads = {}
     for two in (False, True):
         if two:
-            monkeypatch.setenv("PMESH_POINT_CONV_TWO_PASSES", "1")
+            native_options(PMESH_POINT_CONV_TWO_PASSES="1")
         seen = []
         _lib.set_call_hook(lambda name, phase: seen.append(name))
         xt, ft = dev(x, cuda, F32).requires_grad_(True), dev(filt, cuda, F32).requires_grad_(True)

@@ -255,7 +255,11 @@ __global__ __launch_bounds__(kBlock, (H2 && NCB <= 2 && sizeof(TIO) == 4) ? 4 : 
 // wavefront writes for its own tile; the index chain face -> vt_map -> nf_count runs three tiles ahead.
 // Workgroups own contiguous facet ranges (fixed by the problem size only) and leave one partial filter
 // gradient each, summed by reduce_partials in a fixed order.
-template <int NCB, int R, typename TIO>
+// H2: both products as two-piece fp16 products (3 + 6 instructions of 32 cycles per tile and channel block instead of
+// 8 + 16 of 64): the tile's coefficients share one power-of-two scale in both of their layouts, in * s gets one per
+// tile and channel block, and the second product of a tile is taken out of its scale before it joins the running
+// filter gradient.
+template <int NCB, int R, typename TIO, bool H2>
 __global__ __launch_bounds__(kBlock, 2) void f2v_bwd_mfma_k(const TIO *__restrict__ gout, const TIO *__restrict__ in,
                                                          const float *__restrict__ filt,
                                                          const float *__restrict__ coeff,
@@ -294,6 +298,23 @@ __global__ __launch_bounds__(kBlock, 2) void f2v_bwd_mfma_k(const TIO *__restric
     for (int cb = 0; cb < NCB; ++cb)
 #pragma unroll
         for (int i = 0; i < 16; ++i) d2[cb][i] = 0.f;
+    u32x4 bh[NCB], bl[NCB];
+    float inv_beta = 1.f;
+    if constexpr (H2) {
+        float m = 0.f;
+#pragma unroll
+        for (int cb = 0; cb < NCB; ++cb)
+#pragma unroll
+            for (int kk = 0; kk < 8; ++kk) m = fmaxf(m, fabsf(wb[cb][kk]));
+        const float beta = pow2_scale(hwave_fmax(m), &inv_beta);
+#pragma unroll
+        for (int cb = 0; cb < NCB; ++cb) {
+            float t[8];
+#pragma unroll
+            for (int kk = 0; kk < 8; ++kk) t[kk] = wb[cb][kk] * beta;
+            split8h(t, bh[cb], bl[cb]);
+        }
+    }
 
     auto ld_face = [&](int64_t f0, int (&va)[3]) {
         const int64_t f = f0 + col;
@@ -384,13 +405,41 @@ __global__ __launch_bounds__(kBlock, 2) void f2v_bwd_mfma_k(const TIO *__restric
                 xv[cb][i] = cvt_raw(rx, chb[cb], TIO());
             }
         }
+        // (H2) the tile's coefficients, in both layouts, under one scale
+        u32x4 a1h, a1l, a2h[2], a2l[2];
+        float inv_alpha = 1.f;
+        if constexpr (H2) {
+            float m = 0.f;
+#pragma unroll
+            for (int kk = 0; kk < 8; ++kk) m = fmaxf(m, fabsf(a1[kk]));
+            const float alpha = pow2_scale(hwave_fmax(m), &inv_alpha);      // (every lane of the wavefront is here)
+            float t[8];
+#pragma unroll
+            for (int kk = 0; kk < 8; ++kk) t[kk] = a1[kk] * alpha;
+            split8h(t, a1h, a1l);
+#pragma unroll
+            for (int g = 0; g < 2; ++g) {
+#pragma unroll
+                for (int kk = 0; kk < 8; ++kk) t[kk] = a2[8 * g + kk] * alpha;
+                split8h(t, a2h[g], a2l[g]);
+            }
+        }
 #pragma unroll
         for (int cb = 0; cb < NCB; ++cb) {
             f32x16 d;
 #pragma unroll
             for (int i = 0; i < 16; ++i) d[i] = 0.f;
+            if constexpr (H2) {
+                d = mfma_f16(a1l, bh[cb], d);
+                d = mfma_f16(a1h, bl[cb], d);
+                d = mfma_f16(a1h, bh[cb], d);
+                const float unscale = inv_alpha * inv_beta;
 #pragma unroll
-            for (int kk = 0; kk < 8; ++kk) d = __builtin_amdgcn_mfma_f32_32x32x2f32(a1[kk], wb[cb][kk], d, 0, 0, 0);
+                for (int i = 0; i < 16; ++i) d[i] *= unscale;
+            } else {
+#pragma unroll
+                for (int kk = 0; kk < 8; ++kk) d = __builtin_amdgcn_mfma_f32_32x32x2f32(a1[kk], wb[cb][kk], d, 0, 0, 0);
+            }
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
                 const int ri = 8 * (i >> 2) + 4 * h + (i & 3);
@@ -401,9 +450,37 @@ __global__ __launch_bounds__(kBlock, 2) void f2v_bwd_mfma_k(const TIO *__restric
                 st1_pair<R>(const_cast<TIO *>(at_bytes(gin, (unsigned)(f0 + ri) * in_row + chb[cb])), gi,
                             f0 + ri < fend && con[cb] && (R == 1 || !(col & 1)), col);
             }
+            if constexpr (H2) {
+                float D[16], m = 0.f;
 #pragma unroll
-            for (int i = 0; i < 16; ++i)
-                d2[cb] = __builtin_amdgcn_mfma_f32_32x32x2f32(a2[i], xv[cb][i] * sv[cb][i], d2[cb], 0, 0, 0);
+                for (int i = 0; i < 16; ++i) {
+                    D[i] = xv[cb][i] * sv[cb][i];
+                    m = fmaxf(m, fabsf(D[i]));
+                }
+                float inv_delta;
+                const float delta = pow2_scale(hwave_fmax(m), &inv_delta);
+                f32x16 t2;
+#pragma unroll
+                for (int i = 0; i < 16; ++i) t2[i] = 0.f;
+#pragma unroll
+                for (int g = 0; g < 2; ++g) {
+                    float t[8];
+#pragma unroll
+                    for (int kk = 0; kk < 8; ++kk) t[kk] = D[8 * g + kk] * delta;
+                    u32x4 Dh, Dl;
+                    split8h(t, Dh, Dl);
+                    t2 = mfma_f16(a2l[g], Dh, t2);
+                    t2 = mfma_f16(a2h[g], Dl, t2);
+                    t2 = mfma_f16(a2h[g], Dh, t2);
+                }
+                const float unscale2 = inv_alpha * inv_delta;
+#pragma unroll
+                for (int q = 0; q < 8; ++q) d2[cb][q] = fmaf(t2[q], unscale2, d2[cb][q]);      // (rows 0..15: the coefficients)
+            } else {
+#pragma unroll
+                for (int i = 0; i < 16; ++i)
+                    d2[cb] = __builtin_amdgcn_mfma_f32_32x32x2f32(a2[i], xv[cb][i] * sv[cb][i], d2[cb], 0, 0, 0);
+            }
         }
 #pragma unroll
         for (int jj = 0; jj < 3; ++jj) { vo_c[jj] = vo_n[jj]; cnt_c[jj] = cnt_n[jj]; vo_n[jj] = vo_nn[jj]; va_nn[jj] = va_3[jj]; }
@@ -479,10 +556,15 @@ static void f2v_bwd_launch(const TIO *gout, const TIO *in, const float *filt, co
     const unsigned gy = (unsigned)ceil_div(Co, 32);
     const int64_t rows_per_block = ceil_div(ceil_div(Nf, G), 128) * 128;
     const dim3 grid((unsigned)G, gy), block(kBlock);
-    if (r == 1)
-        f2v_bwd_mfma_k<1, 1, TIO><<<grid, block, 0, st>>>(gout, in, filt, coeff, face, nfcount, vtmap, gin, partial, Nf, NvOut, C, Co, rows_per_block);
-    else
-        f2v_bwd_mfma_k<1, 2, TIO><<<grid, block, 0, st>>>(gout, in, filt, coeff, face, nfcount, vtmap, gin, partial, Nf, NvOut, C, Co, rows_per_block);
+#define PM_F2V_BWD(RR, H) f2v_bwd_mfma_k<1, RR, TIO, H><<<grid, block, 0, st>>>(gout, in, filt, coeff, face, nfcount, vtmap, gin, partial, Nf, NvOut, C, Co, rows_per_block)
+    if (options().f2v_fp32mfma) {
+        if (r == 1) PM_F2V_BWD(1, false);
+        else PM_F2V_BWD(2, false);
+    } else {
+        if (r == 1) PM_F2V_BWD(1, true);
+        else PM_F2V_BWD(2, true);
+    }
+#undef PM_F2V_BWD
 }
 
 int f2v_bwd_mfma(const void *gout, const void *in, const float *filt, const float *coeff, const int *face,

@@ -71,9 +71,9 @@ template <int STEP> __device__ __forceinline__ void st1_pair(bf16_t *p, float v,
 // eight dies take contiguous eighths of the vertices (blockIdx.x & 7 = die).
 // H2: the product on the fp16 matrix instruction, both operands split into two fp16 pieces (three piece products of
 // 32 cycles where the fp32 instruction takes eight of 64, and matrix work that runs beside the vector ALU instead of
-// in its place): the filter columns are scaled and split once per wavefront, the coefficients of a pass's 32 entries
-// are brought below 2^14 by one power of two for the wavefront, which leaves the sum again on the way into the
-// vertex sums.
+// in its place): every filter column is scaled by its own power of two and split once per wavefront, the coefficients
+// of a pass's 32 entries are brought below 2^14 by one power of two for the wavefront, and both leave the sum again on
+// the way into the vertex sums.
 template <int NCB, typename TIO, bool H2>
 __global__ __launch_bounds__(kBlock, (H2 && NCB <= 2 && sizeof(TIO) == 4) ? 4 : 1) void f2v_fwd_mfma_k(const TIO *__restrict__ in, const float *__restrict__ filt,
                                                          const float *__restrict__ coeff,
@@ -100,17 +100,18 @@ __global__ __launch_bounds__(kBlock, (H2 && NCB <= 2 && sizeof(TIO) == 4) ? 4 : 
         for (int kk = 0; kk < 8; ++kk) wb[cb][kk] = con[cb] ? filt[(size_t)(8 * h + kk) * Co + co] : 0.f;
     }
 
+    // (H2) every filter column under its own power-of-two scale: a column of small weights keeps its accuracy beside a large one
     u32x4 bh[NCB], bl[NCB];
-    float inv_beta = 1.f;
-    if constexpr (H2) {
-        float m = 0.f;
+    float inv_beta[NCB];
 #pragma unroll
-        for (int cb = 0; cb < NCB; ++cb)
+    for (int cb = 0; cb < NCB; ++cb) {
+        inv_beta[cb] = 1.f;
+        if constexpr (H2) {
+            float m = 0.f;
 #pragma unroll
             for (int kk = 0; kk < 8; ++kk) m = fmaxf(m, fabsf(wb[cb][kk]));
-        const float beta = pow2_scale(hwave_fmax(m), &inv_beta);
-#pragma unroll
-        for (int cb = 0; cb < NCB; ++cb) {
+            m = fmaxf(m, __shfl_xor(m, 32, 64));                       // the column's other eight coefficients
+            const float beta = pow2_scale(m, &inv_beta[cb]);
             float t[8];
 #pragma unroll
             for (int kk = 0; kk < 8; ++kk) t[kk] = wb[cb][kk] * beta;
@@ -192,9 +193,9 @@ __global__ __launch_bounds__(kBlock, (H2 && NCB <= 2 && sizeof(TIO) == 4) ? 4 : 
                 for (int kk = 0; kk < 8; ++kk) a[kk] *= alpha;
                 u32x4 ah, al;
                 split8h(a, ah, al);
-                const float unscale = inv_alpha * inv_beta;
 #pragma unroll
                 for (int cb = 0; cb < NCB; ++cb) {
+                    const float unscale = inv_alpha * inv_beta[cb];
                     f32x16 d;
 #pragma unroll
                     for (int i = 0; i < 16; ++i) d[i] = 0.f;
@@ -256,9 +257,9 @@ __global__ __launch_bounds__(kBlock, (H2 && NCB <= 2 && sizeof(TIO) == 4) ? 4 : 
 // Workgroups own contiguous facet ranges (fixed by the problem size only) and leave one partial filter
 // gradient each, summed by reduce_partials in a fixed order.
 // H2: both products as two-piece fp16 products (3 + 6 instructions of 32 cycles per tile and channel block instead of
-// 8 + 16 of 64): the tile's coefficients share one power-of-two scale in both of their layouts, in * s gets one per
-// tile and channel block, and the second product of a tile is taken out of its scale before it joins the running
-// filter gradient.
+// 8 + 16 of 64): the tile's coefficients share one power-of-two scale in both of their layouts, every filter column
+// and every channel of in * s has its own, and the second product of a tile is taken out of its scales before it
+// joins the running filter gradient.
 template <int NCB, int R, typename TIO, bool H2>
 __global__ __launch_bounds__(kBlock, 2) void f2v_bwd_mfma_k(const TIO *__restrict__ gout, const TIO *__restrict__ in,
                                                          const float *__restrict__ filt,
@@ -298,17 +299,18 @@ __global__ __launch_bounds__(kBlock, 2) void f2v_bwd_mfma_k(const TIO *__restric
     for (int cb = 0; cb < NCB; ++cb)
 #pragma unroll
         for (int i = 0; i < 16; ++i) d2[cb][i] = 0.f;
+    // (H2) every filter column under its own power-of-two scale: a column of small weights keeps its accuracy beside a large one
     u32x4 bh[NCB], bl[NCB];
-    float inv_beta = 1.f;
-    if constexpr (H2) {
-        float m = 0.f;
+    float inv_beta[NCB];
 #pragma unroll
-        for (int cb = 0; cb < NCB; ++cb)
+    for (int cb = 0; cb < NCB; ++cb) {
+        inv_beta[cb] = 1.f;
+        if constexpr (H2) {
+            float m = 0.f;
 #pragma unroll
             for (int kk = 0; kk < 8; ++kk) m = fmaxf(m, fabsf(wb[cb][kk]));
-        const float beta = pow2_scale(hwave_fmax(m), &inv_beta);
-#pragma unroll
-        for (int cb = 0; cb < NCB; ++cb) {
+            m = fmaxf(m, __shfl_xor(m, 32, 64));                       // the column's other eight coefficients
+            const float beta = pow2_scale(m, &inv_beta[cb]);
             float t[8];
 #pragma unroll
             for (int kk = 0; kk < 8; ++kk) t[kk] = wb[cb][kk] * beta;
@@ -433,7 +435,7 @@ __global__ __launch_bounds__(kBlock, 2) void f2v_bwd_mfma_k(const TIO *__restric
                 d = mfma_f16(a1l, bh[cb], d);
                 d = mfma_f16(a1h, bl[cb], d);
                 d = mfma_f16(a1h, bh[cb], d);
-                const float unscale = inv_alpha * inv_beta;
+                const float unscale = inv_alpha * inv_beta[cb];
 #pragma unroll
                 for (int i = 0; i < 16; ++i) d[i] *= unscale;
             } else {
@@ -457,8 +459,9 @@ __global__ __launch_bounds__(kBlock, 2) void f2v_bwd_mfma_k(const TIO *__restric
                     D[i] = xv[cb][i] * sv[cb][i];
                     m = fmaxf(m, fabsf(D[i]));
                 }
+                m = fmaxf(m, __shfl_xor(m, 32, 64));                     // my channel's other sixteen facets
                 float inv_delta;
-                const float delta = pow2_scale(hwave_fmax(m), &inv_delta);
+                const float delta = pow2_scale(m, &inv_delta);            // one scale per channel
                 f32x16 t2;
 #pragma unroll
                 for (int i = 0; i < 16; ++i) t2[i] = 0.f;

@@ -16,7 +16,7 @@ from picassoplus_amd.mesh import topology
 from picassoplus_amd.mesh.layers import sph_harm_values
 from picassoplus_amd.mesh.pi_modules import (conv3d, mesh_conv3d, mesh_pool3d, mesh_unpool3d, pool3d,
                                              texture, unpool3d)
-from util import assert_as_good_as_f32, assert_close, dev, mesh_case, rel_err, strided_vt_map, texture_case
+from util import MEASURED, assert_as_good_as_f32, assert_close, dev, mesh_case, rel_err, strided_vt_map, texture_case
 
 pytestmark = pytest.mark.gpu
 
@@ -220,6 +220,39 @@ def test_f2v_parity(cuda, native_options, mesh, C, r, K, strided, path):
     assert_as_good_as_f32(out, out_ref, loops.f2v_fwd(*a32, dtype=f32), "f2v out")
     assert_as_good_as_f32(xt.grad, gin_ref, gin32, "f2v grad_input")
     assert_as_good_as_f32(ft.grad, gfilt_ref, gfilt32, "f2v grad_filter")
+
+
+@pytest.mark.parametrize("path", ["default", "fp32mfma"])
+def test_f2v_channels_of_very_different_size(cuda, native_options, path):
+    """Filter columns and feature channels nine orders of magnitude apart: every channel is held to 1e-5 of ITS OWN
+    largest value (the matrix-core kernels scale each filter column and each channel of the second product by its own
+    power of two; one scale for all of them would leave the small channels with a few bits)."""
+    say("case f2v channel scales", path)
+    native_options(PMESH_F2V_FP32MFMA="1" if path == "fp32mfma" else "0")
+    v, f = mesh_case("sphere3")
+    rng = np.random.default_rng(14)
+    nv, nf, C, K = v.shape[0], f.shape[0], 64, 16
+    vt_map = np.arange(nv, dtype=np.int32)
+    nfc = np.maximum(S.vertex_facet_count(f, vt_map, nv), 1)
+    col = 10.0 ** rng.uniform(-6, 3, C)
+    x = rng.uniform(-1, 1, (nf, C)) * 10.0 ** rng.uniform(-3, 3, C)
+    filt = rng.normal(0, 0.5, (K, C, 1)) * col[None, :, None]
+    coeff = rng.normal(0, 0.5, (nf, K))
+    gout = rng.normal(0, 1, (nv, C)) * 10.0 ** rng.uniform(-3, 3, C)
+    xt = dev(x, cuda, torch.float32).requires_grad_(True)
+    ft = dev(filt, cuda, torch.float32).requires_grad_(True)
+    out = conv3d.facet2vertex(xt, ft, dev(coeff, cuda, torch.float32), dev(f, cuda), dev(nfc, cuda), dev(vt_map, cuda))
+    out.backward(dev(gout, cuda, torch.float32))
+    torch.cuda.synchronize()
+    # the float32 inputs are the oracle's inputs rounded: compare against the oracle on the rounded inputs
+    r32 = lambda a: a.astype(np.float32).astype(np.float64)
+    out_ref = loops.f2v_fwd(r32(x), r32(filt), r32(coeff), f, nfc, vt_map)
+    gin_ref, gfilt_ref = loops.f2v_bwd(r32(gout), r32(x), r32(filt), r32(coeff), f, nfc, vt_map)
+    for name, got, ref in (("out", out, out_ref), ("grad_input", xt.grad, gin_ref), ("grad_filter", ft.grad[:, :, 0], gfilt_ref[:, :, 0])):
+        got = got.detach().cpu().numpy().astype(np.float64)
+        worst = max(np.abs(got[:, c] - ref[:, c]).max() / np.abs(ref[:, c]).max() for c in range(C))
+        MEASURED.append(("f2v %s, worst channel relative to its own maximum [%s]" % (name, path), worst, 1e-5))
+        assert worst <= 1e-5, (name, worst)
 
 
 def test_f2v_unit_count_is_plain_scatter(cuda):

@@ -364,10 +364,10 @@ def run_conv_layer(args, torch, kind):
                       "facet2facet products one fp16 piece per operand on v_mfma_f32_32x32x16_f16, every sum accumulated in f32"
                       if bf16 else
                       "f32 in HBM; facet2facet products one fp16 piece per operand on v_mfma_f32_32x32x16_f16, f32 accumulate; "
-                      "facet2vertex f32" if args.f2f_half else
-                      "f32 in HBM; facet2facet products on v_mfma_f32_32x32x16_f16 with both operands split into two "
-                      "fp16 pieces (three piece products, about 22 significant bits), f32 accumulate; facet2vertex f32 "
-                      "(filter combination on v_mfma_f32_32x32x2_f32)"),
+                      "facet2vertex sums f32, its filter combination two fp16 pieces per operand" if args.f2f_half else
+                      "f32 in HBM; facet2facet products and facet2vertex's filter combination on v_mfma_f32_32x32x16_f16 with "
+                      "both operands split into two fp16 pieces (three piece products, about 22 significant bits), f32 "
+                      "accumulate; the sums over points and facets in f32"),
                config=dict(workload=name + ("_f2f-half-products" if args.f2f_half and not bf16 else ""), facets=d["nf"], vertices=d["nv"], texture_points=d["T"], channels=C,
                            sh_degree=L, meshes=int(len(d["mf_in"])), algorithmic_bytes=total_bytes))
     if not args.no_cpu_baseline:

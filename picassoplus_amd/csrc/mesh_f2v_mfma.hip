@@ -43,6 +43,22 @@ __device__ __forceinline__ unsigned ld_raw(const bf16_t *base, unsigned byte_off
 {
     return *reinterpret_cast<const unsigned *>(reinterpret_cast<const char *>(base) + (byte_offset & ~3u));
 }
+// The same fetch through a buffer descriptor (base, size in bytes): an offset at or past the size reads zero, so a
+// gather over slots that may be empty needs neither a branch around each fetch nor a zero beforehand -- an empty slot
+// carries the array's size as its offset.
+typedef __amdgpu_buffer_rsrc_t buffer_t;
+__device__ __forceinline__ buffer_t buffer_of(const void *base, unsigned bytes)
+{
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int)bytes, 0x00020000);
+}
+__device__ __forceinline__ unsigned ld_buf(buffer_t b, unsigned byte_offset, float)
+{
+    return __builtin_amdgcn_raw_buffer_load_b32(b, (int)byte_offset, 0, 0);
+}
+__device__ __forceinline__ unsigned ld_buf(buffer_t b, unsigned byte_offset, bf16_t)
+{
+    return __builtin_amdgcn_raw_buffer_load_b32(b, (int)(byte_offset & ~3u), 0, 0);
+}
 __device__ __forceinline__ float cvt_raw(unsigned w, unsigned, float) { return __builtin_bit_cast(float, w); }
 __device__ __forceinline__ float cvt_raw(unsigned w, unsigned byte_offset, bf16_t)
 {
@@ -80,10 +96,11 @@ __global__ __launch_bounds__(kBlock, (H2 && NCB <= 2 && sizeof(TIO) == 4) ? 4 : 
                                                          const int *__restrict__ nfcount,
                                                          const int *__restrict__ rowptr,
                                                          const int *__restrict__ colidx, TIO *__restrict__ out,
-                                                         int64_t NvOut, int C, int r, int Co)
+                                                         int64_t NvOut, int C, int r, int Co, unsigned in_bytes)
 {
     const int l = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int col = l & 31, h = l >> 5, j = col >> 3, s = col & 7;
+    const buffer_t in_buf = buffer_of(in, in_bytes);
     const int co0 = blockIdx.y * (32 * NCB);
     const unsigned row_bytes = (unsigned)C * (unsigned)sizeof(TIO);
 
@@ -164,8 +181,8 @@ __global__ __launch_bounds__(kBlock, (H2 && NCB <= 2 && sizeof(TIO) == 4) ? 4 : 
                 a[0] = t0.x; a[1] = t0.y; a[2] = t0.z; a[3] = t0.w;
                 a[4] = t1.x; a[5] = t1.y; a[6] = t1.z; a[7] = t1.w;
             }
-            // byte offsets of the facet rows my registers pair with
-            const unsigned boff = (f >= 0) ? (unsigned)f * row_bytes : 0xFFFFFFFFu;
+            // byte offsets of the facet rows my registers pair with (an empty slot: past the end, reads zero)
+            const unsigned boff = (f >= 0) ? (unsigned)f * row_bytes : in_bytes;
             unsigned b[16];
 #pragma unroll
             for (int i = 0; i < 16; ++i)
@@ -174,10 +191,7 @@ __global__ __launch_bounds__(kBlock, (H2 && NCB <= 2 && sizeof(TIO) == 4) ? 4 : 
 #pragma unroll
             for (int cb = 0; cb < NCB; ++cb)
 #pragma unroll
-                for (int i = 0; i < 16; ++i) {
-                    xr[cb][i] = 0u;
-                    if (b[i] != 0xFFFFFFFFu && con[cb]) xr[cb][i] = ld_raw(in, b[i] + chb[cb]);
-                }
+                for (int i = 0; i < 16; ++i) xr[cb][i] = ld_buf(in_buf, b[i] + chb[cb], TIO());
             float x[NCB][16];
 #pragma unroll
             for (int cb = 0; cb < NCB; ++cb)
@@ -505,20 +519,22 @@ __global__ __launch_bounds__(kBlock, 2) void f2v_bwd_mfma_k(const TIO *__restric
 
 bool f2v_mfma_ok(int64_t Nf, int C, int r, int K, const void *coeff)
 {
-    return K == 16 && C * r >= 32 && (reinterpret_cast<uintptr_t>(coeff) & 15) == 0 && Nf * (int64_t)C < (int64_t(1) << 30);
+    // (32-bit byte offsets into the feature array, with room for one row past the end)
+    return K == 16 && C * r >= 32 && (reinterpret_cast<uintptr_t>(coeff) & 15) == 0 && (Nf + 1) * (int64_t)C < (int64_t(1) << 30);
 }
 
 template <typename TIO>
 static void f2v_fwd_launch(const TIO *in, const float *filt, const float *coeff, const int *nfcount, const int *rowptr,
-                           const int *colidx, TIO *out, int64_t NvOut, int C, int r, hipStream_t st)
+                           const int *colidx, TIO *out, int64_t Nf, int64_t NvOut, int C, int r, hipStream_t st)
 {
     const int Co = C * r;
+    const unsigned in_bytes = (unsigned)(Nf * C * (int64_t)sizeof(TIO));
     const int ncb = Co <= 32 ? 1 : Co <= 64 ? 2 : Co <= 96 ? 3 : 2;      // wider rows: chunks of 64 channels (more wavefronts in flight)
     const unsigned gy = (unsigned)ceil_div(Co, 32 * ncb);
     const int64_t want = ceil_div(ceil_div(NvOut, 16), 8) * 8;            // 16 vertices per workgroup sweep
     const unsigned gxn = (unsigned)(want < 4096 ? want : 4096);
     const dim3 grid(gxn, gy), block(kBlock);
-#define PM_F2V_FWD(N, H) f2v_fwd_mfma_k<N, TIO, H><<<grid, block, 0, st>>>(in, filt, coeff, nfcount, rowptr, colidx, out, NvOut, C, r, Co)
+#define PM_F2V_FWD(N, H) f2v_fwd_mfma_k<N, TIO, H><<<grid, block, 0, st>>>(in, filt, coeff, nfcount, rowptr, colidx, out, NvOut, C, r, Co, in_bytes)
     if (options().f2v_fp32mfma) {
         switch (ncb) {
         case 1: PM_F2V_FWD(1, false); break;
@@ -536,10 +552,10 @@ static void f2v_fwd_launch(const TIO *in, const float *filt, const float *coeff,
 }
 
 int f2v_fwd_mfma(const void *in, const float *filt, const float *coeff, const int *nfcount, const int *rowptr,
-                 const int *colidx, void *out, int64_t NvOut, int C, int r, hipStream_t st, bool bf16)
+                 const int *colidx, void *out, int64_t Nf, int64_t NvOut, int C, int r, hipStream_t st, bool bf16)
 {
-    if (bf16) f2v_fwd_launch((const bf16_t *)in, filt, coeff, nfcount, rowptr, colidx, (bf16_t *)out, NvOut, C, r, st);
-    else f2v_fwd_launch((const float *)in, filt, coeff, nfcount, rowptr, colidx, (float *)out, NvOut, C, r, st);
+    if (bf16) f2v_fwd_launch((const bf16_t *)in, filt, coeff, nfcount, rowptr, colidx, (bf16_t *)out, Nf, NvOut, C, r, st);
+    else f2v_fwd_launch((const float *)in, filt, coeff, nfcount, rowptr, colidx, (float *)out, Nf, NvOut, C, r, st);
     PM_LAUNCHED("f2v_fwd(mfma)");
     return 0;
 }

@@ -978,7 +978,7 @@ extern "C" int pmesh_f2v_fwd(const float *input, const float *filter, const floa
     const int64_t blocks = ceil_div(NvOut, rs.rpb);
     PM_REQUIRE(grid_ok(blocks), "f2v_fwd: grid too large");
     const int cvec = ((K & 3) == 0 && aligned16(coeff)) ? 1 : 0;
-    if (!force_valu() && f2v_mfma_ok(Nf, C, r, K, coeff)) return f2v_fwd_mfma(input, filter, coeff, nf_count, rowptr, colidx, output, NvOut, C, r, st);
+    if (!force_valu() && f2v_mfma_ok(Nf, C, r, K, coeff)) return f2v_fwd_mfma(input, filter, coeff, nf_count, rowptr, colidx, output, Nf, NvOut, C, r, st);
     if (f2v_fast_ok(C, r, K, {input, filter, output})) {
         // persistent: enough workgroups to fill the chip several times over, each visiting many vertices
         const RowShape fs = row_shape(C * r / 4);
@@ -1063,7 +1063,7 @@ extern "C" int pmesh_f2v_fwd_bf16(const uint16_t *input, const float *filter, co
     PM_REQUIRE(NvOut <= INT32_MAX && Nf <= INT32_MAX / 3, "f2v_fwd_bf16: sizes exceed int32 indexing");
     PM_REQUIRE(f2v_mfma_ok(Nf, C, r, K, coeff) && !(C & 1) && !((reinterpret_cast<uintptr_t>(input) | reinterpret_cast<uintptr_t>(output)) & 3u),
                "f2v_fwd_bf16: bf16 features need 16 coefficients in 16-byte aligned rows, an even channel count and at least 32 output channels (K=%d C=%d r=%d)", K, C, r);
-    return f2v_fwd_mfma(input, filter, coeff, nf_count, rowptr, colidx, output, NvOut, C, r, (hipStream_t)stream, true);
+    return f2v_fwd_mfma(input, filter, coeff, nf_count, rowptr, colidx, output, Nf, NvOut, C, r, (hipStream_t)stream, true);
 }
 
 extern "C" int pmesh_f2v_bwd_bf16(const uint16_t *grad_output, const uint16_t *input, const float *filter,

@@ -14,7 +14,7 @@ bool f2v_mfma_ok(int64_t Nf, int C, int r, int K, const void *coeff);
 
 // bf16: feature rows (in, out) are bf16 (unsigned short) instead of float
 int f2v_fwd_mfma(const void *in, const float *filt, const float *coeff, const int *nfcount, const int *rowptr,
-                 const int *colidx, void *out, int64_t NvOut, int C, int r, hipStream_t st, bool bf16 = false);
+                 const int *colidx, void *out, int64_t Nf, int64_t NvOut, int C, int r, hipStream_t st, bool bf16 = false);
 
 // Backward on the matrix cores: depth multiplier 1 or 2, additionally NvOut * C * r * 4 < 2^32.  G workgroups
 // (f2v_bwd_mfma_blocks) leave G partial filter gradients of 16 * C * r floats in `partial`.

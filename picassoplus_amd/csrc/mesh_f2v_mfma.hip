@@ -295,6 +295,13 @@ __global__ __launch_bounds__(kBlock, 2) void f2v_bwd_mfma_k(const TIO *__restric
     const int64_t fbeg = rb * rows_per_block;
     const int64_t fend = (fbeg + rows_per_block < Nf) ? fbeg + rows_per_block : Nf;
     const unsigned in_row = (unsigned)C * (unsigned)sizeof(TIO), out_row = (unsigned)Co * (unsigned)sizeof(TIO);
+    // Gathers go through buffer descriptors: an offset at or past a descriptor's size reads zero, so neither the rows
+    // beyond this workgroup's range (the feature and coefficient descriptors end at its last facet) nor the corners
+    // without an output vertex (offset = the size of gout) need a branch, a compare or a zero per fetch.
+    const unsigned gout_bytes = (unsigned)NvOut * out_row;
+    const buffer_t gout_buf = buffer_of(gout, gout_bytes);
+    const buffer_t in_buf = buffer_of(in, (unsigned)(fend > 0 ? fend : 0) * in_row);
+    const buffer_t coeff_buf = buffer_of(coeff, (unsigned)(fend > 0 ? fend : 0) * 64u);
 
     float wb[NCB][8];
     unsigned chb[NCB], cob[NCB];
@@ -367,9 +374,9 @@ __global__ __launch_bounds__(kBlock, 2) void f2v_bwd_mfma_k(const TIO *__restric
         // corner table of my tile
         if (h == 0) {
             uint4 m0, m1;
-            m0.x = (vo_c[0] >= 0) ? (unsigned)vo_c[0] * out_row : 0xFFFFFFFFu;
-            m0.y = (vo_c[1] >= 0) ? (unsigned)vo_c[1] * out_row : 0xFFFFFFFFu;
-            m0.z = (vo_c[2] >= 0) ? (unsigned)vo_c[2] * out_row : 0xFFFFFFFFu;
+            m0.x = (vo_c[0] >= 0) ? (unsigned)vo_c[0] * out_row : gout_bytes;
+            m0.y = (vo_c[1] >= 0) ? (unsigned)vo_c[1] * out_row : gout_bytes;
+            m0.z = (vo_c[2] >= 0) ? (unsigned)vo_c[2] * out_row : gout_bytes;
             m0.w = 0u;
             m1.x = __float_as_uint((vo_c[0] >= 0) ? 1.0f / (float)cnt_c[0] : 0.f);
             m1.y = __float_as_uint((vo_c[1] >= 0) ? 1.0f / (float)cnt_c[1] : 0.f);
@@ -395,10 +402,12 @@ __global__ __launch_bounds__(kBlock, 2) void f2v_bwd_mfma_k(const TIO *__restric
             a1[0] = t0.x; a1[1] = t0.y; a1[2] = t0.z; a1[3] = t0.w;
             a1[4] = t1.x; a1[5] = t1.y; a1[6] = t1.z; a1[7] = t1.w;
         }
+        {
+            // (lanes col >= 16 hold no coefficient: an offset that stays past the end with the row steps added)
+            const unsigned cbase = col < 16 ? (unsigned)(f0 + 4 * h) * 64u + 4u * col : 0x80000000u;
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            const int64_t fi = f0 + 8 * (i >> 2) + 4 * h + (i & 3);
-            a2[i] = (fi < fend && col < 16) ? coeff[fi * 16 + col] : 0.f;
+            for (int i = 0; i < 16; ++i)
+                a2[i] = __builtin_bit_cast(float, ld_buf(coeff_buf, cbase + (8 * (i >> 2) + (i & 3)) * 64u, float()));
         }
 
         float sv[NCB][16], xv[NCB][16];
@@ -406,15 +415,11 @@ __global__ __launch_bounds__(kBlock, 2) void f2v_bwd_mfma_k(const TIO *__restric
         for (int i = 0; i < 16; ++i) {
             const int ri = 8 * (i >> 2) + 4 * h + (i & 3);
             const uint4 m0 = meta[wave][ri][0], m1 = meta[wave][ri][1];
-            const bool fok = f0 + ri < fend;
             const unsigned xoff = (unsigned)(f0 + ri) * in_row;
 #pragma unroll
             for (int cb = 0; cb < NCB; ++cb) {
-                unsigned r0 = 0u, r1 = 0u, r2 = 0u, rx = 0u;
-                if (m0.x != 0xFFFFFFFFu && con[cb]) r0 = ld_raw(gout, m0.x + cob[cb]);
-                if (m0.y != 0xFFFFFFFFu && con[cb]) r1 = ld_raw(gout, m0.y + cob[cb]);
-                if (m0.z != 0xFFFFFFFFu && con[cb]) r2 = ld_raw(gout, m0.z + cob[cb]);
-                if (fok && con[cb]) rx = ld_raw(in, xoff + chb[cb]);
+                const unsigned r0 = ld_buf(gout_buf, m0.x + cob[cb], TIO()), r1 = ld_buf(gout_buf, m0.y + cob[cb], TIO());
+                const unsigned r2 = ld_buf(gout_buf, m0.z + cob[cb], TIO()), rx = ld_buf(in_buf, xoff + chb[cb], TIO());
                 // (row offsets are multiples of 4 bytes: the half of the word depends on the column only)
                 const float g0 = cvt_raw(r0, cob[cb], TIO()), g1 = cvt_raw(r1, cob[cb], TIO()), g2 = cvt_raw(r2, cob[cb], TIO());
                 sv[cb][i] = fmaf(g2, __uint_as_float(m1.z), fmaf(g1, __uint_as_float(m1.y), g0 * __uint_as_float(m1.x)));

@@ -1026,7 +1026,7 @@ extern "C" int pmesh_f2v_bwd(const float *grad_output, const float *input, const
     PM_REQUIRE(workspace_bytes >= (size_t)G * K * Co * sizeof(float), "f2v_bwd: workspace too small (%zu bytes)", workspace_bytes);
     const int cvec = ((K & 3) == 0 && aligned16(coeff)) ? 1 : 0;
     float *partial = (float *)workspace;
-    if (!force_valu() && (r == 1 || r == 2) && f2v_mfma_ok(Nf, C, r, K, coeff) && NvOut * (int64_t)Co < (int64_t(1) << 30)) {
+    if (!force_valu() && (r == 1 || r == 2) && f2v_mfma_ok(Nf, C, r, K, coeff) && (NvOut + 1) * (int64_t)Co < (int64_t(1) << 30) && Nf < (int64_t(1) << 25)) {
         const int Gm = f2v_bwd_mfma_blocks(Nf);
         PM_REQUIRE(workspace_bytes >= (size_t)Gm * K * Co * sizeof(float), "f2v_bwd: workspace too small (%zu bytes)", workspace_bytes);
         if (int rc = f2v_bwd_mfma(grad_output, input, filter, coeff, face, nf_count, vt_map, grad_input, partial, Gm, Nf, NvOut, C, r, st)) return rc;
@@ -1086,7 +1086,7 @@ extern "C" int pmesh_f2v_bwd_bf16(const uint16_t *grad_output, const uint16_t *i
         return 0;
     }
     PM_REQUIRE(grad_output && input && filter && coeff && face && nf_count && vt_map && grad_input && workspace, "f2v_bwd_bf16: null pointer");
-    PM_REQUIRE((r == 1 || r == 2) && f2v_mfma_ok(Nf, C, r, K, coeff) && NvOut * (int64_t)Co < (int64_t(1) << 30) && !(C & 1) &&
+    PM_REQUIRE((r == 1 || r == 2) && f2v_mfma_ok(Nf, C, r, K, coeff) && (NvOut + 1) * (int64_t)Co < (int64_t(1) << 30) && Nf < (int64_t(1) << 25) && !(C & 1) &&
                    !((reinterpret_cast<uintptr_t>(input) | reinterpret_cast<uintptr_t>(grad_output) | reinterpret_cast<uintptr_t>(grad_input)) & 3u),
                "f2v_bwd_bf16: bf16 features need 16 coefficients in 16-byte aligned rows, an even channel count, at least 32 output channels and depth multiplier 1 or 2 (K=%d C=%d r=%d)", K, C, r);
     const int Gm = f2v_bwd_mfma_blocks(Nf);

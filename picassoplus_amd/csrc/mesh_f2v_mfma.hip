@@ -60,9 +60,12 @@ __device__ __forceinline__ unsigned ld_buf(buffer_t b, unsigned byte_offset, bf1
     return __builtin_amdgcn_raw_buffer_load_b32(b, (int)(byte_offset & ~3u), 0, 0);
 }
 __device__ __forceinline__ float cvt_raw(unsigned w, unsigned, float) { return __builtin_bit_cast(float, w); }
-__device__ __forceinline__ float cvt_raw(unsigned w, unsigned byte_offset, bf16_t)
+// (the half of the word that holds a bf16 value depends on its column only: `half_sel` is computed once per lane and
+// channel block, the conversion is then one byte permutation: the value's two bytes on top of two zero bytes)
+__device__ __forceinline__ unsigned half_sel(unsigned byte_offset) { return (byte_offset & 2u) ? 0x03020C0Cu : 0x01000C0Cu; }
+__device__ __forceinline__ float cvt_raw(unsigned w, unsigned sel, bf16_t)
 {
-    return __builtin_bit_cast(float, (byte_offset & 2u) ? (w & 0xFFFF0000u) : (w << 16));
+    return __builtin_bit_cast(float, __builtin_amdgcn_perm(w, w, sel));
 }
 // Lanes l and l ^ STEP hold neighbouring values p[0], p[1] (the lane with (lane & STEP) == 0 the first): every lane
 // calls this, `ok` says whether the pair is stored.  STEP = 1: neighbouring lanes; 2: lanes two apart.
@@ -106,13 +109,14 @@ __global__ __launch_bounds__(kBlock, (H2 && NCB <= 2 && sizeof(TIO) == 4) ? 4 : 
 
     // B operands: step kk of half h is coefficient 8h + kk (the A operand uses the same assignment)
     float wb[NCB][8];
-    unsigned chb[NCB];
+    unsigned chb[NCB], xsel[NCB];
     bool con[NCB];
 #pragma unroll
     for (int cb = 0; cb < NCB; ++cb) {
         const int co = co0 + 32 * cb + col;
         con[cb] = co < Co;
         chb[cb] = con[cb] ? (unsigned)(co / r) * (unsigned)sizeof(TIO) : 0u;
+        xsel[cb] = half_sel(chb[cb]);
 #pragma unroll
         for (int kk = 0; kk < 8; ++kk) wb[cb][kk] = con[cb] ? filt[(size_t)(8 * h + kk) * Co + co] : 0.f;
     }
@@ -196,7 +200,7 @@ __global__ __launch_bounds__(kBlock, (H2 && NCB <= 2 && sizeof(TIO) == 4) ? 4 : 
 #pragma unroll
             for (int cb = 0; cb < NCB; ++cb)
 #pragma unroll
-                for (int i = 0; i < 16; ++i) x[cb][i] = cvt_raw(xr[cb][i], chb[cb], TIO());
+                for (int i = 0; i < 16; ++i) x[cb][i] = cvt_raw(xr[cb][i], xsel[cb], TIO());
             if constexpr (H2) {
                 float m = 0.f;
 #pragma unroll
@@ -304,7 +308,7 @@ __global__ __launch_bounds__(kBlock, 2) void f2v_bwd_mfma_k(const TIO *__restric
     const buffer_t coeff_buf = buffer_of(coeff, (unsigned)(fend > 0 ? fend : 0) * 64u);
 
     float wb[NCB][8];
-    unsigned chb[NCB], cob[NCB];
+    unsigned chb[NCB], cob[NCB], xsel[NCB], gsel[NCB];
     bool con[NCB];
 #pragma unroll
     for (int cb = 0; cb < NCB; ++cb) {
@@ -312,6 +316,8 @@ __global__ __launch_bounds__(kBlock, 2) void f2v_bwd_mfma_k(const TIO *__restric
         con[cb] = co < Co;
         chb[cb] = con[cb] ? (unsigned)(co / R) * (unsigned)sizeof(TIO) : 0u;
         cob[cb] = con[cb] ? (unsigned)co * (unsigned)sizeof(TIO) : 0u;
+        xsel[cb] = half_sel(chb[cb]);
+        gsel[cb] = half_sel(cob[cb]);
 #pragma unroll
         for (int kk = 0; kk < 8; ++kk) wb[cb][kk] = con[cb] ? filt[(size_t)(8 * h + kk) * Co + co] : 0.f;
     }
@@ -421,9 +427,9 @@ __global__ __launch_bounds__(kBlock, 2) void f2v_bwd_mfma_k(const TIO *__restric
                 const unsigned r0 = ld_buf(gout_buf, m0.x + cob[cb], TIO()), r1 = ld_buf(gout_buf, m0.y + cob[cb], TIO());
                 const unsigned r2 = ld_buf(gout_buf, m0.z + cob[cb], TIO()), rx = ld_buf(in_buf, xoff + chb[cb], TIO());
                 // (row offsets are multiples of 4 bytes: the half of the word depends on the column only)
-                const float g0 = cvt_raw(r0, cob[cb], TIO()), g1 = cvt_raw(r1, cob[cb], TIO()), g2 = cvt_raw(r2, cob[cb], TIO());
+                const float g0 = cvt_raw(r0, gsel[cb], TIO()), g1 = cvt_raw(r1, gsel[cb], TIO()), g2 = cvt_raw(r2, gsel[cb], TIO());
                 sv[cb][i] = fmaf(g2, __uint_as_float(m1.z), fmaf(g1, __uint_as_float(m1.y), g0 * __uint_as_float(m1.x)));
-                xv[cb][i] = cvt_raw(rx, chb[cb], TIO());
+                xv[cb][i] = cvt_raw(rx, xsel[cb], TIO());
             }
         }
         // (H2) the tile's coefficients, in both layouts, under one scale

@@ -12,6 +12,7 @@ routine is ``pmesh_cluster_vertices_host``, kept as the checker and behind ``PME
 contraction is the average pooling op over the new maps; sorting / unique / scans of integer keys between them are
 PyTorch ops.
 """
+import contextlib
 import ctypes
 import os
 import threading
@@ -26,10 +27,11 @@ from ._check import F32, I32, check_input, same_device, stream_of
 from .geometry import combine_clusters_, compute_triangle_geometry_, count_vertex_adjface_  # noqa: F401 (decimate.py:53-93)
 
 
-def vertex_quadrics(vertexIn, faceIn, geometryIn, useArea=True, wgtBnd=5.0):
+def vertex_quadrics(vertexIn, faceIn, geometryIn, useArea=True, wgtBnd=5.0, own_face=False):
     """Quadric (Nv, 10) of every vertex and the candidate edges of the batch.
 
-    returns (quadric, edge_vi, edge_vj): the unique edges (vi < vj, int32) in ascending (vi, vj) order."""
+    returns (quadric, edge_vi, edge_vj): the unique edges (vi < vj, int32) in ascending (vi, vj) order.
+    ``own_face``: the facets are an earlier round's output, their index range is not checked again."""
     check_input(vertexIn, "vertexIn", 2, F32)
     check_input(faceIn, "faceIn", 2, I32)
     check_input(geometryIn, "geometryIn", 2, F32)
@@ -274,7 +276,7 @@ def cluster_vertices_device(edge_vi, edge_vj, perm, sample, nvIn_cumsum, nv2Remo
     return vt_replace
 
 
-def simplify(vertexIn, faceIn, geometryIn, nvIn_cumsum, mfIn_cumsum, nv2Remove, useArea=True, wgtBnd=5.0):
+def simplify(vertexIn, faceIn, geometryIn, nvIn_cumsum, mfIn_cumsum, nv2Remove, useArea=True, wgtBnd=5.0, own_face=False):
     """One decimation round: the reference's ``mesh_decimation.simplify`` (decimate.cpp:21-89,
     decimate_gpu.cu:618-747).  ``nvIn_cumsum`` / ``mfIn_cumsum``: running totals of vertices / facets per sample.
 
@@ -286,7 +288,7 @@ def simplify(vertexIn, faceIn, geometryIn, nvIn_cumsum, mfIn_cumsum, nv2Remove, 
     useArea, wgtBnd = bool(useArea), float(wgtBnd)
     Nv, D = vertexIn.shape
     dev = vertexIn.device
-    quadric, evi, evj = vertex_quadrics(vertexIn, faceIn, geometryIn, useArea, wgtBnd)
+    quadric, evi, evj = vertex_quadrics(vertexIn, faceIn, geometryIn, useArea, wgtBnd, own_face)
     cost = edge_costs(vertexIn, quadric, evi, evj)
     perm, sample = contraction_order(cost, evi, evj, nvIn_cumsum)
     if evi.is_cuda and os.environ.get("PMESH_DECIMATE_HOST_CLUSTERING") != "1":
@@ -324,8 +326,9 @@ def simplify(vertexIn, faceIn, geometryIn, nvIn_cumsum, mfIn_cumsum, nv2Remove, 
         # contracted vertices stay zero (decimate_gpu.cu:401-441): the average pooling op over a map that sends every
         # representative to its own row
         own_row = torch.where(vt_replace >= 0, torch.arange(Nv, dtype=I32, device=dev), torch.full_like(vt_replace, -1))
-        vertex_out = (mesh_pool3d.avg_forward(vertexIn, vt_replace, own_row, torch.empty((Nv, 1), dtype=F32, device=dev))
-                      if Nv else torch.zeros((0, D), dtype=F32, device=dev))
+        with topology.trusted_indices():                  # (maps made by the kernels above)
+            vertex_out = (mesh_pool3d.avg_forward(vertexIn, vt_replace, own_row, torch.empty((Nv, 1), dtype=F32, device=dev))
+                          if Nv else torch.zeros((0, D), dtype=F32, device=dev))
     return [vertex_out, face_out, degenerate, vt_replace, vt_map, nv_out, mf_out]
 
 
@@ -340,11 +343,14 @@ def mesh_decimation_(vertexIn, faceIn, geometryIn, nvIn, mfIn, nvOut, useArea=Tr
     repIn = torch.zeros(vertexIn.shape[0], dtype=I32, device=dev)
     mapIn = torch.arange(vertexIn.shape[0], dtype=I32, device=dev)
     left = int(nv2Remove.max()) if nv2Remove.numel() else 0
+    rounds = 0
     while left > 0:
         nv_cum = torch.cumsum(nvIn, 0, dtype=I32)
         mf_cum = torch.cumsum(mfIn, 0, dtype=I32)
+        # (from the second round on the facets are the round before's output: valid by construction, not checked again)
         vertexOut, faceOut, isDegenerate, repOut, mapOut, nvOut, mfOut = simplify(
-            vertexIn, faceIn, geometryIn, nv_cum, mf_cum, nv2Remove.contiguous(), useArea, wgtBnd)
+            vertexIn, faceIn, geometryIn, nv_cum, mf_cum, nv2Remove.contiguous(), useArea, wgtBnd, own_face=rounds > 0)
+        rounds += 1
         removed = nvIn - nvOut
         still = (nv2Remove - removed).to(I32)
         # what the host needs of this round, in one transfer: did it remove anything, the sizes of the next round's
@@ -354,9 +360,10 @@ def mesh_decimation_(vertexIn, faceIn, geometryIn, nvIn, mfIn, nvOut, useArea=Tr
             break                                     # nothing left that can be contracted (no candidate edges)
         faceIn = _rows_where(faceOut, ~isDegenerate, mf_total)
         vertexIn = _rows_where(vertexOut, mapOut >= 0, nv_total)
-        geometryIn = compute_triangle_geometry_(vertexIn, faceIn)
+        with topology.trusted_indices():
+            geometryIn = compute_triangle_geometry_(vertexIn, faceIn)
+            repIn, mapIn = combine_clusters_(repIn, mapIn, repOut, mapOut)
         nv2Remove = still
-        repIn, mapIn = combine_clusters_(repIn, mapIn, repOut, mapOut)
         nvIn, mfIn = nvOut, mfOut
     return vertexIn, faceIn, geometryIn, nvIn, mfIn, repIn, mapIn
 

@@ -21,6 +21,7 @@ Cache discipline
            a consumer on another stream waits for that event (nothing is waited for once the
            event has completed, and nothing during stream capture, whose warm-up has run the build).
 """
+import contextlib
 import os
 import threading
 import weakref
@@ -136,10 +137,24 @@ def _checks_enabled():
     return os.environ.get("PICASSO_MESH_SKIP_CHECKS", "0") != "1"
 
 
+_TRUST = threading.local()
+
+
+@contextlib.contextmanager
+def trusted_indices():
+    """Inside this block the index tensors handed to the library are its own kernels' outputs (the rounds of a
+    decimation): their range checks -- one reduction and one synchronisation each -- are skipped."""
+    _TRUST.depth = getattr(_TRUST, "depth", 0) + 1
+    try:
+        yield
+    finally:
+        _TRUST.depth -= 1
+
+
 def _check_range(name, t, lo, hi):
     """One-off validation of an index tensor (one reduction and one synchronisation; only on a cache miss,
-    and not at all with PICASSO_MESH_SKIP_CHECKS=1)."""
-    if t.numel() == 0 or not _checks_enabled():
+    and not at all with PICASSO_MESH_SKIP_CHECKS=1 or inside ``trusted_indices``)."""
+    if t.numel() == 0 or not _checks_enabled() or getattr(_TRUST, "depth", 0):
         return
     mn, mx = (int(x) for x in torch.aminmax(t))
     if mn < lo or mx >= hi:

@@ -222,6 +222,36 @@ def test_f2v_parity(cuda, native_options, mesh, C, r, K, strided, path):
     assert_as_good_as_f32(ft.grad, gfilt_ref, gfilt32, "f2v grad_filter")
 
 
+@pytest.mark.parametrize("cscale,fscale", [(1e-12, 1e6), (1e12, 1e-9), (3e-5, 7e4)])
+def test_f2v_coefficients_and_filters_far_from_one(cuda, cscale, fscale):
+    """The two-piece fp16 products bring coefficients and filter columns into fp16's range by powers of two: inputs
+    twelve orders of magnitude above or below one come out to the same 1e-5 (no overflow to infinity, no loss to
+    fp16's subnormal range), and an all-zero coefficient row stays an exact zero."""
+    say("case f2v magnitudes", cscale, fscale)
+    v, f = mesh_case("sphere3")
+    rng = np.random.default_rng(15)
+    nv, nf, C, K = v.shape[0], f.shape[0], 64, 16
+    vt_map = np.arange(nv, dtype=np.int32)
+    nfc = np.maximum(S.vertex_facet_count(f, vt_map, nv), 1)
+    r32 = lambda a: a.astype(np.float32).astype(np.float64)
+    x = r32(rng.uniform(-1, 1, (nf, C)))
+    filt = r32(rng.normal(0, 0.5, (K, C, 1)) * fscale)
+    coeff = r32(rng.normal(0, 0.5, (nf, K)) * cscale)
+    coeff[::7] = 0.0
+    gout = r32(rng.normal(0, 1, (nv, C)))
+    out_ref = loops.f2v_fwd(x, filt, coeff, f, nfc, vt_map)
+    gin_ref, gfilt_ref = loops.f2v_bwd(gout, x, filt, coeff, f, nfc, vt_map)
+    xt = dev(x, cuda, torch.float32).requires_grad_(True)
+    ft = dev(filt, cuda, torch.float32).requires_grad_(True)
+    out = conv3d.facet2vertex(xt, ft, dev(coeff, cuda, torch.float32), dev(f, cuda), dev(nfc, cuda), dev(vt_map, cuda))
+    out.backward(dev(gout, cuda, torch.float32))
+    torch.cuda.synchronize()
+    assert bool(torch.isfinite(out).all()) and bool(torch.isfinite(xt.grad).all()) and bool(torch.isfinite(ft.grad).all())
+    assert_close(out, out_ref, "f2v out, magnitudes far from one")
+    assert_close(xt.grad, gin_ref, "f2v grad_input, magnitudes far from one")
+    assert_close(ft.grad, gfilt_ref, "f2v grad_filter, magnitudes far from one")
+
+
 @pytest.mark.parametrize("path", ["default", "fp32mfma"])
 def test_f2v_channels_of_very_different_size(cuda, native_options, path):
     """Filter columns and feature channels nine orders of magnitude apart: every channel is held to 1e-5 of ITS OWN

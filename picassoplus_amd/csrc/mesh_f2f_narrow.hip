@@ -14,10 +14,9 @@
 //   workgroup  4 wavefronts, summed through LDS into one partial gradient per workgroup
 #include "common.h"
 #include "f2f_internal.h"
+#include "fp16_split.h"
 
 namespace pmesh {
-
-typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 constexpr int kNarrowPairs = 2;     // facet pairs per iteration (more pairs cost registers, i.e. wavefronts in flight)
 constexpr int kNarrowSlots = 5;     // point slots per lane and round (two points per slot and facet: ten points)
@@ -168,10 +167,13 @@ int f2f_bwd_filter_narrow_partials(const float *gout, const float *tex, const fl
 
 
 // ----------------------------------------------------------------------------------------
-// Forward for the same narrow inputs: out[f, co] = sum_(ci,d) G[f,ci,d] * W[co,ci,d] as fp32 MFMAs whose
-// reduction index runs over the (at most) 64 columns (ci, d):
-//   product    out tile (32 facets x 32 output channels) += G (32 facets x 2 columns) . W^T (2 columns x 32),
-//              32 MFMAs per tile; step s, half h <-> column (ci = s/8, d = 8h + s%8)
+// Forward for the same narrow inputs: out[f, co] = sum_(ci,d) G[f,ci,d] * W[co,ci,d] on the fp16 matrix instruction
+// with both operands split into two fp16 pieces (three piece products), the reduction index running over the (at most)
+// 64 columns (ci, d):
+//   product    out tile (32 facets x 32 output channels) += G (32 facets x 16 columns) . W^T (16 columns x 32), one
+//              step per input channel: step c, half h, element q <-> column (ci = c, d = 8h + q).  Every output
+//              channel's weights carry their own power-of-two scale (set once), the G values of a tile one for the
+//              wavefront; both leave the sums on the way out
 //   lane       (facet l%32 of the tile, half h): forms the 32 G values of its half from the facet's points
 //              (32 bytes of each SH row and the point's texture values); as B operand it holds W of output
 //              channel l%32 for the same columns (registers, loaded once)
@@ -187,14 +189,28 @@ __global__ __launch_bounds__(kBlock) void f2f_fwd_narrow_k(const float *__restri
     const int l = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int m = l & 31, h = l >> 5;
     const int n0 = blockIdx.y * (32 * NT);
-    // B operands: wb[nt][s] = W[n0 + 32nt + m][s/8][8h + s%8]
-    float wb[NT][32];
+    // B operands: pieces of beta * W[n0 + 32nt + m][c][8h .. 8h + 7] for the four steps c
+    u32x4 bh[NT][4], bl[NT][4];
+    float inv_beta[NT];
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
         const int co = n0 + 32 * nt + m;
+        float wv[4][8], mx = 0.f;
 #pragma unroll
-        for (int s = 0; s < 32; ++s)
-            wb[nt][s] = (co < Cout && (s >> 3) < Cin) ? W[((int64_t)co * Cin + (s >> 3)) * 16 + 8 * h + (s & 7)] : 0.f;
+        for (int c = 0; c < 4; ++c)
+#pragma unroll
+            for (int q = 0; q < 8; ++q) {
+                wv[c][q] = (co < Cout && c < Cin) ? W[((int64_t)co * Cin + c) * 16 + 8 * h + q] : 0.f;
+                mx = fmaxf(mx, fabsf(wv[c][q]));
+            }
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));                      // the channel's other half of the columns
+        const float beta = pow2_scale(mx, &inv_beta[nt]);
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+#pragma unroll
+            for (int q = 0; q < 8; ++q) wv[c][q] *= beta;
+            split8h(wv[c], bh[nt][c], bl[nt][c]);
+        }
     }
     const int64_t ntiles = (Nf + 31) >> 5;
     const int64_t tbeg = ((int64_t)blockIdx.x * 4 + wave) * tiles_per_wave;
@@ -244,16 +260,40 @@ __global__ __launch_bounds__(kBlock) void f2f_fwd_narrow_k(const float *__restri
                 }
         }
         const float invK = K > 0 ? 1.0f / (float)K : 0.f;
+        float gm = 0.f;
+#pragma unroll
+        for (int c = 0; c < 4; ++c)
+#pragma unroll
+            for (int q = 0; q < 8; ++q) {
+                G[c][q] *= invK;
+                gm = fmaxf(gm, fabsf(G[c][q]));
+            }
+        float inv_alpha;
+        const float alpha = pow2_scale(hwave_fmax(gm), &inv_alpha);      // (every lane of the wavefront is here)
         f32x16 acc[NT];
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
             for (int i = 0; i < 16; ++i) acc[nt][i] = 0.f;
 #pragma unroll
-        for (int s = 0; s < 32; ++s) {
-            const float a = G[s >> 3][s & 7] * invK;
+        for (int c = 0; c < 4; ++c) {
+            float t[8];
 #pragma unroll
-            for (int nt = 0; nt < NT; ++nt) acc[nt] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, wb[nt][s], acc[nt], 0, 0, 0);
+            for (int q = 0; q < 8; ++q) t[q] = G[c][q] * alpha;
+            u32x4 ah, al;
+            split8h(t, ah, al);
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+                acc[nt] = mfma_f16(al, bh[nt][c], acc[nt]);
+                acc[nt] = mfma_f16(ah, bl[nt][c], acc[nt]);
+                acc[nt] = mfma_f16(ah, bh[nt][c], acc[nt]);
+            }
+        }
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+            const float unscale = inv_alpha * inv_beta[nt];
+#pragma unroll
+            for (int i = 0; i < 16; ++i) acc[nt][i] *= unscale;
         }
         // accumulator: lane (co = n0 + 32nt + m, half h), register i <-> facet 8(i/4) + 4h + i%4 of the tile
 #pragma unroll

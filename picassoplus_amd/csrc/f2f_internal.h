@@ -62,6 +62,7 @@ int f2f16x3_bwd_filter_partials(const void *gout, const void *tex, const float *
 // gradients of Cout*Cin*16 floats are left in `partial` (blocks = f2f_narrow_blocks(Nf) <= kNarrowMaxBlocks).
 constexpr int kNarrowMaxBlocks = 2048;
 bool f2f_narrow_usable(int Cin, int F);
+bool f2f_narrow_bwd_usable(int Cin, int F, int64_t Nf, int Cout);
 int f2f_narrow_blocks(int64_t Nf);
 int f2f_bwd_filter_narrow_partials(const float *gout, const float *tex, const float *sh, const int *cum, float *partial,
                                    int blocks, int64_t T, int64_t Nf, int Cin, int Cout, hipStream_t st);

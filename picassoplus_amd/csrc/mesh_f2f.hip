@@ -421,13 +421,15 @@ static size_t f2f_bwd_ws(int64_t slices, int Cin, int Cout, int F)
 
 extern "C" size_t pmesh_f2f_bwd_workspace_bytes(int Cin, int Cout, int F)
 {
-    return f2f_bwd_ws(f2f_narrow_usable(Cin, F) ? kNarrowMaxBlocks : kFiltMaxSplits, Cin, Cout, F);
+    // (a narrow shape too large for the narrow kernel's 32-bit offsets takes the general kernels: room for either)
+    return f2f_bwd_ws(f2f_narrow_usable(Cin, F) && kNarrowMaxBlocks > kFiltMaxSplits ? kNarrowMaxBlocks : kFiltMaxSplits, Cin, Cout, F);
 }
 
 extern "C" size_t pmesh_f2f_bwd_workspace_bytes_for(int64_t Nf, int Cin, int Cout, int F)
 {
     if (Nf < 0) Nf = 0;
-    return f2f_bwd_ws(f2f_narrow_usable(Cin, F) ? f2f_narrow_blocks(Nf) : filt_splits(Nf), Cin, Cout, F);
+    const int general = filt_splits(Nf), narrow = f2f_narrow_usable(Cin, F) ? f2f_narrow_blocks(Nf) : 0;
+    return f2f_bwd_ws(narrow > general ? narrow : general, Cin, Cout, F);
 }
 
 extern "C" int pmesh_f2f_bwd_texture(const float *grad_output, const float *filter, const float *bary_coeff,
@@ -475,7 +477,7 @@ extern "C" int pmesh_f2f_bwd_filter(const float *grad_output, const float *textu
         return 0;
     }
     PM_REQUIRE(grad_output && texture && bary_coeff && cum_texture && workspace, "f2f_bwd_filter: null pointer");
-    if (!force_generic() && f2f_narrow_usable(Cin, F) && !(reinterpret_cast<uintptr_t>(bary_coeff) & 15u)) {
+    if (!force_generic() && f2f_narrow_bwd_usable(Cin, F, Nf, Cout) && !(reinterpret_cast<uintptr_t>(bary_coeff) & 15u)) {
         const int nb = f2f_narrow_blocks(Nf);
         PM_REQUIRE(workspace_bytes >= (size_t)nb * nW * sizeof(float), "f2f_bwd_filter: workspace too small (%zu bytes)",
                    workspace_bytes);

@@ -1,145 +1,14 @@
-// facet2facet filter gradient for narrow inputs (at most four input channels, 16 SH coefficients) -- the
-// colour input of a network's first block.  gW[co][ci][d] = sum_f gout[f,co] * G[f,ci,d] with
-// G[f,ci,d] = (1/K_f) sum_k tex[k,ci] * sh[k,d] has only Cin * 16 <= 64 columns per facet, so the
-// kernel is a stream over gout, the SH rows and the texture rows:
-//   product    gW^T (columns (ci,d) x 32 output channels) += G^T (columns x 2 facets) . gout (2 x 32), fp32
-//              MFMAs whose reduction index is the facet: the two halves of a wavefront hold the two facets
-//              of a pair
-//   lane       (m, half): point parity m/16, input channel (m/4)%4, d-group m%4.  It loads 16 bytes of an
-//              SH row and one texture value per point and keeps four G values (d = 4*(m%4) + c, c = 0..3)
-//              summed over the points of its parity; component c is the A operand of MFMA c, so rows m and
-//              m + 16 of each product are two partial sums of one column, added at the end
-//   wavefront  a contiguous run of facets in natural order (all reads are sequential), two pairs per
-//              iteration with the loads of all of them in flight together; segment bounds one iteration ahead
-//   workgroup  4 wavefronts, summed through LDS into one partial gradient per workgroup
+// facet2facet for narrow inputs (at most four input channels, 16 SH coefficients) -- the colour input of a network's
+// first block: G[f,ci,d] = (1/K_f) sum_k tex[k,ci] * sh[k,d] has only Cin * 16 <= 64 columns per facet, so both kernels
+// are streams over the SH rows, the texture rows and gout / out, with the products on the fp16 matrix instruction.
 #include "common.h"
 #include "f2f_internal.h"
 #include "fp16_split.h"
 
 namespace pmesh {
 
-constexpr int kNarrowPairs = 2;     // facet pairs per iteration (more pairs cost registers, i.e. wavefronts in flight)
-constexpr int kNarrowSlots = 5;     // point slots per lane and round (two points per slot and facet: ten points)
-
-template <int NT>
-__global__ __launch_bounds__(kBlock) void f2f_bwd_filt_narrow_k(const float *__restrict__ gout, const float *__restrict__ tex,
-                                                                const float *__restrict__ sh, const int *__restrict__ cum,
-                                                                float *__restrict__ partial, int64_t Nf, int T, int Cin,
-                                                                int Cout, int64_t facets_per_wave)
-{
-    __shared__ float red[4][8][64];
-    const int l = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int m = l & 31, h = l >> 5, par = m >> 4, ci = (m >> 2) & 3, dg = m & 3;
-    const int n0 = blockIdx.y * (32 * NT);
-    const bool c_on = ci < Cin;
-    const int64_t fbeg = ((int64_t)blockIdx.x * 4 + wave) * facets_per_wave;
-    const int64_t fend = (fbeg + facets_per_wave < Nf) ? fbeg + facets_per_wave : Nf;
-
-    f32x16 acc[4][NT];
-#pragma unroll
-    for (int c = 0; c < 4; ++c)
-#pragma unroll
-        for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) acc[c][nt][i] = 0.f;
-
-    // segment [k0, k1) of texture points of the facets f0 + 2p + h
-    auto bounds = [&](int64_t f0, int (&k0)[kNarrowPairs], int (&k1)[kNarrowPairs]) {
-#pragma unroll
-        for (int p = 0; p < kNarrowPairs; ++p) {
-            const int64_t f = f0 + 2 * p + h;
-            int a = 0, b = 0;
-            if (f < fend) {
-                a = f ? cum[f - 1] : 0;
-                b = cum[f];
-            }
-            a = a < 0 ? 0 : (a > T ? T : a);
-            b = b < a ? a : (b > T ? T : b);
-            k0[p] = a; k1[p] = b;
-        }
-    };
-
-    int k0[kNarrowPairs], k1[kNarrowPairs];
-    bounds(fbeg, k0, k1);
-    for (int64_t f0 = fbeg; f0 < fend; f0 += 2 * kNarrowPairs) {
-        int nk0[kNarrowPairs], nk1[kNarrowPairs];
-        bounds(f0 + 2 * kNarrowPairs, nk0, nk1);
-
-        float g[kNarrowPairs][NT], G4[kNarrowPairs][4];
-        int kmax = 0;
-#pragma unroll
-        for (int p = 0; p < kNarrowPairs; ++p) {
-            const int64_t f = f0 + 2 * p + h;
-#pragma unroll
-            for (int nt = 0; nt < NT; ++nt) {
-                const int co = n0 + 32 * nt + m;
-                g[p][nt] = (f < fend && co < Cout) ? gout[f * Cout + co] : 0.f;
-            }
-#pragma unroll
-            for (int c = 0; c < 4; ++c) G4[p][c] = 0.f;
-            kmax = (k1[p] - k0[p] > kmax) ? k1[p] - k0[p] : kmax;
-        }
-        // rounds of 2 * kNarrowSlots points per facet, all facets of the iteration in one batch of loads
-        for (int kb = 0; kb == 0 || __builtin_amdgcn_ballot_w64(kb < kmax) != 0ull; kb += 2 * kNarrowSlots) {
-            float4 sv[kNarrowPairs][kNarrowSlots];
-            float tv[kNarrowPairs][kNarrowSlots];
-#pragma unroll
-            for (int p = 0; p < kNarrowPairs; ++p)
-#pragma unroll
-                for (int u = 0; u < kNarrowSlots; ++u) {
-                    const int k = kb + 2 * u + par;
-                    const bool on = k < k1[p] - k0[p];
-                    const int64_t pt = k0[p] + k;
-                    sv[p][u] = on ? *reinterpret_cast<const float4 *>(sh + pt * 16 + 4 * dg) : make_float4(0.f, 0.f, 0.f, 0.f);
-                    tv[p][u] = (on && c_on) ? tex[pt * Cin + ci] : 0.f;
-                }
-#pragma unroll
-            for (int p = 0; p < kNarrowPairs; ++p)
-#pragma unroll
-                for (int u = 0; u < kNarrowSlots; ++u) {
-                    G4[p][0] = fmaf(tv[p][u], sv[p][u].x, G4[p][0]);
-                    G4[p][1] = fmaf(tv[p][u], sv[p][u].y, G4[p][1]);
-                    G4[p][2] = fmaf(tv[p][u], sv[p][u].z, G4[p][2]);
-                    G4[p][3] = fmaf(tv[p][u], sv[p][u].w, G4[p][3]);
-                }
-        }
-#pragma unroll
-        for (int p = 0; p < kNarrowPairs; ++p) {
-            const int K = k1[p] - k0[p];
-            const float invK = K > 0 ? 1.0f / (float)K : 0.f;
-#pragma unroll
-            for (int c = 0; c < 4; ++c)
-#pragma unroll
-                for (int nt = 0; nt < NT; ++nt)
-                    acc[c][nt] = __builtin_amdgcn_mfma_f32_32x32x2f32(G4[p][c] * invK, g[p][nt], acc[c][nt], 0, 0, 0);
-        }
-#pragma unroll
-        for (int p = 0; p < kNarrowPairs; ++p) { k0[p] = nk0[p]; k1[p] = nk1[p]; }
-    }
-
-    // accumulator (c, nt): lane (co = n0 + 32nt + m, half h), register i <-> row 8(i/4) + 4h + i%4; rows r and
-    // r + 16 (registers i and i + 8) are the two point parities of column (ci = r/4, d = 4*(r%4) + c)
-    float *dst = partial + (size_t)blockIdx.x * Cout * Cin * 16;
-#pragma unroll
-    for (int c = 0; c < 4; ++c)
-#pragma unroll
-        for (int nt = 0; nt < NT; ++nt) {
-            __syncthreads();
-#pragma unroll
-            for (int i = 0; i < 8; ++i) red[wave][i][l] = acc[c][nt][i] + acc[c][nt][i + 8];
-            __syncthreads();
-            for (int idx = threadIdx.x; idx < 8 * 64; idx += kBlock) {
-                const int ll = idx & 63, i = idx >> 6;
-                const int row = 8 * (i >> 2) + 4 * (ll >> 5) + (i & 3);
-                const int cc = row >> 2, dd = 4 * (row & 3) + c, co = n0 + 32 * nt + (ll & 31);
-                const float v = (red[0][i][ll] + red[1][i][ll]) + (red[2][i][ll] + red[3][i][ll]);
-                if (cc < Cin && co < Cout) dst[((size_t)co * Cin + cc) * 16 + dd] = v;
-            }
-        }
-}
-
-// The same gradient with the facet as the reduction index of the fp16 matrix instruction (16 facets per step instead of
-// two), both operands split into two fp16 pieces:
+// Filter gradient gW[co][ci][d] = sum_f gout[f,co] * G[f,ci,d] with the facet as the reduction index of the fp16 matrix
+// instruction (16 facets per step), both operands split into two fp16 pieces:
 //   wavefront  a contiguous run of 32-facet tiles.  Lane (facet m, half h) forms the 32 G values of its facet and half
 //              (columns (ci = c, d = 8h + q), as the forward does: 32 bytes of each SH row, the point's texture
 //              values, five points in flight), scaled by one power of two for the tile, into the wavefront's LDS
@@ -338,6 +207,8 @@ __global__ __launch_bounds__(kBlock) void f2f_bwd_filt_narrow_h2_k(const float *
 }
 
 bool f2f_narrow_usable(int Cin, int F) { return F == 16 && Cin <= 4; }       // plus 16-byte aligned SH rows, checked by the caller
+// the filter gradient addresses gout with 32-bit byte offsets (and one that marks a lane without a channel)
+bool f2f_narrow_bwd_usable(int Cin, int F, int64_t Nf, int Cout) { return f2f_narrow_usable(Cin, F) && Nf * (int64_t)Cout < (int64_t(1) << 29); }
 
 // Workgroup count: a function of the facet count only (fixed summation order on any device).
 int f2f_narrow_blocks(int64_t Nf)
@@ -355,21 +226,11 @@ int f2f_bwd_filter_narrow_partials(const float *gout, const float *tex, const fl
     const int64_t gy = ceil_div(Cout, 32 * nt);
     PM_REQUIRE(gy <= 65535, "f2f_bwd_filter: grid too large");
     const dim3 grid((unsigned)blocks, (unsigned)gy);
-    if (!(reinterpret_cast<uintptr_t>(sh) & 15u) && Nf * (int64_t)Cout < (int64_t(1) << 29) && !options().f2f_generic) {
-        // (32-bit byte offsets into gout, with room for the offset that marks a lane without a channel)
-        const int64_t tpw = ceil_div(ceil_div(Nf, 32), (int64_t)blocks * 4);
-        if (nt == 1)
-            f2f_bwd_filt_narrow_h2_k<1><<<grid, dim3(kBlock), 0, st>>>(gout, tex, sh, cum, partial, Nf, (int)T, Cin, Cout, tpw);
-        else
-            f2f_bwd_filt_narrow_h2_k<2><<<grid, dim3(kBlock), 0, st>>>(gout, tex, sh, cum, partial, Nf, (int)T, Cin, Cout, tpw);
-        PM_LAUNCHED("f2f_bwd_filter(narrow, fp16 pieces)");
-        return 0;
-    }
-    const int64_t fpw = ceil_div(ceil_div(Nf, (int64_t)blocks * 4), 2 * kNarrowPairs) * (2 * kNarrowPairs);
+    const int64_t tpw = ceil_div(ceil_div(Nf, 32), (int64_t)blocks * 4);
     if (nt == 1)
-        f2f_bwd_filt_narrow_k<1><<<grid, dim3(kBlock), 0, st>>>(gout, tex, sh, cum, partial, Nf, (int)T, Cin, Cout, fpw);
+        f2f_bwd_filt_narrow_h2_k<1><<<grid, dim3(kBlock), 0, st>>>(gout, tex, sh, cum, partial, Nf, (int)T, Cin, Cout, tpw);
     else
-        f2f_bwd_filt_narrow_k<2><<<grid, dim3(kBlock), 0, st>>>(gout, tex, sh, cum, partial, Nf, (int)T, Cin, Cout, fpw);
+        f2f_bwd_filt_narrow_h2_k<2><<<grid, dim3(kBlock), 0, st>>>(gout, tex, sh, cum, partial, Nf, (int)T, Cin, Cout, tpw);
     PM_LAUNCHED("f2f_bwd_filter(narrow)");
     return 0;
 }

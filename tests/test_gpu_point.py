@@ -350,6 +350,59 @@ def test_dual_block_graph_and_module(cuda):
     assert tuple(y.shape) == (len(xyz), 8) and bool(torch.isfinite(y).all())
 
 
+def test_point_block_step_replays_from_a_hip_graph(cuda):
+    """Forward and backward of the point branch of a dual block (fuzzy convolution with its tail, max pooling to a
+    sampled set, interpolation back; the graphs built beforehand) recorded once as a HIP graph: every replay equals the
+    eager step on the inputs then in the static buffers, with eager steps between the replays."""
+    say("case point graph replay")
+    xyz, nv = cloud(61, [900, 500], scale=1.0)
+    L, radius, C = 3, 0.2, 32
+    X, NV = dev(xyz, cuda), dev(nv, cuda)
+    nn_cnt, nn_idx, _, filt_idx, filt_coeff = point_utils.build_sphere_harmonics(X, X, NV, NV, radius, L=L, nn_uplimit=16)
+    NQ = dev((nv // 4).astype(np.int32), cuda)
+    picked = sample.fps_(X, NV, NQ)
+    Q = X[picked.long()].contiguous()
+    _, pcnt, pidx, _ = nnquery.range_search_(X, Q, NV, NQ, radius=2 * radius, nnsample=32)
+    nn3, d3 = nnquery.knn3_search_(Q, X, NQ, NV)
+    w3 = point_utils.compute_unpool_weight(d3)
+    torch.manual_seed(5)
+    conv = point_layers.PCloudConv3d(C, C, (L + 1) ** 2 + 1, with_bn=False).to(cuda)
+    params = list(conv.parameters())
+    static_x = torch.randn(len(xyz), C, device=cuda, requires_grad=True)
+    static_g = torch.randn(len(xyz), C, device=cuda)
+
+    def step(x, g):
+        y = conv(x, nn_cnt, nn_idx, filt_idx, filt_coeff)
+        p = pool3d.maxPool(y, pcnt, pidx)
+        z = y + unpool3d.interpolate(p, w3, nn3)
+        return [z] + list(torch.autograd.grad(z, [x] + params, g))
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            step(static_x, static_g)                            # warm-up: the pair orders are cached now
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        static_out = step(static_x, static_g)
+    for i in range(3):
+        gen = torch.Generator(device=cuda).manual_seed(300 + i)
+        x = torch.randn(len(xyz), C, device=cuda, generator=gen)
+        g = torch.randn(len(xyz), C, device=cuda, generator=gen)
+        with torch.no_grad():
+            static_x.copy_(x)
+            static_g.copy_(g)
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [t.clone() for t in static_out]
+        eager = step(x.requires_grad_(True), g)
+        torch.cuda.synchronize()
+        for k, (a, b) in enumerate(zip(got, eager)):
+            assert torch.equal(a, b), "replay %d: result %d differs from the eager step" % (i, k)
+
+
 def test_point_argument_errors(cuda):
     say("case point errors")
     db, nvd = cloud(61, [50])

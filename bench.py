@@ -37,7 +37,7 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="scene", choices=["scene", "shapes", "pool", "firstblock", "tail", "hierarchy", "texture", "pcloud", "decimate"],
+    ap.add_argument("--workload", default="scene", choices=["scene", "shapes", "pool", "firstblock", "tail", "f2vtail", "hierarchy", "texture", "pcloud", "decimate"],
                     help="scene: the headline layer (F2F+F2V, C=64); shapes: 16 small meshes V2F+F2F+F2V; pool: "
                          "1024x1024 grid max/avg pool + unpool; firstblock: the scene batch with the reference's first "
                          "block shapes, F2F 3->32 then F2V 32->32 with depth multiplier 2 (pi2_blocks.py:113-130)")
@@ -551,6 +551,62 @@ def run_tail(args, torch):
                             out_channels=Co))
 
 
+def run_f2vtail(args, torch):
+    """The forward of an F2VConv3d module on the scene batch (64 channels, degree 3, 64 outputs, ReLU): the
+    convolution and its pointwise tail as the two native passes (facet2vertex, then the product) and as the one pass
+    that multiplies the vertex rows before they leave the chip, each without and with what a backward pass needs
+    kept (the convolution's rows and the ReLU mask bits)."""
+    from picassoplus_amd import _lib, synthetic as S
+    from picassoplus_amd.mesh.pi_modules import dense, mesh_conv3d
+    dev = torch.device("cuda:0")
+    C, Co = 64, 64
+    d = build_conv_inputs(S.scene_workload(scale=args.scale), C, 3, 3100, tex_counts=1)
+    rng = np.random.default_rng(3101)
+    T = lambda a, dt=None: torch.from_numpy(np.ascontiguousarray(a)).to(dev if dt is None else dev, dtype=dt)
+    face, nfc, vmap = T(d["face"], torch.int32), T(d["nf_count"], torch.int32), T(d["vt_map"], torch.int32)
+    xf = T(rng.uniform(-1, 1, (d["nf"], C)).astype(np.float32))
+    coeff = T(rng.normal(0, 0.5, (d["nf"], 16)).astype(np.float32))
+    filt = T(d["w_f2v"])
+    w = T((rng.normal(0, 1, (C, Co)) / 8).astype(np.float32))
+    b = T(rng.normal(0, 0.3, Co).astype(np.float32))
+    variants = {
+        "two_passes": lambda: dense.dense_tail_forward(mesh_conv3d.facet2vertex_forward(xf, filt, coeff, face, nfc, vmap), w, b, True),
+        "one_pass": lambda: dense.f2v_dense_forward(xf, filt, coeff, face, nfc, vmap, w, b, True),
+        "two_passes_kept": lambda: dense.dense_tail_forward(mesh_conv3d.facet2vertex_forward(xf, filt, coeff, face, nfc, vmap), w, b, True, with_bits=True),
+        "one_pass_kept": lambda: dense.f2v_dense_forward(xf, filt, coeff, face, nfc, vmap, w, b, True, with_bits=True, keep_rows=True),
+    }
+    res, ops = {}, {}
+    for name, fn in variants.items():
+        for _ in range(args.warmup):
+            fn()
+        torch.cuda.synchronize()
+        timer = EventTimer(torch)
+        timer.on = True
+        _lib.set_call_hook(timer)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(args.steps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        _lib.set_call_hook(None)
+        res[name] = e0.elapsed_time(e1) / args.steps
+        ops[name] = {k: round(v, 4) for k, v in timer.summary().items() if k.startswith(("f2v", "dense"))}
+    Nv, Nf = d["nv"], d["nf"]
+    # one pass, nothing kept: facet rows, coefficients, adjacency in; the module's output rows out
+    nb = 4 * Nf * C + 4 * Nf * 16 + 12 * Nf + 8 * Nv + 4 * Nv * Co
+    ms = res["one_pass"]
+    ach = nb / (ms * 1e-3) / 1e9
+    return dict(value=Nv / (ms * 1e-3) / 1e6, unit="Mvertices/s", ms_per_step=ms, variants_ms={k: round(v, 4) for k, v in res.items()},
+                native_calls_ms=ops,
+                dtype="f32 in HBM; both products on the fp16 matrix instructions with operands split into two fp16 pieces "
+                      "(three piece products), f32 accumulate",
+                roofline=dict(bound="hbm", achieved=ach, peak=HBM_PEAK_GBS, unit="GB/s", frac=ach / HBM_PEAK_GBS, traffic=None,
+                              kernel="f2v_dense_fwd", kernel_ms=ops["one_pass"].get("f2v_dense_fwd", ms)),
+                config=dict(workload="scene8x300k_F2VConv3d_forward_C64_L3_64out_relu_fp32", facets=Nf, vertices=Nv,
+                            channels=C, out_channels=Co, algorithmic_bytes=nb))
+
+
 def run_texture(args, torch):
     """Texture points of the scene batch's facets interpolated from 64-channel vertex features, with the SH basis of
     their barycentric coordinates (forward), and the transposed gather (backward)."""
@@ -1009,6 +1065,8 @@ def main():
         res = run_pool(args, torch)
     elif args.workload == "tail":
         res = run_tail(args, torch)
+    elif args.workload == "f2vtail":
+        res = run_f2vtail(args, torch)
     elif args.workload == "hierarchy":
         res = run_hierarchy(args, torch)
     elif args.workload == "texture":

@@ -453,6 +453,24 @@ int pmesh_v2f_dense_fwd(const float *input, const float *filter, const int32_t *
                         uint32_t *relu_bits, float *conv_rows, int64_t Nv, int64_t Nf, int C, int Co,
                         pmesh_stream_t stream);
 
+/* facet2vertex and its tail as ONE pass: replaces mesh_conv3d.facet2vertex_forward (mesh_conv3d.cpp:258-291,
+ * kernel mesh_conv3d_gpu.cu:299-330) followed by the PyTorch ops of F2VConv3d.forward
+ * (picasso/mesh/layers.py:163-174):
+ *   output (NvOut,Co) = act(facet2vertex(input, filter, coeff) (NvOut,C*r) . weight (C*r,Co) + bias) * scale + shift
+ * A wavefront keeps the vertex rows of four passes of the convolution kernel in LDS and multiplies the 16 rows by the
+ * weights on the matrix cores before they leave; conv_rows (NvOut,C*r), when given, also receives them for the
+ * backward pass (pmesh_dense_bwd takes them as its `input`, pmesh_f2v_bwd the gradient that comes out of it).
+ * Supported (pmesh_f2v_dense_supported returns 1): K == 16 with 16-byte aligned coeff rows, C*r == 32 or 64,
+ * Co == 32, 64 or 128; other shapes run pmesh_f2v_fwd and pmesh_dense_fwd.  rowptr / colidx as in pmesh_f2v_fwd;
+ * bias, scale, shift, relu, relu_bits as in pmesh_dense_fwd; workspace (16-byte aligned): the packed weights. */
+int pmesh_f2v_dense_supported(int64_t Nf, int C, int r, int K, int Co, const float *coeff);
+size_t pmesh_f2v_dense_fwd_workspace_bytes(int C, int r, int Co);
+int pmesh_f2v_dense_fwd(const float *input, const float *filter, const float *coeff, const int32_t *nf_count,
+                        const int32_t *rowptr, const int32_t *colidx, const float *weight, const float *bias,
+                        const float *scale, const float *shift, int relu, float *output, uint32_t *relu_bits,
+                        float *conv_rows, void *workspace, size_t workspace_bytes, int64_t Nf, int64_t NvOut, int C,
+                        int r, int K, int Co, pmesh_stream_t stream);
+
 /* The same tail for a convolution that mixes the channels itself (F2FConv3d, picasso/mesh/layers.py:60-64:
  * outputs + biases, activation_fn, BatchNorm): output (N,C) = act(input + bias) * scale + shift, one pass;
  * output may be input.  relu_bits as in pmesh_dense_fwd (NULL, or N * C/32 words when C % 32 == 0 and the rows

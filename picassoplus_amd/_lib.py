@@ -11,7 +11,7 @@ from ctypes import c_char_p, c_float, c_int, c_int64, c_size_t, c_void_p
 _HERE = os.path.dirname(os.path.abspath(__file__))
 # PICASSO_MESH_LIB points at an alternative build of the same ABI (kernel experiments)
 LIB_PATH = os.environ.get("PICASSO_MESH_LIB") or os.path.join(_HERE, "csrc", "libpicasso_mesh.so")
-ABI_VERSION = 19
+ABI_VERSION = 20
 
 P, I, L, Z = c_void_p, c_int, c_int64, c_size_t
 
@@ -105,6 +105,9 @@ SIGNATURES = {
     "pmesh_cluster_attach": (I, [P, P, P, P, L, P, P, P, P]),
     "pmesh_dense_fwd": (I, [P, P, P, P, P, I, P, P, L, I, I, P]),
     "pmesh_v2f_dense_fwd": (I, [P, P, P, P, P, P, P, I, P, P, P, L, L, I, I, P]),
+    "pmesh_f2v_dense_supported": (I, [L, I, I, I, I, P]),
+    "pmesh_f2v_dense_fwd_workspace_bytes": (Z, [I, I, I]),
+    "pmesh_f2v_dense_fwd": (I, [P, P, P, P, P, P, P, P, P, P, I, P, P, P, P, Z, L, L, I, I, I, I, P]),
     "pmesh_dense_bwd_workspace_bytes": (Z, [L, I, I]),
     "pmesh_dense_bwd": (I, [P, P, P, P, P, P, P, P, P, Z, L, I, I, P]),
     "pmesh_bias_act_fwd": (I, [P, P, P, P, I, P, P, L, I, P]),

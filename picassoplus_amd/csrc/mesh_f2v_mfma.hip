@@ -10,6 +10,7 @@
 //     register i of lane (col, h)  <->  vertex i/4 of the four, entry slot 4h + i%4 of its eight.
 // One cross-half exchange per vertex pair and channel block finishes the sum.
 // Against the vector-ALU version this replaces 64 FMAs per entry and four channels by 1/4 of an MFMA.
+#include <type_traits>
 #include "common.h"
 #include "fp16_split.h"
 #include "rows_internal.h"
@@ -259,6 +260,305 @@ __global__ __launch_bounds__(kBlock, (H2 && NCB <= 2 && sizeof(TIO) == 4) ? 4 : 
         e0 = ne0; e1 = ne1; ne0 = me0; ne1 = me1;
         f = nf;
     }
+}
+
+
+// ----------------------------------------------------------------------------------------
+// Forward with the pointwise tail of the convolution module on its store (picasso/mesh/layers.py:163-174 runs
+// the tail as a matmul with depth_weights, + biases, the activation and batch norm after the native op):
+//     out2[v, n] = max(sum_c conv[v, c] * Wd[c, n] + bias[n], floor) * scale[n] + shift[n]
+// The kernel above is kept as it is; a wavefront additionally parks the four vertex rows of every pass over its
+// groups in a private LDS tile and, every four passes, multiplies the 16 rows by the weights: two-piece fp16
+// products on v_mfma_f32_16x16x32_f16 (three piece products per 16 x 16 x 32 block), the rows under one power-of-two
+// scale per tile, every weight column under its own (taken out again with the bias).  The weights sit in LDS in
+// operand layout, packed once per call by f2v_tail_pack_k:
+//     Wp[((s * NTD + nt) * 2 + piece) * 64 + lane] = pieces of beta_n * Wd[32 s + 8 (lane / 16) .. + 7][16 nt + lane % 16]
+//     meta[4 n .. 4 n + 3] = 1 / beta_n, bias_n, scale_n, shift_n
+// A / B operand of the instruction: lane l holds row / column l % 16, reduction indices 8 (l / 16) .. + 7;
+// result: lane l holds column l % 16, rows 4 (l / 16) .. + 3.  NCB = 32-channel blocks of the convolution's
+// rows (its Co = 32 NCB is the product's reduction length), NTD = 16-column tiles of the tail's output.
+typedef float f32x4v __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ f32x4v mfma16_f16(const u32x4 &a, const u32x4 &b, const f32x4v &c)
+{
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+}
+
+__global__ __launch_bounds__(kBlock) void f2v_tail_pack_k(const float *__restrict__ Wd, const float *__restrict__ bias,
+                                                          const float *__restrict__ scale, const float *__restrict__ shift,
+                                                          u32x4 *__restrict__ Wp, float *__restrict__ meta, int Kc, int Cd,
+                                                          int NS, int NTD)
+{
+    const int idx = blockIdx.x * kBlock + threadIdx.x;
+    if (idx >= NS * NTD * 64) return;
+    const int lane = idx & 63, nt = (idx >> 6) % NTD, s = (idx >> 6) / NTD;
+    const int n = 16 * nt + (lane & 15), kg = lane >> 4;
+    float m = 0.f;
+    for (int k = 0; k < Kc; ++k) m = fmaxf(m, fabsf(Wd[(size_t)k * Cd + n]));
+    float inv;
+    const float beta = pow2_scale(m, &inv);
+    float t[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const int k = 32 * s + 8 * kg + j;
+        t[j] = k < Kc ? Wd[(size_t)k * Cd + n] * beta : 0.f;
+    }
+    u32x4 hi, lo;
+    split8h(t, hi, lo);
+    Wp[((size_t)(s * NTD + nt) * 2 + 0) * 64 + lane] = hi;
+    Wp[((size_t)(s * NTD + nt) * 2 + 1) * 64 + lane] = lo;
+    if (s == 0 && kg == 0) {
+        meta[4 * n] = inv;
+        meta[4 * n + 1] = bias ? bias[n] : 0.f;
+        meta[4 * n + 2] = scale ? scale[n] : 1.f;
+        meta[4 * n + 3] = shift ? shift[n] : 0.f;
+    }
+}
+
+constexpr int kTailPad = 4;         // floats between staged rows: 16-byte reads of 16 rows spread over the banks
+
+#ifndef PM_TAIL_OCC
+#define PM_TAIL_OCC 4
+#endif
+template <int NCB, int NTD>
+__global__ __launch_bounds__(kBlock, NTD <= 4 ? PM_TAIL_OCC : 2) void f2v_fwd_tail_k(const float *__restrict__ in, const float *__restrict__ filt,
+                                                         const float *__restrict__ coeff,
+                                                         const int *__restrict__ nfcount,
+                                                         const int *__restrict__ rowptr,
+                                                         const int *__restrict__ colidx, float *__restrict__ conv_out,
+                                                         const u32x4 *__restrict__ Wp, const float *__restrict__ meta,
+                                                         float *__restrict__ out2, unsigned *__restrict__ bits, int relu,
+                                                         int64_t NvOut, int C, int r, unsigned in_bytes)
+{
+    constexpr int Co = 32 * NCB, Cd = 16 * NTD, kRow = Co + kTailPad;
+    __shared__ u32x4 s_W[NCB * NTD * 2 * 64];
+    __shared__ __attribute__((aligned(16))) float s_meta[4 * Cd];
+    __shared__ __attribute__((aligned(16))) float s_stage[kBlock / 64][16 * kRow];
+    const int l = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int col = l & 31, h = l >> 5, j = col >> 3, s = col & 7;
+    const buffer_t in_buf = buffer_of(in, in_bytes);
+    const unsigned row_bytes = (unsigned)C * 4u;
+
+    for (int i = threadIdx.x; i < NCB * NTD * 2 * 64; i += kBlock) s_W[i] = Wp[i];
+    for (int i = threadIdx.x; i < 4 * Cd; i += kBlock) s_meta[i] = meta[i];
+
+    float wb[NCB][8];
+    unsigned chb[NCB];
+#pragma unroll
+    for (int cb = 0; cb < NCB; ++cb) {
+        const int co = 32 * cb + col;
+        chb[cb] = (unsigned)(co / r) * 4u;
+#pragma unroll
+        for (int kk = 0; kk < 8; ++kk) wb[cb][kk] = filt[(size_t)(8 * h + kk) * Co + co];
+    }
+    u32x4 bh[NCB], bl[NCB];
+    float inv_beta[NCB];
+#pragma unroll
+    for (int cb = 0; cb < NCB; ++cb) {
+        float m = 0.f;
+#pragma unroll
+        for (int kk = 0; kk < 8; ++kk) m = fmaxf(m, fabsf(wb[cb][kk]));
+        m = fmaxf(m, __shfl_xor(m, 32, 64));
+        const float beta = pow2_scale(m, &inv_beta[cb]);
+        float t[8];
+#pragma unroll
+        for (int kk = 0; kk < 8; ++kk) t[kk] = wb[cb][kk] * beta;
+        split8h(t, bh[cb], bl[cb]);
+    }
+    __syncthreads();
+
+    const int64_t groups = (NvOut + 3) >> 2, gx = (groups + 7) >> 3;
+    const int xcd = blockIdx.x & 7;
+    const int64_t gstride = (int64_t)(gridDim.x >> 3) * 4;
+    const int64_t gend = ((xcd + 1) * gx < groups) ? (xcd + 1) * gx : groups;
+    int64_t g = xcd * gx + (int64_t)(blockIdx.x >> 3) * 4 + wave;
+    float *stage = s_stage[wave];
+    const float floor_v = relu ? 0.f : -__builtin_inff();
+
+    // the tile's rows (cnt passes of four vertices, the last one at group g_last) times the weights, and the store.
+    // FULL: four passes, every vertex of them inside the array -- no condition on a row.
+    auto flush = [&](auto full_tag, int64_t g_last, int cnt) {
+        constexpr bool FULL = decltype(full_tag)::value;
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        const int r16 = l & 15, kg = l >> 4;
+        const bool rvalid = FULL || (r16 >> 2) < cnt;          // rows of passes that did not happen hold old values
+        float a[NCB][8];
+        float m = 0.f;
+#pragma unroll
+        for (int ks = 0; ks < NCB; ++ks) {
+            const float4 *sp = reinterpret_cast<const float4 *>(stage + r16 * kRow + 32 * ks + 8 * kg);
+            const float4 u = sp[0], v = sp[1];
+            a[ks][0] = rvalid ? u.x : 0.f; a[ks][1] = rvalid ? u.y : 0.f; a[ks][2] = rvalid ? u.z : 0.f; a[ks][3] = rvalid ? u.w : 0.f;
+            a[ks][4] = rvalid ? v.x : 0.f; a[ks][5] = rvalid ? v.y : 0.f; a[ks][6] = rvalid ? v.z : 0.f; a[ks][7] = rvalid ? v.w : 0.f;
+#pragma unroll
+            for (int q = 0; q < 8; ++q) m = fmaxf(m, fabsf(a[ks][q]));
+        }
+        float inv_alpha;
+        const float alpha = pow2_scale(hwave_fmax(m), &inv_alpha);
+        u32x4 ah[NCB], al[NCB];
+#pragma unroll
+        for (int ks = 0; ks < NCB; ++ks) {
+#pragma unroll
+            for (int q = 0; q < 8; ++q) a[ks][q] *= alpha;
+            split8h(a[ks], ah[ks], al[ks]);
+        }
+        // my four rows of the result: pass kg of the tile, vertices 4 g_kg .. + 3
+        const int64_t v0 = 4 * (g_last - (int64_t)((FULL ? 4 : cnt) - 1 - kg) * gstride);
+        const bool qok = FULL || kg < cnt;
+        float *orow = out2 + v0 * Cd + r16;
+        unsigned mine = 0u;                                     // the mask word of row r16 / 2, columns 32 (r16 % 2) .. + 31
+#pragma unroll
+        for (int np = 0; np < NTD / 2; ++np) {
+            f32x4v d[2];
+            float4 mt[2];
+#pragma unroll
+            for (int e = 0; e < 2; ++e) {
+                const int nt = 2 * np + e;
+                d[e] = f32x4v{0.f, 0.f, 0.f, 0.f};
+                mt[e] = reinterpret_cast<const float4 *>(s_meta)[16 * nt + r16];
+            }
+#pragma unroll
+            for (int ks = 0; ks < NCB; ++ks)
+#pragma unroll
+                for (int e = 0; e < 2; ++e) {
+                    const u32x4 *wp = s_W + ((ks * NTD + 2 * np + e) * 2) * 64 + l;
+                    const u32x4 wh = wp[0], wl = wp[64];
+                    d[e] = mfma16_f16(al[ks], wh, d[e]);
+                    d[e] = mfma16_f16(ah[ks], wl, d[e]);
+                    d[e] = mfma16_f16(ah[ks], wh, d[e]);
+                }
+            unsigned long long pos[2][4];
+#pragma unroll
+            for (int e = 0; e < 2; ++e) {
+                const float us = inv_alpha * mt[e].x;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const float v = fmaxf(fmaf(d[e][i], us, mt[e].y), floor_v);
+                    const bool ok = FULL || (qok && v0 + i < NvOut);
+                    if (ok) orow[(int64_t)i * Cd + 16 * (2 * np + e)] = fmaf(v, mt[e].z, mt[e].w);
+                    pos[e][i] = __builtin_amdgcn_ballot_w64(ok && v > 0.f);
+                }
+            }
+            if (bits) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const unsigned word = (unsigned)((pos[0][i] >> (16 * kg)) & 0xFFFFull) |
+                                          ((unsigned)((pos[1][i] >> (16 * kg)) & 0xFFFFull) << 16);
+                    mine = (r16 == (NTD / 2) * i + np) ? word : mine;
+                }
+            }
+        }
+        // lanes 0 .. 2 NTD - 1 of a group of 16 hold the words of its four rows, in the order they lie in memory
+        if (bits && r16 < 2 * NTD) {
+            const int i = r16 / (NTD / 2);
+            if (FULL || (qok && v0 + i < NvOut)) bits[v0 * (Cd / 32) + r16] = mine;
+        }
+        // (the next pass writes the tile again: its reads above are complete, the values sit in registers)
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+    };
+
+    auto bounds = [&](int64_t gg, int &a, int &b) {
+        a = 0; b = 0;
+        const int64_t v = 4 * gg + j;
+        if (gg < gend && v < NvOut) { a = rowptr[v]; b = rowptr[v + 1]; }
+    };
+    int e0, e1, ne0, ne1;
+    bounds(g, e0, e1);
+    bounds(g + gstride, ne0, ne1);
+    int f = (e0 + s < e1) ? colidx[e0 + s] / 3 : -1;
+    int q4 = 0;                                                 // passes parked in the tile
+
+    for (; g < gend; g += gstride) {
+        int me0, me1;
+        bounds(g + 2 * gstride, me0, me1);
+        const int nf = (ne0 + s < ne1) ? colidx[ne0 + s] / 3 : -1;
+        const int64_t vs = 4 * g + 2 * h;
+        const int cnt0 = (vs < NvOut) ? nfcount[vs] : 1, cnt1 = (vs + 1 < NvOut) ? nfcount[vs + 1] : 1;
+        const unsigned long long has = __builtin_amdgcn_ballot_w64(e1 > e0);
+
+        float acc[NCB][4];
+#pragma unroll
+        for (int cb = 0; cb < NCB; ++cb)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) acc[cb][q] = 0.f;
+
+        for (int p = 0;; ++p) {
+            if (p > 0) f = (e0 + 8 * p + s < e1) ? colidx[e0 + 8 * p + s] / 3 : -1;
+            float a[8];
+            {
+                float4 t0 = make_float4(0.f, 0.f, 0.f, 0.f), t1 = t0;
+                if (f >= 0) {
+                    const float4 *cp = reinterpret_cast<const float4 *>(coeff + (int64_t)f * 16 + 8 * h);
+                    t0 = cp[0]; t1 = cp[1];
+                }
+                a[0] = t0.x; a[1] = t0.y; a[2] = t0.z; a[3] = t0.w;
+                a[4] = t1.x; a[5] = t1.y; a[6] = t1.z; a[7] = t1.w;
+            }
+            const unsigned boff = (f >= 0) ? (unsigned)f * row_bytes : in_bytes;
+            unsigned b[16];
+#pragma unroll
+            for (int i = 0; i < 16; ++i)
+                b[i] = (unsigned)__builtin_amdgcn_ds_bpermute((8 * (i >> 2) + 4 * h + (i & 3)) * 4, (int)boff);
+            unsigned xr[NCB][16];
+#pragma unroll
+            for (int cb = 0; cb < NCB; ++cb)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) xr[cb][i] = ld_buf(in_buf, b[i] + chb[cb], float());
+            float m = 0.f;
+#pragma unroll
+            for (int kk = 0; kk < 8; ++kk) m = fmaxf(m, fabsf(a[kk]));
+            float inv_alpha;
+            const float alpha = pow2_scale(hwave_fmax(m), &inv_alpha);
+#pragma unroll
+            for (int kk = 0; kk < 8; ++kk) a[kk] *= alpha;
+            u32x4 ah, al;
+            split8h(a, ah, al);
+#pragma unroll
+            for (int cb = 0; cb < NCB; ++cb) {
+                const float unscale = inv_alpha * inv_beta[cb];
+                f32x16 d;
+#pragma unroll
+                for (int i = 0; i < 16; ++i) d[i] = 0.f;
+                d = mfma_f16(al, bh[cb], d);
+                d = mfma_f16(ah, bl[cb], d);
+                d = mfma_f16(ah, bh[cb], d);
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    float t = 0.f;
+#pragma unroll
+                    for (int i = 4 * q; i < 4 * q + 4; ++i) t = fmaf(d[i], __builtin_bit_cast(float, xr[cb][i]), t);
+                    acc[cb][q] = fmaf(t, unscale, acc[cb][q]);
+                }
+            }
+            if (!__builtin_amdgcn_ballot_w64(e0 + 8 * (p + 1) < e1)) break;
+        }
+
+        const float inv0 = ((has >> (8 * (2 * h))) & 1ull) ? 1.0f / (float)cnt0 : 0.f;
+        const float inv1 = ((has >> (8 * (2 * h + 1))) & 1ull) ? 1.0f / (float)cnt1 : 0.f;
+#pragma unroll
+        for (int cb = 0; cb < NCB; ++cb) {
+            half_swap(acc[cb][0], acc[cb][2]);
+            half_swap(acc[cb][1], acc[cb][3]);
+            const float o0 = (acc[cb][0] + acc[cb][2]) * inv0, o1 = (acc[cb][1] + acc[cb][3]) * inv1;
+            const int co = 32 * cb + col;
+            if (conv_out) {
+                if (vs < NvOut) conv_out[vs * Co + co] = o0;
+                if (vs + 1 < NvOut) conv_out[(vs + 1) * Co + co] = o1;
+            }
+            stage[(4 * q4 + 2 * h) * kRow + co] = o0;
+            stage[(4 * q4 + 2 * h + 1) * kRow + co] = o1;
+        }
+        if (++q4 == 4) {
+            if (4 * g + 3 < NvOut) flush(std::true_type(), g, 4);
+            else flush(std::false_type(), g, 4);
+            q4 = 0;
+        }
+        e0 = ne0; e1 = ne1; ne0 = me0; ne1 = me1;
+        f = nf;
+    }
+    if (q4) flush(std::false_type(), g - gstride, q4);
 }
 
 
@@ -568,6 +868,40 @@ int f2v_fwd_mfma(const void *in, const float *filt, const float *coeff, const in
     if (bf16) f2v_fwd_launch((const bf16_t *)in, filt, coeff, nfcount, rowptr, colidx, (bf16_t *)out, Nf, NvOut, C, r, st);
     else f2v_fwd_launch((const float *)in, filt, coeff, nfcount, rowptr, colidx, (float *)out, Nf, NvOut, C, r, st);
     PM_LAUNCHED("f2v_fwd(mfma)");
+    return 0;
+}
+
+
+bool f2v_tail_ok(int64_t Nf, int C, int r, int K, const void *coeff, int Cd)
+{
+    const int Co = C * r;
+    return f2v_mfma_ok(Nf, C, r, K, coeff) && (Co == 32 || Co == 64) && (Cd == 32 || Cd == 64 || Cd == 128);
+}
+
+size_t f2v_tail_workspace_bytes(int Co, int Cd) { return (size_t)(Co / 32) * (Cd / 16) * 2 * 64 * sizeof(u32x4) + (size_t)4 * Cd * sizeof(float); }
+
+int f2v_fwd_tail(const float *in, const float *filt, const float *coeff, const int *nfcount, const int *rowptr,
+                 const int *colidx, float *conv_out, const float *Wd, const float *bias, const float *scale, const float *shift,
+                 int relu, float *out2, unsigned *bits, void *workspace, int64_t Nf, int64_t NvOut, int C, int r, int Cd,
+                 hipStream_t st)
+{
+    const int Co = C * r, ncb = Co / 32, ntd = Cd / 16;
+    u32x4 *Wp = (u32x4 *)workspace;
+    float *meta = (float *)(Wp + (size_t)ncb * ntd * 2 * 64);
+    f2v_tail_pack_k<<<dim3((unsigned)ceil_div(ncb * ntd * 64, kBlock)), dim3(kBlock), 0, st>>>(Wd, bias, scale, shift, Wp, meta, Co, Cd, ncb, ntd);
+    PM_LAUNCHED("f2v_dense_fwd(pack)");
+    const unsigned in_bytes = (unsigned)(Nf * C * (int64_t)sizeof(float));
+    const int64_t want = ceil_div(ceil_div(NvOut, 16), 8) * 8;
+    const unsigned gxn = (unsigned)(want < 4096 ? want : 4096);
+    const dim3 grid(gxn), block(kBlock);
+#define PM_F2V_TAIL(N, T) f2v_fwd_tail_k<N, T><<<grid, block, 0, st>>>(in, filt, coeff, nfcount, rowptr, colidx, conv_out, Wp, meta, out2, bits, relu, NvOut, C, r, in_bytes)
+    if (ncb == 1) {
+        if (ntd == 2) PM_F2V_TAIL(1, 2); else if (ntd == 4) PM_F2V_TAIL(1, 4); else PM_F2V_TAIL(1, 8);
+    } else {
+        if (ntd == 2) PM_F2V_TAIL(2, 2); else if (ntd == 4) PM_F2V_TAIL(2, 4); else PM_F2V_TAIL(2, 8);
+    }
+#undef PM_F2V_TAIL
+    PM_LAUNCHED("f2v_dense_fwd");
     return 0;
 }
 

@@ -996,6 +996,40 @@ extern "C" int pmesh_f2v_fwd(const float *input, const float *filter, const floa
     return 0;
 }
 
+extern "C" int pmesh_f2v_dense_supported(int64_t Nf, int C, int r, int K, int Co, const float *coeff)
+{
+    return (!force_valu() && !options().f2v_fp32mfma && f2v_tail_ok(Nf, C, r, K, coeff, Co)) ? 1 : 0;
+}
+
+extern "C" size_t pmesh_f2v_dense_fwd_workspace_bytes(int C, int r, int Co)
+{
+    if (C <= 0 || r <= 0 || Co <= 0) return 256;
+    return f2v_tail_workspace_bytes(((C * r + 31) / 32) * 32, ((Co + 15) / 16) * 16) + 256;
+}
+
+extern "C" int pmesh_f2v_dense_fwd(const float *input, const float *filter, const float *coeff,
+                                   const int32_t *nf_count, const int32_t *rowptr, const int32_t *colidx,
+                                   const float *weight, const float *bias, const float *scale, const float *shift,
+                                   int relu, float *output, uint32_t *relu_bits, float *conv_rows, void *workspace,
+                                   size_t workspace_bytes, int64_t Nf, int64_t NvOut, int C, int r, int K, int Co,
+                                   pmesh_stream_t stream)
+{
+    clear_error();
+    PM_DIMS("f2v_dense_fwd");
+    PM_REQUIRE(Nf >= 0 && NvOut >= 0, "f2v_dense_fwd: negative size");
+    if (NvOut == 0) return 0;
+    PM_REQUIRE(input && filter && coeff && nf_count && rowptr && colidx && weight && output && workspace,
+               "f2v_dense_fwd: null pointer");
+    PM_REQUIRE(NvOut <= INT32_MAX && Nf <= INT32_MAX / 3, "f2v_dense_fwd: sizes exceed int32 indexing");
+    PM_REQUIRE(pmesh_f2v_dense_supported(Nf, C, r, K, Co, coeff),
+               "f2v_dense_fwd: takes 16 coefficients in 16-byte aligned rows, 32 or 64 convolution channels and 32, 64 or 128 "
+               "output channels (K=%d C=%d r=%d Co=%d)", K, C, r, Co);
+    PM_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 15u) == 0 && workspace_bytes >= f2v_tail_workspace_bytes(C * r, Co),
+               "f2v_dense_fwd: workspace too small or misaligned (%zu bytes)", workspace_bytes);
+    return f2v_fwd_tail(input, filter, coeff, nf_count, rowptr, colidx, conv_rows, weight, bias, scale, shift, relu, output,
+                        relu_bits, workspace, Nf, NvOut, C, r, Co, (hipStream_t)stream);
+}
+
 extern "C" size_t pmesh_f2v_bwd_workspace_bytes(int C, int r, int K) { return (size_t)1024 * K * C * r * sizeof(float); }
 
 extern "C" int pmesh_f2v_bwd(const float *grad_output, const float *input, const float *filter,

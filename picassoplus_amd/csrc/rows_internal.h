@@ -16,6 +16,17 @@ bool f2v_mfma_ok(int64_t Nf, int C, int r, int K, const void *coeff);
 int f2v_fwd_mfma(const void *in, const float *filt, const float *coeff, const int *nfcount, const int *rowptr,
                  const int *colidx, void *out, int64_t Nf, int64_t NvOut, int C, int r, hipStream_t st, bool bf16 = false);
 
+// facet2vertex with the module's pointwise tail on its store (float rows, 32 or 64 convolution channels C * r,
+// 32 / 64 / 128 tail outputs Cd, the conditions of f2v_mfma_ok): out2 = max(conv . Wd + bias, 0 or -inf) * scale + shift;
+// conv_out (may be null) also receives the convolution's rows, bits (may be null) the mask of positive activations;
+// workspace: f2v_tail_workspace_bytes, 16-byte aligned.
+bool f2v_tail_ok(int64_t Nf, int C, int r, int K, const void *coeff, int Cd);
+size_t f2v_tail_workspace_bytes(int Co, int Cd);
+int f2v_fwd_tail(const float *in, const float *filt, const float *coeff, const int *nfcount, const int *rowptr,
+                 const int *colidx, float *conv_out, const float *Wd, const float *bias, const float *scale, const float *shift,
+                 int relu, float *out2, unsigned *bits, void *workspace, int64_t Nf, int64_t NvOut, int C, int r, int Cd,
+                 hipStream_t st);
+
 // Backward on the matrix cores: depth multiplier 1 or 2, additionally NvOut * C * r * 4 < 2^32.  G workgroups
 // (f2v_bwd_mfma_blocks) leave G partial filter gradients of 16 * C * r floats in `partial`.
 int f2v_bwd_mfma_blocks(int64_t Nf);

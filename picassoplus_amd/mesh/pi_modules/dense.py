@@ -191,6 +191,91 @@ def v2f_dense(input, filter, face, weight, bias, relu=True):
     return V2FDenseFunction.apply(input, filter, face, weight, bias, relu)
 
 
+# ---------------------------------------------------------------- facet2vertex and its tail in one pass
+def f2v_dense_supported(input, filter, coeff, weight):
+    """The one-pass form takes float32 rows, 16 coefficients per facet (degree 3), 32 or 64 convolution channels
+    and 32, 64 or 128 output channels; the library decides (its product switches are part of the answer)."""
+    if input.dtype != F32 or input.dim() != 2 or filter.dim() != 3 or coeff.dim() != 2 or weight.dim() != 2:
+        return False
+    K, C, r = filter.shape
+    if input.shape[1] != C or coeff.shape[1] != K or weight.shape[0] != C * r:
+        return False
+    return bool(_lib.query("pmesh_f2v_dense_supported", input.shape[0], C, r, K, weight.shape[1], coeff.data_ptr()))
+
+
+def f2v_dense_forward(input, filter, coeff, face, nf_count, vt_map, weight, bias=None, relu=True, scale=None, shift=None,
+                      with_bits=False, keep_rows=False):
+    """act(facet2vertex(input, filter, coeff, face, nf_count, vt_map) @ weight + bias) * scale + shift in one kernel: a
+    wavefront multiplies the vertex rows of the convolution by the weights before they leave the chip.
+    input (NfIn,C), filter (K,C,r), coeff (NfIn,K), weight (C*r,Co) -> (NvOut,Co).  ``keep_rows`` also returns the
+    convolution's rows (NvOut,C*r), which the backward pass needs; ``with_bits`` the ReLU mask as bits.
+    Returns out, or (out, bits, rows) when either is asked for."""
+    from .. import topology
+    from . import mesh_conv3d
+    Nf, C, K, r, NvOut, NvIn = mesh_conv3d._f2v_dims(input, filter, coeff, face, nf_count, vt_map)
+    check_input(weight, "weight", 2, F32)
+    Co = weight.shape[1]
+    if weight.shape[0] != C * r:
+        raise RuntimeError("weight must have shape (in_channels * multiplier, out_channels)")
+    for name, t in (("bias", bias), ("scale", scale), ("shift", shift)):
+        if t is not None:
+            check_input(t, name, 1, F32)
+            if t.shape[0] != Co:
+                raise RuntimeError("%s must have out_channels entries" % name)
+    if not f2v_dense_supported(input, filter, coeff, weight):
+        raise RuntimeError("the one-pass facet2vertex tail takes 16 coefficients, 32 or 64 convolution channels and "
+                           "32, 64 or 128 output channels (got K=%d, C*r=%d, Co=%d)" % (K, C * r, Co))
+    dev = same_device(input, filter, coeff, face, nf_count, vt_map, weight, *[t for t in (bias, scale, shift) if t is not None])
+    rowptr, colidx = topology.vertex_csr(face, vt_map, NvOut)
+    with torch.cuda.device(dev):
+        out = torch.empty((NvOut, Co), dtype=F32, device=dev)
+        bits = torch.empty((NvOut, Co // 32), dtype=torch.int32, device=dev) if with_bits else None
+        rows = torch.empty((NvOut, C * r), dtype=F32, device=dev) if keep_rows else None
+        nbytes = _lib.query("pmesh_f2v_dense_fwd_workspace_bytes", C, r, Co)
+        ws = workspace(nbytes, dev)
+        _lib.call("pmesh_f2v_dense_fwd", input.data_ptr(), filter.data_ptr(), coeff.data_ptr(), nf_count.data_ptr(),
+                  rowptr.data_ptr(), colidx.data_ptr(), weight.data_ptr(), _ptr(bias), _ptr(scale), _ptr(shift),
+                  1 if relu else 0, out.data_ptr(), _ptr(bits), _ptr(rows), ws.data_ptr(), nbytes, Nf, NvOut, C, r, K, Co,
+                  stream_of(input))
+    return (out, bits, rows) if (with_bits or keep_rows) else out
+
+
+class F2VDenseFunction(torch.autograd.Function):
+    """facet2vertex, the product with the pointwise weights, the bias and a ReLU (or no activation) as ONE native
+    forward (picasso/mesh/layers.py:163-171 runs them as a native op and three PyTorch ops).  The convolution's rows
+    are kept only when a gradient will need them.  Backward: the tail's gradients from the kept rows, then the
+    convolution's from what the tail hands down."""
+
+    @staticmethod
+    def forward(ctx, input, filter, coeff, face, nf_count, vt_map, weight, bias, relu):
+        for t in (coeff, face, nf_count, vt_map):
+            if t.requires_grad:
+                t.requires_grad = False
+        need = any(ctx.needs_input_grad[i] for i in (0, 1, 6, 7))
+        res = f2v_dense_forward(input, filter, coeff, face, nf_count, vt_map, weight, bias, relu,
+                                with_bits=bool(relu and need), keep_rows=need)
+        out, bits, rows = res if need else (res, None, None)
+        ctx.save_for_backward(input, filter, coeff, face, nf_count, vt_map, weight, bits, rows)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        from . import mesh_conv3d
+        input, filter, coeff, face, nf_count, vt_map, weight, bits, rows = ctx.saved_tensors
+        need_conv = ctx.needs_input_grad[0] or ctx.needs_input_grad[1]
+        grows, gw, gb = dense_tail_backward(grad_output.contiguous(), rows, weight, None, need_input=need_conv, relu_bits=bits)
+        gin = gfilt = None
+        if need_conv:
+            gin, gfilt = mesh_conv3d.facet2vertex_backward(grows, input, filter, coeff, face, nf_count, vt_map)
+        return (gin if ctx.needs_input_grad[0] else None, gfilt if ctx.needs_input_grad[1] else None, None, None, None, None,
+                gw if ctx.needs_input_grad[6] else None, gb if ctx.needs_input_grad[7] else None, None)
+
+
+def f2v_dense(input, filter, coeff, face, nf_count, vt_map, weight, bias, relu=True):
+    """act(facet2vertex(...) @ weight + bias) with gradients for input, filter, weight and bias."""
+    return F2VDenseFunction.apply(input, filter, coeff, face, nf_count, vt_map, weight, bias, relu)
+
+
 # ---------------------------------------------------------------- the tail without a product
 def bits_supported(C, *tensors):
     """The bit form of the ReLU mask of ``bias_act`` needs whole 32-column words and 16-byte aligned rows."""

@@ -350,3 +350,149 @@ def test_v2f_dense_empty_and_refused_shapes(cuda):
         dense.v2f_dense_forward(x, filt, torch.tensor([[0, 1, 10]], dtype=torch.int32, device=cuda), w)
     with pytest.raises(RuntimeError):
         dense.v2f_dense_forward(x.cpu(), filt, face, w)
+
+
+F2V_DENSE_SHAPES = [("sphere2", 32, 1, 32, False), ("sphere3", 64, 1, 64, True), ("room_small", 64, 1, 64, False),
+                    ("fans", 64, 1, 128, False), ("torus", 32, 2, 64, True), ("sphere3", 32, 1, 128, False),
+                    ("tetra", 64, 1, 32, False), ("shapes_small", 16, 2, 32, True), ("octa", 64, 1, 64, True)]
+
+
+@pytest.mark.parametrize("mesh,c,r,co,strided", F2V_DENSE_SHAPES)
+@pytest.mark.parametrize("relu", [True, False])
+def test_f2v_dense_one_pass(cuda, mesh, c, r, co, strided, relu):
+    """facet2vertex + pointwise product + bias + ReLU as one kernel against the float64 oracle composition (oracle:
+    f2v_fwd, then dense_tail_fwd): forward with and without the kept rows / mask bits / frozen norm, every gradient
+    through autograd against the oracle's explicit backward formulas.  Vertex counts that are no multiple of 16 end
+    on a partly filled tile; ``strided`` leaves output vertices without facets (their convolution rows are zero, their
+    outputs the activated bias)."""
+    from oracle import loops
+    from picassoplus_amd import synthetic as S
+    from util import dev, mesh_case, strided_vt_map
+    say("case f2v_dense", mesh, c, r, co, strided, relu)
+    v, f = mesh_case(mesh)
+    nv, nf, K = v.shape[0], f.shape[0], 16
+    rng = np.random.default_rng(c * 1000 + co + r)
+    if strided:
+        vt_map, nvo = strided_vt_map(rng, nv)
+    else:
+        vt_map, nvo = np.arange(nv, dtype=np.int32), nv
+    nfc = np.maximum(S.vertex_facet_count(f, vt_map, nvo), 1)
+    x = rng.uniform(-1, 1, (nf, c)).astype(np.float32)
+    filt = rng.normal(0, 0.5, (K, c, r)).astype(np.float32)
+    coeff = rng.normal(0, 0.5, (nf, K)).astype(np.float32)
+    w = (rng.normal(0, 1, (c * r, co)) / np.sqrt(c * r)).astype(np.float32)
+    b = rng.normal(0, 0.3, co).astype(np.float32)
+    g = rng.normal(0, 1, (nvo, co)).astype(np.float32)
+    xd, fd, cd, wd, bd, gd, face, nfd, vmd = (dev(a, cuda) for a in (x, filt, coeff, w, b, g, f, nfc, vt_map))
+    f64 = np.float64
+    rows64 = loops.f2v_fwd(x.astype(f64), filt.astype(f64), coeff.astype(f64), f, nfc, vt_map)
+    T = lambda a: torch.from_numpy(np.ascontiguousarray(a, np.float64))
+    ref = torch_ref.dense_tail_fwd(T(rows64), T(w), T(b), relu).numpy()
+    assert dense.f2v_dense_supported(xd, fd, cd, wd)
+    out = dense.f2v_dense_forward(xd, fd, cd, face, nfd, vmd, wd, bd, relu)
+    out2, bits, rows = dense.f2v_dense_forward(xd, fd, cd, face, nfd, vmd, wd, bd, relu, with_bits=True, keep_rows=True)
+    torch.cuda.synchronize()
+    assert_close(out, ref, "f2v_dense forward")
+    assert torch.equal(out, out2)
+    assert_close(rows, rows64, "f2v_dense kept rows")
+    # the kept rows are the rows of the convolution kernel, bit for bit
+    from picassoplus_amd.mesh.pi_modules import mesh_conv3d
+    conv = mesh_conv3d.facet2vertex_forward(xd, fd, cd, face, nfd, vmd)
+    assert torch.equal(rows, conv)
+    cols = torch.arange(co, device=cuda)
+    if relu:
+        assert torch.equal(((bits[:, cols // 32] >> (cols % 32)) & 1).bool(), out > 0)
+    f32 = np.float32
+    rows32 = loops.f2v_fwd(x, filt, coeff, f, nfc, vt_map, dtype=f32)
+    z32 = rows32 @ w + b
+    from util import assert_as_good_as_f32
+    assert_as_good_as_f32(out, ref, np.maximum(z32, 0) if relu else z32, "f2v_dense forward")
+    scale, shift = dev(rng.uniform(0.5, 2, co).astype(np.float32), cuda), dev(rng.normal(0, 1, co).astype(np.float32), cuda)
+    outn = dense.f2v_dense_forward(xd, fd, cd, face, nfd, vmd, wd, bd, relu, scale, shift)
+    assert_close(outn, ref * scale.double().cpu().numpy() + shift.double().cpu().numpy(), "f2v_dense with scale/shift")
+    nob = dense.f2v_dense_forward(xd, fd, cd, face, nfd, vmd, wd, None, relu)
+    assert_close(nob, torch_ref.dense_tail_fwd(T(rows64), T(w), T(np.zeros(co)), relu).numpy(), "f2v_dense without a bias")
+    # gradients
+    xg, fg, wg, bg = (t.clone().requires_grad_(True) for t in (xd, fd, wd, bd))
+    y = dense.f2v_dense(xg, fg, cd, face, nfd, vmd, wg, bg, relu)
+    assert torch.equal(y.detach(), out)
+    y.backward(gd)
+    torch.cuda.synchronize()
+    z = rows64 @ w.astype(np.float64) + b
+    safe = (np.abs(z) > 1e-5 * np.abs(z).max()) | (not relu)
+    out64 = np.where(safe, ref, out.double().cpu().numpy())
+    grows, gw, gb = torch_ref.dense_tail_bwd(T(g), T(rows64), T(w), T(out64) if relu else None)
+    gx, gf = loops.f2v_bwd(grows.numpy(), x.astype(f64), filt.astype(f64), coeff.astype(f64), f, nfc, vt_map)
+    assert_close(xg.grad, gx, "f2v_dense grad_input")
+    assert_close(fg.grad, gf, "f2v_dense grad_filter")
+    assert_close(wg.grad, gw.numpy(), "f2v_dense grad_weight")
+    assert_close(bg.grad, gb.numpy(), "f2v_dense grad_bias")
+    with torch.no_grad():
+        assert torch.equal(dense.f2v_dense(xd, fd, cd, face, nfd, vmd, wd, bd, relu), out)
+
+
+def test_f2v_module_takes_the_one_pass_form(cuda, native_options):
+    """Without gradients to record, F2VConv3d calls one native forward where the reference runs the convolution and
+    three PyTorch ops; a training step, shapes the one-pass kernel does not take (other channel counts or degrees) and
+    the vector-ALU switch keep the separate passes."""
+    from picassoplus_amd import _lib
+    from picassoplus_amd import synthetic as S
+    from util import dev, mesh_case
+    native_options(PMESH_F2V_VALU="0", PMESH_F2V_FP32MFMA="0")
+    v, f = mesh_case("sphere2")
+    nv, nf = v.shape[0], f.shape[0]
+    vt_map = np.arange(nv, dtype=np.int32)
+    nfc = np.maximum(S.vertex_facet_count(f, vt_map, nv), 1)
+    face, nfd, vmd = dev(f, cuda), dev(nfc, cuda), dev(vt_map, cuda)
+    x = torch.randn(nf, 64, device=cuda)
+    coeff = torch.randn(nf, 16, device=cuda)
+    calls = []
+    _lib.set_call_hook(lambda name, phase: calls.append(name) if phase == "begin" else None)
+    try:
+        mod = layers.F2VConv3d(64, 64, 3, with_bn=True).to(cuda).eval()
+        with torch.no_grad():
+            y_one = mod(x, face, nfd, vmd, coeff)
+        one = list(calls)
+        del calls[:]
+        y_train = mod(x, face, nfd, vmd, coeff)                 # parameters require gradients: the two passes
+        train = list(calls)
+        del calls[:]
+        with torch.no_grad():
+            layers.F2VConv3d(64, 48, 3, with_bn=False).to(cuda)(x, face, nfd, vmd, coeff)
+        two = list(calls)
+        del calls[:]
+        native_options(PMESH_F2V_VALU="1")
+        with torch.no_grad():
+            layers.F2VConv3d(64, 64, 3, with_bn=False).to(cuda)(x, face, nfd, vmd, coeff)
+        valu = list(calls)
+    finally:
+        _lib.set_call_hook(None)
+    assert "pmesh_f2v_dense_fwd" in one and "pmesh_f2v_fwd" not in one and "pmesh_dense_fwd" not in one, one
+    assert "pmesh_f2v_fwd" in train and "pmesh_dense_fwd" in train and "pmesh_f2v_dense_fwd" not in train, train
+    assert "pmesh_f2v_fwd" in two and "pmesh_dense_fwd" in two, two
+    assert "pmesh_f2v_fwd" in valu and "pmesh_dense_fwd" in valu, valu
+    # both forms of the same module agree to the parity bar
+    assert_close(y_one, y_train.detach().double().cpu().numpy(), "F2VConv3d one pass against two", 2e-6)
+
+
+def test_f2v_dense_refused_shapes(cuda):
+    """Shapes outside the one-pass kernel's range are refused by the op (the module does not send them there) and no
+    output vertices give an empty result."""
+    from util import dev
+    f = np.array([[0, 1, 2], [0, 2, 3]], np.int32)
+    face, nfd, vmd = dev(f, cuda), dev(np.array([2, 1, 2, 1], np.int32), cuda), dev(np.arange(4, dtype=np.int32), cuda)
+    x, filt, coeff = torch.randn(2, 64, device=cuda), torch.randn(16, 64, 1, device=cuda), torch.randn(2, 16, device=cuda)
+    assert dense.f2v_dense_forward(x, filt, coeff, face, nfd, vmd, torch.randn(64, 64, device=cuda)).shape == (4, 64)
+    assert not dense.f2v_dense_supported(x, filt, coeff, torch.randn(64, 48, device=cuda))
+    with pytest.raises(RuntimeError):
+        dense.f2v_dense_forward(x, filt, coeff, face, nfd, vmd, torch.randn(64, 48, device=cuda))
+    with pytest.raises(RuntimeError):
+        dense.f2v_dense_forward(x[:, :24].contiguous(), filt[:, :24].contiguous(), coeff, face, nfd, vmd, torch.randn(24, 64, device=cuda))
+    with pytest.raises(RuntimeError):
+        dense.f2v_dense_forward(x, torch.randn(9, 64, 1, device=cuda), coeff[:, :9].contiguous(), face, nfd, vmd,
+                                torch.randn(64, 64, device=cuda))
+    none = torch.zeros((0,), dtype=torch.int32, device=cuda)
+    nowhere = torch.full((4,), -1, dtype=torch.int32, device=cuda)
+    out, bits, rows = dense.f2v_dense_forward(x, filt, coeff, face, none, nowhere, torch.randn(64, 64, device=cuda), None, True,
+                                              with_bits=True, keep_rows=True)
+    assert out.shape == (0, 64) and bits.shape == (0, 2) and rows.shape == (0, 64)

@@ -292,8 +292,15 @@ __global__ __launch_bounds__(kBlock) void f2v_tail_pack_k(const float *__restric
     if (idx >= NS * NTD * 64) return;
     const int lane = idx & 63, nt = (idx >> 6) % NTD, s = (idx >> 6) / NTD;
     const int n = 16 * nt + (lane & 15), kg = lane >> 4;
+    // the column's largest weight: Kc is 32 or 64, all requests of a batch of 32 leave together
     float m = 0.f;
-    for (int k = 0; k < Kc; ++k) m = fmaxf(m, fabsf(Wd[(size_t)k * Cd + n]));
+    for (int k0 = 0; k0 < Kc; k0 += 32) {
+        float wv[32];
+#pragma unroll
+        for (int k = 0; k < 32; ++k) wv[k] = k0 + k < Kc ? Wd[(size_t)(k0 + k) * Cd + n] : 0.f;
+#pragma unroll
+        for (int k = 0; k < 32; ++k) m = fmaxf(m, fabsf(wv[k]));
+    }
     float inv;
     const float beta = pow2_scale(m, &inv);
     float t[8];

@@ -297,7 +297,7 @@ __global__ __launch_bounds__(kBlock) void f2v_tail_pack_k(const float *__restric
     for (int k0 = 0; k0 < Kc; k0 += 32) {
         float wv[32];
 #pragma unroll
-        for (int k = 0; k < 32; ++k) wv[k] = k0 + k < Kc ? Wd[(size_t)(k0 + k) * Cd + n] : 0.f;
+        for (int k = 0; k < 32; ++k) wv[k] = Wd[(size_t)(k0 + k) * Cd + n];      // (Kc is a multiple of 32)
 #pragma unroll
         for (int k = 0; k < 32; ++k) m = fmaxf(m, fabsf(wv[k]));
     }
@@ -307,7 +307,7 @@ __global__ __launch_bounds__(kBlock) void f2v_tail_pack_k(const float *__restric
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
         const int k = 32 * s + 8 * kg + j;
-        t[j] = k < Kc ? Wd[(size_t)k * Cd + n] * beta : 0.f;
+        t[j] = Wd[(size_t)k * Cd + n] * beta;
     }
     u32x4 hi, lo;
     split8h(t, hi, lo);

@@ -161,6 +161,43 @@ def test_f2v_full_size_adjoints(cuda, scene):
     assert float((y[touched] - 0.75).abs().max()) <= 1e-6
 
 
+def test_f2v_with_its_tail_full_size(cuda, scene):
+    """facet2vertex and its pointwise tail in one pass on the whole scene batch: the kept rows are the convolution
+    kernel's rows bit for bit, the output agrees with the two native passes (each of which is checked against the
+    oracle at this size) and with the float64 oracle composition on sampled vertices, the mask bits with the output."""
+    from oracle import torch_ref as R
+    from picassoplus_amd.mesh.pi_modules import dense, mesh_conv3d
+    d = scene
+    say("case f2v + tail full size", d["nf"], d["nv"])
+    gen = torch.Generator(device=cuda).manual_seed(17)
+    C, Co = d["C"], 64
+    x = torch.randn(d["nf"], C, device=cuda, generator=gen)
+    w = torch.randn(C, Co, device=cuda, generator=gen) / 8
+    b = torch.randn(Co, device=cuda, generator=gen)
+    args = (x, d["w_f2v"], d["coeff"], d["face"], d["nfc"], d["vt_map"])
+    assert dense.f2v_dense_supported(x, d["w_f2v"], d["coeff"], w)
+    out, bits, rows = dense.f2v_dense_forward(*args, w, b, True, with_bits=True, keep_rows=True)
+    conv = mesh_conv3d.facet2vertex_forward(*args)
+    two = dense.dense_tail_forward(conv, w, b, True)
+    torch.cuda.synchronize()
+    assert torch.equal(rows, conv)
+    assert float((out - two).abs().max()) <= 2e-6 * float(two.abs().max())
+    assert torch.equal(dense.f2v_dense_forward(*args, w, b, True), out)
+    cols = torch.arange(Co, device=cuda)
+    assert torch.equal(((bits[:, cols // 32] >> (cols % 32)) & 1).bool(), out > 0)
+    rng = np.random.default_rng(19)
+    f_np = d["face_np"].astype(np.int64)
+    pick_v = np.sort(rng.choice(d["nv"], 2000, replace=False))
+    is_pick = np.zeros(d["nv"], bool)
+    is_pick[pick_v] = True
+    around = np.nonzero(is_pick[f_np].any(1))[0]
+    sub = loops.f2v_fwd(x.cpu().numpy().astype(np.float64)[around], d["w_f2v"].cpu().numpy().astype(np.float64),
+                        d["coeff"].cpu().numpy().astype(np.float64)[around], f_np[around].astype(np.int32),
+                        d["nfc"].cpu().numpy(), np.arange(d["nv"], dtype=np.int32))
+    ref = R.dense_tail_fwd(torch.from_numpy(sub[pick_v]), w.double().cpu(), b.double().cpu(), True).numpy()
+    assert_close(out[torch.from_numpy(pick_v).to(cuda)], ref, "f2v + tail out (sampled vertices)")
+
+
 def test_v2f_full_size_adjoints(cuda, scene):
     d = scene
     gen = torch.Generator(device=cuda).manual_seed(8)

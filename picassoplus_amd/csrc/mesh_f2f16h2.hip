@@ -1657,8 +1657,6 @@ __global__ __launch_bounds__(256, 1) void f2f16h2_bwd_filt_k(const TIO *__restri
 
     // accumulator (cp, t): lane (co = 32t + l32, half h), register i <-> row m = 8(i/4) + 4h + i%4
     // = (channel c0 + 2 NCP w + 2cp + m/16, d = m%16); four consecutive d's per group of four registers
-    // accumulator (cp, t): lane (co = 32t + l32, half h), register i <-> row m = 8(i/4) + 4h + i%4
-    // = (channel c0 + 2 NCP w + 2cp + m/16, d = m%16); four consecutive d's per group of four registers
     const float unscale = sc.S != 0.f ? 1.0f / sc.S : 0.f;
     float *dst = partial + (int64_t)blockIdx.x * Cout * Cin * 16;
 #pragma unroll

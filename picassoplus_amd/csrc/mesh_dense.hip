@@ -1,5 +1,6 @@
-// The pointwise tail of the mesh convolutions on the matrix cores (gfx950, v_mfma_f32_32x32x2_f32, fp32
-// operands and accumulators): out = act(rows . W + bias) [* scale + shift], and its gradients.  The
+// The pointwise tail of the mesh convolutions on the matrix cores (gfx950; v_mfma_f32_32x32x16_bf16 with both
+// operands split exactly into three bf16 pieces, or v_mfma_f32_32x32x2_f32 behind a switch; fp32
+// accumulators): out = act(rows . W + bias) [* scale + shift], and its gradients.  The
 // reference runs this tail as separate PyTorch ops after every convolution (picasso/mesh/layers.py:114-119,
 // 169-174, 232-238: matmul with depth_weights, + biases, activation, batch norm); here the bias, the ReLU and
 // an inference-mode batch norm ride in the epilogue of the product, and the ReLU mask of the backward pass

@@ -4,12 +4,14 @@
 //     x = x1 + x2 + e,   x1 = x rounded to 11 significant bits,  x2 = (x - x1) rounded to 11 bits,  |e| <= 2^-23 |x|
 // and the product is accumulated in fp32 from three piece products,
 //     G.W ~ G2W1 + G1W2 + G1W1                        (the dropped G2W2 is <= 2^-22 relative),
-// three v_mfma_f32_32x32x16_f16 where the three-piece bf16 split needs six, and 24 instead of 44 vector
+// three v_mfma_f32_32x32x16_f16 where the three-piece bf16 split needs six, and 16 instead of 44 vector
 // instructions per eight values split.  fp16 has a narrow exponent range, so both operands are brought
 // to a fixed magnitude by exact power-of-two scales that are taken out of the accumulator at the end:
 //     W' = beta * W        beta from max|W| (one scalar per filter, computed by filter_scale)
 //     G'_f = alpha_f * G_f alpha_f from a bound on max|G_f| = max|tex rows of f| * max|SH rows of f|,
-//                          found by a pre-scan of the facet's rows; it rides on the SH values in registers
+//                          taken from the first fetches of the facet's first sweep with head room (every later
+//                          value is checked against it; a workgroup whose bound did not hold starts over with
+//                          the exact maxima); it rides on the SH values in registers
 // so that |W'|, |G'| < 2^14.  Elements far below their row's maximum (by more than 2^17) fall into fp16's
 // subnormal range and keep an ABSOLUTE error of 2^-25 in scaled units, i.e. below 2^-39 of the row maximum.
 //

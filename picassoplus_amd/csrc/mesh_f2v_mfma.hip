@@ -1,4 +1,5 @@
-// facet2vertex with the filter combination on the matrix cores (fp32 MFMA), 16 SH coefficients.
+// facet2vertex with the filter combination on the matrix cores, 16 SH coefficients: two-piece fp16 products
+// (three v_mfma_f32_32x32x16_f16 per block) by default, the fp32 instruction (eight v_mfma_f32_32x32x2_f32) behind a switch.
 //
 //   w[e,co]   = sum_k coeff[f_e,k] * filt[k,co]        one 32 x 16 x 32 product per 32 entries and 32 channels
 //   out[v,co] = (1/nf[v]) * sum_{e of v} w[e,co] * in[f_e, co/r]

@@ -185,6 +185,17 @@ int pmesh_f2f_bwd_texture(const float *grad_output, const float *filter, const f
                           const int32_t *cum_texture, const int32_t *facet_order, float *grad_texture,
                           void *workspace, size_t workspace_bytes, int64_t T, int64_t Nf, int Cin,
                           int Cout, int F, pmesh_stream_t stream);
+/* pmesh_f2f_bwd_texture with the result ADDED to what grad_texture holds (rows that belong to no facet are left as
+ * they are): a convolution with more than 16 coefficients runs as a sum over blocks of 16 (the texture gradient is
+ * linear in the pair filter x coefficients), and the blocks after the first add onto the first one's result in
+ * place instead of through a separate pass.  No counterpart in the reference.  Only where
+ * pmesh_f2f_bwd_texture_onto_supported returns 1 (F == 16, Cout % 8 == 0, 16-byte aligned arrays). */
+int pmesh_f2f_bwd_texture_onto_supported(const float *grad_output, const float *filter, const float *bary_coeff,
+                                         int Cout, int F);
+int pmesh_f2f_bwd_texture_onto(const float *grad_output, const float *filter, const float *bary_coeff,
+                               const int32_t *cum_texture, const int32_t *facet_order, float *grad_texture,
+                               void *workspace, size_t workspace_bytes, int64_t T, int64_t Nf, int Cin,
+                               int Cout, int F, pmesh_stream_t stream);
 int pmesh_f2f_bwd_filter(const float *grad_output, const float *texture, const float *bary_coeff,
                          const int32_t *cum_texture, const int32_t *facet_order, float *grad_filter,
                          void *workspace, size_t workspace_bytes, int64_t T, int64_t Nf, int Cin,

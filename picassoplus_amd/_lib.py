@@ -11,7 +11,7 @@ from ctypes import c_char_p, c_float, c_int, c_int64, c_size_t, c_void_p
 _HERE = os.path.dirname(os.path.abspath(__file__))
 # PICASSO_MESH_LIB points at an alternative build of the same ABI (kernel experiments)
 LIB_PATH = os.environ.get("PICASSO_MESH_LIB") or os.path.join(_HERE, "csrc", "libpicasso_mesh.so")
-ABI_VERSION = 20
+ABI_VERSION = 21
 
 P, I, L, Z = c_void_p, c_int, c_int64, c_size_t
 
@@ -67,6 +67,8 @@ SIGNATURES = {
     "pmesh_reload_options": (None, []),
     "pmesh_f2f_bwd": (I, [P, P, P, P, P, P, P, P, P, Z, L, L, I, I, I, P]),
     "pmesh_f2f_bwd_texture": (I, [P, P, P, P, P, P, P, Z, L, L, I, I, I, P]),
+    "pmesh_f2f_bwd_texture_onto": (I, [P, P, P, P, P, P, P, Z, L, L, I, I, I, P]),
+    "pmesh_f2f_bwd_texture_onto_supported": (I, [P, P, P, I, I]),
     "pmesh_f2f_bwd_filter": (I, [P, P, P, P, P, P, P, Z, L, L, I, I, I, P]),
     "pmesh_f2f_bwd_bf16_workspace_bytes": (Z, [L, L, I, I, I]),
     "pmesh_f2f_fwd_bf16": (I, [P, P, P, P, P, P, P, Z, L, L, I, I, I, P]),

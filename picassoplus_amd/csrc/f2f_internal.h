@@ -34,7 +34,7 @@ size_t f2f16h2_bwd_texture_workspace_bytes(int Cin, int Cout);
 size_t f2f16h2_bwd_texture_bf16_workspace_bytes(int64_t T, int Cin, int Cout);
 int f2f16h2_bwd_texture(const void *gout, const float *W, const float *sh, const int *cum, const int *order,
                         void *gtex, void *workspace, size_t workspace_bytes, int64_t T, int64_t Nf, int Cin,
-                        int Cout, hipStream_t st, bool half = false, bool bf16 = false);
+                        int Cout, hipStream_t st, bool half = false, bool bf16 = false, bool onto = false);
 
 // texture gradient on the bf16 matrix cores (Cout % 8 == 0, 16-byte aligned grad_output; output channels are
 // taken 64 at a time, later blocks accumulate onto grad_texture)

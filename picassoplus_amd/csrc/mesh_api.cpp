@@ -53,7 +53,7 @@ const Options &options()
 }  // namespace pmesh
 
 extern "C" const char *pmesh_last_error(void) { return pmesh::g_err; }
-extern "C" int pmesh_abi_version(void) { return 20; }
+extern "C" int pmesh_abi_version(void) { return 21; }
 extern "C" void pmesh_reload_options(void)
 {
     std::lock_guard<std::mutex> hold(pmesh::g_options_lock);

@@ -461,6 +461,28 @@ extern "C" int pmesh_f2f_bwd_texture(const float *grad_output, const float *filt
     return 0;
 }
 
+extern "C" int pmesh_f2f_bwd_texture_onto_supported(const float *grad_output, const float *filter, const float *bary_coeff,
+                                                   int Cout, int F)
+{
+    return (!force_generic() && !force_bf16x3() && f2f16x3_usable(filter, bary_coeff, F) &&
+            f2f16x3_bwd_texture_usable(grad_output, Cout)) ? 1 : 0;
+}
+
+extern "C" int pmesh_f2f_bwd_texture_onto(const float *grad_output, const float *filter, const float *bary_coeff,
+                                          const int32_t *cum_texture, const int32_t *facet_order, float *grad_texture,
+                                          void *workspace, size_t workspace_bytes, int64_t T, int64_t Nf, int Cin,
+                                          int Cout, int F, pmesh_stream_t stream)
+{
+    clear_error();
+    PM_F2F_DIMS("f2f_bwd_texture_onto");
+    if (Nf == 0 || T == 0) return 0;
+    PM_REQUIRE(grad_output && filter && bary_coeff && cum_texture && grad_texture, "f2f_bwd_texture_onto: null pointer");
+    PM_REQUIRE(pmesh_f2f_bwd_texture_onto_supported(grad_output, filter, bary_coeff, Cout, F),
+               "f2f_bwd_texture_onto: takes 16 coefficients, a multiple of 8 output channels and 16-byte aligned arrays (F=%d Cout=%d)", F, Cout);
+    return f2f16h2_bwd_texture(grad_output, filter, bary_coeff, cum_texture, facet_order, grad_texture, workspace,
+                               workspace_bytes, T, Nf, Cin, Cout, (hipStream_t)stream, want_half(), false, true);
+}
+
 extern "C" int pmesh_f2f_bwd_filter(const float *grad_output, const float *texture, const float *bary_coeff,
                                     const int32_t *cum_texture, const int32_t *facet_order, float *grad_filter, void *workspace,
                                     size_t workspace_bytes, int64_t T, int64_t Nf, int Cin, int Cout, int F,

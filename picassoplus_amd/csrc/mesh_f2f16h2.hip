@@ -901,7 +901,8 @@ __global__ __launch_bounds__(512, 1) void f2f16h2_bwd_tex_k(const TIN *__restric
                                                             const float *__restrict__ sh,
                                                             const int *__restrict__ cum,
                                                             const int *__restrict__ order, TIO *__restrict__ gtex,
-                                                            int64_t Nf, int T, int Cin, int Cout, int NG, int co0)
+                                                            int64_t Nf, int T, int Cin, int Cout, int NG, int co0,
+                                                            int onto)
 {
     __shared__ u32x4 Ws[3 * kHTChunkMax];
     __shared__ __attribute__((aligned(16))) float s_stage[8][kHTKB * 32 * 16];
@@ -946,7 +947,7 @@ __global__ __launch_bounds__(512, 1) void f2f16h2_bwd_tex_k(const TIN *__restric
     float shs = 0.f;
     // The first sweep starts without a barrier in front (which would wait for the gout rows): every workgroup runs
     // it, and the barrier of its set-up is the one that makes the wavefronts' point counts visible to all.
-#define PM_H2T(N, FIRST, X) h2_tex_sweep<N, NKS, GVEC, HALF, FIRST, TIO>(WpT, sh, gtex, Ws, s_stage[w], s_k0[w], s_K[w], X, bp, kbase, Ks, K, ibeta, shs, sw, Cin, NG, co0 > 0, lane, h)
+#define PM_H2T(N, FIRST, X) h2_tex_sweep<N, NKS, GVEC, HALF, FIRST, TIO>(WpT, sh, gtex, Ws, s_stage[w], s_k0[w], s_K[w], X, bp, kbase, Ks, K, ibeta, shs, sw, Cin, NG, co0 > 0 || onto, lane, h)
     {
         const int sw = 0, kbase = k0;
         const int Ks = K > kHTKB ? kHTKB : K;
@@ -1007,8 +1008,9 @@ __global__ __launch_bounds__(kBlock) void f2f16h2_rows_to_bf16_k(const float *__
 
 int f2f16h2_bwd_texture(const void *gout_, const float *W, const float *sh, const int *cum, const int *order,
                         void *gtex_, void *workspace, size_t workspace_bytes, int64_t T, int64_t Nf, int Cin,
-                        int Cout, hipStream_t st, bool half, bool bf16)
+                        int Cout, hipStream_t st, bool half, bool bf16, bool onto)
 {
+    // onto: the result is added to what grad_texture holds (every block of output channels then adds, the first too)
     const int NG = (Cin + 7) / 8;
     PM_REQUIRE(workspace && workspace_bytes >= f2f16h2_bwd_texture_workspace_bytes(Cin, Cout),
                "f2f_bwd_texture: workspace too small (%zu bytes)", workspace_bytes);
@@ -1036,7 +1038,7 @@ int f2f16h2_bwd_texture(const void *gout_, const float *W, const float *sh, cons
         const int n = NG * 4 * NKS * 64;
         f2f16h2_pack_filter_t_k<<<dim3((unsigned)ceil_div(n, kBlock)), dim3(kBlock), 0, st>>>(W, hdr, WpT, Cin, Cout, NG * 4, NKS, co0);
         PM_LAUNCHED("f2f_bwd_texture(pack)");
-#define PM_TEX(N, G, H, TIN, TIO, DST) f2f16h2_bwd_tex_k<N, G, H, TIN, TIO><<<dim3((unsigned)gx), dim3(512), 0, st>>>((const TIN *)gout_, hdr, WpT, sh, cum, order, (TIO *)(DST), Nf, (int)T, Cin, Cout, NG, co0)
+#define PM_TEX(N, G, H, TIN, TIO, DST) f2f16h2_bwd_tex_k<N, G, H, TIN, TIO><<<dim3((unsigned)gx), dim3(512), 0, st>>>((const TIN *)gout_, hdr, WpT, sh, cum, order, (TIO *)(DST), Nf, (int)T, Cin, Cout, NG, co0, onto ? 1 : 0)
         if (bf16 && gtex32) {
             if (NKS == 2) PM_TEX(2, true, true, bf16_t, float, gtex32);
             else PM_TEX(4, true, true, bf16_t, float, gtex32);

@@ -87,12 +87,13 @@ def _f2v_blocks_of_16(input, filter, coeff):
         return None
     n = (K + 15) // 16
     pad = torch.nn.functional.pad
+    cblocks = topology.coefficient_blocks(coeff)                      # (cut once per coefficient tensor, not per call)
     blocks = []
     for j in range(n):
         if 16 * j + 16 <= K:
-            blocks.append((filter[16 * j:16 * j + 16].contiguous(), coeff[:, 16 * j:16 * j + 16].contiguous()))
+            blocks.append((filter[16 * j:16 * j + 16].contiguous(), cblocks[j]))
         else:                                                        # (only the last block is padded)
-            blocks.append((pad(filter[16 * j:], (0, 0, 0, 0, 0, 16 * j + 16 - K)), pad(coeff[:, 16 * j:], (0, 16 * j + 16 - K))))
+            blocks.append((pad(filter[16 * j:], (0, 0, 0, 0, 0, 16 * j + 16 - K)), cblocks[j]))
     return blocks
 
 
@@ -179,7 +180,8 @@ def _blocks_of_16(input, filter, bary_coeff):
     pad = torch.nn.functional.pad
     cut = lambda t, j: (t[..., 16 * j:16 * j + 16].contiguous() if 16 * j + 16 <= F        # (only the last block is padded)
                         else pad(t[..., 16 * j:], (0, 16 * j + 16 - F)))
-    return [(cut(filter, j), cut(bary_coeff, j)) for j in range(n)]
+    cblocks = topology.coefficient_blocks(bary_coeff)                 # (cut once per coefficient tensor, not per call)
+    return [(cut(filter, j), cblocks[j]) for j in range(n)]
 
 
 def facet2facet_forward(input, filter, bary_coeff, num_texture):
@@ -258,9 +260,21 @@ def facet2facet_backward_selected(grad_output, input, filter, bary_coeff, num_te
         # the texture gradient is the sum over the blocks, the filter gradient their concatenation
         gin, parts = None, []
         for fb, bb in blocks:
-            g_in, g_f = facet2facet_backward_selected(grad_output, input, fb, bb, num_texture, needs)
-            if needs[0]:
-                gin = g_in if gin is None else gin.add_(g_in)
+            if needs[0] and gin is not None and _lib.query("pmesh_f2f_bwd_texture_onto_supported", grad_output.data_ptr(),
+                                                           fb.data_ptr(), bb.data_ptr(), Cout, 16):
+                # the later blocks add their texture gradient onto the first one's in place
+                with torch.cuda.device(dev):
+                    nbytes = _lib.query("pmesh_f2f_bwd_workspace_bytes_for", Nf, Cin, Cout, 16)
+                    ws = workspace(nbytes, dev)
+                    order = topology.facet_order(num_texture, T) if Nf else None
+                    _lib.call("pmesh_f2f_bwd_texture_onto", grad_output.data_ptr(), fb.data_ptr(), bb.data_ptr(),
+                              num_texture.data_ptr(), order.data_ptr() if order is not None else None, gin.data_ptr(),
+                              ws.data_ptr(), nbytes, T, Nf, Cin, Cout, 16, stream_of(input))
+                g_f = facet2facet_backward_selected(grad_output, input, fb, bb, num_texture, (False, needs[1]))[1]
+            else:
+                g_in, g_f = facet2facet_backward_selected(grad_output, input, fb, bb, num_texture, needs)
+                if needs[0]:
+                    gin = g_in if gin is None else gin.add_(g_in)
             parts.append(g_f)
         return [gin, torch.cat(parts, 2)[:, :, :F].contiguous() if needs[1] else None]
     sfx = "_bf16" if input.dtype == BF16 else ""

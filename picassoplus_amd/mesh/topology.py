@@ -47,6 +47,7 @@ class _Entry:
 def clear_cache():
     global _BYTES
     with _LOCK:
+        _BLOCKS.clear()
         for e in _CACHE.values():
             for fin in e.finalizers:
                 fin.detach()
@@ -263,6 +264,41 @@ def running_total(num_texture):
     total = torch.cumsum(num_texture, dim=0, dtype=torch.int)
     _store(key, total, (num_texture,), (total,))
     return total
+
+
+_BLOCKS = {}            # device index -> (key, [blocks]): the coefficient blocks of the tensor seen last on that device
+
+
+def coefficient_blocks(coeff):
+    """A (rows, K) coefficient tensor cut into ceil(K / 16) contiguous blocks of 16 columns, the last one padded
+    with zeros: what the 16-coefficient matrix-core kernels take for other spherical-harmonic degrees.  The
+    blocks of the tensor seen last on a device are kept (the forward and the backward pass of a layer, and the
+    layers of one mesh level, hand in the same tensor), so that they are cut once and not once per native call;
+    they go when the tensor does, or when another one takes their place."""
+    key = _key("b", coeff)
+    dev = coeff.device.index
+    stream = torch.cuda.current_stream(coeff.device).cuda_stream if coeff.is_cuda else None
+    with _LOCK:
+        hit = _BLOCKS.get(dev)
+        if hit is not None and hit[0] == key and hit[2] == stream:      # (another stream cuts its own: no event to wait for)
+            return hit[1]
+    K = coeff.shape[1]
+    pad = torch.nn.functional.pad
+    blocks = [coeff[:, 16 * j:16 * j + 16].contiguous() if 16 * j + 16 <= K else pad(coeff[:, 16 * j:], (0, 16 * j + 16 - K))
+              for j in range((K + 15) // 16)]
+    if torch.cuda.is_current_stream_capturing():
+        return blocks                                   # (a capture keeps its own tensors alive; nothing to share)
+
+    def forget(dev=dev, key=key):
+        with _LOCK:
+            if dev in _BLOCKS and _BLOCKS[dev][0] == key:
+                del _BLOCKS[dev]
+
+    with _LOCK:
+        _BLOCKS[dev] = (key, blocks, stream)
+    fin = weakref.finalize(coeff, forget)
+    fin.atexit = False
+    return blocks
 
 
 def checked_once(kind, owners, extra, check):

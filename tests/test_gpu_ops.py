@@ -531,6 +531,45 @@ def test_f2f_without_facet_order(cuda):
     assert float((w1 - w2).abs().max()) <= 1e-5 * float(w1.abs().max())
 
 
+@pytest.mark.parametrize("nf,Cin,Cout", [(900, 24, 40), (257, 64, 64), (130, 8, 128)])
+def test_f2f_texture_gradient_added_in_place(cuda, nf, Cin, Cout):
+    """pmesh_f2f_bwd_texture_onto adds the texture gradient to what the array holds -- rows that belong to no facet stay
+    as they are -- and gives the plain entry point's result on top of it; the coefficient blocks of another degree are
+    cut once per tensor and cut again when the tensor's contents change."""
+    from picassoplus_amd import _lib
+    say("case f2f texture gradient in place", nf, Cin, Cout)
+    rng = np.random.default_rng(56)
+    counts, bary, _ = texture_case(rng, nf, 9)
+    T = int(counts.sum()) + 5                              # five rows that belong to no facet
+    sh = dev(rng.normal(0, 0.5, (T, 16)), cuda, torch.float32)
+    w = dev(rng.normal(0, 0.3, (Cout, Cin, 16)), cuda, torch.float32)
+    g = dev(rng.normal(0, 1, (nf, Cout)), cuda, torch.float32)
+    cum = torch.cumsum(dev(counts, cuda), 0, dtype=torch.int32)
+    order = topology.facet_order(cum, T)
+    st = torch.cuda.current_stream().cuda_stream
+    nbw = _lib.query("pmesh_f2f_bwd_workspace_bytes", Cin, Cout, 16)
+    ws = torch.empty(nbw, dtype=torch.uint8, device=cuda)
+    assert _lib.query("pmesh_f2f_bwd_texture_onto_supported", g.data_ptr(), w.data_ptr(), sh.data_ptr(), Cout, 16) == 1
+    plain = torch.empty(T, Cin, device=cuda)
+    _lib.call("pmesh_f2f_bwd_texture", g.data_ptr(), w.data_ptr(), sh.data_ptr(), cum.data_ptr(), order.data_ptr(),
+              plain.data_ptr(), ws.data_ptr(), nbw, T, nf, Cin, Cout, 16, st)
+    base = torch.randn(T, Cin, device=cuda)
+    onto = base.clone()
+    _lib.call("pmesh_f2f_bwd_texture_onto", g.data_ptr(), w.data_ptr(), sh.data_ptr(), cum.data_ptr(), order.data_ptr(),
+              onto.data_ptr(), ws.data_ptr(), nbw, T, nf, Cin, Cout, 16, st)
+    torch.cuda.synchronize()
+    assert torch.equal(plain[-5:], torch.zeros(5, Cin, device=cuda)) and torch.equal(onto[-5:], base[-5:])
+    assert float((onto - (base + plain)).abs().max()) <= 2e-7 * float((base.abs() + plain.abs()).max())
+    # other degrees: the cached coefficient blocks follow the tensor's contents
+    sh25 = dev(rng.normal(0, 0.5, (T, 25)), cuda, torch.float32)
+    b1 = topology.coefficient_blocks(sh25)
+    assert topology.coefficient_blocks(sh25) is b1 and len(b1) == 2 and tuple(b1[1].shape) == (T, 16)
+    assert torch.equal(b1[0], sh25[:, :16]) and torch.equal(b1[1][:, :9], sh25[:, 16:]) and not b1[1][:, 9:].any()
+    sh25.mul_(2.0)
+    b2 = topology.coefficient_blocks(sh25)
+    assert b2 is not b1 and torch.equal(b2[0], sh25[:, :16])
+
+
 def test_f2f_shape_sweep(cuda):
     """Seeded sweep over channel counts, facet counts and point counts around the tile sizes of the
     16-coefficient kernels (32-facet wavefront tiles, 4/8/16-channel groups, 64-channel blocks)."""
